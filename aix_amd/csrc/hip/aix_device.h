@@ -1,0 +1,244 @@
+// aix_device.h -- device-side element types, conversions and per-element operators.
+//
+// Shared by the precompiled kernels and by every runtime-generated fused kernel (the text of
+// this file is the hipRTC prelude), so it includes nothing and uses only compiler builtins and
+// the device math library that hipcc/hipRTC declare implicitly.
+//
+// Semantics mirror the reference CPU device (Targets/AIXLib/aixDeviceCPU.cpp) and its software
+// 16-bit floats (Targets/AIXLib/aixFloat16.hpp):
+//   * f16 / bf16 arithmetic happens in f32 and is rounded to 16 bits (RNE) after EVERY operator;
+//   * integer arithmetic wraps; float -> integer conversion saturates and maps NaN to 0
+//     (aixDeviceCPU.cpp:96-117);
+//   * sqrt/log/exp/pow on integer element types evaluate in floating point and saturate back;
+//     sin/cos/tanh on integers truncate toward zero (aixDeviceCPU.cpp:154-242);
+//   * compile with -ffp-contract=off: a*b+c must stay two roundings.
+#ifndef AIX_DEVICE_H
+#define AIX_DEVICE_H
+
+namespace aixd {
+
+typedef signed char        i8;
+typedef unsigned char      u8;
+typedef short              i16;
+typedef unsigned short     u16;
+typedef int                i32;
+typedef unsigned int       u32;
+typedef long long          i64;
+typedef unsigned long long u64;
+typedef _Float16           f16;
+
+// bfloat16 storage word.  Conversion is done on the integer image so that NaN handling is the
+// reference's: truncate and set bit 6 (aixFloat16.hpp:783-805).
+struct bf16 { u16 bits; };
+
+__device__ __forceinline__ float bf16_up(bf16 v) { return __builtin_bit_cast(float, (u32)v.bits << 16); }
+__device__ __forceinline__ bf16 bf16_down(float f)
+{
+    const u32 u = __builtin_bit_cast(u32, f);
+    bf16 r;
+    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) { r.bits = (u16)((u >> 16) | 0x40u); return r; }
+    r.bits = (u16)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);        // round to nearest even
+    return r;
+}
+
+enum { DT_F64 = 0, DT_F32 = 1, DT_F16 = 2, DT_BF16 = 3, DT_I64 = 4, DT_I32 = 5, DT_I16 = 6, DT_I8 = 7, DT_U8 = 8 };
+
+// ---- traits ---------------------------------------------------------------------------------
+// W = type in which one operator is evaluated before rounding back to T.
+template <class T> struct traits;
+template <> struct traits<double> { typedef double W; enum { code = DT_F64, is_float = 1, is_int = 0 }; };
+template <> struct traits<float>  { typedef float  W; enum { code = DT_F32, is_float = 1, is_int = 0 }; };
+template <> struct traits<f16>    { typedef float  W; enum { code = DT_F16, is_float = 1, is_int = 0 }; };
+template <> struct traits<bf16>   { typedef float  W; enum { code = DT_BF16, is_float = 1, is_int = 0 }; };
+template <> struct traits<i64>    { typedef i64 W; typedef u64 U; enum { code = DT_I64, is_float = 0, is_int = 1, is_signed = 1 }; };
+template <> struct traits<i32>    { typedef i32 W; typedef u32 U; enum { code = DT_I32, is_float = 0, is_int = 1, is_signed = 1 }; };
+template <> struct traits<i16>    { typedef i32 W; typedef u32 U; enum { code = DT_I16, is_float = 0, is_int = 1, is_signed = 1 }; };
+template <> struct traits<i8>     { typedef i32 W; typedef u32 U; enum { code = DT_I8,  is_float = 0, is_int = 1, is_signed = 1 }; };
+template <> struct traits<u8>     { typedef i32 W; typedef u32 U; enum { code = DT_U8,  is_float = 0, is_int = 1, is_signed = 0 }; };
+
+template <class T> __device__ __forceinline__ typename traits<T>::W up(T v) { return (typename traits<T>::W)v; }
+template <> __device__ __forceinline__ float up<bf16>(bf16 v) { return bf16_up(v); }
+template <class T> __device__ __forceinline__ T down(typename traits<T>::W v) { return (T)v; }
+template <> __device__ __forceinline__ bf16 down<bf16>(float v) { return bf16_down(v); }
+
+template <class T> __device__ __forceinline__ T zero() { return down<T>((typename traits<T>::W)0); }
+
+// lowest(): aixDeviceCPU.cpp:130-138, aixFloat16.hpp:173-178, 767-772.
+template <class T> __device__ __forceinline__ T lowest();
+template <> __device__ __forceinline__ double lowest<double>() { return -1.7976931348623157e308; }
+template <> __device__ __forceinline__ float  lowest<float>()  { return -3.402823466e38f; }
+template <> __device__ __forceinline__ f16    lowest<f16>()    { return __builtin_bit_cast(f16, (u16)0xFBFF); }
+template <> __device__ __forceinline__ bf16   lowest<bf16>()   { bf16 r; r.bits = 0xFF7F; return r; }
+template <> __device__ __forceinline__ i64    lowest<i64>()    { return (i64)0x8000000000000000ull; }
+template <> __device__ __forceinline__ i32    lowest<i32>()    { return (i32)0x80000000u; }
+template <> __device__ __forceinline__ i16    lowest<i16>()    { return (i16)-32768; }
+template <> __device__ __forceinline__ i8     lowest<i8>()     { return (i8)-128; }
+template <> __device__ __forceinline__ u8     lowest<u8>()     { return (u8)0; }
+
+// ---- conversions ----------------------------------------------------------------------------
+// double -> integer with saturation, NaN -> 0.
+template <class D> __device__ __forceinline__ D sat_from_double(double x);
+template <> __device__ __forceinline__ i64 sat_from_double<i64>(double x)
+{
+    if (x != x) return 0;
+    if (x >= 9223372036854775808.0) return (i64)0x7FFFFFFFFFFFFFFFull;
+    if (x <= -9223372036854775808.0) return (i64)0x8000000000000000ull;
+    return (i64)x;
+}
+template <> __device__ __forceinline__ i32 sat_from_double<i32>(double x)
+{ if (x != x) return 0; x = x < -2147483648.0 ? -2147483648.0 : (x > 2147483647.0 ? 2147483647.0 : x); return (i32)x; }
+template <> __device__ __forceinline__ i16 sat_from_double<i16>(double x)
+{ if (x != x) return 0; x = x < -32768.0 ? -32768.0 : (x > 32767.0 ? 32767.0 : x); return (i16)(i32)x; }
+template <> __device__ __forceinline__ i8 sat_from_double<i8>(double x)
+{ if (x != x) return 0; x = x < -128.0 ? -128.0 : (x > 127.0 ? 127.0 : x); return (i8)(i32)x; }
+template <> __device__ __forceinline__ u8 sat_from_double<u8>(double x)
+{ if (x != x) return 0; x = x < 0.0 ? 0.0 : (x > 255.0 ? 255.0 : x); return (u8)(i32)x; }
+
+// Any element type as double (exact for every type except |i64| > 2^53).
+template <class S> __device__ __forceinline__ double as_double(S v) { return (double)v; }
+template <> __device__ __forceinline__ double as_double<bf16>(bf16 v) { return (double)bf16_up(v); }
+template <> __device__ __forceinline__ double as_double<f16>(f16 v) { return (double)(float)v; }
+
+// convert<S, D>: the value conversion of copy / fill.  Float-like -> integer saturates;
+// everything that targets a 16-bit float goes through float first (aixFloat16.hpp has only a
+// float constructor), everything else is a plain C++ conversion.
+template <class S, class D> struct conv {
+    static __device__ __forceinline__ D run(S v)
+    {
+        if constexpr (traits<S>::is_float && traits<D>::is_int) return sat_from_double<D>(as_double<S>(v));
+        else if constexpr (traits<D>::code == DT_BF16) {
+            if constexpr (traits<S>::code == DT_BF16) return v;
+            else if constexpr (traits<S>::code == DT_F16) return bf16_down((float)v);
+            else return bf16_down((float)v);
+        }
+        else if constexpr (traits<D>::code == DT_F16) {
+            if constexpr (traits<S>::code == DT_BF16) return (f16)bf16_up(v);
+            else return (f16)(float)v;
+        }
+        else if constexpr (traits<S>::code == DT_BF16) return (D)bf16_up(v);
+        else if constexpr (traits<S>::code == DT_F16) return (D)(float)v;
+        else return (D)v;
+    }
+};
+template <class S, class D> __device__ __forceinline__ D convert(S v) { return conv<S, D>::run(v); }
+
+// ---- arithmetic -----------------------------------------------------------------------------
+template <class T> __device__ __forceinline__ T e_add(T a, T b)
+{
+    if constexpr (traits<T>::is_int) { typedef typename traits<T>::U U; return (T)((U)a + (U)b); }
+    else return down<T>(up(a) + up(b));
+}
+template <class T> __device__ __forceinline__ T e_sub(T a, T b)
+{
+    if constexpr (traits<T>::is_int) { typedef typename traits<T>::U U; return (T)((U)a - (U)b); }
+    else return down<T>(up(a) - up(b));
+}
+template <class T> __device__ __forceinline__ T e_mul(T a, T b)
+{
+    if constexpr (traits<T>::is_int) { typedef typename traits<T>::U U; return (T)((U)a * (U)b); }
+    else return down<T>(up(a) * up(b));
+}
+template <class T> __device__ __forceinline__ T e_div(T a, T b)
+{
+    if constexpr (traits<T>::is_int) {
+        // Division by zero and lowest / -1 trap on the CPU; here they are defined: 0 and wrap.
+        typedef typename traits<T>::W W;
+        const W x = (W)a, y = (W)b;
+        if (y == 0) return (T)0;
+        if constexpr (traits<T>::is_signed) { if (y == (W)-1) { typedef typename traits<T>::U U; return (T)((U)0 - (U)a); } }
+        return (T)(x / y);
+    }
+    else return down<T>(up(a) / up(b));
+}
+template <class T> __device__ __forceinline__ T e_neg(T a)
+{
+    if constexpr (traits<T>::is_int) { typedef typename traits<T>::U U; return (T)((U)0 - (U)a); }
+    else return down<T>(-up(a));
+}
+
+// Comparisons in the evaluation type: +-0 equal, NaN unordered (aixFloat16.hpp:66-95).
+template <class T> __device__ __forceinline__ bool e_gt(T a, T b) { return up(a) > up(b); }
+template <class T> __device__ __forceinline__ bool e_lt(T a, T b) { return up(a) < up(b); }
+template <class T> __device__ __forceinline__ bool e_isnan(T a)
+{
+    if constexpr (traits<T>::is_float) { const typename traits<T>::W w = up(a); return w != w; }
+    else return false;
+}
+
+// ---- math -----------------------------------------------------------------------------------
+enum { M_SQRT = 1, M_SIN = 2, M_COS = 3, M_TANH = 4, M_LOG = 5, M_EXP = 6 };
+
+template <int F> __device__ __forceinline__ float math_f32(float x)
+{
+    if constexpr (F == M_SQRT) return __builtin_sqrtf(x);
+    else if constexpr (F == M_SIN) return sinf(x);
+    else if constexpr (F == M_COS) return cosf(x);
+    else if constexpr (F == M_TANH) return tanhf(x);
+    else if constexpr (F == M_LOG) return logf(x);
+    else return expf(x);
+}
+template <int F> __device__ __forceinline__ double math_f64(double x)
+{
+    if constexpr (F == M_SQRT) return __builtin_sqrt(x);
+    else if constexpr (F == M_SIN) return sin(x);
+    else if constexpr (F == M_COS) return cos(x);
+    else if constexpr (F == M_TANH) return tanh(x);
+    else if constexpr (F == M_LOG) return log(x);
+    else return exp(x);
+}
+
+template <int F, class T> __device__ __forceinline__ T e_math(T a)
+{
+    if constexpr (traits<T>::code == DT_F64) return math_f64<F>(a);
+    else if constexpr (traits<T>::is_float) return down<T>(math_f32<F>(up(a)));
+    else {
+        const double r = math_f64<F>((double)a);
+        if constexpr (F == M_SIN || F == M_COS || F == M_TANH) return (T)(i32)r;   // |r| <= 1: truncation
+        else return sat_from_double<T>(r);
+    }
+}
+template <class T> __device__ __forceinline__ T e_sqrt(T a) { return e_math<M_SQRT>(a); }
+template <class T> __device__ __forceinline__ T e_sin(T a)  { return e_math<M_SIN>(a); }
+template <class T> __device__ __forceinline__ T e_cos(T a)  { return e_math<M_COS>(a); }
+template <class T> __device__ __forceinline__ T e_tanh(T a) { return e_math<M_TANH>(a); }
+template <class T> __device__ __forceinline__ T e_log(T a)  { return e_math<M_LOG>(a); }
+template <class T> __device__ __forceinline__ T e_exp(T a)  { return e_math<M_EXP>(a); }
+
+// Integer power as the saturated, truncated real value of base^e (what the CPU's long double
+// evaluation followed by the saturating conversion yields): exact by repeated multiplication on
+// the magnitude, clamped to the range of T; negative exponents give 0 except for bases 0, 1, -1.
+template <class T> __device__ __forceinline__ T int_pow(T base, T e)
+{
+    const i64 b = (i64)base, n = (i64)e;
+    const i64 hi = (i64)(((u64)1 << (8 * sizeof(T) - (traits<T>::is_signed ? 1 : 0))) - 1);   // max of T
+    const i64 lo = traits<T>::is_signed ? -hi - 1 : 0;
+    if (n == 0) return (T)1;
+    if (b == 1) return (T)1;
+    if (b == -1) return (T)((n & 1) ? -1 : 1);
+    if (b == 0) return n > 0 ? (T)0 : (T)hi;                       // 0^negative = +inf -> max
+    if (n < 0) return (T)0;                                        // |b| >= 2: |result| < 1
+    const bool negative = b < 0 && (n & 1);
+    const u64 mag = b < 0 ? (u64)0 - (u64)b : (u64)b;
+    const u64 limit = negative ? (u64)hi + 1 : (u64)hi;            // |lo| or hi
+    u64 r = 1;
+    for (i64 k = 0; k < n; ++k) {
+        if (r > limit / mag) { r = limit + 1; break; }             // would exceed: saturate
+        r *= mag;
+    }
+    if (r > limit) return negative ? (T)lo : (T)hi;
+    return negative ? (T)(i64)((u64)0 - r) : (T)(i64)r;
+}
+
+template <class T> __device__ __forceinline__ T e_pow(T a, T b)
+{
+    if constexpr (traits<T>::code == DT_F64) return pow(a, b);
+    else if constexpr (traits<T>::is_float) return down<T>(powf(up(a), up(b)));
+    else return int_pow<T>(a, b);
+}
+
+// ---- 16-byte vectors of any element type ------------------------------------------------------
+template <class T, int N> struct alignas(sizeof(T) * N) vec { T v[N]; };
+template <class T> struct vec16 { enum { n = 16 / sizeof(T) }; typedef vec<T, 16 / sizeof(T)> type; };
+
+} // namespace aixd
+#endif

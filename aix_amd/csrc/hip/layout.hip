@@ -1,0 +1,366 @@
+// layout.hip -- pure data movement: contiguous (gather a view into a dense tensor), the
+// materialising transpose, sliceSet, tril/triu, indexSelect, indexAdd.
+//
+// Data movement does not look at values, so kernels are instantiated per element SIZE
+// (1, 2, 4, 8 bytes), not per element type.  A 2-D (optionally batched) transposed source is
+// moved through 64x64 LDS tiles so that both the HBM read and the HBM write are coalesced;
+// everything else uses a strided gather with the same three shapes as the elementwise kernels.
+
+#include "common.hpp"
+
+using namespace aixd;
+using namespace aixk;
+
+namespace {
+
+template <int BYTES> struct word;
+template <> struct word<1> { typedef u8 type; };
+template <> struct word<2> { typedef u16 type; };
+template <> struct word<4> { typedef u32 type; };
+template <> struct word<8> { typedef u64 type; };
+
+template <class F> int by_size(int dtype, F&& f)
+{
+    switch (aixk_dtype_size(dtype)) {
+        case 1: return f(u8{});
+        case 2: return f(u16{});
+        case 4: return f(u32{});
+        case 8: return f(u64{});
+        default: return fail(AIXK_EINVAL, "unknown element type %d", dtype);
+    }
+}
+
+// Position of flat logical index i inside one collapsed view.
+template <class IDX> __device__ __forceinline__ u64 locate(const Space<1>& sp, IDX i) { return aixk::locate<1, IDX>(sp, 0, i); }
+
+// ---- strided gather: dst[i] = src[view(i)] -----------------------------------------------------
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void gather_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> sp, u64 n)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock)
+        dst[i] = src[locate<IDX>(sp, (IDX)i)];
+}
+
+// rows: inner dim unit stride, 16-byte chunks
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void gather_rows_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> sp,
+                                                        u64 total_chunks, IDX chunks)
+{
+    typedef typename vec16<W>::type V;
+    constexpr int VEC = vec16<W>::n;
+    Space<1> outer = sp;
+    outer.rank = sp.rank - 1;
+    for (u64 c = (u64)blockIdx.x * kBlock + threadIdx.x; c < total_chunks; c += (u64)gridDim.x * kBlock) {
+        const IDX row = (IDX)(c / chunks);
+        const IDX col = (IDX)(c - (u64)row * chunks) * VEC;
+        const u64 p = locate<IDX>(outer, row) + col;
+        *(V*)(dst + c * VEC) = *(const V*)(src + p);
+    }
+}
+
+// ---- tiled transpose ---------------------------------------------------------------------------
+// Source element (b, r, c) lives at  off + b*sb + r*1 + c*ld   (unit stride along r);
+// destination is dense [B, R, C].  Tile = 64 (r) x 64 (c); 256 lanes.
+// Load: lanes sweep r fastest (coalesced in the source); store: lanes sweep c fastest.
+constexpr int kTile = 64;
+template <class W>
+__global__ __launch_bounds__(kBlock) void transpose_tiled_k(const W* __restrict__ src, W* __restrict__ dst,
+                                                            u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r, u32 tiles_c)
+{
+    __shared__ W tile[kTile][kTile + 1];
+    // XCD-friendly order: consecutive workgroups walk down r so that neighbouring groups share
+    // destination rows' DRAM pages.
+    const u32 t = blockIdx.x;
+    const u32 tr = t % tiles_r, tc = t / tiles_r;
+    const u64 b = blockIdx.y;
+    const u64 r0 = (u64)tr * kTile, c0 = (u64)tc * kTile;
+    const W* s = src + off + b * sb;
+    W* d = dst + b * R * C;
+    const int lx = threadIdx.x & 63, ly = threadIdx.x >> 6;      // 64 x 4
+#pragma unroll 4
+    for (int k = ly; k < kTile; k += 4) {                        // k indexes c within the tile
+        const u64 r = r0 + lx, c = c0 + k;
+        if (r < R && c < C) tile[k][lx] = s[r + c * ld];
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int k = ly; k < kTile; k += 4) {                        // k indexes r within the tile
+        const u64 r = r0 + k, c = c0 + lx;
+        if (r < R && c < C) d[r * C + c] = tile[lx][k];
+    }
+}
+
+// ---- generic strided copy with both sides strided (sliceSet, transpose scatter) ---------------
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void copy_views_k(const W* __restrict__ src, W* __restrict__ dst,
+                                                       Space<1> ssp, Space<1> dsp, u64 n)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock)
+        dst[locate<IDX>(dsp, (IDX)i)] = src[locate<IDX>(ssp, (IDX)i)];
+}
+
+// ---- tril / triu -------------------------------------------------------------------------------
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void tri_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> ssp, Space<1> dsp,
+                                                u64 n, u64 rows, u64 cols, i64 diagonal, int upper)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
+        const i64 r = (i64)((i / cols) % rows), c = (i64)(i % cols);
+        const bool zero = upper ? (c < r + diagonal) : (c > r + diagonal);
+        dst[locate<IDX>(dsp, (IDX)i)] = zero ? (W)0 : src[locate<IDX>(ssp, (IDX)i)];
+    }
+}
+
+// ---- indexSelect -------------------------------------------------------------------------------
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void index_select_k(const W* __restrict__ src, W* __restrict__ dst, const i32* __restrict__ idx,
+                                                         Space<1> ssp, Space<1> isp, u64 n, u64 inner, u64 ni, u64 span)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
+        const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
+        const u64 which = (u64)(i64)idx[locate<IDX>(isp, (IDX)k)];
+        dst[i] = src[locate<IDX>(ssp, (IDX)(o * span + which * inner + e))];
+    }
+}
+
+// ---- indexAdd ----------------------------------------------------------------------------------
+// dst[slot] += src[i] with duplicates summed: atomics.  32/64-bit types use native atomics;
+// 8/16-bit types update their containing 32-bit word with a compare-and-swap loop.
+template <class T> __device__ __forceinline__ void atomic_accumulate(T* base, u64 pos, T val)
+{
+    if constexpr (traits<T>::code == DT_F32) atomicAdd(base + pos, val);
+    else if constexpr (traits<T>::code == DT_F64) atomicAdd(base + pos, val);
+    else if constexpr (traits<T>::code == DT_I32) atomicAdd((int*)base + pos, val);
+    else if constexpr (traits<T>::code == DT_I64) atomicAdd((unsigned long long*)base + pos, (unsigned long long)val);
+    else {
+        const uintptr_t addr = (uintptr_t)(base + pos);
+        u32* wordp = (u32*)(addr & ~(uintptr_t)3);
+        const u32 shift = (u32)(addr & 3) * 8;
+        constexpr u32 mask = sizeof(T) == 1 ? 0xFFu : 0xFFFFu;
+        u32 old = *wordp, assumed;
+        do {
+            assumed = old;
+            typedef typename word<sizeof(T)>::type Wd;
+            const Wd cur_bits = (Wd)((assumed >> shift) & mask);
+            const T cur = __builtin_bit_cast(T, cur_bits);
+            const T nxt = e_add(cur, val);
+            const u32 nxt_bits = (u32)__builtin_bit_cast(Wd, nxt);
+            old = atomicCAS(wordp, assumed, (assumed & ~(mask << shift)) | (nxt_bits << shift));
+        } while (old != assumed);
+    }
+}
+
+template <class T, class IDX>
+__global__ __launch_bounds__(kBlock) void index_add_k(const T* __restrict__ src, T* __restrict__ dst, const i32* __restrict__ idx,
+                                                      Space<1> ssp, Space<1> isp, u64 n, u64 inner, u64 ni, u64 span)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
+        const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
+        const u64 which = (u64)(i64)idx[locate<IDX>(isp, (IDX)k)];
+        atomic_accumulate<T>(dst, o * span + which * inner + e, src[locate<IDX>(ssp, (IDX)i)]);
+    }
+}
+
+// Host routing for dst(dense)[i] = src[view(i)], n elements.
+int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
+{
+    if (n == 0) return AIXK_OK;
+    Space<1> sp;
+    if (!collapse1(src, &sp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const size_t esz = aixk_dtype_size(src->dtype);
+    const unsigned max_blocks = (unsigned)ctx->cus * 32u;
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31);
+
+    // dense already: plain copy
+    if (sp.rank == 0 || (sp.rank == 1 && sp.stride[0][0] == 1)) {
+        AIXK_HIP(hipMemcpyAsync(dst, (const char*)src->data + sp.offset[0] * esz, n * esz, hipMemcpyDeviceToDevice, ctx->stream));
+        return AIXK_OK;
+    }
+    return by_size(src->dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        constexpr int VEC = vec16<W>::n;
+        const W* ps = (const W*)src->data;
+        W* pd = (W*)dst;
+        // 2-D / batched 2-D transposed: [B?, R, C] with strides (sb, 1, ld)
+        if ((sp.rank == 2 && sp.stride[0][0] == 1) || (sp.rank == 3 && sp.stride[0][1] == 1)) {
+            const int o = sp.rank - 2;
+            const uint64_t B = sp.rank == 3 ? sp.shape[0] : 1, sb = sp.rank == 3 ? sp.stride[0][0] : 0;
+            const uint64_t R = sp.shape[o], C = sp.shape[o + 1], ld = sp.stride[0][o + 1];
+            const uint64_t tr = (R + kTile - 1) / kTile, tc = (C + kTile - 1) / kTile;
+            if (ld != 0 && tr * tc < (1ull << 31) && B < 65536) {
+                hipLaunchKernelGGL((transpose_tiled_k<W>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
+                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr, (u32)tc);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            }
+        }
+        // rows: inner dim unit stride and everything 16-byte aligned
+        const int in = sp.rank - 1;
+        if (sp.stride[0][in] == 1 && sp.shape[in] % VEC == 0 && aligned16(pd) && aligned16(ps + sp.offset[0])) {
+            bool ok = true;
+            for (int d = 0; d < in; ++d) if (sp.stride[0][d] % VEC) ok = false;
+            if (ok) {
+                const uint64_t chunks = sp.shape[in] / VEC, total = n / VEC;
+                const unsigned grid = grid_for(total, kBlock, max_blocks);
+                if (small) hipLaunchKernelGGL((gather_rows_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u32)chunks);
+                else hipLaunchKernelGGL((gather_rows_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u64)chunks);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            }
+        }
+        const unsigned grid = grid_for(n, kBlock, max_blocks);
+        if (small) hipLaunchKernelGGL((gather_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)n);
+        else hipLaunchKernelGGL((gather_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)n);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+int copy_views(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t n)
+{
+    if (n == 0) return AIXK_OK;
+    Space<1> ssp, dsp;
+    if (!collapse1(src, &ssp) || !collapse1(dst, &dsp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(dst) < (1ull << 31);
+    return by_size(src->dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
+        if (small) hipLaunchKernelGGL((copy_views_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n);
+        else hipLaunchKernelGGL((copy_views_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+} // namespace
+
+extern "C" {
+
+int32_t aixk_contiguous(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "contiguous: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "contiguous: element types differ");
+    const uint64_t n = dst->size;                    // aixDeviceCPU.cpp:431
+    AIXK_REQUIRE(n == numel(src), "contiguous: dst size does not match the source shape");
+    return gather_into(ctx, src, dst->data, n);
+}
+
+int32_t aixk_transpose(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* out, uint64_t dim0, uint64_t dim1)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(a) && valid_tensor(out), "transpose: bad operand descriptor");
+    AIXK_REQUIRE(a->dtype == out->dtype, "transpose: element types differ");
+    AIXK_REQUIRE((int)dim0 < a->rank && (int)dim1 < a->rank && out->rank == a->rank, "transpose: dims out of range");
+    // Source read through the swapped view; equals the flat read of aixDeviceCPU.cpp:391-405 for
+    // the contiguous sources that function assumes.
+    aixhip_tensor v = *a;
+    v.shape[dim0] = a->shape[dim1]; v.shape[dim1] = a->shape[dim0];
+    v.strides[dim0] = a->strides[dim1]; v.strides[dim1] = a->strides[dim0];
+    uint64_t dense[AIXK_MAX_RANK];
+    row_major_strides(v.rank, v.shape, dense);
+    bool out_dense = true;
+    for (int d = 0; d < v.rank; ++d) if (v.shape[d] > 1 && out->strides[d] != dense[d]) out_dense = false;
+    if (out_dense) return gather_into(ctx, &v, out->data, a->size);
+    aixhip_tensor o = *out;
+    o.offset = 0;                                    // result written from base (aixDeviceCPU.cpp:395-403)
+    std::memcpy(o.shape, v.shape, sizeof(v.shape));
+    return copy_views(ctx, &v, &o, a->size);
+}
+
+int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                       uint64_t dim, uint64_t start, uint64_t end, uint64_t step)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "sliceSet: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "sliceSet: element types differ");
+    AIXK_REQUIRE((int)dim < dst->rank && step > 0 && end >= start, "sliceSet: bad slice");
+    aixhip_tensor window = *dst;                     // the strided window of dst that receives src
+    window.shape[dim] = (end - start + step - 1) / step;
+    window.offset = dst->offset + start * dst->strides[dim];
+    window.strides[dim] = dst->strides[dim] * step;
+    const uint64_t n = src->size;                    // aixDeviceCPU.cpp:477
+    AIXK_REQUIRE(n == numel(&window) && n == numel(src), "sliceSet: source size does not match the slice");
+    AIXK_REQUIRE(start + (window.shape[dim] ? (window.shape[dim] - 1) * step : 0) < dst->shape[dim] || n == 0,
+                 "sliceSet: slice exceeds the destination");
+    return copy_views(ctx, src, &window, n);
+}
+
+int32_t aixk_tri(aixk_ctx* ctx, int upper, const aixhip_tensor* src, const aixhip_tensor* dst, int64_t diagonal)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "tril/triu: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "tril/triu: element types differ");      // aixDeviceMetal.cpp:1160-1161
+    AIXK_REQUIRE(src->rank >= 2, "tril/triu: rank must be at least 2");
+    const uint64_t n = dst->size;                    // aixDeviceCPU.cpp:576
+    if (n == 0) return AIXK_OK;
+    AIXK_REQUIRE(n == numel(src) && n == numel(dst), "tril/triu: sizes differ");
+    Space<1> ssp, dsp;
+    if (!collapse1(src, &ssp) || !collapse1(dst, &dsp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const uint64_t rows = src->shape[src->rank - 2], cols = src->shape[src->rank - 1];
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(dst) < (1ull << 31);
+    return by_size(src->dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
+        if (small) hipLaunchKernelGGL((tri_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n, (u64)rows, (u64)cols, (i64)diagonal, upper);
+        else hipLaunchKernelGGL((tri_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n, (u64)rows, (u64)cols, (i64)diagonal, upper);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+int32_t aixk_index_select(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                          const aixhip_tensor* indices, uint64_t dim)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst) && valid_tensor(indices), "indexSelect: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "indexSelect: element types differ");
+    AIXK_REQUIRE(indices->dtype == AIXK_I32, "indexSelect: indices must be int32");
+    AIXK_REQUIRE((src->rank == 0 && dim == 0) || (int)dim < src->rank, "indexSelect: dim out of range");
+    const uint64_t n = dst->size;                    // aixDeviceCPU.cpp:516
+    if (n == 0) return AIXK_OK;
+    uint64_t inner = 1;
+    for (int d = (int)dim + 1; d < src->rank; ++d) inner *= src->shape[d];
+    const uint64_t span = src->rank ? src->shape[dim] * inner : 0, ni = indices->size;
+    AIXK_REQUIRE(ni > 0, "indexSelect: empty indices");
+    Space<1> ssp, isp;
+    if (!collapse1(src, &ssp) || !collapse1(indices, &isp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && numel(src) < (1ull << 31);
+    return by_size(src->dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
+        if (small) hipLaunchKernelGGL((index_select_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, (const i32*)indices->data, ssp, isp, (u64)n, (u64)inner, (u64)ni, (u64)span);
+        else hipLaunchKernelGGL((index_select_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, (const i32*)indices->data, ssp, isp, (u64)n, (u64)inner, (u64)ni, (u64)span);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+int32_t aixk_index_add(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                       const aixhip_tensor* indices, uint64_t dim)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst) && valid_tensor(indices), "indexAdd: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "indexAdd: element types differ");
+    AIXK_REQUIRE(indices->dtype == AIXK_I32, "indexAdd: indices must be int32");
+    AIXK_REQUIRE((dst->rank == 0 && dim == 0) || (int)dim < dst->rank, "indexAdd: dim out of range");
+    const uint64_t n = src->size;                    // aixDeviceCPU.cpp:550
+    if (n == 0) return AIXK_OK;
+    uint64_t inner = 1;
+    for (int d = (int)dim + 1; d < dst->rank; ++d) inner *= dst->shape[d];
+    const uint64_t span = dst->rank ? dst->shape[dim] * inner : 0, ni = indices->size;
+    AIXK_REQUIRE(ni > 0, "indexAdd: empty indices");
+    Space<1> ssp, isp;
+    if (!collapse1(src, &ssp) || !collapse1(indices, &isp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31);
+    return by_dtype(src->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
+        if (small) hipLaunchKernelGGL((index_add_k<T, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const T*)src->data, (T*)dst->data, (const i32*)indices->data, ssp, isp, (u64)n, (u64)inner, (u64)ni, (u64)span);
+        else hipLaunchKernelGGL((index_add_k<T, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const T*)src->data, (T*)dst->data, (const i32*)indices->data, ssp, isp, (u64)n, (u64)inner, (u64)ni, (u64)span);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+} // extern "C"

@@ -1,0 +1,123 @@
+// matmul.hip -- out[m,n] = a[m,k] . b[k,n] for arbitrary 2-D operand views
+// (aixDeviceCPU.cpp:362-389).
+//
+// Two families:
+//   * f32 / f16 / bf16: MFMA kernels with f32 accumulation (matmul_mfma.hip);
+//   * f64 and the integer types: the LDS-tiled kernel in this file with an accumulator of the
+//     element type (integers wrap as on the CPU); also the fallback for operand layouts the MFMA
+//     kernels do not take.
+// The result is written row-major from out->data.
+
+#include "common.hpp"
+
+using namespace aixd;
+using namespace aixk;
+
+namespace aixk {
+// Implemented in matmul_mfma.hip.  Returns AIXK_OK if it launched, -1 if the shape/layout is not
+// one it handles (caller falls back), or an error status.
+int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+} // namespace aixk
+
+namespace {
+
+template <class T> struct mm_acc { typedef typename traits<T>::W type; };
+template <> struct mm_acc<i64> { typedef u64 type; };
+template <> struct mm_acc<i32> { typedef u32 type; };
+template <> struct mm_acc<i16> { typedef u32 type; };
+template <> struct mm_acc<i8>  { typedef u32 type; };
+template <> struct mm_acc<u8>  { typedef u32 type; };
+
+template <class T> __device__ __forceinline__ typename mm_acc<T>::type mm_up(T v) { return (typename mm_acc<T>::type)up(v); }
+template <class T> __device__ __forceinline__ T mm_down(typename mm_acc<T>::type v)
+{
+    if constexpr (traits<T>::is_int) return (T)v; else return down<T>(v);
+}
+
+constexpr int TM = 64, TN = 64, TK = 16;
+
+struct MatView { u64 off, s0, s1; };
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void matmul_tiled_k(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out,
+                                                         MatView va, MatView vb, u64 M, u64 N, u64 K)
+{
+    typedef typename mm_acc<T>::type A;
+    __shared__ A As[TK][TM + 4];
+    __shared__ A Bs[TK][TN + 4];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;          // 16 x 16 lanes, 4 x 4 outputs each
+    const u64 m0 = (u64)blockIdx.y * TM, n0 = (u64)blockIdx.x * TN;
+    A acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = (A)0;
+
+    for (u64 k0 = 0; k0 < K; k0 += TK) {
+        // A tile: TM x TK, B tile: TK x TN; 1024 elements each, 4 per lane
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int e = threadIdx.x + r * kBlock;
+            const int ak = e & (TK - 1), am = e >> 4;                 // k fastest for A
+            const u64 gm = m0 + am, gk = k0 + ak;
+            As[ak][am] = (gm < M && gk < K) ? mm_up(a[va.off + gm * va.s0 + gk * va.s1]) : (A)0;
+            const int bn = e & (TN - 1), bk = e >> 6;                 // n fastest for B
+            const u64 gn = n0 + bn, gk2 = k0 + bk;
+            Bs[bk][bn] = (gn < N && gk2 < K) ? mm_up(b[vb.off + gk2 * vb.s0 + gn * vb.s1]) : (A)0;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TK; ++kk) {
+            A ra[4], rb[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) ra[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) rb[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += ra[i] * rb[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const u64 gm = m0 + ty * 4 + i;
+        if (gm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const u64 gn = n0 + tx * 4 + j;
+            if (gn < N) out[gm * N + gn] = mm_down<T>(acc[i][j]);
+        }
+    }
+}
+
+} // namespace
+
+extern "C" int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(a) && valid_tensor(b) && valid_tensor(out), "matmul: bad operand descriptor");
+    AIXK_REQUIRE(a->rank == 2 && b->rank == 2, "matmul: operands must be 2-D");            // aixCore.hpp:946-955
+    AIXK_REQUIRE(a->shape[1] == b->shape[0], "matmul: inner dimensions differ");
+    AIXK_REQUIRE(a->dtype == out->dtype && b->dtype == out->dtype, "matmul: operands must have the result's element type");
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    if (M == 0 || N == 0) return AIXK_OK;
+    if (K == 0) return aixk_zero(ctx, out->data, M * N * aixk_dtype_size(out->dtype));
+    AIXK_REQUIRE(out->data != nullptr, "matmul: null result");
+
+    if (out->dtype == AIXK_F32 || out->dtype == AIXK_F16 || out->dtype == AIXK_BF16) {
+        const int rc = matmul_mfma(ctx, a, b, out);
+        if (rc != -1) return rc;
+    }
+    const uint64_t gx = (N + TN - 1) / TN, gy = (M + TM - 1) / TM;
+    AIXK_REQUIRE(gx < (1ull << 31) && gy < 65536, "matmul: shape too large for the generic kernel");
+    const MatView va{a->offset, a->strides[0], a->strides[1]}, vb{b->offset, b->strides[0], b->strides[1]};
+    return by_dtype(out->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        hipLaunchKernelGGL((matmul_tiled_k<T>), dim3((unsigned)gx, (unsigned)gy), dim3(kBlock), 0, ctx->stream,
+                           (const T*)a->data, (const T*)b->data, (T*)out->data, va, vb, (u64)M, (u64)N, (u64)K);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}

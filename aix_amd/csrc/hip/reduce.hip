@@ -1,0 +1,584 @@
+// reduce.hip -- sum / max / argmax over a whole tensor and over subsets of dims
+// (reduceTo, maxTo, argmaxTo, argmaxIndicesTo) for all nine element types.
+//
+// HBM-bound streaming reductions.  Per lane: 16-byte loads, accumulation in registers in a wide
+// type (f32 for f16/bf16, same-width wrap-around for integers, f32/f64 for themselves); per
+// wavefront: a 64-lane shuffle tree; per workgroup: LDS combine of the 4 waves; across
+// workgroups: partials in scratch, combined in a fixed order (results are run-to-run
+// deterministic).
+//
+// Semantics kept from the reference CPU device:
+//   * reduceTo / maxTo accumulate INTO dst (aixDeviceCPU.cpp:449-452, 461-465);
+//   * argmax picks the first maximum in flat logical order; a NaN is never picked unless it is
+//     the first element of its slot (strict '>' scan, aixDeviceCPU.cpp:263-272, 286-295);
+//   * argmaxTo stores (flat / src.strides[dim]) % src.shape[dim] with the source's PHYSICAL
+//     stride (aixDeviceCPU.cpp:293);
+//   * max keeps a NaN only if it is the first element / already in dst (std::max, :250-254).
+// The destination slot of a source element is the reference's right-aligned shape walk
+// (aixDeviceCPU.cpp:627-649), expressed as per-dim weights computed on the host.
+
+#include "common.hpp"
+
+#include <algorithm>
+
+using namespace aixd;
+using namespace aixk;
+
+namespace {
+
+constexpr int kWave = 64;
+constexpr int kWaves = kBlock / kWave;
+
+// ---- accumulators ------------------------------------------------------------------------------
+template <class T> struct sum_acc { typedef typename traits<T>::W type; };
+template <> struct sum_acc<i64> { typedef u64 type; };
+template <> struct sum_acc<i32> { typedef u32 type; };
+template <> struct sum_acc<i16> { typedef u32 type; };
+template <> struct sum_acc<i8>  { typedef u32 type; };
+template <> struct sum_acc<u8>  { typedef u32 type; };
+
+template <class W> __device__ __forceinline__ W neg_inf();
+template <> __device__ __forceinline__ double neg_inf<double>() { return -__builtin_huge_val(); }
+template <> __device__ __forceinline__ float neg_inf<float>() { return -__builtin_huge_valf(); }
+template <> __device__ __forceinline__ i64 neg_inf<i64>() { return lowest<i64>(); }
+template <> __device__ __forceinline__ i32 neg_inf<i32>() { return lowest<i32>(); }
+
+// flags: 1 = holds a non-NaN value, 2 = the slot's first element is NaN
+template <class W> struct ArgAcc { u64 idx; W v; u32 flags; };
+
+template <class T> struct SumOp {
+    typedef typename sum_acc<T>::type Acc;
+    typedef T Out;
+    static __device__ __forceinline__ Acc init() { return (Acc)0; }
+    static __device__ __forceinline__ Acc load(T x, u64, bool) { return (Acc)up(x); }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return a + b; }
+    static __device__ __forceinline__ Acc shfl(Acc v, int d) { return __shfl_down(v, d, kWave); }
+};
+template <class T> struct MaxOp {
+    typedef typename traits<T>::W Acc;
+    typedef T Out;
+    static __device__ __forceinline__ Acc init() { return neg_inf<Acc>(); }
+    static __device__ __forceinline__ Acc load(T x, u64, bool) { const Acc w = up(x); return w != w ? neg_inf<Acc>() : w; }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return b > a ? b : a; }
+    static __device__ __forceinline__ Acc shfl(Acc v, int d) { return __shfl_down(v, d, kWave); }
+};
+template <class T> struct ArgOp {
+    typedef typename traits<T>::W W;
+    typedef ArgAcc<W> Acc;
+    typedef i32 Out;
+    static __device__ __forceinline__ Acc init() { Acc a; a.v = neg_inf<W>(); a.idx = ~0ull; a.flags = 0; return a; }
+    static __device__ __forceinline__ Acc load(T x, u64 flat, bool first)
+    {
+        Acc a; a.v = up(x); a.idx = flat;
+        const bool nan = a.v != a.v;
+        a.flags = nan ? (first ? 2u : 0u) : 1u;
+        return a;
+    }
+    static __device__ __forceinline__ Acc combine(Acc a, Acc b)
+    {
+        const bool av = a.flags & 1u, bv = b.flags & 1u;
+        bool take_b;
+        if (av && bv) take_b = b.v > a.v || (b.v == a.v && b.idx < a.idx);
+        else if (av != bv) take_b = bv;
+        else take_b = b.idx < a.idx;
+        Acc r = take_b ? b : a;
+        r.flags = (r.flags & 1u) | ((a.flags | b.flags) & 2u);
+        return r;
+    }
+    static __device__ __forceinline__ Acc shfl(Acc v, int d)
+    {
+        Acc r;
+        r.idx = (u64)__shfl_down((unsigned long long)v.idx, d, kWave);
+        r.v = __shfl_down(v.v, d, kWave);
+        r.flags = __shfl_down(v.flags, d, kWave);
+        return r;
+    }
+};
+
+template <class Op> __device__ __forceinline__ typename Op::Acc wave_reduce(typename Op::Acc v)
+{
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) v = Op::combine(v, Op::shfl(v, d));
+    return v;                                  // lane 0 holds the result
+}
+
+// Result valid in thread 0.  `smem` holds kWaves accumulators.
+template <class Op> __device__ __forceinline__ typename Op::Acc block_reduce(typename Op::Acc v, typename Op::Acc* smem)
+{
+    v = wave_reduce<Op>(v);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    __syncthreads();                           // smem may still be in use from a previous round
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kWaves; ++w) v = Op::combine(v, smem[w]);
+    }
+    return v;
+}
+
+// ---- landing a finished accumulator --------------------------------------------------------------
+struct Finish {
+    int into;                // 1: combine with what dst holds (reduceTo/maxTo); 0: overwrite (sum/max)
+    int onehot;              // argmax: write 1 at the winner's flat index instead of an index per slot
+    u64 q_stride, q_extent;  // argmax along a dim: stored index = (flat / q_stride) % q_extent; q_stride 0: store flat
+};
+
+// `first` = value of the slot's first element (only read by max in overwrite mode);
+// `first_flat` = flat logical index of the slot's first element (only read by argmax).
+template <class T> __device__ __forceinline__ void land(SumOp<T>, const Finish& f, T* dst, u64 slot, typename SumOp<T>::Acc acc, T, u64)
+{
+    typedef typename SumOp<T>::Acc A;
+    if constexpr (traits<T>::is_int) dst[slot] = f.into ? (T)((A)dst[slot] + acc) : (T)acc;
+    else dst[slot] = f.into ? down<T>(up(dst[slot]) + acc) : down<T>(acc);
+}
+template <class T> __device__ __forceinline__ void land(MaxOp<T>, const Finish& f, T* dst, u64 slot, typename MaxOp<T>::Acc acc, T first, u64)
+{
+    if (f.into) { if (acc > up(dst[slot])) dst[slot] = down<T>(acc); }       // NaN in dst: '>' is false, it stays
+    else dst[slot] = e_isnan(first) ? first : down<T>(acc);                   // a leading NaN sticks
+}
+template <class T> __device__ __forceinline__ void land(ArgOp<T>, const Finish& f, i32* dst, u64 slot, typename ArgOp<T>::Acc acc, T, u64 first_flat)
+{
+    const u64 flat = (acc.flags & 2u) ? first_flat : acc.idx;
+    if (f.onehot) dst[flat] = 1;
+    else dst[slot] = f.q_stride ? (i32)((flat / f.q_stride) % f.q_extent) : (i32)flat;
+}
+
+// ---- whole tensor ----------------------------------------------------------------------------------
+template <class Op, class T, class IDX, bool FLAT>
+__global__ __launch_bounds__(kBlock) void reduce_all_k(const T* __restrict__ src, typename Op::Out* dst, Space<1> sp, u64 n,
+                                                       typename Op::Acc* partials, unsigned int* counter, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    __shared__ Acc smem[kWaves];
+    __shared__ int last;
+    Acc acc = Op::init();
+    if constexpr (FLAT) {
+        typedef typename vec16<T>::type V;
+        constexpr int VEC = vec16<T>::n;
+        constexpr int U = 4;
+        const T* base = src + sp.offset[0];
+        const V* B = (const V*)base;
+        const u64 nvec = n / VEC;
+        const u64 tile = (u64)kBlock * U;
+        for (u64 v0 = (u64)blockIdx.x * tile; v0 < nvec; v0 += (u64)gridDim.x * tile) {
+            V r[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) { const u64 v = v0 + (u64)k * kBlock + threadIdx.x; if (v < nvec) r[k] = B[v]; }
+#pragma unroll
+            for (int k = 0; k < U; ++k) {
+                const u64 v = v0 + (u64)k * kBlock + threadIdx.x;
+                if (v < nvec) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) { const u64 i = v * VEC + e; acc = Op::combine(acc, Op::load(r[k].v[e], i, i == 0)); }
+                }
+            }
+        }
+        const u64 done = nvec * VEC;
+        if (blockIdx.x == 0 && done + threadIdx.x < n) { const u64 i = done + threadIdx.x; acc = Op::combine(acc, Op::load(base[i], i, i == 0)); }
+    } else {
+        for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock)
+            acc = Op::combine(acc, Op::load(src[locate<1, IDX>(sp, 0, (IDX)i)], i, i == 0));
+    }
+    acc = block_reduce<Op>(acc, smem);
+    if (threadIdx.x == 0) {
+        partials[blockIdx.x] = acc;
+        __threadfence();                                     // publish the partial before taking a ticket
+        last = atomicAdd(counter, 1u) == gridDim.x - 1;
+    }
+    __syncthreads();
+    if (!last) return;
+    __threadfence();                                         // see every other workgroup's partial
+    Acc a = Op::init();
+    for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) a = Op::combine(a, partials[i]);
+    a = block_reduce<Op>(a, smem);
+    if (threadIdx.x == 0) {
+        *counter = 0;                                        // ready for the next reduction on this stream
+        land(Op{}, fin, dst, 0, a, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
+    }
+}
+
+// ---- per-slot plans ------------------------------------------------------------------------------
+// Kept dims address the destination slot, reduced dims are folded away.  All extents/strides are
+// those of the jointly collapsed (src strides, dst weights) space; `flat` strides are the
+// row-major strides of that space, which preserve the flat logical index of the original shape.
+struct RedPlan {
+    int nk, nr;
+    u64 k_ext[kMaxDims], k_src[kMaxDims], k_dst[kMaxDims], k_flat[kMaxDims];
+    u64 r_ext[kMaxDims], r_src[kMaxDims], r_flat[kMaxDims];
+    u64 src_off, slots, red;
+};
+
+struct SlotPos { u64 src, dst, flat; };
+
+__device__ __forceinline__ SlotPos slot_pos(const RedPlan& p, u64 slot, int ndims)
+{
+    SlotPos s; s.src = p.src_off; s.dst = 0; s.flat = 0;
+    for (int d = ndims - 1; d >= 0; --d) {
+        const u64 q = slot / p.k_ext[d], c = slot - q * p.k_ext[d];
+        s.src += c * p.k_src[d]; s.dst += c * p.k_dst[d]; s.flat += c * p.k_flat[d];
+        slot = q;
+    }
+    return s;
+}
+
+// inner: exactly one reduced dim, unit source stride.  One group (wave or workgroup) per slot.
+template <class Op, class T, int GROUP, bool VECT>
+__global__ __launch_bounds__(kBlock) void reduce_inner_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    constexpr int per_block = kBlock / GROUP;
+    __shared__ Acc smem[kWaves];
+    const int g = threadIdx.x / GROUP, l = threadIdx.x % GROUP;
+    const u64 L = p.r_ext[0];
+    for (u64 slot0 = (u64)blockIdx.x * per_block; slot0 < p.slots; slot0 += (u64)gridDim.x * per_block) {
+        const u64 slot = slot0 + g;
+        const bool live = slot < p.slots;
+        Acc acc = Op::init();
+        SlotPos s = slot_pos(p, live ? slot : 0, p.nk);
+        if (live) {
+            const T* row = src + s.src;
+            if constexpr (VECT) {
+                typedef typename vec16<T>::type V;
+                constexpr int VEC = vec16<T>::n;
+                constexpr int U = 4;
+                const V* R = (const V*)row;
+                const u64 nvec = L / VEC;
+                for (u64 v0 = 0; v0 < nvec; v0 += (u64)GROUP * U) {
+                    V r[U];
+#pragma unroll
+                    for (int k = 0; k < U; ++k) { const u64 v = v0 + (u64)k * GROUP + l; if (v < nvec) r[k] = R[v]; }
+#pragma unroll
+                    for (int k = 0; k < U; ++k) {
+                        const u64 v = v0 + (u64)k * GROUP + l;
+                        if (v < nvec) {
+#pragma unroll
+                            for (int e = 0; e < VEC; ++e) { const u64 j = v * VEC + e; acc = Op::combine(acc, Op::load(r[k].v[e], s.flat + j * p.r_flat[0], j == 0)); }
+                        }
+                    }
+                }
+            } else {
+                for (u64 j = l; j < L; j += GROUP) acc = Op::combine(acc, Op::load(row[j], s.flat + j * p.r_flat[0], j == 0));
+            }
+        }
+        if constexpr (GROUP == kBlock) acc = block_reduce<Op>(acc, smem);
+        else acc = wave_reduce<Op>(acc);
+        if (live && l == 0) land(Op{}, fin, dst, s.dst, acc, src[s.src], s.flat);
+    }
+}
+
+// outer: one reduced dim R, innermost kept dim C with unit source stride and unit dst weight,
+// optional leading kept dims (blockIdx.z).  Lanes own VEC neighbouring columns; the 4 waves of a
+// workgroup take interleaved rows of the workgroup's row chunk (blockIdx.y).
+template <class Op, class T, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p,
+                                                         u64 rows_per_chunk, typename Op::Acc* partials, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    typedef vec<T, VEC> V;
+    __shared__ Acc sm[kWaves][kWave * VEC];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 c0 = ((u64)blockIdx.x * kWave + lane) * VEC;
+    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const u64 r_begin = (u64)blockIdx.y * rows_per_chunk;
+    const u64 r_end = r_begin + rows_per_chunk < R ? r_begin + rows_per_chunk : R;
+    Acc acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = Op::init();
+    if (c0 < C) {
+        const T* col = src + s.src + c0;
+        constexpr int U = 4;
+        for (u64 r0 = r_begin + wave; r0 < r_end; r0 += (u64)kWaves * U) {
+            V x[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) { const u64 r = r0 + (u64)k * kWaves; if (r < r_end) x[k] = *(const V*)(col + r * p.r_src[0]); }
+#pragma unroll
+            for (int k = 0; k < U; ++k) {
+                const u64 r = r0 + (u64)k * kWaves;
+                if (r < r_end) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e)
+                        acc[e] = Op::combine(acc[e], Op::load(x[k].v[e], s.flat + r * p.r_flat[0] + (c0 + e) * p.k_flat[p.nk - 1], r == 0));
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) sm[wave][lane * VEC + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && c0 < C) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            Acc a = sm[0][lane * VEC + e];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) a = Op::combine(a, sm[w][lane * VEC + e]);
+            const u64 c = c0 + e;
+            if (partials) partials[((u64)blockIdx.z * gridDim.y + blockIdx.y) * C + c] = a;
+            else land(Op{}, fin, dst, s.dst + c, a, src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+        }
+    }
+}
+
+// second stage of `outer` when rows were split over several workgroups
+template <class Op, class T>
+__global__ __launch_bounds__(kBlock) void reduce_outer_finish_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p,
+                                                                unsigned chunks, const typename Op::Acc* __restrict__ partials, Finish fin)
+{
+    const u64 C = p.k_ext[p.nk - 1];
+    for (u64 slot = (u64)blockIdx.x * kBlock + threadIdx.x; slot < p.slots; slot += (u64)gridDim.x * kBlock) {
+        const u64 o = slot / C, c = slot - o * C;
+        typename Op::Acc a = Op::init();
+        for (unsigned k = 0; k < chunks; ++k) a = Op::combine(a, partials[(o * chunks + k) * C + c]);
+        const SlotPos s = slot_pos(p, o, p.nk - 1);
+        land(Op{}, fin, dst, s.dst + c, a, src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+    }
+}
+
+// generic: any mix of kept / reduced dims.  group = 1 lane per slot, or a whole workgroup per slot.
+template <class Op, class T>
+__global__ __launch_bounds__(kBlock) void reduce_generic_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p, int block_per_slot, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    __shared__ Acc smem[kWaves];
+    const u64 groups = block_per_slot ? gridDim.x : (u64)gridDim.x * kBlock;
+    const u64 gid = block_per_slot ? blockIdx.x : (u64)blockIdx.x * kBlock + threadIdx.x;
+    const u64 l = block_per_slot ? threadIdx.x : 0, step = block_per_slot ? kBlock : 1;
+    const u64 rounds = (p.slots + groups - 1) / groups;      // same trip count for every lane of a workgroup
+    for (u64 it = 0; it < rounds; ++it) {
+        const u64 slot = it * groups + gid;
+        const bool live = slot < p.slots;
+        const SlotPos s = slot_pos(p, live ? slot : 0, p.nk);
+        Acc acc = Op::init();
+        if (live) {
+            for (u64 j = l; j < p.red; j += step) {
+                u64 rest = j, pos = s.src, flat = s.flat;
+                for (int d = p.nr - 1; d >= 0; --d) {
+                    const u64 q = rest / p.r_ext[d], c = rest - q * p.r_ext[d];
+                    pos += c * p.r_src[d]; flat += c * p.r_flat[d];
+                    rest = q;
+                }
+                acc = Op::combine(acc, Op::load(src[pos], flat, j == 0));
+            }
+        }
+        if (block_per_slot) acc = block_reduce<Op>(acc, smem);
+        if (live && l == 0) land(Op{}, fin, dst, s.dst, acc, src[s.src], s.flat);
+    }
+}
+
+// ---- host side -------------------------------------------------------------------------------------
+// Per source dim, the multiplier into the flat destination index (0 = reduced away); the walk of
+// aixDeviceCPU.cpp:627-649.
+void dst_weights(const uint64_t* dshape, int drank, const uint64_t* sshape, int srank, uint64_t* weight)
+{
+    int j = drank - 1;
+    uint64_t run = 1;
+    for (int i = srank - 1; i >= 0; --i) {
+        weight[i] = 0;
+        if (j >= 0 && dshape[j] == sshape[i]) { weight[i] = run; run *= dshape[j]; --j; }
+        else if (j >= 0 && dshape[j] == 1) { --j; }
+    }
+}
+
+bool make_plan(const aixhip_tensor* src, const uint64_t* weight, RedPlan* p)
+{
+    const uint64_t* strides[2] = {src->strides, weight};
+    const uint64_t offsets[2] = {src->offset, 0};
+    Space<2> sp;
+    if (!collapse<2>(src->rank, src->shape, strides, offsets, &sp)) return false;
+    uint64_t flat[kMaxDims];
+    row_major_strides(sp.rank, sp.shape, flat);
+    std::memset(p, 0, sizeof(*p));
+    p->src_off = sp.offset[0];
+    p->slots = 1; p->red = 1;
+    for (int d = 0; d < sp.rank; ++d) {
+        if (sp.stride[1][d] != 0) {
+            p->k_ext[p->nk] = sp.shape[d]; p->k_src[p->nk] = sp.stride[0][d]; p->k_dst[p->nk] = sp.stride[1][d]; p->k_flat[p->nk] = flat[d];
+            ++p->nk; p->slots *= sp.shape[d];
+        } else {
+            p->r_ext[p->nr] = sp.shape[d]; p->r_src[p->nr] = sp.stride[0][d]; p->r_flat[p->nr] = flat[d];
+            ++p->nr; p->red *= sp.shape[d];
+        }
+    }
+    for (int d = p->nk; d < kMaxDims; ++d) p->k_ext[d] = 1;
+    for (int d = p->nr; d < kMaxDims; ++d) p->r_ext[d] = 1;
+    return true;
+}
+
+template <class Op, class T>
+int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin);
+
+template <class Op, class T>
+int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, const RedPlan& p, const Finish& fin)
+{
+    typedef typename Op::Acc Acc;
+    constexpr int VEC16 = vec16<T>::n;
+    const T* ps = (const T*)src->data;
+    const unsigned cus = (unsigned)ctx->cus;
+    hipStream_t st = ctx->stream;
+    if (p.slots == 0 || p.red == 0) return AIXK_OK;
+
+    // nothing kept: the whole source folds into dst[0]
+    if (p.nk == 0) return run_all<Op, T>(ctx, src, dst, fin);
+
+    // inner: one reduced dim with unit source stride
+    if (p.nr == 1 && p.r_src[0] == 1 && p.red >= 32) {
+        bool vect = p.red % VEC16 == 0 && aligned16(ps + p.src_off);
+        for (int d = 0; d < p.nk; ++d) if (p.k_src[d] % VEC16) vect = false;
+        const bool big = p.red >= 2048;
+        const uint64_t per_block = big ? 1 : kWaves;
+        const unsigned grid = grid_for(p.slots, (unsigned)per_block, cus * 64u);
+        if (big) {
+            if (vect) hipLaunchKernelGGL((reduce_inner_k<Op, T, kBlock, true>), dim3(grid), dim3(kBlock), 0, st, ps, dst, p, fin);
+            else hipLaunchKernelGGL((reduce_inner_k<Op, T, kBlock, false>), dim3(grid), dim3(kBlock), 0, st, ps, dst, p, fin);
+        } else {
+            if (vect) hipLaunchKernelGGL((reduce_inner_k<Op, T, kWave, true>), dim3(grid), dim3(kBlock), 0, st, ps, dst, p, fin);
+            else hipLaunchKernelGGL((reduce_inner_k<Op, T, kWave, false>), dim3(grid), dim3(kBlock), 0, st, ps, dst, p, fin);
+        }
+        AIXK_HIP(hipGetLastError());
+        return AIXK_OK;
+    }
+    // outer: one reduced dim, innermost kept dim dense on both sides
+    if (p.nr == 1 && p.nk >= 1 && p.k_src[p.nk - 1] == 1 && p.k_dst[p.nk - 1] == 1 && p.k_flat[p.nk - 1] == 1 && p.red >= 8) {
+        const uint64_t C = p.k_ext[p.nk - 1], R = p.r_ext[0], O = p.slots / C;
+        constexpr int VEC = VEC16 < 4 ? VEC16 : 4;
+        bool vect = C % VEC == 0 && ((uintptr_t)(ps + p.src_off) % (sizeof(T) * VEC)) == 0 && p.r_src[0] % VEC == 0;
+        for (int d = 0; d + 1 < p.nk; ++d) if (p.k_src[d] % VEC) vect = false;
+        const int v = vect ? VEC : 1;
+        const uint64_t col_tiles = (C + (uint64_t)kWave * v - 1) / ((uint64_t)kWave * v);
+        if (O <= 65535 && col_tiles < (1ull << 31)) {
+            // split rows until the launch has enough workgroups to fill the chip
+            uint64_t chunks = 1;
+            const uint64_t want = (uint64_t)cus * 8;
+            if (col_tiles * O < want) chunks = std::min<uint64_t>({(want + col_tiles * O - 1) / (col_tiles * O), (R + 63) / 64, (uint64_t)65535});
+            if (chunks < 1) chunks = 1;
+            while (chunks > 1 && chunks * O * C * sizeof(Acc) > ctx->scratch_bytes) chunks /= 2;
+            const uint64_t rows_per_chunk = (R + chunks - 1) / chunks;
+            chunks = (R + rows_per_chunk - 1) / rows_per_chunk;
+            Acc* partials = chunks > 1 ? (Acc*)ctx->scratch : nullptr;
+            const dim3 grid((unsigned)col_tiles, (unsigned)chunks, (unsigned)O);
+            if (vect) hipLaunchKernelGGL((reduce_outer_k<Op, T, VEC>), grid, dim3(kBlock), 0, st, ps, dst, p, (u64)rows_per_chunk, partials, fin);
+            else hipLaunchKernelGGL((reduce_outer_k<Op, T, 1>), grid, dim3(kBlock), 0, st, ps, dst, p, (u64)rows_per_chunk, partials, fin);
+            AIXK_HIP(hipGetLastError());
+            if (chunks > 1) {
+                hipLaunchKernelGGL((reduce_outer_finish_k<Op, T>), dim3(grid_for(p.slots, kBlock, cus * 8u)), dim3(kBlock), 0, st,
+                                   ps, dst, p, (unsigned)chunks, (const Acc*)partials, fin);
+                AIXK_HIP(hipGetLastError());
+            }
+            return AIXK_OK;
+        }
+    }
+    // generic
+    const int block_per_slot = p.red >= 256 && p.slots < (uint64_t)cus * 64;
+    const unsigned grid = block_per_slot ? grid_for(p.slots, 1, cus * 16u) : grid_for(p.slots, kBlock, cus * 16u);
+    hipLaunchKernelGGL((reduce_generic_k<Op, T>), dim3(grid), dim3(kBlock), 0, st, ps, dst, p, block_per_slot, fin);
+    AIXK_HIP(hipGetLastError());
+    return AIXK_OK;
+}
+
+template <class Op, class T>
+int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin)
+{
+    typedef typename Op::Acc Acc;
+    const uint64_t n = a->size;
+    Space<1> sp;
+    if (!collapse1(a, &sp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const T* ps = (const T*)a->data;
+    const bool flat = (sp.rank == 0 || (sp.rank == 1 && sp.stride[0][0] == 1)) && aligned16(ps + sp.offset[0]);
+    const bool small = n < (1ull << 31) && view_extent(a) < (1ull << 31);
+    constexpr int VEC = vec16<T>::n;
+    unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 8, ctx->scratch_bytes / sizeof(Acc));
+    const unsigned grid = flat ? grid_for(n / VEC + 1, kBlock * 4, max_blocks) : grid_for(n, kBlock * 4, max_blocks);
+    Acc* partials = (Acc*)ctx->scratch;
+    if (flat) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
+    else if (small) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
+    else hipLaunchKernelGGL((reduce_all_k<Op, T, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
+    AIXK_HIP(hipGetLastError());
+    return AIXK_OK;
+}
+
+} // namespace
+
+extern "C" {
+
+int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(a) && valid_tensor(out), "reduce: bad operand descriptor");
+    AIXK_REQUIRE(out->data != nullptr, "reduce: null result");
+    if (a->size == 0 && kind == AIXK_SUM) return aixk_zero(ctx, out->data, aixk_dtype_size(out->dtype));
+    AIXK_REQUIRE(a->size > 0 && a->size == numel(a), "reduce: empty or inconsistent source");
+    Finish fin{0, 0, 0, 0};
+    if (kind == AIXK_SUM || kind == AIXK_MAX) {
+        AIXK_REQUIRE(a->dtype == out->dtype, "reduce: operand must have the result's element type");
+        return by_dtype(out->dtype, [&](auto tag) {
+            typedef decltype(tag) T;
+            if (kind == AIXK_SUM) return run_all<SumOp<T>, T>(ctx, a, (T*)out->data, fin);
+            return run_all<MaxOp<T>, T>(ctx, a, (T*)out->data, fin);
+        });
+    }
+    AIXK_REQUIRE(kind == AIXK_ARGMAX || kind == AIXK_ARGMAX_ONEHOT, "reduce: unknown kind %d", kind);
+    // aixDeviceCPU.cpp:1027-1030, 1050-1053
+    AIXK_REQUIRE(out->dtype == AIXK_I32, "argmax supports only int32 data type for its result.");
+    AIXK_REQUIRE(a->size < (1ull << 31), "argmax: index does not fit int32");
+    if (kind == AIXK_ARGMAX_ONEHOT) {
+        fin.onehot = 1;
+        AIXK_TRY(aixk_zero(ctx, out->data, a->size * sizeof(int32_t)));
+    }
+    return by_dtype(a->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        return run_all<ArgOp<T>, T>(ctx, a, (int32_t*)out->data, fin);
+    });
+}
+
+int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "reduceTo: bad operand descriptor");
+    AIXK_REQUIRE(kind == AIXK_SUM || kind == AIXK_MAX, "reduceTo: unknown kind %d", kind);
+    AIXK_REQUIRE(src->dtype == dst->dtype, "reduceTo: element types differ");          // aixDeviceMetal.cpp:787-790
+    if (src->size == 0) return AIXK_OK;
+    AIXK_REQUIRE(src->size == numel(src), "reduceTo: inconsistent source");
+    uint64_t weight[AIXK_MAX_RANK];
+    dst_weights(dst->shape, dst->rank, src->shape, src->rank, weight);
+    RedPlan plan;
+    if (!make_plan(src, weight, &plan)) return fail(AIXK_EINVAL, "reduceTo: view does not collapse to %d dims", kMaxDims);
+    const Finish fin{1, 0, 0, 0};
+    return by_dtype(src->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        if (kind == AIXK_SUM) return run_plan<SumOp<T>, T>(ctx, src, (T*)dst->data, plan, fin);
+        return run_plan<MaxOp<T>, T>(ctx, src, (T*)dst->data, plan, fin);
+    });
+}
+
+int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t dim)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "argmaxTo: bad operand descriptor");
+    // aixDeviceCPU.cpp:1191-1194, 1214-1217
+    AIXK_REQUIRE(dst->dtype == AIXK_I32, "argmaxTo supports only int32 data type for its result.");
+    AIXK_REQUIRE((int)dim < src->rank, "argmaxTo: dim out of range");
+    if (src->size == 0) return AIXK_OK;
+    AIXK_REQUIRE(src->size == numel(src) && src->size < (1ull << 31), "argmaxTo: inconsistent or too large source");
+    uint64_t weight[AIXK_MAX_RANK];
+    Finish fin{0, onehot ? 1 : 0, 0, 0};
+    if (onehot) {
+        AIXK_REQUIRE((int)dim < dst->rank, "argmaxIndicesTo: dim out of range");
+        uint64_t rshape[AIXK_MAX_RANK];
+        for (int d = 0; d < dst->rank; ++d) rshape[d] = d == (int)dim ? 1 : dst->shape[d];   // aixDeviceCPU.cpp:325-326
+        dst_weights(rshape, dst->rank, src->shape, src->rank, weight);
+    } else {
+        AIXK_REQUIRE(src->strides[dim] != 0, "argmaxTo: zero stride along the reduced dim");
+        dst_weights(dst->shape, dst->rank, src->shape, src->rank, weight);
+        fin.q_stride = src->strides[dim];
+        fin.q_extent = src->shape[dim];
+    }
+    RedPlan plan;
+    if (!make_plan(src, weight, &plan)) return fail(AIXK_EINVAL, "argmaxTo: view does not collapse to %d dims", kMaxDims);
+    return by_dtype(src->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        return run_plan<ArgOp<T>, T>(ctx, src, (int32_t*)dst->data, plan, fin);
+    });
+}
+
+} // extern "C"

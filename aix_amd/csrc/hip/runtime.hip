@@ -1,0 +1,312 @@
+// runtime.hip -- context, memory, ordering, timing and the hipRTC kernel cache.
+
+#include "common.hpp"
+
+#include <hip/hiprtc.h>
+
+#include <vector>
+
+namespace aixk {
+
+static thread_local char g_error[1024] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// The text of aix_device.h, embedded at build time (see the Makefile rule for prelude.inc).
+static const char kPrelude[] = {
+#include "prelude.inc"
+    , 0};
+
+namespace {
+__global__ void zero_k(uint4* __restrict__ p, uint64_t n16, unsigned char* __restrict__ tail, unsigned ntail)
+{
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) p[i] = z;
+    if (blockIdx.x == 0 && threadIdx.x < ntail) tail[threadIdx.x] = 0;
+}
+} // namespace
+
+} // namespace aixk
+
+using namespace aixk;
+
+extern "C" {
+
+const char* aixk_last_error(void) { return g_error; }
+
+size_t aixk_dtype_size(int dtype)
+{
+    static const size_t sz[AIXK_DTYPE_COUNT] = {8, 4, 2, 2, 8, 4, 2, 1, 1};
+    return (dtype >= 0 && dtype < AIXK_DTYPE_COUNT) ? sz[dtype] : 0;
+}
+
+int32_t aixk_create(int device_index, aixk_ctx** out)
+{
+    AIXK_REQUIRE(out != nullptr, "create: null out pointer");
+    int count = 0;
+    AIXK_HIP(hipGetDeviceCount(&count));
+    if (count <= 0) return fail(AIXK_EHIP, "no HIP device is visible to this process");
+    AIXK_REQUIRE(device_index >= 0 && device_index < count, "create: device index %d out of range (%d devices)", device_index, count);
+    AIXK_HIP(hipSetDevice(device_index));
+    aixk_ctx* ctx = new aixk_ctx();
+    ctx->device = device_index;
+    AIXK_HIP(hipGetDeviceProperties(&ctx->prop, device_index));
+    ctx->cus = ctx->prop.multiProcessorCount > 0 ? ctx->prop.multiProcessorCount : 256;
+    AIXK_HIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
+    ctx->scratch_bytes = 64u << 20;
+    AIXK_HIP(hipMalloc(&ctx->scratch, ctx->scratch_bytes));
+    AIXK_HIP(hipMalloc((void**)&ctx->counter, 256));
+    AIXK_HIP(hipMemset(ctx->counter, 0, 256));
+    *out = ctx;
+    return AIXK_OK;
+}
+
+int32_t aixk_destroy(aixk_ctx* ctx)
+{
+    if (!ctx) return AIXK_OK;
+    (void)hipSetDevice(ctx->device);
+    (void)hipStreamSynchronize(ctx->stream);
+    for (auto& kv : ctx->rtc) {
+        if (kv.second->m.module) (void)hipModuleUnload(kv.second->m.module);
+        delete kv.second;
+    }
+    (void)hipFree(ctx->scratch);
+    (void)hipFree(ctx->counter);
+    (void)hipStreamDestroy(ctx->stream);
+    delete ctx;
+    return AIXK_OK;
+}
+
+int32_t aixk_info(aixk_ctx* ctx, aixk_device_info* out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(out != nullptr, "info: null out pointer");
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "%s", ctx->prop.name);
+    std::snprintf(out->arch, sizeof(out->arch), "%s", ctx->prop.gcnArchName);
+    out->compute_units = ctx->prop.multiProcessorCount;
+    out->clock_khz = ctx->prop.clockRate;
+    out->large_bar = ctx->prop.isLargeBar;
+    out->wavefront = ctx->prop.warpSize;
+    out->total_mem = ctx->prop.totalGlobalMem;
+    out->lds_per_block = ctx->prop.sharedMemPerBlock;
+    return AIXK_OK;
+}
+
+int32_t aixk_alloc(aixk_ctx* ctx, size_t bytes, int kind, void** out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(out != nullptr, "alloc: null out pointer");
+    const size_t padded = ((bytes ? bytes : 1) + 255) & ~(size_t)255;   // tail lanes of 16-byte kernels stay inside
+    void* p = nullptr;
+    hipError_t e;
+    switch (kind) {
+        case 0: e = hipMalloc(&p, padded); break;
+        case 1:
+            e = hipMallocManaged(&p, padded, hipMemAttachGlobal);
+            if (e == hipSuccess) {
+                (void)hipMemAdvise(p, padded, hipMemAdviseSetPreferredLocation, ctx->device);
+                (void)hipMemAdvise(p, padded, hipMemAdviseSetCoarseGrain, ctx->device);
+                (void)hipMemPrefetchAsync(p, padded, ctx->device, ctx->stream);
+                (void)hipGetLastError();
+            }
+            break;
+        case 2: e = hipHostMalloc(&p, padded, hipHostMallocDefault); break;
+        default: return fail(AIXK_EINVAL, "alloc: unknown memory kind %d", kind);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(AIXK_ENOMEM, "alloc of %zu bytes (kind %d) failed: %s", padded, kind, hipGetErrorString(e));
+    }
+    *out = p;
+    return AIXK_OK;
+}
+
+int32_t aixk_free(aixk_ctx* ctx, void* ptr, int kind)
+{
+    AIXK_TRY(set_device(ctx));
+    if (!ptr) return AIXK_OK;
+    if (kind == 2) AIXK_HIP(hipHostFree(ptr));
+    else AIXK_HIP(hipFree(ptr));
+    return AIXK_OK;
+}
+
+int32_t aixk_copy_in(aixk_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes)
+{
+    AIXK_TRY(set_device(ctx));
+    if (bytes == 0) return AIXK_OK;
+    AIXK_REQUIRE(dst_dev && src_host, "copy_in: null pointer");
+    // pageable source: the runtime stages it before returning, so the caller may reuse it
+    AIXK_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    AIXK_HIP(hipStreamSynchronize(ctx->stream));
+    return AIXK_OK;
+}
+
+int32_t aixk_copy_out(aixk_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes)
+{
+    AIXK_TRY(set_device(ctx));
+    if (bytes == 0) return AIXK_OK;
+    AIXK_REQUIRE(dst_host && src_dev, "copy_out: null pointer");
+    AIXK_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
+    AIXK_HIP(hipStreamSynchronize(ctx->stream));
+    return AIXK_OK;
+}
+
+int32_t aixk_copy_dev(aixk_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes)
+{
+    AIXK_TRY(set_device(ctx));
+    if (bytes == 0) return AIXK_OK;
+    AIXK_REQUIRE(dst_dev && src_dev, "copy_dev: null pointer");
+    AIXK_HIP(hipMemcpyAsync(dst_dev, src_dev, bytes, hipMemcpyDeviceToDevice, ctx->stream));
+    return AIXK_OK;
+}
+
+int32_t aixk_zero(aixk_ctx* ctx, void* dst_dev, size_t bytes)
+{
+    AIXK_TRY(set_device(ctx));
+    if (bytes == 0) return AIXK_OK;
+    AIXK_REQUIRE(dst_dev != nullptr, "zero: null pointer");
+    // A kernel rather than hipMemsetAsync, so that callers may capture this stream in a graph.
+    unsigned char* p = (unsigned char*)dst_dev;
+    const size_t head = ((uintptr_t)p & 15u) ? 16 - ((uintptr_t)p & 15u) : 0;
+    if (head >= bytes) {
+        hipLaunchKernelGGL(zero_k, dim3(1), dim3(kBlock), 0, ctx->stream, (uint4*)nullptr, (uint64_t)0, p, (unsigned)bytes);
+    } else {
+        if (head) hipLaunchKernelGGL(zero_k, dim3(1), dim3(kBlock), 0, ctx->stream, (uint4*)nullptr, (uint64_t)0, p, (unsigned)head);
+        const size_t body = bytes - head, n16 = body / 16, ntail = body % 16;
+        hipLaunchKernelGGL(zero_k, dim3(grid_for(n16 + 1, kBlock, (unsigned)ctx->cus * 16u)), dim3(kBlock), 0, ctx->stream,
+                           (uint4*)(p + head), (uint64_t)n16, p + head + n16 * 16, (unsigned)ntail);
+    }
+    AIXK_HIP(hipGetLastError());
+    return AIXK_OK;
+}
+
+int32_t aixk_sync(aixk_ctx* ctx)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_HIP(hipStreamSynchronize(ctx->stream));
+    return AIXK_OK;
+}
+
+// ---- hipRTC -----------------------------------------------------------------------------------
+const char* aixk_rtc_prelude(void) { return kPrelude; }
+
+int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const char* entry, aixk_module** out, int32_t* was_cached)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(key && source && entry && out, "rtc_get: null argument");
+    auto it = ctx->rtc.find(key);
+    if (it != ctx->rtc.end()) {
+        ++ctx->rtc_hits;
+        *out = it->second;
+        if (was_cached) *was_cached = 1;
+        return AIXK_OK;
+    }
+    ++ctx->rtc_misses;
+    if (was_cached) *was_cached = 0;
+
+    hiprtcProgram prog;
+    const char* header_names[] = {"aix_device.h"};
+    const char* header_texts[] = {kPrelude};
+    hiprtcResult r = hiprtcCreateProgram(&prog, source, "aix_fused.hip", 1, header_texts, header_names);
+    if (r != HIPRTC_SUCCESS) return fail(AIXK_EHIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+    std::string arch = std::string("--offload-arch=") + (ctx->prop.gcnArchName[0] ? ctx->prop.gcnArchName : "gfx950");
+    // IEEE arithmetic: no contraction (a*b+c stays two roundings), no fast-math, correctly rounded
+    // division and square root, no packed-f32 instruction selection.
+    const char* opts[] = {arch.c_str(), "-O3", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
+                          "-fhip-fp32-correctly-rounded-divide-sqrt",
+                          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+    r = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0;
+        hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, '\0');
+        if (n) hiprtcGetProgramLog(prog, &log[0]);
+        hiprtcDestroyProgram(&prog);
+        return fail(AIXK_EHIP, "hipRTC compile failed (%s): %.800s", hiprtcGetErrorString(r), log.c_str());
+    }
+    size_t code_size = 0;
+    hiprtcGetCodeSize(prog, &code_size);
+    std::vector<char> code(code_size);
+    hiprtcGetCode(prog, code.data());
+    hiprtcDestroyProgram(&prog);
+
+    aixk_module* mod = new aixk_module();
+    hipError_t e = hipModuleLoadData(&mod->m.module, code.data());
+    if (e == hipSuccess) e = hipModuleGetFunction(&mod->m.fn, mod->m.module, entry);
+    if (e != hipSuccess) {
+        if (mod->m.module) (void)hipModuleUnload(mod->m.module);
+        delete mod;
+        return fail(AIXK_EHIP, "loading the compiled kernel '%s' failed: %s", entry, hipGetErrorString(e));
+    }
+    ctx->rtc.emplace(key, mod);
+    *out = mod;
+    return AIXK_OK;
+}
+
+int32_t aixk_rtc_launch(aixk_ctx* ctx, aixk_module* mod, uint32_t grid_x, uint32_t block_x, const void* args, size_t args_bytes)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(mod && mod->m.fn, "rtc_launch: null kernel");
+    AIXK_REQUIRE(grid_x > 0 && block_x > 0 && block_x <= 1024, "rtc_launch: bad launch shape %u x %u", grid_x, block_x);
+    AIXK_REQUIRE(args != nullptr || args_bytes == 0, "rtc_launch: null argument block");
+    size_t size = args_bytes;
+    void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    AIXK_HIP(hipModuleLaunchKernel(mod->m.fn, grid_x, 1, 1, block_x, 1, 1, 0, ctx->stream, nullptr, config));
+    return AIXK_OK;
+}
+
+int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses)
+{
+    AIXK_REQUIRE(ctx != nullptr, "null context");
+    if (hits) *hits = ctx->rtc_hits;
+    if (misses) *misses = ctx->rtc_misses;
+    return AIXK_OK;
+}
+
+// ---- timing -----------------------------------------------------------------------------------
+int32_t aixk_event_create(aixk_ctx* ctx, aixk_event** out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(out != nullptr, "event_create: null out pointer");
+    aixk_event* ev = new aixk_event();
+    hipError_t e = hipEventCreate(&ev->ev);
+    if (e != hipSuccess) { delete ev; return fail(AIXK_EHIP, "hipEventCreate: %s", hipGetErrorString(e)); }
+    *out = ev;
+    return AIXK_OK;
+}
+
+int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(ev != nullptr, "event_record: null event");
+    AIXK_HIP(hipEventRecord(ev->ev, ctx->stream));
+    return AIXK_OK;
+}
+
+int32_t aixk_event_elapsed_ms(aixk_ctx* ctx, aixk_event* start, aixk_event* stop, float* ms)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(start && stop && ms, "event_elapsed: null argument");
+    AIXK_HIP(hipEventSynchronize(stop->ev));
+    AIXK_HIP(hipEventElapsedTime(ms, start->ev, stop->ev));
+    return AIXK_OK;
+}
+
+int32_t aixk_event_destroy(aixk_ctx* ctx, aixk_event* ev)
+{
+    if (!ev) return AIXK_OK;
+    if (ctx) (void)hipSetDevice(ctx->device);
+    (void)hipEventDestroy(ev->ev);
+    delete ev;
+    return AIXK_OK;
+}
+
+} // extern "C"

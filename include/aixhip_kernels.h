@@ -1,0 +1,157 @@
+/*
+ * aixhip_kernels.h -- the thin C ABI between host C++ and the gfx950 kernels.
+ *
+ * libaixhip_kernels.so (built by hipcc from aix_amd/csrc/hip) exports exactly these
+ * symbols.  It is the only code in the project that includes HIP headers.  The host-side
+ * device class (DeviceHIP, libaixhip.so) is plain C++20 and talks to the GPU only through
+ * this file: plain pointers, sizes and POD descriptors, no C++ types, no torch types.
+ *
+ * Every launcher is EAGER and ASYNCHRONOUS: it validates its operands on the host, enqueues
+ * its kernels on the context's single in-order stream and returns.  Nothing blocks except
+ * aixk_sync, aixk_copy_out and aixk_event_elapsed_ms.  Status: 0 = ok, AIXK_EINVAL = contract
+ * violation (the reference throws std::invalid_argument there), AIXK_ENOMEM = allocation
+ * failure (std::runtime_error in the reference), AIXK_EHIP = a HIP call failed.
+ * aixk_last_error() returns the message for the last non-zero status on the calling thread.
+ *
+ * Operand semantics follow the reference CPU device (Targets/AIXLib/aixDeviceCPU.cpp):
+ * results are written contiguously from result->data (result offset/strides ignored) unless
+ * stated otherwise; inputs are arbitrary views (offset + strides, stride 0 = broadcast).
+ * All tensor memory must be device memory obtained from aixk_alloc on the same context.
+ */
+#ifndef AIXHIP_KERNELS_H
+#define AIXHIP_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AIXK_MAX_RANK 16
+
+#define AIXK_OK      0
+#define AIXK_EINVAL  1
+#define AIXK_ENOMEM  2
+#define AIXK_EHIP    3
+
+/* Element types, numbered as aix::DataType (Targets/AIXLib/aixCore.hpp:44-55). */
+enum aixk_dtype {
+    AIXK_F64 = 0, AIXK_F32 = 1, AIXK_F16 = 2, AIXK_BF16 = 3,
+    AIXK_I64 = 4, AIXK_I32 = 5, AIXK_I16 = 6, AIXK_I8 = 7, AIXK_U8 = 8,
+    AIXK_DTYPE_COUNT = 9
+};
+
+/* POD image of aix::DeviceTensorParams (Targets/AIXLib/aixCore.hpp:189-198).
+ * offset / size / shape / strides count elements. */
+typedef struct aixhip_tensor {
+    void*    data;
+    int32_t  dtype;
+    int32_t  rank;
+    uint64_t offset;
+    uint64_t size;
+    uint64_t shape[AIXK_MAX_RANK];
+    uint64_t strides[AIXK_MAX_RANK];
+} aixhip_tensor;
+
+typedef struct aixk_ctx aixk_ctx;        /* one GPU, one in-order stream, scratch, JIT cache */
+typedef struct aixk_module aixk_module;  /* a runtime-compiled fused kernel */
+typedef struct aixk_event aixk_event;
+
+typedef struct aixk_device_info {
+    char     name[128];
+    char     arch[64];
+    int32_t  compute_units;
+    int32_t  clock_khz;
+    int32_t  large_bar;          /* 1 if device memory is host-addressable */
+    int32_t  wavefront;
+    uint64_t total_mem;
+    uint64_t lds_per_block;
+} aixk_device_info;
+
+const char* aixk_last_error(void);
+size_t      aixk_dtype_size(int dtype);                 /* aix::Device::dataTypeSize, aixDeviceCPU.cpp:685-700 */
+
+/* ---- context, memory, ordering (aixDevice.hpp:40-42, 82-83) ------------- */
+int32_t aixk_create(int device_index, aixk_ctx** out);
+int32_t aixk_destroy(aixk_ctx* ctx);
+int32_t aixk_info(aixk_ctx* ctx, aixk_device_info* out);
+/* kind: 0 = device memory (hipMalloc), 1 = managed memory preferring the device,
+ *       2 = pinned host memory.  Sizes are padded to a multiple of 256 bytes. */
+int32_t aixk_alloc(aixk_ctx* ctx, size_t bytes, int kind, void** out);
+int32_t aixk_free(aixk_ctx* ctx, void* ptr, int kind);             /* caller has synchronised */
+int32_t aixk_copy_in(aixk_ctx* ctx, void* dst_dev, const void* src_host, size_t bytes);   /* stream-ordered; host buffer reusable on return */
+int32_t aixk_copy_out(aixk_ctx* ctx, void* dst_host, const void* src_dev, size_t bytes);  /* waits for the stream, then copies */
+int32_t aixk_copy_dev(aixk_ctx* ctx, void* dst_dev, const void* src_dev, size_t bytes);
+int32_t aixk_zero(aixk_ctx* ctx, void* dst_dev, size_t bytes);
+int32_t aixk_sync(aixk_ctx* ctx);                                  /* Device::synchronize, aixDevice.hpp:83 */
+
+/* ---- elementwise (aixDevice.hpp:44-48, 53-59) --------------------------- */
+enum aixk_binary_op { AIXK_ADD = 0, AIXK_SUB = 1, AIXK_MUL = 2, AIXK_DIV = 3, AIXK_POW = 4 };
+enum aixk_unary_op  { AIXK_NEG = 0, AIXK_SQRT = 1, AIXK_SIN = 2, AIXK_COS = 3, AIXK_TANH = 4, AIXK_LOG = 5, AIXK_EXP = 6 };
+/* out[i] = a[view(i)] op b[view(i)], i < out->size (pow: i < a->size); element type = out->dtype.
+ * Replaces Device::add/sub/mul/div/pow (aixDeviceCPU.cpp:28-82, 229-242). */
+int32_t aixk_binary(aixk_ctx* ctx, int op, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+/* out[i] = f(a[view(i)]), i < a->size.  Replaces Device::unary/sqrt/sin/cos/tanh/log/exp
+ * (aixDeviceCPU.cpp:84-94, 154-227). */
+int32_t aixk_unary(aixk_ctx* ctx, int op, const aixhip_tensor* a, const aixhip_tensor* out);
+/* Device::fill / fillMin (aixDeviceCPU.cpp:119-138): scalar is HOST memory of scalar_dtype. */
+int32_t aixk_fill(aixk_ctx* ctx, const void* scalar, int scalar_dtype, const aixhip_tensor* out);
+int32_t aixk_fill_min(aixk_ctx* ctx, const aixhip_tensor* out);
+/* Device::copy (aixDeviceCPU.cpp:407-423): flat converting copy of n elements, both device memory. */
+int32_t aixk_cast(aixk_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype, uint64_t n);
+
+/* ---- data movement (aixDevice.hpp:64, 68, 73-80) ------------------------ */
+int32_t aixk_contiguous(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst);      /* aixDeviceCPU.cpp:425-438 */
+int32_t aixk_transpose(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* out, uint64_t dim0, uint64_t dim1); /* :391-405 */
+/* dst is addressed through its offset and strides (the reference GPU device's behaviour). */
+int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                       uint64_t dim, uint64_t start, uint64_t end, uint64_t step);                /* :468-496 */
+int32_t aixk_tri(aixk_ctx* ctx, int upper, const aixhip_tensor* src, const aixhip_tensor* dst, int64_t diagonal); /* :566-622 */
+/* indices: int32, addressed through their own offset and strides. */
+int32_t aixk_index_select(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                          const aixhip_tensor* indices, uint64_t dim);                           /* :498-530 */
+int32_t aixk_index_add(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                       const aixhip_tensor* indices, uint64_t dim);                              /* :532-564 */
+
+/* ---- reductions (aixDevice.hpp:52, 60-62, 69-72) ------------------------ */
+enum aixk_reduce_kind { AIXK_SUM = 0, AIXK_MAX = 1, AIXK_ARGMAX = 2, AIXK_ARGMAX_ONEHOT = 3 };
+/* Whole-tensor reduction into a rank-0 result: Device::sum/max/argmax/argmaxIndices
+ * (aixDeviceCPU.cpp:140-152, 244-318).  ARGMAX kinds need an int32 result. */
+int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out);
+/* dst (op)= reduction of src over the dims dst lacks: Device::reduceTo / maxTo
+ * (aixDeviceCPU.cpp:440-466).  Accumulates INTO dst (caller pre-initialises). kind = SUM|MAX. */
+int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst);
+/* Device::argmaxTo / argmaxIndicesTo (aixDeviceCPU.cpp:275-298, 320-360). onehot=1 scatters ones
+ * into the pre-zeroed int32 dst of src's shape. */
+int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t dim);
+
+/* ---- matmul (aixDevice.hpp:63; aixDeviceCPU.cpp:362-389) ---------------- */
+/* out[m,n] = a[m,k] . b[k,n]; a, b arbitrary 2-D views; f32/f16/bf16 run on MFMA with f32
+ * accumulation, other types on a generic tiled kernel with an accumulator of the element type
+ * (f64 and integers). */
+int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+
+/* ---- runtime-compiled fused elementwise kernels ------------------------- */
+/* Compile `source` (HIP C++, one extern "C" __global__ named `entry`) for gfx950 with hipRTC or
+ * return the cached module for `key`.  *was_cached tells which.  Replaces the reference's
+ * runtime shader compile + pipeline cache (aixDeviceMetalKernelGen.cpp:712-770). */
+int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const char* entry,
+                     aixk_module** out, int32_t* was_cached);
+/* Launch with a packed kernel-argument block (aixDeviceMetalKernelGen.cpp:772-857). */
+int32_t aixk_rtc_launch(aixk_ctx* ctx, aixk_module* mod, uint32_t grid_x, uint32_t block_x,
+                        const void* args, size_t args_bytes);
+/* The device-side header every generated kernel is compiled against (types, conversions, math). */
+const char* aixk_rtc_prelude(void);
+int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);
+
+/* ---- timing on the context's stream ------------------------------------- */
+int32_t aixk_event_create(aixk_ctx* ctx, aixk_event** out);
+int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev);
+int32_t aixk_event_elapsed_ms(aixk_ctx* ctx, aixk_event* start, aixk_event* stop, float* ms); /* waits for stop */
+int32_t aixk_event_destroy(aixk_ctx* ctx, aixk_event* ev);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

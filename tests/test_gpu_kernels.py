@@ -1,0 +1,582 @@
+"""Parity of the gfx950 kernels (through the C ABI of libaixhip_kernels.so) against the CPU oracle
+on identical seeded inputs, following the reference's device-parity pattern
+(Targets/AIXTests/DeviceTests.cpp:199-233: same raw device call on the CPU device and on the
+device under test, then compare).
+
+Tolerances (stated per test):
+  * integers, indices, data movement, casts, fill: bit-exact;
+  * f64/f32/f16/bf16 add, sub, mul, div, negate, sqrt: bit-exact;
+  * f32 sin/cos/tanh/log/exp/pow: <= 2 ulp; f64: <= 4 ulp; f16/bf16: <= 1 ulp of the 16-bit type;
+  * float reductions and f32 matmul: |err| <= 1e-5 x sum|terms| against an exactly accumulated
+    oracle; f16/bf16 additionally allow the final rounding of the result (2^-10 / 2^-8 relative);
+  * f16/bf16 matmul: <= 2e-2 x sum|a||b|.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import aixtest as T
+import gpuharness as G
+from aix_amd import kernels as K
+from oracle import cpuref as O
+
+pytestmark = pytest.mark.gpu
+CPU = O.lib()
+NAMES = O.DTYPE_NAMES
+ids = lambda d: NAMES[d]  # noqa: E731
+
+SIZES = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 32, 33, 63, 64, 65, 127, 128, 129, 255, 256, 257,
+         511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049]      # as DeviceTests.cpp:30-31
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = G.Gpu()
+    yield g
+    g.close()
+    g.ctx.close()
+
+
+def okc(rc):
+    assert rc == 0, rc
+
+
+# ---- elementwise ----------------------------------------------------------------------------------
+def binary_rule(op, dtype):
+    if dtype in T.INT_DTYPES or op != O.POW:
+        return G.EXACT
+    return {O.F32: 2, O.F64: 4, O.F16: 1, O.BF16: 1}[dtype]
+
+
+def unary_rule(op, dtype):
+    if dtype in T.INT_DTYPES or op in (O.NEG, O.SQRT):
+        return G.EXACT
+    return {O.F32: 2, O.F64: 4, O.F16: 1, O.BF16: 1}[dtype]
+
+
+def check_binary(gpu, op, a, b, what):
+    dtype = a.dtype
+    want = T.empty(dtype, a.shape)
+    okc(CPU.binary(op, C.byref(a.desc()), C.byref(b.desc()), C.byref(want.desc())))
+    _, da = gpu.put(a)
+    _, db = gpu.put(b)
+    po, do = gpu.put(T.empty(dtype, a.shape))
+    G.run_gpu(gpu, "aixk_binary", op, G.ref(da), G.ref(db), G.ref(do))
+    got = gpu.fetch(po, want.storage)
+    G.compare(got, want.storage, dtype, binary_rule(op, dtype), what)
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+@pytest.mark.parametrize("op", [O.ADD, O.SUB, O.MUL, O.DIV, O.POW], ids=["add", "sub", "mul", "div", "pow"])
+def test_binary_views(gpu, op, dtype):
+    rng = np.random.default_rng(11000 + op * 16 + dtype)
+    kw = dict(int_span=5 if op == O.POW else 100) if dtype in T.INT_DTYPES else dict(lo=0.05, hi=3.0) if op == O.POW else {}
+    for trial in range(14):
+        shape = T.random_shape(rng, max_rank=5)
+        ka, kb = rng.choice(T.VIEW_KINDS, 2)
+        a = T.view_tensor(rng, dtype, shape, ka, **kw)
+        b = T.view_tensor(rng, dtype, shape, kb, **kw)
+        check_binary(gpu, op, a, b, f"binary op={op} {NAMES[dtype]} {shape} {ka}/{kb}")
+    gpu.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_binary_sizes_and_broadcast_rows(gpu, dtype):
+    """Flat sizes 1..2049 (vector body + tail) and the row / column / scalar broadcast forms the
+    front-end produces (bias add, Tensor op scalar)."""
+    rng = np.random.default_rng(12000 + dtype)
+    for n in SIZES:
+        a = T.contiguous_tensor(rng, dtype, [n])
+        b = T.contiguous_tensor(rng, dtype, [n])
+        check_binary(gpu, O.ADD, a, b, f"add {NAMES[dtype]} n={n}")
+        check_binary(gpu, O.MUL, a, b, f"mul {NAMES[dtype]} n={n}")
+    gpu.release()
+    for rows, cols in [(3, 8), (5, 64), (17, 1024), (64, 96), (7, 33), (130, 2048)]:
+        a = T.contiguous_tensor(rng, dtype, [rows, cols])
+        row = T.HostTensor(T.random_values(rng, cols, dtype), dtype, [rows, cols], [0, 1])
+        col = T.HostTensor(T.random_values(rng, rows, dtype), dtype, [rows, cols], [1, 0])
+        sc = T.HostTensor(T.random_values(rng, 1, dtype), dtype, [rows, cols], [0, 0])
+        for other, name in ((row, "row"), (col, "col"), (sc, "scalar")):
+            check_binary(gpu, O.ADD, a, other, f"add {NAMES[dtype]} [{rows},{cols}] + {name}")
+            check_binary(gpu, O.SUB, other, a, f"sub {NAMES[dtype]} {name} - [{rows},{cols}]")
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+@pytest.mark.parametrize("op", range(7), ids=["neg", "sqrt", "sin", "cos", "tanh", "log", "exp"])
+def test_unary(gpu, op, dtype):
+    rng = np.random.default_rng(13000 + op * 16 + dtype)
+    cases = []
+    for trial in range(8):
+        shape = T.random_shape(rng)
+        cases.append((shape, rng.choice(T.VIEW_KINDS)))
+    cases += [([n], "contig") for n in (1, 5, 64, 257, 2049, 40000)]
+    for shape, kind in cases:
+        lo, hi = (-4.0, 8.0)
+        if op in (O.SQRT, O.LOG):
+            lo, hi = (0.0, 30.0)
+        a = T.view_tensor(rng, dtype, shape, kind, lo=lo, hi=hi, int_span=12)
+        want = T.empty(dtype, shape)
+        okc(CPU.unary(op, C.byref(a.desc()), C.byref(want.desc())))
+        _, da = gpu.put(a)
+        po, do = gpu.put(T.empty(dtype, shape))
+        G.run_gpu(gpu, "aixk_unary", op, G.ref(da), G.ref(do))
+        got = gpu.fetch(po, want.storage)
+        G.compare(got, want.storage, dtype, unary_rule(op, dtype), f"unary op={op} {NAMES[dtype]} {shape} {kind}")
+    gpu.release()
+
+
+def test_unary_f32_special_values(gpu):
+    """Signed zeros, infinities, NaN, denormals and large arguments through every f32 function."""
+    vals = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, -1e-45, 1e-38, 3e-39, 88.7, 89.0, -87.0,
+                     -104.0, 1e10, -1e10, 0.5, 2.0, 3.1415927, 1e-4, 9.0, 16.0, 1e38, 3.4e38, 100.0, 710.0], dtype=np.float32)
+    a = T.HostTensor(vals, O.F32, [vals.size])
+    for op in range(7):
+        want = T.empty(O.F32, a.shape)
+        okc(CPU.unary(op, C.byref(a.desc()), C.byref(want.desc())))
+        _, da = gpu.put(a)
+        po, do = gpu.put(T.empty(O.F32, a.shape))
+        G.run_gpu(gpu, "aixk_unary", op, G.ref(da), G.ref(do))
+        got = gpu.fetch(po, want.storage)
+        G.compare(got, want.storage, O.F32, unary_rule(op, O.F32), f"special values op={op}")
+    gpu.release()
+
+
+def test_f32_transcendental_ulp_histogram(gpu):
+    """1M-point ulp histograms of each f32 function against the oracle; the bound is 2 ulp."""
+    rng = np.random.default_rng(14000)
+    n = 1 << 20
+    for op, lo, hi in ((O.SIN, -20, 20), (O.COS, -20, 20), (O.TANH, -10, 10), (O.EXP, -80, 80), (O.LOG, 1e-30, 1e30)):
+        if op == O.LOG:
+            x = np.exp(rng.uniform(np.log(lo), np.log(hi), n)).astype(np.float32)
+        else:
+            x = rng.uniform(lo, hi, n).astype(np.float32)
+        a = T.HostTensor(x, O.F32, [n])
+        want = T.empty(O.F32, [n])
+        okc(CPU.unary(op, C.byref(a.desc()), C.byref(want.desc())))
+        _, da = gpu.put(a)
+        po, do = gpu.put(T.empty(O.F32, [n]))
+        G.run_gpu(gpu, "aixk_unary", op, G.ref(da), G.ref(do))
+        got = gpu.fetch(po, want.storage)
+        worst, hist = O.ulp_hist_f32(got, want.storage)
+        print(f"ulp histogram op={op}: worst={worst} hist={hist[:6].tolist()}")
+        assert worst <= 2, (op, worst, hist)
+        gpu.release()
+
+
+# ---- fill / fillMin / cast ------------------------------------------------------------------------
+SPECIALS = [0.0, -0.0, 1.0, -1.0, 0.5, 255.0, 256.0, 300.0, -129.0, 32767.6, -32768.9, 65504.0, 65520.0,
+            1e9, -1e9, 3e9, 2147483647.0, 2147483648.0, -2147483649.0, 9.3e18, -9.3e18, 1e30, -1e30,
+            float("inf"), float("-inf"), float("nan"), 1e-8, 6e-8, 5.96e-8, 2.98e-8, 6.1e-5, 3.14]
+
+
+@pytest.mark.parametrize("src", T.ALL_DTYPES, ids=ids)
+def test_cast_and_fill(gpu, src):
+    rng = np.random.default_rng(15000 + src)
+    if src in T.FLOAT_DTYPES:
+        with np.errstate(over="ignore", invalid="ignore"):
+            vals = np.concatenate([np.array(SPECIALS), rng.uniform(-400, 400, 2100), rng.uniform(-1, 1, 64) * 1e6])
+            st = O.to_storage(vals, src)
+    else:
+        info = np.iinfo(O.NP_STORAGE[src])
+        st = np.concatenate([np.array([info.min, info.max, 0, 1, 2], dtype=O.NP_STORAGE[src]),
+                             rng.integers(info.min, info.max, 2100, endpoint=True).astype(O.NP_STORAGE[src])])
+    n = st.size
+    ps = gpu.raw(st.nbytes)
+    gpu.ctx.upload(ps, st)
+    for dst in T.ALL_DTYPES:
+        for count in (n, 1, 13):                                   # vector body + tails
+            want = np.zeros(count, dtype=O.NP_STORAGE[dst])
+            okc(CPU.copy(st.ctypes.data, src, want.ctypes.data, dst, count))
+            pd = gpu.raw(want.nbytes)
+            G.run_gpu(gpu, "aixk_cast", ps, src, pd, dst, count)
+            got = gpu.fetch(pd, want)
+            T.assert_same_bits_nan_ok(got, want, dst, f"cast {NAMES[src]}->{NAMES[dst]} n={count}")
+        # unaligned source and destination (offset by one element)
+        if n > 40:
+            want = np.zeros(33, dtype=O.NP_STORAGE[dst])
+            okc(CPU.copy(st[1:].ctypes.data, src, want.ctypes.data, dst, 33))
+            pd = gpu.raw(want.nbytes + 16)
+            G.run_gpu(gpu, "aixk_cast", ps + st.itemsize, src, pd + want.itemsize, dst, 33)
+            got = np.empty_like(want)
+            gpu.ctx.download(got, pd + want.itemsize)
+            T.assert_same_bits_nan_ok(got, want, dst, f"unaligned cast {NAMES[src]}->{NAMES[dst]}")
+        for k in list(range(0, 40)) + [n - 1]:
+            scalar = st[k:k + 1].copy()
+            for count in (1, 19, 300):
+                want = T.empty(dst, [count])
+                okc(CPU.fill(scalar.ctypes.data, src, C.byref(want.desc())))
+                po, do = gpu.put(T.empty(dst, [count]))
+                G.run_gpu(gpu, "aixk_fill", scalar.ctypes.data, src, G.ref(do))
+                got = gpu.fetch(po, want.storage)
+                T.assert_same_bits_nan_ok(got, want.storage, dst, f"fill {NAMES[src]}->{NAMES[dst]} {scalar} n={count}")
+        gpu.release()
+        ps = gpu.raw(st.nbytes)
+        gpu.ctx.upload(ps, st)
+    want = T.empty(src, [77])
+    okc(CPU.fill_min(C.byref(want.desc())))
+    po, do = gpu.put(T.empty(src, [77]))
+    G.run_gpu(gpu, "aixk_fill_min", G.ref(do))
+    T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"fillMin {NAMES[src]}")
+    gpu.release()
+
+
+# ---- data movement --------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_contiguous_and_transpose(gpu, dtype):
+    rng = np.random.default_rng(16000 + dtype)
+    cases = [(T.random_shape(rng, max_rank=5, max_extent=7), rng.choice(T.VIEW_KINDS)) for _ in range(12)]
+    # 2-D and batched transposes through the LDS-tiled kernel, incl. ragged edges
+    cases += [([n, m], "transposed") for n, m in [(1, 1), (1, 70), (63, 65), (64, 64), (129, 257), (300, 5), (5, 300), (513, 1025)]]
+    cases += [([3, 70, 130], "transposed"), ([96, 256], "sliced"), ([33, 48], "offset")]
+    for shape, kind in cases:
+        src = T.view_tensor(rng, dtype, shape, kind)
+        want = T.empty(dtype, shape)
+        okc(CPU.contiguous(C.byref(src.desc()), C.byref(want.desc())))
+        _, ds = gpu.put(src)
+        po, do = gpu.put(T.empty(dtype, shape))
+        G.run_gpu(gpu, "aixk_contiguous", G.ref(ds), G.ref(do))
+        T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"contiguous {NAMES[dtype]} {shape} {kind} strides={src.strides}")
+        gpu.release()
+    for trial in range(10):
+        shape = T.random_shape(rng, max_rank=4, max_extent=40, max_numel=60000)
+        rank = len(shape)
+        a = T.contiguous_tensor(rng, dtype, shape)
+        d0, d1 = (int(v) for v in rng.integers(0, rank, 2))
+        tshape = list(shape)
+        tshape[d0], tshape[d1] = tshape[d1], tshape[d0]
+        want = T.empty(dtype, tshape)
+        okc(CPU.transpose(C.byref(a.desc()), C.byref(want.desc()), d0, d1))
+        _, da = gpu.put(a)
+        po, do = gpu.put(T.empty(dtype, tshape))
+        G.run_gpu(gpu, "aixk_transpose", G.ref(da), G.ref(do), d0, d1)
+        T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"transpose {NAMES[dtype]} {shape} {d0},{d1}")
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_slice_set_tri_index_ops(gpu, dtype):
+    rng = np.random.default_rng(17000 + dtype)
+    for trial in range(12):
+        shape = T.random_shape(rng, max_rank=4, max_extent=9)
+        rank = len(shape)
+        kind = rng.choice(T.VIEW_KINDS)
+        src = T.view_tensor(rng, dtype, shape, kind)
+        _, dsrc = gpu.put(src)
+        # sliceSet into a strided, offset window (dst offset honoured as on the reference GPU device)
+        dim = int(rng.integers(0, rank))
+        step = int(rng.integers(1, 3))
+        start = int(rng.integers(0, 3))
+        big = list(shape)
+        big[dim] = start + (shape[dim] - 1) * step + 1 + int(rng.integers(0, 2))
+        end = min(big[dim], start + shape[dim] * step)
+        dst = T.view_tensor(rng, dtype, big, rng.choice(["contig", "transposed", "offset", "sliced"]))
+        want = dst.clone()
+        okc(CPU.slice_set(C.byref(src.desc()), C.byref(want.desc()), dim, start, end, step, 1))
+        pd, dd = gpu.put(dst)
+        G.run_gpu(gpu, "aixk_slice_set", G.ref(dsrc), G.ref(dd), dim, start, end, step)
+        T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, f"sliceSet {NAMES[dtype]} {shape}->{big} dim={dim}")
+        # tril / triu
+        if rank >= 2:
+            for upper in (0, 1):
+                diag = int(rng.integers(-3, 4))
+                dst = T.view_tensor(rng, dtype, shape, rng.choice(["contig", "transposed", "sliced", "offset"]))
+                want = dst.clone()
+                okc((CPU.triu if upper else CPU.tril)(C.byref(src.desc()), C.byref(want.desc()), diag))
+                pd, dd = gpu.put(dst)
+                G.run_gpu(gpu, "aixk_tri", upper, G.ref(dsrc), G.ref(dd), diag)
+                T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, f"tri upper={upper} {NAMES[dtype]} {shape} diag={diag}")
+        # indexSelect / indexAdd with strided int32 indices
+        ni = int(rng.integers(1, 7))
+        raw_idx = rng.integers(0, shape[dim], 2 * ni + 1).astype(np.int32)
+        idx = T.HostTensor(raw_idx, O.I32, [ni], [2], 1)
+        _, didx = gpu.put(idx)
+        sel = list(shape)
+        sel[dim] = ni
+        want = T.empty(dtype, sel)
+        okc(CPU.index_select(C.byref(src.desc()), C.byref(want.desc()), C.byref(idx.desc()), dim, 1))
+        po, do = gpu.put(T.empty(dtype, sel))
+        G.run_gpu(gpu, "aixk_index_select", G.ref(dsrc), G.ref(do), G.ref(didx), dim)
+        T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"indexSelect {NAMES[dtype]} {shape} dim={dim}")
+        # updates are small whole numbers so that sums are exact in every float type and the
+        # order in which duplicates are accumulated cannot matter
+        upd_vals = rng.integers(0 if dtype == O.U8 else -3, 4, O.numel(sel)).astype(np.float64)
+        upd = T.HostTensor(O.to_storage(upd_vals, dtype), dtype, sel)
+        acc = T.HostTensor(O.to_storage(rng.integers(0, 5, O.numel(shape)).astype(np.float64), dtype), dtype, shape)
+        want = acc.clone()
+        okc(CPU.index_add(C.byref(upd.desc()), C.byref(want.desc()), C.byref(idx.desc()), dim, 1))
+        _, dupd = gpu.put(upd)
+        pa, dacc = gpu.put(acc)
+        G.run_gpu(gpu, "aixk_index_add", G.ref(dupd), G.ref(dacc), G.ref(didx), dim)
+        T.assert_same_bits(gpu.fetch(pa, want.storage), want.storage, f"indexAdd {NAMES[dtype]} {shape} dim={dim}")
+        gpu.release()
+
+
+# ---- reductions -----------------------------------------------------------------------------------
+def float_sum_tolerance(dtype):
+    # accumulation error bound (relative to sum |x|) + one rounding of the result in its own type
+    return {O.F64: (1e-12, 0.0), O.F32: (1e-5, 0.0), O.F16: (1e-5, 2.0 ** -10), O.BF16: (1e-5, 2.0 ** -8)}[dtype]
+
+
+def check_sum_like(got_storage, dtype, exact, scale, what):
+    tol, final = float_sum_tolerance(dtype)
+    got = O.to_float64(got_storage, dtype)
+    exact = np.asarray(exact, dtype=np.float64)
+    scale = np.asarray(scale, dtype=np.float64)
+    G.assert_close_to_wide(got, exact, scale + (final / max(tol, 1e-300)) * np.abs(exact) + 1e-30, tol, what)
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_reduce_all(gpu, dtype):
+    rng = np.random.default_rng(18000 + dtype)
+    cases = [([n], "contig") for n in SIZES + [70001, 1 << 20]]
+    cases += [(T.random_shape(rng, max_rank=4, max_extent=12, max_numel=20000), rng.choice(T.VIEW_KINDS)) for _ in range(10)]
+    for shape, kind in cases:
+        a = T.view_tensor(rng, dtype, shape, kind, int_span=3)
+        _, da = gpu.put(a)
+        what = f"{NAMES[dtype]} {shape} {kind}"
+        # sum
+        po, do = gpu.put(T.empty(dtype, []))
+        G.run_gpu(gpu, "aixk_reduce_all", K.SUM, G.ref(da), G.ref(do))
+        got = gpu.fetch(po, np.zeros(1, O.NP_STORAGE[dtype]))
+        if dtype in T.INT_DTYPES:
+            want = T.empty(dtype, [])
+            okc(CPU.sum(C.byref(a.desc()), C.byref(want.desc())))
+            T.assert_same_bits(got, want.storage, "sum " + what)
+        else:
+            s, sa = C.c_double(), C.c_double()
+            okc(CPU.sum_wide(C.byref(a.desc()), C.byref(s), C.byref(sa)))
+            check_sum_like(got, dtype, [s.value], [sa.value], "sum " + what)
+        # max, argmax, one-hot: exact
+        for kind_code, name, odt, oshape in ((K.MAX, "max", dtype, []), (K.ARGMAX, "argmax", O.I32, []),
+                                             (K.ARGMAX_ONEHOT, "argmax_indices", O.I32, shape)):
+            want = T.empty(odt, oshape)
+            okc(getattr(CPU, name)(C.byref(a.desc()), C.byref(want.desc())))
+            po, do = gpu.put(T.empty(odt, oshape, fill=-5 if odt == O.I32 else None))
+            G.run_gpu(gpu, "aixk_reduce_all", kind_code, G.ref(da), G.ref(do))
+            T.assert_same_bits_nan_ok(gpu.fetch(po, want.storage), want.storage, odt, f"{name} " + what)
+        gpu.release()
+    # int32-only results (aixDeviceCPU.cpp:1027-1030)
+    a = T.contiguous_tensor(rng, dtype, [4])
+    _, da = gpu.put(a)
+    _, bad = gpu.put(T.empty(O.F32, []))
+    assert gpu.ctx.lib.aixk_reduce_all(gpu.ctx.handle, K.ARGMAX, G.ref(da), G.ref(bad)) == 1
+    assert b"int32" in gpu.ctx.lib.aixk_last_error()
+    gpu.release()
+
+
+@pytest.mark.parametrize("dtype", [O.F64, O.F32, O.F16, O.BF16], ids=ids)
+def test_max_argmax_nan_rules(gpu, dtype):
+    """NaN never wins unless it leads its slot (strict '>' scan / std::max on the CPU)."""
+    base = np.array([1.0, 5.0, np.nan, 7.0, np.nan, 7.0, 2.0, -np.inf], dtype=np.float64)
+    for lead_nan in (False, True):
+        for n in (8, 300, 5000):
+            vals = np.resize(base, n).copy()
+            if lead_nan:
+                vals[0] = np.nan
+            a = T.HostTensor(O.to_storage(vals, dtype), dtype, [n])
+            _, da = gpu.put(a)
+            for kind_code, name, odt, oshape in ((K.MAX, "max", dtype, []), (K.ARGMAX, "argmax", O.I32, []),
+                                                 (K.ARGMAX_ONEHOT, "argmax_indices", O.I32, [n])):
+                want = T.empty(odt, oshape)
+                okc(getattr(CPU, name)(C.byref(a.desc()), C.byref(want.desc())))
+                po, do = gpu.put(T.empty(odt, oshape))
+                G.run_gpu(gpu, "aixk_reduce_all", kind_code, G.ref(da), G.ref(do))
+                T.assert_same_bits_nan_ok(gpu.fetch(po, want.storage), want.storage, odt, f"{name} nan lead={lead_nan} n={n}")
+            # per-row: rows of 4 with NaN in leading / middle positions
+            rows = T.HostTensor(O.to_storage(np.resize(np.array([np.nan, 1, 2, 2, 3, np.nan, 3, 1, -1, -1, np.nan, np.nan]), 96), dtype), dtype, [24, 4])
+            _, dr = gpu.put(rows)
+            want = T.empty(O.I32, [24, 1])
+            okc(CPU.argmax_to(C.byref(rows.desc()), C.byref(want.desc()), 1))
+            po, do = gpu.put(T.empty(O.I32, [24, 1]))
+            G.run_gpu(gpu, "aixk_argmax_to", 0, G.ref(dr), G.ref(do), 1)
+            T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, "argmaxTo with NaN")
+            init = T.HostTensor(O.to_storage(np.resize(np.array([-np.inf, np.nan, 2.5]), 24), dtype), dtype, [24, 1])
+            want = init.clone()
+            okc(CPU.max_to(C.byref(rows.desc()), C.byref(want.desc())))
+            pi, di = gpu.put(init)
+            G.run_gpu(gpu, "aixk_reduce_to", K.MAX, G.ref(dr), G.ref(di))
+            T.assert_same_bits_nan_ok(gpu.fetch(pi, want.storage), want.storage, dtype, "maxTo with NaN")
+            gpu.release()
+
+
+def reduced_shapes(rng, shape):
+    rank = len(shape)
+    outs = []
+    for _ in range(3):
+        mask = [bool(rng.integers(0, 2)) for _ in shape]
+        outs.append([1 if m else e for e, m in zip(shape, mask)])
+    outs.append([1] * rank)
+    k = int(rng.integers(0, rank))
+    outs.append(shape[k:])
+    outs.append([1 if i % 2 else e for i, e in enumerate(shape[k:])])
+    return outs
+
+
+ROUTE_CASES = [  # (source shape, view kind, destination shape) chosen to hit every kernel route
+    ([300, 4096], "contig", [300, 1]),        # inner, workgroup per row, vector loads
+    ([300, 4100], "contig", [300, 1]),        # inner, long ragged rows
+    ([2000, 96], "contig", [2000, 1]),        # inner, wave per row
+    ([64, 100], "sliced", [64, 1]),           # inner, scalar loads
+    ([500, 10], "contig", [500, 1]),          # short rows: generic, lane per slot
+    ([3000, 512], "contig", [1, 512]),        # outer, rows split over workgroups + finish pass
+    ([40, 8192], "contig", [1, 8192]),        # outer, single chunk
+    ([777, 130], "contig", [130]),            # outer, ragged columns, dst rank dropped
+    ([6, 500, 64], "contig", [6, 1, 64]),     # outer with a leading kept dim
+    ([50, 70], "transposed", [50, 1]),        # generic
+    ([9, 40, 33], "contig", [1, 40, 1]),      # two reduced dims: generic, workgroup per slot
+    ([128, 128], "contig", [1, 1]),           # everything folds into one slot
+    ([5, 7], "broadcast", [1, 7]),
+]
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_reduce_to_and_max_to(gpu, dtype):
+    rng = np.random.default_rng(19000 + dtype)
+    cases = list(ROUTE_CASES)
+    for _ in range(8):
+        shape = T.random_shape(rng, max_rank=5, max_extent=6)
+        kind = rng.choice(T.VIEW_KINDS)
+        cases += [(shape, kind, d) for d in reduced_shapes(rng, shape)]
+    for shape, kind, dshape in cases:
+        src = T.view_tensor(rng, dtype, shape, kind, int_span=20)
+        _, ds = gpu.put(src)
+        init = T.contiguous_tensor(rng, dtype, dshape, int_span=5)      # the ops accumulate INTO dst
+        what = f"{NAMES[dtype]} {shape}->{dshape} {kind}"
+        # maxTo: exact
+        want = init.clone()
+        okc(CPU.max_to(C.byref(src.desc()), C.byref(want.desc())))
+        pi, di = gpu.put(init)
+        G.run_gpu(gpu, "aixk_reduce_to", K.MAX, G.ref(ds), G.ref(di))
+        T.assert_same_bits_nan_ok(gpu.fetch(pi, want.storage), want.storage, dtype, "maxTo " + what)
+        # reduceTo
+        pi, di = gpu.put(init)
+        G.run_gpu(gpu, "aixk_reduce_to", K.SUM, G.ref(ds), G.ref(di))
+        got = gpu.fetch(pi, init.storage)
+        if dtype in T.INT_DTYPES:
+            want = init.clone()
+            okc(CPU.reduce_to(C.byref(src.desc()), C.byref(want.desc())))
+            T.assert_same_bits(got, want.storage, "reduceTo " + what)
+        else:
+            exact = init.values().reshape(-1).copy()
+            scale = np.abs(exact)
+            okc(CPU.reduce_to_wide(C.byref(src.desc()), C.byref(init.desc()), exact.ctypes.data, scale.ctypes.data))
+            check_sum_like(got, dtype, exact, scale, "reduceTo " + what)
+        gpu.release()
+
+
+ARG_CASES = [  # (shape, kind, dim)
+    ([512, 700], "contig", 0), ([3000, 256], "contig", 0), ([40, 8192], "contig", 0),
+    ([300, 4096], "contig", 1), ([2000, 96], "contig", 1), ([500, 10], "contig", 1),
+    ([6, 500, 64], "contig", 1), ([9, 40, 33], "contig", 2), ([9, 40, 33], "contig", 0),
+    ([3, 2], "transposed", 1), ([64, 100], "transposed", 0),
+]
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_argmax_to_family(gpu, dtype):
+    rng = np.random.default_rng(20000 + dtype)
+    cases = list(ARG_CASES)
+    for _ in range(12):
+        shape = T.random_shape(rng, max_rank=4, max_extent=6)
+        cases.append((shape, rng.choice(["contig", "contig", "transposed", "sliced", "offset"]), int(rng.integers(0, len(shape)))))
+    for shape, kind, dim in cases:
+        src = T.view_tensor(rng, dtype, shape, kind, int_span=2, lo=-1, hi=1)
+        if dtype in T.FLOAT_DTYPES:                                  # force ties: quantise to 5 levels
+            src.storage[:] = O.to_storage(np.round(O.to_float64(src.storage, dtype) * 2) / 2, dtype)
+        _, ds = gpu.put(src)
+        keep = [1 if d == dim else e for d, e in enumerate(shape)]
+        for dshape in (keep, [e for d, e in enumerate(shape) if d != dim] or [1]):
+            want = T.empty(O.I32, dshape, fill=-7)
+            okc(CPU.argmax_to(C.byref(src.desc()), C.byref(want.desc()), dim))
+            po, do = gpu.put(T.empty(O.I32, dshape, fill=-7))
+            G.run_gpu(gpu, "aixk_argmax_to", 0, G.ref(ds), G.ref(do), dim)
+            T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"argmaxTo {NAMES[dtype]} {shape} dim={dim} {kind} -> {dshape}")
+        want = T.empty(O.I32, shape)
+        okc(CPU.argmax_indices_to(C.byref(src.desc()), C.byref(want.desc()), dim))
+        po, do = gpu.put(T.empty(O.I32, shape))
+        G.run_gpu(gpu, "aixk_argmax_to", 1, G.ref(ds), G.ref(do), dim)
+        T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"argmaxIndicesTo {NAMES[dtype]} {shape} dim={dim} {kind}")
+        gpu.release()
+    src = T.contiguous_tensor(rng, dtype, [4, 4])
+    _, ds = gpu.put(src)
+    _, bad = gpu.put(T.empty(O.F32, [4]))
+    assert gpu.ctx.lib.aixk_argmax_to(gpu.ctx.handle, 0, G.ref(ds), G.ref(bad), 1) == 1
+    gpu.release()
+
+
+# ---- matmul ---------------------------------------------------------------------------------------
+MM_SIZES = [(1, 1, 1), (2, 3, 4), (1, 64, 1), (1, 257, 33), (33, 1, 17), (64, 64, 64), (65, 63, 67), (128, 256, 64),
+            (257, 129, 513), (100, 300, 50), (512, 512, 512), (31, 1024, 9)]   # incl. DeviceTests.cpp:2806-2875 style edges
+
+
+def check_matmul(gpu, a, b, what):
+    dtype = a.dtype
+    m, k, n = a.shape[0], a.shape[1], b.shape[1]
+    _, da = gpu.put(a)
+    _, db = gpu.put(b)
+    po, do = gpu.put(T.empty(dtype, [m, n]))
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+    got = gpu.fetch(po, np.zeros(m * n, O.NP_STORAGE[dtype]))
+    if dtype in T.INT_DTYPES:
+        want = T.empty(dtype, [m, n])
+        okc(CPU.matmul_rows(C.byref(a.desc()), C.byref(b.desc()), C.byref(want.desc()), 8))
+        return T.assert_same_bits(got, want.storage, what)
+    exact = np.zeros(m * n)
+    scale = np.zeros(m * n)
+    okc(CPU.matmul_wide(C.byref(a.desc()), C.byref(b.desc()), exact.ctypes.data, scale.ctypes.data, 8))
+    tol = {O.F64: 1e-12, O.F32: 1e-5, O.F16: 2e-2, O.BF16: 2e-2}[dtype]
+    G.assert_close_to_wide(O.to_float64(got, dtype), exact, scale + 1e-30, tol, what)
+    # and much tighter in practice for the 16-bit types: f32 accumulation + one final rounding
+    if dtype in (O.F16, O.BF16):
+        final = 2.0 ** -10 if dtype == O.F16 else 2.0 ** -8
+        G.assert_close_to_wide(O.to_float64(got, dtype), exact, 1e-5 * scale + final * np.abs(exact) + 1e-30, 1.0, what + " (tight)")
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_matmul(gpu, dtype):
+    rng = np.random.default_rng(21000 + dtype)
+    for (m, k, n) in MM_SIZES:
+        kinds = [("contig", "contig")]
+        if (m, k, n) in ((65, 63, 67), (128, 256, 64), (100, 300, 50), (257, 129, 513)):
+            kinds += [("transposed", "contig"), ("contig", "transposed"), ("transposed", "transposed"), ("offset", "sliced")]
+        for ka, kb in kinds:
+            scale = 1.0 / np.sqrt(k)
+            a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale, int_span=9)
+            b = T.view_tensor(rng, dtype, [k, n], kb, lo=-1, hi=1, int_span=9)
+            check_matmul(gpu, a, b, f"matmul {NAMES[dtype]} {m}x{k}x{n} {ka}/{kb}")
+        gpu.release()
+
+
+def test_matmul_identity_and_ones(gpu):
+    """Mathematical pins: A.I == A exactly; ones[m,k].ones[k,n] == k exactly (f32, f16, bf16)."""
+    rng = np.random.default_rng(22000)
+    for dtype in (O.F32, O.F16, O.BF16):
+        a = T.contiguous_tensor(rng, dtype, [96, 160])
+        eye = T.HostTensor(O.to_storage(np.eye(160).reshape(-1), dtype), dtype, [160, 160])
+        _, da = gpu.put(a)
+        _, de = gpu.put(eye)
+        po, do = gpu.put(T.empty(dtype, [96, 160]))
+        G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(de), G.ref(do))
+        T.assert_same_bits(gpu.fetch(po, a.storage), a.storage, f"A.I {NAMES[dtype]}")
+        ones_a = T.HostTensor(O.to_storage(np.ones(70 * 200), dtype), dtype, [70, 200])
+        ones_b = T.HostTensor(O.to_storage(np.ones(200 * 90), dtype), dtype, [200, 90])
+        _, d1 = gpu.put(ones_a)
+        _, d2 = gpu.put(ones_b)
+        po, do = gpu.put(T.empty(dtype, [70, 90]))
+        G.run_gpu(gpu, "aixk_matmul", G.ref(d1), G.ref(d2), G.ref(do))
+        got = O.to_float64(gpu.fetch(po, np.zeros(70 * 90, O.NP_STORAGE[dtype])), dtype)
+        assert np.all(got == 200.0), f"ones.ones {NAMES[dtype]}"
+        gpu.release()
+
+
+# ---- the reference's own literal vectors through the GPU kernels ----------------------------------
+import goldens  # noqa: E402
+
+_CASES = goldens.load_cases()
+
+
+@pytest.mark.parametrize("case", _CASES, ids=[c["name"] for c in _CASES])
+def test_reference_literals_on_gpu(gpu, case):
+    goldens.run_case(case, G.KernelBackend(gpu))
