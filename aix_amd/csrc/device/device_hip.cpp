@@ -1,0 +1,691 @@
+// device_hip.cpp -- DeviceHIP: host-side logic of the MI355X backend (see device_hip.hpp).
+
+#include "device_hip.hpp"
+
+#include "../../../include/aixhip_kernels.h"
+#include "hipgen.hpp"
+
+#include <algorithm>
+#include <array>
+#include <cstring>
+#include <deque>
+#include <iostream>
+#include <stdexcept>
+
+namespace aix {
+
+#ifndef AIXHIP_USE_AIX_HEADERS
+// In an AIX build these two come from the framework's own library (aixDeviceCPU.cpp:26, 685-700).
+Device::~Device() = default;
+
+size_t Device::dataTypeSize(DataType dtype)
+{
+    static const size_t bytes[DataTypeCount] = {8, 4, 2, 2, 8, 4, 2, 1, 1};
+    return bytes[static_cast<size_t>(dtype)];
+}
+#endif
+
+namespace hip {
+
+using aixhip::fuse::FuseCallbacks;
+using aixhip::fuse::FuseConfig;
+using aixhip::fuse::FuseEngine;
+using aixhip::fuse::FusedSubgraphDescriptor;
+using aixhip::fuse::OpRecord;
+using aixhip::fuse::OpType;
+namespace gen = aixhip::gen;
+
+namespace {
+
+// Freed blocks wait here until the GPU has passed the point at which they were released: the host
+// may write into a reused block directly, which is not ordered with the stream.
+struct Cooling {
+    aixk_event* event;
+    std::vector<std::pair<void*, size_t>> blocks;
+};
+
+struct Extras {
+    std::deque<Cooling> cooling;
+    std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
+    uint64_t hits{0}, misses{0};
+};
+
+std::unordered_map<const DeviceHIP*, Extras>& extras()
+{
+    static std::unordered_map<const DeviceHIP*, Extras> e;
+    return e;
+}
+
+size_t viewEnd(const DeviceTensorParams& p)
+{
+    size_t last = p.offset;
+    for (size_t d = 0; d < p.shape.size(); ++d) {
+        if (p.shape[d] == 0) return p.offset;
+        last += (p.shape[d] - 1) * p.strides[d];
+    }
+    return last + 1;
+}
+
+bool isDense(const DeviceTensorParams& p)
+{
+    size_t run = 1;
+    for (size_t d = p.shape.size(); d-- > 0;) {
+        if (p.shape[d] != 1 && p.strides[d] != run) return false;
+        run *= p.shape[d];
+    }
+    return true;
+}
+
+Stride denseStrides(const Shape& shape)
+{
+    Stride s(shape.size());
+    size_t run = 1;
+    for (size_t d = shape.size(); d-- > 0;) { s[d] = run; run *= shape[d]; }
+    return s;
+}
+
+int binaryCode(OpType t)
+{
+    switch (t) {
+        case OpType::Add: return AIXK_ADD; case OpType::Sub: return AIXK_SUB; case OpType::Mul: return AIXK_MUL;
+        case OpType::Div: return AIXK_DIV; case OpType::Pow: return AIXK_POW; default: return -1;
+    }
+}
+
+int unaryCode(OpType t)
+{
+    switch (t) {
+        case OpType::Negate: return AIXK_NEG; case OpType::Sqrt: return AIXK_SQRT; case OpType::Sin: return AIXK_SIN;
+        case OpType::Cos: return AIXK_COS; case OpType::Tanh: return AIXK_TANH; case OpType::Log: return AIXK_LOG;
+        case OpType::Exp: return AIXK_EXP; default: return -1;
+    }
+}
+
+} // namespace
+
+// ---- construction ------------------------------------------------------------------------------
+DeviceHIP::DeviceHIP(size_t deviceIndex)
+{
+    const int rc = aixk_create((int)deviceIndex, &m_ctx);
+    if (rc != AIXK_OK) throw std::runtime_error(std::string("DeviceHIP: ") + aixk_last_error());
+    aixk_device_info info{};
+    if (aixk_info(m_ctx, &info) == AIXK_OK && info.compute_units > 0) m_cus = info.compute_units;
+    if (aixk_info(m_ctx, &info) == AIXK_OK && !info.large_bar)
+        std::cerr << "DeviceHIP: device memory is not host-addressable on this system; tensors must be moved with "
+                     "copy()/copyToHost() and never dereferenced on the host." << std::endl;
+    FuseConfig cfg;
+    cfg.maxBufferSlots = 24;
+    cfg.supportsStridedFusion = true;
+    extras()[this];
+    setFuseConfig(cfg);
+}
+
+DeviceHIP::~DeviceHIP()
+{
+    try {
+        if (m_engine && m_engine->pendingOps() > 0)
+            std::cerr << "DeviceHIP: destroyed with recorded work that was never synchronised." << std::endl;   // aixDeviceMetal.cpp:146-149
+        if (m_engine) m_engine.reset();
+        if (m_ctx) {
+            aixk_sync(m_ctx);
+            auto& ex = extras()[this];
+            for (auto& c : ex.cooling) { aixk_event_destroy(m_ctx, c.event); for (auto& b : c.blocks) aixk_free(m_ctx, b.first, 0); }
+            for (auto& b : m_limbo) aixk_free(m_ctx, b.first, 0);
+            for (auto& kv : m_pool) for (void* p : kv.second) aixk_free(m_ctx, p, 0);
+            for (auto& kv : m_blocks) aixk_free(m_ctx, (void*)kv.first, 0);
+            aixk_destroy(m_ctx);
+        }
+    } catch (...) {
+    }
+    extras().erase(this);
+}
+
+std::unique_ptr<aix::Device> createDeviceHIP(size_t deviceIndex)
+{
+    try { return std::make_unique<DeviceHIP>(deviceIndex); }
+    catch (const std::exception&) { return nullptr; }             // as createDevice() does for an absent GPU (aixDevices.cpp:28-33)
+}
+
+void DeviceHIP::setFuseConfig(const FuseConfig& cfg)
+{
+    if (m_engine) flush();
+    FuseCallbacks cb;
+    cb.emitFused = [this](const FusedSubgraphDescriptor& d) { emitFused(d); };
+    cb.emitSingle = [this](const OpRecord& op) { emitSingle(op); };
+    cb.finishFlush = [] {};
+    cb.getKernelCacheStats = [this] { return fuseKernelCacheStats(); };
+    m_engine = std::make_unique<FuseEngine>(cfg, std::move(cb));
+    for (auto& kv : m_blocks) m_engine->retainBuffer((void*)kv.first);
+}
+
+std::pair<size_t, size_t> DeviceHIP::fuseKernelCacheStats() const
+{
+    const auto& ex = extras()[this];
+    return {(size_t)ex.hits, (size_t)ex.misses};
+}
+
+void DeviceHIP::check(int status) const
+{
+    if (status == AIXK_OK) return;
+    const std::string msg = std::string("DeviceHIP: ") + aixk_last_error();
+    if (status == AIXK_EINVAL) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
+}
+
+// ---- memory ------------------------------------------------------------------------------------
+const DeviceHIP::Block* DeviceHIP::findBlock(const void* p) const
+{
+    if (!p || m_blocks.empty()) return nullptr;
+    auto it = m_blocks.upper_bound((uintptr_t)p);
+    if (it == m_blocks.begin()) return nullptr;
+    --it;
+    return ((uintptr_t)p < it->first + it->second.bytes) ? &it->second : nullptr;
+}
+
+// 256-byte steps up to 4 KiB, then eight steps per power of two: at most 12.5 % slack, few buckets.
+size_t DeviceHIP::bucketBytes(size_t bytes) const
+{
+    if (bytes < 256) return 256;
+    if (bytes <= 4096) return (bytes + 255) & ~(size_t)255;
+    size_t top = 1;
+    while ((top << 1) <= bytes) top <<= 1;
+    const size_t step = top >> 3;
+    return (bytes + step - 1) & ~(step - 1);
+}
+
+void* DeviceHIP::allocateBlock(size_t bytes, bool track)
+{
+    auto& ex = extras()[this];
+    // blocks whose release point the GPU has passed become reusable
+    while (!ex.cooling.empty()) {
+        int32_t done = 0;
+        if (aixk_event_query(m_ctx, ex.cooling.front().event, &done) != AIXK_OK || !done) break;
+        for (auto& b : ex.cooling.front().blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        aixk_event_destroy(m_ctx, ex.cooling.front().event);
+        ex.cooling.pop_front();
+    }
+    const size_t bucket = bucketBytes(bytes);
+    void* p = nullptr;
+    auto it = m_pool.find(bucket);
+    if (it != m_pool.end() && !it->second.empty()) {
+        p = it->second.back();
+        it->second.pop_back();
+        m_pooledBytes -= bucket;
+    } else if (aixk_alloc(m_ctx, bucket, 0, &p) != AIXK_OK) {
+        // out of memory: finish everything, give cached blocks back, try once more (aixDeviceMetal.cpp:1455-1471)
+        synchronize();
+        emptyCache();
+        if (aixk_alloc(m_ctx, bucket, 0, &p) != AIXK_OK)
+            throw std::runtime_error(std::string("DeviceHIP: GPU memory allocation has failed for size: ") + std::to_string(bytes) + " bytes. " + aixk_last_error());
+    }
+    if (track) {
+        m_blocks[(uintptr_t)p] = Block{bucket};
+        m_liveBytes += bucket;
+        m_engine->retainBuffer(p);
+    }
+    return p;
+}
+
+void* DeviceHIP::allocate(size_t size) { return allocateBlock(size, true); }
+
+void* DeviceHIP::allocate(size_t size, DataType dtype) { return allocateBlock(size * dataTypeSize(dtype), true); }
+
+void DeviceHIP::deallocate(void* memory)
+{
+    if (!memory) return;
+    auto it = m_blocks.find((uintptr_t)memory);
+    if (it == m_blocks.end()) throw std::invalid_argument("DeviceHIP::deallocate() - Found different type of memory to free.");   // aixDeviceMetal.cpp:253-254
+    m_engine->releaseBuffer(memory);
+    m_limbo.emplace_back(memory, it->second.bytes);
+    m_limboBytes += it->second.bytes;
+    m_liveBytes -= it->second.bytes;
+    m_blocks.erase(it);
+    if (m_limboBytes > (size_t(8) << 30)) flush();          // recorded work pins too much freed memory
+}
+
+// Called once the recorded work that might touch freed blocks has been enqueued.
+void DeviceHIP::releaseLimbo()
+{
+    if (m_limbo.empty()) return;
+    auto& ex = extras()[this];
+    Cooling c{};
+    if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
+        c.blocks.swap(m_limbo);
+        ex.cooling.push_back(std::move(c));
+    } else {
+        aixk_sync(m_ctx);
+        for (auto& b : m_limbo) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        m_limbo.clear();
+    }
+    m_limboBytes = 0;
+}
+
+void DeviceHIP::emptyCache()
+{
+    for (auto& kv : m_pool) for (void* p : kv.second) aixk_free(m_ctx, p, 0);
+    m_pool.clear();
+    m_pooledBytes = 0;
+}
+
+void DeviceHIP::flush()
+{
+    m_engine->flush();
+    releaseLimbo();
+}
+
+void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
+{
+    m_engine->recordExternalRead(a);
+    m_engine->recordExternalRead(b);
+    m_engine->recordExternalRead(c);
+    flush();
+}
+
+void DeviceHIP::synchronize()
+{
+    flush();
+    check(aixk_sync(m_ctx));
+    auto& ex = extras()[this];
+    for (auto& c : ex.cooling) {
+        for (auto& b : c.blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        aixk_event_destroy(m_ctx, c.event);
+    }
+    ex.cooling.clear();
+}
+
+void DeviceHIP::copyToHost(void* dstHost, const void* srcDevice, size_t bytes)
+{
+    flushFor(srcDevice);
+    check(aixk_copy_out(m_ctx, dstHost, srcDevice, bytes));
+}
+
+void DeviceHIP::copyFromHost(void* dstDevice, const void* srcHost, size_t bytes)
+{
+    if (!findBlock(dstDevice)) throw std::invalid_argument("DeviceHIP::copyFromHost() result must have GPU memory.");
+    flushFor(dstDevice);
+    check(aixk_copy_in(m_ctx, dstDevice, srcHost, bytes));
+}
+
+// ---- operand handling --------------------------------------------------------------------------
+void DeviceHIP::requireDevice(const DeviceTensorParams& result, const char* op) const
+{
+    if (result.size > 0 && !findBlock(result.data))
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() result must have GPU memory.");      // aixDeviceMetal.cpp:305-306
+}
+
+const void* DeviceHIP::stageRaw(const void* src, size_t bytes)
+{
+    void* tmp = allocateBlock(bytes, false);
+    check(aixk_copy_in(m_ctx, tmp, src, bytes));
+    m_limbo.emplace_back(tmp, bucketBytes(bytes));          // recycled after the work that reads it is enqueued
+    m_limboBytes += bucketBytes(bytes);
+    return tmp;
+}
+
+DeviceTensorParams DeviceHIP::onDevice(const DeviceTensorParams& p)
+{
+    if (!p.data || p.size == 0 || findBlock(p.data)) return p;
+    DeviceTensorParams q = p;                               // a host tensor handed straight to the device (DeviceTests.cpp:209-215)
+    q.data = const_cast<void*>(stageRaw(p.data, viewEnd(p) * dataTypeSize(p.dtype)));
+    return q;
+}
+
+void DeviceHIP::toPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op) const
+{
+    if (p.shape.size() > AIXK_MAX_RANK)
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");    // aixDeviceMetal.cpp:671-672
+    std::memset(out, 0, sizeof(*out));
+    out->data = p.data;
+    out->dtype = (int32_t)p.dtype;
+    out->rank = (int32_t)p.shape.size();
+    out->offset = p.offset;
+    out->size = p.size;
+    for (size_t d = 0; d < p.shape.size(); ++d) { out->shape[d] = p.shape[d]; out->strides[d] = d < p.strides.size() ? p.strides[d] : 0; }
+}
+
+// ---- recorded (fusable) operators --------------------------------------------------------------
+void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& r, const char* op)
+{
+    requireDevice(r, op);
+    if (a.dtype != r.dtype || b.dtype != r.dtype)
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operands must have the result's data type.");
+    if (a.shape.size() > AIXK_MAX_RANK) throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
+    DeviceTensorParams out = r;                             // results are written densely from the base pointer
+    out.offset = 0; out.strides = denseStrides(r.shape); out.isContiguous = true;
+    m_engine->record(t, onDevice(a), onDevice(b), out);
+}
+
+void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op)
+{
+    requireDevice(r, op);
+    if (a.dtype != r.dtype)
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operand must have the result's data type.");
+    if (a.shape.size() > AIXK_MAX_RANK) throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
+    DeviceTensorParams out = r;
+    out.offset = 0; out.strides = denseStrides(r.shape); out.isContiguous = true;
+    out.size = a.size;                                      // unary loops run over the operand (aixDeviceCPU.cpp:90)
+    if (out.shape != a.shape) { out.shape = a.shape; out.strides = denseStrides(a.shape); }
+    m_engine->record(t, onDevice(a), out);
+}
+
+void DeviceHIP::add(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Add, a1, a2, result, "add"); }
+void DeviceHIP::sub(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Sub, a1, a2, result, "sub"); }
+void DeviceHIP::mul(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Mul, a1, a2, result, "mul"); }
+void DeviceHIP::div(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Div, a1, a2, result, "div"); }
+void DeviceHIP::pow(const DeviceTensorParams& a, const DeviceTensorParams& e, const DeviceTensorParams& result) { recordBinary(OpType::Pow, a, e, result, "pow"); }
+void DeviceHIP::unary(const DeviceTensorParams& a1, const DeviceTensorParams& result) { recordUnary(OpType::Negate, a1, result, "unary"); }
+void DeviceHIP::sqrt(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Sqrt, a, result, "sqrt"); }
+void DeviceHIP::sin(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Sin, a, result, "sin"); }
+void DeviceHIP::cos(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Cos, a, result, "cos"); }
+void DeviceHIP::tanh(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Tanh, a, result, "tanh"); }
+void DeviceHIP::log(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Log, a, result, "log"); }
+void DeviceHIP::exp(const DeviceTensorParams& a, const DeviceTensorParams& result) { recordUnary(OpType::Exp, a, result, "exp"); }
+
+void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTensorParams& result)
+{
+    requireDevice(result, "fill");
+    DeviceTensorParams out = result;
+    out.offset = 0; out.strides = denseStrides(result.shape); out.isContiguous = true;
+    m_engine->recordFill(scalar, scalarDType, out);
+}
+
+void DeviceHIP::fillMin(const DeviceTensorParams& result)
+{
+    requireDevice(result, "fillMin");
+    DeviceTensorParams out = result;
+    out.offset = 0; out.strides = denseStrides(result.shape); out.isContiguous = true;
+    m_engine->recordFillMin(out);
+}
+
+// ---- planner callbacks -------------------------------------------------------------------------
+void DeviceHIP::emitSingle(const OpRecord& op)
+{
+    aixhip_tensor a, b, o;
+    toPod(op.output, &o, "emit");
+    if (op.type == OpType::Fill) { check(aixk_fill(m_ctx, op.scalarData.data(), (int)op.scalarDType, &o)); return; }
+    if (op.type == OpType::FillMin) { check(aixk_fill_min(m_ctx, &o)); return; }
+    toPod(op.input0, &a, "emit");
+    if (const int code = binaryCode(op.type); code >= 0) {
+        toPod(op.input1, &b, "emit");
+        check(aixk_binary(m_ctx, code, &a, &b, &o));
+        return;
+    }
+    if (const int code = unaryCode(op.type); code >= 0) { check(aixk_unary(m_ctx, code, &a, &o)); return; }
+    throw std::runtime_error(std::string("DeviceHIP: operator cannot be replayed: ") + aixhip::fuse::opName(op.type));
+}
+
+void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
+{
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
+    const size_t esz = dataTypeSize(d.dtype);
+    const size_t VEC = 16 / esz;
+    const uint64_t n = d.elementCount;
+    if (n == 0 || NO == 0) return;
+
+    // Joint iteration space over the fused shape: dense views get the dense strides of that shape
+    // (their own shape may be a different factorisation of the same count), strided views keep
+    // theirs; one extra dense operand stands for the outputs so dims merge only where they may.
+    const Stride dense = denseStrides(d.shape);
+    const size_t rank = d.shape.size();
+    std::vector<Stride> strides(NI + 1);
+    for (size_t k = 0; k < NI; ++k) {
+        const auto& v = d.inputBuffers[k];
+        if (isDense(v)) strides[k] = dense;
+        else if (v.shape == d.shape) strides[k] = v.strides;
+        else throw std::runtime_error("DeviceHIP: fused kernel received a strided view of a foreign shape");
+    }
+    strides[NI] = dense;
+    // collapse: drop extent-1 dims, merge neighbours where every operand allows it
+    std::vector<uint64_t> shp;
+    std::vector<std::vector<uint64_t>> str(NI + 1);
+    for (size_t dd = 0; dd < rank; ++dd) {
+        if (d.shape[dd] == 1) continue;
+        bool merged = false;
+        if (!shp.empty()) {
+            bool ok = true;
+            for (size_t k = 0; k <= NI; ++k) if (str[k].back() != strides[k][dd] * d.shape[dd]) ok = false;
+            if (ok) {
+                shp.back() *= d.shape[dd];
+                for (size_t k = 0; k <= NI; ++k) str[k].back() = strides[k][dd];
+                merged = true;
+            }
+        }
+        if (!merged) {
+            shp.push_back(d.shape[dd]);
+            for (size_t k = 0; k <= NI; ++k) str[k].push_back(strides[k][dd]);
+        }
+    }
+    if (shp.size() > (size_t)gen::kMaxDims) throw std::invalid_argument("DeviceHIP: fused view does not collapse to 8 dimensions.");
+
+    auto aligned = [](const void* p) { return ((uintptr_t)p & 15u) == 0; };
+    std::vector<const void*> inPtr(NI);
+    std::vector<void*> outPtr(NO);
+    for (size_t k = 0; k < NO; ++k) outPtr[k] = d.outputBuffers[k].data;
+    bool outsAligned = true;
+    for (void* p : outPtr) if (!aligned(p)) outsAligned = false;
+
+    gen::Shape shape = gen::Shape::Gather;
+    uint32_t bmask = 0;
+    uint64_t chunks = 0;
+    const size_t cr = shp.size();
+    if (cr <= 1) {
+        bool ok = outsAligned;
+        for (size_t k = 0; k < NI && ok; ++k) {
+            const uint64_t s = cr ? str[k][0] : 0;
+            const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+            if (cr == 1 && s == 0) bmask |= 1u << k;
+            else if (cr == 1 && s != 1) ok = false;
+            else if (!aligned(base)) ok = false;
+        }
+        if (ok) shape = gen::Shape::Flat;
+    } else {
+        bool ok = outsAligned && shp[cr - 1] % VEC == 0;
+        for (size_t k = 0; k < NI && ok; ++k) {
+            const uint64_t s = str[k][cr - 1];
+            if (s > 1) ok = false;
+            if (s == 1) {
+                const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+                if (!aligned(base)) ok = false;
+                for (size_t dd = 0; dd + 1 < cr; ++dd) if (str[k][dd] % VEC) ok = false;
+            }
+        }
+        if (ok) { shape = gen::Shape::Rows; chunks = shp[cr - 1] / VEC; }
+    }
+
+    gen::Space space;
+    if (shape == gen::Shape::Flat) {
+        for (size_t k = 0; k < NI; ++k) inPtr[k] = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+    } else {
+        space.rank = (uint32_t)cr;
+        for (int dd = 0; dd < gen::kMaxDims; ++dd) space.shape[dd] = dd < (int)cr ? shp[dd] : 1;
+        space.offset.resize(NI);
+        space.stride.resize(NI);
+        for (size_t k = 0; k < NI; ++k) {
+            inPtr[k] = d.inputBuffers[k].data;
+            space.offset[k] = d.inputBuffers[k].offset;
+            for (int dd = 0; dd < gen::kMaxDims; ++dd) space.stride[k][dd] = dd < (int)cr ? str[k][dd] : 0;
+        }
+    }
+
+    auto& ex = extras()[this];
+    const std::string key = gen::signature(d, shape);
+    aixk_module* mod = nullptr;
+    auto it = ex.kernels.find(key);
+    if (it != ex.kernels.end()) { mod = it->second; ++ex.hits; }
+    else {
+        int32_t cached = 0;
+        const std::string src = gen::source(d, shape);
+        check(aixk_rtc_get(m_ctx, key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
+        ex.kernels.emplace(key, mod);
+        ++ex.misses;
+    }
+
+    const auto args = gen::packArgs(d, shape, inPtr, outPtr, n, bmask, shape == gen::Shape::Flat ? nullptr : &space, chunks);
+    uint64_t items, perBlock, cap;
+    if (shape == gen::Shape::Flat) { items = n / VEC + 1; perBlock = (uint64_t)gen::kBlock * gen::flatUnroll(NI); cap = (uint64_t)m_cus * 32; }
+    else if (shape == gen::Shape::Rows) { items = n / VEC; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
+    else { items = n; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
+    uint64_t grid = (items + perBlock - 1) / perBlock;
+    grid = std::max<uint64_t>(1, std::min(grid, cap));
+    check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, args.data(), args.size() * sizeof(uint64_t)));
+}
+
+// ---- operators that run at once ------------------------------------------------------------------
+void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& result)
+{
+    requireDevice(result, "sum");
+    flushFor(a.data, result.data);
+    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "sum"); toPod(result, &pr, "sum");
+    check(aixk_reduce_all(m_ctx, AIXK_SUM, &pa, &pr));
+}
+
+void DeviceHIP::max(const DeviceTensorParams& a, const DeviceTensorParams& result)
+{
+    requireDevice(result, "max");
+    flushFor(a.data, result.data);
+    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "max"); toPod(result, &pr, "max");
+    check(aixk_reduce_all(m_ctx, AIXK_MAX, &pa, &pr));
+}
+
+void DeviceHIP::argmax(const DeviceTensorParams& a, const DeviceTensorParams& result)
+{
+    if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmax supports only int32 data type for its result.");
+    requireDevice(result, "argmax");
+    flushFor(a.data, result.data);
+    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "argmax"); toPod(result, &pr, "argmax");
+    check(aixk_reduce_all(m_ctx, AIXK_ARGMAX, &pa, &pr));
+}
+
+void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorParams& result)
+{
+    if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndices supports only int32 data type for its result.");
+    requireDevice(result, "argmaxIndices");
+    flushFor(a.data, result.data);
+    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "argmaxIndices"); toPod(result, &pr, "argmaxIndices");
+    check(aixk_reduce_all(m_ctx, AIXK_ARGMAX_ONEHOT, &pa, &pr));
+}
+
+void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& result)
+{
+    requireDevice(result, "matmul");
+    flushFor(a.data, b.data, result.data);
+    aixhip_tensor pa, pb, pr; toPod(onDevice(a), &pa, "matmul"); toPod(onDevice(b), &pb, "matmul"); toPod(result, &pr, "matmul");
+    check(aixk_matmul(m_ctx, &pa, &pb, &pr));
+}
+
+void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)
+{
+    requireDevice(result, "transpose");
+    flushFor(a.data, result.data);
+    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "transpose"); toPod(result, &pr, "transpose");
+    check(aixk_transpose(m_ctx, &pa, &pr, dim0, dim1));
+}
+
+void DeviceHIP::copy(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size)
+{
+    if (size == 0) return;
+    if (!findBlock(dst)) throw std::invalid_argument("DeviceHIP::copy() result must have GPU memory.");        // aixDeviceMetal.cpp:714-715
+    flushFor(src, dst);
+    const size_t srcBytes = size * dataTypeSize(srcDType);
+    if (!findBlock(src)) {
+        if (srcDType == dstDType) { check(aixk_copy_in(m_ctx, dst, src, srcBytes)); return; }
+        src = stageRaw(src, srcBytes);
+    }
+    check(aixk_cast(m_ctx, src, (int)srcDType, dst, (int)dstDType, size));
+}
+
+void DeviceHIP::copyImmediate(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size)
+{
+    copy(src, srcDType, dst, dstDType, size);
+    synchronize();
+}
+
+void DeviceHIP::contiguous(const DeviceTensorParams& src, const DeviceTensorParams& dst)
+{
+    requireDevice(dst, "contiguous");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "contiguous"); toPod(dst, &pd, "contiguous");
+    check(aixk_contiguous(m_ctx, &ps, &pd));
+}
+
+void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
+{
+    if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::reduceTo() requires matching source and destination data types.");
+    requireDevice(dst, "reduceTo");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
+    check(aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));
+}
+
+void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
+{
+    if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::maxTo() requires matching source and destination data types.");
+    requireDevice(dst, "maxTo");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "maxTo"); toPod(dst, &pd, "maxTo");
+    check(aixk_reduce_to(m_ctx, AIXK_MAX, &ps, &pd));
+}
+
+void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
+{
+    if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxTo supports only int32 data type for its result.");
+    requireDevice(dst, "argmaxTo");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "argmaxTo"); toPod(dst, &pd, "argmaxTo");
+    check(aixk_argmax_to(m_ctx, 0, &ps, &pd, dim));
+}
+
+void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
+{
+    if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndicesTo supports only int32 data type for its result.");
+    requireDevice(dst, "argmaxIndicesTo");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "argmaxIndicesTo"); toPod(dst, &pd, "argmaxIndicesTo");
+    check(aixk_argmax_to(m_ctx, 1, &ps, &pd, dim));
+}
+
+void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim, size_t start, size_t end, size_t step)
+{
+    if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::sliceSet() requires matching source and destination data types.");
+    requireDevice(dst, "sliceSet");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "sliceSet"); toPod(dst, &pd, "sliceSet");
+    check(aixk_slice_set(m_ctx, &ps, &pd, dim, start, end, step));
+}
+
+void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
+{
+    if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::tril() requires matching source and destination data types.");   // aixDeviceMetal.cpp:1160-1161
+    requireDevice(dst, "tril");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "tril"); toPod(dst, &pd, "tril");
+    check(aixk_tri(m_ctx, 0, &ps, &pd, diagonal));
+}
+
+void DeviceHIP::triu(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
+{
+    if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::triu() requires matching source and destination data types.");
+    requireDevice(dst, "triu");
+    flushFor(src.data, dst.data);
+    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "triu"); toPod(dst, &pd, "triu");
+    check(aixk_tri(m_ctx, 1, &ps, &pd, diagonal));
+}
+
+void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
+{
+    requireDevice(dst, "indexSelect");
+    flushFor(src.data, dst.data, indices.data);
+    aixhip_tensor ps, pd, pi; toPod(onDevice(src), &ps, "indexSelect"); toPod(dst, &pd, "indexSelect"); toPod(onDevice(indices), &pi, "indexSelect");
+    check(aixk_index_select(m_ctx, &ps, &pd, &pi, dim));
+}
+
+void DeviceHIP::indexAdd(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
+{
+    requireDevice(dst, "indexAdd");
+    flushFor(src.data, dst.data, indices.data);
+    aixhip_tensor ps, pd, pi; toPod(onDevice(src), &ps, "indexAdd"); toPod(dst, &pd, "indexAdd"); toPod(onDevice(indices), &pi, "indexAdd");
+    check(aixk_index_add(m_ctx, &ps, &pd, &pi, dim));
+}
+
+} // namespace hip
+} // namespace aix

@@ -1,0 +1,140 @@
+// device_hip.hpp -- aix::Device for one AMD Instinct MI355X (gfx950).
+//
+// Implements the same pure-virtual operator interface the reference's GPU device implements
+// (Targets/AIXLib/aixDevice.hpp:30-84; behavioural template Targets/AIXLib/aixDeviceMetal.cpp), so
+// tensors, autograd, optimizers and examples written against aix::Device run unchanged:
+//
+//     aix::hip::DeviceHIP device;                 // or aix::hip::createDeviceHIP(0)
+//     auto x = aix::tensor(..., { .m_device = &device });
+//
+// Host C++ only: the GPU is reached exclusively through the C ABI of libaixhip_kernels.so
+// (include/aixhip_kernels.h).
+//
+// Execution model
+//   * elementwise operators and fills are RECORDED (fuse.hpp) and run as runtime-compiled fused
+//     kernels at the next flush; every other operator flushes and is enqueued at once;
+//   * everything runs on one in-order stream; results are defined after synchronize();
+//   * allocate() returns device memory that the host can dereference (large-BAR mapping): host
+//     writes are fast, host reads are slow and meant for scalars / debugging / small tensors;
+//   * deallocate() is deferred until the recorded work that may use the block has been enqueued;
+//     blocks are then reused from size buckets;
+//   * input operands may be host pointers (they are staged); results must be this device's memory,
+//     otherwise std::invalid_argument, as on the reference GPU device (aixDeviceMetal.cpp:305-306).
+#pragma once
+
+#include "aix_compat.hpp"
+#include "fuse.hpp"
+
+#include <map>
+#include <memory>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+struct aixk_ctx;
+struct aixhip_tensor;
+
+namespace aix::hip {
+
+class DeviceHIP : public aix::Device {
+public:
+    explicit DeviceHIP(size_t deviceIndex = 0);
+    ~DeviceHIP() override;
+    DeviceHIP(const DeviceHIP&) = delete;
+    DeviceHIP& operator=(const DeviceHIP&) = delete;
+
+    DeviceType type() const override { return aix::kDeviceTypeHIP; }
+    std::string name() const override { return "HIP"; }
+
+    void* allocate(size_t size) override;
+    void* allocate(size_t size, DataType dtype) override;
+    void deallocate(void* memory) override;
+
+    void add(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) override;
+    void sub(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) override;
+    void mul(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) override;
+    void div(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) override;
+    void unary(const DeviceTensorParams& a1, const DeviceTensorParams& result) override;
+
+    void fill(const void* scalar, DataType scalarDType, const DeviceTensorParams& result) override;
+    void fillMin(const DeviceTensorParams& result) override;
+    void sum(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void sqrt(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void sin(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void cos(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void tanh(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void log(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void exp(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void pow(const DeviceTensorParams& a, const DeviceTensorParams& exp, const DeviceTensorParams& result) override;
+    void max(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void argmax(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void argmaxIndices(const DeviceTensorParams& a, const DeviceTensorParams& result) override;
+    void matmul(const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& result) override;
+    void transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1) override;
+
+    void copy(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size) override;
+    void copyImmediate(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size) override;
+    void contiguous(const DeviceTensorParams& src, const DeviceTensorParams& dst) override;
+    void reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst) override;
+    void maxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst) override;
+    void argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim) override;
+    void argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim) override;
+    void sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst,
+                  size_t dim, size_t start, size_t end, size_t step) override;
+    void tril(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal) override;
+    void triu(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal) override;
+    void indexSelect(const DeviceTensorParams& src, const DeviceTensorParams& dst,
+                     const DeviceTensorParams& indices, size_t dim) override;
+    void indexAdd(const DeviceTensorParams& src, const DeviceTensorParams& dst,
+                  const DeviceTensorParams& indices, size_t dim) override;
+
+    void emptyCache() override;
+    void synchronize() override;
+
+    // ---- beyond the interface -------------------------------------------------------------------
+    // Explicit transfers for hosts that should not read device memory through the BAR mapping.
+    void copyToHost(void* dstHost, const void* srcDevice, size_t bytes);     // flushes and waits
+    void copyFromHost(void* dstDevice, const void* srcHost, size_t bytes);   // stream ordered
+    bool isDeviceMemory(const void* p) const { return findBlock(p) != nullptr; }
+
+    void setFuseConfig(const aixhip::fuse::FuseConfig& cfg);                  // flushes first
+    const aixhip::fuse::FuseConfig& fuseConfig() const { return m_engine->config(); }
+    const aixhip::fuse::FlushDiagnostics& lastFlushDiagnostics() const { return m_engine->lastFlushDiagnostics(); }
+    std::pair<size_t, size_t> fuseKernelCacheStats() const;                  // hits, misses (aixDeviceMetal's test hook)
+    void flush();                                                            // plan + enqueue, no wait
+    aixk_ctx* kernelContext() const { return m_ctx; }
+    size_t cachedBytes() const { return m_pooledBytes; }
+    size_t allocatedBytes() const { return m_liveBytes; }
+
+private:
+    struct Block { size_t bytes; };
+
+    const Block* findBlock(const void* p) const;
+    size_t bucketBytes(size_t bytes) const;
+    void* allocateBlock(size_t bytes, bool track);
+    void releaseLimbo();
+    void requireDevice(const DeviceTensorParams& result, const char* op) const;
+    // Returns params whose data is device memory: host operands are staged into a temporary block.
+    DeviceTensorParams onDevice(const DeviceTensorParams& p);
+    const void* stageRaw(const void* src, size_t bytes);
+    void toPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op) const;
+    void check(int status) const;
+    void recordBinary(aixhip::fuse::OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b,
+                      const DeviceTensorParams& r, const char* op);
+    void recordUnary(aixhip::fuse::OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op);
+    void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
+    void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);
+    void emitSingle(const aixhip::fuse::OpRecord& op);
+
+    aixk_ctx* m_ctx{nullptr};
+    std::unique_ptr<aixhip::fuse::FuseEngine> m_engine;
+    std::map<uintptr_t, Block> m_blocks;                       // live allocations by base address
+    std::unordered_map<size_t, std::vector<void*>> m_pool;     // free blocks by bucket size
+    std::vector<std::pair<void*, size_t>> m_limbo;             // freed, but recorded work may still use them
+    size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0};
+    int m_cus{256};
+};
+
+std::unique_ptr<aix::Device> createDeviceHIP(size_t deviceIndex = 0);   // nullptr if no GPU is visible
+
+} // namespace aix::hip

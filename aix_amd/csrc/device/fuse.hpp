@@ -1,0 +1,140 @@
+// fuse.hpp -- the lazy elementwise planner behind DeviceHIP.
+//
+// Same role and the same public surface as the reference's device-agnostic fusion engine
+// (Targets/AIXLib/aixFuse.hpp:29-217): a device records elementwise operators and fills instead of
+// running them; flush() turns the recorded window into fused multi-output kernels plus ordered
+// single operators and hands them to the device through callbacks.  The planning algorithm itself
+// is different (see fuse.cpp): a single pass in program order that grows several open groups at
+// once under explicit read/write hazard rules, treats every fill as a lazily materialised scalar,
+// and classifies contiguity over the buffers that are really loaded or stored -- so an expression
+// such as  tanh(a*b + c) / (1 + exp(-a)) - 0.5*c  becomes ONE dense kernel with three 16-byte
+// loads, one 16-byte store and two immediates per lane group.
+#pragma once
+
+#include "aix_compat.hpp"
+
+#include <cstdint>
+#include <functional>
+#include <optional>
+#include <string>
+#include <unordered_map>
+#include <unordered_set>
+#include <utility>
+#include <vector>
+
+namespace aixhip::fuse {
+
+using aix::DataType;
+using aix::DeviceTensorParams;
+
+// Operator codes; the elementwise ones are the recordable set (aixFuse.hpp:29-88).
+enum class OpType {
+    Add, Sub, Mul, Div, Negate, Sqrt, Sin, Cos, Tanh, Log, Exp, Pow, Fill, FillMin, Cast,
+    Sum, Max, Argmax, ArgmaxIndices, Matmul, Transpose, Copy, Contiguous, ReduceTo, MaxTo,
+    ArgmaxTo, ArgmaxIndicesTo, SliceSet, Tril, Triu, IndexSelect, IndexAdd,
+};
+
+bool isElementwiseOp(OpType t);
+const char* opName(OpType t);
+
+struct FuseConfig {
+    bool   elementwiseFusion     = true;
+    bool   multiOutputKernels    = true;   // let independent ops that share an input join one kernel
+    bool   absorbFills           = true;   // fills feed consumers as immediates and run only if needed
+    bool   diagnostics           = false;
+    size_t flushThreshold        = 200;    // recorded ops that trigger planning
+    size_t maxBufferSlots        = 0;      // pointer arguments one fused kernel may take (must be > 0)
+    bool   supportsStridedFusion = true;   // may fused kernels read broadcast / strided views
+};
+
+struct OpRecord {
+    OpType type{OpType::Add};
+    DeviceTensorParams input0;
+    DeviceTensorParams input1;
+    DeviceTensorParams output;
+    std::vector<uint8_t> scalarData;       // Fill: the scalar in scalarDType
+    DataType scalarDType = DataType::kFloat32;
+    bool hasInput1 = false;
+};
+
+// One fused kernel: ops in execution order.  An operand index below inputBuffers.size() names an
+// external buffer, an index at or above it names the result of ops[index - inputBuffers.size()];
+// SIZE_MAX means "not a tensor" (then the scalar index applies).  scalarData holds the immediates
+// already converted to `dtype`.
+struct FusedSubgraphDescriptor {
+    struct Op {
+        OpType type;
+        size_t inputIndex0  = SIZE_MAX;
+        size_t inputIndex1  = SIZE_MAX;
+        size_t outputIndex  = SIZE_MAX;    // into outputBuffers; SIZE_MAX = value stays in registers
+        size_t scalarIndex0 = SIZE_MAX;
+        size_t scalarIndex1 = SIZE_MAX;
+    };
+    std::vector<Op> ops;
+    std::vector<DeviceTensorParams> inputBuffers;
+    std::vector<DeviceTensorParams> outputBuffers;
+    std::vector<uint8_t> scalarData;
+    DataType dtype{DataType::kFloat32};
+    bool     allContiguous{true};          // every loaded / stored view is dense
+    size_t   elementCount{0};
+    aix::Shape shape;                      // iteration shape (outputs are dense over it)
+};
+
+struct FlushDiagnostics {
+    size_t opsRecorded = 0;
+    size_t fusibleSubgraphs = 0;
+    size_t fusedOps = 0;
+    size_t fallbackOps = 0;
+    size_t dispatchesSaved = 0;
+    size_t fillsAbsorbed = 0;
+    size_t kernelCacheHits = 0;
+    size_t kernelCacheMisses = 0;
+    std::string subgraphSummary;
+    std::string fallbackSummary;
+};
+
+struct FuseCallbacks {
+    std::function<void(const FusedSubgraphDescriptor&)> emitFused;
+    std::function<void(const OpRecord&)> emitSingle;
+    std::function<void()> finishFlush;
+    std::function<std::pair<size_t, size_t>()> getKernelCacheStats = [] { return std::pair<size_t, size_t>{0, 0}; };
+};
+
+// Converts a scalar between element types with the device's conversion rules (saturating
+// float -> integer, NaN -> 0, 16-bit floats by way of float; aixDeviceCPU.cpp:96-117).
+std::vector<uint8_t> convertScalar(const void* scalar, DataType from, DataType to);
+std::vector<uint8_t> lowestScalar(DataType dtype);
+
+class FuseEngine {
+public:
+    FuseEngine(const FuseConfig& config, FuseCallbacks callbacks);
+
+    void record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& output);
+    void record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& input1,
+                const DeviceTensorParams& output);
+    void recordFill(const void* scalar, DataType scalarDType, const DeviceTensorParams& output);
+    void recordFillMin(const DeviceTensorParams& output);
+    void flush();
+
+    const FuseConfig& config() const { return m_config; }
+    const FlushDiagnostics& lastFlushDiagnostics() const;
+    size_t pendingOps() const { return m_pending.size(); }
+
+    void recordExternalRead(const void* buffer);   // the buffer is about to be read outside the planner
+    void retainBuffer(void* buffer);               // allocate(): results written here must reach memory
+    void releaseBuffer(void* buffer);              // deallocate(): nobody will read it after the window
+    void invalidateBuffer(void* buffer);
+
+private:
+    void maybeFlush();
+
+    FuseConfig m_config;
+    FuseCallbacks m_callbacks;
+    std::vector<OpRecord> m_pending;
+    std::unordered_set<const void*> m_live;
+    std::unordered_set<const void*> m_externalReads;
+    std::optional<FlushDiagnostics> m_diagnostics;
+    bool m_flushing{false};
+};
+
+} // namespace aixhip::fuse

@@ -1,0 +1,231 @@
+// hipgen.cpp -- HIP source generation for fused elementwise kernels (see hipgen.hpp).
+
+#include "hipgen.hpp"
+
+#include <array>
+#include <cstring>
+#include <sstream>
+#include <stdexcept>
+
+namespace aixhip::gen {
+
+using fuse::FusedSubgraphDescriptor;
+using fuse::OpType;
+
+namespace {
+
+const char* typeName(aix::DataType t)
+{
+    switch (t) {
+        case aix::DataType::kFloat64:  return "double";
+        case aix::DataType::kFloat32:  return "float";
+        case aix::DataType::kFloat16:  return "f16";
+        case aix::DataType::kBFloat16: return "bf16";
+        case aix::DataType::kInt64:    return "i64";
+        case aix::DataType::kInt32:    return "i32";
+        case aix::DataType::kInt16:    return "i16";
+        case aix::DataType::kInt8:     return "i8";
+        case aix::DataType::kUInt8:    return "u8";
+    }
+    return "float";
+}
+
+const char* shortType(aix::DataType t)
+{
+    static const char* n[] = {"f64", "f32", "f16", "bf16", "i64", "i32", "i16", "i8", "u8"};
+    return n[static_cast<size_t>(t)];
+}
+
+const char* wordName(size_t bytes) { return bytes == 1 ? "u8" : bytes == 2 ? "u16" : bytes == 4 ? "u32" : "u64"; }
+
+const char* fnName(OpType t)
+{
+    switch (t) {
+        case OpType::Add: return "e_add";   case OpType::Sub: return "e_sub";   case OpType::Mul: return "e_mul";
+        case OpType::Div: return "e_div";   case OpType::Pow: return "e_pow";   case OpType::Negate: return "e_neg";
+        case OpType::Sqrt: return "e_sqrt"; case OpType::Sin: return "e_sin";   case OpType::Cos: return "e_cos";
+        case OpType::Tanh: return "e_tanh"; case OpType::Log: return "e_log";   case OpType::Exp: return "e_exp";
+        default: throw std::invalid_argument(std::string("operator cannot be fused: ") + fuse::opName(t));
+    }
+}
+
+bool isBinary(OpType t) { return t == OpType::Add || t == OpType::Sub || t == OpType::Mul || t == OpType::Div || t == OpType::Pow; }
+
+size_t scalarCount(const FusedSubgraphDescriptor& d)
+{
+    return d.scalarData.size() / aix::Device::dataTypeSize(d.dtype);
+}
+
+std::string operandText(const FusedSubgraphDescriptor& d, size_t tensorIndex, size_t scalarIndex)
+{
+    if (tensorIndex != SIZE_MAX) {
+        if (tensorIndex < d.inputBuffers.size()) return "x[" + std::to_string(tensorIndex) + "]";
+        return "v" + std::to_string(tensorIndex - d.inputBuffers.size());
+    }
+    if (scalarIndex != SIZE_MAX) return "s[" + std::to_string(scalarIndex) + "]";
+    throw std::invalid_argument("fused operator without an operand");
+}
+
+// The per-element SSA body shared by the vector loop and the tails.
+void emitBody(std::ostringstream& o, const FusedSubgraphDescriptor& d)
+{
+    o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out)\n{\n";
+    for (size_t k = 0; k < d.ops.size(); ++k) {
+        const auto& op = d.ops[k];
+        o << "    const T v" << k << " = " << fnName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
+        if (isBinary(op.type)) o << ", " << operandText(d, op.inputIndex1, op.scalarIndex1);
+        o << ");\n";
+        if (op.outputIndex != SIZE_MAX) o << "    out[" << op.outputIndex << "] = v" << k << ";\n";
+    }
+    o << "}\n\n";
+}
+
+} // namespace
+
+int flatUnroll(size_t inputs) { return inputs <= 4 ? 4 : (inputs <= 8 ? 2 : 1); }
+
+std::string signature(const FusedSubgraphDescriptor& d, Shape shape)
+{
+    std::ostringstream s;
+    s << shortType(d.dtype) << (shape == Shape::Flat ? "|flat" : shape == Shape::Rows ? "|rows" : "|gather")
+      << "|i" << d.inputBuffers.size() << "o" << d.outputBuffers.size() << "s" << scalarCount(d);
+    for (const auto& op : d.ops) {
+        s << "|" << fuse::opName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
+        if (isBinary(op.type)) s << "," << operandText(d, op.inputIndex1, op.scalarIndex1);
+        s << ")";
+        if (op.outputIndex != SIZE_MAX) s << ">o" << op.outputIndex;
+    }
+    return s.str();
+}
+
+std::string source(const FusedSubgraphDescriptor& d, Shape shape)
+{
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
+    if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
+    const size_t esz = aix::Device::dataTypeSize(d.dtype);
+    const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
+    std::ostringstream o;
+    o << "#include \"aix_device.h\"\nusing namespace aixd;\n"
+      << "// " << signature(d, shape) << "\n"
+      << "typedef " << typeName(d.dtype) << " T;\n"
+      << "typedef " << wordName(esz) << " word_t;\n"
+      << "typedef vec16<T>::type V;\n"
+      << "#define VEC (vec16<T>::n)\n#define NI " << NI << "\n#define NO " << NO << "\n#define NS " << NS << "\n\n";
+    emitBody(o, d);
+
+    o << "struct Args {\n    const T* in[" << AI << "];\n    T* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 n;\n";
+    if (shape == Shape::Flat) o << "    u64 bmask;\n";
+    else o << "    u64 chunks;\n    u64 rank;\n    u64 shape[" << kMaxDims << "];\n    u64 off[" << AI << "];\n    u64 str[" << AI << "][" << kMaxDims << "];\n";
+    o << "};\n\n";
+
+    o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void aix_fused(Args a)\n{\n"
+      << "    T s[" << AS << "];\n";
+    for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
+    if (NS == 0) o << "    s[0] = zero<T>();\n";
+
+    if (shape == Shape::Flat) {
+        const int U = flatUnroll(NI);
+        o << "    T b[" << AI << "];\n";
+        for (size_t k = 0; k < NI; ++k) o << "    b[" << k << "] = ((a.bmask >> " << k << ") & 1) ? a.in[" << k << "][0] : zero<T>();\n";
+        if (NI == 0) o << "    b[0] = zero<T>();\n";
+        o << "    const u64 nvec = a.n / VEC;\n"
+          << "    const u64 tile = (u64)" << kBlock << " * " << U << ";\n"
+          << "    for (u64 v0 = (u64)blockIdx.x * tile; v0 < nvec; v0 += (u64)gridDim.x * tile) {\n";
+        for (size_t k = 0; k < NI; ++k) o << "        V r" << k << "[" << U << "];\n";
+        o << "#pragma unroll\n        for (int k = 0; k < " << U << "; ++k) {\n"
+          << "            const u64 v = v0 + (u64)k * " << kBlock << " + threadIdx.x;\n            if (v < nvec) {\n";
+        for (size_t k = 0; k < NI; ++k)
+            o << "                if (!((a.bmask >> " << k << ") & 1)) r" << k << "[k] = ((const V*)a.in[" << k << "])[v];\n";
+        o << "            }\n        }\n"
+          << "#pragma unroll\n        for (int k = 0; k < " << U << "; ++k) {\n"
+          << "            const u64 v = v0 + (u64)k * " << kBlock << " + threadIdx.x;\n            if (v < nvec) {\n";
+        for (size_t k = 0; k < NO; ++k) o << "                V w" << k << ";\n";
+        o << "#pragma unroll\n                for (int e = 0; e < VEC; ++e) {\n                    T x[" << AI << "], y[" << NO << "];\n";
+        for (size_t k = 0; k < NI; ++k)
+            o << "                    x[" << k << "] = ((a.bmask >> " << k << ") & 1) ? b[" << k << "] : r" << k << "[k].v[e];\n";
+        if (NI == 0) o << "                    x[0] = b[0];\n";
+        o << "                    aix_body(x, s, y);\n";
+        for (size_t k = 0; k < NO; ++k) o << "                    w" << k << ".v[e] = y[" << k << "];\n";
+        o << "                }\n";
+        for (size_t k = 0; k < NO; ++k) o << "                ((V*)a.out[" << k << "])[v] = w" << k << ";\n";
+        o << "            }\n        }\n    }\n"
+          << "    const u64 done = nvec * VEC;\n"
+          << "    if (blockIdx.x == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
+        for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = ((a.bmask >> " << k << ") & 1) ? b[" << k << "] : a.in[" << k << "][i];\n";
+        if (NI == 0) o << "        x[0] = b[0];\n";
+        o << "        aix_body(x, s, y);\n";
+        for (size_t k = 0; k < NO; ++k) o << "        a.out[" << k << "][i] = y[" << k << "];\n";
+        o << "    }\n}\n";
+        return o.str();
+    }
+
+    if (shape == Shape::Rows) {
+        o << "    const int inner = (int)a.rank - 1;\n"
+          << "    const u64 total = a.n / VEC;\n"
+          << "    for (u64 c = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; c < total; c += (u64)gridDim.x * " << kBlock << ") {\n"
+          << "        u64 row = c / a.chunks;\n        const u64 col = (c - row * a.chunks) * VEC;\n"
+          << "        u64 p[" << AI << "];\n";
+        for (size_t k = 0; k < NI; ++k) o << "        p[" << k << "] = a.off[" << k << "];\n";
+        o << "        for (int d = inner - 1; d >= 0; --d) {\n            const u64 q = row / a.shape[d], r = row - q * a.shape[d];\n";
+        for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
+        o << "            row = q;\n        }\n";
+        for (size_t k = 0; k < NI; ++k) {
+            o << "        V r" << k << ";\n"
+              << "        if (a.str[" << k << "][inner] == 0) { const T t = a.in[" << k << "][p[" << k << "]];\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r" << k << ".v[e] = t; }\n"
+              << "        else r" << k << " = *(const V*)(a.in[" << k << "] + p[" << k << "] + col);\n";
+        }
+        for (size_t k = 0; k < NO; ++k) o << "        V w" << k << ";\n";
+        o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
+        for (size_t k = 0; k < NI; ++k) o << "            x[" << k << "] = r" << k << ".v[e];\n";
+        if (NI == 0) o << "            x[0] = zero<T>();\n";
+        o << "            aix_body(x, s, y);\n";
+        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = y[" << k << "];\n";
+        o << "        }\n";
+        for (size_t k = 0; k < NO; ++k) o << "        *(V*)(a.out[" << k << "] + c * VEC) = w" << k << ";\n";
+        o << "    }\n}\n";
+        return o.str();
+    }
+
+    // gather
+    o << "    for (u64 i = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; i < a.n; i += (u64)gridDim.x * " << kBlock << ") {\n"
+      << "        u64 rest = i;\n        u64 p[" << AI << "];\n";
+    for (size_t k = 0; k < NI; ++k) o << "        p[" << k << "] = a.off[" << k << "];\n";
+    o << "        for (int d = (int)a.rank - 1; d >= 0; --d) {\n            const u64 q = rest / a.shape[d], r = rest - q * a.shape[d];\n";
+    for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
+    o << "            rest = q;\n        }\n        T x[" << AI << "], y[" << NO << "];\n";
+    for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = a.in[" << k << "][p[" << k << "]];\n";
+    if (NI == 0) o << "        x[0] = zero<T>();\n";
+    o << "        aix_body(x, s, y);\n";
+    for (size_t k = 0; k < NO; ++k) o << "        a.out[" << k << "][i] = y[" << k << "];\n";
+    o << "    }\n}\n";
+    return o.str();
+}
+
+std::vector<uint64_t> packArgs(const FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
+                               const std::vector<void*>& outputs, uint64_t n, uint32_t broadcastMask, const Space* space,
+                               uint64_t chunksPerRow)
+{
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
+    const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
+    const size_t esz = aix::Device::dataTypeSize(d.dtype);
+    std::vector<uint64_t> a;
+    for (size_t k = 0; k < AI; ++k) a.push_back(k < NI ? (uint64_t)(uintptr_t)inputs[k] : 0);
+    for (size_t k = 0; k < NO; ++k) a.push_back((uint64_t)(uintptr_t)outputs[k]);
+    for (size_t k = 0; k < AS; ++k) {
+        uint64_t bits = 0;
+        if (k < NS) std::memcpy(&bits, d.scalarData.data() + k * esz, esz);     // little endian: low bytes
+        a.push_back(bits);
+    }
+    a.push_back(n);
+    if (shape == Shape::Flat) { a.push_back(broadcastMask); return a; }
+    if (!space) throw std::invalid_argument("strided fused kernel without an iteration space");
+    a.push_back(chunksPerRow);
+    a.push_back(space->rank);
+    for (int dd = 0; dd < kMaxDims; ++dd) a.push_back(space->shape[dd]);
+    for (size_t k = 0; k < AI; ++k) a.push_back(k < NI ? space->offset[k] : 0);
+    for (size_t k = 0; k < AI; ++k)
+        for (int dd = 0; dd < kMaxDims; ++dd) a.push_back(k < NI ? space->stride[k][dd] : 0);
+    return a;
+}
+
+} // namespace aixhip::gen

@@ -1,0 +1,51 @@
+// hipgen.hpp -- turns a fused-subgraph descriptor into HIP C++ source for hipRTC.
+//
+// Replaces the reference's runtime Metal-source generator
+// (Targets/AIXLib/aixDeviceMetalKernelGen.cpp:464-710): same input (a FusedSubgraphDescriptor),
+// same idea (one SSA statement per operator, external inputs loaded once, immediates as kernel
+// arguments so their VALUES never force a recompile), but the emitted text is HIP for gfx950
+// built on the per-element operators of aix_device.h, in one of three launch shapes:
+//   flat    every view dense and 16-byte aligned: 16-byte loads/stores, several in flight;
+//   rows    the innermost dim is dense-or-broadcast for every view: one 16-byte chunk per lane;
+//   gather  any strided view: one element per lane.
+#pragma once
+
+#include "fuse.hpp"
+
+#include <array>
+#include <string>
+#include <vector>
+
+namespace aixhip::gen {
+
+enum class Shape { Flat, Rows, Gather };
+
+// Identity of a generated kernel: element type, launch shape, operator wiring.  Immediates'
+// values, pointers, sizes and strides are arguments and not part of it.
+std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape);
+
+// Source of `extern "C" __global__ void aix_fused(Args)`.
+std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape);
+
+inline const char* entryName() { return "aix_fused"; }
+
+// How many 16-byte vectors per input a lane keeps in flight in the flat shape.
+int flatUnroll(size_t inputs);
+
+constexpr int kMaxDims = 8;
+constexpr int kBlock = 256;
+
+// The iteration space handed to rows / gather kernels.
+struct Space {
+    uint32_t rank{0};
+    uint64_t shape[kMaxDims]{};
+    std::vector<uint64_t> offset;                 // per buffer (inputs then outputs)
+    std::vector<std::array<uint64_t, kMaxDims>> stride;
+};
+
+// Kernel-argument block in the exact layout of the generated `struct Args`.
+std::vector<uint64_t> packArgs(const fuse::FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
+                               const std::vector<void*>& outputs, uint64_t n, uint32_t broadcastMask, const Space* space,
+                               uint64_t chunksPerRow);
+
+} // namespace aixhip::gen

@@ -170,7 +170,7 @@ enum { M_SQRT = 1, M_SIN = 2, M_COS = 3, M_TANH = 4, M_LOG = 5, M_EXP = 6 };
 
 template <int F> __device__ __forceinline__ float math_f32(float x)
 {
-    if constexpr (F == M_SQRT) return __builtin_sqrtf(x);
+    if constexpr (F == M_SQRT) return sqrtf(x);
     else if constexpr (F == M_SIN) return sinf(x);
     else if constexpr (F == M_COS) return cosf(x);
     else if constexpr (F == M_TANH) return tanhf(x);
@@ -179,7 +179,16 @@ template <int F> __device__ __forceinline__ float math_f32(float x)
 }
 template <int F> __device__ __forceinline__ double math_f64(double x)
 {
-    if constexpr (F == M_SQRT) return __builtin_sqrt(x);
+    if constexpr (F == M_SQRT) {
+        // The library routine can be one unit off; one Newton step on the exact residual
+        // (fused multiply-add) makes the result correctly rounded, as the CPU's is.
+        double y = sqrt(x);
+        if (x > 0.0 && x < __builtin_huge_val()) {
+            const double r = __builtin_fma(-y, y, x);
+            y = __builtin_fma(r, 0.5 / y, y);
+        }
+        return y;
+    }
     else if constexpr (F == M_SIN) return sin(x);
     else if constexpr (F == M_COS) return cos(x);
     else if constexpr (F == M_TANH) return tanh(x);

@@ -291,6 +291,16 @@ int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev)
     return AIXK_OK;
 }
 
+int32_t aixk_event_query(aixk_ctx* ctx, aixk_event* ev, int32_t* done)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(ev && done, "event_query: null argument");
+    const hipError_t e = hipEventQuery(ev->ev);
+    if (e == hipSuccess) { *done = 1; return AIXK_OK; }
+    if (e == hipErrorNotReady) { (void)hipGetLastError(); *done = 0; return AIXK_OK; }
+    return fail(AIXK_EHIP, "hipEventQuery: %s", hipGetErrorString(e));
+}
+
 int32_t aixk_event_elapsed_ms(aixk_ctx* ctx, aixk_event* start, aixk_event* stop, float* ms)
 {
     AIXK_TRY(set_device(ctx));

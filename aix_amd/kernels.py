@@ -64,6 +64,7 @@ _SIGNATURES = {
     "aixk_rtc_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "aixk_event_create": [_P, C.POINTER(_P)],
     "aixk_event_record": [_P, _P],
+    "aixk_event_query": [_P, _P, C.POINTER(C.c_int32)],
     "aixk_event_elapsed_ms": [_P, _P, _P, C.POINTER(C.c_float)],
     "aixk_event_destroy": [_P, _P],
 }

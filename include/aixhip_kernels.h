@@ -148,6 +148,7 @@ int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);
 /* ---- timing on the context's stream ------------------------------------- */
 int32_t aixk_event_create(aixk_ctx* ctx, aixk_event** out);
 int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev);
+int32_t aixk_event_query(aixk_ctx* ctx, aixk_event* ev, int32_t* done);              /* never waits */
 int32_t aixk_event_elapsed_ms(aixk_ctx* ctx, aixk_event* start, aixk_event* stop, float* ms); /* waits for stop */
 int32_t aixk_event_destroy(aixk_ctx* ctx, aixk_event* ev);
 

@@ -1,0 +1,387 @@
+// test_planner.cpp -- the fusion planner and the HIP source generator, without a GPU.
+//
+// Pattern of the reference's planner tests (Targets/AIXTests/DeviceTests.cpp:235-289,
+// 1810-1879): drive the engine with fake callbacks that capture what it emits, and check the
+// descriptors.  Additionally every generated kernel source is compiled with hipRTC for gfx950
+// (cross-compilation needs no GPU), so a generator bug fails here, not on the GPU box.
+//
+// Prints one line per check and exits non-zero if any failed.
+
+#include "device/fuse.hpp"
+#include "device/hipgen.hpp"
+
+#include <hip/hiprtc.h>
+
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+#include <string>
+#include <vector>
+
+using namespace aixhip::fuse;
+namespace gen = aixhip::gen;
+using aix::DataType;
+using aix::DeviceTensorParams;
+
+namespace aix {
+Device::~Device() = default;
+size_t Device::dataTypeSize(DataType dtype)
+{
+    static const size_t bytes[DataTypeCount] = {8, 4, 2, 2, 8, 4, 2, 1, 1};
+    return bytes[static_cast<size_t>(dtype)];
+}
+} // namespace aix
+
+static int g_failed = 0;
+static std::string g_prelude;
+
+#define CHECK(cond)                                                                    \
+    do {                                                                               \
+        if (!(cond)) { std::printf("FAIL %s:%d  %s\n", __FILE__, __LINE__, #cond); ++g_failed; } \
+    } while (0)
+
+static DeviceTensorParams T(uintptr_t id, aix::Shape shape, DataType dt = DataType::kFloat32, aix::Stride strides = {}, size_t offset = 0)
+{
+    DeviceTensorParams p;
+    p.data = reinterpret_cast<void*>(id * 0x10000);
+    p.dtype = dt;
+    p.shape = shape;
+    p.offset = offset;
+    size_t n = 1;
+    for (auto e : shape) n *= e;
+    p.size = n;
+    if (strides.empty()) { strides.resize(shape.size()); size_t run = 1; for (size_t d = shape.size(); d-- > 0;) { strides[d] = run; run *= shape[d]; } }
+    p.strides = strides;
+    bool dense = true; size_t run = 1;
+    for (size_t d = shape.size(); d-- > 0;) { if (strides[d] != run) dense = false; run *= shape[d]; }
+    p.isContiguous = dense;
+    return p;
+}
+
+struct Capture {
+    std::vector<FusedSubgraphDescriptor> fused;
+    std::vector<OpRecord> singles;
+    std::vector<std::string> order;           // "F<k>" or "S:<Op>"
+    int finishes = 0;
+    FuseCallbacks callbacks()
+    {
+        FuseCallbacks cb;
+        cb.emitFused = [this](const FusedSubgraphDescriptor& d) { order.push_back("F" + std::to_string(fused.size())); fused.push_back(d); };
+        cb.emitSingle = [this](const OpRecord& op) { order.push_back(std::string("S:") + opName(op.type)); singles.push_back(op); };
+        cb.finishFlush = [this] { ++finishes; };
+        return cb;
+    }
+};
+
+static FuseConfig config(bool fusion = true)
+{
+    FuseConfig c;
+    c.maxBufferSlots = 24;
+    c.diagnostics = true;
+    c.elementwiseFusion = fusion;
+    return c;
+}
+
+// Compiles one generated kernel for gfx950; returns true on success.
+static bool compiles(const FusedSubgraphDescriptor& d, gen::Shape shape)
+{
+    const std::string src = gen::source(d, shape);
+    hiprtcProgram prog;
+    const char* names[] = {"aix_device.h"};
+    const char* texts[] = {g_prelude.c_str()};
+    if (hiprtcCreateProgram(&prog, src.c_str(), "t.hip", 1, texts, names) != HIPRTC_SUCCESS) return false;
+    const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off"};
+    const hiprtcResult r = hiprtcCompileProgram(prog, 4, opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0; hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, 0); if (n) hiprtcGetProgramLog(prog, &log[0]);
+        std::printf("---- hipRTC log ----\n%s\n---- source ----\n%s\n", log.c_str(), src.c_str());
+    }
+    hiprtcDestroyProgram(&prog);
+    return r == HIPRTC_SUCCESS;
+}
+
+static float scalarAt(const FusedSubgraphDescriptor& d, size_t k) { float v; std::memcpy(&v, d.scalarData.data() + 4 * k, 4); return v; }
+
+// tanh(a*b + c) / (1 + exp(-a)) - 0.5*c with every temporary released before the flush.
+static void recordChain(FuseEngine& e, float one, float half, bool releaseTemps, const aix::Shape& shape = {4096, 4096})
+{
+    auto a = T(1, shape), b = T(2, shape), c = T(3, shape), y = T(20, shape);
+    auto t = [&](uintptr_t k) { return T(10 + k, shape); };
+    for (uintptr_t id : {1, 2, 3, 20, 11, 12, 13, 14, 15, 16, 17, 18, 30, 31}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Mul, a, b, t(1));
+    e.record(OpType::Add, t(1), c, t(2));
+    e.record(OpType::Tanh, t(2), t(3));
+    e.record(OpType::Negate, a, t(4));
+    e.record(OpType::Exp, t(4), t(5));
+    auto s1 = T(30, {}), s2 = T(31, {});
+    e.recordFill(&one, DataType::kFloat32, s1);
+    aix::Stride zeros(shape.size(), 0);
+    auto s1b = T(30, shape, DataType::kFloat32, zeros), s2b = T(31, shape, DataType::kFloat32, zeros);
+    e.record(OpType::Add, s1b, t(5), t(6));
+    e.record(OpType::Div, t(3), t(6), t(7));
+    e.recordFill(&half, DataType::kFloat32, s2);
+    e.record(OpType::Mul, s2b, c, t(8));
+    e.record(OpType::Sub, t(7), t(8), y);
+    if (releaseTemps)
+        for (uintptr_t id : {11, 12, 13, 14, 15, 16, 17, 18, 30, 31}) e.releaseBuffer(reinterpret_cast<void*>(id * 0x10000));
+}
+
+static void testChainBecomesOneDenseKernel()
+{
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    recordChain(e, 1.0f, 0.5f, true);
+    CHECK(e.pendingOps() == 11);
+    e.flush();
+    CHECK(cap.finishes == 1);
+    CHECK(cap.singles.empty());
+    CHECK(cap.fused.size() == 1);
+    if (cap.fused.size() != 1) return;
+    const auto& d = cap.fused[0];
+    CHECK(d.ops.size() == 9);                      // the two fills became immediates
+    CHECK(d.inputBuffers.size() == 3);             // a, b, c: each loaded once
+    CHECK(d.outputBuffers.size() == 1);            // only y reaches memory
+    CHECK(d.scalarData.size() == 8);
+    CHECK(scalarAt(d, 0) == 1.0f && scalarAt(d, 1) == 0.5f);
+    CHECK(d.allContiguous);                        // contiguity is judged on materialised buffers only
+    CHECK(d.elementCount == 4096u * 4096u);
+    CHECK(d.dtype == DataType::kFloat32);
+    const auto& diag = e.lastFlushDiagnostics();
+    CHECK(diag.opsRecorded == 11 && diag.fusibleSubgraphs == 1 && diag.fusedOps == 9 && diag.fallbackOps == 0);
+    CHECK(diag.fillsAbsorbed == 2 && diag.dispatchesSaved == 8);
+    CHECK(compiles(d, gen::Shape::Flat));
+    CHECK(compiles(d, gen::Shape::Rows));
+    CHECK(compiles(d, gen::Shape::Gather));
+    // immediates' values are arguments: another value, same kernel identity (DeviceTests.cpp:1774-1807)
+    Capture cap2;
+    FuseEngine e2(config(), cap2.callbacks());
+    recordChain(e2, 1.0f, 0.25f, true);
+    e2.flush();
+    CHECK(cap2.fused.size() == 1);
+    if (cap2.fused.size() == 1) {
+        CHECK(gen::signature(cap2.fused[0], gen::Shape::Flat) == gen::signature(d, gen::Shape::Flat));
+        CHECK(scalarAt(cap2.fused[0], 1) == 0.25f);
+        CHECK(gen::signature(d, gen::Shape::Flat) != gen::signature(d, gen::Shape::Gather));
+    }
+}
+
+static void testLiveTemporariesAreStoredAndFillsRun()
+{
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    recordChain(e, 1.0f, 0.5f, false, {64, 64});
+    e.flush();
+    CHECK(cap.fused.size() == 1);
+    if (cap.fused.size() != 1) return;
+    CHECK(cap.fused[0].outputBuffers.size() == 9);             // t1..t8 and y
+    CHECK(cap.singles.size() == 2);                            // the two scalar tensors are alive: their fills run
+    for (const auto& s : cap.singles) CHECK(s.type == OpType::Fill);
+    CHECK(compiles(cap.fused[0], gen::Shape::Flat));
+}
+
+static void testFusionDisabledReplaysInOrder()
+{
+    Capture cap;
+    FuseEngine e(config(false), cap.callbacks());
+    recordChain(e, 1.0f, 0.5f, true, {8, 8});
+    e.flush();
+    CHECK(cap.fused.empty());
+    CHECK(cap.singles.size() == 11);
+    const OpType want[] = {OpType::Mul, OpType::Add, OpType::Tanh, OpType::Negate, OpType::Exp, OpType::Fill, OpType::Add,
+                           OpType::Div, OpType::Fill, OpType::Mul, OpType::Sub};
+    for (size_t k = 0; k < cap.singles.size() && k < 11; ++k) CHECK(cap.singles[k].type == want[k]);
+}
+
+static void testInPlaceUpdatesKeepProgramOrder()
+{
+    // x = a + b; x += c; x *= x; y = x - a      (in-place: result aliases operand 0, DeviceTests.cpp:1882-1910)
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    aix::Shape s{1000};
+    auto a = T(1, s), b = T(2, s), c = T(3, s), x = T(4, s), y = T(5, s);
+    for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Add, a, b, x);
+    e.record(OpType::Add, x, c, x);
+    e.record(OpType::Mul, x, x, x);
+    e.record(OpType::Sub, x, a, y);
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() != 1) return;
+    const auto& d = cap.fused[0];
+    CHECK(d.ops.size() == 4);
+    CHECK(d.inputBuffers.size() == 3);
+    CHECK(d.outputBuffers.size() == 2);                        // final x and y; earlier values of x never stored
+    size_t stores = 0;
+    for (const auto& op : d.ops) if (op.outputIndex != SIZE_MAX) ++stores;
+    CHECK(stores == 2);
+    CHECK(d.ops[2].outputIndex != SIZE_MAX && d.ops[0].outputIndex == SIZE_MAX && d.ops[1].outputIndex == SIZE_MAX);
+    CHECK(d.ops[2].inputIndex0 == 3 + 1 && d.ops[2].inputIndex1 == 3 + 1);      // x*x reads the register value of op 1
+    CHECK(compiles(d, gen::Shape::Flat));
+}
+
+static void testDifferentViewOfAProducedBufferSplitsKernels()
+{
+    // t = a * b   [64, 32];   u = t^T (stride-swapped view) + c   [32, 64]
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto a = T(1, {64, 32}), b = T(2, {64, 32}), t = T(3, {64, 32}), c = T(4, {32, 64}), u = T(5, {32, 64});
+    auto tT = T(3, {32, 64}, DataType::kFloat32, {1, 32});
+    for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Mul, a, b, t);
+    e.record(OpType::Add, tT, c, u);
+    e.releaseBuffer(t.data);                                   // temporary, but the second op loads it
+    e.flush();
+    CHECK(cap.fused.empty());                                  // two kernels of one op each run as plain operators
+    CHECK(cap.singles.size() == 2);
+    if (cap.singles.size() == 2) { CHECK(cap.singles[0].type == OpType::Mul); CHECK(cap.singles[1].type == OpType::Add); }
+}
+
+static void testWriteAfterReadClosesTheReader()
+{
+    // u = a + b; v = u * u; then a is overwritten: a = c - c.  The kernel reading the old a must run first.
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    aix::Shape s{256};
+    auto a = T(1, s), b = T(2, s), c = T(3, s), u = T(4, s), v = T(5, s);
+    for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Add, a, b, u);
+    e.record(OpType::Mul, u, u, v);
+    e.record(OpType::Sub, c, c, a);
+    e.record(OpType::Negate, a, b);
+    e.flush();
+    CHECK(cap.order.size() == 2);
+    CHECK(cap.fused.size() == 2);
+    if (cap.fused.size() != 2) return;
+    CHECK(cap.fused[0].ops.size() == 2 && cap.fused[0].ops[0].type == OpType::Add);
+    CHECK(cap.fused[1].ops.size() == 2 && cap.fused[1].ops[0].type == OpType::Sub);
+    CHECK(compiles(cap.fused[1], gen::Shape::Flat));
+}
+
+static void testRowBroadcastStaysInOneKernel()
+{
+    // h = x + bias (bias broadcast along rows), r = tanh(h): what Linear + activation records
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto x = T(1, {128, 256}), bias = T(2, {128, 256}, DataType::kFloat32, {0, 1}), h = T(3, {128, 256}), r = T(4, {128, 256});
+    for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Add, x, bias, h);
+    e.record(OpType::Tanh, h, r);
+    e.releaseBuffer(h.data);
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() != 1) return;
+    CHECK(!cap.fused[0].allContiguous);
+    CHECK(cap.fused[0].outputBuffers.size() == 1);
+    CHECK(compiles(cap.fused[0], gen::Shape::Rows));
+    CHECK(compiles(cap.fused[0], gen::Shape::Gather));
+}
+
+static void testDeadCodeIsDropped()
+{
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto a = T(1, {10}), b = T(2, {10}), t = T(3, {10}), u = T(4, {10});
+    for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.record(OpType::Mul, a, b, t);
+    e.record(OpType::Exp, t, u);
+    e.releaseBuffer(t.data);
+    e.releaseBuffer(u.data);
+    e.flush();
+    CHECK(cap.order.empty());
+}
+
+static void testThresholdFlushAndExternalRead()
+{
+    Capture cap;
+    FuseConfig c = config();
+    c.flushThreshold = 4;
+    FuseEngine e(c, cap.callbacks());
+    auto a = T(1, {10}), t = T(2, {10});
+    e.retainBuffer(a.data);
+    e.record(OpType::Exp, a, t);            // t never retained: only an external read keeps it
+    e.record(OpType::Exp, t, t);
+    e.record(OpType::Exp, t, t);
+    CHECK(cap.finishes == 0);
+    e.recordExternalRead(t.data);
+    e.record(OpType::Exp, t, t);            // fourth op: planning runs by itself
+    CHECK(cap.finishes == 1);
+    CHECK(cap.fused.size() == 1);
+    if (cap.fused.size() == 1) CHECK(cap.fused[0].outputBuffers.size() == 1 && cap.fused[0].ops.size() == 4);
+}
+
+static void testFillMinAndIntegerScalars()
+{
+    // m = max-style init: fillMin(t); u = t + a  (int32): the immediate is INT_MIN; a float fill into an int8 tensor saturates
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto a = T(1, {100}, DataType::kInt32), t = T(2, {100}, DataType::kInt32), u = T(3, {100}, DataType::kInt32);
+    for (uintptr_t id : {1, 2, 3}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.recordFillMin(t);
+    e.record(OpType::Add, t, a, u);
+    e.releaseBuffer(t.data);
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() == 1) {
+        int32_t v; std::memcpy(&v, cap.fused[0].scalarData.data(), 4);
+        CHECK(v == INT32_MIN);
+        CHECK(compiles(cap.fused[0], gen::Shape::Flat));
+    }
+    const float big = 300.0f;
+    auto bytes = convertScalar(&big, DataType::kFloat32, DataType::kInt8);
+    CHECK(bytes.size() == 1 && (int8_t)bytes[0] == 127);
+    const float nan = __builtin_nanf("");
+    bytes = convertScalar(&nan, DataType::kFloat32, DataType::kInt32);
+    int32_t z; std::memcpy(&z, bytes.data(), 4);
+    CHECK(z == 0);
+    const float pi = 3.14f;
+    bytes = convertScalar(&pi, DataType::kFloat32, DataType::kFloat16);
+    uint16_t h; std::memcpy(&h, bytes.data(), 2);
+    CHECK(h == 0x4248);                                        // Float16Tests.cpp:25-31
+}
+
+static void testEveryTypeAndOperatorCompiles()
+{
+    const OpType unary[] = {OpType::Negate, OpType::Sqrt, OpType::Sin, OpType::Cos, OpType::Tanh, OpType::Log, OpType::Exp};
+    const OpType binary[] = {OpType::Add, OpType::Sub, OpType::Mul, OpType::Div, OpType::Pow};
+    for (size_t dt = 0; dt < aix::DataTypeCount; ++dt) {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        const DataType t = static_cast<DataType>(dt);
+        auto a = T(1, {50}, t), b = T(2, {50}, t);
+        e.retainBuffer(a.data); e.retainBuffer(b.data);
+        uintptr_t next = 3;
+        DeviceTensorParams cur = a;
+        for (OpType op : binary) { auto o = T(next++, {50}, t); e.record(op, cur, b, o); cur = o; }
+        for (OpType op : unary) { auto o = T(next++, {50}, t); e.record(op, cur, o); cur = o; }
+        e.retainBuffer(cur.data);
+        e.flush();
+        CHECK(cap.fused.size() == 1);
+        if (cap.fused.size() == 1) { CHECK(cap.fused[0].ops.size() == 12); CHECK(compiles(cap.fused[0], gen::Shape::Flat)); }
+    }
+}
+
+int main(int argc, char** argv)
+{
+    if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
+    std::ifstream f(argv[1]);
+    std::stringstream ss; ss << f.rdbuf();
+    g_prelude = ss.str();
+    if (g_prelude.empty()) { std::printf("cannot read %s\n", argv[1]); return 2; }
+
+    testChainBecomesOneDenseKernel();
+    testLiveTemporariesAreStoredAndFillsRun();
+    testFusionDisabledReplaysInOrder();
+    testInPlaceUpdatesKeepProgramOrder();
+    testDifferentViewOfAProducedBufferSplitsKernels();
+    testWriteAfterReadClosesTheReader();
+    testRowBroadcastStaysInOneKernel();
+    testDeadCodeIsDropped();
+    testThresholdFlushAndExternalRead();
+    testFillMinAndIntegerScalars();
+    testEveryTypeAndOperatorCompiles();
+    std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
+    return g_failed ? 1 : 0;
+}

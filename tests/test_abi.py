@@ -27,6 +27,22 @@ def test_kernel_library_exports_every_declared_symbol():
     assert sorted(K.EXPORTED) == names, "the Python binding must cover the header exactly"
 
 
+def test_device_library_exports_every_declared_symbol():
+    from aix_amd import device as D
+    names = declared("aixhip.h", "aixhip_")
+    assert len(names) >= 50
+    lib = D.load()
+    missing = [n for n in names if not hasattr(lib, n)]
+    assert not missing, missing
+    assert sorted(D.EXPORTED) == names, "the Python binding must cover the header exactly"
+    # one entry point per virtual of aix::Device (39 of them: type, name, 3 memory, 32 operators, emptyCache, synchronize)
+    virtuals = ["type", "name", "allocate", "allocate_typed", "deallocate", "add", "sub", "mul", "div", "unary", "fill",
+                "fill_min", "sum", "sqrt", "sin", "cos", "tanh", "log", "exp", "pow", "max", "argmax", "argmax_indices",
+                "matmul", "transpose", "copy", "copy_immediate", "contiguous", "reduce_to", "max_to", "argmax_to",
+                "argmax_indices_to", "slice_set", "tril", "triu", "index_select", "index_add", "empty_cache", "synchronize"]
+    assert len(virtuals) == 39 and all("aixhip_" + v in names for v in virtuals)
+
+
 def test_descriptor_layout_is_shared():
     assert C.sizeof(K.Tensor) == C.sizeof(O.TensorDesc) == 8 + 4 + 4 + 8 + 8 + 16 * 8 * 2
     for (n1, _), (n2, _) in zip(K.Tensor._fields_, O.TensorDesc._fields_):

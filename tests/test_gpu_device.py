@@ -1,0 +1,348 @@
+"""The lazy, fusing device (DeviceHIP behind include/aixhip.h) against the CPU oracle.
+
+These drive the device the way the AIX front-end does -- a fresh result allocation per operator,
+scalars as fills of rank-0 tensors read through stride-0 views, temporaries deallocated before
+synchronize() -- and check results, fusion diagnostics, error behaviour and memory handling.
+Patterns follow Targets/AIXTests/DeviceTests.cpp (queue tests :3074-3552, fusion tests :1774-1910).
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import aixtest as T
+import devharness as H
+import goldens
+from aix_amd import device as D
+from oracle import cpuref as O
+
+pytestmark = pytest.mark.gpu
+CPU = O.lib()
+NAMES = O.DTYPE_NAMES
+EPS32 = 2.0 ** -24
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = H.Dev()
+    yield d
+    d.close()
+
+
+def set_diag(dev, **kw):
+    cfg = dev.dev.fuse_config()
+    cfg.diagnostics = 1
+    for k, v in kw.items():
+        setattr(cfg, k, v)
+    dev.dev.set_fuse_config(cfg)
+
+
+class Recorder:
+    """Builds an expression on the device and, op for op, on the oracle."""
+
+    def __init__(self, dev, dtype, shape):
+        self.dev, self.dtype, self.shape = dev, dtype, list(shape)
+        self.n = O.numel(shape)
+        self.temps = []
+
+    def leaf(self, host):
+        p, d = self.dev.put(host)
+        return {"host": host, "ptr": p, "desc": d}
+
+    def _result(self):
+        host = T.empty(self.dtype, self.shape)
+        p = self.dev.raw(host.storage.nbytes)
+        node = {"host": host, "ptr": p, "desc": H.kdesc(host, p)}
+        self.temps.append(node)
+        return node
+
+    def binary(self, op, x, y):
+        r = self._result()
+        assert CPU.binary(op, C.byref(x["host"].desc()), C.byref(y["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call(["add", "sub", "mul", "div", "pow"][op], H.ref(x["desc"]), H.ref(y["desc"]), H.ref(r["desc"]))
+        return r
+
+    def unary(self, op, x):
+        r = self._result()
+        assert CPU.unary(op, C.byref(x["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call(["unary", "sqrt", "sin", "cos", "tanh", "log", "exp"][op], H.ref(x["desc"]), H.ref(r["desc"]))
+        return r
+
+    def scalar(self, value):
+        """Tensor-level scalar: a rank-0 tensor filled with the value, read through a stride-0 view
+        of the full shape (aixCore.hpp:2384-2388)."""
+        host0 = T.empty(self.dtype, [])
+        v = np.array([value], dtype=np.float32)
+        assert CPU.fill(v.ctypes.data, O.F32, C.byref(host0.desc())) == 0
+        p = self.dev.raw(host0.storage.nbytes)
+        self.dev.dev.call("fill", v.ctypes.data, O.F32, H.ref(H.kdesc(host0, p)))
+        view = T.HostTensor(host0.storage, self.dtype, self.shape, [0] * len(self.shape))
+        node = {"host": view, "ptr": p, "desc": H.kdesc(view, p)}
+        self.temps.append(node)
+        return node
+
+    def free_temps(self, keep=()):
+        for t in self.temps:
+            if not any(t is k for k in keep):
+                self.dev.free(t["ptr"])
+        self.temps = [t for t in self.temps if any(t is k for k in keep)]
+
+
+def build_config0(rec, a, b, c):
+    """y = tanh(a*b + c) / (1 + exp(-a)) - 0.5*c"""
+    t1 = rec.binary(O.MUL, a, b)
+    t2 = rec.binary(O.ADD, t1, c)
+    t3 = rec.unary(O.TANH, t2)
+    t4 = rec.unary(O.NEG, a)
+    t5 = rec.unary(O.EXP, t4)
+    t6 = rec.binary(O.ADD, rec.scalar(1.0), t5)
+    t7 = rec.binary(O.DIV, t3, t6)
+    t8 = rec.binary(O.MUL, rec.scalar(0.5), c)
+    y = rec.binary(O.SUB, t7, t8)
+    return y, t7
+
+
+def test_config0_chain_is_one_fused_kernel(dev):
+    set_diag(dev)
+    rng = np.random.default_rng(0)
+    shape = [1024, 1024]
+    rec = Recorder(dev, O.F32, shape)
+    a, b, c = (rec.leaf(T.contiguous_tensor(rng, O.F32, shape)) for _ in range(3))
+    y, t7 = build_config0(rec, a, b, c)
+    rec.free_temps(keep=(y,))
+    got = dev.fetch(y["ptr"], y["host"].storage)
+    diag = dev.dev.diagnostics()
+    assert diag.fusible_subgraphs == 1 and diag.fused_ops == 9 and diag.fallback_ops == 0, diag.subgraph_summary
+    assert diag.fills_absorbed == 2 and diag.ops_recorded == 11
+    # chain-level bound: tanh and exp may each differ by 2 ulp from the CPU's libm; the quotient
+    # carries that relative error and the final subtraction keeps it absolute.
+    want = y["host"].storage.astype(np.float64)
+    q = np.abs(t7["host"].storage.astype(np.float64))
+    err = np.abs(got.astype(np.float64) - want)
+    assert np.all(err <= 8 * EPS32 * (q + np.abs(want)) + 1e-30), float(err.max())
+    worst, hist = O.ulp_hist_f32(got, y["host"].storage)
+    print("config-0 chain ulp histogram vs CPU chain:", worst, hist[:8].tolist())
+    dev.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=lambda d: NAMES[d])
+def test_random_exact_expressions(dev, dtype):
+    """Random DAGs of exact operators (+ - * negate, scalars, broadcast rows, in-place updates) with
+    temporaries freed before the flush: must equal the op-by-op CPU evaluation bit for bit."""
+    set_diag(dev)
+    rng = np.random.default_rng(31000 + dtype)
+    for trial in range(12):
+        shape = [int(rng.integers(1, 40)), int(rng.integers(1, 70))]
+        rec = Recorder(dev, dtype, shape)
+        kw = dict(int_span=7) if dtype in T.INT_DTYPES else dict(lo=-2, hi=2)
+        nodes = [rec.leaf(T.contiguous_tensor(rng, dtype, shape, **kw)) for _ in range(3)]
+        row = T.HostTensor(T.random_values(rng, shape[1], dtype, **kw), dtype, shape, [0, 1])
+        col = T.HostTensor(T.random_values(rng, shape[0], dtype, **kw), dtype, shape, [1, 0])
+        nodes += [rec.leaf(row), rec.leaf(col)]
+        results = []
+        for step in range(int(rng.integers(3, 14))):
+            kind = rng.integers(0, 10)
+            x = nodes[int(rng.integers(0, len(nodes)))]
+            y = nodes[int(rng.integers(0, len(nodes)))]
+            if kind < 6:
+                r = rec.binary(int(rng.choice([O.ADD, O.SUB, O.MUL])), x, y)
+            elif kind < 8:
+                r = rec.unary(O.NEG, x)
+            else:
+                r = rec.binary(int(rng.choice([O.ADD, O.MUL])), rec.scalar(float(rng.integers(-3, 4))), x)
+            nodes.append(r)
+            results.append(r)
+            if rng.integers(0, 4) == 0 and results:      # in-place update of an earlier result: r2 = r2 op x
+                tgt = results[int(rng.integers(0, len(results)))]
+                op = int(rng.choice([O.ADD, O.SUB, O.MUL]))
+                assert CPU.binary(op, C.byref(tgt["host"].desc()), C.byref(x["host"].desc()), C.byref(tgt["host"].desc())) == 0
+                dev.dev.call(["add", "sub", "mul"][op], H.ref(tgt["desc"]), H.ref(x["desc"]), H.ref(tgt["desc"]))
+        keep = [results[-1]] + [r for r in results[:-1] if rng.integers(0, 3) == 0]
+        rec.free_temps(keep=keep)
+        for r in keep:
+            got = dev.fetch(r["ptr"], r["host"].storage)
+            T.assert_same_bits_nan_ok(got, r["host"].storage, dtype, f"{NAMES[dtype]} trial {trial} shape {shape}")
+        dev.release()
+
+
+def test_fusion_on_off_same_bits(dev):
+    """The fused kernels and the single-operator replay give identical bits (f32, transcendental ops included)."""
+    rng = np.random.default_rng(32000)
+    shape = [333, 257]
+    outs = []
+    for fusion in (1, 0):
+        set_diag(dev, elementwise_fusion=fusion)
+        rec = Recorder(dev, O.F32, shape)
+        r2 = np.random.default_rng(1)
+        a, b, c = (rec.leaf(T.contiguous_tensor(r2, O.F32, shape)) for _ in range(3))
+        y, _ = build_config0(rec, a, b, c)
+        z = rec.unary(O.SIN, rec.binary(O.POW, rec.unary(O.EXP, y), rec.scalar(1.5)))
+        rec.free_temps(keep=(z,))
+        outs.append(dev.fetch(z["ptr"], z["host"].storage))
+        diag = dev.dev.diagnostics()
+        assert (diag.fusible_subgraphs >= 1) == bool(fusion)
+        dev.release()
+    T.assert_same_bits_nan_ok(outs[0], outs[1], O.F32, "fused vs single")
+    set_diag(dev, elementwise_fusion=1)
+
+
+def test_kernel_cache_and_scalar_values(dev):
+    """Different immediates reuse the compiled kernel (DeviceTests.cpp:1774-1807)."""
+    set_diag(dev)
+    rng = np.random.default_rng(33000)
+    shape = [64, 100]
+    h0, m0 = dev.dev.kernel_cache_stats()
+    for k, s in enumerate((0.5, 0.25, 4.0)):
+        rec = Recorder(dev, O.F32, shape)
+        a = rec.leaf(T.contiguous_tensor(rng, O.F32, shape))
+        y = rec.binary(O.ADD, rec.unary(O.COS, rec.binary(O.MUL, rec.scalar(s), a)), rec.scalar(s))
+        rec.free_temps(keep=(y,))
+        got = dev.fetch(y["ptr"], y["host"].storage)
+        assert T.ulp_distance(got, y["host"].storage, O.F32) <= 2
+        dev.release()
+    h1, m1 = dev.dev.kernel_cache_stats()
+    assert m1 - m0 == 1 and h1 - h0 == 2, (h0, m0, h1, m1)
+
+
+def test_pending_work_is_flushed_before_other_operators(dev):
+    """Elementwise work recorded before a reduction / matmul / copy must be visible to it."""
+    set_diag(dev)
+    rng = np.random.default_rng(34000)
+    shape = [96, 160]
+    rec = Recorder(dev, O.F32, shape)
+    a, b = (rec.leaf(T.contiguous_tensor(rng, O.F32, shape)) for _ in range(2))
+    t = rec.binary(O.MUL, a, b)                                    # pending
+    # sum(t)
+    s_host = T.empty(O.F32, [])
+    ps = dev.raw(4)
+    dev.dev.call("sum", H.ref(t["desc"]), H.ref(H.kdesc(s_host, ps)))
+    exact, scale = C.c_double(), C.c_double()
+    assert CPU.sum_wide(C.byref(t["host"].desc()), C.byref(exact), C.byref(scale)) == 0
+    got = dev.fetch(ps, s_host.storage)
+    assert abs(float(got[0]) - exact.value) <= 1e-5 * scale.value
+    # matmul(t, t^T view) after an in-place update of t
+    assert CPU.binary(O.ADD, C.byref(t["host"].desc()), C.byref(a["host"].desc()), C.byref(t["host"].desc())) == 0
+    dev.dev.call("add", H.ref(t["desc"]), H.ref(a["desc"]), H.ref(t["desc"]))
+    tT = T.HostTensor(t["host"].storage, O.F32, [160, 96], [1, 160])
+    m_host = T.empty(O.F32, [96, 96])
+    pm = dev.raw(m_host.storage.nbytes)
+    dev.dev.call("matmul", H.ref(t["desc"]), H.ref(H.kdesc(tT, t["ptr"])), H.ref(H.kdesc(m_host, pm)))
+    exact_m = np.zeros(96 * 96)
+    scale_m = np.zeros(96 * 96)
+    assert CPU.matmul_wide(C.byref(t["host"].desc()), C.byref(tT.desc()), exact_m.ctypes.data, scale_m.ctypes.data, 4) == 0
+    got = dev.fetch(pm, m_host.storage).astype(np.float64)
+    assert np.all(np.abs(got - exact_m) <= 1e-5 * scale_m + 1e-30)
+    # reduceTo into a zero-filled destination (fill recorded, then accumulated into)
+    d_host = T.empty(O.F32, [1, 160])
+    pd = dev.raw(d_host.storage.nbytes)
+    zero = np.zeros(1, np.float32)
+    dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(H.kdesc(d_host, pd)))
+    dev.dev.call("reduce_to", H.ref(t["desc"]), H.ref(H.kdesc(d_host, pd)))
+    exact_r = np.zeros(160)
+    scale_r = np.zeros(160)
+    assert CPU.reduce_to_wide(C.byref(t["host"].desc()), C.byref(d_host.desc()), exact_r.ctypes.data, scale_r.ctypes.data) == 0
+    got = dev.fetch(pd, d_host.storage).astype(np.float64)
+    assert np.all(np.abs(got - exact_r) <= 1e-5 * scale_r + 1e-30)
+    dev.release()
+
+
+def test_host_operands_and_error_convention(dev):
+    rng = np.random.default_rng(35000)
+    a = T.contiguous_tensor(rng, O.F32, [50, 20])
+    b = T.view_tensor(rng, O.F32, [50, 20], "transposed")
+    want = T.empty(O.F32, [50, 20])
+    assert CPU.binary(O.ADD, C.byref(a.desc()), C.byref(b.desc()), C.byref(want.desc())) == 0
+    # host tensors handed straight to the device as sources (DeviceTests.cpp:209-215)
+    out = T.empty(O.F32, [50, 20])
+    po = dev.raw(out.storage.nbytes)
+    dev.dev.call("add", H.ref(H.kdesc(a, a.storage.ctypes.data)), H.ref(H.kdesc(b, b.storage.ctypes.data)), H.ref(H.kdesc(out, po)))
+    T.assert_same_bits(dev.fetch(po, out.storage), want.storage, "host sources")
+    # a host result is refused (aixDeviceMetal.cpp:305-306)
+    rc = dev.dev.status("add", H.ref(H.kdesc(a, a.storage.ctypes.data)), H.ref(H.kdesc(b, b.storage.ctypes.data)),
+                        H.ref(H.kdesc(out, out.storage.ctypes.data)))
+    assert rc == 1 and b"result must have GPU memory" in dev.dev.lib.aixhip_last_error()
+    # int32-only argmax results (aixDeviceCPU.cpp:1027-1030)
+    pa, da = dev.put(a)
+    bad = T.empty(O.F32, [])
+    pb = dev.raw(4)
+    assert dev.dev.status("argmax", H.ref(da), H.ref(H.kdesc(bad, pb))) == 1
+    assert b"int32" in dev.dev.lib.aixhip_last_error()
+    # freeing memory the device does not own (aixDeviceMetal.cpp:253-254)
+    assert dev.dev.lib.aixhip_deallocate(dev.dev.handle, a.storage.ctypes.data) == 1
+    # copy into host memory is refused, copy from host memory converts
+    u8 = np.zeros(4, np.uint8)
+    src = O.to_storage(np.array([-1.0, 0.0, 42.0, 300.0]), O.BF16)
+    assert dev.dev.status("copy", src.ctypes.data, O.BF16, u8.ctypes.data, O.U8, 4) == 1
+    pd = dev.raw(4)
+    dev.dev.call("copy_immediate", src.ctypes.data, O.BF16, pd, O.U8, 4)
+    assert dev.fetch(pd, u8).tolist() == [0, 0, 42, 255]          # DeviceTests.cpp:1282-1305
+    dev.release()
+
+
+def test_host_dereference_of_device_memory(dev):
+    """allocate() returns memory the host may write and (slowly) read directly, as the AIX
+    front-end does for item(), printing and test set-up (DeviceTests.cpp:185-189)."""
+    n = 4096
+    pa, pb, po = dev.raw(n * 4, keep=True), dev.raw(n * 4, keep=True), dev.raw(n * 4, keep=True)
+    a_host = T.empty(O.F32, [n])
+    for round_ in range(3):                                        # same addresses, new data each round
+        x = np.random.default_rng(round_).uniform(-1, 1, n).astype(np.float32)
+        y = np.random.default_rng(100 + round_).uniform(-1, 1, n).astype(np.float32)
+        C.memmove(pa, x.ctypes.data, n * 4)                        # direct host stores into device memory
+        C.memmove(pb, y.ctypes.data, n * 4)
+        dev.dev.call("mul", H.ref(H.kdesc(a_host, pa)), H.ref(H.kdesc(a_host, pb)), H.ref(H.kdesc(a_host, po)))
+        dev.dev.synchronize()
+        got = np.empty(n, np.float32)
+        C.memmove(got.ctypes.data, po, n * 4)                      # direct host loads from device memory
+        T.assert_same_bits(got, x * y, f"round {round_}")
+    dev.release()
+
+
+def test_1024_chained_in_place_adds_without_sync(dev):
+    """DeviceTests.cpp:3478-3500: 1024 in-place adds on 1 Mi elements, one synchronize at the end."""
+    n = 1 << 20
+    x = T.HostTensor(np.zeros(n, np.float32), O.F32, [n])
+    one = T.HostTensor(np.ones(n, np.float32), O.F32, [n])
+    px, dx = dev.put(x)
+    p1, d1 = dev.put(one)
+    for _ in range(1024):
+        dev.dev.call("add", H.ref(dx), H.ref(d1), H.ref(dx))
+    got = dev.fetch(px, x.storage)
+    assert np.all(got == 1024.0)
+    dev.release()
+
+
+def test_temporaries_are_recycled(dev):
+    """A long allocate / compute / free loop without synchronize keeps memory bounded."""
+    rng = np.random.default_rng(36000)
+    n = 1 << 18
+    a = T.contiguous_tensor(rng, O.F32, [n])
+    pa, da = dev.put(a)
+    acc = T.HostTensor(np.zeros(n, np.float32), O.F32, [n])
+    pacc, dacc = dev.put(acc)
+    for it in range(400):
+        pt = dev.raw(n * 4, keep=False)
+        dt = H.kdesc(acc, pt)
+        dev.dev.call("mul", H.ref(da), H.ref(da), H.ref(dt))
+        dev.dev.call("add", H.ref(dacc), H.ref(dt), H.ref(dacc))
+        dev.dev.deallocate(pt)
+        if it % 50 == 49:
+            dev.dev.flush()
+    got = dev.fetch(pacc, acc.storage)
+    want = np.zeros(n, np.float32)
+    sq = a.storage * a.storage
+    for _ in range(400):
+        want += sq
+    T.assert_same_bits(got, want, "accumulated squares")
+    live, cached = C.c_uint64(), C.c_uint64()
+    D.check(dev.dev.lib.aixhip_memory_stats(dev.dev.handle, C.byref(live), C.byref(cached)))
+    assert cached.value <= 160 * n * 4, cached.value
+    dev.release()
+
+
+_CASES = goldens.load_cases()
+
+
+@pytest.mark.parametrize("case", _CASES, ids=[c["name"] for c in _CASES])
+def test_reference_literals_on_device(dev, case):
+    goldens.run_case(case, H.DeviceBackend(dev))

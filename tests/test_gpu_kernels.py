@@ -50,6 +50,11 @@ def binary_rule(op, dtype):
 
 
 def unary_rule(op, dtype):
+    if op == O.SQRT and dtype == O.F64:
+        # The CPU evaluates sqrt in 80-bit long double and rounds a second time to double
+        # (aixDeviceCPU.cpp:162-163); about 1 result in 10^4 is then one unit away from the
+        # correctly rounded double the GPU returns.
+        return 1
     if dtype in T.INT_DTYPES or op in (O.NEG, O.SQRT):
         return G.EXACT
     return {O.F32: 2, O.F64: 4, O.F16: 1, O.BF16: 1}[dtype]
