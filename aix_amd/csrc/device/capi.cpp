@@ -66,6 +66,10 @@ DeviceHIP& D(aixhip_device* dev)
 
 } // namespace
 
+namespace aix::hip {
+DeviceHIP* fromHandle(::aixhip_device* handle) { return &D(handle); }
+}
+
 extern "C" {
 
 const char* aixhip_last_error(void) { return g_error; }

@@ -508,21 +508,23 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     }
 
     auto& ex = extras()[this];
-    const std::string key = gen::signature(d, shape);
+    bool noAlias = true;                                     // in-place updates: an output that is also an input
+    for (const auto& ob : d.outputBuffers) for (const auto& ib : d.inputBuffers) if (ob.data == ib.data) noAlias = false;
+    const std::string key = gen::signature(d, shape, bmask, noAlias);
     aixk_module* mod = nullptr;
     auto it = ex.kernels.find(key);
     if (it != ex.kernels.end()) { mod = it->second; ++ex.hits; }
     else {
         int32_t cached = 0;
-        const std::string src = gen::source(d, shape);
+        const std::string src = gen::source(d, shape, bmask, noAlias);
         check(aixk_rtc_get(m_ctx, key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
         ex.kernels.emplace(key, mod);
         ++ex.misses;
     }
 
-    const auto args = gen::packArgs(d, shape, inPtr, outPtr, n, bmask, shape == gen::Shape::Flat ? nullptr : &space, chunks);
+    const auto args = gen::packArgs(d, shape, inPtr, outPtr, n, shape == gen::Shape::Flat ? nullptr : &space, chunks);
     uint64_t items, perBlock, cap;
-    if (shape == gen::Shape::Flat) { items = n / VEC + 1; perBlock = (uint64_t)gen::kBlock * gen::flatUnroll(NI); cap = (uint64_t)m_cus * 32; }
+    if (shape == gen::Shape::Flat) { items = n / VEC + 1; perBlock = gen::kBlock; cap = 1u << 22; }
     else if (shape == gen::Shape::Rows) { items = n / VEC; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     else { items = n; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     uint64_t grid = (items + perBlock - 1) / perBlock;

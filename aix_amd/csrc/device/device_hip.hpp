@@ -33,6 +33,7 @@
 
 struct aixk_ctx;
 struct aixhip_tensor;
+struct aixhip_device;
 
 namespace aix::hip {
 
@@ -136,5 +137,8 @@ private:
 };
 
 std::unique_ptr<aix::Device> createDeviceHIP(size_t deviceIndex = 0);   // nullptr if no GPU is visible
+
+// The C++ device behind a handle of the C ABI (include/aixhip.h); throws on a null handle.
+DeviceHIP* fromHandle(::aixhip_device* handle);
 
 } // namespace aix::hip

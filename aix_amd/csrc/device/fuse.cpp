@@ -126,6 +126,7 @@ struct Group {
     std::vector<std::pair<DeviceTensorParams, size_t>> defs;   // view -> latest defining op
     std::vector<DeviceTensorParams> loads;                     // distinct views loaded from memory
     bool open{true};
+    bool absorbed{false};                                      // merged into another group
     bool hasScalar{false};
 };
 
@@ -303,9 +304,15 @@ private:
                     if (!m_groups[g].open) continue;
                     const auto* def = findDef(m_groups[g], in[k]->data);
                     if (!def) continue;
-                    if (sameView(def->first, *in[k]) && compatible(m_groups[g], op) && (target == SIZE_MAX || target == g)) {
+                    const bool usable = sameView(def->first, *in[k]) && compatible(m_groups[g], op);
+                    if (usable && (target == SIZE_MAX || target == g)) {
                         resolved[k] = Operand{Operand::kValue, def->second};
                         target = g;
+                    } else if (usable && mergeable(m_groups[target], m_groups[g])) {
+                        // both operands come from open groups: open groups are independent of each
+                        // other, so the two become one kernel
+                        resolved[k] = Operand{Operand::kValue, def->second};
+                        mergeInto(target, g);
                     } else {
                         closeGroup(g);
                         closedSomething = true;
@@ -384,6 +391,41 @@ private:
         const bool opDense = isDense(op.output) && (!op.input0.data || isDense(op.input0)) &&
                              (!op.hasInput1 || !op.input1.data || isDense(op.input1));
         return g.dense && opDense;
+    }
+
+    bool mergeable(const Group& a, const Group& b) const
+    {
+        if (a.dtype != b.dtype || a.count != b.count) return false;
+        if (!(a.shape == b.shape) && !(a.dense && b.dense)) return false;
+        size_t loads = a.loads.size();
+        for (const auto& v : b.loads) {
+            bool known = false;
+            for (const auto& w : a.loads) if (sameView(v, w)) known = true;
+            if (!known) ++loads;
+        }
+        return loads + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;
+    }
+
+    // Folds open group `from` into open group `into` (no hazards can exist between open groups).
+    void mergeInto(size_t into, size_t from)
+    {
+        Group& a = m_groups[into];
+        Group& b = m_groups[from];
+        std::vector<size_t> ops(a.ops.size() + b.ops.size());
+        std::merge(a.ops.begin(), a.ops.end(), b.ops.begin(), b.ops.end(), ops.begin());     // program order
+        a.ops.swap(ops);
+        for (auto& d : b.defs) a.defs.push_back(d);
+        for (const auto& v : b.loads) {
+            bool known = false;
+            for (const auto& w : a.loads) if (sameView(v, w)) known = true;
+            if (!known) a.loads.push_back(v);
+        }
+        a.dense = a.dense && b.dense;
+        a.hasScalar = a.hasScalar || b.hasScalar;
+        for (size_t w : b.ops) m_groupOf[w] = into;
+        b.ops.clear(); b.defs.clear(); b.loads.clear();
+        b.open = false;                                     // absorbed: never emitted on its own
+        b.absorbed = true;
     }
 
     size_t slotsAfterJoin(const Group& g, const OpRecord& op, const Operand* resolved) const
@@ -530,6 +572,11 @@ const FlushDiagnostics& FuseEngine::lastFlushDiagnostics() const
 void FuseEngine::flush()
 {
     if (m_flushing) return;                  // callbacks may call back into the device
+    if (m_pending.empty()) {                 // nothing recorded: the previous flush's diagnostics stay readable
+        m_externalReads.clear();
+        m_callbacks.finishFlush();
+        return;
+    }
     m_flushing = true;
     struct Reset { bool& f; ~Reset() { f = false; } } reset{m_flushing};
 

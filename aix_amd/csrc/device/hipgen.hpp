@@ -22,15 +22,15 @@ enum class Shape { Flat, Rows, Gather };
 
 // Identity of a generated kernel: element type, launch shape, operator wiring.  Immediates'
 // values, pointers, sizes and strides are arguments and not part of it.
-std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape);
+// For the flat shape two more facts are compiled in: which inputs are a single broadcast element
+// (bit k of broadcastMask), and whether no output aliases an input (the pointers may then be
+// declared __restrict__).
+std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
 
 // Source of `extern "C" __global__ void aix_fused(Args)`.
-std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape);
+std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
 
 inline const char* entryName() { return "aix_fused"; }
-
-// How many 16-byte vectors per input a lane keeps in flight in the flat shape.
-int flatUnroll(size_t inputs);
 
 constexpr int kMaxDims = 8;
 constexpr int kBlock = 256;
@@ -45,7 +45,7 @@ struct Space {
 
 // Kernel-argument block in the exact layout of the generated `struct Args`.
 std::vector<uint64_t> packArgs(const fuse::FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
-                               const std::vector<void*>& outputs, uint64_t n, uint32_t broadcastMask, const Space* space,
+                               const std::vector<void*>& outputs, uint64_t n, const Space* space,
                                uint64_t chunksPerRow);
 
 } // namespace aixhip::gen

@@ -1,0 +1,312 @@
+// value.hpp -- a small tensor-value front-end over aix::Device.
+//
+// This is the CALLER side of the device interface: it decides what a device sees, exactly the way
+// the AIX front-end does (Targets/AIXLib/aixCore.hpp) --
+//   * every operator allocates a fresh contiguous result from the device (:1414-1427);
+//   * operands of different shape become stride-0 broadcast VIEWS, no copy (:599-629, 1616-1638);
+//   * `tensor op scalar` materialises the scalar as a rank-0 tensor with fill() and reads it
+//     through a broadcast view (:2384-2388);
+//   * transpose / reshape of contiguous data / select are views (:979-994);
+//   * reductions along dims are fill(0 | lowest) followed by reduceTo / maxTo (:632-639, 873-891);
+//   * temporaries release their storage (Device::deallocate) as soon as the expression is done,
+//     usually long before the device has run anything.
+// It exists so that the benchmark and the training example can drive DeviceHIP (or any other
+// aix::Device) with the op stream AIX itself would produce.  It is not a port of AIX's tensor
+// classes: no printing, no serialisation, no dtype promotion beyond what the drivers need.
+#pragma once
+
+#include "../device/aix_compat.hpp"
+
+#include <cstring>
+#include <memory>
+#include <numeric>
+#include <stdexcept>
+#include <vector>
+
+namespace aixfe {
+
+using aix::DataType;
+using aix::Device;
+using aix::DeviceTensorParams;
+using aix::Shape;
+using aix::Stride;
+
+inline size_t numel(const Shape& s) { size_t n = 1; for (auto e : s) n *= e; return n; }
+
+inline Stride denseStrides(const Shape& s)
+{
+    Stride st(s.size());
+    size_t run = 1;
+    for (size_t d = s.size(); d-- > 0;) { st[d] = run; run *= s[d]; }
+    return st;
+}
+
+inline Shape broadcastShapes(const Shape& a, const Shape& b)
+{
+    const size_t r = std::max(a.size(), b.size());
+    Shape out(r);
+    for (size_t i = 0; i < r; ++i) {
+        const size_t ea = i < r - a.size() ? 1 : a[i - (r - a.size())];
+        const size_t eb = i < r - b.size() ? 1 : b[i - (r - b.size())];
+        if (ea != eb && ea != 1 && eb != 1) throw std::invalid_argument("shapes cannot be broadcast together");
+        out[i] = ea == 1 ? eb : ea;
+    }
+    return out;
+}
+
+class Value {
+public:
+    Value() = default;
+
+    // Uninitialised contiguous tensor.
+    Value(Device* dev, DataType dt, Shape shape) : m_dev(dev), m_dt(dt), m_shape(std::move(shape))
+    {
+        m_strides = denseStrides(m_shape);
+        m_store = std::make_shared<Storage>(dev, dev->allocate(std::max<size_t>(numel(m_shape), 1), dt));
+    }
+
+    // Every element = v (one device fill).
+    static Value full(Device* dev, DataType dt, const Shape& shape, float v)
+    {
+        Value t(dev, dt, shape);
+        dev->fill(&v, DataType::kFloat32, t.params());
+        return t;
+    }
+
+    // From host memory of the same element type (Device::copy, host source).
+    static Value fromHost(Device* dev, DataType dt, const Shape& shape, const void* host)
+    {
+        Value t(dev, dt, shape);
+        dev->copy(host, dt, t.data(), dt, numel(shape));
+        return t;
+    }
+
+    bool defined() const { return (bool)m_store; }
+    Device* device() const { return m_dev; }
+    DataType dtype() const { return m_dt; }
+    const Shape& shape() const { return m_shape; }
+    const Stride& strides() const { return m_strides; }
+    size_t size() const { return numel(m_shape); }
+    void* data() const { return m_store ? m_store->ptr : nullptr; }
+    size_t offset() const { return m_offset; }
+    bool isContiguous() const { return m_strides == denseStrides(m_shape); }
+
+    DeviceTensorParams params() const
+    {
+        DeviceTensorParams p;
+        p.data = data(); p.dtype = m_dt; p.isContiguous = isContiguous(); p.offset = m_offset;
+        p.shape = m_shape; p.size = size(); p.strides = m_strides;
+        return p;
+    }
+
+    // ---- views ------------------------------------------------------------------------------
+    Value broadcastTo(const Shape& target) const
+    {
+        if (target == m_shape) return *this;
+        if (target.size() < m_shape.size()) throw std::invalid_argument("broadcastTo: rank shrinks");
+        Value v = *this;
+        v.m_shape = target;
+        v.m_strides.assign(target.size(), 0);
+        const size_t lead = target.size() - m_shape.size();
+        for (size_t i = 0; i < m_shape.size(); ++i) {
+            if (m_shape[i] == target[lead + i]) v.m_strides[lead + i] = m_strides[i];
+            else if (m_shape[i] != 1) throw std::invalid_argument("broadcastTo: incompatible shape");
+        }
+        return v;
+    }
+
+    Value transpose(size_t d0, size_t d1) const
+    {
+        Value v = *this;
+        std::swap(v.m_shape[d0], v.m_shape[d1]);
+        std::swap(v.m_strides[d0], v.m_strides[d1]);
+        return v;
+    }
+
+    Value reshape(const Shape& s) const
+    {
+        if (numel(s) != size()) throw std::invalid_argument("reshape: element count differs");
+        Value v = isContiguous() ? *this : contiguous();
+        v.m_shape = s;
+        v.m_strides = denseStrides(s);
+        return v;
+    }
+
+    // index `i` along the first dim: a view with an offset (how batched matmuls are issued)
+    Value select0(size_t i) const
+    {
+        Value v = *this;
+        v.m_offset += i * m_strides[0];
+        v.m_shape.erase(v.m_shape.begin());
+        v.m_strides.erase(v.m_strides.begin());
+        return v;
+    }
+
+    Value contiguous() const
+    {
+        if (isContiguous() && m_offset == 0) return *this;
+        Value r(m_dev, m_dt, m_shape);
+        m_dev->contiguous(params(), r.params());
+        return r;
+    }
+
+    Value to(DataType dt) const
+    {
+        if (dt == m_dt) return *this;
+        Value src = contiguous();
+        Value r(m_dev, dt, m_shape);
+        m_dev->copy(static_cast<const char*>(src.data()) + src.m_offset * Device::dataTypeSize(m_dt), m_dt, r.data(), dt, size());
+        return r;
+    }
+
+    // ---- elementwise ------------------------------------------------------------------------
+    using BinaryFn = void (Device::*)(const DeviceTensorParams&, const DeviceTensorParams&, const DeviceTensorParams&);
+    using UnaryFn = void (Device::*)(const DeviceTensorParams&, const DeviceTensorParams&);
+
+    Value binary(BinaryFn fn, const Value& other) const
+    {
+        if (other.m_dt != m_dt) throw std::invalid_argument("binary: element types differ");
+        if (m_shape == other.m_shape) {
+            Value r(m_dev, m_dt, m_shape);
+            (m_dev->*fn)(params(), other.params(), r.params());
+            return r;
+        }
+        const Shape bc = broadcastShapes(m_shape, other.m_shape);
+        const Value l = broadcastTo(bc), rr = other.broadcastTo(bc);
+        Value r(m_dev, m_dt, bc);
+        (m_dev->*fn)(l.params(), rr.params(), r.params());
+        return r;
+    }
+
+    // tensor op scalar: rank-0 tensor + broadcast view
+    Value binaryScalar(BinaryFn fn, float s, bool scalarFirst = false) const
+    {
+        const Value sc = full(m_dev, m_dt, Shape{}, s).broadcastTo(m_shape);
+        Value r(m_dev, m_dt, m_shape);
+        if (scalarFirst) (m_dev->*fn)(sc.params(), params(), r.params());
+        else (m_dev->*fn)(params(), sc.params(), r.params());
+        return r;
+    }
+
+    Value& inPlace(BinaryFn fn, const Value& other)
+    {
+        const Value rhs = other.m_shape == m_shape ? other : other.broadcastTo(m_shape);
+        (m_dev->*fn)(params(), rhs.params(), params());
+        return *this;
+    }
+
+    Value unary(UnaryFn fn) const
+    {
+        Value r(m_dev, m_dt, m_shape);
+        (m_dev->*fn)(params(), r.params());
+        return r;
+    }
+
+    Value operator+(const Value& o) const { return binary(&Device::add, o); }
+    Value operator-(const Value& o) const { return binary(&Device::sub, o); }
+    Value operator*(const Value& o) const { return binary(&Device::mul, o); }
+    Value operator/(const Value& o) const { return binary(&Device::div, o); }
+    Value operator+(float s) const { return binaryScalar(&Device::add, s); }
+    Value operator-(float s) const { return binaryScalar(&Device::sub, s); }
+    Value operator*(float s) const { return binaryScalar(&Device::mul, s); }
+    Value operator/(float s) const { return binaryScalar(&Device::div, s); }
+    friend Value operator+(float s, const Value& v) { return v.binaryScalar(&Device::add, s, true); }
+    friend Value operator-(float s, const Value& v) { return v.binaryScalar(&Device::sub, s, true); }
+    friend Value operator*(float s, const Value& v) { return v.binaryScalar(&Device::mul, s, true); }
+    friend Value operator/(float s, const Value& v) { return v.binaryScalar(&Device::div, s, true); }
+    Value operator-() const { return unary(&Device::unary); }
+    Value& operator+=(const Value& o) { return inPlace(&Device::add, o); }
+    Value& operator-=(const Value& o) { return inPlace(&Device::sub, o); }
+    Value& operator*=(const Value& o) { return inPlace(&Device::mul, o); }
+    Value sqrt() const { return unary(&Device::sqrt); }
+    Value exp() const { return unary(&Device::exp); }
+    Value log() const { return unary(&Device::log); }
+    Value tanh() const { return unary(&Device::tanh); }
+    Value sin() const { return unary(&Device::sin); }
+    Value cos() const { return unary(&Device::cos); }
+    Value pow(float e) const { return binaryScalar(&Device::pow, e); }
+
+    void fill(float v) { m_dev->fill(&v, DataType::kFloat32, params()); }
+
+    // ---- reductions ---------------------------------------------------------------------------
+    Value sum() const
+    {
+        Value r(m_dev, m_dt, Shape{});
+        m_dev->sum(params(), r.params());
+        return r;
+    }
+
+    // Sum down to `target` (right-aligned, 1 = reduced): zero-fill then accumulate.
+    Value reduceTo(const Shape& target) const
+    {
+        if (target == m_shape) return *this;
+        Value r = full(m_dev, m_dt, target, 0.0f);
+        m_dev->reduceTo(params(), r.params());
+        return r;
+    }
+
+    Value sum(size_t dim, bool keepDim) const
+    {
+        Shape kept = m_shape;
+        kept[dim] = 1;
+        Value r = reduceTo(kept);
+        return keepDim ? r : r.squeeze(dim);
+    }
+
+    Value max(size_t dim, bool keepDim) const
+    {
+        Shape kept = m_shape;
+        kept[dim] = 1;
+        Value r(m_dev, m_dt, kept);
+        m_dev->fillMin(r.params());
+        m_dev->maxTo(params(), r.params());
+        return keepDim ? r : r.squeeze(dim);
+    }
+
+    Value argmax(size_t dim, bool keepDim) const
+    {
+        Shape kept = m_shape;
+        kept[dim] = 1;
+        Value r(m_dev, DataType::kInt32, kept);
+        m_dev->argmaxTo(params(), r.params(), dim);
+        return keepDim ? r : r.squeeze(dim);
+    }
+
+    Value mean() const { return sum() / (float)size(); }
+
+    Value squeeze(size_t dim) const
+    {
+        Value v = *this;
+        v.m_shape.erase(v.m_shape.begin() + (long)dim);
+        v.m_strides.erase(v.m_strides.begin() + (long)dim);
+        return v;
+    }
+
+    Value matmul(const Value& b) const
+    {
+        if (m_shape.size() != 2 || b.m_shape.size() != 2 || m_shape[1] != b.m_shape[0])
+            throw std::invalid_argument("matmul: operands must be 2-D with matching inner dimension");
+        Value r(m_dev, m_dt, Shape{m_shape[0], b.m_shape[1]});
+        m_dev->matmul(params(), b.params(), r.params());
+        return r;
+    }
+
+private:
+    struct Storage {
+        Device* dev;
+        void* ptr;
+        Storage(Device* d, void* p) : dev(d), ptr(p) {}
+        ~Storage() { if (dev && ptr) dev->deallocate(ptr); }
+        Storage(const Storage&) = delete;
+        Storage& operator=(const Storage&) = delete;
+    };
+
+    Device* m_dev{nullptr};
+    DataType m_dt{DataType::kFloat32};
+    Shape m_shape;
+    Stride m_strides;
+    size_t m_offset{0};
+    std::shared_ptr<Storage> m_store;
+};
+
+} // namespace aixfe

@@ -17,8 +17,6 @@ using namespace aixk;
 
 namespace {
 
-constexpr int kUnroll = 4;
-
 template <int OP, class T> struct Bin {
     static __device__ __forceinline__ T run(T a, T b)
     {
@@ -40,10 +38,11 @@ static_assert(AIXK_SQRT == M_SQRT && AIXK_SIN == M_SIN && AIXK_COS == M_COS && A
               AIXK_LOG == M_LOG && AIXK_EXP == M_EXP, "unary op codes must match the math selectors");
 
 // ---- flat ------------------------------------------------------------------------------------
-// NIN = 1 or 2 inputs.  An input flagged `scalar` is a single broadcast element.
-template <class F, class T, int NIN>
-__global__ __launch_bounds__(kBlock) void ew_flat(const T* __restrict__ a, const T* __restrict__ b,
-                                                  T* __restrict__ out, u64 n, int a_scalar, int b_scalar)
+// NIN = 1 or 2 inputs.  AS / BS: that input is a single broadcast element.  One 16-byte vector per
+// operand per lane and one workgroup per 256 vectors: many small groups in flight overlap their
+// load and compute phases better than a long per-lane loop (measured on the fused chain).
+template <class F, class T, int NIN, bool AS, bool BS>
+__global__ __launch_bounds__(kBlock) void ew_flat(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out, u64 n)
 {
     typedef typename vec16<T>::type V;
     constexpr int VEC = vec16<T>::n;
@@ -51,42 +50,27 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const T* __restrict__ a, const
     const V* A = (const V*)a;
     const V* B = (const V*)b;
     V* O = (V*)out;
-    T sa = a_scalar ? a[0] : zero<T>();
-    T sb = zero<T>();
-    if constexpr (NIN == 2) sb = b_scalar ? b[0] : zero<T>();
-
-    const u64 tile = (u64)kBlock * kUnroll;
-    for (u64 v0 = (u64)blockIdx.x * tile; v0 < nvec; v0 += (u64)gridDim.x * tile) {
-        V ra[kUnroll], rb[kUnroll];
+    T sa = zero<T>(), sb = zero<T>();
+    if constexpr (AS) sa = a[0];
+    if constexpr (NIN == 2 && BS) sb = b[0];
+    for (u64 v = (u64)blockIdx.x * kBlock + threadIdx.x; v < nvec; v += (u64)gridDim.x * kBlock) {
+        V ra, rb, r;
+        if constexpr (!AS) ra = A[v];
+        if constexpr (NIN == 2 && !BS) rb = B[v];
 #pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
-            const u64 v = v0 + (u64)k * kBlock + threadIdx.x;
-            if (v < nvec) {
-                if (!a_scalar) ra[k] = A[v];
-                if constexpr (NIN == 2) if (!b_scalar) rb[k] = B[v];
-            }
+        for (int e = 0; e < VEC; ++e) {
+            const T x = AS ? sa : ra.v[e];
+            if constexpr (NIN == 2) { const T y = BS ? sb : rb.v[e]; r.v[e] = F::run(x, y); }
+            else r.v[e] = F::run(x);
         }
-#pragma unroll
-        for (int k = 0; k < kUnroll; ++k) {
-            const u64 v = v0 + (u64)k * kBlock + threadIdx.x;
-            if (v < nvec) {
-                V r;
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const T x = a_scalar ? sa : ra[k].v[e];
-                    if constexpr (NIN == 2) { const T y = b_scalar ? sb : rb[k].v[e]; r.v[e] = F::run(x, y); }
-                    else r.v[e] = F::run(x);
-                }
-                O[v] = r;
-            }
-        }
+        O[v] = r;
     }
     // tail (< VEC elements) by the first lanes of block 0
     const u64 done = nvec * VEC;
     if (blockIdx.x == 0 && done + threadIdx.x < n) {
         const u64 i = done + threadIdx.x;
-        const T x = a_scalar ? sa : a[i];
-        if constexpr (NIN == 2) { const T y = b_scalar ? sb : b[i]; out[i] = F::run(x, y); }
+        const T x = AS ? sa : a[i];
+        if constexpr (NIN == 2) { const T y = BS ? sb : b[i]; out[i] = F::run(x, y); }
         else out[i] = F::run(x);
     }
 }
@@ -163,8 +147,6 @@ int launch_ew(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, con
     const T* pa = (const T*)a->data;
     const T* pb = NIN == 2 ? (const T*)b->data : pa;
     T* po = (T*)out->data;
-    const unsigned max_blocks = (unsigned)ctx->cus * 16u;
-
     // flat: rank 0 (single element / all-broadcast) or rank 1 with strides in {0,1}
     const bool flat_shape = sp.rank == 0 || (sp.rank == 1 && sp.stride[0][0] <= 1 && sp.stride[1][0] <= 1);
     if (flat_shape) {
@@ -173,9 +155,14 @@ int launch_ew(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, con
         const T* qa = pa + sp.offset[0];
         const T* qb = pb + sp.offset[1];
         if ((as || aligned16(qa)) && (bs || aligned16(qb)) && aligned16(po)) {
-            const unsigned grid = grid_for(n / VEC + 1, kBlock * kUnroll, max_blocks);
-            hipLaunchKernelGGL((ew_flat<F, T, NIN>), dim3(grid), dim3(kBlock), 0, ctx->stream, qa, qb, po, (u64)n,
-                               sp.rank == 0 ? 0 : as, sp.rank == 0 ? 0 : bs);
+            const unsigned grid = grid_for(n / VEC + 1, kBlock, 1u << 22);
+            const int fa = sp.rank == 0 ? 0 : as, fb = (NIN == 2 && sp.rank != 0) ? bs : 0;
+#define AIXK_FLAT(AS_, BS_) hipLaunchKernelGGL((ew_flat<F, T, NIN, AS_, BS_>), dim3(grid), dim3(kBlock), 0, ctx->stream, qa, qb, po, (u64)n)
+            if (fa && fb) AIXK_FLAT(true, true);
+            else if (fa) AIXK_FLAT(true, false);
+            else if (fb) AIXK_FLAT(false, true);
+            else AIXK_FLAT(false, false);
+#undef AIXK_FLAT
             AIXK_HIP(hipGetLastError());
             return AIXK_OK;
         }
@@ -195,7 +182,7 @@ int launch_ew(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, con
         }
         if (ok) {
             const uint64_t chunks = sp.shape[in] / VEC, total = n / VEC;
-            const unsigned grid = grid_for(total, kBlock, max_blocks * 4);
+            const unsigned grid = grid_for(total, kBlock, 1u << 22);
             if (small)
                 hipLaunchKernelGGL((ew_rows<F, T, NIN, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, pa, pb, po, sp, (u64)total, (u32)chunks);
             else
@@ -204,7 +191,7 @@ int launch_ew(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, con
             return AIXK_OK;
         }
     }
-    const unsigned grid = grid_for(n, kBlock, max_blocks * 4);
+    const unsigned grid = grid_for(n, kBlock, 1u << 22);
     if (small)
         hipLaunchKernelGGL((ew_gather<F, T, NIN, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, pa, pb, po, sp, (u64)n);
     else
@@ -375,7 +362,7 @@ int32_t aixk_cast(aixk_ctx* ctx, const void* src, int src_dtype, void* dst, int 
             if constexpr (traits<S>::code == traits<D>::code) return (int)AIXK_OK;
             else {
                 constexpr int K = 16 / (sizeof(S) < sizeof(D) ? sizeof(S) : sizeof(D));
-                const unsigned max_blocks = (unsigned)ctx->cus * 16u;
+                const unsigned max_blocks = 1u << 22;              // one chunk per lane
                 if (aligned16(src) && aligned16(dst))
                     hipLaunchKernelGGL((cast_flat<S, D>), dim3(grid_for(n / K + 1, kBlock, max_blocks)), dim3(kBlock), 0, ctx->stream,
                                        (const S*)src, (D*)dst, (u64)n);

@@ -90,6 +90,41 @@ __global__ __launch_bounds__(kBlock) void transpose_tiled_k(const W* __restrict_
     }
 }
 
+// Same tile walk with 16-byte global accesses on both sides (whole tiles only, everything
+// 16-byte aligned): a lane loads VEC consecutive r of one c, scatters them into the LDS tile as
+// tile[r][c], and later gathers VEC consecutive c of one r for a 16-byte store.
+template <class W>
+__global__ __launch_bounds__(kBlock) void transpose_vec_k(const W* __restrict__ src, W* __restrict__ dst,
+                                                          u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r)
+{
+    typedef typename vec16<W>::type V;
+    constexpr int VEC = vec16<W>::n;
+    constexpr int LPR = kTile / VEC;          // lanes covering one tile row
+    constexpr int RPP = kBlock / LPR;         // tile rows covered per pass
+    __shared__ W tile[kTile][kTile + 1];
+    const u32 t = blockIdx.x;
+    const u32 tr = t % tiles_r, tc = t / tiles_r;
+    const u64 b = blockIdx.y;
+    const u64 r0 = (u64)tr * kTile, c0 = (u64)tc * kTile;
+    const W* s = src + off + b * sb;
+    W* d = dst + b * R * C;
+    const int lv = (threadIdx.x % LPR) * VEC, lp = threadIdx.x / LPR;
+#pragma unroll
+    for (int cc = lp; cc < kTile; cc += RPP) {
+        const V v = *(const V*)(s + (r0 + lv) + (c0 + cc) * ld);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) tile[lv + e][cc] = v.v[e];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int rr = lp; rr < kTile; rr += RPP) {
+        V v;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v.v[e] = tile[rr][lv + e];
+        *(V*)(d + (r0 + rr) * C + c0 + lv) = v;
+    }
+}
+
 // ---- generic strided copy with both sides strided (sliceSet, transpose scatter) ---------------
 template <class W, class IDX>
 __global__ __launch_bounds__(kBlock) void copy_views_k(const W* __restrict__ src, W* __restrict__ dst,
@@ -187,6 +222,14 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
             const uint64_t B = sp.rank == 3 ? sp.shape[0] : 1, sb = sp.rank == 3 ? sp.stride[0][0] : 0;
             const uint64_t R = sp.shape[o], C = sp.shape[o + 1], ld = sp.stride[0][o + 1];
             const uint64_t tr = (R + kTile - 1) / kTile, tc = (C + kTile - 1) / kTile;
+            const bool whole = R % kTile == 0 && C % kTile == 0 && ld % VEC == 0 && sb % VEC == 0 &&
+                               aligned16(ps + sp.offset[0]) && aligned16(pd);
+            if (ld != 0 && whole && tr * tc < (1ull << 31) && B < 65536) {
+                hipLaunchKernelGGL((transpose_vec_k<W>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
+                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            }
             if (ld != 0 && tr * tc < (1ull << 31) && B < 65536) {
                 hipLaunchKernelGGL((transpose_tiled_k<W>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
                                    ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr, (u32)tc);

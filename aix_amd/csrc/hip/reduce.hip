@@ -44,7 +44,8 @@ template <> __device__ __forceinline__ i64 neg_inf<i64>() { return lowest<i64>()
 template <> __device__ __forceinline__ i32 neg_inf<i32>() { return lowest<i32>(); }
 
 // flags: 1 = holds a non-NaN value, 2 = the slot's first element is NaN
-template <class W> struct ArgAcc { u64 idx; W v; u32 flags; };
+// idx: flat logical index (argmax sources are limited to 2^31 elements on the host side)
+template <class W> struct ArgAcc { W v; u32 idx; u32 flags; };
 
 template <class T> struct SumOp {
     typedef typename sum_acc<T>::type Acc;
@@ -52,6 +53,7 @@ template <class T> struct SumOp {
     static __device__ __forceinline__ Acc init() { return (Acc)0; }
     static __device__ __forceinline__ Acc load(T x, u64, bool) { return (Acc)up(x); }
     static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return a + b; }
+    static __device__ __forceinline__ void step(Acc& a, T x, u64, bool) { a += (Acc)up(x); }
     static __device__ __forceinline__ Acc shfl(Acc v, int d) { return __shfl_down(v, d, kWave); }
 };
 template <class T> struct MaxOp {
@@ -60,16 +62,25 @@ template <class T> struct MaxOp {
     static __device__ __forceinline__ Acc init() { return neg_inf<Acc>(); }
     static __device__ __forceinline__ Acc load(T x, u64, bool) { const Acc w = up(x); return w != w ? neg_inf<Acc>() : w; }
     static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return b > a ? b : a; }
+    static __device__ __forceinline__ void step(Acc& a, T x, u64, bool) { const Acc w = up(x); if (w > a) a = w; }      // NaN: '>' is false
     static __device__ __forceinline__ Acc shfl(Acc v, int d) { return __shfl_down(v, d, kWave); }
 };
 template <class T> struct ArgOp {
     typedef typename traits<T>::W W;
     typedef ArgAcc<W> Acc;
     typedef i32 Out;
-    static __device__ __forceinline__ Acc init() { Acc a; a.v = neg_inf<W>(); a.idx = ~0ull; a.flags = 0; return a; }
+    static __device__ __forceinline__ Acc init() { Acc a; a.v = neg_inf<W>(); a.idx = ~0u; a.flags = 0; return a; }
+    // In-order scan by one lane: indices only grow, so an equal value never replaces the holder.
+    static __device__ __forceinline__ void step(Acc& a, T x, u64 flat, bool first)
+    {
+        const W w = up(x);
+        const bool nan = w != w;
+        if (!nan && (!(a.flags & 1u) || w > a.v)) { a.v = w; a.idx = (u32)flat; a.flags |= 1u; }
+        if (first && nan) a.flags |= 2u;
+    }
     static __device__ __forceinline__ Acc load(T x, u64 flat, bool first)
     {
-        Acc a; a.v = up(x); a.idx = flat;
+        Acc a; a.v = up(x); a.idx = (u32)flat;
         const bool nan = a.v != a.v;
         a.flags = nan ? (first ? 2u : 0u) : 1u;
         return a;
@@ -88,7 +99,7 @@ template <class T> struct ArgOp {
     static __device__ __forceinline__ Acc shfl(Acc v, int d)
     {
         Acc r;
-        r.idx = (u64)__shfl_down((unsigned long long)v.idx, d, kWave);
+        r.idx = __shfl_down(v.idx, d, kWave);
         r.v = __shfl_down(v.v, d, kWave);
         r.flags = __shfl_down(v.flags, d, kWave);
         return r;
@@ -147,11 +158,10 @@ template <class T> __device__ __forceinline__ void land(ArgOp<T>, const Finish& 
 // ---- whole tensor ----------------------------------------------------------------------------------
 template <class Op, class T, class IDX, bool FLAT>
 __global__ __launch_bounds__(kBlock) void reduce_all_k(const T* __restrict__ src, typename Op::Out* dst, Space<1> sp, u64 n,
-                                                       typename Op::Acc* partials, unsigned int* counter, Finish fin)
+                                                       typename Op::Acc* partials, Finish fin)
 {
     typedef typename Op::Acc Acc;
     __shared__ Acc smem[kWaves];
-    __shared__ int last;
     Acc acc = Op::init();
     if constexpr (FLAT) {
         typedef typename vec16<T>::type V;
@@ -170,32 +180,36 @@ __global__ __launch_bounds__(kBlock) void reduce_all_k(const T* __restrict__ src
                 const u64 v = v0 + (u64)k * kBlock + threadIdx.x;
                 if (v < nvec) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) { const u64 i = v * VEC + e; acc = Op::combine(acc, Op::load(r[k].v[e], i, i == 0)); }
+                    for (int e = 0; e < VEC; ++e) { const u64 i = v * VEC + e; Op::step(acc, r[k].v[e], i, i == 0); }
                 }
             }
         }
         const u64 done = nvec * VEC;
-        if (blockIdx.x == 0 && done + threadIdx.x < n) { const u64 i = done + threadIdx.x; acc = Op::combine(acc, Op::load(base[i], i, i == 0)); }
+        if (blockIdx.x == 0 && done + threadIdx.x < n) { const u64 i = done + threadIdx.x; Op::step(acc, base[i], i, i == 0); }
     } else {
         for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock)
-            acc = Op::combine(acc, Op::load(src[locate<1, IDX>(sp, 0, (IDX)i)], i, i == 0));
+            Op::step(acc, src[locate<1, IDX>(sp, 0, (IDX)i)], i, i == 0);
     }
     acc = block_reduce<Op>(acc, smem);
     if (threadIdx.x == 0) {
-        partials[blockIdx.x] = acc;
-        __threadfence();                                     // publish the partial before taking a ticket
-        last = atomicAdd(counter, 1u) == gridDim.x - 1;
+        if (gridDim.x == 1) land(Op{}, fin, dst, 0, acc, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
+        else partials[blockIdx.x] = acc;
     }
-    __syncthreads();
-    if (!last) return;
-    __threadfence();                                         // see every other workgroup's partial
+}
+
+// Second pass of the whole-tensor reduction: one workgroup folds the partials in index order.
+// (A kernel boundary instead of an in-kernel "last group finishes" hand-off: the device-scope
+// fences that hand-off needs cost more than a second launch on this multi-die part.)
+template <class Op, class T, class IDX>
+__global__ __launch_bounds__(kBlock) void reduce_all_finish_k(const T* __restrict__ src, typename Op::Out* dst, Space<1> sp,
+                                                              const typename Op::Acc* __restrict__ partials, unsigned count, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    __shared__ Acc smem[kWaves];
     Acc a = Op::init();
-    for (unsigned i = threadIdx.x; i < gridDim.x; i += kBlock) a = Op::combine(a, partials[i]);
+    for (unsigned i = threadIdx.x; i < count; i += kBlock) a = Op::combine(a, partials[i]);
     a = block_reduce<Op>(a, smem);
-    if (threadIdx.x == 0) {
-        *counter = 0;                                        // ready for the next reduction on this stream
-        land(Op{}, fin, dst, 0, a, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
-    }
+    if (threadIdx.x == 0) land(Op{}, fin, dst, 0, a, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
 }
 
 // ---- per-slot plans ------------------------------------------------------------------------------
@@ -253,12 +267,12 @@ __global__ __launch_bounds__(kBlock) void reduce_inner_k(const T* __restrict__ s
                         const u64 v = v0 + (u64)k * GROUP + l;
                         if (v < nvec) {
 #pragma unroll
-                            for (int e = 0; e < VEC; ++e) { const u64 j = v * VEC + e; acc = Op::combine(acc, Op::load(r[k].v[e], s.flat + j * p.r_flat[0], j == 0)); }
+                            for (int e = 0; e < VEC; ++e) { const u64 j = v * VEC + e; Op::step(acc, r[k].v[e], s.flat + j * p.r_flat[0], j == 0); }
                         }
                     }
                 }
             } else {
-                for (u64 j = l; j < L; j += GROUP) acc = Op::combine(acc, Op::load(row[j], s.flat + j * p.r_flat[0], j == 0));
+                for (u64 j = l; j < L; j += GROUP) Op::step(acc, row[j], s.flat + j * p.r_flat[0], j == 0);
             }
         }
         if constexpr (GROUP == kBlock) acc = block_reduce<Op>(acc, smem);
@@ -299,7 +313,7 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ s
                 if (r < r_end) {
 #pragma unroll
                     for (int e = 0; e < VEC; ++e)
-                        acc[e] = Op::combine(acc[e], Op::load(x[k].v[e], s.flat + r * p.r_flat[0] + (c0 + e) * p.k_flat[p.nk - 1], r == 0));
+                        Op::step(acc[e], x[k].v[e], s.flat + r * p.r_flat[0] + (c0 + e) * p.k_flat[p.nk - 1], r == 0);
                 }
             }
         }
@@ -358,7 +372,7 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_k(const T* __restrict__
                     pos += c * p.r_src[d]; flat += c * p.r_flat[d];
                     rest = q;
                 }
-                acc = Op::combine(acc, Op::load(src[pos], flat, j == 0));
+                Op::step(acc, src[pos], flat, j == 0);
             }
         }
         if (block_per_slot) acc = block_reduce<Op>(acc, smem);
@@ -487,13 +501,18 @@ int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const 
     const bool flat = (sp.rank == 0 || (sp.rank == 1 && sp.stride[0][0] == 1)) && aligned16(ps + sp.offset[0]);
     const bool small = n < (1ull << 31) && view_extent(a) < (1ull << 31);
     constexpr int VEC = vec16<T>::n;
-    unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 8, ctx->scratch_bytes / sizeof(Acc));
+    unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 16, ctx->scratch_bytes / sizeof(Acc));
     const unsigned grid = flat ? grid_for(n / VEC + 1, kBlock * 4, max_blocks) : grid_for(n, kBlock * 4, max_blocks);
     Acc* partials = (Acc*)ctx->scratch;
-    if (flat) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
-    else if (small) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
-    else hipLaunchKernelGGL((reduce_all_k<Op, T, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, ctx->counter, fin);
+    if (flat) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
+    else if (small) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
+    else hipLaunchKernelGGL((reduce_all_k<Op, T, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
     AIXK_HIP(hipGetLastError());
+    if (grid > 1) {
+        if (small) hipLaunchKernelGGL((reduce_all_finish_k<Op, T, u32>), dim3(1), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (const Acc*)partials, grid, fin);
+        else hipLaunchKernelGGL((reduce_all_finish_k<Op, T, u64>), dim3(1), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (const Acc*)partials, grid, fin);
+        AIXK_HIP(hipGetLastError());
+    }
     return AIXK_OK;
 }
 

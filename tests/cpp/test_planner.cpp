@@ -168,6 +168,39 @@ static void testChainBecomesOneDenseKernel()
     }
 }
 
+static void testOperandOrderDoesNotSplitTheKernel()
+{
+    // C++ leaves the evaluation order of a - b open: record the right operand's subtree first.
+    // t8 = 0.5*c starts its own group, the rest grows another; the final sub joins them.
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    aix::Shape shape{512, 512};
+    auto a = T(1, shape), b = T(2, shape), c = T(3, shape), y = T(20, shape);
+    auto t = [&](uintptr_t k) { return T(10 + k, shape); };
+    for (uintptr_t id : {1, 2, 3, 20, 11, 12, 13, 14, 15, 16, 17, 18, 30, 31}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    const float one = 1.0f, half = 0.5f;
+    aix::Stride zeros(2, 0);
+    e.recordFill(&half, DataType::kFloat32, T(31, {}));
+    e.record(OpType::Mul, T(31, shape, DataType::kFloat32, zeros), c, t(8));
+    e.recordFill(&one, DataType::kFloat32, T(30, {}));
+    e.record(OpType::Negate, a, t(4));
+    e.record(OpType::Exp, t(4), t(5));
+    e.record(OpType::Add, T(30, shape, DataType::kFloat32, zeros), t(5), t(6));
+    e.record(OpType::Mul, a, b, t(1));
+    e.record(OpType::Add, t(1), c, t(2));
+    e.record(OpType::Tanh, t(2), t(3));
+    e.record(OpType::Div, t(3), t(6), t(7));
+    e.record(OpType::Sub, t(7), t(8), y);
+    for (uintptr_t id : {11, 12, 13, 14, 15, 16, 17, 18, 30, 31}) e.releaseBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.flush();
+    CHECK(cap.singles.empty());
+    CHECK(cap.fused.size() == 1);
+    if (cap.fused.size() != 1) return;
+    CHECK(cap.fused[0].ops.size() == 9 && cap.fused[0].inputBuffers.size() == 3 && cap.fused[0].outputBuffers.size() == 1);
+    CHECK(cap.fused[0].ops[0].type == OpType::Mul && cap.fused[0].ops.back().type == OpType::Sub);     // program order kept
+    CHECK(compiles(cap.fused[0], gen::Shape::Flat));
+}
+
 static void testLiveTemporariesAreStoredAndFillsRun()
 {
     Capture cap;
@@ -372,6 +405,7 @@ int main(int argc, char** argv)
     if (g_prelude.empty()) { std::printf("cannot read %s\n", argv[1]); return 2; }
 
     testChainBecomesOneDenseKernel();
+    testOperandOrderDoesNotSplitTheKernel();
     testLiveTemporariesAreStoredAndFillsRun();
     testFusionDisabledReplaysInOrder();
     testInPlaceUpdatesKeepProgramOrder();

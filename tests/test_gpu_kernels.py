@@ -235,6 +235,7 @@ def test_contiguous_and_transpose(gpu, dtype):
     # 2-D and batched transposes through the LDS-tiled kernel, incl. ragged edges
     cases += [([n, m], "transposed") for n, m in [(1, 1), (1, 70), (63, 65), (64, 64), (129, 257), (300, 5), (5, 300), (513, 1025)]]
     cases += [([3, 70, 130], "transposed"), ([96, 256], "sliced"), ([33, 48], "offset")]
+    cases += [([128, 192], "transposed"), ([3, 64, 128], "transposed"), ([256, 64], "transposed")]   # whole tiles: 16-byte path
     for shape, kind in cases:
         src = T.view_tensor(rng, dtype, shape, kind)
         want = T.empty(dtype, shape)
