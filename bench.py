@@ -103,6 +103,31 @@ def cpu_chain(a, b, c):
     return y, t7, dt, kind
 
 
+def calibrate_copy(steps):
+    """K launches of ew_flat<negate, f32> over 16 Mi elements: reads 67 108 864 B, writes 67 108 864 B per launch."""
+    from aix_amd import kernels as K
+    ctx = K.Context(0)
+    n = 1 << 24
+    src, dst = ctx.alloc(n * 4), ctx.alloc(n * 4)
+    ctx.upload(src, np.ones(n, np.float32))
+    d_in, d_out = K.Tensor(), K.Tensor()
+    for d, p in ((d_in, src), (d_out, dst)):
+        d.data, d.dtype, d.rank, d.offset, d.size = p, K.F32, 1, 0, n
+        d.shape[0], d.strides[0] = n, 1
+    e0, e1 = ctx.event(), ctx.event()
+    ctx.call("aixk_unary", K.NEG, C.byref(d_in), C.byref(d_out))
+    ctx.sync()
+    ctx.record(e0)
+    for _ in range(steps):
+        ctx.call("aixk_unary", K.NEG, C.byref(d_in), C.byref(d_out))
+    ctx.record(e1)
+    ms = ctx.elapsed_ms(e0, e1)
+    print(json.dumps({"workload": "calibration: negate f32, 16 Mi elements", "bytes_read_per_launch": n * 4,
+                      "bytes_written_per_launch": n * 4, "launches": steps + 1, "us_per_launch": round(ms * 1e3 / steps, 2),
+                      "GBps": round(2 * n * 4 / (ms / steps * 1e-3) / 1e9, 1)}))
+    ctx.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -110,9 +135,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="run only a plain copy-shaped kernel (negate, 64 MiB in + 64 MiB out per launch): the known-size "
+                         "reference that hardware counter readings (FETCH_SIZE / WRITE_SIZE) are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend drives one GPU per process and this build measures exactly one; run with --gpus 1")
+    if args.calibrate_copy:
+        return calibrate_copy(args.steps)
 
     from aix_amd import device as D
     lib = load_driver()
@@ -145,7 +175,9 @@ def main():
                    "fusion": {"ops_recorded": int(diag.ops_recorded), "kernels": int(diag.fusible_subgraphs),
                               "fused_ops": int(diag.fused_ops), "fills_absorbed": int(diag.fills_absorbed),
                               "single_ops": int(diag.fallback_ops), "jit_cache_hits": hits, "jit_cache_misses": misses}},
-        "roofline": roofline("hbm", algo_bytes / (kernel_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s"),
+        # traffic: HBM bytes per launch from the FETCH_SIZE + WRITE_SIZE counter passes, scaled by the readings of
+        # a copy kernel of known size (profiles/aix_fused_c0_f32_4096x4096.md); a measured constant, not live.
+        "roofline": roofline("hbm", algo_bytes / (kernel_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", traffic=268409963),
     }
     out["roofline"]["kernel"] = "aix_fused (f32|flat|i3o1s2, 9 ops)"
     out["roofline"]["kernel_us"] = round(kernel_ms * 1e3, 2)
