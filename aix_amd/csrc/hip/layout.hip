@@ -407,3 +407,8 @@ int32_t aixk_index_add(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_ten
 }
 
 } // extern "C"
+
+namespace aixk {
+// dst (dense, n elements) = the logical contents of `src`; used by the GEMM to make operands K-contiguous.
+int gather_dense(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n) { return gather_into(ctx, src, dst, n); }
+} // namespace aixk

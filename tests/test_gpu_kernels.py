@@ -555,6 +555,23 @@ def test_matmul(gpu, dtype):
         gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16], ids=ids)
+def test_matmul_mfma_tiles(gpu, dtype):
+    """Shapes that run on the matrix cores: ragged M and N against both workgroup tile sizes, every
+    operand layout (row-major, transposed view, sliced, offset), K tails inside a K step."""
+    rng = np.random.default_rng(23000 + dtype)
+    cases = [((256, 256, 256), "contig", "contig"), ((300, 520, 264), "contig", "contig"), ((1000, 72, 130), "contig", "transposed"),
+             ((129, 1048, 131), "transposed", "contig"), ((640, 136, 384), "transposed", "transposed"),
+             ((200, 200, 200), "sliced", "offset"), ((96, 4096, 80), "contig", "contig"),
+             ((2085, 512, 4101), "contig", "contig"), ((2048, 264, 4096), "contig", "transposed")]     # 256x256 tiles
+    for (m, k, n), ka, kb in cases:
+        scale = 1.0 / np.sqrt(k)
+        a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
+        b = T.view_tensor(rng, dtype, [k, n], kb, lo=-1, hi=1)
+        check_matmul(gpu, a, b, f"mfma matmul {NAMES[dtype]} {m}x{k}x{n} {ka}/{kb}")
+        gpu.release()
+
+
 def test_matmul_identity_and_ones(gpu):
     """Mathematical pins: A.I == A exactly; ones[m,k].ones[k,n] == k exactly (f32, f16, bf16)."""
     rng = np.random.default_rng(22000)
