@@ -1,19 +1,18 @@
 // matmul_mfma.hip -- GEMM on the matrix cores for f32 / f16 / bf16, f32 accumulation.
 //
-// One core kernel shape per precision, both operands K-contiguous in memory ("NT": A is [M,K] with
-// unit stride along K, B is given as [N,K] with unit stride along K):
+// Core kernels, all with both operands K-contiguous in memory ("NT": A is [M,K] with unit stride
+// along K, B is given as [N,K] with unit stride along K):
 //
-//   16-bit  v_mfma_f32_32x32x16_{bf16,f16}; workgroup tile 256x256 (or 128x128 for small
-//           problems) x BK=64, 4 waves in a 2x2 arrangement, each wave 4x4 (2x2) MFMA tiles with
-//           the accumulators resident in the 512-entry unified register file;
-//   f32     v_mfma_f32_32x32x2f32; workgroup tile 128x128 x BK=32, each wave 2x2 MFMA tiles.
+//   16-bit, whole tiles   gemm_nt16_direct_k: 256x256x64 workgroup tile, LDS filled by LDS-direct
+//                         global loads, swizzled layout, explicit software pipeline (see there);
+//   16-bit, any shape     gemm_nt16_k: 256x256 or 128x128 tile x BK=64, bounds-checked register
+//                         staging, padded LDS rows; edges and small problems;
+//   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 tile x BK=32.
 //
-// Per K-step: 16-byte global loads into registers for step t+1 are issued before the MFMAs of step
-// t, then written to the other LDS buffer (double buffered, one barrier per step).  LDS rows are
-// padded by 16 bytes so that the 8 lanes served per LDS cycle by ds_read_b128 hit 32 distinct
-// banks.  Every lane feeds the MFMA with 8 (f32: 4) consecutive K values of one row; because A and
-// B use the same lane->K assignment, the dot products are independent of how the instruction
-// numbers K internally.
+// All use 4 waves in a 2x2 arrangement with the accumulators resident in the 512-entry unified
+// register file.  Every lane feeds the MFMA with 8 (f32: 4) consecutive K values of one row;
+// because A and B use the same lane->K assignment, the dot products are independent of how the
+// instruction numbers K internally.
 //
 // Workgroups are numbered so that the 32 groups resident on one XCD (dispatch is round-robin over
 // the 8 XCDs) cover a compact 4 x 8 block of output tiles and share A/B panels in that XCD's L2.
@@ -65,12 +64,22 @@ template <class T> struct Mma16;
 template <> struct Mma16<bf16> {
     static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c)
     { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0); }
-    static __device__ __forceinline__ bf16 out(float v) { return bf16_down(v); }
+    static __device__ __forceinline__ bf16 out(float v)       // bf16_down without a branch (the epilogue holds 256 live accumulators)
+    {
+        const u32 u = __builtin_bit_cast(u32, v);
+        const bool nan = (u & 0x7FFFFFFFu) > 0x7F800000u;
+        bf16 r;
+        r.bits = (u16)(nan ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16));
+        return r;
+    }
+    static __device__ __forceinline__ u32 pack(float lo, float hi) { return (u32)out(lo).bits | ((u32)out(hi).bits << 16); }
 };
 template <> struct Mma16<f16> {
     static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c)
     { return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0); }
     static __device__ __forceinline__ f16 out(float v) { return (f16)v; }
+    static __device__ __forceinline__ u32 pack(float lo, float hi)
+    { return (u32)__builtin_bit_cast(u16, (f16)lo) | ((u32)__builtin_bit_cast(u16, (f16)hi) << 16); }
 };
 
 // ---- 16-bit operands ---------------------------------------------------------------------------
@@ -168,6 +177,139 @@ __global__ __launch_bounds__(256) void gemm_nt16_k(GemmArgs g)
             }
         }
 }
+
+// ---- 16-bit operands, 256 x 256 x 64 tile fed by LDS-direct loads ---------------------------------
+// For M, N multiples of 256 and K a multiple of 64.  Two 64 KB LDS stages; each wave fills its share
+// of the next stage with global_load_lds_dwordx4 (16 bytes per lane straight into LDS, no staging
+// registers, whole 128-byte rows per 8 lanes so every L2 request is a full line).  One load
+// instruction deposits 1 KB contiguously (lane L at byte 16 L), so padding is impossible; instead
+// the 16-byte k-chunk q of row r is kept in slot q ^ f(r), f(r) = ((r >> 1) & 7) ^ ((r & 1) << 2),
+// which makes the ds_read_b128 fragment reads (32 consecutive rows, one slot) conflict-free for
+// both 8-lane/32-bank and 16-lane/64-bank service; the producing lane applies the same
+// permutation to the global address it fetches.
+//
+// A K-step is four phases of 16 MFMAs (one 16-wide K slice each) on double-buffered fragments: the
+// LDS reads of the next slice and the loads of the tile after next are spread between the MFMAs in
+// fenced sub-blocks of 4 (the scheduler otherwise serialises "read, wait, 4 MFMAs").  The step's
+// single barrier sits before the last phase, whose MFMAs cover the first fragment reads from the
+// other stage.  The compiler does not track LDS-direct loads against LDS reads, so the waits
+// before each barrier are explicit (s_waitcnt vmcnt), and the barrier is the bare instruction.
+#define AIX_SB() __builtin_amdgcn_sched_barrier(0)
+#define AIX_WAIT(VM, LGKM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (((VM) >> 4) << 14) | 0x70 | ((LGKM) << 8))
+#define AIX_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+#define AIX_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
+template <class T>
+__global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
+{
+    constexpr int BM = 256, BK = 64, TI = 4, TJ = 4, STAGE = 2 * 256 * BK * 2;     // 65536 bytes: A rows then B rows
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    u32 tm, tn;
+    tile_of(g, tm, tn);
+    const u64 m0 = (u64)tm * 256, n0 = (u64)tn * 256;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), wm = wave >> 1, wn = wave & 1;
+    // producer: wave w fills rows 64 w .. 64 w + 63 of both operands, 8 chunks of 8 rows each
+    const int lr = lane >> 3;
+    const int fe = (lr >> 1) ^ ((lr & 1) << 2);              // f(row) in even chunks; odd chunks: fe ^ 4
+    const int q0 = (lane & 7) ^ fe, q1 = q0 ^ 4;
+    const char* A = (const char*)g.a + (m0 + wave * 64) * g.lda * 2;
+    const char* B = (const char*)g.b + (n0 + wave * 64) * g.ldb * 2;
+    const u32 oa0 = (u32)((lr * g.lda + q0 * 8) * 2), oa1 = (u32)((lr * g.lda + q1 * 8) * 2);
+    const u32 ob0 = (u32)((lr * g.ldb + q0 * 8) * 2), ob1 = (u32)((lr * g.ldb + q1 * 8) * 2);
+    const u64 ca = 16 * g.lda, cb = 16 * g.ldb;               // bytes between 8-row chunks
+    const int steps = (int)(g.K / BK);
+    // consumer: lane reads row (lane & 31) of a 32-row block, k-chunk 2 kk + (lane >> 5)
+    const int r15 = lane & 15;
+    const int slot0 = (lane >> 5) ^ (((r15 >> 1) & 7) ^ ((r15 & 1) << 2));
+    const int fra = (wm * 128 + (lane & 31)) * 128 + slot0 * 16;
+    const int frb = BM * 128 + (wn * 128 + (lane & 31)) * 128 + slot0 * 16;
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    u32x4 fa[2][TI], fb[2][TJ];
+
+    // load n of a tile (0..15): n < 8 is chunk n of A, otherwise chunk n - 8 of B
+#define AIX_LD(N, KO, BO) { if ((N) < 8) __builtin_amdgcn_global_load_lds(AIX_GLB(A + ((N) * ca + (KO)) + (((N) & 1) ? oa1 : oa0)), AIX_LDS(smem + (BO) + (wave * 8 + (N)) * 1024), 16, 0, 0); \
+    else __builtin_amdgcn_global_load_lds(AIX_GLB(B + (((N) - 8) * cb + (KO)) + (((N) & 1) ? ob1 : ob0)), AIX_LDS(smem + (BO) + BM * 128 + (wave * 8 + (N) - 8) * 1024), 16, 0, 0); }
+#define AIX_RDA(F, BO, KK, I) fa[F][I] = *(const u32x4*)(smem + (BO) + (fra ^ ((KK) * 32)) + (I) * 4096);
+#define AIX_RDB(F, BO, KK, J) fb[F][J] = *(const u32x4*)(smem + (BO) + (frb ^ ((KK) * 32)) + (J) * 4096);
+#define AIX_ROW(F, I) { _Pragma("unroll") for (int j = 0; j < TJ; ++j) acc[I][j] = Mma16<T>::run(fa[F][I], fb[F][j], acc[I][j]); }
+    // MFMAs on fragment set FC while set FN is read from stage RBO, slice KK; loads L0.. of the tile at byte KO go to stage LBO
+#define AIX_PHASE(FC, FN, RBO, KK, KO, LBO, L0, L1, L2, L3, L4, L5) \
+    AIX_RDA(FN, RBO, KK, 0) AIX_RDA(FN, RBO, KK, 1) if (L0 >= 0) AIX_LD(L0, KO, LBO) if (L4 >= 0) AIX_LD(L4, KO, LBO) AIX_ROW(FC, 0) AIX_SB(); \
+    AIX_RDA(FN, RBO, KK, 2) AIX_RDA(FN, RBO, KK, 3) if (L1 >= 0) AIX_LD(L1, KO, LBO) if (L5 >= 0) AIX_LD(L5, KO, LBO) AIX_ROW(FC, 1) AIX_SB(); \
+    AIX_RDB(FN, RBO, KK, 0) AIX_RDB(FN, RBO, KK, 1) if (L2 >= 0) AIX_LD(L2, KO, LBO) AIX_ROW(FC, 2) AIX_SB(); \
+    AIX_RDB(FN, RBO, KK, 2) AIX_RDB(FN, RBO, KK, 3) if (L3 >= 0) AIX_LD(L3, KO, LBO) AIX_ROW(FC, 3) AIX_SB();
+
+    // Tiles past the end re-read the last tile into a stage nobody consumes any more.
+    {
+        const u64 k1 = (u64)(1 < steps ? 1 : 0) * (BK * 2);
+#pragma unroll
+        for (int n = 0; n < 16; ++n) AIX_LD(n, 0, 0)
+#pragma unroll
+        for (int n = 0; n < 6; ++n) AIX_LD(n, k1, STAGE)
+    }
+    AIX_SB();
+    AIX_WAIT(6, 15);                                          // tile 0 has landed (6 younger loads may be in flight)
+    __builtin_amdgcn_s_barrier();
+    AIX_SB();
+    AIX_RDA(0, 0, 0, 0) AIX_RDA(0, 0, 0, 1) AIX_RDA(0, 0, 0, 2) AIX_RDA(0, 0, 0, 3)
+    AIX_RDB(0, 0, 0, 0) AIX_RDB(0, 0, 0, 1) AIX_RDB(0, 0, 0, 2) AIX_RDB(0, 0, 0, 3)
+    for (int kt = 0; kt < steps; ++kt) {
+        const int bo = (kt & 1) * STAGE, nbo = bo ^ STAGE;
+        const u64 k1 = (u64)(kt + 1 < steps ? kt + 1 : steps - 1) * (BK * 2);
+        const u64 k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1) * (BK * 2);
+        AIX_PHASE(0, 1, bo, 1, k1, nbo, 6, 7, 8, 9, 10, -1)
+        AIX_PHASE(1, 0, bo, 2, k1, nbo, 11, 12, 13, 14, 15, -1)
+        AIX_PHASE(0, 1, bo, 3, k1, nbo, -1, -1, -1, -1, -1, -1)
+        AIX_WAIT(0, 0);                                       // tile kt+1 complete in the other stage; own reads of this stage done
+        __builtin_amdgcn_s_barrier();
+        AIX_SB();
+        AIX_PHASE(1, 0, nbo, 0, k2, bo, 0, 1, 2, 3, 4, 5)
+    }
+#undef AIX_PHASE
+#undef AIX_ROW
+#undef AIX_RDB
+#undef AIX_RDA
+#undef AIX_LD
+    AIX_WAIT(0, 0);                                           // stray loads have landed before LDS is reused
+    __builtin_amdgcn_s_barrier();
+    AIX_SB();
+
+    // Epilogue through LDS, each wave on its own 20 KB: a 32-row slab of the wave's 128 x 128 block
+    // is laid out row-major (pitch 132 floats), read back as runs of 8 columns, rounded and stored
+    // with 16-byte writes (256 contiguous bytes per row).
+    constexpr int PITCH = 132;
+    float* slab = (float*)smem + wave * (32 * PITCH + 1024);
+    u16* C = (u16*)g.c;
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                slab[((v >> 2) * 8 + (lane >> 5) * 4 + (v & 3)) * PITCH + j * 32 + (lane & 31)] = acc[i][j][v];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int grp = lane + 64 * t, row = grp >> 4, cg = grp & 15;
+            const f32x4 lo = *(const f32x4*)(slab + row * PITCH + cg * 8);
+            const f32x4 hi = *(const f32x4*)(slab + row * PITCH + cg * 8 + 4);
+            u32x4 o;
+            o.x = Mma16<T>::pack(lo.x, lo.y); o.y = Mma16<T>::pack(lo.z, lo.w);
+            o.z = Mma16<T>::pack(hi.x, hi.y); o.w = Mma16<T>::pack(hi.z, hi.w);
+            *(u32x4*)(C + (m0 + wm * 128 + i * 32 + row) * g.N + n0 + wn * 128 + cg * 8) = o;
+        }
+    }
+}
+#undef AIX_GLB
+#undef AIX_LDS
+#undef AIX_WAIT
+#undef AIX_SB
 
 // ---- f32 operands ------------------------------------------------------------------------------
 // 128 x 128 workgroup tile, BK = 32; LDS row = 32 floats + 4 padding = 144 bytes.  A lane reads 4
@@ -341,7 +483,12 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         return AIXK_OK;
     }
     const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= (uint64_t)ctx->cus / 2;
-    if (big) {
+    if (big && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && lda < (1ull << 27) && ldb < (1ull << 27)) {
+        constexpr size_t lds = 2 * 65536;
+        const u32 n = grid_of(256, 256);
+        if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_direct_k<bf16>, lds)); hipLaunchKernelGGL((gemm_nt16_direct_k<bf16>), dim3(n), dim3(256), lds, ctx->stream, g); }
+        else { AIXK_TRY(set_lds(gemm_nt16_direct_k<f16>, lds)); hipLaunchKernelGGL((gemm_nt16_direct_k<f16>), dim3(n), dim3(256), lds, ctx->stream, g); }
+    } else if (big) {
         constexpr size_t lds = 2 * (256 + 256) * 72 * 2;
         const u32 n = grid_of(256, 256);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }

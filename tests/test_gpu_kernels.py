@@ -563,7 +563,10 @@ def test_matmul_mfma_tiles(gpu, dtype):
     cases = [((256, 256, 256), "contig", "contig"), ((300, 520, 264), "contig", "contig"), ((1000, 72, 130), "contig", "transposed"),
              ((129, 1048, 131), "transposed", "contig"), ((640, 136, 384), "transposed", "transposed"),
              ((200, 200, 200), "sliced", "offset"), ((96, 4096, 80), "contig", "contig"),
-             ((2085, 512, 4101), "contig", "contig"), ((2048, 264, 4096), "contig", "transposed")]     # 256x256 tiles
+             ((2085, 512, 4101), "contig", "contig"), ((2048, 264, 4096), "contig", "transposed"),     # 256x256 tiles
+             # whole 256x256 tiles and K steps of 64: the LDS-direct kernel (1, 2, 3 and 5 K steps; swizzled and plain tile numbering)
+             ((2048, 64, 4096), "contig", "transposed"), ((2048, 128, 4096), "contig", "contig"),
+             ((4096, 192, 2048), "transposed", "contig"), ((2304, 320, 3840), "contig", "transposed")]
     for (m, k, n), ka, kb in cases:
         scale = 1.0 / np.sqrt(k)
         a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
