@@ -9,6 +9,7 @@
 
 #include "../../../include/aixhip.h"
 #include "../device/device_hip.hpp"
+#include "../frontend/mlp.hpp"
 #include "../frontend/value.hpp"
 
 #include <chrono>
@@ -159,6 +160,19 @@ int aixbench_matmul(aixhip_device* handle, int dtype, uint64_t M, uint64_t N, ui
         t.stop(&res->wall_s, &res->gpu_ms);
         res->steps = steps;
         if (out) dev->copyToHost(out, r[0].data(), M * N * aix::Device::dataTypeSize(dt));
+    });
+}
+
+// Config 3: MLP training (in -> hidden -> hidden -> out, ReLU, softmax + cross-entropy, Adam) for
+// `steps` steps from the given host parameters; losses[steps], step_seconds[steps] (may be NULL).
+int aixbench_mlp(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
+                 const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds)
+{
+    return guarded([&] {
+        DeviceHIP* dev = aix::hip::fromHandle(handle);
+        const aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr};
+        const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
+        aixfe::runMlp(dev, cfg, host, losses, step_seconds);
     });
 }
 

@@ -1,0 +1,375 @@
+// autograd.hpp -- reverse-mode differentiation over aixfe::Value, generating the op stream the
+// reference's autograd generates (Targets/AIXLib/aixCore.hpp:1790-1857, 2014-2309).
+//
+// What a device sees during backward() depends on how the caller differentiates, so this mirrors
+// the reference's scheme rather than a textbook tape:
+//   * every result is a node holding its value, its input nodes and one backward function;
+//   * backward(seed) on a node calls that function at once, which computes the seeds of the inputs
+//     with ordinary Value operators and RECURSES into them -- no topological ordering and no
+//     accumulation at interior nodes, so a node reachable along p paths is differentiated p times
+//     (softmax + cross-entropy reaches the logits along 4 paths; everything below them runs 4x);
+//   * leaves add the seed into their gradient buffer (grad += seed);
+//   * binary operators first bring both operands to the common shape with broadcastTo(), which
+//     is itself a node whose backward is reduceTo() of the seed;
+//   * `tensor op scalar` wraps the scalar in a rank-0 tensor and broadcasts it (:2384-2438).
+// Only the operators the training drivers need are present.
+#pragma once
+
+#include "value.hpp"
+
+#include <functional>
+#include <utility>
+
+namespace aixfe {
+
+struct Node;
+using NodePtr = std::shared_ptr<Node>;
+
+// aixCore.hpp:1790-1857
+struct Node {
+    Value value;
+    bool requireGrad{false};
+    bool retainGrad{false};
+    bool isLeaf{true};
+    std::vector<NodePtr> inputs;
+    size_t dim0{0}, dim1{0};
+    bool keepDim{false};
+    std::function<void(Node*, const Value&)> backwardFn;
+
+    Node(Value v, bool req) : value(std::move(v)), requireGrad(req) {}
+
+    void backward(const Value& seed)
+    {
+        if (retainGrad) grad() += seed;
+        if (requireGrad || retainGrad) backwardFn(this, seed);
+    }
+
+    Value& grad()
+    {
+        if (!m_grad.defined()) {
+            m_grad = Value(value.device(), value.dtype(), value.shape());
+            m_grad.fill(0.0f);
+        }
+        return m_grad;
+    }
+
+    void setBackward(std::vector<NodePtr> in, std::function<void(Node*, const Value&)> fn)
+    {
+        if (requireGrad || retainGrad) { inputs = std::move(in); backwardFn = std::move(fn); }
+    }
+
+private:
+    Value m_grad;
+};
+
+class Tensor {
+public:
+    Tensor() = default;
+
+    // Leaf from an existing value.
+    explicit Tensor(Value v, bool requireGrad = false) : m_node(std::make_shared<Node>(std::move(v), requireGrad))
+    {
+        m_node->backwardFn = defaultBackward;
+    }
+
+    // Leaf filled with one number (aixCore.hpp:1907-1913).
+    Tensor(float v, const Shape& shape, Device* dev, DataType dt = DataType::kFloat32, bool requireGrad = false)
+        : Tensor(Value::full(dev, dt, shape, v), requireGrad) {}
+
+    static Tensor fromHost(Device* dev, DataType dt, const Shape& shape, const void* host, bool requireGrad = false)
+    {
+        return Tensor(Value::fromHost(dev, dt, shape, host), requireGrad);
+    }
+
+    const Value& value() const { return m_node->value; }
+    Value& value() { return m_node->value; }
+    Value& grad() const { return m_node->grad(); }
+    const Shape& shape() const { return m_node->value.shape(); }
+    DataType dtype() const { return m_node->value.dtype(); }
+    Device* device() const { return m_node->value.device(); }
+    bool isRequireGrad() const { return m_node->requireGrad; }
+    void zeroGrad() const { m_node->grad().fill(0.0f); }
+    const NodePtr& node() const { return m_node; }
+
+    // aixCore.hpp:1923-1933: seed of ones.
+    void backward() const
+    {
+        if (value().size() != 1) throw std::invalid_argument("backward() requires a one-element tensor");
+        m_node->backward(Value::full(device(), dtype(), shape(), 1.0f));
+    }
+
+    // ---- shape ------------------------------------------------------------------------------
+    Tensor broadcastTo(const Shape& s) const
+    {
+        if (shape() == s) return *this;
+        Tensor r = makeResult(value().broadcastTo(s), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.reduceTo(n->inputs[0]->value.shape()));
+        });
+        return r;
+    }
+
+    Tensor transpose(size_t d0, size_t d1) const
+    {
+        Tensor r = makeResult(value().transpose(d0, d1), isRequireGrad());
+        r.m_node->dim0 = d0; r.m_node->dim1 = d1;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.transpose(n->dim0, n->dim1));
+        });
+        return r;
+    }
+
+    Tensor unsqueeze(size_t dim) const
+    {
+        Tensor r = makeResult(value().unsqueeze(dim), isRequireGrad());
+        r.m_node->dim0 = dim;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.squeeze(n->dim0));
+        });
+        return r;
+    }
+
+    Tensor squeeze(size_t dim) const
+    {
+        Tensor r = makeResult(value().squeeze(dim), isRequireGrad());
+        r.m_node->dim0 = dim;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.unsqueeze(n->dim0));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2702-2779; catBackwardFunc :2292-2309
+    static Tensor cat(const std::vector<Tensor>& parts, size_t dim)
+    {
+        if (parts.empty()) throw std::invalid_argument("cat: no tensors");
+        if (parts.size() == 1) return parts[0];
+        bool anyGrad = false, anyNonLeaf = false;
+        std::vector<Value> values;
+        std::vector<NodePtr> inputs;
+        for (const auto& p : parts) {
+            anyGrad |= p.isRequireGrad(); anyNonLeaf |= !p.m_node->isLeaf;
+            values.push_back(p.value()); inputs.push_back(p.m_node);
+        }
+        Tensor r = makeResult(Value::cat(values, dim), anyGrad, anyNonLeaf);
+        r.m_node->dim0 = dim;
+        r.m_node->setBackward(std::move(inputs), [](Node* n, const Value& seed) {
+            size_t at = 0;
+            for (auto& in : n->inputs) {
+                const size_t ext = in->value.shape()[n->dim0];
+                if (in->requireGrad || in->retainGrad) in->backward(seed.slice(n->dim0, at, at + ext, 1));
+                at += ext;
+            }
+        });
+        return r;
+    }
+
+    // ---- arithmetic (aixCore.hpp:2317-2438) -----------------------------------------------------
+    Tensor operator+(const Tensor& o) const
+    {
+        return binary(o, [](const Value& a, const Value& b) { return a + b; }, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2) return;
+            if (n->inputs[0] == n->inputs[1]) { n->inputs[0]->backward(seed + seed); return; }
+            if (wants(n->inputs[0])) n->inputs[0]->backward(seed);
+            if (wants(n->inputs[1])) n->inputs[1]->backward(seed);
+        });
+    }
+
+    Tensor operator-(const Tensor& o) const
+    {
+        return binary(o, [](const Value& a, const Value& b) { return a - b; }, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2 || n->inputs[0] == n->inputs[1]) return;
+            if (wants(n->inputs[0])) n->inputs[0]->backward(seed);
+            if (wants(n->inputs[1])) n->inputs[1]->backward(-seed);
+        });
+    }
+
+    Tensor operator*(const Tensor& o) const
+    {
+        return binary(o, [](const Value& a, const Value& b) { return a * b; }, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2) return;
+            if (n->inputs[0] == n->inputs[1]) {
+                const Value g = n->inputs[0]->value * seed;
+                n->inputs[0]->backward(g + g);
+                return;
+            }
+            if (wants(n->inputs[0])) n->inputs[0]->backward(n->inputs[1]->value * seed);
+            if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value * seed);
+        });
+    }
+
+    Tensor operator/(const Tensor& o) const
+    {
+        return binary(o, [](const Value& a, const Value& b) { return a / b; }, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2) return;
+            if (wants(n->inputs[0])) n->inputs[0]->backward(seed / n->inputs[1]->value);
+            if (wants(n->inputs[1]))
+                n->inputs[1]->backward(-n->inputs[0]->value * seed / (n->inputs[1]->value * n->inputs[1]->value));
+        });
+    }
+
+    Tensor operator-() const
+    {
+        Tensor r = makeResult(-value(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(-seed);
+        });
+        return r;
+    }
+
+    Tensor operator+(float s) const { return *this + scalar(s, false); }
+    Tensor operator-(float s) const { return *this - scalar(s, false); }
+    Tensor operator*(float s) const { return *this * scalar(s, false); }
+    Tensor operator/(float s) const { return *this / scalar(s, false); }
+    friend Tensor operator+(float s, const Tensor& t) { return t.scalar(s, true) + t; }
+    friend Tensor operator-(float s, const Tensor& t) { return t.scalar(s, true) - t; }
+    friend Tensor operator*(float s, const Tensor& t) { return t.scalar(s, true) * t; }
+    friend Tensor operator/(float s, const Tensor& t) { return t.scalar(s, true) / t; }
+
+    // ---- math (aixCore.hpp:2440-2480; backward :2123-2163) ------------------------------------------
+    Tensor exp() const
+    {
+        Tensor r = makeResult(value().exp(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed * n->value);
+        });
+        return r;
+    }
+
+    Tensor log() const
+    {
+        Tensor r = makeResult(value().log(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed / n->inputs[0]->value);
+        });
+        return r;
+    }
+
+    Tensor tanh() const
+    {
+        Tensor r = makeResult(value().tanh(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward((n->value * n->value).withScalar(&Device::sub, 1.0f, true) * seed);
+        });
+        return r;
+    }
+
+    Tensor sqrt() const
+    {
+        Tensor r = makeResult(value().sqrt(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(n->value.withScalar(&Device::div, 0.5f, true) * seed);
+        });
+        return r;
+    }
+
+    // ---- reductions (aixCore.hpp:2482-2521; backward :2165-2176, 2235-2252) --------------------
+    Tensor sum() const
+    {
+        Tensor r = makeResult(value().sum(), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.broadcastTo(n->inputs[0]->value.shape()));
+        });
+        return r;
+    }
+
+    Tensor sum(size_t dim, bool keepDim = false) const
+    {
+        Tensor r = makeResult(value().sum(dim, keepDim), isRequireGrad());
+        r.m_node->dim0 = dim; r.m_node->keepDim = keepDim;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            const Shape& orig = n->inputs[0]->value.shape();
+            n->inputs[0]->backward(n->keepDim ? seed.broadcastTo(orig) : seed.unsqueeze(n->dim0).broadcastTo(orig));
+        });
+        return r;
+    }
+
+    Tensor mean() const { return sum() / (float)value().size(); }
+    Tensor mean(size_t dim, bool keepDim = false) const { return sum(dim, keepDim) / (float)shape()[dim]; }
+
+    Tensor max(size_t dim, bool keepDim = false) const
+    {
+        Tensor r = makeResult(value().max(dim, keepDim), isRequireGrad());
+        r.m_node->dim0 = dim;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed * n->inputs[0]->value.argmaxIndices(n->dim0));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2557-2569; matmulBackwardFunc :2178-2194
+    Tensor matmul(const Tensor& o) const
+    {
+        Tensor r = makeResult(value().matmul(o.value()), isRequireGrad() || o.isRequireGrad(), !m_node->isLeaf || !o.m_node->isLeaf);
+        r.m_node->setBackward({m_node, o.m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2) return;
+            if (n->inputs[0] == n->inputs[1]) {
+                const Value xT = n->inputs[0]->value.transpose(0, 1);
+                n->inputs[0]->backward(seed.matmul(xT) + xT.matmul(seed));
+                return;
+            }
+            if (wants(n->inputs[0])) n->inputs[0]->backward(seed.matmul(n->inputs[1]->value.transpose(0, 1)));
+            if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value.transpose(0, 1).matmul(seed));
+        });
+        return r;
+    }
+
+private:
+    static bool wants(const NodePtr& n) { return n->requireGrad || n->retainGrad; }
+
+    // aixCore.hpp:2017-2024
+    static void defaultBackward(Node* n, const Value& seed)
+    {
+        if (n->requireGrad && !n->retainGrad) n->grad() += seed;
+    }
+
+    // aixCore.hpp:2783-2796
+    Tensor makeResult(Value v, bool anyGrad) const { return makeResult(std::move(v), anyGrad, !m_node->isLeaf); }
+    static Tensor makeResult(Value v, bool anyGrad, bool anyNonLeaf)
+    {
+        Tensor r;
+        r.m_node = std::make_shared<Node>(std::move(v), anyGrad);
+        r.m_node->isLeaf = !anyGrad && !anyNonLeaf;
+        r.m_node->backwardFn = defaultBackward;
+        return r;
+    }
+
+    // The scalar operand of `tensor op scalar`: rank-0 tensor seen through a broadcast view.  When
+    // the scalar is on the left it inherits requireGrad from the tensor (aixCore.hpp:2408-2438).
+    Tensor scalar(float s, bool onLeft) const
+    {
+        return Tensor(s, Shape{}, device(), dtype(), onLeft && isRequireGrad()).broadcastTo(shape());
+    }
+
+    template <class Fwd, class Bwd> Tensor binary(const Tensor& o, Fwd fwd, Bwd bwd) const
+    {
+        const Shape bc = shape() == o.shape() ? shape() : broadcastShapes(shape(), o.shape());
+        const Tensor lhs = broadcastTo(bc), rhs = o.broadcastTo(bc);
+        Tensor r = makeResult(fwd(lhs.value(), rhs.value()), isRequireGrad() || o.isRequireGrad(),
+                              !lhs.m_node->isLeaf || !rhs.m_node->isLeaf);
+        r.m_node->setBackward({lhs.m_node, rhs.m_node}, bwd);
+        return r;
+    }
+
+    NodePtr m_node;
+};
+
+inline Tensor matmul(const Tensor& a, const Tensor& b) { return a.matmul(b); }
+inline Tensor exp(const Tensor& a) { return a.exp(); }
+inline Tensor log(const Tensor& a) { return a.log(); }
+inline Tensor tanh(const Tensor& a) { return a.tanh(); }
+inline Tensor mean(const Tensor& a) { return a.mean(); }
+
+} // namespace aixfe

@@ -31,6 +31,8 @@ using aix::DeviceTensorParams;
 using aix::Shape;
 using aix::Stride;
 
+inline bool isFloat(DataType dt) { return static_cast<size_t>(dt) <= static_cast<size_t>(DataType::kBFloat16); }
+
 inline size_t numel(const Shape& s) { size_t n = 1; for (auto e : s) n *= e; return n; }
 
 inline Stride denseStrides(const Shape& s)
@@ -165,7 +167,13 @@ public:
 
     Value binary(BinaryFn fn, const Value& other) const
     {
-        if (other.m_dt != m_dt) throw std::invalid_argument("binary: element types differ");
+        if (other.m_dt != m_dt) {
+            // operands are first converted to the promoted type (aixCore.hpp:1616-1630); the drivers
+            // only ever mix a floating tensor with an integer mask, which promotes to the float type
+            const bool lf = isFloat(m_dt), rf = isFloat(other.m_dt);
+            if (lf == rf) throw std::invalid_argument("binary: unsupported mix of element types");
+            return lf ? binary(fn, other.to(m_dt)) : to(other.m_dt).binary(fn, other);
+        }
         if (m_shape == other.m_shape) {
             Value r(m_dev, m_dt, m_shape);
             (m_dev->*fn)(params(), other.params(), r.params());
@@ -228,6 +236,15 @@ public:
 
     void fill(float v) { m_dev->fill(&v, DataType::kFloat32, params()); }
 
+    // `value op scalar` as the reference's value class does it (aixCore.hpp:715-777): the scalar
+    // becomes a FULL-SHAPE filled tensor, then the ordinary binary operator runs.  (The float
+    // operators above follow its autograd class instead: rank-0 tensor + broadcast view, :2384-2438.)
+    Value withScalar(BinaryFn fn, float s, bool scalarFirst = false) const
+    {
+        const Value sc = full(m_dev, m_dt, m_shape, s);
+        return scalarFirst ? sc.binary(fn, *this) : binary(fn, sc);
+    }
+
     // ---- reductions ---------------------------------------------------------------------------
     Value sum() const
     {
@@ -274,9 +291,69 @@ public:
 
     Value mean() const { return sum() / (float)size(); }
 
+    // 1 where the element is the (first) maximum along `dim`, 0 elsewhere, int32 (aixCore.hpp:927-941).
+    Value argmaxIndices(size_t dim) const
+    {
+        Value r = full(m_dev, DataType::kInt32, m_shape, 0.0f);
+        m_dev->argmaxIndicesTo(params(), r.params(), dim);
+        return r;
+    }
+
+    // aixCore.hpp:1060-1087
+    Value unsqueeze(size_t dim) const
+    {
+        Value v = *this;
+        size_t inserted = 1;
+        if (!m_shape.empty() && dim < m_shape.size()) inserted = m_strides[dim] * m_shape[dim];
+        v.m_shape.insert(v.m_shape.begin() + (long)dim, 1);
+        v.m_strides.insert(v.m_strides.begin() + (long)dim, inserted);
+        return v;
+    }
+
+    // A strided window along `dim` (view; aixCore.hpp:1089-1145).
+    Value slice(size_t dim, size_t start, size_t end, size_t step = 1) const
+    {
+        if (dim >= m_shape.size() || step < 1 || start >= end || end > m_shape[dim]) throw std::invalid_argument("slice: bad range");
+        Value v = *this;
+        v.m_offset += start * m_strides[dim];
+        v.m_strides[dim] *= step;
+        v.m_shape[dim] = (end - start + step - 1) / step;
+        return v;
+    }
+
+    // Write `src` into that window of *this (in place; aixCore.hpp:1147-1204 with inPlace = true).
+    void sliceSetInPlace(const Value& src, size_t dim, size_t start, size_t end, size_t step = 1) const
+    {
+        m_dev->sliceSet(src.params(), params(), dim, start, end, step);
+    }
+
+    // aixCore.hpp:1348-1402: a fresh tensor, one sliceSet per part.
+    static Value cat(const std::vector<Value>& parts, size_t dim)
+    {
+        if (parts.empty()) throw std::invalid_argument("cat: no tensors");
+        Shape shape = parts[0].m_shape;
+        for (size_t i = 1; i < parts.size(); ++i) shape[dim] += parts[i].m_shape[dim];
+        Value r(parts[0].m_dev, parts[0].m_dt, shape);
+        size_t at = 0;
+        for (const auto& p : parts) { r.sliceSetInPlace(p, dim, at, at + p.m_shape[dim]); at += p.m_shape[dim]; }
+        return r;
+    }
+
+    // First element on the host, after a synchronize(); device memory is host-readable on both
+    // backends (plain memory on the CPU, large-BAR mapping on the GPU).
+    float item() const
+    {
+        if (m_dt != DataType::kFloat32) throw std::invalid_argument("item: f32 only");
+        m_dev->synchronize();
+        float v;
+        std::memcpy(&v, static_cast<const char*>(data()) + m_offset * sizeof(float), sizeof(float));
+        return v;
+    }
+
     Value squeeze(size_t dim) const
     {
         Value v = *this;
+        if (dim >= m_shape.size() || m_shape[dim] != 1) return v;
         v.m_shape.erase(v.m_shape.begin() + (long)dim);
         v.m_strides.erase(v.m_strides.begin() + (long)dim);
         return v;

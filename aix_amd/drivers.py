@@ -1,0 +1,66 @@
+"""ctypes binding of the native driver loops (libaixhip_bench.so): whole AIX-style programs
+(expression chains, reductions, GEMM sweeps, the MLP training loop) issued from C++ through the
+tensor front-end into DeviceHIP, so that no Python sits inside a step."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import device as D
+from ._build import library_path
+
+_PF = C.POINTER(C.c_float)
+_PPF = C.POINTER(_PF)
+_lib = None
+
+
+class BenchResult(C.Structure):
+    _fields_ = [("wall_s", C.c_double), ("gpu_ms", C.c_float), ("steps", C.c_int32), ("reserved", C.c_int32)]
+
+
+def load():
+    """Load libaixhip_bench.so.  Never builds, never falls back."""
+    global _lib
+    if _lib is None:
+        D.load()
+        path = library_path("libaixhip_bench.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError(f"{path} is not built; run __graft_entry__.build()")
+        lib = C.CDLL(path)
+        P = C.c_void_p
+        lib.aixbench_last_error.restype = C.c_char_p
+        lib.aixbench_fused_chain.argtypes = [P, C.c_uint64, C.c_uint64, P, P, P, C.c_int, C.c_int, C.POINTER(BenchResult), P]
+        lib.aixbench_reduce_item.argtypes = [P, C.c_int, C.c_uint64, C.c_uint64, P, P, C.c_int, C.c_int, C.POINTER(BenchResult), P]
+        lib.aixbench_matmul.argtypes = [P, C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64, P, P, C.c_int, C.c_int,
+                                        C.POINTER(BenchResult), P]
+        lib.aixbench_mlp.argtypes = [P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, _PF, _PF, _PPF, _PPF,
+                                     _PF, C.POINTER(C.c_double)]
+        _lib = lib
+    return _lib
+
+
+def run(fn, *args):
+    lib = load()
+    if getattr(lib, fn)(*args) != 0:
+        raise RuntimeError(f"{fn}: {lib.aixbench_last_error().decode()}")
+
+
+def _pointer_array(arrays):
+    arr = (_PF * len(arrays))()
+    for i, a in enumerate(arrays):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+        arr[i] = a.ctypes.data_as(_PF)
+    return arr
+
+
+def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data):
+    """Train the MLP (n_in -> hidden -> hidden -> n_out, ReLU, softmax + cross-entropy, Adam) for
+    `steps` steps on `dev` from host arrays data = (x, onehot, [w1, w2, w3], [b1, b2, b3]).
+    Returns (loss per step, seconds per step)."""
+    x, y, w, b = data
+    losses = np.zeros(steps, dtype=np.float32)
+    secs = np.zeros(steps, dtype=np.float64)
+    pw, pb = _pointer_array(w), _pointer_array(b)
+    run("aixbench_mlp", dev.handle, batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+        pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
+    return losses, secs

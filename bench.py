@@ -229,6 +229,35 @@ def main():
                            "ms_per_step": round(r.wall_s * 1e3 / steps_mm, 5),
                            "value": round(flops * steps_mm / r.wall_s / 1e12, 2), "unit": "TFLOP/s",
                            "roofline": roofline("mfma", flops / (r.gpu_ms / steps_mm * 1e-3) / 1e12, MFMA_PEAK_TFLOPS[dt_name], "TFLOP/s")})
+        # configs[3]: MLP training step (autograd + Adam); the CPU device runs the first steps of the same program
+        from aix_amd import drivers as GD
+        from oracle import drivers as OD
+        shape = (4096, 784, 2048, 10)
+        data = OD.mlp_data(*shape)
+        mlp_steps = 100
+        losses, secs = GD.mlp(dev, *shape, mlp_steps, 1e-3, data)
+        steady = secs[1:]                                   # step 0 carries the JIT compilations
+        flops = 2.0 * shape[0] * (shape[1] * shape[2] + shape[2] * shape[2] + shape[2] * shape[3])      # forward products
+        # backward: 4 traversals (softmax + cross-entropy reach the logits along 4 paths), each dW3, dH2, dW2, dH1, dW1
+        flops_step = flops + 4 * (2 * flops - 2.0 * shape[0] * shape[1] * shape[2])
+        mlp = {"workload": "configs[3] MLP 784-2048-2048-10, batch 4096, f32, ReLU, softmax + cross-entropy, Adam lr 1e-3, "
+                           "100 steps, loss read back every step",
+               "ms_per_step": round(float(steady.mean()) * 1e3, 4), "value": round(1.0 / float(steady.mean()), 2), "unit": "steps/s",
+               "first_step_ms": round(float(secs[0]) * 1e3, 2), "flop_per_step": flops_step,
+               "roofline": roofline("mfma", flops_step / float(steady.mean()) / 1e12, MFMA_PEAK_TFLOPS["f32"], "TFLOP/s"),
+               "loss": [round(float(l), 6) for l in losses[[0, 1, 2, 9, 49, 99]]]}
+        if not args.no_cpu:
+            threads = min(16, os.cpu_count() or 1)
+            cpu_steps = 2
+            want, cpu_secs, (ops, matmuls) = OD.oracle_mlp(*shape, cpu_steps, 1e-3, data, threads=threads)
+            rel = np.abs(losses[:cpu_steps].astype(np.float64) - want) / np.abs(want)
+            mlp["cpu_baseline"] = {"value": round(cpu_steps / float(cpu_secs.sum()), 4), "unit": "steps/s", "cores": threads, "kind": "port",
+                                   "sample": f"the first {cpu_steps} steps of the same program on the CPU oracle device "
+                                             f"({float(cpu_secs.sum()):.1f} s; {matmuls // cpu_steps} matmuls, {ops // cpu_steps} operator calls per step; "
+                                             f"matmul rows on {threads} threads, everything else on 1)"}
+            mlp["parity"] = {"checked_against": "cpu_baseline losses", "steps": cpu_steps, "max_rel_dev": float(rel.max()),
+                             "ok": bool(rel.max() <= 1e-4), "rule": "|loss_gpu - loss_cpu| <= 1e-4 |loss_cpu| on the first steps"}
+        extras.append(mlp)
         out["extras"] = extras
 
     dev.close()

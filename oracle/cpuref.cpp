@@ -182,6 +182,35 @@ inline uint64_t phys(const cpuref_tensor* t, uint64_t i)
     return pos;
 }
 
+// phys(t, i) for i = start, start + 1, ...: the same positions, produced by carrying a
+// multi-index instead of dividing anew for every element.  With `weight` (one multiplier per
+// dimension) it also carries sum(coordinate * weight), which is DstMap::map(i).
+struct Cursor {
+    const cpuref_tensor* t;
+    const uint64_t* weight;
+    uint64_t pos, mapped;
+    uint64_t idx[CPUREF_MAX_RANK];
+    Cursor(const cpuref_tensor* tensor, uint64_t start = 0, const uint64_t* w = nullptr) : t(tensor), weight(w), pos(tensor->offset), mapped(0)
+    {
+        for (int d = t->rank - 1; d >= 0; --d) {
+            const uint64_t ext = t->shape[d];
+            idx[d] = ext ? start % ext : 0;
+            if (ext) start /= ext;
+            pos += idx[d] * t->strides[d];
+            if (weight) mapped += idx[d] * weight[d];
+        }
+    }
+    inline void next()
+    {
+        for (int d = t->rank - 1; d >= 0; --d) {
+            if (++idx[d] < t->shape[d]) { pos += t->strides[d]; if (weight) mapped += weight[d]; return; }
+            pos -= (t->shape[d] - 1) * t->strides[d];
+            if (weight) mapped -= (t->shape[d] - 1) * weight[d];
+            idx[d] = 0;
+        }
+    }
+};
+
 // For every source dimension, the multiplier that maps its coordinate into the flat
 // index of the (smaller) destination.  Same walk as aixDeviceCPU.cpp:627-649: source
 // dims are scanned from the last; a destination dim is consumed when it equals the
@@ -228,6 +257,22 @@ template <class T> inline long double to_ld(T v)
     if constexpr (is_half16<T>::value) return (long double)(float)v; else return (long double)v;
 }
 
+// One output row of the i, j, k nest reordered to i, k, j: every out[i][j] still starts from
+// zero and receives a[i][k] * b[k][j] for k = 0, 1, ... in that order, each product rounded
+// before it is added (no contraction), so the result is bit-identical to the nest above; only
+// independent outputs are interleaved, which lets the j loop run on vector registers.
+template <class T>
+__attribute__((target_clones("avx2", "default")))
+void matmul_row_ikj(const T* arow, uint64_t as1, const T* b, uint64_t bs0, T* orow, uint64_t n, uint64_t kk)
+{
+    for (uint64_t j = 0; j < n; ++j) orow[j] = T(0);
+    for (uint64_t k = 0; k < kk; ++k) {
+        const T x = arow[k * as1];
+        const T* brow = b + k * bs0;
+        for (uint64_t j = 0; j < n; ++j) orow[j] = orow[j] + x * brow[j];
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -246,13 +291,14 @@ int cpuref_binary(int op, const cpuref_tensor* a, const cpuref_tensor* b, const 
     return by_dtype(out->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* pa = (const T*)a->data; const T* pb = (const T*)b->data; T* po = (T*)out->data;
+        Cursor ca(a), cb(b);
         if (op == CPUREF_POW) {
-            for (uint64_t i = 0; i < a->size; ++i)
-                po[i] = convert_value<long double, T>(std::pow(to_ld(pa[phys(a, i)]), to_ld(pb[phys(b, i)])));
+            for (uint64_t i = 0; i < a->size; ++i, ca.next(), cb.next())
+                po[i] = convert_value<long double, T>(std::pow(to_ld(pa[ca.pos]), to_ld(pb[cb.pos])));
             return;
         }
-        for (uint64_t i = 0; i < out->size; ++i) {
-            const T x = pa[phys(a, i)], y = pb[phys(b, i)];
+        for (uint64_t i = 0; i < out->size; ++i, ca.next(), cb.next()) {
+            const T x = pa[ca.pos], y = pb[cb.pos];
             po[i] = op == CPUREF_ADD ? t_add(x, y) : op == CPUREF_SUB ? t_sub(x, y)
                   : op == CPUREF_MUL ? t_mul(x, y) : t_div(x, y);
         }
@@ -269,8 +315,9 @@ int cpuref_unary(int op, const cpuref_tensor* a, const cpuref_tensor* out)
     return by_dtype(out->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* pa = (const T*)a->data; T* po = (T*)out->data;
-        for (uint64_t i = 0; i < a->size; ++i) {
-            const T x = pa[phys(a, i)];
+        Cursor ca(a);
+        for (uint64_t i = 0; i < a->size; ++i, ca.next()) {
+            const T x = pa[ca.pos];
             switch (op) {
                 case CPUREF_NEG:  po[i] = t_neg(x); break;
                 case CPUREF_SQRT: po[i] = convert_value<long double, T>(std::sqrt(to_ld(x))); break;
@@ -342,7 +389,8 @@ int cpuref_contiguous(const cpuref_tensor* src, const cpuref_tensor* dst)
     return by_dtype(src->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* ps = (const T*)src->data; T* pd = (T*)dst->data;
-        for (uint64_t i = 0; i < dst->size; ++i) pd[i] = ps[phys(src, i)];
+        Cursor cs(src);
+        for (uint64_t i = 0; i < dst->size; ++i, cs.next()) pd[i] = ps[cs.pos];
     });
 }
 
@@ -435,9 +483,10 @@ int cpuref_reduce_to(const cpuref_tensor* src, const cpuref_tensor* dst)
         using T = decltype(tag);
         const T* ps = (const T*)src->data; T* pd = (T*)dst->data;
         DstMap m; m.build(dst->shape, dst->rank, src->shape, src->rank);
-        for (uint64_t i = 0; i < src->size; ++i) {
-            T& slot = pd[m.map(i, src->shape, src->rank)];
-            slot = t_add(slot, ps[phys(src, i)]);
+        Cursor cs(src, 0, m.weight);
+        for (uint64_t i = 0; i < src->size; ++i, cs.next()) {
+            T& slot = pd[cs.mapped];
+            slot = t_add(slot, ps[cs.pos]);
         }
     });
 }
@@ -449,9 +498,10 @@ int cpuref_max_to(const cpuref_tensor* src, const cpuref_tensor* dst)
         using T = decltype(tag);
         const T* ps = (const T*)src->data; T* pd = (T*)dst->data;
         DstMap m; m.build(dst->shape, dst->rank, src->shape, src->rank);
-        for (uint64_t i = 0; i < src->size; ++i) {
-            T& slot = pd[m.map(i, src->shape, src->rank)];
-            slot = t_max(slot, ps[phys(src, i)]);
+        Cursor cs(src, 0, m.weight);
+        for (uint64_t i = 0; i < src->size; ++i, cs.next()) {
+            T& slot = pd[cs.mapped];
+            slot = t_max(slot, ps[cs.pos]);
         }
     });
 }
@@ -493,9 +543,10 @@ int cpuref_argmax_indices_to(const cpuref_tensor* src, const cpuref_tensor* dst,
         std::vector<char> seen(slots, 0);
         std::vector<uint64_t> where(slots, 0);
         DstMap m; m.build(rshape, dst->rank, src->shape, src->rank);
-        for (uint64_t i = 0; i < src->size; ++i) {
-            const uint64_t s = m.map(i, src->shape, src->rank);
-            const T x = ps[phys(src, i)];
+        Cursor cs(src, 0, m.weight);
+        for (uint64_t i = 0; i < src->size; ++i, cs.next()) {
+            const uint64_t s = cs.mapped;
+            const T x = ps[cs.pos];
             if (!seen[s] || t_gt(x, best[s])) { seen[s] = 1; best[s] = x; where[s] = i; }
         }
         for (uint64_t s = 0; s < slots; ++s) pd[(int32_t)where[s]] = 1;
@@ -512,6 +563,35 @@ int cpuref_matmul(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_t
 int cpuref_matmul_rows(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads)
 {
     if (a->rank != 2 || b->rank != 2) return CPUREF_EINVAL;
+    if (out->dtype == CPUREF_F32 || out->dtype == CPUREF_F64) {
+        // f32 / f64: the reordered nest.  B is first copied to a dense [K, N] array if its rows are not unit-stride.
+        return by_dtype(out->dtype, [&](auto tag) {
+            using T = decltype(tag);
+            if constexpr (std::is_same_v<T, float> || std::is_same_v<T, double>) {
+                const uint64_t m = a->shape[0], n = b->shape[1], kk = a->shape[1];
+                const T* pa = (const T*)a->data + a->offset; T* po = (T*)out->data;
+                const T* pb = (const T*)b->data + b->offset;
+                uint64_t bs0 = b->strides[0];
+                std::vector<T> dense;
+                if (b->strides[1] != 1 && n > 1) {
+                    dense.resize(kk * n);
+                    for (uint64_t k = 0; k < kk; ++k) for (uint64_t j = 0; j < n; ++j) dense[k * n + j] = pb[k * b->strides[0] + j * b->strides[1]];
+                    pb = dense.data(); bs0 = n;
+                }
+                auto rows = [&](uint64_t r0, uint64_t r1) {
+                    for (uint64_t i = r0; i < r1; ++i) matmul_row_ikj<T>(pa + i * a->strides[0], a->strides[1], pb, bs0, po + i * n, n, kk);
+                };
+                if (threads <= 1 || m < 2) { rows(0, m); return; }
+                std::vector<std::thread> pool;
+                const uint64_t per = (m + threads - 1) / threads;
+                for (int t = 0; t < threads; ++t) {
+                    const uint64_t r0 = std::min<uint64_t>(m, t * per), r1 = std::min<uint64_t>(m, r0 + per);
+                    if (r0 < r1) pool.emplace_back(rows, r0, r1);
+                }
+                for (auto& th : pool) th.join();
+            }
+        });
+    }
     return by_dtype(out->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* pa = (const T*)a->data; const T* pb = (const T*)b->data; T* po = (T*)out->data;

@@ -1,0 +1,97 @@
+"""ctypes binding of the driver loops on the CPU side: oracle/liboracle_drivers.so (the
+front-end + autograd + Adam headers of the product compiled against the oracle device) and,
+where it was built, oracle/_ref/libaixref_drivers.so (the same loop written with the reference's
+own classes).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, __graft_entry__.smoke() and bench.py's
+cpu_baseline leg.  The product package never imports this module.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+_PF = C.POINTER(C.c_float)
+_PPF = C.POINTER(_PF)
+
+
+def mlp_data(batch, n_in, hidden, n_out, seed_w=0, seed_x=5, seed_y=6):
+    """Synthetic inputs of the MLP configuration: X ~ U(0,1), one-hot labels uniform over the
+    classes, weights and biases U(-1,1)/sqrt(fan_in); all f32, generated on the host."""
+    x = np.random.default_rng(seed_x).random((batch, n_in), dtype=np.float32)
+    labels = np.random.default_rng(seed_y).integers(0, n_out, size=batch)
+    y = np.zeros((batch, n_out), dtype=np.float32)
+    y[np.arange(batch), labels] = 1.0
+    rng = np.random.default_rng(seed_w)
+    dims = [(n_in, hidden), (hidden, hidden), (hidden, n_out)]
+    w = [((rng.random(d, dtype=np.float32) * 2 - 1) / np.float32(np.sqrt(d[0]))).astype(np.float32) for d in dims]
+    b = [((rng.random((1, d[1]), dtype=np.float32) * 2 - 1) / np.float32(np.sqrt(d[0]))).astype(np.float32) for d in dims]
+    return x, y, w, b
+
+
+def pointer_array(arrays):
+    """float** over a list of contiguous f32 arrays (keep the list alive while it is used)."""
+    arr = (_PF * len(arrays))()
+    for i, a in enumerate(arrays):
+        assert a.dtype == np.float32 and a.flags.c_contiguous
+        arr[i] = a.ctypes.data_as(_PF)
+    return arr
+
+
+_oracle = None
+_ref = None
+
+
+def oracle_lib():
+    global _oracle
+    if _oracle is None:
+        path = os.path.join(HERE, "liboracle_drivers.so")
+        if not os.path.exists(path):
+            from . import cpuref
+            cpuref.build(ref=False)
+        _oracle = C.CDLL(path)
+        _oracle.oracle_mlp.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float,
+                                       _PF, _PF, _PPF, _PPF, _PF, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
+        _oracle.oracle_drivers_last_error.restype = C.c_char_p
+    return _oracle
+
+
+def ref_lib():
+    """The loop on the reference's own classes, or None where oracle/_ref was not built."""
+    global _ref
+    if _ref is None:
+        path = os.path.join(HERE, "_ref", "libaixref_drivers.so")
+        if not os.path.exists(path):
+            return None
+        _ref = C.CDLL(path)
+        _ref.aixref_mlp.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float,
+                                    _PF, _PF, _PPF, _PPF, _PF, C.POINTER(C.c_uint64)]
+        _ref.aixref_drivers_last_error.restype = C.c_char_p
+    return _ref
+
+
+def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1):
+    """Losses per step, seconds per step and (operator calls, matmul calls) of the oracle run."""
+    x, y, w, b = data
+    losses = np.zeros(steps, dtype=np.float32)
+    secs = np.zeros(steps, dtype=np.float64)
+    counts = (C.c_uint64 * 2)()
+    pw, pb = pointer_array(w), pointer_array(b)
+    rc = oracle_lib().oracle_mlp(threads, batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+                                 pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), counts)
+    if rc != 0:
+        raise RuntimeError(oracle_lib().oracle_drivers_last_error().decode())
+    return losses, secs, (int(counts[0]), int(counts[1]))
+
+
+def ref_mlp(batch, n_in, hidden, n_out, steps, lr, data):
+    x, y, w, b = data
+    losses = np.zeros(steps, dtype=np.float32)
+    counts = (C.c_uint64 * 2)()
+    pw, pb = pointer_array(w), pointer_array(b)
+    rc = ref_lib().aixref_mlp(batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+                              pw, pb, losses.ctypes.data_as(_PF), counts)
+    if rc != 0:
+        raise RuntimeError(ref_lib().aixref_drivers_last_error().decode())
+    return losses, int(counts[1])

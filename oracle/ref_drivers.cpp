@@ -1,0 +1,74 @@
+// ref_drivers.cpp -- the benchmark's MLP training loop written against the reference's OWN tensor,
+// autograd, nn and optimizer classes (<aix.hpp>) on its own aix::DeviceCPU.
+//
+// TEST INFRASTRUCTURE ONLY, built only where the reference tree is present (oracle/Makefile,
+// target `ref`), compiled with the reference's sources from where they lie.  It pins the
+// front-end restatement (aix_amd/csrc/frontend): the same model, data and loop run through
+// aixfe::Tensor on the oracle device must give the same losses bit for bit and the same number of
+// matmul calls, which shows that both generate the same operator stream.
+
+#include <aix.hpp>
+
+#include <cstdio>
+#include <cstdint>
+
+namespace {
+
+struct CountingCPU final : aix::DeviceCPU {
+    uint64_t matmuls{0};
+    void matmul(const aix::DeviceTensorParams& a, const aix::DeviceTensorParams& b, const aix::DeviceTensorParams& r) override
+    {
+        ++matmuls;
+        aix::DeviceCPU::matmul(a, b, r);
+    }
+};
+
+aix::Tensor relu(const aix::Tensor& x, aix::Device* dev)
+{
+    aix::Shape lifted = x.shape();
+    lifted.insert(lifted.begin(), 1);
+    const aix::Tensor zeros(0.0f, lifted, { .m_dtype = x.dataType(), .m_device = dev });
+    return aix::Tensor::cat({x.unsqueeze(0), zeros}, 0).max(0);
+}
+
+thread_local char g_err[512] = "";
+
+} // namespace
+
+extern "C" {
+
+const char* aixref_drivers_last_error(void) { return g_err; }
+
+int aixref_mlp(uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
+               const float* x, const float* y, const float* const* w, const float* const* b, float* losses, uint64_t* counts)
+{
+    try {
+        CountingCPU dev;
+        const aix::TensorOptions plain{ .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
+        const aix::TensorOptions param{ .m_requireGrad = true, .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
+        const auto F32 = aix::DataType::kFloat32;
+        aix::Tensor X(x, batch * in, F32, aix::Shape{batch, in}, plain);
+        aix::Tensor Y(y, batch * out, F32, aix::Shape{batch, out}, plain);
+        aix::Tensor w1(w[0], in * hidden, F32, aix::Shape{in, hidden}, param), b1(b[0], hidden, F32, aix::Shape{1, hidden}, param);
+        aix::Tensor w2(w[1], hidden * hidden, F32, aix::Shape{hidden, hidden}, param), b2(b[1], hidden, F32, aix::Shape{1, hidden}, param);
+        aix::Tensor w3(w[2], hidden * out, F32, aix::Shape{hidden, out}, param), b3(b[2], out, F32, aix::Shape{1, out}, param);
+        aix::optim::Adam opt(std::vector<aix::Tensor>{w1, b1, w2, b2, w3, b3}, lr);
+        aix::nn::Softmax softmax(1, true);
+        aix::nn::CrossEntropyLoss lossFn;
+        for (int s = 0; s < steps; ++s) {
+            opt.zeroGrad();
+            auto h1 = relu(aix::matmul(X, w1) + b1, &dev);
+            auto h2 = relu(aix::matmul(h1, w2) + b2, &dev);
+            auto logits = aix::matmul(h2, w3) + b3;
+            auto loss = lossFn(softmax.forward(logits), Y);
+            loss.backward();
+            opt.step();
+            dev.synchronize();
+            losses[s] = loss.value().item<float>();
+        }
+        if (counts) counts[1] = dev.matmuls;
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
+
+} // extern "C"

@@ -1,0 +1,35 @@
+"""The autograd / nn / optimizer front-end (aix_amd/csrc/frontend) against the reference's own
+classes: the same MLP training loop, once through aixfe::Tensor on the oracle device and once
+through aix::Tensor on the reference's DeviceCPU (oracle/_ref, built from the reference's sources).
+Both devices are bit-identical operator by operator (tests/test_oracle_vs_ref.py), so equal loss
+traces, bit for bit over many Adam steps, and equal matmul counts show that the front-end issues
+the operator stream the reference's autograd issues (same backward formulas, same path-wise
+recursion, same scalar handling)."""
+import numpy as np
+import pytest
+
+from oracle import drivers
+
+pytestmark = pytest.mark.skipif(drivers.ref_lib() is None, reason="oracle/_ref not built (no reference tree)")
+
+
+@pytest.mark.parametrize("shape", [(8, 12, 16, 5), (32, 20, 24, 10), (5, 7, 3, 2)], ids=str)
+def test_mlp_loss_trace_bit_identical(shape):
+    batch, n_in, hidden, n_out = shape
+    steps = 25
+    data = drivers.mlp_data(batch, n_in, hidden, n_out)
+    got, _, (ops, matmuls) = drivers.oracle_mlp(batch, n_in, hidden, n_out, steps, 1e-3, data)
+    want, ref_matmuls = drivers.ref_mlp(batch, n_in, hidden, n_out, steps, 1e-3, data)
+    assert np.all(np.isfinite(want)) and want[-1] < want[0], "reference loss should fall"
+    assert got.view(np.uint32).tolist() == want.view(np.uint32).tolist()
+    assert matmuls == ref_matmuls
+    # 3 forward products + 4 backward traversals (softmax and cross-entropy reach the logits
+    # along 4 paths) of 5 products each (dW3, dH2, dW2, dH1, dW1) per step
+    assert matmuls == steps * (3 + 4 * 5)
+
+
+def test_threads_do_not_change_the_trace():
+    data = drivers.mlp_data(64, 30, 40, 10)
+    one, _, _ = drivers.oracle_mlp(64, 30, 40, 10, 5, 1e-3, data, threads=1)
+    four, _, _ = drivers.oracle_mlp(64, 30, 40, 10, 5, 1e-3, data, threads=4)
+    assert one.view(np.uint32).tolist() == four.view(np.uint32).tolist()
