@@ -4,12 +4,14 @@
 
 #include "../../../include/aixhip_kernels.h"
 #include "hipgen.hpp"
+#include "scalar_convert.hpp"
 
 #include <algorithm>
 #include <array>
 #include <cstring>
 #include <deque>
 #include <iostream>
+#include <limits>
 #include <stdexcept>
 
 namespace aix {
@@ -610,22 +612,57 @@ void DeviceHIP::contiguous(const DeviceTensorParams& src, const DeviceTensorPara
     check(aixk_contiguous(m_ctx, &ps, &pd));
 }
 
+// The front-end always initialises the destination of reduceTo / maxTo right before the call
+// (fill(0) / fillMin(), aixCore.hpp:632-639, 873-891).  While that fill is still waiting in the
+// planner's window it is taken out and handed to the reduction kernel as the value every
+// destination element "holds", which saves the fill's launch and its pass over dst.
+static bool lowestBits(DataType dt, uint64_t* bits)
+{
+    switch (dt) {
+        case DataType::kFloat64:  { const double v = -std::numeric_limits<double>::max(); std::memcpy(bits, &v, 8); return true; }
+        case DataType::kFloat32:  { const float v = -std::numeric_limits<float>::max(); std::memcpy(bits, &v, 4); return true; }
+        case DataType::kFloat16:  *bits = 0xFBFFu; return true;
+        case DataType::kBFloat16: *bits = 0xFF7Fu; return true;
+        case DataType::kInt64:    { const int64_t v = std::numeric_limits<int64_t>::min(); std::memcpy(bits, &v, 8); return true; }
+        case DataType::kInt32:    { const int32_t v = std::numeric_limits<int32_t>::min(); std::memcpy(bits, &v, 4); return true; }
+        case DataType::kInt16:    { const int16_t v = std::numeric_limits<int16_t>::min(); std::memcpy(bits, &v, 2); return true; }
+        case DataType::kInt8:     { const int8_t v = std::numeric_limits<int8_t>::min(); std::memcpy(bits, &v, 1); return true; }
+        case DataType::kUInt8:    *bits = 0; return true;
+    }
+    return false;
+}
+
+bool DeviceHIP::takeInit(const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t* bits)
+{
+    if (src.data == dst.data || src.size == 0) return false;
+    aixhip::fuse::OpRecord fill;
+    if (!m_engine->takeTrailingFill(dst, &fill)) return false;
+    *bits = 0;
+    if (fill.type == OpType::FillMin) return lowestBits(dst.dtype, bits);
+    const auto v = aixhip::scalar::decode(fill.scalarData.data(), static_cast<int>(fill.scalarDType));
+    return aixhip::scalar::encode(v, static_cast<int>(dst.dtype), bits) != 0;
+}
+
 void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::reduceTo() requires matching source and destination data types.");
     requireDevice(dst, "reduceTo");
+    uint64_t init = 0;
+    const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
-    check(aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));
+    check(folded ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));
 }
 
 void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::maxTo() requires matching source and destination data types.");
     requireDevice(dst, "maxTo");
+    uint64_t init = 0;
+    const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "maxTo"); toPod(dst, &pd, "maxTo");
-    check(aixk_reduce_to(m_ctx, AIXK_MAX, &ps, &pd));
+    check(folded ? aixk_reduce_to_init(m_ctx, AIXK_MAX, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_MAX, &ps, &pd));
 }
 
 void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)

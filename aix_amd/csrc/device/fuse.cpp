@@ -625,6 +625,25 @@ void FuseEngine::flush()
     m_externalReads.clear();
 }
 
+bool FuseEngine::takeTrailingFill(const DeviceTensorParams& output, OpRecord* fill)
+{
+    if (m_flushing || !output.data) return false;
+    for (size_t k = m_pending.size(); k-- > 0;) {
+        const OpRecord& op = m_pending[k];
+        const bool reads = op.type != OpType::Fill && op.type != OpType::FillMin &&
+                           (op.input0.data == output.data || (op.hasInput1 && op.input1.data == output.data));
+        if (reads) return false;
+        if (op.output.data != output.data) continue;
+        if ((op.type != OpType::Fill && op.type != OpType::FillMin) || op.output.dtype != output.dtype ||
+            op.output.offset != output.offset || op.output.size != output.size || !output.isContiguous || !op.output.isContiguous)
+            return false;
+        *fill = op;
+        m_pending.erase(m_pending.begin() + (long)k);
+        return true;
+    }
+    return false;
+}
+
 void FuseEngine::recordExternalRead(const void* buffer) { if (buffer) m_externalReads.insert(buffer); }
 void FuseEngine::retainBuffer(void* buffer) { if (buffer) m_live.insert(buffer); }
 void FuseEngine::releaseBuffer(void* buffer) { if (buffer) { m_live.erase(buffer); m_externalReads.erase(buffer); } }

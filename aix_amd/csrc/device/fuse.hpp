@@ -120,6 +120,10 @@ public:
     const FlushDiagnostics& lastFlushDiagnostics() const;
     size_t pendingOps() const { return m_pending.size(); }
 
+    // If the newest pending operator touching output.data is a fill / fillMin of exactly this dense
+    // tensor, remove it from the window and hand it over (the caller folds it into the operator
+    // it is about to run eagerly); false and no change otherwise.
+    bool takeTrailingFill(const DeviceTensorParams& output, OpRecord* fill);
     void recordExternalRead(const void* buffer);   // the buffer is about to be read outside the planner
     void retainBuffer(void* buffer);               // allocate(): results written here must reach memory
     void releaseBuffer(void* buffer);              // deallocate(): nobody will read it after the window

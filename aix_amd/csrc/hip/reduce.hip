@@ -130,22 +130,30 @@ template <class Op> __device__ __forceinline__ typename Op::Acc block_reduce(typ
 
 // ---- landing a finished accumulator --------------------------------------------------------------
 struct Finish {
-    int into;                // 1: combine with what dst holds (reduceTo/maxTo); 0: overwrite (sum/max)
+    int into;                // 1: combine with what dst holds (reduceTo/maxTo); 0: overwrite (sum/max);
+                             // 2: combine with `init` as if dst held it everywhere (dst itself is never read)
     int onehot;              // argmax: write 1 at the winner's flat index instead of an index per slot
     u64 q_stride, q_extent;  // argmax along a dim: stored index = (flat / q_stride) % q_extent; q_stride 0: store flat
+    u64 init;                // into == 2: the value, in the low bytes, in the destination's element type
 };
+
+template <class T> __device__ __forceinline__ T held(const Finish& f, const T* dst, u64 slot)
+{
+    if (f.into == 2) { T v; __builtin_memcpy(&v, &f.init, sizeof(T)); return v; }
+    return dst[slot];
+}
 
 // `first` = value of the slot's first element (only read by max in overwrite mode);
 // `first_flat` = flat logical index of the slot's first element (only read by argmax).
 template <class T> __device__ __forceinline__ void land(SumOp<T>, const Finish& f, T* dst, u64 slot, typename SumOp<T>::Acc acc, T, u64)
 {
     typedef typename SumOp<T>::Acc A;
-    if constexpr (traits<T>::is_int) dst[slot] = f.into ? (T)((A)dst[slot] + acc) : (T)acc;
-    else dst[slot] = f.into ? down<T>(up(dst[slot]) + acc) : down<T>(acc);
+    if constexpr (traits<T>::is_int) dst[slot] = f.into ? (T)((A)held(f, dst, slot) + acc) : (T)acc;
+    else dst[slot] = f.into ? down<T>(up(held(f, dst, slot)) + acc) : down<T>(acc);
 }
 template <class T> __device__ __forceinline__ void land(MaxOp<T>, const Finish& f, T* dst, u64 slot, typename MaxOp<T>::Acc acc, T first, u64)
 {
-    if (f.into) { if (acc > up(dst[slot])) dst[slot] = down<T>(acc); }       // NaN in dst: '>' is false, it stays
+    if (f.into) { const T was = held(f, dst, slot); if (acc > up(was)) dst[slot] = down<T>(acc); else if (f.into == 2) dst[slot] = was; }   // NaN in dst: '>' is false, it stays
     else dst[slot] = e_isnan(first) ? first : down<T>(acc);                   // a leading NaN sticks
 }
 template <class T> __device__ __forceinline__ void land(ArgOp<T>, const Finish& f, i32* dst, u64 slot, typename ArgOp<T>::Acc acc, T, u64 first_flat)
@@ -527,7 +535,7 @@ int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const a
     AIXK_REQUIRE(out->data != nullptr, "reduce: null result");
     if (a->size == 0 && kind == AIXK_SUM) return aixk_zero(ctx, out->data, aixk_dtype_size(out->dtype));
     AIXK_REQUIRE(a->size > 0 && a->size == numel(a), "reduce: empty or inconsistent source");
-    Finish fin{0, 0, 0, 0};
+    Finish fin{0, 0, 0, 0, 0};
     if (kind == AIXK_SUM || kind == AIXK_MAX) {
         AIXK_REQUIRE(a->dtype == out->dtype, "reduce: operand must have the result's element type");
         return by_dtype(out->dtype, [&](auto tag) {
@@ -550,9 +558,22 @@ int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const a
     });
 }
 
+static int32_t reduce_to_impl(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, const uint64_t* init);
+
 int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst)
 {
+    return reduce_to_impl(ctx, kind, src, dst, nullptr);
+}
+
+int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t init_bits)
+{
+    return reduce_to_impl(ctx, kind, src, dst, &init_bits);
+}
+
+static int32_t reduce_to_impl(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, const uint64_t* init)
+{
     AIXK_TRY(set_device(ctx));
+    if (init && src->size == 0 && valid_tensor(dst)) return aixk_fill(ctx, init, dst->dtype, dst);
     AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "reduceTo: bad operand descriptor");
     AIXK_REQUIRE(kind == AIXK_SUM || kind == AIXK_MAX, "reduceTo: unknown kind %d", kind);
     AIXK_REQUIRE(src->dtype == dst->dtype, "reduceTo: element types differ");          // aixDeviceMetal.cpp:787-790
@@ -562,7 +583,12 @@ int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const 
     dst_weights(dst->shape, dst->rank, src->shape, src->rank, weight);
     RedPlan plan;
     if (!make_plan(src, weight, &plan)) return fail(AIXK_EINVAL, "reduceTo: view does not collapse to %d dims", kMaxDims);
-    const Finish fin{1, 0, 0, 0};
+    if (init && (dst->size != plan.slots || plan.red == 0)) {
+        // not one landing per destination element: initialise the ordinary way, then accumulate
+        AIXK_TRY(aixk_fill(ctx, init, dst->dtype, dst));
+        init = nullptr;
+    }
+    const Finish fin{init ? 2 : 1, 0, 0, 0, init ? *init : 0};
     return by_dtype(src->dtype, [&](auto tag) {
         typedef decltype(tag) T;
         if (kind == AIXK_SUM) return run_plan<SumOp<T>, T>(ctx, src, (T*)dst->data, plan, fin);

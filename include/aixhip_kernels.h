@@ -122,6 +122,11 @@ int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const a
 /* dst (op)= reduction of src over the dims dst lacks: Device::reduceTo / maxTo
  * (aixDeviceCPU.cpp:440-466).  Accumulates INTO dst (caller pre-initialises). kind = SUM|MAX. */
 int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst);
+/* The same with the pre-initialisation folded in: every dst element is taken to hold `init_bits`
+ * (a value of dst's element type in the low bytes) and is written exactly once, never read.  It is
+ * what fill(0) / fillMin() followed by reduceTo / maxTo computes (aixCore.hpp:632-639, 873-891)
+ * without the separate fill pass over dst. */
+int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t init_bits);
 /* Device::argmaxTo / argmaxIndicesTo (aixDeviceCPU.cpp:275-298, 320-360). onehot=1 scatters ones
  * into the pre-zeroed int32 dst of src's shape. */
 int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t dim);

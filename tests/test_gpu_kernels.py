@@ -438,6 +438,32 @@ ROUTE_CASES = [  # (source shape, view kind, destination shape) chosen to hit ev
 
 
 @pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_reduce_to_with_folded_initialisation(gpu, dtype):
+    """aixk_reduce_to_init(init) == fill(init) followed by aixk_reduce_to, bit for bit (same kernels,
+    the destination's old contents replaced by a constant), on every route; and with garbage in dst
+    beforehand to show dst is never read.  MAX with the lowest value is what max(dim) issues."""
+    rng = np.random.default_rng(19500 + dtype)
+    lowest = {O.F64: np.array([-np.finfo(np.float64).max]), O.F32: np.array([-np.finfo(np.float32).max], np.float32),
+              O.F16: np.array([0xFBFF], np.uint16), O.BF16: np.array([0xFF7F], np.uint16),
+              O.I64: np.array([np.iinfo(np.int64).min]), O.I32: np.array([np.iinfo(np.int32).min], np.int32),
+              O.I16: np.array([np.iinfo(np.int16).min], np.int16), O.I8: np.array([-128], np.int8), O.U8: np.array([0], np.uint8)}[dtype]
+    for shape, kind, dshape in ROUTE_CASES:
+        src = T.view_tensor(rng, dtype, shape, kind, int_span=20)
+        _, ds = gpu.put(src)
+        for code, bits_arr in ((K.SUM, np.zeros(1, O.NP_STORAGE[dtype])), (K.SUM, O.to_storage(np.array([3.0]), dtype)), (K.MAX, lowest)):
+            bits = int.from_bytes(bits_arr.tobytes()[:O.ITEMSIZE[dtype]], "little")
+            filled = T.HostTensor(np.resize(bits_arr.view(O.NP_STORAGE[dtype]), max(1, int(np.prod(dshape)))).copy(), dtype, dshape)
+            pa, da = gpu.put(filled)
+            G.run_gpu(gpu, "aixk_reduce_to", code, G.ref(ds), G.ref(da))
+            want = gpu.fetch(pa, filled.storage)
+            garbage = T.contiguous_tensor(rng, dtype, dshape, int_span=50)
+            pb, db = gpu.put(garbage)
+            G.run_gpu(gpu, "aixk_reduce_to_init", code, G.ref(ds), G.ref(db), C.c_uint64(bits))
+            T.assert_same_bits_nan_ok(gpu.fetch(pb, filled.storage), want, dtype, f"reduce_to_init {NAMES[dtype]} {shape}->{dshape} {kind} code {code}")
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
 def test_reduce_to_and_max_to(gpu, dtype):
     rng = np.random.default_rng(19000 + dtype)
     cases = list(ROUTE_CASES)
