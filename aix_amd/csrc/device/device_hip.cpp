@@ -48,6 +48,7 @@ struct Cooling {
 
 struct Extras {
     std::deque<Cooling> cooling;
+    unsigned flushesSinceEvent{0};
     std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
     uint64_t hits{0}, misses{0};
 };
@@ -246,10 +247,16 @@ void DeviceHIP::deallocate(void* memory)
 }
 
 // Called once the recorded work that might touch freed blocks has been enqueued.
+// An event costs a marker packet between two kernels (a few microseconds of idle GPU), so it is
+// not recorded after every flush: freed blocks wait until 16 flushes have passed or until they
+// amount to 32 MiB and an eighth of what the device holds otherwise, whichever comes first.
 void DeviceHIP::releaseLimbo()
 {
     if (m_limbo.empty()) return;
     auto& ex = extras()[this];
+    const size_t enough = std::max<size_t>(size_t(32) << 20, (m_liveBytes + m_pooledBytes) / 8);
+    if (++ex.flushesSinceEvent < 16 && m_limboBytes < enough) return;
+    ex.flushesSinceEvent = 0;
     Cooling c{};
     if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
         c.blocks.swap(m_limbo);
@@ -293,6 +300,11 @@ void DeviceHIP::synchronize()
         aixk_event_destroy(m_ctx, c.event);
     }
     ex.cooling.clear();
+    // everything recorded has been enqueued and has finished: blocks freed since the last event are idle too
+    for (auto& b : m_limbo) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+    m_limbo.clear();
+    m_limboBytes = 0;
+    ex.flushesSinceEvent = 0;
 }
 
 void DeviceHIP::copyToHost(void* dstHost, const void* srcDevice, size_t bytes)

@@ -50,6 +50,7 @@ template <class W> struct ArgAcc { W v; u32 idx; u32 flags; };
 template <class T> struct SumOp {
     typedef typename sum_acc<T>::type Acc;
     typedef T Out;
+    static constexpr bool kTracksIndex = false;
     static __device__ __forceinline__ Acc init() { return (Acc)0; }
     static __device__ __forceinline__ Acc load(T x, u64, bool) { return (Acc)up(x); }
     static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return a + b; }
@@ -59,6 +60,7 @@ template <class T> struct SumOp {
 template <class T> struct MaxOp {
     typedef typename traits<T>::W Acc;
     typedef T Out;
+    static constexpr bool kTracksIndex = false;
     static __device__ __forceinline__ Acc init() { return neg_inf<Acc>(); }
     static __device__ __forceinline__ Acc load(T x, u64, bool) { const Acc w = up(x); return w != w ? neg_inf<Acc>() : w; }
     static __device__ __forceinline__ Acc combine(Acc a, Acc b) { return b > a ? b : a; }
@@ -69,6 +71,7 @@ template <class T> struct ArgOp {
     typedef typename traits<T>::W W;
     typedef ArgAcc<W> Acc;
     typedef i32 Out;
+    static constexpr bool kTracksIndex = true;
     static __device__ __forceinline__ Acc init() { Acc a; a.v = neg_inf<W>(); a.idx = ~0u; a.flags = 0; return a; }
     // In-order scan by one lane: indices only grow, so an equal value never replaces the holder.
     static __device__ __forceinline__ void step(Acc& a, T x, u64 flat, bool first)
@@ -320,10 +323,15 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ s
                 const u64 r = r0 + (u64)k * kWaves;
                 if (r < r_end) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e)
-                        Op::step(acc[e], x[k].v[e], s.flat + r * p.r_flat[0] + (c0 + e) * p.k_flat[p.nk - 1], r == 0);
+                    for (int e = 0; e < VEC; ++e) Op::step(acc[e], x[k].v[e], r, r == 0);     // the row stands in for the flat index
                 }
             }
+        }
+        // A lane scans one column with ascending rows, so the row orders candidates exactly as the
+        // flat index would; the (64-bit) flat index is formed once per column, not per element.
+        if constexpr (Op::kTracksIndex) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) if (acc[e].flags & 1u) acc[e].idx = (u32)(s.flat + (u64)acc[e].idx * p.r_flat[0] + (c0 + e) * p.k_flat[p.nk - 1]);
         }
     }
 #pragma unroll
@@ -342,18 +350,39 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ s
     }
 }
 
-// second stage of `outer` when rows were split over several workgroups
+// second stage of `outer` when rows were split over several workgroups: 64 slots per workgroup,
+// the four waves take every fourth chunk (independent loads in flight), LDS folds the four.
 template <class Op, class T>
 __global__ __launch_bounds__(kBlock) void reduce_outer_finish_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p,
                                                                 unsigned chunks, const typename Op::Acc* __restrict__ partials, Finish fin)
 {
+    typedef typename Op::Acc Acc;
+    __shared__ Acc sm[kWaves][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const u64 C = p.k_ext[p.nk - 1];
-    for (u64 slot = (u64)blockIdx.x * kBlock + threadIdx.x; slot < p.slots; slot += (u64)gridDim.x * kBlock) {
-        const u64 o = slot / C, c = slot - o * C;
-        typename Op::Acc a = Op::init();
-        for (unsigned k = 0; k < chunks; ++k) a = Op::combine(a, partials[(o * chunks + k) * C + c]);
-        const SlotPos s = slot_pos(p, o, p.nk - 1);
-        land(Op{}, fin, dst, s.dst + c, a, src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+    for (u64 base = (u64)blockIdx.x * kWave; base < p.slots; base += (u64)gridDim.x * kWave) {
+        const u64 slot = base + lane;
+        const bool live = slot < p.slots;
+        const u64 o = live ? slot / C : 0, c = live ? slot - o * C : 0;
+        Acc a = Op::init();
+        if (live) {
+            const Acc* col = partials + o * chunks * C + c;
+            unsigned k = wave;
+            for (; k + 3 * kWaves < chunks; k += 4 * kWaves) {
+                const Acc x0 = col[(u64)k * C], x1 = col[(u64)(k + kWaves) * C], x2 = col[(u64)(k + 2 * kWaves) * C], x3 = col[(u64)(k + 3 * kWaves) * C];
+                a = Op::combine(Op::combine(Op::combine(Op::combine(a, x0), x1), x2), x3);
+            }
+            for (; k < chunks; k += kWaves) a = Op::combine(a, col[(u64)k * C]);
+        }
+        __syncthreads();
+        sm[wave][lane] = a;
+        __syncthreads();
+        if (wave == 0 && live) {
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) a = Op::combine(a, sm[w][lane]);
+            const SlotPos s = slot_pos(p, o, p.nk - 1);
+            land(Op{}, fin, dst, s.dst + c, a, src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+        }
     }
 }
 
@@ -483,7 +512,7 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
             else hipLaunchKernelGGL((reduce_outer_k<Op, T, 1>), grid, dim3(kBlock), 0, st, ps, dst, p, (u64)rows_per_chunk, partials, fin);
             AIXK_HIP(hipGetLastError());
             if (chunks > 1) {
-                hipLaunchKernelGGL((reduce_outer_finish_k<Op, T>), dim3(grid_for(p.slots, kBlock, cus * 8u)), dim3(kBlock), 0, st,
+                hipLaunchKernelGGL((reduce_outer_finish_k<Op, T>), dim3(grid_for(p.slots, kWave, cus * 8u)), dim3(kBlock), 0, st,
                                    ps, dst, p, (unsigned)chunks, (const Acc*)partials, fin);
                 AIXK_HIP(hipGetLastError());
             }
