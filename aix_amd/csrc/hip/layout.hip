@@ -92,36 +92,43 @@ __global__ __launch_bounds__(kBlock) void transpose_tiled_k(const W* __restrict_
 
 // Same tile walk with 16-byte global accesses on both sides (whole tiles only, everything
 // 16-byte aligned): a lane loads VEC consecutive r of one c, scatters them into the LDS tile as
-// tile[r][c], and later gathers VEC consecutive c of one r for a 16-byte store.
-template <class W>
+// tile[r][c], and later gathers VEC consecutive c of one r for a 16-byte store.  TR x TC is the
+// tile in elements (TR along the source's contiguous dim).  Measured on [8192,8192] f32: the
+// access pattern, not LDS, sets the pace; 128 x 64 (512-byte read runs, 256-byte write runs) with
+// four tiles that are neighbours along the destination's contiguous dim numbered consecutively
+// is the fastest of the shapes tried (5.3 TB/s against 6.0 TB/s for a plain copy).
+template <class W, int TR, int TC>
 __global__ __launch_bounds__(kBlock) void transpose_vec_k(const W* __restrict__ src, W* __restrict__ dst,
-                                                          u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r)
+                                                          u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r, u32 tiles_c)
 {
     typedef typename vec16<W>::type V;
     constexpr int VEC = vec16<W>::n;
-    constexpr int LPR = kTile / VEC;          // lanes covering one tile row
-    constexpr int RPP = kBlock / LPR;         // tile rows covered per pass
-    __shared__ W tile[kTile][kTile + 1];
+    constexpr int LPR = TR / VEC, RPP = kBlock / LPR;      // lanes per source row, source rows per pass
+    constexpr int LPW = TC / VEC, WPP = kBlock / LPW;      // lanes per destination row, destination rows per pass
+    __shared__ W tile[TR][TC + 1];
     const u32 t = blockIdx.x;
-    const u32 tr = t % tiles_r, tc = t / tiles_r;
+    u32 tr, tc;
+    if (tiles_c % 4 == 0) { tc = (t / (4 * tiles_r)) * 4 + t % 4; tr = (t / 4) % tiles_r; }
+    else { tr = t % tiles_r; tc = t / tiles_r; }
     const u64 b = blockIdx.y;
-    const u64 r0 = (u64)tr * kTile, c0 = (u64)tc * kTile;
+    const u64 r0 = (u64)tr * TR, c0 = (u64)tc * TC;
     const W* s = src + off + b * sb;
     W* d = dst + b * R * C;
     const int lv = (threadIdx.x % LPR) * VEC, lp = threadIdx.x / LPR;
 #pragma unroll
-    for (int cc = lp; cc < kTile; cc += RPP) {
+    for (int cc = lp; cc < TC; cc += RPP) {
         const V v = *(const V*)(s + (r0 + lv) + (c0 + cc) * ld);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) tile[lv + e][cc] = v.v[e];
     }
     __syncthreads();
+    const int wv = (threadIdx.x % LPW) * VEC, wp = threadIdx.x / LPW;
 #pragma unroll
-    for (int rr = lp; rr < kTile; rr += RPP) {
+    for (int rr = wp; rr < TR; rr += WPP) {
         V v;
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v.v[e] = tile[rr][lv + e];
-        *(V*)(d + (r0 + rr) * C + c0 + lv) = v;
+        for (int e = 0; e < VEC; ++e) v.v[e] = tile[rr][wv + e];
+        *(V*)(d + (r0 + rr) * C + c0 + wv) = v;
     }
 }
 
@@ -222,11 +229,18 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
             const uint64_t B = sp.rank == 3 ? sp.shape[0] : 1, sb = sp.rank == 3 ? sp.stride[0][0] : 0;
             const uint64_t R = sp.shape[o], C = sp.shape[o + 1], ld = sp.stride[0][o + 1];
             const uint64_t tr = (R + kTile - 1) / kTile, tc = (C + kTile - 1) / kTile;
-            const bool whole = R % kTile == 0 && C % kTile == 0 && ld % VEC == 0 && sb % VEC == 0 &&
-                               aligned16(ps + sp.offset[0]) && aligned16(pd);
-            if (ld != 0 && whole && tr * tc < (1ull << 31) && B < 65536) {
-                hipLaunchKernelGGL((transpose_vec_k<W>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
-                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr);
+            const bool vecok = ld != 0 && ld % VEC == 0 && sb % VEC == 0 && aligned16(ps + sp.offset[0]) && aligned16(pd) && B < 65536;
+            // tile in elements: 512-byte read runs where the shape allows, else 64 x 64
+            constexpr int BIG_R = 128, BIG_C = sizeof(W) >= 4 ? 64 : 128;
+            if (vecok && sizeof(W) <= 4 && R % BIG_R == 0 && C % BIG_C == 0 && (R / BIG_R) * (C / BIG_C) < (1ull << 31)) {
+                hipLaunchKernelGGL((transpose_vec_k<W, BIG_R, BIG_C>), dim3((unsigned)((R / BIG_R) * (C / BIG_C)), (unsigned)B), dim3(kBlock), 0, ctx->stream,
+                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)(R / BIG_R), (u32)(C / BIG_C));
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            }
+            if (vecok && R % kTile == 0 && C % kTile == 0 && tr * tc < (1ull << 31)) {
+                hipLaunchKernelGGL((transpose_vec_k<W, kTile, kTile>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
+                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr, (u32)tc);
                 AIXK_HIP(hipGetLastError());
                 return (int)AIXK_OK;
             }
