@@ -350,6 +350,49 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ s
     }
 }
 
+// `outer` for wide rows: the four waves sit side by side, so a workgroup reads 256 * VEC
+// consecutive columns (4 KB of f32) of each row and every lane owns its columns outright -- no
+// LDS stage.  Long contiguous runs per row are what the strided walk needs to approach the
+// bandwidth of the unit-stride routes.
+template <class Op, class T, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p,
+                                                              u64 rows_per_chunk, typename Op::Acc* partials, Finish fin)
+{
+    typedef typename Op::Acc Acc;
+    typedef vec<T, VEC> V;
+    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 c0 = ((u64)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (c0 >= C) return;
+    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const u64 r_begin = (u64)blockIdx.y * rows_per_chunk;
+    const u64 r_end = r_begin + rows_per_chunk < R ? r_begin + rows_per_chunk : R;
+    Acc acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = Op::init();
+    const T* col = src + s.src + c0;
+    constexpr int U = 8;
+    for (u64 r0 = r_begin; r0 < r_end; r0 += U) {
+        V x[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * p.r_src[0]);
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            const u64 r = r0 + k;
+            if (r < r_end) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) Op::step(acc[e], x[k].v[e], r, r == 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        const u64 c = c0 + e;
+        if constexpr (Op::kTracksIndex) { if (acc[e].flags & 1u) acc[e].idx = (u32)(s.flat + (u64)acc[e].idx * p.r_flat[0] + c * p.k_flat[p.nk - 1]); }
+        if (partials) partials[((u64)blockIdx.z * gridDim.y + blockIdx.y) * C + c] = acc[e];
+        else land(Op{}, fin, dst, s.dst + c, acc[e], src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+    }
+}
+
 // second stage of `outer` when rows were split over several workgroups: 64 slots per workgroup,
 // the four waves take every fourth chunk (independent loads in flight), LDS folds the four.
 template <class Op, class T>
@@ -496,6 +539,25 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
         bool vect = C % VEC == 0 && ((uintptr_t)(ps + p.src_off) % (sizeof(T) * VEC)) == 0 && p.r_src[0] % VEC == 0;
         for (int d = 0; d + 1 < p.nk; ++d) if (p.k_src[d] % VEC) vect = false;
         const int v = vect ? VEC : 1;
+        // wide rows: workgroups of 256 * v columns, rows split into chunks of at least 16
+        if (vect && C >= (uint64_t)kBlock * v * 2 && R >= 64 && O <= 65535) {
+            const uint64_t tiles = (C + (uint64_t)kBlock * v - 1) / ((uint64_t)kBlock * v);
+            const uint64_t want = (uint64_t)cus * (sizeof(Acc) > 8 ? 2 : 8);      // wide partial records: fewer, longer chunks
+            uint64_t chunks = tiles * O < want ? std::min<uint64_t>({(want + tiles * O - 1) / (tiles * O), (R + 15) / 16, (uint64_t)65535}) : 1;
+            while (chunks > 1 && chunks * O * C * sizeof(Acc) > ctx->scratch_bytes) chunks /= 2;
+            const uint64_t rows_per_chunk = (R + chunks - 1) / chunks;
+            chunks = (R + rows_per_chunk - 1) / rows_per_chunk;
+            Acc* partials = chunks > 1 ? (Acc*)ctx->scratch : nullptr;
+            hipLaunchKernelGGL((reduce_outer_wide_k<Op, T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st,
+                               ps, dst, p, (u64)rows_per_chunk, partials, fin);
+            AIXK_HIP(hipGetLastError());
+            if (chunks > 1) {
+                hipLaunchKernelGGL((reduce_outer_finish_k<Op, T>), dim3(grid_for(p.slots, kWave, cus * 8u)), dim3(kBlock), 0, st,
+                                   ps, dst, p, (unsigned)chunks, (const Acc*)partials, fin);
+                AIXK_HIP(hipGetLastError());
+            }
+            return AIXK_OK;
+        }
         const uint64_t col_tiles = (C + (uint64_t)kWave * v - 1) / ((uint64_t)kWave * v);
         if (O <= 65535 && col_tiles < (1ull << 31)) {
             // split rows until the launch has enough workgroups to fill the chip

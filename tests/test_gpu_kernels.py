@@ -434,6 +434,8 @@ ROUTE_CASES = [  # (source shape, view kind, destination shape) chosen to hit ev
     ([9, 40, 33], "contig", [1, 40, 1]),      # two reduced dims: generic, workgroup per slot
     ([128, 128], "contig", [1, 1]),           # everything folds into one slot
     ([5, 7], "broadcast", [1, 7]),
+    ([130, 2304], "contig", [1, 2304]),       # outer, wide rows: workgroups side by side, rows split into chunks
+    ([3, 70, 2048], "contig", [3, 1, 2048]),  # the same with a leading kept dim
 ]
 
 
