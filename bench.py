@@ -134,6 +134,9 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--extras", default="c1,c2,c3",
+                    help="which of the other configurations to run besides the headline (comma list of c1, c2, c3): "
+                         "lets a profiler run cover one workload at a time")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="run only a plain copy-shaped kernel (negate, 64 MiB in + 64 MiB out per launch): the known-size "
@@ -196,6 +199,8 @@ def main():
     # ---- other single-GPU configurations (reported, not the headline) -----------------------------
     if not args.no_extras:
         extras = []
+        chosen = set(args.extras.split(","))
+    if not args.no_extras and "c1" in chosen:
         n = 8192
         rng1 = np.random.default_rng(1)
         x = rng1.standard_normal((n, n), dtype=np.float32)
@@ -213,22 +218,41 @@ def main():
                            "value": round(nbytes * steps / r.wall_s / 1e9, 1), "unit": "GB/s",
                            "roofline": roofline("hbm", nbytes / (r.gpu_ms / steps * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s")})
         del x
-        for dt_code, dt_name, np_dt, m in ((1, "f32", np.float32, 4096), (3, "bf16", np.uint16, 4096), (2, "f16", np.float16, 4096)):
-            ra = np.random.default_rng(3).uniform(-1, 1, (m, m)).astype(np.float32) / np.sqrt(m)
-            rb = np.random.default_rng(4).uniform(-1, 1, (m, m)).astype(np.float32) / np.sqrt(m)
-            if dt_name == "bf16":
-                from oracle.cpuref import f32_to_bf16_bits
-                ha, hb = f32_to_bf16_bits(ra), f32_to_bf16_bits(rb)
-            else:
-                ha, hb = ra.astype(np_dt), rb.astype(np_dt)
+    if not args.no_extras and "c2" in chosen:
+        from oracle.cpuref import f32_to_bf16_bits
+        host = {}
+
+        def operands(dt_name, m, batch=1):
+            key = (dt_name, m, batch)
+            if key not in host:
+                ra = np.random.default_rng(3).uniform(-1, 1, (batch, m, m)).astype(np.float32) / np.sqrt(m)
+                rb = np.random.default_rng(4).uniform(-1, 1, (batch, m, m)).astype(np.float32) / np.sqrt(m)
+                if dt_name == "bf16":
+                    host[key] = (f32_to_bf16_bits(ra), f32_to_bf16_bits(rb))
+                else:
+                    np_dt = np.float32 if dt_name == "f32" else np.float16
+                    host[key] = (ra.astype(np_dt), rb.astype(np_dt))
+            return host[key]
+
+        codes = {"f32": 1, "f16": 2, "bf16": 3}
+        layouts = {"NN": 0, "NT": 1, "TN": 2}
+        sweep = [("f32", 4096, "NN", 1, 20), ("bf16", 4096, "NN", 1, 20), ("f16", 4096, "NN", 1, 20),
+                 ("bf16", 4096, "NT", 1, 20), ("bf16", 4096, "TN", 1, 20), ("f32", 4096, "NT", 1, 20),
+                 ("bf16", 1024, "NN", 1, 50), ("bf16", 8192, "NN", 1, 5), ("f32", 1024, "NN", 1, 50), ("f32", 8192, "NN", 1, 3),
+                 ("bf16", 512, "NN", 64, 20)]
+        for dt_name, m, lay, batch, steps_mm in sweep:
+            ha, hb = operands(dt_name, m, batch)
             r = BenchResult()
-            steps_mm = 20
-            run(lib, "aixbench_matmul", dev.handle, dt_code, m, m, m, 0, 1, ha.ctypes.data, hb.ctypes.data, steps_mm, 2, C.byref(r), None)
-            flops = 2.0 * m * m * m
-            extras.append({"workload": f"configs[2] matmul {dt_name} {m}^3 (f32 accumulation)",
+            run(lib, "aixbench_matmul", dev.handle, codes[dt_name], m, m, m, layouts[lay], batch, ha.ctypes.data, hb.ctypes.data,
+                steps_mm, 2, C.byref(r), None)
+            flops = 2.0 * m * m * m * batch
+            what = f"{m}^3" if batch == 1 else f"{batch} x [{m},{m}]x[{m},{m}] (one matmul call per select(0,i) view)"
+            extras.append({"workload": f"configs[2] matmul {dt_name} {what} {lay} (f32 accumulation)",
                            "ms_per_step": round(r.wall_s * 1e3 / steps_mm, 5),
                            "value": round(flops * steps_mm / r.wall_s / 1e12, 2), "unit": "TFLOP/s",
                            "roofline": roofline("mfma", flops / (r.gpu_ms / steps_mm * 1e-3) / 1e12, MFMA_PEAK_TFLOPS[dt_name], "TFLOP/s")})
+        host.clear()
+    if not args.no_extras and "c3" in chosen:
         # configs[3]: MLP training step (autograd + Adam); the CPU device runs the first steps of the same program
         from aix_amd import drivers as GD
         from oracle import drivers as OD
@@ -258,6 +282,7 @@ def main():
             mlp["parity"] = {"checked_against": "cpu_baseline losses", "steps": cpu_steps, "max_rel_dev": float(rel.max()),
                              "ok": bool(rel.max() <= 1e-4), "rule": "|loss_gpu - loss_cpu| <= 1e-4 |loss_cpu| on the first steps"}
         extras.append(mlp)
+    if not args.no_extras:
         out["extras"] = extras
 
     dev.close()
