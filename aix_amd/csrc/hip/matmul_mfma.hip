@@ -198,7 +198,33 @@ __global__ __launch_bounds__(256) void gemm_nt16_k(GemmArgs g)
 #define AIX_WAIT(VM, LGKM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (((VM) >> 4) << 14) | 0x70 | ((LGKM) << 8))
 #define AIX_LDS(p) ((__attribute__((address_space(3))) void*)(p))
 #define AIX_GLB(p) ((const __attribute__((address_space(1))) void*)(p))
-template <class T>
+//
+// An operand may also be given the other way round -- A as [K, M] with unit stride along M (a
+// transposed view, "T" form), B as [K, N] with unit stride along N (plain row-major) -- and is then
+// consumed where it lies: its stage holds 64 k-rows of 512 bytes (LDS-direct chunks of 2 k-rows),
+// and the MFMA fragments, which need 8 consecutive k per lane, are assembled by
+// ds_read_b64_tr_b16: in every group of 16 lanes, lane j points at 4 consecutive elements
+// ("row" j) and lane i receives element i & 3 of rows (i >> 2) + 4 e, e = 0..3.  With lane j
+// pointing at X[k + (j >> 2)][n + 4 (j & 3) ..], lane i receives X[k .. k + 3][n + i]: four k of
+// its own column; two such reads make a fragment.  The four k-rows of a group are 512 bytes
+// apart (same banks), so the 16-byte chunk c of k-row k is kept in slot c ^ 4 (k & 3): the 64 bytes
+// that two neighbouring groups read from each of their four k-rows then fall into disjoint banks.
+//
+// The read is issued through inline assembly: given the builtin, the compiler orders it behind every
+// LDS-direct load in flight (s_waitcnt vmcnt(0) before each read), which serialises the pipeline.
+// The price is that the compiler no longer knows the result is pending, so every phase that consumes
+// such fragments starts with an explicit s_waitcnt lgkmcnt(0).
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x4 tr_fragment(const unsigned char* lds_addr)
+{
+    const u32 addr = (u32)(size_t)(__attribute__((address_space(3))) const unsigned char*)lds_addr;
+    u32x2 lo, hi;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(hi) : "v"(addr));       // k + 4
+    return u32x4{lo.x, lo.y, hi.x, hi.y};
+}
+
+template <class T, bool AT, bool BT>
 __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
 {
     constexpr int BM = 256, BK = 64, TI = 4, TJ = 4, STAGE = 2 * 256 * BK * 2;     // 65536 bytes: A rows then B rows
@@ -208,21 +234,31 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
     const u64 m0 = (u64)tm * 256, n0 = (u64)tn * 256;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), wm = wave >> 1, wn = wave & 1;
-    // producer: wave w fills rows 64 w .. 64 w + 63 of both operands, 8 chunks of 8 rows each
+    // producer, K-contiguous operand: wave w fills rows 64 w .. 64 w + 63, 8 chunks of 8 rows (128 B) each
     const int lr = lane >> 3;
     const int fe = (lr >> 1) ^ ((lr & 1) << 2);              // f(row) in even chunks; odd chunks: fe ^ 4
     const int q0 = (lane & 7) ^ fe, q1 = q0 ^ 4;
-    const char* A = (const char*)g.a + (m0 + wave * 64) * g.lda * 2;
-    const char* B = (const char*)g.b + (n0 + wave * 64) * g.ldb * 2;
-    const u32 oa0 = (u32)((lr * g.lda + q0 * 8) * 2), oa1 = (u32)((lr * g.lda + q1 * 8) * 2);
-    const u32 ob0 = (u32)((lr * g.ldb + q0 * 8) * 2), ob1 = (u32)((lr * g.ldb + q1 * 8) * 2);
-    const u64 ca = 16 * g.lda, cb = 16 * g.ldb;               // bytes between 8-row chunks
+    // producer, T-form operand: wave w fills k-rows 16 w .. 16 w + 15, 8 chunks of 2 k-rows (512 B) each;
+    // lane = (k-row lane >> 5, slot lane & 31) fetches chunk slot ^ 4 (k & 3), k & 3 = 2 (chunk & 1) + (lane >> 5)
+    const int tk = lane >> 5, ts0 = (lane & 31) ^ (4 * tk), ts1 = ts0 ^ 8;
+    const char* A = AT ? (const char*)g.a + m0 * 2 + (u64)(wave * 16) * g.lda * 2 : (const char*)g.a + (m0 + wave * 64) * g.lda * 2;
+    const char* B = BT ? (const char*)g.b + n0 * 2 + (u64)(wave * 16) * g.ldb * 2 : (const char*)g.b + (n0 + wave * 64) * g.ldb * 2;
+    const u32 oa0 = AT ? (u32)((tk * g.lda + ts0 * 8) * 2) : (u32)((lr * g.lda + q0 * 8) * 2);
+    const u32 oa1 = AT ? (u32)((tk * g.lda + ts1 * 8) * 2) : (u32)((lr * g.lda + q1 * 8) * 2);
+    const u32 ob0 = BT ? (u32)((tk * g.ldb + ts0 * 8) * 2) : (u32)((lr * g.ldb + q0 * 8) * 2);
+    const u32 ob1 = BT ? (u32)((tk * g.ldb + ts1 * 8) * 2) : (u32)((lr * g.ldb + q1 * 8) * 2);
+    const u64 ca = (AT ? 4 : 16) * g.lda, cb = (BT ? 4 : 16) * g.ldb;      // bytes between chunks
+    const u64 sa = AT ? (u64)BK * g.lda * 2 : (u64)BK * 2, sb = BT ? (u64)BK * g.ldb * 2 : (u64)BK * 2;   // bytes between K-steps
     const int steps = (int)(g.K / BK);
-    // consumer: lane reads row (lane & 31) of a 32-row block, k-chunk 2 kk + (lane >> 5)
+    // consumer, K-contiguous operand: lane reads row (lane & 31) of a 32-row block, k-chunk 2 kk + (lane >> 5)
     const int r15 = lane & 15;
     const int slot0 = (lane >> 5) ^ (((r15 >> 1) & 7) ^ ((r15 & 1) << 2));
-    const int fra = (wm * 128 + (lane & 31)) * 128 + slot0 * 16;
-    const int frb = BM * 128 + (wn * 128 + (lane & 31)) * 128 + slot0 * 16;
+    // consumer, T-form operand: lane j of a 16-lane group points at k-row (8 (lane >> 5) + (j >> 2)) [+ 16 kk, + 4],
+    // columns 16 ((lane >> 4) & 1) + 4 (j & 3) .. + 3 of the 32-column block; the block index enters by XOR (bits 6-7)
+    const int tq = r15 >> 2, tn4 = 4 * (r15 & 3), tc = (16 * ((lane >> 4) & 1) + tn4) >> 3;
+    const int tlane = (8 * (lane >> 5) + tq) * 512 + (tn4 & 4) * 2;
+    const int fra = AT ? tlane + (((16 * wm + tc) ^ (4 * tq)) * 16) : (wm * 128 + (lane & 31)) * 128 + slot0 * 16;
+    const int frb = BM * 128 + (BT ? tlane + (((16 * wn + tc) ^ (4 * tq)) * 16) : (wn * 128 + (lane & 31)) * 128 + slot0 * 16);
 
     f32x16 acc[TI][TJ];
 #pragma unroll
@@ -234,13 +270,16 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
     u32x4 fa[2][TI], fb[2][TJ];
 
     // load n of a tile (0..15): n < 8 is chunk n of A, otherwise chunk n - 8 of B
-#define AIX_LD(N, KO, BO) { if ((N) < 8) __builtin_amdgcn_global_load_lds(AIX_GLB(A + ((N) * ca + (KO)) + (((N) & 1) ? oa1 : oa0)), AIX_LDS(smem + (BO) + (wave * 8 + (N)) * 1024), 16, 0, 0); \
-    else __builtin_amdgcn_global_load_lds(AIX_GLB(B + (((N) - 8) * cb + (KO)) + (((N) & 1) ? ob1 : ob0)), AIX_LDS(smem + (BO) + BM * 128 + (wave * 8 + (N) - 8) * 1024), 16, 0, 0); }
-#define AIX_RDA(F, BO, KK, I) fa[F][I] = *(const u32x4*)(smem + (BO) + (fra ^ ((KK) * 32)) + (I) * 4096);
-#define AIX_RDB(F, BO, KK, J) fb[F][J] = *(const u32x4*)(smem + (BO) + (frb ^ ((KK) * 32)) + (J) * 4096);
+#define AIX_LD(N, KI, BO) { if ((N) < 8) __builtin_amdgcn_global_load_lds(AIX_GLB(A + ((N) * ca + (KI) * sa) + (((N) & 1) ? oa1 : oa0)), AIX_LDS(smem + (BO) + (wave * 8 + (N)) * 1024), 16, 0, 0); \
+    else __builtin_amdgcn_global_load_lds(AIX_GLB(B + (((N) - 8) * cb + (KI) * sb) + (((N) & 1) ? ob1 : ob0)), AIX_LDS(smem + (BO) + BM * 128 + (wave * 8 + (N) - 8) * 1024), 16, 0, 0); }
+#define AIX_RDA(F, BO, KK, I) { if constexpr (AT) fa[F][I] = tr_fragment(smem + (BO) + (fra ^ ((I) * 64)) + (KK) * 8192); \
+    else fa[F][I] = *(const u32x4*)(smem + (BO) + (fra ^ ((KK) * 32)) + (I) * 4096); }
+#define AIX_RDB(F, BO, KK, J) { if constexpr (BT) fb[F][J] = tr_fragment(smem + (BO) + (frb ^ ((J) * 64)) + (KK) * 8192); \
+    else fb[F][J] = *(const u32x4*)(smem + (BO) + (frb ^ ((KK) * 32)) + (J) * 4096); }
 #define AIX_ROW(F, I) { _Pragma("unroll") for (int j = 0; j < TJ; ++j) acc[I][j] = Mma16<T>::run(fa[F][I], fb[F][j], acc[I][j]); }
-    // MFMAs on fragment set FC while set FN is read from stage RBO, slice KK; loads L0.. of the tile at byte KO go to stage LBO
+    // MFMAs on fragment set FC while set FN is read from stage RBO, slice KK; loads L0.. of K-tile KO go to stage LBO
 #define AIX_PHASE(FC, FN, RBO, KK, KO, LBO, L0, L1, L2, L3, L4, L5) \
+    if constexpr (AT || BT) { AIX_SB(); __builtin_amdgcn_s_waitcnt(0xC07F); AIX_SB(); }     /* lgkmcnt(0): fragment set FC has arrived */ \
     AIX_RDA(FN, RBO, KK, 0) AIX_RDA(FN, RBO, KK, 1) if (L0 >= 0) AIX_LD(L0, KO, LBO) if (L4 >= 0) AIX_LD(L4, KO, LBO) AIX_ROW(FC, 0) AIX_SB(); \
     AIX_RDA(FN, RBO, KK, 2) AIX_RDA(FN, RBO, KK, 3) if (L1 >= 0) AIX_LD(L1, KO, LBO) if (L5 >= 0) AIX_LD(L5, KO, LBO) AIX_ROW(FC, 1) AIX_SB(); \
     AIX_RDB(FN, RBO, KK, 0) AIX_RDB(FN, RBO, KK, 1) if (L2 >= 0) AIX_LD(L2, KO, LBO) AIX_ROW(FC, 2) AIX_SB(); \
@@ -248,9 +287,9 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
 
     // Tiles past the end re-read the last tile into a stage nobody consumes any more.
     {
-        const u64 k1 = (u64)(1 < steps ? 1 : 0) * (BK * 2);
+        const u64 k1 = 1 < steps ? 1 : 0;
 #pragma unroll
-        for (int n = 0; n < 16; ++n) AIX_LD(n, 0, 0)
+        for (int n = 0; n < 16; ++n) AIX_LD(n, (u64)0, 0)
 #pragma unroll
         for (int n = 0; n < 6; ++n) AIX_LD(n, k1, STAGE)
     }
@@ -262,8 +301,7 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
     AIX_RDB(0, 0, 0, 0) AIX_RDB(0, 0, 0, 1) AIX_RDB(0, 0, 0, 2) AIX_RDB(0, 0, 0, 3)
     for (int kt = 0; kt < steps; ++kt) {
         const int bo = (kt & 1) * STAGE, nbo = bo ^ STAGE;
-        const u64 k1 = (u64)(kt + 1 < steps ? kt + 1 : steps - 1) * (BK * 2);
-        const u64 k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1) * (BK * 2);
+        const u64 k1 = (u64)(kt + 1 < steps ? kt + 1 : steps - 1), k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1);
         AIX_PHASE(0, 1, bo, 1, k1, nbo, 6, 7, 8, 9, 10, -1)
         AIX_PHASE(1, 0, bo, 2, k1, nbo, 11, 12, 13, 14, 15, -1)
         AIX_PHASE(0, 1, bo, 3, k1, nbo, -1, -1, -1, -1, -1, -1)
@@ -441,6 +479,43 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
     if (K % kq != 0 || M * N < 64 * 64) return -1;                // odd K / tiny outputs: LDS-tiled kernel
     if (((M + 127) / 128) * ((N + 127) / 128) >= (1ull << 31)) return -1;
 
+    // 16-bit, whole 256 x 256 x 64 tiles, enough of them: every operand layout is consumed where it lies
+    // (K-contiguous, or "T" form with unit stride along M / N), no gathers.
+    if (esz == 2 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (M / 256) * (N / 256) >= (uint64_t)ctx->cus / 2 &&
+        (M / 256) * (N / 256) < (1ull << 31)) {
+        const char* qa = (const char*)a->data + a->offset * esz;
+        const char* qb = (const char*)b->data + b->offset * esz;
+        const bool a_k = a->strides[1] == 1, a_m = a->strides[0] == 1;
+        const bool b_k = b->strides[0] == 1, b_n = b->strides[1] == 1;
+        const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
+        if ((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && la < (1ull << 27) && lb < (1ull << 27) && aligned16(qa) && aligned16(qb)) {
+            GemmArgs g{};
+            g.a = qa; g.b = qb; g.c = out->data;
+            g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+            g.tiles_m = (u32)(M / 256); g.tiles_n = (u32)(N / 256);
+            const u32 n = g.tiles_m * g.tiles_n;
+            g.swizzle = n % 8u == 0 ? 1u : 0u;
+            constexpr size_t lds = 2 * 65536;
+            const bool at = !a_k, bt = !b_k;
+            auto launch = [&](auto kernel) {
+                AIXK_TRY(set_lds(kernel, lds));
+                hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            };
+            if (out->dtype == AIXK_BF16) {
+                if (!at && !bt) return launch(gemm_nt16_direct_k<bf16, false, false>);
+                if (!at && bt) return launch(gemm_nt16_direct_k<bf16, false, true>);
+                if (at && !bt) return launch(gemm_nt16_direct_k<bf16, true, false>);
+                return launch(gemm_nt16_direct_k<bf16, true, true>);
+            }
+            if (!at && !bt) return launch(gemm_nt16_direct_k<f16, false, false>);
+            if (!at && bt) return launch(gemm_nt16_direct_k<f16, false, true>);
+            if (at && !bt) return launch(gemm_nt16_direct_k<f16, true, false>);
+            return launch(gemm_nt16_direct_k<f16, true, true>);
+        }
+    }
+
     // A as [M,K] and B as [N,K], both with unit stride along K and 16-byte aligned rows
     const char* pa = (const char*)a->data + a->offset * esz;
     uint64_t lda = a->strides[0];
@@ -483,12 +558,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         return AIXK_OK;
     }
     const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= (uint64_t)ctx->cus / 2;
-    if (big && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && lda < (1ull << 27) && ldb < (1ull << 27)) {
-        constexpr size_t lds = 2 * 65536;
-        const u32 n = grid_of(256, 256);
-        if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_direct_k<bf16>, lds)); hipLaunchKernelGGL((gemm_nt16_direct_k<bf16>), dim3(n), dim3(256), lds, ctx->stream, g); }
-        else { AIXK_TRY(set_lds(gemm_nt16_direct_k<f16>, lds)); hipLaunchKernelGGL((gemm_nt16_direct_k<f16>), dim3(n), dim3(256), lds, ctx->stream, g); }
-    } else if (big) {
+    if (big) {
         constexpr size_t lds = 2 * (256 + 256) * 72 * 2;
         const u32 n = grid_of(256, 256);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }

@@ -594,7 +594,8 @@ def test_matmul_mfma_tiles(gpu, dtype):
              ((2085, 512, 4101), "contig", "contig"), ((2048, 264, 4096), "contig", "transposed"),     # 256x256 tiles
              # whole 256x256 tiles and K steps of 64: the LDS-direct kernel (1, 2, 3 and 5 K steps; swizzled and plain tile numbering)
              ((2048, 64, 4096), "contig", "transposed"), ((2048, 128, 4096), "contig", "contig"),
-             ((4096, 192, 2048), "transposed", "contig"), ((2304, 320, 3840), "contig", "transposed")]
+             ((4096, 192, 2048), "transposed", "contig"), ((2304, 320, 3840), "contig", "transposed"),
+             ((2048, 256, 4096), "transposed", "transposed"), ((4096, 128, 2048), "contig", "sliced")]
     for (m, k, n), ka, kb in cases:
         scale = 1.0 / np.sqrt(k)
         a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
