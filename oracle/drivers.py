@@ -95,3 +95,38 @@ def ref_mlp(batch, n_in, hidden, n_out, steps, lr, data):
     if rc != 0:
         raise RuntimeError(ref_lib().aixref_drivers_last_error().decode())
     return losses, int(counts[1])
+
+
+def ref_hip_lib_path():
+    path = os.path.join(HERE, "_ref", "libaixref_hip_drivers.so")
+    return path if os.path.exists(path) else None
+
+
+def _ref_hip_mlp_here(batch, n_in, hidden, n_out, steps, lr):
+    """Runs in a process of its own (see ref_hip_mlp): the reference's front-end on DeviceHIP."""
+    lib = C.CDLL(ref_hip_lib_path())
+    lib.aixref_mlp_hip.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, _PF, _PF, _PPF, _PPF, _PF]
+    lib.aixref_drivers_last_error.restype = C.c_char_p
+    x, y, w, b = mlp_data(batch, n_in, hidden, n_out)
+    losses = np.zeros(steps, dtype=np.float32)
+    pw, pb = pointer_array(w), pointer_array(b)
+    rc = lib.aixref_mlp_hip(batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF), pw, pb, losses.ctypes.data_as(_PF))
+    if rc != 0:
+        raise RuntimeError(lib.aixref_drivers_last_error().decode())
+    return losses
+
+
+def ref_hip_mlp(batch, n_in, hidden, n_out, steps, lr):
+    """The MLP loop written with the reference's own classes, run on the GPU backend (default
+    mlp_data inputs).  A separate process, because that library carries a DeviceHIP built against
+    the reference's headers, which must not meet the product's own build of the class in one process."""
+    import json
+    import subprocess
+    import sys
+    code = ("import json, sys; sys.path.insert(0, %r); from oracle import drivers as d; "
+            "print(json.dumps([float(v) for v in d._ref_hip_mlp_here(%d, %d, %d, %d, %d, %r)]))"
+            % (os.path.dirname(HERE), batch, n_in, hidden, n_out, steps, lr))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
+    if out.returncode != 0:
+        raise RuntimeError("reference front-end on DeviceHIP failed: " + out.stderr[-2000:])
+    return np.array(json.loads(out.stdout.strip().splitlines()[-1]), dtype=np.float32)

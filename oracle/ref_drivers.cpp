@@ -8,6 +8,9 @@
 // matmul calls, which shows that both generate the same operator stream.
 
 #include <aix.hpp>
+#ifdef AIXREF_WITH_HIP
+#include "../aix_amd/csrc/device/device_hip.hpp"      // built with AIXHIP_USE_AIX_HEADERS: derives from the reference's aix::Device
+#endif
 
 #include <cstdio>
 #include <cstdint>
@@ -39,36 +42,66 @@ extern "C" {
 
 const char* aixref_drivers_last_error(void) { return g_err; }
 
+}   // extern "C"
+
+namespace {
+
+// The loop itself, on whatever aix::Device it is given -- nothing in it names a backend.
+void mlp_loop(aix::Device& dev, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
+              const float* x, const float* y, const float* const* w, const float* const* b, float* losses)
+{
+    const aix::TensorOptions plain{ .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
+    const aix::TensorOptions param{ .m_requireGrad = true, .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
+    const auto F32 = aix::DataType::kFloat32;
+    aix::Tensor X(x, batch * in, F32, aix::Shape{batch, in}, plain);
+    aix::Tensor Y(y, batch * out, F32, aix::Shape{batch, out}, plain);
+    aix::Tensor w1(w[0], in * hidden, F32, aix::Shape{in, hidden}, param), b1(b[0], hidden, F32, aix::Shape{1, hidden}, param);
+    aix::Tensor w2(w[1], hidden * hidden, F32, aix::Shape{hidden, hidden}, param), b2(b[1], hidden, F32, aix::Shape{1, hidden}, param);
+    aix::Tensor w3(w[2], hidden * out, F32, aix::Shape{hidden, out}, param), b3(b[2], out, F32, aix::Shape{1, out}, param);
+    aix::optim::Adam opt(std::vector<aix::Tensor>{w1, b1, w2, b2, w3, b3}, lr);
+    aix::nn::Softmax softmax(1, true);
+    aix::nn::CrossEntropyLoss lossFn;
+    for (int s = 0; s < steps; ++s) {
+        opt.zeroGrad();
+        auto h1 = relu(aix::matmul(X, w1) + b1, &dev);
+        auto h2 = relu(aix::matmul(h1, w2) + b2, &dev);
+        auto logits = aix::matmul(h2, w3) + b3;
+        auto loss = lossFn(softmax.forward(logits), Y);
+        loss.backward();
+        opt.step();
+        dev.synchronize();
+        losses[s] = loss.value().item<float>();
+    }
+    dev.synchronize();
+}
+
+} // namespace
+
+extern "C" {
+
 int aixref_mlp(uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
                const float* x, const float* y, const float* const* w, const float* const* b, float* losses, uint64_t* counts)
 {
     try {
         CountingCPU dev;
-        const aix::TensorOptions plain{ .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
-        const aix::TensorOptions param{ .m_requireGrad = true, .m_dtype = aix::DataType::kFloat32, .m_device = &dev };
-        const auto F32 = aix::DataType::kFloat32;
-        aix::Tensor X(x, batch * in, F32, aix::Shape{batch, in}, plain);
-        aix::Tensor Y(y, batch * out, F32, aix::Shape{batch, out}, plain);
-        aix::Tensor w1(w[0], in * hidden, F32, aix::Shape{in, hidden}, param), b1(b[0], hidden, F32, aix::Shape{1, hidden}, param);
-        aix::Tensor w2(w[1], hidden * hidden, F32, aix::Shape{hidden, hidden}, param), b2(b[1], hidden, F32, aix::Shape{1, hidden}, param);
-        aix::Tensor w3(w[2], hidden * out, F32, aix::Shape{hidden, out}, param), b3(b[2], out, F32, aix::Shape{1, out}, param);
-        aix::optim::Adam opt(std::vector<aix::Tensor>{w1, b1, w2, b2, w3, b3}, lr);
-        aix::nn::Softmax softmax(1, true);
-        aix::nn::CrossEntropyLoss lossFn;
-        for (int s = 0; s < steps; ++s) {
-            opt.zeroGrad();
-            auto h1 = relu(aix::matmul(X, w1) + b1, &dev);
-            auto h2 = relu(aix::matmul(h1, w2) + b2, &dev);
-            auto logits = aix::matmul(h2, w3) + b3;
-            auto loss = lossFn(softmax.forward(logits), Y);
-            loss.backward();
-            opt.step();
-            dev.synchronize();
-            losses[s] = loss.value().item<float>();
-        }
+        mlp_loop(dev, batch, in, hidden, out, steps, lr, x, y, w, b, losses);
         if (counts) counts[1] = dev.matmuls;
         return 0;
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
 }
+
+#ifdef AIXREF_WITH_HIP
+// The same loop, the reference's own front-end, on the MI355X backend: aix::hip::DeviceHIP handed to
+// aix::Tensor exactly as README.MD:166-188 hands it the Metal device.
+int aixref_mlp_hip(uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
+                   const float* x, const float* y, const float* const* w, const float* const* b, float* losses)
+{
+    try {
+        aix::hip::DeviceHIP dev;
+        mlp_loop(dev, batch, in, hidden, out, steps, lr, x, y, w, b, losses);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
+#endif
 
 } // extern "C"

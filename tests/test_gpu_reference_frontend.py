@@ -1,0 +1,38 @@
+"""The reference's own front-end on the GPU backend.
+
+oracle/_ref/libaixref_hip_drivers.so is built where the reference tree is present: the reference's
+aix.hpp (Tensor, autograd, nn::Softmax, nn::CrossEntropyLoss, optim::Adam), its DeviceCPU sources, and
+this repository's DeviceHIP host sources compiled against those headers, so that DeviceHIP derives
+from the framework's own aix::Device and is handed to aix::Tensor like any other device.  The MLP
+training loop then runs unchanged on it; its losses are compared with the same loop on the
+reference's CPU device (small case, literal reference arithmetic) and with the restated front-end on
+the product build of DeviceHIP (same operator stream, so the same numbers bit for bit)."""
+import numpy as np
+import pytest
+
+from oracle import drivers as OD
+
+pytestmark = [pytest.mark.gpu,
+              pytest.mark.skipif(OD.ref_hip_lib_path() is None or OD.ref_lib() is None, reason="oracle/_ref not built (no reference tree)")]
+
+
+def test_reference_tensor_autograd_adam_run_unchanged_on_device_hip():
+    shape, steps = (64, 48, 32, 10), 60
+    on_gpu = OD.ref_hip_mlp(*shape, steps, 1e-3)
+    on_cpu, _ = OD.ref_mlp(*shape, steps, 1e-3, OD.mlp_data(*shape))
+    rel = np.abs(on_gpu.astype(np.float64) - on_cpu) / np.abs(on_cpu)
+    print(f"reference front-end, {shape} x{steps}: CPU {on_cpu[0]:.6f} -> {on_cpu[-1]:.6f}, DeviceHIP {on_gpu[-1]:.6f}, max rel dev {rel.max():.3e}")
+    assert np.all(np.isfinite(on_gpu)) and on_cpu[-1] < on_cpu[0]
+    assert rel.max() <= 1e-4
+
+
+def test_restated_front_end_issues_the_same_stream_on_the_gpu():
+    from aix_amd import device as D, drivers as GD
+    shape, steps = (128, 784, 64, 10), 25
+    via_reference = OD.ref_hip_mlp(*shape, steps, 1e-3)
+    dev = D.Device(0)
+    try:
+        via_restatement, _ = GD.mlp(dev, *shape, steps, 1e-3, OD.mlp_data(*shape))
+    finally:
+        dev.close()
+    assert via_reference.view(np.uint32).tolist() == via_restatement.view(np.uint32).tolist()
