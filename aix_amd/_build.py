@@ -9,10 +9,10 @@ def library_path(name):
     return os.path.join(HERE, name)
 
 
-def build(jobs=8, verbose=False):
-    """Compile every HIP extension for gfx950 and the host library.  Always recompiles what is
-    out of date; raises on the first compiler error."""
-    cmd = ["make", "-C", os.path.join(HERE, "csrc"), f"-j{jobs}", "all"]
+def build(jobs=8, verbose=False, force=False):
+    """Compile every HIP extension for gfx950 and the host library; raises on the first compiler
+    error.  force=True recompiles every source even where an up-to-date library is present."""
+    cmd = ["make", "-C", os.path.join(HERE, "csrc"), f"-j{jobs}", "all"] + (["-B"] if force else [])
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         print(res.stdout[-8000:])

@@ -94,11 +94,13 @@ def to_float64(storage, dtype):
     return np.asarray(storage).astype(np.float64)
 
 
-def build(ref=True):
-    """(Re)build the oracle; the reference-backed library only where the reference exists."""
-    subprocess.check_call(["make", "-s", "-C", HERE, "all"])
+def build(ref=True, force=False):
+    """(Re)build the oracle; the reference-backed libraries only where the reference exists.
+    force=True recompiles even what is up to date."""
+    extra = ["-B"] if force else []
+    subprocess.check_call(["make", "-s", "-C", HERE, "all"] + extra)
     if ref and os.path.isdir(os.environ.get("AIX_REFERENCE_DIR", "/root/reference")):
-        subprocess.check_call(["make", "-s", "-C", HERE, "ref"])
+        subprocess.check_call(["make", "-s", "-C", HERE, "ref"] + extra)
 
 
 _T = C.POINTER(TensorDesc)
