@@ -10,6 +10,7 @@
 #include "../../../include/aixhip.h"
 #include "../device/device_hip.hpp"
 #include "../frontend/mlp.hpp"
+#include "../frontend/transformer.hpp"
 #include "../frontend/value.hpp"
 
 #include <chrono>
@@ -165,14 +166,28 @@ int aixbench_matmul(aixhip_device* handle, int dtype, uint64_t M, uint64_t N, ui
 
 // Config 3: MLP training (in -> hidden -> hidden -> out, ReLU, softmax + cross-entropy, Adam) for
 // `steps` steps from the given host parameters; losses[steps], step_seconds[steps] (may be NULL).
-int aixbench_mlp(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
+// single_pass = 0 differentiates as the reference does (once per path), 1 once per node.
+int aixbench_mlp(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
                  const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds)
 {
     return guarded([&] {
         DeviceHIP* dev = aix::hip::fromHandle(handle);
-        const aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr};
+        const aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr, single_pass};
         const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
         aixfe::runMlp(dev, cfg, host, losses, step_seconds);
+    });
+}
+
+// Config 4: decoder-only transformer forward + backward (frontend/transformer.hpp); params in the order of
+// aixfe::transformerParamShapes; losses[steps], grad_norms[steps * param_count], step_seconds[steps] (may be NULL).
+int aixbench_transformer(aixhip_device* handle, uint64_t layers, uint64_t d_model, uint64_t heads, uint64_t seq, uint64_t batch,
+                         uint64_t vocab, int steps, const int32_t* tokens, const float* const* params,
+                         float* losses, float* grad_norms, double* step_seconds)
+{
+    return guarded([&] {
+        DeviceHIP* dev = aix::hip::fromHandle(handle);
+        const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps};
+        aixfe::runTransformer(dev, cfg, tokens, params, losses, grad_norms, step_seconds);
     });
 }
 

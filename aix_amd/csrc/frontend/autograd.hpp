@@ -18,6 +18,7 @@
 #include "value.hpp"
 
 #include <functional>
+#include <unordered_set>
 #include <utility>
 
 namespace aixfe {
@@ -32,17 +33,26 @@ struct Node {
     bool retainGrad{false};
     bool isLeaf{true};
     std::vector<NodePtr> inputs;
-    size_t dim0{0}, dim1{0};
+    size_t dim0{0}, dim1{0}, start{0}, end{0};
+    ssize_t diagonal{0};
     bool keepDim{false};
+    Value indices;
     std::function<void(Node*, const Value&)> backwardFn;
 
     Node(Value v, bool req) : value(std::move(v)), requireGrad(req) {}
 
     void backward(const Value& seed)
     {
+        if (accumulating()) {                       // single-pass mode: gather the seed, the driver calls backwardFn once
+            pending = pending.defined() ? pending + seed : seed;
+            return;
+        }
         if (retainGrad) grad() += seed;
         if (requireGrad || retainGrad) backwardFn(this, seed);
     }
+
+    static bool& accumulating() { static thread_local bool on = false; return on; }
+    Value pending;                                  // sum of the seeds received so far (single-pass mode)
 
     Value& grad()
     {
@@ -98,7 +108,100 @@ public:
         m_node->backward(Value::full(device(), dtype(), shape(), 1.0f));
     }
 
+    // Single-pass differentiation: nodes are visited in reverse topological order and each one is
+    // differentiated ONCE with the sum of the seeds that reached it.  The reference has no such mode
+    // (its recursion revisits a node once per path, which is exponential in the number of residual
+    // branches of a transformer); the backward formulas are the same ones, only the traversal differs.
+    void backwardOnce() const
+    {
+        if (value().size() != 1) throw std::invalid_argument("backward() requires a one-element tensor");
+        std::vector<Node*> order;
+        std::vector<std::pair<Node*, size_t>> stack{{m_node.get(), 0}};
+        std::unordered_set<Node*> seen{m_node.get()};
+        while (!stack.empty()) {                      // iterative post-order DFS
+            auto& [n, next] = stack.back();
+            if (next < n->inputs.size()) {
+                Node* in = n->inputs[next++].get();
+                if (seen.insert(in).second) stack.push_back({in, 0});
+            } else { order.push_back(n); stack.pop_back(); }
+        }
+        Node::accumulating() = true;
+        try {
+            m_node->pending = Value::full(device(), dtype(), shape(), 1.0f);
+            for (size_t k = order.size(); k-- > 0;) {
+                Node* n = order[k];
+                if (!n->pending.defined()) continue;
+                const Value seed = std::move(n->pending);
+                n->pending = Value();
+                if (n->retainGrad) n->grad() += seed;
+                if (n->requireGrad || n->retainGrad) n->backwardFn(n, seed);
+            }
+        } catch (...) { Node::accumulating() = false; throw; }
+        Node::accumulating() = false;
+    }
+
     // ---- shape ------------------------------------------------------------------------------
+    // aixCore.hpp:1973-1978
+    Tensor reshape(const Shape& s) const
+    {
+        Tensor r = makeResult(value().reshape(s), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.reshape(n->inputs[0]->value.shape()));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2004-2010; backward casts the seed back (:2052-2057)
+    Tensor to(DataType dt) const
+    {
+        if (dtype() == dt) return *this;
+        Tensor r = makeResult(value().to(dt), isRequireGrad());
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.to(n->inputs[0]->value.dtype()));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2597-2608; backward scatters the seed into zeros (:2228-2233)
+    Tensor slice(size_t dim, size_t start, size_t end, size_t step = 1) const
+    {
+        Tensor r = makeResult(value().slice(dim, start, end, step), isRequireGrad());
+        r.m_node->dim0 = dim; r.m_node->dim1 = step; r.m_node->start = start; r.m_node->end = end;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(n->inputs[0]->value.sliceSet(seed, n->dim0, n->start, n->end, n->dim1));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2664-2670
+    Tensor tril(ssize_t diagonal = 0) const
+    {
+        Tensor r = makeResult(value().tril(diagonal), isRequireGrad());
+        r.m_node->diagonal = diagonal;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            n->inputs[0]->backward(seed.tril(n->diagonal));
+        });
+        return r;
+    }
+
+    // aixCore.hpp:2680-2700; backward adds the seed's rows into zeros (:2284-2290)
+    Tensor indexSelect(size_t dim, const Value& indices) const
+    {
+        Tensor r = makeResult(value().indexSelect(dim, indices), isRequireGrad(), !m_node->isLeaf);
+        r.m_node->dim0 = dim; r.m_node->indices = indices;
+        r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.empty()) return;
+            const Value zeros = Value::full(seed.device(), seed.dtype(), n->inputs[0]->value.shape(), 0.0f);
+            zeros.indexAddInPlace(n->dim0, n->indices, seed);
+            n->inputs[0]->backward(zeros);
+        });
+        return r;
+    }
+
     Tensor broadcastTo(const Shape& s) const
     {
         if (shape() == s) return *this;
@@ -262,6 +365,19 @@ public:
         return r;
     }
 
+    // aixCore.hpp:2533-2540; backward :2165-2176 (only the base is differentiated: the exponent is a constant)
+    Tensor pow(float e) const
+    {
+        const Tensor ex = Tensor(e, Shape{}, device(), dtype()).broadcastTo(shape());
+        Tensor r = makeResult(value().pow(ex.value()), isRequireGrad(), !m_node->isLeaf);
+        r.m_node->setBackward({m_node, ex.m_node}, [](Node* n, const Value& seed) {
+            if (n->inputs.size() < 2) return;
+            if (wants(n->inputs[0]))
+                n->inputs[0]->backward(seed * n->inputs[1]->value * n->inputs[0]->value.pow(n->inputs[1]->value.withScalar(&Device::sub, 1.0f)));
+        });
+        return r;
+    }
+
     Tensor sqrt() const
     {
         Tensor r = makeResult(value().sqrt(), isRequireGrad());
@@ -297,6 +413,15 @@ public:
 
     Tensor mean() const { return sum() / (float)value().size(); }
     Tensor mean(size_t dim, bool keepDim = false) const { return sum(dim, keepDim) / (float)shape()[dim]; }
+
+    // aixCore.hpp:2626-2633
+    Tensor var(size_t dim, bool unbiased = true, bool keepDim = false) const
+    {
+        const Tensor deviation = *this - mean(dim, true);
+        const size_t count = unbiased ? shape()[dim] - 1 : shape()[dim];
+        const Tensor v = (deviation * deviation).sum(dim, true) / float(count);
+        return keepDim ? v : v.squeeze(dim);
+    }
 
     Tensor max(size_t dim, bool keepDim = false) const
     {

@@ -15,6 +15,7 @@ struct MlpConfig {
     uint64_t batch, in, hidden, out;
     int32_t steps;
     float lr;
+    int32_t singlePass;       // 0: the reference's path-by-path backward(); 1: Tensor::backwardOnce()
 };
 
 struct MlpHost {              // host arrays, f32, row-major
@@ -40,7 +41,7 @@ inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* l
         opt.zeroGrad();
         const Tensor logits = l3.forward(relu(l2.forward(relu(l1.forward(x)))));
         const Tensor loss = crossEntropy(softmax(logits, 1, true), y);
-        loss.backward();
+        if (cfg.singlePass) loss.backwardOnce(); else loss.backward();
         opt.step();
         losses[s] = loss.value().item();          // synchronizes
         if (step_seconds) step_seconds[s] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();

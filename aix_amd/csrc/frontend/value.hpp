@@ -339,6 +339,45 @@ public:
         return r;
     }
 
+    // aixCore.hpp:1320-1346
+    Value tril(ssize_t diagonal = 0) const
+    {
+        Value r(m_dev, m_dt, m_shape);
+        m_dev->tril(params(), r.params(), diagonal);
+        return r;
+    }
+
+    // Zero-padded copy of `src` into the window of a tensor shaped like *this (aixCore.hpp:1147-1204, not in place).
+    Value sliceSet(const Value& src, size_t dim, size_t start, size_t end, size_t step = 1) const
+    {
+        Value r = full(m_dev, m_dt, m_shape, 0.0f);
+        m_dev->sliceSet(src.params(), r.params(), dim, start, end, step);
+        return r;
+    }
+
+    // Rows (dim = 0) or other slabs picked by an int32 index vector (aixCore.hpp:1217-1247).
+    Value indexSelect(size_t dim, const Value& indices) const
+    {
+        Shape shape = m_shape;
+        shape[dim] = indices.shape().empty() ? 1 : indices.shape()[0];
+        Value r(m_dev, m_dt, shape);
+        m_dev->indexSelect(params(), r.params(), indices.params(), dim);
+        return r;
+    }
+
+    // *this[indices] += source, in place (aixCore.hpp:1249-1294 with inPlace = true).
+    void indexAddInPlace(size_t dim, const Value& indices, const Value& source) const
+    {
+        m_dev->indexAdd(source.params(), params(), indices.params(), dim);
+    }
+
+    Value pow(const Value& e) const
+    {
+        Value r(m_dev, m_dt, m_shape);
+        m_dev->pow(params(), e.params(), r.params());
+        return r;
+    }
+
     // First element on the host, after a synchronize(); device memory is host-readable on both
     // backends (plain memory on the CPU, large-BAR mapping on the GPU).
     float item() const

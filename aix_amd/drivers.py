@@ -33,7 +33,7 @@ def load():
         lib.aixbench_reduce_item.argtypes = [P, C.c_int, C.c_uint64, C.c_uint64, P, P, C.c_int, C.c_int, C.POINTER(BenchResult), P]
         lib.aixbench_matmul.argtypes = [P, C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_uint64, P, P, C.c_int, C.c_int,
                                         C.POINTER(BenchResult), P]
-        lib.aixbench_mlp.argtypes = [P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, _PF, _PF, _PPF, _PPF,
+        lib.aixbench_mlp.argtypes = [P, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int, _PF, _PF, _PPF, _PPF,
                                      _PF, C.POINTER(C.c_double)]
         _lib = lib
     return _lib
@@ -53,14 +53,32 @@ def _pointer_array(arrays):
     return arr
 
 
-def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data):
+def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data, single_pass=False):
     """Train the MLP (n_in -> hidden -> hidden -> n_out, ReLU, softmax + cross-entropy, Adam) for
     `steps` steps on `dev` from host arrays data = (x, onehot, [w1, w2, w3], [b1, b2, b3]).
+    single_pass=True differentiates once per node instead of once per path (the reference's way).
     Returns (loss per step, seconds per step)."""
     x, y, w, b = data
     losses = np.zeros(steps, dtype=np.float32)
     secs = np.zeros(steps, dtype=np.float64)
     pw, pb = _pointer_array(w), _pointer_array(b)
-    run("aixbench_mlp", dev.handle, batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+    run("aixbench_mlp", dev.handle, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
         pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
     return losses, secs
+
+
+def transformer(dev, cfg, steps, data):
+    """Forward + backward of the decoder-only transformer for `steps` steps on `dev`;
+    cfg = (layers, d_model, heads, seq, batch, vocab), data = (int32 tokens [batch * seq], list of f32
+    parameter arrays in the order of frontend/transformer.hpp).  Returns (losses, gradient norms
+    [steps, parameters], seconds per step)."""
+    tokens, params = data
+    lib = load()
+    lib.aixbench_transformer.argtypes = [C.c_void_p] + [C.c_uint64] * 6 + [C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
+    losses = np.zeros(steps, np.float32)
+    norms = np.zeros((steps, len(params)), np.float32)
+    secs = np.zeros(steps, np.float64)
+    pp = _pointer_array(params)
+    run("aixbench_transformer", dev.handle, *cfg, steps, tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
+        norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
+    return losses, norms, secs

@@ -51,7 +51,7 @@ def oracle_lib():
             from . import cpuref
             cpuref.build(ref=False)
         _oracle = C.CDLL(path)
-        _oracle.oracle_mlp.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float,
+        _oracle.oracle_mlp.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int,
                                        _PF, _PF, _PPF, _PPF, _PF, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
         _oracle.oracle_drivers_last_error.restype = C.c_char_p
     return _oracle
@@ -71,14 +71,14 @@ def ref_lib():
     return _ref
 
 
-def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1):
+def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pass=False):
     """Losses per step, seconds per step and (operator calls, matmul calls) of the oracle run."""
     x, y, w, b = data
     losses = np.zeros(steps, dtype=np.float32)
     secs = np.zeros(steps, dtype=np.float64)
     counts = (C.c_uint64 * 2)()
     pw, pb = pointer_array(w), pointer_array(b)
-    rc = oracle_lib().oracle_mlp(threads, batch, n_in, hidden, n_out, steps, lr, x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+    rc = oracle_lib().oracle_mlp(threads, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
                                  pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), counts)
     if rc != 0:
         raise RuntimeError(oracle_lib().oracle_drivers_last_error().decode())
@@ -130,3 +130,47 @@ def ref_hip_mlp(batch, n_in, hidden, n_out, steps, lr):
     if out.returncode != 0:
         raise RuntimeError("reference front-end on DeviceHIP failed: " + out.stderr[-2000:])
     return np.array(json.loads(out.stdout.strip().splitlines()[-1]), dtype=np.float32)
+
+
+# ---- transformer (configs[4]) ------------------------------------------------------------------------
+def transformer_param_shapes(layers, d, heads, seq, batch, vocab):
+    """Parameter order of aix_amd/csrc/frontend/transformer.hpp."""
+    shapes = [(vocab, d), (seq, d)]
+    for _ in range(layers):
+        shapes += [(1, d), (1, d), (d, d), (1, d), (d, d), (1, d), (d, d), (1, d), (d, d), (1, d),
+                   (1, d), (1, d), (d, 4 * d), (1, 4 * d), (4 * d, d), (1, d)]
+    shapes += [(1, d), (1, d), (d, vocab)]
+    return shapes
+
+
+def transformer_data(layers, d, heads, seq, batch, vocab, seed_tok=7, seed_w=8):
+    """Token ids U[0, vocab), weights N(0, 0.02) (LayerNorm gains 1, all biases 0), f32 on the host."""
+    tokens = np.random.default_rng(seed_tok).integers(0, vocab, size=batch * seq).astype(np.int32)
+    rng = np.random.default_rng(seed_w)
+    params = []
+    for shape in transformer_param_shapes(layers, d, heads, seq, batch, vocab):
+        if shape[0] == 1:
+            params.append(np.zeros(shape, np.float32))
+        else:
+            params.append((rng.standard_normal(shape) * 0.02).astype(np.float32))
+    # LayerNorm gains are the [1, d] arrays at block offsets 0 and 10, and the first of the last three
+    gains = [2 + 16 * l + o for l in range(layers) for o in (0, 10)] + [2 + 16 * layers]
+    for g in gains:
+        params[g][:] = 1.0
+    return tokens, params
+
+
+def oracle_transformer(cfg, steps, data, threads=1):
+    """cfg = (layers, d, heads, seq, batch, vocab).  Returns (losses, grad norms [steps, P], seconds)."""
+    tokens, params = data
+    lib = oracle_lib()
+    lib.oracle_transformer.argtypes = [C.c_int] + [C.c_uint64] * 6 + [C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
+    losses = np.zeros(steps, np.float32)
+    norms = np.zeros((steps, len(params)), np.float32)
+    secs = np.zeros(steps, np.float64)
+    pp = pointer_array(params)
+    rc = lib.oracle_transformer(threads, *cfg, steps, tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
+                                norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
+    if rc != 0:
+        raise RuntimeError(lib.oracle_drivers_last_error().decode())
+    return losses, norms, secs

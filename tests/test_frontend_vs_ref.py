@@ -33,3 +33,15 @@ def test_threads_do_not_change_the_trace():
     one, _, _ = drivers.oracle_mlp(64, 30, 40, 10, 5, 1e-3, data, threads=1)
     four, _, _ = drivers.oracle_mlp(64, 30, 40, 10, 5, 1e-3, data, threads=4)
     assert one.view(np.uint32).tolist() == four.view(np.uint32).tolist()
+
+
+def test_single_pass_backward_gives_the_same_gradients():
+    """Tensor::backwardOnce() (each node differentiated once with the summed seed) against the
+    reference's recursion (once per path): same formulas, different summation order, so the loss
+    traces of 30 Adam steps agree to rounding."""
+    shape = (48, 20, 24, 10)
+    data = drivers.mlp_data(*shape)
+    per_path, _, (ops_a, mm_a) = drivers.oracle_mlp(*shape, 30, 1e-3, data)
+    once, _, (ops_b, mm_b) = drivers.oracle_mlp(*shape, 30, 1e-3, data, single_pass=True)
+    assert np.all(np.abs(per_path.astype(np.float64) - once) <= 2e-6 * np.abs(per_path))
+    assert mm_b == 30 * (3 + 5) and mm_a == 30 * (3 + 4 * 5)

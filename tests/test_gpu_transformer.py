@@ -1,0 +1,41 @@
+"""Decoder-only transformer forward + backward (aix_amd/csrc/frontend/transformer.hpp, bf16 activations,
+f32 master parameters) on DeviceHIP against the CPU device, at reduced sizes the CPU finishes in
+seconds: the loss and the L2 norm of every parameter's gradient are compared.
+
+Tolerance: 2e-2 relative, the bar for 16-bit work with f32 accumulation.  The devices differ by
+design in how they add bf16 numbers (the GPU accumulates reductions and matmuls in f32 and rounds
+once; the CPU device rounds to bf16 after every addition), which is the larger part of what is
+observed; the observed deviations are printed."""
+import numpy as np
+import pytest
+
+from oracle import drivers as OD
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    from aix_amd import device as D
+    d = D.Device(0)
+    yield d
+    d.close()
+
+
+@pytest.mark.parametrize("cfg", [(2, 64, 4, 32, 2, 128), (1, 32, 2, 24, 3, 80), (3, 128, 8, 64, 2, 256)], ids=str)
+def test_loss_and_gradient_norms_match_the_cpu_device(dev, cfg):
+    from aix_amd import drivers as GD
+    data = OD.transformer_data(*cfg)
+    want_l, want_n, _ = OD.oracle_transformer(cfg, 2, data, threads=16)
+    got_l, got_n, secs = GD.transformer(dev, cfg, 2, data)
+    rel_l = np.abs(got_l.astype(np.float64) - want_l) / np.abs(want_l)
+    big = want_n > 1e-3 * want_n.max()                # norms that are not numerically zero (biases start at 0 but have gradients)
+    rel_n = np.abs(got_n.astype(np.float64) - want_n)[big] / want_n[big]
+    print(f"transformer {cfg}: loss {want_l[0]:.6f} (cpu) {got_l[0]:.6f} (gpu), rel dev {rel_l.max():.2e}; "
+          f"{int(big.sum())} gradient norms, max rel dev {rel_n.max():.2e}, median {np.median(rel_n):.2e}; gpu {secs[1] * 1e3:.1f} ms/step")
+    assert np.all(np.isfinite(got_l)) and np.all(np.isfinite(got_n))
+    assert abs(want_l[0] - np.log(cfg[5]) / cfg[5]) < 0.05 * want_l[0], "untrained model: loss is ln(V) / V with the reference's mean over all elements"
+    # no optimizer step: both steps see the same parameters (embedding gradients are summed with atomics, in any order)
+    assert got_l[0] == got_l[1] and np.allclose(got_n[0], got_n[1], rtol=1e-3, atol=0)
+    assert rel_l.max() <= 2e-2
+    assert rel_n.max() <= 2e-2
