@@ -142,7 +142,14 @@ struct PendingFill {
 
 class Planner {
 public:
-    Planner(const std::vector<OpRecord>& ops, const FuseConfig& cfg, const std::unordered_set<const void*>& live)
+    // A buffer outlives the window if somebody still holds it or if it is about to be read outside the planner.
+    struct Liveness {
+        const std::unordered_set<const void*>& held;
+        const std::unordered_set<const void*>& external;
+        size_t count(const void* p) const { return held.count(p) || external.count(p) ? 1 : 0; }
+    };
+
+    Planner(const std::vector<OpRecord>& ops, const FuseConfig& cfg, Liveness live)
         : m_ops(ops), m_cfg(cfg), m_live(live), m_operands(ops.size()), m_groupOf(ops.size(), SIZE_MAX) {}
 
     void run()
@@ -503,7 +510,7 @@ private:
 
     const std::vector<OpRecord>& m_ops;
     const FuseConfig& m_cfg;
-    const std::unordered_set<const void*>& m_live;
+    const Liveness m_live;
     std::vector<std::array<Operand, 2>> m_operands;
     std::vector<size_t> m_groupOf;
     std::vector<Group> m_groups;
@@ -585,8 +592,7 @@ void FuseEngine::flush()
     std::vector<OpRecord> window;
     window.swap(m_pending);
     // buffers about to be read outside the planner count as alive for this window
-    std::unordered_set<const void*> live = m_live;
-    live.insert(m_externalReads.begin(), m_externalReads.end());
+    const Planner::Liveness live{m_live, m_externalReads};
 
     size_t fusedKernels = 0, fusedOps = 0, singles = 0, absorbed = 0;
     std::ostringstream groupsText;
