@@ -399,29 +399,44 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
         for (int i = 0; i < CB; ++i) { const int c = tid + 256 * i; *(f32x4*)&Bs[buf][c >> 3][(c & 7) * 4] = rb[i]; }
     };
 
+    // Fragments are double buffered: the four ds_read_b128 of the next 8-wide K slice are issued
+    // under the 16 MFMAs of the current one; the tile for the next step goes to the other LDS buffer
+    // under the third slice; the step's barrier sits before the last slice, whose MFMAs cover the
+    // first fragment reads from that buffer.  sched_barrier keeps the phases apart (left alone,
+    // the compiler emits "4 reads, wait, 16 MFMAs" per slice and exposes the LDS latency each time).
+    f32x4 fa[2][TI], fb[2][TJ];
+    auto read_frags = [&](int set, int buf, int kk) {
+#pragma unroll
+        for (int i = 0; i < TI; ++i) fa[set][i] = *(const f32x4*)&As[buf][wm * WM + i * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) fb[set][j] = *(const f32x4*)&Bs[buf][wn * WN + j * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
+    };
+    auto mma = [&](int set) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i][s], fb[set][j][s], acc[i][j], 0, 0, 0);
+    };
     const u64 steps = (g.K + BK - 1) / BK;
     load_global(0);
     store_lds(0);
     __syncthreads();
+    read_frags(0, 0, 0);
     for (u64 kt = 0; kt < steps; ++kt) {
         const int buf = (int)(kt & 1);
-        if (kt + 1 < steps) load_global((kt + 1) * BK);
-#pragma unroll
-        for (int kk = 0; kk < BK / 8; ++kk) {
-            f32x4 fa[TI], fb[TJ];
-#pragma unroll
-            for (int i = 0; i < TI; ++i) fa[i] = *(const f32x4*)&As[buf][wm * WM + i * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
-#pragma unroll
-            for (int j = 0; j < TJ; ++j) fb[j] = *(const f32x4*)&Bs[buf][wn * WN + j * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int i = 0; i < TI; ++i)
-#pragma unroll
-                    for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
-        }
-        if (kt + 1 < steps) store_lds(buf ^ 1);
+        load_global((kt + 1 < steps ? kt + 1 : kt) * BK);       // past the end: the last tile again, into a buffer nobody reads
+        read_frags(1, buf, 1); mma(0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(0, buf, 2); mma(1);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(1, buf, 3); store_lds(buf ^ 1); mma(0);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(0, buf ^ 1, 0); mma(1);
+        __builtin_amdgcn_sched_barrier(0);
     }
 
     float* C = (float*)g.c;
