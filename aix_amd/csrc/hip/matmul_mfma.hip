@@ -352,10 +352,11 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
 // ---- f32 operands ------------------------------------------------------------------------------
 // 128 x 128 workgroup tile, BK = 32; LDS row = 32 floats + 4 padding = 144 bytes.  A lane reads 4
 // consecutive K of its row with one ds_read_b128 and spends them on 4 successive 32x32x2 MFMAs.
+template <int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
 {
-    constexpr int BM = 128, BN = 128, BK = 32, LDR = BK + 4;
-    constexpr int WM = 64, WN = 64, TI = 2, TJ = 2;
+    constexpr int BK = 32, LDR = BK + 4;
+    constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
     constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;      // 4 each
     extern __shared__ __attribute__((aligned(16))) unsigned char smem32[];
     float (*As)[BM][LDR] = (float (*)[BM][LDR])smem32;                       // [2][BM][LDR]
@@ -492,7 +493,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
     const size_t esz = aixk_dtype_size(out->dtype);
     const uint64_t kq = 16 / esz;                                 // elements per 16-byte chunk
     if (K % kq != 0 || M * N < 64 * 64) return -1;                // odd K / tiny outputs: LDS-tiled kernel
-    if (((M + 127) / 128) * ((N + 127) / 128) >= (1ull << 31)) return -1;
+    if (((M + 63) / 64) * ((N + 63) / 64) >= (1ull << 31)) return -1;
 
     // 16-bit, whole 256 x 256 x 64 tiles, enough of them: every operand layout is consumed where it lies
     // (K-contiguous, or "T" form with unit stride along M / N), no gathers.
@@ -564,11 +565,20 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         g.swizzle = n % 8u == 0 ? 1u : 0u;
         return n;
     };
+    // problems that 128 x 128 tiles cannot spread over the chip twice use 64 x 64 tiles
+    const bool small_tiles = ((M + 127) / 128) * ((N + 127) / 128) < (uint64_t)ctx->cus * 2;
     if (out->dtype == AIXK_F32) {
-        constexpr size_t lds = 2 * (128 + 128) * 36 * sizeof(float);
-        const u32 n = grid_of(128, 128);
-        AIXK_TRY(set_lds(gemm_nt32_k, lds));
-        hipLaunchKernelGGL(gemm_nt32_k, dim3(n), dim3(256), lds, ctx->stream, g);
+        if (small_tiles) {
+            constexpr size_t lds = 2 * (64 + 64) * 36 * sizeof(float);
+            const u32 n = grid_of(64, 64);
+            AIXK_TRY(set_lds(gemm_nt32_k<64, 64>, lds));
+            hipLaunchKernelGGL((gemm_nt32_k<64, 64>), dim3(n), dim3(256), lds, ctx->stream, g);
+        } else {
+            constexpr size_t lds = 2 * (128 + 128) * 36 * sizeof(float);
+            const u32 n = grid_of(128, 128);
+            AIXK_TRY(set_lds(gemm_nt32_k<128, 128>, lds));
+            hipLaunchKernelGGL((gemm_nt32_k<128, 128>), dim3(n), dim3(256), lds, ctx->stream, g);
+        }
         AIXK_HIP(hipGetLastError());
         return AIXK_OK;
     }
@@ -578,6 +588,11 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         const u32 n = grid_of(256, 256);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }
         else { AIXK_TRY(set_lds(gemm_nt16_k<f16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<f16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }
+    } else if (small_tiles) {
+        constexpr size_t lds = 2 * (64 + 64) * 72 * 2;
+        const u32 n = grid_of(64, 64);
+        if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 64, 64>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 64, 64>), dim3(n), dim3(256), lds, ctx->stream, g); }
+        else { AIXK_TRY(set_lds(gemm_nt16_k<f16, 64, 64>, lds)); hipLaunchKernelGGL((gemm_nt16_k<f16, 64, 64>), dim3(n), dim3(256), lds, ctx->stream, g); }
     } else {
         constexpr size_t lds = 2 * (128 + 128) * 72 * 2;
         const u32 n = grid_of(128, 128);
