@@ -42,10 +42,11 @@ struct Timer {
         t0 = std::chrono::steady_clock::now();
         aixk_event_record(dev->kernelContext(), e0);
     }
-    void stop(double* wall_s, float* gpu_ms)
+    void stop(double* wall_s, float* gpu_ms, int32_t* enqueue_us = nullptr)
     {
         dev->flush();
         aixk_event_record(dev->kernelContext(), e1);
+        if (enqueue_us) *enqueue_us = (int32_t)(std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() * 1e6);
         dev->synchronize();
         *wall_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         aixk_event_elapsed_ms(dev->kernelContext(), e0, e1, gpu_ms);
@@ -66,7 +67,7 @@ typedef struct aixbench_result {
     double wall_s;        // K steps, synchronize to synchronize
     float  gpu_ms;        // same region between two events on the device's stream
     int32_t steps;
-    int32_t reserved;
+    int32_t enqueue_us;   // host time to issue the K steps (before waiting for the device)
 } aixbench_result;
 
 const char* aixbench_last_error(void) { return g_err; }
@@ -91,7 +92,7 @@ int aixbench_fused_chain(aixhip_device* handle, uint64_t rows, uint64_t cols, co
         Timer t(dev);
         t.start();
         for (int i = 0; i < steps; ++i) step();
-        t.stop(&res->wall_s, &res->gpu_ms);
+        t.stop(&res->wall_s, &res->gpu_ms, &res->enqueue_us);
         res->steps = steps;
         if (y_out) dev->copyToHost(y_out, y.data(), rows * cols * sizeof(float));
     });
@@ -124,7 +125,7 @@ int aixbench_reduce_item(aixhip_device* handle, int which, uint64_t rows, uint64
         Timer t(dev);
         t.start();
         for (int i = 0; i < steps; ++i) step();
-        t.stop(&res->wall_s, &res->gpu_ms);
+        t.stop(&res->wall_s, &res->gpu_ms, &res->enqueue_us);
         res->steps = steps;
         if (out) dev->copyToHost(out, r.data(), r.size() * aix::Device::dataTypeSize(r.dtype()));
     });
@@ -158,7 +159,7 @@ int aixbench_matmul(aixhip_device* handle, int dtype, uint64_t M, uint64_t N, ui
         Timer t(dev);
         t.start();
         for (int i = 0; i < steps; ++i) step();
-        t.stop(&res->wall_s, &res->gpu_ms);
+        t.stop(&res->wall_s, &res->gpu_ms, &res->enqueue_us);
         res->steps = steps;
         if (out) dev->copyToHost(out, r[0].data(), M * N * aix::Device::dataTypeSize(dt));
     });

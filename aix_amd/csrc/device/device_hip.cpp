@@ -35,6 +35,7 @@ using aixhip::fuse::FuseEngine;
 using aixhip::fuse::FusedSubgraphDescriptor;
 using aixhip::fuse::OpRecord;
 using aixhip::fuse::OpType;
+using aixhip::fuse::View;
 namespace gen = aixhip::gen;
 
 namespace {
@@ -44,47 +45,27 @@ namespace {
 struct Cooling {
     aixk_event* event;
     std::vector<std::pair<void*, size_t>> blocks;
+    size_t bytes{0};
 };
 
-struct Extras {
-    std::deque<Cooling> cooling;
-    unsigned flushesSinceEvent{0};
-    std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
-    uint64_t hits{0}, misses{0};
-};
-
-std::unordered_map<const DeviceHIP*, Extras>& extras()
-{
-    static std::unordered_map<const DeviceHIP*, Extras> e;
-    return e;
-}
-
-size_t viewEnd(const DeviceTensorParams& p)
+size_t viewEnd(const View& p)
 {
     size_t last = p.offset;
-    for (size_t d = 0; d < p.shape.size(); ++d) {
+    for (size_t d = 0; d < p.rank; ++d) {
         if (p.shape[d] == 0) return p.offset;
         last += (p.shape[d] - 1) * p.strides[d];
     }
     return last + 1;
 }
 
-bool isDense(const DeviceTensorParams& p)
+size_t viewEnd(const aixhip_tensor& p)
 {
-    size_t run = 1;
-    for (size_t d = p.shape.size(); d-- > 0;) {
-        if (p.shape[d] != 1 && p.strides[d] != run) return false;
-        run *= p.shape[d];
+    size_t last = p.offset;
+    for (int d = 0; d < p.rank; ++d) {
+        if (p.shape[d] == 0) return p.offset;
+        last += (p.shape[d] - 1) * p.strides[d];
     }
-    return true;
-}
-
-Stride denseStrides(const Shape& shape)
-{
-    Stride s(shape.size());
-    size_t run = 1;
-    for (size_t d = shape.size(); d-- > 0;) { s[d] = run; run *= shape[d]; }
-    return s;
+    return last + 1;
 }
 
 int binaryCode(OpType t)
@@ -106,6 +87,86 @@ int unaryCode(OpType t)
 
 } // namespace
 
+struct DeviceHIP::Extras {
+    std::deque<Cooling> cooling;
+    size_t coolingBytes{0};
+    unsigned flushesSinceEvent{0};
+    std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
+    uint64_t hits{0}, misses{0};
+    // working storage of emitFused, kept from kernel to kernel
+    std::string key;
+    std::vector<uint64_t> args;
+    gen::Space space;
+};
+
+// ---- block table -------------------------------------------------------------------------------
+DeviceHIP::Block* DeviceHIP::BlockTable::find(const void* base) const
+{
+    if (m_slots.empty()) return nullptr;
+    const uintptr_t key = (uintptr_t)base;
+    const size_t mask = m_slots.size() - 1;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i].key == key) return &m_slots[i].block;
+        if (m_slots[i].key == 0) return nullptr;
+    }
+}
+
+DeviceHIP::Block* DeviceHIP::BlockTable::findContaining(const void* p) const
+{
+    const uintptr_t a = (uintptr_t)p;
+    for (const auto& s : m_slots) if (s.key > 1 && a >= s.key && a < s.key + s.block.bytes) return &s.block;
+    return nullptr;
+}
+
+void DeviceHIP::BlockTable::grow()
+{
+    std::vector<Slot> old;
+    old.swap(m_slots);
+    size_t capacity = 256;
+    while (capacity < m_count * 4) capacity <<= 1;
+    m_slots.assign(capacity, Slot{});
+    m_shift = 64;
+    for (size_t c = capacity; c > 1; c >>= 1) --m_shift;
+    m_used = m_count;
+    const size_t mask = capacity - 1;
+    for (const auto& s : old) {
+        if (s.key <= 1) continue;
+        size_t i = slotOf(s.key);
+        while (m_slots[i].key != 0) i = (i + 1) & mask;
+        m_slots[i] = s;
+    }
+}
+
+void DeviceHIP::BlockTable::insert(void* base, size_t bytes)
+{
+    const uintptr_t key = (uintptr_t)base;
+    if ((m_used + 1) * 2 > m_slots.size()) grow();
+    const size_t mask = m_slots.size() - 1;
+    size_t grave = SIZE_MAX;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i].key == key) { m_slots[i].block = Block{bytes}; return; }
+        if (m_slots[i].key == 1 && grave == SIZE_MAX) grave = i;
+        if (m_slots[i].key == 0) {
+            if (grave != SIZE_MAX) i = grave; else ++m_used;
+            m_slots[i].key = key;
+            m_slots[i].block = Block{bytes};
+            ++m_count;
+            return;
+        }
+    }
+}
+
+bool DeviceHIP::BlockTable::erase(void* base, size_t* bytes)
+{
+    if (m_slots.empty()) return false;
+    const uintptr_t key = (uintptr_t)base;
+    const size_t mask = m_slots.size() - 1;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i].key == key) { *bytes = m_slots[i].block.bytes; m_slots[i].key = 1; --m_count; return true; }
+        if (m_slots[i].key == 0) return false;
+    }
+}
+
 // ---- construction ------------------------------------------------------------------------------
 DeviceHIP::DeviceHIP(size_t deviceIndex)
 {
@@ -113,13 +174,14 @@ DeviceHIP::DeviceHIP(size_t deviceIndex)
     if (rc != AIXK_OK) throw std::runtime_error(std::string("DeviceHIP: ") + aixk_last_error());
     aixk_device_info info{};
     if (aixk_info(m_ctx, &info) == AIXK_OK && info.compute_units > 0) m_cus = info.compute_units;
+    m_totalBytes = info.total_mem;
     if (aixk_info(m_ctx, &info) == AIXK_OK && !info.large_bar)
         std::cerr << "DeviceHIP: device memory is not host-addressable on this system; tensors must be moved with "
                      "copy()/copyToHost() and never dereferenced on the host." << std::endl;
     FuseConfig cfg;
     cfg.maxBufferSlots = 24;
     cfg.supportsStridedFusion = true;
-    extras()[this];
+    m_extras = std::make_unique<Extras>();
     setFuseConfig(cfg);
 }
 
@@ -131,16 +193,15 @@ DeviceHIP::~DeviceHIP()
         if (m_engine) m_engine.reset();
         if (m_ctx) {
             aixk_sync(m_ctx);
-            auto& ex = extras()[this];
+            auto& ex = *m_extras;
             for (auto& c : ex.cooling) { aixk_event_destroy(m_ctx, c.event); for (auto& b : c.blocks) aixk_free(m_ctx, b.first, 0); }
             for (auto& b : m_limbo) aixk_free(m_ctx, b.first, 0);
             for (auto& kv : m_pool) for (void* p : kv.second) aixk_free(m_ctx, p, 0);
-            for (auto& kv : m_blocks) aixk_free(m_ctx, (void*)kv.first, 0);
+            m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) aixk_free(m_ctx, base, 0); });
             aixk_destroy(m_ctx);
         }
     } catch (...) {
     }
-    extras().erase(this);
 }
 
 std::unique_ptr<aix::Device> createDeviceHIP(size_t deviceIndex)
@@ -158,13 +219,12 @@ void DeviceHIP::setFuseConfig(const FuseConfig& cfg)
     cb.finishFlush = [] {};
     cb.getKernelCacheStats = [this] { return fuseKernelCacheStats(); };
     m_engine = std::make_unique<FuseEngine>(cfg, std::move(cb));
-    for (auto& kv : m_blocks) m_engine->retainBuffer((void*)kv.first);
+    m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) m_engine->retainBuffer(base); });
 }
 
 std::pair<size_t, size_t> DeviceHIP::fuseKernelCacheStats() const
 {
-    const auto& ex = extras()[this];
-    return {(size_t)ex.hits, (size_t)ex.misses};
+    return {(size_t)m_extras->hits, (size_t)m_extras->misses};
 }
 
 void DeviceHIP::check(int status) const
@@ -179,10 +239,8 @@ void DeviceHIP::check(int status) const
 const DeviceHIP::Block* DeviceHIP::findBlock(const void* p) const
 {
     if (!p || m_blocks.empty()) return nullptr;
-    auto it = m_blocks.upper_bound((uintptr_t)p);
-    if (it == m_blocks.begin()) return nullptr;
-    --it;
-    return ((uintptr_t)p < it->first + it->second.bytes) ? &it->second : nullptr;
+    if (const Block* exact = m_blocks.find(p)) return exact;
+    return m_blocks.findContaining(p);
 }
 
 // 256-byte steps up to 4 KiB, then eight steps per power of two: at most 12.5 % slack, few buckets.
@@ -198,12 +256,13 @@ size_t DeviceHIP::bucketBytes(size_t bytes) const
 
 void* DeviceHIP::allocateBlock(size_t bytes, bool track)
 {
-    auto& ex = extras()[this];
+    auto& ex = *m_extras;
     // blocks whose release point the GPU has passed become reusable
     while (!ex.cooling.empty()) {
         int32_t done = 0;
         if (aixk_event_query(m_ctx, ex.cooling.front().event, &done) != AIXK_OK || !done) break;
         for (auto& b : ex.cooling.front().blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        ex.coolingBytes -= ex.cooling.front().bytes;
         aixk_event_destroy(m_ctx, ex.cooling.front().event);
         ex.cooling.pop_front();
     }
@@ -222,7 +281,7 @@ void* DeviceHIP::allocateBlock(size_t bytes, bool track)
             throw std::runtime_error(std::string("DeviceHIP: GPU memory allocation has failed for size: ") + std::to_string(bytes) + " bytes. " + aixk_last_error());
     }
     if (track) {
-        m_blocks[(uintptr_t)p] = Block{bucket};
+        m_blocks.insert(p, bucket);
         m_liveBytes += bucket;
         m_engine->retainBuffer(p);
     }
@@ -236,30 +295,64 @@ void* DeviceHIP::allocate(size_t size, DataType dtype) { return allocateBlock(si
 void DeviceHIP::deallocate(void* memory)
 {
     if (!memory) return;
-    auto it = m_blocks.find((uintptr_t)memory);
-    if (it == m_blocks.end()) throw std::invalid_argument("DeviceHIP::deallocate() - Found different type of memory to free.");   // aixDeviceMetal.cpp:253-254
+    Block* block = m_blocks.find(memory);
+    if (!block || block->freed) throw std::invalid_argument("DeviceHIP::deallocate() - Found different type of memory to free.");   // aixDeviceMetal.cpp:253-254
+    block->freed = true;                                    // stays in the table until the block leaves m_limbo: work recorded on it may still mark it
+    const size_t bytes = block->bytes;
     m_engine->releaseBuffer(memory);
-    m_limbo.emplace_back(memory, it->second.bytes);
-    m_limboBytes += it->second.bytes;
-    m_liveBytes -= it->second.bytes;
-    m_blocks.erase(it);
+    m_limbo.emplace_back(memory, bytes);
+    m_limboBytes += bytes;
+    m_liveBytes -= bytes;
     if (m_limboBytes > (size_t(8) << 30)) flush();          // recorded work pins too much freed memory
 }
 
+void DeviceHIP::markTouched(const void* p)
+{
+    if (!p || m_blocks.empty()) return;
+    Block* b = m_blocks.find(p);
+    if (!b) b = m_blocks.findContaining(p);
+    if (b) b->touched = true;
+}
+
 // Called once the recorded work that might touch freed blocks has been enqueued.
-// An event costs a marker packet between two kernels (a few microseconds of idle GPU), so it is
-// not recorded after every flush: freed blocks wait until 16 flushes have passed or until they
-// amount to 32 MiB and an eighth of what the device holds otherwise, whichever comes first.
+//
+// A freed block that no enqueued work has referenced since it was allocated -- a temporary whose
+// value stayed in registers of a fused kernel, an absorbed fill -- is idle and goes straight back
+// to the pool.  The others wait for the GPU to pass an event.  An event costs a marker packet
+// between two kernels (a few microseconds of idle GPU), so it is not recorded after every flush:
+// such blocks wait until 16 flushes have passed or until they amount to a thousandth of the card
+// (288 MiB of 288 GiB; at least 32 MiB) and an eighth of what the device holds otherwise,
+// whichever comes first.
 void DeviceHIP::releaseLimbo()
 {
     if (m_limbo.empty()) return;
-    auto& ex = extras()[this];
-    const size_t enough = std::max<size_t>(size_t(32) << 20, (m_liveBytes + m_pooledBytes) / 8);
+    auto& ex = *m_extras;
+    size_t kept = 0;
+    for (size_t k = 0; k < m_limbo.size(); ++k) {
+        const auto entry = m_limbo[k];
+        const Block* b = m_blocks.find(entry.first);        // staging blocks are not in the table: always used
+        if (b && !b->touched) {
+            size_t bytes = 0;
+            m_blocks.erase(entry.first, &bytes);
+            m_pool[entry.second].push_back(entry.first);
+            m_pooledBytes += entry.second;
+            m_limboBytes -= entry.second;
+        } else {
+            m_limbo[kept++] = entry;
+        }
+    }
+    m_limbo.resize(kept);
+    if (m_limbo.empty()) return;
+
+    const size_t enough = std::max<size_t>({size_t(32) << 20, m_totalBytes >> 10, (m_liveBytes + m_pooledBytes) / 8});
     if (++ex.flushesSinceEvent < 16 && m_limboBytes < enough) return;
     ex.flushesSinceEvent = 0;
+    for (const auto& entry : m_limbo) { size_t bytes = 0; m_blocks.erase(entry.first, &bytes); }
     Cooling c{};
     if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
         c.blocks.swap(m_limbo);
+        c.bytes = m_limboBytes;
+        ex.coolingBytes += c.bytes;
         ex.cooling.push_back(std::move(c));
     } else {
         aixk_sync(m_ctx);
@@ -287,6 +380,9 @@ void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
     m_engine->recordExternalRead(a);
     m_engine->recordExternalRead(b);
     m_engine->recordExternalRead(c);
+    markTouched(a);                                         // the caller is about to enqueue work on them
+    markTouched(b);
+    markTouched(c);
     flush();
 }
 
@@ -294,14 +390,15 @@ void DeviceHIP::synchronize()
 {
     flush();
     check(aixk_sync(m_ctx));
-    auto& ex = extras()[this];
+    auto& ex = *m_extras;
     for (auto& c : ex.cooling) {
         for (auto& b : c.blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
         aixk_event_destroy(m_ctx, c.event);
     }
     ex.cooling.clear();
+    ex.coolingBytes = 0;
     // everything recorded has been enqueued and has finished: blocks freed since the last event are idle too
-    for (auto& b : m_limbo) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+    for (auto& b : m_limbo) { size_t bytes = 0; m_blocks.erase(b.first, &bytes); m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
     m_limbo.clear();
     m_limboBytes = 0;
     ex.flushesSinceEvent = 0;
@@ -336,12 +433,11 @@ const void* DeviceHIP::stageRaw(const void* src, size_t bytes)
     return tmp;
 }
 
-DeviceTensorParams DeviceHIP::onDevice(const DeviceTensorParams& p)
+void DeviceHIP::onDevice(View& v)
 {
-    if (!p.data || p.size == 0 || findBlock(p.data)) return p;
-    DeviceTensorParams q = p;                               // a host tensor handed straight to the device (DeviceTests.cpp:209-215)
-    q.data = const_cast<void*>(stageRaw(p.data, viewEnd(p) * dataTypeSize(p.dtype)));
-    return q;
+    if (!v.data || v.size == 0 || findBlock(v.data)) return;
+    // a host tensor handed straight to the device (DeviceTests.cpp:209-215)
+    v.data = const_cast<void*>(stageRaw(v.data, viewEnd(v) * dataTypeSize(v.dtype)));
 }
 
 void DeviceHIP::toPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op) const
@@ -357,16 +453,37 @@ void DeviceHIP::toPod(const DeviceTensorParams& p, aixhip_tensor* out, const cha
     for (size_t d = 0; d < p.shape.size(); ++d) { out->shape[d] = p.shape[d]; out->strides[d] = d < p.strides.size() ? p.strides[d] : 0; }
 }
 
+void DeviceHIP::toPod(const View& v, aixhip_tensor* out) const
+{
+    std::memset(out, 0, sizeof(*out));
+    out->data = v.data;
+    out->dtype = (int32_t)v.dtype;
+    out->rank = (int32_t)v.rank;
+    out->offset = v.offset;
+    out->size = v.size;
+    for (size_t d = 0; d < v.rank; ++d) { out->shape[d] = v.shape[d]; out->strides[d] = v.strides[d]; }
+}
+
+void DeviceHIP::stagedPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op)
+{
+    toPod(p, out, op);
+    if (!out->data || out->size == 0 || findBlock(out->data)) return;
+    out->data = const_cast<void*>(stageRaw(out->data, viewEnd(*out) * dataTypeSize(p.dtype)));
+}
+
 // ---- recorded (fusable) operators --------------------------------------------------------------
 void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& r, const char* op)
 {
     requireDevice(r, op);
     if (a.dtype != r.dtype || b.dtype != r.dtype)
         throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operands must have the result's data type.");
-    if (a.shape.size() > AIXK_MAX_RANK) throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
-    DeviceTensorParams out = r;                             // results are written densely from the base pointer
-    out.offset = 0; out.strides = denseStrides(r.shape); out.isContiguous = true;
-    m_engine->record(t, onDevice(a), onDevice(b), out);
+    if (a.shape.size() > AIXK_MAX_RANK || b.shape.size() > AIXK_MAX_RANK || r.shape.size() > AIXK_MAX_RANK)
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
+    View va(a), vb(b), out(r);
+    out.makeDense();                                        // results are written densely from the base pointer
+    onDevice(va);
+    onDevice(vb);
+    m_engine->record(t, va, vb, out);
 }
 
 void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op)
@@ -374,12 +491,14 @@ void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceT
     requireDevice(r, op);
     if (a.dtype != r.dtype)
         throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operand must have the result's data type.");
-    if (a.shape.size() > AIXK_MAX_RANK) throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
-    DeviceTensorParams out = r;
-    out.offset = 0; out.strides = denseStrides(r.shape); out.isContiguous = true;
+    if (a.shape.size() > AIXK_MAX_RANK || r.shape.size() > AIXK_MAX_RANK)
+        throw std::invalid_argument(std::string("DeviceHIP::") + op + "() supports at most 16 dimensions.");
+    View va(a), out(r);
     out.size = a.size;                                      // unary loops run over the operand (aixDeviceCPU.cpp:90)
-    if (out.shape != a.shape) { out.shape = a.shape; out.strides = denseStrides(a.shape); }
-    m_engine->record(t, onDevice(a), out);
+    if (!out.sameShape(va)) { out.rank = va.rank; std::memcpy(out.shape, va.shape, va.rank * sizeof(size_t)); }
+    out.makeDense();
+    onDevice(va);
+    m_engine->record(t, va, out);
 }
 
 void DeviceHIP::add(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Add, a1, a2, result, "add"); }
@@ -398,16 +517,16 @@ void DeviceHIP::exp(const DeviceTensorParams& a, const DeviceTensorParams& resul
 void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTensorParams& result)
 {
     requireDevice(result, "fill");
-    DeviceTensorParams out = result;
-    out.offset = 0; out.strides = denseStrides(result.shape); out.isContiguous = true;
+    View out(result);
+    out.makeDense();
     m_engine->recordFill(scalar, scalarDType, out);
 }
 
 void DeviceHIP::fillMin(const DeviceTensorParams& result)
 {
     requireDevice(result, "fillMin");
-    DeviceTensorParams out = result;
-    out.offset = 0; out.strides = denseStrides(result.shape); out.isContiguous = true;
+    View out(result);
+    out.makeDense();
     m_engine->recordFillMin(out);
 }
 
@@ -415,12 +534,15 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
 void DeviceHIP::emitSingle(const OpRecord& op)
 {
     aixhip_tensor a, b, o;
-    toPod(op.output, &o, "emit");
+    markTouched(op.output.data);
+    markTouched(op.input0.data);
+    if (op.hasInput1) markTouched(op.input1.data);
+    toPod(op.output, &o);
     if (op.type == OpType::Fill) { check(aixk_fill(m_ctx, op.scalarData.data(), (int)op.scalarDType, &o)); return; }
     if (op.type == OpType::FillMin) { check(aixk_fill_min(m_ctx, &o)); return; }
-    toPod(op.input0, &a, "emit");
+    toPod(op.input0, &a);
     if (const int code = binaryCode(op.type); code >= 0) {
-        toPod(op.input1, &b, "emit");
+        toPod(op.input1, &b);
         check(aixk_binary(m_ctx, code, &a, &b, &o));
         return;
     }
@@ -430,68 +552,75 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 
 void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 {
+    constexpr size_t kMaxOperands = 64;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     const size_t esz = dataTypeSize(d.dtype);
     const size_t VEC = 16 / esz;
     const uint64_t n = d.elementCount;
     if (n == 0 || NO == 0) return;
+    const size_t rank = d.shape.size();
+    if (NI + 1 > kMaxOperands || NO > kMaxOperands || rank > aixhip::fuse::kMaxRank)
+        throw std::invalid_argument("DeviceHIP: fused kernel with too many operands or dimensions.");
 
     // Joint iteration space over the fused shape: dense views get the dense strides of that shape
     // (their own shape may be a different factorisation of the same count), strided views keep
     // theirs; one extra dense operand stands for the outputs so dims merge only where they may.
-    const Stride dense = denseStrides(d.shape);
-    const size_t rank = d.shape.size();
-    std::vector<Stride> strides(NI + 1);
+    size_t dense[aixhip::fuse::kMaxRank];
+    { size_t run = 1; for (size_t dd = rank; dd-- > 0;) { dense[dd] = run; run *= d.shape[dd]; } }
+    const size_t* strides[kMaxOperands];
     for (size_t k = 0; k < NI; ++k) {
         const auto& v = d.inputBuffers[k];
-        if (isDense(v)) strides[k] = dense;
-        else if (v.shape == d.shape) strides[k] = v.strides;
+        if (v.dense) strides[k] = dense;
+        else if (v.sameShape(d.shape)) strides[k] = v.strides;
         else throw std::runtime_error("DeviceHIP: fused kernel received a strided view of a foreign shape");
     }
     strides[NI] = dense;
     // collapse: drop extent-1 dims, merge neighbours where every operand allows it
-    std::vector<uint64_t> shp;
-    std::vector<std::vector<uint64_t>> str(NI + 1);
+    uint64_t shp[aixhip::fuse::kMaxRank];
+    uint64_t str[kMaxOperands][aixhip::fuse::kMaxRank];
+    size_t cr = 0;
     for (size_t dd = 0; dd < rank; ++dd) {
         if (d.shape[dd] == 1) continue;
         bool merged = false;
-        if (!shp.empty()) {
+        if (cr > 0) {
             bool ok = true;
-            for (size_t k = 0; k <= NI; ++k) if (str[k].back() != strides[k][dd] * d.shape[dd]) ok = false;
+            for (size_t k = 0; k <= NI; ++k) if (str[k][cr - 1] != strides[k][dd] * d.shape[dd]) ok = false;
             if (ok) {
-                shp.back() *= d.shape[dd];
-                for (size_t k = 0; k <= NI; ++k) str[k].back() = strides[k][dd];
+                shp[cr - 1] *= d.shape[dd];
+                for (size_t k = 0; k <= NI; ++k) str[k][cr - 1] = strides[k][dd];
                 merged = true;
             }
         }
         if (!merged) {
-            shp.push_back(d.shape[dd]);
-            for (size_t k = 0; k <= NI; ++k) str[k].push_back(strides[k][dd]);
+            shp[cr] = d.shape[dd];
+            for (size_t k = 0; k <= NI; ++k) str[k][cr] = strides[k][dd];
+            ++cr;
         }
     }
-    if (shp.size() > (size_t)gen::kMaxDims) throw std::invalid_argument("DeviceHIP: fused view does not collapse to 8 dimensions.");
+    if (cr > (size_t)gen::kMaxDims) throw std::invalid_argument("DeviceHIP: fused view does not collapse to 8 dimensions.");
 
     auto aligned = [](const void* p) { return ((uintptr_t)p & 15u) == 0; };
-    std::vector<const void*> inPtr(NI);
-    std::vector<void*> outPtr(NO);
-    for (size_t k = 0; k < NO; ++k) outPtr[k] = d.outputBuffers[k].data;
+    const void* inPtr[kMaxOperands];
+    void* outPtr[kMaxOperands];
     bool outsAligned = true;
-    for (void* p : outPtr) if (!aligned(p)) outsAligned = false;
+    for (size_t k = 0; k < NO; ++k) { outPtr[k] = d.outputBuffers[k].data; if (!aligned(outPtr[k])) outsAligned = false; }
+    for (size_t k = 0; k < NO; ++k) markTouched(d.outputBuffers[k].data);
+    for (size_t k = 0; k < NI; ++k) markTouched(d.inputBuffers[k].data);
 
     gen::Shape shape = gen::Shape::Gather;
     uint32_t bmask = 0;
     uint64_t chunks = 0;
-    const size_t cr = shp.size();
     if (cr <= 1) {
         bool ok = outsAligned;
         for (size_t k = 0; k < NI && ok; ++k) {
             const uint64_t s = cr ? str[k][0] : 0;
             const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
-            if (cr == 1 && s == 0) bmask |= 1u << k;
+            if (cr == 1 && s == 0) { if (k < 32) bmask |= 1u << k; else ok = false; }
             else if (cr == 1 && s != 1) ok = false;
             else if (!aligned(base)) ok = false;
         }
         if (ok) shape = gen::Shape::Flat;
+        else bmask = 0;
     } else {
         bool ok = outsAligned && shp[cr - 1] % VEC == 0;
         for (size_t k = 0; k < NI && ok; ++k) {
@@ -506,7 +635,8 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         if (ok) { shape = gen::Shape::Rows; chunks = shp[cr - 1] / VEC; }
     }
 
-    gen::Space space;
+    auto& ex = *m_extras;
+    gen::Space& space = ex.space;
     if (shape == gen::Shape::Flat) {
         for (size_t k = 0; k < NI; ++k) inPtr[k] = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
     } else {
@@ -521,29 +651,28 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         }
     }
 
-    auto& ex = extras()[this];
     bool noAlias = true;                                     // in-place updates: an output that is also an input
     for (const auto& ob : d.outputBuffers) for (const auto& ib : d.inputBuffers) if (ob.data == ib.data) noAlias = false;
-    const std::string key = gen::signature(d, shape, bmask, noAlias);
+    gen::signatureInto(ex.key, d, shape, bmask, noAlias);
     aixk_module* mod = nullptr;
-    auto it = ex.kernels.find(key);
+    auto it = ex.kernels.find(ex.key);
     if (it != ex.kernels.end()) { mod = it->second; ++ex.hits; }
     else {
         int32_t cached = 0;
         const std::string src = gen::source(d, shape, bmask, noAlias);
-        check(aixk_rtc_get(m_ctx, key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
-        ex.kernels.emplace(key, mod);
+        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
+        ex.kernels.emplace(ex.key, mod);
         ++ex.misses;
     }
 
-    const auto args = gen::packArgs(d, shape, inPtr, outPtr, n, shape == gen::Shape::Flat ? nullptr : &space, chunks);
+    gen::packArgsInto(ex.args, d, shape, inPtr, outPtr, n, shape == gen::Shape::Flat ? nullptr : &space, chunks);
     uint64_t items, perBlock, cap;
     if (shape == gen::Shape::Flat) { items = n / VEC + 1; perBlock = gen::kBlock; cap = 1u << 22; }
     else if (shape == gen::Shape::Rows) { items = n / VEC; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     else { items = n; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     uint64_t grid = (items + perBlock - 1) / perBlock;
     grid = std::max<uint64_t>(1, std::min(grid, cap));
-    check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, args.data(), args.size() * sizeof(uint64_t)));
+    check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
 }
 
 // ---- operators that run at once ------------------------------------------------------------------
@@ -551,7 +680,7 @@ void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& resul
 {
     requireDevice(result, "sum");
     flushFor(a.data, result.data);
-    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "sum"); toPod(result, &pr, "sum");
+    aixhip_tensor pa, pr; stagedPod(a, &pa, "sum"); toPod(result, &pr, "sum");
     check(aixk_reduce_all(m_ctx, AIXK_SUM, &pa, &pr));
 }
 
@@ -559,7 +688,7 @@ void DeviceHIP::max(const DeviceTensorParams& a, const DeviceTensorParams& resul
 {
     requireDevice(result, "max");
     flushFor(a.data, result.data);
-    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "max"); toPod(result, &pr, "max");
+    aixhip_tensor pa, pr; stagedPod(a, &pa, "max"); toPod(result, &pr, "max");
     check(aixk_reduce_all(m_ctx, AIXK_MAX, &pa, &pr));
 }
 
@@ -568,7 +697,7 @@ void DeviceHIP::argmax(const DeviceTensorParams& a, const DeviceTensorParams& re
     if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmax supports only int32 data type for its result.");
     requireDevice(result, "argmax");
     flushFor(a.data, result.data);
-    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "argmax"); toPod(result, &pr, "argmax");
+    aixhip_tensor pa, pr; stagedPod(a, &pa, "argmax"); toPod(result, &pr, "argmax");
     check(aixk_reduce_all(m_ctx, AIXK_ARGMAX, &pa, &pr));
 }
 
@@ -577,7 +706,7 @@ void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorPar
     if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndices supports only int32 data type for its result.");
     requireDevice(result, "argmaxIndices");
     flushFor(a.data, result.data);
-    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "argmaxIndices"); toPod(result, &pr, "argmaxIndices");
+    aixhip_tensor pa, pr; stagedPod(a, &pa, "argmaxIndices"); toPod(result, &pr, "argmaxIndices");
     check(aixk_reduce_all(m_ctx, AIXK_ARGMAX_ONEHOT, &pa, &pr));
 }
 
@@ -585,7 +714,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
 {
     requireDevice(result, "matmul");
     flushFor(a.data, b.data, result.data);
-    aixhip_tensor pa, pb, pr; toPod(onDevice(a), &pa, "matmul"); toPod(onDevice(b), &pb, "matmul"); toPod(result, &pr, "matmul");
+    aixhip_tensor pa, pb, pr; stagedPod(a, &pa, "matmul"); stagedPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
     check(aixk_matmul(m_ctx, &pa, &pb, &pr));
 }
 
@@ -593,7 +722,7 @@ void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams&
 {
     requireDevice(result, "transpose");
     flushFor(a.data, result.data);
-    aixhip_tensor pa, pr; toPod(onDevice(a), &pa, "transpose"); toPod(result, &pr, "transpose");
+    aixhip_tensor pa, pr; stagedPod(a, &pa, "transpose"); toPod(result, &pr, "transpose");
     check(aixk_transpose(m_ctx, &pa, &pr, dim0, dim1));
 }
 
@@ -620,7 +749,7 @@ void DeviceHIP::contiguous(const DeviceTensorParams& src, const DeviceTensorPara
 {
     requireDevice(dst, "contiguous");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "contiguous"); toPod(dst, &pd, "contiguous");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "contiguous"); toPod(dst, &pd, "contiguous");
     check(aixk_contiguous(m_ctx, &ps, &pd));
 }
 
@@ -662,7 +791,7 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
     check(folded ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));
 }
 
@@ -673,7 +802,7 @@ void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& d
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "maxTo"); toPod(dst, &pd, "maxTo");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "maxTo"); toPod(dst, &pd, "maxTo");
     check(folded ? aixk_reduce_to_init(m_ctx, AIXK_MAX, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_MAX, &ps, &pd));
 }
 
@@ -682,7 +811,7 @@ void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxTo");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "argmaxTo"); toPod(dst, &pd, "argmaxTo");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "argmaxTo"); toPod(dst, &pd, "argmaxTo");
     check(aixk_argmax_to(m_ctx, 0, &ps, &pd, dim));
 }
 
@@ -691,7 +820,7 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndicesTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxIndicesTo");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "argmaxIndicesTo"); toPod(dst, &pd, "argmaxIndicesTo");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "argmaxIndicesTo"); toPod(dst, &pd, "argmaxIndicesTo");
     check(aixk_argmax_to(m_ctx, 1, &ps, &pd, dim));
 }
 
@@ -700,7 +829,7 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::sliceSet() requires matching source and destination data types.");
     requireDevice(dst, "sliceSet");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "sliceSet"); toPod(dst, &pd, "sliceSet");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "sliceSet"); toPod(dst, &pd, "sliceSet");
     check(aixk_slice_set(m_ctx, &ps, &pd, dim, start, end, step));
 }
 
@@ -709,7 +838,7 @@ void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& ds
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::tril() requires matching source and destination data types.");   // aixDeviceMetal.cpp:1160-1161
     requireDevice(dst, "tril");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "tril"); toPod(dst, &pd, "tril");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "tril"); toPod(dst, &pd, "tril");
     check(aixk_tri(m_ctx, 0, &ps, &pd, diagonal));
 }
 
@@ -718,7 +847,7 @@ void DeviceHIP::triu(const DeviceTensorParams& src, const DeviceTensorParams& ds
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::triu() requires matching source and destination data types.");
     requireDevice(dst, "triu");
     flushFor(src.data, dst.data);
-    aixhip_tensor ps, pd; toPod(onDevice(src), &ps, "triu"); toPod(dst, &pd, "triu");
+    aixhip_tensor ps, pd; stagedPod(src, &ps, "triu"); toPod(dst, &pd, "triu");
     check(aixk_tri(m_ctx, 1, &ps, &pd, diagonal));
 }
 
@@ -726,7 +855,7 @@ void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorPar
 {
     requireDevice(dst, "indexSelect");
     flushFor(src.data, dst.data, indices.data);
-    aixhip_tensor ps, pd, pi; toPod(onDevice(src), &ps, "indexSelect"); toPod(dst, &pd, "indexSelect"); toPod(onDevice(indices), &pi, "indexSelect");
+    aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexSelect"); toPod(dst, &pd, "indexSelect"); stagedPod(indices, &pi, "indexSelect");
     check(aixk_index_select(m_ctx, &ps, &pd, &pi, dim));
 }
 
@@ -734,7 +863,7 @@ void DeviceHIP::indexAdd(const DeviceTensorParams& src, const DeviceTensorParams
 {
     requireDevice(dst, "indexAdd");
     flushFor(src.data, dst.data, indices.data);
-    aixhip_tensor ps, pd, pi; toPod(onDevice(src), &ps, "indexAdd"); toPod(dst, &pd, "indexAdd"); toPod(onDevice(indices), &pi, "indexAdd");
+    aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexAdd"); toPod(dst, &pd, "indexAdd"); stagedPod(indices, &pi, "indexAdd");
     check(aixk_index_add(m_ctx, &ps, &pd, &pi, dim));
 }
 

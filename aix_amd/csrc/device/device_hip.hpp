@@ -25,7 +25,6 @@
 #include "aix_compat.hpp"
 #include "fuse.hpp"
 
-#include <map>
 #include <memory>
 #include <string>
 #include <unordered_map>
@@ -108,17 +107,45 @@ public:
     size_t allocatedBytes() const { return m_liveBytes; }
 
 private:
-    struct Block { size_t bytes; };
+    struct Block {
+        size_t bytes;
+        bool touched{false};     // enqueued GPU work has referenced the block since it was allocated
+        bool freed{false};       // deallocate() has been called; the block waits in m_limbo
+    };
+    struct Extras;
+
+    // Live allocations by base address.  Operands normally carry a block's base pointer (views
+    // differ by offset), so the lookup is one probe of an open-addressing table; a pointer into the
+    // middle of a block, or a host pointer, falls back to a scan.
+    class BlockTable {
+    public:
+        Block* find(const void* base) const;
+        Block* findContaining(const void* p) const;
+        void insert(void* base, size_t bytes);
+        bool erase(void* base, size_t* bytes);
+        bool empty() const { return m_count == 0; }
+        template <class F> void forEach(F f) const { for (const auto& s : m_slots) if (s.key > 1) f((void*)s.key, s.block); }
+    private:
+        struct Slot { uintptr_t key{0}; mutable Block block{0}; };   // key 0 = never used, 1 = erased
+        size_t slotOf(uintptr_t key) const { return (size_t)(((key >> 6) * 0x9E3779B97F4A7C15ull) >> m_shift); }
+        void grow();
+        std::vector<Slot> m_slots;
+        size_t m_count{0}, m_used{0};
+        unsigned m_shift{64};
+    };
 
     const Block* findBlock(const void* p) const;
     size_t bucketBytes(size_t bytes) const;
     void* allocateBlock(size_t bytes, bool track);
     void releaseLimbo();
+    void markTouched(const void* p);
     void requireDevice(const DeviceTensorParams& result, const char* op) const;
-    // Returns params whose data is device memory: host operands are staged into a temporary block.
-    DeviceTensorParams onDevice(const DeviceTensorParams& p);
+    // Makes the view's data device memory: a host operand is staged into a temporary block.
+    void onDevice(aixhip::fuse::View& v);
     const void* stageRaw(const void* src, size_t bytes);
     void toPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op) const;
+    void toPod(const aixhip::fuse::View& v, aixhip_tensor* out) const;
+    void stagedPod(const DeviceTensorParams& p, aixhip_tensor* out, const char* op);      // toPod + staging of a host operand
     void check(int status) const;
     void recordBinary(aixhip::fuse::OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b,
                       const DeviceTensorParams& r, const char* op);
@@ -130,10 +157,11 @@ private:
 
     aixk_ctx* m_ctx{nullptr};
     std::unique_ptr<aixhip::fuse::FuseEngine> m_engine;
-    std::map<uintptr_t, Block> m_blocks;                       // live allocations by base address
+    std::unique_ptr<Extras> m_extras;                          // kernel cache, cooling blocks, scratch vectors
+    BlockTable m_blocks;
     std::unordered_map<size_t, std::vector<void*>> m_pool;     // free blocks by bucket size
     std::vector<std::pair<void*, size_t>> m_limbo;             // freed, but recorded work may still use them
-    size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0};
+    size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0}, m_totalBytes{0};
     int m_cus{256};
 };
 

@@ -58,54 +58,168 @@ const char* opName(OpType t)
     return names[static_cast<size_t>(t)];
 }
 
+size_t convertScalarInto(const void* scalar, DataType from, DataType to, uint8_t* out)
+{
+    const auto v = scalar::decode(scalar, static_cast<int>(from));
+    return scalar::encode(v, static_cast<int>(to), out);
+}
+
+size_t lowestScalarInto(DataType dtype, uint8_t* out)
+{
+    auto put = [&](auto v) { std::memcpy(out, &v, sizeof(v)); return sizeof(v); };
+    switch (dtype) {
+        case DataType::kFloat64:  return put(std::numeric_limits<double>::lowest());
+        case DataType::kFloat32:  return put(std::numeric_limits<float>::lowest());
+        case DataType::kFloat16:  return put((uint16_t)0xFBFF);          // aixFloat16.hpp:173-178
+        case DataType::kBFloat16: return put((uint16_t)0xFF7F);          // aixFloat16.hpp:767-772
+        case DataType::kInt64:    return put(std::numeric_limits<int64_t>::lowest());
+        case DataType::kInt32:    return put(std::numeric_limits<int32_t>::lowest());
+        case DataType::kInt16:    return put(std::numeric_limits<int16_t>::lowest());
+        case DataType::kInt8:     return put(std::numeric_limits<int8_t>::lowest());
+        case DataType::kUInt8:    return put((uint8_t)0);
+    }
+    return 0;
+}
+
 std::vector<uint8_t> convertScalar(const void* scalar, DataType from, DataType to)
 {
-    std::vector<uint8_t> out(8, 0);
-    const auto v = scalar::decode(scalar, static_cast<int>(from));
-    out.resize(scalar::encode(v, static_cast<int>(to), out.data()));
-    return out;
+    uint8_t bytes[8] = {};
+    const size_t n = convertScalarInto(scalar, from, to, bytes);
+    return std::vector<uint8_t>(bytes, bytes + n);
 }
 
 std::vector<uint8_t> lowestScalar(DataType dtype)
 {
-    std::vector<uint8_t> out(8, 0);
-    auto put = [&](auto v) { std::memcpy(out.data(), &v, sizeof(v)); out.resize(sizeof(v)); };
-    switch (dtype) {
-        case DataType::kFloat64:  put(std::numeric_limits<double>::lowest()); break;
-        case DataType::kFloat32:  put(std::numeric_limits<float>::lowest()); break;
-        case DataType::kFloat16:  put((uint16_t)0xFBFF); break;          // aixFloat16.hpp:173-178
-        case DataType::kBFloat16: put((uint16_t)0xFF7F); break;          // aixFloat16.hpp:767-772
-        case DataType::kInt64:    put(std::numeric_limits<int64_t>::lowest()); break;
-        case DataType::kInt32:    put(std::numeric_limits<int32_t>::lowest()); break;
-        case DataType::kInt16:    put(std::numeric_limits<int16_t>::lowest()); break;
-        case DataType::kInt8:     put(std::numeric_limits<int8_t>::lowest()); break;
-        case DataType::kUInt8:    put((uint8_t)0); break;
-    }
-    return out;
+    uint8_t bytes[8] = {};
+    const size_t n = lowestScalarInto(dtype, bytes);
+    return std::vector<uint8_t>(bytes, bytes + n);
 }
 
+// ---- View --------------------------------------------------------------------------------------
 namespace {
 
-bool sameView(const DeviceTensorParams& a, const DeviceTensorParams& b)
-{
-    return a.data == b.data && a.dtype == b.dtype && a.offset == b.offset && a.shape == b.shape && a.strides == b.strides;
-}
-
-bool isDense(const DeviceTensorParams& p)
+bool denseLayout(const size_t* shape, const size_t* strides, size_t rank)
 {
     size_t run = 1;
-    for (size_t d = p.shape.size(); d-- > 0;) {
-        if (p.shape[d] != 1 && p.strides[d] != run) return false;
-        run *= p.shape[d];
+    for (size_t d = rank; d-- > 0;) {
+        if (shape[d] != 1 && strides[d] != run) return false;
+        run *= shape[d];
     }
     return true;
 }
 
+} // namespace
+
+View::View(const DeviceTensorParams& p)
+    : data(p.data), dtype(p.dtype), rank((uint32_t)p.shape.size()), offset(p.offset), size(p.size)
+{
+    if (p.shape.size() > kMaxRank) throw std::invalid_argument("aixhip: tensors of more than 16 dimensions are not supported.");
+    for (size_t d = 0; d < rank; ++d) { shape[d] = p.shape[d]; strides[d] = d < p.strides.size() ? p.strides[d] : 0; }
+    dense = denseLayout(shape, strides, rank);
+}
+
+bool View::sameShape(const aix::Shape& s) const
+{
+    if (s.size() != rank) return false;
+    for (size_t d = 0; d < rank; ++d) if (s[d] != shape[d]) return false;
+    return true;
+}
+
+void View::makeDense()
+{
+    offset = 0;
+    size_t run = 1;
+    for (size_t d = rank; d-- > 0;) { strides[d] = run; run *= shape[d]; }
+    dense = true;
+}
+
+DeviceTensorParams View::params() const
+{
+    DeviceTensorParams p;
+    p.data = data; p.dtype = dtype; p.isContiguous = dense; p.offset = offset; p.size = size;
+    p.shape.assign(shape, shape + rank);
+    p.strides.assign(strides, strides + rank);
+    return p;
+}
+
+// ---- PointerSet --------------------------------------------------------------------------------
+bool PointerSet::contains(const void* p) const
+{
+    if (m_slots.empty()) return false;
+    const uintptr_t key = (uintptr_t)p;
+    const size_t mask = m_slots.size() - 1;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i] == key) return true;
+        if (m_slots[i] == 0) return false;
+    }
+}
+
+void PointerSet::grow()
+{
+    std::vector<uintptr_t> old;
+    old.swap(m_slots);
+    size_t capacity = 64;
+    while (capacity < m_count * 4) capacity <<= 1;
+    m_slots.assign(capacity, 0);
+    m_shift = 64;
+    for (size_t c = capacity; c > 1; c >>= 1) --m_shift;
+    m_used = m_count;
+    const size_t mask = capacity - 1;
+    for (uintptr_t key : old) {
+        if (key <= 1) continue;
+        size_t i = slotOf(key);
+        while (m_slots[i] != 0) i = (i + 1) & mask;
+        m_slots[i] = key;
+    }
+}
+
+void PointerSet::insert(const void* p)
+{
+    const uintptr_t key = (uintptr_t)p;
+    if (key <= 1) return;
+    if ((m_used + 1) * 2 > m_slots.size()) grow();
+    const size_t mask = m_slots.size() - 1;
+    size_t grave = SIZE_MAX;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i] == key) return;
+        if (m_slots[i] == 1 && grave == SIZE_MAX) grave = i;
+        if (m_slots[i] == 0) {
+            if (grave != SIZE_MAX) m_slots[grave] = key;
+            else { m_slots[i] = key; ++m_used; }
+            ++m_count;
+            return;
+        }
+    }
+}
+
+void PointerSet::erase(const void* p)
+{
+    if (m_slots.empty()) return;
+    const uintptr_t key = (uintptr_t)p;
+    if (key <= 1) return;
+    const size_t mask = m_slots.size() - 1;
+    for (size_t i = slotOf(key);; i = (i + 1) & mask) {
+        if (m_slots[i] == key) { m_slots[i] = 1; --m_count; return; }
+        if (m_slots[i] == 0) return;
+    }
+}
+
+namespace {
+
+bool sameView(const View& a, const View& b)
+{
+    return a.data == b.data && a.dtype == b.dtype && a.offset == b.offset && a.rank == b.rank &&
+           std::memcmp(a.shape, b.shape, a.rank * sizeof(size_t)) == 0 &&
+           std::memcmp(a.strides, b.strides, a.rank * sizeof(size_t)) == 0;
+}
+
+bool isDense(const View& p) { return p.dense; }
+
 // One past the last element position the view touches.
-size_t viewEnd(const DeviceTensorParams& p)
+size_t viewEnd(const View& p)
 {
     size_t last = p.offset;
-    for (size_t d = 0; d < p.shape.size(); ++d) {
+    for (size_t d = 0; d < p.rank; ++d) {
         if (p.shape[d] == 0) return p.offset;
         last += (p.shape[d] - 1) * p.strides[d];
     }
@@ -117,17 +231,30 @@ struct Operand {
     size_t index{SIZE_MAX};          // kValue: defining op (window index); kScalar: fill op (window index)
 };
 
+// A view inside the window: operand `slot` (0, 1 = inputs, 2 = output) of operator `op`.
+struct ViewRef {
+    uint32_t op;
+    uint32_t slot;
+};
+
 struct Group {
     DataType dtype{DataType::kFloat32};
     size_t count{0};
-    aix::Shape shape;
+    const View* shape{nullptr};                                // the view whose shape is the iteration space
     bool dense{true};                                          // every loaded view so far is dense
     std::vector<size_t> ops;                                   // window indices, program order
-    std::vector<std::pair<DeviceTensorParams, size_t>> defs;   // view -> latest defining op
-    std::vector<DeviceTensorParams> loads;                     // distinct views loaded from memory
+    std::vector<size_t> defs;                                  // per defined view: the latest operator defining it
+    std::vector<ViewRef> loads;                                // distinct views loaded from memory
     bool open{true};
     bool absorbed{false};                                      // merged into another group
     bool hasScalar{false};
+
+    void reset()
+    {
+        dtype = DataType::kFloat32; count = 0; shape = nullptr; dense = true;
+        ops.clear(); defs.clear(); loads.clear();
+        open = true; absorbed = false; hasScalar = false;
+    }
 };
 
 struct Emit {
@@ -136,57 +263,74 @@ struct Emit {
 };
 
 struct PendingFill {
+    const void* buffer;
     size_t op;                       // window index
     size_t size;                     // elements filled from the base pointer
 };
+
+} // namespace
 
 class Planner {
 public:
     // A buffer outlives the window if somebody still holds it or if it is about to be read outside the planner.
     struct Liveness {
-        const std::unordered_set<const void*>& held;
-        const std::unordered_set<const void*>& external;
-        size_t count(const void* p) const { return held.count(p) || external.count(p) ? 1 : 0; }
+        const PointerSet* held{nullptr};
+        const std::vector<const void*>* external{nullptr};
+        bool count(const void* p) const
+        {
+            if (held->contains(p)) return true;
+            for (const void* e : *external) if (e == p) return true;
+            return false;
+        }
     };
 
-    Planner(const std::vector<OpRecord>& ops, const FuseConfig& cfg, Liveness live)
-        : m_ops(ops), m_cfg(cfg), m_live(live), m_operands(ops.size()), m_groupOf(ops.size(), SIZE_MAX) {}
+    explicit Planner(const FuseConfig& cfg) : m_cfg(cfg) {}
 
-    void run()
+    void run(const std::vector<OpRecord>& ops, Liveness live)
     {
-        for (size_t i = 0; i < m_ops.size(); ++i) {
-            const auto& op = m_ops[i];
+        m_ops = &ops;
+        m_live = live;
+        m_operands.assign(ops.size(), {});
+        m_groupOf.assign(ops.size(), SIZE_MAX);
+        m_groupCount = 0;
+        m_emits.clear();
+        m_fills.clear();
+        m_fillsAbsorbed = 0;
+
+        for (size_t i = 0; i < ops.size(); ++i) {
+            const auto& op = ops[i];
             if (op.type == OpType::Fill || op.type == OpType::FillMin) placeFill(i);
             else if (isElementwiseOp(op.type) && op.type != OpType::Cast && m_cfg.elementwiseFusion) placeOp(i);
             else placeSingle(i);
         }
-        for (size_t g = 0; g < m_groups.size(); ++g) closeGroup(g);
+        for (size_t g = 0; g < m_groupCount; ++g) closeGroup(g);
         // fills nobody could absorb completely: run them if the buffer outlives the window
-        std::vector<size_t> rest;
-        for (auto& [buf, pf] : m_fills) if (m_live.count(buf)) rest.push_back(pf.op);
-        std::sort(rest.begin(), rest.end());
-        for (size_t op : rest) m_emits.push_back({false, op});
+        m_rest.clear();
+        for (const auto& pf : m_fills) if (m_live.count(pf.buffer)) m_rest.push_back(pf.op);
+        std::sort(m_rest.begin(), m_rest.end());
+        for (size_t op : m_rest) m_emits.push_back({false, op});
         m_fills.clear();
         decideStores();
     }
 
     const std::vector<Emit>& emits() const { return m_emits; }
-    const std::vector<Group>& groups() const { return m_groups; }
+    const Group& group(size_t g) const { return m_groups[g]; }
     size_t fillsAbsorbed() const { return m_fillsAbsorbed; }
 
     // A group of one operator without immediates runs as a plain single operator.
     bool emitsAsSingle(const Group& g) const { return g.ops.size() == 1 && !g.hasScalar; }
 
-    FusedSubgraphDescriptor describe(const Group& g) const
+    void describe(const Group& g, FusedSubgraphDescriptor& d)
     {
-        FusedSubgraphDescriptor d;
+        const auto& ops = *m_ops;
+        d.ops.clear(); d.inputBuffers.clear(); d.outputBuffers.clear(); d.scalarData.clear();
         d.dtype = g.dtype;
         d.elementCount = g.count;
-        d.shape = g.shape;
+        d.shape.assign(g.shape->shape, g.shape->shape + g.shape->rank);
         d.allContiguous = true;
-        std::unordered_map<size_t, size_t> position;          // window index -> position in d.ops
-        std::unordered_map<size_t, size_t> scalarSlot;        // fill op -> scalar index
-        auto inputSlot = [&](const DeviceTensorParams& v) {
+        m_position.resize(ops.size());                        // window index -> position in d.ops (this group's ops only)
+        m_scalarSlots.clear();                                // fill op -> scalar index
+        auto inputSlot = [&](const View& v) {
             for (size_t k = 0; k < d.inputBuffers.size(); ++k) if (sameView(d.inputBuffers[k], v)) return k;
             d.inputBuffers.push_back(v);
             if (!isDense(v)) d.allContiguous = false;
@@ -194,34 +338,38 @@ public:
         };
         // external inputs first, so that value indices (inputs.size() + position) are stable
         for (size_t w : g.ops) {
-            const auto& op = m_ops[w];
+            const auto& op = ops[w];
             if (m_operands[w][0].kind == Operand::kMemory) inputSlot(op.input0);
             if (m_operands[w][1].kind == Operand::kMemory) inputSlot(op.input1);
         }
         const size_t nIn = d.inputBuffers.size();
         const size_t esz = aix::Device::dataTypeSize(g.dtype);
         auto scalarIndex = [&](size_t fillOp) {
-            auto it = scalarSlot.find(fillOp);
-            if (it != scalarSlot.end()) return it->second;
-            const auto& f = m_ops[fillOp];
-            auto bytes = f.type == OpType::FillMin ? lowestScalar(g.dtype)
-                                                   : convertScalar(f.scalarData.data(), f.scalarDType, g.dtype);
+            for (const auto& known : m_scalarSlots) if (known.first == fillOp) return known.second;
+            const auto& f = ops[fillOp];
+            uint8_t bytes[8] = {};
+            const size_t n = f.type == OpType::FillMin ? lowestScalarInto(g.dtype, bytes)
+                                                       : convertScalarInto(f.scalarData.data(), f.scalarDType, g.dtype, bytes);
             const size_t slot = d.scalarData.size() / esz;
-            d.scalarData.insert(d.scalarData.end(), bytes.begin(), bytes.end());
-            scalarSlot[fillOp] = slot;
+            d.scalarData.insert(d.scalarData.end(), bytes, bytes + n);
+            m_scalarSlots.emplace_back(fillOp, slot);
             return slot;
         };
         for (size_t w : g.ops) {
-            const auto& op = m_ops[w];
+            const auto& op = ops[w];
             FusedSubgraphDescriptor::Op o;
             o.type = op.type;
-            const DeviceTensorParams* in[2] = {&op.input0, &op.input1};
+            const View* in[2] = {&op.input0, &op.input1};
             size_t* idx[2] = {&o.inputIndex0, &o.inputIndex1};
             size_t* sc[2] = {&o.scalarIndex0, &o.scalarIndex1};
             for (int k = 0; k < 2; ++k) {
                 const auto& operand = m_operands[w][k];
                 if (operand.kind == Operand::kMemory) *idx[k] = inputSlot(*in[k]);
-                else if (operand.kind == Operand::kValue) *idx[k] = nIn + position.at(operand.index);
+                else if (operand.kind == Operand::kValue) {
+                    if (m_groupOf[operand.index] != m_groupOf[w] || operand.index >= w)
+                        throw std::logic_error("fusion planner: a register operand is not defined earlier in the same kernel");
+                    *idx[k] = nIn + m_position[operand.index];
+                }
                 else if (operand.kind == Operand::kScalar) *sc[k] = scalarIndex(operand.index);
             }
             if (m_store[w]) {
@@ -229,45 +377,71 @@ public:
                 d.outputBuffers.push_back(op.output);
                 if (!isDense(op.output)) d.allContiguous = false;
             }
-            position[w] = d.ops.size();
+            m_position[w] = d.ops.size();
             d.ops.push_back(o);
         }
-        return d;
     }
 
 private:
+    const OpRecord& at(size_t i) const { return (*m_ops)[i]; }
+    const View& view(ViewRef r) const
+    {
+        const auto& op = at(r.op);
+        return r.slot == 0 ? op.input0 : r.slot == 1 ? op.input1 : op.output;
+    }
+    const View& defView(size_t definingOp) const { return at(definingOp).output; }
+
+    PendingFill* findFill(const void* buffer)
+    {
+        for (auto& pf : m_fills) if (pf.buffer == buffer) return &pf;
+        return nullptr;
+    }
+    void eraseFill(const void* buffer)
+    {
+        for (size_t k = 0; k < m_fills.size(); ++k)
+            if (m_fills[k].buffer == buffer) { m_fills[k] = m_fills.back(); m_fills.pop_back(); return; }
+    }
+
+    size_t newGroup()
+    {
+        if (m_groupCount == m_groups.size()) m_groups.emplace_back();
+        m_groups[m_groupCount].reset();
+        return m_groupCount++;
+    }
+
     // ---- fills --------------------------------------------------------------------------------
     void placeFill(size_t i)
     {
-        const auto& out = m_ops[i].output;
+        const auto& out = at(i).output;
         if (!m_cfg.absorbFills || !m_cfg.elementwiseFusion) { placeSingle(i); return; }
         // groups that see the buffer's previous content must run before anything overwrites it
         closeGroupsTouching(out.data, SIZE_MAX, nullptr);
-        auto it = m_fills.find(out.data);
-        if (it != m_fills.end() && it->second.size > out.size) materialise(out.data);   // older, larger fill survives underneath
-        m_fills[out.data] = PendingFill{i, out.size};                                   // written flat from the base pointer
+        PendingFill* known = findFill(out.data);
+        if (known && known->size > out.size) { materialise(out.data); known = nullptr; }   // older, larger fill survives underneath
+        if (known) { known->op = i; known->size = out.size; }
+        else m_fills.push_back(PendingFill{out.data, i, out.size});                        // written flat from the base pointer
     }
 
     void materialise(const void* buffer)
     {
-        auto it = m_fills.find(buffer);
-        if (it == m_fills.end()) return;
-        m_emits.push_back({false, it->second.op});
-        m_fills.erase(it);
+        const PendingFill* pf = findFill(buffer);
+        if (!pf) return;
+        m_emits.push_back({false, pf->op});
+        eraseFill(buffer);
     }
 
     // ---- operators that cannot be fused ----------------------------------------------------------
     void placeSingle(size_t i)
     {
-        const auto& op = m_ops[i];
-        for (const DeviceTensorParams* in : {&op.input0, &op.input1}) {
+        const auto& op = at(i);
+        for (const View* in : {&op.input0, &op.input1}) {
             if (!in->data) continue;
             materialise(in->data);
             closeWriters(in->data);
         }
         if (op.output.data) {
             closeGroupsTouching(op.output.data, SIZE_MAX, nullptr);
-            if (op.type == OpType::Fill || op.type == OpType::FillMin) m_fills.erase(op.output.data);
+            if (op.type == OpType::Fill || op.type == OpType::FillMin) eraseFill(op.output.data);
             else materialise(op.output.data);
         }
         if (op.input0.data) m_operands[i][0].kind = Operand::kMemory;
@@ -278,9 +452,9 @@ private:
     // ---- fusable operators ---------------------------------------------------------------------
     void placeOp(size_t i)
     {
-        const auto& op = m_ops[i];
+        const auto& op = at(i);
         const bool binary = op.hasInput1;
-        const DeviceTensorParams* in[2] = {&op.input0, binary ? &op.input1 : nullptr};
+        const View* in[2] = {&op.input0, binary ? &op.input1 : nullptr};
 
         if (!m_cfg.supportsStridedFusion) {
             const bool dense = isDense(op.output) && (!in[0]->data || isDense(*in[0])) && (!in[1] || !in[1]->data || isDense(*in[1]));
@@ -298,27 +472,26 @@ private:
                 resolved[k] = Operand{};
                 if (!in[k] || !in[k]->data) continue;
                 // an unmaterialised fill covering everything the view can touch -> immediate
-                auto f = m_fills.find(in[k]->data);
-                if (f != m_fills.end()) {
-                    if (in[k]->dtype == m_ops[f->second.op].output.dtype && viewEnd(*in[k]) <= f->second.size) {
-                        resolved[k] = Operand{Operand::kScalar, f->second.op};
+                if (const PendingFill* f = findFill(in[k]->data)) {
+                    if (in[k]->dtype == at(f->op).output.dtype && viewEnd(*in[k]) <= f->size) {
+                        resolved[k] = Operand{Operand::kScalar, f->op};
                         continue;
                     }
                     materialise(in[k]->data);
                 }
                 resolved[k].kind = Operand::kMemory;
-                for (size_t g = 0; g < m_groups.size(); ++g) {
+                for (size_t g = 0; g < m_groupCount; ++g) {
                     if (!m_groups[g].open) continue;
-                    const auto* def = findDef(m_groups[g], in[k]->data);
-                    if (!def) continue;
-                    const bool usable = sameView(def->first, *in[k]) && compatible(m_groups[g], op);
+                    const size_t def = findDef(m_groups[g], in[k]->data);
+                    if (def == SIZE_MAX) continue;
+                    const bool usable = sameView(defView(def), *in[k]) && compatible(m_groups[g], op);
                     if (usable && (target == SIZE_MAX || target == g)) {
-                        resolved[k] = Operand{Operand::kValue, def->second};
+                        resolved[k] = Operand{Operand::kValue, def};
                         target = g;
                     } else if (usable && mergeable(m_groups[target], m_groups[g])) {
                         // both operands come from open groups: open groups are independent of each
                         // other, so the two become one kernel
-                        resolved[k] = Operand{Operand::kValue, def->second};
+                        resolved[k] = Operand{Operand::kValue, def};
                         mergeInto(target, g);
                     } else {
                         closeGroup(g);
@@ -330,12 +503,10 @@ private:
 
             // no producer inside the window: share loads with an open group of the same shape
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t g = 0; g < m_groups.size() && target == SIZE_MAX; ++g) {
+                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
                     if (!m_groups[g].open || !compatible(m_groups[g], op)) continue;
                     for (int k = 0; k < 2; ++k)
-                        if (resolved[k].kind == Operand::kMemory)
-                            for (const auto& v : m_groups[g].loads)
-                                if (sameView(v, *in[k])) target = g;
+                        if (resolved[k].kind == Operand::kMemory && loads(m_groups[g], *in[k])) target = g;
                 }
             }
 
@@ -349,27 +520,23 @@ private:
         }
 
         // a fill that this operator overwrites completely never has to run
-        auto f = m_fills.find(op.output.data);
-        if (f != m_fills.end()) {
-            if (isDense(op.output) && op.output.offset == 0 && op.output.size >= f->second.size) m_fills.erase(f);
+        if (const PendingFill* f = findFill(op.output.data)) {
+            if (isDense(op.output) && op.output.offset == 0 && op.output.size >= f->size) eraseFill(op.output.data);
             else materialise(op.output.data);
         }
 
         if (target == SIZE_MAX) {
-            Group g;
-            g.dtype = op.output.dtype;
-            g.count = op.output.size;
-            g.shape = op.output.shape;
-            m_groups.push_back(std::move(g));
-            target = m_groups.size() - 1;
+            target = newGroup();
+            Group& fresh = m_groups[target];
+            fresh.dtype = op.output.dtype;
+            fresh.count = op.output.size;
+            fresh.shape = &op.output;
         }
         Group& g = m_groups[target];
         for (int k = 0; k < 2; ++k) {
             m_operands[i][k] = resolved[k];
             if (resolved[k].kind == Operand::kMemory) {
-                bool known = false;
-                for (const auto& v : g.loads) if (sameView(v, *in[k])) known = true;
-                if (!known) g.loads.push_back(*in[k]);
+                if (!loads(g, *in[k])) g.loads.push_back(ViewRef{(uint32_t)i, (uint32_t)k});
                 if (!isDense(*in[k])) g.dense = false;
             } else if (resolved[k].kind == Operand::kScalar) {
                 g.hasScalar = true;
@@ -377,16 +544,23 @@ private:
             }
         }
         bool redefined = false;
-        for (auto& def : g.defs) if (sameView(def.first, op.output)) { def.second = i; redefined = true; }
-        if (!redefined) g.defs.emplace_back(op.output, i);
+        for (auto& def : g.defs) if (sameView(defView(def), op.output)) { def = i; redefined = true; }
+        if (!redefined) g.defs.push_back(i);
         g.ops.push_back(i);
         m_groupOf[i] = target;
     }
 
-    static const std::pair<DeviceTensorParams, size_t>* findDef(const Group& g, const void* buffer)
+    // The latest operator of the group that defines a view of `buffer`, SIZE_MAX if none does.
+    size_t findDef(const Group& g, const void* buffer) const
     {
-        for (const auto& def : g.defs) if (def.first.data == buffer) return &def;
-        return nullptr;
+        for (size_t def : g.defs) if (defView(def).data == buffer) return def;
+        return SIZE_MAX;
+    }
+
+    bool loads(const Group& g, const View& v) const
+    {
+        for (const ViewRef& r : g.loads) if (sameView(view(r), v)) return true;
+        return false;
     }
 
     // Same element type and iteration space: identical shape, or equal element counts when both
@@ -394,7 +568,7 @@ private:
     bool compatible(const Group& g, const OpRecord& op) const
     {
         if (g.dtype != op.output.dtype || g.count != op.output.size) return false;
-        if (g.shape == op.output.shape) return true;
+        if (g.shape->sameShape(op.output)) return true;
         const bool opDense = isDense(op.output) && (!op.input0.data || isDense(op.input0)) &&
                              (!op.hasInput1 || !op.input1.data || isDense(op.input1));
         return g.dense && opDense;
@@ -403,14 +577,10 @@ private:
     bool mergeable(const Group& a, const Group& b) const
     {
         if (a.dtype != b.dtype || a.count != b.count) return false;
-        if (!(a.shape == b.shape) && !(a.dense && b.dense)) return false;
-        size_t loads = a.loads.size();
-        for (const auto& v : b.loads) {
-            bool known = false;
-            for (const auto& w : a.loads) if (sameView(v, w)) known = true;
-            if (!known) ++loads;
-        }
-        return loads + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;
+        if (!a.shape->sameShape(*b.shape) && !(a.dense && b.dense)) return false;
+        size_t count = a.loads.size();
+        for (const ViewRef& r : b.loads) if (!loads(a, view(r))) ++count;
+        return count + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;
     }
 
     // Folds open group `from` into open group `into` (no hazards can exist between open groups).
@@ -418,15 +588,11 @@ private:
     {
         Group& a = m_groups[into];
         Group& b = m_groups[from];
-        std::vector<size_t> ops(a.ops.size() + b.ops.size());
-        std::merge(a.ops.begin(), a.ops.end(), b.ops.begin(), b.ops.end(), ops.begin());     // program order
-        a.ops.swap(ops);
-        for (auto& d : b.defs) a.defs.push_back(d);
-        for (const auto& v : b.loads) {
-            bool known = false;
-            for (const auto& w : a.loads) if (sameView(v, w)) known = true;
-            if (!known) a.loads.push_back(v);
-        }
+        m_merged.resize(a.ops.size() + b.ops.size());
+        std::merge(a.ops.begin(), a.ops.end(), b.ops.begin(), b.ops.end(), m_merged.begin());     // program order
+        a.ops.assign(m_merged.begin(), m_merged.end());
+        for (size_t def : b.defs) a.defs.push_back(def);
+        for (const ViewRef& r : b.loads) if (!loads(a, view(r))) a.loads.push_back(r);
         a.dense = a.dense && b.dense;
         a.hasScalar = a.hasScalar || b.hasScalar;
         for (size_t w : b.ops) m_groupOf[w] = into;
@@ -438,12 +604,10 @@ private:
     size_t slotsAfterJoin(const Group& g, const OpRecord& op, const Operand* resolved) const
     {
         size_t slots = g.loads.size() + g.defs.size() + 1;     // every def may have to be stored
-        const DeviceTensorParams* in[2] = {&op.input0, &op.input1};
+        const View* in[2] = {&op.input0, &op.input1};
         for (int k = 0; k < 2; ++k) {
             if (resolved[k].kind != Operand::kMemory) continue;
-            bool known = false;
-            for (const auto& v : g.loads) if (sameView(v, *in[k])) known = true;
-            if (!known) ++slots;
+            if (!loads(g, *in[k])) ++slots;
         }
         return slots;
     }
@@ -451,16 +615,22 @@ private:
     // Closes every open group that loads or defines `buffer`, except that the group `keep` may go
     // on if it only ever sees the buffer through exactly the view `same` (in-place elementwise
     // update).  Returns true if it closed anything.
-    bool closeGroupsTouching(const void* buffer, size_t keep, const DeviceTensorParams* same)
+    bool closeGroupsTouching(const void* buffer, size_t keep, const View* same)
     {
         bool closed = false;
         if (!buffer) return false;
-        for (size_t g = 0; g < m_groups.size(); ++g) {
+        for (size_t g = 0; g < m_groupCount; ++g) {
             Group& grp = m_groups[g];
             if (!grp.open) continue;
             bool touches = false, conflicting = false;
-            for (const auto& v : grp.loads) if (v.data == buffer) { touches = true; if (!same || !sameView(v, *same)) conflicting = true; }
-            for (const auto& d : grp.defs) if (d.first.data == buffer) { touches = true; if (!same || !sameView(d.first, *same)) conflicting = true; }
+            for (const ViewRef& r : grp.loads) {
+                const View& v = view(r);
+                if (v.data == buffer) { touches = true; if (!same || !sameView(v, *same)) conflicting = true; }
+            }
+            for (size_t def : grp.defs) {
+                const View& v = defView(def);
+                if (v.data == buffer) { touches = true; if (!same || !sameView(v, *same)) conflicting = true; }
+            }
             if (!touches) continue;
             if (g == keep && !conflicting) continue;
             closeGroup(g);
@@ -471,8 +641,8 @@ private:
 
     void closeWriters(const void* buffer)
     {
-        for (size_t g = 0; g < m_groups.size(); ++g)
-            if (m_groups[g].open && findDef(m_groups[g], buffer)) closeGroup(g);
+        for (size_t g = 0; g < m_groupCount; ++g)
+            if (m_groups[g].open && findDef(m_groups[g], buffer) != SIZE_MAX) closeGroup(g);
     }
 
     void closeGroup(size_t g)
@@ -487,20 +657,21 @@ private:
     // view is stored.
     void decideStores()
     {
-        m_store.assign(m_ops.size(), false);
-        for (size_t g = 0; g < m_groups.size(); ++g)
-            for (const auto& def : m_groups[g].defs)
-                if (m_live.count(def.first.data)) m_store[def.second] = true;
-        for (size_t j = 0; j < m_ops.size(); ++j) {
-            const DeviceTensorParams* in[2] = {&m_ops[j].input0, &m_ops[j].input1};
+        const size_t n = m_ops->size();
+        m_store.assign(n, 0);
+        for (size_t g = 0; g < m_groupCount; ++g)
+            for (size_t def : m_groups[g].defs)
+                if (m_live.count(defView(def).data)) m_store[def] = 1;
+        for (size_t j = 0; j < n; ++j) {
+            const View* in[2] = {&at(j).input0, &at(j).input1};
             for (int k = 0; k < 2; ++k) {
                 if (m_operands[j][k].kind != Operand::kMemory || !in[k]->data) continue;
                 for (size_t w = j; w-- > 0;) {
-                    if (m_ops[w].output.data != in[k]->data) continue;
+                    if (at(w).output.data != in[k]->data) continue;
                     if (m_groupOf[w] != SIZE_MAX) {
                         // the value that must be in memory is the group's last definition of that view
-                        for (const auto& def : m_groups[m_groupOf[w]].defs)
-                            if (sameView(def.first, m_ops[w].output)) m_store[def.second] = true;
+                        for (size_t def : m_groups[m_groupOf[w]].defs)
+                            if (sameView(defView(def), at(w).output)) m_store[def] = 1;
                     }
                     break;
                 }
@@ -508,19 +679,20 @@ private:
         }
     }
 
-    const std::vector<OpRecord>& m_ops;
     const FuseConfig& m_cfg;
-    const Liveness m_live;
+    const std::vector<OpRecord>* m_ops{nullptr};
+    Liveness m_live;
     std::vector<std::array<Operand, 2>> m_operands;
     std::vector<size_t> m_groupOf;
-    std::vector<Group> m_groups;
+    std::vector<Group> m_groups;             // [0, m_groupCount) belong to the current window
+    size_t m_groupCount{0};
     std::vector<Emit> m_emits;
-    std::unordered_map<const void*, PendingFill> m_fills;
-    std::vector<bool> m_store;
+    std::vector<PendingFill> m_fills;
+    std::vector<uint8_t> m_store;
+    std::vector<size_t> m_rest, m_merged, m_position;
+    std::vector<std::pair<size_t, size_t>> m_scalarSlots;
     size_t m_fillsAbsorbed{0};
 };
-
-} // namespace
 
 // ---- FuseEngine --------------------------------------------------------------------------------
 FuseEngine::FuseEngine(const FuseConfig& config, FuseCallbacks callbacks) : m_config(config), m_callbacks(std::move(callbacks))
@@ -529,44 +701,50 @@ FuseEngine::FuseEngine(const FuseConfig& config, FuseCallbacks callbacks) : m_co
     if (!m_callbacks.emitFused || !m_callbacks.emitSingle || !m_callbacks.finishFlush)
         throw std::invalid_argument("FuseEngine requires emitFused, emitSingle and finishFlush callbacks.");
     if (!m_callbacks.getKernelCacheStats) m_callbacks.getKernelCacheStats = [] { return std::pair<size_t, size_t>{0, 0}; };
+    m_planner = std::make_unique<Planner>(m_config);
 }
+
+FuseEngine::~FuseEngine() = default;
 
 void FuseEngine::maybeFlush()
 {
     if (m_pending.size() >= m_config.flushThreshold) flush();
 }
 
-void FuseEngine::record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& output)
+OpRecord& FuseEngine::append(OpType type)
 {
-    OpRecord r;
-    r.type = type; r.input0 = input0; r.output = output;
-    m_pending.push_back(std::move(r));
+    m_pending.emplace_back();
+    OpRecord& r = m_pending.back();
+    r.type = type;
+    return r;
+}
+
+void FuseEngine::record(OpType type, const View& input0, const View& output)
+{
+    OpRecord& r = append(type);
+    r.input0 = input0; r.output = output;
     maybeFlush();
 }
 
-void FuseEngine::record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& input1, const DeviceTensorParams& output)
+void FuseEngine::record(OpType type, const View& input0, const View& input1, const View& output)
 {
-    OpRecord r;
-    r.type = type; r.input0 = input0; r.input1 = input1; r.output = output; r.hasInput1 = true;
-    m_pending.push_back(std::move(r));
+    OpRecord& r = append(type);
+    r.input0 = input0; r.input1 = input1; r.output = output; r.hasInput1 = true;
     maybeFlush();
 }
 
-void FuseEngine::recordFill(const void* scalar, DataType scalarDType, const DeviceTensorParams& output)
+void FuseEngine::recordFill(const void* scalar, DataType scalarDType, const View& output)
 {
-    OpRecord r;
-    r.type = OpType::Fill; r.output = output; r.scalarDType = scalarDType;
-    const size_t n = aix::Device::dataTypeSize(scalarDType);
-    r.scalarData.assign(static_cast<const uint8_t*>(scalar), static_cast<const uint8_t*>(scalar) + n);
-    m_pending.push_back(std::move(r));
+    OpRecord& r = append(OpType::Fill);
+    r.output = output; r.scalarDType = scalarDType;
+    std::memcpy(r.scalarData.data(), scalar, aix::Device::dataTypeSize(scalarDType));
     maybeFlush();
 }
 
-void FuseEngine::recordFillMin(const DeviceTensorParams& output)
+void FuseEngine::recordFillMin(const View& output)
 {
-    OpRecord r;
-    r.type = OpType::FillMin; r.output = output;
-    m_pending.push_back(std::move(r));
+    OpRecord& r = append(OpType::FillMin);
+    r.output = output;
     maybeFlush();
 }
 
@@ -589,29 +767,29 @@ void FuseEngine::flush()
 
     if (m_config.diagnostics) { m_diagnostics.emplace(); m_diagnostics->opsRecorded = m_pending.size(); }
 
-    std::vector<OpRecord> window;
-    window.swap(m_pending);
+    m_window.clear();
+    m_window.swap(m_pending);                // operators recorded by callbacks belong to the next window
+    const std::vector<OpRecord>& window = m_window;
     // buffers about to be read outside the planner count as alive for this window
-    const Planner::Liveness live{m_live, m_externalReads};
+    const Planner::Liveness live{&m_live, &m_externalReads};
 
-    size_t fusedKernels = 0, fusedOps = 0, singles = 0, absorbed = 0;
-    std::ostringstream groupsText;
-    if (!window.empty()) {
-        Planner plan(window, m_config, live);
-        plan.run();
-        for (const auto& e : plan.emits()) {
-            if (!e.fused) { m_callbacks.emitSingle(window[e.index]); ++singles; continue; }
-            const auto& g = plan.groups()[e.index];
-            if (plan.emitsAsSingle(g)) { m_callbacks.emitSingle(window[g.ops[0]]); ++singles; continue; }
-            auto desc = plan.describe(g);
-            if (desc.outputBuffers.empty()) continue;          // nothing of it is ever read: dead code
-            m_callbacks.emitFused(desc);
-            if (fusedKernels) groupsText << ", ";
-            groupsText << desc.ops.size() << " ops";
-            ++fusedKernels;
-            fusedOps += desc.ops.size();
+    size_t fusedKernels = 0, fusedOps = 0, singles = 0;
+    std::string groupsText;
+    Planner& plan = *m_planner;
+    plan.run(window, live);
+    for (const auto& e : plan.emits()) {
+        if (!e.fused) { m_callbacks.emitSingle(window[e.index]); ++singles; continue; }
+        const auto& g = plan.group(e.index);
+        if (plan.emitsAsSingle(g)) { m_callbacks.emitSingle(window[g.ops[0]]); ++singles; continue; }
+        plan.describe(g, m_descriptor);
+        if (m_descriptor.outputBuffers.empty()) continue;          // nothing of it is ever read: dead code
+        m_callbacks.emitFused(m_descriptor);
+        if (m_config.diagnostics) {
+            if (fusedKernels) groupsText += ", ";
+            groupsText += std::to_string(m_descriptor.ops.size()) + " ops";
         }
-        absorbed = plan.fillsAbsorbed();
+        ++fusedKernels;
+        fusedOps += m_descriptor.ops.size();
     }
     m_callbacks.finishFlush();
 
@@ -621,8 +799,8 @@ void FuseEngine::flush()
         d.fusedOps = fusedOps;
         d.fallbackOps = singles;
         d.dispatchesSaved = fusedOps - fusedKernels;
-        d.fillsAbsorbed = absorbed;
-        d.subgraphSummary = std::to_string(fusedKernels) + " subgraphs" + (fusedKernels ? " (" + groupsText.str() + ")" : "");
+        d.fillsAbsorbed = plan.fillsAbsorbed();
+        d.subgraphSummary = std::to_string(fusedKernels) + " subgraphs" + (fusedKernels ? " (" + groupsText + ")" : "");
         d.fallbackSummary = std::to_string(singles) + " individual ops";
         auto [hits, misses] = m_callbacks.getKernelCacheStats();
         d.kernelCacheHits = hits;
@@ -631,7 +809,7 @@ void FuseEngine::flush()
     m_externalReads.clear();
 }
 
-bool FuseEngine::takeTrailingFill(const DeviceTensorParams& output, OpRecord* fill)
+bool FuseEngine::takeTrailingFill(const View& output, OpRecord* fill)
 {
     if (m_flushing || !output.data) return false;
     for (size_t k = m_pending.size(); k-- > 0;) {
@@ -641,7 +819,7 @@ bool FuseEngine::takeTrailingFill(const DeviceTensorParams& output, OpRecord* fi
         if (reads) return false;
         if (op.output.data != output.data) continue;
         if ((op.type != OpType::Fill && op.type != OpType::FillMin) || op.output.dtype != output.dtype ||
-            op.output.offset != output.offset || op.output.size != output.size || !output.isContiguous || !op.output.isContiguous)
+            op.output.offset != output.offset || op.output.size != output.size || !output.dense || !op.output.dense)
             return false;
         *fill = op;
         m_pending.erase(m_pending.begin() + (long)k);
@@ -650,9 +828,23 @@ bool FuseEngine::takeTrailingFill(const DeviceTensorParams& output, OpRecord* fi
     return false;
 }
 
-void FuseEngine::recordExternalRead(const void* buffer) { if (buffer) m_externalReads.insert(buffer); }
+void FuseEngine::recordExternalRead(const void* buffer)
+{
+    if (!buffer) return;
+    for (const void* known : m_externalReads) if (known == buffer) return;
+    m_externalReads.push_back(buffer);
+}
+
 void FuseEngine::retainBuffer(void* buffer) { if (buffer) m_live.insert(buffer); }
-void FuseEngine::releaseBuffer(void* buffer) { if (buffer) { m_live.erase(buffer); m_externalReads.erase(buffer); } }
+
+void FuseEngine::releaseBuffer(void* buffer)
+{
+    if (!buffer) return;
+    m_live.erase(buffer);
+    for (size_t k = 0; k < m_externalReads.size(); ++k)
+        if (m_externalReads[k] == buffer) { m_externalReads[k] = m_externalReads.back(); m_externalReads.pop_back(); break; }
+}
+
 void FuseEngine::invalidateBuffer(void*) {}
 
 } // namespace aixhip::fuse

@@ -13,12 +13,13 @@
 
 #include "aix_compat.hpp"
 
+#include <array>
 #include <cstdint>
+#include <cstring>
 #include <functional>
+#include <memory>
 #include <optional>
 #include <string>
-#include <unordered_map>
-#include <unordered_set>
 #include <utility>
 #include <vector>
 
@@ -47,12 +48,47 @@ struct FuseConfig {
     bool   supportsStridedFusion = true;   // may fused kernels read broadcast / strided views
 };
 
+// An operand as the planner keeps it: the fields of aix::DeviceTensorParams with the extents and
+// strides held in place, so that recording an operator allocates nothing.  `dense` says that the
+// view walks its elements in memory order without gaps (extent-1 dimensions may carry any stride).
+constexpr size_t kMaxRank = 16;
+
+struct View {
+    void*    data{nullptr};
+    DataType dtype{DataType::kFloat32};
+    bool     dense{true};
+    uint32_t rank{0};
+    size_t   offset{0};
+    size_t   size{0};
+    size_t   shape[kMaxRank];              // [0, rank) are meaningful
+    size_t   strides[kMaxRank];
+
+    View() {}
+    View(const DeviceTensorParams& p);     // std::invalid_argument beyond kMaxRank dimensions
+    View(const View& o) { assign(o); }
+    View& operator=(const View& o) { if (this != &o) assign(o); return *this; }
+
+    bool sameShape(const View& o) const { return rank == o.rank && std::memcmp(shape, o.shape, rank * sizeof(size_t)) == 0; }
+    bool sameShape(const aix::Shape& s) const;
+    void makeDense();                      // offset 0 and the dense strides of `shape`
+    aix::Shape shapeVector() const { return aix::Shape(shape, shape + rank); }
+    DeviceTensorParams params() const;
+
+private:
+    void assign(const View& o)
+    {
+        data = o.data; dtype = o.dtype; dense = o.dense; rank = o.rank; offset = o.offset; size = o.size;
+        std::memcpy(shape, o.shape, rank * sizeof(size_t));
+        std::memcpy(strides, o.strides, rank * sizeof(size_t));
+    }
+};
+
 struct OpRecord {
     OpType type{OpType::Add};
-    DeviceTensorParams input0;
-    DeviceTensorParams input1;
-    DeviceTensorParams output;
-    std::vector<uint8_t> scalarData;       // Fill: the scalar in scalarDType
+    View input0;
+    View input1;
+    View output;
+    std::array<uint8_t, 8> scalarData{};   // Fill: the scalar in scalarDType
     DataType scalarDType = DataType::kFloat32;
     bool hasInput1 = false;
 };
@@ -71,14 +107,16 @@ struct FusedSubgraphDescriptor {
         size_t scalarIndex1 = SIZE_MAX;
     };
     std::vector<Op> ops;
-    std::vector<DeviceTensorParams> inputBuffers;
-    std::vector<DeviceTensorParams> outputBuffers;
+    std::vector<View> inputBuffers;
+    std::vector<View> outputBuffers;
     std::vector<uint8_t> scalarData;
     DataType dtype{DataType::kFloat32};
     bool     allContiguous{true};          // every loaded / stored view is dense
     size_t   elementCount{0};
     aix::Shape shape;                      // iteration shape (outputs are dense over it)
 };
+// The descriptor handed to emitFused is reused from kernel to kernel: a callback that wants to keep
+// it copies it.
 
 struct FlushDiagnostics {
     size_t opsRecorded = 0;
@@ -104,16 +142,38 @@ struct FuseCallbacks {
 // float -> integer, NaN -> 0, 16-bit floats by way of float; aixDeviceCPU.cpp:96-117).
 std::vector<uint8_t> convertScalar(const void* scalar, DataType from, DataType to);
 std::vector<uint8_t> lowestScalar(DataType dtype);
+// The same without the vector: writes at most 8 bytes to `out` and returns how many.
+size_t convertScalarInto(const void* scalar, DataType from, DataType to, uint8_t* out);
+size_t lowestScalarInto(DataType dtype, uint8_t* out);
+
+// A set of buffer addresses that neither allocates per insertion nor chases pointers on lookup
+// (open addressing; allocate() / deallocate() of every temporary pass through it).
+class PointerSet {
+public:
+    bool contains(const void* p) const;
+    void insert(const void* p);
+    void erase(const void* p);
+    size_t size() const { return m_count; }
+
+private:
+    size_t slotOf(uintptr_t key) const { return (size_t)(((key >> 6) * 0x9E3779B97F4A7C15ull) >> m_shift); }
+    void grow();
+    std::vector<uintptr_t> m_slots;        // 0 = never used, 1 = erased
+    size_t m_count{0}, m_used{0};
+    unsigned m_shift{64};
+};
+
+class Planner;
 
 class FuseEngine {
 public:
     FuseEngine(const FuseConfig& config, FuseCallbacks callbacks);
+    ~FuseEngine();
 
-    void record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& output);
-    void record(OpType type, const DeviceTensorParams& input0, const DeviceTensorParams& input1,
-                const DeviceTensorParams& output);
-    void recordFill(const void* scalar, DataType scalarDType, const DeviceTensorParams& output);
-    void recordFillMin(const DeviceTensorParams& output);
+    void record(OpType type, const View& input0, const View& output);
+    void record(OpType type, const View& input0, const View& input1, const View& output);
+    void recordFill(const void* scalar, DataType scalarDType, const View& output);
+    void recordFillMin(const View& output);
     void flush();
 
     const FuseConfig& config() const { return m_config; }
@@ -123,7 +183,7 @@ public:
     // If the newest pending operator touching output.data is a fill / fillMin of exactly this dense
     // tensor, remove it from the window and hand it over (the caller folds it into the operator
     // it is about to run eagerly); false and no change otherwise.
-    bool takeTrailingFill(const DeviceTensorParams& output, OpRecord* fill);
+    bool takeTrailingFill(const View& output, OpRecord* fill);
     void recordExternalRead(const void* buffer);   // the buffer is about to be read outside the planner
     void retainBuffer(void* buffer);               // allocate(): results written here must reach memory
     void releaseBuffer(void* buffer);              // deallocate(): nobody will read it after the window
@@ -134,9 +194,13 @@ private:
 
     FuseConfig m_config;
     FuseCallbacks m_callbacks;
-    std::vector<OpRecord> m_pending;
-    std::unordered_set<const void*> m_live;
-    std::unordered_set<const void*> m_externalReads;
+    OpRecord& append(OpType type);
+    std::vector<OpRecord> m_pending;       // capacity is kept from window to window
+    std::vector<OpRecord> m_window;
+    PointerSet m_live;
+    std::vector<const void*> m_externalReads;
+    std::unique_ptr<Planner> m_planner;    // its working storage is kept from window to window
+    FusedSubgraphDescriptor m_descriptor;
     std::optional<FlushDiagnostics> m_diagnostics;
     bool m_flushing{false};
 };

@@ -82,19 +82,52 @@ void emitBody(std::ostringstream& o, const FusedSubgraphDescriptor& d)
 
 } // namespace
 
+namespace {
+
+void appendNumber(std::string& out, uint64_t v, unsigned base = 10)
+{
+    char digits[24];
+    int n = 0;
+    do { const unsigned r = (unsigned)(v % base); digits[n++] = (char)(r < 10 ? '0' + r : 'a' + (r - 10)); v /= base; } while (v);
+    while (n) out.push_back(digits[--n]);
+}
+
+void appendOperand(std::string& out, const FusedSubgraphDescriptor& d, size_t tensorIndex, size_t scalarIndex)
+{
+    if (tensorIndex != SIZE_MAX) {
+        if (tensorIndex < d.inputBuffers.size()) { out += "x["; appendNumber(out, tensorIndex); out += ']'; }
+        else { out += 'v'; appendNumber(out, tensorIndex - d.inputBuffers.size()); }
+        return;
+    }
+    if (scalarIndex == SIZE_MAX) throw std::invalid_argument("fused operator without an operand");
+    out += "s["; appendNumber(out, scalarIndex); out += ']';
+}
+
+} // namespace
+
+void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
+{
+    s.clear();
+    s += shortType(d.dtype);
+    s += shape == Shape::Flat ? "|flat" : shape == Shape::Rows ? "|rows" : "|gather";
+    if (shape == Shape::Flat) { s += noAlias ? 'r' : 'a'; appendNumber(s, broadcastMask, 16); }
+    s += "|i"; appendNumber(s, d.inputBuffers.size());
+    s += 'o';  appendNumber(s, d.outputBuffers.size());
+    s += 's';  appendNumber(s, scalarCount(d));
+    for (const auto& op : d.ops) {
+        s += '|'; s += fuse::opName(op.type); s += '(';
+        appendOperand(s, d, op.inputIndex0, op.scalarIndex0);
+        if (isBinary(op.type)) { s += ','; appendOperand(s, d, op.inputIndex1, op.scalarIndex1); }
+        s += ')';
+        if (op.outputIndex != SIZE_MAX) { s += ">o"; appendNumber(s, op.outputIndex); }
+    }
+}
+
 std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
 {
-    std::ostringstream s;
-    s << shortType(d.dtype) << (shape == Shape::Flat ? "|flat" : shape == Shape::Rows ? "|rows" : "|gather");
-    if (shape == Shape::Flat) s << (noAlias ? "r" : "a") << std::hex << broadcastMask << std::dec;
-    s << "|i" << d.inputBuffers.size() << "o" << d.outputBuffers.size() << "s" << scalarCount(d);
-    for (const auto& op : d.ops) {
-        s << "|" << fuse::opName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
-        if (isBinary(op.type)) s << "," << operandText(d, op.inputIndex1, op.scalarIndex1);
-        s << ")";
-        if (op.outputIndex != SIZE_MAX) s << ">o" << op.outputIndex;
-    }
-    return s.str();
+    std::string s;
+    signatureInto(s, d, shape, broadcastMask, noAlias);
+    return s;
 }
 
 std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
@@ -202,13 +235,13 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     return o.str();
 }
 
-std::vector<uint64_t> packArgs(const FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
-                               const std::vector<void*>& outputs, uint64_t n, const Space* space, uint64_t chunksPerRow)
+void packArgsInto(std::vector<uint64_t>& a, const FusedSubgraphDescriptor& d, Shape shape, const void* const* inputs,
+                  void* const* outputs, uint64_t n, const Space* space, uint64_t chunksPerRow)
 {
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
     const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
     const size_t esz = aix::Device::dataTypeSize(d.dtype);
-    std::vector<uint64_t> a;
+    a.clear();
     for (size_t k = 0; k < AI; ++k) a.push_back(k < NI ? (uint64_t)(uintptr_t)inputs[k] : 0);
     for (size_t k = 0; k < NO; ++k) a.push_back((uint64_t)(uintptr_t)outputs[k]);
     for (size_t k = 0; k < AS; ++k) {
@@ -217,7 +250,7 @@ std::vector<uint64_t> packArgs(const FusedSubgraphDescriptor& d, Shape shape, co
         a.push_back(bits);
     }
     a.push_back(n);
-    if (shape == Shape::Flat) return a;
+    if (shape == Shape::Flat) return;
     if (!space) throw std::invalid_argument("strided fused kernel without an iteration space");
     a.push_back(chunksPerRow);
     a.push_back(space->rank);
@@ -225,6 +258,13 @@ std::vector<uint64_t> packArgs(const FusedSubgraphDescriptor& d, Shape shape, co
     for (size_t k = 0; k < AI; ++k) a.push_back(k < NI ? space->offset[k] : 0);
     for (size_t k = 0; k < AI; ++k)
         for (int dd = 0; dd < kMaxDims; ++dd) a.push_back(k < NI ? space->stride[k][dd] : 0);
+}
+
+std::vector<uint64_t> packArgs(const FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
+                               const std::vector<void*>& outputs, uint64_t n, const Space* space, uint64_t chunksPerRow)
+{
+    std::vector<uint64_t> a;
+    packArgsInto(a, d, shape, inputs.data(), outputs.data(), n, space, chunksPerRow);
     return a;
 }
 

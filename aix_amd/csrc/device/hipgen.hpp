@@ -26,6 +26,8 @@ enum class Shape { Flat, Rows, Gather };
 // (bit k of broadcastMask), and whether no output aliases an input (the pointers may then be
 // declared __restrict__).
 std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
+// The same text written into `out` (cleared first; its capacity is reused from call to call).
+void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias);
 
 // Source of `extern "C" __global__ void aix_fused(Args)`.
 std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
@@ -47,5 +49,8 @@ struct Space {
 std::vector<uint64_t> packArgs(const fuse::FusedSubgraphDescriptor& d, Shape shape, const std::vector<const void*>& inputs,
                                const std::vector<void*>& outputs, uint64_t n, const Space* space,
                                uint64_t chunksPerRow);
+// The same into `a` (cleared first); inputs / outputs hold one pointer per descriptor buffer.
+void packArgsInto(std::vector<uint64_t>& a, const fuse::FusedSubgraphDescriptor& d, Shape shape, const void* const* inputs,
+                  void* const* outputs, uint64_t n, const Space* space, uint64_t chunksPerRow);
 
 } // namespace aixhip::gen

@@ -61,10 +61,12 @@ public:
     Value() = default;
 
     // Uninitialised contiguous tensor.
-    Value(Device* dev, DataType dt, Shape shape) : m_dev(dev), m_dt(dt), m_shape(std::move(shape))
+    Value(Device* dev, DataType dt, Shape shape) : m_dev(dev)
     {
-        m_strides = denseStrides(m_shape);
-        m_store = std::make_shared<Storage>(dev, dev->allocate(std::max<size_t>(numel(m_shape), 1), dt));
+        m_p.dtype = dt;
+        m_p.shape = std::move(shape);
+        m_p.strides = denseStrides(m_p.shape);
+        m_store = std::make_shared<Storage>(dev, dev->allocate(std::max<size_t>(numel(m_p.shape), 1), dt));
     }
 
     // Every element = v (one device fill).
@@ -85,34 +87,39 @@ public:
 
     bool defined() const { return (bool)m_store; }
     Device* device() const { return m_dev; }
-    DataType dtype() const { return m_dt; }
-    const Shape& shape() const { return m_shape; }
-    const Stride& strides() const { return m_strides; }
-    size_t size() const { return numel(m_shape); }
+    DataType dtype() const { return m_p.dtype; }
+    const Shape& shape() const { return m_p.shape; }
+    const Stride& strides() const { return m_p.strides; }
+    size_t size() const { return numel(m_p.shape); }
     void* data() const { return m_store ? m_store->ptr : nullptr; }
-    size_t offset() const { return m_offset; }
-    bool isContiguous() const { return m_strides == denseStrides(m_shape); }
-
-    DeviceTensorParams params() const
+    size_t offset() const { return m_p.offset; }
+    bool isContiguous() const
     {
-        DeviceTensorParams p;
-        p.data = data(); p.dtype = m_dt; p.isContiguous = isContiguous(); p.offset = m_offset;
-        p.shape = m_shape; p.size = size(); p.strides = m_strides;
-        return p;
+        size_t run = 1;
+        for (size_t d = m_p.shape.size(); d-- > 0;) { if (m_p.strides[d] != run) return false; run *= m_p.shape[d]; }
+        return true;
+    }
+
+    // What the device sees of this value.  The reference is to a member that this call brings up
+    // to date: it stays valid while the value lives and is not reshaped.
+    const DeviceTensorParams& params() const
+    {
+        m_p.data = data(); m_p.isContiguous = isContiguous(); m_p.size = size();
+        return m_p;
     }
 
     // ---- views ------------------------------------------------------------------------------
     Value broadcastTo(const Shape& target) const
     {
-        if (target == m_shape) return *this;
-        if (target.size() < m_shape.size()) throw std::invalid_argument("broadcastTo: rank shrinks");
+        if (target == m_p.shape) return *this;
+        if (target.size() < m_p.shape.size()) throw std::invalid_argument("broadcastTo: rank shrinks");
         Value v = *this;
-        v.m_shape = target;
-        v.m_strides.assign(target.size(), 0);
-        const size_t lead = target.size() - m_shape.size();
-        for (size_t i = 0; i < m_shape.size(); ++i) {
-            if (m_shape[i] == target[lead + i]) v.m_strides[lead + i] = m_strides[i];
-            else if (m_shape[i] != 1) throw std::invalid_argument("broadcastTo: incompatible shape");
+        v.m_p.shape = target;
+        v.m_p.strides.assign(target.size(), 0);
+        const size_t lead = target.size() - m_p.shape.size();
+        for (size_t i = 0; i < m_p.shape.size(); ++i) {
+            if (m_p.shape[i] == target[lead + i]) v.m_p.strides[lead + i] = m_p.strides[i];
+            else if (m_p.shape[i] != 1) throw std::invalid_argument("broadcastTo: incompatible shape");
         }
         return v;
     }
@@ -120,8 +127,8 @@ public:
     Value transpose(size_t d0, size_t d1) const
     {
         Value v = *this;
-        std::swap(v.m_shape[d0], v.m_shape[d1]);
-        std::swap(v.m_strides[d0], v.m_strides[d1]);
+        std::swap(v.m_p.shape[d0], v.m_p.shape[d1]);
+        std::swap(v.m_p.strides[d0], v.m_p.strides[d1]);
         return v;
     }
 
@@ -129,8 +136,8 @@ public:
     {
         if (numel(s) != size()) throw std::invalid_argument("reshape: element count differs");
         Value v = isContiguous() ? *this : contiguous();
-        v.m_shape = s;
-        v.m_strides = denseStrides(s);
+        v.m_p.shape = s;
+        v.m_p.strides = denseStrides(s);
         return v;
     }
 
@@ -138,26 +145,26 @@ public:
     Value select0(size_t i) const
     {
         Value v = *this;
-        v.m_offset += i * m_strides[0];
-        v.m_shape.erase(v.m_shape.begin());
-        v.m_strides.erase(v.m_strides.begin());
+        v.m_p.offset += i * m_p.strides[0];
+        v.m_p.shape.erase(v.m_p.shape.begin());
+        v.m_p.strides.erase(v.m_p.strides.begin());
         return v;
     }
 
     Value contiguous() const
     {
-        if (isContiguous() && m_offset == 0) return *this;
-        Value r(m_dev, m_dt, m_shape);
+        if (isContiguous() && m_p.offset == 0) return *this;
+        Value r(m_dev, m_p.dtype, m_p.shape);
         m_dev->contiguous(params(), r.params());
         return r;
     }
 
     Value to(DataType dt) const
     {
-        if (dt == m_dt) return *this;
+        if (dt == m_p.dtype) return *this;
         Value src = contiguous();
-        Value r(m_dev, dt, m_shape);
-        m_dev->copy(static_cast<const char*>(src.data()) + src.m_offset * Device::dataTypeSize(m_dt), m_dt, r.data(), dt, size());
+        Value r(m_dev, dt, m_p.shape);
+        m_dev->copy(static_cast<const char*>(src.data()) + src.m_p.offset * Device::dataTypeSize(m_p.dtype), m_p.dtype, r.data(), dt, size());
         return r;
     }
 
@@ -167,21 +174,21 @@ public:
 
     Value binary(BinaryFn fn, const Value& other) const
     {
-        if (other.m_dt != m_dt) {
+        if (other.m_p.dtype != m_p.dtype) {
             // operands are first converted to the promoted type (aixCore.hpp:1616-1630); the drivers
             // only ever mix a floating tensor with an integer mask, which promotes to the float type
-            const bool lf = isFloat(m_dt), rf = isFloat(other.m_dt);
+            const bool lf = isFloat(m_p.dtype), rf = isFloat(other.m_p.dtype);
             if (lf == rf) throw std::invalid_argument("binary: unsupported mix of element types");
-            return lf ? binary(fn, other.to(m_dt)) : to(other.m_dt).binary(fn, other);
+            return lf ? binary(fn, other.to(m_p.dtype)) : to(other.m_p.dtype).binary(fn, other);
         }
-        if (m_shape == other.m_shape) {
-            Value r(m_dev, m_dt, m_shape);
+        if (m_p.shape == other.m_p.shape) {
+            Value r(m_dev, m_p.dtype, m_p.shape);
             (m_dev->*fn)(params(), other.params(), r.params());
             return r;
         }
-        const Shape bc = broadcastShapes(m_shape, other.m_shape);
+        const Shape bc = broadcastShapes(m_p.shape, other.m_p.shape);
         const Value l = broadcastTo(bc), rr = other.broadcastTo(bc);
-        Value r(m_dev, m_dt, bc);
+        Value r(m_dev, m_p.dtype, bc);
         (m_dev->*fn)(l.params(), rr.params(), r.params());
         return r;
     }
@@ -189,8 +196,8 @@ public:
     // tensor op scalar: rank-0 tensor + broadcast view
     Value binaryScalar(BinaryFn fn, float s, bool scalarFirst = false) const
     {
-        const Value sc = full(m_dev, m_dt, Shape{}, s).broadcastTo(m_shape);
-        Value r(m_dev, m_dt, m_shape);
+        const Value sc = full(m_dev, m_p.dtype, Shape{}, s).broadcastTo(m_p.shape);
+        Value r(m_dev, m_p.dtype, m_p.shape);
         if (scalarFirst) (m_dev->*fn)(sc.params(), params(), r.params());
         else (m_dev->*fn)(params(), sc.params(), r.params());
         return r;
@@ -198,14 +205,14 @@ public:
 
     Value& inPlace(BinaryFn fn, const Value& other)
     {
-        const Value rhs = other.m_shape == m_shape ? other : other.broadcastTo(m_shape);
+        const Value rhs = other.m_p.shape == m_p.shape ? other : other.broadcastTo(m_p.shape);
         (m_dev->*fn)(params(), rhs.params(), params());
         return *this;
     }
 
     Value unary(UnaryFn fn) const
     {
-        Value r(m_dev, m_dt, m_shape);
+        Value r(m_dev, m_p.dtype, m_p.shape);
         (m_dev->*fn)(params(), r.params());
         return r;
     }
@@ -241,14 +248,14 @@ public:
     // operators above follow its autograd class instead: rank-0 tensor + broadcast view, :2384-2438.)
     Value withScalar(BinaryFn fn, float s, bool scalarFirst = false) const
     {
-        const Value sc = full(m_dev, m_dt, m_shape, s);
+        const Value sc = full(m_dev, m_p.dtype, m_p.shape, s);
         return scalarFirst ? sc.binary(fn, *this) : binary(fn, sc);
     }
 
     // ---- reductions ---------------------------------------------------------------------------
     Value sum() const
     {
-        Value r(m_dev, m_dt, Shape{});
+        Value r(m_dev, m_p.dtype, Shape{});
         m_dev->sum(params(), r.params());
         return r;
     }
@@ -256,15 +263,15 @@ public:
     // Sum down to `target` (right-aligned, 1 = reduced): zero-fill then accumulate.
     Value reduceTo(const Shape& target) const
     {
-        if (target == m_shape) return *this;
-        Value r = full(m_dev, m_dt, target, 0.0f);
+        if (target == m_p.shape) return *this;
+        Value r = full(m_dev, m_p.dtype, target, 0.0f);
         m_dev->reduceTo(params(), r.params());
         return r;
     }
 
     Value sum(size_t dim, bool keepDim) const
     {
-        Shape kept = m_shape;
+        Shape kept = m_p.shape;
         kept[dim] = 1;
         Value r = reduceTo(kept);
         return keepDim ? r : r.squeeze(dim);
@@ -272,9 +279,9 @@ public:
 
     Value max(size_t dim, bool keepDim) const
     {
-        Shape kept = m_shape;
+        Shape kept = m_p.shape;
         kept[dim] = 1;
-        Value r(m_dev, m_dt, kept);
+        Value r(m_dev, m_p.dtype, kept);
         m_dev->fillMin(r.params());
         m_dev->maxTo(params(), r.params());
         return keepDim ? r : r.squeeze(dim);
@@ -282,7 +289,7 @@ public:
 
     Value argmax(size_t dim, bool keepDim) const
     {
-        Shape kept = m_shape;
+        Shape kept = m_p.shape;
         kept[dim] = 1;
         Value r(m_dev, DataType::kInt32, kept);
         m_dev->argmaxTo(params(), r.params(), dim);
@@ -294,7 +301,7 @@ public:
     // 1 where the element is the (first) maximum along `dim`, 0 elsewhere, int32 (aixCore.hpp:927-941).
     Value argmaxIndices(size_t dim) const
     {
-        Value r = full(m_dev, DataType::kInt32, m_shape, 0.0f);
+        Value r = full(m_dev, DataType::kInt32, m_p.shape, 0.0f);
         m_dev->argmaxIndicesTo(params(), r.params(), dim);
         return r;
     }
@@ -304,20 +311,20 @@ public:
     {
         Value v = *this;
         size_t inserted = 1;
-        if (!m_shape.empty() && dim < m_shape.size()) inserted = m_strides[dim] * m_shape[dim];
-        v.m_shape.insert(v.m_shape.begin() + (long)dim, 1);
-        v.m_strides.insert(v.m_strides.begin() + (long)dim, inserted);
+        if (!m_p.shape.empty() && dim < m_p.shape.size()) inserted = m_p.strides[dim] * m_p.shape[dim];
+        v.m_p.shape.insert(v.m_p.shape.begin() + (long)dim, 1);
+        v.m_p.strides.insert(v.m_p.strides.begin() + (long)dim, inserted);
         return v;
     }
 
     // A strided window along `dim` (view; aixCore.hpp:1089-1145).
     Value slice(size_t dim, size_t start, size_t end, size_t step = 1) const
     {
-        if (dim >= m_shape.size() || step < 1 || start >= end || end > m_shape[dim]) throw std::invalid_argument("slice: bad range");
+        if (dim >= m_p.shape.size() || step < 1 || start >= end || end > m_p.shape[dim]) throw std::invalid_argument("slice: bad range");
         Value v = *this;
-        v.m_offset += start * m_strides[dim];
-        v.m_strides[dim] *= step;
-        v.m_shape[dim] = (end - start + step - 1) / step;
+        v.m_p.offset += start * m_p.strides[dim];
+        v.m_p.strides[dim] *= step;
+        v.m_p.shape[dim] = (end - start + step - 1) / step;
         return v;
     }
 
@@ -331,18 +338,18 @@ public:
     static Value cat(const std::vector<Value>& parts, size_t dim)
     {
         if (parts.empty()) throw std::invalid_argument("cat: no tensors");
-        Shape shape = parts[0].m_shape;
-        for (size_t i = 1; i < parts.size(); ++i) shape[dim] += parts[i].m_shape[dim];
-        Value r(parts[0].m_dev, parts[0].m_dt, shape);
+        Shape shape = parts[0].m_p.shape;
+        for (size_t i = 1; i < parts.size(); ++i) shape[dim] += parts[i].m_p.shape[dim];
+        Value r(parts[0].m_dev, parts[0].m_p.dtype, shape);
         size_t at = 0;
-        for (const auto& p : parts) { r.sliceSetInPlace(p, dim, at, at + p.m_shape[dim]); at += p.m_shape[dim]; }
+        for (const auto& p : parts) { r.sliceSetInPlace(p, dim, at, at + p.m_p.shape[dim]); at += p.m_p.shape[dim]; }
         return r;
     }
 
     // aixCore.hpp:1320-1346
     Value tril(ssize_t diagonal = 0) const
     {
-        Value r(m_dev, m_dt, m_shape);
+        Value r(m_dev, m_p.dtype, m_p.shape);
         m_dev->tril(params(), r.params(), diagonal);
         return r;
     }
@@ -350,7 +357,7 @@ public:
     // Zero-padded copy of `src` into the window of a tensor shaped like *this (aixCore.hpp:1147-1204, not in place).
     Value sliceSet(const Value& src, size_t dim, size_t start, size_t end, size_t step = 1) const
     {
-        Value r = full(m_dev, m_dt, m_shape, 0.0f);
+        Value r = full(m_dev, m_p.dtype, m_p.shape, 0.0f);
         m_dev->sliceSet(src.params(), r.params(), dim, start, end, step);
         return r;
     }
@@ -358,9 +365,9 @@ public:
     // Rows (dim = 0) or other slabs picked by an int32 index vector (aixCore.hpp:1217-1247).
     Value indexSelect(size_t dim, const Value& indices) const
     {
-        Shape shape = m_shape;
+        Shape shape = m_p.shape;
         shape[dim] = indices.shape().empty() ? 1 : indices.shape()[0];
-        Value r(m_dev, m_dt, shape);
+        Value r(m_dev, m_p.dtype, shape);
         m_dev->indexSelect(params(), r.params(), indices.params(), dim);
         return r;
     }
@@ -373,7 +380,7 @@ public:
 
     Value pow(const Value& e) const
     {
-        Value r(m_dev, m_dt, m_shape);
+        Value r(m_dev, m_p.dtype, m_p.shape);
         m_dev->pow(params(), e.params(), r.params());
         return r;
     }
@@ -382,27 +389,27 @@ public:
     // backends (plain memory on the CPU, large-BAR mapping on the GPU).
     float item() const
     {
-        if (m_dt != DataType::kFloat32) throw std::invalid_argument("item: f32 only");
+        if (m_p.dtype != DataType::kFloat32) throw std::invalid_argument("item: f32 only");
         m_dev->synchronize();
         float v;
-        std::memcpy(&v, static_cast<const char*>(data()) + m_offset * sizeof(float), sizeof(float));
+        std::memcpy(&v, static_cast<const char*>(data()) + m_p.offset * sizeof(float), sizeof(float));
         return v;
     }
 
     Value squeeze(size_t dim) const
     {
         Value v = *this;
-        if (dim >= m_shape.size() || m_shape[dim] != 1) return v;
-        v.m_shape.erase(v.m_shape.begin() + (long)dim);
-        v.m_strides.erase(v.m_strides.begin() + (long)dim);
+        if (dim >= m_p.shape.size() || m_p.shape[dim] != 1) return v;
+        v.m_p.shape.erase(v.m_p.shape.begin() + (long)dim);
+        v.m_p.strides.erase(v.m_p.strides.begin() + (long)dim);
         return v;
     }
 
     Value matmul(const Value& b) const
     {
-        if (m_shape.size() != 2 || b.m_shape.size() != 2 || m_shape[1] != b.m_shape[0])
+        if (m_p.shape.size() != 2 || b.m_p.shape.size() != 2 || m_p.shape[1] != b.m_p.shape[0])
             throw std::invalid_argument("matmul: operands must be 2-D with matching inner dimension");
-        Value r(m_dev, m_dt, Shape{m_shape[0], b.m_shape[1]});
+        Value r(m_dev, m_p.dtype, Shape{m_p.shape[0], b.m_p.shape[1]});
         m_dev->matmul(params(), b.params(), r.params());
         return r;
     }
@@ -418,10 +425,7 @@ private:
     };
 
     Device* m_dev{nullptr};
-    DataType m_dt{DataType::kFloat32};
-    Shape m_shape;
-    Stride m_strides;
-    size_t m_offset{0};
+    mutable DeviceTensorParams m_p;        // dtype, offset, shape and strides live here; data / size / isContiguous are set by params()
     std::shared_ptr<Storage> m_store;
 };
 

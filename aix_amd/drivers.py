@@ -15,7 +15,7 @@ _lib = None
 
 
 class BenchResult(C.Structure):
-    _fields_ = [("wall_s", C.c_double), ("gpu_ms", C.c_float), ("steps", C.c_int32), ("reserved", C.c_int32)]
+    _fields_ = [("wall_s", C.c_double), ("gpu_ms", C.c_float), ("steps", C.c_int32), ("enqueue_us", C.c_int32)]
 
 
 def load():

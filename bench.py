@@ -35,7 +35,7 @@ MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
 
 
 class BenchResult(C.Structure):
-    _fields_ = [("wall_s", C.c_double), ("gpu_ms", C.c_float), ("steps", C.c_int32), ("reserved", C.c_int32)]
+    _fields_ = [("wall_s", C.c_double), ("gpu_ms", C.c_float), ("steps", C.c_int32), ("enqueue_us", C.c_int32)]
 
 
 def load_driver():

@@ -14,6 +14,7 @@ import aixtest as T
 import devharness as H
 import goldens
 from aix_amd import device as D
+from aix_amd import kernels as K
 from oracle import cpuref as O
 
 pytestmark = pytest.mark.gpu
@@ -337,6 +338,38 @@ def test_temporaries_are_recycled(dev):
     live, cached = C.c_uint64(), C.c_uint64()
     D.check(dev.dev.lib.aixhip_memory_stats(dev.dev.handle, C.byref(live), C.byref(cached)))
     assert cached.value <= 160 * n * 4, cached.value
+    dev.release()
+
+
+def test_used_temporaries_are_recycled(dev):
+    """The same for temporaries that enqueued work really wrote (an eager operator per iteration):
+    they come back once the GPU has passed an event, so 1.6 GiB of them hold a few hundred MiB."""
+    rng = np.random.default_rng(36001)
+    rows, cols = 1024, 1024
+    a = T.contiguous_tensor(rng, O.F32, [rows, cols])
+    pa, da = dev.put(a)
+    acc = T.HostTensor(np.zeros(rows * cols, np.float32), O.F32, [cols, rows])
+    pacc, dacc = dev.put(acc)
+    loops = 400
+    for it in range(loops):
+        pt = dev.raw(rows * cols * 4, keep=False)
+        dt = H.kdesc(acc, pt)
+        dev.dev.call("transpose", H.ref(da), H.ref(dt), 0, 1)          # runs at once: the block is used
+        dev.dev.call("add", H.ref(dacc), H.ref(dt), H.ref(dacc))
+        dev.dev.deallocate(pt)
+    got = dev.fetch(pacc, acc.storage)
+    want = np.zeros(rows * cols, np.float32)
+    at = np.ascontiguousarray(a.storage.reshape(rows, cols).T).reshape(-1)
+    for _ in range(loops):
+        want += at
+    T.assert_same_bits(got, want, "accumulated transposes")
+    live, cached = C.c_uint64(), C.c_uint64()
+    D.check(dev.dev.lib.aixhip_memory_stats(dev.dev.handle, C.byref(live), C.byref(cached)))
+    info = K.DeviceInfo()
+    K.check(K.load().aixk_info(dev.dev.kernel_context(), C.byref(info)))
+    floor = max(32 << 20, info.total_mem >> 10)
+    assert cached.value <= 3 * floor, (cached.value, floor)
+    assert cached.value < loops * rows * cols * 4 // 2
     dev.release()
 
 

@@ -236,6 +236,7 @@ def test_contiguous_and_transpose(gpu, dtype):
     cases += [([n, m], "transposed") for n, m in [(1, 1), (1, 70), (63, 65), (64, 64), (129, 257), (300, 5), (5, 300), (513, 1025)]]
     cases += [([3, 70, 130], "transposed"), ([96, 256], "sliced"), ([33, 48], "offset")]
     cases += [([128, 192], "transposed"), ([3, 64, 128], "transposed"), ([256, 64], "transposed")]   # whole tiles: 16-byte path
+    cases += [([256, 384], "transposed"), ([384, 256], "transposed"), ([2, 256, 128], "transposed")]  # whole 128 x 64 / 128 x 128 tiles, grouped order
     for shape, kind in cases:
         src = T.view_tensor(rng, dtype, shape, kind)
         want = T.empty(dtype, shape)
