@@ -349,6 +349,115 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
 #undef AIX_WAIT
 #undef AIX_SB
 
+// ---- 16-bit operands, small problems --------------------------------------------------------------
+// For outputs that 64 x 64 tiles cannot spread over the chip (the per-head matmuls of attention,
+// [512, 64] x [64, 512] and the like): a 32 x 32 tile per workgroup and the K dimension split over the
+// workgroup's four waves.  Wave w owns the 64-wide K steps w, w + 4, ...: it fetches its own operand
+// tiles (8 independent 16-byte loads per lane, the next step's in flight under the current step's
+// MFMAs), stages them in its own part of LDS and never waits for the other waves -- with so few
+// workgroups nothing else hides the latency of a K step, so the chain is made a quarter as long --
+// and the four partial tiles are added through LDS at the end.
+//
+// Both operands are consumed where they lie.  A K-contiguous operand is staged as [row][k] (pitch 72
+// elements) and read with ds_read_b128, as in gemm_nt16_k.  A T-form operand (A given as [K, M] with
+// unit stride along M, B as plain row-major [K, N]) is staged as it comes, [k][row] with a pitch of
+// 96 elements, and the fragments -- 8 consecutive k per lane -- are assembled by ds_read_b64_tr_b16
+// (see gemm_nt16_direct_k for the lane mapping); 192 bytes between k-rows put the four k-rows that a
+// group of 16 lanes reads, and the two groups of a half-wave, into disjoint banks.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+template <int PT>
+__device__ __forceinline__ u32x4 tr_fragment_lds(const u16* p)
+{
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * PT));     // k + 4
+    const u32x2 l = __builtin_bit_cast(u32x2, lo), h = __builtin_bit_cast(u32x2, hi);
+    return u32x4{l.x, l.y, h.x, h.y};
+}
+
+template <bool AT, bool BT> struct Small16 {
+    static constexpr int BM = 32, BN = 32, BK = 64, PK = BK + 8, PT = 96;
+    static constexpr int SA = AT ? BK * PT : BM * PK, SB = BT ? BK * PT : BN * PK;      // elements per wave
+    static constexpr size_t kLds = (size_t)4 * (SA + SB) * 2 > 16384 ? (size_t)4 * (SA + SB) * 2 : 16384;   // the stages double as the reduction buffer
+};
+
+template <class T, bool AT, bool BT>
+__global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g)
+{
+    typedef Small16<AT, BT> S;
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, PK = S::PK, PT = S::PT, SA = S::SA, SB = S::SB;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_small[];
+
+    u32 tm, tn;
+    tile_of(g, tm, tn);
+    const u64 m0 = (u64)tm * BM, n0 = (u64)tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const u16* A = (const u16*)g.a;
+    const u16* B = (const u16*)g.b;
+    u16* as = (u16*)smem_small + wave * (SA + SB);           // this wave's stage
+    u16* bs = as + SA;
+
+    // four 16-byte chunks per lane, operand and step: chunk c = lane + 64 i is (row c / 8, k 8 (c % 8)) of a
+    // K-contiguous tile, (k-row c / 4, column 8 (c % 4)) of a T-form tile
+    u32x4 ra[4], rb[4];
+    auto load_global = [&](u64 k0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = lane + 64 * i;
+            if constexpr (AT) { const u64 k = k0 + (c >> 2), m = m0 + (c & 3) * 8; ra[i] = (k < g.K && m < g.M) ? *(const u32x4*)(A + k * g.lda + m) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 m = m0 + (c >> 3), k = k0 + (c & 7) * 8; ra[i] = (m < g.M && k < g.K) ? *(const u32x4*)(A + m * g.lda + k) : (u32x4){0, 0, 0, 0}; }
+            if constexpr (BT) { const u64 k = k0 + (c >> 2), n = n0 + (c & 3) * 8; rb[i] = (k < g.K && n < g.N) ? *(const u32x4*)(B + k * g.ldb + n) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 n = n0 + (c >> 3), k = k0 + (c & 7) * 8; rb[i] = (n < g.N && k < g.K) ? *(const u32x4*)(B + n * g.ldb + k) : (u32x4){0, 0, 0, 0}; }
+        }
+    };
+    auto store_lds = [&] {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int c = lane + 64 * i;
+            *(u32x4*)(as + (AT ? (c >> 2) * PT + (c & 3) * 8 : (c >> 3) * PK + (c & 7) * 8)) = ra[i];
+            *(u32x4*)(bs + (BT ? (c >> 2) * PT + (c & 3) * 8 : (c >> 3) * PK + (c & 7) * 8)) = rb[i];
+        }
+    };
+    // fragment addresses inside a stage for the 16-wide K slice 0; slice kk adds 16 k
+    const int j = lane & 15;
+    const int tro = (8 * (lane >> 5) + (j >> 2)) * PT + 16 * ((lane >> 4) & 1) + 4 * (j & 3);
+    const int kro = (lane & 31) * PK + (lane >> 5) * 8;
+
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.0f;
+
+    const u64 steps = (g.K + BK - 1) / BK;
+    u64 kt = (u64)wave;
+    if (kt < steps) load_global(kt * BK);
+    for (; kt < steps; kt += 4) {
+        store_lds();                                          // the wave's LDS operations execute in order: no barrier inside a wave
+        if (kt + 4 < steps) load_global((kt + 4) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            u32x4 fa, fb;
+            if constexpr (AT) fa = tr_fragment_lds<PT>(as + tro + kk * 16 * PT); else fa = *(const u32x4*)(as + kro + kk * 16);
+            if constexpr (BT) fb = tr_fragment_lds<PT>(bs + tro + kk * 16 * PT); else fb = *(const u32x4*)(bs + kro + kk * 16);
+            acc = Mma16<T>::run(fa, fb, acc);
+        }
+    }
+
+    // add the four waves' partial tiles: slot e = 64 v + lane holds accumulator element v of lane `lane`
+    __syncthreads();
+    float* red = (float*)smem_small;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[wave * 1024 + v * 64 + lane] = acc[v];
+    __syncthreads();
+    T* C = (T*)g.c;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = tid + 256 * i, v = e >> 6, l = e & 63;
+        const float sum = (red[e] + red[1024 + e]) + (red[2048 + e] + red[3072 + e]);
+        const u64 row = m0 + (v >> 2) * 8 + (l >> 5) * 4 + (v & 3), col = n0 + (l & 31);
+        if (row < g.M && col < g.N) C[row * g.N + col] = Mma16<T>::out(sum);
+    }
+}
+
 // ---- f32 operands ------------------------------------------------------------------------------
 // 128 x 128 workgroup tile, BK = 32; LDS row = 32 floats + 4 padding = 144 bytes.  A lane reads 4
 // consecutive K of its row with one ds_read_b128 and spends them on 4 successive 32x32x2 MFMAs.
@@ -529,6 +638,41 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
             if (!at && bt) return launch(gemm_nt16_direct_k<f16, false, true>);
             if (at && !bt) return launch(gemm_nt16_direct_k<f16, true, false>);
             return launch(gemm_nt16_direct_k<f16, true, true>);
+        }
+    }
+
+    // 16-bit, outputs that 64 x 64 tiles cannot spread over the chip: 32 x 32 tiles, K split over the waves,
+    // every operand layout consumed where it lies
+    if (esz == 2 && ((M + 63) / 64) * ((N + 63) / 64) < (uint64_t)ctx->cus) {
+        const char* qa = (const char*)a->data + a->offset * esz;
+        const char* qb = (const char*)b->data + b->offset * esz;
+        const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 8 == 0;
+        const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 8 == 0;
+        const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
+        if ((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && aligned16(qa) && aligned16(qb)) {
+            GemmArgs g{};
+            g.a = qa; g.b = qb; g.c = out->data;
+            g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+            g.tiles_m = (u32)((M + 31) / 32); g.tiles_n = (u32)((N + 31) / 32);
+            const u32 n = g.tiles_m * g.tiles_n;
+            g.swizzle = n % 8u == 0 ? 1u : 0u;
+            const bool at = !a_k, bt = !b_k;
+            auto launch = [&](auto kernel, size_t lds) {
+                AIXK_TRY(set_lds(kernel, lds));
+                hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            };
+            if (out->dtype == AIXK_BF16) {
+                if (!at && !bt) return launch(gemm_small16_k<bf16, false, false>, Small16<false, false>::kLds);
+                if (!at && bt) return launch(gemm_small16_k<bf16, false, true>, Small16<false, true>::kLds);
+                if (at && !bt) return launch(gemm_small16_k<bf16, true, false>, Small16<true, false>::kLds);
+                return launch(gemm_small16_k<bf16, true, true>, Small16<true, true>::kLds);
+            }
+            if (!at && !bt) return launch(gemm_small16_k<f16, false, false>, Small16<false, false>::kLds);
+            if (!at && bt) return launch(gemm_small16_k<f16, false, true>, Small16<false, true>::kLds);
+            if (at && !bt) return launch(gemm_small16_k<f16, true, false>, Small16<true, false>::kLds);
+            return launch(gemm_small16_k<f16, true, true>, Small16<true, true>::kLds);
         }
     }
 

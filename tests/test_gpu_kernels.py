@@ -605,6 +605,22 @@ def test_matmul_mfma_tiles(gpu, dtype):
         gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16], ids=ids)
+def test_matmul_small_tiles(gpu, dtype):
+    """16-bit outputs too small for 64 x 64 tiles to fill the chip (attention heads and the like): the
+    32 x 32-tile kernel that splits K over its four waves, every operand layout consumed in place --
+    one to nine K steps, ragged tiles, K tails, extents that are no multiple of 8 (those are gathered)."""
+    rng = np.random.default_rng(23500 + dtype)
+    layouts = [("contig", "contig"), ("contig", "transposed"), ("transposed", "contig"), ("transposed", "transposed")]
+    for (m, k, n) in [(512, 64, 512), (512, 512, 64), (64, 512, 512), (96, 40, 72), (72, 200, 88), (64, 8, 64), (104, 576, 40), (99, 64, 101)]:
+        for ka, kb in layouts + [("sliced", "offset")]:
+            scale = 1.0 / np.sqrt(k)
+            a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
+            b = T.view_tensor(rng, dtype, [k, n], kb, lo=-1, hi=1)
+            check_matmul(gpu, a, b, f"small matmul {NAMES[dtype]} {m}x{k}x{n} {ka}/{kb}")
+        gpu.release()
+
+
 def test_matmul_identity_and_ones(gpu):
     """Mathematical pins: A.I == A exactly; ones[m,k].ones[k,n] == k exactly (f32, f16, bf16)."""
     rng = np.random.default_rng(22000)
