@@ -533,14 +533,15 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
         return AIXK_OK;
     }
     // outer: one reduced dim, innermost kept dim dense on both sides
-    if (p.nr == 1 && p.nk >= 1 && p.k_src[p.nk - 1] == 1 && p.k_dst[p.nk - 1] == 1 && p.k_flat[p.nk - 1] == 1 && p.red >= 8) {
+    if (p.nr == 1 && p.nk >= 1 && p.k_src[p.nk - 1] == 1 && p.k_dst[p.nk - 1] == 1 && p.k_flat[p.nk - 1] == 1 && p.red >= 2) {
         const uint64_t C = p.k_ext[p.nk - 1], R = p.r_ext[0], O = p.slots / C;
         constexpr int VEC = VEC16 < 4 ? VEC16 : 4;
         bool vect = C % VEC == 0 && ((uintptr_t)(ps + p.src_off) % (sizeof(T) * VEC)) == 0 && p.r_src[0] % VEC == 0;
         for (int d = 0; d + 1 < p.nk; ++d) if (p.k_src[d] % VEC) vect = false;
         const int v = vect ? VEC : 1;
-        // wide rows: workgroups of 256 * v columns, rows split into chunks of at least 16
-        if (vect && C >= (uint64_t)kBlock * v * 2 && R >= 64 && O <= 65535) {
+        // wide rows: workgroups of 256 * v columns, rows split into chunks of at least 16 (a handful of rows --
+        // the pair axis of a composed ReLU, say -- is one chunk: every lane folds its columns outright)
+        if (vect && C >= (uint64_t)kBlock * v * 2 && (R >= 64 || R < 8) && O <= 65535) {
             const uint64_t tiles = (C + (uint64_t)kBlock * v - 1) / ((uint64_t)kBlock * v);
             const uint64_t want = (uint64_t)cus * (sizeof(Acc) > 8 ? 2 : 8);      // wide partial records: fewer, longer chunks
             uint64_t chunks = tiles * O < want ? std::min<uint64_t>({(want + tiles * O - 1) / (tiles * O), (R + 15) / 16, (uint64_t)65535}) : 1;
