@@ -396,6 +396,105 @@ static void testEveryTypeAndOperatorCompiles()
     }
 }
 
+static void testPointerSetGrowsAndForgets()
+{
+    PointerSet set;
+    CHECK(!set.contains(reinterpret_cast<void*>(0x1000)));
+    const size_t n = 50000;
+    for (size_t i = 1; i <= n; ++i) set.insert(reinterpret_cast<void*>(i * 0x100));
+    CHECK(set.size() == n);
+    bool all = true;
+    for (size_t i = 1; i <= n; ++i) if (!set.contains(reinterpret_cast<void*>(i * 0x100))) all = false;
+    CHECK(all);
+    CHECK(!set.contains(reinterpret_cast<void*>((n + 1) * 0x100)) && !set.contains(reinterpret_cast<void*>(0x80)));
+    set.insert(reinterpret_cast<void*>(0x100));                      // twice: still one member
+    CHECK(set.size() == n);
+    for (size_t i = 1; i <= n; i += 2) set.erase(reinterpret_cast<void*>(i * 0x100));
+    CHECK(set.size() == n / 2);
+    bool odd_gone = true, even_there = true;
+    for (size_t i = 1; i <= n; ++i) {
+        const bool in = set.contains(reinterpret_cast<void*>(i * 0x100));
+        if (i % 2 == 1 && in) odd_gone = false;
+        if (i % 2 == 0 && !in) even_there = false;
+    }
+    CHECK(odd_gone && even_there);
+    // allocate / free churn over the same addresses: graves are reused, lookups stay exact
+    for (int round = 0; round < 200; ++round)
+        for (size_t i = 1; i <= 300; i += 2) {
+            void* p = reinterpret_cast<void*>(i * 0x100);
+            set.insert(p);
+            if (!set.contains(p)) { CHECK(false); return; }
+            set.erase(p);
+        }
+    CHECK(set.size() == n / 2);
+}
+
+static void testViewLimitsAndRoundTrip()
+{
+    auto p = T(5, {3, 1, 4}, DataType::kInt16, {4, 99, 1}, 7);           // an extent-1 dimension may carry any stride
+    View v(p);
+    CHECK(v.rank == 3 && v.dense && v.offset == 7 && v.size == 12 && v.dtype == DataType::kInt16);
+    const auto q = v.params();
+    CHECK(q.data == p.data && q.shape == p.shape && q.strides == p.strides && q.offset == 7 && q.size == 12);
+    View w(T(5, {3, 4}, DataType::kInt16, {1, 3}));
+    CHECK(!w.dense);
+    w.makeDense();
+    CHECK(w.dense && w.offset == 0 && w.strides[0] == 4 && w.strides[1] == 1);
+    bool threw = false;
+    try { View too(T(6, aix::Shape(17, 1))); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw);
+    View copy = v;                                                        // copies carry only the meaningful extents
+    CHECK(copy.sameShape(v) && copy.strides[1] == 99 && copy.sameShape(aix::Shape{3, 1, 4}) && !copy.sameShape(aix::Shape{3, 4}));
+}
+
+static void testEngineStorageIsReusedAcrossWindows()
+{
+    // many windows through one engine: the descriptor handed out is the engine's own and is refilled,
+    // results do not depend on what earlier windows left behind
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    for (int round = 0; round < 50; ++round) {
+        const aix::Shape shape{64, (size_t)(8 + round)};
+        recordChain(e, 1.0f, 0.5f, true, shape);
+        if (round % 3 == 0) {                                            // a second, unrelated kernel in the same window
+            auto x = T(40, {10}), y = T(41, {10}), z = T(42, {10});
+            for (uintptr_t id : {40, 41, 42}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+            e.record(OpType::Add, x, y, z);
+            e.record(OpType::Exp, z, z);
+        }
+        e.flush();
+    }
+    CHECK(cap.fused.size() == 50 + 17);
+    bool ok = true;
+    size_t chains = 0;
+    for (const auto& d : cap.fused) {
+        if (d.ops.size() == 9) { ++chains; if (d.inputBuffers.size() != 3 || d.outputBuffers.size() != 1 || d.scalarData.size() != 8) ok = false; }
+        else if (d.ops.size() != 2 || d.inputBuffers.size() != 2 || d.outputBuffers.size() != 1 || d.elementCount != 10) ok = false;
+    }
+    CHECK(ok && chains == 50);
+}
+
+static void testTrailingFillIsHandedOver()
+{
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto a = T(1, {8, 8}), d = T(2, {8}), other = T(3, {8});
+    for (uintptr_t id : {1, 2, 3}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    const float zero = 0.0f, seven = 7.0f;
+    e.recordFill(&seven, DataType::kFloat32, other);
+    e.recordFill(&zero, DataType::kFloat32, d);
+    OpRecord fill;
+    CHECK(e.takeTrailingFill(d, &fill));                                  // newest operator on d is a fill of all of d
+    CHECK(fill.type == OpType::Fill && fill.output.data == d.data && e.pendingOps() == 1);
+    float got; std::memcpy(&got, fill.scalarData.data(), 4);
+    CHECK(got == 0.0f);
+    CHECK(!e.takeTrailingFill(d, &fill));                                 // nothing left for d
+    e.recordFill(&zero, DataType::kFloat32, d);
+    e.record(OpType::Add, d, other, a.data == nullptr ? d : T(4, {8}));   // somebody reads d after the fill
+    CHECK(!e.takeTrailingFill(d, &fill));
+    e.flush();
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -416,6 +515,10 @@ int main(int argc, char** argv)
     testThresholdFlushAndExternalRead();
     testFillMinAndIntegerScalars();
     testEveryTypeAndOperatorCompiles();
+    testPointerSetGrowsAndForgets();
+    testViewLimitsAndRoundTrip();
+    testEngineStorageIsReusedAcrossWindows();
+    testTrailingFillIsHandedOver();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

@@ -373,6 +373,29 @@ def test_used_temporaries_are_recycled(dev):
     dev.release()
 
 
+def test_interior_pointer_operands(dev):
+    """Operands and results may point into the middle of an allocation (two tensors carved out of one
+    block): the device recognises them as its own memory, orders the work and frees the block once."""
+    rng = np.random.default_rng(36500)
+    n = 1 << 16
+    lo = T.contiguous_tensor(rng, O.F32, [n])
+    hi = T.contiguous_tensor(rng, O.F32, [n])
+    big = dev.raw(2 * n * 4)
+    dev.dev.from_host(big, lo.storage)
+    dev.dev.from_host(big + n * 4, hi.storage)
+    d_lo, d_hi = H.kdesc(lo, big), H.kdesc(hi, big + n * 4)
+    out = dev.raw(n * 4)
+    dev.dev.call("add", H.ref(d_lo), H.ref(d_hi), H.ref(H.kdesc(lo, out)))
+    T.assert_same_bits(dev.fetch(out, lo.storage), lo.storage + hi.storage, "sum of the two halves")
+    dev.dev.call("mul", H.ref(d_lo), H.ref(d_lo), H.ref(d_hi))             # result through an interior pointer
+    dev.dev.call("sum", H.ref(d_hi), H.ref(H.kdesc(T.empty(O.F32, [1]), out)))   # an operator that runs at once reads it
+    T.assert_same_bits(dev.fetch(big + n * 4, hi.storage), lo.storage * lo.storage, "square written into the upper half")
+    got = dev.fetch(out, np.zeros(1, np.float32))
+    want = np.float64((lo.storage.astype(np.float64) ** 2).sum())
+    assert abs(float(got[0]) - want) <= 1e-5 * want
+    dev.release()
+
+
 _CASES = goldens.load_cases()
 
 
