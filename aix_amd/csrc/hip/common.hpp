@@ -57,6 +57,10 @@ struct aixk_ctx {
     void* scratch{nullptr};
     size_t scratch_bytes{0};
     unsigned int* counter{nullptr};
+    // matmul: K-contiguous copies of operands whose layout the kernels cannot consume in place
+    // (A and B); grown on demand, ordered on `stream` like everything else
+    void* gemm_ws[2]{nullptr, nullptr};
+    size_t gemm_ws_bytes[2]{0, 0};
     // runtime-compiled kernels by signature
     std::unordered_map<std::string, aixk_module*> rtc;
     uint64_t rtc_hits{0}, rtc_misses{0};

@@ -459,17 +459,25 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g)
 }
 
 // ---- f32 operands ------------------------------------------------------------------------------
-// 128 x 128 workgroup tile, BK = 32; LDS row = 32 floats + 4 padding = 144 bytes.  A lane reads 4
-// consecutive K of its row with one ds_read_b128 and spends them on 4 successive 32x32x2 MFMAs.
-template <int BM, int BN>
+// 128 x 128 (or 64 x 64) workgroup tile, BK = 32.  v_mfma_f32_32x32x2f32 takes one element per lane
+// and operand -- lane l holds A[row l % 32][k l / 32] -- so both operand forms feed it directly:
+//   K-contiguous (A as [M, K], B given as [N, K]): staged [row][k], 32 floats + 4 padding per row;
+//     a lane reads 4 consecutive k of its row with one ds_read_b128 and spends them on 4 MFMAs;
+//   T form (A given as [K, M] with unit stride along M, B as plain row-major [K, N]): staged as it
+//     comes, [k][row] with a pitch of BM + 8 floats; a lane reads its column of 4 consecutive k-rows
+//     with 4 ds_read_b32 (32 consecutive floats per half-wave; the other half-wave's rows k + 4 start
+//     32 banks away), no transposing copy beforehand.
+template <int BM, int BN, bool AT, bool BT>
 __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
 {
     constexpr int BK = 32, LDR = BK + 4;
     constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
-    constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;      // 4 each
+    constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;      // 16-byte chunks per lane, operand and step
+    constexpr int PA = AT ? BM + 8 : LDR, PB = BT ? BN + 8 : LDR;          // floats per LDS row
+    constexpr int SA = (AT ? BK : BM) * PA, SB = (BT ? BK : BN) * PB;      // floats per stage
     extern __shared__ __attribute__((aligned(16))) unsigned char smem32[];
-    float (*As)[BM][LDR] = (float (*)[BM][LDR])smem32;                       // [2][BM][LDR]
-    float (*Bs)[BN][LDR] = (float (*)[BN][LDR])(smem32 + sizeof(float) * 2 * BM * LDR);
+    float* As = (float*)smem32;                                            // [2][SA]
+    float* Bs = As + 2 * SA;                                               // [2][SB]
 
     u32 tm, tn;
     tile_of(g, tm, tn);
@@ -487,39 +495,59 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    // chunk c of a K-contiguous tile is (row c / 8, k 4 (c % 8)); of a T-form tile (k-row c / (B / 4), column 4 (c % (B / 4)))
     f32x4 ra[CA], rb[CB];
     auto load_global = [&](u64 k0) {
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
-            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
-            const u64 r = m0 + row, k = k0 + kc * 4;
-            ra[i] = (r < g.M && k < g.K) ? *(const f32x4*)(A + r * g.lda + k) : (f32x4){0, 0, 0, 0};
+            const int c = tid + 256 * i;
+            if constexpr (AT) { const u64 k = k0 + c / (BM / 4), m = m0 + (c % (BM / 4)) * 4; ra[i] = (k < g.K && m < g.M) ? *(const f32x4*)(A + k * g.lda + m) : (f32x4){0, 0, 0, 0}; }
+            else { const u64 r = m0 + (c >> 3), k = k0 + (c & 7) * 4; ra[i] = (r < g.M && k < g.K) ? *(const f32x4*)(A + r * g.lda + k) : (f32x4){0, 0, 0, 0}; }
         }
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
-            const int c = tid + 256 * i, row = c >> 3, kc = c & 7;
-            const u64 r = n0 + row, k = k0 + kc * 4;
-            rb[i] = (r < g.N && k < g.K) ? *(const f32x4*)(B + r * g.ldb + k) : (f32x4){0, 0, 0, 0};
+            const int c = tid + 256 * i;
+            if constexpr (BT) { const u64 k = k0 + c / (BN / 4), n = n0 + (c % (BN / 4)) * 4; rb[i] = (k < g.K && n < g.N) ? *(const f32x4*)(B + k * g.ldb + n) : (f32x4){0, 0, 0, 0}; }
+            else { const u64 r = n0 + (c >> 3), k = k0 + (c & 7) * 4; rb[i] = (r < g.N && k < g.K) ? *(const f32x4*)(B + r * g.ldb + k) : (f32x4){0, 0, 0, 0}; }
         }
     };
     auto store_lds = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < CA; ++i) { const int c = tid + 256 * i; *(f32x4*)&As[buf][c >> 3][(c & 7) * 4] = ra[i]; }
+        for (int i = 0; i < CA; ++i) {
+            const int c = tid + 256 * i;
+            *(f32x4*)(As + buf * SA + (AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : (c >> 3) * PA + (c & 7) * 4)) = ra[i];
+        }
 #pragma unroll
-        for (int i = 0; i < CB; ++i) { const int c = tid + 256 * i; *(f32x4*)&Bs[buf][c >> 3][(c & 7) * 4] = rb[i]; }
+        for (int i = 0; i < CB; ++i) {
+            const int c = tid + 256 * i;
+            *(f32x4*)(Bs + buf * SB + (BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : (c >> 3) * PB + (c & 7) * 4)) = rb[i];
+        }
     };
 
-    // Fragments are double buffered: the four ds_read_b128 of the next 8-wide K slice are issued
-    // under the 16 MFMAs of the current one; the tile for the next step goes to the other LDS buffer
-    // under the third slice; the step's barrier sits before the last slice, whose MFMAs cover the
-    // first fragment reads from that buffer.  sched_barrier keeps the phases apart (left alone,
-    // the compiler emits "4 reads, wait, 16 MFMAs" per slice and exposes the LDS latency each time).
+    // Fragments are double buffered: the reads of the next 8-wide K slice are issued under the 16
+    // MFMAs of the current one; the tile for the next step goes to the other LDS buffer under the
+    // third slice; the step's barrier sits before the last slice, whose MFMAs cover the first
+    // fragment reads from that buffer.  sched_barrier keeps the phases apart (left alone, the
+    // compiler emits "4 reads, wait, 16 MFMAs" per slice and exposes the LDS latency each time).
     f32x4 fa[2][TI], fb[2][TJ];
     auto read_frags = [&](int set, int buf, int kk) {
+        const int k = kk * 8 + (lane >> 5) * 4;
 #pragma unroll
-        for (int i = 0; i < TI; ++i) fa[set][i] = *(const f32x4*)&As[buf][wm * WM + i * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
+        for (int i = 0; i < TI; ++i) {
+            const int row = wm * WM + i * 32 + (lane & 31);
+            if constexpr (AT) {
 #pragma unroll
-        for (int j = 0; j < TJ; ++j) fb[set][j] = *(const f32x4*)&Bs[buf][wn * WN + j * 32 + (lane & 31)][kk * 8 + (lane >> 5) * 4];
+                for (int e = 0; e < 4; ++e) fa[set][i][e] = As[buf * SA + (k + e) * PA + row];
+            } else fa[set][i] = *(const f32x4*)(As + buf * SA + row * PA + k);
+        }
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const int row = wn * WN + j * 32 + (lane & 31);
+            if constexpr (BT) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) fb[set][j][e] = Bs[buf * SB + (k + e) * PB + row];
+            } else fb[set][j] = *(const f32x4*)(Bs + buf * SB + row * PB + k);
+        }
     };
     auto mma = [&](int set) {
 #pragma unroll
@@ -564,20 +592,21 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
 }
 
 // Workspace for operands that have to be made K-contiguous; grows on demand, lives with the
-// process (all use is ordered on the context's single stream).
-struct Workspace { void* ptr{nullptr}; size_t bytes{0}; };
-Workspace g_ws[2];
-
-int workspace(int which, size_t bytes, void** out)
+// context (all use is ordered on the context's single stream).
+int workspace(aixk_ctx* ctx, int which, size_t bytes, void** out)
 {
-    Workspace& w = g_ws[which];
-    if (w.bytes < bytes) {
-        if (w.ptr) { AIXK_HIP(hipDeviceSynchronize()); AIXK_HIP(hipFree(w.ptr)); w.ptr = nullptr; w.bytes = 0; }
+    if (ctx->gemm_ws_bytes[which] < bytes) {
+        if (ctx->gemm_ws[which]) {
+            AIXK_HIP(hipStreamSynchronize(ctx->stream));
+            AIXK_HIP(hipFree(ctx->gemm_ws[which]));
+            ctx->gemm_ws[which] = nullptr;
+            ctx->gemm_ws_bytes[which] = 0;
+        }
         const size_t want = (bytes + (size_t(1) << 20)) & ~((size_t(1) << 20) - 1);
-        if (hipMalloc(&w.ptr, want) != hipSuccess) { (void)hipGetLastError(); return fail(AIXK_ENOMEM, "matmul workspace of %zu bytes", want); }
-        w.bytes = want;
+        if (hipMalloc(&ctx->gemm_ws[which], want) != hipSuccess) { (void)hipGetLastError(); ctx->gemm_ws[which] = nullptr; return fail(AIXK_ENOMEM, "matmul workspace of %zu bytes", want); }
+        ctx->gemm_ws_bytes[which] = want;
     }
-    *out = w.ptr;
+    *out = ctx->gemm_ws[which];
     return AIXK_OK;
 }
 
@@ -641,9 +670,10 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         }
     }
 
-    // 16-bit, outputs that 64 x 64 tiles cannot spread over the chip: 32 x 32 tiles, K split over the waves,
-    // every operand layout consumed where it lies
-    if (esz == 2 && ((M + 63) / 64) * ((N + 63) / 64) < (uint64_t)ctx->cus) {
+    // 16-bit, outputs that 64 x 64 tiles cannot spread over the chip twice: 32 x 32 tiles, K split over the waves,
+    // every operand layout consumed where it lies (measured against the 64 x 64 route: 1024^3 NN 23.9 -> 15.2 us;
+    // beyond two tiles per compute unit the larger tiles win)
+    if (esz == 2 && ((M + 63) / 64) * ((N + 63) / 64) < (uint64_t)ctx->cus * 2) {
         const char* qa = (const char*)a->data + a->offset * esz;
         const char* qb = (const char*)b->data + b->offset * esz;
         const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 8 == 0;
@@ -676,12 +706,70 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         }
     }
 
-    // A as [M,K] and B as [N,K], both with unit stride along K and 16-byte aligned rows
+    auto grid_of = [&](GemmArgs& g, uint64_t bm, uint64_t bn) {
+        g.tiles_m = (u32)((M + bm - 1) / bm);
+        g.tiles_n = (u32)((N + bn - 1) / bn);
+        const u32 n = g.tiles_m * g.tiles_n;
+        g.swizzle = n % 8u == 0 ? 1u : 0u;
+        return n;
+    };
+    // problems that 128 x 128 tiles cannot spread over the chip twice use 64 x 64 tiles
+    const bool small_tiles = ((M + 127) / 128) * ((N + 127) / 128) < (uint64_t)ctx->cus * 2;
+
+    // f32: either operand form is consumed where it lies (K-contiguous, or unit stride along M / N with an extent
+    // that is a multiple of 4); anything else is gathered into K-contiguous scratch first
+    if (out->dtype == AIXK_F32) {
+        const char* pa = (const char*)a->data + a->offset * esz;
+        const char* pb = (const char*)b->data + b->offset * esz;
+        const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 4 == 0;
+        const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 4 == 0;
+        uint64_t lda = a_k ? a->strides[0] : a->strides[1], ldb = b_k ? b->strides[1] : b->strides[0];
+        bool at = !a_k && a_m, bt = !b_k && b_n;
+        if (!(a_k || a_m) || lda % 4 != 0 || !aligned16(pa)) {
+            void* ws;
+            AIXK_TRY(workspace(ctx, 0, M * K * esz, &ws));
+            AIXK_TRY(gather_dense(ctx, a, ws, M * K));
+            pa = (const char*)ws; lda = K; at = false;
+        }
+        if (!(b_k || b_n) || ldb % 4 != 0 || !aligned16(pb)) {
+            aixhip_tensor bt_view = *b;                           // the [N,K] view of b
+            bt_view.shape[0] = N; bt_view.shape[1] = K;
+            bt_view.strides[0] = b->strides[1]; bt_view.strides[1] = b->strides[0];
+            void* ws;
+            AIXK_TRY(workspace(ctx, 1, N * K * esz, &ws));
+            AIXK_TRY(gather_dense(ctx, &bt_view, ws, N * K));
+            pb = (const char*)ws; ldb = K; bt = false;
+        }
+        GemmArgs g{};
+        g.a = pa; g.b = pb; g.c = out->data;
+        g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
+        auto launch = [&](auto kernel, uint64_t tile, size_t lds) {
+            const u32 n = grid_of(g, tile, tile);
+            AIXK_TRY(set_lds(kernel, lds));
+            hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
+            AIXK_HIP(hipGetLastError());
+            return (int)AIXK_OK;
+        };
+        // stage sizes: K-contiguous rows x 36 floats, T form 32 k-rows x (tile + 8) floats
+        auto lds_of = [](size_t tile, bool ta, bool tb) { return 2 * sizeof(float) * ((ta ? 32 * (tile + 8) : tile * 36) + (tb ? 32 * (tile + 8) : tile * 36)); };
+        if (small_tiles) {
+            if (!at && !bt) return launch(gemm_nt32_k<64, 64, false, false>, 64, lds_of(64, false, false));
+            if (!at && bt) return launch(gemm_nt32_k<64, 64, false, true>, 64, lds_of(64, false, true));
+            if (at && !bt) return launch(gemm_nt32_k<64, 64, true, false>, 64, lds_of(64, true, false));
+            return launch(gemm_nt32_k<64, 64, true, true>, 64, lds_of(64, true, true));
+        }
+        if (!at && !bt) return launch(gemm_nt32_k<128, 128, false, false>, 128, lds_of(128, false, false));
+        if (!at && bt) return launch(gemm_nt32_k<128, 128, false, true>, 128, lds_of(128, false, true));
+        if (at && !bt) return launch(gemm_nt32_k<128, 128, true, false>, 128, lds_of(128, true, false));
+        return launch(gemm_nt32_k<128, 128, true, true>, 128, lds_of(128, true, true));
+    }
+
+    // 16-bit: A as [M,K] and B as [N,K], both with unit stride along K and 16-byte aligned rows
     const char* pa = (const char*)a->data + a->offset * esz;
     uint64_t lda = a->strides[0];
     if (!(a->strides[1] == 1 || K == 1) || lda % kq != 0 || !aligned16(pa)) {
         void* ws;
-        AIXK_TRY(workspace(0, M * K * esz, &ws));
+        AIXK_TRY(workspace(ctx, 0, M * K * esz, &ws));
         AIXK_TRY(gather_dense(ctx, a, ws, M * K));
         pa = (const char*)ws;
         lda = K;
@@ -693,7 +781,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         bt.shape[0] = N; bt.shape[1] = K;
         bt.strides[0] = b->strides[1]; bt.strides[1] = b->strides[0];
         void* ws;
-        AIXK_TRY(workspace(1, N * K * esz, &ws));
+        AIXK_TRY(workspace(ctx, 1, N * K * esz, &ws));
         AIXK_TRY(gather_dense(ctx, &bt, ws, N * K));
         pb = (const char*)ws;
         ldb = K;
@@ -702,44 +790,21 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
     GemmArgs g{};
     g.a = pa; g.b = pb; g.c = out->data;
     g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
-    auto grid_of = [&](uint64_t bm, uint64_t bn) {
-        g.tiles_m = (u32)((M + bm - 1) / bm);
-        g.tiles_n = (u32)((N + bn - 1) / bn);
-        const u32 n = g.tiles_m * g.tiles_n;
-        g.swizzle = n % 8u == 0 ? 1u : 0u;
-        return n;
-    };
-    // problems that 128 x 128 tiles cannot spread over the chip twice use 64 x 64 tiles
-    const bool small_tiles = ((M + 127) / 128) * ((N + 127) / 128) < (uint64_t)ctx->cus * 2;
-    if (out->dtype == AIXK_F32) {
-        if (small_tiles) {
-            constexpr size_t lds = 2 * (64 + 64) * 36 * sizeof(float);
-            const u32 n = grid_of(64, 64);
-            AIXK_TRY(set_lds(gemm_nt32_k<64, 64>, lds));
-            hipLaunchKernelGGL((gemm_nt32_k<64, 64>), dim3(n), dim3(256), lds, ctx->stream, g);
-        } else {
-            constexpr size_t lds = 2 * (128 + 128) * 36 * sizeof(float);
-            const u32 n = grid_of(128, 128);
-            AIXK_TRY(set_lds(gemm_nt32_k<128, 128>, lds));
-            hipLaunchKernelGGL((gemm_nt32_k<128, 128>), dim3(n), dim3(256), lds, ctx->stream, g);
-        }
-        AIXK_HIP(hipGetLastError());
-        return AIXK_OK;
-    }
+    auto grid16 = [&](uint64_t bm, uint64_t bn) { return grid_of(g, bm, bn); };
     const bool big = ((M + 255) / 256) * ((N + 255) / 256) >= (uint64_t)ctx->cus / 2;
     if (big) {
         constexpr size_t lds = 2 * (256 + 256) * 72 * 2;
-        const u32 n = grid_of(256, 256);
+        const u32 n = grid16(256, 256);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }
         else { AIXK_TRY(set_lds(gemm_nt16_k<f16, 256, 256>, lds)); hipLaunchKernelGGL((gemm_nt16_k<f16, 256, 256>), dim3(n), dim3(256), lds, ctx->stream, g); }
     } else if (small_tiles) {
         constexpr size_t lds = 2 * (64 + 64) * 72 * 2;
-        const u32 n = grid_of(64, 64);
+        const u32 n = grid16(64, 64);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 64, 64>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 64, 64>), dim3(n), dim3(256), lds, ctx->stream, g); }
         else { AIXK_TRY(set_lds(gemm_nt16_k<f16, 64, 64>, lds)); hipLaunchKernelGGL((gemm_nt16_k<f16, 64, 64>), dim3(n), dim3(256), lds, ctx->stream, g); }
     } else {
         constexpr size_t lds = 2 * (128 + 128) * 72 * 2;
-        const u32 n = grid_of(128, 128);
+        const u32 n = grid16(128, 128);
         if (out->dtype == AIXK_BF16) { AIXK_TRY(set_lds(gemm_nt16_k<bf16, 128, 128>, lds)); hipLaunchKernelGGL((gemm_nt16_k<bf16, 128, 128>), dim3(n), dim3(256), lds, ctx->stream, g); }
         else { AIXK_TRY(set_lds(gemm_nt16_k<f16, 128, 128>, lds)); hipLaunchKernelGGL((gemm_nt16_k<f16, 128, 128>), dim3(n), dim3(256), lds, ctx->stream, g); }
     }

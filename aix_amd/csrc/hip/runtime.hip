@@ -79,6 +79,7 @@ int32_t aixk_destroy(aixk_ctx* ctx)
     }
     (void)hipFree(ctx->scratch);
     (void)hipFree(ctx->counter);
+    for (void* ws : ctx->gemm_ws) if (ws) (void)hipFree(ws);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return AIXK_OK;
