@@ -75,9 +75,51 @@ void mlp_loop(aix::Device& dev, uint64_t batch, uint64_t in, uint64_t hidden, ui
     dev.synchronize();
 }
 
+// The reference's XOR example (Targets/AIXExamples/XORMetalApp/Main.cpp) as a function of the device:
+// nn::Sequential of Linear / Tanh, MSELoss, Adam, parameters created on the host and moved with
+// Module::to(device) / to(dtype), inputs built from double literals and converted on the device,
+// the loss read through item<float>() after synchronize().  losses[epochs], predictions[4].
+void xor_loop(aix::Device& dev, aix::DataType dtype, size_t hidden1, size_t hidden2, int epochs, float lr, float* losses, float* predictions)
+{
+    aix::manualSeed(1234);                                  // identical initial parameters on every device
+    aix::nn::Sequential model;
+    model.add(aix::nn::Linear(2, hidden1));
+    model.add(aix::nn::Tanh());
+    model.add(aix::nn::Linear(hidden1, hidden2));
+    model.add(aix::nn::Tanh());
+    model.add(aix::nn::Linear(hidden2, 1));
+    model.to(dev);
+    model.to(dtype);
+    auto inputs = aix::tensor({0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0}, {4, 2}).to(dev).to(dtype);
+    auto targets = aix::tensor({0.0, 1.0, 1.0, 0.0}, {4, 1}).to(dev).to(dtype);
+    aix::optim::Adam optimizer(model.parameters(), lr);
+    auto lossFunc = aix::nn::MSELoss();
+    for (int epoch = 0; epoch < epochs; ++epoch) {
+        auto loss = lossFunc(model.forward(inputs), targets);
+        optimizer.zeroGrad();
+        loss.backward();
+        optimizer.step();
+        loss = loss.to(aix::DataType::kFloat32);
+        dev.synchronize();
+        losses[epoch] = loss.value().item<float>();
+    }
+    auto final = model.forward(inputs).to(aix::DataType::kFloat32);
+    dev.synchronize();
+    for (int i = 0; i < 4; ++i) predictions[i] = final.value().data<float>()[i];
+}
+
 } // namespace
 
 extern "C" {
+
+int aixref_xor(int dtype, uint64_t hidden1, uint64_t hidden2, int epochs, float lr, float* losses, float* predictions)
+{
+    try {
+        aix::DeviceCPU dev;
+        xor_loop(dev, static_cast<aix::DataType>(dtype), hidden1, hidden2, epochs, lr, losses, predictions);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
 
 int aixref_mlp(uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr,
                const float* x, const float* y, const float* const* w, const float* const* b, float* losses, uint64_t* counts)
@@ -99,6 +141,15 @@ int aixref_mlp_hip(uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, i
     try {
         aix::hip::DeviceHIP dev;
         mlp_loop(dev, batch, in, hidden, out, steps, lr, x, y, w, b, losses);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
+
+int aixref_xor_hip(int dtype, uint64_t hidden1, uint64_t hidden2, int epochs, float lr, float* losses, float* predictions)
+{
+    try {
+        aix::hip::DeviceHIP dev;
+        xor_loop(dev, static_cast<aix::DataType>(dtype), hidden1, hidden2, epochs, lr, losses, predictions);
         return 0;
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
 }

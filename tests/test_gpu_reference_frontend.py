@@ -36,3 +36,22 @@ def test_restated_front_end_issues_the_same_stream_on_the_gpu():
     finally:
         dev.close()
     assert via_reference.view(np.uint32).tolist() == via_restatement.view(np.uint32).tolist()
+
+
+@pytest.mark.parametrize("dtype,first,tol", [(1, 12, 2e-4), (2, 3, 5e-2), (3, 3, 1e-1)], ids=["f32", "f16", "bf16"])
+def test_reference_xor_example_runs_unchanged_on_device_hip(dtype, first, tol):
+    """The reference's XOR example (nn::Sequential of Linear / Tanh, MSELoss, Adam; parameters made on
+    the host and moved with Module::to(device) / to(dtype), double literals converted on the device,
+    item<float>() after synchronize()) with DeviceHIP in place of its GPU device: the first epochs'
+    losses follow the same program on the reference's CPU device, and in f32 both runs learn XOR."""
+    hidden1, hidden2, epochs = 64, 32, 400 if dtype == 1 else 6
+    cpu_losses, cpu_pred = OD.ref_xor(dtype, hidden1, hidden2, epochs, 0.01)
+    gpu_losses, gpu_pred = OD.ref_hip_xor(dtype, hidden1, hidden2, epochs, 0.01)
+    rel = np.abs(gpu_losses[:first].astype(np.float64) - cpu_losses[:first]) / np.abs(cpu_losses[:first])
+    print(f"XOR dtype {dtype}: CPU {cpu_losses[:4]} ... {cpu_losses[-1]:.3e}; DeviceHIP {gpu_losses[:4]} ... {gpu_losses[-1]:.3e}; max rel dev of the first {first}: {rel.max():.3e}")
+    assert np.all(np.isfinite(gpu_losses))
+    assert rel.max() <= tol
+    if dtype == 1:
+        want = np.array([0.0, 1.0, 1.0, 0.0])
+        assert cpu_losses[-1] < 1e-3 and gpu_losses[-1] < 1e-3
+        assert np.abs(cpu_pred - want).max() < 5e-2 and np.abs(gpu_pred - want).max() < 5e-2
