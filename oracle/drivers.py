@@ -171,6 +171,30 @@ def ref_hip_xor(dtype, hidden1, hidden2, epochs, lr):
     return np.array(losses, dtype=np.float32), np.array(preds, dtype=np.float32)
 
 
+def _ref_hip_xor_save_load_here(hidden1, hidden2, epochs, lr, path):
+    lib = C.CDLL(ref_hip_lib_path())
+    lib.aixref_xor_save_load_hip.argtypes = [C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_char_p, _PF]
+    lib.aixref_drivers_last_error.restype = C.c_char_p
+    preds = np.zeros(12, dtype=np.float32)
+    if lib.aixref_xor_save_load_hip(hidden1, hidden2, epochs, lr, path.encode(), preds.ctypes.data_as(_PF)) != 0:
+        raise RuntimeError(lib.aixref_drivers_last_error().decode())
+    return preds
+
+
+def ref_hip_xor_save_load(hidden1, hidden2, epochs, lr, path):
+    """nn::save from DeviceHIP, nn::load into DeviceHIP and into the CPU device; 3 x 4 predictions (separate process)."""
+    import json
+    import subprocess
+    import sys
+    code = ("import json, sys; sys.path.insert(0, %r); from oracle import drivers as d; "
+            "print(json.dumps([float(v) for v in d._ref_hip_xor_save_load_here(%d, %d, %d, %r, %r)]))"
+            % (os.path.dirname(HERE), hidden1, hidden2, epochs, lr, path))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=600)
+    if out.returncode != 0:
+        raise RuntimeError("nn::save / nn::load on DeviceHIP failed: " + out.stderr[-2000:])
+    return np.array(json.loads(out.stdout.strip().splitlines()[-1]), dtype=np.float32).reshape(3, 4)
+
+
 # ---- transformer (configs[4]) ------------------------------------------------------------------------
 def transformer_param_shapes(layers, d, heads, seq, batch, vocab):
     """Parameter order of aix_amd/csrc/frontend/transformer.hpp."""

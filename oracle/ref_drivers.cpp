@@ -153,6 +153,61 @@ int aixref_xor_hip(int dtype, uint64_t hidden1, uint64_t hidden2, int epochs, fl
         return 0;
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
 }
+
+// nn::save of a model trained on DeviceHIP (the host reads the parameters straight out of device memory), then
+// nn::load into a fresh model on DeviceHIP (the host writes them straight into device memory) and into one on the
+// reference's CPU device; predictions[0..3] trained model, [4..7] reloaded on DeviceHIP, [8..11] reloaded on the CPU.
+int aixref_xor_save_load_hip(uint64_t hidden1, uint64_t hidden2, int epochs, float lr, const char* path, float* predictions)
+{
+    try {
+        const auto F32 = aix::DataType::kFloat32;
+        auto build = [&](aix::nn::Sequential& m) {
+            m.add(aix::nn::Linear(2, hidden1)); m.add(aix::nn::Tanh());
+            m.add(aix::nn::Linear(hidden1, hidden2)); m.add(aix::nn::Tanh());
+            m.add(aix::nn::Linear(hidden2, 1));
+        };
+        auto predict = [&](aix::nn::Sequential& m, aix::Device& dev, float* out) {
+            auto inputs = aix::tensor({0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0}, {4, 2}).to(dev).to(F32);
+            auto y = m.forward(inputs);
+            dev.synchronize();
+            for (int i = 0; i < 4; ++i) out[i] = y.value().data<float>()[i];
+        };
+        aix::hip::DeviceHIP dev;
+        aix::manualSeed(99);
+        aix::nn::Sequential model;
+        build(model);
+        model.to(dev);
+        auto inputs = aix::tensor({0.0, 0.0, 0.0, 1.0, 1.0, 0.0, 1.0, 1.0}, {4, 2}).to(dev).to(F32);
+        auto targets = aix::tensor({0.0, 1.0, 1.0, 0.0}, {4, 1}).to(dev).to(F32);
+        aix::optim::Adam optimizer(model.parameters(), lr);
+        auto lossFunc = aix::nn::MSELoss();
+        for (int epoch = 0; epoch < epochs; ++epoch) {
+            auto loss = lossFunc(model.forward(inputs), targets);
+            optimizer.zeroGrad();
+            loss.backward();
+            optimizer.step();
+        }
+        dev.synchronize();
+        predict(model, dev, predictions);
+        aix::nn::save(model, path);
+
+        aix::manualSeed(7);                                     // different initial values: everything must come from the file
+        aix::nn::Sequential onGpu;
+        build(onGpu);
+        onGpu.to(dev);
+        dev.synchronize();
+        aix::nn::load(onGpu, path);
+        predict(onGpu, dev, predictions + 4);
+
+        aix::DeviceCPU cpu;
+        aix::nn::Sequential onCpu;
+        build(onCpu);
+        onCpu.to(cpu);
+        aix::nn::load(onCpu, path);
+        predict(onCpu, cpu, predictions + 8);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
 #endif
 
 } // extern "C"

@@ -55,3 +55,16 @@ def test_reference_xor_example_runs_unchanged_on_device_hip(dtype, first, tol):
         want = np.array([0.0, 1.0, 1.0, 0.0])
         assert cpu_losses[-1] < 1e-3 and gpu_losses[-1] < 1e-3
         assert np.abs(cpu_pred - want).max() < 5e-2 and np.abs(gpu_pred - want).max() < 5e-2
+
+
+def test_reference_save_and_load_through_device_memory(tmp_path):
+    """nn::save reads the parameters of a model trained on DeviceHIP straight out of device memory and
+    nn::load writes them straight into it (aixNeuralNetwork.hpp:258-301): a fresh model on DeviceHIP
+    loaded from the file predicts bit for bit what the trained one does, one on the reference's CPU
+    device the same within f32 rounding of tanh."""
+    preds = OD.ref_hip_xor_save_load(64, 32, 300, 0.01, str(tmp_path / "xor.bin"))
+    trained, on_gpu, on_cpu = preds
+    print("trained", trained, "reloaded on DeviceHIP", on_gpu, "reloaded on the CPU device", on_cpu)
+    assert trained.view(np.uint32).tolist() == on_gpu.view(np.uint32).tolist()
+    assert np.abs(on_cpu - trained).max() <= 1e-5
+    assert np.abs(trained - np.array([0.0, 1.0, 1.0, 0.0])).max() < 5e-2
