@@ -1,0 +1,181 @@
+"""The benchmark's own sizes through size-independent properties.
+
+The element-by-element oracle comparisons of test_gpu_kernels.py run at sizes the CPU oracle finishes in
+seconds.  Here the kernels run at the sizes the benchmark quotes -- [8192, 8192] f32 for the reductions,
+the broadcast add and the transpose copy, 4096^3 (and one 8192^3) for the matmuls -- and are checked
+with what the mathematics fixes at any size:
+
+  * exact operators (max, argmax, x + v, transpose) against numpy on the same data, bit for bit;
+    transpose twice is the identity;
+  * sums against float64 sums within 1e-5 * sum|x| (the accumulation order is the implementation's);
+  * matmul: C . 1 = A . (B . 1) (a checksum of every element of C, evaluated in float64 from the inputs in
+    O(n^2)), 96 randomly chosen entries against float64 dot products, A . I = A exactly -- for every
+    operand layout the kernels consume in place.
+
+Everything goes through the C ABI of libaixhip_kernels.so."""
+import numpy as np
+import pytest
+
+import aixtest as T
+import gpuharness as G
+from oracle import cpuref as O
+
+pytestmark = pytest.mark.gpu
+NAMES = O.DTYPE_NAMES
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = G.Gpu()
+    yield g
+    g.close()
+    g.ctx.close()
+
+
+@pytest.fixture(scope="module")
+def big():
+    """x [8192, 8192] f32 with many exact ties (quantised to 1/64) and v [8192]."""
+    rng = np.random.default_rng(5150)
+    x = (np.round(rng.uniform(-1, 1, (8192, 8192)) * 64) / 64).astype(np.float32)
+    v = rng.uniform(-1, 1, 8192).astype(np.float32)
+    return x, v
+
+
+def _tensor(arr, dtype, shape, strides=None):
+    return T.HostTensor(arr.reshape(-1), dtype, shape, strides)
+
+
+def test_reductions_at_benchmark_size(gpu, big):
+    x, _ = big
+    R, Cn = x.shape
+    src = _tensor(x, O.F32, [R, Cn])
+    _, ds = gpu.put(src)
+    abs_rows = np.abs(x, dtype=np.float64).sum(axis=1)
+
+    # sum(1): fill(0) + reduceTo into [R, 1]
+    out = T.empty(O.F32, [R, 1], fill=0)
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_reduce_to", 0, G.ref(ds), G.ref(do))
+    got = gpu.fetch(po, out.storage).astype(np.float64)
+    want = x.sum(axis=1, dtype=np.float64)
+    assert np.all(np.abs(got - want) <= 1e-5 * abs_rows + 1e-30), float(np.abs(got - want).max())
+
+    # max(1): lowest + maxTo; exact
+    out = T.empty(O.F32, [R, 1], fill=float(np.finfo(np.float32).min))
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_reduce_to", 1, G.ref(ds), G.ref(do))
+    T.assert_same_bits(gpu.fetch(po, out.storage), x.max(axis=1), "max(1) at [8192, 8192]")
+
+    # argmax(0): the first maximum of every column (the data is full of ties)
+    out = T.empty(O.I32, [1, Cn], fill=-1)
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_argmax_to", 0, G.ref(ds), G.ref(do), 0)
+    T.assert_same_bits(gpu.fetch(po, out.storage), x.argmax(axis=0).astype(np.int32), "argmax(0) at [8192, 8192]")
+
+    # sum(): everything into one element
+    out = T.empty(O.F32, [1], fill=0)
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_reduce_all", 0, G.ref(ds), G.ref(do))
+    got = float(gpu.fetch(po, out.storage)[0])
+    want = float(x.sum(dtype=np.float64))
+    assert abs(got - want) <= 1e-5 * float(abs_rows.sum()), (got, want)
+    gpu.release()
+
+
+def test_broadcast_add_and_transpose_at_benchmark_size(gpu, big):
+    x, v = big
+    R, Cn = x.shape
+    px, dx = gpu.put(_tensor(x, O.F32, [R, Cn]))
+    _, dv = gpu.put(_tensor(v, O.F32, [R, Cn], [0, 1]))              # the row vector read through a stride-0 view
+    out = T.empty(O.F32, [R, Cn])
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_binary", O.ADD, G.ref(dx), G.ref(dv), G.ref(do))
+    T.assert_same_bits(gpu.fetch(po, out.storage), (x + v[None, :]).reshape(-1), "x + v at [8192, 8192]")
+
+    # x.transpose(0, 1).contiguous(): a gather through the transposed view; twice gives x back
+    d_t = G.kdesc(_tensor(x, O.F32, [Cn, R], [1, Cn]), px)             # the transposed view of the device copy of x
+    G.run_gpu(gpu, "aixk_contiguous", G.ref(d_t), G.ref(do))
+    once = gpu.fetch(po, out.storage)
+    T.assert_same_bits(once, np.ascontiguousarray(x.T).reshape(-1), "transpose copy at [8192, 8192]")
+    pb, db = gpu.put(T.empty(O.F32, [R, Cn]))
+    d_tt = G.kdesc(_tensor(x, O.F32, [R, Cn], [1, R]), po)             # the transposed view of the transposed copy
+    G.run_gpu(gpu, "aixk_contiguous", G.ref(d_tt), G.ref(db))
+    T.assert_same_bits(gpu.fetch(pb, out.storage), x.reshape(-1), "transpose twice")
+    gpu.release()
+
+
+def _matmul_properties(gpu, dtype, n, layout, rng, tol_rel):
+    """A [n, n] . B [n, n] with A and / or B held transposed in memory (layout 'NN', 'NT', 'TN', 'TT':
+    T = the operand is stored as its transpose and read through a transposed view)."""
+    scale = 1.0 / np.sqrt(n)
+    a_store = O.to_storage(rng.uniform(-scale, scale, n * n), dtype)
+    b_store = O.to_storage(rng.uniform(-1, 1, n * n), dtype)
+    a_t, b_t = layout[0] == "T", layout[1] == "T"
+    # logical A[i, k]: stored row-major, or stored as [k, i] and viewed with strides (1, n)
+    A = O.to_float64(a_store, dtype).reshape(n, n)
+    B = O.to_float64(b_store, dtype).reshape(n, n)
+    if a_t:
+        A = A.T
+    if b_t:
+        B = B.T
+    ha = T.HostTensor(a_store, dtype, [n, n], [1, n] if a_t else None)
+    hb = T.HostTensor(b_store, dtype, [n, n], [1, n] if b_t else None)
+    _, da = gpu.put(ha)
+    _, db = gpu.put(hb)
+    out = T.empty(dtype, [n, n])
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+    Cg = O.to_float64(gpu.fetch(po, out.storage), dtype).reshape(n, n)
+
+    # checksum of every element: C . 1 = A . (B . 1); bound = rounding of the output type on sum_j |C_ij| plus
+    # the accumulation bound on |A| . (|B| . 1)
+    eps_out = {O.F32: 2.0 ** -24, O.F16: 2.0 ** -11, O.BF16: 2.0 ** -8}[dtype]
+    want_rows = A @ B.sum(axis=1)
+    mag_rows = np.abs(A) @ np.abs(B).sum(axis=1)
+    got_rows = Cg.sum(axis=1)
+    bound = eps_out * np.abs(Cg).sum(axis=1) + tol_rel * mag_rows
+    bad = np.abs(got_rows - want_rows) > bound
+    assert not bad.any(), f"{NAMES[dtype]} {n}^3 {layout}: row checksum off by {float(np.abs(got_rows - want_rows).max())} (bound {float(bound.min())})"
+    # the same over columns catches a transposed or permuted result that keeps the row sums
+    want_cols = A.sum(axis=0) @ B
+    got_cols = Cg.sum(axis=0)
+    mag_cols = np.abs(A).sum(axis=0) @ np.abs(B)
+    bound = eps_out * np.abs(Cg).sum(axis=0) + tol_rel * mag_cols
+    assert np.all(np.abs(got_cols - want_cols) <= bound), f"{NAMES[dtype]} {n}^3 {layout}: column checksum"
+    # single entries against float64 dot products
+    idx = rng.integers(0, n, size=(96, 2))
+    for i, j in idx:
+        want = float(A[i, :] @ B[:, j])
+        mag = float(np.abs(A[i, :]) @ np.abs(B[:, j]))
+        assert abs(Cg[i, j] - want) <= eps_out * abs(want) + tol_rel * mag + 1e-30, (layout, int(i), int(j), Cg[i, j], want)
+    gpu.release()
+
+
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN", "TT"])
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=lambda d: NAMES[d])
+def test_matmul_4096_cubed_16bit(gpu, dtype, layout):
+    _matmul_properties(gpu, dtype, 4096, layout, np.random.default_rng(6000 + dtype), 1e-5)
+
+
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+def test_matmul_4096_cubed_f32(gpu, layout):
+    _matmul_properties(gpu, O.F32, 4096, layout, np.random.default_rng(6100), 1e-5)
+
+
+def test_matmul_8192_cubed_bf16(gpu):
+    _matmul_properties(gpu, O.BF16, 8192, "NN", np.random.default_rng(6200), 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16], ids=lambda d: NAMES[d])
+def test_matmul_identity_at_4096(gpu, dtype):
+    """A . I == A exactly at the benchmark size (every product is a * 1 or a * 0, every sum exact)."""
+    n = 4096
+    rng = np.random.default_rng(6300 + dtype)
+    a = T.HostTensor(O.to_storage(rng.uniform(-1, 1, n * n), dtype), dtype, [n, n])
+    eye = T.HostTensor(O.to_storage(np.eye(n).reshape(-1), dtype), dtype, [n, n])
+    _, da = gpu.put(a)
+    _, de = gpu.put(eye)
+    po, do = gpu.put(T.empty(dtype, [n, n]))
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(de), G.ref(do))
+    T.assert_same_bits(gpu.fetch(po, a.storage), a.storage, f"A.I {NAMES[dtype]} at 4096")
+    gpu.release()
