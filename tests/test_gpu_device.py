@@ -103,10 +103,10 @@ def build_config0(rec, a, b, c):
     return y, t7
 
 
-def test_config0_chain_is_one_fused_kernel(dev):
+@pytest.mark.parametrize("shape", [[1024, 1024], [4096, 4096]], ids=["1024", "benchmark-size"])
+def test_config0_chain_is_one_fused_kernel(dev, shape):
     set_diag(dev)
     rng = np.random.default_rng(0)
-    shape = [1024, 1024]
     rec = Recorder(dev, O.F32, shape)
     a, b, c = (rec.leaf(T.contiguous_tensor(rng, O.F32, shape)) for _ in range(3))
     y, t7 = build_config0(rec, a, b, c)
