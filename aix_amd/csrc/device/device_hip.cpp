@@ -538,6 +538,11 @@ void DeviceHIP::emitSingle(const OpRecord& op)
     markTouched(op.input0.data);
     if (op.hasInput1) markTouched(op.input1.data);
     toPod(op.output, &o);
+    if (op.type == OpType::Cast) {
+        check(aixk_cast(m_ctx, (const char*)op.input0.data + op.input0.offset * dataTypeSize(op.input0.dtype), (int)op.input0.dtype,
+                        (char*)op.output.data + op.output.offset * dataTypeSize(op.output.dtype), (int)op.output.dtype, op.output.size));
+        return;
+    }
     if (op.type == OpType::Fill) { check(aixk_fill(m_ctx, op.scalarData.data(), (int)op.scalarDType, &o)); return; }
     if (op.type == OpType::FillMin) { check(aixk_fill_min(m_ctx, &o)); return; }
     toPod(op.input0, &a);
@@ -614,7 +619,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         bool ok = outsAligned;
         for (size_t k = 0; k < NI && ok; ++k) {
             const uint64_t s = cr ? str[k][0] : 0;
-            const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+            const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * dataTypeSize(d.inputBuffers[k].dtype);
             if (cr == 1 && s == 0) { if (k < 32) bmask |= 1u << k; else ok = false; }
             else if (cr == 1 && s != 1) ok = false;
             else if (!aligned(base)) ok = false;
@@ -627,7 +632,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
             const uint64_t s = str[k][cr - 1];
             if (s > 1) ok = false;
             if (s == 1) {
-                const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+                const char* base = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * dataTypeSize(d.inputBuffers[k].dtype);
                 if (!aligned(base)) ok = false;
                 for (size_t dd = 0; dd + 1 < cr; ++dd) if (str[k][dd] % VEC) ok = false;
             }
@@ -638,7 +643,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     auto& ex = *m_extras;
     gen::Space& space = ex.space;
     if (shape == gen::Shape::Flat) {
-        for (size_t k = 0; k < NI; ++k) inPtr[k] = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * esz;
+        for (size_t k = 0; k < NI; ++k) inPtr[k] = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * dataTypeSize(d.inputBuffers[k].dtype);
     } else {
         space.rank = (uint32_t)cr;
         for (int dd = 0; dd < gen::kMaxDims; ++dd) space.shape[dd] = dd < (int)cr ? shp[dd] : 1;
@@ -730,6 +735,20 @@ void DeviceHIP::copy(const void* src, DataType srcDType, void* dst, DataType dst
 {
     if (size == 0) return;
     if (!findBlock(dst)) throw std::invalid_argument("DeviceHIP::copy() result must have GPU memory.");        // aixDeviceMetal.cpp:714-715
+    // Both ends whole device blocks: the conversion is recorded and fuses into the kernel that produces its
+    // operand (converted at the store) or into the one that consumes its result (converted at the load).
+    // The planner tells buffers apart by base address, so pointers into the middle of a block run at once.
+    {
+        const Block* sb = m_blocks.find(src);
+        const Block* db = m_blocks.find(dst);
+        if (sb && db && !sb->freed && !db->freed && src != dst) {
+            View in, out;
+            in.data = const_cast<void*>(src); in.dtype = srcDType; in.rank = 1; in.shape[0] = size; in.strides[0] = 1; in.size = size;
+            out.data = dst; out.dtype = dstDType; out.rank = 1; out.shape[0] = size; out.strides[0] = 1; out.size = size;
+            m_engine->record(OpType::Cast, in, out);
+            return;
+        }
+    }
     flushFor(src, dst);
     const size_t srcBytes = size * dataTypeSize(srcDType);
     if (!findBlock(src)) {

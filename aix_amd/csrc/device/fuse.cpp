@@ -215,6 +215,14 @@ bool sameView(const View& a, const View& b)
 
 bool isDense(const View& p) { return p.dense; }
 
+// The same elements in the same flat order: identical views, or two dense views of one buffer that
+// start at the same element and have the same count (a [rows, cols] result read back as [rows * cols]).
+bool sameElements(const View& a, const View& b)
+{
+    if (sameView(a, b)) return true;
+    return a.dense && b.dense && a.data == b.data && a.dtype == b.dtype && a.offset == b.offset && a.size == b.size;
+}
+
 // One past the last element position the view touches.
 size_t viewEnd(const View& p)
 {
@@ -300,7 +308,7 @@ public:
         for (size_t i = 0; i < ops.size(); ++i) {
             const auto& op = ops[i];
             if (op.type == OpType::Fill || op.type == OpType::FillMin) placeFill(i);
-            else if (isElementwiseOp(op.type) && op.type != OpType::Cast && m_cfg.elementwiseFusion) placeOp(i);
+            else if (isElementwiseOp(op.type) && m_cfg.elementwiseFusion) placeOp(i);
             else placeSingle(i);
         }
         for (size_t g = 0; g < m_groupCount; ++g) closeGroup(g);
@@ -455,6 +463,12 @@ private:
         const auto& op = at(i);
         const bool binary = op.hasInput1;
         const View* in[2] = {&op.input0, binary ? &op.input1 : nullptr};
+        // A cast changes the element type between its operand and its result.  Kernels compute in ONE
+        // type and convert at their loads and stores, so a cast is fused at one of its two ends: it
+        // joins the kernel that holds its operand in a register as a last step (the value is stored
+        // converted; nothing in that kernel may use it further), or it starts / joins a kernel of
+        // its result type whose load of the operand converts.
+        const bool isCast = op.type == OpType::Cast;
 
         if (!m_cfg.supportsStridedFusion) {
             const bool dense = isDense(op.output) && (!in[0]->data || isDense(*in[0])) && (!in[1] || !in[1]->data || isDense(*in[1]));
@@ -472,8 +486,9 @@ private:
                 resolved[k] = Operand{};
                 if (!in[k] || !in[k]->data) continue;
                 // an unmaterialised fill covering everything the view can touch -> immediate
+                // (not for a cast: the immediate would skip the rounding to the fill's own type)
                 if (const PendingFill* f = findFill(in[k]->data)) {
-                    if (in[k]->dtype == at(f->op).output.dtype && viewEnd(*in[k]) <= f->size) {
+                    if (!isCast && in[k]->dtype == at(f->op).output.dtype && viewEnd(*in[k]) <= f->size) {
                         resolved[k] = Operand{Operand::kScalar, f->op};
                         continue;
                     }
@@ -484,7 +499,7 @@ private:
                     if (!m_groups[g].open) continue;
                     const size_t def = findDef(m_groups[g], in[k]->data);
                     if (def == SIZE_MAX) continue;
-                    const bool usable = sameView(defView(def), *in[k]) && compatible(m_groups[g], op);
+                    const bool usable = sameElements(defView(def), *in[k]) && compatible(m_groups[g], op, in[k]->dtype);
                     if (usable && (target == SIZE_MAX || target == g)) {
                         resolved[k] = Operand{Operand::kValue, def};
                         target = g;
@@ -504,7 +519,7 @@ private:
             // no producer inside the window: share loads with an open group of the same shape
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
                 for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
-                    if (!m_groups[g].open || !compatible(m_groups[g], op)) continue;
+                    if (!m_groups[g].open || !compatible(m_groups[g], op, op.output.dtype)) continue;
                     for (int k = 0; k < 2; ++k)
                         if (resolved[k].kind == Operand::kMemory && loads(m_groups[g], *in[k])) target = g;
                 }
@@ -533,6 +548,7 @@ private:
             fresh.shape = &op.output;
         }
         Group& g = m_groups[target];
+        adoptShape(g, op);
         for (int k = 0; k < 2; ++k) {
             m_operands[i][k] = resolved[k];
             if (resolved[k].kind == Operand::kMemory) {
@@ -563,21 +579,33 @@ private:
         return false;
     }
 
-    // Same element type and iteration space: identical shape, or equal element counts when both
-    // sides only touch dense views (then the flat index is all that matters).
-    bool compatible(const Group& g, const OpRecord& op) const
+    // `type` is the element type the operator would compute in inside the group: its result type, or for
+    // a cast that takes a register value the operand's type.
+    // Strided views are bound to the shape they were made for; dense views (and every result) only need
+    // the element count, since the flat index is all that matters for them.  So with different shapes the
+    // two can still share a kernel if one side is all dense: a dense operator rides on the group's shape,
+    // a dense group adopts the shape of an operator that brings strided views (see adoptShape()).
+    static bool denseOperands(const OpRecord& op)
     {
-        if (g.dtype != op.output.dtype || g.count != op.output.size) return false;
+        return isDense(op.output) && (!op.input0.data || isDense(op.input0)) && (!op.hasInput1 || !op.input1.data || isDense(op.input1));
+    }
+
+    bool compatible(const Group& g, const OpRecord& op, DataType type) const
+    {
+        if (g.dtype != type || g.count != op.output.size) return false;
         if (g.shape->sameShape(op.output)) return true;
-        const bool opDense = isDense(op.output) && (!op.input0.data || isDense(op.input0)) &&
-                             (!op.hasInput1 || !op.input1.data || isDense(op.input1));
-        return g.dense && opDense;
+        return g.dense || denseOperands(op);
+    }
+
+    static void adoptShape(Group& g, const OpRecord& op)
+    {
+        if (!g.shape->sameShape(op.output) && !denseOperands(op)) g.shape = &op.output;      // g.dense held, or compatible() had refused
     }
 
     bool mergeable(const Group& a, const Group& b) const
     {
         if (a.dtype != b.dtype || a.count != b.count) return false;
-        if (!a.shape->sameShape(*b.shape) && !(a.dense && b.dense)) return false;
+        if (!a.shape->sameShape(*b.shape) && !a.dense && !b.dense) return false;
         size_t count = a.loads.size();
         for (const ViewRef& r : b.loads) if (!loads(a, view(r))) ++count;
         return count + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;
@@ -593,6 +621,7 @@ private:
         a.ops.assign(m_merged.begin(), m_merged.end());
         for (size_t def : b.defs) a.defs.push_back(def);
         for (const ViewRef& r : b.loads) if (!loads(a, view(r))) a.loads.push_back(r);
+        if (!a.shape->sameShape(*b.shape) && !b.dense) a.shape = b.shape;        // a is all dense then: it adopts the shape b's strided views need
         a.dense = a.dense && b.dense;
         a.hasScalar = a.hasScalar || b.hasScalar;
         for (size_t w : b.ops) m_groupOf[w] = into;

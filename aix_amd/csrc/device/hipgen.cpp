@@ -66,15 +66,19 @@ std::string operandText(const FusedSubgraphDescriptor& d, size_t tensorIndex, si
     throw std::invalid_argument("fused operator without an operand");
 }
 
-// The per-element SSA body shared by the vector loop and the tails.
+// The per-element SSA body shared by the vector loop and the tails.  Every value has the kernel's
+// one element type T: loads convert to it and stores convert from it, so a cast is the identity here.
 void emitBody(std::ostringstream& o, const FusedSubgraphDescriptor& d)
 {
     o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out)\n{\n";
     for (size_t k = 0; k < d.ops.size(); ++k) {
         const auto& op = d.ops[k];
-        o << "    const T v" << k << " = " << fnName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
-        if (isBinary(op.type)) o << ", " << operandText(d, op.inputIndex1, op.scalarIndex1);
-        o << ");\n";
+        if (op.type == OpType::Cast) o << "    const T v" << k << " = " << operandText(d, op.inputIndex0, op.scalarIndex0) << ";\n";
+        else {
+            o << "    const T v" << k << " = " << fnName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
+            if (isBinary(op.type)) o << ", " << operandText(d, op.inputIndex1, op.scalarIndex1);
+            o << ");\n";
+        }
         if (op.outputIndex != SIZE_MAX) o << "    out[" << op.outputIndex << "] = v" << k << ";\n";
     }
     o << "}\n\n";
@@ -114,6 +118,11 @@ void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape
     s += "|i"; appendNumber(s, d.inputBuffers.size());
     s += 'o';  appendNumber(s, d.outputBuffers.size());
     s += 's';  appendNumber(s, scalarCount(d));
+    // buffers of another element type than the kernel's (fused casts): part of the identity
+    for (size_t k = 0; k < d.inputBuffers.size(); ++k)
+        if (d.inputBuffers[k].dtype != d.dtype) { s += "|x"; appendNumber(s, k); s += ':'; s += shortType(d.inputBuffers[k].dtype); }
+    for (size_t k = 0; k < d.outputBuffers.size(); ++k)
+        if (d.outputBuffers[k].dtype != d.dtype) { s += "|y"; appendNumber(s, k); s += ':'; s += shortType(d.outputBuffers[k].dtype); }
     for (const auto& op : d.ops) {
         s += '|'; s += fuse::opName(op.type); s += '(';
         appendOperand(s, d, op.inputIndex0, op.scalarIndex0);
@@ -141,11 +150,19 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
       << "// " << signature(d, shape, broadcastMask, noAlias) << "\n"
       << "typedef " << typeName(d.dtype) << " T;\n"
       << "typedef " << wordName(esz) << " word_t;\n"
-      << "typedef vec16<T>::type V;\n"
-      << "#define VEC (vec16<T>::n)\n#define NI " << NI << "\n#define NO " << NO << "\n#define NS " << NS << "\n\n";
+      << "#define VEC (vec16<T>::n)\n#define NI " << NI << "\n#define NO " << NO << "\n#define NS " << NS << "\n";
+    // Buffers carry their own element type (a fused cast makes it differ from T): loads convert to T,
+    // stores convert from it.  Same type: the bits pass through untouched.
+    for (size_t k = 0; k < NI; ++k) o << "typedef " << typeName(d.inputBuffers[k].dtype) << " I" << k << ";\n";
+    for (size_t k = 0; k < NO; ++k) o << "typedef " << typeName(d.outputBuffers[k].dtype) << " O" << k << ";\n";
+    o << "\n";
+    auto in_same = [&](size_t k) { return d.inputBuffers[k].dtype == d.dtype; };
+    auto out_same = [&](size_t k) { return d.outputBuffers[k].dtype == d.dtype; };
+    auto to_t = [&](size_t k, const std::string& e) { return in_same(k) ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
+    auto from_t = [&](size_t k, const std::string& e) { return out_same(k) ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
     emitBody(o, d);
 
-    o << "struct Args {\n    const T* in[" << AI << "];\n    T* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 n;\n";
+    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 n;\n";
     if (shape != Shape::Flat) o << "    u64 chunks;\n    u64 rank;\n    u64 shape[" << kMaxDims << "];\n    u64 off[" << AI << "];\n    u64 str[" << AI << "][" << kMaxDims << "];\n";
     o << "};\n\n";
 
@@ -153,30 +170,32 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
+    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = (const I" << k << "*)a.in[" << k << "];\n";
+    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = (O" << k << "*)a.out[" << k << "];\n";
 
     if (shape == Shape::Flat) {
-        // One 16-byte vector per operand per lane and as many workgroups as there are vectors:
-        // the hardware overlaps the groups' load and compute phases far better than a long
-        // per-lane loop does (measured: 87 % of HBM peak for a 3-load / 1-store tanh+exp+div body).
+        // One vector of VEC elements per operand per lane (16 bytes of T) and as many workgroups as
+        // there are vectors: the hardware overlaps the groups' load and compute phases far better than
+        // a long per-lane loop does (measured: 87 % of HBM peak for a 3-load / 1-store tanh+exp+div body).
         const char* rs = noAlias ? " __restrict__" : "";
         auto bc = [&](size_t k) { return ((broadcastMask >> k) & 1u) != 0; };
         for (size_t k = 0; k < NI; ++k) {
-            if (bc(k)) o << "    const T b" << k << " = a.in[" << k << "][0];\n";
-            else o << "    const V*" << rs << " p" << k << " = (const V*)a.in[" << k << "];\n";
+            if (bc(k)) o << "    const T b" << k << " = " << to_t(k, "in" + std::to_string(k) + "[0]") << ";\n";
+            else o << "    const vec<I" << k << ", VEC>*" << rs << " p" << k << " = (const vec<I" << k << ", VEC>*)in" << k << ";\n";
         }
-        for (size_t k = 0; k < NO; ++k) o << "    V*" << rs << " q" << k << " = (V*)a.out[" << k << "];\n";
+        for (size_t k = 0; k < NO; ++k) o << "    vec<O" << k << ", VEC>*" << rs << " q" << k << " = (vec<O" << k << ", VEC>*)out" << k << ";\n";
         o << "    const u64 nvec = a.n / VEC;\n"
           << "    for (u64 v = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; v < nvec; v += (u64)gridDim.x * " << kBlock << ") {\n";
-        for (size_t k = 0; k < NI; ++k) if (!bc(k)) o << "        const V r" << k << " = p" << k << "[v];\n";
-        for (size_t k = 0; k < NO; ++k) o << "        V w" << k << ";\n";
+        for (size_t k = 0; k < NI; ++k) if (!bc(k)) o << "        const vec<I" << k << ", VEC> r" << k << " = p" << k << "[v];\n";
+        for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
         o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
         for (size_t k = 0; k < NI; ++k) {
             if (bc(k)) o << "            x[" << k << "] = b" << k << ";\n";
-            else o << "            x[" << k << "] = r" << k << ".v[e];\n";
+            else o << "            x[" << k << "] = " << to_t(k, "r" + std::to_string(k) + ".v[e]") << ";\n";
         }
         if (NI == 0) o << "            x[0] = zero<T>();\n";
         o << "            aix_body(x, s, y);\n";
-        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = y[" << k << "];\n";
+        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
         for (size_t k = 0; k < NO; ++k) o << "        q" << k << "[v] = w" << k << ";\n";
         o << "    }\n"
@@ -184,11 +203,11 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
           << "    if (blockIdx.x == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
         for (size_t k = 0; k < NI; ++k) {
             if (bc(k)) o << "        x[" << k << "] = b" << k << ";\n";
-            else o << "        x[" << k << "] = a.in[" << k << "][i];\n";
+            else o << "        x[" << k << "] = " << to_t(k, "in" + std::to_string(k) + "[i]") << ";\n";
         }
         if (NI == 0) o << "        x[0] = zero<T>();\n";
         o << "        aix_body(x, s, y);\n";
-        for (size_t k = 0; k < NO; ++k) o << "        a.out[" << k << "][i] = y[" << k << "];\n";
+        for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "    }\n}\n";
         return o.str();
     }
@@ -204,18 +223,18 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
         o << "            row = q;\n        }\n";
         for (size_t k = 0; k < NI; ++k) {
-            o << "        V r" << k << ";\n"
-              << "        if (a.str[" << k << "][inner] == 0) { const T t = a.in[" << k << "][p[" << k << "]];\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r" << k << ".v[e] = t; }\n"
-              << "        else r" << k << " = *(const V*)(a.in[" << k << "] + p[" << k << "] + col);\n";
+            o << "        vec<I" << k << ", VEC> r" << k << ";\n"
+              << "        if (a.str[" << k << "][inner] == 0) { const I" << k << " t = in" << k << "[p[" << k << "]];\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r" << k << ".v[e] = t; }\n"
+              << "        else r" << k << " = *(const vec<I" << k << ", VEC>*)(in" << k << " + p[" << k << "] + col);\n";
         }
-        for (size_t k = 0; k < NO; ++k) o << "        V w" << k << ";\n";
+        for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
         o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
-        for (size_t k = 0; k < NI; ++k) o << "            x[" << k << "] = r" << k << ".v[e];\n";
+        for (size_t k = 0; k < NI; ++k) o << "            x[" << k << "] = " << to_t(k, "r" + std::to_string(k) + ".v[e]") << ";\n";
         if (NI == 0) o << "            x[0] = zero<T>();\n";
         o << "            aix_body(x, s, y);\n";
-        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = y[" << k << "];\n";
+        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
-        for (size_t k = 0; k < NO; ++k) o << "        *(V*)(a.out[" << k << "] + c * VEC) = w" << k << ";\n";
+        for (size_t k = 0; k < NO; ++k) o << "        *(vec<O" << k << ", VEC>*)(out" << k << " + c * VEC) = w" << k << ";\n";
         o << "    }\n}\n";
         return o.str();
     }
@@ -227,10 +246,10 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     o << "        for (int d = (int)a.rank - 1; d >= 0; --d) {\n            const u64 q = rest / a.shape[d], r = rest - q * a.shape[d];\n";
     for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
     o << "            rest = q;\n        }\n        T x[" << AI << "], y[" << NO << "];\n";
-    for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = a.in[" << k << "][p[" << k << "]];\n";
+    for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = " << to_t(k, "in" + std::to_string(k) + "[p[" + std::to_string(k) + "]]") << ";\n";
     if (NI == 0) o << "        x[0] = zero<T>();\n";
     o << "        aix_body(x, s, y);\n";
-    for (size_t k = 0; k < NO; ++k) o << "        a.out[" << k << "][i] = y[" << k << "];\n";
+    for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
     o << "    }\n}\n";
     return o.str();
 }

@@ -495,6 +495,98 @@ static void testTrailingFillIsHandedOver()
     e.flush();
 }
 
+static void testCastsFuseAtTheirLoadOrStoreEnd()
+{
+    const aix::Shape shape{128, 96};
+    const size_t n = 128 * 96;
+    // (a * b) converted to bf16: the conversion joins the kernel that holds the product in a register
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto a = T(1, shape), b = T(2, shape), t = T(3, shape);
+        auto flat = T(3, {n}), out = T(4, {n}, DataType::kBFloat16);
+        for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        e.record(OpType::Mul, a, b, t);
+        e.record(OpType::Cast, flat, out);
+        e.releaseBuffer(reinterpret_cast<void*>(3 * 0x10000));
+        e.flush();
+        CHECK(cap.singles.empty() && cap.fused.size() == 1);
+        if (cap.fused.size() == 1) {
+            const auto& d = cap.fused[0];
+            CHECK(d.dtype == DataType::kFloat32 && d.ops.size() == 2 && d.inputBuffers.size() == 2 && d.outputBuffers.size() == 1);
+            CHECK(d.outputBuffers[0].dtype == DataType::kBFloat16 && d.outputBuffers[0].data == out.data);
+            CHECK(compiles(d, gen::Shape::Flat) && compiles(d, gen::Shape::Rows) && compiles(d, gen::Shape::Gather));
+            CHECK(gen::signature(d, gen::Shape::Flat).find("|y0:bf16") != std::string::npos);
+        }
+    }
+    // an int32 mask converted to f32 and multiplied: the conversion happens at the load of the kernel that multiplies
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto mask = T(1, {n}, DataType::kInt32), asFloat = T(2, {n}), asFloat2d = T(2, shape), g = T(3, shape), y = T(4, shape);
+        for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        e.record(OpType::Cast, mask, asFloat);
+        e.record(OpType::Mul, asFloat2d, g, y);
+        e.releaseBuffer(reinterpret_cast<void*>(2 * 0x10000));
+        e.flush();
+        CHECK(cap.singles.empty() && cap.fused.size() == 1);
+        if (cap.fused.size() == 1) {
+            const auto& d = cap.fused[0];
+            CHECK(d.dtype == DataType::kFloat32 && d.ops.size() == 2 && d.outputBuffers.size() == 1);
+            CHECK(d.inputBuffers.size() == 2 && d.inputBuffers[0].dtype == DataType::kInt32 && d.inputBuffers[1].dtype == DataType::kFloat32);
+            CHECK(compiles(d, gen::Shape::Flat) && compiles(d, gen::Shape::Rows) && compiles(d, gen::Shape::Gather));
+        }
+    }
+    // the converted value read again in its new type: a second kernel, after the first; a fill is never an
+    // immediate of a cast (its rounding to the fill's own type would be lost)
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto a = T(1, {n}), h = T(2, {n}, DataType::kFloat16), h2 = T(3, {n}, DataType::kFloat16), c = T(5, {n}, DataType::kFloat16), cf = T(6, {n});
+        for (uintptr_t id : {1, 2, 3, 5, 6}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        const float tenth = 0.1f;
+        e.record(OpType::Exp, a, a);                 // in place, f32
+        e.record(OpType::Cast, a, h);                // joins as the last step of that kernel
+        e.record(OpType::Add, h, h, h2);             // f16: must load h from memory
+        e.recordFill(&tenth, DataType::kFloat32, c); // f16 tensor filled with 0.1
+        e.record(OpType::Cast, c, cf);               // f16 -> f32: needs the rounded value
+        e.flush();
+        CHECK(cap.order.size() == 4 && cap.order[0] == "F0");
+        CHECK(cap.fused.size() == 1 && cap.singles.size() == 3);
+        if (cap.fused.size() == 1) {
+            CHECK(cap.fused[0].dtype == DataType::kFloat32 && cap.fused[0].ops.size() == 2 && cap.fused[0].outputBuffers.size() == 2);
+            CHECK(cap.fused[0].outputBuffers[1].dtype == DataType::kFloat16);
+        }
+        if (cap.singles.size() == 3) {                    // a lone operator runs as the plain operator
+            CHECK(cap.singles[0].type == OpType::Fill && cap.singles[1].type == OpType::Add && cap.singles[2].type == OpType::Cast);
+            CHECK(cap.singles[1].input0.data == h.data && cap.singles[2].input0.dtype == DataType::kFloat16);
+        }
+    }
+    // every pair of element types, at the load and at the store
+    const DataType all[] = {DataType::kFloat64, DataType::kFloat32, DataType::kFloat16, DataType::kBFloat16, DataType::kInt64,
+                            DataType::kInt32, DataType::kInt16, DataType::kInt8, DataType::kUInt8};
+    int built = 0;
+    for (DataType from : all)
+        for (DataType to : all) {
+            if (from == to) continue;
+            Capture cap;
+            FuseEngine e(config(), cap.callbacks());
+            auto x = T(1, {n}, from), xt = T(2, {n}, to), y = T(3, {n}, to), back = T(4, {n}, from);
+            for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+            e.record(OpType::Cast, x, xt);           // load end
+            e.record(OpType::Add, xt, xt, y);
+            e.record(OpType::Cast, y, back);         // store end
+            e.releaseBuffer(reinterpret_cast<void*>(2 * 0x10000));
+            e.flush();
+            if (cap.fused.size() != 1 || !cap.singles.empty()) { CHECK(false); continue; }
+            const auto& d = cap.fused[0];
+            if (!(d.dtype == to && d.ops.size() == 3 && d.outputBuffers.size() == 2)) { CHECK(false); continue; }
+            if (!compiles(d, gen::Shape::Flat) || !compiles(d, gen::Shape::Gather)) { CHECK(false); continue; }
+            ++built;
+        }
+    CHECK(built == 72);
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -519,6 +611,7 @@ int main(int argc, char** argv)
     testViewLimitsAndRoundTrip();
     testEngineStorageIsReusedAcrossWindows();
     testTrailingFillIsHandedOver();
+    testCastsFuseAtTheirLoadOrStoreEnd();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

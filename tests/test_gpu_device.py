@@ -315,6 +315,8 @@ def test_1024_chained_in_place_adds_without_sync(dev):
 
 def test_temporaries_are_recycled(dev):
     """A long allocate / compute / free loop without synchronize keeps memory bounded."""
+    dev.dev.synchronize()
+    dev.dev.call("empty_cache")                              # blocks cached by earlier tests do not count
     rng = np.random.default_rng(36000)
     n = 1 << 18
     a = T.contiguous_tensor(rng, O.F32, [n])
@@ -344,6 +346,8 @@ def test_temporaries_are_recycled(dev):
 def test_used_temporaries_are_recycled(dev):
     """The same for temporaries that enqueued work really wrote (an eager operator per iteration):
     they come back once the GPU has passed an event, so 1.6 GiB of them hold a few hundred MiB."""
+    dev.dev.synchronize()
+    dev.dev.call("empty_cache")
     rng = np.random.default_rng(36001)
     rows, cols = 1024, 1024
     a = T.contiguous_tensor(rng, O.F32, [rows, cols])
@@ -393,6 +397,58 @@ def test_interior_pointer_operands(dev):
     got = dev.fetch(out, np.zeros(1, np.float32))
     want = np.float64((lo.storage.astype(np.float64) ** 2).sum())
     assert abs(float(got[0]) - want) <= 1e-5 * want
+    dev.release()
+
+
+def _special_storage(rng, dtype, n):
+    if dtype in T.FLOAT_DTYPES:
+        with np.errstate(over="ignore", invalid="ignore"):
+            vals = np.concatenate([np.array([0.0, -0.0, 1.0, -1.0, 0.5, 255.4, 255.6, -0.4, 300.0, -129.0, 32767.6, -40000.0, 3.0e9, -3.0e9,
+                                             1e19, -1e19, 65504.0, 1e-8, np.inf, -np.inf, np.nan]), rng.uniform(-400, 400, n - 21)])
+            return O.to_storage(vals, dtype)
+    info = np.iinfo(O.NP_STORAGE[dtype])
+    return np.concatenate([np.array([info.min, info.max, 0, 1, 2], dtype=O.NP_STORAGE[dtype]),
+                           rng.integers(info.min, info.max, n - 5, endpoint=True).astype(O.NP_STORAGE[dtype])])
+
+
+@pytest.mark.parametrize("src", T.ALL_DTYPES, ids=lambda d: NAMES[d])
+def test_recorded_casts_fuse_and_keep_the_conversion_rules(dev, src):
+    """Device-to-device copy() is recorded: it runs inside the kernel that consumes its result (converted at
+    the load) or produces its operand (converted at the store).  Every pair of element types, special
+    values included, against the CPU device operator by operator: y = (x.to(D) + x.to(D)).to(S), both
+    intermediate tensors released before the flush, and the plain single cast."""
+    set_diag(dev)
+    rng = np.random.default_rng(37000 + src)
+    n = 2100 + 13                                            # vector body + tail
+    st = _special_storage(rng, src, n)
+    x = T.HostTensor(st, src, [n])
+    px, dx = dev.put(x)
+    for dst in T.ALL_DTYPES:
+        if dst == src:
+            continue
+        what = f"{NAMES[src]} -> {NAMES[dst]}"
+        # CPU: copy, add, copy back
+        xd = T.empty(dst, [n]); yd = T.empty(dst, [n]); back = T.empty(src, [n]); plain = T.empty(dst, [n])
+        assert CPU.copy(st.ctypes.data, src, xd.storage.ctypes.data, dst, n) == 0
+        with np.errstate(all="ignore"):
+            assert CPU.binary(O.ADD, C.byref(xd.desc()), C.byref(xd.desc()), C.byref(yd.desc())) == 0
+        assert CPU.copy(yd.storage.ctypes.data, dst, back.storage.ctypes.data, src, n) == 0
+        # device: the same stream, temporaries freed before anything runs
+        p_xd, p_yd, p_back = dev.raw(xd.storage.nbytes, keep=False), dev.raw(yd.storage.nbytes, keep=False), dev.raw(back.storage.nbytes)
+        dev.dev.call("copy", px, src, p_xd, dst, n)
+        dev.dev.call("add", H.ref(H.kdesc(xd, p_xd)), H.ref(H.kdesc(xd, p_xd)), H.ref(H.kdesc(yd, p_yd)))
+        dev.dev.call("copy", p_yd, dst, p_back, src, n)
+        dev.dev.deallocate(p_xd)
+        dev.dev.deallocate(p_yd)
+        got = dev.fetch(p_back, back.storage)
+        diag = dev.dev.diagnostics()
+        assert diag.fusible_subgraphs == 1 and diag.fused_ops == 3 and diag.fallback_ops == 0, (what, diag.subgraph_summary, diag.fallback_summary)
+        T.assert_same_bits_nan_ok(got, back.storage, src, "fused cast, add, cast back: " + what)
+        # a cast on its own runs as the plain conversion kernel
+        p_plain = dev.raw(plain.storage.nbytes)
+        dev.dev.call("copy", px, src, p_plain, dst, n)
+        got = dev.fetch(p_plain, plain.storage)
+        T.assert_same_bits_nan_ok(got, xd.storage, dst, "single cast: " + what)
     dev.release()
 
 
