@@ -45,7 +45,6 @@ namespace {
 struct Cooling {
     aixk_event* event;
     std::vector<std::pair<void*, size_t>> blocks;
-    size_t bytes{0};
 };
 
 size_t viewEnd(const View& p)
@@ -89,7 +88,6 @@ int unaryCode(OpType t)
 
 struct DeviceHIP::Extras {
     std::deque<Cooling> cooling;
-    size_t coolingBytes{0};
     unsigned flushesSinceEvent{0};
     std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
     uint64_t hits{0}, misses{0};
@@ -262,7 +260,6 @@ void* DeviceHIP::allocateBlock(size_t bytes, bool track)
         int32_t done = 0;
         if (aixk_event_query(m_ctx, ex.cooling.front().event, &done) != AIXK_OK || !done) break;
         for (auto& b : ex.cooling.front().blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
-        ex.coolingBytes -= ex.cooling.front().bytes;
         aixk_event_destroy(m_ctx, ex.cooling.front().event);
         ex.cooling.pop_front();
     }
@@ -351,8 +348,6 @@ void DeviceHIP::releaseLimbo()
     Cooling c{};
     if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
         c.blocks.swap(m_limbo);
-        c.bytes = m_limboBytes;
-        ex.coolingBytes += c.bytes;
         ex.cooling.push_back(std::move(c));
     } else {
         aixk_sync(m_ctx);
@@ -396,7 +391,6 @@ void DeviceHIP::synchronize()
         aixk_event_destroy(m_ctx, c.event);
     }
     ex.cooling.clear();
-    ex.coolingBytes = 0;
     // everything recorded has been enqueued and has finished: blocks freed since the last event are idle too
     for (auto& b : m_limbo) { size_t bytes = 0; m_blocks.erase(b.first, &bytes); m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
     m_limbo.clear();
