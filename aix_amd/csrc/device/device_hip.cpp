@@ -477,6 +477,15 @@ void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const Device
     out.makeDense();                                        // results are written densely from the base pointer
     onDevice(va);
     onDevice(vb);
+    if (va.rank > (uint32_t)gen::kMaxDims || vb.rank > (uint32_t)gen::kMaxDims) {
+        // generated kernels index at most 8 collapsed dimensions; views of higher rank (which may not collapse
+        // that far) run on the precompiled operator, which takes all 16
+        flushFor(va.data, vb.data, out.data);
+        aixhip_tensor pa, pb, po;
+        toPod(va, &pa); toPod(vb, &pb); toPod(out, &po);
+        check(aixk_binary(m_ctx, binaryCode(t), &pa, &pb, &po));
+        return;
+    }
     m_engine->record(t, va, vb, out);
 }
 
@@ -492,6 +501,13 @@ void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceT
     if (!out.sameShape(va)) { out.rank = va.rank; std::memcpy(out.shape, va.shape, va.rank * sizeof(size_t)); }
     out.makeDense();
     onDevice(va);
+    if (va.rank > (uint32_t)gen::kMaxDims) {
+        flushFor(va.data, out.data);
+        aixhip_tensor pa, po;
+        toPod(va, &pa); toPod(out, &po);
+        check(aixk_unary(m_ctx, unaryCode(t), &pa, &po));
+        return;
+    }
     m_engine->record(t, va, out);
 }
 

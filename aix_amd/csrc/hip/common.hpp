@@ -18,7 +18,7 @@
 
 namespace aixk {
 
-constexpr int kMaxDims = 8;              // rank of a collapsed iteration space the kernels accept
+constexpr int kMaxDims = AIXK_MAX_RANK;  // rank of a collapsed iteration space the kernels accept: any view the descriptor can hold
 constexpr int kBlock = 256;              // threads per workgroup: 4 wavefronts of 64
 
 int fail(int code, const char* fmt, ...);
