@@ -203,3 +203,73 @@ def test_rank_16_views_through_the_device(gpu):
         dev.release()
     finally:
         dev.close()
+
+
+def test_more_than_four_giga_elements(gpu):
+    """2^32 + 4099 uint8 elements: every flat index beyond 32 bits.  add, cast, fill, max and the
+    strided gather (a [2, n/2] transpose would not fit the ragged count, so a sliced view: every second
+    element of the first half) against numpy."""
+    n = (1 << 32) + 4099
+    rng = np.random.default_rng(44000)
+    a = rng.integers(0, 256, n, dtype=np.uint8)
+    b = rng.integers(0, 256, n, dtype=np.uint8)
+    pa, pb, po = gpu.raw(n), gpu.raw(n), gpu.raw(n)
+    gpu.ctx.upload(pa, a)
+    gpu.ctx.upload(pb, b)
+    da, db, do = _desc(pa, O.U8, [n]), _desc(pb, O.U8, [n]), _desc(po, O.U8, [n])
+    G.run_gpu(gpu, "aixk_binary", O.ADD, G.ref(da), G.ref(db), G.ref(do))
+    got = np.empty(n, np.uint8)
+    gpu.ctx.download(got, po)
+    want = a + b                                             # uint8 wraps, as the device does
+    assert np.array_equal(got[-8192:], want[-8192:]) and np.array_equal(got[:8192], want[:8192])
+    assert np.array_equal(got, want), "uint8 add beyond 2^32 elements"
+    # max over everything, and with the only 255 placed past the 32-bit boundary
+    a2 = np.minimum(a, 254)
+    a2[(1 << 32) + 77] = 255
+    gpu.ctx.upload(pa, a2)
+    pm = gpu.raw(256)
+    G.run_gpu(gpu, "aixk_reduce_all", 1, G.ref(da), G.ref(_desc(pm, O.U8, [1])))
+    m = np.zeros(1, np.uint8)
+    gpu.ctx.download(m, pm)
+    assert m[0] == 255
+    # cast to int8 over the whole range (integer to integer is the plain C++ conversion: it wraps)
+    G.run_gpu(gpu, "aixk_cast", pa, O.U8, po, O.I8, n)
+    gpu.ctx.download(got, po)
+    assert np.array_equal(got, a2), "u8 -> i8 cast beyond 2^32 elements"
+    # fill, then check both ends and the total
+    seven = np.array([7], np.uint8)
+    G.run_gpu(gpu, "aixk_fill", seven.ctypes.data, O.U8, G.ref(do))
+    gpu.ctx.download(got, po)
+    assert got.min() == 7 and got.max() == 7
+    # strided gather with offsets and strides beyond 32 bits: every second element of the upper half
+    half = n // 2
+    cnt = (n - half) // 2
+    src = _desc(pa, O.U8, [cnt], [2], offset=half)
+    G.run_gpu(gpu, "aixk_contiguous", G.ref(src), G.ref(_desc(po, O.U8, [cnt])))
+    gpu.ctx.download(got, po)
+    assert np.array_equal(got[:cnt], a2[half:half + 2 * cnt:2]), "strided gather beyond 2^32"
+    gpu.release()
+
+
+def test_generated_kernel_beyond_four_giga_elements():
+    """The same count through the lazy device: y = (a + b) * a as one generated kernel on uint8."""
+    import devharness as H
+    dev = H.Dev()
+    try:
+        n = (1 << 32) + 4099
+        rng = np.random.default_rng(44001)
+        a = T.HostTensor(rng.integers(0, 256, n, dtype=np.uint8), O.U8, [n])
+        b = T.HostTensor(rng.integers(0, 256, n, dtype=np.uint8), O.U8, [n])
+        pa, da = dev.put(a)
+        pb, db = dev.put(b)
+        pt, py = dev.raw(n, keep=False), dev.raw(n)
+        dt, dy = H.kdesc(a, pt), H.kdesc(a, py)
+        dev.dev.call("add", H.ref(da), H.ref(db), H.ref(dt))
+        dev.dev.call("mul", H.ref(dt), H.ref(da), H.ref(dy))
+        dev.dev.deallocate(pt)
+        got = dev.fetch(py, a.storage)
+        want = (a.storage + b.storage) * a.storage          # uint8 arithmetic wraps on both sides
+        assert np.array_equal(got, want)
+        dev.release()
+    finally:
+        dev.close()
