@@ -112,6 +112,7 @@ DeviceHIP::Block* DeviceHIP::BlockTable::find(const void* base) const
 DeviceHIP::Block* DeviceHIP::BlockTable::findContaining(const void* p) const
 {
     const uintptr_t a = (uintptr_t)p;
+    if (a < m_lo || a >= m_hi) return nullptr;
     for (const auto& s : m_slots) if (s.key > 1 && a >= s.key && a < s.key + s.block.bytes) return &s.block;
     return nullptr;
 }
@@ -138,6 +139,8 @@ void DeviceHIP::BlockTable::grow()
 void DeviceHIP::BlockTable::insert(void* base, size_t bytes)
 {
     const uintptr_t key = (uintptr_t)base;
+    if (key < m_lo) m_lo = key;
+    if (key + bytes > m_hi) m_hi = key + bytes;
     if ((m_used + 1) * 2 > m_slots.size()) grow();
     const size_t mask = m_slots.size() - 1;
     size_t grave = SIZE_MAX;

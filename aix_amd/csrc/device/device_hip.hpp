@@ -25,6 +25,7 @@
 #include "aix_compat.hpp"
 #include "fuse.hpp"
 
+#include <cstdint>
 #include <memory>
 #include <string>
 #include <unordered_map>
@@ -132,6 +133,7 @@ private:
         std::vector<Slot> m_slots;
         size_t m_count{0}, m_used{0};
         unsigned m_shift{64};
+        uintptr_t m_lo{UINTPTR_MAX}, m_hi{0};                   // every block ever inserted lies in [m_lo, m_hi): host pointers miss at once
     };
 
     const Block* findBlock(const void* p) const;
