@@ -587,6 +587,47 @@ static void testCastsFuseAtTheirLoadOrStoreEnd()
     CHECK(built == 72);
 }
 
+static void testDenseSidesAdoptTheStridedSidesShape()
+{
+    const size_t r = 48, c = 32, n = r * c;
+    auto flat = [&](uintptr_t id) { return T(id, {n}); };
+    auto mat = [&](uintptr_t id) { return T(id, {r, c}); };
+    auto rowOf = [&](uintptr_t id) { return T(id, {r, c}, DataType::kFloat32, {0, 1}); };     // a [c] vector broadcast over rows
+    auto colOf = [&](uintptr_t id) { return T(id, {c, r}, DataType::kFloat32, {0, 1}); };     // another shape with the same count
+    // a dense group opened on a flat view takes on the shape of an operator that brings a broadcast view,
+    // and a [rows, cols] result read back flat is the same register value
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        e.record(OpType::Exp, flat(1), flat(2));                 // dense, shape [n]
+        e.record(OpType::Mul, mat(2), rowOf(3), mat(4));         // reads the flat result as [r, c]; broadcast operand
+        e.record(OpType::Negate, flat(4), flat(5));              // a dense operator rides on the adopted shape
+        e.releaseBuffer(reinterpret_cast<void*>(2 * 0x10000));
+        e.releaseBuffer(reinterpret_cast<void*>(4 * 0x10000));
+        e.flush();
+        CHECK(cap.singles.empty() && cap.fused.size() == 1);
+        if (cap.fused.size() == 1) {
+            const auto& d = cap.fused[0];
+            CHECK(d.ops.size() == 3 && d.inputBuffers.size() == 2 && d.outputBuffers.size() == 1 && !d.allContiguous);
+            CHECK(d.shape == (aix::Shape{r, c}));
+            CHECK(compiles(d, gen::Shape::Rows) && compiles(d, gen::Shape::Gather));
+        }
+    }
+    // two sides that both bring strided views of different shapes cannot share an iteration space
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        for (uintptr_t id : {1, 2, 3, 4, 5, 6}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        e.record(OpType::Add, mat(1), rowOf(2), mat(3));         // bound to [r, c]
+        e.record(OpType::Mul, T(3, {c, r}), colOf(4), T(5, {c, r}));   // the dense result viewed as [c, r], with a [c, r] broadcast
+        e.flush();
+        CHECK(cap.order.size() == 2);                            // two launches, in program order
+        size_t launches = cap.fused.size() + cap.singles.size();
+        CHECK(launches == 2);
+    }
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -612,6 +653,7 @@ int main(int argc, char** argv)
     testEngineStorageIsReusedAcrossWindows();
     testTrailingFillIsHandedOver();
     testCastsFuseAtTheirLoadOrStoreEnd();
+    testDenseSidesAdoptTheStridedSidesShape();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }
