@@ -860,9 +860,13 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::sliceSet() requires matching source and destination data types.");
     requireDevice(dst, "sliceSet");
+    // the backward of a slice fills the destination (zeros of the input's shape) right before the call:
+    // a fill still waiting in the window becomes the value written outside the slice, in the same pass
+    uint64_t init = 0;
+    const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "sliceSet"); toPod(dst, &pd, "sliceSet");
-    check(aixk_slice_set(m_ctx, &ps, &pd, dim, start, end, step));
+    check(folded ? aixk_slice_set_init(m_ctx, &ps, &pd, dim, start, end, step, init) : aixk_slice_set(m_ctx, &ps, &pd, dim, start, end, step));
 }
 
 void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)

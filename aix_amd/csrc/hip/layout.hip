@@ -141,6 +141,23 @@ __global__ __launch_bounds__(kBlock) void copy_views_k(const W* __restrict__ src
         dst[locate<IDX>(dsp, (IDX)i)] = src[locate<IDX>(ssp, (IDX)i)];
 }
 
+// ---- fill + sliceSet in one pass ----------------------------------------------------------------
+// dst is dense: element i is (o, c, e) = (i / (D inner), (i / inner) % D, i % inner) around the sliced dim.
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void slice_set_init_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> ssp, u64 n,
+                                                           u64 inner, u64 extent, u64 start, u64 end, u64 step, u64 count, W init)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
+        const u64 q = i / inner, e = i - q * inner, o = q / extent, c = q - o * extent;
+        W v = init;
+        if (c >= start && c < end) {
+            const u64 k = (c - start) / step;
+            if (start + k * step == c) v = src[locate<IDX>(ssp, (IDX)((o * count + k) * inner + e))];
+        }
+        dst[i] = v;
+    }
+}
+
 // ---- tril / triu -------------------------------------------------------------------------------
 template <class W, class IDX>
 __global__ __launch_bounds__(kBlock) void tri_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> ssp, Space<1> dsp,
@@ -341,6 +358,42 @@ int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_ten
     AIXK_REQUIRE(start + (window.shape[dim] ? (window.shape[dim] - 1) * step : 0) < dst->shape[dim] || n == 0,
                  "sliceSet: slice exceeds the destination");
     return copy_views(ctx, src, &window, n);
+}
+
+int32_t aixk_slice_set_init(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                            uint64_t dim, uint64_t start, uint64_t end, uint64_t step, uint64_t init_bits)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "sliceSet: bad operand descriptor");
+    AIXK_REQUIRE(src->dtype == dst->dtype, "sliceSet: element types differ");
+    AIXK_REQUIRE((int)dim < dst->rank && step > 0 && end >= start, "sliceSet: bad slice");
+    uint64_t dense[AIXK_MAX_RANK];
+    row_major_strides(dst->rank, dst->shape, dense);
+    bool is_dense = dst->offset == 0 && dst->size == numel(dst);
+    for (int d = 0; d < dst->rank; ++d) if (dst->shape[d] != 1 && dst->strides[d] != dense[d]) is_dense = false;
+    AIXK_REQUIRE(is_dense, "sliceSet with initialisation: the destination must be dense");
+    const uint64_t count = (end - start + step - 1) / step;
+    uint64_t window = count;
+    for (int d = 0; d < dst->rank; ++d) if (d != (int)dim) window *= dst->shape[d];
+    AIXK_REQUIRE(src->size == window && window == numel(src), "sliceSet: source size does not match the slice");
+    AIXK_REQUIRE(count == 0 || start + (count - 1) * step < dst->shape[dim], "sliceSet: slice exceeds the destination");
+    const uint64_t n = dst->size;
+    if (n == 0) return AIXK_OK;
+    uint64_t inner = 1;
+    for (int d = (int)dim + 1; d < dst->rank; ++d) inner *= dst->shape[d];
+    Space<1> ssp;
+    if (!collapse1(src, &ssp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+    const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31);
+    return by_size(src->dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
+        if (small) hipLaunchKernelGGL((slice_set_init_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, (u64)n,
+                                      (u64)inner, (u64)dst->shape[dim], (u64)start, (u64)end, (u64)step, (u64)count, (W)init_bits);
+        else hipLaunchKernelGGL((slice_set_init_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, (u64)n,
+                                (u64)inner, (u64)dst->shape[dim], (u64)start, (u64)end, (u64)step, (u64)count, (W)init_bits);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
 }
 
 int32_t aixk_tri(aixk_ctx* ctx, int upper, const aixhip_tensor* src, const aixhip_tensor* dst, int64_t diagonal)

@@ -52,6 +52,7 @@ _SIGNATURES = {
     "aixk_contiguous": [_P, _T, _T],
     "aixk_transpose": [_P, _T, _T, C.c_uint64, C.c_uint64],
     "aixk_slice_set": [_P, _T, _T, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64],
+    "aixk_slice_set_init": [_P, _T, _T, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64],
     "aixk_tri": [_P, C.c_int, _T, _T, C.c_int64],
     "aixk_index_select": [_P, _T, _T, _T, C.c_uint64],
     "aixk_index_add": [_P, _T, _T, _T, C.c_uint64],

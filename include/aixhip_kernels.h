@@ -107,6 +107,12 @@ int32_t aixk_transpose(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tenso
 /* dst is addressed through its offset and strides (the reference GPU device's behaviour). */
 int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
                        uint64_t dim, uint64_t start, uint64_t end, uint64_t step);                /* :468-496 */
+/* The same with the destination's initialisation folded in: dst (dense, offset 0) is written exactly once --
+ * `init_bits` (a value of its element type in the low bytes) outside the slice, src inside.  It is what
+ * fill(v) followed by sliceSet computes (the backward of a slice: zeros of the input's shape, then the
+ * gradient set into the slice, aixCore.hpp:1200-1203, 2237-2241) without the separate fill pass over dst. */
+int32_t aixk_slice_set_init(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
+                            uint64_t dim, uint64_t start, uint64_t end, uint64_t step, uint64_t init_bits);
 int32_t aixk_tri(aixk_ctx* ctx, int upper, const aixhip_tensor* src, const aixhip_tensor* dst, int64_t diagonal); /* :566-622 */
 /* indices: int32, addressed through their own offset and strides. */
 int32_t aixk_index_select(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,

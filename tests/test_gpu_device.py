@@ -452,6 +452,29 @@ def test_recorded_casts_fuse_and_keep_the_conversion_rules(dev, src):
     dev.release()
 
 
+def test_fill_is_folded_into_slice_set(dev):
+    """The backward of a slice: zeros of the input's shape, then the gradient set into the slice.  The pending
+    fill becomes the value the one sliceSet pass writes outside the slice (no fill kernel runs); a fill that
+    something else has read in between stays a fill."""
+    set_diag(dev)
+    rng = np.random.default_rng(38000)
+    for dtype in (O.F32, O.BF16, O.I32):
+        big, part = [40, 96], [40, 32]
+        g = T.contiguous_tensor(rng, dtype, part, int_span=50)
+        pg, dg = dev.put(g)
+        want = T.empty(dtype, big)
+        zero = np.zeros(1, np.float32)
+        assert CPU.fill(zero.ctypes.data, O.F32, C.byref(want.desc())) == 0
+        assert CPU.slice_set(C.byref(g.desc()), C.byref(want.desc()), 1, 32, 64, 1, 1) == 0
+        pz = dev.raw(want.storage.nbytes)
+        dz = H.kdesc(want, pz)
+        dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(dz))
+        dev.dev.call("slice_set", H.ref(dg), H.ref(dz), 1, 32, 64, 1)
+        got = dev.fetch(pz, want.storage)
+        T.assert_same_bits(got, want.storage, f"fill + sliceSet folded, {NAMES[dtype]}")
+    dev.release()
+
+
 _CASES = goldens.load_cases()
 
 

@@ -284,6 +284,15 @@ def test_slice_set_tri_index_ops(gpu, dtype):
         pd, dd = gpu.put(dst)
         G.run_gpu(gpu, "aixk_slice_set", G.ref(dsrc), G.ref(dd), dim, start, end, step)
         T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, f"sliceSet {NAMES[dtype]} {shape}->{big} dim={dim}")
+        # the same with the destination's initialisation folded in: fill(v) + sliceSet in one pass over a dense dst
+        scalar = T.random_values(rng, 1, dtype, int_span=50)
+        want = T.empty(dtype, big)
+        okc(CPU.fill(scalar.ctypes.data, dtype, C.byref(want.desc())))
+        okc(CPU.slice_set(C.byref(src.desc()), C.byref(want.desc()), dim, start, end, step, 1))
+        pd, dd = gpu.put(T.empty(dtype, big, fill=3))                   # every element must be overwritten
+        bits = int(np.frombuffer(scalar.tobytes().ljust(8, b"\0"), dtype=np.uint64)[0])
+        G.run_gpu(gpu, "aixk_slice_set_init", G.ref(dsrc), G.ref(dd), dim, start, end, step, bits)
+        T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, f"fill + sliceSet {NAMES[dtype]} {shape}->{big} dim={dim}")
         # tril / triu
         if rank >= 2:
             for upper in (0, 1):
