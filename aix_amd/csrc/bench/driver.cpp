@@ -181,13 +181,14 @@ int aixbench_mlp(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hi
 
 // Config 4: decoder-only transformer forward + backward (frontend/transformer.hpp); params in the order of
 // aixfe::transformerParamShapes; losses[steps], grad_norms[steps * param_count], step_seconds[steps] (may be NULL).
+// stacked_attention = 0: one 2-D matmul per (sequence, head), the reference's interface as it is; 1: matmul on stacks.
 int aixbench_transformer(aixhip_device* handle, uint64_t layers, uint64_t d_model, uint64_t heads, uint64_t seq, uint64_t batch,
-                         uint64_t vocab, int steps, const int32_t* tokens, const float* const* params,
+                         uint64_t vocab, int steps, int stacked_attention, const int32_t* tokens, const float* const* params,
                          float* losses, float* grad_norms, double* step_seconds)
 {
     return guarded([&] {
         DeviceHIP* dev = aix::hip::fromHandle(handle);
-        const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps};
+        const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps, stacked_attention};
         aixfe::runTransformer(dev, cfg, tokens, params, losses, grad_norms, step_seconds);
     });
 }

@@ -733,7 +733,9 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
     requireDevice(result, "matmul");
     flushFor(a.data, b.data, result.data);
     aixhip_tensor pa, pb, pr; stagedPod(a, &pa, "matmul"); stagedPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
-    check(aixk_matmul(m_ctx, &pa, &pb, &pr));
+    // operands with leading dims in front of the matrix dims: a stack of products (beyond the reference, whose
+    // matmul is 2-D only, aixCore.hpp:943-976)
+    check(a.shape.size() > 2 ? aixk_matmul_batched(m_ctx, &pa, &pb, &pr) : aixk_matmul(m_ctx, &pa, &pb, &pr));
 }
 
 void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)

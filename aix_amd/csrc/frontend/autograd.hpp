@@ -434,19 +434,21 @@ public:
         return r;
     }
 
-    // aixCore.hpp:2557-2569; matmulBackwardFunc :2178-2194
+    // aixCore.hpp:2557-2569; matmulBackwardFunc :2178-2194.  Stacks of matrices (rank above 2) transpose their
+    // last two dims.
     Tensor matmul(const Tensor& o) const
     {
         Tensor r = makeResult(value().matmul(o.value()), isRequireGrad() || o.isRequireGrad(), !m_node->isLeaf || !o.m_node->isLeaf);
         r.m_node->setBackward({m_node, o.m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.size() < 2) return;
+            const size_t rank = seed.shape().size(), d0 = rank - 2, d1 = rank - 1;
             if (n->inputs[0] == n->inputs[1]) {
-                const Value xT = n->inputs[0]->value.transpose(0, 1);
+                const Value xT = n->inputs[0]->value.transpose(d0, d1);
                 n->inputs[0]->backward(seed.matmul(xT) + xT.matmul(seed));
                 return;
             }
-            if (wants(n->inputs[0])) n->inputs[0]->backward(seed.matmul(n->inputs[1]->value.transpose(0, 1)));
-            if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value.transpose(0, 1).matmul(seed));
+            if (wants(n->inputs[0])) n->inputs[0]->backward(seed.matmul(n->inputs[1]->value.transpose(d0, d1)));
+            if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value.transpose(d0, d1).matmul(seed));
         });
         return r;
     }

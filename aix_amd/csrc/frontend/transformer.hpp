@@ -13,6 +13,11 @@
 // The interface has no batch dimension, so attention is issued the way an AIX program has to issue
 // it: projections as one [tokens, d] matmul each, then row slices per sequence and column slices
 // per head (views), 2-D matmuls on those, cat() to put heads and sequences back together.
+//
+// stackedAttention = 1 uses what this device adds to the interface, matmul on stacks of matrices:
+// q, k, v are seen as [batch, heads, seq, d / heads] views (reshape + transpose, no copy), the
+// scores of all sequences and heads are one [batch, heads, seq, seq] tensor, and mask, softmax and
+// the product with v are one operator each over it.  The arithmetic per element is the same.
 #pragma once
 
 #include "nn.hpp"
@@ -25,6 +30,7 @@ namespace aixfe {
 struct TransformerConfig {
     uint64_t layers, dModel, heads, seq, batch, vocab;
     int32_t steps;
+    int32_t stackedAttention{0};
 };
 
 // Parameter order (all f32, row-major):
@@ -100,20 +106,28 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
             const Tensor q = matmul(h, W[at + 2]) + W[at + 3];
             const Tensor k = matmul(h, W[at + 4]) + W[at + 5];
             const Tensor v = matmul(h, W[at + 6]) + W[at + 7];
-            std::vector<Tensor> sequences;
-            for (uint64_t b = 0; b < c.batch; ++b) {
-                const Tensor qb = q.slice(0, b * c.seq, (b + 1) * c.seq), kb = k.slice(0, b * c.seq, (b + 1) * c.seq),
-                             vb = v.slice(0, b * c.seq, (b + 1) * c.seq);
-                std::vector<Tensor> heads;
-                for (uint64_t hd = 0; hd < c.heads; ++hd) {
-                    const Tensor qh = qb.slice(1, hd * dh, (hd + 1) * dh), kh = kb.slice(1, hd * dh, (hd + 1) * dh),
-                                 vh = vb.slice(1, hd * dh, (hd + 1) * dh);
-                    const Tensor scores = (matmul(qh, kh.transpose(0, 1)) * scale).tril() + mask;
-                    heads.push_back(matmul(softmax(scores, 1, true), vh));
+            Tensor attn;
+            if (c.stackedAttention) {
+                const Shape split{c.batch, c.seq, c.heads, dh};
+                const Tensor q4 = q.reshape(split).transpose(1, 2), k4 = k.reshape(split).transpose(1, 2), v4 = v.reshape(split).transpose(1, 2);
+                const Tensor scores = (matmul(q4, k4.transpose(2, 3)) * scale).tril() + mask;         // [batch, heads, seq, seq]
+                attn = matmul(softmax(scores, 3, true), v4).transpose(1, 2).reshape(Shape{T, d});
+            } else {
+                std::vector<Tensor> sequences;
+                for (uint64_t b = 0; b < c.batch; ++b) {
+                    const Tensor qb = q.slice(0, b * c.seq, (b + 1) * c.seq), kb = k.slice(0, b * c.seq, (b + 1) * c.seq),
+                                 vb = v.slice(0, b * c.seq, (b + 1) * c.seq);
+                    std::vector<Tensor> heads;
+                    for (uint64_t hd = 0; hd < c.heads; ++hd) {
+                        const Tensor qh = qb.slice(1, hd * dh, (hd + 1) * dh), kh = kb.slice(1, hd * dh, (hd + 1) * dh),
+                                     vh = vb.slice(1, hd * dh, (hd + 1) * dh);
+                        const Tensor scores = (matmul(qh, kh.transpose(0, 1)) * scale).tril() + mask;
+                        heads.push_back(matmul(softmax(scores, 1, true), vh));
+                    }
+                    sequences.push_back(Tensor::cat(heads, 1));
                 }
-                sequences.push_back(Tensor::cat(heads, 1));
+                attn = Tensor::cat(sequences, 0);
             }
-            const Tensor attn = Tensor::cat(sequences, 0);
             x = x + (matmul(attn, W[at + 8]) + W[at + 9]);
             const Tensor h2 = layerNorm(x, P[at + 10], P[at + 11]);
             x = x + (matmul(gelu(matmul(h2, W[at + 12]) + W[at + 13]), W[at + 14]) + W[at + 15]);

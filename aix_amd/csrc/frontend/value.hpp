@@ -17,6 +17,7 @@
 
 #include "../device/aix_compat.hpp"
 
+#include <algorithm>
 #include <cstring>
 #include <memory>
 #include <numeric>
@@ -405,13 +406,19 @@ public:
         return v;
     }
 
+    // 2-D operands as in the reference (aixCore.hpp:943-976).  Beyond it: operands of one rank above 2 with the
+    // same leading dims are a stack of products, one per leading index, in a single device call.
     Value matmul(const Value& b) const
     {
-        if (m_p.shape.size() != 2 || b.m_p.shape.size() != 2 || m_p.shape[1] != b.m_p.shape[0])
-            throw std::invalid_argument("matmul: operands must be 2-D with matching inner dimension");
-        Value r(m_dev, m_p.dtype, Shape{m_p.shape[0], b.m_p.shape[1]});
-        m_dev->matmul(params(), b.params(), r.params());
-        return r;
+        const size_t r = m_p.shape.size();
+        if (r < 2 || b.m_p.shape.size() != r || m_p.shape[r - 1] != b.m_p.shape[r - 2] ||
+            !std::equal(m_p.shape.begin(), m_p.shape.end() - 2, b.m_p.shape.begin()))
+            throw std::invalid_argument("matmul: operands must be 2-D (or stacks with the same leading dims) with matching inner dimension");
+        Shape out(m_p.shape.begin(), m_p.shape.end() - 1);
+        out.push_back(b.m_p.shape[r - 1]);
+        Value res(m_dev, m_p.dtype, out);
+        m_dev->matmul(params(), b.params(), res.params());
+        return res;
     }
 
 private:

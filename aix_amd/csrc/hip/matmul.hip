@@ -17,6 +17,9 @@ namespace aixk {
 // Implemented in matmul_mfma.hip.  Returns AIXK_OK if it launched, -1 if the shape/layout is not
 // one it handles (caller falls back), or an error status.
 int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+// The same for a stack of products (a, b, out: the 2-D descriptors of the first matrices; batch: the joint
+// collapsed space of the leading dims, operands a, b, out).
+int matmul_mfma_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>& batch);
 } // namespace aixk
 
 namespace {
@@ -120,4 +123,62 @@ extern "C" int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixh
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     });
+}
+
+// out[..., m, n] = a[..., m, k] . b[..., k, n]: one product per index of the leading dims, which a, b and out share
+// (any of them may be a view: permuted, sliced, stride 0).  The results are written densely, row-major over
+// (leading dims, m, n), from out->data.
+extern "C" int32_t aixk_matmul_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(a) && valid_tensor(b) && valid_tensor(out), "matmul: bad operand descriptor");
+    AIXK_REQUIRE(a->rank >= 2 && a->rank == b->rank && a->rank == out->rank, "matmul: operands and result must have the same rank, at least 2");
+    if (a->rank == 2) return aixk_matmul(ctx, a, b, out);
+    const int nb = a->rank - 2;
+    for (int d = 0; d < nb; ++d)
+        AIXK_REQUIRE(a->shape[d] == b->shape[d] && a->shape[d] == out->shape[d], "matmul: leading dimensions differ");
+    AIXK_REQUIRE(a->shape[nb + 1] == b->shape[nb], "matmul: inner dimensions differ");
+    AIXK_REQUIRE(out->shape[nb] == a->shape[nb] && out->shape[nb + 1] == b->shape[nb + 1], "matmul: result shape does not match the operands");
+    AIXK_REQUIRE(a->dtype == out->dtype && b->dtype == out->dtype, "matmul: operands must have the result's element type");
+    const uint64_t M = a->shape[nb], K = a->shape[nb + 1], N = b->shape[nb + 1];
+    uint64_t count = 1;
+    for (int d = 0; d < nb; ++d) count *= a->shape[d];
+    if (count == 0 || M == 0 || N == 0) return AIXK_OK;
+    const size_t esz = aixk_dtype_size(out->dtype);
+    AIXK_REQUIRE(out->data != nullptr, "matmul: null result");
+    if (K == 0) return aixk_zero(ctx, out->data, count * M * N * esz);
+
+    // the leading dims as one joint iteration space; the result's strides are those of a dense stack
+    uint64_t dense[AIXK_MAX_RANK];
+    { uint64_t run = M * N; for (int d = nb - 1; d >= 0; --d) { dense[d] = run; run *= a->shape[d]; } }
+    const uint64_t* strides[3] = {a->strides, b->strides, dense};
+    const uint64_t offsets[3] = {0, 0, 0};
+    Space<3> batch;
+    AIXK_REQUIRE(collapse<3>(nb, a->shape, strides, offsets, &batch), "matmul: leading dims do not collapse to %d", kMaxDims);
+
+    auto matrix = [](const aixhip_tensor* t, int nb) {
+        aixhip_tensor m = *t;
+        m.rank = 2;
+        m.shape[0] = t->shape[nb]; m.shape[1] = t->shape[nb + 1];
+        m.strides[0] = t->strides[nb]; m.strides[1] = t->strides[nb + 1];
+        m.size = m.shape[0] * m.shape[1];
+        return m;
+    };
+    aixhip_tensor a2 = matrix(a, nb), b2 = matrix(b, nb), o2 = matrix(out, nb);
+    o2.offset = 0; o2.strides[0] = N; o2.strides[1] = 1;
+    if (out->dtype == AIXK_F16 || out->dtype == AIXK_BF16) {
+        const int rc = matmul_mfma_batched(ctx, &a2, &b2, &o2, batch);
+        if (rc != -1) return rc;
+    }
+    // one launch per product
+    uint64_t coord[kMaxDims] = {};
+    for (uint64_t i = 0; i < count; ++i) {
+        uint64_t oa = a->offset, ob = b->offset;
+        for (int d = 0; d < batch.rank; ++d) { oa += coord[d] * batch.stride[0][d]; ob += coord[d] * batch.stride[1][d]; }
+        a2.offset = oa; b2.offset = ob;
+        o2.data = (char*)out->data + i * M * N * esz;
+        AIXK_TRY(aixk_matmul(ctx, &a2, &b2, &o2));
+        for (int d = batch.rank - 1; d >= 0; --d) { if (++coord[d] < batch.shape[d]) break; coord[d] = 0; }
+    }
+    return AIXK_OK;
 }

@@ -45,6 +45,14 @@ struct GemmArgs {
     u32 tiles_m, tiles_n, swizzle;  // swizzle = 1: XCD-aware numbering is a bijection for this grid
 };
 
+// A stack of independent products in one launch: blockIdx.y numbers the matrices in row-major order of up to
+// three (collapsed) leading dims; every matrix of A / B starts sa / sb elements further per step of its dim,
+// results are dense, sc elements apart.  rank 0: a single product.
+struct BatchArgs {
+    u32 rank, ext[3];
+    u64 sa[3], sb[3], sc;
+};
+
 // blockIdx -> output tile, XCD-aware and grouped (4 tile rows per column sweep).
 __device__ __forceinline__ void tile_of(const GemmArgs& g, u32& tm, u32& tn)
 {
@@ -382,7 +390,7 @@ template <bool AT, bool BT> struct Small16 {
 };
 
 template <class T, bool AT, bool BT>
-__global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g)
+__global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
 {
     typedef Small16<AT, BT> S;
     constexpr int BM = S::BM, BN = S::BN, BK = S::BK, PK = S::PK, PT = S::PT, SA = S::SA, SB = S::SB;
@@ -394,6 +402,16 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const u16* A = (const u16*)g.a;
     const u16* B = (const u16*)g.b;
+    T* C = (T*)g.c;
+    if (bt.rank) {                                           // uniform over the workgroup: scalar arithmetic
+        u32 rest = blockIdx.y;
+        for (int d = (int)bt.rank - 1; d >= 0; --d) {
+            const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
+            A += (u64)c * bt.sa[d]; B += (u64)c * bt.sb[d];
+            rest = q;
+        }
+        C += (u64)blockIdx.y * bt.sc;
+    }
     u16* as = (u16*)smem_small + wave * (SA + SB);           // this wave's stage
     u16* bs = as + SA;
 
@@ -448,7 +466,6 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g)
 #pragma unroll
     for (int v = 0; v < 16; ++v) red[wave * 1024 + v * 64 + lane] = acc[v];
     __syncthreads();
-    T* C = (T*)g.c;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int e = tid + 256 * i, v = e >> 6, l = e & 63;
@@ -621,9 +638,71 @@ template <class K> int set_lds(K kernel, size_t bytes)
     return AIXK_OK;
 }
 
+
+// gemm_small16_k on the last two dims of a / b (rank 2 descriptors), `batch` = the joint collapsed space of the
+// leading dims (operands 0, 1, 2 = a, b, out) or null for one product.  -1: a layout the kernel does not take.
+int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    constexpr size_t esz = 2;
+    const char* qa = (const char*)a->data + a->offset * esz;
+    const char* qb = (const char*)b->data + b->offset * esz;
+    const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 8 == 0;
+    const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 8 == 0;
+    const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
+    if (!((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && aligned16(qa) && aligned16(qb))) return -1;
+    BatchArgs bt{};
+    uint64_t count = 1;
+    if (batch) {
+        if (batch->rank > 3) return -1;
+        bt.rank = (u32)batch->rank;
+        for (int d = 0; d < batch->rank; ++d) {
+            if (batch->shape[d] >= (1ull << 31) || batch->stride[0][d] % 8 != 0 || batch->stride[1][d] % 8 != 0) return -1;   // every matrix 16-byte aligned
+            bt.ext[d] = (u32)batch->shape[d]; bt.sa[d] = batch->stride[0][d]; bt.sb[d] = batch->stride[1][d];
+            count *= batch->shape[d];
+        }
+        if (count > 65535) return -1;
+        bt.sc = M * N;
+        if (bt.rank == 0) { bt.rank = 1; bt.ext[0] = 1; }
+    }
+    GemmArgs g{};
+    g.a = qa; g.b = qb; g.c = out->data;
+    g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+    g.tiles_m = (u32)((M + 31) / 32); g.tiles_n = (u32)((N + 31) / 32);
+    const u32 n = g.tiles_m * g.tiles_n;
+    g.swizzle = n % 8u == 0 ? 1u : 0u;
+    const bool at = !a_k, tb = !b_k;
+    auto launch = [&](auto kernel, size_t lds) {
+        AIXK_TRY(set_lds(kernel, lds));
+        hipLaunchKernelGGL(kernel, dim3(n, (unsigned)count), dim3(256), lds, ctx->stream, g, bt);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    };
+    if (out->dtype == AIXK_BF16) {
+        if (!at && !tb) return launch(gemm_small16_k<bf16, false, false>, Small16<false, false>::kLds);
+        if (!at && tb) return launch(gemm_small16_k<bf16, false, true>, Small16<false, true>::kLds);
+        if (at && !tb) return launch(gemm_small16_k<bf16, true, false>, Small16<true, false>::kLds);
+        return launch(gemm_small16_k<bf16, true, true>, Small16<true, true>::kLds);
+    }
+    if (!at && !tb) return launch(gemm_small16_k<f16, false, false>, Small16<false, false>::kLds);
+    if (!at && tb) return launch(gemm_small16_k<f16, false, true>, Small16<false, true>::kLds);
+    if (at && !tb) return launch(gemm_small16_k<f16, true, false>, Small16<true, false>::kLds);
+    return launch(gemm_small16_k<f16, true, true>, Small16<true, true>::kLds);
+}
+
 } // namespace
 
 namespace aixk {
+
+// A stack of 16-bit products small enough for the 32 x 32 tiles, in one launch.  -1: not handled here.
+int matmul_mfma_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>& batch)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    if (aixk_dtype_size(out->dtype) != 2 || (out->dtype != AIXK_BF16 && out->dtype != AIXK_F16)) return -1;
+    if (K % 8 != 0 || M * N < 64 * 64) return -1;                  // as for a single product
+    if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 2) return -1;     // each product fills the chip by itself: one launch each
+    return launch_small16(ctx, a, b, out, &batch);
+}
 
 int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)
 {
@@ -674,36 +753,8 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
     // every operand layout consumed where it lies (measured against the 64 x 64 route: 1024^3 NN 23.9 -> 15.2 us;
     // beyond two tiles per compute unit the larger tiles win)
     if (esz == 2 && ((M + 63) / 64) * ((N + 63) / 64) < (uint64_t)ctx->cus * 2) {
-        const char* qa = (const char*)a->data + a->offset * esz;
-        const char* qb = (const char*)b->data + b->offset * esz;
-        const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 8 == 0;
-        const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 8 == 0;
-        const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
-        if ((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && aligned16(qa) && aligned16(qb)) {
-            GemmArgs g{};
-            g.a = qa; g.b = qb; g.c = out->data;
-            g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
-            g.tiles_m = (u32)((M + 31) / 32); g.tiles_n = (u32)((N + 31) / 32);
-            const u32 n = g.tiles_m * g.tiles_n;
-            g.swizzle = n % 8u == 0 ? 1u : 0u;
-            const bool at = !a_k, bt = !b_k;
-            auto launch = [&](auto kernel, size_t lds) {
-                AIXK_TRY(set_lds(kernel, lds));
-                hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
-                AIXK_HIP(hipGetLastError());
-                return (int)AIXK_OK;
-            };
-            if (out->dtype == AIXK_BF16) {
-                if (!at && !bt) return launch(gemm_small16_k<bf16, false, false>, Small16<false, false>::kLds);
-                if (!at && bt) return launch(gemm_small16_k<bf16, false, true>, Small16<false, true>::kLds);
-                if (at && !bt) return launch(gemm_small16_k<bf16, true, false>, Small16<true, false>::kLds);
-                return launch(gemm_small16_k<bf16, true, true>, Small16<true, true>::kLds);
-            }
-            if (!at && !bt) return launch(gemm_small16_k<f16, false, false>, Small16<false, false>::kLds);
-            if (!at && bt) return launch(gemm_small16_k<f16, false, true>, Small16<false, true>::kLds);
-            if (at && !bt) return launch(gemm_small16_k<f16, true, false>, Small16<true, false>::kLds);
-            return launch(gemm_small16_k<f16, true, true>, Small16<true, true>::kLds);
-        }
+        const int rc = launch_small16(ctx, a, b, out, nullptr);
+        if (rc != -1) return rc;
     }
 
     auto grid_of = [&](GemmArgs& g, uint64_t bm, uint64_t bn) {

@@ -67,18 +67,19 @@ def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data, single_pass=False):
     return losses, secs
 
 
-def transformer(dev, cfg, steps, data):
+def transformer(dev, cfg, steps, data, stacked=False):
     """Forward + backward of the decoder-only transformer for `steps` steps on `dev`;
     cfg = (layers, d_model, heads, seq, batch, vocab), data = (int32 tokens [batch * seq], list of f32
     parameter arrays in the order of frontend/transformer.hpp).  Returns (losses, gradient norms
-    [steps, parameters], seconds per step)."""
+    [steps, parameters], seconds per step).  stacked: attention as matmuls on [batch, heads, ...] stacks (one
+    operator per layer and step of the attention) instead of one 2-D matmul per sequence and head."""
     tokens, params = data
     lib = load()
-    lib.aixbench_transformer.argtypes = [C.c_void_p] + [C.c_uint64] * 6 + [C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
+    lib.aixbench_transformer.argtypes = [C.c_void_p] + [C.c_uint64] * 6 + [C.c_int, C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
     losses = np.zeros(steps, np.float32)
     norms = np.zeros((steps, len(params)), np.float32)
     secs = np.zeros(steps, np.float64)
     pp = _pointer_array(params)
-    run("aixbench_transformer", dev.handle, *cfg, steps, tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
+    run("aixbench_transformer", dev.handle, *cfg, steps, int(stacked), tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
         norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
     return losses, norms, secs

@@ -289,34 +289,38 @@ def main():
         cfg = (6, 768, 12, 512, 16, 8192)
         data = OD.transformer_data(*cfg)
         t_steps = 4
-        losses, norms, secs = GD.transformer(dev, cfg, t_steps, data)
-        steady = float(secs[1:].mean())
         tokens = cfg[3] * cfg[4]
         d, v, s_len, layers = cfg[1], cfg[5], cfg[3], cfg[0]
         # forward products: 12 d^2 per token and layer (qkv, out, MLP), 2 s d per token and layer (scores, mix, causal half
         # not skipped), d v per token (output projection); backward = 2 x forward
         fwd = 2.0 * tokens * (layers * (12 * d * d + 2 * s_len * d) + d * v)
-        tf = {"workload": "configs[4] decoder-only transformer forward+backward: 6 layers, d 768, 12 heads, seq 512, batch 16, vocab 8192, "
-                          "GELU MLP 4x, LayerNorm, causal softmax attention as per-(batch, head) 2-D matmuls, bf16 activations, f32 masters",
-              "ms_per_step": round(steady * 1e3, 2), "value": round(tokens / steady, 1), "unit": "tokens/s",
-              "first_step_ms": round(float(secs[0]) * 1e3, 1), "flop_per_step": 3 * fwd,
-              "roofline": roofline("mfma", 3 * fwd / steady / 1e12, MFMA_PEAK_TFLOPS["bf16"], "TFLOP/s"),
-              "loss": round(float(losses[-1]), 7), "loss_expected_untrained": round(float(np.log(v) / v), 7)}
-        if not args.no_cpu:
-            small = (3, 128, 8, 64, 2, 256)
-            sdata = OD.transformer_data(*small)
-            threads = min(16, os.cpu_count() or 1)
-            want_l, want_n, cpu_secs = OD.oracle_transformer(small, 2, sdata, threads=threads)
-            got_l, got_n, _ = GD.transformer(dev, small, 2, sdata)
-            big = want_n[0] > 1e-3 * want_n[0].max()
-            rel_n = float((np.abs(got_n[0].astype(np.float64) - want_n[0])[big] / want_n[0][big]).max())
-            rel_l = float(abs(float(got_l[0]) - float(want_l[0])) / abs(float(want_l[0])))
-            tf["cpu_baseline"] = {"value": round(small[3] * small[4] / float(cpu_secs[1]), 1), "unit": "tokens/s", "cores": threads, "kind": "port",
-                                  "sample": f"a reduced model {small} (layers, d, heads, seq, batch, vocab), one step on the CPU oracle device "
-                                            f"({float(cpu_secs[1]):.2f} s); the full configuration is out of reach of the CPU device"}
-            tf["parity"] = {"checked_against": "cpu_baseline run (reduced model)", "loss_rel_dev": rel_l, "grad_norm_max_rel_dev": rel_n,
-                            "ok": bool(rel_l <= 2e-2 and rel_n <= 2e-2), "rule": "loss and every parameter's gradient norm within 2e-2 relative"}
-        extras.append(tf)
+        # attention issued (1) the way the reference's interface allows -- one 2-D matmul per (sequence, head) on sliced
+        # views -- and (2) with matmul on [batch, heads, ...] stacks, which this device adds to that interface
+        for stacked, how in ((False, "causal softmax attention as per-(batch, head) 2-D matmuls"),
+                             (True, "causal softmax attention as matmuls on [batch, heads, seq, .] stacks (an extension of the interface)")):
+            losses, norms, secs = GD.transformer(dev, cfg, t_steps, data, stacked=stacked)
+            steady = float(secs[1:].mean())
+            tf = {"workload": "configs[4] decoder-only transformer forward+backward: 6 layers, d 768, 12 heads, seq 512, batch 16, vocab 8192, "
+                              f"GELU MLP 4x, LayerNorm, {how}, bf16 activations, f32 masters",
+                  "ms_per_step": round(steady * 1e3, 2), "value": round(tokens / steady, 1), "unit": "tokens/s",
+                  "first_step_ms": round(float(secs[0]) * 1e3, 1), "flop_per_step": 3 * fwd,
+                  "roofline": roofline("mfma", 3 * fwd / steady / 1e12, MFMA_PEAK_TFLOPS["bf16"], "TFLOP/s"),
+                  "loss": round(float(losses[-1]), 7), "loss_expected_untrained": round(float(np.log(v) / v), 7)}
+            if not args.no_cpu:
+                small = (3, 128, 8, 64, 2, 256)
+                sdata = OD.transformer_data(*small)
+                threads = min(16, os.cpu_count() or 1)
+                want_l, want_n, cpu_secs = OD.oracle_transformer(small, 2, sdata, threads=threads, stacked=stacked)
+                got_l, got_n, _ = GD.transformer(dev, small, 2, sdata, stacked=stacked)
+                big = want_n[0] > 1e-3 * want_n[0].max()
+                rel_n = float((np.abs(got_n[0].astype(np.float64) - want_n[0])[big] / want_n[0][big]).max())
+                rel_l = float(abs(float(got_l[0]) - float(want_l[0])) / abs(float(want_l[0])))
+                tf["cpu_baseline"] = {"value": round(small[3] * small[4] / float(cpu_secs[1]), 1), "unit": "tokens/s", "cores": threads, "kind": "port",
+                                      "sample": f"a reduced model {small} (layers, d, heads, seq, batch, vocab), one step on the CPU oracle device "
+                                                f"({float(cpu_secs[1]):.2f} s); the full configuration is out of reach of the CPU device"}
+                tf["parity"] = {"checked_against": "cpu_baseline run (reduced model, the same program)", "loss_rel_dev": rel_l, "grad_norm_max_rel_dev": rel_n,
+                                "ok": bool(rel_l <= 2e-2 and rel_n <= 2e-2), "rule": "loss and every parameter's gradient norm within 2e-2 relative"}
+            extras.append(tf)
     if not args.no_extras:
         out["extras"] = extras
 

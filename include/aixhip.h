@@ -75,6 +75,8 @@ int32_t aixhip_pow(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tens
 int32_t aixhip_max(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tensor* result);
 int32_t aixhip_argmax(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tensor* result);
 int32_t aixhip_argmax_indices(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tensor* result);
+/* matmul: 2-D operands as in the reference; operands and result of the same rank above 2 are a stack of
+ * products over their shared leading dims (an extension, see aixk_matmul_batched). */
 int32_t aixhip_matmul(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* result);
 int32_t aixhip_transpose(aixhip_device* dev, const aixhip_tensor* a, const aixhip_tensor* result, size_t dim0, size_t dim1);
 

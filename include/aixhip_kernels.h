@@ -142,6 +142,14 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
  * accumulation, other types on a generic tiled kernel with an accumulator of the element type
  * (f64 and integers). */
 int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+/* An extension of the above: the reference multiplies 2-D operands only (aixCore.hpp:943-976), so an
+ * AIX program issues attention as one matmul per (sequence, head) on sliced views.  Here a, b and out
+ * may carry the same leading dims in front of the matrix dims: out[..., m, n] = a[..., m, k] . b[..., k, n],
+ * one product per index of the leading dims, exactly what the 2-D entry point computes for each.
+ * a and b may be any views (permuted, sliced, stride 0); the results are written densely from
+ * out->data.  Stacks of small 16-bit products run as ONE launch; everything else is issued product by
+ * product through the 2-D entry point.  Rank 2 is the 2-D entry point. */
+int32_t aixk_matmul_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
 
 /* ---- runtime-compiled fused elementwise kernels ------------------------- */
 /* Compile `source` (HIP C++, one extern "C" __global__ named `entry`) for gfx950 with hipRTC or

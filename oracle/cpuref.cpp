@@ -731,6 +731,42 @@ int cpuref_reduce_to_wide(const cpuref_tensor* src, const cpuref_tensor* dst_lik
     });
 }
 
+int cpuref_matmul_stack(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads)
+{
+    if (a->rank < 2 || a->rank != b->rank || a->rank != out->rank) return CPUREF_EINVAL;
+    const int nb = a->rank - 2;
+    uint64_t count = 1;
+    for (int d = 0; d < nb; ++d) {
+        if (a->shape[d] != b->shape[d] || a->shape[d] != out->shape[d]) return CPUREF_EINVAL;
+        count *= a->shape[d];
+    }
+    auto matrix = [nb](const cpuref_tensor* t) {
+        cpuref_tensor m = *t;
+        m.rank = 2;
+        m.shape[0] = t->shape[nb]; m.shape[1] = t->shape[nb + 1];
+        m.strides[0] = t->strides[nb]; m.strides[1] = t->strides[nb + 1];
+        m.size = m.shape[0] * m.shape[1];
+        return m;
+    };
+    cpuref_tensor a2 = matrix(a), b2 = matrix(b), o2 = matrix(out);
+    if (a2.shape[1] != b2.shape[0]) return CPUREF_EINVAL;
+    const uint64_t per = a2.shape[0] * b2.shape[1] * cpuref_dtype_size(out->dtype);
+    o2.offset = 0; o2.strides[0] = b2.shape[1]; o2.strides[1] = 1;
+    for (uint64_t i = 0; i < count; ++i) {
+        uint64_t rest = i, oa = a->offset, ob = b->offset;
+        for (int d = nb - 1; d >= 0; --d) {
+            const uint64_t c = rest % a->shape[d];
+            rest /= a->shape[d];
+            oa += c * a->strides[d]; ob += c * b->strides[d];
+        }
+        a2.offset = oa; b2.offset = ob;
+        o2.data = (char*)out->data + i * per;
+        const int rc = cpuref_matmul_rows(&a2, &b2, &o2, threads);
+        if (rc != CPUREF_OK) return rc;
+    }
+    return CPUREF_OK;
+}
+
 int cpuref_matmul_wide(const cpuref_tensor* a, const cpuref_tensor* b, double* out64, double* abs64, int threads)
 {
     if (a->rank != 2 || b->rank != 2 || a->dtype != b->dtype) return CPUREF_EINVAL;

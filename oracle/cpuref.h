@@ -95,6 +95,11 @@ int cpuref_matmul_wide(const cpuref_tensor* a, const cpuref_tensor* b, double* o
 /* Same arithmetic, operand order and rounding as cpuref_matmul (accumulator of the
  * element type, k ascending) with rows spread over threads; bit-identical to it. */
 int cpuref_matmul_rows(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads);
+/* Not in the reference (its matmul is 2-D only, aixCore.hpp:943-976): a, b, out of one rank above 2 with
+ * the same leading dims; cpuref_matmul_rows on the matrices of every leading index in turn, results
+ * dense from out->data.  Pinned by that function and, for the indexing of the stack, by integer
+ * stacks against numpy.matmul (tests/test_oracle_golden.py). */
+int cpuref_matmul_stack(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads);
 
 /* ---- helpers for tests --------------------------------------------------- */
 /* Distance in units in the last place between two f32 arrays: returns the maximum,

@@ -38,11 +38,11 @@ int oracle_mlp(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64
 
 // Same contract as aixbench_transformer.
 int oracle_transformer(int threads, uint64_t layers, uint64_t d_model, uint64_t heads, uint64_t seq, uint64_t batch, uint64_t vocab,
-                       int steps, const int32_t* tokens, const float* const* params, float* losses, float* grad_norms, double* step_seconds)
+                       int steps, int stacked_attention, const int32_t* tokens, const float* const* params, float* losses, float* grad_norms, double* step_seconds)
 {
     try {
         oracle::OracleDevice dev(threads);
-        const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps};
+        const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps, stacked_attention};
         aixfe::runTransformer(&dev, cfg, tokens, params, losses, grad_norms, step_seconds);
         return 0;
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }

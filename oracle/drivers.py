@@ -223,16 +223,16 @@ def transformer_data(layers, d, heads, seq, batch, vocab, seed_tok=7, seed_w=8):
     return tokens, params
 
 
-def oracle_transformer(cfg, steps, data, threads=1):
+def oracle_transformer(cfg, steps, data, threads=1, stacked=False):
     """cfg = (layers, d, heads, seq, batch, vocab).  Returns (losses, grad norms [steps, P], seconds)."""
     tokens, params = data
     lib = oracle_lib()
-    lib.oracle_transformer.argtypes = [C.c_int] + [C.c_uint64] * 6 + [C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
+    lib.oracle_transformer.argtypes = [C.c_int] + [C.c_uint64] * 6 + [C.c_int, C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
     losses = np.zeros(steps, np.float32)
     norms = np.zeros((steps, len(params)), np.float32)
     secs = np.zeros(steps, np.float64)
     pp = pointer_array(params)
-    rc = lib.oracle_transformer(threads, *cfg, steps, tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
+    rc = lib.oracle_transformer(threads, *cfg, steps, int(stacked), tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
                                 norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
     if rc != 0:
         raise RuntimeError(lib.oracle_drivers_last_error().decode())

@@ -47,7 +47,11 @@ public:
     void max(const P& a, const P& r) override { ok(cpuref_max(d(a), d(r))); ++ops; }
     void argmax(const P& a, const P& r) override { ok(cpuref_argmax(d(a), d(r))); ++ops; }
     void argmaxIndices(const P& a, const P& r) override { ok(cpuref_argmax_indices(d(a), d(r))); ++ops; }
-    void matmul(const P& a, const P& b, const P& r) override { ok(cpuref_matmul_rows(d(a), d(b), d(r), m_threads)); ++ops; ++matmuls; }
+    void matmul(const P& a, const P& b, const P& r) override
+    {
+        ok(a.shape.size() > 2 ? cpuref_matmul_stack(d(a), d(b), d(r), m_threads) : cpuref_matmul_rows(d(a), d(b), d(r), m_threads));
+        ++ops; ++matmuls;
+    }
     void transpose(const P& a, const P& r, size_t d0, size_t d1) override { ok(cpuref_transpose(d(a), d(r), d0, d1)); ++ops; }
     void copy(const void* s, aix::DataType st, void* t, aix::DataType tt, size_t n) override { ok(cpuref_copy(s, (int)st, t, (int)tt, n)); }
     void copyImmediate(const void* s, aix::DataType st, void* t, aix::DataType tt, size_t n) override { copy(s, st, t, tt, n); }

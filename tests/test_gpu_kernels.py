@@ -656,6 +656,124 @@ def test_matmul_identity_and_ones(gpu):
         gpu.release()
 
 
+# ---- stacks of products (beyond the reference: its matmul is 2-D only) -----------------------------
+def _matrix_of(ht, index):
+    """The 2-D view of matrix `index` (a tuple over the leading dims) of a stacked HostTensor."""
+    nb = len(ht.shape) - 2
+    off = ht.offset + sum(i * s for i, s in zip(index, ht.strides[:nb]))
+    return T.HostTensor(ht.storage, ht.dtype, ht.shape[nb:], ht.strides[nb:], off)
+
+
+def check_matmul_stack(gpu, a, b, what, against_each=True):
+    """aixk_matmul_batched against (1) the oracle's stack -- integers bit for bit, floats within the matmul bar of
+    the exactly accumulated products -- and (2) aixk_matmul issued matrix by matrix on the same views, bit for bit."""
+    dtype = a.dtype
+    lead, m, k, n = a.shape[:-2], a.shape[-2], a.shape[-1], b.shape[-1]
+    count = int(np.prod(lead))
+    pa, da = gpu.put(a)
+    pb, db = gpu.put(b)
+    po, do = gpu.put(T.empty(dtype, lead + [m, n]))
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(da), G.ref(db), G.ref(do))
+    got = gpu.fetch(po, np.zeros(count * m * n, O.NP_STORAGE[dtype]))
+    if dtype in T.INT_DTYPES:
+        want = T.empty(dtype, lead + [m, n])
+        okc(CPU.matmul_stack(C.byref(a.desc()), C.byref(b.desc()), C.byref(want.desc()), 8))
+        T.assert_same_bits(got, want.storage, what)
+    tol = {O.F64: 1e-12, O.F32: 1e-5, O.F16: 2e-2, O.BF16: 2e-2}.get(dtype)
+    p1, d1 = gpu.put(T.empty(dtype, [m, n]))
+    for flat, index in enumerate(np.ndindex(*lead)):
+        a2, b2 = _matrix_of(a, index), _matrix_of(b, index)
+        mine = got[flat * m * n:(flat + 1) * m * n]
+        if dtype not in T.INT_DTYPES:
+            exact = np.zeros(m * n)
+            scale = np.zeros(m * n)
+            okc(CPU.matmul_wide(C.byref(a2.desc()), C.byref(b2.desc()), exact.ctypes.data, scale.ctypes.data, 8))
+            G.assert_close_to_wide(O.to_float64(mine, dtype), exact, scale + 1e-30, tol, f"{what} matrix {index}")
+        if against_each:
+            G.run_gpu(gpu, "aixk_matmul", G.ref(G.kdesc(a2, pa)), G.ref(G.kdesc(b2, pb)), G.ref(d1))
+            T.assert_same_bits(mine, gpu.fetch(p1, mine), f"{what} matrix {index} against the 2-D entry point")
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16, O.F32, O.I32], ids=ids)
+def test_matmul_stacks(gpu, dtype):
+    """Attention-shaped stacks through every view the front-end builds: q, k, v stored [batch, seq, heads, d]
+    and seen as [batch, heads, seq, d] (permuted leading dims), k transposed on its last two dims, a
+    transposed first operand (the gradient products), a second operand shared by the whole stack (stride 0),
+    sliced stacks with an offset, ragged extents.  The 16-bit cases run as one launch, f32 and integers as
+    one launch per matrix."""
+    rng = np.random.default_rng(24000 + dtype)
+    B, H, S, D = 2, 3, 96, 64
+    def draw(count, lo, hi):
+        return O.to_storage(rng.integers(-9, 9, count) if dtype in T.INT_DTYPES else rng.uniform(lo, hi, count), dtype)
+    q = draw(B * S * H * D, -0.2, 0.2)
+    kk = draw(B * S * H * D, -1, 1)
+    heads = [S * H * D, D, H * D, 1]                       # [batch, heads, seq, d] over [batch, seq, heads, d] storage
+    heads_t = [S * H * D, D, 1, H * D]                     # ... with the last two dims transposed: [batch, heads, d, seq]
+    q4 = T.HostTensor(q, dtype, [B, H, S, D], heads)
+    kT = T.HostTensor(kk, dtype, [B, H, D, S], heads_t)
+    check_matmul_stack(gpu, q4, kT, f"scores {NAMES[dtype]}")                                  # [S, D] . [D, S]
+    p = T.HostTensor(draw(B * H * S * S, -0.1, 0.1), dtype, [B, H, S, S])
+    v4 = T.HostTensor(kk, dtype, [B, H, S, D], heads)
+    check_matmul_stack(gpu, p, v4, f"p.v {NAMES[dtype]}")                                      # [S, S] . [S, D]
+    pT = T.HostTensor(p.storage, dtype, [B, H, S, S], [H * S * S, S * S, 1, S])
+    check_matmul_stack(gpu, pT, v4, f"pT.v {NAMES[dtype]}")                                    # transposed first operand
+    check_matmul_stack(gpu, p, T.HostTensor(kk, dtype, [B, H, S, D], [0, 0, H * D, 1]), f"shared second operand {NAMES[dtype]}")
+    gpu.release()
+    # a slice of a stack (offset, fewer matrices than stored), ragged extents, rank 3
+    wide = T.HostTensor(draw(5 * 72 * 104, -0.2, 0.2), dtype, [3, 72, 88], [72 * 104, 104, 1], offset=72 * 104 + 8)
+    other = T.HostTensor(draw(4 * 88 * 80, -1, 1), dtype, [3, 88, 80], None, offset=88 * 80)
+    check_matmul_stack(gpu, wide, other, f"sliced stack {NAMES[dtype]}")
+    # matrices too small or too odd for the matrix-core route
+    check_matmul_stack(gpu, T.HostTensor(draw(7 * 5 * 3, -1, 1), dtype, [7, 5, 3]), T.HostTensor(draw(7 * 3 * 4, -1, 1), dtype, [7, 3, 4]),
+                       f"tiny stack {NAMES[dtype]}")
+    gpu.release()
+
+
+def test_matmul_stack_edges(gpu):
+    """Rank 2 is the 2-D entry point; empty stacks and K = 0; more matrices than one launch numbers (stride-0
+    stacks of one product: every result matrix equals the single product); mismatched operands are refused."""
+    rng = np.random.default_rng(24500)
+    dtype = O.BF16
+    a = T.HostTensor(O.to_storage(rng.uniform(-0.3, 0.3, 64 * 16), dtype), dtype, [64, 16])
+    b = T.HostTensor(O.to_storage(rng.uniform(-1, 1, 16 * 64), dtype), dtype, [16, 64])
+    pa, da = gpu.put(a)
+    pb, db = gpu.put(b)
+    p1, d1 = gpu.put(T.empty(dtype, [64, 64]))
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(d1))
+    one = gpu.fetch(p1, np.zeros(64 * 64, np.uint16))
+    p2, d2 = gpu.put(T.empty(dtype, [64, 64], fill=7))
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(da), G.ref(db), G.ref(d2))
+    T.assert_same_bits(gpu.fetch(p2, one), one, "rank 2 through the stacked entry point")
+    for count in (3, 65535, 65536 + 5):
+        sa = T.HostTensor(a.storage, dtype, [count, 64, 16], [0, 16, 1])
+        sb = T.HostTensor(b.storage, dtype, [count, 16, 64], [0, 64, 1])
+        po, do = gpu.put(T.empty(dtype, [count, 64, 64], fill=7))
+        G.run_gpu(gpu, "aixk_matmul_batched", G.ref(G.kdesc(sa, pa)), G.ref(G.kdesc(sb, pb)), G.ref(do))
+        got = gpu.fetch(po, np.zeros(count * 4096, np.uint16)).reshape(count, 4096)
+        assert np.all(got == one[None, :]), f"{count} copies of one product"
+        gpu.release()
+        pa, da = gpu.put(a)
+        pb, db = gpu.put(b)
+    # empty stack: nothing written; K = 0: zeros
+    po, do = gpu.put(T.empty(dtype, [2, 4, 4], fill=7))
+    empty_a, empty_b, empty_o = G.kdesc(T.HostTensor(a.storage, dtype, [0, 4, 8]), pa), G.kdesc(T.HostTensor(b.storage, dtype, [0, 8, 4]), pb), G.kdesc(T.empty(dtype, [0, 4, 4]), po)
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(empty_a), G.ref(empty_b), G.ref(empty_o))
+    assert np.all(gpu.fetch(po, np.zeros(32, np.uint16)) == 7)
+    k0_a, k0_b = G.kdesc(T.HostTensor(a.storage, dtype, [2, 4, 0]), pa), G.kdesc(T.HostTensor(b.storage, dtype, [2, 0, 4]), pb)
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(k0_a), G.ref(k0_b), G.ref(do))
+    assert np.all(gpu.fetch(po, np.zeros(32, np.uint16)) == 0)
+    # refusals
+    lib = gpu.ctx.lib
+    three = G.kdesc(T.HostTensor(a.storage, dtype, [2, 8, 16]), pa)
+    other_lead = G.kdesc(T.HostTensor(b.storage, dtype, [3, 16, 8]), pb)
+    out3 = G.kdesc(T.empty(dtype, [2, 8, 8]), po)
+    assert lib.aixk_matmul_batched(gpu.ctx.handle, G.ref(three), G.ref(other_lead), G.ref(out3)) != 0          # leading dims differ
+    assert lib.aixk_matmul_batched(gpu.ctx.handle, G.ref(three), G.ref(db), G.ref(out3)) != 0                  # ranks differ
+    bad_inner = G.kdesc(T.HostTensor(b.storage, dtype, [2, 8, 8]), pb)
+    assert lib.aixk_matmul_batched(gpu.ctx.handle, G.ref(three), G.ref(bad_inner), G.ref(out3)) != 0           # inner dims differ
+    gpu.release()
+
+
 # ---- the reference's own literal vectors through the GPU kernels ----------------------------------
 import goldens  # noqa: E402
 

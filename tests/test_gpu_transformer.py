@@ -22,12 +22,15 @@ def dev():
     d.close()
 
 
+@pytest.mark.parametrize("stacked", [False, True], ids=["per_head", "stacked"])
 @pytest.mark.parametrize("cfg", [(2, 64, 4, 32, 2, 128), (1, 32, 2, 24, 3, 80), (3, 128, 8, 64, 2, 256)], ids=str)
-def test_loss_and_gradient_norms_match_the_cpu_device(dev, cfg):
+def test_loss_and_gradient_norms_match_the_cpu_device(dev, cfg, stacked):
+    """per_head: attention as one 2-D matmul per (sequence, head), the reference's interface as it is;
+    stacked: as matmuls on [batch, heads, ...] stacks, the same program on both devices."""
     from aix_amd import drivers as GD
     data = OD.transformer_data(*cfg)
-    want_l, want_n, _ = OD.oracle_transformer(cfg, 2, data, threads=16)
-    got_l, got_n, secs = GD.transformer(dev, cfg, 2, data)
+    want_l, want_n, _ = OD.oracle_transformer(cfg, 2, data, threads=16, stacked=stacked)
+    got_l, got_n, secs = GD.transformer(dev, cfg, 2, data, stacked=stacked)
     rel_l = np.abs(got_l.astype(np.float64) - want_l) / np.abs(want_l)
     big = want_n > 1e-3 * want_n.max()                # norms that are not numerically zero (biases start at 0 but have gradients)
     rel_n = np.abs(got_n.astype(np.float64) - want_n)[big] / want_n[big]
@@ -39,3 +42,20 @@ def test_loss_and_gradient_norms_match_the_cpu_device(dev, cfg):
     assert got_l[0] == got_l[1] and np.allclose(got_n[0], got_n[1], rtol=1e-3, atol=0)
     assert rel_l.max() <= 2e-2
     assert rel_n.max() <= 2e-2
+
+
+def test_stacked_attention_against_per_head_attention_on_the_gpu(dev):
+    """The two ways of issuing attention on the same device: the same arithmetic per element, so the losses and
+    gradient norms agree far inside the 16-bit bar (the difference left is the order in which atomics and
+    multi-workgroup reductions add)."""
+    from aix_amd import drivers as GD
+    cfg = (2, 128, 4, 128, 3, 256)
+    data = OD.transformer_data(*cfg)
+    loop_l, loop_n, loop_s = GD.transformer(dev, cfg, 2, data)
+    stack_l, stack_n, stack_s = GD.transformer(dev, cfg, 2, data, stacked=True)
+    big = loop_n > 1e-3 * loop_n.max()
+    rel = np.abs(stack_n.astype(np.float64) - loop_n)[big] / loop_n[big]
+    print(f"{cfg}: loss {loop_l[0]:.6f} (per head) {stack_l[0]:.6f} (stacked); gradient norms max rel dev {rel.max():.2e}; "
+          f"{loop_s[1] * 1e3:.1f} ms/step per head, {stack_s[1] * 1e3:.1f} ms/step stacked")
+    assert abs(float(stack_l[0]) - float(loop_l[0])) <= 1e-5 * abs(float(loop_l[0]))
+    assert rel.max() <= 1e-3

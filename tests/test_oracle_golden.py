@@ -154,6 +154,45 @@ def test_sum_reduce_matmul_invariants():
     np.testing.assert_allclose(lit.storage, wide, rtol=0, atol=23 * 2 ** -23 * (np.abs(R) @ np.abs(S)).max())
 
 
+def test_matmul_stack_is_the_2d_matmul_per_leading_index():
+    """cpuref_matmul_stack (an extension: the reference's matmul is 2-D only) adds nothing but the walk over the
+    leading dims: integer stacks equal numpy.matmul exactly, through permuted, sliced and stride-0 views, and a
+    float stack equals cpuref_matmul on each pair of matrices bit for bit."""
+    rng = np.random.default_rng(450)
+    # [2, 3, 5, 4] . [2, 3, 4, 6] on int32, operands seen through views of larger arrays
+    base_a = rng.integers(-9, 9, (5, 2, 3, 8)).astype(np.int32)            # stored [m, p, q, 2k]: a[p, q, m, k] = base[m, p, q, 2k]
+    base_b = rng.integers(-9, 9, (3, 4, 6)).astype(np.int32)               # stored [q, k, n]: the same for every p (stride 0)
+    ta = T.HostTensor(base_a, O.I32, [2, 3, 5, 4], [3 * 8, 8, 2 * 3 * 8, 2])
+    tb = T.HostTensor(base_b, O.I32, [2, 3, 4, 6], [0, 24, 6, 1])
+    out = T.empty(O.I32, [2, 3, 5, 6])
+    assert CPU.matmul_stack(C.byref(ta.desc()), C.byref(tb.desc()), C.byref(out.desc()), 2) == 0
+    A = base_a[:, :, :, ::2].transpose(1, 2, 0, 3).astype(np.int64)
+    B = np.broadcast_to(base_b.astype(np.int64), (2, 3, 4, 6))
+    np.testing.assert_array_equal(out.storage.reshape(2, 3, 5, 6), A @ B)
+    # an offset moves every matrix of the stack
+    tb_off = T.HostTensor(base_b, O.I32, [2, 2, 4, 6], [0, 24, 6, 1], offset=24)
+    ta2 = T.HostTensor(base_a, O.I32, [2, 2, 5, 4], [3 * 8, 8, 2 * 3 * 8, 2])
+    out = T.empty(O.I32, [2, 2, 5, 6])
+    assert CPU.matmul_stack(C.byref(ta2.desc()), C.byref(tb_off.desc()), C.byref(out.desc()), 1) == 0
+    np.testing.assert_array_equal(out.storage.reshape(2, 2, 5, 6), A[:, :2] @ B[:, 1:])
+    # floats: the bits of the 2-D function, matrix by matrix
+    for dtype in (O.F32, O.BF16):
+        fa = O.to_storage(rng.uniform(-1, 1, 4 * 7 * 9), dtype)
+        fb = O.to_storage(rng.uniform(-1, 1, 4 * 9 * 5), dtype)
+        sa, sb = T.HostTensor(fa, dtype, [4, 7, 9]), T.HostTensor(fb, dtype, [4, 9, 5])
+        stack = T.empty(dtype, [4, 7, 5])
+        assert CPU.matmul_stack(C.byref(sa.desc()), C.byref(sb.desc()), C.byref(stack.desc()), 3) == 0
+        for i in range(4):
+            one = T.empty(dtype, [7, 5])
+            a2 = T.HostTensor(fa, dtype, [7, 9], offset=i * 63)
+            b2 = T.HostTensor(fb, dtype, [9, 5], offset=i * 45)
+            assert CPU.matmul(C.byref(a2.desc()), C.byref(b2.desc()), C.byref(one.desc())) == 0
+            T.assert_same_bits(stack.storage[i * 35:(i + 1) * 35], one.storage, f"stack matrix {i}")
+    # ranks must agree, leading dims must agree
+    bad = T.HostTensor(base_b, O.I32, [3, 4, 6])
+    assert CPU.matmul_stack(C.byref(ta.desc()), C.byref(bad.desc()), C.byref(out.desc()), 1) != 0
+
+
 def test_argmax_first_maximum_brute_force():
     rng = np.random.default_rng(500)
     for _ in range(50):
