@@ -24,6 +24,9 @@
 
 #include "common.hpp"
 
+#include <algorithm>
+#include <type_traits>
+
 using namespace aixd;
 using namespace aixk;
 
@@ -475,6 +478,161 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
     }
 }
 
+// ---- 16-bit operands, mid-size problems and stacks of matrices --------------------------------------
+// Everything between the two kernels above: outputs of a few hundred tiles (a [8192, 768] activation times a
+// [768, 768] weight), weight gradients with few tiles and a very long K ([768, 8192] x [8192, 768]), and stacks of
+// attention-sized products.  BM x BN workgroup tile (128 x 128, 128 x 64, 64 x 64), BK = 32, four waves 2 x 2,
+// two LDS stages filled from registers (the next step's global loads are in flight under this step's MFMAs), one
+// barrier per step; 41 KB of LDS at most, so several workgroups share a compute unit and overlap each other's
+// barriers and LDS reads.  Both operand forms are consumed where they lie, exactly as in gemm_small16_k:
+// K-contiguous staged [row][k] with a pitch of 40 elements (80 bytes: 16 consecutive rows start in 16 different
+// groups of four banks), T form staged [k][row] with a pitch of tile + 32 elements (64 or 192 bytes modulo 256: the
+// four k-rows a group of 16 lanes reads, and the two groups of a half-wave, fall into disjoint banks).
+//
+// blockIdx.y numbers the matrices of a stack (BatchArgs).  blockIdx.z numbers K splits: split s multiplies K steps
+// [s * per_split, (s + 1) * per_split) and, when there is more than one split, stores its f32 partial tile in
+// `partial` ([split][matrix][M][N]) for splitk_finish_k to add up in split order and round once.
+struct SplitArgs { float* partial; u32 splits, per_split; u64 matrices; };
+
+template <int BM, int BN, int BK_, bool AT, bool BT> struct Tile16 {
+    static constexpr int BK = BK_, PK = BK + 8, PA = BM + 32, PB = BN + 32;
+    static constexpr int SA = AT ? BK * PA : BM * PK, SB = BT ? BK * PB : BN * PK;       // elements per stage
+    static constexpr size_t kLds = (size_t)2 * (SA + SB) * 2;
+};
+
+template <class T, int BM, int BN, int BKT, bool AT, bool BT>
+__global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, SplitArgs sk)
+{
+    typedef Tile16<BM, BN, BKT, AT, BT> S;
+    constexpr int BK = S::BK, PK = S::PK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
+    constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
+    constexpr int CA = BM * (BK / 8) / 256, CB = BN * (BK / 8) / 256;        // 16-byte chunks per lane and step
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_tile[];
+    u16* As = (u16*)smem_tile;                            // [2][SA]
+    u16* Bs = As + 2 * SA;                                // [2][SB]
+
+    u32 tm, tn;
+    tile_of(g, tm, tn);
+    const u64 m0 = (u64)tm * BM, n0 = (u64)tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const u16* A = (const u16*)g.a;
+    const u16* B = (const u16*)g.b;
+    if (bt.rank) {                                           // uniform over the workgroup: scalar arithmetic
+        u32 rest = blockIdx.y;
+        for (int d = (int)bt.rank - 1; d >= 0; --d) {
+            const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
+            A += (u64)c * bt.sa[d]; B += (u64)c * bt.sb[d];
+            rest = q;
+        }
+    }
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    u32x4 ra[CA], rb[CB];
+    auto load_global = [&](u64 k0) {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            const int c = tid + 256 * i;
+            if constexpr (AT) { const u64 k = k0 + c / (BM / 8), m = m0 + (c % (BM / 8)) * 8; ra[i] = (k < g.K && m < g.M) ? *(const u32x4*)(A + k * g.lda + m) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 m = m0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; ra[i] = (m < g.M && k < g.K) ? *(const u32x4*)(A + m * g.lda + k) : (u32x4){0, 0, 0, 0}; }
+        }
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const int c = tid + 256 * i;
+            if constexpr (BT) { const u64 k = k0 + c / (BN / 8), n = n0 + (c % (BN / 8)) * 8; rb[i] = (k < g.K && n < g.N) ? *(const u32x4*)(B + k * g.ldb + n) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 n = n0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; rb[i] = (n < g.N && k < g.K) ? *(const u32x4*)(B + n * g.ldb + k) : (u32x4){0, 0, 0, 0}; }
+        }
+    };
+    auto store_lds = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            const int c = tid + 256 * i;
+            *(u32x4*)(As + buf * SA + (AT ? (c / (BM / 8)) * PA + (c % (BM / 8)) * 8 : (c / (BK / 8)) * PK + (c % (BK / 8)) * 8)) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const int c = tid + 256 * i;
+            *(u32x4*)(Bs + buf * SB + (BT ? (c / (BN / 8)) * PB + (c % (BN / 8)) * 8 : (c / (BK / 8)) * PK + (c % (BK / 8)) * 8)) = rb[i];
+        }
+    };
+    // fragment addresses inside a stage for the wave's first 32 rows and the 16-wide K slice 0
+    const int j16 = lane & 15;
+    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM
+                       : (wm * WM + (lane & 31)) * PK + (lane >> 5) * 8;
+    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN
+                       : (wn * WN + (lane & 31)) * PK + (lane >> 5) * 8;
+
+    const u64 steps = (g.K + BK - 1) / BK;
+    const u64 first = (u64)blockIdx.z * sk.per_split;
+    const u64 last = first + sk.per_split < steps ? first + sk.per_split : steps;
+    if (first < last) {
+        load_global(first * BK);
+        store_lds(0);
+    }
+    __syncthreads();
+    for (u64 kt = first; kt < last; ++kt) {
+        const int buf = (int)((kt - first) & 1);
+        if (kt + 1 < last) load_global((kt + 1) * BK);
+        const u16* as = As + buf * SA + fa0;
+        const u16* bs = Bs + buf * SB + fb0;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            u32x4 fa[TI], fb[TJ];
+#pragma unroll
+            for (int i = 0; i < TI; ++i) {
+                if constexpr (AT) fa[i] = tr_fragment_lds<PA>(as + i * 32 + kk * 16 * PA); else fa[i] = *(const u32x4*)(as + i * 32 * PK + kk * 16);
+            }
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+                if constexpr (BT) fb[j] = tr_fragment_lds<PB>(bs + j * 32 + kk * 16 * PB); else fb[j] = *(const u32x4*)(bs + j * 32 * PK + kk * 16);
+            }
+#pragma unroll
+            for (int i = 0; i < TI; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) acc[i][j] = Mma16<T>::run(fa[i], fb[j], acc[i][j]);
+        }
+        if (kt + 1 < last) store_lds(buf ^ 1);
+        __syncthreads();
+    }
+
+    // accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
+    const u64 plane = g.M * g.N;
+    T* C = (T*)g.c + (u64)blockIdx.y * plane;
+    float* P = sk.splits > 1 ? sk.partial + ((u64)blockIdx.z * sk.matrices + blockIdx.y) * plane : nullptr;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const u64 col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const u64 row = m0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                if (row < g.M && col < g.N) {
+                    if (P) P[row * g.N + col] = acc[i][j][v];
+                    else C[row * g.N + col] = Mma16<T>::out(acc[i][j][v]);
+                }
+            }
+        }
+}
+
+// out[e] = the partial results of all K splits added in split order, rounded once.
+template <class T>
+__global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__ partial, T* __restrict__ out, u64 total, u32 splits)
+{
+    for (u64 e = (u64)blockIdx.x * 256 + threadIdx.x; e < total; e += (u64)gridDim.x * 256) {
+        float sum = partial[e];
+        for (u32 s = 1; s < splits; ++s) sum += partial[(u64)s * total + e];
+        out[e] = Mma16<T>::out(sum);
+    }
+}
+
 // ---- f32 operands ------------------------------------------------------------------------------
 // 128 x 128 (or 64 x 64) workgroup tile, BK = 32.  v_mfma_f32_32x32x2f32 takes one element per lane
 // and operand -- lane l holds A[row l % 32][k l / 32] -- so both operand forms feed it directly:
@@ -690,18 +848,134 @@ int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b
     return launch(gemm_small16_k<f16, true, true>, Small16<true, true>::kLds);
 }
 
+
+// K step of gemm_tile16_k by tile height: the 64 x 64 tile wants 64 (fewer barriers per byte; 1536^3 NT 25.7 -> 21.2 us),
+// the 128-row tiles 32 (more workgroups per compute unit; the transformer's shapes are 5 % faster overall).
+constexpr int tile16_bk(int bm) { return bm == 64 ? 64 : 32; }
+
+// gemm_tile16_k on the last two dims of a / b, `batch` as for launch_small16.  tile: 0 = 64 x 64, 1 = 128 x 64,
+// 2 = 128 x 128; splits: K splits wanted (1 = none).  -1: a layout the kernel does not take.
+int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch,
+                  int tile, uint64_t splits)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    constexpr size_t esz = 2;
+    const char* qa = (const char*)a->data + a->offset * esz;
+    const char* qb = (const char*)b->data + b->offset * esz;
+    const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 8 == 0;
+    const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 8 == 0;
+    const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
+    if (!((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && aligned16(qa) && aligned16(qb))) return -1;
+    BatchArgs bt{};
+    uint64_t count = 1;
+    if (batch) {
+        if (batch->rank > 3) return -1;
+        bt.rank = (u32)batch->rank;
+        for (int d = 0; d < batch->rank; ++d) {
+            if (batch->shape[d] >= (1ull << 31) || batch->stride[0][d] % 8 != 0 || batch->stride[1][d] % 8 != 0) return -1;
+            bt.ext[d] = (u32)batch->shape[d]; bt.sa[d] = batch->stride[0][d]; bt.sb[d] = batch->stride[1][d];
+            count *= batch->shape[d];
+        }
+        if (count > 65535) return -1;
+        bt.sc = M * N;
+    }
+    const uint64_t bm = tile == 0 ? 64 : 128, bn = tile == 2 ? 128 : 64;
+    GemmArgs g{};
+    g.a = qa; g.b = qb; g.c = out->data;
+    g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+    g.tiles_m = (u32)((M + bm - 1) / bm); g.tiles_n = (u32)((N + bn - 1) / bn);
+    const u32 n = g.tiles_m * g.tiles_n;
+    g.swizzle = n % 8u == 0 ? 1u : 0u;
+    const uint64_t bk = (uint64_t)tile16_bk((int)bm);
+    const uint64_t steps = (K + bk - 1) / bk;
+    if (splits > steps) splits = steps;
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    SplitArgs sk{};
+    sk.per_split = (u32)((steps + splits - 1) / splits);
+    sk.splits = (u32)((steps + sk.per_split - 1) / sk.per_split);
+    sk.matrices = count;
+    if (sk.splits > 1) {
+        void* ws;
+        AIXK_TRY(workspace(ctx, 0, (size_t)sk.splits * count * M * N * sizeof(float), &ws));
+        sk.partial = (float*)ws;
+    }
+    const bool at = !a_k, tb = !b_k;
+    auto launch = [&](auto kernel, size_t lds) {
+        AIXK_TRY(set_lds(kernel, lds));
+        hipLaunchKernelGGL(kernel, dim3(n, (unsigned)count, sk.splits), dim3(256), lds, ctx->stream, g, bt, sk);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    };
+    auto by_form = [&](auto dtype_tag, auto bm_tag, auto bn_tag) {
+        typedef decltype(dtype_tag) T;
+        constexpr int BM = decltype(bm_tag)::value, BN = decltype(bn_tag)::value, BK = tile16_bk(BM);
+        if (!at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, false>, Tile16<BM, BN, BK, false, false>::kLds);
+        if (!at && tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, true>, Tile16<BM, BN, BK, false, true>::kLds);
+        if (at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, true, false>, Tile16<BM, BN, BK, true, false>::kLds);
+        return launch(gemm_tile16_k<T, BM, BN, BK, true, true>, Tile16<BM, BN, BK, true, true>::kLds);
+    };
+    auto by_tile = [&](auto dtype_tag) {
+        if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{});
+        if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{});
+        return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{});
+    };
+    const int rc = out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
+    if (rc != AIXK_OK || sk.splits == 1) return rc;
+    const uint64_t total = count * M * N;
+    const unsigned blocks = grid_for(total, 256, (unsigned)ctx->cus * 16u);
+    if (out->dtype == AIXK_BF16) hipLaunchKernelGGL((splitk_finish_k<bf16>), dim3(blocks), dim3(256), 0, ctx->stream, (const float*)sk.partial, (bf16*)out->data, (u64)total, sk.splits);
+    else hipLaunchKernelGGL((splitk_finish_k<f16>), dim3(blocks), dim3(256), 0, ctx->stream, (const float*)sk.partial, (f16*)out->data, (u64)total, sk.splits);
+    AIXK_HIP(hipGetLastError());
+    return AIXK_OK;
+}
+
+// Which kernel multiplies 16-bit operands whose layouts are consumed in place (everything the LDS-direct kernel does
+// not take).  Measured on the shapes of a d = 768 transformer step at 8192 tokens, in microseconds, old route -> new:
+// [8192,768]x[768,768] 28 -> 23, [8192,3072]^T-free x [3072,768] 76 -> 67, weight gradients [768,8192]x[8192,768]
+// 73 -> 32 (8 K splits) and [768,8192]x[8192,3072] 113 -> 72 (4 splits), stacks of 192 attention products
+// [512,64]x[64,512] 121 -> 42, [512,512]x[512,64] 52 -> 27, [512,512]^T x [512,64] 92 -> 27.
+int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    const uint64_t cus = (uint64_t)ctx->cus;
+    uint64_t count = 1;
+    if (batch) for (int d = 0; d < batch->rank; ++d) count *= batch->shape[d];
+    const uint64_t t64 = ((M + 63) / 64) * ((N + 63) / 64), t128 = ((M + 127) / 128) * ((N + 127) / 128), t12864 = ((M + 127) / 128) * ((N + 63) / 64);
+    auto splits_for = [&](uint64_t groups, uint64_t steps, uint64_t fill) {        // long K, few workgroups: split K over workgroups
+        if (K < 4096 || groups >= fill * cus) return (uint64_t)1;
+        return std::max<uint64_t>(1, std::min<uint64_t>(steps / 16, (fill * cus + groups - 1) / groups));
+    };
+    if (batch) {
+        // stacks: thin results (attention's [seq, head dim]) on 128 x 64 tiles, everything else on 128 x 128
+        if (M <= 64) return launch_tile16(ctx, a, b, out, batch, 0, splits_for(t64 * count, (K + 63) / 64 * 2, 4));
+        if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, splits_for(t12864 * count, (K + 31) / 32, 2));
+        return launch_tile16(ctx, a, b, out, batch, 2, splits_for(t128 * count, (K + 31) / 32, 2));
+    }
+    if (t64 < 2 * cus) {
+        // outputs that 64 x 64 tiles cannot spread over the chip twice: with a long K, 64 x 64 tiles and K split over
+        // workgroups; otherwise 32 x 32 tiles with K split over the waves (1024^3 NN: 11.8 us against 12.7)
+        if (K >= 4096) return launch_tile16(ctx, a, b, out, nullptr, 0, splits_for(t64, (K + 63) / 64 * 2, 4));
+        return launch_small16(ctx, a, b, out, nullptr);
+    }
+    if (K >= 4096 && t128 < 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 2, splits_for(t128, (K + 31) / 32, 2));
+    if (t128 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
+    if (t12864 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 1, 1);
+    return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
+}
+
 } // namespace
 
 namespace aixk {
 
-// A stack of 16-bit products small enough for the 32 x 32 tiles, in one launch.  -1: not handled here.
+// A stack of 16-bit products that do not fill the chip one by one, in one launch.  -1: not handled here.
 int matmul_mfma_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>& batch)
 {
     const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
     if (aixk_dtype_size(out->dtype) != 2 || (out->dtype != AIXK_BF16 && out->dtype != AIXK_F16)) return -1;
     if (K % 8 != 0 || M * N < 64 * 64) return -1;                  // as for a single product
     if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 2) return -1;     // each product fills the chip by itself: one launch each
-    return launch_small16(ctx, a, b, out, &batch);
+    return route16(ctx, a, b, out, &batch);
 }
 
 int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)
@@ -749,11 +1023,9 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         }
     }
 
-    // 16-bit, outputs that 64 x 64 tiles cannot spread over the chip twice: 32 x 32 tiles, K split over the waves,
-    // every operand layout consumed where it lies (measured against the 64 x 64 route: 1024^3 NN 23.9 -> 15.2 us;
-    // beyond two tiles per compute unit the larger tiles win)
-    if (esz == 2 && ((M + 63) / 64) * ((N + 63) / 64) < (uint64_t)ctx->cus * 2) {
-        const int rc = launch_small16(ctx, a, b, out, nullptr);
+    // 16-bit, operands consumed where they lie (K-contiguous or T form): tiles and K splits by shape
+    if (esz == 2) {
+        const int rc = route16(ctx, a, b, out, nullptr);
         if (rc != -1) return rc;
     }
 

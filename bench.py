@@ -135,7 +135,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--extras", default="c1,c2,c3,c4",
-                    help="which of the other configurations to run besides the headline (comma list of c1, c2, c3, c4): "
+                    help="which of the other configurations to run besides the headline (comma list of c1, c2, c3, c4; c4loop / c4stack "
+                         "= one of c4's two ways of issuing attention): "
                          "lets a profiler run cover one workload at a time")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -282,7 +283,7 @@ def main():
             mlp["parity"] = {"checked_against": "cpu_baseline losses", "steps": cpu_steps, "max_rel_dev": float(rel.max()),
                              "ok": bool(rel.max() <= 1e-4), "rule": "|loss_gpu - loss_cpu| <= 1e-4 |loss_cpu| on the first steps"}
         extras.append(mlp)
-    if not args.no_extras and "c4" in chosen:
+    if not args.no_extras and chosen & {"c4", "c4loop", "c4stack"}:
         # configs[4]: decoder-only transformer forward + backward composed from device operators
         from aix_amd import drivers as GD
         from oracle import drivers as OD
@@ -298,6 +299,8 @@ def main():
         # views -- and (2) with matmul on [batch, heads, ...] stacks, which this device adds to that interface
         for stacked, how in ((False, "causal softmax attention as per-(batch, head) 2-D matmuls"),
                              (True, "causal softmax attention as matmuls on [batch, heads, seq, .] stacks (an extension of the interface)")):
+            if "c4" not in chosen and ("c4stack" if stacked else "c4loop") not in chosen:
+                continue
             losses, norms, secs = GD.transformer(dev, cfg, t_steps, data, stacked=stacked)
             steady = float(secs[1:].mean())
             tf = {"workload": "configs[4] decoder-only transformer forward+backward: 6 layers, d 768, 12 heads, seq 512, batch 16, vocab 8192, "

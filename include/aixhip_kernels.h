@@ -145,7 +145,8 @@ int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
 /* An extension of the above: the reference multiplies 2-D operands only (aixCore.hpp:943-976), so an
  * AIX program issues attention as one matmul per (sequence, head) on sliced views.  Here a, b and out
  * may carry the same leading dims in front of the matrix dims: out[..., m, n] = a[..., m, k] . b[..., k, n],
- * one product per index of the leading dims, exactly what the 2-D entry point computes for each.
+ * one product per index of the leading dims, what the 2-D entry point computes for each (f32 accumulation,
+ * one rounding; the order in which the f32 partial sums are added may differ from the 2-D route's).
  * a and b may be any views (permuted, sliced, stride 0); the results are written densely from
  * out->data.  Stacks of small 16-bit products run as ONE launch; everything else is issued product by
  * product through the 2-D entry point.  Rank 2 is the 2-D entry point. */

@@ -666,7 +666,10 @@ def _matrix_of(ht, index):
 
 def check_matmul_stack(gpu, a, b, what, against_each=True):
     """aixk_matmul_batched against (1) the oracle's stack -- integers bit for bit, floats within the matmul bar of
-    the exactly accumulated products -- and (2) aixk_matmul issued matrix by matrix on the same views, bit for bit."""
+    the exactly accumulated products -- and (2) aixk_matmul issued matrix by matrix on the same views: bit for bit
+    where the stack is issued product by product (f32, integers); the one-launch 16-bit route may add the f32
+    partial sums in another order than the 2-D route picks for a single small product, so there the two agree to
+    f32 accumulation error plus the final rounding."""
     dtype = a.dtype
     lead, m, k, n = a.shape[:-2], a.shape[-2], a.shape[-1], b.shape[-1]
     count = int(np.prod(lead))
@@ -691,7 +694,13 @@ def check_matmul_stack(gpu, a, b, what, against_each=True):
             G.assert_close_to_wide(O.to_float64(mine, dtype), exact, scale + 1e-30, tol, f"{what} matrix {index}")
         if against_each:
             G.run_gpu(gpu, "aixk_matmul", G.ref(G.kdesc(a2, pa)), G.ref(G.kdesc(b2, pb)), G.ref(d1))
-            T.assert_same_bits(mine, gpu.fetch(p1, mine), f"{what} matrix {index} against the 2-D entry point")
+            single = gpu.fetch(p1, mine)
+            if dtype in (O.F16, O.BF16):
+                final = 2.0 ** -10 if dtype == O.F16 else 2.0 ** -8
+                G.assert_close_to_wide(O.to_float64(mine, dtype), O.to_float64(single, dtype), 1e-5 * scale + final * np.abs(exact) + 1e-30, 1.0,
+                                       f"{what} matrix {index} against the 2-D entry point")
+            else:
+                T.assert_same_bits(mine, single, f"{what} matrix {index} against the 2-D entry point")
 
 
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16, O.F32, O.I32], ids=ids)
