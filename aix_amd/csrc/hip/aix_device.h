@@ -241,7 +241,14 @@ template <class T> __device__ __forceinline__ T int_pow(T base, T e)
 template <class T> __device__ __forceinline__ T e_pow(T a, T b)
 {
     if constexpr (traits<T>::code == DT_F64) return pow(a, b);
-    else if constexpr (traits<T>::is_float) return down<T>(powf(up(a), up(b)));
+    else if constexpr (traits<T>::is_float) {
+        // squares and cubes (GELU's x^3 and its derivative) as products: two roundings at most, inside the 2 ulp of
+        // powf, a fraction of its cost; the exponent usually is one scalar for the whole tensor, so the branch is uniform
+        const float x = up(a), e = up(b);
+        if (e == 2.0f) return down<T>(x * x);
+        if (e == 3.0f) return down<T>(x * x * x);
+        return down<T>(powf(x, e));
+    }
     else return int_pow<T>(a, b);
 }
 

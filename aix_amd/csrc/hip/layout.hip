@@ -170,6 +170,31 @@ __global__ __launch_bounds__(kBlock) void tri_k(const W* __restrict__ src, W* __
     }
 }
 
+// Dense source and destination, rows of whole 16-byte vectors: a lane owns one vector (all of it in one row), reads it
+// only if some of it is kept and writes 16 bytes; the zeroed triangle is never read.
+template <class W>
+__global__ __launch_bounds__(kBlock) void tri_vec_k(const W* __restrict__ src, W* __restrict__ dst, u64 nvec, u64 rows, u64 cols, i64 diagonal, int upper)
+{
+    constexpr int VEC = 16 / sizeof(W);
+    typedef vec<W, VEC> V;
+    const u64 v = (u64)blockIdx.x * kBlock + threadIdx.x;
+    if (v >= nvec) return;
+    const u64 i = v * VEC;
+    const i64 r = (i64)((i / cols) % rows), c = (i64)(i % cols);
+    const i64 edge = r + diagonal;                       // lower: columns above `edge` are zeroed; upper: columns below it
+    const bool none = upper ? (c + VEC - 1 < edge) : (c > edge);
+    V x;
+    if (none) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x.v[e] = (W)0;
+    } else {
+        x = *(const V*)(src + i);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) if (upper ? (c + e < edge) : (c + e > edge)) x.v[e] = (W)0;
+    }
+    *(V*)(dst + i) = x;
+}
+
 // ---- indexSelect -------------------------------------------------------------------------------
 template <class W, class IDX>
 __global__ __launch_bounds__(kBlock) void index_select_k(const W* __restrict__ src, W* __restrict__ dst, const i32* __restrict__ idx,
@@ -411,6 +436,15 @@ int32_t aixk_tri(aixk_ctx* ctx, int upper, const aixhip_tensor* src, const aixhi
     const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(dst) < (1ull << 31);
     return by_size(src->dtype, [&](auto tag) {
         typedef decltype(tag) W;
+        constexpr uint64_t VEC = 16 / sizeof(W);
+        const bool dense = (ssp.rank == 0 || (ssp.rank == 1 && ssp.stride[0][0] == 1)) && (dsp.rank == 0 || (dsp.rank == 1 && dsp.stride[0][0] == 1));
+        const W* ps = (const W*)src->data + ssp.offset[0];
+        W* pd = (W*)dst->data + dsp.offset[0];
+        if (dense && cols % VEC == 0 && aligned16(ps) && aligned16(pd) && n / VEC / kBlock < (1ull << 31)) {
+            hipLaunchKernelGGL((tri_vec_k<W>), dim3((unsigned)((n / VEC + kBlock - 1) / kBlock)), dim3(kBlock), 0, ctx->stream, ps, pd, (u64)(n / VEC), (u64)rows, (u64)cols, (i64)diagonal, upper);
+            AIXK_HIP(hipGetLastError());
+            return (int)AIXK_OK;
+        }
         const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
         if (small) hipLaunchKernelGGL((tri_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n, (u64)rows, (u64)cols, (i64)diagonal, upper);
         else hipLaunchKernelGGL((tri_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n, (u64)rows, (u64)cols, (i64)diagonal, upper);

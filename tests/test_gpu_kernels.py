@@ -86,6 +86,25 @@ def test_binary_views(gpu, op, dtype):
     gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16], ids=ids)
+def test_pow_squares_and_cubes(gpu, dtype):
+    """Exponents 2 and 3 are evaluated as products (GELU's x^3 and its derivative): the same bar as every other
+    pow against the CPU's long-double powl, over signs, zeros, tiny and huge bases, infinities and NaN, with the
+    exponent as a broadcast scalar and as a full tensor that mixes 2, 3 and other exponents."""
+    rng = np.random.default_rng(11900 + dtype)
+    n = 4096
+    base = np.concatenate([rng.uniform(-30, 30, n - 24), [0.0, -0.0, 1.0, -1.0, 1e-13, -1e-13, 1e-20, 3e12, -3e12, 1e19, -1e19, 2.5e38,
+                                                           np.inf, -np.inf, np.nan, 65504.0, -65504.0, 6e-8, 255.0, -255.0, 0.5, -0.5, 1e-5, -1e-5]])
+    a = T.HostTensor(O.to_storage(base, dtype), dtype, [n])
+    for e in (2.0, 3.0):
+        b = T.HostTensor(O.to_storage(np.array([e]), dtype), dtype, [n], [0])
+        check_binary(gpu, O.POW, a, b, f"pow {NAMES[dtype]} exponent {e} (scalar)")
+    mixed = T.HostTensor(O.to_storage(rng.choice([2.0, 3.0, 2.5, -1.0, 0.0, 1.0], n), dtype), dtype, [n])
+    positive = T.HostTensor(O.to_storage(np.abs(base) + 0.05, dtype), dtype, [n])
+    check_binary(gpu, O.POW, positive, mixed, f"pow {NAMES[dtype]} mixed exponents")
+    gpu.release()
+
+
 @pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
 def test_binary_sizes_and_broadcast_rows(gpu, dtype):
     """Flat sizes 1..2049 (vector body + tail) and the row / column / scalar broadcast forms the
@@ -653,6 +672,24 @@ def test_matmul_identity_and_ones(gpu):
         G.run_gpu(gpu, "aixk_matmul", G.ref(d1), G.ref(d2), G.ref(do))
         got = O.to_float64(gpu.fetch(po, np.zeros(70 * 90, O.NP_STORAGE[dtype])), dtype)
         assert np.all(got == 200.0), f"ones.ones {NAMES[dtype]}"
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
+def test_tri_on_dense_stacks(gpu, dtype):
+    """tril / triu of dense tensors whose rows are whole 16-byte vectors (a stack of attention score matrices):
+    the vector kernel, every diagonal from all-zero to all-kept, vectors that straddle the edge."""
+    rng = np.random.default_rng(26000 + dtype)
+    for shape in ([2, 3, 24, 32], [40, 48], [5, 16, 64]):
+        src = T.contiguous_tensor(rng, dtype, shape, int_span=50)
+        _, dsrc = gpu.put(src)
+        for upper in (0, 1):
+            for diag in (-shape[-2] - 1, -7, -1, 0, 1, 5, 13, shape[-1] + 1):
+                want = T.empty(dtype, shape, fill=3)
+                okc((CPU.triu if upper else CPU.tril)(C.byref(src.desc()), C.byref(want.desc()), diag))
+                pd, dd = gpu.put(T.empty(dtype, shape, fill=3))
+                G.run_gpu(gpu, "aixk_tri", upper, G.ref(dsrc), G.ref(dd), diag)
+                T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, f"tri upper={upper} {NAMES[dtype]} {shape} diag={diag}")
         gpu.release()
 
 
