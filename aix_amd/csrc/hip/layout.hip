@@ -8,6 +8,8 @@
 
 #include "common.hpp"
 
+#include <utility>
+
 using namespace aixd;
 using namespace aixk;
 
@@ -55,6 +57,33 @@ __global__ __launch_bounds__(kBlock) void gather_rows_k(const W* __restrict__ sr
         const IDX col = (IDX)(c - (u64)row * chunks) * VEC;
         const u64 p = locate<IDX>(outer, row) + col;
         *(V*)(dst + c * VEC) = *(const V*)(src + p);
+    }
+}
+
+// rows again, walked in the order of the SOURCE: when consecutive destination rows are far apart in the source (heads
+// and positions swapped: 64 KB hops that keep landing on the same memory channel) but consecutive source rows are
+// close together in the destination, the lanes follow the source and scatter whole rows instead.  dims: outermost
+// first, the last one varies fastest; both offsets in elements.
+struct RowWalk {
+    int rank;
+    u64 ext[kMaxDims], src[kMaxDims], dst[kMaxDims];
+    u64 src_off;
+};
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void permute_rows_k(const W* __restrict__ src, W* __restrict__ dst, RowWalk w, u64 total_chunks, IDX chunks)
+{
+    typedef typename vec16<W>::type V;
+    constexpr int VEC = vec16<W>::n;
+    for (u64 c = (u64)blockIdx.x * kBlock + threadIdx.x; c < total_chunks; c += (u64)gridDim.x * kBlock) {
+        IDX row = (IDX)(c / chunks);
+        const IDX col = (IDX)(c - (u64)row * chunks) * VEC;
+        u64 ps = w.src_off + col, pd = col;
+        for (int d = w.rank - 1; d >= 0; --d) {
+            const IDX ext = (IDX)w.ext[d], q = row / ext, k = row - q * ext;
+            ps += (u64)k * w.src[d]; pd += (u64)k * w.dst[d];
+            row = q;
+        }
+        *(V*)(dst + pd) = *(const V*)(src + ps);
     }
 }
 
@@ -301,6 +330,24 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
             if (ok) {
                 const uint64_t chunks = sp.shape[in] / VEC, total = n / VEC;
                 const unsigned grid = grid_for(total, kBlock, max_blocks);
+                // the walk in source order, if its hop between consecutive rows (in the destination) is the shorter one
+                if (in >= 2) {
+                    RowWalk w{};
+                    w.rank = in; w.src_off = sp.offset[0];
+                    uint64_t run = sp.shape[in];
+                    bool plain = true;
+                    for (int d = in - 1; d >= 0; --d) { w.ext[d] = sp.shape[d]; w.src[d] = sp.stride[0][d]; w.dst[d] = run; run *= sp.shape[d]; if (sp.stride[0][d] == 0) plain = false; }
+                    const uint64_t hop_here = w.src[in - 1] * sizeof(W);
+                    for (int i = 1; i < in; ++i)                       // insertion sort by source stride, largest first
+                        for (int j = i; j > 0 && w.src[j] > w.src[j - 1]; --j) { std::swap(w.ext[j], w.ext[j - 1]); std::swap(w.src[j], w.src[j - 1]); std::swap(w.dst[j], w.dst[j - 1]); }
+                    const uint64_t hop_there = w.dst[in - 1] * sizeof(W);
+                    if (plain && hop_here >= 4096 && hop_there < hop_here) {
+                        if (small) hipLaunchKernelGGL((permute_rows_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u32)chunks);
+                        else hipLaunchKernelGGL((permute_rows_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u64)chunks);
+                        AIXK_HIP(hipGetLastError());
+                        return (int)AIXK_OK;
+                    }
+                }
                 if (small) hipLaunchKernelGGL((gather_rows_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u32)chunks);
                 else hipLaunchKernelGGL((gather_rows_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u64)chunks);
                 AIXK_HIP(hipGetLastError());

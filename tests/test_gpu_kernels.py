@@ -281,6 +281,35 @@ def test_contiguous_and_transpose(gpu, dtype):
         gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.I8, O.F64], ids=ids)
+def test_contiguous_of_permuted_rows(gpu, dtype):
+    """Copies whose unit of movement is a whole row while the dims in front of it are permuted -- attention's
+    [batch, heads, seq, d] <-> [batch, seq, heads, d] -- with hops of 4 KB and more between consecutive rows on the
+    source side: walked in source order.  Also a permutation of three leading dims, a sliced source with an offset,
+    and the mirror case (short hops in the source), which stays on the destination-order kernel."""
+    rng = np.random.default_rng(16500 + dtype)
+    esz = np.dtype(O.NP_STORAGE[dtype]).itemsize
+    d = 64 // esz * 2                                                   # rows of 128 bytes
+    for (B, H, S) in ((2, 3, 40), (1, 5, 33)):
+        stored = T.random_values(rng, B * H * S * d + 3 * d, dtype, int_span=100)
+        views = {
+            "heads<->seq": T.HostTensor(stored, dtype, [B, S, H, d], [H * S * d, d, S * d, 1]),
+            "seq<->heads, short hops": T.HostTensor(stored, dtype, [B, H, S, d], [H * S * d, d, H * d, 1]),
+            "offset": T.HostTensor(stored, dtype, [B, S, H, d], [H * S * d, d, S * d, 1], offset=2 * d),
+        }
+        big = T.random_values(rng, 3 * 4 * 5 * 2 * 4096 // esz, dtype, int_span=100)
+        row = 4096 // esz
+        views["three dims"] = T.HostTensor(big, dtype, [5, 4, 3, 2, d], [2 * row, 5 * 2 * row, 4 * 5 * 2 * row, row, 1])
+        for name, src in views.items():
+            want = T.empty(dtype, src.shape)
+            okc(CPU.contiguous(C.byref(src.desc()), C.byref(want.desc())))
+            _, ds = gpu.put(src)
+            po, do = gpu.put(T.empty(dtype, src.shape))
+            G.run_gpu(gpu, "aixk_contiguous", G.ref(ds), G.ref(do))
+            T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"contiguous {NAMES[dtype]} {name} {src.shape} strides={src.strides}")
+        gpu.release()
+
+
 @pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
 def test_slice_set_tri_index_ops(gpu, dtype):
     rng = np.random.default_rng(17000 + dtype)
