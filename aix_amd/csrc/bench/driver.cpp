@@ -134,19 +134,27 @@ int aixbench_reduce_item(aixhip_device* handle, int which, uint64_t rows, uint64
 // Config 2: C = A[M,K] . B[K,N]; element type dtype (1 f32, 2 f16, 3 bf16); a, b are host arrays of
 // that type.  layout: 0 NN, 1 NT (b given as [N,K], used through a transposed view), 2 TN (a given
 // as [K,M]).  batch > 1: a, b hold `batch` matrices and each step issues `batch` matmuls on
-// select(0, i) views, as the interface has no batch dim.
+// select(0, i) views, as the interface has no batch dim; layout + 4: ONE matmul on the [batch, ., .] stacks instead
+// (the extension of matmul to operands with leading dims).
 int aixbench_matmul(aixhip_device* handle, int dtype, uint64_t M, uint64_t N, uint64_t K, int layout, uint64_t batch,
                     const void* a, const void* b, int steps, int warmup, aixbench_result* res, void* out)
 {
     return guarded([&] {
         DeviceHIP* dev = aix::hip::fromHandle(handle);
         const DataType dt = static_cast<DataType>(dtype);
+        const bool stacked = (layout & 4) != 0;
+        layout &= 3;
         const Shape sa = layout == 2 ? Shape{batch, K, M} : Shape{batch, M, K};
         const Shape sb = layout == 1 ? Shape{batch, N, K} : Shape{batch, K, N};
         Value A = Value::fromHost(dev, dt, sa, a);
         Value B = Value::fromHost(dev, dt, sb, b);
         std::vector<Value> r(batch);
         auto step = [&] {
+            if (stacked) {
+                r[0] = (layout == 2 ? A.transpose(1, 2) : A).matmul(layout == 1 ? B.transpose(1, 2) : B);
+                dev->flush();
+                return;
+            }
             for (uint64_t i = 0; i < batch; ++i) {
                 Value ai = A.select0(i), bi = B.select0(i);
                 if (layout == 2) ai = ai.transpose(0, 1);

@@ -27,17 +27,21 @@ typedef long long          i64;
 typedef unsigned long long u64;
 typedef _Float16           f16;
 
-// bfloat16 storage word.  Conversion is done on the integer image so that NaN handling is the
-// reference's: truncate and set bit 6 (aixFloat16.hpp:783-805).
+// bfloat16 storage word.  f32 -> bf16 is the hardware conversion (v_cvt_pk_bf16_f32): round to nearest even,
+// and a NaN keeps its upper payload bits and gets bit 6 set -- on every one of the 2^32 inputs the value the
+// reference computes on the integer image, ((u + 0x7FFF + ((u >> 16) & 1)) >> 16, NaN: (u >> 16) | 0x40;
+// aixFloat16.hpp:783-805), in one instruction instead of seven.
 struct bf16 { u16 bits; };
 
 __device__ __forceinline__ float bf16_up(bf16 v) { return __builtin_bit_cast(float, (u32)v.bits << 16); }
 __device__ __forceinline__ bf16 bf16_down(float f)
 {
-    const u32 u = __builtin_bit_cast(u32, f);
+    // through inline assembly: given the conversion as an fptrunc, this compiler's instruction selection fails on
+    // some negations that feed it
+    u32 packed;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %1" : "=v"(packed) : "v"(f));
     bf16 r;
-    if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu)) { r.bits = (u16)((u >> 16) | 0x40u); return r; }
-    r.bits = (u16)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);        // round to nearest even
+    r.bits = (u16)packed;
     return r;
 }
 

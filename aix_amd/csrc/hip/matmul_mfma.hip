@@ -75,14 +75,7 @@ template <class T> struct Mma16;
 template <> struct Mma16<bf16> {
     static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c)
     { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0); }
-    static __device__ __forceinline__ bf16 out(float v)       // bf16_down without a branch (the epilogue holds 256 live accumulators)
-    {
-        const u32 u = __builtin_bit_cast(u32, v);
-        const bool nan = (u & 0x7FFFFFFFu) > 0x7F800000u;
-        bf16 r;
-        r.bits = (u16)(nan ? ((u >> 16) | 0x40u) : ((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16));
-        return r;
-    }
+    static __device__ __forceinline__ bf16 out(float v) { return bf16_down(v); }
     static __device__ __forceinline__ u32 pack(float lo, float hi) { return (u32)out(lo).bits | ((u32)out(hi).bits << 16); }
 };
 template <> struct Mma16<f16> {

@@ -240,14 +240,16 @@ def main():
         sweep = [("f32", 4096, "NN", 1, 20), ("bf16", 4096, "NN", 1, 20), ("f16", 4096, "NN", 1, 20),
                  ("bf16", 4096, "NT", 1, 20), ("bf16", 4096, "TN", 1, 20), ("f32", 4096, "NT", 1, 20),
                  ("bf16", 1024, "NN", 1, 50), ("bf16", 8192, "NN", 1, 5), ("f32", 1024, "NN", 1, 50), ("f32", 8192, "NN", 1, 3),
-                 ("bf16", 512, "NN", 64, 20)]
+                 ("bf16", 512, "NN", 64, 20), ("bf16", 512, "NN", -64, 20)]
         for dt_name, m, lay, batch, steps_mm in sweep:
+            stacked, batch = batch < 0, abs(batch)                 # negative: one matmul on the [batch, m, m] stacks
             ha, hb = operands(dt_name, m, batch)
             r = BenchResult()
-            run(lib, "aixbench_matmul", dev.handle, codes[dt_name], m, m, m, layouts[lay], batch, ha.ctypes.data, hb.ctypes.data,
+            run(lib, "aixbench_matmul", dev.handle, codes[dt_name], m, m, m, layouts[lay] + (4 if stacked else 0), batch, ha.ctypes.data, hb.ctypes.data,
                 steps_mm, 2, C.byref(r), None)
             flops = 2.0 * m * m * m * batch
-            what = f"{m}^3" if batch == 1 else f"{batch} x [{m},{m}]x[{m},{m}] (one matmul call per select(0,i) view)"
+            what = f"{m}^3" if batch == 1 else f"{batch} x [{m},{m}]x[{m},{m}] " + (
+                "(one matmul call on the [64, 512, 512] stacks: an extension of the interface)" if stacked else "(one matmul call per select(0,i) view)")
             extras.append({"workload": f"configs[2] matmul {dt_name} {what} {lay} (f32 accumulation)",
                            "ms_per_step": round(r.wall_s * 1e3 / steps_mm, 5),
                            "value": round(flops * steps_mm / r.wall_s / 1e12, 2), "unit": "TFLOP/s",

@@ -246,6 +246,25 @@ def test_cast_and_fill(gpu, src):
     gpu.release()
 
 
+def test_f32_to_bf16_every_class_of_input(gpu):
+    """The device rounds f32 to bf16 with the hardware conversion; the reference does it on the integer image
+    (aixFloat16.hpp:783-805: round to nearest even; NaN = upper half with bit 6 set).  All 65 536 upper halves
+    x 48 lower halves (the rounding boundary and its neighbours, zero, all ones, random) -- every exponent,
+    every NaN payload class, infinities, subnormals -- must give the same 16 bits, NaN payloads included."""
+    rng = np.random.default_rng(15500)
+    low = np.concatenate([np.array([0, 1, 2, 0x7FFE, 0x7FFF, 0x8000, 0x8001, 0x8002, 0xFFFE, 0xFFFF, 0x4000, 0xC000], np.uint32),
+                          rng.integers(0, 0x10000, 36).astype(np.uint32)])
+    bits = ((np.arange(0x10000, dtype=np.uint32)[:, None] << 16) | low[None, :]).reshape(-1)
+    src = bits.view(np.float32)
+    want = np.zeros(src.size, np.uint16)
+    okc(CPU.copy(src.ctypes.data, O.F32, want.ctypes.data, O.BF16, src.size))
+    ps, pd = gpu.raw(src.nbytes), gpu.raw(want.nbytes)
+    gpu.ctx.upload(ps, src)
+    G.run_gpu(gpu, "aixk_cast", ps, O.F32, pd, O.BF16, src.size)
+    T.assert_same_bits(gpu.fetch(pd, want), want, "f32 -> bf16")
+    gpu.release()
+
+
 # ---- data movement --------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
 def test_contiguous_and_transpose(gpu, dtype):
