@@ -52,15 +52,19 @@ struct aixk_ctx {
     hipStream_t stream{nullptr};
     hipDeviceProp_t prop{};
     int cus{256};
-    // scratch for multi-block reductions: partial results + a completion counter (zeroed at
-    // creation; the last block of each reduction resets it).
+    // scratch for multi-block reductions: partial results
     void* scratch{nullptr};
     size_t scratch_bytes{0};
+    // 256 bytes of flags, zeroed at creation.  Word 0: set to `gemm_seq` by a split-plane f32 matmul that met an
+    // infinity or a NaN in its operands (the IEEE-faithful kernel then redoes the product); launches are numbered,
+    // so the word never has to be cleared.
     unsigned int* counter{nullptr};
+    unsigned int gemm_seq{0};
     // matmul: K-contiguous copies of operands whose layout the kernels cannot consume in place
-    // (A and B); grown on demand, ordered on `stream` like everything else
-    void* gemm_ws[2]{nullptr, nullptr};
-    size_t gemm_ws_bytes[2]{0, 0};
+    // (0: A, 1: B) and the f32 partial results of K splits (2); grown on demand, ordered on `stream`
+    // like everything else
+    void* gemm_ws[3]{nullptr, nullptr, nullptr};
+    size_t gemm_ws_bytes[3]{0, 0, 0};
     // runtime-compiled kernels by signature
     std::unordered_map<std::string, aixk_module*> rtc;
     uint64_t rtc_hits{0}, rtc_misses{0};

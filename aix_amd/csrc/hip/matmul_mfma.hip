@@ -626,6 +626,186 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
     }
 }
 
+// ---- f32 operands on the bf16 matrix pipe ------------------------------------------------------------
+// The f32 MFMA runs at 1/16 of the bf16 rate.  An f32 value is the exact sum of three bf16 values (8 + 8 + 8
+// significand bits: hi = x truncated to its upper 16 bits, mid = RNE(x - hi), lo = RNE(x - hi - mid); the exponent
+// range is the same, so nothing overflows or underflows that f32 itself does not), and a product of two bf16 values
+// is exact in f32.  So A . B = sum over the six plane pairs (hi hi, hi mid, mid hi, mid mid, hi lo, lo hi) of bf16
+// MFMAs accumulating in f32; the three pairs left out (mid lo, lo mid, lo lo) are below 2^-23 of |a| |b| per term --
+// the size of f32's own rounding of a product -- and the accumulation is the f32 accumulation of the matrix unit
+// either way.  Six bf16 MFMAs cost 6/16 of one f32 MFMA of the same shape.
+//
+// gemm_x3_k: 128 x 128 x 32 tile, four waves 2 x 2.  The operands are read from memory as f32 (K-contiguous or T
+// form, 16-byte chunks of four values), split in registers, and staged as three bf16 planes per operand with the
+// layouts of gemm_tile16_k (so the fragment reads, including ds_read_b64_tr_b16 for T-form operands, are the same);
+// a wave reads 12 fragments per 24 MFMAs.  One LDS stage of 60 KB (two workgroups per compute unit) and two barriers
+// per K step: the next step's global loads are in flight during the MFMAs.  blockIdx.z numbers K splits as in
+// gemm_tile16_k.
+//
+// Infinities and NaNs do not survive the split (inf - inf, and inf times a zero mid or lo plane of the other operand):
+// a lane that loads one stores the launch's number into a flag word, and the f32 MFMA kernel that is always launched
+// right behind -- its workgroups return at once unless the flag carries this number -- redoes the whole product with
+// IEEE arithmetic.
+template <bool AT, bool BT> struct TileX3 {
+    static constexpr int BM = 128, BN = 128, BK = 32, PK = BK + 8, PA = BM + 32, PB = BN + 32;
+    static constexpr int SA = AT ? BK * PA : BM * PK, SB = BT ? BK * PB : BN * PK;       // bf16 elements per plane
+    static constexpr size_t kLds = (size_t)3 * (SA + SB) * 2;
+};
+
+__device__ __forceinline__ u32 cvt_pk_bf16(float lo, float hi)
+{
+    u32 r;
+    asm("v_cvt_pk_bf16_f32 %0, %1, %2" : "=v"(r) : "v"(lo), "v"(hi));
+    return r;
+}
+
+// four f32 -> three word pairs of four bf16 (element e in bits 16 (e & 1) of word e / 2)
+__device__ __forceinline__ bool all_finite(const u32x4 x)
+{
+    return ((x.x & 0x7F800000u) != 0x7F800000u) && ((x.y & 0x7F800000u) != 0x7F800000u) && ((x.z & 0x7F800000u) != 0x7F800000u) && ((x.w & 0x7F800000u) != 0x7F800000u);
+}
+__device__ __forceinline__ void split3(const u32x4 x, u32x2& h, u32x2& m, u32x2& l)
+{
+    const u32 xs[4] = {x.x, x.y, x.z, x.w};
+    float r[4];
+    u32 hb[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { hb[e] = xs[e] & 0xFFFF0000u; r[e] = __builtin_bit_cast(float, xs[e]) - __builtin_bit_cast(float, hb[e]); }
+    h.x = (hb[0] >> 16) | hb[1]; h.y = (hb[2] >> 16) | hb[3];
+    m.x = cvt_pk_bf16(r[0], r[1]); m.y = cvt_pk_bf16(r[2], r[3]);
+    const float s0 = r[0] - __builtin_bit_cast(float, m.x << 16), s1 = r[1] - __builtin_bit_cast(float, m.x & 0xFFFF0000u);
+    const float s2 = r[2] - __builtin_bit_cast(float, m.y << 16), s3 = r[3] - __builtin_bit_cast(float, m.y & 0xFFFF0000u);
+    l.x = cvt_pk_bf16(s0, s1); l.y = cvt_pk_bf16(s2, s3);
+}
+
+template <bool AT, bool BT>
+__global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* flag, u32 seq)
+{
+    typedef TileX3<AT, BT> S;
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, PK = S::PK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
+    constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
+    constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;        // 16-byte chunks (4 values) per lane and step
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_x3[];
+    u16* As = (u16*)smem_x3;                              // [3][SA]
+    u16* Bs = As + 3 * SA;                                // [3][SB]
+
+    u32 tm, tn;
+    tile_of(g, tm, tn);
+    const u64 m0 = (u64)tm * BM, n0 = (u64)tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const float* A = (const float*)g.a;
+    const float* B = (const float*)g.b;
+
+    f32x16 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    u32x4 ra[CA], rb[CB];
+    auto load_global = [&](u64 k0) {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            const int c = tid + 256 * i;
+            if constexpr (AT) { const u64 k = k0 + c / (BM / 4), m = m0 + (c % (BM / 4)) * 4; ra[i] = (k < g.K && m < g.M) ? *(const u32x4*)(A + k * g.lda + m) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 m = m0 + c / (BK / 4), k = k0 + (c % (BK / 4)) * 4; ra[i] = (m < g.M && k < g.K) ? *(const u32x4*)(A + m * g.lda + k) : (u32x4){0, 0, 0, 0}; }
+        }
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const int c = tid + 256 * i;
+            if constexpr (BT) { const u64 k = k0 + c / (BN / 4), n = n0 + (c % (BN / 4)) * 4; rb[i] = (k < g.K && n < g.N) ? *(const u32x4*)(B + k * g.ldb + n) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 n = n0 + c / (BK / 4), k = k0 + (c % (BK / 4)) * 4; rb[i] = (n < g.N && k < g.K) ? *(const u32x4*)(B + n * g.ldb + k) : (u32x4){0, 0, 0, 0}; }
+        }
+    };
+    auto store_lds = [&] {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) {
+            const int c = tid + 256 * i;
+            const int at = AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
+            u32x2 h, m, l;
+            if (!all_finite(ra[i])) *flag = seq;
+            split3(ra[i], h, m, l);
+            *(u32x2*)(As + at) = h; *(u32x2*)(As + SA + at) = m; *(u32x2*)(As + 2 * SA + at) = l;
+        }
+#pragma unroll
+        for (int i = 0; i < CB; ++i) {
+            const int c = tid + 256 * i;
+            const int at = BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
+            u32x2 h, m, l;
+            if (!all_finite(rb[i])) *flag = seq;
+            split3(rb[i], h, m, l);
+            *(u32x2*)(Bs + at) = h; *(u32x2*)(Bs + SB + at) = m; *(u32x2*)(Bs + 2 * SB + at) = l;
+        }
+    };
+    const int j16 = lane & 15;
+    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM
+                       : (wm * WM + (lane & 31)) * PK + (lane >> 5) * 8;
+    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN
+                       : (wn * WN + (lane & 31)) * PK + (lane >> 5) * 8;
+
+    const u64 steps = (g.K + BK - 1) / BK;
+    const u64 first = (u64)blockIdx.z * sk.per_split;
+    const u64 last = first + sk.per_split < steps ? first + sk.per_split : steps;
+    if (first < last) load_global(first * BK);
+    for (u64 kt = first; kt < last; ++kt) {
+        store_lds();
+        __syncthreads();
+        if (kt + 1 < last) load_global((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            u32x4 fa[3][TI], fb[3][TJ];
+#pragma unroll
+            for (int p = 0; p < 3; ++p) {
+#pragma unroll
+                for (int i = 0; i < TI; ++i) {
+                    const u16* q = As + p * SA + fa0;
+                    if constexpr (AT) fa[p][i] = tr_fragment_lds<PA>(q + i * 32 + kk * 16 * PA); else fa[p][i] = *(const u32x4*)(q + i * 32 * PK + kk * 16);
+                }
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) {
+                    const u16* q = Bs + p * SB + fb0;
+                    if constexpr (BT) fb[p][j] = tr_fragment_lds<PB>(q + j * 32 + kk * 16 * PB); else fb[p][j] = *(const u32x4*)(q + j * 32 * PK + kk * 16);
+                }
+            }
+            // smallest contributions first; four independent accumulators between two uses of the same one
+            constexpr int pa[6] = {2, 0, 1, 1, 0, 0}, pb[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+            for (int t = 0; t < 6; ++t)
+#pragma unroll
+                for (int i = 0; i < TI; ++i)
+#pragma unroll
+                    for (int j = 0; j < TJ; ++j) acc[i][j] = Mma16<bf16>::run(fa[pa[t]][i], fb[pb[t]][j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+
+    const u64 plane = g.M * g.N;
+    float* C = sk.splits > 1 ? sk.partial + (u64)blockIdx.z * plane : (float*)g.c;
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) {
+            const u64 col = n0 + wn * WN + j * 32 + (lane & 31);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const u64 row = m0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
+                if (row < g.M && col < g.N) C[row * g.N + col] = acc[i][j][v];
+            }
+        }
+}
+
+__global__ __launch_bounds__(256) void splitk_finish_f32_k(const float* __restrict__ partial, float* __restrict__ out, u64 total, u32 splits)
+{
+    for (u64 e = (u64)blockIdx.x * 256 + threadIdx.x; e < total; e += (u64)gridDim.x * 256) {
+        float sum = partial[e];
+        for (u32 s = 1; s < splits; ++s) sum += partial[(u64)s * total + e];
+        out[e] = sum;
+    }
+}
+
 // ---- f32 operands ------------------------------------------------------------------------------
 // 128 x 128 (or 64 x 64) workgroup tile, BK = 32.  v_mfma_f32_32x32x2f32 takes one element per lane
 // and operand -- lane l holds A[row l % 32][k l / 32] -- so both operand forms feed it directly:
@@ -636,8 +816,9 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
 //     with 4 ds_read_b32 (32 consecutive floats per half-wave; the other half-wave's rows k + 4 start
 //     32 banks away), no transposing copy beforehand.
 template <int BM, int BN, bool AT, bool BT>
-__global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g)
+__global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, const u32* only_if, u32 seq)
 {
+    if (only_if && *only_if != seq) return;                                // stand-by launch behind gemm_x3_k: nothing to redo
     constexpr int BK = 32, LDR = BK + 4;
     constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
     constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;      // 16-byte chunks per lane, operand and step
@@ -890,7 +1071,7 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
     sk.matrices = count;
     if (sk.splits > 1) {
         void* ws;
-        AIXK_TRY(workspace(ctx, 0, (size_t)sk.splits * count * M * N * sizeof(float), &ws));
+        AIXK_TRY(workspace(ctx, 2, (size_t)sk.splits * count * M * N * sizeof(float), &ws));
         sk.partial = (float*)ws;
     }
     const bool at = !a_k, tb = !b_k;
@@ -1059,10 +1240,52 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         GemmArgs g{};
         g.a = pa; g.b = pb; g.c = out->data;
         g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
+        // enough 128 x 128 tiles: on the bf16 pipe, each operand as three bf16 planes (gemm_x3_k); with few tiles and a
+        // long K, K is split over workgroups
+        const uint64_t t128 = ((M + 127) / 128) * ((N + 127) / 128), fill = 2 * (uint64_t)ctx->cus, steps = (K + 31) / 32;
+        // two workgroups per compute unit hide each other's split-and-stage phases: with fewer tiles than that, K is split
+        // over workgroups if it is long enough, else the f32 MFMA kernels below take the product
+        uint64_t splits = 1;
+        if (t128 < fill && K >= 2048) splits = std::min<uint64_t>({steps / 16, (fill + t128 - 1) / t128, (uint64_t)64});
+        const u32* only_if = nullptr;          // set: the launches below stand by behind gemm_x3_k
+        u32 seq = 0;
+        if (t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 2) {
+            const u32 n = grid_of(g, 128, 128);
+            SplitArgs sk{};
+            sk.per_split = (u32)((steps + splits - 1) / splits);
+            sk.splits = (u32)((steps + sk.per_split - 1) / sk.per_split);
+            sk.matrices = 1;
+            if (sk.splits > 1) {
+                void* ws;
+                AIXK_TRY(workspace(ctx, 2, (size_t)sk.splits * M * N * sizeof(float), &ws));
+                sk.partial = (float*)ws;
+            }
+            if (++ctx->gemm_seq == 0) ++ctx->gemm_seq;                     // 0 is what the flag word holds at creation
+            seq = ctx->gemm_seq;
+            auto launch_x3 = [&](auto kernel, size_t lds) {
+                AIXK_TRY(set_lds(kernel, lds));
+                hipLaunchKernelGGL(kernel, dim3(n, 1, sk.splits), dim3(256), lds, ctx->stream, g, sk, (u32*)ctx->counter, seq);
+                AIXK_HIP(hipGetLastError());
+                return (int)AIXK_OK;
+            };
+            int rc;
+            if (!at && !bt) rc = launch_x3(gemm_x3_k<false, false>, TileX3<false, false>::kLds);
+            else if (!at && bt) rc = launch_x3(gemm_x3_k<false, true>, TileX3<false, true>::kLds);
+            else if (at && !bt) rc = launch_x3(gemm_x3_k<true, false>, TileX3<true, false>::kLds);
+            else rc = launch_x3(gemm_x3_k<true, true>, TileX3<true, true>::kLds);
+            if (rc != AIXK_OK) return rc;
+            if (sk.splits > 1) {
+                const uint64_t total = M * N;
+                hipLaunchKernelGGL(splitk_finish_f32_k, dim3(grid_for(total, 256, (unsigned)ctx->cus * 16u)), dim3(256), 0, ctx->stream,
+                                   (const float*)sk.partial, (float*)out->data, (u64)total, sk.splits);
+                AIXK_HIP(hipGetLastError());
+            }
+            only_if = (const u32*)ctx->counter;                            // an infinity or a NaN among the operands: redo with IEEE arithmetic
+        }
         auto launch = [&](auto kernel, uint64_t tile, size_t lds) {
             const u32 n = grid_of(g, tile, tile);
             AIXK_TRY(set_lds(kernel, lds));
-            hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
+            hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g, only_if, seq);
             AIXK_HIP(hipGetLastError());
             return (int)AIXK_OK;
         };

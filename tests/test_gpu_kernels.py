@@ -701,6 +701,46 @@ def test_matmul_small_tiles(gpu, dtype):
         gpu.release()
 
 
+def test_matmul_f32_large_tiles_special_values(gpu):
+    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes in registers.
+    Rows with an infinity, a NaN, both infinities, or a value next to FLT_MAX must come out as IEEE arithmetic has
+    them (inf, NaN, NaN, finite); their neighbours in the same 16-byte chunk and everything else stay within the
+    f32 matmul bar; subnormal inputs count as what they are."""
+    rng = np.random.default_rng(25500)
+    m, k, n = 4096, 256, 2048
+    A = (rng.uniform(-1, 1, (m, k)) / np.sqrt(k)).astype(np.float32)
+    B = rng.uniform(0.1, 1.0, (k, n)).astype(np.float32)
+    A[7, 5] = np.inf
+    A[130, 9] = np.nan
+    A[131, 250] = -np.inf
+    A[300, 3], A[300, 77] = np.inf, -np.inf
+    A[1000, :] = 0.0
+    A[1000, 17] = np.float32(3.3e38)                  # times at most 1: finite in f32, would be inf if rounded up to bf16 first
+    A[2000, :] = np.float32(1e-41)                    # subnormal inputs
+    for layout in ("NN", "TN"):
+        a = T.HostTensor(A if layout == "NN" else np.ascontiguousarray(A.T), O.F32, [m, k], None if layout == "NN" else [1, m])
+        b = T.HostTensor(B, O.F32, [k, n])
+        _, da = gpu.put(a)
+        _, db = gpu.put(b)
+        po, do = gpu.put(T.empty(O.F32, [m, n]))
+        G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+        got = gpu.fetch(po, np.zeros(m * n, np.float32)).reshape(m, n)
+        assert np.all(got[7] == np.inf), layout
+        assert np.all(np.isnan(got[130])) and np.all(np.isnan(got[300])), layout
+        assert np.all(got[131] == -np.inf), layout
+        with np.errstate(invalid="ignore", over="ignore"):
+            exact = A.astype(np.float64) @ B.astype(np.float64)
+            scale = np.abs(A).astype(np.float64) @ np.abs(B).astype(np.float64)
+        ordinary = np.ones(m, bool)
+        ordinary[[7, 130, 131, 300]] = False
+        assert np.all(np.isfinite(got[ordinary])), layout
+        err = np.abs(got[ordinary] - exact[ordinary])
+        assert np.all(err <= 1e-5 * scale[ordinary] + 1e-44), (layout, float((err / (scale[ordinary] + 1e-300)).max()))
+        # and far inside the bar in practice: three planes carry all 24 bits
+        assert np.all(err[:6] <= 4e-7 * scale[ordinary][:6]), layout
+        gpu.release()
+
+
 def test_matmul_identity_and_ones(gpu):
     """Mathematical pins: A.I == A exactly; ones[m,k].ones[k,n] == k exactly (f32, f16, bf16)."""
     rng = np.random.default_rng(22000)
