@@ -1,25 +1,26 @@
 // matmul_mfma.hip -- GEMM on the matrix cores for f32 / f16 / bf16, f32 accumulation.
 //
-// Core kernels, all with both operands K-contiguous in memory ("NT": A is [M,K] with unit stride
-// along K, B is given as [N,K] with unit stride along K):
+// Kernels (A is [M,K], B is [K,N]; "K-contiguous" = unit stride along K, "T form" = unit stride along M / N):
 //
 //   16-bit, whole tiles   gemm_nt16_direct_k: 256x256x64 workgroup tile, LDS filled by LDS-direct
-//                         global loads, swizzled layout, explicit software pipeline (see there);
-//   16-bit, any shape     gemm_nt16_k: 256x256 or 128x128 tile x BK=64, bounds-checked register
-//                         staging, padded LDS rows; edges and small problems;
-//   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 tile x BK=32.
+//                         global loads, swizzled layout, explicit software pipeline; both operand forms;
+//   16-bit, mid-size      gemm_tile16_k: 128x128 / 128x64 / 64x64 tiles, register staging, both operand
+//                         forms, stacks of matrices (blockIdx.y) and K splits over workgroups (blockIdx.z);
+//   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
+//   16-bit, odd layouts   gemm_nt16_k: K-contiguous operands only, bounds-checked (others are gathered first);
+//   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
+//   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 or 64x64 tile x BK=32, both operand forms.
 //
-// All use 4 waves in a 2x2 arrangement with the accumulators resident in the 512-entry unified
-// register file.  Every lane feeds the MFMA with 8 (f32: 4) consecutive K values of one row;
-// because A and B use the same lane->K assignment, the dot products are independent of how the
-// instruction numbers K internally.
+// All use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
+// resident in the 512-entry unified register file.  Every lane feeds the 16-bit MFMA with 8 consecutive K
+// values of one row; because A and B use the same lane->K assignment, the dot products are independent of
+// how the instruction numbers K internally.
 //
 // Workgroups are numbered so that the 32 groups resident on one XCD (dispatch is round-robin over
 // the 8 XCDs) cover a compact 4 x 8 block of output tiles and share A/B panels in that XCD's L2.
 //
-// Operands that are not K-contiguous (plain row-major B, transposed-view A, sliced views) are
-// first gathered into K-contiguous scratch by the tiled transpose; odd K (not a multiple of 8
-// elements for 16-bit, 4 for f32) falls back to the LDS-tiled kernel in matmul.hip.
+// Odd K (not a multiple of 8 elements for 16-bit, 4 for f32) falls back to the LDS-tiled kernel in
+// matmul.hip.
 #pragma clang fp contract(fast)
 
 #include "common.hpp"
