@@ -3,8 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extras] [--no-cpu]
 
-Prints ONE JSON line.  The headline is BASELINE.json's first metric, fused-elementwise GB/s, on
-its configuration: f32 a, b, c of shape [4096, 4096] ~ U(-1, 1), seed 0,
+Prints ONE JSON line.  The headline is the reference benchmark's first metric, fused-elementwise
+GB/s, on its configuration: f32 a, b, c of shape [4096, 4096] ~ U(-1, 1), seed 0,
 y = tanh(a*b + c) / (1 + exp(-a)) - 0.5*c, evaluated lazily through the device interface so that
 the fusion planner emits one kernel.  A step is one evaluation (11 recorded device operators ->
 1 fused kernel); inputs are resident in HBM before the timed region; K steps are issued from the
@@ -16,7 +16,8 @@ native driver (libaixhip_bench.so) between two synchronize() calls.
   cpu_baseline = the same expression on the reference CPU device path, one thread
 
 "extras" carries the other single-GPU configurations (reductions / broadcast / transpose at
-[8192, 8192], matmul) with their own roofline entries; they are reported, not the headline.
+[8192, 8192], matmul, the MLP training step, the transformer step in its two ways of issuing
+attention) with their own roofline entries; they are reported, not the headline.
 """
 import argparse
 import ctypes as C
