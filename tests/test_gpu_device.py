@@ -481,3 +481,42 @@ _CASES = goldens.load_cases()
 @pytest.mark.parametrize("case", _CASES, ids=[c["name"] for c in _CASES])
 def test_reference_literals_on_device(dev, case):
     goldens.run_case(case, H.DeviceBackend(dev))
+
+
+def test_matmul_on_stacks_through_the_device(dev):
+    """matmul with operands of rank above 2 (beyond the reference's 2-D matmul): a stack of products through the
+    device interface -- elementwise work pending on an operand is flushed first, the [batch, heads, seq, d] view of
+    a [batch * seq, heads * d] activation is consumed without a copy, a host-memory operand is staged, and
+    operands whose leading dims differ are refused with the reference's exception type."""
+    rng = np.random.default_rng(36000)
+    B, Hd, S, D = 2, 3, 64, 32
+    dtype = O.BF16
+    rec = Recorder(dev, dtype, [B * S, Hd * D])
+    x = rec.leaf(T.contiguous_tensor(rng, dtype, [B * S, Hd * D], lo=-0.3, hi=0.3))
+    y = rec.leaf(T.contiguous_tensor(rng, dtype, [B * S, Hd * D], lo=-0.3, hi=0.3))
+    q = rec.binary(O.ADD, x, y)                                     # pending when the matmul is called
+    heads = [S * Hd * D, D, Hd * D, 1]
+    q4 = T.HostTensor(q["host"].storage, dtype, [B, Hd, S, D], heads)
+    kT = T.HostTensor(y["host"].storage, dtype, [B, Hd, D, S], [S * Hd * D, D, 1, Hd * D])
+    out = T.empty(dtype, [B, Hd, S, S])
+    po = dev.raw(out.storage.nbytes)
+    dev.dev.call("matmul", H.ref(H.kdesc(q4, q["ptr"])), H.ref(H.kdesc(kT, y["ptr"])), H.ref(H.kdesc(out, po)))
+    got = O.to_float64(dev.fetch(po, out.storage), dtype).reshape(B, Hd, S, S)
+    want = O.to_float64(q4.gather(), dtype) @ O.to_float64(kT.gather(), dtype)
+    scale = np.abs(O.to_float64(q4.gather(), dtype)) @ np.abs(O.to_float64(kT.gather(), dtype))
+    assert np.all(np.abs(got - want) <= 1e-5 * scale + 2.0 ** -8 * np.abs(want) + 1e-30)
+    # a host-memory second operand (staged into device memory first), f32 stack issued product by product
+    a32 = T.contiguous_tensor(rng, O.F32, [3, 40, 24], lo=-1, hi=1)
+    b32 = T.contiguous_tensor(rng, O.F32, [3, 24, 56], lo=-1, hi=1)
+    pa, da = dev.put(a32)
+    o32 = T.empty(O.F32, [3, 40, 56])
+    po32 = dev.raw(o32.storage.nbytes)
+    dev.dev.call("matmul", H.ref(da), H.ref(H.kdesc(b32, b32.storage.ctypes.data)), H.ref(H.kdesc(o32, po32)))
+    got32 = dev.fetch(po32, o32.storage).astype(np.float64).reshape(3, 40, 56)
+    want32 = a32.gather().astype(np.float64) @ b32.gather().astype(np.float64)
+    assert np.all(np.abs(got32 - want32) <= 1e-5 * (np.abs(a32.gather()).astype(np.float64) @ np.abs(b32.gather()).astype(np.float64)))
+    # leading dims that differ: refused
+    bad = T.HostTensor(b32.storage, O.F32, [2, 24, 56])
+    with pytest.raises(Exception):
+        dev.dev.call("matmul", H.ref(da), H.ref(H.kdesc(bad, bad.storage.ctypes.data)), H.ref(H.kdesc(o32, po32)))
+    dev.release()
