@@ -110,7 +110,7 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
             if (c.stackedAttention) {
                 const Shape split{c.batch, c.seq, c.heads, dh};
                 const Tensor q4 = q.reshape(split).transpose(1, 2), k4 = k.reshape(split).transpose(1, 2), v4 = v.reshape(split).transpose(1, 2);
-                const Tensor scores = (matmul(q4, k4.transpose(2, 3)) * scale).tril() + mask;         // [batch, heads, seq, seq]
+                const Tensor scores = matmul(q4, k4.transpose(2, 3)).tril() * scale + mask;         // [batch, heads, seq, seq]; scale and mask fuse
                 attn = matmul(softmax(scores, 3, true), v4).transpose(1, 2).reshape(Shape{T, d});
             } else {
                 std::vector<Tensor> sequences;
@@ -121,7 +121,7 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
                     for (uint64_t hd = 0; hd < c.heads; ++hd) {
                         const Tensor qh = qb.slice(1, hd * dh, (hd + 1) * dh), kh = kb.slice(1, hd * dh, (hd + 1) * dh),
                                      vh = vb.slice(1, hd * dh, (hd + 1) * dh);
-                        const Tensor scores = (matmul(qh, kh.transpose(0, 1)) * scale).tril() + mask;
+                        const Tensor scores = matmul(qh, kh.transpose(0, 1)).tril() * scale + mask;
                         heads.push_back(matmul(softmax(scores, 1, true), vh));
                     }
                     sequences.push_back(Tensor::cat(heads, 1));
