@@ -514,6 +514,8 @@ ROUTE_CASES = [  # (source shape, view kind, destination shape) chosen to hit ev
     ([130, 2304], "contig", [1, 2304]),       # outer, wide rows: workgroups side by side, rows split into chunks
     ([3, 70, 2048], "contig", [3, 1, 2048]),  # the same with a leading kept dim
     ([2, 64, 2048], "contig", [1, 64, 2048]), # a handful of rows (the pair axis of a composed ReLU): wide route, one chunk
+    ([1100, 2048], "contig", [1, 2048]),      # outer, many dense rows a workgroup holds whole: one sequential stream per workgroup
+    ([2, 1030, 5120], "contig", [2, 1, 5120]),# the same with a leading kept dim and five column tiles per lane
     ([3, 6000, 64], "contig", [3, 6000, 1]),  # very many short rows (softmax rows of a stack of score matrices): several rows per wave
     ([17001, 48], "contig", [17001, 1]),      # the same, rows that leave lanes idle, a ragged last group of rows
     ([7, 4100], "contig", [1, 4100]),         # the same, ragged columns
@@ -588,7 +590,7 @@ ARG_CASES = [  # (shape, kind, dim)
     ([6, 500, 64], "contig", 1), ([9, 40, 33], "contig", 2), ([9, 40, 33], "contig", 0),
     ([3, 2], "transposed", 1), ([64, 100], "transposed", 0),
     ([2, 40, 2048], "contig", 0), ([5, 4100], "contig", 0), ([3, 2, 1024], "contig", 1),    # a handful of rows, wide and narrow columns
-    ([20000, 64], "contig", 1),                                                               # very many short rows: several rows per wave
+    ([20000, 64], "contig", 1), ([1100, 3072], "contig", 0),                                                               # very many short rows: several rows per wave
 ]
 
 
