@@ -768,6 +768,28 @@ def test_matmul_identity_and_ones(gpu):
         gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16, O.I16, O.F32], ids=ids)
+def test_index_add_with_many_duplicates(gpu, dtype):
+    """Embedding-gradient shapes: hundreds of updates landing on a few dozen rows (16-bit types update two
+    neighbouring elements per compare-and-swap).  Whole-number updates keep every partial sum exact, so the
+    order in which duplicates arrive cannot matter and the result equals the CPU's bit for bit."""
+    rng = np.random.default_rng(27000 + dtype)
+    for shape, dim, ni in (([50, 64], 0, 700), ([4, 9, 6], 1, 40), ([3, 5, 8], 2, 64), ([7, 10], 0, 33)):
+        sel = list(shape)
+        sel[dim] = ni
+        idx = T.HostTensor(rng.integers(0, shape[dim], ni).astype(np.int32), O.I32, [ni])
+        upd = T.HostTensor(O.to_storage(rng.integers(-2, 3, O.numel(sel)).astype(np.float64), dtype), dtype, sel)
+        acc = T.HostTensor(O.to_storage(rng.integers(-4, 5, O.numel(shape)).astype(np.float64), dtype), dtype, shape)
+        want = acc.clone()
+        okc(CPU.index_add(C.byref(upd.desc()), C.byref(want.desc()), C.byref(idx.desc()), dim, 1))
+        _, didx = gpu.put(idx)
+        _, dupd = gpu.put(upd)
+        pa, dacc = gpu.put(acc)
+        G.run_gpu(gpu, "aixk_index_add", G.ref(dupd), G.ref(dacc), G.ref(didx), dim)
+        T.assert_same_bits(gpu.fetch(pa, want.storage), want.storage, f"indexAdd {NAMES[dtype]} {shape} dim={dim} x{ni}")
+        gpu.release()
+
+
 @pytest.mark.parametrize("dtype", T.ALL_DTYPES, ids=ids)
 def test_tri_on_dense_stacks(gpu, dtype):
     """tril / triu of dense tensors whose rows are whole 16-byte vectors (a stack of attention score matrices):
