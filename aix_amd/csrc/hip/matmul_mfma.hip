@@ -643,10 +643,12 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
 // per K step: the next step's global loads are in flight during the MFMAs.  blockIdx.z numbers K splits as in
 // gemm_tile16_k.
 //
-// Infinities and NaNs do not survive the split (inf - inf, and inf times a zero mid or lo plane of the other operand):
-// a lane that loads one stores the launch's number into a flag word, and the f32 MFMA kernel that is always launched
-// right behind -- its workgroups return at once unless the flag carries this number -- redoes the whole product with
-// IEEE arithmetic.
+// Infinities and NaNs do not survive the split (inf - inf, and inf times a zero mid or lo plane of the other operand),
+// but they cannot hide either: every operand element meets a nonzero hi plane or a zero, so a non-finite input leaves
+// an infinity or a NaN in some accumulator of its row or column.  A lane that ends up with one stores the launch's
+// number into a flag word, and the f32 MFMA kernel that is always launched right behind -- its workgroups return at
+// once unless the flag carries this number -- redoes the whole product with IEEE arithmetic (which also covers sums
+// that overflow on their own: the redo returns the same infinities).
 template <bool AT, bool BT> struct TileX3 {
     static constexpr int BM = 128, BN = 128, BK = 32, PK = BK + 8, PA = BM + 32, PB = BN + 32;
     static constexpr int SA = AT ? BK * PA : BM * PK, SB = BT ? BK * PB : BN * PK;       // bf16 elements per plane
@@ -661,10 +663,6 @@ __device__ __forceinline__ u32 cvt_pk_bf16(float lo, float hi)
 }
 
 // four f32 -> three word pairs of four bf16 (element e in bits 16 (e & 1) of word e / 2)
-__device__ __forceinline__ bool all_finite(const u32x4 x)
-{
-    return ((x.x & 0x7F800000u) != 0x7F800000u) && ((x.y & 0x7F800000u) != 0x7F800000u) && ((x.z & 0x7F800000u) != 0x7F800000u) && ((x.w & 0x7F800000u) != 0x7F800000u);
-}
 __device__ __forceinline__ void split3(const u32x4 x, u32x2& h, u32x2& m, u32x2& l)
 {
     const u32 xs[4] = {x.x, x.y, x.z, x.w};
@@ -727,7 +725,6 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
             const int c = tid + 256 * i;
             const int at = AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
             u32x2 h, m, l;
-            if (!all_finite(ra[i])) *flag = seq;
             split3(ra[i], h, m, l);
             *(u32x2*)(As + at) = h; *(u32x2*)(As + SA + at) = m; *(u32x2*)(As + 2 * SA + at) = l;
         }
@@ -736,7 +733,6 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
             const int c = tid + 256 * i;
             const int at = BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
             u32x2 h, m, l;
-            if (!all_finite(rb[i])) *flag = seq;
             split3(rb[i], h, m, l);
             *(u32x2*)(Bs + at) = h; *(u32x2*)(Bs + SB + at) = m; *(u32x2*)(Bs + 2 * SB + at) = l;
         }
@@ -785,6 +781,7 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
 
     const u64 plane = g.M * g.N;
     float* C = sk.splits > 1 ? sk.partial + (u64)blockIdx.z * plane : (float*)g.c;
+    float probe = 0.0f;                                   // NaN as soon as one accumulator is an infinity or a NaN (x * 0)
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -794,8 +791,10 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
             for (int v = 0; v < 16; ++v) {
                 const u64 row = m0 + wm * WM + i * 32 + (v >> 2) * 8 + (lane >> 5) * 4 + (v & 3);
                 if (row < g.M && col < g.N) C[row * g.N + col] = acc[i][j][v];
+                probe = __builtin_fmaf(acc[i][j][v], 0.0f, probe);
             }
         }
+    if (probe != probe) *flag = seq;
 }
 
 __global__ __launch_bounds__(256) void splitk_finish_f32_k(const float* __restrict__ partial, float* __restrict__ out, u64 total, u32 splits)
