@@ -1249,7 +1249,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         if (t128 < fill && K >= 2048) splits = std::min<uint64_t>({steps / 16, (fill + t128 - 1) / t128, (uint64_t)64});
         const u32* only_if = nullptr;          // set: the launches below stand by behind gemm_x3_k
         u32 seq = 0;
-        if (t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 2) {
+        if (t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 4) {
             const u32 n = grid_of(g, 128, 128);
             SplitArgs sk{};
             sk.per_split = (u32)((steps + splits - 1) / splits);
