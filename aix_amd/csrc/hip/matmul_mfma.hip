@@ -816,7 +816,7 @@ __global__ __launch_bounds__(256) void splitk_finish_f32_k(const float* __restri
 //     with 4 ds_read_b32 (32 consecutive floats per half-wave; the other half-wave's rows k + 4 start
 //     32 banks away), no transposing copy beforehand.
 template <int BM, int BN, bool AT, bool BT>
-__global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, const u32* only_if, u32 seq)
+__global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, SplitArgs sk, const u32* only_if, u32 seq)
 {
     if (only_if && *only_if != seq) return;                                // stand-by launch behind gemm_x3_k: nothing to redo
     constexpr int BK = 32, LDR = BK + 4;
@@ -906,14 +906,18 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, const u32* only_i
 #pragma unroll
                 for (int j = 0; j < TJ; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[set][i][s], fb[set][j][s], acc[i][j], 0, 0, 0);
     };
+    // blockIdx.z numbers K splits (few tiles, long K: [2048, 4096] x [4096, 10]): split s multiplies its share of the K
+    // steps and stores an f32 partial tile for splitk_finish_f32_k
     const u64 steps = (g.K + BK - 1) / BK;
-    load_global(0);
+    const u64 first = (u64)blockIdx.z * sk.per_split;
+    const u64 last = first + sk.per_split < steps ? first + sk.per_split : steps;
+    load_global(first * BK);
     store_lds(0);
     __syncthreads();
     read_frags(0, 0, 0);
-    for (u64 kt = 0; kt < steps; ++kt) {
-        const int buf = (int)(kt & 1);
-        load_global((kt + 1 < steps ? kt + 1 : kt) * BK);       // past the end: the last tile again, into a buffer nobody reads
+    for (u64 kt = first; kt < last; ++kt) {
+        const int buf = (int)((kt - first) & 1);
+        load_global((kt + 1 < last ? kt + 1 : kt) * BK);        // past the end: the last tile again, into a buffer nobody reads
         read_frags(1, buf, 1); mma(0);
         __builtin_amdgcn_sched_barrier(0);
         read_frags(0, buf, 2); mma(1);
@@ -926,7 +930,7 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, const u32* only_i
         __builtin_amdgcn_sched_barrier(0);
     }
 
-    float* C = (float*)g.c;
+    float* C = sk.splits > 1 ? sk.partial + (u64)blockIdx.z * g.M * g.N : (float*)g.c;
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -1284,9 +1288,26 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         }
         auto launch = [&](auto kernel, uint64_t tile, size_t lds) {
             const u32 n = grid_of(g, tile, tile);
+            // few tiles and a long K (a weight gradient with ten output columns): K split over workgroups
+            SplitArgs sk{};
+            uint64_t ksplits = 1;
+            if (!only_if && n < (u32)ctx->cus && K >= 2048) ksplits = std::max<uint64_t>(1, std::min<uint64_t>({steps / 8, (fill + n - 1) / n, (uint64_t)64}));
+            sk.per_split = (u32)((steps + ksplits - 1) / ksplits);
+            sk.splits = (u32)((steps + sk.per_split - 1) / sk.per_split);
+            sk.matrices = 1;
+            if (sk.splits > 1) {
+                void* ws;
+                AIXK_TRY(workspace(ctx, 2, (size_t)sk.splits * M * N * sizeof(float), &ws));
+                sk.partial = (float*)ws;
+            }
             AIXK_TRY(set_lds(kernel, lds));
-            hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g, only_if, seq);
+            hipLaunchKernelGGL(kernel, dim3(n, 1, sk.splits), dim3(256), lds, ctx->stream, g, sk, only_if, seq);
             AIXK_HIP(hipGetLastError());
+            if (sk.splits > 1) {
+                hipLaunchKernelGGL(splitk_finish_f32_k, dim3(grid_for(M * N, 256, (unsigned)ctx->cus * 16u)), dim3(256), 0, ctx->stream,
+                                   (const float*)sk.partial, (float*)out->data, (u64)(M * N), sk.splits);
+                AIXK_HIP(hipGetLastError());
+            }
             return (int)AIXK_OK;
         };
         // stage sizes: K-contiguous rows x 36 floats, T form 32 k-rows x (tile + 8) floats
