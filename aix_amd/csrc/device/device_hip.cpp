@@ -853,9 +853,17 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
 {
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndicesTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxIndicesTo");
+    // the caller zero-fills the destination right before the call (aixCore.hpp:927-941): a fill still waiting in
+    // the window is folded into the operator
+    uint64_t init = 0;
+    const bool folded = takeInit(src, dst, &init);
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "argmaxIndicesTo"); toPod(dst, &pd, "argmaxIndicesTo");
-    check(aixk_argmax_to(m_ctx, 1, &ps, &pd, dim));
+    if (folded && init != 0) {                                       // not the zero fill: put it back as a pass of its own
+        const int32_t value = (int32_t)init;
+        check(aixk_fill(m_ctx, &value, AIXK_I32, &pd));
+    }
+    check(aixk_argmax_to(m_ctx, folded && init == 0 ? 2 : 1, &ps, &pd, dim));
 }
 
 void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim, size_t start, size_t end, size_t step)

@@ -393,6 +393,40 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restric
     }
 }
 
+// argmaxIndicesTo over a handful of rows with the zero-initialisation of the destination folded in (the pair axis of a
+// composed ReLU: fill(0) + argmaxIndicesTo on [2, 4096, 2048]): a lane owns VEC columns, finds the winning row of each
+// and writes the whole one-hot column block -- R dense 16-byte stores -- instead of a fill pass plus scattered ones.
+template <class T, int VEC>
+__global__ __launch_bounds__(kBlock) void argmax_onehot_rows_k(const T* __restrict__ src, i32* __restrict__ dst, RedPlan p)
+{
+    typedef ArgOp<T> Op;
+    typedef typename Op::Acc Acc;
+    typedef vec<T, VEC> V;
+    typedef vec<i32, VEC> O;
+    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 c0 = ((u64)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (c0 >= C) return;
+    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const T* col = src + s.src + c0;
+    Acc acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = Op::init();
+    for (u64 r = 0; r < R; ++r) {
+        const V x = *(const V*)(col + r * p.r_src[0]);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) Op::step(acc[e], x.v[e], r, r == 0);
+    }
+    u32 winner[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) winner[e] = (acc[e].flags & 2u) ? 0u : acc[e].idx;      // a leading NaN wins (as land() has it)
+    for (u64 r = 0; r < R; ++r) {
+        O out;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out.v[e] = winner[e] == (u32)r ? 1 : 0;
+        *(O*)(dst + s.flat + r * p.r_flat[0] + c0) = out;
+    }
+}
+
 // second stage of `outer` when rows were split over several workgroups: 64 slots per workgroup,
 // the four waves take every fourth chunk (independent loads in flight), LDS folds the four.
 template <class Op, class T>
@@ -502,6 +536,20 @@ bool make_plan(const aixhip_tensor* src, const uint64_t* weight, RedPlan* p)
 template <class Op, class T>
 int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin);
 
+// Does argmax_onehot_rows_k take this plan?  One reduced dim of fewer than 8 rows, the innermost kept dim dense on both
+// sides, everything aligned for VEC-wide accesses.
+template <class T>
+bool onehot_rows_route(const RedPlan& p, const T* ps, const void* dst)
+{
+    constexpr int VEC16 = vec16<T>::n, VEC = VEC16 < 4 ? VEC16 : 4;
+    if (!(p.nr == 1 && p.nk >= 1 && p.k_src[p.nk - 1] == 1 && p.k_dst[p.nk - 1] == 1 && p.k_flat[p.nk - 1] == 1 && p.red >= 2)) return false;
+    const uint64_t C = p.k_ext[p.nk - 1], R = p.r_ext[0], O = p.slots / C;
+    if (R >= 8 || O > 65535 || C % VEC != 0 || C / VEC / kBlock >= (1ull << 31)) return false;
+    if (((uintptr_t)(ps + p.src_off) % (sizeof(T) * VEC)) != 0 || p.r_src[0] % VEC != 0 || p.r_flat[0] % VEC != 0 || !aligned16(dst)) return false;
+    for (int d = 0; d + 1 < p.nk; ++d) if (p.k_src[d] % VEC || p.k_flat[d] % VEC) return false;
+    return true;
+}
+
 template <class Op, class T>
 int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, const RedPlan& p, const Finish& fin)
 {
@@ -539,6 +587,15 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
         bool vect = C % VEC == 0 && ((uintptr_t)(ps + p.src_off) % (sizeof(T) * VEC)) == 0 && p.r_src[0] % VEC == 0;
         for (int d = 0; d + 1 < p.nk; ++d) if (p.k_src[d] % VEC) vect = false;
         const int v = vect ? VEC : 1;
+        // one-hot argmax over a handful of rows whose destination this call also has to zero: written densely in one pass
+        if constexpr (Op::kTracksIndex) {
+            if (fin.onehot == 2 && onehot_rows_route<T>(p, ps, dst)) {
+                const uint64_t tiles = (C / VEC + kBlock - 1) / kBlock;
+                hipLaunchKernelGGL((argmax_onehot_rows_k<T, VEC>), dim3((unsigned)tiles, 1, (unsigned)O), dim3(kBlock), 0, st, ps, (i32*)dst, p);
+                AIXK_HIP(hipGetLastError());
+                return AIXK_OK;
+            }
+        }
         // wide rows: workgroups of 256 * v columns, rows split into chunks of at least 16 (a handful of rows --
         // the pair axis of a composed ReLU, say -- is one chunk: every lane folds its columns outright)
         if (vect && C >= (uint64_t)kBlock * v * 2 && (R >= 64 || R < 8) && O <= 65535) {
@@ -698,7 +755,7 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
     if (src->size == 0) return AIXK_OK;
     AIXK_REQUIRE(src->size == numel(src) && src->size < (1ull << 31), "argmaxTo: inconsistent or too large source");
     uint64_t weight[AIXK_MAX_RANK];
-    Finish fin{0, onehot ? 1 : 0, 0, 0};
+    Finish fin{0, onehot, 0, 0};
     if (onehot) {
         AIXK_REQUIRE((int)dim < dst->rank, "argmaxIndicesTo: dim out of range");
         uint64_t rshape[AIXK_MAX_RANK];
@@ -714,6 +771,11 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
     if (!make_plan(src, weight, &plan)) return fail(AIXK_EINVAL, "argmaxTo: view does not collapse to %d dims", kMaxDims);
     return by_dtype(src->dtype, [&](auto tag) {
         typedef decltype(tag) T;
+        if (fin.onehot == 2 && !onehot_rows_route<T>(plan, (const T*)src->data, dst->data)) {
+            // the zero-initialisation this call owes, as a pass of its own, then ones scattered as usual
+            AIXK_TRY(aixk_zero(ctx, dst->data, src->size * sizeof(int32_t)));
+            fin.onehot = 1;
+        }
         return run_plan<ArgOp<T>, T>(ctx, src, (int32_t*)dst->data, plan, fin);
     });
 }

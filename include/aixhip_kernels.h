@@ -134,7 +134,9 @@ int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const 
  * without the separate fill pass over dst. */
 int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t init_bits);
 /* Device::argmaxTo / argmaxIndicesTo (aixDeviceCPU.cpp:275-298, 320-360). onehot=1 scatters ones
- * into the pre-zeroed int32 dst of src's shape. */
+ * into the pre-zeroed int32 dst of src's shape; onehot=2 also zeroes dst first (the fill(0) the
+ * caller issues before argmaxIndicesTo, aixCore.hpp:927-941, folded in: over a handful of rows the
+ * one-hot block is then written densely in a single pass). */
 int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t dim);
 
 /* ---- matmul (aixDevice.hpp:63; aixDeviceCPU.cpp:362-389) ---------------- */

@@ -520,3 +520,27 @@ def test_matmul_on_stacks_through_the_device(dev):
     with pytest.raises(Exception):
         dev.dev.call("matmul", H.ref(da), H.ref(H.kdesc(bad, bad.storage.ctypes.data)), H.ref(H.kdesc(o32, po32)))
     dev.release()
+
+
+def test_fill_is_folded_into_argmax_indices_to(dev):
+    """The mask of a max() backward: an int32 tensor of src's shape filled with 0, then argmaxIndicesTo scatters
+    ones into it.  A zero fill still waiting in the window is folded into the operator (over a handful of rows
+    the one-hot block is written densely in one pass); any other pending value is put back first, because
+    the operator only ever writes the ones."""
+    set_diag(dev)
+    rng = np.random.default_rng(39000)
+    for shape, dim in (([2, 64, 256], 0), ([300, 40], 1), ([5, 1024], 0)):
+        src = T.contiguous_tensor(rng, O.F32, shape, lo=-1, hi=1)
+        src.storage[:] = np.round(src.storage * 2) / 2                       # ties: the first maximum wins
+        _, dsrc = dev.put(src)
+        for value in (0.0, 5.0):
+            want = T.empty(O.I32, shape)
+            v = np.array([value], np.float32)
+            assert CPU.fill(v.ctypes.data, O.F32, C.byref(want.desc())) == 0
+            assert CPU.argmax_indices_to(C.byref(src.desc()), C.byref(want.desc()), dim) == 0
+            pm = dev.raw(want.storage.nbytes)
+            dm = H.kdesc(want, pm)
+            dev.dev.call("fill", v.ctypes.data, O.F32, H.ref(dm))
+            dev.dev.call("argmax_indices_to", H.ref(dsrc), H.ref(dm), dim)
+            T.assert_same_bits(dev.fetch(pm, want.storage), want.storage, f"fill({value}) + argmaxIndicesTo {shape} dim={dim}")
+    dev.release()

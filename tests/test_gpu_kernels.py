@@ -590,7 +590,7 @@ ARG_CASES = [  # (shape, kind, dim)
     ([6, 500, 64], "contig", 1), ([9, 40, 33], "contig", 2), ([9, 40, 33], "contig", 0),
     ([3, 2], "transposed", 1), ([64, 100], "transposed", 0),
     ([2, 40, 2048], "contig", 0), ([5, 4100], "contig", 0), ([3, 2, 1024], "contig", 1),    # a handful of rows, wide and narrow columns
-    ([20000, 64], "contig", 1), ([1100, 3072], "contig", 0),                                                               # very many short rows: several rows per wave
+    ([20000, 64], "contig", 1), ([1100, 3072], "contig", 0), ([2, 300, 64], "contig", 0), ([4, 2, 1028], "contig", 1), ([7, 36], "contig", 0),                                                               # very many short rows: several rows per wave
 ]
 
 
@@ -618,6 +618,10 @@ def test_argmax_to_family(gpu, dtype):
         po, do = gpu.put(T.empty(O.I32, shape))
         G.run_gpu(gpu, "aixk_argmax_to", 1, G.ref(ds), G.ref(do), dim)
         T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"argmaxIndicesTo {NAMES[dtype]} {shape} dim={dim} {kind}")
+        # the same with the zero-fill of the destination folded in: whatever dst held is overwritten
+        po, do = gpu.put(T.empty(O.I32, shape, fill=7))
+        G.run_gpu(gpu, "aixk_argmax_to", 2, G.ref(ds), G.ref(do), dim)
+        T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"fill(0) + argmaxIndicesTo {NAMES[dtype]} {shape} dim={dim} {kind}")
         gpu.release()
     src = T.contiguous_tensor(rng, dtype, [4, 4])
     _, ds = gpu.put(src)
