@@ -151,6 +151,58 @@ def _matmul_properties(gpu, dtype, n, layout, rng, tol_rel):
     gpu.release()
 
 
+def _rect_properties(gpu, dtype, m, k, n, layout, rng, tol_rel):
+    """The same checks for A [m, k] . B [k, n]: row and column checksums of every element of C against float64
+    from the inputs in O(mk + kn), and 64 single entries against float64 dot products."""
+    a_t, b_t = layout[0] == "T", layout[1] == "T"
+    a_store = O.to_storage(rng.uniform(-1, 1, m * k) / np.sqrt(k), dtype)
+    b_store = O.to_storage(rng.uniform(-1, 1, k * n), dtype)
+    A = O.to_float64(a_store, dtype).reshape((k, m) if a_t else (m, k))
+    B = O.to_float64(b_store, dtype).reshape((n, k) if b_t else (k, n))
+    A = A.T if a_t else A
+    B = B.T if b_t else B
+    ha = T.HostTensor(a_store, dtype, [m, k], [1, m] if a_t else None)
+    hb = T.HostTensor(b_store, dtype, [k, n], [1, k] if b_t else None)
+    _, da = gpu.put(ha)
+    _, db = gpu.put(hb)
+    out = T.empty(dtype, [m, n])
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+    Cg = O.to_float64(gpu.fetch(po, out.storage), dtype).reshape(m, n)
+    eps_out = {O.F32: 2.0 ** -24, O.F16: 2.0 ** -11, O.BF16: 2.0 ** -8}[dtype]
+    what = f"{NAMES[dtype]} [{m},{k}]x[{k},{n}] {layout}"
+    got, want, mag = Cg.sum(axis=1), A @ B.sum(axis=1), np.abs(A) @ np.abs(B).sum(axis=1)
+    assert np.all(np.abs(got - want) <= eps_out * np.abs(Cg).sum(axis=1) + tol_rel * mag), what + ": row checksum"
+    got, want, mag = Cg.sum(axis=0), A.sum(axis=0) @ B, np.abs(A).sum(axis=0) @ np.abs(B)
+    assert np.all(np.abs(got - want) <= eps_out * np.abs(Cg).sum(axis=0) + tol_rel * mag), what + ": column checksum"
+    for i, j in zip(rng.integers(0, m, 64), rng.integers(0, n, 64)):
+        want = float(A[i, :] @ B[:, j])
+        assert abs(Cg[i, j] - want) <= eps_out * abs(want) + tol_rel * float(np.abs(A[i, :]) @ np.abs(B[:, j])) + 1e-30, (what, int(i), int(j))
+    gpu.release()
+
+
+@pytest.mark.parametrize("case", [
+    (8192, 768, 768, "NT"), (8192, 768, 768, "NN"), (8192, 3072, 768, "NN"),      # activations x weights: 128 x 64 tiles
+    (768, 8192, 768, "TN"), (768, 8192, 768, "TT"),                                 # a weight gradient (x^T . dy, both given row-major) and the same with dy transposed: 64 x 64 tiles, K split 8 ways
+    (768, 8192, 3072, "TT"), (3072, 8192, 768, "TN"),                               # 128 x 128 tiles, K split 4 ways
+    (768, 8192, 8192, "TT"),                                                        # the output projection's gradient: K split 2 ways
+], ids=lambda c: f"{c[0]}x{c[1]}x{c[2]}{c[3]}")
+def test_matmul_transformer_shapes_bf16(gpu, case):
+    """The mid-size products of a d = 768 transformer step at 8192 tokens, at their real shapes: every tile
+    size of the mid-size kernel, with and without K splits, operands consumed where they lie."""
+    m, k, n, layout = case
+    _rect_properties(gpu, O.BF16, m, k, n, layout, np.random.default_rng(6400 + m + n), 1e-5)
+
+
+@pytest.mark.parametrize("case", [(4096, 784, 2048, "NN"), (2048, 4096, 2048, "TT"), (784, 4096, 2048, "TT"), (2048, 4096, 10, "TN"), (4096, 2048, 2048, "NT")],
+                         ids=lambda c: f"{c[0]}x{c[1]}x{c[2]}{c[3]}")
+def test_matmul_mlp_shapes_f32(gpu, case):
+    """The products of the 784-2048-2048-10 MLP at batch 4096, at their real shapes: the split-plane kernel with
+    and without K splits, and the f32 MFMA kernel with K splits for the ten-column weight gradient."""
+    m, k, n, layout = case
+    _rect_properties(gpu, O.F32, m, k, n, layout, np.random.default_rng(6500 + m + n), 1e-5)
+
+
 @pytest.mark.parametrize("layout", ["NN", "NT", "TN", "TT"])
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=lambda d: NAMES[d])
 def test_matmul_4096_cubed_16bit(gpu, dtype, layout):
