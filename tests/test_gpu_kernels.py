@@ -894,6 +894,42 @@ def test_matmul_stacks(gpu, dtype):
     gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.I32], ids=ids)
+def test_matmul_stacks_random_views(gpu, dtype):
+    """Stacks with one to three leading dims in a random storage order (so the leading dims of a and b collapse
+    differently, or not at all), an operand shared along a random leading dim (stride 0), extents that are and are not
+    multiples of the 16-byte chunk, matrices stored transposed: against the oracle's stack and the 2-D entry point."""
+    rng = np.random.default_rng(24800 + dtype)
+    for trial in range(10):
+        nlead = int(rng.integers(1, 4))
+        lead = [int(v) for v in rng.integers(1, 4, nlead)]
+        m, k, n = (int(v) for v in rng.choice([8, 24, 40, 64, 72, 96, 100], 3))
+        if trial % 3 == 0:
+            m, n = 64, 64                                            # large enough for the one-launch route (16-bit types)
+            k = int(rng.choice([16, 64, 136]))
+
+        def operand(rows, cols):
+            """Random storage order of the leading dims, matrix stored plain or transposed, maybe shared along one dim."""
+            order = list(rng.permutation(nlead))
+            shared = int(rng.integers(0, nlead)) if rng.random() < 0.3 else -1
+            transposed = rng.random() < 0.5
+            strides = [0] * nlead
+            run = rows * cols
+            for d in reversed(order):
+                if d == shared:
+                    continue
+                strides[d] = run
+                run *= lead[d]
+            offset = int(rng.integers(0, 3)) * 8
+            values = rng.integers(-9, 9, run + offset) if dtype in T.INT_DTYPES else rng.uniform(-1, 1, run + offset) / np.sqrt(k)
+            mat = [1, rows] if transposed else [cols, 1]
+            return T.HostTensor(O.to_storage(values, dtype), dtype, lead + [rows, cols], strides + mat, offset)
+
+        a, b = operand(m, k), operand(k, n)
+        check_matmul_stack(gpu, a, b, f"random stack {NAMES[dtype]} lead={lead} {m}x{k}x{n} a.strides={a.strides} b.strides={b.strides}")
+        gpu.release()
+
+
 def test_matmul_stack_edges(gpu):
     """Rank 2 is the 2-D entry point; empty stacks and K = 0; more matrices than one launch numbers (stride-0
     stacks of one product: every result matrix equals the single product); mismatched operands are refused."""
