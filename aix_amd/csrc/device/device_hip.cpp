@@ -559,6 +559,7 @@ void DeviceHIP::emitSingle(const OpRecord& op)
     if (op.type == OpType::Fill) { check(aixk_fill(m_ctx, op.scalarData.data(), (int)op.scalarDType, &o)); return; }
     if (op.type == OpType::FillMin) { check(aixk_fill_min(m_ctx, &o)); return; }
     toPod(op.input0, &a);
+    if (op.type == OpType::Tril || op.type == OpType::Triu) { check(aixk_tri(m_ctx, op.type == OpType::Triu ? 1 : 0, &a, &o, op.triDiagonal)); return; }
     if (const int code = binaryCode(op.type); code >= 0) {
         toPod(op.input1, &b);
         check(aixk_binary(m_ctx, code, &a, &b, &o));
@@ -883,6 +884,7 @@ void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& ds
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::tril() requires matching source and destination data types.");   // aixDeviceMetal.cpp:1160-1161
     requireDevice(dst, "tril");
+    if (recordTri(OpType::Tril, src, dst, diagonal)) return;
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "tril"); toPod(dst, &pd, "tril");
     check(aixk_tri(m_ctx, 0, &ps, &pd, diagonal));
@@ -892,9 +894,26 @@ void DeviceHIP::triu(const DeviceTensorParams& src, const DeviceTensorParams& ds
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::triu() requires matching source and destination data types.");
     requireDevice(dst, "triu");
+    if (recordTri(OpType::Triu, src, dst, diagonal)) return;
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "triu"); toPod(dst, &pd, "triu");
     check(aixk_tri(m_ctx, 1, &ps, &pd, diagonal));
+}
+
+// tril / triu join the window as elementwise operators (the scale, the mask and the triangle of attention scores become
+// one kernel) when both ends are this device's memory, the destination is a whole dense tensor of the source's shape
+// and the views fit the generated kernels; everything else runs at once.
+bool DeviceHIP::recordTri(OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
+{
+    if (src.shape.size() < 2 || src.shape.size() > (size_t)gen::kMaxDims || src.shape != dst.shape || src.size == 0 || src.size != dst.size) return false;
+    if (!dst.isContiguous || dst.offset != 0 || !findBlock(src.data)) return false;
+    size_t count = 1;
+    for (auto e : src.shape) count *= e;
+    if (count != src.size) return false;
+    View in(src), out(dst);
+    out.makeDense();
+    m_engine->recordTri(type, in, out, (int64_t)diagonal);
+    return true;
 }
 
 void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)

@@ -152,6 +152,7 @@ private:
     void recordBinary(aixhip::fuse::OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b,
                       const DeviceTensorParams& r, const char* op);
     void recordUnary(aixhip::fuse::OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op);
+    bool recordTri(aixhip::fuse::OpType t, const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal);
     bool takeInit(const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t* bits);
     void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);

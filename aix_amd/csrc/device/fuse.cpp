@@ -43,6 +43,7 @@ bool isElementwiseOp(OpType t)
         case OpType::Add: case OpType::Sub: case OpType::Mul: case OpType::Div: case OpType::Negate:
         case OpType::Sqrt: case OpType::Sin: case OpType::Cos: case OpType::Tanh: case OpType::Log:
         case OpType::Exp: case OpType::Pow: case OpType::Fill: case OpType::FillMin: case OpType::Cast:
+        case OpType::Tril: case OpType::Triu:                 // when recorded (FuseEngine::recordTri)
             return true;
         default:
             return false;
@@ -331,7 +332,7 @@ public:
     void describe(const Group& g, FusedSubgraphDescriptor& d)
     {
         const auto& ops = *m_ops;
-        d.ops.clear(); d.inputBuffers.clear(); d.outputBuffers.clear(); d.scalarData.clear();
+        d.ops.clear(); d.inputBuffers.clear(); d.outputBuffers.clear(); d.scalarData.clear(); d.opParams.clear();
         d.dtype = g.dtype;
         d.elementCount = g.count;
         d.shape.assign(g.shape->shape, g.shape->shape + g.shape->rank);
@@ -379,6 +380,10 @@ public:
                     *idx[k] = nIn + m_position[operand.index];
                 }
                 else if (operand.kind == Operand::kScalar) *sc[k] = scalarIndex(operand.index);
+            }
+            if (op.type == OpType::Tril || op.type == OpType::Triu) {
+                o.paramIndex = d.opParams.size() / 3;
+                d.opParams.push_back(op.triRows); d.opParams.push_back(op.triCols); d.opParams.push_back((uint64_t)op.triDiagonal);
             }
             if (m_store[w]) {
                 o.outputIndex = d.outputBuffers.size();
@@ -767,6 +772,15 @@ void FuseEngine::recordFill(const void* scalar, DataType scalarDType, const View
     OpRecord& r = append(OpType::Fill);
     r.output = output; r.scalarDType = scalarDType;
     std::memcpy(r.scalarData.data(), scalar, aix::Device::dataTypeSize(scalarDType));
+    maybeFlush();
+}
+
+void FuseEngine::recordTri(OpType type, const View& input, const View& output, int64_t diagonal)
+{
+    if ((type != OpType::Tril && type != OpType::Triu) || input.rank < 2) throw std::invalid_argument("recordTri: tril / triu of a tensor of rank 2 or more");
+    OpRecord& r = append(type);
+    r.input0 = input; r.output = output;
+    r.triRows = input.shape[input.rank - 2]; r.triCols = input.shape[input.rank - 1]; r.triDiagonal = diagonal;
     maybeFlush();
 }
 

@@ -91,6 +91,9 @@ struct OpRecord {
     std::array<uint8_t, 8> scalarData{};   // Fill: the scalar in scalarDType
     DataType scalarDType = DataType::kFloat32;
     bool hasInput1 = false;
+    // Tril / Triu recorded as elementwise operators: the extents of the last two dims and the diagonal
+    uint64_t triRows{0}, triCols{0};
+    int64_t triDiagonal{0};
 };
 
 // One fused kernel: ops in execution order.  An operand index below inputBuffers.size() names an
@@ -105,8 +108,10 @@ struct FusedSubgraphDescriptor {
         size_t outputIndex  = SIZE_MAX;    // into outputBuffers; SIZE_MAX = value stays in registers
         size_t scalarIndex0 = SIZE_MAX;
         size_t scalarIndex1 = SIZE_MAX;
+        size_t paramIndex   = SIZE_MAX;    // Tril / Triu: its (rows, cols, diagonal) triple in opParams
     };
     std::vector<Op> ops;
+    std::vector<uint64_t> opParams;        // run-time integers of index-dependent operators, three per Tril / Triu
     std::vector<View> inputBuffers;
     std::vector<View> outputBuffers;
     std::vector<uint8_t> scalarData;
@@ -174,6 +179,8 @@ public:
     void record(OpType type, const View& input0, const View& input1, const View& output);
     void recordFill(const void* scalar, DataType scalarDType, const View& output);
     void recordFillMin(const View& output);
+    // tril / triu of `input` (its last two dims) as an elementwise operator: the kept part passes through, the rest is 0
+    void recordTri(OpType type, const View& input, const View& output, int64_t diagonal);
     void flush();
 
     const FuseConfig& config() const { return m_config; }

@@ -56,6 +56,15 @@ size_t scalarCount(const FusedSubgraphDescriptor& d)
     return d.scalarData.size() / aix::Device::dataTypeSize(d.dtype);
 }
 
+bool isTri(OpType t) { return t == OpType::Tril || t == OpType::Triu; }
+
+size_t triCount(const FusedSubgraphDescriptor& d)
+{
+    size_t n = 0;
+    for (const auto& op : d.ops) if (isTri(op.type)) ++n;
+    return n;
+}
+
 std::string operandText(const FusedSubgraphDescriptor& d, size_t tensorIndex, size_t scalarIndex)
 {
     if (tensorIndex != SIZE_MAX) {
@@ -70,10 +79,15 @@ std::string operandText(const FusedSubgraphDescriptor& d, size_t tensorIndex, si
 // one element type T: loads convert to it and stores convert from it, so a cast is the identity here.
 void emitBody(std::ostringstream& o, const FusedSubgraphDescriptor& d)
 {
-    o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out)\n{\n";
+    // kernels with a tril / triu also get the element's flat logical index and the operators' (rows, cols, diagonal)
+    if (triCount(d)) o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out, int e, const TriPos* tpos, const u64* tp)\n{\n";
+    else o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out)\n{\n";
     for (size_t k = 0; k < d.ops.size(); ++k) {
         const auto& op = d.ops[k];
         if (op.type == OpType::Cast) o << "    const T v" << k << " = " << operandText(d, op.inputIndex0, op.scalarIndex0) << ";\n";
+        else if (isTri(op.type))
+            o << "    const T v" << k << " = tri_keeps(tpos[" << op.paramIndex << "], e, tp[" << 3 * op.paramIndex << "], tp[" << 3 * op.paramIndex + 1 << "], (i64)tp["
+              << 3 * op.paramIndex + 2 << "], " << (op.type == OpType::Triu ? 1 : 0) << ") ? " << operandText(d, op.inputIndex0, op.scalarIndex0) << " : zero<T>();\n";
         else {
             o << "    const T v" << k << " = " << fnName(op.type) << "(" << operandText(d, op.inputIndex0, op.scalarIndex0);
             if (isBinary(op.type)) o << ", " << operandText(d, op.inputIndex1, op.scalarIndex1);
@@ -141,8 +155,9 @@ std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t br
 
 std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
 {
-    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d), NT = triCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
+    if (d.opParams.size() != 3 * NT) throw std::invalid_argument("fused kernel: tril / triu without its parameters");
     const size_t esz = aix::Device::dataTypeSize(d.dtype);
     const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
     std::ostringstream o;
@@ -162,7 +177,9 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     auto from_t = [&](size_t k, const std::string& e) { return out_same(k) ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
     emitBody(o, d);
 
-    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 n;\n";
+    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n";
+    if (NT) o << "    u64 tp[" << 3 * NT << "];\n";
+    o << "    u64 n;\n";
     if (shape != Shape::Flat) o << "    u64 chunks;\n    u64 rank;\n    u64 shape[" << kMaxDims << "];\n    u64 off[" << AI << "];\n    u64 str[" << AI << "][" << kMaxDims << "];\n";
     o << "};\n\n";
 
@@ -188,25 +205,27 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
           << "    for (u64 v = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; v < nvec; v += (u64)gridDim.x * " << kBlock << ") {\n";
         for (size_t k = 0; k < NI; ++k) if (!bc(k)) o << "        const vec<I" << k << ", VEC> r" << k << " = p" << k << "[v];\n";
         for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
+        if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(v * VEC, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
         o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
         for (size_t k = 0; k < NI; ++k) {
             if (bc(k)) o << "            x[" << k << "] = b" << k << ";\n";
             else o << "            x[" << k << "] = " << to_t(k, "r" + std::to_string(k) + ".v[e]") << ";\n";
         }
         if (NI == 0) o << "            x[0] = zero<T>();\n";
-        o << "            aix_body(x, s, y);\n";
+        o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
         for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
         for (size_t k = 0; k < NO; ++k) o << "        q" << k << "[v] = w" << k << ";\n";
         o << "    }\n"
           << "    const u64 done = nvec * VEC;\n"
           << "    if (blockIdx.x == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
+        if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(i, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
         for (size_t k = 0; k < NI; ++k) {
             if (bc(k)) o << "        x[" << k << "] = b" << k << ";\n";
             else o << "        x[" << k << "] = " << to_t(k, "in" + std::to_string(k) + "[i]") << ";\n";
         }
         if (NI == 0) o << "        x[0] = zero<T>();\n";
-        o << "        aix_body(x, s, y);\n";
+        o << "        aix_body(x, s, y" << (NT ? ", 0, tpos, a.tp" : "") << ");\n";
         for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "    }\n}\n";
         return o.str();
@@ -228,10 +247,11 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
               << "        else r" << k << " = *(const vec<I" << k << ", VEC>*)(in" << k << " + p[" << k << "] + col);\n";
         }
         for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
+        if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(c * VEC, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
         o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
         for (size_t k = 0; k < NI; ++k) o << "            x[" << k << "] = " << to_t(k, "r" + std::to_string(k) + ".v[e]") << ";\n";
         if (NI == 0) o << "            x[0] = zero<T>();\n";
-        o << "            aix_body(x, s, y);\n";
+        o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
         for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
         for (size_t k = 0; k < NO; ++k) o << "        *(vec<O" << k << ", VEC>*)(out" << k << " + c * VEC) = w" << k << ";\n";
@@ -242,13 +262,14 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     // gather
     o << "    for (u64 i = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; i < a.n; i += (u64)gridDim.x * " << kBlock << ") {\n"
       << "        u64 rest = i;\n        u64 p[" << AI << "];\n";
+    if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(i, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
     for (size_t k = 0; k < NI; ++k) o << "        p[" << k << "] = a.off[" << k << "];\n";
     o << "        for (int d = (int)a.rank - 1; d >= 0; --d) {\n            const u64 q = rest / a.shape[d], r = rest - q * a.shape[d];\n";
     for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
     o << "            rest = q;\n        }\n        T x[" << AI << "], y[" << NO << "];\n";
     for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = " << to_t(k, "in" + std::to_string(k) + "[p[" + std::to_string(k) + "]]") << ";\n";
     if (NI == 0) o << "        x[0] = zero<T>();\n";
-    o << "        aix_body(x, s, y);\n";
+    o << "        aix_body(x, s, y" << (NT ? ", 0, tpos, a.tp" : "") << ");\n";
     for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
     o << "    }\n}\n";
     return o.str();
@@ -268,6 +289,7 @@ void packArgsInto(std::vector<uint64_t>& a, const FusedSubgraphDescriptor& d, Sh
         if (k < NS) std::memcpy(&bits, d.scalarData.data() + k * esz, esz);     // little endian: low bytes
         a.push_back(bits);
     }
+    for (uint64_t v : d.opParams) a.push_back(v);
     a.push_back(n);
     if (shape == Shape::Flat) return;
     if (!space) throw std::invalid_argument("strided fused kernel without an iteration space");

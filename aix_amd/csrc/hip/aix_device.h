@@ -256,6 +256,31 @@ template <class T> __device__ __forceinline__ T e_pow(T a, T b)
     else return int_pow<T>(a, b);
 }
 
+// tril / triu as an elementwise predicate over the flat logical index of a tensor whose last two dims are [rows, cols]:
+// tril keeps columns up to row + diagonal, triu columns from row + diagonal on.  The (row, column) of a vector's first
+// element is found once per vector (two divisions, 32-bit when everything fits); its other elements step the column.
+struct TriPos { i64 r, c; };
+__device__ __forceinline__ TriPos tri_origin(u64 i, u64 rows, u64 cols)
+{
+    TriPos p;
+    if (((i | rows | cols) >> 32) == 0) {
+        const u32 q = (u32)i / (u32)cols;
+        p.c = (i64)((u32)i - q * (u32)cols);
+        p.r = (i64)(q % (u32)rows);
+    } else {
+        const u64 q = i / cols;
+        p.c = (i64)(i - q * cols);
+        p.r = (i64)(q % rows);
+    }
+    return p;
+}
+__device__ __forceinline__ bool tri_keeps(TriPos p, int e, u64 rows, u64 cols, i64 diagonal, int upper)
+{
+    i64 c = p.c + e, r = p.r;
+    while (c >= (i64)cols) { c -= (i64)cols; if (++r == (i64)rows) r = 0; }      // the vector runs over the end of a row
+    return upper ? c >= r + diagonal : c <= r + diagonal;
+}
+
 // ---- 16-byte vectors of any element type ------------------------------------------------------
 template <class T, int N> struct alignas(sizeof(T) * N) vec { T v[N]; };
 template <class T> struct vec16 { enum { n = 16 / sizeof(T) }; typedef vec<T, 16 / sizeof(T)> type; };

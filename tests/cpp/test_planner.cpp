@@ -628,6 +628,60 @@ static void testDenseSidesAdoptTheStridedSidesShape()
     }
 }
 
+static void testTrilJoinsItsNeighbours()
+{
+    // attention scores: tril(s) * scale + mask (mask broadcast over the stack): one kernel; the triangle's extents and
+    // diagonal travel as run-time integers, so another diagonal or stack size reuses the compiled kernel
+    for (int upper = 0; upper < 2; ++upper) {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        const aix::Shape shape{3, 4, 64, 64};
+        auto s = T(1, shape, DataType::kBFloat16), t = T(2, shape, DataType::kBFloat16), scaled = T(3, shape, DataType::kBFloat16), out = T(4, shape, DataType::kBFloat16);
+        auto mask = T(5, shape, DataType::kBFloat16, {0, 0, 64, 1});
+        auto scale0 = T(6, {}, DataType::kBFloat16);
+        auto scale = T(6, shape, DataType::kBFloat16, {0, 0, 0, 0});
+        for (uintptr_t id : {1, 2, 3, 4, 5, 6}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        const float eighth = 0.125f;
+        e.recordTri(upper ? OpType::Triu : OpType::Tril, View(s), View(t), -2);
+        e.recordFill(&eighth, DataType::kFloat32, View(scale0));
+        e.record(OpType::Mul, View(t), View(scale), View(scaled));
+        e.record(OpType::Add, View(scaled), View(mask), View(out));
+        for (uintptr_t id : {2, 3, 6}) e.releaseBuffer(reinterpret_cast<void*>(id * 0x10000));
+        e.flush();
+        CHECK(cap.fused.size() == 1 && cap.singles.empty());
+        if (cap.fused.size() != 1) continue;
+        const auto& d = cap.fused[0];
+        CHECK(d.ops.size() == 3 && d.ops[0].type == (upper ? OpType::Triu : OpType::Tril) && d.ops[0].paramIndex == 0);
+        CHECK(d.opParams.size() == 3 && d.opParams[0] == 64 && d.opParams[1] == 64 && (int64_t)d.opParams[2] == -2);
+        CHECK(d.outputBuffers.size() == 1 && d.inputBuffers.size() == 2);
+        CHECK(compiles(d, gen::Shape::Rows));
+        CHECK(compiles(d, gen::Shape::Gather));
+        const std::string sig = gen::signature(d, gen::Shape::Rows, 0, true);
+        CHECK(sig.find(upper ? "Triu(" : "Tril(") != std::string::npos && sig.find("-2") == std::string::npos);
+        const auto args = gen::packArgs(d, gen::Shape::Flat, {nullptr, nullptr}, {nullptr}, 3 * 4 * 64 * 64, nullptr, 0);
+        CHECK(args.size() == 2 + 1 + 1 + 3 + 1);                  // inputs, output, the scale, (rows, cols, diagonal), n
+    }
+    // alone in its window it runs as the plain operator
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto a = T(1, {8, 8}), b = T(2, {8, 8});
+    for (uintptr_t id : {1, 2}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.recordTri(OpType::Tril, View(a), View(b), 1);
+    e.flush();
+    CHECK(cap.fused.empty() && cap.singles.size() == 1 && cap.singles[0].type == OpType::Tril && cap.singles[0].triDiagonal == 1);
+    // a flat chain of dense tensors: the flat launch shape compiles with the index-dependent operator too
+    Capture flat;
+    FuseEngine f(config(), flat.callbacks());
+    auto x = T(1, {16, 32, 32}), y = T(2, {16, 32, 32}), z = T(3, {16, 32, 32});
+    for (uintptr_t id : {1, 2, 3}) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    f.record(OpType::Exp, View(x), View(y));
+    f.recordTri(OpType::Triu, View(y), View(z), 0);
+    f.releaseBuffer(y.data);
+    f.flush();
+    CHECK(flat.fused.size() == 1 && flat.singles.empty());
+    if (flat.fused.size() == 1) { CHECK(flat.fused[0].allContiguous); CHECK(compiles(flat.fused[0], gen::Shape::Flat)); }
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -654,6 +708,7 @@ int main(int argc, char** argv)
     testTrailingFillIsHandedOver();
     testCastsFuseAtTheirLoadOrStoreEnd();
     testDenseSidesAdoptTheStridedSidesShape();
+    testTrilJoinsItsNeighbours();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

@@ -544,3 +544,49 @@ def test_fill_is_folded_into_argmax_indices_to(dev):
             dev.dev.call("argmax_indices_to", H.ref(dsrc), H.ref(dm), dim)
             T.assert_same_bits(dev.fetch(pm, want.storage), want.storage, f"fill({value}) + argmaxIndicesTo {shape} dim={dim}")
     dev.release()
+
+
+def test_tril_and_triu_join_the_fused_kernels(dev):
+    """tril / triu recorded as elementwise operators: attention's tril(s) * scale + mask is ONE generated kernel
+    (the triangle's extents and diagonal are run-time integers of it), negate -> triu over a dense stack takes the flat
+    launch shape, a transposed source the gather shape; results against the CPU oracle operator by operator."""
+    set_diag(dev)
+    rng = np.random.default_rng(40000)
+    for dtype in (O.BF16, O.F32):
+        for shape, diag, upper in (([2, 3, 40, 48], 0, 0), ([2, 3, 40, 48], -3, 1), ([5, 33, 20], 4, 0), ([64, 64], 1, 1)):
+            rec = Recorder(dev, dtype, shape)
+            s = rec.leaf(T.contiguous_tensor(rng, dtype, shape, lo=-2, hi=2))
+            mask_store = T.random_values(rng, shape[-2] * shape[-1], dtype, lo=-1, hi=1)
+            mask = rec.leaf(T.HostTensor(mask_store, dtype, shape, [0] * (len(shape) - 2) + [shape[-1], 1]))   # uploads flush: before recording
+            # oracle: tril, then * scale, then + mask (mask broadcast over the leading dims)
+            t_host = T.empty(dtype, shape)
+            assert (CPU.triu if upper else CPU.tril)(C.byref(s["host"].desc()), C.byref(t_host.desc()), diag) == 0
+            pt = dev.raw(t_host.storage.nbytes)
+            t = {"host": t_host, "ptr": pt, "desc": H.kdesc(t_host, pt)}
+            dev.dev.call("triu" if upper else "tril", H.ref(s["desc"]), H.ref(t["desc"]), diag)
+            scaled = rec.binary(O.MUL, t, rec.scalar(0.125))
+            out = rec.binary(O.ADD, scaled, mask)
+            got = dev.fetch(out["ptr"], out["host"].storage)
+            T.assert_same_bits(got, out["host"].storage, f"tri(upper={upper}, {diag}) * scale + mask {NAMES[dtype]} {shape}")
+            diagn = dev.dev.diagnostics()
+            assert diagn.fusible_subgraphs == 1 and diagn.fused_ops == 3, diagn.subgraph_summary     # (the scalar's own fill also runs: its tensor is still alive)
+            dev.release()
+        # negate -> triu on a dense stack (flat launch shape), and tril of a transposed view (gather shape) feeding a negate
+        shape = [4, 32, 32]
+        rec = Recorder(dev, dtype, shape)
+        x = rec.leaf(T.contiguous_tensor(rng, dtype, shape, lo=-1, hi=1))
+        e = rec.unary(O.NEG, x)                                         # (exact on both devices)
+        z_host = T.empty(dtype, shape)
+        assert CPU.triu(C.byref(e["host"].desc()), C.byref(z_host.desc()), -1) == 0
+        pz = dev.raw(z_host.storage.nbytes)
+        dev.dev.call("triu", H.ref(e["desc"]), H.ref(H.kdesc(z_host, pz)), -1)
+        T.assert_same_bits(dev.fetch(pz, z_host.storage), z_host.storage, f"negate -> triu {NAMES[dtype]}")
+        xt = T.HostTensor(x["host"].storage, dtype, shape, [32 * 32, 1, 32])
+        w_host = T.empty(dtype, shape)
+        assert CPU.tril(C.byref(xt.desc()), C.byref(w_host.desc()), 2) == 0
+        pw = dev.raw(w_host.storage.nbytes)
+        w = {"host": w_host, "ptr": pw, "desc": H.kdesc(w_host, pw)}
+        dev.dev.call("tril", H.ref(H.kdesc(xt, x["ptr"])), H.ref(w["desc"]), 2)
+        neg = rec.unary(O.NEG, w)
+        T.assert_same_bits(dev.fetch(neg["ptr"], neg["host"].storage), neg["host"].storage, f"tril(transposed view) -> negate {NAMES[dtype]}")
+        dev.release()
