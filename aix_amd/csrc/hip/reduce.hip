@@ -427,6 +427,45 @@ __global__ __launch_bounds__(kBlock) void argmax_onehot_rows_k(const T* __restri
     }
 }
 
+// argmaxIndicesTo along a unit-stride dim with the zero-initialisation folded in (the mask of a softmax's max() backward:
+// fill(0) + argmaxIndicesTo over rows of 512): a wave finds the winner of a row -- the arithmetic of
+// reduce_inner_k<ArgOp, T, kWave, .> -- and writes the row's one-hot block densely, 16 bytes per lane and step.
+template <class T, bool VECT>
+__global__ __launch_bounds__(kBlock) void argmax_onehot_inner_k(const T* __restrict__ src, i32* __restrict__ dst, RedPlan p)
+{
+    typedef ArgOp<T> Op;
+    typedef typename Op::Acc Acc;
+    typedef typename vec16<T>::type V;
+    constexpr int VEC = vec16<T>::n;
+    typedef vec<i32, 4> O4;
+    const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
+    const u64 L = p.r_ext[0];
+    for (u64 slot = (u64)blockIdx.x * kWaves + w; slot < p.slots; slot += (u64)gridDim.x * kWaves) {
+        const SlotPos s = slot_pos(p, slot, p.nk);
+        const T* row = src + s.src;
+        Acc acc = Op::init();                                                           // candidates carry their position in the row
+        if constexpr (VECT) {
+            for (u64 v = l; v < L / VEC; v += kWave) {
+                const V x = *(const V*)(row + v * VEC);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) { const u64 j = v * VEC + e; Op::step(acc, x.v[e], j, j == 0); }
+            }
+        } else {
+            for (u64 j = l; j < L; j += kWave) Op::step(acc, row[j], j, j == 0);
+        }
+        acc = wave_reduce<Op>(acc);
+        const u32 mine = (acc.flags & 2u) ? 0u : acc.idx;                               // a leading NaN wins (as land() has it)
+        const u32 winner = __shfl(mine, 0, kWave);
+        i32* out = dst + s.flat;                                                         // the row is contiguous in the flat order
+        for (u64 j0 = (u64)l * 4; j0 < L; j0 += (u64)kWave * 4) {
+            O4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v.v[e] = (u32)(j0 + e) == winner ? 1 : 0;
+            *(O4*)(out + j0) = v;
+        }
+    }
+}
+
 // second stage of `outer` when rows were split over several workgroups: 64 slots per workgroup,
 // the four waves take every fourth chunk (independent loads in flight), LDS folds the four.
 template <class Op, class T>
@@ -538,6 +577,16 @@ int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const 
 
 // Does argmax_onehot_rows_k take this plan?  One reduced dim of fewer than 8 rows, the innermost kept dim dense on both
 // sides, everything aligned for VEC-wide accesses.
+// Does argmax_onehot_inner_k take this plan?  One reduced dim with unit source stride that is also the innermost dim of
+// the flat order, rows of a multiple of 4 elements that start 16-byte aligned in the destination.
+inline bool onehot_inner_route(const RedPlan& p, const void* dst)
+{
+    if (!(p.nk >= 1 && p.nr == 1 && p.r_src[0] == 1 && p.r_flat[0] == 1 && p.red >= 32 && p.red % 4 == 0 && p.red < (1ull << 31))) return false;
+    if (!aligned16(dst)) return false;
+    for (int d = 0; d < p.nk; ++d) if (p.k_flat[d] % 4) return false;
+    return true;
+}
+
 template <class T>
 bool onehot_rows_route(const RedPlan& p, const T* ps, const void* dst)
 {
@@ -564,6 +613,18 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
     if (p.nk == 0) return run_all<Op, T>(ctx, src, dst, fin);
 
     // inner: one reduced dim with unit source stride
+    if constexpr (Op::kTracksIndex) {
+        if (fin.onehot == 2 && onehot_inner_route(p, dst)) {
+            // a row per wave, all rows in flight at once
+            bool vect = p.red % VEC16 == 0 && aligned16(ps + p.src_off);
+            for (int d = 0; d < p.nk; ++d) if (p.k_src[d] % VEC16) vect = false;
+            const unsigned rows_grid = grid_for(p.slots, kWaves, 1u << 30);
+            if (vect) hipLaunchKernelGGL((argmax_onehot_inner_k<T, true>), dim3(rows_grid), dim3(kBlock), 0, st, ps, (i32*)dst, p);
+            else hipLaunchKernelGGL((argmax_onehot_inner_k<T, false>), dim3(rows_grid), dim3(kBlock), 0, st, ps, (i32*)dst, p);
+            AIXK_HIP(hipGetLastError());
+            return AIXK_OK;
+        }
+    }
     if (p.nr == 1 && p.r_src[0] == 1 && p.red >= 32) {
         bool vect = p.red % VEC16 == 0 && aligned16(ps + p.src_off);
         for (int d = 0; d < p.nk; ++d) if (p.k_src[d] % VEC16) vect = false;
@@ -771,7 +832,7 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
     if (!make_plan(src, weight, &plan)) return fail(AIXK_EINVAL, "argmaxTo: view does not collapse to %d dims", kMaxDims);
     return by_dtype(src->dtype, [&](auto tag) {
         typedef decltype(tag) T;
-        if (fin.onehot == 2 && !onehot_rows_route<T>(plan, (const T*)src->data, dst->data)) {
+        if (fin.onehot == 2 && !onehot_rows_route<T>(plan, (const T*)src->data, dst->data) && !onehot_inner_route(plan, dst->data)) {
             // the zero-initialisation this call owes, as a pass of its own, then ones scattered as usual
             AIXK_TRY(aixk_zero(ctx, dst->data, src->size * sizeof(int32_t)));
             fin.onehot = 1;
