@@ -478,19 +478,30 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
 // attention-sized products.  BM x BN workgroup tile (128 x 128, 128 x 64, 64 x 64), BK = 32, four waves 2 x 2,
 // two LDS stages filled from registers (the next step's global loads are in flight under this step's MFMAs), one
 // barrier per step; 41 KB of LDS at most, so several workgroups share a compute unit and overlap each other's
-// barriers and LDS reads.  Both operand forms are consumed where they lie, exactly as in gemm_small16_k:
-// K-contiguous staged [row][k] with a pitch of 40 elements (80 bytes: 16 consecutive rows start in 16 different
-// groups of four banks), T form staged [k][row] with a pitch of tile + 32 elements (64 or 192 bytes modulo 256: the
-// four k-rows a group of 16 lanes reads, and the two groups of a half-wave, fall into disjoint banks).
+// barriers and LDS reads.  Both operand forms are consumed where they lie: K-contiguous staged [row][k], unpadded, with
+// the 16-byte chunks of a row XOR-swizzled (kswz below); T form staged [k][row] with a pitch of tile + 32 elements (64 or
+// 192 bytes modulo 256: the four k-rows a group of 16 lanes reads with ds_read_b64_tr_b16, and the two groups of a
+// half-wave, fall into disjoint banks).  SQ_LDS_BANK_CONFLICT = 0 for both.
 //
 // blockIdx.y numbers the matrices of a stack (BatchArgs).  blockIdx.z numbers K splits: split s multiplies K steps
 // [s * per_split, (s + 1) * per_split) and, when there is more than one split, stores its f32 partial tile in
 // `partial` ([split][matrix][M][N]) for splitk_finish_k to add up in split order and round once.
 struct SplitArgs { float* partial; u32 splits, per_split; u64 matrices; };
 
+// K-contiguous operands are staged without padding: row r keeps its 16-byte k-chunk q in slot q ^ kswz<BK>(r).  A group of 8
+// (or 16) lanes that writes whole rows then covers 128 (256) contiguous bytes, and the fragment reads -- 32 consecutive
+// rows, one chunk -- fall into disjoint banks under both an 8-lane / 32-bank and a 16-lane / 64-bank service (padded rows
+// of 80 bytes read without conflicts but cost a third of the LDS cycles in write conflicts, by SQ_LDS_BANK_CONFLICT).
+// Only bits 0..3 of r enter, so a row's swizzle is known from the lane that owns it.
+template <int BK> __device__ __forceinline__ int kswz(int r)
+{
+    if constexpr (BK == 64) return ((r >> 1) & 7) ^ ((r & 1) << 2);          // 8 chunks per row (gemm_nt16_direct_k's)
+    else return (r ^ (r >> 2)) & 3;                                           // 4 chunks per row
+}
+
 template <int BM, int BN, int BK_, bool AT, bool BT> struct Tile16 {
-    static constexpr int BK = BK_, PK = BK + 8, PA = BM + 32, PB = BN + 32;
-    static constexpr int SA = AT ? BK * PA : BM * PK, SB = BT ? BK * PB : BN * PK;       // elements per stage
+    static constexpr int BK = BK_, PA = BM + 32, PB = BN + 32;
+    static constexpr int SA = AT ? BK * PA : BM * BK, SB = BT ? BK * PB : BN * BK;       // elements per stage
     static constexpr size_t kLds = (size_t)2 * (SA + SB) * 2;
 };
 
@@ -498,9 +509,10 @@ template <class T, int BM, int BN, int BKT, bool AT, bool BT>
 __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, SplitArgs sk)
 {
     typedef Tile16<BM, BN, BKT, AT, BT> S;
-    constexpr int BK = S::BK, PK = S::PK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
+    constexpr int BK = S::BK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
     constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
     constexpr int CA = BM * (BK / 8) / 256, CB = BN * (BK / 8) / 256;        // 16-byte chunks per lane and step
+    constexpr int CH = BK / 8;                                                // chunks per K-contiguous row
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_tile[];
     u16* As = (u16*)smem_tile;                            // [2][SA]
     u16* Bs = As + 2 * SA;                                // [2][SB]
@@ -548,20 +560,19 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             const int c = tid + 256 * i;
-            *(u32x4*)(As + buf * SA + (AT ? (c / (BM / 8)) * PA + (c % (BM / 8)) * 8 : (c / (BK / 8)) * PK + (c % (BK / 8)) * 8)) = ra[i];
+            *(u32x4*)(As + buf * SA + (AT ? (c / (BM / 8)) * PA + (c % (BM / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = ra[i];
         }
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
             const int c = tid + 256 * i;
-            *(u32x4*)(Bs + buf * SB + (BT ? (c / (BN / 8)) * PB + (c % (BN / 8)) * 8 : (c / (BK / 8)) * PK + (c % (BK / 8)) * 8)) = rb[i];
+            *(u32x4*)(Bs + buf * SB + (BT ? (c / (BN / 8)) * PB + (c % (BN / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = rb[i];
         }
     };
-    // fragment addresses inside a stage for the wave's first 32 rows and the 16-wide K slice 0
-    const int j16 = lane & 15;
-    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM
-                       : (wm * WM + (lane & 31)) * PK + (lane >> 5) * 8;
-    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN
-                       : (wn * WN + (lane & 31)) * PK + (lane >> 5) * 8;
+    // fragment addresses inside a stage for the wave's first 32 rows: T form for the 16-wide K slice 0; K-contiguous: the
+    // row's start, the chunk (lane / 32 + 2 kk) goes through the row's swizzle
+    const int j16 = lane & 15, swz = kswz<BK>(lane & 31), half = lane >> 5;
+    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM : (wm * WM + (lane & 31)) * BK;
+    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN : (wn * WN + (lane & 31)) * BK;
 
     const u64 steps = (g.K + BK - 1) / BK;
     const u64 first = (u64)blockIdx.z * sk.per_split;
@@ -579,13 +590,14 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
             u32x4 fa[TI], fb[TJ];
+            const int slot = ((half + 2 * kk) ^ swz) * 8;
 #pragma unroll
             for (int i = 0; i < TI; ++i) {
-                if constexpr (AT) fa[i] = tr_fragment_lds<PA>(as + i * 32 + kk * 16 * PA); else fa[i] = *(const u32x4*)(as + i * 32 * PK + kk * 16);
+                if constexpr (AT) fa[i] = tr_fragment_lds<PA>(as + i * 32 + kk * 16 * PA); else fa[i] = *(const u32x4*)(as + i * 32 * BK + slot);
             }
 #pragma unroll
             for (int j = 0; j < TJ; ++j) {
-                if constexpr (BT) fb[j] = tr_fragment_lds<PB>(bs + j * 32 + kk * 16 * PB); else fb[j] = *(const u32x4*)(bs + j * 32 * PK + kk * 16);
+                if constexpr (BT) fb[j] = tr_fragment_lds<PB>(bs + j * 32 + kk * 16 * PB); else fb[j] = *(const u32x4*)(bs + j * 32 * BK + slot);
             }
 #pragma unroll
             for (int i = 0; i < TI; ++i)
@@ -639,7 +651,7 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
 // gemm_x3_k: 128 x 128 x 32 tile, four waves 2 x 2.  The operands are read from memory as f32 (K-contiguous or T
 // form, 16-byte chunks of four values), split in registers, and staged as three bf16 planes per operand with the
 // layouts of gemm_tile16_k (so the fragment reads, including ds_read_b64_tr_b16 for T-form operands, are the same);
-// a wave reads 12 fragments per 24 MFMAs.  One LDS stage of 60 KB (two workgroups per compute unit) and two barriers
+// a wave reads 12 fragments per 24 MFMAs.  One LDS stage of 48-60 KB (two workgroups per compute unit) and two barriers
 // per K step: the next step's global loads are in flight during the MFMAs.  blockIdx.z numbers K splits as in
 // gemm_tile16_k.
 //
@@ -650,8 +662,8 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
 // once unless the flag carries this number -- redoes the whole product with IEEE arithmetic (which also covers sums
 // that overflow on their own: the redo returns the same infinities).
 template <bool AT, bool BT> struct TileX3 {
-    static constexpr int BM = 128, BN = 128, BK = 32, PK = BK + 8, PA = BM + 32, PB = BN + 32;
-    static constexpr int SA = AT ? BK * PA : BM * PK, SB = BT ? BK * PB : BN * PK;       // bf16 elements per plane
+    static constexpr int BM = 128, BN = 128, BK = 32, PA = BM + 32, PB = BN + 32;
+    static constexpr int SA = AT ? BK * PA : BM * BK, SB = BT ? BK * PB : BN * BK;       // bf16 elements per plane
     static constexpr size_t kLds = (size_t)3 * (SA + SB) * 2;
 };
 
@@ -681,9 +693,12 @@ template <bool AT, bool BT>
 __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* flag, u32 seq)
 {
     typedef TileX3<AT, BT> S;
-    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, PK = S::PK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
+    constexpr int BM = S::BM, BN = S::BN, BK = S::BK, PA = S::PA, PB = S::PB, SA = S::SA, SB = S::SB;
     constexpr int WM = BM / 2, WN = BN / 2, TI = WM / 32, TJ = WN / 32;
     constexpr int CA = BM * (BK / 4) / 256, CB = BN * (BK / 4) / 256;        // 16-byte chunks (4 values) per lane and step
+    constexpr int C4 = BK / 4;                                                // 4-value chunks per K-contiguous row
+    // K-contiguous plane rows are unpadded and swizzled (kswz): the 4 values of chunk k4 are one half of 16-byte slot k4 / 2
+    auto kplace = [](int c) { const int r = c / C4, k4 = c % C4; return r * BK + (((k4 >> 1) ^ kswz<BK>(r)) * 8) + (k4 & 1) * 4; };
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_x3[];
     u16* As = (u16*)smem_x3;                              // [3][SA]
     u16* Bs = As + 3 * SA;                                // [3][SB]
@@ -723,7 +738,7 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             const int c = tid + 256 * i;
-            const int at = AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
+            const int at = AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : kplace(c);
             u32x2 h, m, l;
             split3(ra[i], h, m, l);
             *(u32x2*)(As + at) = h; *(u32x2*)(As + SA + at) = m; *(u32x2*)(As + 2 * SA + at) = l;
@@ -731,17 +746,15 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
             const int c = tid + 256 * i;
-            const int at = BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : (c / (BK / 4)) * PK + (c % (BK / 4)) * 4;
+            const int at = BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : kplace(c);
             u32x2 h, m, l;
             split3(rb[i], h, m, l);
             *(u32x2*)(Bs + at) = h; *(u32x2*)(Bs + SB + at) = m; *(u32x2*)(Bs + 2 * SB + at) = l;
         }
     };
-    const int j16 = lane & 15;
-    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM
-                       : (wm * WM + (lane & 31)) * PK + (lane >> 5) * 8;
-    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN
-                       : (wn * WN + (lane & 31)) * PK + (lane >> 5) * 8;
+    const int j16 = lane & 15, swz = kswz<BK>(lane & 31), half = lane >> 5;
+    const int fa0 = AT ? (8 * (lane >> 5) + (j16 >> 2)) * PA + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wm * WM : (wm * WM + (lane & 31)) * BK;
+    const int fb0 = BT ? (8 * (lane >> 5) + (j16 >> 2)) * PB + 16 * ((lane >> 4) & 1) + 4 * (j16 & 3) + wn * WN : (wn * WN + (lane & 31)) * BK;
 
     const u64 steps = (g.K + BK - 1) / BK;
     const u64 first = (u64)blockIdx.z * sk.per_split;
@@ -754,17 +767,18 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
             u32x4 fa[3][TI], fb[3][TJ];
+            const int slot = ((half + 2 * kk) ^ swz) * 8;
 #pragma unroll
             for (int p = 0; p < 3; ++p) {
 #pragma unroll
                 for (int i = 0; i < TI; ++i) {
                     const u16* q = As + p * SA + fa0;
-                    if constexpr (AT) fa[p][i] = tr_fragment_lds<PA>(q + i * 32 + kk * 16 * PA); else fa[p][i] = *(const u32x4*)(q + i * 32 * PK + kk * 16);
+                    if constexpr (AT) fa[p][i] = tr_fragment_lds<PA>(q + i * 32 + kk * 16 * PA); else fa[p][i] = *(const u32x4*)(q + i * 32 * BK + slot);
                 }
 #pragma unroll
                 for (int j = 0; j < TJ; ++j) {
                     const u16* q = Bs + p * SB + fb0;
-                    if constexpr (BT) fb[p][j] = tr_fragment_lds<PB>(q + j * 32 + kk * 16 * PB); else fb[p][j] = *(const u32x4*)(q + j * 32 * PK + kk * 16);
+                    if constexpr (BT) fb[p][j] = tr_fragment_lds<PB>(q + j * 32 + kk * 16 * PB); else fb[p][j] = *(const u32x4*)(q + j * 32 * BK + slot);
                 }
             }
             // smallest contributions first; four independent accumulators between two uses of the same one
