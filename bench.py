@@ -262,6 +262,15 @@ def main():
                                             f"this algorithm is the bf16 peak / 6 = {MFMA_PEAK_TFLOPS['bf16'] / 6:.1f} TFLOP/s "
                                             f"(frac {line['roofline']['achieved'] / (MFMA_PEAK_TFLOPS['bf16'] / 6):.3f}); peak and frac above are the f32 MFMA's")
             extras.append(line)
+        # the same 4096^3 bf16 product on all-zero operands: same kernel, same instruction stream, no bits toggling in the
+        # matrix pipe -- the gap to the line above is the clock the part gives up under the power of real operands
+        hz = np.zeros((4096, 4096), np.uint16)
+        r = BenchResult()
+        run(lib, "aixbench_matmul", dev.handle, codes["bf16"], 4096, 4096, 4096, 0, 1, hz.ctypes.data, hz.ctypes.data, 20, 2, C.byref(r), None)
+        flops = 2.0 * 4096 ** 3
+        extras.append({"workload": "configs[2] matmul bf16 4096^3 NN, ALL-ZERO operands (diagnostic of the power limit, not a result)",
+                       "ms_per_step": round(r.wall_s * 1e3 / 20, 5), "value": round(flops * 20 / r.wall_s / 1e12, 2), "unit": "TFLOP/s",
+                       "roofline": roofline("mfma", flops / (r.gpu_ms / 20 * 1e-3) / 1e12, MFMA_PEAK_TFLOPS["bf16"], "TFLOP/s")})
         host.clear()
     if not args.no_extras and "c3" in chosen:
         # configs[3]: MLP training step (autograd + Adam); the CPU device runs the first steps of the same program
