@@ -476,9 +476,10 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
 // Everything between the two kernels above: outputs of a few hundred tiles (a [8192, 768] activation times a
 // [768, 768] weight), weight gradients with few tiles and a very long K ([768, 8192] x [8192, 768]), and stacks of
 // attention-sized products.  BM x BN workgroup tile (128 x 128, 128 x 64, 64 x 64), BK = 32, four waves 2 x 2,
-// two LDS stages filled from registers (the next step's global loads are in flight under this step's MFMAs), one
-// barrier per step; 41 KB of LDS at most, so several workgroups share a compute unit and overlap each other's
-// barriers and LDS reads.  Both operand forms are consumed where they lie: K-contiguous staged [row][k], unpadded, with
+// two LDS stages filled from registers -- for interior tiles from a ring of register stages that keeps the global
+// loads of the next 2-3 K steps in flight, for edge tiles one step ahead -- one barrier per step; 41 KB of LDS at
+// most, so several workgroups share a compute unit and overlap each other's barriers and LDS reads.  Results leave
+// through LDS as 16-byte stores.  Both operand forms are consumed where they lie: K-contiguous staged [row][k], unpadded, with
 // the 16-byte chunks of a row XOR-swizzled (kswz below); T form staged [k][row] with a pitch of tile + 32 elements (64 or
 // 192 bytes modulo 256: the four k-rows a group of 16 lanes reads with ds_read_b64_tr_b16, and the two groups of a
 // half-wave, fall into disjoint banks).  SQ_LDS_BANK_CONFLICT = 0 for both.
@@ -541,31 +542,56 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    u32x4 ra[CA], rb[CB];
-    auto load_global = [&](u64 k0) {
+    // Register stages between global memory and LDS.  A tile whose rows, columns and K steps all lie inside the operands
+    // ("interior") is fetched by unconditional loads, DEPTH K-steps ahead: only then can the in-order load counter tell
+    // "the oldest tile has arrived" from "everything has arrived" (a load under a bounds check is a branch, and behind a
+    // branch the compiler waits for every load in flight), and with 4-8 MFMAs per wave and step nothing but that distance
+    // covers the latency of a load.  Edge tiles take the checked loads, one step ahead.
+    constexpr int DEPTH = BM * BN >= 128 * 128 ? 2 : 3;            // registers: the 128 x 128 tile keeps three waves per SIMD with 2
+    u32x4 ra[DEPTH][CA], rb[DEPTH][CB];
+    auto load_global = [&](u64 k0, u32x4* pa, u32x4* pb) {
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             const int c = tid + 256 * i;
-            if constexpr (AT) { const u64 k = k0 + c / (BM / 8), m = m0 + (c % (BM / 8)) * 8; ra[i] = (k < g.K && m < g.M) ? *(const u32x4*)(A + k * g.lda + m) : (u32x4){0, 0, 0, 0}; }
-            else { const u64 m = m0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; ra[i] = (m < g.M && k < g.K) ? *(const u32x4*)(A + m * g.lda + k) : (u32x4){0, 0, 0, 0}; }
+            if constexpr (AT) { const u64 k = k0 + c / (BM / 8), m = m0 + (c % (BM / 8)) * 8; pa[i] = (k < g.K && m < g.M) ? *(const u32x4*)(A + k * g.lda + m) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 m = m0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; pa[i] = (m < g.M && k < g.K) ? *(const u32x4*)(A + m * g.lda + k) : (u32x4){0, 0, 0, 0}; }
         }
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
             const int c = tid + 256 * i;
-            if constexpr (BT) { const u64 k = k0 + c / (BN / 8), n = n0 + (c % (BN / 8)) * 8; rb[i] = (k < g.K && n < g.N) ? *(const u32x4*)(B + k * g.ldb + n) : (u32x4){0, 0, 0, 0}; }
-            else { const u64 n = n0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; rb[i] = (n < g.N && k < g.K) ? *(const u32x4*)(B + n * g.ldb + k) : (u32x4){0, 0, 0, 0}; }
+            if constexpr (BT) { const u64 k = k0 + c / (BN / 8), n = n0 + (c % (BN / 8)) * 8; pb[i] = (k < g.K && n < g.N) ? *(const u32x4*)(B + k * g.ldb + n) : (u32x4){0, 0, 0, 0}; }
+            else { const u64 n = n0 + c / (BK / 8), k = k0 + (c % (BK / 8)) * 8; pb[i] = (n < g.N && k < g.K) ? *(const u32x4*)(B + n * g.ldb + k) : (u32x4){0, 0, 0, 0}; }
         }
     };
-    auto store_lds = [&](int buf) {
+    // the same without checks: the lane's part of the address once, the K step enters as a uniform offset
+    const u16 *ga[CA], *gb[CB];
+#pragma unroll
+    for (int i = 0; i < CA; ++i) {
+        const int c = tid + 256 * i;
+        ga[i] = AT ? A + (u64)(c / (BM / 8)) * g.lda + m0 + (c % (BM / 8)) * 8 : A + (m0 + c / (BK / 8)) * g.lda + (c % (BK / 8)) * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < CB; ++i) {
+        const int c = tid + 256 * i;
+        gb[i] = BT ? B + (u64)(c / (BN / 8)) * g.ldb + n0 + (c % (BN / 8)) * 8 : B + (n0 + c / (BK / 8)) * g.ldb + (c % (BK / 8)) * 8;
+    }
+    const u64 ka = AT ? (u64)BK * g.lda : (u64)BK, kb = BT ? (u64)BK * g.ldb : (u64)BK;      // elements per K step
+    auto load_interior = [&](u64 kt, u32x4* pa, u32x4* pb) {
+#pragma unroll
+        for (int i = 0; i < CA; ++i) pa[i] = *(const u32x4*)(ga[i] + kt * ka);
+#pragma unroll
+        for (int i = 0; i < CB; ++i) pb[i] = *(const u32x4*)(gb[i] + kt * kb);
+    };
+    auto store_lds = [&](int buf, const u32x4* pa, const u32x4* pb) {
 #pragma unroll
         for (int i = 0; i < CA; ++i) {
             const int c = tid + 256 * i;
-            *(u32x4*)(As + buf * SA + (AT ? (c / (BM / 8)) * PA + (c % (BM / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = ra[i];
+            *(u32x4*)(As + buf * SA + (AT ? (c / (BM / 8)) * PA + (c % (BM / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = pa[i];
         }
 #pragma unroll
         for (int i = 0; i < CB; ++i) {
             const int c = tid + 256 * i;
-            *(u32x4*)(Bs + buf * SB + (BT ? (c / (BN / 8)) * PB + (c % (BN / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = rb[i];
+            *(u32x4*)(Bs + buf * SB + (BT ? (c / (BN / 8)) * PB + (c % (BN / 8)) * 8 : (c / CH) * BK + ((c % CH) ^ kswz<BK>(c / CH)) * 8)) = pb[i];
         }
     };
     // fragment addresses inside a stage for the wave's first 32 rows: T form for the 16-wide K slice 0; K-contiguous: the
@@ -577,14 +603,7 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
     const u64 steps = (g.K + BK - 1) / BK;
     const u64 first = (u64)blockIdx.z * sk.per_split;
     const u64 last = first + sk.per_split < steps ? first + sk.per_split : steps;
-    if (first < last) {
-        load_global(first * BK);
-        store_lds(0);
-    }
-    __syncthreads();
-    for (u64 kt = first; kt < last; ++kt) {
-        const int buf = (int)((kt - first) & 1);
-        if (kt + 1 < last) load_global((kt + 1) * BK);
+    auto multiply = [&](int buf) {
         const u16* as = As + buf * SA + fa0;
         const u16* bs = Bs + buf * SB + fb0;
 #pragma unroll
@@ -604,7 +623,44 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 #pragma unroll
                 for (int j = 0; j < TJ; ++j) acc[i][j] = Mma16<T>::run(fa[i], fb[j], acc[i][j]);
         }
-        if (kt + 1 < last) store_lds(buf ^ 1);
+    };
+    // (short K: the ring's first loads would fetch the last tile over and over)
+    const bool interior = m0 + BM <= g.M && n0 + BN <= g.N && g.K % BK == 0 && last - first >= 2 * DEPTH + 2;
+    u64 kt = first;
+    if (first < last) {
+        if (interior) {
+            // ring slot d holds tile t + 1 when step t = first + d (mod DEPTH) begins; tiles past the end re-read the last one
+            const u64 end = last - 1;
+            load_interior(first, ra[0], rb[0]);
+            store_lds(0, ra[0], rb[0]);
+#pragma unroll
+            for (int d = 0; d < DEPTH; ++d) { const u64 t = first + 1 + d; load_interior(t < end ? t : end, ra[d], rb[d]); }
+            __syncthreads();
+            // whole turns of the ring, in a loop without exits between the steps (an exit would merge states in which different
+            // slots hold the youngest loads, and the wait for one slot would become a wait for all)
+            for (; kt + DEPTH <= last; kt += DEPTH) {
+#pragma unroll
+                for (int d = 0; d < DEPTH; ++d) {
+                    const u64 t = kt + d, nt = t + 1 + DEPTH;
+                    const int buf = (int)((t - first) & 1);
+                    store_lds(buf ^ 1, ra[d], rb[d]);                 // tile t + 1 (behind the last step: a copy nobody reads)
+                    load_interior(nt < end ? nt : end, ra[d], rb[d]);
+                    multiply(buf);
+                    __syncthreads();
+                }
+            }
+        } else {
+            load_global(first * BK, ra[0], rb[0]);
+            store_lds(0, ra[0], rb[0]);
+        }
+    }
+    __syncthreads();
+    // edge tiles, and the steps an interior tile has left after the last whole turn (its tile kt is staged already)
+    for (; kt < last; ++kt) {
+        const int buf = (int)((kt - first) & 1);
+        if (kt + 1 < last) load_global((kt + 1) * BK, ra[0], rb[0]);
+        multiply(buf);
+        if (kt + 1 < last) store_lds(buf ^ 1, ra[0], rb[0]);
         __syncthreads();
     }
 
@@ -612,6 +668,36 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
     const u64 plane = g.M * g.N;
     T* C = (T*)g.c + (u64)blockIdx.y * plane;
     float* P = sk.splits > 1 ? sk.partial + ((u64)blockIdx.z * sk.matrices + blockIdx.y) * plane : nullptr;
+    if (!P && g.N % 8 == 0 && ((size_t)g.c & 15) == 0) {
+        // Through LDS (free after the last barrier), each wave on its own 32 x 32 slab: written as the MFMA leaves it (a lane
+        // = a column), read back as runs of 8 columns, rounded and stored 16 bytes per lane: an eighth of the store
+        // instructions of two-byte stores straight from the accumulators (4-8 % of a [8192, 768] x [768, 768] product; the
+        // f32 partial tiles of a K split gain nothing from the detour and go out directly).
+        constexpr int PITCH = 36;
+        static_assert((size_t)4 * 32 * PITCH * 4 <= S::kLds, "the epilogue slabs fit into the stages");
+        float* slab = (float*)smem_tile + wave * (32 * PITCH);
+#pragma unroll
+        for (int i = 0; i < TI; ++i)
+#pragma unroll
+            for (int j = 0; j < TJ; ++j) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) slab[((v >> 2) * 8 + (lane >> 5) * 4 + (v & 3)) * PITCH + (lane & 31)] = acc[i][j][v];
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    const int grp = lane + 64 * t, r = grp >> 2, cg = grp & 3;
+                    const f32x4 lo = *(const f32x4*)(slab + r * PITCH + cg * 8);
+                    const f32x4 hi = *(const f32x4*)(slab + r * PITCH + cg * 8 + 4);
+                    const u64 row = m0 + wm * WM + i * 32 + r, col = n0 + wn * WN + j * 32 + cg * 8;
+                    if (row < g.M && col < g.N) {
+                        u32x4 o;
+                        o.x = Mma16<T>::pack(lo.x, lo.y); o.y = Mma16<T>::pack(lo.z, lo.w);
+                        o.z = Mma16<T>::pack(hi.x, hi.y); o.w = Mma16<T>::pack(hi.z, hi.w);
+                        *(u32x4*)(C + row * g.N + col) = o;
+                    }
+                }
+            }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
@@ -1151,7 +1237,7 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         return launch_small16(ctx, a, b, out, nullptr);
     }
     if (K >= 4096 && t128 < 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 2, splits_for(t128, (K + 31) / 32, 2));
-    if (t128 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
+    if (t128 >= cus + cus / 2) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
     if (t12864 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 1, 1);
     return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
 }

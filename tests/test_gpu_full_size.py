@@ -181,8 +181,24 @@ def _rect_properties(gpu, dtype, m, k, n, layout, rng, tol_rel):
     gpu.release()
 
 
+@pytest.mark.parametrize("tile", [(2048, 3072), (2048, 2048), (1024, 2048)], ids=["128x128", "128x64", "64x64"])
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN", "TT"])
+def test_matmul_prefetch_ring_every_remainder(gpu, tile, layout):
+    """Interior tiles of the mid-size kernel fetch their operands several K steps ahead through a ring of register stages
+    and finish the steps left over after the last whole turn of the ring one step ahead; tiles on a ragged edge take
+    bounds-checked loads throughout.  Every number of left-over steps for rings of 2 and 3 stages, with whole tiles only
+    and with a ragged last tile row and column next to interior tiles, for each tile size and operand form."""
+    m, n = tile
+    bk = 64 if tile == (1024, 2048) else 32
+    rng = np.random.default_rng(6600 + m + n)
+    for steps in (7, 8, 9, 10, 11, 12, 13):
+        _rect_properties(gpu, O.BF16, m, steps * bk, n, layout, rng, 1e-5)
+    _rect_properties(gpu, O.F16, m - 40, 11 * bk, n - 24, layout, rng, 1e-5)
+    _rect_properties(gpu, O.BF16, m - 8, 10 * bk + 8, n, layout, rng, 1e-5)         # K not a whole number of steps: checked loads everywhere
+
+
 @pytest.mark.parametrize("case", [
-    (8192, 768, 768, "NT"), (8192, 768, 768, "NN"), (8192, 3072, 768, "NN"),      # activations x weights: 128 x 64 tiles
+    (8192, 768, 768, "NT"), (8192, 768, 768, "NN"), (8192, 3072, 768, "NN"),      # activations x weights: 128 x 128 / 128 x 64 tiles
     (768, 8192, 768, "TN"), (768, 8192, 768, "TT"),                                 # a weight gradient (x^T . dy, both given row-major) and the same with dy transposed: 64 x 64 tiles, K split 8 ways
     (768, 8192, 3072, "TT"), (3072, 8192, 768, "TN"),                               # 128 x 128 tiles, K split 4 ways
     (768, 8192, 8192, "TT"),                                                        # the output projection's gradient: K split 2 ways
