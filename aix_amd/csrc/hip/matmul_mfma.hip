@@ -1230,13 +1230,29 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, splits_for(t12864 * count, (K + 31) / 32, 2));
         return launch_tile16(ctx, a, b, out, batch, 2, splits_for(t128 * count, (K + 31) / 32, 2));
     }
+    if (K >= 4096 && t128 < 2 * cus && M >= 128 && N >= 128) {
+        // a long K and few tiles (weight gradients): 128 x 128 tiles, K split over workgroups.  Splits shorten every
+        // workgroup's chain of K steps, as long as the workgroups still find a compute unit each (a second round of
+        // workgroups doubles the time), and each adds an f32 copy of the result to write and read back: with a step and
+        // a MB of partial result at the same price (about 0.3 us) the cheapest split count by this sum was the measured
+        // optimum, or within 3 % of it, on [768, 768 | 2304 | 3072 | 8192] x K 8192, 768^2, 1024^2 and 1536^2 x K 4096,
+        // 512^2 x K 8192 and [2048, 1024] x K 16384 (3, 2, 6, 2, 6, 4, 3, 8, 2 splits).
+        const uint64_t steps = (K + 31) / 32, most = std::max<uint64_t>(1, std::min<uint64_t>(steps / 16, 16));
+        const double mb = (double)M * (double)N * 4e-6;
+        uint64_t splits = 1;
+        double least = 0.0;
+        for (uint64_t sp = 1; sp <= most; ++sp) {
+            const double cost = (double)((t128 * sp + cus - 1) / cus) * (double)((steps + sp - 1) / sp) + (sp > 1 ? (double)sp * mb : 0.0);
+            if (sp == 1 || cost < least) { least = cost; splits = sp; }
+        }
+        return launch_tile16(ctx, a, b, out, nullptr, 2, splits);
+    }
     if (t64 < 2 * cus) {
         // outputs that 64 x 64 tiles cannot spread over the chip twice: with a long K, 64 x 64 tiles and K split over
         // workgroups; otherwise 32 x 32 tiles with K split over the waves (1024^3 NN: 11.8 us against 12.7)
         if (K >= 4096) return launch_tile16(ctx, a, b, out, nullptr, 0, splits_for(t64, (K + 63) / 64 * 2, 4));
         return launch_small16(ctx, a, b, out, nullptr);
     }
-    if (K >= 4096 && t128 < 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 2, splits_for(t128, (K + 31) / 32, 2));
     if (t128 >= cus + cus / 2) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
     if (t12864 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 1, 1);
     return launch_tile16(ctx, a, b, out, nullptr, 0, 1);

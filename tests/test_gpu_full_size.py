@@ -199,9 +199,10 @@ def test_matmul_prefetch_ring_every_remainder(gpu, tile, layout):
 
 @pytest.mark.parametrize("case", [
     (8192, 768, 768, "NT"), (8192, 768, 768, "NN"), (8192, 3072, 768, "NN"),      # activations x weights: 128 x 128 / 128 x 64 tiles
-    (768, 8192, 768, "TN"), (768, 8192, 768, "TT"),                                 # a weight gradient (x^T . dy, both given row-major) and the same with dy transposed: 64 x 64 tiles, K split 8 ways
-    (768, 8192, 3072, "TT"), (3072, 8192, 768, "TN"),                               # 128 x 128 tiles, K split 4 ways
+    (768, 8192, 768, "TN"), (768, 8192, 768, "TT"),                                 # a weight gradient (x^T . dy, both given row-major) and the same with dy transposed: 128 x 128 tiles, K split 6 ways
+    (768, 8192, 3072, "TT"), (3072, 8192, 768, "TN"), (768, 8192, 2304, "TT"),      # K split 3 and 2 ways
     (768, 8192, 8192, "TT"),                                                        # the output projection's gradient: K split 2 ways
+    (64, 8192, 768, "TN"), (512, 4096, 96, "NN"),                                   # a long K under a result less than a 128 x 128 tile wide: 64 x 64 tiles, K split
 ], ids=lambda c: f"{c[0]}x{c[1]}x{c[2]}{c[3]}")
 def test_matmul_transformer_shapes_bf16(gpu, case):
     """The mid-size products of a d = 768 transformer step at 8192 tokens, at their real shapes: every tile
