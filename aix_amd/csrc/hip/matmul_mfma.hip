@@ -1249,8 +1249,11 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
     }
     if (t64 < 2 * cus) {
         // outputs that 64 x 64 tiles cannot spread over the chip twice: with a long K, 64 x 64 tiles and K split over
-        // workgroups; otherwise 32 x 32 tiles with K split over the waves (1024^3 NN: 11.8 us against 12.7)
+        // workgroups; from half a tile per compute unit on, 64 x 64 tiles as they are (their interior tiles prefetch three K
+        // steps ahead: 1024^3 NN 12.0 -> 8.7 us, [1024,1024] x K 2048 20.3 -> 13.3, 1280^3 TN 37.5 -> 14.2); below that, 32 x 32
+        // tiles with K split over the waves (512^3: 4.3 us against 5.9)
         if (K >= 4096) return launch_tile16(ctx, a, b, out, nullptr, 0, splits_for(t64, (K + 63) / 64 * 2, 4));
+        if (2 * t64 > cus) return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
         return launch_small16(ctx, a, b, out, nullptr);
     }
     if (t128 >= cus + cus / 2) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
