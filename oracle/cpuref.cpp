@@ -23,6 +23,16 @@
 //                                       routine), bounded against float64
 //   * sum/reduceTo/matmul            -- literals, linearity/identity invariants and
 //                                       float64 brute force
+//   * the accuracy oracles sum_wide,
+//     reduce_to_wide, matmul_wide    -- math.fsum / float64 numpy over the logical
+//                                       contents of every view kind and every
+//                                       destination shape; integers stored as floats
+//                                       must come out exact and equal to the
+//                                       reference's own sum / reduceTo
+//                                       (tests/test_oracle_wide.py)
+//   * ulp_hist_f32 (the 2-ulp rule)  -- hand-built pairs: +-0, neighbours across 0
+//                                       and across powers of two, NaN against NaN
+//                                       and against numbers (same file)
 // No function of this file is "parity unpinned".
 
 #include "cpuref.h"
