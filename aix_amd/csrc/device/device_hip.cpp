@@ -736,7 +736,16 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
     aixhip_tensor pa, pb, pr; stagedPod(a, &pa, "matmul"); stagedPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
     // operands with leading dims in front of the matrix dims: a stack of products (beyond the reference, whose
     // matmul is 2-D only, aixCore.hpp:943-976)
-    check(a.shape.size() > 2 ? aixk_matmul_batched(m_ctx, &pa, &pb, &pr) : aixk_matmul(m_ctx, &pa, &pb, &pr));
+    auto run = [&] { return a.shape.size() > 2 ? aixk_matmul_batched(m_ctx, &pa, &pb, &pr) : aixk_matmul(m_ctx, &pa, &pb, &pr); };
+    int status = run();
+    if (status == AIXK_ENOMEM) {
+        // the kernel layer's own workspaces (gathered operands, K-split partials) are outside the pool: give the
+        // cached blocks back to the driver and try once more, as allocateBlock() does for the pool's own requests
+        synchronize();
+        emptyCache();
+        status = run();
+    }
+    check(status);
 }
 
 void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)

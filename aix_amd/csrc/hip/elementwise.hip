@@ -41,8 +41,10 @@ static_assert(AIXK_SQRT == M_SQRT && AIXK_SIN == M_SIN && AIXK_COS == M_COS && A
 // NIN = 1 or 2 inputs.  AS / BS: that input is a single broadcast element.  One 16-byte vector per
 // operand per lane and one workgroup per 256 vectors: many small groups in flight overlap their
 // load and compute phases better than a long per-lane loop (measured on the fused chain).
+// `out` may be one of the inputs (in-place operators, aixCore.hpp:1447, 1451), so in these three kernels it
+// and the inputs carry no restrict qualifier: every lane reads its elements before it writes the same addresses.
 template <class F, class T, int NIN, bool AS, bool BS>
-__global__ __launch_bounds__(kBlock) void ew_flat(const T* __restrict__ a, const T* __restrict__ b, T* __restrict__ out, u64 n)
+__global__ __launch_bounds__(kBlock) void ew_flat(const T* a, const T* b, T* out, u64 n)
 {
     typedef typename vec16<T>::type V;
     constexpr int VEC = vec16<T>::n;
@@ -78,8 +80,8 @@ __global__ __launch_bounds__(kBlock) void ew_flat(const T* __restrict__ a, const
 // ---- rows ------------------------------------------------------------------------------------
 // Space dims: [outer..., inner]; inner strides are 1 or 0 for inputs.  `chunks` = inner / VEC.
 template <class F, class T, int NIN, class IDX>
-__global__ __launch_bounds__(kBlock) void ew_rows(const T* __restrict__ a, const T* __restrict__ b,
-                                                  T* __restrict__ out, Space<2> sp, u64 total_chunks, IDX chunks)
+__global__ __launch_bounds__(kBlock) void ew_rows(const T* a, const T* b,
+                                                  T* out, Space<2> sp, u64 total_chunks, IDX chunks)
 {
     typedef typename vec16<T>::type V;
     constexpr int VEC = vec16<T>::n;
@@ -115,8 +117,8 @@ __global__ __launch_bounds__(kBlock) void ew_rows(const T* __restrict__ a, const
 
 // ---- gather ----------------------------------------------------------------------------------
 template <class F, class T, int NIN, class IDX>
-__global__ __launch_bounds__(kBlock) void ew_gather(const T* __restrict__ a, const T* __restrict__ b,
-                                                    T* __restrict__ out, Space<2> sp, u64 n)
+__global__ __launch_bounds__(kBlock) void ew_gather(const T* a, const T* b,
+                                                    T* out, Space<2> sp, u64 n)
 {
     for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
         IDX rest = (IDX)i;

@@ -225,13 +225,18 @@ __global__ __launch_bounds__(kBlock) void tri_vec_k(const W* __restrict__ src, W
 }
 
 // ---- indexSelect -------------------------------------------------------------------------------
+// The reference checks the range of the indices only by a host-side assert after a synchronize
+// (aixCore.hpp:1242, 1640-1650).  Here an index outside [0, extent) touches no memory: indexSelect
+// writes a zero for it, indexAdd skips it.
 template <class W, class IDX>
 __global__ __launch_bounds__(kBlock) void index_select_k(const W* __restrict__ src, W* __restrict__ dst, const i32* __restrict__ idx,
                                                          Space<1> ssp, Space<1> isp, u64 n, u64 inner, u64 ni, u64 span)
 {
     for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
         const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
-        const u64 which = (u64)(i64)idx[locate<IDX>(isp, (IDX)k)];
+        const i32 at = idx[locate<IDX>(isp, (IDX)k)];
+        const u64 which = (u64)(i64)at;
+        if (at < 0 || which * inner >= (span ? span : inner)) { dst[i] = (W)0; continue; }          // index outside the source: no access, a zero
         dst[i] = src[locate<IDX>(ssp, (IDX)(o * span + which * inner + e))];
     }
 }
@@ -269,7 +274,9 @@ __global__ __launch_bounds__(kBlock) void index_add_k(const T* __restrict__ src,
 {
     for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < n; i += (u64)gridDim.x * kBlock) {
         const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
-        const u64 which = (u64)(i64)idx[locate<IDX>(isp, (IDX)k)];
+        const i32 at = idx[locate<IDX>(isp, (IDX)k)];
+        const u64 which = (u64)(i64)at;
+        if (at < 0 || which * inner >= (span ? span : inner)) continue;                               // index outside the destination: nothing is written
         atomic_accumulate<T>(dst, o * span + which * inner + e, src[locate<IDX>(ssp, (IDX)i)]);
     }
 }
@@ -285,7 +292,9 @@ __global__ __launch_bounds__(kBlock) void index_add_pairs_k(const T* __restrict_
     typedef typename word<sizeof(T)>::type Wd;
     for (u64 i = ((u64)blockIdx.x * kBlock + threadIdx.x) * 2; i < n; i += (u64)gridDim.x * kBlock * 2) {
         const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
-        const u64 which = (u64)(i64)idx[locate<IDX>(isp, (IDX)k)];
+        const i32 at = idx[locate<IDX>(isp, (IDX)k)];
+        const u64 which = (u64)(i64)at;
+        if (at < 0 || which * inner >= (span ? span : inner)) continue;
         const T lo = src[locate<IDX>(ssp, (IDX)i)], hi = src[locate<IDX>(ssp, (IDX)(i + 1))];
         u32* wordp = (u32*)(dst + o * span + which * inner + e);
         u32 old = *wordp, assumed;

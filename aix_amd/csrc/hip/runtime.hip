@@ -57,13 +57,23 @@ int32_t aixk_create(int device_index, aixk_ctx** out)
     AIXK_HIP(hipSetDevice(device_index));
     aixk_ctx* ctx = new aixk_ctx();
     ctx->device = device_index;
-    AIXK_HIP(hipGetDeviceProperties(&ctx->prop, device_index));
-    ctx->cus = ctx->prop.multiProcessorCount > 0 ? ctx->prop.multiProcessorCount : 256;
-    AIXK_HIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
-    ctx->scratch_bytes = 64u << 20;
-    AIXK_HIP(hipMalloc(&ctx->scratch, ctx->scratch_bytes));
-    AIXK_HIP(hipMalloc((void**)&ctx->counter, 256));
-    AIXK_HIP(hipMemset(ctx->counter, 0, 256));
+    const int32_t rc = [ctx, device_index]() -> int32_t {
+        AIXK_HIP(hipGetDeviceProperties(&ctx->prop, device_index));
+        ctx->cus = ctx->prop.multiProcessorCount > 0 ? ctx->prop.multiProcessorCount : 256;
+        AIXK_HIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
+        ctx->scratch_bytes = 64u << 20;
+        AIXK_HIP(hipMalloc(&ctx->scratch, ctx->scratch_bytes));
+        AIXK_HIP(hipMalloc((void**)&ctx->counter, 256));
+        AIXK_HIP(hipMemset(ctx->counter, 0, 256));
+        return AIXK_OK;
+    }();
+    if (rc != AIXK_OK) {                              // nothing of a half-built context survives
+        if (ctx->counter) (void)hipFree(ctx->counter);
+        if (ctx->scratch) (void)hipFree(ctx->scratch);
+        if (ctx->stream) (void)hipStreamDestroy(ctx->stream);
+        delete ctx;
+        return rc;
+    }
     *out = ctx;
     return AIXK_OK;
 }

@@ -673,11 +673,23 @@ static inline int64_t index_at(const cpuref_tensor* idx, uint64_t k, int strided
     return ((const int32_t*)idx->data)[strided ? phys(idx, k) : k];
 }
 
+// The reference only asserts the range of the indices on the host (aixCore.hpp:1242, 1640-1650) and then reads or
+// writes out of bounds.  The oracle refuses such a call before it touches anything.
+static bool indices_in_range(const cpuref_tensor* idx, int strided, uint64_t extent)
+{
+    for (uint64_t k = 0; k < idx->size; ++k) {
+        const int64_t v = index_at(idx, k, strided);
+        if (v < 0 || (uint64_t)v >= extent) return false;
+    }
+    return true;
+}
+
 // aixDeviceCPU.cpp:498-530: iterate dst.size; dst contiguous from base.
 int cpuref_index_select(const cpuref_tensor* src, const cpuref_tensor* dst,
                         const cpuref_tensor* indices, uint64_t dim, int strided_indices)
 {
     if (indices->dtype != CPUREF_I32) return CPUREF_EINVAL;
+    if (!indices_in_range(indices, strided_indices, src->rank ? src->shape[dim] : 1)) return CPUREF_EINVAL;
     return by_dtype(src->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* ps = (const T*)src->data; T* pd = (T*)dst->data;
@@ -697,6 +709,7 @@ int cpuref_index_add(const cpuref_tensor* src, const cpuref_tensor* dst,
                      const cpuref_tensor* indices, uint64_t dim, int strided_indices)
 {
     if (indices->dtype != CPUREF_I32) return CPUREF_EINVAL;
+    if (!indices_in_range(indices, strided_indices, dst->rank ? dst->shape[dim] : 1)) return CPUREF_EINVAL;
     return by_dtype(src->dtype, [&](auto tag) {
         using T = decltype(tag);
         const T* ps = (const T*)src->data; T* pd = (T*)dst->data;
