@@ -55,6 +55,8 @@ struct aixk_ctx {
     // scratch for multi-block reductions: partial results
     void* scratch{nullptr};
     size_t scratch_bytes{0};
+    // this device's address of the static scratch array of reduce.hip (the entry point that allocates nothing)
+    void* static_scratch{nullptr};
     // 256 bytes of flags, zeroed at creation.  Word 0: set to `gemm_seq` by a split-plane f32 matmul that met an
     // infinity or a NaN in its operands (the IEEE-faithful kernel then redoes the product); launches are numbered,
     // so the word never has to be cleared.
@@ -74,6 +76,8 @@ struct aixk_module { aixk::RtcModule m; };
 struct aixk_event { hipEvent_t ev{nullptr}; };
 
 namespace aixk {
+
+int resolve_static_scratch(aixk_ctx* ctx);          // reduce.hip; called once per context by aixk_create
 
 inline int set_device(aixk_ctx* ctx)
 {

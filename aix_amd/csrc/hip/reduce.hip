@@ -24,7 +24,28 @@
 using namespace aixd;
 using namespace aixk;
 
+// Static device memory for the entry point that may not allocate (aixk_reduce_all_noalloc): the partial results of one
+// whole-tensor reduction, at most 4096 workgroups x 16 bytes.  Every GPU the library runs on holds its own copy at its
+// own address until the process ends.  The name is a host-side stand-in, never a device address: host code uses the
+// per-device pointer hipGetSymbolAddress returns (kept in the context), and the kernels take that pointer as an
+// argument like the pooled scratch.
+static __device__ __align__(256) unsigned char scratch[65536];
+
+namespace aixk {
+int resolve_static_scratch(aixk_ctx* ctx)
+{
+    void* ptr = nullptr;
+    AIXK_HIP(hipSetDevice(ctx->device));
+    AIXK_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+    ctx->static_scratch = ptr;
+    return AIXK_OK;
+}
+} // namespace aixk
+
 namespace {
+
+constexpr size_t kStaticScratchBytes = 65536;
+constexpr uint64_t kStaticMaxElements = 1ull << 31;
 
 constexpr int kWave = 64;
 constexpr int kWaves = kBlock / kWave;
@@ -573,7 +594,7 @@ bool make_plan(const aixhip_tensor* src, const uint64_t* weight, RedPlan* p)
 }
 
 template <class Op, class T>
-int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin);
+int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin, void* fixed = nullptr);
 
 // Does argmax_onehot_rows_k take this plan?  One reduced dim of fewer than 8 rows, the innermost kept dim dense on both
 // sides, everything aligned for VEC-wide accesses.
@@ -708,8 +729,10 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
     return AIXK_OK;
 }
 
+// `fixed` = the per-device address of the static scratch array when the caller may not allocate (then the launch must be
+// the one the pooled scratch would get, or the call is refused), else null.
 template <class Op, class T>
-int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin)
+int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const Finish& fin, void* fixed)
 {
     typedef typename Op::Acc Acc;
     const uint64_t n = a->size;
@@ -721,7 +744,9 @@ int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const 
     constexpr int VEC = vec16<T>::n;
     unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 16, ctx->scratch_bytes / sizeof(Acc));
     const unsigned grid = flat ? grid_for(n / VEC + 1, kBlock * 4, max_blocks) : grid_for(n, kBlock * 4, max_blocks);
-    Acc* partials = (Acc*)ctx->scratch;
+    if (fixed && (size_t)grid * sizeof(Acc) > kStaticScratchBytes)
+        return fail(AIXK_EINVAL, "reduce (no-allocation entry point): %u partial results of %zu bytes exceed the %zu-byte static scratch", grid, sizeof(Acc), kStaticScratchBytes);
+    Acc* partials = (Acc*)(fixed ? fixed : ctx->scratch);
     if (flat) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
     else if (small) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
     else hipLaunchKernelGGL((reduce_all_k<Op, T, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
@@ -738,9 +763,8 @@ int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const 
 
 extern "C" {
 
-int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out)
+static int32_t reduce_all_impl(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out, void* fixed)
 {
-    AIXK_TRY(set_device(ctx));
     AIXK_REQUIRE(valid_tensor(a) && valid_tensor(out), "reduce: bad operand descriptor");
     AIXK_REQUIRE(out->data != nullptr, "reduce: null result");
     if (a->size == 0 && kind == AIXK_SUM) return aixk_zero(ctx, out->data, aixk_dtype_size(out->dtype));
@@ -750,8 +774,8 @@ int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const a
         AIXK_REQUIRE(a->dtype == out->dtype, "reduce: operand must have the result's element type");
         return by_dtype(out->dtype, [&](auto tag) {
             typedef decltype(tag) T;
-            if (kind == AIXK_SUM) return run_all<SumOp<T>, T>(ctx, a, (T*)out->data, fin);
-            return run_all<MaxOp<T>, T>(ctx, a, (T*)out->data, fin);
+            if (kind == AIXK_SUM) return run_all<SumOp<T>, T>(ctx, a, (T*)out->data, fin, fixed);
+            return run_all<MaxOp<T>, T>(ctx, a, (T*)out->data, fin, fixed);
         });
     }
     AIXK_REQUIRE(kind == AIXK_ARGMAX || kind == AIXK_ARGMAX_ONEHOT, "reduce: unknown kind %d", kind);
@@ -764,8 +788,28 @@ int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const a
     }
     return by_dtype(a->dtype, [&](auto tag) {
         typedef decltype(tag) T;
-        return run_all<ArgOp<T>, T>(ctx, a, (int32_t*)out->data, fin);
+        return run_all<ArgOp<T>, T>(ctx, a, (int32_t*)out->data, fin, fixed);
     });
+}
+
+int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out)
+{
+    AIXK_TRY(set_device(ctx));
+    return reduce_all_impl(ctx, kind, a, out, nullptr);
+}
+
+// The same reduction for callers that may not allocate (stream capture, serving loops, harnesses that forbid
+// hipMalloc): the partial results of the workgroups live in the static device array `scratch` of this file instead
+// of the context's pooled scratch.  No hipMalloc / hipFree / allocating library call is made on this path.  The
+// array is shared by every call on the GPU and keeps the last call's contents; each launch overwrites the partials
+// it reads, so nothing has to be cleared, but two calls that overlap on one GPU (two contexts, two streams) race.
+int32_t aixk_reduce_all_noalloc(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(ctx->static_scratch != nullptr, "reduce (no-allocation entry point): the static scratch of device %d was not resolved", ctx->device);
+    AIXK_REQUIRE(a != nullptr && a->size <= kStaticMaxElements,
+                 "reduce (no-allocation entry point): at most %llu elements per call", (unsigned long long)kStaticMaxElements);
+    return reduce_all_impl(ctx, kind, a, out, ctx->static_scratch);
 }
 
 static int32_t reduce_to_impl(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, const uint64_t* init);

@@ -65,7 +65,7 @@ int32_t aixk_create(int device_index, aixk_ctx** out)
         AIXK_HIP(hipMalloc(&ctx->scratch, ctx->scratch_bytes));
         AIXK_HIP(hipMalloc((void**)&ctx->counter, 256));
         AIXK_HIP(hipMemset(ctx->counter, 0, 256));
-        return AIXK_OK;
+        return aixk::resolve_static_scratch(ctx);
     }();
     if (rc != AIXK_OK) {                              // nothing of a half-built context survives
         if (ctx->counter) (void)hipFree(ctx->counter);

@@ -57,6 +57,7 @@ _SIGNATURES = {
     "aixk_index_select": [_P, _T, _T, _T, C.c_uint64],
     "aixk_index_add": [_P, _T, _T, _T, C.c_uint64],
     "aixk_reduce_all": [_P, C.c_int, _T, _T],
+    "aixk_reduce_all_noalloc": [_P, C.c_int, _T, _T],
     "aixk_reduce_to": [_P, C.c_int, _T, _T],
     "aixk_reduce_to_init": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
