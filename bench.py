@@ -33,6 +33,10 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}
+# large f32 products run as six bf16 MFMAs per product term (three bf16 planes per operand): that pipe's ceiling for them
+X3_PEAK_TFLOPS = MFMA_PEAK_TFLOPS["bf16"] / 6
+# configs[1]: HBM bytes per step (all launches of the item) from the counter passes, item index -> bytes; None = not measured
+C1_TRAFFIC = {}
 
 
 class BenchResult(C.Structure):
@@ -102,6 +106,57 @@ def cpu_chain(a, b, c):
     y = binary(O.SUB, t7, binary(O.MUL, scalar(0.5), c, xs=zeros))
     dt = time.perf_counter() - t0
     return y, t7, dt, kind
+
+
+def cpu_c1_items(x, v):
+    """The six configs[1] items on the CPU device path at full size, one thread, as the front-end issues them
+    (fill + reduceTo, fillMin + maxTo, argmaxTo, sum, add with a stride-0 view, contiguous of a transposed view).
+    Returns {item index: (seconds, result array)} and the kind of CPU path."""
+    from oracle import cpuref as O
+    ref = O.ref_lib()
+    lib, kind = (ref, "reference") if ref is not None else (O.lib(), "port")
+    n = x.shape[0]
+    X = O.desc_of(x, O.F32, [n, n])
+    out = {}
+
+    def timed(fn):
+        t0 = time.perf_counter()
+        fn()
+        return time.perf_counter() - t0
+
+    def sum1():
+        assert lib.fill(np.zeros(1, np.float32).ctypes.data, O.F32, C.byref(O.desc_of(r, O.F32, [n, 1]))) == 0
+        assert lib.reduce_to(C.byref(X), C.byref(O.desc_of(r, O.F32, [n, 1]))) == 0
+
+    def max1():
+        assert lib.fill_min(C.byref(O.desc_of(r, O.F32, [n, 1]))) == 0
+        assert lib.max_to(C.byref(X), C.byref(O.desc_of(r, O.F32, [n, 1]))) == 0
+
+    r = np.empty(n, np.float32)
+    out[0] = (timed(sum1), r.copy())
+    out[1] = (timed(max1), r.copy())
+    ri = np.empty(n, np.int32)
+    out[2] = (timed(lambda: lib.argmax_to(C.byref(X), C.byref(O.desc_of(ri, O.I32, [n])), 0)), ri)
+    r0 = np.empty(1, np.float32)
+    out[3] = (timed(lambda: lib.sum(C.byref(X), C.byref(O.desc_of(r0, O.F32, [])))), r0)
+    big = np.empty((n, n), np.float32)
+    out[4] = (timed(lambda: lib.binary(O.ADD, C.byref(X), C.byref(O.desc_of(v, O.F32, [n, n], [0, 1])), C.byref(O.desc_of(big, O.F32, [n, n])))), big.copy())
+    out[5] = (timed(lambda: lib.contiguous(C.byref(O.desc_of(x, O.F32, [n, n], [1, n])), C.byref(O.desc_of(big, O.F32, [n, n])))), big)
+    return out, kind
+
+
+def cpu_matmul_seconds(dt_name, m):
+    """One m^3 product (NN) on the CPU device path, one thread; operands drawn like the GPU's."""
+    from oracle import cpuref as O
+    ref = O.ref_lib()
+    lib, kind = (ref, "reference") if ref is not None else (O.lib(), "port")
+    code = {"f32": O.F32, "f16": O.F16, "bf16": O.BF16}[dt_name]
+    a = O.to_storage(np.random.default_rng(3).uniform(-1, 1, m * m) / np.sqrt(m), code)
+    b = O.to_storage(np.random.default_rng(4).uniform(-1, 1, m * m) / np.sqrt(m), code)
+    c = np.empty(m * m, O.NP_STORAGE[code])
+    t0 = time.perf_counter()
+    assert lib.matmul(C.byref(O.desc_of(a, code, [m, m])), C.byref(O.desc_of(b, code, [m, m])), C.byref(O.desc_of(c, code, [m, m]))) == 0
+    return time.perf_counter() - t0, kind
 
 
 def calibrate_copy(steps):
@@ -213,12 +268,31 @@ def main():
                  (3, "sum()", N * 4 + 4), (4, "x + v (row broadcast)", 2 * N * 4 + n * 4),
                  (5, "x.transpose(0,1).contiguous()", 2 * N * 4)]
         steps = max(10, args.steps // 4)
+        # HBM bytes per launch of each item's dominant kernel from FETCH_SIZE + WRITE_SIZE counter passes scaled by a copy
+        # kernel of known size (profiles/reductions_c1_f32_8192x8192.md); measured constants, not live
+        traffic = C1_TRAFFIC
+        cpu, cpu_kind = cpu_c1_items(x, v) if not args.no_cpu else ({}, None)
         for which, name, nbytes in items:
             r = BenchResult()
-            run(lib, "aixbench_reduce_item", dev.handle, which, n, n, x.ctypes.data, v.ctypes.data, steps, 3, C.byref(r), None)
-            extras.append({"workload": f"configs[1] f32 [8192,8192]: {name}", "ms_per_step": round(r.wall_s * 1e3 / steps, 5),
-                           "value": round(nbytes * steps / r.wall_s / 1e9, 1), "unit": "GB/s",
-                           "roofline": roofline("hbm", nbytes / (r.gpu_ms / steps * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s")})
+            got = np.empty(n if which < 3 else (1 if which == 3 else N), np.int32 if which == 2 else np.float32)
+            run(lib, "aixbench_reduce_item", dev.handle, which, n, n, x.ctypes.data, v.ctypes.data, steps, 3, C.byref(r), got.ctypes.data)
+            line = {"workload": f"configs[1] f32 [8192,8192]: {name}", "ms_per_step": round(r.wall_s * 1e3 / steps, 5),
+                    "value": round(nbytes * steps / r.wall_s / 1e9, 1), "unit": "GB/s",
+                    "roofline": roofline("hbm", nbytes / (r.gpu_ms / steps * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", traffic=traffic.get(which))}
+            if which in cpu:
+                secs, want = cpu[which]
+                line["cpu_baseline"] = {"value": round(nbytes / secs / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": cpu_kind,
+                                        "sample": f"the full [8192,8192] item once on the CPU device ({secs:.2f} s), one thread of {os.cpu_count()}"}
+                if which in (0, 3):                         # float sums: the CPU adds sequentially in f32, the GPU in a tree
+                    exact = x.astype(np.float64).sum(axis=1) if which == 0 else np.array([x.astype(np.float64).sum()])
+                    mag = np.abs(x).astype(np.float64).sum(axis=1) if which == 0 else np.array([np.abs(x).astype(np.float64).sum()])
+                    err = float((np.abs(got.astype(np.float64) - exact) / mag).max())
+                    cpu_err = float((np.abs(want.reshape(-1).astype(np.float64) - exact) / mag).max())
+                    line["parity"] = {"checked_against": "float64 sums of the same data", "ok": bool(err <= 1e-5), "max_err_over_sum_abs": err,
+                                      "cpu_device_err_over_sum_abs": cpu_err, "rule": "|err| <= 1e-5 * sum|x|"}
+                else:
+                    line["parity"] = {"checked_against": "cpu_baseline result", "ok": bool(np.array_equal(got.reshape(-1), want.reshape(-1))), "rule": "bit-exact"}
+            extras.append(line)
         del x
     if not args.no_extras and "c2" in chosen:
         from oracle.cpuref import f32_to_bf16_bits
@@ -238,9 +312,16 @@ def main():
 
         codes = {"f32": 1, "f16": 2, "bf16": 3}
         layouts = {"NN": 0, "NT": 1, "TN": 2}
+        # the CPU device beside it: f32 at 1024^3 and the 16-bit types at 512^3 measured, other sizes scaled by M*N*K and labelled
+        cpu_mm = {}
+        if not args.no_cpu:
+            for dt_name, m_cpu in (("f32", 1024), ("bf16", 512), ("f16", 512)):
+                secs, kind = cpu_matmul_seconds(dt_name, m_cpu)
+                cpu_mm[dt_name] = (secs, m_cpu, kind)
         sweep = [("f32", 4096, "NN", 1, 20), ("bf16", 4096, "NN", 1, 20), ("f16", 4096, "NN", 1, 20),
                  ("bf16", 4096, "NT", 1, 20), ("bf16", 4096, "TN", 1, 20), ("f32", 4096, "NT", 1, 20),
-                 ("bf16", 1024, "NN", 1, 50), ("bf16", 8192, "NN", 1, 5), ("f32", 1024, "NN", 1, 50), ("f32", 8192, "NN", 1, 3),
+                 ("bf16", 1024, "NN", 1, 50), ("f16", 1024, "NN", 1, 50), ("f32", 1024, "NN", 1, 50),
+                 ("bf16", 8192, "NN", 1, 5), ("f16", 8192, "NN", 1, 5), ("f32", 8192, "NN", 1, 3),
                  ("bf16", 512, "NN", 64, 20), ("bf16", 512, "NN", -64, 20)]
         for dt_name, m, lay, batch, steps_mm in sweep:
             stacked, batch = batch < 0, abs(batch)                 # negative: one matmul on the [batch, m, m] stacks
@@ -251,16 +332,23 @@ def main():
             flops = 2.0 * m * m * m * batch
             what = f"{m}^3" if batch == 1 else f"{batch} x [{m},{m}]x[{m},{m}] " + (
                 "(one matmul call on the [64, 512, 512] stacks: an extension of the interface)" if stacked else "(one matmul call per select(0,i) view)")
+            x3 = dt_name == "f32" and ((m + 127) // 128) ** 2 >= 448          # the route the library takes (matmul_mfma.hip)
+            peak = X3_PEAK_TFLOPS if x3 else MFMA_PEAK_TFLOPS[dt_name]
             line = {"workload": f"configs[2] matmul {dt_name} {what} {lay} (f32 accumulation)",
                     "ms_per_step": round(r.wall_s * 1e3 / steps_mm, 5),
                     "value": round(flops * steps_mm / r.wall_s / 1e12, 2), "unit": "TFLOP/s",
-                    "roofline": roofline("mfma", flops / (r.gpu_ms / steps_mm * 1e-3) / 1e12, MFMA_PEAK_TFLOPS[dt_name], "TFLOP/s")}
-            if dt_name == "f32" and m >= 2048:
-                # large f32 products run on the bf16 matrix pipe: each operand as three bf16 planes, six bf16 MFMAs per product
-                # term, f32 accumulation -- so the published f32 MFMA peak is not a ceiling for them
-                line["roofline"]["note"] = ("f32 operands split into three bf16 planes, 6 bf16 MFMAs per f32 MFMA's worth of work: the ceiling of "
-                                            f"this algorithm is the bf16 peak / 6 = {MFMA_PEAK_TFLOPS['bf16'] / 6:.1f} TFLOP/s "
-                                            f"(frac {line['roofline']['achieved'] / (MFMA_PEAK_TFLOPS['bf16'] / 6):.3f}); peak and frac above are the f32 MFMA's")
+                    "roofline": roofline("mfma", flops / (r.gpu_ms / steps_mm * 1e-3) / 1e12, round(peak, 1), "TFLOP/s")}
+            if x3:
+                line["roofline"]["note"] = ("f32 operands split into three bf16 planes, six bf16 MFMAs per product term, f32 accumulation: the pipe this "
+                                            f"kernel runs on peaks at 2500 / 6 = {X3_PEAK_TFLOPS:.1f} TFLOP/s for it (peak and frac above); against the "
+                                            f"f32 MFMA's published {MFMA_PEAK_TFLOPS['f32']} TFLOP/s the achieved rate is "
+                                            f"{line['roofline']['achieved'] / MFMA_PEAK_TFLOPS['f32']:.2f}x")
+            if cpu_mm:
+                secs, m_cpu, kind = cpu_mm[dt_name]
+                scaled = secs * (m / m_cpu) ** 3 * batch
+                line["cpu_baseline"] = {"value": round(flops / scaled / 1e12, 9), "unit": "TFLOP/s", "cores": 1, "kind": kind,
+                                        "sample": f"{dt_name} {m_cpu}^3 NN once on the CPU device ({secs:.1f} s, one thread)" + (
+                                            "" if (m == m_cpu and batch == 1) else f"; EXTRAPOLATED to this line's size in proportion to M*N*K ({scaled:.0f} s if run)")}
             extras.append(line)
         # the same 4096^3 bf16 product on all-zero operands: same kernel, same instruction stream, no bits toggling in the
         # matrix pipe -- the gap to the line above is the clock the part gives up under the power of real operands
@@ -284,11 +372,13 @@ def main():
         flops = 2.0 * shape[0] * (shape[1] * shape[2] + shape[2] * shape[2] + shape[2] * shape[3])      # forward products
         # backward: 4 traversals (softmax + cross-entropy reach the logits along 4 paths), each dW3, dH2, dW2, dH1, dW1
         flops_step = flops + 4 * (2 * flops - 2.0 * shape[0] * shape[1] * shape[2])
+        useful = flops + (2 * flops - 2.0 * shape[0] * shape[1] * shape[2])       # what one traversal of the backward pass needs
         mlp = {"workload": "configs[3] MLP 784-2048-2048-10, batch 4096, f32, ReLU, softmax + cross-entropy, Adam lr 1e-3, "
                            "100 steps, loss read back every step",
                "ms_per_step": round(float(steady.mean()) * 1e3, 4), "value": round(1.0 / float(steady.mean()), 2), "unit": "steps/s",
-               "first_step_ms": round(float(secs[0]) * 1e3, 2), "flop_per_step": flops_step,
-               "roofline": roofline("mfma", flops_step / float(steady.mean()) / 1e12, MFMA_PEAK_TFLOPS["f32"], "TFLOP/s"),
+               "first_step_ms": round(float(secs[0]) * 1e3, 2), "flop_per_step_issued": flops_step, "flop_per_step_useful": useful,
+               "useful_TFLOPs": round(useful / float(steady.mean()) / 1e12, 2),
+               "roofline": roofline("mfma", flops_step / float(steady.mean()) / 1e12, round(X3_PEAK_TFLOPS, 1), "TFLOP/s"),
                "loss": [round(float(l), 6) for l in losses[[0, 1, 2, 9, 49, 99]]]}
         if not args.no_cpu:
             threads = min(16, os.cpu_count() or 1)
@@ -301,6 +391,9 @@ def main():
                                              f"matmul rows on {threads} threads, everything else on 1)"}
             mlp["parity"] = {"checked_against": "cpu_baseline losses", "steps": cpu_steps, "max_rel_dev": float(rel.max()),
                              "ok": bool(rel.max() <= 1e-4), "rule": "|loss_gpu - loss_cpu| <= 1e-4 |loss_cpu| on the first steps"}
+        mlp["roofline"]["note"] = ("issued work: the reference's backward recursion differentiates once per path, so the five backward products run "
+                                   f"4 times ({flops_step / 1e9:.0f} GFLOP per step, what AIX issues on any device); one traversal would need "
+                                   f"{useful / 1e9:.0f} GFLOP (useful_TFLOPs). The products run on the split-plane bf16 route, hence its peak.")
         extras.append(mlp)
     if not args.no_extras and chosen & {"c4", "c4loop", "c4stack"}:
         # configs[4]: decoder-only transformer forward + backward composed from device operators

@@ -1,0 +1,115 @@
+// stub_kernels.cpp -- a host-only stand-in for libaixhip_kernels.so (include/aixhip_kernels.h) for the sanitizer
+// builds of the device's host code (the counterpart of the reference's ASan / TSan configurations,
+// CMakeLists.txt:25, 47-53).  Memory comes from the host heap under a settable budget, events complete after a
+// settable number of queries, every compute entry point only counts its call: what runs under the sanitizers is
+// DeviceHIP's own bookkeeping -- block table, buckets, limbo, cooling lists, the planner and the source generator.
+// TEST INFRASTRUCTURE ONLY; never linked into the product.
+#include "aixhip_kernels.h"
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+
+struct aixk_ctx { size_t budget{SIZE_MAX}, held{0}; int event_delay{0}; uint64_t launches{0}, allocs{0}, frees{0}, syncs{0}, hits{0}, misses{0}; };
+struct aixk_module { int dummy; };
+struct aixk_event { int countdown{0}; bool recorded{false}; };
+
+static thread_local char g_error[256] = "";
+static aixk_module g_module;
+static std::atomic<long long> g_held_everywhere{0};        // bytes handed out and not yet returned, over all contexts
+static std::atomic<int> g_fail_matmuls{0};                 // the next n matmul calls report AIXK_ENOMEM
+
+extern "C" {
+
+// test controls (not part of the product ABI)
+void stub_set_budget(aixk_ctx* c, size_t bytes) { c->budget = bytes; }
+void stub_set_event_delay(aixk_ctx* c, int queries) { c->event_delay = queries; }
+size_t stub_held(aixk_ctx* c) { return c->held; }
+uint64_t stub_launches(aixk_ctx* c) { return c->launches; }
+uint64_t stub_allocs(aixk_ctx* c) { return c->allocs; }
+uint64_t stub_frees(aixk_ctx* c) { return c->frees; }
+uint64_t stub_syncs(aixk_ctx* c) { return c->syncs; }
+long long stub_held_everywhere(void) { return g_held_everywhere.load(); }
+void stub_fail_next_matmuls(int n) { g_fail_matmuls = n; }
+
+const char* aixk_last_error(void) { return g_error; }
+size_t aixk_dtype_size(int dtype) { static const size_t sz[9] = {8, 4, 2, 2, 8, 4, 2, 1, 1}; return dtype >= 0 && dtype < 9 ? sz[dtype] : 0; }
+int32_t aixk_create(int, aixk_ctx** out) { *out = new aixk_ctx(); return AIXK_OK; }
+int32_t aixk_destroy(aixk_ctx* c) { delete c; return AIXK_OK; }
+int32_t aixk_info(aixk_ctx*, aixk_device_info* out)
+{
+    std::memset(out, 0, sizeof(*out));
+    std::snprintf(out->name, sizeof(out->name), "stub");
+    out->compute_units = 256; out->large_bar = 1; out->wavefront = 64; out->total_mem = 1ull << 30;
+    return AIXK_OK;
+}
+int32_t aixk_alloc(aixk_ctx* c, size_t bytes, int, void** out)
+{
+    if (c->held + bytes > c->budget) { std::snprintf(g_error, sizeof(g_error), "stub: out of memory (%zu held, %zu asked)", c->held, bytes); return AIXK_ENOMEM; }
+    void* p = nullptr;
+    if (posix_memalign(&p, 256, bytes + sizeof(size_t) * 32) != 0) return AIXK_ENOMEM;
+    *(size_t*)p = bytes;                                   // size header in front of the 256-byte aligned block
+    c->held += bytes; ++c->allocs; g_held_everywhere += (long long)bytes;
+    *out = (char*)p + 256;
+    return AIXK_OK;
+}
+int32_t aixk_free(aixk_ctx* c, void* ptr, int)
+{
+    if (!ptr) return AIXK_OK;
+    void* base = (char*)ptr - 256;
+    c->held -= *(size_t*)base; ++c->frees; g_held_everywhere -= (long long)*(size_t*)base;
+    std::free(base);
+    return AIXK_OK;
+}
+int32_t aixk_copy_in(aixk_ctx* c, void* d, const void* s, size_t n) { ++c->launches; std::memcpy(d, s, n); return AIXK_OK; }
+int32_t aixk_copy_out(aixk_ctx* c, void* d, const void* s, size_t n) { ++c->launches; std::memcpy(d, s, n); return AIXK_OK; }
+int32_t aixk_copy_dev(aixk_ctx* c, void* d, const void* s, size_t n) { ++c->launches; std::memmove(d, s, n); return AIXK_OK; }
+int32_t aixk_zero(aixk_ctx* c, void* d, size_t n) { ++c->launches; std::memset(d, 0, n); return AIXK_OK; }
+int32_t aixk_sync(aixk_ctx* c) { ++c->syncs; return AIXK_OK; }
+
+#define STUB_OP(name, ...) int32_t name(aixk_ctx* c, __VA_ARGS__) { ++c->launches; return AIXK_OK; }
+STUB_OP(aixk_binary, int, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_unary, int, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_fill, const void*, int, const aixhip_tensor*)
+STUB_OP(aixk_fill_min, const aixhip_tensor*)
+STUB_OP(aixk_cast, const void*, int, void*, int, uint64_t)
+STUB_OP(aixk_contiguous, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_transpose, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t)
+STUB_OP(aixk_slice_set, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t, uint64_t, uint64_t)
+STUB_OP(aixk_slice_set_init, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t, uint64_t, uint64_t, uint64_t)
+STUB_OP(aixk_tri, int, const aixhip_tensor*, const aixhip_tensor*, int64_t)
+STUB_OP(aixk_index_select, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
+STUB_OP(aixk_index_add, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
+STUB_OP(aixk_reduce_all, int, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_reduce_all_noalloc, int, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_reduce_to, int, const aixhip_tensor*, const aixhip_tensor*)
+STUB_OP(aixk_reduce_to_init, int, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
+STUB_OP(aixk_argmax_to, int, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
+int32_t aixk_matmul(aixk_ctx* c, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
+{
+    if (g_fail_matmuls > 0) { --g_fail_matmuls; std::snprintf(g_error, sizeof(g_error), "stub: matmul workspace"); return AIXK_ENOMEM; }
+    ++c->launches;
+    return AIXK_OK;
+}
+STUB_OP(aixk_matmul_batched, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
+
+int32_t aixk_rtc_get(aixk_ctx* c, const char*, const char*, const char*, aixk_module** out, int32_t* was_cached)
+{
+    ++c->misses;
+    *out = &g_module;
+    if (was_cached) *was_cached = 0;
+    return AIXK_OK;
+}
+STUB_OP(aixk_rtc_launch, aixk_module*, uint32_t, uint32_t, const void*, size_t)
+const char* aixk_rtc_prelude(void) { return ""; }
+int32_t aixk_rtc_stats(aixk_ctx* c, uint64_t* hits, uint64_t* misses) { *hits = c->hits; *misses = c->misses; return AIXK_OK; }
+
+int32_t aixk_event_create(aixk_ctx*, aixk_event** out) { *out = new aixk_event(); return AIXK_OK; }
+int32_t aixk_event_record(aixk_ctx* c, aixk_event* e) { e->recorded = true; e->countdown = c->event_delay; return AIXK_OK; }
+int32_t aixk_event_query(aixk_ctx*, aixk_event* e, int32_t* done) { *done = e->recorded && e->countdown-- <= 0; return AIXK_OK; }
+int32_t aixk_event_elapsed_ms(aixk_ctx*, aixk_event*, aixk_event*, float* ms) { *ms = 0.f; return AIXK_OK; }
+int32_t aixk_event_destroy(aixk_ctx*, aixk_event* e) { delete e; return AIXK_OK; }
+
+} // extern "C"

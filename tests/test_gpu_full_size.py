@@ -2,8 +2,9 @@
 
 The element-by-element oracle comparisons of test_gpu_kernels.py run at sizes the CPU oracle finishes in
 seconds.  Here the kernels run at the sizes the benchmark quotes -- [8192, 8192] f32 for the reductions,
-the broadcast add and the transpose copy, 4096^3 (and one 8192^3) for the matmuls -- and are checked
-with what the mathematics fixes at any size:
+the broadcast add and the transpose copy, 1024^3, 4096^3 and 8192^3 in f32 / bf16 / f16 and the batch of 64 512^3
+products for the matmuls -- and are checked with what the mathematics fixes at any size (1024^3 and the batch are
+small enough for the exactly accumulated oracle on every element):
 
   * exact operators (max, argmax, x + v, transpose) against numpy on the same data, bit for bit;
     transpose twice is the identity;
@@ -13,6 +14,8 @@ with what the mathematics fixes at any size:
     operand layout the kernels consume in place.
 
 Everything goes through the C ABI of libaixhip_kernels.so."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -22,6 +25,7 @@ from oracle import cpuref as O
 
 pytestmark = pytest.mark.gpu
 NAMES = O.DTYPE_NAMES
+CPU = O.lib()
 
 
 @pytest.fixture(scope="module")
@@ -233,6 +237,76 @@ def test_matmul_4096_cubed_f32(gpu, layout):
 
 def test_matmul_8192_cubed_bf16(gpu):
     _matmul_properties(gpu, O.BF16, 8192, "NN", np.random.default_rng(6200), 1e-5)
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.F16], ids=lambda d: NAMES[d])
+def test_matmul_8192_cubed_f32_f16(gpu, dtype):
+    _matmul_properties(gpu, dtype, 8192, "NN", np.random.default_rng(6210 + dtype), 1e-5)
+
+
+@pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16, O.F16], ids=lambda d: NAMES[d])
+def test_matmul_1024_cubed(gpu, dtype, layout):
+    """The smallest size of the sweep, every element: at 1024^3 the exactly accumulated oracle is affordable, so this
+    is a full comparison (|err| <= 1e-5 x sum|a||b| plus the rounding of the result type), not a checksum."""
+    n = 1024
+    rng = np.random.default_rng(6220 + dtype)
+    a_t, b_t = layout[0] == "T", layout[1] == "T"
+    a = T.HostTensor(O.to_storage(rng.uniform(-1, 1, n * n) / np.sqrt(n), dtype), dtype, [n, n], [1, n] if a_t else None)
+    b = T.HostTensor(O.to_storage(rng.uniform(-1, 1, n * n) / np.sqrt(n), dtype), dtype, [n, n], [1, n] if b_t else None)
+    _, da = gpu.put(a)
+    _, db = gpu.put(b)
+    out = T.empty(dtype, [n, n])
+    po, do = gpu.put(out)
+    G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+    got = O.to_float64(gpu.fetch(po, out.storage), dtype)
+    exact, mag = np.zeros(n * n), np.zeros(n * n)
+    assert CPU.matmul_wide(C.byref(a.desc()), C.byref(b.desc()), exact.ctypes.data, mag.ctypes.data, 16) == 0
+    eps_out = {O.F32: 2.0 ** -24, O.F16: 2.0 ** -11, O.BF16: 2.0 ** -8}[dtype]
+    bad = np.abs(got - exact) > eps_out * np.abs(exact) + 1e-5 * mag + 1e-30
+    assert not bad.any(), f"{NAMES[dtype]} 1024^3 {layout}: {int(bad.sum())} elements beyond the bound"
+    gpu.release()
+
+
+def _stack_data(rng, dtype, count, n):
+    a = T.HostTensor(O.to_storage(rng.uniform(-1, 1, count * n * n) / np.sqrt(n), dtype), dtype, [count, n, n])
+    b = T.HostTensor(O.to_storage(rng.uniform(-1, 1, count * n * n) / np.sqrt(n), dtype), dtype, [count, n, n])
+    exact, mag = np.zeros(count * n * n), np.zeros(count * n * n)
+    for i in range(count):
+        a2 = T.HostTensor(a.storage, dtype, [n, n], None, i * n * n)
+        b2 = T.HostTensor(b.storage, dtype, [n, n], None, i * n * n)
+        e, m = np.zeros(n * n), np.zeros(n * n)
+        assert CPU.matmul_wide(C.byref(a2.desc()), C.byref(b2.desc()), e.ctypes.data, m.ctypes.data, 16) == 0
+        exact[i * n * n:(i + 1) * n * n], mag[i * n * n:(i + 1) * n * n] = e, m
+    return a, b, exact, mag
+
+
+def test_matmul_batch_of_64_bf16_both_forms(gpu):
+    """[64, 512, 512] x [64, 512, 512] bf16, every element against the exactly accumulated oracle: once as the
+    interface has it (64 matmul calls on select(0, i) views, offset != 0, aixCore.hpp:943-976) and once as one call on
+    the stacks; the two forms must also agree with each other within the rounding of the result type."""
+    count, n, dtype = 64, 512, O.BF16
+    a, b, exact, mag = _stack_data(np.random.default_rng(6230), dtype, count, n)
+    pa, da = gpu.put(a)
+    pb, db = gpu.put(b)
+    out = T.empty(dtype, [count, n, n])
+    bound = 2.0 ** -8 * np.abs(exact) + 1e-5 * mag + 1e-30
+    # 64 calls on views of the stacks
+    po, _ = gpu.put(out)
+    for i in range(count):
+        va = G.kdesc(T.HostTensor(a.storage, dtype, [n, n], None, i * n * n), pa)
+        vb = G.kdesc(T.HostTensor(b.storage, dtype, [n, n], None, i * n * n), pb)
+        vo = G.kdesc(T.HostTensor(out.storage, dtype, [n, n]), po + i * n * n * 2)
+        G.run_gpu(gpu, "aixk_matmul", G.ref(va), G.ref(vb), G.ref(vo))
+    per_call = O.to_float64(gpu.fetch(po, out.storage), dtype)
+    assert np.all(np.abs(per_call - exact) <= bound), "64 calls on select(0, i) views"
+    # one call on the stacks
+    po2, do2 = gpu.put(out)
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(da), G.ref(db), G.ref(do2))
+    stacked = O.to_float64(gpu.fetch(po2, out.storage), dtype)
+    assert np.all(np.abs(stacked - exact) <= bound), "one call on the [64, 512, 512] stacks"
+    assert np.all(np.abs(stacked - per_call) <= 2.0 ** -7 * np.abs(exact) + 2e-5 * mag + 1e-30)
+    gpu.release()
 
 
 @pytest.mark.parametrize("dtype", [O.F32, O.BF16], ids=lambda d: NAMES[d])
