@@ -9,6 +9,7 @@
 #include <algorithm>
 #include <array>
 #include <cstring>
+#include <cstdlib>
 #include <deque>
 #include <iostream>
 #include <limits>
@@ -95,6 +96,11 @@ struct DeviceHIP::Extras {
     std::string key;
     std::vector<uint64_t> args;
     gen::Space space;
+    // results of at least this many bytes are written with non-temporal stores (the kernel layer's rule, same override)
+    size_t streamStoreMinBytes = [] {
+        const char* e = std::getenv("AIXHIP_STREAM_STORE_MIN_BYTES");
+        return e && *e ? (size_t)std::strtoull(e, nullptr, 10) : (size_t)AIXK_STREAM_STORE_MIN_BYTES;
+    }();
 };
 
 // ---- block table -------------------------------------------------------------------------------
@@ -672,13 +678,16 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 
     bool noAlias = true;                                     // in-place updates: an output that is also an input
     for (const auto& ob : d.outputBuffers) for (const auto& ib : d.inputBuffers) if (ob.data == ib.data) noAlias = false;
-    gen::signatureInto(ex.key, d, shape, bmask, noAlias);
+    size_t storedBytes = 0;                                  // large results leave through non-temporal stores
+    for (const auto& ob : d.outputBuffers) storedBytes += n * dataTypeSize(ob.dtype);
+    const bool streamOut = storedBytes >= ex.streamStoreMinBytes;
+    gen::signatureInto(ex.key, d, shape, bmask, noAlias, streamOut);
     aixk_module* mod = nullptr;
     auto it = ex.kernels.find(ex.key);
     if (it != ex.kernels.end()) { mod = it->second; ++ex.hits; }
     else {
         int32_t cached = 0;
-        const std::string src = gen::source(d, shape, bmask, noAlias);
+        const std::string src = gen::source(d, shape, bmask, noAlias, streamOut);
         check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
         ex.kernels.emplace(ex.key, mod);
         ++ex.misses;

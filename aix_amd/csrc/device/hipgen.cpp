@@ -123,11 +123,12 @@ void appendOperand(std::string& out, const FusedSubgraphDescriptor& d, size_t te
 
 } // namespace
 
-void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
+void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut)
 {
     s.clear();
     s += shortType(d.dtype);
     s += shape == Shape::Flat ? "|flat" : shape == Shape::Rows ? "|rows" : "|gather";
+    if (streamOut && shape != Shape::Gather) s += "|nt";
     if (shape == Shape::Flat) { s += noAlias ? 'r' : 'a'; appendNumber(s, broadcastMask, 16); }
     s += "|i"; appendNumber(s, d.inputBuffers.size());
     s += 'o';  appendNumber(s, d.outputBuffers.size());
@@ -146,14 +147,14 @@ void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape
     }
 }
 
-std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
+std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut)
 {
     std::string s;
-    signatureInto(s, d, shape, broadcastMask, noAlias);
+    signatureInto(s, d, shape, broadcastMask, noAlias, streamOut);
     return s;
 }
 
-std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias)
+std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut)
 {
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d), NT = triCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
@@ -162,7 +163,8 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
     std::ostringstream o;
     o << "#include \"aix_device.h\"\nusing namespace aixd;\n"
-      << "// " << signature(d, shape, broadcastMask, noAlias) << "\n"
+      << "// " << signature(d, shape, broadcastMask, noAlias, streamOut) << "\n"
+      << "#define AIX_NT " << (streamOut ? "true" : "false") << "\n"
       << "typedef " << typeName(d.dtype) << " T;\n"
       << "typedef " << wordName(esz) << " word_t;\n"
       << "#define VEC (vec16<T>::n)\n#define NI " << NI << "\n#define NO " << NO << "\n#define NS " << NS << "\n";
@@ -215,7 +217,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
         for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
-        for (size_t k = 0; k < NO; ++k) o << "        q" << k << "[v] = w" << k << ";\n";
+        for (size_t k = 0; k < NO; ++k) o << "        store_sel<AIX_NT>(q" << k << " + v, w" << k << ");\n";
         o << "    }\n"
           << "    const u64 done = nvec * VEC;\n"
           << "    if (blockIdx.x == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
@@ -241,11 +243,11 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         o << "        for (int d = inner - 1; d >= 0; --d) {\n            const u64 q = row / a.shape[d], r = row - q * a.shape[d];\n";
         for (size_t k = 0; k < NI; ++k) o << "            p[" << k << "] += r * a.str[" << k << "][d];\n";
         o << "            row = q;\n        }\n";
-        for (size_t k = 0; k < NI; ++k) {
-            o << "        vec<I" << k << ", VEC> r" << k << ";\n"
-              << "        if (a.str[" << k << "][inner] == 0) { const I" << k << " t = in" << k << "[p[" << k << "]];\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r" << k << ".v[e] = t; }\n"
-              << "        else r" << k << " = *(const vec<I" << k << ", VEC>*)(in" << k << " + p[" << k << "] + col);\n";
-        }
+        // all loads first and without branches (row_vec_ptr / row_vec_fix in the device header say why)
+        for (size_t k = 0; k < NI; ++k)
+            o << "        vec<I" << k << ", VEC> r" << k << " = *row_vec_ptr<I" << k << ", VEC>(in" << k << " + p[" << k << "], col, a.str[" << k << "][inner] == 0);\n";
+        for (size_t k = 0; k < NI; ++k)
+            o << "        r" << k << " = row_vec_fix<I" << k << ", VEC>(r" << k << ", in" << k << " + p[" << k << "], a.str[" << k << "][inner] == 0);\n";
         for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
         if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(c * VEC, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
         o << "#pragma unroll\n        for (int e = 0; e < VEC; ++e) {\n            T x[" << AI << "], y[" << NO << "];\n";
@@ -254,7 +256,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
         for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
         o << "        }\n";
-        for (size_t k = 0; k < NO; ++k) o << "        *(vec<O" << k << ", VEC>*)(out" << k << " + c * VEC) = w" << k << ";\n";
+        for (size_t k = 0; k < NO; ++k) o << "        store_sel<AIX_NT>((vec<O" << k << ", VEC>*)(out" << k << " + c * VEC), w" << k << ");\n";
         o << "    }\n}\n";
         return o.str();
     }

@@ -24,13 +24,14 @@ enum class Shape { Flat, Rows, Gather };
 // values, pointers, sizes and strides are arguments and not part of it.
 // For the flat shape two more facts are compiled in: which inputs are a single broadcast element
 // (bit k of broadcastMask), and whether no output aliases an input (the pointers may then be
-// declared __restrict__).
-std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
+// declared __restrict__).  streamOut (flat and rows shapes): the results leave through non-temporal stores -- large results
+// that nothing reads back from cache.
+std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false);
 // The same text written into `out` (cleared first; its capacity is reused from call to call).
-void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias);
+void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut = false);
 
 // Source of `extern "C" __global__ void aix_fused(Args)`.
-std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true);
+std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false);
 
 inline const char* entryName() { return "aix_fused"; }
 

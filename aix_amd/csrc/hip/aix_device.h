@@ -285,5 +285,57 @@ __device__ __forceinline__ bool tri_keeps(TriPos p, int e, u64 rows, u64 cols, i
 template <class T, int N> struct alignas(sizeof(T) * N) vec { T v[N]; };
 template <class T> struct vec16 { enum { n = 16 / sizeof(T) }; typedef vec<T, 16 / sizeof(T)> type; };
 
+// An operand of a row-shaped kernel: the 16-byte vector at row + col, or -- the operand is broadcast along the row --
+// copies of the one element *row.  Without a branch: a branch per operand makes the compiler wait for the first
+// operand's data before it issues the second operand's load (two memory latencies per lane instead of one; measured
+// 86 -> 74 us on x[8192, 8192] + v[8192]).  The broadcast element is fetched as the aligned 16 bytes around it (a
+// naturally aligned 16-byte block holding a valid element lies in the same page: the read cannot fault) and picked
+// out afterwards.
+template <class T, int N> __device__ __forceinline__ const vec<T, N>* row_vec_ptr(const T* row, u64 col, bool bcast)
+{
+    // as an offset from `row`, so that the pointer keeps its (global) address space
+    const long long off = bcast ? -(long long)((u64)row & (u64)(sizeof(T) * N - 1)) : (long long)(col * sizeof(T));
+    return (const vec<T, N>*)((const char*)row + off);
+}
+template <class T, int N> __device__ __forceinline__ vec<T, N> row_vec_fix(vec<T, N> v, const T* row, bool bcast)
+{
+    const unsigned k = (unsigned)(((u64)row & (u64)(sizeof(T) * N - 1)) / sizeof(T));
+    T s = v.v[0];
+#pragma unroll
+    for (int j = 1; j < N; ++j) s = k == (unsigned)j ? v.v[j] : s;
+#pragma unroll
+    for (int e = 0; e < N; ++e) v.v[e] = bcast ? s : v.v[e];
+    return v;
+}
+
+// Stores of values that this kernel and its neighbours will not read again.  A non-temporal store does not allocate its
+// line in the caches on the way out: on results of tens of megabytes that is worth 15 % of a copy-shaped kernel's time
+// (negate over 256 MiB: 87 -> 74 us; the transpose copy: 93 -> 79 us); small results are stored normally so that the
+// next kernel finds them in cache.
+template <class V> __device__ __forceinline__ void store_nt(V* p, const V& v)
+{
+    if constexpr (sizeof(V) == 16) { typedef unsigned int w4 __attribute__((ext_vector_type(4))); __builtin_nontemporal_store(__builtin_bit_cast(w4, v), (w4*)p); }
+    else if constexpr (sizeof(V) == 8) __builtin_nontemporal_store(__builtin_bit_cast(unsigned long long, v), (unsigned long long*)p);
+    else if constexpr (sizeof(V) == 4) __builtin_nontemporal_store(__builtin_bit_cast(unsigned int, v), (unsigned int*)p);
+    else if constexpr (sizeof(V) == 2) __builtin_nontemporal_store(__builtin_bit_cast(unsigned short, v), (unsigned short*)p);
+    else if constexpr (sizeof(V) == 1) __builtin_nontemporal_store(__builtin_bit_cast(unsigned char, v), (unsigned char*)p);
+    else if constexpr (sizeof(V) % 16 == 0 && alignof(V) >= 16) {
+        typedef unsigned int w4 __attribute__((ext_vector_type(4)));
+        struct Pieces { w4 q[sizeof(V) / 16]; };
+        const Pieces pieces = __builtin_bit_cast(Pieces, v);
+#pragma unroll
+        for (unsigned k = 0; k < sizeof(V) / 16; ++k) __builtin_nontemporal_store(pieces.q[k], (w4*)p + k);
+    }
+    else *p = v;
+}
+// The hint is a compile-time choice of the kernel: chosen at run time inside one kernel, the optimiser folds the two
+// branches' stores into ONE plain store and the hint is lost (and fencing them apart with empty asm statements makes
+// every wave wait for its store before it may retire: 74 -> 84 us on the row-broadcast add).
+template <bool NT, class V> __device__ __forceinline__ void store_sel(V* p, const V& v)
+{
+    if constexpr (NT) store_nt(p, v);
+    else *p = v;
+}
+
 } // namespace aixd
 #endif

@@ -77,6 +77,8 @@ struct aixk_event { hipEvent_t ev{nullptr}; };
 
 namespace aixk {
 
+size_t stream_store_min_bytes();                      // runtime.hip: AIXK_STREAM_STORE_MIN_BYTES or its environment override
+inline bool streams_out(size_t bytes) { return bytes >= stream_store_min_bytes(); }
 int resolve_static_scratch(aixk_ctx* ctx);          // reduce.hip; called once per context by aixk_create
 
 inline int set_device(aixk_ctx* ctx)

@@ -44,7 +44,7 @@ __global__ __launch_bounds__(kBlock) void gather_k(const W* __restrict__ src, W*
 }
 
 // rows: inner dim unit stride, 16-byte chunks
-template <class W, class IDX>
+template <class W, class IDX, bool NT>
 __global__ __launch_bounds__(kBlock) void gather_rows_k(const W* __restrict__ src, W* __restrict__ dst, Space<1> sp,
                                                         u64 total_chunks, IDX chunks)
 {
@@ -56,7 +56,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_k(const W* __restrict__ sr
         const IDX row = (IDX)(c / chunks);
         const IDX col = (IDX)(c - (u64)row * chunks) * VEC;
         const u64 p = locate<IDX>(outer, row) + col;
-        *(V*)(dst + c * VEC) = *(const V*)(src + p);
+        store_sel<NT>((V*)(dst + c * VEC), *(const V*)(src + p));
     }
 }
 
@@ -69,7 +69,7 @@ struct RowWalk {
     u64 ext[kMaxDims], src[kMaxDims], dst[kMaxDims];
     u64 src_off;
 };
-template <class W, class IDX>
+template <class W, class IDX, bool NT>
 __global__ __launch_bounds__(kBlock) void permute_rows_k(const W* __restrict__ src, W* __restrict__ dst, RowWalk w, u64 total_chunks, IDX chunks)
 {
     typedef typename vec16<W>::type V;
@@ -83,7 +83,7 @@ __global__ __launch_bounds__(kBlock) void permute_rows_k(const W* __restrict__ s
             ps += (u64)k * w.src[d]; pd += (u64)k * w.dst[d];
             row = q;
         }
-        *(V*)(dst + pd) = *(const V*)(src + ps);
+        store_sel<NT>((V*)(dst + pd), *(const V*)(src + ps));
     }
 }
 
@@ -122,19 +122,22 @@ __global__ __launch_bounds__(kBlock) void transpose_tiled_k(const W* __restrict_
 // Same tile walk with 16-byte global accesses on both sides (whole tiles only, everything
 // 16-byte aligned): a lane loads VEC consecutive r of one c, scatters them into the LDS tile as
 // tile[r][c], and later gathers VEC consecutive c of one r for a 16-byte store.  TR x TC is the
-// tile in elements (TR along the source's contiguous dim).  Measured on [8192,8192] f32: the
-// access pattern, not LDS, sets the pace; 128 x 64 (512-byte read runs, 256-byte write runs) with
-// four tiles that are neighbours along the destination's contiguous dim numbered consecutively
-// is the fastest of the shapes tried (5.3 TB/s against 6.0 TB/s for a plain copy).
-template <class W, int TR, int TC>
-__global__ __launch_bounds__(kBlock) void transpose_vec_k(const W* __restrict__ src, W* __restrict__ dst,
-                                                          u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r, u32 tiles_c)
+// tile in elements (TR along the source's contiguous dim), BLOCK the lanes of a workgroup.
+// Measured on [8192,8192] f32 (us; a plain copy of the same bytes: 89, with non-temporal stores 73):
+// 64 x 64 / 256 lanes 111, 128 x 64 / 256 lanes 102, 128 x 128 / 512 lanes 93 -- longer runs on both
+// sides (512 bytes) and 8 loads per lane in flight -- and 79 with the result leaving through
+// non-temporal stores; four tiles that are neighbours along the destination's contiguous dim are
+// numbered consecutively (one tile after another along either dim: 95-103).
+template <class W, int TR, int TC, int BLOCK, bool NT>
+__global__ __launch_bounds__(BLOCK) void transpose_vec_k(const W* __restrict__ src, W* __restrict__ dst,
+                                                         u64 R, u64 C, u64 ld, u64 sb, u64 off, u32 tiles_r, u32 tiles_c)
 {
     typedef typename vec16<W>::type V;
     constexpr int VEC = vec16<W>::n;
-    constexpr int LPR = TR / VEC, RPP = kBlock / LPR;      // lanes per source row, source rows per pass
-    constexpr int LPW = TC / VEC, WPP = kBlock / LPW;      // lanes per destination row, destination rows per pass
-    __shared__ W tile[TR][TC + 1];
+    constexpr int LPR = TR / VEC, RPP = BLOCK / LPR;       // lanes per source row, source rows per pass
+    constexpr int LPW = TC / VEC, WPP = BLOCK / LPW;       // lanes per destination row, destination rows per pass
+    extern __shared__ __align__(16) unsigned char transpose_lds[];
+    W (*tile)[TC + 1] = (W (*)[TC + 1])transpose_lds;
     const u32 t = blockIdx.x;
     u32 tr, tc;
     if (tiles_c % 4 == 0) { tc = (t / (4 * tiles_r)) * 4 + t % 4; tr = (t / 4) % tiles_r; }
@@ -157,7 +160,8 @@ __global__ __launch_bounds__(kBlock) void transpose_vec_k(const W* __restrict__ 
         V v;
 #pragma unroll
         for (int e = 0; e < VEC; ++e) v.v[e] = tile[rr][wv + e];
-        *(V*)(d + (r0 + rr) * C + c0 + wv) = v;
+        if constexpr (NT) store_nt((V*)(d + (r0 + rr) * C + c0 + wv), v);
+        else *(V*)(d + (r0 + rr) * C + c0 + wv) = v;
     }
 }
 
@@ -327,6 +331,7 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
         constexpr int VEC = vec16<W>::n;
         const W* ps = (const W*)src->data;
         W* pd = (W*)dst;
+        const bool nt = streams_out(n * sizeof(W));         // a large result leaves through non-temporal stores
         // 2-D / batched 2-D transposed: [B?, R, C] with strides (sb, 1, ld)
         if ((sp.rank == 2 && sp.stride[0][0] == 1) || (sp.rank == 3 && sp.stride[0][1] == 1)) {
             const int o = sp.rank - 2;
@@ -334,20 +339,29 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
             const uint64_t R = sp.shape[o], C = sp.shape[o + 1], ld = sp.stride[0][o + 1];
             const uint64_t tr = (R + kTile - 1) / kTile, tc = (C + kTile - 1) / kTile;
             const bool vecok = ld != 0 && ld % VEC == 0 && sb % VEC == 0 && aligned16(ps + sp.offset[0]) && aligned16(pd) && B < 65536;
-            // tile in elements: 512-byte read runs where the shape allows, else 64 x 64
-            constexpr int BIG_R = 128, BIG_C = sizeof(W) >= 4 ? 64 : 128;
-            if (vecok && sizeof(W) <= 4 && R % BIG_R == 0 && C % BIG_C == 0 && (R / BIG_R) * (C / BIG_C) < (1ull << 31)) {
-                hipLaunchKernelGGL((transpose_vec_k<W, BIG_R, BIG_C>), dim3((unsigned)((R / BIG_R) * (C / BIG_C)), (unsigned)B), dim3(kBlock), 0, ctx->stream,
-                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)(R / BIG_R), (u32)(C / BIG_C));
+            // tile in elements: 512-byte runs on both sides where the shape allows (128 x 128 of 4 bytes, 256 x 256 of
+            // 2 would not fit: 128 x 128 there too), else 64 x 64
+            auto launch_t = [&](auto kernel, uint64_t TR, uint64_t TC, unsigned block) {
+                const size_t lds = sizeof(W) * TR * (TC + 1);
+                hipLaunchKernelGGL(kernel, dim3((unsigned)((R / TR) * (C / TC)), (unsigned)B), dim3(block), lds, ctx->stream,
+                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)(R / TR), (u32)(C / TC));
                 AIXK_HIP(hipGetLastError());
                 return (int)AIXK_OK;
+            };
+            if (vecok && sizeof(W) <= 4 && sizeof(W) >= 2 && R % 128 == 0 && C % 128 == 0 && (R / 128) * (C / 128) < (1ull << 31) && (R / 128) * (C / 128) * B >= (uint64_t)ctx->cus)
+            {
+                if constexpr (sizeof(W) * 128 * 129 > 65536) {               // beyond the default limit of dynamic LDS: raised once
+                    static bool raised = false;
+                    if (!raised) {
+                        AIXK_HIP(hipFuncSetAttribute((const void*)transpose_vec_k<W, 128, 128, 512, true>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(W) * 128 * 129)));
+                        AIXK_HIP(hipFuncSetAttribute((const void*)transpose_vec_k<W, 128, 128, 512, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)(sizeof(W) * 128 * 129)));
+                        raised = true;
+                    }
+                }
+                return nt ? launch_t(transpose_vec_k<W, 128, 128, 512, true>, 128, 128, 512) : launch_t(transpose_vec_k<W, 128, 128, 512, false>, 128, 128, 512);
             }
-            if (vecok && R % kTile == 0 && C % kTile == 0 && tr * tc < (1ull << 31)) {
-                hipLaunchKernelGGL((transpose_vec_k<W, kTile, kTile>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
-                                   ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr, (u32)tc);
-                AIXK_HIP(hipGetLastError());
-                return (int)AIXK_OK;
-            }
+            if (vecok && R % kTile == 0 && C % kTile == 0 && tr * tc < (1ull << 31))
+                return nt ? launch_t(transpose_vec_k<W, kTile, kTile, kBlock, true>, kTile, kTile, kBlock) : launch_t(transpose_vec_k<W, kTile, kTile, kBlock, false>, kTile, kTile, kBlock);
             if (ld != 0 && tr * tc < (1ull << 31) && B < 65536) {
                 hipLaunchKernelGGL((transpose_tiled_k<W>), dim3((unsigned)(tr * tc), (unsigned)B), dim3(kBlock), 0, ctx->stream,
                                    ps, pd, (u64)R, (u64)C, (u64)ld, (u64)sb, (u64)sp.offset[0], (u32)tr, (u32)tc);
@@ -375,14 +389,18 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
                         for (int j = i; j > 0 && w.src[j] > w.src[j - 1]; --j) { std::swap(w.ext[j], w.ext[j - 1]); std::swap(w.src[j], w.src[j - 1]); std::swap(w.dst[j], w.dst[j - 1]); }
                     const uint64_t hop_there = w.dst[in - 1] * sizeof(W);
                     if (plain && hop_here >= 4096 && hop_there < hop_here) {
-                        if (small) hipLaunchKernelGGL((permute_rows_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u32)chunks);
-                        else hipLaunchKernelGGL((permute_rows_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u64)chunks);
+                        if (small) { if (nt) hipLaunchKernelGGL((permute_rows_k<W, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u32)chunks);
+                                     else hipLaunchKernelGGL((permute_rows_k<W, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u32)chunks); }
+                        else { if (nt) hipLaunchKernelGGL((permute_rows_k<W, u64, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u64)chunks);
+                               else hipLaunchKernelGGL((permute_rows_k<W, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, w, (u64)total, (u64)chunks); }
                         AIXK_HIP(hipGetLastError());
                         return (int)AIXK_OK;
                     }
                 }
-                if (small) hipLaunchKernelGGL((gather_rows_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u32)chunks);
-                else hipLaunchKernelGGL((gather_rows_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u64)chunks);
+                if (small) { if (nt) hipLaunchKernelGGL((gather_rows_k<W, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u32)chunks);
+                             else hipLaunchKernelGGL((gather_rows_k<W, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u32)chunks); }
+                else { if (nt) hipLaunchKernelGGL((gather_rows_k<W, u64, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u64)chunks);
+                       else hipLaunchKernelGGL((gather_rows_k<W, u64, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, pd, sp, (u64)total, (u64)chunks); }
                 AIXK_HIP(hipGetLastError());
                 return (int)AIXK_OK;
             }

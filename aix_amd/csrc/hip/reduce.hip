@@ -239,7 +239,16 @@ __global__ __launch_bounds__(kBlock) void reduce_all_finish_k(const T* __restric
     typedef typename Op::Acc Acc;
     __shared__ Acc smem[kWaves];
     Acc a = Op::init();
-    for (unsigned i = threadIdx.x; i < count; i += kBlock) a = Op::combine(a, partials[i]);
+    // batches of 8 loads in flight per lane: one after the other the (up to 16) loads of a lane are a chain of memory
+    // latencies, most of this kernel's time
+    constexpr unsigned U = 8;
+    for (unsigned i0 = threadIdx.x; i0 < count; i0 += kBlock * U) {
+        Acc r[U];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < count) r[k] = partials[i0 + k * kBlock];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < count) a = Op::combine(a, r[k]);
+    }
     a = block_reduce<Op>(a, smem);
     if (threadIdx.x == 0) land(Op{}, fin, dst, 0, a, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
 }
@@ -487,6 +496,82 @@ __global__ __launch_bounds__(kBlock) void argmax_onehot_inner_k(const T* __restr
     }
 }
 
+// argmax down the columns of wide rows with the rows split into chunks: the record a lane keeps per column is the
+// pair (value, row) and the scan is a bare `x > best` -- three instructions per element against the seven of
+// ArgOp::step -- and the partial records are 8 bytes instead of 12 (16 for 8-byte elements).  A strict `>` from minus
+// infinity never picks a NaN and keeps the first of equal values; what it cannot tell apart -- a column chunk whose
+// values are all NaN or the lowest value of the type -- is left as row = ~0 and settled by argmax_cols_finish_k.
+template <class W> struct ColRec { W v; u32 row; };
+template <> struct ColRec<double> { double v; u32 row; u32 pad; };
+template <> struct ColRec<i64> { i64 v; u32 row; u32 pad; };
+
+template <class T, int VEC>
+__global__ __launch_bounds__(kBlock) void argmax_cols_k(const T* __restrict__ src, RedPlan p, u64 rows_per_chunk, ColRec<typename traits<T>::W>* __restrict__ partials)
+{
+    typedef typename traits<T>::W W;
+    typedef vec<T, VEC> V;
+    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 c0 = ((u64)blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (c0 >= C) return;
+    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const u64 r_begin = (u64)blockIdx.y * rows_per_chunk;
+    const u64 r_end = r_begin + rows_per_chunk < R ? r_begin + rows_per_chunk : R;
+    W best[VEC]; u32 row[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) { best[e] = neg_inf<W>(); row[e] = ~0u; }
+    const T* col = src + s.src + c0;
+    constexpr int U = 8;
+    for (u64 r0 = r_begin; r0 < r_end; r0 += U) {
+        V x[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * p.r_src[0]);
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+            if (r0 + k < r_end) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) { const W w = up(x[k].v[e]); const bool more = w > best[e]; best[e] = more ? w : best[e]; row[e] = more ? (u32)(r0 + k) : row[e]; }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        ColRec<W> rec{};
+        rec.v = best[e]; rec.row = row[e];
+        partials[((u64)blockIdx.z * gridDim.y + blockIdx.y) * C + c0 + e] = rec;
+    }
+}
+
+// Second stage: a lane folds the chunk records of one column in chunk order (rows ascend with the chunks, so a later
+// record wins only with a strictly greater value), all its loads in flight at once, and lands the result.  A leading
+// NaN wins, as everywhere in this file.  A column no chunk found anything in holds only NaNs and lowest values: if its
+// first element is not a NaN it is such a lowest value and the first of them, so row 0 wins there too.
+template <class T>
+__global__ __launch_bounds__(kBlock) void argmax_cols_finish_k(const T* __restrict__ src, i32* dst, RedPlan p, unsigned chunks,
+                                                               const ColRec<typename traits<T>::W>* __restrict__ partials, Finish fin)
+{
+    typedef typename traits<T>::W W;
+    const u64 C = p.k_ext[p.nk - 1];
+    const u64 slot = (u64)blockIdx.x * kBlock + threadIdx.x;
+    if (slot >= p.slots) return;
+    const u64 o = slot / C, c = slot - o * C;
+    const ColRec<W>* col = partials + o * chunks * C + c;
+    W best = neg_inf<W>(); u32 row = ~0u;
+    constexpr unsigned U = 8;
+    for (unsigned k0 = 0; k0 < chunks; k0 += U) {
+        ColRec<W> r[U];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (k0 + k < chunks) r[k] = col[(u64)(k0 + k) * C];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (k0 + k < chunks && r[k].row != ~0u && (row == ~0u || r[k].v > best)) { best = r[k].v; row = r[k].row; }
+    }
+    const SlotPos s = slot_pos(p, o, p.nk - 1);
+    const T* first = src + s.src + c;
+    if (e_isnan(*first) || row == ~0u) row = 0;
+    const u64 flat = s.flat + (u64)row * p.r_flat[0] + c * p.k_flat[p.nk - 1];
+    if (fin.onehot) dst[flat] = 1;
+    else dst[s.dst + c] = fin.q_stride ? (i32)((flat / fin.q_stride) % fin.q_extent) : (i32)flat;
+}
+
 // second stage of `outer` when rows were split over several workgroups: 64 slots per workgroup,
 // the four waves take every fourth chunk (independent loads in flight), LDS folds the four.
 template <class Op, class T>
@@ -682,11 +767,39 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
         // the pair axis of a composed ReLU, say -- is one chunk: every lane folds its columns outright)
         if (vect && C >= (uint64_t)kBlock * v * 2 && (R >= 64 || R < 8) && O <= 65535) {
             const uint64_t tiles = (C + (uint64_t)kBlock * v - 1) / ((uint64_t)kBlock * v);
-            const uint64_t want = (uint64_t)cus * (sizeof(Acc) > 8 ? 2 : 8);      // wide partial records: fewer, longer chunks
+            // about one workgroup per compute unit for argmax (its partial records are wide and the second stage reads
+            // them all), eight for sums and maxima; the sweep itself runs at the same pace from 32 to 256 chunks
+            const uint64_t want = (uint64_t)cus * (Op::kTracksIndex ? 1 : 8);
             uint64_t chunks = tiles * O < want ? std::min<uint64_t>({(want + tiles * O - 1) / (tiles * O), (R + 15) / 16, (uint64_t)65535}) : 1;
             while (chunks > 1 && chunks * O * C * sizeof(Acc) > ctx->scratch_bytes) chunks /= 2;
-            const uint64_t rows_per_chunk = (R + chunks - 1) / chunks;
+            uint64_t rows_per_chunk = (R + chunks - 1) / chunks;
+            // The workgroups of a launch start together and walk their chunks in step.  If the chunks lie a multiple of
+            // 4 MiB apart (128 rows of 32 KiB, say) all of them ask the same memory channels for different DRAM rows at
+            // every step; the same happens within a few rows of such a distance.  Chunks are lengthened until their
+            // distance is at least 8 rows away from every multiple of 4 MiB (measured on [8192, 8192] f32: 128 rows per
+            // chunk 50 us, 127 or 129 rows 47-49 us, 136 rows 41 us).
+            if (chunks > 1) {
+                const uint64_t pitch = p.r_src[0] * sizeof(T), period = 4ull << 20, guard = 8 * pitch;
+                if (pitch > 0 && guard * 2 < period)
+                    for (int tries = 0; tries < 64; ++tries) {
+                        const uint64_t phase = (rows_per_chunk * pitch) % period;
+                        if (phase >= guard && phase <= period - guard) break;
+                        ++rows_per_chunk;
+                    }
+            }
             chunks = (R + rows_per_chunk - 1) / rows_per_chunk;
+            if constexpr (Op::kTracksIndex) {
+                // the (value, row) sweep with its own second stage
+                typedef ColRec<typename traits<T>::W> Rec;
+                if (chunks > 1 && fin.onehot != 2 && R < (1ull << 32) - 1 && chunks * O * C * sizeof(Rec) <= ctx->scratch_bytes) {
+                    Rec* recs = (Rec*)ctx->scratch;
+                    hipLaunchKernelGGL((argmax_cols_k<T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st, ps, p, (u64)rows_per_chunk, recs);
+                    AIXK_HIP(hipGetLastError());
+                    hipLaunchKernelGGL((argmax_cols_finish_k<T>), dim3((unsigned)((p.slots + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, ps, (i32*)dst, p, (unsigned)chunks, (const Rec*)recs, fin);
+                    AIXK_HIP(hipGetLastError());
+                    return AIXK_OK;
+                }
+            }
             Acc* partials = chunks > 1 ? (Acc*)ctx->scratch : nullptr;
             hipLaunchKernelGGL((reduce_outer_wide_k<Op, T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st,
                                ps, dst, p, (u64)rows_per_chunk, partials, fin);

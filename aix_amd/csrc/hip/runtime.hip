@@ -2,6 +2,8 @@
 
 #include "common.hpp"
 
+#include <cstdlib>
+
 #include <hip/hiprtc.h>
 
 #include <vector>
@@ -36,6 +38,17 @@ __global__ void zero_k(uint4* __restrict__ p, uint64_t n16, unsigned char* __res
 } // namespace aixk
 
 using namespace aixk;
+
+namespace aixk {
+size_t stream_store_min_bytes()
+{
+    static const size_t value = [] {
+        const char* e = std::getenv("AIXHIP_STREAM_STORE_MIN_BYTES");
+        return e && *e ? (size_t)std::strtoull(e, nullptr, 10) : (size_t)AIXK_STREAM_STORE_MIN_BYTES;
+    }();
+    return value;
+}
+} // namespace aixk
 
 extern "C" {
 

@@ -35,6 +35,10 @@ extern "C" {
 #define AIXK_ENOMEM  2
 #define AIXK_EHIP    3
 
+/* Results of at least this many bytes are written with non-temporal (streaming) stores; smaller ones stay in cache
+ * for the kernel that reads them next.  The environment variable AIXHIP_STREAM_STORE_MIN_BYTES overrides it. */
+#define AIXK_STREAM_STORE_MIN_BYTES (32ull << 20)
+
 /* Element types, numbered as aix::DataType (Targets/AIXLib/aixCore.hpp:44-55). */
 enum aixk_dtype {
     AIXK_F64 = 0, AIXK_F32 = 1, AIXK_F16 = 2, AIXK_BF16 = 3,
