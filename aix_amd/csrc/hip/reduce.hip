@@ -266,6 +266,12 @@ struct RedPlan {
 
 struct SlotPos { u64 src, dst, flat; };
 
+// What the column sweeps need of a plan, as plain kernel arguments: read out of the (1 KB) plan in the kernel they
+// cost a chain of dependent scalar loads at the head of every workgroup -- several microseconds where a workgroup
+// lives for ten.  `slot0` is the position of the first leading slot; with more leading slots (gridDim.z > 1) the
+// kernel still walks the plan.
+struct OuterDirect { u64 C, R, r_src, r_flat, k_flat; SlotPos slot0; };
+
 __device__ __forceinline__ SlotPos slot_pos(const RedPlan& p, u64 slot, int ndims)
 {
     SlotPos s; s.src = p.src_off; s.dst = 0; s.flat = 0;
@@ -385,15 +391,15 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_k(const T* __restrict__ s
 // LDS stage.  Long contiguous runs per row are what the strided walk needs to approach the
 // bandwidth of the unit-stride routes.
 template <class Op, class T, int VEC>
-__global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restrict__ src, typename Op::Out* dst, RedPlan p,
+__global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restrict__ src, typename Op::Out* dst, OuterDirect d, RedPlan p,
                                                               u64 rows_per_chunk, typename Op::Acc* partials, Finish fin)
 {
     typedef typename Op::Acc Acc;
     typedef vec<T, VEC> V;
-    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 C = d.C, R = d.R;
     const u64 c0 = ((u64)blockIdx.x * kBlock + threadIdx.x) * VEC;
     if (c0 >= C) return;
-    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const SlotPos s = gridDim.z == 1 ? d.slot0 : slot_pos(p, blockIdx.z, p.nk - 1);
     const u64 r_begin = (u64)blockIdx.y * rows_per_chunk;
     const u64 r_end = r_begin + rows_per_chunk < R ? r_begin + rows_per_chunk : R;
     Acc acc[VEC];
@@ -404,7 +410,7 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restric
     for (u64 r0 = r_begin; r0 < r_end; r0 += U) {
         V x[U];
 #pragma unroll
-        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * p.r_src[0]);
+        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * d.r_src);
 #pragma unroll
         for (int k = 0; k < U; ++k) {
             const u64 r = r0 + k;
@@ -417,9 +423,9 @@ __global__ __launch_bounds__(kBlock) void reduce_outer_wide_k(const T* __restric
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
         const u64 c = c0 + e;
-        if constexpr (Op::kTracksIndex) { if (acc[e].flags & 1u) acc[e].idx = (u32)(s.flat + (u64)acc[e].idx * p.r_flat[0] + c * p.k_flat[p.nk - 1]); }
+        if constexpr (Op::kTracksIndex) { if (acc[e].flags & 1u) acc[e].idx = (u32)(s.flat + (u64)acc[e].idx * d.r_flat + c * d.k_flat); }
         if (partials) partials[((u64)blockIdx.z * gridDim.y + blockIdx.y) * C + c] = acc[e];
-        else land(Op{}, fin, dst, s.dst + c, acc[e], src[s.src + c], s.flat + c * p.k_flat[p.nk - 1]);
+        else land(Op{}, fin, dst, s.dst + c, acc[e], src[s.src + c], s.flat + c * d.k_flat);
     }
 }
 
@@ -506,14 +512,14 @@ template <> struct ColRec<double> { double v; u32 row; u32 pad; };
 template <> struct ColRec<i64> { i64 v; u32 row; u32 pad; };
 
 template <class T, int VEC>
-__global__ __launch_bounds__(kBlock) void argmax_cols_k(const T* __restrict__ src, RedPlan p, u64 rows_per_chunk, ColRec<typename traits<T>::W>* __restrict__ partials)
+__global__ __launch_bounds__(kBlock) void argmax_cols_k(const T* __restrict__ src, OuterDirect d, RedPlan p, u64 rows_per_chunk, ColRec<typename traits<T>::W>* __restrict__ partials)
 {
     typedef typename traits<T>::W W;
     typedef vec<T, VEC> V;
-    const u64 C = p.k_ext[p.nk - 1], R = p.r_ext[0];
+    const u64 C = d.C, R = d.R;
     const u64 c0 = ((u64)blockIdx.x * kBlock + threadIdx.x) * VEC;
     if (c0 >= C) return;
-    const SlotPos s = slot_pos(p, blockIdx.z, p.nk - 1);
+    const SlotPos s = gridDim.z == 1 ? d.slot0 : slot_pos(p, blockIdx.z, p.nk - 1);
     const u64 r_begin = (u64)blockIdx.y * rows_per_chunk;
     const u64 r_end = r_begin + rows_per_chunk < R ? r_begin + rows_per_chunk : R;
     W best[VEC]; u32 row[VEC];
@@ -524,7 +530,7 @@ __global__ __launch_bounds__(kBlock) void argmax_cols_k(const T* __restrict__ sr
     for (u64 r0 = r_begin; r0 < r_end; r0 += U) {
         V x[U];
 #pragma unroll
-        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * p.r_src[0]);
+        for (int k = 0; k < U; ++k) if (r0 + k < r_end) x[k] = *(const V*)(col + (r0 + k) * d.r_src);
 #pragma unroll
         for (int k = 0; k < U; ++k) {
             if (r0 + k < r_end) {
@@ -546,28 +552,43 @@ __global__ __launch_bounds__(kBlock) void argmax_cols_k(const T* __restrict__ sr
 // NaN wins, as everywhere in this file.  A column no chunk found anything in holds only NaNs and lowest values: if its
 // first element is not a NaN it is such a lowest value and the first of them, so row 0 wins there too.
 template <class T>
-__global__ __launch_bounds__(kBlock) void argmax_cols_finish_k(const T* __restrict__ src, i32* dst, RedPlan p, unsigned chunks,
+__global__ __launch_bounds__(kBlock) void argmax_cols_finish_k(const T* __restrict__ src, i32* dst, OuterDirect d, RedPlan p, u64 slots, unsigned chunks,
                                                                const ColRec<typename traits<T>::W>* __restrict__ partials, Finish fin)
 {
     typedef typename traits<T>::W W;
-    const u64 C = p.k_ext[p.nk - 1];
-    const u64 slot = (u64)blockIdx.x * kBlock + threadIdx.x;
-    if (slot >= p.slots) return;
-    const u64 o = slot / C, c = slot - o * C;
-    const ColRec<W>* col = partials + o * chunks * C + c;
+    typedef ColRec<W> Rec;
+    __shared__ Rec sm[kWaves][kWave];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const u64 C = d.C;
+    const u64 slot = (u64)blockIdx.x * kWave + lane;           // 64 columns per workgroup; wave w folds chunks w, w + 4, ...
+    const bool live = slot < slots;
+    const u64 o = live ? slot / C : 0, c = live ? slot - o * C : 0;
     W best = neg_inf<W>(); u32 row = ~0u;
-    constexpr unsigned U = 8;
-    for (unsigned k0 = 0; k0 < chunks; k0 += U) {
-        ColRec<W> r[U];
+    if (live) {
+        const Rec* col = partials + o * chunks * C + c;
+        constexpr unsigned U = 8;
+        for (unsigned k0 = wave; k0 < chunks; k0 += kWaves * U) {
+            Rec r[U];
 #pragma unroll
-        for (unsigned k = 0; k < U; ++k) if (k0 + k < chunks) r[k] = col[(u64)(k0 + k) * C];
+            for (unsigned k = 0; k < U; ++k) if (k0 + k * kWaves < chunks) r[k] = col[(u64)(k0 + k * kWaves) * C];
 #pragma unroll
-        for (unsigned k = 0; k < U; ++k) if (k0 + k < chunks && r[k].row != ~0u && (row == ~0u || r[k].v > best)) { best = r[k].v; row = r[k].row; }
+            for (unsigned k = 0; k < U; ++k) if (k0 + k * kWaves < chunks && r[k].row != ~0u && (row == ~0u || r[k].v > best)) { best = r[k].v; row = r[k].row; }
+        }
     }
-    const SlotPos s = slot_pos(p, o, p.nk - 1);
+    Rec mine{}; mine.v = best; mine.row = row;
+    sm[wave][lane] = mine;
+    __syncthreads();
+    if (wave != 0 || !live) return;
+    // the waves hold interleaved chunks: among equal values the lower row wins
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+        const Rec r = sm[w][lane];
+        if (r.row != ~0u && (row == ~0u || r.v > best || (r.v == best && r.row < row))) { best = r.v; row = r.row; }
+    }
+    const SlotPos s = slots == C ? d.slot0 : slot_pos(p, o, p.nk - 1);
     const T* first = src + s.src + c;
     if (e_isnan(*first) || row == ~0u) row = 0;
-    const u64 flat = s.flat + (u64)row * p.r_flat[0] + c * p.k_flat[p.nk - 1];
+    const u64 flat = s.flat + (u64)row * d.r_flat + c * d.k_flat;
     if (fin.onehot) dst[flat] = 1;
     else dst[s.dst + c] = fin.q_stride ? (i32)((flat / fin.q_stride) % fin.q_extent) : (i32)flat;
 }
@@ -705,6 +726,14 @@ bool onehot_rows_route(const RedPlan& p, const T* ps, const void* dst)
     return true;
 }
 
+inline OuterDirect outer_direct(const RedPlan& p)
+{
+    OuterDirect d;
+    d.C = p.k_ext[p.nk - 1]; d.R = p.r_ext[0]; d.r_src = p.r_src[0]; d.r_flat = p.r_flat[0]; d.k_flat = p.k_flat[p.nk - 1];
+    d.slot0.src = p.src_off; d.slot0.dst = 0; d.slot0.flat = 0;
+    return d;
+}
+
 template <class Op, class T>
 int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, const RedPlan& p, const Finish& fin)
 {
@@ -767,9 +796,10 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
         // the pair axis of a composed ReLU, say -- is one chunk: every lane folds its columns outright)
         if (vect && C >= (uint64_t)kBlock * v * 2 && (R >= 64 || R < 8) && O <= 65535) {
             const uint64_t tiles = (C + (uint64_t)kBlock * v - 1) / ((uint64_t)kBlock * v);
-            // about one workgroup per compute unit for argmax (its partial records are wide and the second stage reads
-            // them all), eight for sums and maxima; the sweep itself runs at the same pace from 32 to 256 chunks
-            const uint64_t want = (uint64_t)cus * (Op::kTracksIndex ? 1 : 8);
+            // two workgroups per compute unit: the sweep runs at the same pace from 32 to 256 chunks (41 us on [8192, 8192]
+            // f32), the second stage costs a microsecond per 30 chunks, and with one workgroup per compute unit the pace
+            // depends on details of the instruction stream (41 or 47-49 us for near-identical kernels)
+            const uint64_t want = (uint64_t)cus * 2;
             uint64_t chunks = tiles * O < want ? std::min<uint64_t>({(want + tiles * O - 1) / (tiles * O), (R + 15) / 16, (uint64_t)65535}) : 1;
             while (chunks > 1 && chunks * O * C * sizeof(Acc) > ctx->scratch_bytes) chunks /= 2;
             uint64_t rows_per_chunk = (R + chunks - 1) / chunks;
@@ -793,16 +823,16 @@ int run_plan(aixk_ctx* ctx, const aixhip_tensor* src, typename Op::Out* dst, con
                 typedef ColRec<typename traits<T>::W> Rec;
                 if (chunks > 1 && fin.onehot != 2 && R < (1ull << 32) - 1 && chunks * O * C * sizeof(Rec) <= ctx->scratch_bytes) {
                     Rec* recs = (Rec*)ctx->scratch;
-                    hipLaunchKernelGGL((argmax_cols_k<T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st, ps, p, (u64)rows_per_chunk, recs);
+                    hipLaunchKernelGGL((argmax_cols_k<T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st, ps, outer_direct(p), p, (u64)rows_per_chunk, recs);
                     AIXK_HIP(hipGetLastError());
-                    hipLaunchKernelGGL((argmax_cols_finish_k<T>), dim3((unsigned)((p.slots + kBlock - 1) / kBlock)), dim3(kBlock), 0, st, ps, (i32*)dst, p, (unsigned)chunks, (const Rec*)recs, fin);
+                    hipLaunchKernelGGL((argmax_cols_finish_k<T>), dim3((unsigned)((p.slots + kWave - 1) / kWave)), dim3(kBlock), 0, st, ps, (i32*)dst, outer_direct(p), p, (u64)p.slots, (unsigned)chunks, (const Rec*)recs, fin);
                     AIXK_HIP(hipGetLastError());
                     return AIXK_OK;
                 }
             }
             Acc* partials = chunks > 1 ? (Acc*)ctx->scratch : nullptr;
             hipLaunchKernelGGL((reduce_outer_wide_k<Op, T, VEC>), dim3((unsigned)tiles, (unsigned)chunks, (unsigned)O), dim3(kBlock), 0, st,
-                               ps, dst, p, (u64)rows_per_chunk, partials, fin);
+                               ps, dst, outer_direct(p), p, (u64)rows_per_chunk, partials, fin);
             AIXK_HIP(hipGetLastError());
             if (chunks > 1) {
                 hipLaunchKernelGGL((reduce_outer_finish_k<Op, T>), dim3(grid_for(p.slots, kWave, cus * 8u)), dim3(kBlock), 0, st,
