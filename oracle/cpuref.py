@@ -11,7 +11,13 @@ import subprocess
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+REF_BUILT_NOTE = os.path.join(HERE, "ref_built.note")
 MAX_RANK = 16
+
+
+def ref_expected():
+    """True where this tree was built with the reference present: oracle/_ref must then be there too."""
+    return os.path.exists(REF_BUILT_NOTE)
 
 F64, F32, F16, BF16, I64, I32, I16, I8, U8 = range(9)
 DTYPE_NAMES = ["f64", "f32", "f16", "bf16", "i64", "i32", "i16", "i8", "u8"]
@@ -101,6 +107,10 @@ def build(ref=True, force=False):
     subprocess.check_call(["make", "-s", "-C", HERE, "all"] + extra)
     if ref and os.path.isdir(os.environ.get("AIX_REFERENCE_DIR", "/root/reference")):
         subprocess.check_call(["make", "-s", "-C", HERE, "ref"] + extra)
+        # a note beside (not inside) _ref/ that the reference-backed libraries belong to this tree: a test that finds
+        # the note but not the libraries fails instead of skipping
+        with open(REF_BUILT_NOTE, "w") as f:
+            f.write("oracle/_ref was built from the reference tree by oracle/Makefile (target ref)\n")
 
 
 _T = C.POINTER(TensorDesc)

@@ -237,3 +237,31 @@ def oracle_transformer(cfg, steps, data, threads=1, stacked=False):
     if rc != 0:
         raise RuntimeError(lib.oracle_drivers_last_error().decode())
     return losses, norms, secs
+
+
+# ---- the reference's device test cases (oracle/ref_drivers.cpp: deviceChecks) --------------------------------------
+def _device_checks_here(on_hip):
+    lib = C.CDLL(ref_hip_lib_path() if on_hip else os.path.join(HERE, "_ref", "libaixref_drivers.so"))
+    lib.aixref_device_checks.argtypes = [C.c_int, C.c_char_p, C.c_uint64, C.POINTER(C.c_int)]
+    lib.aixref_drivers_last_error.restype = C.c_char_p
+    report = C.create_string_buffer(1 << 16)
+    checks = C.c_int(0)
+    failures = lib.aixref_device_checks(int(on_hip), report, len(report), C.byref(checks))
+    if failures < 0:
+        raise RuntimeError(lib.aixref_drivers_last_error().decode())
+    return failures, checks.value, report.value.decode()
+
+
+def ref_device_checks(on_hip):
+    """The reference's device test cases with its own classes around the device under test: its CPU device standing in
+    (on_hip False; must pass trivially) or DeviceHIP (separate process, see ref_hip_mlp).  (failures, checks, report)."""
+    import json
+    import subprocess
+    import sys
+    code = ("import json, sys; sys.path.insert(0, %r); from oracle import drivers as d; print(json.dumps(d._device_checks_here(%r)))"
+            % (os.path.dirname(HERE), bool(on_hip)))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=1200)
+    if out.returncode != 0:
+        raise RuntimeError("device checks failed to run: " + out.stderr[-2000:])
+    failures, checks, report = json.loads(out.stdout.strip().splitlines()[-1])
+    return failures, checks, report

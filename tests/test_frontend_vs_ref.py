@@ -45,3 +45,10 @@ def test_single_pass_backward_gives_the_same_gradients():
     once, _, (ops_b, mm_b) = drivers.oracle_mlp(*shape, 30, 1e-3, data, single_pass=True)
     assert np.all(np.abs(per_path.astype(np.float64) - once) <= 2e-6 * np.abs(per_path))
     assert mm_b == 30 * (3 + 5) and mm_a == 30 * (3 + 4 * 5)
+
+
+def test_reference_device_test_cases_pass_on_the_reference_cpu_device():
+    """A check of the checks: the device cases of oracle/ref_drivers.cpp (deviceChecks) with the reference's CPU device
+    standing in as the device under test must pass without a failure."""
+    failures, checks, report = drivers.ref_device_checks(False)
+    assert checks > 5000 and failures == 0, report

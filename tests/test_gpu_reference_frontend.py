@@ -10,10 +10,17 @@ the product build of DeviceHIP (same operator stream, so the same numbers bit fo
 import numpy as np
 import pytest
 
-from oracle import drivers as OD
+from oracle import cpuref, drivers as OD
 
+MISSING = OD.ref_hip_lib_path() is None or OD.ref_lib() is None
+# a tree that was never built next to the reference has no oracle/_ref: skip; a tree that was, and lost it: fail loudly
 pytestmark = [pytest.mark.gpu,
-              pytest.mark.skipif(OD.ref_hip_lib_path() is None or OD.ref_lib() is None, reason="oracle/_ref not built (no reference tree)")]
+              pytest.mark.skipif(MISSING and not cpuref.ref_expected(), reason="oracle/_ref not built (no reference tree)")]
+
+
+@pytest.fixture(autouse=True)
+def _reference_libraries_are_there():
+    assert not MISSING, "this tree was built with the reference present (oracle/ref_built.note) but oracle/_ref/*.so is missing"
 
 
 def test_reference_tensor_autograd_adam_run_unchanged_on_device_hip():
@@ -68,3 +75,14 @@ def test_reference_save_and_load_through_device_memory(tmp_path):
     assert trained.view(np.uint32).tolist() == on_gpu.view(np.uint32).tolist()
     assert np.abs(on_cpu - trained).max() <= 1e-5
     assert np.abs(trained - np.array([0.0, 1.0, 1.0, 0.0])).max() < 5e-2
+
+
+def test_reference_device_test_cases_on_device_hip():
+    """The cases of the reference's device test file -- every operator against its CPU device over the reference's test
+    sizes and all nine element types, 200 queued operator pairs with autograd, 1024 chained adds on a million elements,
+    1000 Adam steps without a synchronize, the benchmark's XOR model -- written with the reference's own TensorValue /
+    Tensor / nn / optim classes (oracle/ref_drivers.cpp: deviceChecks) and run with DeviceHIP as the device under test."""
+    failures, checks, report = OD.ref_device_checks(True)
+    print(f"{checks} checks, {failures} failures\n{report}")
+    assert checks > 5000
+    assert failures == 0, report
