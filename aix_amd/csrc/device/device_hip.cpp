@@ -96,6 +96,10 @@ struct DeviceHIP::Extras {
     std::string key;
     std::vector<uint64_t> args;
     gen::Space space;
+    // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
+    struct Group { std::vector<aixhip_tensor> a, b, out; };
+    std::array<Group, 4> groups;
+    bool anyPending() const { for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
     // results of at least this many bytes are written with non-temporal stores (the kernel layer's rule, same override)
     size_t streamStoreMinBytes = [] {
         const char* e = std::getenv("AIXHIP_STREAM_STORE_MIN_BYTES");
@@ -197,6 +201,7 @@ DeviceHIP::~DeviceHIP()
     try {
         if (m_engine && m_engine->pendingOps() > 0)
             std::cerr << "DeviceHIP: destroyed with recorded work that was never synchronised." << std::endl;   // aixDeviceMetal.cpp:146-149
+        if (m_ctx && m_extras && m_extras->anyPending()) issueMatmulGroup();           // matmul calls still waiting for company
         if (m_engine) m_engine.reset();
         if (m_ctx) {
             aixk_sync(m_ctx);
@@ -375,6 +380,7 @@ void DeviceHIP::emptyCache()
 
 void DeviceHIP::flush()
 {
+    issueMatmulGroup();                                     // pending products were called before anything now in the window was recorded
     m_engine->flush();
     releaseLimbo();
 }
@@ -552,6 +558,7 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
 // ---- planner callbacks -------------------------------------------------------------------------
 void DeviceHIP::emitSingle(const OpRecord& op)
 {
+    issueMatmulGroup();
     aixhip_tensor a, b, o;
     markTouched(op.output.data);
     markTouched(op.input0.data);
@@ -577,6 +584,7 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 
 void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 {
+    issueMatmulGroup();
     constexpr size_t kMaxOperands = 64;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     const size_t esz = dataTypeSize(d.dtype);
@@ -738,9 +746,54 @@ void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorPar
     check(aixk_reduce_all(m_ctx, AIXK_ARGMAX_ONEHOT, &pa, &pr));
 }
 
+// The interface has no batch dimension (aixCore.hpp:943-976), so attention over (sequence, head) pairs, or any batch of
+// small products, arrives as a run of matmul calls of one shape.  One launch per call leaves the chip mostly idle (a
+// [512, 512] x [512, 512] bf16 product: 4.4 us for 0.3 us of arithmetic), so such calls are not issued at once: a small
+// 16-bit product whose operands lie in device memory joins the group of pending products if it has their shape and
+// operand layout and depends on none of them, and the group is issued as ONE launch when anything else happens -- an
+// operator of another kind is enqueued, recorded operators are planned, the window is flushed or synchronised.  The
+// reference batches its dispatches for the same reason (aixDeviceMetal.cpp:1344-1389).
 void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& result)
 {
     requireDevice(result, "matmul");
+    auto& ex = *m_extras;
+    const bool sixteen = result.dtype == DataType::kFloat16 || result.dtype == DataType::kBFloat16;
+    if (sixteen && a.shape.size() == 2 && b.shape.size() == 2 && result.shape.size() == 2 && a.dtype == result.dtype && b.dtype == result.dtype &&
+        a.size && b.size && findBlock(a.data) && findBlock(b.data)) {
+        const size_t M = a.shape[0], K = a.shape[1], N = b.shape[1];
+        const bool small = K % 8 == 0 && M * N >= 64 * 64 && ((M + 63) / 64) * ((N + 63) / 64) < (size_t)m_cus * 2;
+        if (small && b.shape[0] == K && result.shape[0] == M && result.shape[1] == N) {
+            // recorded operators that produce an operand, or that still use the result's buffer, go first (and so does
+            // every pending product); any other recorded operator may as well run after the product
+            if (m_engine->pendingWrites(a.data) || m_engine->pendingWrites(b.data) || m_engine->pendingTouches(result.data)) {
+                m_engine->recordExternalRead(a.data);
+                m_engine->recordExternalRead(b.data);
+                flush();
+            }
+            aixhip_tensor pa, pb, pr; toPod(a, &pa, "matmul"); toPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
+            // it may read no pending result and overwrite nothing pending: all pending products are then independent of
+            // each other, whatever group they wait in, and the groups may be issued in any order
+            bool independent = true;
+            for (const auto& g : ex.groups)
+                for (size_t i = 0; independent && i < g.out.size(); ++i)
+                    independent = g.out[i].data != pa.data && g.out[i].data != pb.data && g.out[i].data != pr.data &&
+                                  g.a[i].data != pr.data && g.b[i].data != pr.data;
+            if (!independent) issueMatmulGroup();
+            // the group of its shape and operand layout (forward and backward products of attention alternate between
+            // two or three of them), or the emptiest slot
+            Extras::Group* into = nullptr;
+            for (auto& g : ex.groups) {
+                if (g.out.empty()) { if (!into) into = &g; continue; }
+                const aixhip_tensor &ga = g.a[0], &gb = g.b[0];
+                if (g.out[0].dtype == pr.dtype && ga.shape[0] == M && ga.shape[1] == K && gb.shape[1] == N && ga.strides[0] == pa.strides[0] &&
+                    ga.strides[1] == pa.strides[1] && gb.strides[0] == pb.strides[0] && gb.strides[1] == pb.strides[1] && g.out.size() < 4096) { into = &g; break; }
+            }
+            if (!into) { issueMatmulGroup(); into = &ex.groups[0]; }
+            into->a.push_back(pa); into->b.push_back(pb); into->out.push_back(pr);
+            markTouched(a.data); markTouched(b.data); markTouched(result.data);
+            return;
+        }
+    }
     flushFor(a.data, b.data, result.data);
     aixhip_tensor pa, pb, pr; stagedPod(a, &pa, "matmul"); stagedPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
     // operands with leading dims in front of the matrix dims: a stack of products (beyond the reference, whose
@@ -753,6 +806,20 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
         synchronize();
         emptyCache();
         status = run();
+    }
+    check(status);
+}
+
+void DeviceHIP::issueMatmulGroup()
+{
+    auto& ex = *m_extras;
+    int status = AIXK_OK;
+    for (auto& g : ex.groups) {
+        if (g.out.empty()) continue;
+        const uint32_t count = (uint32_t)g.out.size();
+        if (status == AIXK_OK)
+            status = count == 1 ? aixk_matmul(m_ctx, &g.a[0], &g.b[0], &g.out[0]) : aixk_matmul_grouped(m_ctx, g.a.data(), g.b.data(), g.out.data(), count);
+        g.a.clear(); g.b.clear(); g.out.clear();
     }
     check(status);
 }

@@ -157,6 +157,7 @@ private:
     void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void emitSingle(const aixhip::fuse::OpRecord& op);
+    void issueMatmulGroup();                                 // the pending matmul calls as one launch (see matmul())
 
     aixk_ctx* m_ctx{nullptr};
     std::unique_ptr<aixhip::fuse::FuseEngine> m_engine;

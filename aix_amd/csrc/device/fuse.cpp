@@ -871,6 +871,21 @@ bool FuseEngine::takeTrailingFill(const View& output, OpRecord* fill)
     return false;
 }
 
+bool FuseEngine::pendingWrites(const void* buffer) const
+{
+    if (!buffer) return false;
+    for (const OpRecord& op : m_pending) if (op.output.data == buffer) return true;
+    return false;
+}
+
+bool FuseEngine::pendingTouches(const void* buffer) const
+{
+    if (!buffer) return false;
+    for (const OpRecord& op : m_pending)
+        if (op.output.data == buffer || op.input0.data == buffer || (op.hasInput1 && op.input1.data == buffer)) return true;
+    return false;
+}
+
 void FuseEngine::recordExternalRead(const void* buffer)
 {
     if (!buffer) return;

@@ -191,6 +191,8 @@ public:
     // tensor, remove it from the window and hand it over (the caller folds it into the operator
     // it is about to run eagerly); false and no change otherwise.
     bool takeTrailingFill(const View& output, OpRecord* fill);
+    bool pendingWrites(const void* buffer) const;  // a recorded operator of the window writes the buffer
+    bool pendingTouches(const void* buffer) const; // ... reads or writes it
     void recordExternalRead(const void* buffer);   // the buffer is about to be read outside the planner
     void retainBuffer(void* buffer);               // allocate(): results written here must reach memory
     void releaseBuffer(void* buffer);              // deallocate(): nobody will read it after the window

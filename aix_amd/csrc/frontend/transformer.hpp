@@ -113,19 +113,25 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
                 const Tensor scores = matmul(q4, k4.transpose(2, 3)).tril() * scale + mask;         // [batch, heads, seq, seq]; scale and mask fuse
                 attn = matmul(softmax(scores, 3, true), v4).transpose(1, 2).reshape(Shape{T, d});
             } else {
-                std::vector<Tensor> sequences;
+                // One 2-D product per (sequence, head), as the interface has it, written stage by stage -- all score products,
+                // then every head's mask and softmax, then all mixing products -- so that a device that batches runs of
+                // equal-shaped matmul calls finds such runs (the arithmetic per head is the same in any order).
+                const uint64_t pairs = c.batch * c.heads;
+                std::vector<Tensor> qh(pairs), kh(pairs), vh(pairs), raw(pairs), prob(pairs), mixed(pairs);
                 for (uint64_t b = 0; b < c.batch; ++b) {
                     const Tensor qb = q.slice(0, b * c.seq, (b + 1) * c.seq), kb = k.slice(0, b * c.seq, (b + 1) * c.seq),
                                  vb = v.slice(0, b * c.seq, (b + 1) * c.seq);
-                    std::vector<Tensor> heads;
                     for (uint64_t hd = 0; hd < c.heads; ++hd) {
-                        const Tensor qh = qb.slice(1, hd * dh, (hd + 1) * dh), kh = kb.slice(1, hd * dh, (hd + 1) * dh),
-                                     vh = vb.slice(1, hd * dh, (hd + 1) * dh);
-                        const Tensor scores = matmul(qh, kh.transpose(0, 1)).tril() * scale + mask;
-                        heads.push_back(matmul(softmax(scores, 1, true), vh));
+                        const uint64_t i = b * c.heads + hd;
+                        qh[i] = qb.slice(1, hd * dh, (hd + 1) * dh); kh[i] = kb.slice(1, hd * dh, (hd + 1) * dh); vh[i] = vb.slice(1, hd * dh, (hd + 1) * dh);
                     }
-                    sequences.push_back(Tensor::cat(heads, 1));
                 }
+                for (uint64_t i = 0; i < pairs; ++i) raw[i] = matmul(qh[i], kh[i].transpose(0, 1));
+                for (uint64_t i = 0; i < pairs; ++i) prob[i] = softmax(raw[i].tril() * scale + mask, 1, true);
+                for (uint64_t i = 0; i < pairs; ++i) mixed[i] = matmul(prob[i], vh[i]);
+                std::vector<Tensor> sequences;
+                for (uint64_t b = 0; b < c.batch; ++b)
+                    sequences.push_back(Tensor::cat(std::vector<Tensor>(mixed.begin() + (long)(b * c.heads), mixed.begin() + (long)((b + 1) * c.heads)), 1));
                 attn = Tensor::cat(sequences, 0);
             }
             x = x + (matmul(attn, W[at + 8]) + W[at + 9]);

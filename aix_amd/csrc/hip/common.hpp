@@ -67,6 +67,13 @@ struct aixk_ctx {
     // like everything else
     void* gemm_ws[3]{nullptr, nullptr, nullptr};
     size_t gemm_ws_bytes[3]{0, 0, 0};
+    // small tables that kernels read from device memory (the operand addresses of a grouped launch): a pinned host ring
+    // and its device twin, filled slot by slot and copied on the stream; an event per lap guards the reuse of a slot
+    char* table_host{nullptr};
+    char* table_dev{nullptr};
+    size_t table_bytes{0}, table_used{0};
+    hipEvent_t table_lap[2]{nullptr, nullptr};
+    int table_half{0};
     // runtime-compiled kernels by signature
     std::unordered_map<std::string, aixk_module*> rtc;
     uint64_t rtc_hits{0}, rtc_misses{0};
@@ -79,7 +86,10 @@ namespace aixk {
 
 size_t stream_store_min_bytes();                      // runtime.hip: AIXK_STREAM_STORE_MIN_BYTES or its environment override
 inline bool streams_out(size_t bytes) { return bytes >= stream_store_min_bytes(); }
-int resolve_static_scratch(aixk_ctx* ctx);          // reduce.hip; called once per context by aixk_create
+int resolve_static_scratch(aixk_ctx* ctx);
+// runtime.hip: `bytes` of table space: where the host writes it and where kernels will find it once table_upload() has run
+int table_slot(aixk_ctx* ctx, size_t bytes, void** host, const void** dev);
+int table_upload(aixk_ctx* ctx, const void* host, const void* dev, size_t bytes);          // reduce.hip; called once per context by aixk_create
 
 inline int set_device(aixk_ctx* ctx)
 {

@@ -20,6 +20,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
 // The same for a stack of products (a, b, out: the 2-D descriptors of the first matrices; batch: the joint
 // collapsed space of the leading dims, operands a, b, out).
 int matmul_mfma_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>& batch);
+int matmul_mfma_grouped(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, uint32_t count);
 } // namespace aixk
 
 namespace {
@@ -128,6 +129,25 @@ extern "C" int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixh
 // out[..., m, n] = a[..., m, k] . b[..., k, n]: one product per index of the leading dims, which a, b and out share
 // (any of them may be a view: permuted, sliced, stride 0).  The results are written densely, row-major over
 // (leading dims, m, n), from out->data.
+extern "C" int32_t aixk_matmul_grouped(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(count == 0 || (a && b && out), "matmul group: null operand arrays");
+    if (count >= 2) {
+        bool plain = true;
+        for (uint32_t i = 0; i < count && plain; ++i)
+            plain = valid_tensor(&a[i]) && valid_tensor(&b[i]) && valid_tensor(&out[i]) && a[i].rank == 2 && b[i].rank == 2 && out[i].rank == 2 &&
+                    a[i].shape[1] == b[i].shape[0] && out[i].shape[0] == a[i].shape[0] && out[i].shape[1] == b[i].shape[1] && out[i].data != nullptr &&
+                    a[i].shape[0] && b[i].shape[1] && a[i].shape[1];
+        if (plain) {
+            const int rc = matmul_mfma_grouped(ctx, a, b, out, count);
+            if (rc != -1) return rc;
+        }
+    }
+    for (uint32_t i = 0; i < count; ++i) AIXK_TRY(aixk_matmul(ctx, &a[i], &b[i], &out[i]));    // one by one, every check of the single call
+    return AIXK_OK;
+}
+
 extern "C" int32_t aixk_matmul_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)
 {
     AIXK_TRY(set_device(ctx));

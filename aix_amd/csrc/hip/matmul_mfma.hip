@@ -52,9 +52,12 @@ struct GemmArgs {
 // A stack of independent products in one launch: blockIdx.y numbers the matrices in row-major order of up to
 // three (collapsed) leading dims; every matrix of A / B starts sa / sb elements further per step of its dim,
 // results are dense, sc elements apart.  rank 0: a single product.
+// `table` set: the matrices are unrelated buffers instead -- three addresses (A, B, C) per matrix in device memory, in
+// the order of blockIdx.y (a group of separate matmul calls issued as one launch).
 struct BatchArgs {
     u32 rank, ext[3];
     u64 sa[3], sb[3], sc;
+    const u64* table;
 };
 
 // blockIdx -> output tile, XCD-aware and grouped (4 tile rows per column sweep).
@@ -400,7 +403,10 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
     const u16* A = (const u16*)g.a;
     const u16* B = (const u16*)g.b;
     T* C = (T*)g.c;
-    if (bt.rank) {                                           // uniform over the workgroup: scalar arithmetic
+    if (bt.table) {
+        const u64* entry = bt.table + 3 * (u64)blockIdx.y;
+        A = (const u16*)entry[0]; B = (const u16*)entry[1]; C = (T*)entry[2];
+    } else if (bt.rank) {                                    // uniform over the workgroup: scalar arithmetic
         u32 rest = blockIdx.y;
         for (int d = (int)bt.rank - 1; d >= 0; --d) {
             const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
@@ -525,7 +531,10 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
     const int wm = wave >> 1, wn = wave & 1;
     const u16* A = (const u16*)g.a;
     const u16* B = (const u16*)g.b;
-    if (bt.rank) {                                           // uniform over the workgroup: scalar arithmetic
+    if (bt.table) {
+        const u64* entry = bt.table + 3 * (u64)blockIdx.y;
+        A = (const u16*)entry[0]; B = (const u16*)entry[1];
+    } else if (bt.rank) {                                    // uniform over the workgroup: scalar arithmetic
         u32 rest = blockIdx.y;
         for (int d = (int)bt.rank - 1; d >= 0; --d) {
             const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
@@ -666,7 +675,7 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 
     // accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
     const u64 plane = g.M * g.N;
-    T* C = (T*)g.c + (u64)blockIdx.y * plane;
+    T* C = bt.table ? (T*)bt.table[3 * (u64)blockIdx.y + 2] : (T*)g.c + (u64)blockIdx.y * plane;
     float* P = sk.splits > 1 ? sk.partial + ((u64)blockIdx.z * sk.matrices + blockIdx.y) * plane : nullptr;
     if (!P && g.N % 8 == 0 && ((size_t)g.c & 15) == 0) {
         // Through LDS (free after the last barrier), each wave on its own 32 x 32 slab: written as the MFMA leaves it (a lane
@@ -1077,7 +1086,7 @@ template <class K> int set_lds(K kernel, size_t bytes)
 
 // gemm_small16_k on the last two dims of a / b (rank 2 descriptors), `batch` = the joint collapsed space of the
 // leading dims (operands 0, 1, 2 = a, b, out) or null for one product.  -1: a layout the kernel does not take.
-int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch)
+int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch, const u64* table = nullptr)
 {
     const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
     constexpr size_t esz = 2;
@@ -1100,6 +1109,7 @@ int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b
         if (count > 65535) return -1;
         bt.sc = M * N;
         if (bt.rank == 0) { bt.rank = 1; bt.ext[0] = 1; }
+        bt.table = table;
     }
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
@@ -1134,7 +1144,7 @@ constexpr int tile16_bk(int bm) { return bm == 64 ? 64 : 32; }
 // gemm_tile16_k on the last two dims of a / b, `batch` as for launch_small16.  tile: 0 = 64 x 64, 1 = 128 x 64,
 // 2 = 128 x 128; splits: K splits wanted (1 = none).  -1: a layout the kernel does not take.
 int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch,
-                  int tile, uint64_t splits)
+                  int tile, uint64_t splits, const u64* table = nullptr)
 {
     const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
     constexpr size_t esz = 2;
@@ -1156,6 +1166,7 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         }
         if (count > 65535) return -1;
         bt.sc = M * N;
+        bt.table = table;
     }
     const uint64_t bm = tile == 0 ? 64 : 128, bn = tile == 2 ? 128 : 64;
     GemmArgs g{};
@@ -1213,7 +1224,7 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
 // [8192,768]x[768,768] 28 -> 23, [8192,3072]^T-free x [3072,768] 76 -> 67, weight gradients [768,8192]x[8192,768]
 // 73 -> 32 (8 K splits) and [768,8192]x[8192,3072] 113 -> 72 (4 splits), stacks of 192 attention products
 // [512,64]x[64,512] 121 -> 42, [512,512]x[512,64] 52 -> 27, [512,512]^T x [512,64] 92 -> 27.
-int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch)
+int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch, const u64* table = nullptr)
 {
     const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
     const uint64_t cus = (uint64_t)ctx->cus;
@@ -1226,9 +1237,10 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
     };
     if (batch) {
         // stacks: thin results (attention's [seq, head dim]) on 128 x 64 tiles, everything else on 128 x 128
-        if (M <= 64) return launch_tile16(ctx, a, b, out, batch, 0, splits_for(t64 * count, (K + 63) / 64 * 2, 4));
-        if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, splits_for(t12864 * count, (K + 31) / 32, 2));
-        return launch_tile16(ctx, a, b, out, batch, 2, splits_for(t128 * count, (K + 31) / 32, 2));
+        // a group of separate products (table): no K splits -- their partial planes assume one dense stack of results
+        if (M <= 64) return launch_tile16(ctx, a, b, out, batch, 0, table ? 1 : splits_for(t64 * count, (K + 63) / 64 * 2, 4), table);
+        if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, table ? 1 : splits_for(t12864 * count, (K + 31) / 32, 2), table);
+        return launch_tile16(ctx, a, b, out, batch, 2, table ? 1 : splits_for(t128 * count, (K + 31) / 32, 2), table);
     }
     if (K >= 4096 && t128 < 2 * cus && M >= 128 && N >= 128) {
         // a long K and few tiles (weight gradients): 128 x 128 tiles, K split over workgroups.  Splits shorten every
@@ -1273,6 +1285,38 @@ int matmul_mfma_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tens
     if (K % 8 != 0 || M * N < 64 * 64) return -1;                  // as for a single product
     if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 2) return -1;     // each product fills the chip by itself: one launch each
     return route16(ctx, a, b, out, &batch);
+}
+
+// `count` separate 16-bit products of one shape and one operand layout (only the buffers differ) in one launch: the
+// kernels of the stacks, with the three addresses of every product read from a table in device memory.  -1: not
+// handled here (the caller issues them one by one).
+int matmul_mfma_grouped(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, uint32_t count)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    if (out->dtype != AIXK_BF16 && out->dtype != AIXK_F16) return -1;
+    if (count < 2 || count > 65535 || K % 8 != 0 || M * N < 64 * 64) return -1;
+    if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 2) return -1;       // each product fills the chip by itself
+    for (uint32_t i = 0; i < count; ++i) {
+        if (a[i].dtype != out->dtype || b[i].dtype != out->dtype || out[i].dtype != out->dtype) return -1;
+        if (a[i].shape[0] != M || a[i].shape[1] != K || b[i].shape[0] != K || b[i].shape[1] != N) return -1;
+        if (a[i].strides[0] != a->strides[0] || a[i].strides[1] != a->strides[1] || b[i].strides[0] != b->strides[0] || b[i].strides[1] != b->strides[1]) return -1;
+        if (!aligned16((const char*)a[i].data + a[i].offset * 2) || !aligned16((const char*)b[i].data + b[i].offset * 2) || !aligned16(out[i].data)) return -1;
+    }
+    u64* host = nullptr;
+    const u64* dev = nullptr;
+    AIXK_TRY(table_slot(ctx, (size_t)count * 3 * sizeof(u64), (void**)&host, (const void**)&dev));
+    for (uint32_t i = 0; i < count; ++i) {
+        host[3 * i] = (u64)(uintptr_t)((const char*)a[i].data + a[i].offset * 2);
+        host[3 * i + 1] = (u64)(uintptr_t)((const char*)b[i].data + b[i].offset * 2);
+        host[3 * i + 2] = (u64)(uintptr_t)out[i].data;
+    }
+    AIXK_TRY(table_upload(ctx, host, dev, (size_t)count * 3 * sizeof(u64)));
+    Space<3> batch{};
+    batch.rank = 1;
+    batch.shape[0] = count;
+    aixhip_tensor o2 = out[0];
+    o2.offset = 0; o2.strides[0] = N; o2.strides[1] = 1;
+    return route16(ctx, &a[0], &b[0], &o2, &batch, dev);
 }
 
 int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out)

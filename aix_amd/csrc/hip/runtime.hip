@@ -40,6 +40,43 @@ __global__ void zero_k(uint4* __restrict__ p, uint64_t n16, unsigned char* __res
 using namespace aixk;
 
 namespace aixk {
+// The ring is used in two halves.  Moving on to a half records an event behind the work that used the other half and
+// waits for the event that was recorded when this half was left the last time: by then every copy out of it and every
+// kernel reading its device twin has finished.  The wait only ever blocks a host that is a whole half (hundreds of
+// grouped launches) ahead of the GPU.
+int table_slot(aixk_ctx* ctx, size_t bytes, void** host, const void** dev)
+{
+    bytes = (bytes + 255) & ~(size_t)255;
+    if (!ctx->table_host) {
+        ctx->table_bytes = 1u << 20;
+        AIXK_HIP(hipHostMalloc((void**)&ctx->table_host, ctx->table_bytes, hipHostMallocDefault));
+        AIXK_HIP(hipMalloc((void**)&ctx->table_dev, ctx->table_bytes));
+        AIXK_HIP(hipEventCreateWithFlags(&ctx->table_lap[0], hipEventDisableTiming));
+        AIXK_HIP(hipEventCreateWithFlags(&ctx->table_lap[1], hipEventDisableTiming));
+        AIXK_HIP(hipEventRecord(ctx->table_lap[0], ctx->stream));
+        AIXK_HIP(hipEventRecord(ctx->table_lap[1], ctx->stream));
+    }
+    const size_t half = ctx->table_bytes / 2;
+    if (bytes > half) return fail(AIXK_EINVAL, "table of %zu bytes exceeds the ring", bytes);
+    if (ctx->table_used + bytes > half) {
+        AIXK_HIP(hipEventRecord(ctx->table_lap[ctx->table_half], ctx->stream));      // behind everything that used this half
+        ctx->table_half ^= 1;
+        AIXK_HIP(hipEventSynchronize(ctx->table_lap[ctx->table_half]));              // the half we return to is idle
+        ctx->table_used = 0;
+    }
+    const size_t at = (size_t)ctx->table_half * half + ctx->table_used;
+    ctx->table_used += bytes;
+    *host = ctx->table_host + at;
+    *dev = ctx->table_dev + at;
+    return AIXK_OK;
+}
+
+int table_upload(aixk_ctx* ctx, const void* host, const void* dev, size_t bytes)
+{
+    AIXK_HIP(hipMemcpyAsync(const_cast<void*>(dev), host, bytes, hipMemcpyHostToDevice, ctx->stream));
+    return AIXK_OK;
+}
+
 size_t stream_store_min_bytes()
 {
     static const size_t value = [] {
@@ -99,6 +136,12 @@ int32_t aixk_destroy(aixk_ctx* ctx)
     for (auto& kv : ctx->rtc) {
         if (kv.second->m.module) (void)hipModuleUnload(kv.second->m.module);
         delete kv.second;
+    }
+    if (ctx->table_host) {
+        (void)hipHostFree(ctx->table_host);
+        (void)hipFree(ctx->table_dev);
+        (void)hipEventDestroy(ctx->table_lap[0]);
+        (void)hipEventDestroy(ctx->table_lap[1]);
     }
     (void)hipFree(ctx->scratch);
     (void)hipFree(ctx->counter);

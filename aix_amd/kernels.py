@@ -63,6 +63,7 @@ _SIGNATURES = {
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_matmul": [_P, _T, _T, _T],
     "aixk_matmul_batched": [_P, _T, _T, _T],
+    "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],
     "aixk_rtc_get": [_P, C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_P), C.POINTER(C.c_int32)],
     "aixk_rtc_launch": [_P, _P, C.c_uint32, C.c_uint32, _P, C.c_size_t],
     "aixk_rtc_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],

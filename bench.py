@@ -327,11 +327,13 @@ def main():
             stacked, batch = batch < 0, abs(batch)                 # negative: one matmul on the [batch, m, m] stacks
             ha, hb = operands(dt_name, m, batch)
             r = BenchResult()
+            # small products: enough untimed steps for the device's block pool to reach its steady state (results freed in one
+            # step come back from their cooling period a few steps later; until then every result is a fresh hipMalloc)
             run(lib, "aixbench_matmul", dev.handle, codes[dt_name], m, m, m, layouts[lay] + (4 if stacked else 0), batch, ha.ctypes.data, hb.ctypes.data,
-                steps_mm, 2, C.byref(r), None)
+                steps_mm, 40 if m <= 1024 else 2, C.byref(r), None)
             flops = 2.0 * m * m * m * batch
             what = f"{m}^3" if batch == 1 else f"{batch} x [{m},{m}]x[{m},{m}] " + (
-                "(one matmul call on the [64, 512, 512] stacks: an extension of the interface)" if stacked else "(one matmul call per select(0,i) view)")
+                "(one matmul call on the [64, 512, 512] stacks: an extension of the interface)" if stacked else "(one matmul call per select(0,i) view; the device issues the run of 64 calls as one grouped launch)")
             x3 = dt_name == "f32" and ((m + 127) // 128) ** 2 >= 448          # the route the library takes (matmul_mfma.hip)
             peak = X3_PEAK_TFLOPS if x3 else MFMA_PEAK_TFLOPS[dt_name]
             line = {"workload": f"configs[2] matmul {dt_name} {what} {lay} (f32 accumulation)",

@@ -164,6 +164,11 @@ int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
  * out->data.  Stacks of small 16-bit products run as ONE launch; everything else is issued product by
  * product through the 2-D entry point.  Rank 2 is the 2-D entry point. */
 int32_t aixk_matmul_batched(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+/* `count` separate products -- a[i] . b[i] -> out[i], the descriptors in three arrays -- issued together: what a run of
+ * Device::matmul calls on same-shaped operands asks for (aixCore.hpp:943-976 has no batch dimension, so attention over
+ * (sequence, head) pairs arrives as such a run).  16-bit products of one shape and operand layout that do not fill the
+ * chip one by one run as ONE launch; anything else one by one, with the result of aixk_matmul for every product. */
+int32_t aixk_matmul_grouped(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, uint32_t count);
 
 /* ---- runtime-compiled fused elementwise kernels ------------------------- */
 /* Compile `source` (HIP C++, one extern "C" __global__ named `entry`) for gfx950 with hipRTC or

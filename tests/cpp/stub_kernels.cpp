@@ -94,6 +94,11 @@ int32_t aixk_matmul(aixk_ctx* c, const aixhip_tensor*, const aixhip_tensor*, con
     return AIXK_OK;
 }
 STUB_OP(aixk_matmul_batched, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
+int32_t aixk_matmul_grouped(aixk_ctx* c, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, uint32_t count)
+{
+    for (uint32_t i = 0; i < count; ++i) { const int32_t rc = aixk_matmul(c, a + i, b + i, out + i); if (rc != AIXK_OK) return rc; }
+    return AIXK_OK;
+}
 
 int32_t aixk_rtc_get(aixk_ctx* c, const char*, const char*, const char*, aixk_module** out, int32_t* was_cached)
 {
