@@ -96,6 +96,8 @@ struct DeviceHIP::Extras {
     std::string key;
     std::vector<uint64_t> args;
     gen::Space space;
+    // row reductions are recorded and fused with the operators around them (AIXHIP_FUSE_ROW_REDUCTIONS=0 switches it off)
+    bool fuseRowReductions = [] { const char* e = std::getenv("AIXHIP_FUSE_ROW_REDUCTIONS"); return !(e && e[0] == '0'); }();
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
     struct Group { std::vector<aixhip_tensor> a, b, out; };
     std::array<Group, 4> groups;
@@ -572,6 +574,12 @@ void DeviceHIP::emitSingle(const OpRecord& op)
     if (op.type == OpType::Fill) { check(aixk_fill(m_ctx, op.scalarData.data(), (int)op.scalarDType, &o)); return; }
     if (op.type == OpType::FillMin) { check(aixk_fill_min(m_ctx, &o)); return; }
     toPod(op.input0, &a);
+    if (aixhip::fuse::isRowReduce(op.type)) {               // a recorded row reduction that found no company: the stand-alone kernel
+        uint64_t init = 0;
+        std::memcpy(&init, op.scalarData.data(), dataTypeSize(op.output.dtype));
+        check(aixk_reduce_to_init(m_ctx, op.type == OpType::ReduceTo ? AIXK_SUM : AIXK_MAX, &a, &o, init));
+        return;
+    }
     if (op.type == OpType::Tril || op.type == OpType::Triu) { check(aixk_tri(m_ctx, op.type == OpType::Triu ? 1 : 0, &a, &o, op.triDiagonal)); return; }
     if (const int code = binaryCode(op.type); code >= 0) {
         toPod(op.input1, &b);
@@ -594,6 +602,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     const size_t rank = d.shape.size();
     if (NI + 1 > kMaxOperands || NO > kMaxOperands || rank > aixhip::fuse::kMaxRank)
         throw std::invalid_argument("DeviceHIP: fused kernel with too many operands or dimensions.");
+    if (d.rowLength) { emitRowProgram(d); return; }
 
     // Joint iteration space over the fused shape: dense views get the dense strides of that shape
     // (their own shape may be a different factorisation of the same count), strided views keep
@@ -708,6 +717,45 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     else { items = n; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     uint64_t grid = (items + perBlock - 1) / perBlock;
     grid = std::max<uint64_t>(1, std::min(grid, cap));
+    check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
+}
+
+// A fused kernel that holds row reductions: a wave or a workgroup per row (hipgen.hpp: row programs).
+void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
+{
+    auto& ex = *m_extras;
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
+    gen::RowGeometry geo;
+    if (!gen::rowGeometry(d, &geo)) throw std::logic_error("DeviceHIP: a row program the generator cannot lay out");
+    const void* inPtr[64];
+    void* outPtr[64];
+    size_t storedBytes = 0;
+    for (size_t k = 0; k < NI; ++k) {
+        markTouched(d.inputBuffers[k].data);
+        inPtr[k] = (const char*)d.inputBuffers[k].data + d.inputBuffers[k].offset * dataTypeSize(d.inputBuffers[k].dtype);
+    }
+    for (size_t k = 0; k < NO; ++k) {
+        markTouched(d.outputBuffers[k].data);
+        outPtr[k] = (char*)d.outputBuffers[k].data + d.outputBuffers[k].offset * dataTypeSize(d.outputBuffers[k].dtype);
+        storedBytes += d.outputBuffers[k].size * dataTypeSize(d.outputBuffers[k].dtype);
+    }
+    const bool streamOut = storedBytes >= ex.streamStoreMinBytes;
+    gen::rowSignatureInto(ex.key, d, geo, streamOut);
+    aixk_module* mod = nullptr;
+    auto it = ex.kernels.find(ex.key);
+    if (it != ex.kernels.end()) { mod = it->second; ++ex.hits; }
+    else {
+        int32_t cached = 0;
+        const std::string src = gen::rowSource(d, geo, streamOut);
+        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
+        ex.kernels.emplace(ex.key, mod);
+        ++ex.misses;
+    }
+    gen::packRowArgsInto(ex.args, d, inPtr, outPtr);
+    const uint64_t rows = d.elementCount / d.rowLength;
+    const uint64_t rowsPerBlock = geo.lanes == 64 ? gen::kBlock / 64 : 1;
+    uint64_t grid = (rows + rowsPerBlock - 1) / rowsPerBlock;
+    grid = std::max<uint64_t>(1, std::min<uint64_t>(grid, (uint64_t)m_cus * 64));
     check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
 }
 
@@ -904,12 +952,38 @@ bool DeviceHIP::takeInit(const DeviceTensorParams& src, const DeviceTensorParams
     return aixhip::scalar::encode(v, static_cast<int>(dst.dtype), bits) != 0;
 }
 
+// A sum / maximum over the last dimension of a dense floating-point tensor whose destination's initialisation could be
+// folded in is not run at once but recorded: the planner fuses it with the elementwise operators around it into one
+// kernel that works row by row (max -> sub -> exp -> sum -> div of aixNeuralNetwork.hpp:188-192 reads its operand once;
+// mean, variance and normalisation of a LayerNorm likewise).  The fused kernel adds a row up in the stand-alone row
+// kernel's order, so fusing changes no bits; rows that kernel does not take (shorter than 32 elements) are not recorded.
+// Everything else runs at once as before.
+bool DeviceHIP::recordRowReduction(OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init)
+{
+    if (!m_engine->config().elementwiseFusion || !m_extras->fuseRowReductions) return false;
+    if (src.dtype != DataType::kFloat32 && src.dtype != DataType::kFloat16 && src.dtype != DataType::kBFloat16 && src.dtype != DataType::kFloat64) return false;
+    if (src.shape.empty() || src.shape.size() > AIXK_MAX_RANK || !src.isContiguous || !findBlock(src.data) || src.size == 0) return false;
+    const size_t L = src.shape.back(), esz = dataTypeSize(src.dtype), vec = 16 / esz;
+    if (L < 32 || L % vec != 0 || src.offset % vec != 0 || src.size % L != 0 || dst.size != src.size / L) return false;
+    if (L / vec > 8 * (L >= 2048 ? 256u : 64u)) return false;              // more than 8 vectors per lane: the stand-alone kernel
+    // the destination: the source's shape with the last dim 1 or dropped, dense
+    if (!dst.isContiguous || dst.offset != 0) return false;
+    const size_t lead = src.shape.size() - 1;
+    if (dst.shape.size() != lead && !(dst.shape.size() == lead + 1 && dst.shape.back() == 1)) return false;
+    for (size_t d = 0; d < lead; ++d) if (dst.shape[d] != src.shape[d]) return false;
+    View in(src), out(dst);
+    out.makeDense();
+    m_engine->recordRowReduce(type, in, out, &init, L);
+    return true;
+}
+
 void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::reduceTo() requires matching source and destination data types.");
     requireDevice(dst, "reduceTo");
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
+    if (folded && recordRowReduction(OpType::ReduceTo, src, dst, init)) return;
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
     check(folded ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));
@@ -921,6 +995,7 @@ void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& d
     requireDevice(dst, "maxTo");
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
+    if (folded && recordRowReduction(OpType::MaxTo, src, dst, init)) return;
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "maxTo"); toPod(dst, &pd, "maxTo");
     check(folded ? aixk_reduce_to_init(m_ctx, AIXK_MAX, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_MAX, &ps, &pd));

@@ -157,6 +157,8 @@ private:
     void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void emitSingle(const aixhip::fuse::OpRecord& op);
+    void emitRowProgram(const aixhip::fuse::FusedSubgraphDescriptor& d);
+    bool recordRowReduction(aixhip::fuse::OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init);
     void issueMatmulGroup();                                 // the pending matmul calls as one launch (see matmul())
 
     aixk_ctx* m_ctx{nullptr};

@@ -205,6 +205,35 @@ void PointerSet::erase(const void* p)
     }
 }
 
+// The trailing run of dimensions of `v` that make up one row of `length` elements, or -1: rows are the last dimensions
+// whose extents multiply to `length`.
+static int rowSplit(const View& v, size_t length)
+{
+    size_t run = 1;
+    int d = (int)v.rank;
+    while (d > 0 && run < length) { --d; run *= v.shape[d]; }
+    return run == length ? d : -1;
+}
+
+RowOperand rowOperandKind(const View& v, size_t rows, size_t length)
+{
+    if (!v.data || rows == 0 || length == 0) return RowOperand::None;
+    const size_t vec = 16 / aix::Device::dataTypeSize(v.dtype);
+    if (v.size == rows * length) {
+        if (v.dense) return v.offset % vec == 0 ? RowOperand::Dense : RowOperand::None;
+        const int split = rowSplit(v, length);
+        if (split < 0) return RowOperand::None;
+        // strides of the row dims and of the leading dims: all zero, or those of a dense tensor
+        auto zeros = [&](int from, int to) { for (int d = from; d < to; ++d) if (v.shape[d] > 1 && v.strides[d] != 0) return false; return true; };
+        auto dense = [&](int from, int to) { size_t run = 1; for (int d = to - 1; d >= from; --d) { if (v.shape[d] > 1 && v.strides[d] != run) return false; run *= v.shape[d]; } return true; };
+        if (zeros(split, (int)v.rank) && dense(0, split)) return RowOperand::PerRowBroadcast;            // one value per row, repeated along it
+        if (dense(split, (int)v.rank) && zeros(0, split)) return v.offset % vec == 0 ? RowOperand::RowVector : RowOperand::None;   // one row for all rows
+        return RowOperand::None;
+    }
+    if (v.size == rows && v.dense) return RowOperand::PerRow;
+    return RowOperand::None;
+}
+
 namespace {
 
 bool sameView(const View& a, const View& b)
@@ -257,12 +286,16 @@ struct Group {
     bool open{true};
     bool absorbed{false};                                      // merged into another group
     bool hasScalar{false};
+    size_t rowLen{0};                                          // > 0: a row program over rows of this many elements (it holds a row reduction)
+    bool hasTri{false};                                        // holds a tril / triu (their flat index arithmetic is not available row by row)
+
+    size_t rows() const { return rowLen ? count / rowLen : 0; }
 
     void reset()
     {
         dtype = DataType::kFloat32; count = 0; shape = nullptr; dense = true;
         ops.clear(); defs.clear(); loads.clear();
-        open = true; absorbed = false; hasScalar = false;
+        open = true; absorbed = false; hasScalar = false; rowLen = 0; hasTri = false;
     }
 };
 
@@ -300,6 +333,7 @@ public:
         m_ops = &ops;
         m_live = live;
         m_operands.assign(ops.size(), {});
+        m_perRow.assign(ops.size(), 0);
         m_groupOf.assign(ops.size(), SIZE_MAX);
         m_groupCount = 0;
         m_emits.clear();
@@ -310,6 +344,7 @@ public:
             const auto& op = ops[i];
             if (op.type == OpType::Fill || op.type == OpType::FillMin) placeFill(i);
             else if (isElementwiseOp(op.type) && m_cfg.elementwiseFusion) placeOp(i);
+            else if (isRowReduce(op.type) && op.rowLength && m_cfg.elementwiseFusion && m_cfg.supportsStridedFusion) placeReduce(i);
             else placeSingle(i);
         }
         for (size_t g = 0; g < m_groupCount; ++g) closeGroup(g);
@@ -327,7 +362,7 @@ public:
     size_t fillsAbsorbed() const { return m_fillsAbsorbed; }
 
     // A group of one operator without immediates runs as a plain single operator.
-    bool emitsAsSingle(const Group& g) const { return g.ops.size() == 1 && !g.hasScalar; }
+    bool emitsAsSingle(const Group& g) const { return g.ops.size() == 1 && (!g.hasScalar || isRowReduce(at(g.ops[0]).type)); }
 
     void describe(const Group& g, FusedSubgraphDescriptor& d)
     {
@@ -337,6 +372,7 @@ public:
         d.elementCount = g.count;
         d.shape.assign(g.shape->shape, g.shape->shape + g.shape->rank);
         d.allContiguous = true;
+        d.rowLength = g.rowLen;
         m_position.resize(ops.size());                        // window index -> position in d.ops (this group's ops only)
         m_scalarSlots.clear();                                // fill op -> scalar index
         auto inputSlot = [&](const View& v) {
@@ -380,6 +416,12 @@ public:
                     *idx[k] = nIn + m_position[operand.index];
                 }
                 else if (operand.kind == Operand::kScalar) *sc[k] = scalarIndex(operand.index);
+            }
+            o.perRow = m_perRow[w] != 0;
+            if (isRowReduce(op.type)) {
+                // the value the destination was initialised with (already in the group's element type) as an immediate
+                o.scalarIndex1 = d.scalarData.size() / esz;
+                d.scalarData.insert(d.scalarData.end(), op.scalarData.data(), op.scalarData.data() + esz);
             }
             if (op.type == OpType::Tril || op.type == OpType::Triu) {
                 o.paramIndex = d.opParams.size() / 3;
@@ -504,7 +546,7 @@ private:
                     if (!m_groups[g].open) continue;
                     const size_t def = findDef(m_groups[g], in[k]->data);
                     if (def == SIZE_MAX) continue;
-                    const bool usable = sameElements(defView(def), *in[k]) && compatible(m_groups[g], op, in[k]->dtype);
+                    const bool usable = valueUsable(m_groups[g], def, *in[k], op) && compatible(m_groups[g], op, in[k]->dtype);
                     if (usable && (target == SIZE_MAX || target == g)) {
                         resolved[k] = Operand{Operand::kValue, def};
                         target = g;
@@ -533,6 +575,11 @@ private:
             // hazards on the output buffer
             if (closeGroupsTouching(op.output.data, target, &op.output)) continue;
             if (target != SIZE_MAX && slotsAfterJoin(m_groups[target], op, resolved) > m_cfg.maxBufferSlots) {
+                closeGroup(target);
+                continue;
+            }
+            // a row program takes its memory operands row by row: whole rows, one value per row, or one row for all
+            if (target != SIZE_MAX && m_groups[target].rowLen && !rowOperandsFit(m_groups[target], op, resolved)) {
                 closeGroup(target);
                 continue;
             }
@@ -569,6 +616,112 @@ private:
         if (!redefined) g.defs.push_back(i);
         g.ops.push_back(i);
         m_groupOf[i] = target;
+        if (op.type == OpType::Tril || op.type == OpType::Triu) g.hasTri = true;
+        m_perRow[i] = g.rowLen && op.output.size == g.rows() && op.output.size != g.count;
+    }
+
+    // ---- row reductions ------------------------------------------------------------------------------
+    // sum / maximum over the rows of a dense [rows, length] operand.  It joins the open kernel that holds the operand in
+    // registers, or one that loads it, if that kernel can work row by row (rowsFit); later operators of the kernel may
+    // use the per-row result -- repeated along the row, or in arithmetic on per-row values -- without a pass over memory
+    // in between: max -> sub -> exp -> sum -> div of a softmax is one kernel, one read of the operand.
+    void placeReduce(size_t i)
+    {
+        const auto& op = at(i);
+        const View& in = op.input0;
+        const size_t L = op.rowLength;
+        size_t target = SIZE_MAX;
+        Operand resolved{};
+        for (;;) {
+            bool closedSomething = false;
+            target = SIZE_MAX;
+            resolved = Operand{};
+            if (findFill(in.data)) materialise(in.data);
+            resolved.kind = Operand::kMemory;
+            for (size_t g = 0; g < m_groupCount; ++g) {
+                if (!m_groups[g].open) continue;
+                const size_t def = findDef(m_groups[g], in.data);
+                if (def == SIZE_MAX) continue;
+                const Group& grp = m_groups[g];
+                const bool usable = target == SIZE_MAX && !m_perRow[def] && at(def).type != OpType::Cast && sameElements(defView(def), in) &&
+                                    grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L);
+                if (usable) { resolved = Operand{Operand::kValue, def}; target = g; }
+                else { closeGroup(g); closedSomething = true; }
+            }
+            if (closedSomething) continue;
+            if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
+                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
+                    const Group& grp = m_groups[g];
+                    if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
+                }
+            }
+            if (closeGroupsTouching(op.output.data, target, &op.output)) continue;
+            if (target != SIZE_MAX) {
+                const Group& grp = m_groups[target];
+                size_t slots = grp.loads.size() + grp.defs.size() + 1;
+                if (resolved.kind == Operand::kMemory && !loads(grp, in)) ++slots;
+                if (slots > m_cfg.maxBufferSlots) { closeGroup(target); continue; }
+            }
+            break;
+        }
+        if (findFill(op.output.data)) eraseFill(op.output.data);     // the reduction defines every element of its destination
+        if (target == SIZE_MAX) {
+            target = newGroup();
+            Group& fresh = m_groups[target];
+            fresh.dtype = in.dtype;
+            fresh.count = in.size;
+            fresh.shape = &op.input0;
+        }
+        Group& g = m_groups[target];
+        g.rowLen = L;
+        m_operands[i][0] = resolved;
+        if (resolved.kind == Operand::kMemory && !loads(g, in)) g.loads.push_back(ViewRef{(uint32_t)i, 0});
+        g.defs.push_back(i);
+        g.ops.push_back(i);
+        m_groupOf[i] = target;
+        m_perRow[i] = 1;
+    }
+
+    // Can the group work on rows of `length` elements?  It does already, or everything it loads and stores fits rows.
+    bool rowsFit(const Group& g, size_t length) const
+    {
+        if (g.rowLen) return g.rowLen == length;
+        if (g.hasTri || length == 0 || g.count % length != 0) return false;
+        const size_t rows = g.count / length;
+        for (const ViewRef& r : g.loads) {
+            const RowOperand k = rowOperandKind(view(r), rows, length);
+            if (k != RowOperand::Dense && k != RowOperand::PerRowBroadcast && k != RowOperand::RowVector) return false;
+        }
+        for (size_t def : g.defs) if (rowOperandKind(defView(def), rows, length) != RowOperand::Dense) return false;
+        return true;
+    }
+
+    // The memory operands and the result of `op` as a member of row program `g`.
+    bool rowOperandsFit(const Group& g, const OpRecord& op, const Operand* resolved) const
+    {
+        const size_t rows = g.rows();
+        const bool per = op.output.size == rows && op.output.size != g.count;
+        if (op.type == OpType::Tril || op.type == OpType::Triu) return false;
+        if (rowOperandKind(op.output, rows, g.rowLen) != (per ? RowOperand::PerRow : RowOperand::Dense)) return false;
+        const View* in[2] = {&op.input0, op.hasInput1 ? &op.input1 : nullptr};
+        for (int k = 0; k < 2; ++k) {
+            if (!in[k] || !in[k]->data || resolved[k].kind != Operand::kMemory) continue;
+            const RowOperand kind = rowOperandKind(*in[k], rows, g.rowLen);
+            if (per ? kind != RowOperand::PerRow : (kind != RowOperand::Dense && kind != RowOperand::PerRowBroadcast && kind != RowOperand::RowVector)) return false;
+        }
+        return true;
+    }
+
+    // May `op` take the value that operator `def` of group `g` defines, seeing it through view `v`?
+    bool valueUsable(const Group& g, size_t def, const View& v, const OpRecord& op) const
+    {
+        if (!m_perRow[def]) return sameElements(defView(def), v);
+        // a per-row value: to an operator on per-row values it is the same elements; to an operator on whole rows it is the
+        // destination seen with the row dimension(s) broadcast
+        if (op.output.size == g.rows() && op.output.size != g.count) return sameElements(defView(def), v);
+        const View& d = defView(def);
+        return op.output.size == g.count && v.data == d.data && v.dtype == d.dtype && v.offset == d.offset &&
+               rowOperandKind(v, g.rows(), g.rowLen) == RowOperand::PerRowBroadcast;
     }
 
     // The latest operator of the group that defines a view of `buffer`, SIZE_MAX if none does.
@@ -597,6 +750,12 @@ private:
 
     bool compatible(const Group& g, const OpRecord& op, DataType type) const
     {
+        if (g.rowLen) {
+            // a row program takes operators on whole rows and operators on per-row values; what their memory operands
+            // look like is checked once the operands are resolved (rowOperandsFit)
+            if (g.dtype != type || op.type == OpType::Tril || op.type == OpType::Triu) return false;
+            return op.output.size == g.count || op.output.size == g.rows();
+        }
         if (g.dtype != type || g.count != op.output.size) return false;
         if (g.shape->sameShape(op.output)) return true;
         return g.dense || denseOperands(op);
@@ -609,6 +768,7 @@ private:
 
     bool mergeable(const Group& a, const Group& b) const
     {
+        if (a.rowLen || b.rowLen) return false;                // row programs grow operator by operator only
         if (a.dtype != b.dtype || a.count != b.count) return false;
         if (!a.shape->sameShape(*b.shape) && !a.dense && !b.dense) return false;
         size_t count = a.loads.size();
@@ -629,6 +789,7 @@ private:
         if (!a.shape->sameShape(*b.shape) && !b.dense) a.shape = b.shape;        // a is all dense then: it adopts the shape b's strided views need
         a.dense = a.dense && b.dense;
         a.hasScalar = a.hasScalar || b.hasScalar;
+        a.hasTri = a.hasTri || b.hasTri;
         for (size_t w : b.ops) m_groupOf[w] = into;
         b.ops.clear(); b.defs.clear(); b.loads.clear();
         b.open = false;                                     // absorbed: never emitted on its own
@@ -718,6 +879,7 @@ private:
     Liveness m_live;
     std::vector<std::array<Operand, 2>> m_operands;
     std::vector<size_t> m_groupOf;
+    std::vector<uint8_t> m_perRow;           // the operator yields one value per row of its (row program) group
     std::vector<Group> m_groups;             // [0, m_groupCount) belong to the current window
     size_t m_groupCount{0};
     std::vector<Emit> m_emits;
@@ -781,6 +943,17 @@ void FuseEngine::recordTri(OpType type, const View& input, const View& output, i
     OpRecord& r = append(type);
     r.input0 = input; r.output = output;
     r.triRows = input.shape[input.rank - 2]; r.triCols = input.shape[input.rank - 1]; r.triDiagonal = diagonal;
+    maybeFlush();
+}
+
+void FuseEngine::recordRowReduce(OpType type, const View& input, const View& output, const void* init, size_t rowLength)
+{
+    if (!isRowReduce(type) || rowLength == 0 || input.size % rowLength != 0 || output.size != input.size / rowLength || input.dtype != output.dtype)
+        throw std::invalid_argument("recordRowReduce: a sum / maximum over the rows of a [rows, length] operand into one value per row");
+    OpRecord& r = append(type);
+    r.input0 = input; r.output = output; r.rowLength = rowLength;
+    r.scalarDType = output.dtype;
+    std::memcpy(r.scalarData.data(), init, aix::Device::dataTypeSize(output.dtype));
     maybeFlush();
 }
 

@@ -36,6 +36,8 @@ enum class OpType {
 };
 
 bool isElementwiseOp(OpType t);
+// ReduceTo / MaxTo recorded as row reductions (FuseEngine::recordRowReduce): sum / maximum over the last, dense dimension
+inline bool isRowReduce(OpType t) { return t == OpType::ReduceTo || t == OpType::MaxTo; }
 const char* opName(OpType t);
 
 struct FuseConfig {
@@ -94,7 +96,16 @@ struct OpRecord {
     // Tril / Triu recorded as elementwise operators: the extents of the last two dims and the diagonal
     uint64_t triRows{0}, triCols{0};
     int64_t triDiagonal{0};
+    // ReduceTo / MaxTo recorded as a row reduction: elements per row of input0 (its last dimension); scalarData then holds
+    // the value the destination was initialised with, in the destination's element type (the folded fill)
+    size_t rowLength{0};
 };
+
+// How a view takes part in a kernel that works row by row on [rows, length] data (a "row program"): element for element,
+// one value per row repeated along the row, one row repeated for every row, one value per row (operand of a per-row
+// operator), or not at all.
+enum class RowOperand { Dense, PerRowBroadcast, RowVector, PerRow, None };
+RowOperand rowOperandKind(const View& v, size_t rows, size_t length);
 
 // One fused kernel: ops in execution order.  An operand index below inputBuffers.size() names an
 // external buffer, an index at or above it names the result of ops[index - inputBuffers.size()];
@@ -109,6 +120,7 @@ struct FusedSubgraphDescriptor {
         size_t scalarIndex0 = SIZE_MAX;
         size_t scalarIndex1 = SIZE_MAX;
         size_t paramIndex   = SIZE_MAX;    // Tril / Triu: its (rows, cols, diagonal) triple in opParams
+        bool   perRow       = false;       // row programs: the operator yields one value per row (a reduction, or arithmetic on such values)
     };
     std::vector<Op> ops;
     std::vector<uint64_t> opParams;        // run-time integers of index-dependent operators, three per Tril / Triu
@@ -119,6 +131,10 @@ struct FusedSubgraphDescriptor {
     bool     allContiguous{true};          // every loaded / stored view is dense
     size_t   elementCount{0};
     aix::Shape shape;                      // iteration shape (outputs are dense over it)
+    // Row program: the kernel handles rows of `rowLength` elements (elementCount / rowLength of them) and may hold
+    // ReduceTo / MaxTo operators -- sum / maximum over a row, combined with the immediate scalarIndex1 the destination was
+    // initialised with -- whose per-row results later operators of the same kernel use.  0: a plain elementwise kernel.
+    size_t   rowLength{0};
 };
 // The descriptor handed to emitFused is reused from kernel to kernel: a callback that wants to keep
 // it copies it.
@@ -181,6 +197,9 @@ public:
     void recordFillMin(const View& output);
     // tril / triu of `input` (its last two dims) as an elementwise operator: the kept part passes through, the rest is 0
     void recordTri(OpType type, const View& input, const View& output, int64_t diagonal);
+    // ReduceTo / MaxTo over the last dimension (`rowLength` elements, dense) of `input` into the dense `output`, whose
+    // pending initialisation the caller has taken out of the window: `init` is that value in output's element type.
+    void recordRowReduce(OpType type, const View& input, const View& output, const void* init, size_t rowLength);
     void flush();
 
     const FuseConfig& config() const { return m_config; }

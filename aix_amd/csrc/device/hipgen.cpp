@@ -6,6 +6,7 @@
 #include <cstring>
 #include <sstream>
 #include <stdexcept>
+#include <vector>
 
 namespace aixhip::gen {
 
@@ -275,6 +276,200 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
     o << "    }\n}\n";
     return o.str();
+}
+
+// ---- row programs ------------------------------------------------------------------------------------------------------
+bool rowGeometry(const FusedSubgraphDescriptor& d, RowGeometry* g)
+{
+    if (!d.rowLength || d.elementCount % d.rowLength) return false;
+    const size_t vec = 16 / aix::Device::dataTypeSize(d.dtype);
+    if (d.rowLength % vec) return false;
+    g->lanes = d.rowLength >= 2048 ? 256 : 64;                     // the stand-alone reduction's choice (reduce.hip), for identical sums
+    const size_t nvec = d.rowLength / vec;
+    g->vectors = (int)((nvec + (size_t)g->lanes - 1) / (size_t)g->lanes);
+    return g->vectors >= 1 && g->vectors <= 8;
+}
+
+namespace {
+
+char kindLetter(fuse::RowOperand k)
+{
+    switch (k) {
+        case fuse::RowOperand::Dense: return 'd';
+        case fuse::RowOperand::PerRowBroadcast: return 'b';
+        case fuse::RowOperand::RowVector: return 'r';
+        case fuse::RowOperand::PerRow: return 'p';
+        default: return '?';
+    }
+}
+
+fuse::RowOperand inputKind(const FusedSubgraphDescriptor& d, size_t k)
+{
+    const fuse::RowOperand kind = fuse::rowOperandKind(d.inputBuffers[k], d.elementCount / d.rowLength, d.rowLength);
+    if (kind == fuse::RowOperand::None) throw std::invalid_argument("row program: an operand that is neither rows, nor one value per row, nor one row");
+    return kind;
+}
+
+} // namespace
+
+void rowSignatureInto(std::string& s, const FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut)
+{
+    s.clear();
+    s += shortType(d.dtype);
+    s += "|row"; appendNumber(s, (uint64_t)g.lanes); s += 'x'; appendNumber(s, (uint64_t)g.vectors);
+    if (streamOut) s += "|nt";
+    s += "|i"; appendNumber(s, d.inputBuffers.size());
+    s += 'o';  appendNumber(s, d.outputBuffers.size());
+    s += 's';  appendNumber(s, scalarCount(d));
+    s += '|';
+    for (size_t k = 0; k < d.inputBuffers.size(); ++k) s += kindLetter(inputKind(d, k));
+    for (size_t k = 0; k < d.inputBuffers.size(); ++k)
+        if (d.inputBuffers[k].dtype != d.dtype) { s += "|x"; appendNumber(s, k); s += ':'; s += shortType(d.inputBuffers[k].dtype); }
+    for (size_t k = 0; k < d.outputBuffers.size(); ++k)
+        if (d.outputBuffers[k].dtype != d.dtype) { s += "|y"; appendNumber(s, k); s += ':'; s += shortType(d.outputBuffers[k].dtype); }
+    for (const auto& op : d.ops) {
+        s += '|'; s += fuse::opName(op.type); if (op.perRow) s += '\''; s += '(';
+        appendOperand(s, d, op.inputIndex0, op.scalarIndex0);
+        if (isBinary(op.type) || fuse::isRowReduce(op.type)) { s += ','; appendOperand(s, d, op.inputIndex1, op.scalarIndex1); }
+        s += ')';
+        if (op.outputIndex != SIZE_MAX) { s += ">o"; appendNumber(s, op.outputIndex); }
+    }
+}
+
+std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut)
+{
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
+    if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
+    if (triCount(d)) throw std::invalid_argument("row program: tril / triu cannot be part of it");
+    const size_t esz = aix::Device::dataTypeSize(d.dtype);
+    const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
+    std::vector<fuse::RowOperand> kinds(NI);
+    for (size_t k = 0; k < NI; ++k) kinds[k] = inputKind(d, k);
+    std::string sig;
+    rowSignatureInto(sig, d, g, streamOut);
+    std::ostringstream o;
+    o << "#include \"aix_device.h\"\nusing namespace aixd;\n// " << sig << "\n"
+      << "#define AIX_NT " << (streamOut ? "true" : "false") << "\n"
+      << "typedef " << typeName(d.dtype) << " T;\ntypedef traits<T>::W W;\ntypedef " << wordName(esz) << " word_t;\n"
+      << "#define VEC (vec16<T>::n)\n#define NV " << g.vectors << "\n#define G " << g.lanes << "\n";
+    for (size_t k = 0; k < NI; ++k) o << "typedef " << typeName(d.inputBuffers[k].dtype) << " I" << k << ";\n";
+    for (size_t k = 0; k < NO; ++k) o << "typedef " << typeName(d.outputBuffers[k].dtype) << " O" << k << ";\n";
+    auto to_t = [&](size_t k, const std::string& e) { return d.inputBuffers[k].dtype == d.dtype ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
+    auto from_t = [&](size_t k, const std::string& e) { return d.outputBuffers[k].dtype == d.dtype ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
+    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 rows;\n    u64 len;\n};\n\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void aix_fused(Args a)\n{\n"
+      << "    __shared__ W red[4];\n    (void)red;\n"
+      << "    T s[" << AS << "];\n";
+    for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
+    if (NS == 0) o << "    s[0] = zero<T>();\n";
+    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = (const I" << k << "*)a.in[" << k << "];\n";
+    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = (O" << k << "*)a.out[" << k << "];\n";
+    o << "    const u32 lane = threadIdx.x % G;\n"
+      << "    const u64 nvec = a.len / VEC;\n"
+      << "    const W lowestW = (W)(-__builtin_huge_val());\n    (void)lowestW;\n";
+    if (g.lanes == 64) o << "    for (u64 row = (u64)blockIdx.x * " << kBlock / 64 << " + threadIdx.x / 64; row < a.rows; row += (u64)gridDim.x * " << kBlock / 64 << ") {\n";
+    else o << "    for (u64 row = blockIdx.x; row < a.rows; row += gridDim.x) {\n";
+    // operands: whole rows (their own or the one shared row) as vectors, per-row values as scalars
+    for (size_t k = 0; k < NI; ++k) {
+        if (kinds[k] == fuse::RowOperand::Dense || kinds[k] == fuse::RowOperand::RowVector) {
+            const char* base = kinds[k] == fuse::RowOperand::Dense ? " + row * a.len" : "";
+            o << "        T x" << k << "[NV][VEC];\n#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n"
+              << "            const u64 v = lane + (u64)j * G;\n"
+              << "            vec<I" << k << ", VEC> r;\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r.v[e] = zero<I" << k << ">();\n"
+              << "            if (v < nvec) r = ((const vec<I" << k << ", VEC>*)(in" << k << base << "))[v];\n"
+              << "#pragma unroll\n            for (int e = 0; e < VEC; ++e) x" << k << "[j][e] = " << to_t(k, "r.v[e]") << ";\n        }\n";
+        } else {
+            o << "        const T q" << k << " = " << to_t(k, "in" + std::to_string(k) + "[row]") << ";\n";
+        }
+    }
+    auto fullOperand = [&](size_t tensorIndex, size_t scalarIndex) -> std::string {
+        if (tensorIndex != SIZE_MAX) {
+            if (tensorIndex < NI) {
+                if (kinds[tensorIndex] == fuse::RowOperand::PerRowBroadcast) return "q" + std::to_string(tensorIndex);
+                if (kinds[tensorIndex] == fuse::RowOperand::PerRow) throw std::invalid_argument("row program: a per-row operand of an operator on whole rows");
+                return "x" + std::to_string(tensorIndex) + "[j][e]";
+            }
+            const size_t m = tensorIndex - NI;
+            return d.ops[m].perRow ? "p" + std::to_string(m) : "v" + std::to_string(m) + "[j][e]";
+        }
+        if (scalarIndex != SIZE_MAX) return "s[" + std::to_string(scalarIndex) + "]";
+        throw std::invalid_argument("fused operator without an operand");
+    };
+    auto rowOperand = [&](size_t tensorIndex, size_t scalarIndex) -> std::string {
+        if (tensorIndex != SIZE_MAX) {
+            if (tensorIndex < NI) {
+                if (kinds[tensorIndex] != fuse::RowOperand::PerRow) throw std::invalid_argument("row program: a row operand of an operator on per-row values");
+                return "q" + std::to_string(tensorIndex);
+            }
+            const size_t m = tensorIndex - NI;
+            if (!d.ops[m].perRow) throw std::invalid_argument("row program: a row value used by an operator on per-row values");
+            return "p" + std::to_string(m);
+        }
+        if (scalarIndex != SIZE_MAX) return "s[" + std::to_string(scalarIndex) + "]";
+        throw std::invalid_argument("fused operator without an operand");
+    };
+    for (size_t k = 0; k < d.ops.size(); ++k) {
+        const auto& op = d.ops[k];
+        if (fuse::isRowReduce(op.type)) {
+            const bool sum = op.type == OpType::ReduceTo;
+            const std::string init = "s[" + std::to_string(op.scalarIndex1) + "]";
+            o << "        W a" << k << " = " << (sum ? "(W)0" : "lowestW") << ";\n#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n"
+              << "            if (lane + (u64)j * G < nvec) {\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) { const W w = up(" << fullOperand(op.inputIndex0, op.scalarIndex0) << "); ";
+            if (sum) o << "a" << k << " += w; }\n"; else o << "if (w > a" << k << ") a" << k << " = w; }\n";
+            o << "            }\n        }\n"
+              << "        a" << k << " = " << (sum ? "row_sum" : "row_max") << "<G>(a" << k << ", red);\n";
+            // combined with the value the destination was initialised with, as the stand-alone kernels land their results
+            if (sum) o << "        const T p" << k << " = down<T>(up(" << init << ") + a" << k << ");\n";
+            else o << "        const T p" << k << " = a" << k << " > up(" << init << ") ? down<T>(a" << k << ") : " << init << ";\n";
+            if (op.outputIndex != SIZE_MAX) o << "        if (lane == 0) out" << op.outputIndex << "[row] = " << from_t(op.outputIndex, "p" + std::to_string(k)) << ";\n";
+            continue;
+        }
+        if (op.perRow) {
+            o << "        const T p" << k << " = ";
+            if (op.type == OpType::Cast) o << rowOperand(op.inputIndex0, op.scalarIndex0);
+            else {
+                o << fnName(op.type) << "(" << rowOperand(op.inputIndex0, op.scalarIndex0);
+                if (isBinary(op.type)) o << ", " << rowOperand(op.inputIndex1, op.scalarIndex1);
+                o << ")";
+            }
+            o << ";\n";
+            if (op.outputIndex != SIZE_MAX) o << "        if (lane == 0) out" << op.outputIndex << "[row] = " << from_t(op.outputIndex, "p" + std::to_string(k)) << ";\n";
+            continue;
+        }
+        o << "        T v" << k << "[NV][VEC];\n#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) v" << k << "[j][e] = ";
+        if (op.type == OpType::Cast) o << fullOperand(op.inputIndex0, op.scalarIndex0);
+        else {
+            o << fnName(op.type) << "(" << fullOperand(op.inputIndex0, op.scalarIndex0);
+            if (isBinary(op.type)) o << ", " << fullOperand(op.inputIndex1, op.scalarIndex1);
+            o << ")";
+        }
+        o << ";\n        }\n";
+        if (op.outputIndex != SIZE_MAX) {
+            const size_t q = op.outputIndex;
+            o << "#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n            const u64 v = lane + (u64)j * G;\n            if (v < nvec) {\n"
+              << "                vec<O" << q << ", VEC> w;\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) w.v[e] = " << from_t(q, "v" + std::to_string(k) + "[j][e]") << ";\n"
+              << "                store_sel<AIX_NT>((vec<O" << q << ", VEC>*)(out" << q << " + row * a.len) + v, w);\n            }\n        }\n";
+        }
+    }
+    o << "    }\n}\n";
+    return o.str();
+}
+
+void packRowArgsInto(std::vector<uint64_t>& a, const FusedSubgraphDescriptor& d, const void* const* inputs, void* const* outputs)
+{
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
+    const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
+    const size_t esz = aix::Device::dataTypeSize(d.dtype);
+    a.clear();
+    for (size_t k = 0; k < AI; ++k) a.push_back(k < NI ? (uint64_t)(uintptr_t)inputs[k] : 0);
+    for (size_t k = 0; k < NO; ++k) a.push_back((uint64_t)(uintptr_t)outputs[k]);
+    for (size_t k = 0; k < AS; ++k) {
+        uint64_t bits = 0;
+        if (k < NS) std::memcpy(&bits, d.scalarData.data() + k * esz, esz);
+        a.push_back(bits);
+    }
+    a.push_back(d.elementCount / d.rowLength);
+    a.push_back(d.rowLength);
 }
 
 void packArgsInto(std::vector<uint64_t>& a, const FusedSubgraphDescriptor& d, Shape shape, const void* const* inputs,

@@ -33,6 +33,21 @@ void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Sha
 // Source of `extern "C" __global__ void aix_fused(Args)`.
 std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false);
 
+// ---- row programs (descriptor.rowLength > 0) ------------------------------------------------------------------------
+// A kernel that works row by row on [rows, rowLength] data: a wave (rows shorter than 2048 elements) or a workgroup per
+// row, the row's vectors in registers, sums / maxima over the row by shuffles (and LDS across the four waves) in the
+// order of the stand-alone reduction kernels, so that fused and unfused results are the same bits.
+struct RowGeometry {
+    int lanes{64};          // lanes per row: 64 or 256
+    int vectors{1};         // 16-byte vectors per lane and row (compile-time; the tail of a row is masked)
+};
+// false: the descriptor cannot run as a row program (row too long, not a whole number of vectors)
+bool rowGeometry(const fuse::FusedSubgraphDescriptor& d, RowGeometry* g);
+void rowSignatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut);
+std::string rowSource(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut);
+// Args of a row program: in[], out[], immediates, rows, rowLength
+void packRowArgsInto(std::vector<uint64_t>& a, const fuse::FusedSubgraphDescriptor& d, const void* const* inputs, void* const* outputs);
+
 inline const char* entryName() { return "aix_fused"; }
 
 constexpr int kMaxDims = 8;

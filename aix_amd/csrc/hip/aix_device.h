@@ -308,6 +308,38 @@ template <class T, int N> __device__ __forceinline__ vec<T, N> row_vec_fix(vec<T
     return v;
 }
 
+// Sum / maximum of one value per lane over the LANES (64: a wave, 256: the workgroup's four waves through `red`) lanes
+// that share a row, returned to every one of them.  The order is that of the stand-alone reduction kernels -- shuffle
+// tree down to lane 0 of a wave, then wave 0's result combined with waves 1, 2, 3 in turn -- so that a sum formed
+// inside a fused kernel has the bits of the same sum formed by itself.
+template <int LANES, class W> __device__ __forceinline__ W row_sum(W v, W* red)
+{
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) v += __shfl_down(v, d, 64);
+    if constexpr (LANES == 64) return __shfl(v, 0, 64);
+    else {
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        return ((red[0] + red[1]) + red[2]) + red[3];
+    }
+}
+template <int LANES, class W> __device__ __forceinline__ W row_max(W v, W* red)
+{
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) { const W o = __shfl_down(v, d, 64); v = o > v ? o : v; }
+    if constexpr (LANES == 64) return __shfl(v, 0, 64);
+    else {
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        W r = red[0];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) r = red[w] > r ? red[w] : r;
+        return r;
+    }
+}
+
 // Stores of values that this kernel and its neighbours will not read again.  A non-temporal store does not allocate its
 // line in the caches on the way out: on results of tens of megabytes that is worth 15 % of a copy-shaped kernel's time
 // (negate over 256 MiB: 87 -> 74 us; the transpose copy: 93 -> 79 us); small results are stored normally so that the

@@ -13,6 +13,7 @@
 #include <hip/hiprtc.h>
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <iostream>
@@ -682,6 +683,161 @@ static void testTrilJoinsItsNeighbours()
     if (flat.fused.size() == 1) { CHECK(flat.fused[0].allContiguous); CHECK(compiles(flat.fused[0], gen::Shape::Flat)); }
 }
 
+// Compiles one generated row program for gfx950.
+static bool compilesRow(const FusedSubgraphDescriptor& d)
+{
+    gen::RowGeometry geo;
+    if (!gen::rowGeometry(d, &geo)) { std::printf("no row geometry\n"); return false; }
+    const std::string src = gen::rowSource(d, geo, false);
+    if (std::getenv("AIX_PRINT_ROW_SOURCES")) std::printf("%s\n", src.c_str());
+    hiprtcProgram prog;
+    const char* names[] = {"aix_device.h"};
+    const char* texts[] = {g_prelude.c_str()};
+    if (hiprtcCreateProgram(&prog, src.c_str(), "r.hip", 1, texts, names) != HIPRTC_SUCCESS) return false;
+    const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off"};
+    const hiprtcResult r = hiprtcCompileProgram(prog, 4, opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0; hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, 0); if (n) hiprtcGetProgramLog(prog, &log[0]);
+        std::printf("---- hipRTC log ----\n%s\n---- source ----\n%s\n", log.c_str(), src.c_str());
+    }
+    hiprtcDestroyProgram(&prog);
+    return r == HIPRTC_SUCCESS;
+}
+
+static void recordSoftmax(FuseEngine& e, DataType dt, size_t rows, size_t L, uintptr_t base = 0)
+{
+    // (x - x.max(-1, true)).exp() / that.sum(-1, true)   (aixNeuralNetwork.hpp:188-192)
+    auto id = [&](uintptr_t k) { return base + k; };
+    auto x = T(id(1), {rows, L}, dt), m = T(id(2), {rows, 1}, dt), d = T(id(3), {rows, L}, dt), ex = T(id(4), {rows, L}, dt);
+    auto s = T(id(5), {rows, 1}, dt), y = T(id(6), {rows, L}, dt);
+    auto mB = T(id(2), {rows, L}, dt, {1, 0}), sB = T(id(5), {rows, L}, dt, {1, 0});
+    for (uintptr_t k = 1; k <= 6; ++k) e.retainBuffer(reinterpret_cast<void*>(id(k) * 0x10000));
+    uint8_t lowest[8] = {}, zero[8] = {};
+    lowestScalarInto(dt, lowest);
+    e.recordRowReduce(OpType::MaxTo, View(x), View(m), lowest, L);
+    e.record(OpType::Sub, View(x), View(mB), View(d));
+    e.record(OpType::Exp, View(d), View(ex));
+    e.recordRowReduce(OpType::ReduceTo, View(ex), View(s), zero, L);
+    e.record(OpType::Div, View(ex), View(sB), View(y));
+    for (uintptr_t k : {2, 3, 4, 5}) e.releaseBuffer(reinterpret_cast<void*>(id(k) * 0x10000));
+}
+
+static void testSoftmaxBecomesOneRowProgram()
+{
+    for (DataType dt : {DataType::kFloat32, DataType::kBFloat16, DataType::kFloat16, DataType::kFloat64}) {
+        for (size_t L : {64, 1024, 4096}) {
+            Capture cap;
+            FuseEngine e(config(), cap.callbacks());
+            recordSoftmax(e, dt, 512, L);
+            e.flush();
+            CHECK(cap.fused.size() == 1 && cap.singles.empty());
+            if (cap.fused.size() != 1) continue;
+            const auto& d = cap.fused[0];
+            CHECK(d.rowLength == L && d.elementCount == 512 * L && d.dtype == dt);
+            CHECK(d.ops.size() == 5 && d.inputBuffers.size() == 1 && d.outputBuffers.size() == 1);
+            CHECK(d.ops[0].type == OpType::MaxTo && d.ops[0].perRow && d.ops[0].outputIndex == SIZE_MAX && d.ops[0].scalarIndex1 != SIZE_MAX);
+            CHECK(d.ops[1].type == OpType::Sub && !d.ops[1].perRow && d.ops[1].inputIndex1 == 1 + 0);       // the maximum from registers
+            CHECK(d.ops[3].type == OpType::ReduceTo && d.ops[3].perRow);
+            CHECK(d.ops[4].type == OpType::Div && d.ops[4].outputIndex == 0);
+            gen::RowGeometry geo;
+            CHECK(gen::rowGeometry(d, &geo) && geo.lanes == (L >= 2048 ? 256 : 64));
+            CHECK(compilesRow(d));
+            std::vector<uint64_t> args;
+            const void* in[1] = {nullptr}; void* out[1] = {nullptr};
+            gen::packRowArgsInto(args, d, in, out);
+            CHECK(args.size() == 1 + 1 + d.scalarData.size() / aix::Device::dataTypeSize(dt) + 2);
+        }
+    }
+    // the per-row results stay visible when somebody still holds them: they are stored by the same kernel
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto x = T(1, {128, 256}), m = T(2, {128, 1}), y = T(3, {128, 256});
+        auto mB = T(2, {128, 256}, DataType::kFloat32, {1, 0});
+        for (uintptr_t k : {1, 2, 3}) e.retainBuffer(reinterpret_cast<void*>(k * 0x10000));
+        uint8_t lowest[8]; lowestScalarInto(DataType::kFloat32, lowest);
+        e.recordRowReduce(OpType::MaxTo, View(x), View(m), lowest, 256);
+        e.record(OpType::Sub, View(x), View(mB), View(y));
+        e.flush();
+        CHECK(cap.fused.size() == 1 && cap.singles.empty());
+        if (cap.fused.size() == 1) {
+            CHECK(cap.fused[0].outputBuffers.size() == 2 && cap.fused[0].ops[0].outputIndex != SIZE_MAX);
+            CHECK(compilesRow(cap.fused[0]));
+        }
+    }
+    // a reduction with no elementwise company runs as the stand-alone operator, its initial value travelling along
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto x = T(1, {128, 256}), m = T(2, {128, 1});
+        for (uintptr_t k : {1, 2}) e.retainBuffer(reinterpret_cast<void*>(k * 0x10000));
+        const float seven = 7.0f;
+        e.recordRowReduce(OpType::ReduceTo, View(x), View(m), &seven, 256);
+        e.flush();
+        CHECK(cap.fused.empty() && cap.singles.size() == 1 && cap.singles[0].type == OpType::ReduceTo && cap.singles[0].rowLength == 256);
+        float got; std::memcpy(&got, cap.singles[0].scalarData.data(), 4);
+        CHECK(got == 7.0f);
+    }
+    // with fusion off every record replays alone and in order
+    {
+        Capture cap;
+        FuseEngine e(config(false), cap.callbacks());
+        recordSoftmax(e, DataType::kFloat32, 64, 128);
+        e.flush();
+        CHECK(cap.fused.empty() && cap.singles.size() == 5);
+        CHECK(cap.order == (std::vector<std::string>{"S:MaxTo", "S:Sub", "S:Exp", "S:ReduceTo", "S:Div"}));
+    }
+    // two softmaxes of different row lengths in one window: two kernels
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        recordSoftmax(e, DataType::kFloat32, 64, 128);
+        recordSoftmax(e, DataType::kFloat32, 32, 256, 100);
+        e.flush();
+        CHECK(cap.fused.size() == 2 && cap.singles.empty());
+        if (cap.fused.size() == 2) CHECK(cap.fused[0].rowLength == 128 && cap.fused[1].rowLength == 256);
+    }
+}
+
+static void testLayerNormPiecesShareOneRowProgram()
+{
+    // mean = sum(x)/L; d = x - mean; var = sum(d*d)/L; y = d / sqrt(var + eps) * gamma + beta
+    const size_t rows = 256, L = 768;
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto full = [&](uintptr_t k) { return T(k, {rows, L}); };
+    auto col = [&](uintptr_t k) { return T(k, {rows, 1}); };
+    auto colB = [&](uintptr_t k) { return T(k, {rows, L}, DataType::kFloat32, {1, 0}); };
+    auto rowB = [&](uintptr_t k) { return T(k, {rows, L}, DataType::kFloat32, {0, 1}); };
+    auto scalarB = [&](uintptr_t k) { return T(k, {rows, 1}, DataType::kFloat32, {0, 0}); };
+    for (uintptr_t k = 1; k <= 20; ++k) e.retainBuffer(reinterpret_cast<void*>(k * 0x10000));
+    const float zero = 0.0f, len = (float)L, eps = 1e-5f;
+    e.recordRowReduce(OpType::ReduceTo, View(full(1)), View(col(2)), &zero, L);
+    e.recordFill(&len, DataType::kFloat32, View(T(3, {})));
+    e.record(OpType::Div, View(col(2)), View(scalarB(3)), View(col(4)));          // mean, one value per row
+    e.record(OpType::Sub, View(full(1)), View(colB(4)), View(full(5)));
+    e.record(OpType::Mul, View(full(5)), View(full(5)), View(full(6)));
+    e.recordRowReduce(OpType::ReduceTo, View(full(6)), View(col(7)), &zero, L);
+    e.record(OpType::Div, View(col(7)), View(scalarB(3)), View(col(8)));          // variance
+    e.recordFill(&eps, DataType::kFloat32, View(T(9, {})));
+    e.record(OpType::Add, View(col(8)), View(scalarB(9)), View(col(10)));
+    e.record(OpType::Sqrt, View(col(10)), View(col(11)));
+    e.record(OpType::Div, View(full(5)), View(colB(11)), View(full(12)));
+    e.record(OpType::Mul, View(full(12)), View(rowB(13)), View(full(14)));        // gamma: one row for every row
+    e.record(OpType::Add, View(full(14)), View(rowB(15)), View(full(16)));
+    for (uintptr_t k : {2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 14}) e.releaseBuffer(reinterpret_cast<void*>(k * 0x10000));
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() != 1) { for (auto& o : cap.order) std::printf("  %s\n", o.c_str()); return; }
+    const auto& d = cap.fused[0];
+    CHECK(d.rowLength == L && d.inputBuffers.size() == 3 && d.outputBuffers.size() == 1 && d.ops.size() == 11);
+    size_t perRow = 0;
+    for (const auto& o : d.ops) perRow += o.perRow;
+    CHECK(perRow == 6);                                                           // two sums, mean, variance, + eps, sqrt
+    CHECK(compilesRow(d));
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -709,6 +865,8 @@ int main(int argc, char** argv)
     testCastsFuseAtTheirLoadOrStoreEnd();
     testDenseSidesAdoptTheStridedSidesShape();
     testTrilJoinsItsNeighbours();
+    testSoftmaxBecomesOneRowProgram();
+    testLayerNormPiecesShareOneRowProgram();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

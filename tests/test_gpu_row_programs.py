@@ -1,0 +1,307 @@
+"""Row programs: sums and maxima over the last dimension recorded by the lazy device and fused with the elementwise
+operators around them into one generated kernel -- Softmax (Targets/AIXLib/aixNeuralNetwork.hpp:188-192: max -> sub ->
+exp -> sum -> div) and the pieces of a LayerNorm.
+
+Each case is driven the way the front-end does (fresh result per operator, fillMin / fill of the destination before
+maxTo / reduceTo as in aixCore.hpp:873-891, temporaries freed before the read) three ways: fused, with fusion switched
+off (the stand-alone kernels, each checked against the oracle in its own tests), and operator by operator on the CPU
+oracle.  Bars: fused and unfused give the SAME BITS wherever there is more than one row (the fused kernel sums a row
+in the stand-alone row kernel's order; a single row is a whole-tensor sum there, in another order); against the oracle
+chain, whose sums run in index order, 1e-5 of the largest result for f32 and 1e-12 for f64.  The 16-bit types add a row
+up in bf16 / f16 on the CPU, one rounding per element (aixDeviceCPU.cpp reduceTo accumulates in the element type), which
+loses whole digits over a row; their results are held against the same expression in float64 on the same inputs
+instead: 2e-2 of the largest result for softmax (4 rounded operators), 4e-2 for the 11 of a LayerNorm.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import aixtest as T
+import devharness as H
+from oracle import cpuref as O
+
+pytestmark = pytest.mark.gpu
+CPU = O.lib()
+NAMES = O.DTYPE_NAMES
+TOL = {O.F64: 1e-12, O.F32: 1e-5, O.F16: 2e-2, O.BF16: 2e-2}
+
+
+@pytest.fixture(scope="module")
+def dev():
+    d = H.Dev()
+    yield d
+    d.close()
+
+
+def set_fusion(dev, on):
+    cfg = dev.dev.fuse_config()
+    cfg.diagnostics = 1
+    cfg.elementwise_fusion = 1 if on else 0
+    dev.dev.set_fuse_config(cfg)
+
+
+class Front:
+    """Records on the device and, operator for operator, on the oracle."""
+
+    def __init__(self, dev, dtype):
+        self.dev, self.dtype, self.temps, self.leaves = dev, dtype, [], []
+
+    def leaf(self, host):
+        p, d = self.dev.put(host)
+        node = {"host": host, "ptr": p, "desc": d}
+        self.leaves.append(node)
+        return node
+
+    def result(self, shape):
+        host = T.empty(self.dtype, shape)
+        p = self.dev.raw(host.storage.nbytes)
+        node = {"host": host, "ptr": p, "desc": H.kdesc(host, p)}
+        self.temps.append(node)
+        return node
+
+    def over_rows(self, node, shape):
+        """[..., 1] read as [..., L] (stride 0 in the last dim), what broadcastTo hands the device."""
+        lead = O.row_major(list(shape[:-1]) + [1])[:-1]
+        view = T.HostTensor(node["host"].storage, self.dtype, shape, lead + [0])
+        return {"host": view, "ptr": node["ptr"], "desc": H.kdesc(view, node["ptr"])}
+
+    def over_all(self, node, shape):
+        view = T.HostTensor(node["host"].storage, self.dtype, shape, [0] * len(shape))
+        return {"host": view, "ptr": node["ptr"], "desc": H.kdesc(view, node["ptr"])}
+
+    def row_vector(self, node, shape):
+        view = T.HostTensor(node["host"].storage, self.dtype, shape, [0] * (len(shape) - 1) + [1])
+        return {"host": view, "ptr": node["ptr"], "desc": H.kdesc(view, node["ptr"])}
+
+    def binary(self, op, x, y, shape):
+        r = self.result(shape)
+        assert CPU.binary(op, C.byref(x["host"].desc()), C.byref(y["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call(["add", "sub", "mul", "div", "pow"][op], H.ref(x["desc"]), H.ref(y["desc"]), H.ref(r["desc"]))
+        return r
+
+    def unary(self, op, x, shape):
+        r = self.result(shape)
+        assert CPU.unary(op, C.byref(x["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call(["unary", "sqrt", "sin", "cos", "tanh", "log", "exp"][op], H.ref(x["desc"]), H.ref(r["desc"]))
+        return r
+
+    def scalar(self, value):
+        r = self.result([])
+        v = np.array([value], dtype=np.float32)
+        assert CPU.fill(v.ctypes.data, O.F32, C.byref(r["host"].desc())) == 0
+        self.dev.dev.call("fill", v.ctypes.data, O.F32, H.ref(r["desc"]))
+        return r
+
+    def row_max(self, x, shape):
+        r = self.result(list(shape[:-1]) + [1])
+        assert CPU.fill_min(C.byref(r["host"].desc())) == 0 and CPU.max_to(C.byref(x["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call("fill_min", H.ref(r["desc"]))
+        self.dev.dev.call("max_to", H.ref(x["desc"]), H.ref(r["desc"]))
+        return r
+
+    def row_sum(self, x, shape):
+        r = self.result(list(shape[:-1]) + [1])
+        zero = np.zeros(1, np.float32)
+        assert CPU.fill(zero.ctypes.data, O.F32, C.byref(r["host"].desc())) == 0 and CPU.reduce_to(C.byref(x["host"].desc()), C.byref(r["host"].desc())) == 0
+        self.dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(r["desc"]))
+        self.dev.dev.call("reduce_to", H.ref(x["desc"]), H.ref(r["desc"]))
+        return r
+
+    def free_temps(self, keep=()):
+        for t in self.temps:
+            if not any(t is k for k in keep):
+                self.dev.free(t["ptr"])
+        self.temps = [t for t in self.temps if any(t is k for k in keep)]
+
+
+def softmax(f, x, shape):
+    m = f.row_max(x, shape)
+    d = f.binary(O.SUB, x, f.over_rows(m, shape), shape)
+    e = f.unary(O.EXP, d, shape)
+    s = f.row_sum(e, shape)
+    return f.binary(O.DIV, e, f.over_rows(s, shape), shape)
+
+
+def layer_norm(f, x, gamma, beta, shape):
+    col = list(shape[:-1]) + [1]
+    length = f.scalar(float(shape[-1]))
+    mean = f.binary(O.DIV, f.row_sum(x, shape), f.over_all(length, col), col)
+    d = f.binary(O.SUB, x, f.over_rows(mean, shape), shape)
+    var = f.binary(O.DIV, f.row_sum(f.binary(O.MUL, d, d, shape), shape), f.over_all(length, col), col)
+    std = f.unary(O.SQRT, f.binary(O.ADD, var, f.over_all(f.scalar(1e-5), col), col), col)
+    n = f.binary(O.DIV, d, f.over_rows(std, shape), shape)
+    return f.binary(O.ADD, f.binary(O.MUL, n, f.row_vector(gamma, shape), shape), f.row_vector(beta, shape), shape)
+
+
+def close_enough(got, want, dtype, what, tol=None):
+    g, w = O.to_float64(got, dtype), O.to_float64(want, dtype)
+    both_nan = np.isnan(g) & np.isnan(w)
+    assert np.array_equal(np.isnan(g), np.isnan(w)), what
+    scale = max(float(np.nanmax(np.abs(w), initial=0.0)), 1e-30)
+    err = np.where(both_nan, 0.0, np.abs(g - w))
+    tol = TOL[dtype] if tol is None else tol
+    assert float(err.max(initial=0.0)) <= tol * scale, f"{what}: {float(err.max())} vs {tol * scale}"
+
+
+def np_softmax(x):
+    e = np.exp(x - x.max(axis=-1, keepdims=True))
+    return e / e.sum(axis=-1, keepdims=True)
+
+
+def run_both(dev, dtype, shape, build, seed, expect_fused_ops=None, lo=-4.0, hi=4.0, poke=None, exact=None, tol16=2e-2):
+    outs, want, leaves = [], None, None
+    for fusion in (True, False):
+        set_fusion(dev, fusion)
+        f = Front(dev, dtype)
+        rng = np.random.default_rng(seed)
+        host = T.contiguous_tensor(rng, dtype, shape, lo=lo, hi=hi)
+        if poke is not None:
+            poke(host)
+        x = f.leaf(host)
+        f.leaves = []
+        y = build(f, x, rng)
+        f.free_temps(keep=(y,))
+        outs.append(dev.fetch(y["ptr"], y["host"].storage))
+        if fusion and expect_fused_ops is not None:
+            diag = dev.dev.diagnostics()
+            assert diag.fusible_subgraphs == 1 and diag.fused_ops == expect_fused_ops and diag.fallback_ops == 0, \
+                (diag.fusible_subgraphs, diag.fused_ops, diag.fallback_ops, diag.subgraph_summary, diag.fallback_summary)
+        want = y["host"].storage
+        leaves = [O.to_float64(host.storage, dtype).reshape(shape)] + [O.to_float64(t["host"].storage, dtype) for t in f.leaves]
+        dev.release()
+    set_fusion(dev, True)
+    what = f"{NAMES[dtype]} {shape}"
+    if O.numel(shape[:-1]) > 1:
+        T.assert_same_bits_nan_ok(outs[0], outs[1], dtype, "fused vs stand-alone kernels " + what)
+    else:
+        close_enough(outs[0], outs[1], dtype, "fused vs stand-alone kernels " + what)
+    if dtype in (O.F32, O.F64):
+        close_enough(outs[0], want, dtype, "fused vs oracle " + what)
+    if exact is not None:
+        with np.errstate(all="ignore"):
+            ideal = exact(*leaves).reshape(-1)
+        tol = {O.F64: 1e-12, O.F32: 1e-5}.get(dtype, tol16)
+        close_enough(outs[0], O.to_storage(ideal, dtype), dtype, "fused vs float64 " + what, tol)
+    return outs[0]
+
+
+# rows shorter than 2048 elements take a wave each, longer ones a workgroup; [9, 1000] and [3, 520] end inside a lane's
+# vector run; 3-D shapes reduce the last dim only
+FUSED_SHAPES = [[64, 128], [9, 1000], [33, 2048], [5, 4096], [3, 520], [4, 6, 64], [2, 3, 5, 256], [1, 512], [300, 64]]
+
+
+@pytest.mark.parametrize("dtype", T.FLOAT_DTYPES, ids=lambda d: NAMES[d])
+def test_softmax_is_one_kernel_and_matches(dev, dtype):
+    for k, shape in enumerate(FUSED_SHAPES):
+        got = run_both(dev, dtype, shape, lambda f, x, rng: softmax(f, x, shape), 500 + k, expect_fused_ops=5, exact=np_softmax)
+        rows = O.to_float64(got, dtype).reshape(-1, shape[-1]).sum(axis=1)
+        assert np.all(np.abs(rows - 1.0) <= (4e-2 if dtype in (O.F16, O.BF16) else 1e-5)), shape     # what the mathematics fixes
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16], ids=lambda d: NAMES[d])
+def test_rows_the_row_program_does_not_take(dev, dtype):
+    """Too long for the registers of a workgroup, not a whole number of 16-byte vectors, or a handful of elements: the
+    reductions run as the stand-alone kernels between fused elementwise kernels; same results."""
+    vec = 16 // O.ITEMSIZE[dtype]
+    for k, shape in enumerate(([2, 8 * 256 * vec * 2], [16, 100 + vec // 2 + 1], [40, 24], [40, 7], [5, 1])):
+        run_both(dev, dtype, shape, lambda f, x, rng: softmax(f, x, shape), 600 + k, exact=np_softmax)
+
+
+@pytest.mark.parametrize("dtype", T.FLOAT_DTYPES, ids=lambda d: NAMES[d])
+def test_layer_norm_pieces_are_one_kernel(dev, dtype):
+    for k, shape in enumerate(([48, 768], [7, 4096], [2, 5, 256])):
+        def build(f, x, rng):
+            gamma = f.leaf(T.contiguous_tensor(rng, dtype, [shape[-1]], lo=0.5, hi=1.5))
+            beta = f.leaf(T.contiguous_tensor(rng, dtype, [shape[-1]], lo=-0.5, hi=0.5))
+            return layer_norm(f, x, gamma, beta, shape)
+
+        def exact(x, gamma, beta):
+            d = x - x.mean(axis=-1, keepdims=True)
+            return d / np.sqrt((d * d).mean(axis=-1, keepdims=True) + np.float64(np.float32(1e-5))) * gamma + beta
+        run_both(dev, dtype, shape, build, 700 + k, expect_fused_ops=11, exact=exact, tol16=4e-2)
+
+
+def test_special_values_in_rows(dev):
+    """A row of -inf (its maximum is -inf, x - max is NaN), a NaN in a row (maxTo skips it as std::max does,
+    aixDeviceCPU.cpp maxTo; the sum carries it), +inf, and a row of one repeated value."""
+    shape = [8, 256]
+
+    def poke(host):
+        v = host.storage.reshape(shape)
+        v[1, :] = -np.inf
+        v[2, 17] = np.nan
+        v[3, 200] = np.inf
+        v[4, :] = 3.25
+        v[5, 0] = np.nan
+    run_both(dev, O.F32, shape, lambda f, x, rng: softmax(f, x, shape), 800, expect_fused_ops=5, poke=poke, exact=np_softmax)
+
+
+def test_row_results_somebody_still_holds_are_stored(dev):
+    """The per-row maximum and sum are read after the window as well: the one kernel stores them too."""
+    shape = [37, 512]
+    for fusion in (True, False):
+        set_fusion(dev, fusion)
+        f = Front(dev, O.F32)
+        x = f.leaf(T.contiguous_tensor(np.random.default_rng(900), O.F32, shape, lo=-3, hi=3))
+        m = f.row_max(x, shape)
+        d = f.binary(O.SUB, x, f.over_rows(m, shape), shape)
+        s = f.row_sum(d, shape)
+        y = f.binary(O.DIV, d, f.over_rows(s, shape), shape)
+        f.free_temps(keep=(y, m, s))
+        got_y = dev.fetch(y["ptr"], y["host"].storage)
+        if fusion:
+            diag = dev.dev.diagnostics()
+            assert diag.fusible_subgraphs == 1 and diag.fused_ops == 4 and diag.fallback_ops == 0, diag.subgraph_summary
+        T.assert_same_bits(dev.fetch(m["ptr"], m["host"].storage), m["host"].storage, "row maxima (exact)")
+        close_enough(dev.fetch(s["ptr"], s["host"].storage), s["host"].storage, O.F32, "row sums")
+        close_enough(got_y, y["host"].storage, O.F32, "quotients")
+        dev.release()
+    set_fusion(dev, True)
+
+
+def test_source_overwritten_after_its_reduction(dev):
+    """max over x, then x += 1 in place, then x - max: the maximum is of the old x, the difference of the new one."""
+    shape = [20, 384]
+    outs = []
+    for fusion in (True, False):
+        set_fusion(dev, fusion)
+        f = Front(dev, O.F32)
+        x = f.leaf(T.contiguous_tensor(np.random.default_rng(901), O.F32, shape, lo=-3, hi=3))
+        x["host"] = x["host"].clone()
+        m = f.row_max(x, shape)
+        one = f.scalar(1.0)
+        ob = f.over_all(one, shape)
+        assert CPU.binary(O.ADD, C.byref(x["host"].desc()), C.byref(ob["host"].desc()), C.byref(x["host"].desc())) == 0
+        dev.dev.call("add", H.ref(x["desc"]), H.ref(ob["desc"]), H.ref(x["desc"]))
+        y = f.binary(O.SUB, x, f.over_rows(m, shape), shape)
+        f.free_temps(keep=(y,))
+        outs.append(dev.fetch(y["ptr"], y["host"].storage))
+        T.assert_same_bits(outs[-1], y["host"].storage, f"(x + 1) - max(x), fusion={fusion}")     # every step is exact or correctly rounded
+        dev.release()
+    set_fusion(dev, True)
+
+
+def test_initial_value_of_the_destination_takes_part(dev):
+    """reduceTo adds to, and maxTo compares with, what the destination was filled with (aixDeviceCPU.cpp reduceTo /
+    maxTo accumulate into dst): a fill of 10 before the row sum, a fill of 2.5 before the row maximum."""
+    shape = [12, 320]
+    for fusion in (True, False):
+        set_fusion(dev, fusion)
+        f = Front(dev, O.F32)
+        x = f.leaf(T.contiguous_tensor(np.random.default_rng(902), O.F32, shape, lo=-3, hi=3))
+        col = [12, 1]
+        s, m = f.result(col), f.result(col)
+        for node, value, cpu, name in ((s, 10.0, CPU.reduce_to, "reduce_to"), (m, 2.5, CPU.max_to, "max_to")):
+            v = np.array([value], np.float32)
+            assert CPU.fill(v.ctypes.data, O.F32, C.byref(node["host"].desc())) == 0 and cpu(C.byref(x["host"].desc()), C.byref(node["host"].desc())) == 0
+            dev.dev.call("fill", v.ctypes.data, O.F32, H.ref(node["desc"]))
+            dev.dev.call(name, H.ref(x["desc"]), H.ref(node["desc"]))
+        y = f.binary(O.MUL, f.binary(O.SUB, x, f.over_rows(s, shape), shape), f.over_rows(m, shape), shape)
+        f.free_temps(keep=(y, m))
+        close_enough(dev.fetch(y["ptr"], y["host"].storage), y["host"].storage, O.F32, f"(x - (10 + sum)) * max(2.5, max), fusion={fusion}")
+        got_m = dev.fetch(m["ptr"], m["host"].storage)
+        T.assert_same_bits(got_m, m["host"].storage, "maxima with a floor")
+        assert got_m.min() >= 2.5
+        dev.release()
+    set_fusion(dev, True)
