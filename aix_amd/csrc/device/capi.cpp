@@ -160,7 +160,7 @@ int32_t aixhip_get_fuse_config(aixhip_device* dev, aixhip_fuse_config* out)
         if (!out) throw std::invalid_argument("null out pointer");
         const auto& c = D(dev).fuseConfig();
         *out = aixhip_fuse_config{c.elementwiseFusion, c.multiOutputKernels, c.absorbFills, c.diagnostics,
-                                  c.flushThreshold, c.maxBufferSlots, c.supportsStridedFusion, 0};
+                                  c.flushThreshold, c.maxBufferSlots, c.supportsStridedFusion, !c.deferIdleFills};
     });
 }
 
@@ -176,6 +176,7 @@ int32_t aixhip_set_fuse_config(aixhip_device* dev, const aixhip_fuse_config* cfg
         c.flushThreshold = cfg->flush_threshold ? cfg->flush_threshold : 1;
         c.maxBufferSlots = cfg->max_buffer_slots;
         c.supportsStridedFusion = cfg->supports_strided_fusion != 0;
+        c.deferIdleFills = cfg->eager_idle_fills == 0;
         D(dev).setFuseConfig(c);
     });
 }

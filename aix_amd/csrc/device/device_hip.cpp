@@ -121,6 +121,15 @@ DeviceHIP::Block* DeviceHIP::BlockTable::find(const void* base) const
     }
 }
 
+const void* DeviceHIP::BlockTable::baseOf(const void* p) const
+{
+    if (find(p)) return p;
+    const uintptr_t a = (uintptr_t)p;
+    if (a < m_lo || a >= m_hi) return nullptr;
+    for (const auto& s : m_slots) if (s.key > 1 && a >= s.key && a < s.key + s.block.bytes) return (const void*)s.key;
+    return nullptr;
+}
+
 DeviceHIP::Block* DeviceHIP::BlockTable::findContaining(const void* p) const
 {
     const uintptr_t a = (uintptr_t)p;
@@ -232,6 +241,7 @@ void DeviceHIP::setFuseConfig(const FuseConfig& cfg)
     cb.emitSingle = [this](const OpRecord& op) { emitSingle(op); };
     cb.finishFlush = [] {};
     cb.getKernelCacheStats = [this] { return fuseKernelCacheStats(); };
+    cb.blockBase = [this](const void* p) { return m_blocks.baseOf(p); };
     m_engine = std::make_unique<FuseEngine>(cfg, std::move(cb));
     m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) m_engine->retainBuffer(base); });
 }
@@ -316,7 +326,7 @@ void DeviceHIP::deallocate(void* memory)
     m_limbo.emplace_back(memory, bytes);
     m_limboBytes += bytes;
     m_liveBytes -= bytes;
-    if (m_limboBytes > (size_t(8) << 30)) flush();          // recorded work pins too much freed memory
+    if (m_limboBytes > (size_t(8) << 30)) flushWindow(false);   // recorded work pins too much freed memory
 }
 
 void DeviceHIP::markTouched(const void* p)
@@ -380,22 +390,39 @@ void DeviceHIP::emptyCache()
     m_pooledBytes = 0;
 }
 
-void DeviceHIP::flush()
+void DeviceHIP::flush() { flushWindow(true); }
+
+// final: nothing recorded stays behind.  Otherwise fills that nothing recorded so far uses may wait (FuseEngine::flush).
+void DeviceHIP::flushWindow(bool final)
 {
     issueMatmulGroup();                                     // pending products were called before anything now in the window was recorded
-    m_engine->flush();
+    m_engine->flush(final);
     releaseLimbo();
 }
 
 void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
 {
-    m_engine->recordExternalRead(a);
-    m_engine->recordExternalRead(b);
-    m_engine->recordExternalRead(c);
+    for (const void* p : {a, b, c}) {
+        if (!p) continue;
+        m_engine->recordExternalRead(p);
+        const void* base = m_blocks.baseOf(p);              // an operand may point into the middle of a block
+        if (base && base != p) m_engine->recordExternalRead(base);
+    }
     markTouched(a);                                         // the caller is about to enqueue work on them
     markTouched(b);
     markTouched(c);
-    flush();
+    flushWindow(false);
+}
+
+// The planner orders recorded operators by the addresses of their buffers.  An operand that points into the middle of
+// a block (pointer arithmetic by a caller of the C ABI; the front-end names a block's start and an offset) would escape
+// that: operators with such an operand are recorded into a window of their own.
+bool DeviceHIP::fenceInterior(const void* a, const void* b, const void* c)
+{
+    bool any = false;
+    for (const void* p : {a, b, c}) if (p && !m_blocks.find(p) && m_blocks.baseOf(p)) any = true;
+    if (any) flushFor(a, b, c);
+    return any;
 }
 
 void DeviceHIP::synchronize()
@@ -503,7 +530,9 @@ void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const Device
         check(aixk_binary(m_ctx, binaryCode(t), &pa, &pb, &po));
         return;
     }
+    const bool fenced = fenceInterior(va.data, vb.data, out.data);
     m_engine->record(t, va, vb, out);
+    if (fenced) flushFor(out.data);                         // (names the result: somebody may read it through the block's start)
 }
 
 void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op)
@@ -525,7 +554,9 @@ void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceT
         check(aixk_unary(m_ctx, unaryCode(t), &pa, &po));
         return;
     }
+    const bool fenced = fenceInterior(va.data, out.data);
     m_engine->record(t, va, out);
+    if (fenced) flushFor(out.data);
 }
 
 void DeviceHIP::add(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Add, a1, a2, result, "add"); }
@@ -546,7 +577,9 @@ void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTenso
     requireDevice(result, "fill");
     View out(result);
     out.makeDense();
+    const bool fenced = fenceInterior(out.data);
     m_engine->recordFill(scalar, scalarDType, out);
+    if (fenced) flushFor(out.data);
 }
 
 void DeviceHIP::fillMin(const DeviceTensorParams& result)
@@ -554,7 +587,9 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
     requireDevice(result, "fillMin");
     View out(result);
     out.makeDense();
+    const bool fenced = fenceInterior(out.data);
     m_engine->recordFillMin(out);
+    if (fenced) flushFor(out.data);
 }
 
 // ---- planner callbacks -------------------------------------------------------------------------
@@ -705,7 +740,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     else {
         int32_t cached = 0;
         const std::string src = gen::source(d, shape, bmask, noAlias, streamOut);
-        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
+        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(d, shape).c_str(), &mod, &cached));
         ex.kernels.emplace(ex.key, mod);
         ++ex.misses;
     }
@@ -747,7 +782,7 @@ void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
     else {
         int32_t cached = 0;
         const std::string src = gen::rowSource(d, geo, streamOut);
-        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::entryName(), &mod, &cached));
+        check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), gen::rowEntryName(d, geo).c_str(), &mod, &cached));
         ex.kernels.emplace(ex.key, mod);
         ++ex.misses;
     }
@@ -816,7 +851,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             if (m_engine->pendingWrites(a.data) || m_engine->pendingWrites(b.data) || m_engine->pendingTouches(result.data)) {
                 m_engine->recordExternalRead(a.data);
                 m_engine->recordExternalRead(b.data);
-                flush();
+                flushWindow(false);
             }
             aixhip_tensor pa, pb, pr; toPod(a, &pa, "matmul"); toPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
             // it may read no pending result and overwrite nothing pending: all pending products are then independent of
@@ -962,7 +997,7 @@ bool DeviceHIP::recordRowReduction(OpType type, const DeviceTensorParams& src, c
 {
     if (!m_engine->config().elementwiseFusion || !m_extras->fuseRowReductions) return false;
     if (src.dtype != DataType::kFloat32 && src.dtype != DataType::kFloat16 && src.dtype != DataType::kBFloat16 && src.dtype != DataType::kFloat64) return false;
-    if (src.shape.empty() || src.shape.size() > AIXK_MAX_RANK || !src.isContiguous || !findBlock(src.data) || src.size == 0) return false;
+    if (src.shape.empty() || src.shape.size() > AIXK_MAX_RANK || !src.isContiguous || !m_blocks.find(src.data) || !m_blocks.find(dst.data) || src.size == 0) return false;
     const size_t L = src.shape.back(), esz = dataTypeSize(src.dtype), vec = 16 / esz;
     if (L < 32 || L % vec != 0 || src.offset % vec != 0 || src.size % L != 0 || dst.size != src.size / L) return false;
     if (L / vec > 8 * (L >= 2048 ? 256u : 64u)) return false;              // more than 8 vectors per lane: the stand-alone kernel
@@ -1066,7 +1101,7 @@ void DeviceHIP::triu(const DeviceTensorParams& src, const DeviceTensorParams& ds
 bool DeviceHIP::recordTri(OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
 {
     if (src.shape.size() < 2 || src.shape.size() > (size_t)gen::kMaxDims || src.shape != dst.shape || src.size == 0 || src.size != dst.size) return false;
-    if (!dst.isContiguous || dst.offset != 0 || !findBlock(src.data)) return false;
+    if (!dst.isContiguous || dst.offset != 0 || !m_blocks.find(src.data) || !m_blocks.find(dst.data)) return false;   // (blocks by their start)
     size_t count = 1;
     for (auto e : src.shape) count *= e;
     if (count != src.size) return false;

@@ -122,6 +122,7 @@ private:
     public:
         Block* find(const void* base) const;
         Block* findContaining(const void* p) const;
+        const void* baseOf(const void* p) const;            // start of the block p lies in; nullptr for host memory
         void insert(void* base, size_t bytes);
         bool erase(void* base, size_t* bytes);
         bool empty() const { return m_count == 0; }
@@ -155,6 +156,8 @@ private:
     bool recordTri(aixhip::fuse::OpType t, const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal);
     bool takeInit(const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t* bits);
     void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
+    void flushWindow(bool final);
+    bool fenceInterior(const void* a, const void* b = nullptr, const void* c = nullptr);   // true: flush again once the operator is recorded
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void emitSingle(const aixhip::fuse::OpRecord& op);
     void emitRowProgram(const aixhip::fuse::FusedSubgraphDescriptor& d);

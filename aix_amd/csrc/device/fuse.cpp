@@ -904,7 +904,49 @@ FuseEngine::~FuseEngine() = default;
 
 void FuseEngine::maybeFlush()
 {
-    if (m_pending.size() >= m_config.flushThreshold) flush();
+    if (m_pending.size() >= m_config.flushThreshold) flush(false);
+}
+
+void FuseEngine::wake(const void* operand)
+{
+    if (!operand || m_waiting.empty()) return;
+    const void* base = m_callbacks.blockBase ? m_callbacks.blockBase(operand) : operand;
+    if (!base || !m_waitingBuffers.contains(base)) return;
+    size_t kept = 0;
+    for (size_t k = 0; k < m_waiting.size(); ++k) {
+        if (m_waiting[k].output.data == base) { m_pending.push_back(m_waiting[k]); m_pending.back().hasWaited = true; }
+        else { if (kept != k) m_waiting[kept] = m_waiting[k]; ++kept; }
+    }
+    m_waiting.resize(kept);
+    m_waitingBuffers.erase(base);
+}
+
+// Moves the window's idle fills (see flush()) from m_window to m_waiting.
+void FuseEngine::setAsideIdleFills()
+{
+    auto isFill = [](const OpRecord& op) { return op.type == OpType::Fill || op.type == OpType::FillMin; };
+    size_t kept = 0;
+    bool moved = false;
+    for (size_t i = 0; i < m_window.size(); ++i) {
+        const OpRecord& op = m_window[i];
+        bool idle = isFill(op) && !op.hasWaited && op.output.dense && op.output.offset == 0 && m_live.contains(op.output.data) &&
+                    !m_waitingBuffers.contains(op.output.data);
+        if (idle) for (const void* r : m_externalReads) if (r == op.output.data) { idle = false; break; }
+        if (idle) {
+            const void* buf = op.output.data;
+            for (size_t j = 0; j < m_window.size() && idle; ++j) {
+                if (j == i) continue;
+                const OpRecord& o = m_window[j];
+                if (o.output.data == buf || o.input0.data == buf || (o.hasInput1 && o.input1.data == buf)) idle = false;
+            }
+            // (the records already moved sit at [0, kept) or were set aside: one set aside touched another buffer, or this
+            // fill's buffer would be in m_waitingBuffers)
+        }
+        if (idle) { m_waiting.push_back(op); m_waitingBuffers.insert(op.output.data); moved = true; continue; }
+        if (kept != i) m_window[kept] = m_window[i];
+        ++kept;
+    }
+    if (moved) m_window.resize(kept);
 }
 
 OpRecord& FuseEngine::append(OpType type)
@@ -917,6 +959,7 @@ OpRecord& FuseEngine::append(OpType type)
 
 void FuseEngine::record(OpType type, const View& input0, const View& output)
 {
+    wake(input0.data); wake(output.data);
     OpRecord& r = append(type);
     r.input0 = input0; r.output = output;
     maybeFlush();
@@ -924,6 +967,7 @@ void FuseEngine::record(OpType type, const View& input0, const View& output)
 
 void FuseEngine::record(OpType type, const View& input0, const View& input1, const View& output)
 {
+    wake(input0.data); wake(input1.data); wake(output.data);
     OpRecord& r = append(type);
     r.input0 = input0; r.input1 = input1; r.output = output; r.hasInput1 = true;
     maybeFlush();
@@ -931,6 +975,7 @@ void FuseEngine::record(OpType type, const View& input0, const View& input1, con
 
 void FuseEngine::recordFill(const void* scalar, DataType scalarDType, const View& output)
 {
+    wake(output.data);
     OpRecord& r = append(OpType::Fill);
     r.output = output; r.scalarDType = scalarDType;
     std::memcpy(r.scalarData.data(), scalar, aix::Device::dataTypeSize(scalarDType));
@@ -940,6 +985,7 @@ void FuseEngine::recordFill(const void* scalar, DataType scalarDType, const View
 void FuseEngine::recordTri(OpType type, const View& input, const View& output, int64_t diagonal)
 {
     if ((type != OpType::Tril && type != OpType::Triu) || input.rank < 2) throw std::invalid_argument("recordTri: tril / triu of a tensor of rank 2 or more");
+    wake(input.data); wake(output.data);
     OpRecord& r = append(type);
     r.input0 = input; r.output = output;
     r.triRows = input.shape[input.rank - 2]; r.triCols = input.shape[input.rank - 1]; r.triDiagonal = diagonal;
@@ -950,6 +996,7 @@ void FuseEngine::recordRowReduce(OpType type, const View& input, const View& out
 {
     if (!isRowReduce(type) || rowLength == 0 || input.size % rowLength != 0 || output.size != input.size / rowLength || input.dtype != output.dtype)
         throw std::invalid_argument("recordRowReduce: a sum / maximum over the rows of a [rows, length] operand into one value per row");
+    wake(input.data); wake(output.data);
     OpRecord& r = append(type);
     r.input0 = input; r.output = output; r.rowLength = rowLength;
     r.scalarDType = output.dtype;
@@ -959,6 +1006,7 @@ void FuseEngine::recordRowReduce(OpType type, const View& input, const View& out
 
 void FuseEngine::recordFillMin(const View& output)
 {
+    wake(output.data);
     OpRecord& r = append(OpType::FillMin);
     r.output = output;
     maybeFlush();
@@ -970,9 +1018,14 @@ const FlushDiagnostics& FuseEngine::lastFlushDiagnostics() const
     return m_diagnostics ? *m_diagnostics : empty;
 }
 
-void FuseEngine::flush()
+void FuseEngine::flush(bool final)
 {
     if (m_flushing) return;                  // callbacks may call back into the device
+    if (final && !m_waiting.empty()) {       // every waiting fill runs now; nothing recorded since touches their buffers
+        m_pending.insert(m_pending.begin(), m_waiting.begin(), m_waiting.end());
+        for (const OpRecord& op : m_waiting) m_waitingBuffers.erase(op.output.data);
+        m_waiting.clear();
+    }
     if (m_pending.empty()) {                 // nothing recorded: the previous flush's diagnostics stay readable
         m_externalReads.clear();
         m_callbacks.finishFlush();
@@ -985,6 +1038,7 @@ void FuseEngine::flush()
 
     m_window.clear();
     m_window.swap(m_pending);                // operators recorded by callbacks belong to the next window
+    if (!final && m_config.deferIdleFills && m_config.elementwiseFusion && m_config.absorbFills) setAsideIdleFills();
     const std::vector<OpRecord>& window = m_window;
     // buffers about to be read outside the planner count as alive for this window
     const Planner::Liveness live{&m_live, &m_externalReads};
@@ -1028,6 +1082,7 @@ void FuseEngine::flush()
 bool FuseEngine::takeTrailingFill(const View& output, OpRecord* fill)
 {
     if (m_flushing || !output.data) return false;
+    wake(output.data);
     for (size_t k = m_pending.size(); k-- > 0;) {
         const OpRecord& op = m_pending[k];
         const bool reads = op.type != OpType::Fill && op.type != OpType::FillMin &&
@@ -1044,16 +1099,18 @@ bool FuseEngine::takeTrailingFill(const View& output, OpRecord* fill)
     return false;
 }
 
-bool FuseEngine::pendingWrites(const void* buffer) const
+bool FuseEngine::pendingWrites(const void* buffer)
 {
     if (!buffer) return false;
+    wake(buffer);
     for (const OpRecord& op : m_pending) if (op.output.data == buffer) return true;
     return false;
 }
 
-bool FuseEngine::pendingTouches(const void* buffer) const
+bool FuseEngine::pendingTouches(const void* buffer)
 {
     if (!buffer) return false;
+    wake(buffer);
     for (const OpRecord& op : m_pending)
         if (op.output.data == buffer || op.input0.data == buffer || (op.hasInput1 && op.input1.data == buffer)) return true;
     return false;
@@ -1062,6 +1119,7 @@ bool FuseEngine::pendingTouches(const void* buffer) const
 void FuseEngine::recordExternalRead(const void* buffer)
 {
     if (!buffer) return;
+    wake(buffer);
     for (const void* known : m_externalReads) if (known == buffer) return;
     m_externalReads.push_back(buffer);
 }
@@ -1072,6 +1130,13 @@ void FuseEngine::releaseBuffer(void* buffer)
 {
     if (!buffer) return;
     m_live.erase(buffer);
+    if (!m_waiting.empty() && m_waitingBuffers.contains(buffer)) {          // nobody will ever read what the fill would write
+        size_t kept = 0;
+        for (size_t k = 0; k < m_waiting.size(); ++k)
+            if (m_waiting[k].output.data != buffer) { if (kept != k) m_waiting[kept] = m_waiting[k]; ++kept; }
+        m_waiting.resize(kept);
+        m_waitingBuffers.erase(buffer);
+    }
     for (size_t k = 0; k < m_externalReads.size(); ++k)
         if (m_externalReads[k] == buffer) { m_externalReads[k] = m_externalReads.back(); m_externalReads.pop_back(); break; }
 }

@@ -48,6 +48,7 @@ struct FuseConfig {
     size_t flushThreshold        = 200;    // recorded ops that trigger planning
     size_t maxBufferSlots        = 0;      // pointer arguments one fused kernel may take (must be > 0)
     bool   supportsStridedFusion = true;   // may fused kernels read broadcast / strided views
+    bool   deferIdleFills        = true;   // a fill nothing else in its window touches waits for its first user (see flush())
 };
 
 // An operand as the planner keeps it: the fields of aix::DeviceTensorParams with the extents and
@@ -99,6 +100,9 @@ struct OpRecord {
     // ReduceTo / MaxTo recorded as a row reduction: elements per row of input0 (its last dimension); scalarData then holds
     // the value the destination was initialised with, in the destination's element type (the folded fill)
     size_t rowLength{0};
+    // Fill / FillMin: the fill has waited outside the window and was brought back because somebody names its buffer: it
+    // runs with the window it is in now
+    bool hasWaited{false};
 };
 
 // How a view takes part in a kernel that works row by row on [rows, length] data (a "row program"): element for element,
@@ -157,6 +161,9 @@ struct FuseCallbacks {
     std::function<void(const OpRecord&)> emitSingle;
     std::function<void()> finishFlush;
     std::function<std::pair<size_t, size_t>()> getKernelCacheStats = [] { return std::pair<size_t, size_t>{0, 0}; };
+    // The start of the allocation an operand pointer lies in (operands may point into the middle of a block); an
+    // engine without it takes every pointer for a block of its own.
+    std::function<const void*(const void*)> blockBase;
 };
 
 // Converts a scalar between element types with the device's conversion rules (saturating
@@ -200,7 +207,15 @@ public:
     // ReduceTo / MaxTo over the last dimension (`rowLength` elements, dense) of `input` into the dense `output`, whose
     // pending initialisation the caller has taken out of the window: `init` is that value in output's element type.
     void recordRowReduce(OpType type, const View& input, const View& output, const void* init, size_t rowLength);
-    void flush();
+    // Plans and emits the window.  A fill (fill / fillMin of a whole dense buffer that allocate() handed out) that no
+    // other operator of the window touches, and that nobody outside is about to read, is not emitted unless `final`:
+    // it waits, outside the window, until an operator naming its buffer is recorded (it then rejoins the window ahead
+    // of that operator and is usually absorbed as an immediate), until the buffer is read outside the planner
+    // (recordExternalRead, takeTrailingFill, pendingWrites / pendingTouches), or until a final flush; a buffer released
+    // in between takes its fill along.  zeroGrad() followed, a whole forward and backward pass later, by the first
+    // accumulation into the gradient is the case this is for (aixCore.hpp zeroGrad, accumulateGrad).
+    void flush(bool final = true);
+    size_t waitingFills() const { return m_waiting.size(); }
 
     const FuseConfig& config() const { return m_config; }
     const FlushDiagnostics& lastFlushDiagnostics() const;
@@ -210,8 +225,8 @@ public:
     // tensor, remove it from the window and hand it over (the caller folds it into the operator
     // it is about to run eagerly); false and no change otherwise.
     bool takeTrailingFill(const View& output, OpRecord* fill);
-    bool pendingWrites(const void* buffer) const;  // a recorded operator of the window writes the buffer
-    bool pendingTouches(const void* buffer) const; // ... reads or writes it
+    bool pendingWrites(const void* buffer);        // a recorded operator of the window writes the buffer
+    bool pendingTouches(const void* buffer);       // ... reads or writes it
     void recordExternalRead(const void* buffer);   // the buffer is about to be read outside the planner
     void retainBuffer(void* buffer);               // allocate(): results written here must reach memory
     void releaseBuffer(void* buffer);              // deallocate(): nobody will read it after the window
@@ -219,6 +234,8 @@ public:
 
 private:
     void maybeFlush();
+    void wake(const void* operand);                // the waiting fills of the operand's buffer rejoin the window
+    void setAsideIdleFills();
 
     FuseConfig m_config;
     FuseCallbacks m_callbacks;
@@ -227,6 +244,8 @@ private:
     std::vector<OpRecord> m_window;
     PointerSet m_live;
     std::vector<const void*> m_externalReads;
+    std::vector<OpRecord> m_waiting;       // fills set aside by flush(false), oldest first
+    PointerSet m_waitingBuffers;
     std::unique_ptr<Planner> m_planner;    // its working storage is kept from window to window
     FusedSubgraphDescriptor m_descriptor;
     std::optional<FlushDiagnostics> m_diagnostics;

@@ -13,6 +13,28 @@ namespace aixhip::gen {
 using fuse::FusedSubgraphDescriptor;
 using fuse::OpType;
 
+static std::string entryNameWith(const fuse::FusedSubgraphDescriptor& d, const char* tag)
+{
+    static const char* const types[] = {"f64", "f32", "f16", "bf16", "i64", "i32", "i16", "i8", "u8"};
+    std::string name = std::string("aix_fused_") + types[static_cast<size_t>(d.dtype)] + "_" + tag + "_";
+    for (const auto& op : d.ops) {
+        const char* n = fuse::opName(op.type);
+        if (name.size() + std::strlen(n) > 116) { name += "_etc"; break; }
+        name += n;
+    }
+    return name;
+}
+
+std::string entryName(const fuse::FusedSubgraphDescriptor& d, Shape shape)
+{
+    return entryNameWith(d, shape == Shape::Flat ? "flat" : shape == Shape::Rows ? "rows" : "gather");
+}
+
+std::string rowEntryName(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g)
+{
+    return entryNameWith(d, g.lanes == 64 ? "row64" : "row256");
+}
+
 namespace {
 
 const char* typeName(aix::DataType t)
@@ -186,7 +208,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     if (shape != Shape::Flat) o << "    u64 chunks;\n    u64 rank;\n    u64 shape[" << kMaxDims << "];\n    u64 off[" << AI << "];\n    u64 str[" << AI << "][" << kMaxDims << "];\n";
     o << "};\n\n";
 
-    o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void aix_fused(Args a)\n{\n"
+    o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << entryName(d, shape) << "(Args a)\n{\n"
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
@@ -357,7 +379,7 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     auto to_t = [&](size_t k, const std::string& e) { return d.inputBuffers[k].dtype == d.dtype ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
     auto from_t = [&](size_t k, const std::string& e) { return d.outputBuffers[k].dtype == d.dtype ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
     o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 rows;\n    u64 len;\n};\n\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void aix_fused(Args a)\n{\n"
+      << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "(Args a)\n{\n"
       << "    __shared__ W red[4];\n    (void)red;\n"
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";

@@ -30,7 +30,7 @@ std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint3
 // The same text written into `out` (cleared first; its capacity is reused from call to call).
 void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut = false);
 
-// Source of `extern "C" __global__ void aix_fused(Args)`.
+// Source of `extern "C" __global__ void <entryName>(Args)`.
 std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false);
 
 // ---- row programs (descriptor.rowLength > 0) ------------------------------------------------------------------------
@@ -48,7 +48,10 @@ std::string rowSource(const fuse::FusedSubgraphDescriptor& d, const RowGeometry&
 // Args of a row program: in[], out[], immediates, rows, rowLength
 void packRowArgsInto(std::vector<uint64_t>& a, const fuse::FusedSubgraphDescriptor& d, const void* const* inputs, void* const* outputs);
 
-inline const char* entryName() { return "aix_fused"; }
+// The kernel's symbol: "aix_fused_<type>_<launch shape>_<operators in order>" (what a profiler's trace shows), at most
+// 120 characters.
+std::string entryName(const fuse::FusedSubgraphDescriptor& d, Shape shape);
+std::string rowEntryName(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g);
 
 constexpr int kMaxDims = 8;
 constexpr int kBlock = 256;

@@ -14,7 +14,7 @@ _P = C.c_void_p
 class FuseConfig(C.Structure):
     _fields_ = [("elementwise_fusion", C.c_int32), ("multi_output_kernels", C.c_int32), ("absorb_fills", C.c_int32),
                 ("diagnostics", C.c_int32), ("flush_threshold", C.c_uint64), ("max_buffer_slots", C.c_uint64),
-                ("supports_strided_fusion", C.c_int32), ("reserved", C.c_int32)]
+                ("supports_strided_fusion", C.c_int32), ("eager_idle_fills", C.c_int32)]
 
 
 class FlushDiagnostics(C.Structure):

@@ -239,7 +239,7 @@ def main():
         # a copy kernel of known size (profiles/aix_fused_c0_f32_4096x4096.md); a measured constant, not live.
         "roofline": roofline("hbm", algo_bytes / (kernel_ms * 1e-3) / 1e9, HBM_PEAK_GBS, "GB/s", traffic=268409963),
     }
-    out["roofline"]["kernel"] = "aix_fused (f32|flat|i3o1s2, 9 ops)"
+    out["roofline"]["kernel"] = "aix_fused_f32_flat_MulAddTanhNegateExpAddDivMulSub"
     out["roofline"]["kernel_us"] = round(kernel_ms * 1e3, 2)
 
     # ---- the reference CPU path on the same inputs --------------------------------------------------

@@ -121,7 +121,8 @@ typedef struct aixhip_fuse_config {
     uint64_t flush_threshold;
     uint64_t max_buffer_slots;
     int32_t  supports_strided_fusion;
-    int32_t  reserved;
+    int32_t  eager_idle_fills;        /* 1: a fill nothing in its window uses runs at once; 0 (default): it waits for its
+                                         first user or the next synchronize / flush and is usually absorbed there */
 } aixhip_fuse_config;
 int32_t aixhip_get_fuse_config(aixhip_device* dev, aixhip_fuse_config* out);
 int32_t aixhip_set_fuse_config(aixhip_device* dev, const aixhip_fuse_config* cfg);

@@ -838,6 +838,99 @@ static void testLayerNormPiecesShareOneRowProgram()
     CHECK(compilesRow(d));
 }
 
+static void testIdleFillsWaitForTheirFirstUser()
+{
+    // zeroGrad() ... a long time later ... grad = grad + g: the fill is held back by the flushes in between and ends up
+    // as an immediate of the accumulation; nothing is launched for it
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto grad = T(1, {512, 64}), g = T(2, {512, 64}), other = T(3, {512, 64}), sink = T(4, {512, 64});
+        for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        const float zero = 0.0f;
+        e.recordFill(&zero, DataType::kFloat32, View(grad));
+        e.record(OpType::Exp, View(other), View(sink));
+        e.flush(false);
+        CHECK(cap.singles.size() == 1 && cap.singles[0].type == OpType::Exp && cap.fused.empty() && e.waitingFills() == 1);
+        e.flush(false);                                             // an empty window changes nothing
+        CHECK(e.waitingFills() == 1 && cap.singles.size() == 1);
+        CHECK(e.pendingOps() == 0);
+        e.record(OpType::Add, View(grad), View(g), View(grad));
+        CHECK(e.waitingFills() == 0 && e.pendingOps() == 2);        // the fill rejoined the window ahead of its user
+        e.flush(false);
+        CHECK(cap.fused.size() == 1 && cap.singles.size() == 1);
+        if (cap.fused.size() == 1) {
+            const auto& d = cap.fused[0];
+            CHECK(d.ops.size() == 1 && d.inputBuffers.size() == 1 && d.inputBuffers[0].data == g.data && d.ops[0].scalarIndex0 != SIZE_MAX);
+            CHECK(scalarAt(d, d.ops[0].scalarIndex0) == 0.0f);
+        }
+    }
+    // a final flush runs what waits; a released buffer takes its fill along; a fill somebody in the window uses, a fill of
+    // part of a buffer and a fill of memory the device did not hand out never wait
+    {
+        Capture cap;
+        FuseEngine e(config(), cap.callbacks());
+        auto a = T(1, {100}), b = T(2, {100}), c = T(3, {100}), part = T(4, {50}, DataType::kFloat32, {}, 8), foreign = T(9, {100});
+        for (uintptr_t id : {1, 2, 3, 4}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        const float one = 1.0f;
+        e.recordFill(&one, DataType::kFloat32, View(a));
+        e.recordFill(&one, DataType::kFloat32, View(b));
+        e.recordFillMin(View(c));
+        e.recordFill(&one, DataType::kFloat32, View(part));
+        e.recordFill(&one, DataType::kFloat32, View(foreign));
+        e.flush(false);
+        CHECK(e.waitingFills() == 3 && cap.singles.size() == 1);    // `part` ran; nobody can read `foreign`: dropped
+        if (std::getenv("AIX_TEST_VERBOSE")) { std::printf("waiting %zu singles %zu fused %zu\n", e.waitingFills(), cap.singles.size(), cap.fused.size()); for (auto& o : cap.order) std::printf("  %s\n", o.c_str()); }
+        e.releaseBuffer(b.data);
+        CHECK(e.waitingFills() == 2);
+        e.flush();
+        CHECK(e.waitingFills() == 0 && cap.singles.size() == 3);
+        CHECK(cap.singles[1].type == OpType::Fill && cap.singles[1].output.data == a.data && cap.singles[2].type == OpType::FillMin);
+    }
+    // reading the buffer outside the planner, asking whether work on it is pending, or folding the fill into an eager
+    // operator brings it back; so does an operand that points into the middle of the filled block (the device fences such
+    // operands with flushes of its own: the planner orders operators by buffer address)
+    {
+        Capture cap;
+        auto cb = cap.callbacks();
+        cb.blockBase = [](const void* p) { return reinterpret_cast<const void*>(reinterpret_cast<uintptr_t>(p) & ~uintptr_t(0xFFFF)); };
+        FuseEngine e(config(), cb);
+        auto a = T(1, {100}), b = T(2, {100}), c = T(3, {100}), d = T(4, {100}), out = T(5, {50});
+        for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+        const float two = 2.0f;
+        for (auto* t : {&a, &b, &c, &d}) e.recordFill(&two, DataType::kFloat32, View(*t));
+        e.flush(false);
+        CHECK(e.waitingFills() == 4 && cap.singles.empty());
+        e.recordExternalRead(a.data);
+        CHECK(e.waitingFills() == 3 && e.pendingOps() == 1);
+        CHECK(e.pendingWrites(b.data) && e.waitingFills() == 2 && e.pendingOps() == 2);
+        OpRecord fill;
+        CHECK(e.takeTrailingFill(View(c), &fill) && fill.type == OpType::Fill && e.waitingFills() == 1 && e.pendingOps() == 2);
+        auto inside = T(4, {50});
+        inside.data = reinterpret_cast<char*>(inside.data) + 200;   // elements [50, 100) of d by pointer
+        e.record(OpType::Negate, View(inside), View(out));
+        CHECK(e.waitingFills() == 0 && e.pendingOps() == 4);
+        e.flush(false);
+        CHECK(e.waitingFills() == 0);                               // a fill that has waited runs with the window it rejoined
+        size_t fills = 0;
+        for (const auto& op : cap.singles) fills += op.type == OpType::Fill;
+        CHECK(fills == 3 && cap.singles.size() == 4);               // a, b, d and the negate (c's fill was handed over)
+    }
+    // switched off: every fill runs in its own window
+    {
+        Capture cap;
+        FuseConfig c = config();
+        c.deferIdleFills = false;
+        FuseEngine e(c, cap.callbacks());
+        auto a = T(1, {100});
+        e.retainBuffer(a.data);
+        const float one = 1.0f;
+        e.recordFill(&one, DataType::kFloat32, View(a));
+        e.flush(false);
+        CHECK(e.waitingFills() == 0 && cap.singles.size() == 1);
+    }
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -867,6 +960,7 @@ int main(int argc, char** argv)
     testTrilJoinsItsNeighbours();
     testSoftmaxBecomesOneRowProgram();
     testLayerNormPiecesShareOneRowProgram();
+    testIdleFillsWaitForTheirFirstUser();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

@@ -590,3 +590,61 @@ def test_tril_and_triu_join_the_fused_kernels(dev):
         neg = rec.unary(O.NEG, w)
         T.assert_same_bits(dev.fetch(neg["ptr"], neg["host"].storage), neg["host"].storage, f"tril(transposed view) -> negate {NAMES[dtype]}")
         dev.release()
+
+
+def test_idle_fills_wait_for_their_first_user(dev):
+    """zeroGrad() and, a pass later, the accumulation into the gradient: the fill is not launched when the flushes in
+    between come (nothing there names its buffer); it becomes an immediate of the accumulation.  Reading the buffer, a
+    synchronize(), or an operand pointing into the block bring a waiting fill back in time."""
+    set_diag(dev)
+    rng = np.random.default_rng(41000)
+    n = 50000
+    x = T.contiguous_tensor(rng, O.F32, [n])
+    other = T.contiguous_tensor(rng, O.F32, [64, 32])
+    _, dx = dev.put(x)
+    _, dother = dev.put(other)
+    pg = dev.raw(n * 4)
+    dg = H.kdesc(x, pg)
+    zero, three, five, seven = (np.array([v], np.float32) for v in (0.0, 3.0, 5.0, 7.0))
+    dev.dev.synchronize()
+    dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(dg))
+    pt = dev.raw(other.storage.nbytes)
+    dev.dev.call("transpose", H.ref(dother), H.ref(H.kdesc(T.empty(O.F32, [32, 64]), pt)), 0, 1)   # runs at once: a flush
+    diag = dev.dev.diagnostics()
+    assert diag.ops_recorded == 1 and diag.fallback_ops == 0 and diag.fusible_subgraphs == 0, (diag.ops_recorded, diag.fallback_ops)
+    dev.dev.call("add", H.ref(dg), H.ref(dx), H.ref(dg))                   # grad = grad + x
+    got = dev.fetch(pg, x.storage)
+    diag = dev.dev.diagnostics()
+    assert diag.ops_recorded == 2 and diag.fusible_subgraphs == 1 and diag.fills_absorbed == 1 and diag.fallback_ops == 0, diag.subgraph_summary
+    T.assert_same_bits(got, x.storage + np.float32(0), "0 + x")
+    # read back with nothing else recorded / after a synchronize
+    ph = dev.raw(n * 4)
+    dev.dev.call("fill", three.ctypes.data, O.F32, H.ref(H.kdesc(x, ph)))
+    dev.dev.call("transpose", H.ref(dother), H.ref(H.kdesc(T.empty(O.F32, [32, 64]), pt)), 0, 1)
+    assert np.all(dev.fetch(ph, x.storage) == 3.0)
+    dev.dev.call("fill", five.ctypes.data, O.F32, H.ref(H.kdesc(x, ph)))
+    dev.dev.call("transpose", H.ref(dother), H.ref(H.kdesc(T.empty(O.F32, [32, 64]), pt)), 0, 1)
+    dev.dev.synchronize()
+    host_view = (C.c_float * n).from_address(ph)                             # device memory is host-visible (large BAR)
+    assert host_view[0] == 5.0 and host_view[n - 1] == 5.0
+    # a waiting fill whose buffer is released is never launched; the block is reused at once
+    pk = dev.raw(1 << 20, keep=False)
+    dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(H.kdesc(T.empty(O.F32, [1 << 18]), pk)))
+    dev.dev.call("transpose", H.ref(dother), H.ref(H.kdesc(T.empty(O.F32, [32, 64]), pt)), 0, 1)
+    dev.dev.deallocate(pk)
+    dev.dev.synchronize()
+    # operands that point into the middle of a filled block, and a fill through such a pointer
+    half = 4096
+    big = dev.raw(2 * half * 4)
+    whole = T.empty(O.F32, [2 * half])
+    upper = T.empty(O.F32, [half])
+    dev.dev.call("fill", five.ctypes.data, O.F32, H.ref(H.kdesc(whole, big)))
+    dev.dev.call("transpose", H.ref(dother), H.ref(H.kdesc(T.empty(O.F32, [32, 64]), pt)), 0, 1)
+    pout = dev.raw(half * 4)
+    dev.dev.call("unary", H.ref(H.kdesc(upper, big + half * 4)), H.ref(H.kdesc(upper, pout)))
+    assert np.all(dev.fetch(pout, upper.storage) == -5.0)
+    dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(H.kdesc(upper, big + half * 4)))
+    dev.dev.synchronize()
+    got = dev.fetch(big, whole.storage)
+    assert np.all(got[:half] == 5.0) and np.all(got[half:] == 7.0)
+    dev.release()
