@@ -195,6 +195,15 @@ int32_t aixhip_last_flush_diagnostics(aixhip_device* dev, aixhip_flush_diagnosti
     });
 }
 
+int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint64_t* kernels)
+{
+    return guarded([&] {
+        const auto s = D(dev).batchedLaunchStats();
+        if (launches) *launches = s.first;
+        if (kernels) *kernels = s.second;
+    });
+}
+
 int32_t aixhip_fuse_kernel_cache_stats(aixhip_device* dev, uint64_t* hits, uint64_t* misses)
 {
     return guarded([&] {

@@ -96,6 +96,22 @@ struct DeviceHIP::Extras {
     std::string key;
     std::vector<uint64_t> args;
     gen::Space space;
+    // Consecutive flat kernels of one signature that do not depend on one another (Adam's update of parameter after
+    // parameter, aixOptimizer.hpp:112-140; the per-parameter casts of a mixed-precision step) leave as ONE launch: their
+    // argument blocks travel in a table, each with a share of the grid (AIXHIP_BATCH_FLAT_KERNELS=0 switches it off).
+    struct FlatBatch {
+        std::string key;
+        aixk_module* single{nullptr};
+        aixk_module* many{nullptr};
+        size_t words{0};                    // uint64 words per argument block
+        std::vector<uint64_t> table;
+        std::vector<uint32_t> starts;       // first workgroup of each block's share; the total last
+        aixhip::fuse::PointerSet reads, writes;
+        uint32_t count() const { return starts.empty() ? 0 : (uint32_t)starts.size() - 1; }
+        void clear() { table.clear(); starts.clear(); reads.clear(); writes.clear(); single = many = nullptr; words = 0; }
+    } batch;
+    bool batchFlatKernels = [] { const char* e = std::getenv("AIXHIP_BATCH_FLAT_KERNELS"); return !(e && e[0] == '0'); }();
+    uint64_t batchedLaunches{0}, batchedKernels{0};
     // row reductions are recorded and fused with the operators around them (AIXHIP_FUSE_ROW_REDUCTIONS=0 switches it off)
     bool fuseRowReductions = [] { const char* e = std::getenv("AIXHIP_FUSE_ROW_REDUCTIONS"); return !(e && e[0] == '0'); }();
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
@@ -239,11 +255,18 @@ void DeviceHIP::setFuseConfig(const FuseConfig& cfg)
     FuseCallbacks cb;
     cb.emitFused = [this](const FusedSubgraphDescriptor& d) { emitFused(d); };
     cb.emitSingle = [this](const OpRecord& op) { emitSingle(op); };
-    cb.finishFlush = [] {};
+    cb.finishFlush = [this] { issueFlatBatch(); };
     cb.getKernelCacheStats = [this] { return fuseKernelCacheStats(); };
     cb.blockBase = [this](const void* p) { return m_blocks.baseOf(p); };
-    m_engine = std::make_unique<FuseEngine>(cfg, std::move(cb));
+    FuseConfig own = cfg;
+    own.loneCastsAsKernels = m_extras->batchFlatKernels;    // so that runs of them leave as one launch (issueFlatBatch)
+    m_engine = std::make_unique<FuseEngine>(own, std::move(cb));
     m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) m_engine->retainBuffer(base); });
+}
+
+std::pair<size_t, size_t> DeviceHIP::batchedLaunchStats() const
+{
+    return {(size_t)m_extras->batchedLaunches, (size_t)m_extras->batchedKernels};
 }
 
 std::pair<size_t, size_t> DeviceHIP::fuseKernelCacheStats() const
@@ -396,7 +419,8 @@ void DeviceHIP::flush() { flushWindow(true); }
 void DeviceHIP::flushWindow(bool final)
 {
     issueMatmulGroup();                                     // pending products were called before anything now in the window was recorded
-    m_engine->flush(final);
+    try { m_engine->flush(final); }
+    catch (...) { m_extras->batch.clear(); throw; }
     releaseLimbo();
 }
 
@@ -595,6 +619,7 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
 // ---- planner callbacks -------------------------------------------------------------------------
 void DeviceHIP::emitSingle(const OpRecord& op)
 {
+    issueFlatBatch();
     issueMatmulGroup();
     aixhip_tensor a, b, o;
     markTouched(op.output.data);
@@ -752,12 +777,65 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     else { items = n; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
     uint64_t grid = (items + perBlock - 1) / perBlock;
     grid = std::max<uint64_t>(1, std::min(grid, cap));
+
+    auto& B = ex.batch;
+    if (shape == gen::Shape::Flat && ex.batchFlatKernels) {
+        // joins the kernels waiting to leave together, or starts the next such run
+        bool joins = B.count() != 0 && B.key == ex.key && B.count() < 256 && (uint64_t)B.starts.back() + grid < (1u << 30) &&
+                     (B.table.size() + ex.args.size()) * sizeof(uint64_t) < (200u << 10);
+        if (joins) {
+            for (size_t k = 0; k < NI && joins; ++k) if (B.writes.contains(d.inputBuffers[k].data)) joins = false;
+            for (size_t k = 0; k < NO && joins; ++k)
+                if (B.writes.contains(d.outputBuffers[k].data) || B.reads.contains(d.outputBuffers[k].data)) joins = false;
+        }
+        if (!joins) issueFlatBatch();
+        if (B.count() == 0) { B.key = ex.key; B.single = mod; B.words = ex.args.size(); B.starts.push_back(0); }
+        else if (!B.many) {
+            ex.key += "|many";
+            auto many = ex.kernels.find(ex.key);
+            if (many != ex.kernels.end()) { B.many = many->second; ++ex.hits; }
+            else {
+                int32_t cached = 0;
+                const std::string src = gen::source(d, shape, bmask, noAlias, streamOut, true);
+                check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), (gen::entryName(d, shape) + "_many").c_str(), &B.many, &cached));
+                ex.kernels.emplace(ex.key, B.many);
+                ++ex.misses;
+            }
+        }
+        B.table.insert(B.table.end(), ex.args.begin(), ex.args.end());
+        B.starts.push_back(B.starts.back() + (uint32_t)grid);
+        for (size_t k = 0; k < NI; ++k) B.reads.insert(d.inputBuffers[k].data);
+        for (size_t k = 0; k < NO; ++k) B.writes.insert(d.outputBuffers[k].data);
+        return;
+    }
+    issueFlatBatch();
     check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
+}
+
+// The flat kernels that wait in the batch (emitFused) leave: alone as an ordinary launch, several as one launch of the
+// kernel's many-blocks form.  Everything else that enqueues work during a flush calls this first.
+void DeviceHIP::issueFlatBatch()
+{
+    auto& B = m_extras->batch;
+    const uint32_t count = B.count();
+    if (count == 0) return;
+    struct Clear { Extras::FlatBatch& b; ~Clear() { b.clear(); } } clear{B};
+    if (count == 1) {
+        check(aixk_rtc_launch(m_ctx, B.single, B.starts[1], gen::kBlock, B.table.data(), B.words * sizeof(uint64_t)));
+        return;
+    }
+    const size_t startsOffset = B.table.size() * sizeof(uint64_t);
+    B.table.resize(B.table.size() + (B.starts.size() * sizeof(uint32_t) + 7) / 8);
+    std::memcpy((char*)B.table.data() + startsOffset, B.starts.data(), B.starts.size() * sizeof(uint32_t));
+    check(aixk_rtc_launch_many(m_ctx, B.many, gen::kBlock, B.table.data(), B.table.size() * sizeof(uint64_t), startsOffset, count));
+    ++m_extras->batchedLaunches;
+    m_extras->batchedKernels += count;
 }
 
 // A fused kernel that holds row reductions: a wave or a workgroup per row (hipgen.hpp: row programs).
 void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
 {
+    issueFlatBatch();
     auto& ex = *m_extras;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     gen::RowGeometry geo;

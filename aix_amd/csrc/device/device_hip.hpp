@@ -102,6 +102,7 @@ public:
     const aixhip::fuse::FuseConfig& fuseConfig() const { return m_engine->config(); }
     const aixhip::fuse::FlushDiagnostics& lastFlushDiagnostics() const { return m_engine->lastFlushDiagnostics(); }
     std::pair<size_t, size_t> fuseKernelCacheStats() const;                  // hits, misses (aixDeviceMetal's test hook)
+    std::pair<size_t, size_t> batchedLaunchStats() const;                    // launches that carried several flat kernels, kernels carried
     void flush();                                                            // plan + enqueue, no wait
     aixk_ctx* kernelContext() const { return m_ctx; }
     size_t cachedBytes() const { return m_pooledBytes; }
@@ -161,6 +162,7 @@ private:
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void emitSingle(const aixhip::fuse::OpRecord& op);
     void emitRowProgram(const aixhip::fuse::FusedSubgraphDescriptor& d);
+    void issueFlatBatch();
     bool recordRowReduction(aixhip::fuse::OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init);
     void issueMatmulGroup();                                 // the pending matmul calls as one launch (see matmul())
 

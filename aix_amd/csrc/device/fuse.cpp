@@ -1050,7 +1050,8 @@ void FuseEngine::flush(bool final)
     for (const auto& e : plan.emits()) {
         if (!e.fused) { m_callbacks.emitSingle(window[e.index]); ++singles; continue; }
         const auto& g = plan.group(e.index);
-        if (plan.emitsAsSingle(g)) { m_callbacks.emitSingle(window[g.ops[0]]); ++singles; continue; }
+        const bool castKernel = m_config.loneCastsAsKernels && g.ops.size() == 1 && window[g.ops[0]].type == OpType::Cast;
+        if (plan.emitsAsSingle(g) && !castKernel) { m_callbacks.emitSingle(window[g.ops[0]]); ++singles; continue; }
         plan.describe(g, m_descriptor);
         if (m_descriptor.outputBuffers.empty()) continue;          // nothing of it is ever read: dead code
         m_callbacks.emitFused(m_descriptor);

@@ -13,6 +13,7 @@
 
 #include "aix_compat.hpp"
 
+#include <algorithm>
 #include <array>
 #include <cstdint>
 #include <cstring>
@@ -48,6 +49,7 @@ struct FuseConfig {
     size_t flushThreshold        = 200;    // recorded ops that trigger planning
     size_t maxBufferSlots        = 0;      // pointer arguments one fused kernel may take (must be > 0)
     bool   supportsStridedFusion = true;   // may fused kernels read broadcast / strided views
+    bool   loneCastsAsKernels    = false;  // a cast with no company is emitted as a one-operator kernel (emitFused), not as a single
     bool   deferIdleFills        = true;   // a fill nothing else in its window touches waits for its first user (see flush())
 };
 
@@ -181,6 +183,7 @@ public:
     bool contains(const void* p) const;
     void insert(const void* p);
     void erase(const void* p);
+    void clear() { if (m_used) { std::fill(m_slots.begin(), m_slots.end(), (uintptr_t)0); m_count = m_used = 0; } }
     size_t size() const { return m_count; }
 
 private:

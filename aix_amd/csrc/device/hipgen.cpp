@@ -177,8 +177,9 @@ std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t br
     return s;
 }
 
-std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut)
+std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut, bool many)
 {
+    if (many && shape != Shape::Flat) throw std::invalid_argument("only flat kernels have a many-blocks form");
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d), NT = triCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
     if (d.opParams.size() != 3 * NT) throw std::invalid_argument("fused kernel: tril / triu without its parameters");
@@ -208,8 +209,18 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     if (shape != Shape::Flat) o << "    u64 chunks;\n    u64 rank;\n    u64 shape[" << kMaxDims << "];\n    u64 off[" << AI << "];\n    u64 str[" << AI << "][" << kMaxDims << "];\n";
     o << "};\n\n";
 
-    o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << entryName(d, shape) << "(Args a)\n{\n"
-      << "    T s[" << AS << "];\n";
+    if (many) {
+        // one launch for several argument blocks: the workgroup finds the block whose share of the grid it is in
+        o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << entryName(d, shape) << "_many(const Args* table, const u32* starts, u32 count)\n{\n"
+          << "    u32 lo = 0, hi = count;\n"
+          << "    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (starts[mid] <= blockIdx.x) lo = mid; else hi = mid; }\n"
+          << "    const Args a = table[lo];\n"
+          << "    const u32 BID = blockIdx.x - starts[lo], GDIM = starts[lo + 1] - starts[lo];\n";
+    } else {
+        o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << entryName(d, shape) << "(Args a)\n{\n"
+          << "    const u32 BID = blockIdx.x, GDIM = gridDim.x;\n    (void)BID; (void)GDIM;\n";
+    }
+    o << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
     for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = (const I" << k << "*)a.in[" << k << "];\n";
@@ -227,7 +238,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         }
         for (size_t k = 0; k < NO; ++k) o << "    vec<O" << k << ", VEC>*" << rs << " q" << k << " = (vec<O" << k << ", VEC>*)out" << k << ";\n";
         o << "    const u64 nvec = a.n / VEC;\n"
-          << "    for (u64 v = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; v < nvec; v += (u64)gridDim.x * " << kBlock << ") {\n";
+          << "    for (u64 v = (u64)BID * " << kBlock << " + threadIdx.x; v < nvec; v += (u64)GDIM * " << kBlock << ") {\n";
         for (size_t k = 0; k < NI; ++k) if (!bc(k)) o << "        const vec<I" << k << ", VEC> r" << k << " = p" << k << "[v];\n";
         for (size_t k = 0; k < NO; ++k) o << "        vec<O" << k << ", VEC> w" << k << ";\n";
         if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(v * VEC, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
@@ -243,7 +254,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         for (size_t k = 0; k < NO; ++k) o << "        store_sel<AIX_NT>(q" << k << " + v, w" << k << ");\n";
         o << "    }\n"
           << "    const u64 done = nvec * VEC;\n"
-          << "    if (blockIdx.x == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
+          << "    if (BID == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
         if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(i, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
         for (size_t k = 0; k < NI; ++k) {
             if (bc(k)) o << "        x[" << k << "] = b" << k << ";\n";

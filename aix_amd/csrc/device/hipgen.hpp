@@ -30,8 +30,12 @@ std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint3
 // The same text written into `out` (cleared first; its capacity is reused from call to call).
 void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut = false);
 
-// Source of `extern "C" __global__ void <entryName>(Args)`.
-std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false);
+// Source of `extern "C" __global__ void <entryName>(Args)`.  many (flat shape only): of
+// `<entryName>_many(const Args* table, const u32* starts, u32 count)` instead -- the same body for `count` argument
+// blocks in one launch, workgroups [starts[k], starts[k + 1]) working on table[k] (Adam's update of every parameter,
+// the per-parameter casts of a mixed-precision step).
+std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false,
+                   bool many = false);
 
 // ---- row programs (descriptor.rowLength > 0) ------------------------------------------------------------------------
 // A kernel that works row by row on [rows, rowLength] data: a wave (rows shorter than 2048 elements) or a workgroup per

@@ -318,6 +318,29 @@ int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const c
     return AIXK_OK;
 }
 
+int32_t aixk_rtc_launch_many(aixk_ctx* ctx, aixk_module* mod, uint32_t block_x, const void* table, size_t table_bytes,
+                             size_t starts_offset, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(mod && mod->m.fn, "rtc_launch_many: null kernel");
+    AIXK_REQUIRE(table && count > 0 && block_x > 0 && block_x <= 1024, "rtc_launch_many: bad arguments");
+    AIXK_REQUIRE(starts_offset % 4 == 0 && starts_offset + ((size_t)count + 1) * 4 <= table_bytes && table_bytes <= (256u << 10),
+                 "rtc_launch_many: table of %zu bytes, starts at %zu, %u blocks", table_bytes, starts_offset, count);
+    const uint32_t* starts = (const uint32_t*)((const char*)table + starts_offset);
+    for (uint32_t k = 0; k < count; ++k) AIXK_REQUIRE(starts[k] < starts[k + 1], "rtc_launch_many: empty or unordered share %u", k);
+    AIXK_REQUIRE(starts[0] == 0, "rtc_launch_many: the first share starts at workgroup %u", starts[0]);
+    void* host = nullptr;
+    const void* dev = nullptr;
+    AIXK_TRY(aixk::table_slot(ctx, table_bytes, &host, &dev));
+    std::memcpy(host, table, table_bytes);
+    AIXK_TRY(aixk::table_upload(ctx, host, dev, table_bytes));
+    struct { uint64_t table; uint64_t starts; uint32_t count; uint32_t pad; } args{(uint64_t)(uintptr_t)dev, (uint64_t)(uintptr_t)dev + starts_offset, count, 0};
+    size_t size = sizeof(args);
+    void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &size, HIP_LAUNCH_PARAM_END};
+    AIXK_HIP(hipModuleLaunchKernel(mod->m.fn, starts[count], 1, 1, block_x, 1, 1, 0, ctx->stream, nullptr, config));
+    return AIXK_OK;
+}
+
 int32_t aixk_rtc_launch(aixk_ctx* ctx, aixk_module* mod, uint32_t grid_x, uint32_t block_x, const void* args, size_t args_bytes)
 {
     AIXK_TRY(set_device(ctx));

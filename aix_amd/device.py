@@ -57,6 +57,7 @@ _SIGNATURES = {
     "aixhip_set_fuse_config": [_P, C.POINTER(FuseConfig)],
     "aixhip_last_flush_diagnostics": [_P, C.POINTER(FlushDiagnostics)],
     "aixhip_fuse_kernel_cache_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "aixhip_batched_launch_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "aixhip_memory_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
 }
 _OTHER = {
@@ -166,6 +167,11 @@ class Device:
         h, m = C.c_uint64(), C.c_uint64()
         check(self.lib.aixhip_fuse_kernel_cache_stats(self.handle, C.byref(h), C.byref(m)))
         return h.value, m.value
+
+    def batched_launch_stats(self):
+        n, k = C.c_uint64(), C.c_uint64()
+        check(self.lib.aixhip_batched_launch_stats(self.handle, C.byref(n), C.byref(k)))
+        return n.value, k.value
 
     def kernel_context(self):
         return _P(self.lib.aixhip_kernel_context(self.handle))

@@ -66,6 +66,7 @@ _SIGNATURES = {
     "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],
     "aixk_rtc_get": [_P, C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_P), C.POINTER(C.c_int32)],
     "aixk_rtc_launch": [_P, _P, C.c_uint32, C.c_uint32, _P, C.c_size_t],
+    "aixk_rtc_launch_many": [_P, _P, C.c_uint32, _P, C.c_size_t, C.c_size_t, C.c_uint32],
     "aixk_rtc_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "aixk_event_create": [_P, C.POINTER(_P)],
     "aixk_event_record": [_P, _P],

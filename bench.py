@@ -403,7 +403,7 @@ def main():
         from oracle import drivers as OD
         cfg = (6, 768, 12, 512, 16, 8192)
         data = OD.transformer_data(*cfg)
-        t_steps = 4
+        t_steps = 8
         tokens = cfg[3] * cfg[4]
         d, v, s_len, layers = cfg[1], cfg[5], cfg[3], cfg[0]
         # forward products: 12 d^2 per token and layer (qkv, out, MLP), 2 s d per token and layer (scores, mix, causal half
@@ -416,7 +416,8 @@ def main():
             if "c4" not in chosen and ("c4stack" if stacked else "c4loop") not in chosen:
                 continue
             losses, norms, secs = GD.transformer(dev, cfg, t_steps, data, stacked=stacked)
-            steady = float(secs[1:].mean())
+            steady = float(np.median(secs[2:]))               # the first steps compile kernels and warm the allocator up
+            print(f"configs[4] stacked={stacked} step times ms: {[round(float(x) * 1e3, 2) for x in secs]}", file=sys.stderr)
             tf = {"workload": "configs[4] decoder-only transformer forward+backward: 6 layers, d 768, 12 heads, seq 512, batch 16, vocab 8192, "
                               f"GELU MLP 4x, LayerNorm, {how}, bf16 activations, f32 masters",
                   "ms_per_step": round(steady * 1e3, 2), "value": round(tokens / steady, 1), "unit": "tokens/s",

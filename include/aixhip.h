@@ -137,6 +137,9 @@ typedef struct aixhip_flush_diagnostics {
 int32_t aixhip_last_flush_diagnostics(aixhip_device* dev, aixhip_flush_diagnostics* out);
 /* DeviceMetal::fuseKernelCacheStats (Targets/AIXTests/DeviceTests.cpp:1774-1807). */
 int32_t aixhip_fuse_kernel_cache_stats(aixhip_device* dev, uint64_t* hits, uint64_t* misses);
+/* Launches that carried several generated kernels of one signature at once (Adam's update of parameter after parameter
+ * as one launch), and how many kernels they carried, since the device was created.  No counterpart in the reference. */
+int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint64_t* kernels);
 /* The kernel-layer context of this device (stream, events) for timing with aixk_event_*. */
 aixk_ctx* aixhip_kernel_context(aixhip_device* dev);
 int32_t aixhip_memory_stats(aixhip_device* dev, uint64_t* live_bytes, uint64_t* cached_bytes);

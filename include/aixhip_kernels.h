@@ -179,6 +179,15 @@ int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const c
 /* Launch with a packed kernel-argument block (aixDeviceMetalKernelGen.cpp:772-857). */
 int32_t aixk_rtc_launch(aixk_ctx* ctx, aixk_module* mod, uint32_t grid_x, uint32_t block_x,
                         const void* args, size_t args_bytes);
+/* One launch for `count` argument blocks of one kernel body.  The module's entry must have the form
+ * `extern "C" __global__ void f(const Args* table, const uint32_t* starts, uint32_t count)`: `table` (host memory here,
+ * `table_bytes` of it) holds the `count` argument blocks back to back and, `starts_offset` bytes in, count + 1 uint32 --
+ * the first workgroup of every block's share of the grid and, last, the grid size.  The table is copied to device
+ * memory in stream order; the host's copy may be reused as soon as the call returns.  AIXK_EINVAL if the table exceeds
+ * 256 KiB or the shares are not in ascending order.  No counterpart in the reference, whose Adam updates one parameter
+ * per dispatch (aixOptimizer.hpp:112-140). */
+int32_t aixk_rtc_launch_many(aixk_ctx* ctx, aixk_module* mod, uint32_t block_x, const void* table, size_t table_bytes,
+                             size_t starts_offset, uint32_t count);
 /* The device-side header every generated kernel is compiled against (types, conversions, math). */
 const char* aixk_rtc_prelude(void);
 int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);

@@ -931,6 +931,59 @@ static void testIdleFillsWaitForTheirFirstUser()
     }
 }
 
+static void testLoneCastsAsKernelsAndTheManyBlocksForm()
+{
+    // the per-parameter casts of a mixed-precision step: each a one-operator kernel of one signature, so that the device
+    // can send them off together; the many-blocks form of a flat kernel compiles
+    Capture cap;
+    FuseConfig c = config();
+    c.loneCastsAsKernels = true;
+    FuseEngine e(c, cap.callbacks());
+    for (uintptr_t k = 0; k < 3; ++k) {
+        auto src = T(1 + 2 * k, {100 + 28 * k}), dst = T(2 + 2 * k, {100 + 28 * k}, DataType::kBFloat16);
+        e.retainBuffer(src.data); e.retainBuffer(dst.data);
+        e.record(OpType::Cast, View(src), View(dst));
+    }
+    e.flush();
+    CHECK(cap.fused.size() == 3 && cap.singles.empty());
+    if (cap.fused.size() != 3) return;
+    const std::string sig = gen::signature(cap.fused[0], gen::Shape::Flat, 0, true);
+    CHECK(sig == gen::signature(cap.fused[1], gen::Shape::Flat, 0, true) && sig == gen::signature(cap.fused[2], gen::Shape::Flat, 0, true));
+    CHECK(compiles(cap.fused[0], gen::Shape::Flat));
+    const auto& d = cap.fused[0];
+    const std::string src = gen::source(d, gen::Shape::Flat, 0, true, false, true);
+    CHECK(src.find(gen::entryName(d, gen::Shape::Flat) + "_many(const Args* table, const u32* starts, u32 count)") != std::string::npos);
+    hiprtcProgram prog;
+    const char* names[] = {"aix_device.h"};
+    const char* texts[] = {g_prelude.c_str()};
+    CHECK(hiprtcCreateProgram(&prog, src.c_str(), "m.hip", 1, texts, names) == HIPRTC_SUCCESS);
+    const char* opts[] = {"--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off"};
+    const hiprtcResult r = hiprtcCompileProgram(prog, 4, opts);
+    if (r != HIPRTC_SUCCESS) {
+        size_t n = 0; hiprtcGetProgramLogSize(prog, &n);
+        std::string log(n, 0); if (n) hiprtcGetProgramLog(prog, &log[0]);
+        std::printf("---- hipRTC log ----\n%s\n---- source ----\n%s\n", log.c_str(), src.c_str());
+    }
+    CHECK(r == HIPRTC_SUCCESS);
+    hiprtcDestroyProgram(&prog);
+    bool threw = false;
+    try { (void)gen::source(d, gen::Shape::Rows, 0, true, false, true); } catch (const std::invalid_argument&) { threw = true; }
+    CHECK(threw);
+    // the chain of the benchmark in its many-blocks form
+    Capture chain;
+    FuseEngine f(config(), chain.callbacks());
+    recordChain(f, 1.0f, 0.5f, true);
+    f.flush();
+    CHECK(chain.fused.size() == 1);
+    if (chain.fused.size() == 1) {
+        const std::string many = gen::source(chain.fused[0], gen::Shape::Flat, 0, true, false, true);
+        hiprtcProgram p2;
+        CHECK(hiprtcCreateProgram(&p2, many.c_str(), "m2.hip", 1, texts, names) == HIPRTC_SUCCESS);
+        CHECK(hiprtcCompileProgram(p2, 4, opts) == HIPRTC_SUCCESS);
+        hiprtcDestroyProgram(&p2);
+    }
+}
+
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::printf("usage: test_planner <path to aix_device.h>\n"); return 2; }
@@ -961,6 +1014,7 @@ int main(int argc, char** argv)
     testSoftmaxBecomesOneRowProgram();
     testLayerNormPiecesShareOneRowProgram();
     testIdleFillsWaitForTheirFirstUser();
+    testLoneCastsAsKernelsAndTheManyBlocksForm();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

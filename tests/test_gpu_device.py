@@ -648,3 +648,63 @@ def test_idle_fills_wait_for_their_first_user(dev):
     got = dev.fetch(big, whole.storage)
     assert np.all(got[:half] == 5.0) and np.all(got[half:] == 7.0)
     dev.release()
+
+
+def test_runs_of_equal_flat_kernels_leave_as_one_launch(dev):
+    """Adam's update of parameter after parameter (aixOptimizer.hpp:112-140), the per-parameter casts of a
+    mixed-precision step: generated flat kernels of one signature that do not depend on one another are sent off in one
+    launch, each with its own argument block and share of the grid.  Results against the oracle operator by operator
+    (exact: multiply and add, correctly rounded on both sides); sizes from one element to a million, ragged tails."""
+    set_diag(dev)
+    rng = np.random.default_rng(42000)
+    sizes = [1, 3, 4, 5, 255, 256, 1000, 4096, 65537, 1 << 20, 7, 300000]
+    before = dev.dev.batched_launch_stats()
+    nodes = []
+    recs = [Recorder(dev, O.F32, [n]) for n in sizes]
+    leaves = [rec.leaf(T.contiguous_tensor(rng, O.F32, [n])) for rec, n in zip(recs, sizes)]      # (uploads flush: all of them first)
+    for rec, x in zip(recs, leaves):
+        y = rec.binary(O.ADD, rec.binary(O.MUL, x, rec.scalar(2.0)), rec.scalar(1.0))
+        nodes.append((rec, y))
+    for rec, y in nodes:
+        rec.free_temps(keep=(y,))
+    got = [dev.fetch(y["ptr"], y["host"].storage) for _, y in nodes]
+    after = dev.dev.batched_launch_stats()
+    assert after[0] - before[0] == 1 and after[1] - before[1] == len(sizes), (before, after)
+    for (rec, y), g, n in zip(nodes, got, sizes):
+        T.assert_same_bits(g, y["host"].storage, f"2x + 1 over {n} elements, batched")
+    dev.release()
+    # kernels that depend on one another stay apart: z = 2y + 1 reads the y of the kernel before it
+    rec = Recorder(dev, O.F32, [5000])
+    x = rec.leaf(T.contiguous_tensor(rng, O.F32, [5000]))
+    y = rec.binary(O.ADD, rec.binary(O.MUL, x, rec.scalar(2.0)), rec.scalar(1.0))
+    dev.dev.flush()
+    before = dev.dev.batched_launch_stats()
+    chain = [y]
+    for _ in range(3):
+        # each link is recorded after a use of the previous result outside the kernel, so that it is a kernel of its own
+        chain.append(rec.binary(O.ADD, rec.binary(O.MUL, chain[-1], rec.scalar(2.0)), rec.scalar(1.0)))
+    got = dev.fetch(chain[-1]["ptr"], chain[-1]["host"].storage)
+    T.assert_same_bits(got, chain[-1]["host"].storage, "three dependent links")
+    for link in chain[:-1]:
+        T.assert_same_bits(dev.fetch(link["ptr"], link["host"].storage), link["host"].storage, "a link's own result")
+    dev.release()
+    # casts of several tensors (f32 -> bf16, bf16 -> f32): one launch each way, values as the single operator gives them
+    srcs = [T.contiguous_tensor(rng, O.F32, [n], lo=-300, hi=300) for n in (10, 513, 70000, 8)]
+    before = dev.dev.batched_launch_stats()
+    outs = []
+    for s in srcs:
+        ps, _ = dev.put(s)
+        pd = dev.raw(s.size * 2)
+        outs.append(pd)
+    dev.dev.synchronize()
+    ptrs = [dev.live[-2 * len(srcs) + 2 * k] for k in range(len(srcs))]
+    for s, ps, pd in zip(srcs, ptrs, outs):
+        dev.dev.call("copy", ps, O.F32, pd, O.BF16, s.size)
+    got = [dev.fetch(pd, np.zeros(s.size, np.uint16)) for s, pd in zip(srcs, outs)]
+    after = dev.dev.batched_launch_stats()
+    assert after[0] - before[0] == 1 and after[1] - before[1] == len(srcs), (before, after)
+    for s, g in zip(srcs, got):
+        want = np.zeros(s.size, np.uint16)
+        assert CPU.copy(s.storage.ctypes.data, O.F32, want.ctypes.data, O.BF16, s.size) == 0
+        T.assert_same_bits(g, want, f"f32 -> bf16 over {s.size} elements, batched")
+    dev.release()
