@@ -59,7 +59,12 @@ def _compare(dev, shape, steps, threads=16, envelope=False):
 
 
 def test_small_mlp_100_steps(dev):
+    before = dev.batched_launch_stats()
     _compare(dev, (64, 48, 32, 10), 100)
+    launches, kernels = (a - b for a, b in zip(dev.batched_launch_stats(), before))
+    print(f"launches that carried several kernels: {launches}, kernels carried: {kernels}")
+    # Adam's update (aixOptimizer.hpp:112-140) of the six parameters: one launch per step, not six
+    assert launches >= 100 and kernels >= 500          # (one parameter's update shares its kernel with the end of backward)
 
 
 def test_ragged_mlp(dev):
