@@ -8,6 +8,7 @@
 
 #include <algorithm>
 #include <array>
+#include <cstdio>
 #include <cstring>
 #include <cstdlib>
 #include <deque>
@@ -87,6 +88,10 @@ int unaryCode(OpType t)
 
 } // namespace
 
+// AIXHIP_TRACE=1: one line on stderr per kernel or operator the device enqueues (what ran, in which order, how large).
+static const bool kTrace = [] { const char* e = std::getenv("AIXHIP_TRACE"); return e && e[0] == '1'; }();
+#define AIXHIP_TRACE(...) do { if (kTrace) { std::fprintf(stderr, "[aixhip] " __VA_ARGS__); std::fputc('\n', stderr); } } while (0)
+
 struct DeviceHIP::Extras {
     std::deque<Cooling> cooling;
     unsigned flushesSinceEvent{0};
@@ -110,6 +115,7 @@ struct DeviceHIP::Extras {
         uint32_t count() const { return starts.empty() ? 0 : (uint32_t)starts.size() - 1; }
         void clear() { table.clear(); starts.clear(); reads.clear(); writes.clear(); single = many = nullptr; words = 0; }
     } batch;
+    std::vector<aixk_fill_item> smallFills;   // consecutive fills of small live buffers (the rank-0 constants of an expression): one launch
     bool batchFlatKernels = [] { const char* e = std::getenv("AIXHIP_BATCH_FLAT_KERNELS"); return !(e && e[0] == '0'); }();
     uint64_t batchedLaunches{0}, batchedKernels{0};
     // row reductions are recorded and fused with the operators around them (AIXHIP_FUSE_ROW_REDUCTIONS=0 switches it off)
@@ -420,12 +426,13 @@ void DeviceHIP::flushWindow(bool final)
 {
     issueMatmulGroup();                                     // pending products were called before anything now in the window was recorded
     try { m_engine->flush(final); }
-    catch (...) { m_extras->batch.clear(); throw; }
+    catch (...) { m_extras->batch.clear(); m_extras->smallFills.clear(); throw; }
     releaseLimbo();
 }
 
 void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
 {
+    AIXHIP_TRACE("-- operator outside the planner (%zu recorded)", m_engine->pendingOps());
     for (const void* p : {a, b, c}) {
         if (!p) continue;
         m_engine->recordExternalRead(p);
@@ -619,8 +626,26 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
 // ---- planner callbacks -------------------------------------------------------------------------
 void DeviceHIP::emitSingle(const OpRecord& op)
 {
-    issueFlatBatch();
+    const bool smallFill = (op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels;
+    if (!smallFill || m_extras->batch.count()) issueFlatBatch();            // (a fill joins the fills before it)
     issueMatmulGroup();
+    AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
+    if ((op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels) {
+        // small fills that follow one another leave together (issueFlatBatch sends them off ahead of whatever comes next)
+        aixk_fill_item item{};
+        uint8_t bytes[8] = {};
+        const size_t esz = op.type == OpType::Fill ? aixhip::fuse::convertScalarInto(op.scalarData.data(), op.scalarDType, op.output.dtype, bytes)
+                                                   : aixhip::fuse::lowestScalarInto(op.output.dtype, bytes);
+        std::memcpy(&item.bits, bytes, esz);
+        item.dst = (char*)op.output.data + op.output.offset * esz;
+        item.elements = (uint32_t)op.output.size;
+        item.element_size = (uint32_t)esz;
+        markTouched(op.output.data);
+        for (const auto& f : m_extras->smallFills)
+            if (f.dst == item.dst) { issueFlatBatch(); break; }             // a second fill of the same buffer comes after the first
+        m_extras->smallFills.push_back(item);
+        return;
+    }
     aixhip_tensor a, b, o;
     markTouched(op.output.data);
     markTouched(op.input0.data);
@@ -778,6 +803,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     uint64_t grid = (items + perBlock - 1) / perBlock;
     grid = std::max<uint64_t>(1, std::min(grid, cap));
 
+    AIXHIP_TRACE("%s  %llu elements, %zu in %zu out", gen::entryName(d, shape).c_str(), (unsigned long long)n, NI, NO);
     auto& B = ex.batch;
     if (shape == gen::Shape::Flat && ex.batchFlatKernels) {
         // joins the kernels waiting to leave together, or starts the next such run
@@ -816,6 +842,11 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 // kernel's many-blocks form.  Everything else that enqueues work during a flush calls this first.
 void DeviceHIP::issueFlatBatch()
 {
+    if (!m_extras->smallFills.empty()) {
+        auto& fills = m_extras->smallFills;
+        struct Clear { std::vector<aixk_fill_item>& f; ~Clear() { f.clear(); } } clearFills{fills};
+        check(aixk_fill_many(m_ctx, fills.data(), (uint32_t)fills.size()));
+    }
     auto& B = m_extras->batch;
     const uint32_t count = B.count();
     if (count == 0) return;
@@ -865,6 +896,7 @@ void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
         ++ex.misses;
     }
     gen::packRowArgsInto(ex.args, d, inPtr, outPtr);
+    AIXHIP_TRACE("%s  rows of %zu, %zu elements, %zu in %zu out", gen::rowEntryName(d, geo).c_str(), d.rowLength, d.elementCount, NI, NO);
     const uint64_t rows = d.elementCount / d.rowLength;
     const uint64_t rowsPerBlock = geo.lanes == 64 ? gen::kBlock / 64 : 1;
     uint64_t grid = (rows + rowsPerBlock - 1) / rowsPerBlock;
@@ -875,6 +907,7 @@ void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
 // ---- operators that run at once ------------------------------------------------------------------
 void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    AIXHIP_TRACE("sum");
     requireDevice(result, "sum");
     flushFor(a.data, result.data);
     aixhip_tensor pa, pr; stagedPod(a, &pa, "sum"); toPod(result, &pr, "sum");
@@ -883,6 +916,7 @@ void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& resul
 
 void DeviceHIP::max(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    AIXHIP_TRACE("max");
     requireDevice(result, "max");
     flushFor(a.data, result.data);
     aixhip_tensor pa, pr; stagedPod(a, &pa, "max"); toPod(result, &pr, "max");
@@ -917,6 +951,7 @@ void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorPar
 void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& result)
 {
     requireDevice(result, "matmul");
+    AIXHIP_TRACE("matmul rank %zu, %zu x %zu elements", a.shape.size(), a.size, b.size);
     auto& ex = *m_extras;
     const bool sixteen = result.dtype == DataType::kFloat16 || result.dtype == DataType::kBFloat16;
     if (sixteen && a.shape.size() == 2 && b.shape.size() == 2 && result.shape.size() == 2 && a.dtype == result.dtype && b.dtype == result.dtype &&
@@ -987,6 +1022,7 @@ void DeviceHIP::issueMatmulGroup()
 
 void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)
 {
+    AIXHIP_TRACE("transpose");
     requireDevice(result, "transpose");
     flushFor(a.data, result.data);
     aixhip_tensor pa, pr; stagedPod(a, &pa, "transpose"); toPod(result, &pr, "transpose");
@@ -1028,6 +1064,7 @@ void DeviceHIP::copyImmediate(const void* src, DataType srcDType, void* dst, Dat
 
 void DeviceHIP::contiguous(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    AIXHIP_TRACE("contiguous");
     requireDevice(dst, "contiguous");
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "contiguous"); toPod(dst, &pd, "contiguous");
@@ -1092,6 +1129,7 @@ bool DeviceHIP::recordRowReduction(OpType type, const DeviceTensorParams& src, c
 
 void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    AIXHIP_TRACE("reduceTo");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::reduceTo() requires matching source and destination data types.");
     requireDevice(dst, "reduceTo");
     uint64_t init = 0;
@@ -1104,6 +1142,7 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
 
 void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    AIXHIP_TRACE("maxTo");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::maxTo() requires matching source and destination data types.");
     requireDevice(dst, "maxTo");
     uint64_t init = 0;
@@ -1116,6 +1155,7 @@ void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& d
 
 void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
 {
+    AIXHIP_TRACE("argmaxTo");
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxTo");
     flushFor(src.data, dst.data);
@@ -1125,6 +1165,7 @@ void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams
 
 void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
 {
+    AIXHIP_TRACE("argmaxIndicesTo");
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndicesTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxIndicesTo");
     // the caller zero-fills the destination right before the call (aixCore.hpp:927-941): a fill still waiting in
@@ -1142,6 +1183,7 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
 
 void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim, size_t start, size_t end, size_t step)
 {
+    AIXHIP_TRACE("sliceSet");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::sliceSet() requires matching source and destination data types.");
     requireDevice(dst, "sliceSet");
     // the backward of a slice fills the destination (zeros of the input's shape) right before the call:
@@ -1191,6 +1233,7 @@ bool DeviceHIP::recordTri(OpType type, const DeviceTensorParams& src, const Devi
 
 void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
 {
+    AIXHIP_TRACE("indexSelect");
     requireDevice(dst, "indexSelect");
     flushFor(src.data, dst.data, indices.data);
     aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexSelect"); toPod(dst, &pd, "indexSelect"); stagedPod(indices, &pi, "indexSelect");
@@ -1199,6 +1242,7 @@ void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorPar
 
 void DeviceHIP::indexAdd(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
 {
+    AIXHIP_TRACE("indexAdd");
     requireDevice(dst, "indexAdd");
     flushFor(src.data, dst.data, indices.data);
     aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexAdd"); toPod(dst, &pd, "indexAdd"); stagedPod(indices, &pi, "indexAdd");

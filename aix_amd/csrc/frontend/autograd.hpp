@@ -12,6 +12,12 @@
 //   * binary operators first bring both operands to the common shape with broadcastTo(), which
 //     is itself a node whose backward is reduceTo() of the seed;
 //   * `tensor op scalar` wraps the scalar in a rank-0 tensor and broadcasts it (:2384-2438).
+//   * a node's value is kept for as long as somebody can still read it: a Tensor handle, the node's own backward
+//     formula (exp, tanh, sqrt) or a consumer's (mul, div, pow, log, max, matmul read their operands).  Once the last
+//     handle is gone and no formula reads it, the storage is released and only shape and type stay -- the sum of a
+//     residual branch, a masked score tensor, the pieces of a LayerNorm need not stay in memory (or be written to it at
+//     all: a fused kernel stores only what is alive).  The reference keeps every intermediate value alive until the
+//     graph dies (aixCore.hpp:1790-1857); the operators issued and their results are the same.
 // Only the operators the training drivers need are present.
 #pragma once
 
@@ -38,6 +44,8 @@ struct Node {
     bool keepDim{false};
     Value indices;
     std::function<void(Node*, const Value&)> backwardFn;
+    int handles{0};                                 // Tensor objects that name this node
+    int readers{0};                                 // backward formulas (its own, its consumers') that read `value`
 
     Node(Value v, bool req) : value(std::move(v)), requireGrad(req) {}
 
@@ -63,9 +71,20 @@ struct Node {
         return m_grad;
     }
 
-    void setBackward(std::vector<NodePtr> in, std::function<void(Node*, const Value&)> fn)
+    // readsInputs: bit k set = the formula reads inputs[k]->value; readsOwn: it reads this node's value
+    void setBackward(std::vector<NodePtr> in, std::function<void(Node*, const Value&)> fn, unsigned readsInputs = 0, bool readsOwn = false)
     {
-        if (requireGrad || retainGrad) { inputs = std::move(in); backwardFn = std::move(fn); }
+        if (requireGrad || retainGrad) {
+            inputs = std::move(in); backwardFn = std::move(fn);
+            for (size_t k = 0; k < inputs.size(); ++k) if ((readsInputs >> k) & 1u) ++inputs[k]->readers;
+            if (readsOwn) ++readers;
+        }
+    }
+
+    // The last handle is gone: nobody but a backward formula can read the value any more.
+    void handleReleased()
+    {
+        if (--handles == 0 && readers == 0 && !retainGrad && !(isLeaf && requireGrad)) value.releaseStorage();
     }
 
 private:
@@ -75,11 +94,25 @@ private:
 class Tensor {
 public:
     Tensor() = default;
+    Tensor(const Tensor& o) : m_node(o.m_node) { if (m_node) ++m_node->handles; }
+    Tensor(Tensor&& o) noexcept : m_node(std::move(o.m_node)) { o.m_node.reset(); }
+    Tensor& operator=(const Tensor& o)
+    {
+        if (this != &o && m_node != o.m_node) { drop(); m_node = o.m_node; if (m_node) ++m_node->handles; }
+        return *this;
+    }
+    Tensor& operator=(Tensor&& o) noexcept
+    {
+        if (this != &o) { drop(); m_node = std::move(o.m_node); o.m_node.reset(); }
+        return *this;
+    }
+    ~Tensor() { drop(); }
 
     // Leaf from an existing value.
     explicit Tensor(Value v, bool requireGrad = false) : m_node(std::make_shared<Node>(std::move(v), requireGrad))
     {
         m_node->backwardFn = defaultBackward;
+        m_node->handles = 1;
     }
 
     // Leaf filled with one number (aixCore.hpp:1907-1913).
@@ -302,7 +335,7 @@ public:
             }
             if (wants(n->inputs[0])) n->inputs[0]->backward(n->inputs[1]->value * seed);
             if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value * seed);
-        });
+        }, 1);
     }
 
     Tensor operator/(const Tensor& o) const
@@ -312,7 +345,7 @@ public:
             if (wants(n->inputs[0])) n->inputs[0]->backward(seed / n->inputs[1]->value);
             if (wants(n->inputs[1]))
                 n->inputs[1]->backward(-n->inputs[0]->value * seed / (n->inputs[1]->value * n->inputs[1]->value));
-        });
+        }, 2);
     }
 
     Tensor operator-() const
@@ -341,7 +374,7 @@ public:
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
             n->inputs[0]->backward(seed * n->value);
-        });
+        }, 0, true);
         return r;
     }
 
@@ -351,7 +384,7 @@ public:
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
             n->inputs[0]->backward(seed / n->inputs[0]->value);
-        });
+        }, 1);
         return r;
     }
 
@@ -361,7 +394,7 @@ public:
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
             n->inputs[0]->backward((n->value * n->value).withScalar(&Device::sub, 1.0f, true) * seed);
-        });
+        }, 0, true);
         return r;
     }
 
@@ -374,7 +407,7 @@ public:
             if (n->inputs.size() < 2) return;
             if (wants(n->inputs[0]))
                 n->inputs[0]->backward(seed * n->inputs[1]->value * n->inputs[0]->value.pow(n->inputs[1]->value.withScalar(&Device::sub, 1.0f)));
-        });
+        }, 3);
         return r;
     }
 
@@ -384,7 +417,7 @@ public:
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
             n->inputs[0]->backward(n->value.withScalar(&Device::div, 0.5f, true) * seed);
-        });
+        }, 0, true);
         return r;
     }
 
@@ -430,7 +463,7 @@ public:
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
             n->inputs[0]->backward(seed * n->inputs[0]->value.argmaxIndices(n->dim0));
-        });
+        }, 1);
         return r;
     }
 
@@ -449,7 +482,7 @@ public:
             }
             if (wants(n->inputs[0])) n->inputs[0]->backward(seed.matmul(n->inputs[1]->value.transpose(d0, d1)));
             if (wants(n->inputs[1])) n->inputs[1]->backward(n->inputs[0]->value.transpose(d0, d1).matmul(seed));
-        });
+        }, 3);
         return r;
     }
 
@@ -470,6 +503,7 @@ private:
         r.m_node = std::make_shared<Node>(std::move(v), anyGrad);
         r.m_node->isLeaf = !anyGrad && !anyNonLeaf;
         r.m_node->backwardFn = defaultBackward;
+        r.m_node->handles = 1;
         return r;
     }
 
@@ -480,15 +514,23 @@ private:
         return Tensor(s, Shape{}, device(), dtype(), onLeft && isRequireGrad()).broadcastTo(shape());
     }
 
-    template <class Fwd, class Bwd> Tensor binary(const Tensor& o, Fwd fwd, Bwd bwd) const
+    // reads: which operands' values the backward formula reads: 0 none (add, sub), 1 "the other operand of every
+    // operand that wants a gradient" (mul), 2 "the divisor if anybody wants a gradient, the dividend if the divisor does" (div)
+    template <class Fwd, class Bwd> Tensor binary(const Tensor& o, Fwd fwd, Bwd bwd, int reads = 0) const
     {
         const Shape bc = shape() == o.shape() ? shape() : broadcastShapes(shape(), o.shape());
         const Tensor lhs = broadcastTo(bc), rhs = o.broadcastTo(bc);
         Tensor r = makeResult(fwd(lhs.value(), rhs.value()), isRequireGrad() || o.isRequireGrad(),
                               !lhs.m_node->isLeaf || !rhs.m_node->isLeaf);
-        r.m_node->setBackward({lhs.m_node, rhs.m_node}, bwd);
+        unsigned mask = 0;
+        const bool wl = wants(lhs.m_node), wr = wants(rhs.m_node);
+        if (reads == 1) mask = lhs.m_node == rhs.m_node ? 1u : (wl ? 2u : 0u) | (wr ? 1u : 0u);
+        if (reads == 2) mask = (wl || wr ? 2u : 0u) | (wr ? 1u : 0u);
+        r.m_node->setBackward({lhs.m_node, rhs.m_node}, bwd, mask);
         return r;
     }
+
+    void drop() noexcept { if (m_node) { m_node->handleReleased(); m_node.reset(); } }
 
     NodePtr m_node;
 };

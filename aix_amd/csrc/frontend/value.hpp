@@ -87,6 +87,8 @@ public:
     }
 
     bool defined() const { return (bool)m_store; }
+    // Gives the memory up; shape, strides and type stay readable (what a backward formula needs of a value nobody reads).
+    void releaseStorage() { m_store.reset(); }
     Device* device() const { return m_dev; }
     DataType dtype() const { return m_p.dtype; }
     const Shape& shape() const { return m_p.shape; }
@@ -105,6 +107,7 @@ public:
     // to date: it stays valid while the value lives and is not reshaped.
     const DeviceTensorParams& params() const
     {
+        if (!m_store) throw std::logic_error("aixfe::Value: the value's memory has been released (no backward formula was to read it)");
         m_p.data = data(); m_p.isContiguous = isContiguous(); m_p.size = size();
         return m_p;
     }

@@ -295,6 +295,20 @@ template <class S, class D> __global__ __launch_bounds__(kBlock) void fill_cvt_v
     if (blockIdx.x == 0 && done + threadIdx.x < n) out[done + threadIdx.x] = s;
 }
 
+// Small fills of one launch (aixk_fill_many): workgroup k writes item k.
+struct FillItems { static constexpr int kMost = 32; u64 dst[kMost]; u64 bits[kMost]; u32 n[kMost]; u32 esz[kMost]; };
+__global__ __launch_bounds__(kBlock) void fill_items_k(FillItems it)
+{
+    const u32 k = blockIdx.x, n = it.n[k], esz = it.esz[k];
+    const u64 bits = it.bits[k];
+    for (u32 i = threadIdx.x; i < n; i += kBlock) {
+        if (esz == 1) ((u8*)it.dst[k])[i] = (u8)bits;
+        else if (esz == 2) ((u16*)it.dst[k])[i] = (u16)bits;
+        else if (esz == 4) ((u32*)it.dst[k])[i] = (u32)bits;
+        else ((u64*)it.dst[k])[i] = bits;
+    }
+}
+
 template <class T> __global__ void fill_min_k(T* __restrict__ out, u64 n)
 {
     const T v = lowest<T>();
@@ -365,6 +379,25 @@ int32_t aixk_fill(aixk_ctx* ctx, const void* scalar, int scalar_dtype, const aix
             return (int)AIXK_OK;
         });
     });
+}
+
+int32_t aixk_fill_many(aixk_ctx* ctx, const aixk_fill_item* items, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(items != nullptr || count == 0, "fill_many: null items");
+    for (uint32_t at = 0; at < count; at += FillItems::kMost) {
+        FillItems it{};
+        const uint32_t now = count - at < (uint32_t)FillItems::kMost ? count - at : (uint32_t)FillItems::kMost;
+        for (uint32_t k = 0; k < now; ++k) {
+            const aixk_fill_item& f = items[at + k];
+            AIXK_REQUIRE(f.dst != nullptr && (f.element_size == 1 || f.element_size == 2 || f.element_size == 4 || f.element_size == 8) &&
+                         f.elements <= 65536 && ((uintptr_t)f.dst % f.element_size) == 0, "fill_many: bad item %u", at + k);
+            it.dst[k] = (u64)(uintptr_t)f.dst; it.bits[k] = f.bits; it.n[k] = f.elements; it.esz[k] = f.element_size;
+        }
+        hipLaunchKernelGGL(fill_items_k, dim3(now), dim3(kBlock), 0, ctx->stream, it);
+        AIXK_HIP(hipGetLastError());
+    }
+    return AIXK_OK;
 }
 
 int32_t aixk_fill_min(aixk_ctx* ctx, const aixhip_tensor* out)

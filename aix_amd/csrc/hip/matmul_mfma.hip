@@ -25,6 +25,8 @@
 
 #include "common.hpp"
 
+#include <cstdio>
+#include <cstdlib>
 #include <algorithm>
 #include <type_traits>
 
@@ -1142,7 +1144,7 @@ int launch_small16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b
 constexpr int tile16_bk(int bm) { return bm == 64 ? 64 : 32; }
 
 // gemm_tile16_k on the last two dims of a / b, `batch` as for launch_small16.  tile: 0 = 64 x 64, 1 = 128 x 64,
-// 2 = 128 x 128; splits: K splits wanted (1 = none).  -1: a layout the kernel does not take.
+// 2 = 128 x 128, 3 = 128 x 192, 4 = 192 x 128; splits: K splits wanted (1 = none).  -1: a layout the kernel does not take.
 int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch,
                   int tile, uint64_t splits, const u64* table = nullptr)
 {
@@ -1168,7 +1170,7 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         bt.sc = M * N;
         bt.table = table;
     }
-    const uint64_t bm = tile == 0 ? 64 : 128, bn = tile == 2 ? 128 : 64;
+    const uint64_t bm = tile == 0 ? 64 : tile == 4 ? 192 : 128, bn = tile == 2 || tile == 4 ? 128 : tile == 3 ? 192 : 64;
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
     g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
@@ -1207,6 +1209,8 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
     auto by_tile = [&](auto dtype_tag) {
         if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{});
         if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{});
+        if (tile == 3) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 192>{});
+        if (tile == 4) return by_form(dtype_tag, std::integral_constant<int, 192>{}, std::integral_constant<int, 128>{});
         return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{});
     };
     const int rc = out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
@@ -1242,6 +1246,11 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, table ? 1 : splits_for(t12864 * count, (K + 31) / 32, 2), table);
         return launch_tile16(ctx, a, b, out, batch, 2, table ? 1 : splits_for(t128 * count, (K + 31) / 32, 2), table);
     }
+    if (const char* force = std::getenv("AIXK_PROBE_TILE16")) {       // probe: "tile" or "tile,splits"
+        int tile = 2; unsigned long long sp = 1;
+        std::sscanf(force, "%d,%llu", &tile, &sp);
+        return launch_tile16(ctx, a, b, out, nullptr, tile, sp);
+    }
     if (K >= 4096 && t128 < 2 * cus && M >= 128 && N >= 128) {
         // a long K and few tiles (weight gradients): 128 x 128 tiles, K split over workgroups.  Splits shorten every
         // workgroup's chain of K steps, as long as the workgroups still find a compute unit each (a second round of
@@ -1251,13 +1260,29 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         // 512^2 x K 8192 and [2048, 1024] x K 16384 (3, 2, 6, 2, 6, 4, 3, 8, 2 splits).
         const uint64_t steps = (K + 31) / 32, most = std::max<uint64_t>(1, std::min<uint64_t>(steps / 16, 16));
         const double mb = (double)M * (double)N * 4e-6;
+        // Workgroups per compute unit -> cost of a K step of all of them, in steps of one workgroup alone: two share a
+        // compute unit at 1.5 (they cover each other's barriers), a third and every further pair queue behind
+        // ([768, 8192] x [8192, 8192] on 128 x 128 tiles: 0.45 us per step alone, 0.69 at 1.5 per unit, 1.17 at 3).
+        auto sharing = [](uint64_t per_unit) { return per_unit <= 1 ? 1.0 : per_unit == 2 ? 1.5 : per_unit % 2 ? 1.5 * (double)(per_unit - 1) / 2 + 1.0 : 1.5 * (double)per_unit / 2; };
         uint64_t splits = 1;
+        int tile = 2;
         double least = 0.0;
-        for (uint64_t sp = 1; sp <= most; ++sp) {
-            const double cost = (double)((t128 * sp + cus - 1) / cus) * (double)((steps + sp - 1) / sp) + (sp > 1 ? (double)sp * mb : 0.0);
-            if (sp == 1 || cost < least) { least = cost; splits = sp; }
+        // The same sum for 128 x 192 and 192 x 128 tiles where they divide the result (the widths of a d = 768 model are
+        // multiples of 192, not of 256); a step of theirs costs 1.47 steps of a 128 x 128 tile (0.66 us against 0.45).  They win where their count
+        // fills the chip in whole rounds and 128 x 128 tiles leave half a round: [768, 8192] x [8192, 8192] 185 -> 147 us
+        // (192 x 128, 2 splits), [8192, 8192] x [8192, 768] 194 -> 145 us (128 x 192, 2 splits); elsewhere the 128 x 128
+        // choice stays unless another is a twentieth cheaper.
+        for (int cand = 2; cand <= 4; ++cand) {
+            if (cand == 3 && (N % 192 != 0 || M % 128 != 0)) continue;
+            if (cand == 4 && (M % 192 != 0 || N % 128 != 0)) continue;
+            const uint64_t tiles = cand == 2 ? t128 : cand == 3 ? (M / 128) * (N / 192) : (M / 192) * (N / 128);
+            const double weight = cand == 2 ? 1.0 : 1.47;
+            for (uint64_t sp = 1; sp <= most; ++sp) {
+                const double cost = weight * sharing((tiles * sp + cus - 1) / cus) * (double)((steps + sp - 1) / sp) + (sp > 1 ? (double)sp * mb : 0.0);
+                if ((cand == 2 && sp == 1) || cost < least * (cand == tile ? 1.0 : 0.95)) { least = cost; splits = sp; tile = cand; }
+            }
         }
-        return launch_tile16(ctx, a, b, out, nullptr, 2, splits);
+        return launch_tile16(ctx, a, b, out, nullptr, tile, splits);
     }
     if (t64 < 2 * cus) {
         // outputs that 64 x 64 tiles cannot spread over the chip twice: with a long K, 64 x 64 tiles and K split over

@@ -19,6 +19,11 @@ class Tensor(C.Structure):
                 ("shape", C.c_uint64 * MAX_RANK), ("strides", C.c_uint64 * MAX_RANK)]
 
 
+class FillItem(C.Structure):
+    """aixk_fill_item"""
+    _fields_ = [("dst", C.c_void_p), ("bits", C.c_uint64), ("elements", C.c_uint32), ("element_size", C.c_uint32)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("large_bar", C.c_int32), ("wavefront", C.c_int32),
@@ -48,6 +53,7 @@ _SIGNATURES = {
     "aixk_unary": [_P, C.c_int, _T, _T],
     "aixk_fill": [_P, _P, C.c_int, _T],
     "aixk_fill_min": [_P, _T],
+    "aixk_fill_many": [_P, _P, C.c_uint32],
     "aixk_cast": [_P, _P, C.c_int, _P, C.c_int, C.c_uint64],
     "aixk_contiguous": [_P, _T, _T],
     "aixk_transpose": [_P, _T, _T, C.c_uint64, C.c_uint64],

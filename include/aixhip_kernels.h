@@ -102,6 +102,12 @@ int32_t aixk_unary(aixk_ctx* ctx, int op, const aixhip_tensor* a, const aixhip_t
 /* Device::fill / fillMin (aixDeviceCPU.cpp:119-138): scalar is HOST memory of scalar_dtype. */
 int32_t aixk_fill(aixk_ctx* ctx, const void* scalar, int scalar_dtype, const aixhip_tensor* out);
 int32_t aixk_fill_min(aixk_ctx* ctx, const aixhip_tensor* out);
+/* `count` small fills in one launch (the rank-0 constants of an expression, `tensor op scalar` of
+ * aixCore.hpp:2384-2438, are filled one Device::fill each): item k writes `elements` copies of the low `element_size`
+ * bytes of `bits` -- the value already in the destination's element type -- from `dst` on.  AIXK_EINVAL for an
+ * element size other than 1, 2, 4, 8 or more than 65536 elements in one item. */
+typedef struct aixk_fill_item { void* dst; uint64_t bits; uint32_t elements; uint32_t element_size; } aixk_fill_item;
+int32_t aixk_fill_many(aixk_ctx* ctx, const aixk_fill_item* items, uint32_t count);
 /* Device::copy (aixDeviceCPU.cpp:407-423): flat converting copy of n elements, both device memory. */
 int32_t aixk_cast(aixk_ctx* ctx, const void* src, int src_dtype, void* dst, int dst_dtype, uint64_t n);
 

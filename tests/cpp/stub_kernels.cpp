@@ -108,6 +108,7 @@ int32_t aixk_rtc_get(aixk_ctx* c, const char*, const char*, const char*, aixk_mo
     return AIXK_OK;
 }
 STUB_OP(aixk_rtc_launch, aixk_module*, uint32_t, uint32_t, const void*, size_t)
+STUB_OP(aixk_fill_many, const aixk_fill_item*, uint32_t)
 STUB_OP(aixk_rtc_launch_many, aixk_module*, uint32_t, const void*, size_t, size_t, uint32_t)
 const char* aixk_rtc_prelude(void) { return ""; }
 int32_t aixk_rtc_stats(aixk_ctx* c, uint64_t* hits, uint64_t* misses) { *hits = c->hits; *misses = c->misses; return AIXK_OK; }
