@@ -1170,14 +1170,14 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         bt.sc = M * N;
         bt.table = table;
     }
-    const uint64_t bm = tile == 0 ? 64 : tile == 4 ? 192 : 128, bn = tile == 2 || tile == 4 ? 128 : tile == 3 ? 192 : 64;
+    const uint64_t bm = tile == 0 ? 64 : tile == 4 ? 192 : 128, bn = tile == 2 || tile == 4 || tile == 5 ? 128 : tile == 3 ? 192 : 64;
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
     g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
     g.tiles_m = (u32)((M + bm - 1) / bm); g.tiles_n = (u32)((N + bn - 1) / bn);
     const u32 n = g.tiles_m * g.tiles_n;
     g.swizzle = n % 8u == 0 ? 1u : 0u;
-    const uint64_t bk = (uint64_t)tile16_bk((int)bm);
+    const uint64_t bk = tile == 5 ? 64 : (uint64_t)tile16_bk((int)bm);
     const uint64_t steps = (K + bk - 1) / bk;
     if (splits > steps) splits = steps;
     if (splits > 64) splits = 64;
@@ -1198,20 +1198,22 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     };
-    auto by_form = [&](auto dtype_tag, auto bm_tag, auto bn_tag) {
+    auto by_form = [&](auto dtype_tag, auto bm_tag, auto bn_tag, auto bk_tag) {
         typedef decltype(dtype_tag) T;
-        constexpr int BM = decltype(bm_tag)::value, BN = decltype(bn_tag)::value, BK = tile16_bk(BM);
+        constexpr int BM = decltype(bm_tag)::value, BN = decltype(bn_tag)::value, BK = decltype(bk_tag)::value ? decltype(bk_tag)::value : tile16_bk(BM);
         if (!at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, false>, Tile16<BM, BN, BK, false, false>::kLds);
         if (!at && tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, true>, Tile16<BM, BN, BK, false, true>::kLds);
         if (at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, true, false>, Tile16<BM, BN, BK, true, false>::kLds);
         return launch(gemm_tile16_k<T, BM, BN, BK, true, true>, Tile16<BM, BN, BK, true, true>::kLds);
     };
     auto by_tile = [&](auto dtype_tag) {
-        if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{});
-        if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{});
-        if (tile == 3) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 192>{});
-        if (tile == 4) return by_form(dtype_tag, std::integral_constant<int, 192>{}, std::integral_constant<int, 128>{});
-        return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{});
+        constexpr std::integral_constant<int, 0> usual{};
+        if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{}, usual);
+        if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, usual);
+        if (tile == 3) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 192>{}, usual);
+        if (tile == 4) return by_form(dtype_tag, std::integral_constant<int, 192>{}, std::integral_constant<int, 128>{}, usual);
+        if (tile == 5) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{});
+        return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, usual);
     };
     const int rc = out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
     if (rc != AIXK_OK || sk.splits == 1) return rc;

@@ -4,8 +4,8 @@ oracle device, plus the same run with 1 % of the second weight matrix moved by o
 measure of how far rounding alone moves this trace on the CPU, which sets the envelope the GPU trace is held to.
 
 The oracle device runs the product's front-end headers on oracle/cpuref (its f32 matmul is the i-k-j reordering of the
-reference's loop nest, bit-identical to it: tests/test_frontend_vs_ref.py, tests/test_oracle_vs_ref.py).  About
-15 minutes per run on 8 cores; run from the repository root:  python tests/golden/make_mlp_c3_trace.py [threads]"""
+reference's loop nest, bit-identical to it: tests/test_frontend_vs_ref.py, tests/test_oracle_vs_ref.py).  Each of the
+two runs takes about 65-80 minutes on 6 threads (38 s per step); run from the repository root:  python tests/golden/make_mlp_c3_trace.py [threads]"""
 import json
 import os
 import sys

@@ -75,3 +75,38 @@ def test_ragged_mlp(dev):
 def test_mnist_shaped_mlp_100_steps(dev):
     """784 -> 256 -> 256 -> 10, batch 512: the configuration's layout at a size the CPU finishes in seconds."""
     _compare(dev, (512, 784, 256, 10), 100, envelope=True)
+
+
+def test_full_size_mlp_against_the_committed_cpu_trace(dev):
+    """The configuration at its real size -- 784 -> 2048 -> 2048 -> 10, batch 4096, 100 steps -- against the per-step
+    losses of the CPU oracle device committed in tests/golden/mlp_c3_trace.json (tests/golden/make_mlp_c3_trace.py
+    wrote it from the same seeded host data; over two hours of CPU time, so it is not rerun here).  The first forward
+    pass (step 0): 1e-5 relative, the bar of its matmuls and reductions (observed 3e-7).  Steps 1-4: 1e-4 -- Adam's first
+    updates have the size of the learning rate whatever the gradient's size (m / sqrt(v) = +-1 after one step), so a
+    gradient entry near zero whose sign differs by rounding moves its weight by twice the learning rate: with 6 million
+    weights the loss of the next steps differs at the 1e-5 level (observed 1.0e-5 at step 2), not at that of the
+    arithmetic.  Whole trace: the envelope the fixture itself measures -- 20 x the deviation of the CPU's own run with
+    1 % of W2 moved by one unit in the last place (never more than 0.1)."""
+    import json
+    import os
+    from aix_amd import drivers as GD
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mlp_c3_trace.json")) as f:
+        fixture = json.load(f)
+    batch, n_in, hidden, n_out = fixture["shape"]
+    assert (batch, n_in, hidden, n_out) == (4096, 784, 2048, 10) and fixture["steps"] == 100
+    want = np.frombuffer(bytes.fromhex("".join(fixture["losses_hex"])), dtype=np.float32).astype(np.float64)
+    assert np.array_equal(want, np.array(fixture["losses"]))
+    other = np.array(fixture["losses_one_ulp_perturbed"])
+    spread = float((np.abs(other - want) / np.abs(want)).max())
+    tol = min(0.1, max(1e-3, 20 * spread))
+    data = OD.mlp_data(batch, n_in, hidden, n_out)
+    got, secs = GD.mlp(dev, batch, n_in, hidden, n_out, fixture["steps"], fixture["lr"], data)
+    rel = np.abs(got.astype(np.float64) - want) / np.abs(want)
+    print(f"full-size MLP x100: loss {want[0]:.6f} -> {want[-1]:.6f} (cpu fixture), {got[-1]:.6f} (gpu); max rel dev {rel.max():.3e} at step "
+          f"{int(rel.argmax())}; first 5 steps {rel[:5].max():.3e}; CPU's own one-ulp spread {spread:.3e} -> tolerance {tol:.3e}; "
+          f"gpu {np.median(secs[1:]) * 1e3:.2f} ms/step against {fixture['cpu_seconds_per_step']:.1f} s/step on {fixture['threads']} CPU threads")
+    print("relative deviation per step:", " ".join(f"{v:.1e}" for v in rel))
+    assert np.all(np.isfinite(got)) and got[-1] < got[0]
+    assert rel[0] <= 1e-5, "first forward pass"
+    assert rel[:5].max() <= 1e-4, "first 5 steps"
+    assert rel.max() <= tol
