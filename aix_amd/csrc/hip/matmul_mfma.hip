@@ -385,6 +385,16 @@ __device__ __forceinline__ u32x4 tr_fragment_lds(const u16* p)
     return u32x4{l.x, l.y, h.x, h.y};
 }
 
+// An address read from a table in memory, as a pointer the compiler knows to be global memory: a pointer made from a
+// plain integer is "flat", every access through it (and through anything selected between it and a kernel argument) is a
+// flat_load that counts against the LDS counter too, and the waits before every LDS operation and barrier then cover
+// the global loads in flight -- the register ring of gemm_tile16_k degenerates to "wait for everything" ([8192, 768] x
+// [768, 768]: 18.6 -> 22.4 us).
+template <class T> __device__ __forceinline__ T* global_ptr(u64 address)
+{
+    return (T*)(__attribute__((address_space(1))) T*)address;
+}
+
 template <bool AT, bool BT> struct Small16 {
     static constexpr int BM = 32, BN = 32, BK = 64, PK = BK + 8, PT = 96;
     static constexpr int SA = AT ? BK * PT : BM * PK, SB = BT ? BK * PT : BN * PK;      // elements per wave
@@ -407,7 +417,7 @@ __global__ __launch_bounds__(256) void gemm_small16_k(GemmArgs g, BatchArgs bt)
     T* C = (T*)g.c;
     if (bt.table) {
         const u64* entry = bt.table + 3 * (u64)blockIdx.y;
-        A = (const u16*)entry[0]; B = (const u16*)entry[1]; C = (T*)entry[2];
+        A = global_ptr<const u16>(entry[0]); B = global_ptr<const u16>(entry[1]); C = global_ptr<T>(entry[2]);
     } else if (bt.rank) {                                    // uniform over the workgroup: scalar arithmetic
         u32 rest = blockIdx.y;
         for (int d = (int)bt.rank - 1; d >= 0; --d) {
@@ -514,7 +524,7 @@ template <int BM, int BN, int BK_, bool AT, bool BT> struct Tile16 {
     static constexpr size_t kLds = (size_t)2 * (SA + SB) * 2;
 };
 
-template <class T, int BM, int BN, int BKT, bool AT, bool BT>
+template <class T, int BM, int BN, int BKT, bool AT, bool BT, int RING = 0>
 __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, SplitArgs sk)
 {
     typedef Tile16<BM, BN, BKT, AT, BT> S;
@@ -535,7 +545,7 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
     const u16* B = (const u16*)g.b;
     if (bt.table) {
         const u64* entry = bt.table + 3 * (u64)blockIdx.y;
-        A = (const u16*)entry[0]; B = (const u16*)entry[1];
+        A = global_ptr<const u16>(entry[0]); B = global_ptr<const u16>(entry[1]);
     } else if (bt.rank) {                                    // uniform over the workgroup: scalar arithmetic
         u32 rest = blockIdx.y;
         for (int d = (int)bt.rank - 1; d >= 0; --d) {
@@ -558,7 +568,7 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
     // "the oldest tile has arrived" from "everything has arrived" (a load under a bounds check is a branch, and behind a
     // branch the compiler waits for every load in flight), and with 4-8 MFMAs per wave and step nothing but that distance
     // covers the latency of a load.  Edge tiles take the checked loads, one step ahead.
-    constexpr int DEPTH = BM * BN >= 128 * 128 ? 2 : 3;            // registers: the 128 x 128 tile keeps three waves per SIMD with 2
+    constexpr int DEPTH = RING ? RING : BM * BN >= 128 * 128 ? 2 : 3;      // registers: the 128 x 128 tile keeps three waves per SIMD with 2
     u32x4 ra[DEPTH][CA], rb[DEPTH][CB];
     auto load_global = [&](u64 k0, u32x4* pa, u32x4* pb) {
 #pragma unroll
@@ -677,7 +687,7 @@ __global__ __launch_bounds__(256) void gemm_tile16_k(GemmArgs g, BatchArgs bt, S
 
     // accumulator element v of lane l: row 8*(v/4) + 4*(l/32) + v%4, column l%32 of its 32x32 tile
     const u64 plane = g.M * g.N;
-    T* C = bt.table ? (T*)bt.table[3 * (u64)blockIdx.y + 2] : (T*)g.c + (u64)blockIdx.y * plane;
+    T* C = bt.table ? global_ptr<T>(bt.table[3 * (u64)blockIdx.y + 2]) : (T*)g.c + (u64)blockIdx.y * plane;
     float* P = sk.splits > 1 ? sk.partial + ((u64)blockIdx.z * sk.matrices + blockIdx.y) * plane : nullptr;
     if (!P && g.N % 8 == 0 && ((size_t)g.c & 15) == 0) {
         // Through LDS (free after the last barrier), each wave on its own 32 x 32 slab: written as the MFMA leaves it (a lane
@@ -1170,14 +1180,14 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         bt.sc = M * N;
         bt.table = table;
     }
-    const uint64_t bm = tile == 0 ? 64 : tile == 4 ? 192 : 128, bn = tile == 2 || tile == 4 || tile == 5 ? 128 : tile == 3 ? 192 : 64;
+    const uint64_t bm = tile == 0 ? 64 : tile == 4 ? 192 : 128, bn = tile == 2 || tile == 4 ? 128 : tile == 3 ? 192 : 64;
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
     g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
     g.tiles_m = (u32)((M + bm - 1) / bm); g.tiles_n = (u32)((N + bn - 1) / bn);
     const u32 n = g.tiles_m * g.tiles_n;
     g.swizzle = n % 8u == 0 ? 1u : 0u;
-    const uint64_t bk = tile == 5 ? 64 : (uint64_t)tile16_bk((int)bm);
+    const uint64_t bk = (uint64_t)tile16_bk((int)bm);
     const uint64_t steps = (K + bk - 1) / bk;
     if (splits > steps) splits = steps;
     if (splits > 64) splits = 64;
@@ -1198,22 +1208,22 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     };
-    auto by_form = [&](auto dtype_tag, auto bm_tag, auto bn_tag, auto bk_tag) {
+    auto by_form = [&](auto dtype_tag, auto bm_tag, auto bn_tag, auto bk_tag, auto ring_tag) {
         typedef decltype(dtype_tag) T;
         constexpr int BM = decltype(bm_tag)::value, BN = decltype(bn_tag)::value, BK = decltype(bk_tag)::value ? decltype(bk_tag)::value : tile16_bk(BM);
-        if (!at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, false>, Tile16<BM, BN, BK, false, false>::kLds);
-        if (!at && tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, true>, Tile16<BM, BN, BK, false, true>::kLds);
-        if (at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, true, false>, Tile16<BM, BN, BK, true, false>::kLds);
-        return launch(gemm_tile16_k<T, BM, BN, BK, true, true>, Tile16<BM, BN, BK, true, true>::kLds);
+        constexpr int RING = decltype(ring_tag)::value;
+        if (!at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, false, RING>, Tile16<BM, BN, BK, false, false>::kLds);
+        if (!at && tb) return launch(gemm_tile16_k<T, BM, BN, BK, false, true, RING>, Tile16<BM, BN, BK, false, true>::kLds);
+        if (at && !tb) return launch(gemm_tile16_k<T, BM, BN, BK, true, false, RING>, Tile16<BM, BN, BK, true, false>::kLds);
+        return launch(gemm_tile16_k<T, BM, BN, BK, true, true, RING>, Tile16<BM, BN, BK, true, true>::kLds);
     };
     auto by_tile = [&](auto dtype_tag) {
         constexpr std::integral_constant<int, 0> usual{};
-        if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{}, usual);
-        if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, usual);
-        if (tile == 3) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 192>{}, usual);
-        if (tile == 4) return by_form(dtype_tag, std::integral_constant<int, 192>{}, std::integral_constant<int, 128>{}, usual);
-        if (tile == 5) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{});
-        return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, usual);
+        if (tile == 0) return by_form(dtype_tag, std::integral_constant<int, 64>{}, std::integral_constant<int, 64>{}, usual, usual);
+        if (tile == 1) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 64>{}, usual, usual);
+        if (tile == 3) return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 192>{}, usual, usual);
+        if (tile == 4) return by_form(dtype_tag, std::integral_constant<int, 192>{}, std::integral_constant<int, 128>{}, usual, usual);
+        return by_form(dtype_tag, std::integral_constant<int, 128>{}, std::integral_constant<int, 128>{}, usual, usual);
     };
     const int rc = out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
     if (rc != AIXK_OK || sk.splits == 1) return rc;
@@ -1248,42 +1258,44 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, table ? 1 : splits_for(t12864 * count, (K + 31) / 32, 2), table);
         return launch_tile16(ctx, a, b, out, batch, 2, table ? 1 : splits_for(t128 * count, (K + 31) / 32, 2), table);
     }
-    if (const char* force = std::getenv("AIXK_PROBE_TILE16")) {       // probe: "tile" or "tile,splits"
-        int tile = 2; unsigned long long sp = 1;
-        std::sscanf(force, "%d,%llu", &tile, &sp);
-        return launch_tile16(ctx, a, b, out, nullptr, tile, sp);
-    }
-    if (K >= 4096 && t128 < 2 * cus && M >= 128 && N >= 128) {
-        // a long K and few tiles (weight gradients): 128 x 128 tiles, K split over workgroups.  Splits shorten every
-        // workgroup's chain of K steps, as long as the workgroups still find a compute unit each (a second round of
-        // workgroups doubles the time), and each adds an f32 copy of the result to write and read back: with a step and
-        // a MB of partial result at the same price (about 0.3 us) the cheapest split count by this sum was the measured
-        // optimum, or within 3 % of it, on [768, 768 | 2304 | 3072 | 8192] x K 8192, 768^2, 1024^2 and 1536^2 x K 4096,
-        // 512^2 x K 8192 and [2048, 1024] x K 16384 (3, 2, 6, 2, 6, 4, 3, 8, 2 splits).
-        const uint64_t steps = (K + 31) / 32, most = std::max<uint64_t>(1, std::min<uint64_t>(steps / 16, 16));
+    // Tiles and K splits by a two-term cost in units of one K step (32 deep) of a lone 128 x 128 workgroup: the steps of the
+    // workgroups that share a compute unit, plus -- with K split over workgroups -- the f32 partial results to write and
+    // add up.  Measured on a d = 768 transformer's products at 8192 tokens (us per step of a lone workgroup: 128 x 128 0.32-0.45
+    // by operand form, 128 x 192 and 192 x 128 1.4 times that; two workgroups on one compute unit take 1.6 steps for a step
+    // of each, a third and every further pair queue behind; a MB of partial result costs 2 steps):
+    //   [8192, 768] x [768, 768]: 384 tiles of 128 x 128 (1.5 per unit) 20.3 us, 256 tiles of 128 x 192 18.5
+    //   [8192, 3072] x [3072, 768]: 60.8 -> 51.6; [8192, 8192] x [8192, 768]: 155.8 -> 135.9 (no split; 2 splits 144)
+    //   [768, 8192] x [8192, 8192]: 160 -> 139 (192 x 128); [768, 8192] x [8192, 768]: 80.8 unsplit, 27.5 with 7 splits
+    //   [768, 8192] x [8192, 3072]: 86.7 unsplit, 63 (128 x 128, 3 splits) / 62 (128 x 192, 5 splits)
+    // The 192-wide tiles enter where they divide the result (the widths of a d = 768 model are multiples of 192, not of
+    // 256); the 128 x 128 choice stays unless another is a twentieth cheaper.
+    auto sharing = [](uint64_t per_unit) { return per_unit <= 1 ? 1.0 : per_unit % 2 ? 1.6 * (double)(per_unit - 1) / 2 + 1.0 : 1.6 * (double)per_unit / 2; };
+    auto cheapest = [&](uint64_t most, int* tile_out) {
+        const uint64_t steps = (K + 31) / 32;
         const double mb = (double)M * (double)N * 4e-6;
-        // Workgroups per compute unit -> cost of a K step of all of them, in steps of one workgroup alone: two share a
-        // compute unit at 1.5 (they cover each other's barriers), a third and every further pair queue behind
-        // ([768, 8192] x [8192, 8192] on 128 x 128 tiles: 0.45 us per step alone, 0.69 at 1.5 per unit, 1.17 at 3).
-        auto sharing = [](uint64_t per_unit) { return per_unit <= 1 ? 1.0 : per_unit == 2 ? 1.5 : per_unit % 2 ? 1.5 * (double)(per_unit - 1) / 2 + 1.0 : 1.5 * (double)per_unit / 2; };
         uint64_t splits = 1;
         int tile = 2;
         double least = 0.0;
-        // The same sum for 128 x 192 and 192 x 128 tiles where they divide the result (the widths of a d = 768 model are
-        // multiples of 192, not of 256); a step of theirs costs 1.47 steps of a 128 x 128 tile (0.66 us against 0.45).  They win where their count
-        // fills the chip in whole rounds and 128 x 128 tiles leave half a round: [768, 8192] x [8192, 8192] 185 -> 147 us
-        // (192 x 128, 2 splits), [8192, 8192] x [8192, 768] 194 -> 145 us (128 x 192, 2 splits); elsewhere the 128 x 128
-        // choice stays unless another is a twentieth cheaper.
         for (int cand = 2; cand <= 4; ++cand) {
             if (cand == 3 && (N % 192 != 0 || M % 128 != 0)) continue;
             if (cand == 4 && (M % 192 != 0 || N % 128 != 0)) continue;
             const uint64_t tiles = cand == 2 ? t128 : cand == 3 ? (M / 128) * (N / 192) : (M / 192) * (N / 128);
-            const double weight = cand == 2 ? 1.0 : 1.47;
+            const double weight = cand == 2 ? 1.0 : 1.4;
             for (uint64_t sp = 1; sp <= most; ++sp) {
-                const double cost = weight * sharing((tiles * sp + cus - 1) / cus) * (double)((steps + sp - 1) / sp) + (sp > 1 ? (double)sp * mb : 0.0);
+                const double cost = weight * sharing((tiles * sp + cus - 1) / cus) * (double)((steps + sp - 1) / sp) + (sp > 1 ? 2.0 * (double)sp * mb : 0.0);
                 if ((cand == 2 && sp == 1) || cost < least * (cand == tile ? 1.0 : 0.95)) { least = cost; splits = sp; tile = cand; }
             }
         }
+        *tile_out = tile;
+        return splits;
+    };
+    if (K >= 4096 && t128 < 2 * cus && M >= 128 && N >= 128) {
+        // a long K and few tiles (weight gradients): K split over workgroups.  Splits shorten every workgroup's chain of K
+        // steps, as long as the workgroups still find a compute unit each, and each adds an f32 copy of the result to write
+        // and read back.
+        int tile = 2;
+        const uint64_t steps = (K + 31) / 32;
+        const uint64_t splits = cheapest(std::max<uint64_t>(1, std::min<uint64_t>(steps / 16, 16)), &tile);
         return launch_tile16(ctx, a, b, out, nullptr, tile, splits);
     }
     if (t64 < 2 * cus) {
@@ -1295,7 +1307,11 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         if (2 * t64 > cus) return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
         return launch_small16(ctx, a, b, out, nullptr);
     }
-    if (t128 >= cus + cus / 2) return launch_tile16(ctx, a, b, out, nullptr, 2, 1);
+    if (t128 >= cus) {                                     // (2048^3: 256 tiles of 128 x 128 27.4 us, 512 of 128 x 64 33.0)
+        int tile = 2;
+        (void)cheapest(1, &tile);
+        return launch_tile16(ctx, a, b, out, nullptr, tile, 1);
+    }
     if (t12864 >= 2 * cus) return launch_tile16(ctx, a, b, out, nullptr, 1, 1);
     return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
 }

@@ -109,27 +109,28 @@ def test_broadcast_add_and_transpose_at_benchmark_size(gpu, big):
 
 
 def _matmul_properties(gpu, dtype, n, layout, rng, tol_rel):
-    """A [n, n] . B [n, n] with A and / or B held transposed in memory (layout 'NN', 'NT', 'TN', 'TT':
-    T = the operand is stored as its transpose and read through a transposed view)."""
-    scale = 1.0 / np.sqrt(n)
-    a_store = O.to_storage(rng.uniform(-scale, scale, n * n), dtype)
-    b_store = O.to_storage(rng.uniform(-1, 1, n * n), dtype)
+    """A [m, k] . B [k, n] (n: one extent for m = k = n, or (m, k, n)) with A and / or B held transposed in memory
+    (layout 'NN', 'NT', 'TN', 'TT': T = the operand is stored as its transpose and read through a transposed view)."""
+    m, k, n = (n, n, n) if isinstance(n, int) else n
+    scale = 1.0 / np.sqrt(k)
+    a_store = O.to_storage(rng.uniform(-scale, scale, m * k), dtype)
+    b_store = O.to_storage(rng.uniform(-1, 1, k * n), dtype)
     a_t, b_t = layout[0] == "T", layout[1] == "T"
-    # logical A[i, k]: stored row-major, or stored as [k, i] and viewed with strides (1, n)
-    A = O.to_float64(a_store, dtype).reshape(n, n)
-    B = O.to_float64(b_store, dtype).reshape(n, n)
+    # logical A[i, k]: stored row-major, or stored as [k, i] and viewed with strides (1, m)
+    A = O.to_float64(a_store, dtype).reshape((k, m) if a_t else (m, k))
+    B = O.to_float64(b_store, dtype).reshape((n, k) if b_t else (k, n))
     if a_t:
         A = A.T
     if b_t:
         B = B.T
-    ha = T.HostTensor(a_store, dtype, [n, n], [1, n] if a_t else None)
-    hb = T.HostTensor(b_store, dtype, [n, n], [1, n] if b_t else None)
+    ha = T.HostTensor(a_store, dtype, [m, k], [1, m] if a_t else None)
+    hb = T.HostTensor(b_store, dtype, [k, n], [1, k] if b_t else None)
     _, da = gpu.put(ha)
     _, db = gpu.put(hb)
-    out = T.empty(dtype, [n, n])
+    out = T.empty(dtype, [m, n])
     po, do = gpu.put(out)
     G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
-    Cg = O.to_float64(gpu.fetch(po, out.storage), dtype).reshape(n, n)
+    Cg = O.to_float64(gpu.fetch(po, out.storage), dtype).reshape(m, n)
 
     # checksum of every element: C . 1 = A . (B . 1); bound = rounding of the output type on sum_j |C_ij| plus
     # the accumulation bound on |A| . (|B| . 1)
@@ -147,7 +148,7 @@ def _matmul_properties(gpu, dtype, n, layout, rng, tol_rel):
     bound = eps_out * np.abs(Cg).sum(axis=0) + tol_rel * mag_cols
     assert np.all(np.abs(got_cols - want_cols) <= bound), f"{NAMES[dtype]} {n}^3 {layout}: column checksum"
     # single entries against float64 dot products
-    idx = rng.integers(0, n, size=(96, 2))
+    idx = np.stack([rng.integers(0, m, size=96), rng.integers(0, n, size=96)], axis=1)
     for i, j in idx:
         want = float(A[i, :] @ B[:, j])
         mag = float(np.abs(A[i, :]) @ np.abs(B[:, j]))
@@ -228,6 +229,20 @@ def test_matmul_mlp_shapes_f32(gpu, case):
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=lambda d: NAMES[d])
 def test_matmul_4096_cubed_16bit(gpu, dtype, layout):
     _matmul_properties(gpu, dtype, 4096, layout, np.random.default_rng(6000 + dtype), 1e-5)
+
+
+# the products of a d = 768 transformer step at 8192 tokens: results of 256-384 tiles (128 x 192 and 192 x 128 tiles where
+# the widths are multiples of 192), weight gradients with K = 8192 split over workgroups, the output projection's gradients
+TRANSFORMER_PRODUCTS = [((8192, 768, 768), "NN"), ((8192, 768, 768), "NT"), ((8192, 768, 768), "TN"), ((8192, 768, 768), "TT"),
+                        ((8192, 3072, 768), "NN"), ((8192, 3072, 768), "NT"), ((8192, 768, 3072), "NN"), ((8192, 768, 3072), "NT"),
+                        ((8192, 8192, 768), "NT"), ((768, 8192, 8192), "TN"), ((768, 8192, 768), "TN"), ((768, 8192, 3072), "TN"),
+                        ((3072, 8192, 768), "TN"), ((2048, 2048, 2048), "NN"), ((1536, 768, 8192), "NN"), ((768, 8192, 8192), "NN")]
+
+
+@pytest.mark.parametrize("shape,layout", TRANSFORMER_PRODUCTS, ids=[f"{s[0]}x{s[1]}x{s[2]}-{l}" for s, l in TRANSFORMER_PRODUCTS])
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=lambda d: NAMES[d])
+def test_matmul_transformer_shapes(gpu, dtype, shape, layout):
+    _matmul_properties(gpu, dtype, shape, layout, np.random.default_rng(6300 + dtype), 1e-5)
 
 
 @pytest.mark.parametrize("layout", ["NN", "NT", "TN"])
