@@ -223,8 +223,8 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     o << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
-    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = (const I" << k << "*)a.in[" << k << "];\n";
-    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = (O" << k << "*)a.out[" << k << "];\n";
+    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = global_ptr<const I" << k << ">((u64)a.in[" << k << "]);\n";
+    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = global_ptr<O" << k << ">((u64)a.out[" << k << "]);\n";
 
     if (shape == Shape::Flat) {
         // One vector of VEC elements per operand per lane (16 bytes of T) and as many workgroups as
@@ -395,8 +395,8 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
-    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = (const I" << k << "*)a.in[" << k << "];\n";
-    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = (O" << k << "*)a.out[" << k << "];\n";
+    for (size_t k = 0; k < NI; ++k) o << "    const I" << k << "* in" << k << " = global_ptr<const I" << k << ">((u64)a.in[" << k << "]);\n";
+    for (size_t k = 0; k < NO; ++k) o << "    O" << k << "* out" << k << " = global_ptr<O" << k << ">((u64)a.out[" << k << "]);\n";
     o << "    const u32 lane = threadIdx.x % G;\n"
       << "    const u64 nvec = a.len / VEC;\n"
       << "    const W lowestW = (W)(-__builtin_huge_val());\n    (void)lowestW;\n";

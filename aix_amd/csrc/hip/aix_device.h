@@ -369,5 +369,15 @@ template <bool NT, class V> __device__ __forceinline__ void store_sel(V* p, cons
     else *p = v;
 }
 
+// An address that arrives as plain data (read from a table in memory, a field of an argument block copied from one), as
+// a pointer the compiler knows to be global memory.  A pointer made from a plain integer is "flat": every access through
+// it is a flat_load / flat_store, which counts against the LDS counter too, so the waits before LDS operations and
+// barriers then cover the global loads in flight (gemm_tile16_k's register ring degenerated to "wait for everything":
+// [8192, 768] x [768, 768] 18.6 -> 22.4 us until its table addresses went through here).
+template <class T> __device__ __forceinline__ T* global_ptr(u64 address)
+{
+    return (T*)(__attribute__((address_space(1))) T*)address;
+}
+
 } // namespace aixd
 #endif

@@ -302,10 +302,10 @@ __global__ __launch_bounds__(kBlock) void fill_items_k(FillItems it)
     const u32 k = blockIdx.x, n = it.n[k], esz = it.esz[k];
     const u64 bits = it.bits[k];
     for (u32 i = threadIdx.x; i < n; i += kBlock) {
-        if (esz == 1) ((u8*)it.dst[k])[i] = (u8)bits;
-        else if (esz == 2) ((u16*)it.dst[k])[i] = (u16)bits;
-        else if (esz == 4) ((u32*)it.dst[k])[i] = (u32)bits;
-        else ((u64*)it.dst[k])[i] = bits;
+        if (esz == 1) global_ptr<u8>(it.dst[k])[i] = (u8)bits;
+        else if (esz == 2) global_ptr<u16>(it.dst[k])[i] = (u16)bits;
+        else if (esz == 4) global_ptr<u32>(it.dst[k])[i] = (u32)bits;
+        else global_ptr<u64>(it.dst[k])[i] = bits;
     }
 }
 

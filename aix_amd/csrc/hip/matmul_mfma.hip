@@ -385,16 +385,6 @@ __device__ __forceinline__ u32x4 tr_fragment_lds(const u16* p)
     return u32x4{l.x, l.y, h.x, h.y};
 }
 
-// An address read from a table in memory, as a pointer the compiler knows to be global memory: a pointer made from a
-// plain integer is "flat", every access through it (and through anything selected between it and a kernel argument) is a
-// flat_load that counts against the LDS counter too, and the waits before every LDS operation and barrier then cover
-// the global loads in flight -- the register ring of gemm_tile16_k degenerates to "wait for everything" ([8192, 768] x
-// [768, 768]: 18.6 -> 22.4 us).
-template <class T> __device__ __forceinline__ T* global_ptr(u64 address)
-{
-    return (T*)(__attribute__((address_space(1))) T*)address;
-}
-
 template <bool AT, bool BT> struct Small16 {
     static constexpr int BM = 32, BN = 32, BK = 64, PK = BK + 8, PT = 96;
     static constexpr int SA = AT ? BK * PT : BM * PK, SB = BT ? BK * PT : BN * PK;      // elements per wave

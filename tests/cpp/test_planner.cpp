@@ -952,6 +952,7 @@ static void testLoneCastsAsKernelsAndTheManyBlocksForm()
     CHECK(compiles(cap.fused[0], gen::Shape::Flat));
     const auto& d = cap.fused[0];
     const std::string src = gen::source(d, gen::Shape::Flat, 0, true, false, true);
+    if (std::getenv("AIX_PRINT_MANY_SOURCE")) std::printf("%s\n", src.c_str());
     CHECK(src.find(gen::entryName(d, gen::Shape::Flat) + "_many(const Args* table, const u32* starts, u32 count)") != std::string::npos);
     hiprtcProgram prog;
     const char* names[] = {"aix_device.h"};
