@@ -1297,7 +1297,7 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         if (2 * t64 > cus) return launch_tile16(ctx, a, b, out, nullptr, 0, 1);
         return launch_small16(ctx, a, b, out, nullptr);
     }
-    if (t128 >= cus) {                                     // (2048^3: 256 tiles of 128 x 128 27.4 us, 512 of 128 x 64 33.0)
+    if (2 * t128 >= cus) {                                 // (2048^3: 256 tiles of 128 x 128 27.4 us, 512 of 128 x 64 33.0; 1536^3: 144 tiles 19.6, 576 of 64 x 64 22.1)
         int tile = 2;
         (void)cheapest(1, &tile);
         return launch_tile16(ctx, a, b, out, nullptr, tile, 1);
