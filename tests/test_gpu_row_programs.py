@@ -305,3 +305,112 @@ def test_initial_value_of_the_destination_takes_part(dev):
         assert got_m.min() >= 2.5
         dev.release()
     set_fusion(dev, True)
+
+
+def _random_program(dev, rng, dtype, rows, length, steps, fusion):
+    """One random program of exact operators on small integer values (every sum and product stays exactly representable,
+    so the order of a sum does not matter and all three evaluations must agree bit for bit): full [rows, length] tensors,
+    one-value-per-row tensors from row maxima and row sums (fills folded or not), broadcasts of them, a row vector, scalars,
+    in-place updates, operators that run at once in between (which flush the window), temporaries freed along the way."""
+    set_fusion(dev, fusion)
+    f = Front(dev, dtype)
+    shape, col = [rows, length], [rows, 1]
+    small = lambda n: O.to_storage(rng.integers(-2, 3, n).astype(np.float64), dtype)            # noqa: E731
+    full = [f.leaf(T.HostTensor(small(rows * length), dtype, shape)) for _ in range(3)]
+    cols = [f.leaf(T.HostTensor(small(rows), dtype, col))]
+    vec = f.leaf(T.HostTensor(small(length), dtype, [length]))
+    bound = {id(t): 2.0 for t in full + cols}                        # largest magnitude a tensor can hold
+    limit = 2.0 ** (7 if dtype in (O.F16, O.BF16) else 20)           # 16-bit types: integers up to 256 are exact
+    kept = []
+    for step in range(steps):
+        kind = int(rng.integers(0, 12))
+        x = full[int(rng.integers(0, len(full)))]
+        if kind < 3:                                                 # full op full
+            y = full[int(rng.integers(0, len(full)))]
+            op = int(rng.choice([O.ADD, O.SUB, O.MUL]))
+            b = bound[id(x)] * bound[id(y)] if op == O.MUL else bound[id(x)] + bound[id(y)]
+            if b > limit:
+                continue
+            r = f.binary(op, x, y, shape)
+            bound[id(r)] = b
+            full.append(r)
+        elif kind < 5:                                               # full op (one value per row, broadcast along the row)
+            c = cols[int(rng.integers(0, len(cols)))]
+            op = int(rng.choice([O.ADD, O.SUB, O.MUL]))
+            b = bound[id(x)] * bound[id(c)] if op == O.MUL else bound[id(x)] + bound[id(c)]
+            if b > limit:
+                continue
+            r = f.binary(op, x, f.over_rows(c, shape), shape)
+            bound[id(r)] = b
+            full.append(r)
+        elif kind == 5:                                              # full op row vector / scalar
+            if bound[id(x)] + 2 > limit:
+                continue
+            other = f.row_vector(vec, shape) if rng.integers(0, 2) else f.over_all(f.scalar(float(rng.integers(-2, 3))), shape)
+            r = f.binary(int(rng.choice([O.ADD, O.SUB])), x, other, shape)
+            bound[id(r)] = bound[id(x)] + 2
+            full.append(r)
+        elif kind == 6:
+            r = f.unary(O.NEG, x, shape)
+            bound[id(r)] = bound[id(x)]
+            full.append(r)
+        elif kind < 9:                                               # row maximum / row sum
+            if kind == 7:
+                r = f.row_max(x, shape)
+                bound[id(r)] = bound[id(x)]
+            else:
+                if bound[id(x)] * length > limit:
+                    continue
+                r = f.row_sum(x, shape)
+                bound[id(r)] = bound[id(x)] * length
+            cols.append(r)
+        elif kind == 9:                                              # per-row arithmetic
+            a, c = cols[int(rng.integers(0, len(cols)))], cols[int(rng.integers(0, len(cols)))]
+            if bound[id(a)] + bound[id(c)] > limit:
+                continue
+            r = f.binary(int(rng.choice([O.ADD, O.SUB])), a, c, col)
+            bound[id(r)] = bound[id(a)] + bound[id(c)]
+            cols.append(r)
+        elif kind == 10:                                             # in-place update of an earlier result
+            y = full[int(rng.integers(0, len(full)))]
+            if x is y or bound[id(x)] + bound[id(y)] > limit or not any(x is t for t in f.temps):
+                continue
+            assert CPU.binary(O.ADD, C.byref(x["host"].desc()), C.byref(y["host"].desc()), C.byref(x["host"].desc())) == 0
+            dev.dev.call("add", H.ref(x["desc"]), H.ref(y["desc"]), H.ref(x["desc"]))
+            bound[id(x)] += bound[id(y)]
+        else:                                                        # an operator that runs at once: contiguous copy of a transposed view
+            t_view = T.HostTensor(x["host"].storage, dtype, [length, rows], [1, length])
+            r = f.result([length, rows])
+            assert CPU.contiguous(C.byref(t_view.desc()), C.byref(r["host"].desc())) == 0
+            dev.dev.call("contiguous", H.ref(H.kdesc(t_view, x["ptr"])), H.ref(r["desc"]))
+            kept.append(r)
+        if rng.integers(0, 5) == 0 and len(f.temps) > 4:             # free a temporary nobody will name again
+            victim = f.temps[int(rng.integers(0, len(f.temps)))]
+            if not any(victim is k for k in kept) and victim is not full[-1]:
+                full = [t for t in full if t is not victim]
+                cols = [t for t in cols if t is not victim] or cols
+                if any(t is victim for t in full + cols):
+                    continue
+                f.temps = [t for t in f.temps if t is not victim]
+                dev.free(victim["ptr"])
+    kept += [t for t in (full[-3:] + cols[-2:]) if any(t is k for k in f.temps)]
+    f.free_temps(keep=kept)
+    got = [(dev.fetch(t["ptr"], t["host"].storage), t["host"].storage.copy()) for t in kept]
+    dev.release()
+    return got
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16, O.F64], ids=lambda d: NAMES[d])
+def test_random_programs_with_row_reductions(dev, dtype):
+    for trial in range(10):
+        seed = 9000 + 100 * dtype + trial
+        rows = int(np.random.default_rng(seed).integers(1, 24))
+        length = int(np.random.default_rng(seed + 1).choice([32, 64, 96, 256, 1000 if dtype != O.BF16 else 1024, 2048]))
+        fused = _random_program(dev, np.random.default_rng(seed), dtype, rows, length, 30, True)
+        plain = _random_program(dev, np.random.default_rng(seed), dtype, rows, length, 30, False)
+        assert len(fused) == len(plain) and len(fused) > 0
+        for k, ((g1, want), (g2, _)) in enumerate(zip(fused, plain)):
+            what = f"{NAMES[dtype]} trial {trial} [{rows}, {length}] tensor {k}"
+            T.assert_same_bits(g1, want, "fused vs oracle " + what)
+            T.assert_same_bits(g2, want, "unfused vs oracle " + what)
+    set_fusion(dev, True)
