@@ -59,3 +59,25 @@ def test_stacked_attention_against_per_head_attention_on_the_gpu(dev):
           f"{loop_s[1] * 1e3:.1f} ms/step per head, {stack_s[1] * 1e3:.1f} ms/step stacked")
     assert abs(float(stack_l[0]) - float(loop_l[0])) <= 1e-5 * abs(float(loop_l[0]))
     assert rel.max() <= 1e-3
+
+
+def test_full_size_configuration_both_ways(dev):
+    """The configuration at its real size (6 layers, d 768, 12 heads, seq 512, batch 16, vocab 8192), which no CPU device
+    finishes in a test's time: the program with per-(sequence, head) attention -- the reference's interface as it is,
+    36 000 kernels of the small-product, grouped-launch and row-program paths -- and the program on stacks -- 780 launches
+    of the large-tile paths -- share no GEMM route and no softmax launch shape, and must still agree: loss to 1e-4,
+    every parameter's gradient norm to 1e-2 (the reduced sizes above pin both programs to the CPU device at 2e-2).  The
+    untrained loss is ln(V) / V with the reference's mean over all elements."""
+    from aix_amd import drivers as GD
+    cfg = (6, 768, 12, 512, 16, 8192)
+    data = OD.transformer_data(*cfg)
+    stack_l, stack_n, stack_s = GD.transformer(dev, cfg, 2, data, stacked=True)
+    loop_l, loop_n, loop_s = GD.transformer(dev, cfg, 2, data)
+    assert np.all(np.isfinite(stack_l)) and np.all(np.isfinite(stack_n)) and np.all(np.isfinite(loop_n))
+    big = loop_n > 1e-3 * loop_n.max()
+    rel = np.abs(stack_n.astype(np.float64) - loop_n)[big] / loop_n[big]
+    print(f"{cfg}: loss {loop_l[0]:.7f} (per head) {stack_l[0]:.7f} (stacked), ln(V)/V = {np.log(cfg[5]) / cfg[5]:.7f}; {int(big.sum())} gradient norms, "
+          f"max rel dev {rel.max():.2e}; {loop_s[1] * 1e3:.1f} ms/step per head, {stack_s[1] * 1e3:.1f} ms/step stacked")
+    assert abs(float(stack_l[0]) - np.log(cfg[5]) / cfg[5]) < 0.05 * float(stack_l[0])
+    assert abs(float(stack_l[0]) - float(loop_l[0])) <= 1e-4 * abs(float(loop_l[0]))
+    assert rel.max() <= 1e-2
