@@ -197,6 +197,79 @@ static void stress(unsigned seed, int rounds)
     CHECK(stub_held(ctx) == 0 && stub_allocs(ctx) == stub_frees(ctx));
 }
 
+// The host side of what the device does between the interface and the kernels -- recorded row reductions and row
+// programs, fills that wait for their first user, runs of equal flat kernels and small fills sent off together,
+// operands that point into the middle of a block -- driven with random traffic on the stub layer: what runs (under the
+// sanitizers) is the planner, the generator, the batch tables and the waiting lists; the kernels only count.
+static DeviceTensorParams tensor(void* p, std::vector<size_t> shape, DataType dt = DataType::kFloat32, std::vector<size_t> strides = {}, size_t offset = 0)
+{
+    DeviceTensorParams t;
+    t.data = p; t.dtype = dt; t.shape = shape; t.offset = offset;
+    size_t n = 1;
+    for (auto e : shape) n *= e;
+    t.size = n;
+    if (strides.empty()) { strides.resize(shape.size()); size_t run = 1; for (size_t d = shape.size(); d-- > 0;) { strides[d] = run; run *= shape[d]; } }
+    bool dense = true; size_t run = 1;
+    for (size_t d = shape.size(); d-- > 0;) { if (strides[d] != run) dense = false; run *= shape[d]; }
+    t.strides = strides; t.isContiguous = dense;
+    return t;
+}
+
+static void planner_traffic(unsigned seed, int rounds)
+{
+    DeviceHIP dev;
+    aixk_ctx* ctx = dev.kernelContext();
+    std::mt19937 rng(seed);
+    const size_t rows = 24, len = 256, n = rows * len;
+    std::vector<void*> full, cols;
+    auto fresh_full = [&] { void* p = dev.allocate(n * 4); full.push_back(p); return p; };
+    auto fresh_col = [&] { void* p = dev.allocate(rows * 4); cols.push_back(p); return p; };
+    for (int i = 0; i < 3; ++i) fresh_full();
+    fresh_col();
+    const float zero = 0.0f, two = 2.0f;
+    for (int i = 0; i < rounds; ++i) {
+        const unsigned what = rng() % 100;
+        void* x = full[rng() % full.size()];
+        if (what < 25) {                                               // elementwise, full op full
+            void* y = full[rng() % full.size()];
+            dev.add(tensor(x, {rows, len}), tensor(y, {rows, len}), tensor(fresh_full(), {rows, len}));
+        } else if (what < 35) {                                        // full op (one value per row)
+            void* c = cols[rng() % cols.size()];
+            dev.sub(tensor(x, {rows, len}), tensor(c, {rows, len}, DataType::kFloat32, {1, 0}), tensor(fresh_full(), {rows, len}));
+        } else if (what < 45) {                                        // row maximum / row sum with the fill in front
+            void* c = fresh_col();
+            if (what & 1) { dev.fillMin(tensor(c, {rows, 1})); dev.maxTo(tensor(x, {rows, len}), tensor(c, {rows, 1})); }
+            else { dev.fill(&zero, DataType::kFloat32, tensor(c, {rows, 1})); dev.reduceTo(tensor(x, {rows, len}), tensor(c, {rows, 1})); }
+        } else if (what < 55) {                                        // a fill that may wait; sometimes of a block that dies at once
+            void* p = fresh_full();
+            dev.fill(&two, DataType::kFloat32, tensor(p, {rows, len}));
+            if (what & 1) { dev.deallocate(p); full.pop_back(); }
+        } else if (what < 62) {                                        // small fills in a row (rank-0 constants)
+            for (int k = 0; k < 3; ++k) { void* c = fresh_col(); dev.fill(&two, DataType::kFloat32, tensor(c, {})); }
+        } else if (what < 70) {                                        // runs of equal flat kernels: y_k = -x_k
+            for (int k = 0; k < 4; ++k) dev.unary(tensor(full[rng() % full.size()], {n}), tensor(fresh_full(), {n}));
+        } else if (what < 76) {                                        // an operand inside a block
+            dev.unary(tensor((char*)x + 64 * 4, {len}), tensor(fresh_full(), {len}));
+        } else if (what < 84) {                                        // an operator that runs at once
+            dev.transpose(tensor(x, {rows, len}), tensor(fresh_full(), {len, rows}), 0, 1);
+        } else if (what < 92 && full.size() > 4) {                     // temporaries die
+            const size_t k = 3 + rng() % (full.size() - 3);
+            dev.deallocate(full[k]); full[k] = full.back(); full.pop_back();
+            if (cols.size() > 2) { dev.deallocate(cols.back()); cols.pop_back(); }
+        } else if (what < 97) {
+            dev.flush();
+        } else {
+            dev.synchronize();
+        }
+    }
+    dev.synchronize();
+    CHECK(stub_launches(ctx) > 0);
+    for (void* p : full) dev.deallocate(p);
+    for (void* p : cols) dev.deallocate(p);
+    dev.synchronize();
+    CHECK(dev.allocatedBytes() == 0);
+}
+
 static void test_destruction_returns_everything()
 {
     const long long before = stub_held_everywhere();
@@ -223,10 +296,13 @@ int main(int argc, char** argv)
     test_out_of_memory_retry();
     test_destruction_returns_everything();
     for (unsigned seed = 1; seed <= 4; ++seed) stress(seed, 20000);
+    for (unsigned seed = 21; seed <= 24; ++seed) planner_traffic(seed, 3000);
     if (threads) {
         // one device per thread is the contract (no locks inside a device): two devices side by side must share nothing
         std::thread t1(stress, 11u, 20000), t2(stress, 12u, 20000);
         t1.join(); t2.join();
+        std::thread t3(planner_traffic, 31u, 2000), t4(planner_traffic, 32u, 2000);
+        t3.join(); t4.join();
     }
     CHECK(stub_held_everywhere() == 0);
     if (g_failed) { std::printf("%d allocator checks FAILED\n", g_failed); return 1; }
