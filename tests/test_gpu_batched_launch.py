@@ -1,0 +1,129 @@
+"""The two kernel-layer entry points that carry several pieces of work in one launch, through the C ABI:
+aixk_fill_many (small fills, each item a pattern already in its destination's element type) and aixk_rtc_launch_many
+(several argument blocks of one runtime-compiled kernel, each with its share of the grid).  Results against numpy (fills
+and an exact elementwise body), sizes down to one element and ragged tails, and the argument checks both promise."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import gpuharness as G
+from aix_amd import kernels as K
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    g = G.Gpu()
+    yield g
+    g.close()
+    g.ctx.close()
+
+
+def _items(entries):
+    arr = (K.FillItem * len(entries))()
+    for k, (dst, bits, n, esz) in enumerate(entries):
+        arr[k].dst, arr[k].bits, arr[k].elements, arr[k].element_size = dst, bits, n, esz
+    return arr
+
+
+def test_fill_many_writes_every_item_and_nothing_else(gpu):
+    rng = np.random.default_rng(51000)
+    cases = []      # (pointer to the guarded buffer, elements, element size, pattern)
+    for esz, dtype in ((1, np.uint8), (2, np.uint16), (4, np.uint32), (8, np.uint64)):
+        for n in (1, 2, 255, 256, 257, 4099, 65536):
+            pattern = int(rng.integers(1, 2 ** (8 * esz - 1), dtype=np.uint64))
+            p = gpu.raw((n + 32) * esz)                              # 16 guard elements on either side
+            gpu.ctx.upload(p, np.full(n + 32, 0x5A, dtype=np.uint8).repeat(esz)[: (n + 32) * esz].copy())
+            cases.append((p, n, esz, dtype, pattern))
+    entries = [(p + 16 * esz, pattern, n, esz) for p, n, esz, _, pattern in cases]
+    G.run_gpu(gpu, "aixk_fill_many", _items(entries), len(entries))
+    for p, n, esz, dtype, pattern in cases:
+        got = gpu.fetch(p, np.zeros(n + 32, dtype))
+        guard = np.frombuffer(bytes([0x5A]) * esz, dtype=dtype)[0]
+        assert np.all(got[16:16 + n] == dtype(pattern & (2 ** (8 * esz) - 1))), (n, esz)
+        assert np.all(got[:16] == guard) and np.all(got[16 + n:] == guard), ("guards", n, esz)
+    # 40 items in one call (at most 32 travel with a launch: two launches inside), every one on an address of its own
+    many = [(cases[k % len(cases)][0] + (16 + k // len(cases)) * cases[k % len(cases)][2], k + 1, 1, cases[k % len(cases)][2]) for k in range(40)]
+    G.run_gpu(gpu, "aixk_fill_many", _items(many), len(many))
+    for dst, bits, _, esz in many:
+        got = gpu.fetch(dst, np.zeros(1, {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[esz]))
+        assert int(got[0]) == bits
+    gpu.release()
+
+
+def test_fill_many_checks_its_items(gpu):
+    p = gpu.raw(1 << 20)
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    assert lib.aixk_fill_many(h, _items([(p, 1, 4, 3)]), 1) == 1            # element size 3
+    assert lib.aixk_fill_many(h, _items([(p, 1, 65537, 4)]), 1) == 1        # too many elements for one item
+    assert lib.aixk_fill_many(h, _items([(p + 2, 1, 4, 4)]), 1) == 1        # misaligned for its element size
+    assert lib.aixk_fill_many(h, _items([(None, 1, 4, 4)]), 1) == 1         # null destination
+    assert lib.aixk_fill_many(h, None, 0) == 0                              # nothing to do is fine
+    gpu.ctx.sync()
+    gpu.release()
+
+
+SOURCE = r"""
+#include "aix_device.h"
+using namespace aixd;
+struct Args { const float* x; float* y; float scale; float shift; u64 n; };
+extern "C" __global__ __launch_bounds__(256) void axpb_many(const Args* table, const u32* starts, u32 count)
+{
+    u32 lo = 0, hi = count;
+    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (starts[mid] <= blockIdx.x) lo = mid; else hi = mid; }
+    const Args a = table[lo];
+    const u32 bid = blockIdx.x - starts[lo], gdim = starts[lo + 1] - starts[lo];
+    const float* x = global_ptr<const float>((u64)a.x);
+    float* y = global_ptr<float>((u64)a.y);
+    for (u64 i = (u64)bid * 256 + threadIdx.x; i < a.n; i += (u64)gdim * 256) y[i] = x[i] * a.scale + a.shift;
+}
+"""
+
+
+class Args(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("y", C.c_void_p), ("scale", C.c_float), ("shift", C.c_float), ("n", C.c_uint64)]
+
+
+def _table(blocks, grids):
+    """Argument blocks back to back, then count + 1 uint32: the first workgroup of every share and the grid size."""
+    raw = b"".join(bytes(b) for b in blocks)
+    starts = np.concatenate([[0], np.cumsum(grids)]).astype(np.uint32)
+    return raw + starts.tobytes(), len(raw)
+
+
+def test_launch_many_runs_every_argument_block(gpu):
+    rng = np.random.default_rng(52000)
+    mod = C.c_void_p()
+    cached = C.c_int32()
+    G.run_gpu(gpu, "aixk_rtc_get", b"test|axpb_many", SOURCE.encode(), b"axpb_many", C.byref(mod), C.byref(cached))
+    sizes = [1, 255, 256, 257, 1000, 65537, 3, 300000]
+    xs = [rng.integers(-8, 9, n).astype(np.float32) for n in sizes]               # small integers: a*x + b is exact
+    blocks, grids, outs = [], [], []
+    for k, (n, x) in enumerate(zip(sizes, xs)):
+        px, py = gpu.raw(n * 4), gpu.raw(n * 4)
+        gpu.ctx.upload(px, x)
+        blocks.append(Args(px, py, float(k + 1), float(-k), n))
+        grids.append(max(1, min((n + 255) // 256, 7 + k)))                       # some shares loop, some do not
+        outs.append(py)
+    table, starts_offset = _table(blocks, grids)
+    buf = C.create_string_buffer(table, len(table))
+    G.run_gpu(gpu, "aixk_rtc_launch_many", mod, 256, buf, len(table), starts_offset, len(blocks))
+    buf.raw = b"\0" * len(table)                                                 # the host's copy may be reused as soon as the call returns
+    for k, (x, py) in enumerate(zip(xs, outs)):
+        got = gpu.fetch(py, x)
+        assert np.array_equal(got, x * np.float32(k + 1) + np.float32(-k)), sizes[k]
+    # the checks: shares out of order, a first share that does not start at 0, a table too large, starts outside the table
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    bad, off = _table(blocks[:2], [4, 4])
+    starts = np.frombuffer(bad[off:], np.uint32).copy()
+    for wrong in ([0, 4, 4], [1, 4, 8], [0, 8, 4]):
+        t = bad[:off] + np.array(wrong, np.uint32).tobytes()
+        assert lib.aixk_rtc_launch_many(h, mod, 256, C.create_string_buffer(t, len(t)), len(t), off, 2) == 1, wrong
+    assert lib.aixk_rtc_launch_many(h, mod, 256, C.create_string_buffer(bad, len(bad)), len(bad), off + 8, 2) == 1       # starts run past the end
+    big = b"\0" * ((256 << 10) + 8)
+    assert lib.aixk_rtc_launch_many(h, mod, 256, C.create_string_buffer(big, len(big)), len(big), 0, 1) == 1
+    assert lib.aixk_rtc_launch_many(h, mod, 256, None, 0, 0, 0) == 1
+    gpu.ctx.sync()
+    gpu.release()
