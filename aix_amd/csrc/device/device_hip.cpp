@@ -123,7 +123,9 @@ struct DeviceHIP::Extras {
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
     struct Group { std::vector<aixhip_tensor> a, b, out; };
     std::array<Group, 4> groups;
-    bool anyPending() const { for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
+    // sliceSet calls waiting to leave as one launch (see DeviceHIP::sliceSet)
+    std::vector<aixk_slice_item> slices;
+    bool anyPending() const { if (!slices.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
     // results of at least this many bytes are written with non-temporal stores (the kernel layer's rule, same override)
     size_t streamStoreMinBytes = [] {
         const char* e = std::getenv("AIXHIP_STREAM_STORE_MIN_BYTES");
@@ -234,7 +236,7 @@ DeviceHIP::~DeviceHIP()
     try {
         if (m_engine && m_engine->pendingOps() > 0)
             std::cerr << "DeviceHIP: destroyed with recorded work that was never synchronised." << std::endl;   // aixDeviceMetal.cpp:146-149
-        if (m_ctx && m_extras && m_extras->anyPending()) issueMatmulGroup();           // matmul calls still waiting for company
+        if (m_ctx && m_extras && m_extras->anyPending()) issuePending();           // matmul calls still waiting for company
         if (m_engine) m_engine.reset();
         if (m_ctx) {
             aixk_sync(m_ctx);
@@ -424,7 +426,7 @@ void DeviceHIP::flush() { flushWindow(true); }
 // final: nothing recorded stays behind.  Otherwise fills that nothing recorded so far uses may wait (FuseEngine::flush).
 void DeviceHIP::flushWindow(bool final)
 {
-    issueMatmulGroup();                                     // pending products were called before anything now in the window was recorded
+    issuePending();                                     // pending products were called before anything now in the window was recorded
     try { m_engine->flush(final); }
     catch (...) { m_extras->batch.clear(); m_extras->smallFills.clear(); throw; }
     releaseLimbo();
@@ -628,7 +630,7 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 {
     const bool smallFill = (op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels;
     if (!smallFill || m_extras->batch.count()) issueFlatBatch();            // (a fill joins the fills before it)
-    issueMatmulGroup();
+    issuePending();
     AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
     if ((op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels) {
         // small fills that follow one another leave together (issueFlatBatch sends them off ahead of whatever comes next)
@@ -677,7 +679,7 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 
 void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 {
-    issueMatmulGroup();
+    issuePending();
     constexpr size_t kMaxOperands = 64;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     const size_t esz = dataTypeSize(d.dtype);
@@ -974,7 +976,9 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
                 for (size_t i = 0; independent && i < g.out.size(); ++i)
                     independent = g.out[i].data != pa.data && g.out[i].data != pb.data && g.out[i].data != pr.data &&
                                   g.a[i].data != pr.data && g.b[i].data != pr.data;
-            if (!independent) issueMatmulGroup();
+            for (size_t i = 0; independent && i < ex.slices.size(); ++i)
+                independent = ex.slices[i].dst.data != pa.data && ex.slices[i].dst.data != pb.data && ex.slices[i].dst.data != pr.data && ex.slices[i].src.data != pr.data;
+            if (!independent) issuePending();
             // the group of its shape and operand layout (forward and backward products of attention alternate between
             // two or three of them), or the emptiest slot
             Extras::Group* into = nullptr;
@@ -984,7 +988,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
                 if (g.out[0].dtype == pr.dtype && ga.shape[0] == M && ga.shape[1] == K && gb.shape[1] == N && ga.strides[0] == pa.strides[0] &&
                     ga.strides[1] == pa.strides[1] && gb.strides[0] == pb.strides[0] && gb.strides[1] == pb.strides[1] && g.out.size() < 4096) { into = &g; break; }
             }
-            if (!into) { issueMatmulGroup(); into = &ex.groups[0]; }
+            if (!into) { issuePending(); into = &ex.groups[0]; }
             into->a.push_back(pa); into->b.push_back(pb); into->out.push_back(pr);
             markTouched(a.data); markTouched(b.data); markTouched(result.data);
             return;
@@ -1006,10 +1010,16 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
     check(status);
 }
 
-void DeviceHIP::issueMatmulGroup()
+void DeviceHIP::issuePending()
 {
     auto& ex = *m_extras;
     int status = AIXK_OK;
+    if (!ex.slices.empty()) {
+        status = ex.slices.size() == 1 ? aixk_slice_set(m_ctx, &ex.slices[0].src, &ex.slices[0].dst, ex.slices[0].dim, ex.slices[0].start, ex.slices[0].end, ex.slices[0].step)
+                                       : aixk_slice_set_many(m_ctx, ex.slices.data(), (uint32_t)ex.slices.size());
+        if (ex.slices.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.slices.size(); }
+        ex.slices.clear();
+    }
     for (auto& g : ex.groups) {
         if (g.out.empty()) continue;
         const uint32_t count = (uint32_t)g.out.size();
@@ -1181,6 +1191,13 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
     check(aixk_argmax_to(m_ctx, folded && init == 0 ? 2 : 1, &ps, &pd, dim));
 }
 
+// A cat() is one sliceSet per part into a fresh tensor (aixCore.hpp:1348-1402), the seed of a tensor whose slices were
+// used is one per slice (:2228-2233): runs of calls that copy a few KB each and do not depend on one another.  Like
+// small matmul calls they are not issued at once: a call whose operands lie in device memory waits, and the run leaves
+// as ONE launch when anything else happens.  A call joins the run if it reads nothing a waiting call (sliceSet or
+// matmul) writes and writes nothing a waiting call reads or writes -- two windows of one destination count as apart
+// when the destination is described the same way both times and the windows are ranges of one dim (step 1) that do not
+// overlap; otherwise what waits is issued first.
 void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim, size_t start, size_t end, size_t step)
 {
     AIXHIP_TRACE("sliceSet");
@@ -1190,6 +1207,42 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
     // a fill still waiting in the window becomes the value written outside the slice, in the same pass
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
+    auto& ex = *m_extras;
+    if (!folded && ex.batchFlatKernels && src.size && findBlock(src.data) && findBlock(dst.data) && src.data != dst.data &&
+        src.shape.size() <= AIXK_MAX_RANK && dst.shape.size() <= AIXK_MAX_RANK && dim < dst.shape.size() && step >= 1 && end > start) {
+        aixk_slice_item item{};
+        toPod(src, &item.src, "sliceSet"); toPod(dst, &item.dst, "sliceSet");
+        item.dim = dim; item.start = start; item.end = end; item.step = step;
+        // what aixk_slice_set checks, so that a bad call is reported here and now by the path below
+        const uint64_t count = (end - start + step - 1) / step;
+        uint64_t window = count, whole = 1;
+        for (size_t d = 0; d < dst.shape.size(); ++d) if (d != dim) window *= dst.shape[d];
+        for (size_t d = 0; d < src.shape.size(); ++d) whole *= src.shape[d];
+        if (window == src.size && whole == src.size && start + (count - 1) * step < dst.shape[dim]) {
+            if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {      // recorded producers and users go first
+                m_engine->recordExternalRead(src.data);
+                flushWindow(false);
+            }
+            bool independent = ex.slices.size() < AIXK_SLICE_ITEMS_MAX &&
+                               (ex.slices.empty() || dataTypeSize(static_cast<DataType>(ex.slices[0].src.dtype)) == dataTypeSize(src.dtype));
+            for (const auto& g : ex.groups)
+                for (size_t i = 0; independent && i < g.out.size(); ++i)
+                    independent = g.out[i].data != src.data && g.out[i].data != dst.data && g.a[i].data != dst.data && g.b[i].data != dst.data;
+            for (size_t i = 0; independent && i < ex.slices.size(); ++i) {
+                const aixk_slice_item& w = ex.slices[i];
+                independent = w.dst.data != src.data && w.src.data != dst.data;
+                if (independent && w.dst.data == dst.data) {
+                    independent = w.dim == dim && w.step == 1 && step == 1 && (w.end <= start || end <= w.start) && w.dst.rank == item.dst.rank &&
+                                  w.dst.offset == item.dst.offset && !std::memcmp(w.dst.shape, item.dst.shape, sizeof(item.dst.shape)) &&
+                                  !std::memcmp(w.dst.strides, item.dst.strides, sizeof(item.dst.strides));
+                }
+            }
+            if (!independent) issuePending();
+            ex.slices.push_back(item);
+            markTouched(src.data); markTouched(dst.data);
+            return;
+        }
+    }
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "sliceSet"); toPod(dst, &pd, "sliceSet");
     check(folded ? aixk_slice_set_init(m_ctx, &ps, &pd, dim, start, end, step, init) : aixk_slice_set(m_ctx, &ps, &pd, dim, start, end, step));

@@ -164,7 +164,7 @@ private:
     void emitRowProgram(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void issueFlatBatch();
     bool recordRowReduction(aixhip::fuse::OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init);
-    void issueMatmulGroup();                                 // the pending matmul calls as one launch (see matmul())
+    void issuePending();                                     // the waiting matmul and sliceSet calls, one launch per run (see matmul(), sliceSet())
 
     aixk_ctx* m_ctx{nullptr};
     std::unique_ptr<aixhip::fuse::FuseEngine> m_engine;

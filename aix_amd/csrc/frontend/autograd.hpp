@@ -23,6 +23,8 @@
 
 #include "value.hpp"
 
+#include <algorithm>
+#include <atomic>
 #include <functional>
 #include <unordered_set>
 #include <utility>
@@ -46,6 +48,7 @@ struct Node {
     std::function<void(Node*, const Value&)> backwardFn;
     int handles{0};                                 // Tensor objects that name this node
     int readers{0};                                 // backward formulas (its own, its consumers') that read `value`
+    uint64_t serial{nextSerial()};                  // creation order: a node is always younger than its inputs
 
     Node(Value v, bool req) : value(std::move(v)), requireGrad(req) {}
 
@@ -59,8 +62,50 @@ struct Node {
         if (requireGrad || retainGrad) backwardFn(this, seed);
     }
 
+    // The seed of a slice of this node: `seed` in the window, zero elsewhere (aixCore.hpp:2228-2233).  Single-pass mode
+    // only notes the window; takeSeed() puts all of them together.
+    void backwardWindow(const Value& seed, size_t dim, size_t from, size_t to, size_t step)
+    {
+        if (accumulating()) { windows.push_back({seed, dim, from, to, step}); return; }
+        backward(value.sliceSet(seed, dim, from, to, step));
+    }
+
+    // Single-pass mode: the sum of everything that reached this node, which then holds nothing.  Windows that do not
+    // overlap -- the per-head slices of a projection, the parts a cat() was made of -- are written into ONE tensor of
+    // zeros, a sliceSet of the window's size each; a sum of zero-padded tensors, one per window, holds the same numbers.
+    Value takeSeed()
+    {
+        Value seed = std::move(pending);
+        pending = Value();
+        if (windows.empty()) return seed;
+        std::vector<Window> w = std::move(windows);
+        windows.clear();
+        bool apart = !seed.defined();
+        for (size_t k = 0; apart && k < w.size(); ++k) {
+            apart = w[k].dim == w[0].dim && w[k].step == 1;
+            for (size_t j = 0; apart && j < k; ++j) apart = w[k].to <= w[j].from || w[j].to <= w[k].from;
+        }
+        if (apart) {
+            size_t covered = 0;
+            for (const auto& x : w) covered += x.to - x.from;
+            // windows that leave nothing out (every head of a projection was used): no zeros to start from
+            seed = covered == value.shape()[w[0].dim] ? Value(value.device(), value.dtype(), value.shape())
+                                                      : Value::full(value.device(), value.dtype(), value.shape(), 0.0f);
+            for (const auto& x : w) seed.sliceSetInPlace(x.seed, x.dim, x.from, x.to, x.step);
+            return seed;
+        }
+        for (const auto& x : w) {
+            const Value padded = value.sliceSet(x.seed, x.dim, x.from, x.to, x.step);
+            seed = seed.defined() ? seed + padded : padded;
+        }
+        return seed;
+    }
+
     static bool& accumulating() { static thread_local bool on = false; return on; }
+    static uint64_t nextSerial() { static std::atomic<uint64_t> n{0}; return ++n; }
     Value pending;                                  // sum of the seeds received so far (single-pass mode)
+    struct Window { Value seed; size_t dim, from, to, step; };
+    std::vector<Window> windows;                    // seeds of slices of this node, not yet part of `pending`
 
     Value& grad()
     {
@@ -141,31 +186,28 @@ public:
         m_node->backward(Value::full(device(), dtype(), shape(), 1.0f));
     }
 
-    // Single-pass differentiation: nodes are visited in reverse topological order and each one is
-    // differentiated ONCE with the sum of the seeds that reached it.  The reference has no such mode
-    // (its recursion revisits a node once per path, which is exponential in the number of residual
-    // branches of a transformer); the backward formulas are the same ones, only the traversal differs.
+    // Single-pass differentiation: nodes are visited youngest first -- the reverse of the order the program created
+    // them in, which is a reverse topological order -- and each one is differentiated ONCE with the sum of the seeds
+    // that reached it.  A program written stage by stage (all heads' score products, then all their softmaxes, ...) is
+    // differentiated stage by stage too, so a device that batches runs of equal calls finds the same runs in the
+    // backward pass.  The reference has no such mode (its recursion revisits a node once per path, which is
+    // exponential in the number of residual branches of a transformer); the backward formulas are the same ones,
+    // only the traversal differs.
     void backwardOnce() const
     {
         if (value().size() != 1) throw std::invalid_argument("backward() requires a one-element tensor");
-        std::vector<Node*> order;
-        std::vector<std::pair<Node*, size_t>> stack{{m_node.get(), 0}};
+        std::vector<Node*> order{m_node.get()};
         std::unordered_set<Node*> seen{m_node.get()};
-        while (!stack.empty()) {                      // iterative post-order DFS
-            auto& [n, next] = stack.back();
-            if (next < n->inputs.size()) {
-                Node* in = n->inputs[next++].get();
-                if (seen.insert(in).second) stack.push_back({in, 0});
-            } else { order.push_back(n); stack.pop_back(); }
-        }
+        for (size_t k = 0; k < order.size(); ++k)     // everything the result depends on
+            for (const auto& in : order[k]->inputs)
+                if (seen.insert(in.get()).second) order.push_back(in.get());
+        std::sort(order.begin(), order.end(), [](const Node* a, const Node* b) { return a->serial > b->serial; });
         Node::accumulating() = true;
         try {
             m_node->pending = Value::full(device(), dtype(), shape(), 1.0f);
-            for (size_t k = order.size(); k-- > 0;) {
-                Node* n = order[k];
-                if (!n->pending.defined()) continue;
-                const Value seed = std::move(n->pending);
-                n->pending = Value();
+            for (Node* n : order) {
+                if (!n->pending.defined() && n->windows.empty()) continue;
+                const Value seed = n->takeSeed();
                 if (n->retainGrad) n->grad() += seed;
                 if (n->requireGrad || n->retainGrad) n->backwardFn(n, seed);
             }
@@ -204,7 +246,7 @@ public:
         r.m_node->dim0 = dim; r.m_node->dim1 = step; r.m_node->start = start; r.m_node->end = end;
         r.m_node->setBackward({m_node}, [](Node* n, const Value& seed) {
             if (n->inputs.empty()) return;
-            n->inputs[0]->backward(n->inputs[0]->value.sliceSet(seed, n->dim0, n->start, n->end, n->dim1));
+            n->inputs[0]->backwardWindow(seed, n->dim0, n->start, n->end, n->dim1);
         });
         return r;
     }

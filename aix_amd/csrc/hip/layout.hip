@@ -174,6 +174,24 @@ __global__ __launch_bounds__(kBlock) void copy_views_k(const W* __restrict__ src
         dst[locate<IDX>(dsp, (IDX)i)] = src[locate<IDX>(ssp, (IDX)i)];
 }
 
+// Several such copies in one launch: item k's views and element count come from a table in device memory, its share of
+// the grid from `starts` (count + 1 ascending numbers, the last one the grid size).
+struct CopyItem { u64 src, dst, n, pad; Space<1> ssp, dsp; };
+
+template <class W, class IDX>
+__global__ __launch_bounds__(kBlock) void copy_views_many_k(const CopyItem* __restrict__ items, const u32* __restrict__ starts, u32 count)
+{
+    u32 lo = 0, hi = count;
+    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (starts[mid] <= blockIdx.x) lo = mid; else hi = mid; }
+    const CopyItem& it = items[lo];
+    const u32 first = starts[lo], share = starts[lo + 1] - first;
+    const W* src = global_ptr<const W>(it.src);
+    W* dst = global_ptr<W>(it.dst);
+    const u64 n = it.n;
+    for (u64 i = (u64)(blockIdx.x - first) * kBlock + threadIdx.x; i < n; i += (u64)share * kBlock)
+        dst[locate<IDX>(it.dsp, (IDX)i)] = src[locate<IDX>(it.ssp, (IDX)i)];
+}
+
 // ---- fill + sliceSet in one pass ----------------------------------------------------------------
 // dst is dense: element i is (o, c, e) = (i / (D inner), (i / inner) % D, i % inner) around the sliced dim.
 template <class W, class IDX>
@@ -481,6 +499,55 @@ int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_ten
     AIXK_REQUIRE(start + (window.shape[dim] ? (window.shape[dim] - 1) * step : 0) < dst->shape[dim] || n == 0,
                  "sliceSet: slice exceeds the destination");
     return copy_views(ctx, src, &window, n);
+}
+
+int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    if (count == 0) return AIXK_OK;
+    AIXK_REQUIRE(items, "sliceSet of several items: no items");
+    AIXK_REQUIRE(count <= AIXK_SLICE_ITEMS_MAX, "sliceSet of several items: more than %d items", (int)AIXK_SLICE_ITEMS_MAX);
+    const size_t esz = aixk_dtype_size(items[0].src.dtype);
+    const size_t table_bytes = (size_t)count * sizeof(CopyItem), all_bytes = table_bytes + ((size_t)count + 1) * sizeof(u32);
+    char* host = nullptr;                            // built where the copy engine will read it
+    const char* dev = nullptr;
+    AIXK_TRY(table_slot(ctx, all_bytes, (void**)&host, (const void**)&dev));
+    CopyItem* table = (CopyItem*)host;
+    u32* starts = (u32*)(host + table_bytes);
+    bool small = true;
+    u32 grid = 0;
+    for (uint32_t k = 0; k < count; ++k) {
+        const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
+        const uint64_t dim = items[k].dim, start = items[k].start, end = items[k].end, step = items[k].step;
+        AIXK_REQUIRE(valid_tensor(src) && valid_tensor(dst), "sliceSet: bad operand descriptor");
+        AIXK_REQUIRE(src->dtype == dst->dtype, "sliceSet: element types differ");
+        AIXK_REQUIRE(aixk_dtype_size(src->dtype) == esz, "sliceSet of several items: element sizes differ");
+        AIXK_REQUIRE((int)dim < dst->rank && step > 0 && end >= start, "sliceSet: bad slice");
+        aixhip_tensor window = *dst;
+        window.shape[dim] = (end - start + step - 1) / step;
+        window.offset = dst->offset + start * dst->strides[dim];
+        window.strides[dim] = dst->strides[dim] * step;
+        const uint64_t n = src->size;
+        AIXK_REQUIRE(n > 0 && n == numel(&window) && n == numel(src), "sliceSet: source size does not match the slice");
+        AIXK_REQUIRE(start + (window.shape[dim] - 1) * step < dst->shape[dim], "sliceSet: slice exceeds the destination");
+        CopyItem& it = table[k];
+        it.src = (u64)(uintptr_t)src->data; it.dst = (u64)(uintptr_t)dst->data; it.n = n; it.pad = 0;
+        if (!collapse1(src, &it.ssp) || !collapse1(&window, &it.dsp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
+        small = small && n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(&window) < (1ull << 31);
+        starts[k] = grid;
+        const unsigned share = grid_for(n, kBlock, (unsigned)ctx->cus * 4u);
+        AIXK_REQUIRE((uint64_t)grid + share < (1ull << 31), "sliceSet of several items: grid too large");
+        grid += share;
+    }
+    starts[count] = grid;
+    AIXK_TRY(table_upload(ctx, host, dev, all_bytes));
+    return by_size(items[0].src.dtype, [&](auto tag) {
+        typedef decltype(tag) W;
+        if (small) hipLaunchKernelGGL((copy_views_many_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const CopyItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
+        else hipLaunchKernelGGL((copy_views_many_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const CopyItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
 }
 
 int32_t aixk_slice_set_init(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,

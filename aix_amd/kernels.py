@@ -24,6 +24,11 @@ class FillItem(C.Structure):
     _fields_ = [("dst", C.c_void_p), ("bits", C.c_uint64), ("elements", C.c_uint32), ("element_size", C.c_uint32)]
 
 
+class SliceItem(C.Structure):
+    """aixk_slice_item"""
+    _fields_ = [("src", Tensor), ("dst", Tensor), ("dim", C.c_uint64), ("start", C.c_uint64), ("end", C.c_uint64), ("step", C.c_uint64)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("large_bar", C.c_int32), ("wavefront", C.c_int32),
@@ -58,6 +63,7 @@ _SIGNATURES = {
     "aixk_contiguous": [_P, _T, _T],
     "aixk_transpose": [_P, _T, _T, C.c_uint64, C.c_uint64],
     "aixk_slice_set": [_P, _T, _T, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64],
+    "aixk_slice_set_many": [_P, _P, C.c_uint32],
     "aixk_slice_set_init": [_P, _T, _T, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64],
     "aixk_tri": [_P, C.c_int, _T, _T, C.c_int64],
     "aixk_index_select": [_P, _T, _T, _T, C.c_uint64],

@@ -117,6 +117,14 @@ int32_t aixk_transpose(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tenso
 /* dst is addressed through its offset and strides (the reference GPU device's behaviour). */
 int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst,
                        uint64_t dim, uint64_t start, uint64_t end, uint64_t step);                /* :468-496 */
+/* `count` sliceSet calls in one launch (the parts of a cat(), aixCore.hpp:1348-1402, and the windows the backward pass
+ * of slices writes, :2228-2233, arrive as runs of Device::sliceSet calls that do not depend on one another): item k is
+ * aixk_slice_set(src, dst, dim, start, end, step) of its fields.  All items have one element size; the caller
+ * guarantees that no item reads or overwrites what another one writes.  AIXK_EINVAL for more than
+ * AIXK_SLICE_ITEMS_MAX items, an empty item, or an item aixk_slice_set would reject; nothing is launched then. */
+#define AIXK_SLICE_ITEMS_MAX 512
+typedef struct aixk_slice_item { aixhip_tensor src, dst; uint64_t dim, start, end, step; } aixk_slice_item;
+int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_t count);
 /* The same with the destination's initialisation folded in: dst (dense, offset 0) is written exactly once --
  * `init_bits` (a value of its element type in the low bytes) outside the slice, src inside.  It is what
  * fill(v) followed by sliceSet computes (the backward of a slice: zeros of the input's shape, then the

@@ -78,6 +78,7 @@ STUB_OP(aixk_cast, const void*, int, void*, int, uint64_t)
 STUB_OP(aixk_contiguous, const aixhip_tensor*, const aixhip_tensor*)
 STUB_OP(aixk_transpose, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t)
 STUB_OP(aixk_slice_set, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t, uint64_t, uint64_t)
+STUB_OP(aixk_slice_set_many, const aixk_slice_item*, uint32_t)
 STUB_OP(aixk_slice_set_init, const aixhip_tensor*, const aixhip_tensor*, uint64_t, uint64_t, uint64_t, uint64_t, uint64_t)
 STUB_OP(aixk_tri, int, const aixhip_tensor*, const aixhip_tensor*, int64_t)
 STUB_OP(aixk_index_select, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*, uint64_t)

@@ -1,14 +1,19 @@
-"""The two kernel-layer entry points that carry several pieces of work in one launch, through the C ABI:
-aixk_fill_many (small fills, each item a pattern already in its destination's element type) and aixk_rtc_launch_many
-(several argument blocks of one runtime-compiled kernel, each with its share of the grid).  Results against numpy (fills
-and an exact elementwise body), sizes down to one element and ragged tails, and the argument checks both promise."""
+"""The kernel-layer entry points that carry several pieces of work in one launch, through the C ABI: aixk_fill_many
+(small fills, each item a pattern already in its destination's element type), aixk_rtc_launch_many (several argument
+blocks of one runtime-compiled kernel, each with its share of the grid) and aixk_slice_set_many (several sliceSet calls).
+Results against numpy (fills and an exact elementwise body) and the CPU oracle's sliceSet, sizes down to one element and
+ragged tails, and the argument checks they promise."""
 import ctypes as C
 
 import numpy as np
 import pytest
 
+import aixtest as T
 import gpuharness as G
 from aix_amd import kernels as K
+from oracle import cpuref as O
+
+CPU = O.lib()
 
 pytestmark = pytest.mark.gpu
 
@@ -126,4 +131,76 @@ def test_launch_many_runs_every_argument_block(gpu):
     assert lib.aixk_rtc_launch_many(h, mod, 256, C.create_string_buffer(big, len(big)), len(big), 0, 1) == 1
     assert lib.aixk_rtc_launch_many(h, mod, 256, None, 0, 0, 0) == 1
     gpu.ctx.sync()
+    gpu.release()
+
+
+def _slice_items(entries):
+    arr = (K.SliceItem * len(entries))()
+    for k, (src, dst, dim, start, end, step) in enumerate(entries):
+        arr[k].src, arr[k].dst, arr[k].dim, arr[k].start, arr[k].end, arr[k].step = src, dst, dim, start, end, step
+    return arr
+
+
+@pytest.mark.parametrize("dtype", [O.F32, O.BF16, O.I8, O.F64], ids=["f32", "bf16", "i8", "f64"])
+def test_slice_set_many_is_slice_set_item_by_item(gpu, dtype):
+    """Random sources (contiguous, transposed, sliced, offset views) into windows of separate destinations, and a
+    destination that receives all its column blocks from different sources (a cat): bit-identical to the oracle's
+    sliceSet applied item by item."""
+    rng = np.random.default_rng(53000 + dtype)
+    entries, checks = [], []
+    for trial in range(40):
+        shape = T.random_shape(rng, max_rank=4, max_extent=9)
+        src = T.view_tensor(rng, dtype, shape, rng.choice(T.VIEW_KINDS))
+        _, dsrc = gpu.put(src)
+        dim = int(rng.integers(0, len(shape)))
+        step, start = int(rng.integers(1, 3)), int(rng.integers(0, 3))
+        big = list(shape)
+        big[dim] = start + (shape[dim] - 1) * step + 1 + int(rng.integers(0, 2))
+        end = min(big[dim], start + shape[dim] * step)
+        dst = T.view_tensor(rng, dtype, big, rng.choice(["contig", "transposed", "offset", "sliced"]))
+        want = dst.clone()
+        assert CPU.slice_set(C.byref(src.desc()), C.byref(want.desc()), dim, start, end, step, 1) == 0
+        pd, dd = gpu.put(dst)
+        entries.append((dsrc, dd, dim, start, end, step))
+        checks.append((pd, want, f"item {trial} {shape}->{big} dim={dim}"))
+    # one destination, twelve column blocks, every one from a source of its own (the last a strided view)
+    rows, width, parts = 37, 8, 12
+    whole = T.empty(dtype, [rows, width * parts], fill=3)
+    want = whole.clone()
+    pw, dw = gpu.put(whole)
+    for k in range(parts):
+        src = T.view_tensor(rng, dtype, [rows, width], "transposed" if k == parts - 1 else "contig")
+        _, dsrc = gpu.put(src)
+        assert CPU.slice_set(C.byref(src.desc()), C.byref(want.desc()), 1, k * width, (k + 1) * width, 1, 1) == 0
+        entries.append((dsrc, dw, 1, k * width, (k + 1) * width, 1))
+    checks.append((pw, want, "twelve column blocks of one destination"))
+    G.run_gpu(gpu, "aixk_slice_set_many", _slice_items(entries), len(entries))
+    for pd, want, what in checks:
+        T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, "sliceSet of several items: " + what)
+    gpu.release()
+
+
+def test_slice_set_many_checks_its_items(gpu):
+    rng = np.random.default_rng(54000)
+    src = T.contiguous_tensor(rng, O.F32, [4, 8])
+    dst = T.empty(O.F32, [4, 32], fill=1)
+    other = T.contiguous_tensor(rng, O.BF16, [4, 8])
+    obig = T.empty(O.BF16, [4, 32], fill=1)
+    _, ds = gpu.put(src)
+    pd, dd = gpu.put(dst)
+    _, d16 = gpu.put(other)
+    _, d16big = gpu.put(obig)
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    good = (ds, dd, 1, 0, 8, 1)
+    assert lib.aixk_slice_set_many(h, None, 0) == 0                                           # nothing to do is fine
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (ds, dd, 1, 28, 36, 1)]), 2) == 1    # window beyond the destination
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (ds, dd, 1, 8, 12, 1)]), 2) == 1     # source larger than the window
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (ds, dd, 2, 8, 16, 1)]), 2) == 1     # no such dim
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (ds, dd, 1, 8, 16, 0)]), 2) == 1     # step 0
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (ds, d16big, 1, 8, 16, 1)]), 2) == 1   # element types differ within an item
+    assert lib.aixk_slice_set_many(h, _slice_items([good, (d16, d16big, 1, 8, 16, 1)]), 2) == 1  # element sizes differ between items
+    assert lib.aixk_slice_set_many(h, _slice_items([good] * 513), 513) == 1                    # more items than one call takes
+    gpu.ctx.sync()
+    got = gpu.fetch(pd, dst.storage)
+    assert np.all(got == 1), "a refused call must launch nothing"
     gpu.release()

@@ -475,6 +475,96 @@ def test_fill_is_folded_into_slice_set(dev):
     dev.release()
 
 
+def test_runs_of_slice_sets_leave_as_one_launch(dev):
+    """cat() is one sliceSet per part (aixCore.hpp:1348-1402), the seed of a sliced tensor one per slice (:2228-2233):
+    calls that do not depend on one another wait and leave in one launch.  Every scenario against the oracle applying
+    the same calls one after the other: parts of one destination, windows that overlap (the later call wins), a
+    destination that is the next call's source, recorded operators before and after, a matmul on the result."""
+    set_diag(dev)
+    rng = np.random.default_rng(43000)
+    dtype = O.BF16
+    rows, width, parts = 64, 32, 12
+
+    def oracle_set(src, dst, dim, a, b):
+        assert CPU.slice_set(C.byref(src.desc()), C.byref(dst.desc()), dim, a, b, 1, 1) == 0
+
+    # 1. a cat of twelve column blocks and, into another tensor, four row blocks: one launch for all sixteen
+    whole, tall = T.empty(dtype, [rows, width * parts], fill=7), T.empty(dtype, [4 * rows, width], fill=7)
+    pw, dw = dev.put(whole)
+    pt, dt = dev.put(tall)
+    srcs = [T.contiguous_tensor(rng, dtype, [rows, width]) for _ in range(parts + 4)]
+    ups = [dev.put(x) for x in srcs]
+    dev.dev.synchronize()
+    before = dev.dev.batched_launch_stats()
+    for k in range(parts):
+        oracle_set(srcs[k], whole, 1, k * width, (k + 1) * width)
+        dev.dev.call("slice_set", H.ref(ups[k][1]), H.ref(dw), 1, k * width, (k + 1) * width, 1)
+    for k in range(4):
+        oracle_set(srcs[parts + k], tall, 0, k * rows, (k + 1) * rows)
+        dev.dev.call("slice_set", H.ref(ups[parts + k][1]), H.ref(dt), 0, k * rows, (k + 1) * rows, 1)
+    got_w, got_t = dev.fetch(pw, whole.storage), dev.fetch(pt, tall.storage)
+    after = dev.dev.batched_launch_stats()
+    assert after[0] - before[0] == 1 and after[1] - before[1] == parts + 4, (before, after)
+    T.assert_same_bits(got_w, whole.storage, "twelve column blocks")
+    T.assert_same_bits(got_t, tall.storage, "four row blocks")
+    # 2. windows that overlap, a strided window, the same window twice: the calls keep their order
+    for k, (a, b) in enumerate([(0, 32), (16, 48), (16, 48), (40, 72)]):
+        oracle_set(srcs[k], whole, 1, a, b)
+        dev.dev.call("slice_set", H.ref(ups[k][1]), H.ref(dw), 1, a, b, 1)
+    assert CPU.slice_set(C.byref(srcs[5].desc()), C.byref(whole.desc()), 1, 100, 164, 2, 1) == 0
+    dev.dev.call("slice_set", H.ref(ups[5][1]), H.ref(dw), 1, 100, 164, 2)
+    oracle_set(srcs[6], whole, 1, 101, 133)
+    dev.dev.call("slice_set", H.ref(ups[6][1]), H.ref(dw), 1, 101, 133, 1)
+    T.assert_same_bits(dev.fetch(pw, whole.storage), whole.storage, "overlapping windows")
+    # 3. a destination that the next call reads, and a source that is overwritten after it was read
+    mid, last = T.empty(dtype, [rows, 2 * width], fill=1), T.empty(dtype, [rows, 4 * width], fill=2)
+    pm, dm = dev.put(mid)
+    pl, dl = dev.put(last)
+    oracle_set(srcs[0], mid, 1, 0, width)
+    dev.dev.call("slice_set", H.ref(ups[0][1]), H.ref(dm), 1, 0, width, 1)
+    oracle_set(mid, last, 1, 2 * width, 4 * width)
+    dev.dev.call("slice_set", H.ref(dm), H.ref(dl), 1, 2 * width, 4 * width, 1)
+    oracle_set(srcs[1], mid, 1, 0, width)                                         # after `last` took its copy
+    dev.dev.call("slice_set", H.ref(ups[1][1]), H.ref(dm), 1, 0, width, 1)
+    T.assert_same_bits(dev.fetch(pl, last.storage), last.storage, "chain: the copy of the destination before it changed")
+    T.assert_same_bits(dev.fetch(pm, mid.storage), mid.storage, "chain: the destination after its second window")
+    # 4. recorded operators on either side: the source is a recorded sum, the destination is negated afterwards
+    rec = Recorder(dev, dtype, [rows, width])
+    x, y = rec.leaf(srcs[2]), rec.leaf(srcs[3])
+    total = rec.binary(O.ADD, x, y)                                               # pending when sliceSet is called
+    oracle_set(total["host"], mid, 1, width, 2 * width)
+    dev.dev.call("slice_set", H.ref(total["desc"]), H.ref(dm), 1, width, 2 * width, 1)
+    rec2 = Recorder(dev, dtype, [rows, 2 * width])
+    neg = rec2.unary(O.NEG, {"host": mid, "ptr": pm, "desc": dm})                  # recorded while the sliceSet waits
+    oracle_set(srcs[4], mid, 1, 0, width)                                         # and the destination changes again
+    dev.dev.call("slice_set", H.ref(ups[4][1]), H.ref(dm), 1, 0, width, 1)
+    T.assert_same_bits(dev.fetch(neg["ptr"], neg["host"].storage), neg["host"].storage, "negation of the destination as it was")
+    T.assert_same_bits(dev.fetch(pm, mid.storage), mid.storage, "destination after the negation was recorded")
+    # 5. a matmul on a destination whose parts are still waiting, and a sliceSet of its result
+    a = T.empty(dtype, [64, 64], fill=0)
+    pa, da = dev.put(a)
+    halves = [T.contiguous_tensor(rng, dtype, [64, 32], lo=-1, hi=1) for _ in range(2)]
+    for k, hlf in enumerate(halves):
+        _, dh = dev.put(hlf)
+        oracle_set(hlf, a, 1, 32 * k, 32 * (k + 1))
+        dev.dev.call("slice_set", H.ref(dh), H.ref(da), 1, 32 * k, 32 * (k + 1), 1)
+    b = T.contiguous_tensor(rng, dtype, [64, 64], lo=-1, hi=1)
+    _, db = dev.put(b)
+    prod = T.empty(dtype, [64, 64])
+    pp = dev.raw(prod.storage.nbytes)
+    dp = H.kdesc(prod, pp)
+    dev.dev.call("matmul", H.ref(da), H.ref(db), H.ref(dp))
+    wide = T.empty(dtype, [64, 128], fill=5)
+    pwd, dwd = dev.put(wide)
+    dev.dev.call("slice_set", H.ref(dp), H.ref(dwd), 1, 64, 128, 1)
+    raw = dev.fetch(pwd, wide.storage).reshape(64, 128)
+    got = O.to_float64(raw[:, 64:], dtype)
+    want = O.to_float64(a.storage, dtype).reshape(64, 64) @ O.to_float64(b.storage, dtype).reshape(64, 64)
+    assert np.all(raw[:, :64] == 5)
+    assert np.max(np.abs(got - want)) <= 2e-2 * np.max(np.abs(want)), "matmul of the assembled operand, set into a window"   # bf16 result: 2e-2 relative
+    dev.release()
+
+
 _CASES = goldens.load_cases()
 
 
