@@ -123,9 +123,28 @@ struct DeviceHIP::Extras {
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
     struct Group { std::vector<aixhip_tensor> a, b, out; };
     std::array<Group, 4> groups;
-    // sliceSet calls waiting to leave as one launch (see DeviceHIP::sliceSet)
+    // sliceSet and argmaxIndicesTo calls waiting to leave as one launch each (see DeviceHIP::sliceSet, argmaxIndicesTo)
     std::vector<aixk_slice_item> slices;
-    bool anyPending() const { if (!slices.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
+    std::vector<aixk_argmax_item> onehots;
+    // what the waiting calls of all three kinds read and write (block starts), so that a new call knows in one lookup
+    // whether it may wait beside them; per destination of waiting sliceSet calls, how it was described and the windows
+    // written so far
+    aixhip::fuse::PointerSet waitReads, waitWrites;
+    struct SliceWindows { aixhip_tensor dst; uint64_t dim; std::vector<std::pair<uint64_t, uint64_t>> ranges; };
+    std::unordered_map<const void*, SliceWindows> sliceDsts;
+    bool anyPending() const { if (!slices.empty() || !onehots.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
+    // a call that reads r0, r1 and writes w neither uses what waits nor is used by it
+    bool apartFromWaiting(const void* r0, const void* r1, const void* w) const
+    {
+        if ((r0 && waitWrites.contains(r0)) || (r1 && waitWrites.contains(r1))) return false;
+        return !waitWrites.contains(w) && !waitReads.contains(w);
+    }
+    void noteWaiting(const void* r0, const void* r1, const void* w)
+    {
+        if (r0) waitReads.insert(r0);
+        if (r1) waitReads.insert(r1);
+        waitWrites.insert(w);
+    }
     // results of at least this many bytes are written with non-temporal stores (the kernel layer's rule, same override)
     size_t streamStoreMinBytes = [] {
         const char* e = std::getenv("AIXHIP_STREAM_STORE_MIN_BYTES");
@@ -268,6 +287,8 @@ void DeviceHIP::setFuseConfig(const FuseConfig& cfg)
     cb.blockBase = [this](const void* p) { return m_blocks.baseOf(p); };
     FuseConfig own = cfg;
     own.loneCastsAsKernels = m_extras->batchFlatKernels;    // so that runs of them leave as one launch (issueFlatBatch)
+    own.groupEqualKernels = m_extras->batchFlatKernels;     // and so that such runs form where the program interleaves kinds
+    if (const char* e = std::getenv("AIXHIP_FLUSH_THRESHOLD"); e && *e) own.flushThreshold = std::max<size_t>(1, std::strtoull(e, nullptr, 10));
     m_engine = std::make_unique<FuseEngine>(own, std::move(cb));
     m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) m_engine->retainBuffer(base); });
 }
@@ -806,38 +827,47 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     grid = std::max<uint64_t>(1, std::min(grid, cap));
 
     AIXHIP_TRACE("%s  %llu elements, %zu in %zu out", gen::entryName(d, shape).c_str(), (unsigned long long)n, NI, NO);
-    auto& B = ex.batch;
-    if (shape == gen::Shape::Flat && ex.batchFlatKernels) {
-        // joins the kernels waiting to leave together, or starts the next such run
-        bool joins = B.count() != 0 && B.key == ex.key && B.count() < 256 && (uint64_t)B.starts.back() + grid < (1u << 30) &&
-                     (B.table.size() + ex.args.size()) * sizeof(uint64_t) < (200u << 10);
-        if (joins) {
-            for (size_t k = 0; k < NI && joins; ++k) if (B.writes.contains(d.inputBuffers[k].data)) joins = false;
-            for (size_t k = 0; k < NO && joins; ++k)
-                if (B.writes.contains(d.outputBuffers[k].data) || B.reads.contains(d.outputBuffers[k].data)) joins = false;
-        }
-        if (!joins) issueFlatBatch();
-        if (B.count() == 0) { B.key = ex.key; B.single = mod; B.words = ex.args.size(); B.starts.push_back(0); }
-        else if (!B.many) {
-            ex.key += "|many";
-            auto many = ex.kernels.find(ex.key);
-            if (many != ex.kernels.end()) { B.many = many->second; ++ex.hits; }
-            else {
-                int32_t cached = 0;
-                const std::string src = gen::source(d, shape, bmask, noAlias, streamOut, true);
-                check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), (gen::entryName(d, shape) + "_many").c_str(), &B.many, &cached));
-                ex.kernels.emplace(ex.key, B.many);
-                ++ex.misses;
-            }
-        }
-        B.table.insert(B.table.end(), ex.args.begin(), ex.args.end());
-        B.starts.push_back(B.starts.back() + (uint32_t)grid);
-        for (size_t k = 0; k < NI; ++k) B.reads.insert(d.inputBuffers[k].data);
-        for (size_t k = 0; k < NO; ++k) B.writes.insert(d.outputBuffers[k].data);
+    if (ex.batchFlatKernels) {
+        joinBatch(d, mod, gen::entryName(d, shape), grid, [&] { return gen::source(d, shape, bmask, noAlias, streamOut, true); });
         return;
     }
     issueFlatBatch();
     check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
+}
+
+// The kernel whose signature is in Extras::key and whose argument block is in Extras::args joins the kernels waiting to
+// leave together -- same kernel, reads nothing they write, writes nothing they read or write -- or sends them off and
+// starts the next run.  manySource gives the text of the kernel's many-blocks form when that has to be compiled.
+void DeviceHIP::joinBatch(const FusedSubgraphDescriptor& d, aixk_module* mod, const std::string& entry, uint64_t grid, const std::function<std::string()>& manySource)
+{
+    auto& ex = *m_extras;
+    auto& B = ex.batch;
+    const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
+    bool joins = B.count() != 0 && B.key == ex.key && B.count() < 256 && (uint64_t)B.starts.back() + grid < (1u << 30) &&
+                 (B.table.size() + ex.args.size()) * sizeof(uint64_t) < (200u << 10);
+    if (joins) {
+        for (size_t k = 0; k < NI && joins; ++k) if (B.writes.contains(d.inputBuffers[k].data)) joins = false;
+        for (size_t k = 0; k < NO && joins; ++k)
+            if (B.writes.contains(d.outputBuffers[k].data) || B.reads.contains(d.outputBuffers[k].data)) joins = false;
+    }
+    if (!joins) issueFlatBatch();
+    if (B.count() == 0) { B.key = ex.key; B.single = mod; B.words = ex.args.size(); B.starts.push_back(0); }
+    else if (!B.many) {
+        ex.key += "|many";
+        auto many = ex.kernels.find(ex.key);
+        if (many != ex.kernels.end()) { B.many = many->second; ++ex.hits; }
+        else {
+            int32_t cached = 0;
+            const std::string src = manySource();
+            check(aixk_rtc_get(m_ctx, ex.key.c_str(), src.c_str(), (entry + "_many").c_str(), &B.many, &cached));
+            ex.kernels.emplace(ex.key, B.many);
+            ++ex.misses;
+        }
+    }
+    B.table.insert(B.table.end(), ex.args.begin(), ex.args.end());
+    B.starts.push_back(B.starts.back() + (uint32_t)grid);
+    for (size_t k = 0; k < NI; ++k) B.reads.insert(d.inputBuffers[k].data);
+    for (size_t k = 0; k < NO; ++k) B.writes.insert(d.outputBuffers[k].data);
 }
 
 // The flat kernels that wait in the batch (emitFused) leave: alone as an ordinary launch, several as one launch of the
@@ -868,7 +898,6 @@ void DeviceHIP::issueFlatBatch()
 // A fused kernel that holds row reductions: a wave or a workgroup per row (hipgen.hpp: row programs).
 void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
 {
-    issueFlatBatch();
     auto& ex = *m_extras;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     gen::RowGeometry geo;
@@ -903,6 +932,11 @@ void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
     const uint64_t rowsPerBlock = geo.lanes == 64 ? gen::kBlock / 64 : 1;
     uint64_t grid = (rows + rowsPerBlock - 1) / rowsPerBlock;
     grid = std::max<uint64_t>(1, std::min<uint64_t>(grid, (uint64_t)m_cus * 64));
+    if (ex.batchFlatKernels) {
+        joinBatch(d, mod, gen::rowEntryName(d, geo), grid, [&] { return gen::rowSource(d, geo, streamOut, true); });
+        return;
+    }
+    issueFlatBatch();
     check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
 }
 
@@ -969,16 +1003,9 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
                 flushWindow(false);
             }
             aixhip_tensor pa, pb, pr; toPod(a, &pa, "matmul"); toPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
-            // it may read no pending result and overwrite nothing pending: all pending products are then independent of
+            // it may read no waiting result and overwrite nothing that waits: all waiting calls are then independent of
             // each other, whatever group they wait in, and the groups may be issued in any order
-            bool independent = true;
-            for (const auto& g : ex.groups)
-                for (size_t i = 0; independent && i < g.out.size(); ++i)
-                    independent = g.out[i].data != pa.data && g.out[i].data != pb.data && g.out[i].data != pr.data &&
-                                  g.a[i].data != pr.data && g.b[i].data != pr.data;
-            for (size_t i = 0; independent && i < ex.slices.size(); ++i)
-                independent = ex.slices[i].dst.data != pa.data && ex.slices[i].dst.data != pb.data && ex.slices[i].dst.data != pr.data && ex.slices[i].src.data != pr.data;
-            if (!independent) issuePending();
+            if (!ex.apartFromWaiting(pa.data, pb.data, pr.data)) issuePending();
             // the group of its shape and operand layout (forward and backward products of attention alternate between
             // two or three of them), or the emptiest slot
             Extras::Group* into = nullptr;
@@ -990,6 +1017,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             }
             if (!into) { issuePending(); into = &ex.groups[0]; }
             into->a.push_back(pa); into->b.push_back(pb); into->out.push_back(pr);
+            ex.noteWaiting(pa.data, pb.data, pr.data);
             markTouched(a.data); markTouched(b.data); markTouched(result.data);
             return;
         }
@@ -1020,6 +1048,14 @@ void DeviceHIP::issuePending()
         if (ex.slices.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.slices.size(); }
         ex.slices.clear();
     }
+    if (!ex.onehots.empty()) {
+        if (status == AIXK_OK)
+            status = ex.onehots.size() == 1 ? aixk_argmax_to(m_ctx, 2, &ex.onehots[0].src, &ex.onehots[0].dst, ex.onehots[0].dim)
+                                            : aixk_argmax_onehot_many(m_ctx, ex.onehots.data(), (uint32_t)ex.onehots.size());
+        if (ex.onehots.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.onehots.size(); }
+        ex.onehots.clear();
+    }
+    ex.waitReads.clear(); ex.waitWrites.clear(); ex.sliceDsts.clear();
     for (auto& g : ex.groups) {
         if (g.out.empty()) continue;
         const uint32_t count = (uint32_t)g.out.size();
@@ -1173,6 +1209,9 @@ void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams
     check(aixk_argmax_to(m_ctx, 0, &ps, &pd, dim));
 }
 
+// The mask of max()'s backward pass (aixCore.hpp:2170-2175) is asked for head after head: like small matmul calls, a
+// call whose zero fill was folded in and whose operands lie in device memory waits for company and leaves with it in one
+// launch (see matmul(), sliceSet()).
 void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
 {
     AIXHIP_TRACE("argmaxIndicesTo");
@@ -1182,6 +1221,23 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
     // the window is folded into the operator
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
+    auto& ex = *m_extras;
+    if (folded && init == 0 && ex.batchFlatKernels && src.size && src.size < (size_t(1) << 31) && dst.size == src.size && findBlock(src.data) && findBlock(dst.data) &&
+        src.data != dst.data && src.isContiguous && dst.isContiguous && dst.offset == 0 && src.shape == dst.shape && !src.shape.empty() &&
+        dim + 1 == src.shape.size() && src.shape.size() <= AIXK_MAX_RANK) {
+        if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {          // recorded producers and users go first
+            m_engine->recordExternalRead(src.data);
+            flushWindow(false);
+        }
+        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.apartFromWaiting(src.data, nullptr, dst.data)) issuePending();
+        aixk_argmax_item item{};
+        toPod(src, &item.src, "argmaxIndicesTo"); toPod(dst, &item.dst, "argmaxIndicesTo");
+        item.dim = dim;
+        ex.onehots.push_back(item);
+        ex.noteWaiting(src.data, nullptr, dst.data);
+        markTouched(src.data); markTouched(dst.data);
+        return;
+    }
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "argmaxIndicesTo"); toPod(dst, &pd, "argmaxIndicesTo");
     if (folded && init != 0) {                                       // not the zero fill: put it back as a pass of its own
@@ -1225,19 +1281,25 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
             }
             bool independent = ex.slices.size() < AIXK_SLICE_ITEMS_MAX &&
                                (ex.slices.empty() || dataTypeSize(static_cast<DataType>(ex.slices[0].src.dtype)) == dataTypeSize(src.dtype));
-            for (const auto& g : ex.groups)
-                for (size_t i = 0; independent && i < g.out.size(); ++i)
-                    independent = g.out[i].data != src.data && g.out[i].data != dst.data && g.a[i].data != dst.data && g.b[i].data != dst.data;
-            for (size_t i = 0; independent && i < ex.slices.size(); ++i) {
-                const aixk_slice_item& w = ex.slices[i];
-                independent = w.dst.data != src.data && w.src.data != dst.data;
-                if (independent && w.dst.data == dst.data) {
-                    independent = w.dim == dim && w.step == 1 && step == 1 && (w.end <= start || end <= w.start) && w.dst.rank == item.dst.rank &&
-                                  w.dst.offset == item.dst.offset && !std::memcmp(w.dst.shape, item.dst.shape, sizeof(item.dst.shape)) &&
-                                  !std::memcmp(w.dst.strides, item.dst.strides, sizeof(item.dst.strides));
-                }
+            auto windows = ex.sliceDsts.find(dst.data);
+            if (independent && windows != ex.sliceDsts.end()) {
+                // another window of a destination that waits: apart if nothing that waits reads the destination, it is
+                // described the same way, and the ranges do not meet
+                const auto& w = windows->second;
+                independent = !ex.waitWrites.contains(src.data) && !ex.waitReads.contains(dst.data) && w.dim == dim && step == 1 && w.dst.rank == item.dst.rank &&
+                              w.dst.offset == item.dst.offset && !std::memcmp(w.dst.shape, item.dst.shape, sizeof(item.dst.shape)) &&
+                              !std::memcmp(w.dst.strides, item.dst.strides, sizeof(item.dst.strides));
+                for (size_t i = 0; independent && i < w.ranges.size(); ++i) independent = w.ranges[i].second <= start || end <= w.ranges[i].first;
+            } else if (independent) {
+                independent = ex.apartFromWaiting(src.data, nullptr, dst.data);
             }
             if (!independent) issuePending();
+            if (step == 1) {
+                auto& w = ex.sliceDsts[dst.data];
+                if (w.ranges.empty()) { w.dst = item.dst; w.dim = dim; }
+                w.ranges.emplace_back(start, end);
+            }
+            ex.noteWaiting(src.data, nullptr, dst.data);
             ex.slices.push_back(item);
             markTouched(src.data); markTouched(dst.data);
             return;

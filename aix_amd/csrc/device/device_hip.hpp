@@ -26,12 +26,14 @@
 #include "fuse.hpp"
 
 #include <cstdint>
+#include <functional>
 #include <memory>
 #include <string>
 #include <unordered_map>
 #include <vector>
 
 struct aixk_ctx;
+struct aixk_module;
 struct aixhip_tensor;
 struct aixhip_device;
 
@@ -164,6 +166,7 @@ private:
     void emitRowProgram(const aixhip::fuse::FusedSubgraphDescriptor& d);
     void issueFlatBatch();
     bool recordRowReduction(aixhip::fuse::OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init);
+    void joinBatch(const aixhip::fuse::FusedSubgraphDescriptor& d, aixk_module* mod, const std::string& entry, uint64_t grid, const std::function<std::string()>& manySource);
     void issuePending();                                     // the waiting matmul and sliceSet calls, one launch per run (see matmul(), sliceSet())
 
     aixk_ctx* m_ctx{nullptr};

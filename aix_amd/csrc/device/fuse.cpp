@@ -1047,7 +1047,52 @@ void FuseEngine::flush(bool final)
     std::string groupsText;
     Planner& plan = *m_planner;
     plan.run(window, live);
-    for (const auto& e : plan.emits()) {
+    // The planner's list is one valid order; any order that keeps two kernels apart only where one touches what the other
+    // writes is as good.  Kernels are sent off level by level -- a kernel's level is one more than the highest level of
+    // an earlier kernel it depends on -- and kind by kind within a level, so that the same operator applied to tensor
+    // after tensor (one attention head after the other) comes out as a run of equal kernels even when the program
+    // interleaves it with others; the device sends such runs off as one launch.  Reads and writes are taken per
+    // operator (every input, every output of every operator of a kernel): more than a kernel really loads and stores,
+    // which can only add dependences.
+    m_order.clear();
+    m_touched.clear();
+    if (!(m_config.groupEqualKernels && m_config.elementwiseFusion)) {
+        for (size_t k = 0; k < plan.emits().size(); ++k) m_order.push_back({0, 0, k});
+    } else {
+        const auto& emits = plan.emits();
+        auto each = [&](const Emit& e, auto&& fn) {
+            if (!e.fused) { fn(window[e.index]); return; }
+            for (size_t op : plan.group(e.index).ops) fn(window[op]);
+        };
+        for (size_t k = 0; k < emits.size(); ++k) {
+            uint32_t level = 0;
+            uint64_t kind = emits[k].fused ? 0xcbf29ce484222325ull : 0x84222325cbf29ce4ull;
+            each(emits[k], [&](const OpRecord& op) {
+                kind = (kind ^ (uint64_t)op.type ^ ((uint64_t)op.output.dtype << 8) ^ ((uint64_t)op.rowLength << 16)) * 0x100000001b3ull;
+                const bool fill = op.type == OpType::Fill || op.type == OpType::FillMin;
+                for (const void* r : {fill ? nullptr : op.input0.data, op.hasInput1 ? op.input1.data : nullptr}) {
+                    if (!r) continue;
+                    auto it = m_touched.find(r);
+                    if (it != m_touched.end()) level = std::max(level, it->second.first);
+                }
+                auto it = m_touched.find(op.output.data);
+                if (it != m_touched.end()) level = std::max({level, it->second.first, it->second.second});
+            });
+            each(emits[k], [&](const OpRecord& op) {
+                const bool fill = op.type == OpType::Fill || op.type == OpType::FillMin;
+                for (const void* r : {fill ? nullptr : op.input0.data, op.hasInput1 ? op.input1.data : nullptr})
+                    if (r) { auto& t = m_touched[r]; t.second = std::max(t.second, level + 1); }
+                auto& t = m_touched[op.output.data];
+                t.first = std::max(t.first, level + 1);
+            });
+            m_order.push_back({level, kind, k});
+        }
+        std::sort(m_order.begin(), m_order.end(), [](const Order& a, const Order& b) {
+            return a.level != b.level ? a.level < b.level : a.kind != b.kind ? a.kind < b.kind : a.at < b.at;
+        });
+    }
+    for (const Order& o : m_order) {
+        const auto& e = plan.emits()[o.at];
         if (!e.fused) { m_callbacks.emitSingle(window[e.index]); ++singles; continue; }
         const auto& g = plan.group(e.index);
         const bool castKernel = m_config.loneCastsAsKernels && g.ops.size() == 1 && window[g.ops[0]].type == OpType::Cast;

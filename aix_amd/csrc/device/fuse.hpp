@@ -22,6 +22,7 @@
 #include <optional>
 #include <string>
 #include <utility>
+#include <unordered_map>
 #include <vector>
 
 namespace aixhip::fuse {
@@ -51,6 +52,7 @@ struct FuseConfig {
     bool   supportsStridedFusion = true;   // may fused kernels read broadcast / strided views
     bool   loneCastsAsKernels    = false;  // a cast with no company is emitted as a one-operator kernel (emitFused), not as a single
     bool   deferIdleFills        = true;   // a fill nothing else in its window touches waits for its first user (see flush())
+    bool   groupEqualKernels     = false;  // kernels leave level by level and kind by kind instead of in the planner's order (see flush())
 };
 
 // An operand as the planner keeps it: the fields of aix::DeviceTensorParams with the extents and
@@ -251,6 +253,11 @@ private:
     PointerSet m_waitingBuffers;
     std::unique_ptr<Planner> m_planner;    // its working storage is kept from window to window
     FusedSubgraphDescriptor m_descriptor;
+    // flush(): the order kernels leave in (level, kind, place in the planner's list) and, per buffer, one more than the
+    // highest level of a kernel that wrote / read it so far
+    struct Order { uint32_t level; uint64_t kind; size_t at; };
+    std::vector<Order> m_order;
+    std::unordered_map<const void*, std::pair<uint32_t, uint32_t>> m_touched;
     std::optional<FlushDiagnostics> m_diagnostics;
     bool m_flushing{false};
 };

@@ -179,7 +179,6 @@ std::string signature(const FusedSubgraphDescriptor& d, Shape shape, uint32_t br
 
 std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut, bool many)
 {
-    if (many && shape != Shape::Flat) throw std::invalid_argument("only flat kernels have a many-blocks form");
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d), NT = triCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
     if (d.opParams.size() != 3 * NT) throw std::invalid_argument("fused kernel: tril / triu without its parameters");
@@ -270,7 +269,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     if (shape == Shape::Rows) {
         o << "    const int inner = (int)a.rank - 1;\n"
           << "    const u64 total = a.n / VEC;\n"
-          << "    for (u64 c = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; c < total; c += (u64)gridDim.x * " << kBlock << ") {\n"
+          << "    for (u64 c = (u64)BID * " << kBlock << " + threadIdx.x; c < total; c += (u64)GDIM * " << kBlock << ") {\n"
           << "        u64 row = c / a.chunks;\n        const u64 col = (c - row * a.chunks) * VEC;\n"
           << "        u64 p[" << AI << "];\n";
         for (size_t k = 0; k < NI; ++k) o << "        p[" << k << "] = a.off[" << k << "];\n";
@@ -296,7 +295,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     }
 
     // gather
-    o << "    for (u64 i = (u64)blockIdx.x * " << kBlock << " + threadIdx.x; i < a.n; i += (u64)gridDim.x * " << kBlock << ") {\n"
+    o << "    for (u64 i = (u64)BID * " << kBlock << " + threadIdx.x; i < a.n; i += (u64)GDIM * " << kBlock << ") {\n"
       << "        u64 rest = i;\n        u64 p[" << AI << "];\n";
     if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(i, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
     for (size_t k = 0; k < NI; ++k) o << "        p[" << k << "] = a.off[" << k << "];\n";
@@ -369,7 +368,7 @@ void rowSignatureInto(std::string& s, const FusedSubgraphDescriptor& d, const Ro
     }
 }
 
-std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut)
+std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut, bool many)
 {
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
@@ -389,9 +388,18 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     for (size_t k = 0; k < NO; ++k) o << "typedef " << typeName(d.outputBuffers[k].dtype) << " O" << k << ";\n";
     auto to_t = [&](size_t k, const std::string& e) { return d.inputBuffers[k].dtype == d.dtype ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
     auto from_t = [&](size_t k, const std::string& e) { return d.outputBuffers[k].dtype == d.dtype ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
-    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 rows;\n    u64 len;\n};\n\n"
-      << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "(Args a)\n{\n"
-      << "    __shared__ W red[4];\n    (void)red;\n"
+    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 rows;\n    u64 len;\n};\n\n";
+    if (many) {
+        o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "_many(const Args* table, const u32* starts, u32 count)\n{\n"
+          << "    u32 lo = 0, hi = count;\n"
+          << "    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (starts[mid] <= blockIdx.x) lo = mid; else hi = mid; }\n"
+          << "    const Args a = table[lo];\n"
+          << "    const u32 BID = blockIdx.x - starts[lo], GDIM = starts[lo + 1] - starts[lo];\n";
+    } else {
+        o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "(Args a)\n{\n"
+          << "    const u32 BID = blockIdx.x, GDIM = gridDim.x;\n";
+    }
+    o << "    __shared__ W red[4];\n    (void)red;\n"
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
     if (NS == 0) o << "    s[0] = zero<T>();\n";
@@ -400,8 +408,8 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     o << "    const u32 lane = threadIdx.x % G;\n"
       << "    const u64 nvec = a.len / VEC;\n"
       << "    const W lowestW = (W)(-__builtin_huge_val());\n    (void)lowestW;\n";
-    if (g.lanes == 64) o << "    for (u64 row = (u64)blockIdx.x * " << kBlock / 64 << " + threadIdx.x / 64; row < a.rows; row += (u64)gridDim.x * " << kBlock / 64 << ") {\n";
-    else o << "    for (u64 row = blockIdx.x; row < a.rows; row += gridDim.x) {\n";
+    if (g.lanes == 64) o << "    for (u64 row = (u64)BID * " << kBlock / 64 << " + threadIdx.x / 64; row < a.rows; row += (u64)GDIM * " << kBlock / 64 << ") {\n";
+    else o << "    for (u64 row = BID; row < a.rows; row += GDIM) {\n";
     // operands: whole rows (their own or the one shared row) as vectors, per-row values as scalars
     for (size_t k = 0; k < NI; ++k) {
         if (kinds[k] == fuse::RowOperand::Dense || kinds[k] == fuse::RowOperand::RowVector) {

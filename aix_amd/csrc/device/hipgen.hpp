@@ -30,10 +30,10 @@ std::string signature(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint3
 // The same text written into `out` (cleared first; its capacity is reused from call to call).
 void signatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask, bool noAlias, bool streamOut = false);
 
-// Source of `extern "C" __global__ void <entryName>(Args)`.  many (flat shape only): of
+// Source of `extern "C" __global__ void <entryName>(Args)`.  many: of
 // `<entryName>_many(const Args* table, const u32* starts, u32 count)` instead -- the same body for `count` argument
 // blocks in one launch, workgroups [starts[k], starts[k + 1]) working on table[k] (Adam's update of every parameter,
-// the per-parameter casts of a mixed-precision step).
+// the per-parameter casts of a mixed-precision step, one operator applied head by head).
 std::string source(const fuse::FusedSubgraphDescriptor& d, Shape shape, uint32_t broadcastMask = 0, bool noAlias = true, bool streamOut = false,
                    bool many = false);
 
@@ -48,7 +48,7 @@ struct RowGeometry {
 // false: the descriptor cannot run as a row program (row too long, not a whole number of vectors)
 bool rowGeometry(const fuse::FusedSubgraphDescriptor& d, RowGeometry* g);
 void rowSignatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut);
-std::string rowSource(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut);
+std::string rowSource(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut, bool many = false);     // (many: as for source())
 // Args of a row program: in[], out[], immediates, rows, rowLength
 void packRowArgsInto(std::vector<uint64_t>& a, const fuse::FusedSubgraphDescriptor& d, const void* const* inputs, void* const* outputs);
 

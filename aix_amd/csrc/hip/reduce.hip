@@ -502,6 +502,47 @@ __global__ __launch_bounds__(kBlock) void argmax_onehot_inner_k(const T* __restr
     }
 }
 
+// The same for several tensors of dense rows in one launch (the masks of max()'s backward, head after head): item k's
+// addresses and extents come from a table in device memory, its share of the grid from `starts`.
+struct OnehotItem { u64 src, dst, rows, len; };
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void argmax_onehot_inner_many_k(const OnehotItem* __restrict__ items, const u32* __restrict__ starts, u32 count)
+{
+    typedef ArgOp<T> Op;
+    typedef typename Op::Acc Acc;
+    typedef typename vec16<T>::type V;
+    constexpr int VEC = vec16<T>::n;
+    typedef vec<i32, 4> O4;
+    u32 lo = 0, hi = count;
+    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (starts[mid] <= blockIdx.x) lo = mid; else hi = mid; }
+    const OnehotItem it = items[lo];
+    const u32 first = starts[lo], share = starts[lo + 1] - first;
+    const T* src = global_ptr<const T>(it.src);
+    i32* dst = global_ptr<i32>(it.dst);
+    const int w = threadIdx.x / kWave, l = threadIdx.x % kWave;
+    const u64 L = it.len;
+    for (u64 slot = (u64)(blockIdx.x - first) * kWaves + w; slot < it.rows; slot += (u64)share * kWaves) {
+        const T* row = src + slot * L;
+        Acc acc = Op::init();
+        for (u64 v = l; v < L / VEC; v += kWave) {
+            const V x = *(const V*)(row + v * VEC);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) { const u64 j = v * VEC + e; Op::step(acc, x.v[e], j, j == 0); }
+        }
+        acc = wave_reduce<Op>(acc);
+        const u32 mine = (acc.flags & 2u) ? 0u : acc.idx;
+        const u32 winner = __shfl(mine, 0, kWave);
+        i32* out = dst + slot * L;
+        for (u64 j0 = (u64)l * 4; j0 < L; j0 += (u64)kWave * 4) {
+            O4 v;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v.v[e] = (u32)(j0 + e) == winner ? 1 : 0;
+            *(O4*)(out + j0) = v;
+        }
+    }
+}
+
 // argmax down the columns of wide rows with the rows split into chunks: the record a lane keeps per column is the
 // pair (value, row) and the scan is a bare `x > best` -- three instructions per element against the seven of
 // ArgOp::step -- and the partial records are 8 bytes instead of 12 (16 for 8-byte elements).  A strict `>` from minus
@@ -1025,6 +1066,57 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
             fin.onehot = 1;
         }
         return run_plan<ArgOp<T>, T>(ctx, src, (int32_t*)dst->data, plan, fin);
+    });
+}
+
+int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    if (count == 0) return AIXK_OK;
+    AIXK_REQUIRE(items, "argmaxIndicesTo of several items: no items");
+    // one launch if every item is dense rows of one element type reduced along the last dim, else item by item
+    bool together = count >= 2 && count <= AIXK_ARGMAX_ITEMS_MAX;
+    const int dtype = items[0].src.dtype;
+    for (uint32_t k = 0; k < count && together; ++k) {
+        const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
+        together = valid_tensor(src) && valid_tensor(dst) && src->dtype == dtype && dst->dtype == AIXK_I32 && src->rank >= 1 &&
+                   (int)items[k].dim == src->rank - 1 && dst->rank == src->rank && src->size > 0 && src->size == numel(src) && src->size < (1ull << 31) &&
+                   dst->size == src->size && dst->offset == 0 && aligned16(dst->data);
+        if (!together) break;
+        const uint64_t L = src->shape[src->rank - 1], vec = 16 / aixk_dtype_size(dtype);
+        uint64_t dense[AIXK_MAX_RANK];
+        row_major_strides(src->rank, src->shape, dense);
+        for (int d = 0; d < src->rank; ++d)
+            if (dst->shape[d] != src->shape[d] || (src->shape[d] != 1 && (src->strides[d] != dense[d] || dst->strides[d] != dense[d]))) together = false;
+        together = together && L >= 32 && L % 4 == 0 && L % vec == 0 && aligned16((const char*)src->data + src->offset * aixk_dtype_size(dtype));
+    }
+    if (!together) {
+        for (uint32_t k = 0; k < count; ++k) AIXK_TRY(aixk_argmax_to(ctx, 2, &items[k].src, &items[k].dst, items[k].dim));
+        return AIXK_OK;
+    }
+    const size_t table_bytes = (size_t)count * sizeof(OnehotItem), all_bytes = table_bytes + ((size_t)count + 1) * sizeof(u32);
+    char* host = nullptr;
+    const char* dev = nullptr;
+    AIXK_TRY(table_slot(ctx, all_bytes, (void**)&host, (const void**)&dev));
+    OnehotItem* table = (OnehotItem*)host;
+    u32* starts = (u32*)(host + table_bytes);
+    u32 grid = 0;
+    for (uint32_t k = 0; k < count; ++k) {
+        const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
+        const uint64_t L = src->shape[src->rank - 1], rows = src->size / L;
+        table[k].src = (u64)(uintptr_t)((const char*)src->data + src->offset * aixk_dtype_size(dtype));
+        table[k].dst = (u64)(uintptr_t)dst->data;
+        table[k].rows = rows; table[k].len = L;
+        starts[k] = grid;
+        grid += grid_for(rows, kWaves, 1u << 20);
+    }
+    starts[count] = grid;
+    AIXK_TRY(table_upload(ctx, host, dev, all_bytes));
+    return by_dtype(dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        hipLaunchKernelGGL((argmax_onehot_inner_many_k<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const OnehotItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
     });
 }
 

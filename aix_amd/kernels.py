@@ -29,6 +29,11 @@ class SliceItem(C.Structure):
     _fields_ = [("src", Tensor), ("dst", Tensor), ("dim", C.c_uint64), ("start", C.c_uint64), ("end", C.c_uint64), ("step", C.c_uint64)]
 
 
+class ArgmaxItem(C.Structure):
+    """aixk_argmax_item"""
+    _fields_ = [("src", Tensor), ("dst", Tensor), ("dim", C.c_uint64)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("large_bar", C.c_int32), ("wavefront", C.c_int32),
@@ -73,6 +78,7 @@ _SIGNATURES = {
     "aixk_reduce_to": [_P, C.c_int, _T, _T],
     "aixk_reduce_to_init": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
+    "aixk_argmax_onehot_many": [_P, _P, C.c_uint32],
     "aixk_matmul": [_P, _T, _T, _T],
     "aixk_matmul_batched": [_P, _T, _T, _T],
     "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],

@@ -163,6 +163,14 @@ int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, c
  * caller issues before argmaxIndicesTo, aixCore.hpp:927-941, folded in: over a handful of rows the
  * one-hot block is then written densely in a single pass). */
 int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t dim);
+/* `count` argmaxIndicesTo calls, each with the zero fill of its destination folded in (item k is
+ * aixk_argmax_to(ctx, 2, src, dst, dim) of its fields): the masks that the backward pass of max() asks for head after
+ * head (aixCore.hpp:927-941, 2170-2175).  One launch when every item is a dense tensor of one element type reduced along its
+ * last dim (rows of at least 32 elements, a multiple of 4 and of 16 bytes) and there are at most AIXK_ARGMAX_ITEMS_MAX
+ * items, otherwise item by item in order.  The caller guarantees that no item reads what another one writes. */
+#define AIXK_ARGMAX_ITEMS_MAX 1024
+typedef struct aixk_argmax_item { aixhip_tensor src, dst; uint64_t dim; } aixk_argmax_item;
+int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, uint32_t count);
 
 /* ---- matmul (aixDevice.hpp:63; aixDeviceCPU.cpp:362-389) ---------------- */
 /* out[m,n] = a[m,k] . b[k,n]; a, b arbitrary 2-D views; f32/f16/bf16 run on MFMA with f32

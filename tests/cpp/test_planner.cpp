@@ -967,9 +967,33 @@ static void testLoneCastsAsKernelsAndTheManyBlocksForm()
     }
     CHECK(r == HIPRTC_SUCCESS);
     hiprtcDestroyProgram(&prog);
-    bool threw = false;
-    try { (void)gen::source(d, gen::Shape::Rows, 0, true, false, true); } catch (const std::invalid_argument&) { threw = true; }
-    CHECK(threw);
+    // the other launch shapes and a row program have the form too (one operator applied head by head)
+    auto compilesText = [&](const std::string& text, const std::string& entry) {
+        if (text.find(entry + "_many(const Args* table, const u32* starts, u32 count)") == std::string::npos) return false;
+        hiprtcProgram p3;
+        if (hiprtcCreateProgram(&p3, text.c_str(), "m3.hip", 1, texts, names) != HIPRTC_SUCCESS) return false;
+        const hiprtcResult r3 = hiprtcCompileProgram(p3, 4, opts);
+        if (r3 != HIPRTC_SUCCESS) {
+            size_t n = 0; hiprtcGetProgramLogSize(p3, &n);
+            std::string log(n, 0); if (n) hiprtcGetProgramLog(p3, &log[0]);
+            std::printf("---- hipRTC log ----\n%s\n---- source ----\n%s\n", log.c_str(), text.c_str());
+        }
+        hiprtcDestroyProgram(&p3);
+        return r3 == HIPRTC_SUCCESS;
+    };
+    CHECK(compilesText(gen::source(d, gen::Shape::Rows, 0, true, false, true), gen::entryName(d, gen::Shape::Rows)));
+    CHECK(compilesText(gen::source(d, gen::Shape::Gather, 0, true, false, true), gen::entryName(d, gen::Shape::Gather)));
+    {
+        Capture rows;
+        FuseEngine g(config(), rows.callbacks());
+        recordSoftmax(g, DataType::kBFloat16, 8, 512);
+        g.flush();
+        CHECK(rows.fused.size() == 1);
+        gen::RowGeometry geo;
+        if (rows.fused.size() == 1 && gen::rowGeometry(rows.fused[0], &geo))
+            CHECK(compilesText(gen::rowSource(rows.fused[0], geo, false, true), gen::rowEntryName(rows.fused[0], geo)));
+        else CHECK(false);
+    }
     // the chain of the benchmark in its many-blocks form
     Capture chain;
     FuseEngine f(config(), chain.callbacks());
@@ -983,6 +1007,73 @@ static void testLoneCastsAsKernelsAndTheManyBlocksForm()
         CHECK(hiprtcCompileProgram(p2, 4, opts) == HIPRTC_SUCCESS);
         hiprtcDestroyProgram(&p2);
     }
+}
+
+static void testEqualKernelsLeaveSideBySide()
+{
+    // head after head, three kernels each: b = tril(a)^2, y = b - max(b) row by row (a triangle cannot be part of a row
+    // program), c = triu(y)^2.  The planner closes a kernel when the next one reads its result, so its list goes
+    // A0 B0 A1 B1 ... and the C's last; with groupEqualKernels the A's leave side by side, then the B's, then the C's,
+    // and a kernel that depends on another never overtakes it, also through a buffer written twice.
+    auto run = [&](bool group, std::vector<FusedSubgraphDescriptor>* fused, std::vector<OpRecord>* singles) {
+        Capture cap;
+        FuseConfig c = config();
+        c.groupEqualKernels = group;
+        FuseEngine e(c, cap.callbacks());
+        uint8_t lowest[8] = {};
+        lowestScalarInto(DataType::kFloat32, lowest);
+        auto P = [](uintptr_t id) { return reinterpret_cast<void*>(id * 0x10000); };
+        for (uintptr_t k = 0; k < 4; ++k) {
+            const uintptr_t id = 10 * (k + 1);
+            auto a = T(id + 1, {8, 256}), t = T(id + 2, {8, 256}), b = T(id + 3, {8, 256}), m = T(id + 4, {8, 1}), y = T(id + 5, {8, 256});
+            auto u = T(id + 6, {8, 256}), c2 = T(id + 7, {8, 256});
+            auto mB = T(id + 4, {8, 256}, DataType::kFloat32, {1, 0});
+            for (uintptr_t j = 1; j <= 7; ++j) e.retainBuffer(P(id + j));
+            e.recordTri(OpType::Tril, View(a), View(t), 0);
+            e.record(OpType::Mul, View(t), View(t), View(b));
+            e.releaseBuffer(P(id + 2));
+            e.recordRowReduce(OpType::MaxTo, View(b), View(m), lowest, 256);
+            e.record(OpType::Sub, View(b), View(mB), View(y));
+            e.releaseBuffer(P(id + 4));
+            e.recordTri(OpType::Triu, View(y), View(u), 0);
+            e.record(OpType::Mul, View(u), View(u), View(c2));
+            e.releaseBuffer(P(id + 6));
+        }
+        // one buffer written by two kernels in turn: z = exp(a_0) (alive) is read by a row program, then z = sqrt(a_1)
+        auto a0 = T(11, {8, 256}), a1 = T(21, {8, 256}), z = T(90, {8, 256}), mz = T(91, {8, 1});
+        for (uintptr_t id : {90, 91}) e.retainBuffer(P(id));
+        e.recordTri(OpType::Tril, View(a0), View(z), 3);
+        e.recordRowReduce(OpType::MaxTo, View(z), View(mz), lowest, 256);
+        e.recordTri(OpType::Tril, View(a1), View(z), 4);
+        e.flush();
+        *fused = cap.fused; *singles = cap.singles;
+        if (std::getenv("AIX_TEST_VERBOSE")) for (auto& o : cap.order) std::printf("  %s %s\n", group ? "grouped" : "plain  ", o.c_str());
+    };
+    std::vector<FusedSubgraphDescriptor> fa, fb;
+    std::vector<OpRecord> sa, sb;
+    run(false, &fa, &sa);
+    run(true, &fb, &sb);
+    CHECK(fa.size() == 12 && fb.size() == 12 && sa.size() == 3 && sb.size() == 3);
+    if (fa.size() != 12 || fb.size() != 12 || sb.size() != 3) return;
+    auto kindOf = [](const FusedSubgraphDescriptor& d) { return d.ops[0].type == OpType::Tril ? 'A' : d.ops[0].type == OpType::Triu ? 'C' : 'B'; };
+    std::string plain, grouped;
+    for (const auto& d : fa) plain += kindOf(d);
+    for (const auto& d : fb) grouped += kindOf(d);
+    CHECK(plain == "ABABABABCCCC");
+    CHECK(grouped == "AAAABBBBCCCC");
+    // each head's three kernels in order (B reads A's output, C reads B's)
+    for (uintptr_t k = 0; k < 4; ++k) {
+        const void* b = reinterpret_cast<const void*>((10 * (k + 1) + 3) * 0x10000);
+        const void* y = reinterpret_cast<const void*>((10 * (k + 1) + 5) * 0x10000);
+        size_t ia = SIZE_MAX, ib = SIZE_MAX, ic = SIZE_MAX;
+        for (size_t j = 0; j < fb.size(); ++j) {
+            for (const auto& o : fb[j].outputBuffers) { if (o.data == b) ia = j; if (o.data == y) ib = j; }
+            for (const auto& in : fb[j].inputBuffers) if (in.data == y && kindOf(fb[j]) == 'C') ic = j;
+        }
+        CHECK(ia < ib && ib < ic && ic != SIZE_MAX);
+    }
+    // the two writers of z and the reader between them (single operators) keep their order
+    CHECK(sb[0].type == OpType::Tril && sb[0].triDiagonal == 3 && sb[1].type == OpType::MaxTo && sb[2].type == OpType::Tril && sb[2].triDiagonal == 4);
 }
 
 int main(int argc, char** argv)
@@ -1016,6 +1107,7 @@ int main(int argc, char** argv)
     testLayerNormPiecesShareOneRowProgram();
     testIdleFillsWaitForTheirFirstUser();
     testLoneCastsAsKernelsAndTheManyBlocksForm();
+    testEqualKernelsLeaveSideBySide();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
 }

@@ -1,6 +1,7 @@
 """The kernel-layer entry points that carry several pieces of work in one launch, through the C ABI: aixk_fill_many
 (small fills, each item a pattern already in its destination's element type), aixk_rtc_launch_many (several argument
-blocks of one runtime-compiled kernel, each with its share of the grid) and aixk_slice_set_many (several sliceSet calls).
+blocks of one runtime-compiled kernel, each with its share of the grid), aixk_slice_set_many (several sliceSet calls) and
+aixk_argmax_onehot_many (several argmaxIndicesTo calls with their zero fill).
 Results against numpy (fills and an exact elementwise body) and the CPU oracle's sliceSet, sizes down to one element and
 ragged tails, and the argument checks they promise."""
 import ctypes as C
@@ -203,4 +204,48 @@ def test_slice_set_many_checks_its_items(gpu):
     gpu.ctx.sync()
     got = gpu.fetch(pd, dst.storage)
     assert np.all(got == 1), "a refused call must launch nothing"
+    gpu.release()
+
+
+def _argmax_items(entries):
+    arr = (K.ArgmaxItem * len(entries))()
+    for k, (src, dst, dim) in enumerate(entries):
+        arr[k].src, arr[k].dst, arr[k].dim = src, dst, dim
+    return arr
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.F16], ids=["bf16", "f32", "f16"])
+def test_argmax_onehot_many_is_fill_and_argmax_indices_item_by_item(gpu, dtype):
+    """Dense tensors reduced along their last dim leave in one launch; a set with an item of another kind (another dim,
+    a strided source) runs item by item.  Either way every destination equals zeros + the oracle's argmaxIndicesTo:
+    ties (values on a coarse grid) go to the first maximum, a row of NaNs picks its first element."""
+    rng = np.random.default_rng(55000 + dtype)
+
+    def case(shape, dim, kind="contig"):
+        src = T.view_tensor(rng, dtype, shape, kind, lo=-2, hi=2)
+        vals = O.to_float64(src.storage, dtype)
+        src.storage[:] = O.to_storage(np.round(vals * 4) / 4, dtype)
+        if shape[-1] >= 64:
+            src.storage[: shape[-1]] = O.to_storage(np.full(shape[-1], np.nan), dtype)       # the first row: NaNs only
+        want = T.empty(O.I32, shape)
+        assert CPU.argmax_indices_to(C.byref(src.desc()), C.byref(want.desc()), dim) == 0
+        _, dsrc = gpu.put(src)
+        pd, dd = gpu.put(T.empty(O.I32, shape, fill=9))                                      # every element must be written
+        return (dsrc, dd, dim), (pd, want, f"{shape} dim={dim} {kind}")
+
+    together = [case([64, 512], 1), case([3, 40, 64], 2), case([1, 32], 1), case([517, 96], 1), case([2, 2, 2, 128], 3)]
+    G.run_gpu(gpu, "aixk_argmax_onehot_many", _argmax_items([c[0] for c in together]), len(together))
+    for _, (pd, want, what) in together:
+        T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, "argmaxIndicesTo of several items, one launch: " + what)
+    mixed = [case([64, 512], 1), case([40, 64], 0), case([8, 48], 1, "transposed"), case([5, 30], 1)]
+    G.run_gpu(gpu, "aixk_argmax_onehot_many", _argmax_items([c[0] for c in mixed]), len(mixed))
+    for _, (pd, want, what) in mixed:
+        T.assert_same_bits(gpu.fetch(pd, want.storage), want.storage, "argmaxIndicesTo of several items, item by item: " + what)
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    assert lib.aixk_argmax_onehot_many(h, None, 0) == 0
+    bad_src, bad_dst, _ = together[0][0]
+    wrong = K.Tensor.from_buffer_copy(bad_dst)
+    wrong.dtype = O.F32
+    assert lib.aixk_argmax_onehot_many(h, _argmax_items([together[1][0], (bad_src, wrong, 1)]), 2) == 1      # result must be int32
+    gpu.ctx.sync()
     gpu.release()

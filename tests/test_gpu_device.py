@@ -636,6 +636,54 @@ def test_fill_is_folded_into_argmax_indices_to(dev):
     dev.release()
 
 
+def test_runs_of_argmax_indices_to_leave_as_one_launch(dev):
+    """The masks of max()'s backward pass, head after head (aixCore.hpp:2170-2175): calls whose zero fill was folded in
+    wait and leave in one launch; a recorded operator that reads a mask, a source that a recorded operator produces, and
+    a mask whose buffer is also the next call's source keep their order.  Against the oracle call by call."""
+    set_diag(dev)
+    rng = np.random.default_rng(44000)
+    dtype = O.BF16
+    shape = [64, 128]
+    zero = np.zeros(1, np.float32)
+
+    def mask_of(src_host, src_desc):
+        want = T.empty(O.I32, shape)
+        assert CPU.fill(zero.ctypes.data, O.F32, C.byref(want.desc())) == 0
+        assert CPU.argmax_indices_to(C.byref(src_host.desc()), C.byref(want.desc()), 1) == 0
+        pm = dev.raw(want.storage.nbytes)
+        dm = H.kdesc(want, pm)
+        dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(dm))
+        dev.dev.call("argmax_indices_to", H.ref(src_desc), H.ref(dm), 1)
+        return pm, dm, want
+
+    srcs = [T.contiguous_tensor(rng, dtype, shape, lo=-1, hi=1) for _ in range(6)]
+    ups = [dev.put(x) for x in srcs]
+    dev.dev.synchronize()
+    before = dev.dev.batched_launch_stats()
+    masks = [mask_of(x, d) for x, (_, d) in zip(srcs, ups)]
+    got = [dev.fetch(pm, want.storage) for pm, _, want in masks]
+    after = dev.dev.batched_launch_stats()
+    assert after[0] - before[0] == 1 and after[1] - before[1] == len(srcs), (before, after)
+    for g, (_, _, want) in zip(got, masks):
+        T.assert_same_bits(g, want.storage, "six masks in one launch")
+    # a source that is a recorded sum, and a recorded conversion + product that reads the mask while it waits
+    rec = Recorder(dev, dtype, shape)
+    x, y = rec.leaf(srcs[0]), rec.leaf(srcs[1])
+    total = rec.binary(O.ADD, x, y)
+    pm, dm, want = mask_of(total["host"], total["desc"])
+    as16 = T.empty(dtype, shape)
+    assert CPU.copy(want.storage.ctypes.data, O.I32, as16.storage.ctypes.data, dtype, want.size) == 0
+    p16 = dev.raw(as16.storage.nbytes)
+    dev.dev.call("copy", pm, O.I32, p16, dtype, want.size)
+    prod = rec.binary(O.MUL, {"host": as16, "ptr": p16, "desc": H.kdesc(as16, p16)}, x)
+    # the next mask overwrites a buffer that the waiting product still reads: x's own storage is its destination's source
+    pm2, dm2, want2 = mask_of(prod["host"], prod["desc"])
+    T.assert_same_bits(dev.fetch(prod["ptr"], prod["host"].storage), prod["host"].storage, "mask * x, recorded while the mask waited")
+    T.assert_same_bits(dev.fetch(pm, want.storage), want.storage, "mask of a recorded sum")
+    T.assert_same_bits(dev.fetch(pm2, want2.storage), want2.storage, "mask of the product")
+    dev.release()
+
+
 def test_tril_and_triu_join_the_fused_kernels(dev):
     """tril / triu recorded as elementwise operators: attention's tril(s) * scale + mask is ONE generated kernel
     (the triangle's extents and diagonal are run-time integers of it), negate -> triu over a dense stack takes the flat
