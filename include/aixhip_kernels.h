@@ -121,7 +121,8 @@ int32_t aixk_slice_set(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_ten
  * of slices writes, :2228-2233, arrive as runs of Device::sliceSet calls that do not depend on one another): item k is
  * aixk_slice_set(src, dst, dim, start, end, step) of its fields.  All items have one element size; the caller
  * guarantees that no item reads or overwrites what another one writes.  AIXK_EINVAL for more than
- * AIXK_SLICE_ITEMS_MAX items, an empty item, or an item aixk_slice_set would reject; nothing is launched then. */
+ * AIXK_SLICE_ITEMS_MAX items, an empty item, or an item aixk_slice_set would reject; nothing is launched then.
+ * No counterpart in the reference's interface (one Device::sliceSet call per part there). */
 #define AIXK_SLICE_ITEMS_MAX 512
 typedef struct aixk_slice_item { aixhip_tensor src, dst; uint64_t dim, start, end, step; } aixk_slice_item;
 int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_t count);
@@ -167,7 +168,8 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
  * aixk_argmax_to(ctx, 2, src, dst, dim) of its fields): the masks that the backward pass of max() asks for head after
  * head (aixCore.hpp:927-941, 2170-2175).  One launch when every item is a dense tensor of one element type reduced along its
  * last dim (rows of at least 32 elements, a multiple of 4 and of 16 bytes) and there are at most AIXK_ARGMAX_ITEMS_MAX
- * items, otherwise item by item in order.  The caller guarantees that no item reads what another one writes. */
+ * items, otherwise item by item in order.  The caller guarantees that no item reads what another one writes.
+ * No counterpart in the reference's interface (one Device::argmaxIndicesTo call per tensor there). */
 #define AIXK_ARGMAX_ITEMS_MAX 1024
 typedef struct aixk_argmax_item { aixhip_tensor src, dst; uint64_t dim; } aixk_argmax_item;
 int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, uint32_t count);
