@@ -250,8 +250,26 @@ static void planner_traffic(unsigned seed, int rounds)
             for (int k = 0; k < 4; ++k) dev.unary(tensor(full[rng() % full.size()], {n}), tensor(fresh_full(), {n}));
         } else if (what < 76) {                                        // an operand inside a block
             dev.unary(tensor((char*)x + 64 * 4, {len}), tensor(fresh_full(), {len}));
-        } else if (what < 84) {                                        // an operator that runs at once
+        } else if (what < 79) {                                        // an operator that runs at once
             dev.transpose(tensor(x, {rows, len}), tensor(fresh_full(), {len, rows}), 0, 1);
+        } else if (what < 82) {                                        // a cat: row blocks of a fresh tensor, the sources may die at once
+            void* whole = fresh_full();
+            for (size_t k = 0; k < 4; ++k) {
+                void* part = dev.allocate(n);                          // [rows / 4, len] of f32
+                dev.unary(tensor(x, {rows / 4, len}), tensor(part, {rows / 4, len}));
+                dev.sliceSet(tensor(part, {rows / 4, len}), tensor(whole, {rows, len}), 0, k * (rows / 4), (k + 1) * (rows / 4), 1);
+                dev.deallocate(part);
+            }
+            if (what & 1) dev.sliceSet(tensor(x, {rows / 4, len}), tensor(whole, {rows, len}), 0, 3, 3 + rows / 4, 1);      // overlaps two of them
+        } else if (what < 84) {                                        // masks of max()'s backward, then a matmul that waits beside them
+            for (int k = 0; k < 3; ++k) {
+                void* mask = fresh_full();
+                dev.fill(&zero, DataType::kFloat32, tensor(mask, {rows, len}, DataType::kInt32));
+                dev.argmaxIndicesTo(tensor(full[rng() % (full.size() - 1)], {rows, len}), tensor(mask, {rows, len}, DataType::kInt32), 1);
+            }
+            void* h = dev.allocate(n * 4);
+            full.push_back(h);
+            dev.matmul(tensor(x, {64, 64}, DataType::kBFloat16), tensor(full[0], {64, 64}, DataType::kBFloat16), tensor(h, {64, 64}, DataType::kBFloat16));
         } else if (what < 92 && full.size() > 4) {                     // temporaries die
             const size_t k = 3 + rng() % (full.size() - 3);
             dev.deallocate(full[k]); full[k] = full.back(); full.pop_back();
