@@ -85,6 +85,18 @@ def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pa
     return losses, secs, (int(counts[0]), int(counts[1]))
 
 
+def oracle_slice_gradients(which, rows, cols, x, w):
+    """(gradient by the reference's recursion, gradient by the single-pass traversal) of slicing program `which`."""
+    out = np.zeros((2, rows, cols), dtype=np.float32)
+    lib = oracle_lib()
+    lib.oracle_slice_gradients.argtypes = [C.c_int, C.c_uint64, C.c_uint64, _PF, _PF, _PF]
+    rc = lib.oracle_slice_gradients(which, rows, cols, np.ascontiguousarray(x, np.float32).ctypes.data_as(_PF),
+                                    np.ascontiguousarray(w, np.float32).ctypes.data_as(_PF), out.ctypes.data_as(_PF))
+    if rc != 0:
+        raise RuntimeError(lib.oracle_drivers_last_error().decode())
+    return out[0], out[1]
+
+
 def ref_mlp(batch, n_in, hidden, n_out, steps, lr, data):
     x, y, w, b = data
     losses = np.zeros(steps, dtype=np.float32)

@@ -47,6 +47,38 @@ def test_single_pass_backward_gives_the_same_gradients():
     assert mm_b == 30 * (3 + 5) and mm_a == 30 * (3 + 4 * 5)
 
 
+@pytest.mark.parametrize("which", range(7), ids=["cover", "gap", "overlap", "beside_a_seed", "two_dims", "strided", "heads_and_cat"])
+def test_single_pass_backward_of_slices(which):
+    """The single-pass traversal gathers the seeds of slices as windows and writes windows of one dim that do not overlap
+    into one tensor (aixCore.hpp:2228-2233 builds a zero-padded tensor per slice and adds them up): the gradient of the
+    sliced tensor must come out as the reference's recursion gives it, and as calculus does.  Small integers: exact."""
+    rows, cols = 8, 16
+    rng = np.random.default_rng(61000 + which)
+    x = rng.integers(-3, 4, (rows, cols)).astype(np.float32)
+    w = rng.integers(1, 4, (rows, cols)).astype(np.float32)
+    by_recursion, single_pass = drivers.oracle_slice_gradients(which, rows, cols, x, w)
+    assert np.array_equal(by_recursion, single_pass)
+    c2, c4, r2 = cols // 2, cols // 4, rows // 2
+    k = np.zeros((rows, cols), np.float64)                         # d loss / d h
+    if which == 0:
+        k[:, :c4] += 2; k[:, c4:c2] += 3; k[:, c2:] += 5
+    elif which == 1:
+        k[:, :c4] += 2; k[:, c2:] += 5
+    elif which == 2:
+        k[:, :c2] += 2; k[:, c4:] += 3
+    elif which == 3:
+        k[:, :c2] += 2; k[:, c2:] += 3; k += 2 * x * w
+    elif which == 4:
+        k[:, :c2] += 2; k[r2:, :] += 3
+    elif which == 5:
+        k[0::2, :] += 2; k[1::2, :] += 3
+    else:
+        for b in range(2):
+            for h in range(4):
+                k[b * r2:(b + 1) * r2, h * c4:(h + 1) * c4] = (h + 1 + 4 * b) * w[b * r2:(b + 1) * r2, h * c4:(h + 1) * c4]
+    assert np.array_equal(single_pass.astype(np.float64), k * w)
+
+
 def test_reference_device_test_cases_pass_on_the_reference_cpu_device():
     """A check of the checks: the device cases of oracle/ref_drivers.cpp (deviceChecks) with the reference's CPU device
     standing in as the device under test must pass without a failure."""
