@@ -768,7 +768,17 @@ private:
 
     bool mergeable(const Group& a, const Group& b) const
     {
-        if (a.rowLen || b.rowLen) return false;                // row programs grow operator by operator only
+        if (a.rowLen || b.rowLen) {
+            // a row program takes in a kernel of plain elementwise operators (or another program over rows of the same
+            // length) if everything that one loads and stores fits the rows: the conversion of a mask that a row
+            // program multiplies with then happens at the program's load instead of in a pass of its own
+            const size_t length = a.rowLen ? a.rowLen : b.rowLen;
+            if (a.dtype != b.dtype || a.count != b.count || !rowsFit(a, length) || !rowsFit(b, length)) return false;
+            if (a.hasTri || b.hasTri) return false;
+            size_t slots = a.loads.size();
+            for (const ViewRef& r : b.loads) if (!loads(a, view(r))) ++slots;
+            return slots + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;
+        }
         if (a.dtype != b.dtype || a.count != b.count) return false;
         if (!a.shape->sameShape(*b.shape) && !a.dense && !b.dense) return false;
         size_t count = a.loads.size();
@@ -790,6 +800,7 @@ private:
         a.dense = a.dense && b.dense;
         a.hasScalar = a.hasScalar || b.hasScalar;
         a.hasTri = a.hasTri || b.hasTri;
+        if (!a.rowLen) a.rowLen = b.rowLen;
         for (size_t w : b.ops) m_groupOf[w] = into;
         b.ops.clear(); b.defs.clear(); b.loads.clear();
         b.open = false;                                     // absorbed: never emitted on its own

@@ -1009,6 +1009,45 @@ static void testLoneCastsAsKernelsAndTheManyBlocksForm()
     }
 }
 
+static void testRowProgramTakesInAPlainKernel()
+{
+    // max()'s backward inside a softmax gradient: m = rowmax(x) ... c = cast(mask: int32 -> f32), y = c * m (m broadcast
+    // along the row).  The cast starts a kernel of its own (nothing defines or loads its operand); when the product needs
+    // both the cast's value and the row program's per-row value, the two kernels become one: the mask is converted at
+    // the row program's load, there is no pass that writes a converted copy.
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    const size_t rows = 16, L = 512;
+    auto x = T(1, {rows, L}), m = T(2, {rows, 1}), mask = T(3, {rows, L}, DataType::kInt32), c = T(4, {rows, L}), y = T(5, {rows, L});
+    auto mB = T(2, {rows, L}, DataType::kFloat32, {1, 0});
+    for (uintptr_t id : {1, 2, 3, 4, 5}) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    uint8_t lowest[8] = {};
+    lowestScalarInto(DataType::kFloat32, lowest);
+    e.recordRowReduce(OpType::MaxTo, View(x), View(m), lowest, L);
+    e.record(OpType::Cast, View(mask), View(c));
+    e.record(OpType::Mul, View(c), View(mB), View(y));
+    e.releaseBuffer(reinterpret_cast<void*>(uintptr_t(4) * 0x10000));
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() != 1) return;
+    const auto& d = cap.fused[0];
+    CHECK(d.rowLength == L && d.ops.size() == 3 && d.inputBuffers.size() == 2);
+    bool sawMask = false;
+    for (const auto& in : d.inputBuffers) if (in.dtype == DataType::kInt32) sawMask = true;
+    CHECK(sawMask);
+    CHECK(d.outputBuffers.size() == 2);                         // m and y; the converted mask is never stored
+    CHECK(compilesRow(d));
+    // a plain kernel with a triangle stays apart (its index arithmetic is not available row by row)
+    Capture cap2;
+    FuseEngine f(config(), cap2.callbacks());
+    for (uintptr_t id : {1, 2, 3, 4, 5}) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    f.recordRowReduce(OpType::MaxTo, View(x), View(m), lowest, L);
+    f.recordTri(OpType::Tril, View(T(3, {rows, L})), View(c), 0);
+    f.record(OpType::Mul, View(c), View(mB), View(y));
+    f.flush();
+    CHECK(cap2.fused.size() + cap2.singles.size() >= 2);
+}
+
 static void testEqualKernelsLeaveSideBySide()
 {
     // head after head, three kernels each: b = tril(a)^2, y = b - max(b) row by row (a triangle cannot be part of a row
@@ -1107,6 +1146,7 @@ int main(int argc, char** argv)
     testLayerNormPiecesShareOneRowProgram();
     testIdleFillsWaitForTheirFirstUser();
     testLoneCastsAsKernelsAndTheManyBlocksForm();
+    testRowProgramTakesInAPlainKernel();
     testEqualKernelsLeaveSideBySide();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;
