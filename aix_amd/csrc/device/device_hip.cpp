@@ -244,7 +244,8 @@ DeviceHIP::DeviceHIP(size_t deviceIndex)
         std::cerr << "DeviceHIP: device memory is not host-addressable on this system; tensors must be moved with "
                      "copy()/copyToHost() and never dereferenced on the host." << std::endl;
     FuseConfig cfg;
-    cfg.maxBufferSlots = 24;
+    cfg.maxBufferSlots = 40;                                 // (pointer arguments are cheap here; 24 cut GeLU's backward formula, 11 loads and 6 stores, in two)
+    if (const char* e = std::getenv("AIXHIP_MAX_BUFFER_SLOTS"); e && *e) cfg.maxBufferSlots = std::max<size_t>(4, std::min<size_t>(60, std::strtoull(e, nullptr, 10)));
     cfg.supportsStridedFusion = true;
     m_extras = std::make_unique<Extras>();
     setFuseConfig(cfg);
