@@ -219,6 +219,8 @@ RowOperand rowOperandKind(const View& v, size_t rows, size_t length)
 {
     if (!v.data || rows == 0 || length == 0) return RowOperand::None;
     const size_t vec = 16 / aix::Device::dataTypeSize(v.dtype);
+    bool still = v.size > 1;                                                   // one element seen everywhere: a scalar tensor, broadcast
+    for (uint32_t d = 0; d < v.rank; ++d) if (v.shape[d] > 1 && v.strides[d] != 0) still = false;
     if (v.size == rows * length) {
         if (v.dense) return v.offset % vec == 0 ? RowOperand::Dense : RowOperand::None;
         const int split = rowSplit(v, length);
@@ -227,14 +229,35 @@ RowOperand rowOperandKind(const View& v, size_t rows, size_t length)
         auto zeros = [&](int from, int to) { for (int d = from; d < to; ++d) if (v.shape[d] > 1 && v.strides[d] != 0) return false; return true; };
         auto dense = [&](int from, int to) { size_t run = 1; for (int d = to - 1; d >= from; --d) { if (v.shape[d] > 1 && v.strides[d] != run) return false; run *= v.shape[d]; } return true; };
         if (zeros(split, (int)v.rank) && dense(0, split)) return RowOperand::PerRowBroadcast;            // one value per row, repeated along it
-        if (dense(split, (int)v.rank) && zeros(0, split)) return v.offset % vec == 0 ? RowOperand::RowVector : RowOperand::None;   // one row for all rows
+        if (still) return RowOperand::Single;
+        // a dense block of whole rows that comes round again and again: one row for all rows, or the [seq, seq] mask of
+        // attention under [batch, heads, seq, seq] scores (the dims in front of the block have stride 0)
+        int from = (int)v.rank;
+        { size_t run = 1; while (from > 0 && (v.shape[from - 1] == 1 || v.strides[from - 1] == run)) { --from; run *= v.shape[from]; } }
+        if (from > split) return RowOperand::None;
+        while (from < split && !zeros(0, from)) ++from;            // (extent-1 dims may sit on either side)
+        if (zeros(0, from) && dense(from, (int)v.rank)) return v.offset % vec == 0 ? RowOperand::RowVector : RowOperand::None;
         return RowOperand::None;
     }
     if (v.size == rows && v.dense) return RowOperand::PerRow;
+    if (v.size == rows && still) return RowOperand::Single;
     return RowOperand::None;
 }
 
+size_t rowOperandPeriod(const View& v, size_t rows, size_t length)
+{
+    if (rowOperandKind(v, rows, length) != RowOperand::RowVector) return 0;
+    // the dims with a stride: everything behind the zero-stride dims in front
+    size_t block = 1;
+    int d = 0;
+    while (d < (int)v.rank && (v.shape[d] == 1 || v.strides[d] == 0)) ++d;
+    for (; d < (int)v.rank; ++d) block *= v.shape[d];
+    return block / length ? block / length : 1;
+}
+
 namespace {
+
+bool isTriOp(OpType t) { return t == OpType::Tril || t == OpType::Triu; }
 
 bool sameView(const View& a, const View& b)
 {
@@ -686,11 +709,12 @@ private:
     bool rowsFit(const Group& g, size_t length) const
     {
         if (g.rowLen) return g.rowLen == length;
-        if (g.hasTri || length == 0 || g.count % length != 0) return false;
+        if (length == 0 || g.count % length != 0) return false;
+        if (g.hasTri) for (size_t op : g.ops) if (isTriOp(at(op).type) && at(op).triCols != length) return false;
         const size_t rows = g.count / length;
         for (const ViewRef& r : g.loads) {
             const RowOperand k = rowOperandKind(view(r), rows, length);
-            if (k != RowOperand::Dense && k != RowOperand::PerRowBroadcast && k != RowOperand::RowVector) return false;
+            if (k != RowOperand::Dense && k != RowOperand::PerRowBroadcast && k != RowOperand::RowVector && k != RowOperand::Single) return false;
         }
         for (size_t def : g.defs) if (rowOperandKind(defView(def), rows, length) != RowOperand::Dense) return false;
         return true;
@@ -701,12 +725,13 @@ private:
     {
         const size_t rows = g.rows();
         const bool per = op.output.size == rows && op.output.size != g.count;
-        if (op.type == OpType::Tril || op.type == OpType::Triu) return false;
+        if (isTriOp(op.type) && (per || op.triCols != g.rowLen)) return false;        // a matrix row must be a row of the program
         if (rowOperandKind(op.output, rows, g.rowLen) != (per ? RowOperand::PerRow : RowOperand::Dense)) return false;
         const View* in[2] = {&op.input0, op.hasInput1 ? &op.input1 : nullptr};
         for (int k = 0; k < 2; ++k) {
             if (!in[k] || !in[k]->data || resolved[k].kind != Operand::kMemory) continue;
             const RowOperand kind = rowOperandKind(*in[k], rows, g.rowLen);
+            if (kind == RowOperand::Single) continue;
             if (per ? kind != RowOperand::PerRow : (kind != RowOperand::Dense && kind != RowOperand::PerRowBroadcast && kind != RowOperand::RowVector)) return false;
         }
         return true;
@@ -753,7 +778,8 @@ private:
         if (g.rowLen) {
             // a row program takes operators on whole rows and operators on per-row values; what their memory operands
             // look like is checked once the operands are resolved (rowOperandsFit)
-            if (g.dtype != type || op.type == OpType::Tril || op.type == OpType::Triu) return false;
+            if (g.dtype != type) return false;
+            if (isTriOp(op.type)) return op.output.size == g.count && op.triCols == g.rowLen;
             return op.output.size == g.count || op.output.size == g.rows();
         }
         if (g.dtype != type || g.count != op.output.size) return false;
@@ -774,7 +800,6 @@ private:
             // program multiplies with then happens at the program's load instead of in a pass of its own
             const size_t length = a.rowLen ? a.rowLen : b.rowLen;
             if (a.dtype != b.dtype || a.count != b.count || !rowsFit(a, length) || !rowsFit(b, length)) return false;
-            if (a.hasTri || b.hasTri) return false;
             size_t slots = a.loads.size();
             for (const ViewRef& r : b.loads) if (!loads(a, view(r))) ++slots;
             return slots + a.defs.size() + b.defs.size() + 1 <= m_cfg.maxBufferSlots;

@@ -110,10 +110,13 @@ struct OpRecord {
 };
 
 // How a view takes part in a kernel that works row by row on [rows, length] data (a "row program"): element for element,
-// one value per row repeated along the row, one row repeated for every row, one value per row (operand of a per-row
-// operator), or not at all.
-enum class RowOperand { Dense, PerRowBroadcast, RowVector, PerRow, None };
+// one value per row repeated along the row, a dense block of one or more whole rows that every so many rows see again
+// (one row for all rows: gamma of a LayerNorm; the [seq, seq] mask under [batch, heads, seq, seq] scores), one value per
+// row (operand of a per-row operator), one element seen from everywhere (a scalar tensor, broadcast), or not at all.
+enum class RowOperand { Dense, PerRowBroadcast, RowVector, PerRow, Single, None };
 RowOperand rowOperandKind(const View& v, size_t rows, size_t length);
+// RowVector operands: how many rows the block holds that every row sees as (row % period); 0 for the other kinds.
+size_t rowOperandPeriod(const View& v, size_t rows, size_t length);
 
 // One fused kernel: ops in execution order.  An operand index below inputBuffers.size() names an
 // external buffer, an index at or above it names the result of ops[index - inputBuffers.size()];

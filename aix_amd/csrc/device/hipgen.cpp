@@ -331,6 +331,7 @@ char kindLetter(fuse::RowOperand k)
         case fuse::RowOperand::PerRowBroadcast: return 'b';
         case fuse::RowOperand::RowVector: return 'r';
         case fuse::RowOperand::PerRow: return 'p';
+        case fuse::RowOperand::Single: return 's';
         default: return '?';
     }
 }
@@ -372,7 +373,8 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
 {
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size(), NS = scalarCount(d);
     if (NO == 0) throw std::invalid_argument("fused kernel without outputs");
-    if (triCount(d)) throw std::invalid_argument("row program: tril / triu cannot be part of it");
+    const size_t NT = triCount(d);
+    if (d.opParams.size() != 3 * NT) throw std::invalid_argument("fused kernel: tril / triu without its parameters");
     const size_t esz = aix::Device::dataTypeSize(d.dtype);
     const size_t AI = NI ? NI : 1, AS = NS ? NS : 1;
     std::vector<fuse::RowOperand> kinds(NI);
@@ -388,7 +390,9 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     for (size_t k = 0; k < NO; ++k) o << "typedef " << typeName(d.outputBuffers[k].dtype) << " O" << k << ";\n";
     auto to_t = [&](size_t k, const std::string& e) { return d.inputBuffers[k].dtype == d.dtype ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
     auto from_t = [&](size_t k, const std::string& e) { return d.outputBuffers[k].dtype == d.dtype ? e : "convert<T, O" + std::to_string(k) + ">(" + e + ")"; };
-    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 rows;\n    u64 len;\n};\n\n";
+    o << "struct Args {\n    const void* in[" << AI << "];\n    void* out[" << NO << "];\n    u64 sc[" << AS << "];\n    u64 per[" << AI << "];\n";
+    if (NT) o << "    u64 tp[" << 3 * NT << "];\n";
+    o << "    u64 rows;\n    u64 len;\n};\n\n";
     if (many) {
         o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "_many(const Args* table, const u32* starts, u32 count)\n{\n"
           << "    u32 lo = 0, hi = count;\n"
@@ -413,12 +417,15 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     // operands: whole rows (their own or the one shared row) as vectors, per-row values as scalars
     for (size_t k = 0; k < NI; ++k) {
         if (kinds[k] == fuse::RowOperand::Dense || kinds[k] == fuse::RowOperand::RowVector) {
-            const char* base = kinds[k] == fuse::RowOperand::Dense ? " + row * a.len" : "";
+            // (a block of rows that comes round again: row % period, period 1 for the one row all rows share)
+            const std::string base = kinds[k] == fuse::RowOperand::Dense ? " + row * a.len" : " + (row % a.per[" + std::to_string(k) + "]) * a.len";
             o << "        T x" << k << "[NV][VEC];\n#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n"
               << "            const u64 v = lane + (u64)j * G;\n"
               << "            vec<I" << k << ", VEC> r;\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) r.v[e] = zero<I" << k << ">();\n"
               << "            if (v < nvec) r = ((const vec<I" << k << ", VEC>*)(in" << k << base << "))[v];\n"
               << "#pragma unroll\n            for (int e = 0; e < VEC; ++e) x" << k << "[j][e] = " << to_t(k, "r.v[e]") << ";\n        }\n";
+        } else if (kinds[k] == fuse::RowOperand::Single) {
+            o << "        const T q" << k << " = " << to_t(k, "in" + std::to_string(k) + "[0]") << ";\n";
         } else {
             o << "        const T q" << k << " = " << to_t(k, "in" + std::to_string(k) + "[row]") << ";\n";
         }
@@ -426,7 +433,7 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     auto fullOperand = [&](size_t tensorIndex, size_t scalarIndex) -> std::string {
         if (tensorIndex != SIZE_MAX) {
             if (tensorIndex < NI) {
-                if (kinds[tensorIndex] == fuse::RowOperand::PerRowBroadcast) return "q" + std::to_string(tensorIndex);
+                if (kinds[tensorIndex] == fuse::RowOperand::PerRowBroadcast || kinds[tensorIndex] == fuse::RowOperand::Single) return "q" + std::to_string(tensorIndex);
                 if (kinds[tensorIndex] == fuse::RowOperand::PerRow) throw std::invalid_argument("row program: a per-row operand of an operator on whole rows");
                 return "x" + std::to_string(tensorIndex) + "[j][e]";
             }
@@ -439,7 +446,7 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
     auto rowOperand = [&](size_t tensorIndex, size_t scalarIndex) -> std::string {
         if (tensorIndex != SIZE_MAX) {
             if (tensorIndex < NI) {
-                if (kinds[tensorIndex] != fuse::RowOperand::PerRow) throw std::invalid_argument("row program: a row operand of an operator on per-row values");
+                if (kinds[tensorIndex] != fuse::RowOperand::PerRow && kinds[tensorIndex] != fuse::RowOperand::Single) throw std::invalid_argument("row program: a row operand of an operator on per-row values");
                 return "q" + std::to_string(tensorIndex);
             }
             const size_t m = tensorIndex - NI;
@@ -477,6 +484,22 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
             if (op.outputIndex != SIZE_MAX) o << "        if (lane == 0) out" << op.outputIndex << "[row] = " << from_t(op.outputIndex, "p" + std::to_string(k)) << ";\n";
             continue;
         }
+        if (isTri(op.type)) {
+            // the row of the program is a row of the matrix: its number within the matrix, the element's column, the diagonal
+            const size_t q = 3 * op.paramIndex;
+            o << "        T v" << k << "[NV][VEC];\n        {\n            const i64 r = (i64)(row % a.tp[" << q << "]) + (i64)a.tp[" << q + 2 << "];\n"
+              << "#pragma unroll\n            for (int j = 0; j < NV; ++j) {\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) {\n"
+              << "                    const i64 c = (i64)((lane + (u64)j * G) * VEC + e);\n"
+              << "                    v" << k << "[j][e] = (" << (op.type == OpType::Triu ? "c >= r" : "c <= r") << ") ? " << fullOperand(op.inputIndex0, op.scalarIndex0) << " : zero<T>();\n"
+              << "                }\n            }\n        }\n";
+            if (op.outputIndex != SIZE_MAX) {
+                const size_t qo = op.outputIndex;
+                o << "#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n            const u64 v = lane + (u64)j * G;\n            if (v < nvec) {\n"
+                  << "                vec<O" << qo << ", VEC> w;\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) w.v[e] = " << from_t(qo, "v" + std::to_string(k) + "[j][e]") << ";\n"
+                  << "                store_sel<AIX_NT>((vec<O" << qo << ", VEC>*)(out" << qo << " + row * a.len) + v, w);\n            }\n        }\n";
+            }
+            continue;
+        }
         o << "        T v" << k << "[NV][VEC];\n#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n#pragma unroll\n            for (int e = 0; e < VEC; ++e) v" << k << "[j][e] = ";
         if (op.type == OpType::Cast) o << fullOperand(op.inputIndex0, op.scalarIndex0);
         else {
@@ -509,7 +532,13 @@ void packRowArgsInto(std::vector<uint64_t>& a, const FusedSubgraphDescriptor& d,
         if (k < NS) std::memcpy(&bits, d.scalarData.data() + k * esz, esz);
         a.push_back(bits);
     }
-    a.push_back(d.elementCount / d.rowLength);
+    const size_t rows = d.elementCount / d.rowLength;
+    for (size_t k = 0; k < AI; ++k) {
+        const size_t period = k < NI ? fuse::rowOperandPeriod(d.inputBuffers[k], rows, d.rowLength) : 0;
+        a.push_back(period ? period : 1);
+    }
+    for (uint64_t v : d.opParams) a.push_back(v);
+    a.push_back(rows);
     a.push_back(d.rowLength);
 }
 

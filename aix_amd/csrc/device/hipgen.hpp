@@ -49,7 +49,8 @@ struct RowGeometry {
 bool rowGeometry(const fuse::FusedSubgraphDescriptor& d, RowGeometry* g);
 void rowSignatureInto(std::string& out, const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut);
 std::string rowSource(const fuse::FusedSubgraphDescriptor& d, const RowGeometry& g, bool streamOut, bool many = false);     // (many: as for source())
-// Args of a row program: in[], out[], immediates, rows, rowLength
+// Args of a row program: in[], out[], immediates, per input the period of its block of rows (1 where it has none), the
+// (rows, cols, diagonal) of every tril / triu, rows, rowLength
 void packRowArgsInto(std::vector<uint64_t>& a, const fuse::FusedSubgraphDescriptor& d, const void* const* inputs, void* const* outputs);
 
 // The kernel's symbol: "aix_fused_<type>_<launch shape>_<operators in order>" (what a profiler's trace shows), at most

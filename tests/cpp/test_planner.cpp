@@ -746,7 +746,7 @@ static void testSoftmaxBecomesOneRowProgram()
             std::vector<uint64_t> args;
             const void* in[1] = {nullptr}; void* out[1] = {nullptr};
             gen::packRowArgsInto(args, d, in, out);
-            CHECK(args.size() == 1 + 1 + d.scalarData.size() / aix::Device::dataTypeSize(dt) + 2);
+            CHECK(args.size() == 1 + 1 + d.scalarData.size() / aix::Device::dataTypeSize(dt) + 1 + 2);      // in, out, immediates, the input's period, rows, length
         }
     }
     // the per-row results stay visible when somebody still holds them: they are stored by the same kernel
@@ -1037,24 +1037,56 @@ static void testRowProgramTakesInAPlainKernel()
     CHECK(sawMask);
     CHECK(d.outputBuffers.size() == 2);                         // m and y; the converted mask is never stored
     CHECK(compilesRow(d));
-    // a plain kernel with a triangle stays apart (its index arithmetic is not available row by row)
+    // attention's forward pass in one kernel: tril(s) * scale + mask, then the softmax of the rows -- the triangle's rows
+    // are the program's rows, the [seq, seq] mask under [heads, seq, seq] scores is a block of rows that comes round again
     Capture cap2;
     FuseEngine f(config(), cap2.callbacks());
-    for (uintptr_t id : {1, 2, 3, 4, 5}) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
-    f.recordRowReduce(OpType::MaxTo, View(x), View(m), lowest, L);
-    f.recordTri(OpType::Tril, View(T(3, {rows, L})), View(c), 0);
-    f.record(OpType::Mul, View(c), View(mB), View(y));
+    const size_t heads = 3, seq = 64;
+    auto sc = T(11, {heads, seq, seq}), t1 = T(12, {heads, seq, seq}), t2 = T(13, {heads, seq, seq}), t3 = T(14, {heads, seq, seq});
+    auto half = T(15, {}), halfB = T(15, {heads, seq, seq}, DataType::kFloat32, {0, 0, 0});
+    auto msk = T(16, {seq, seq}), mskB = T(16, {heads, seq, seq}, DataType::kFloat32, {0, seq, 1});
+    auto mx = T(17, {heads, seq, 1}), mxB = T(17, {heads, seq, seq}, DataType::kFloat32, {seq, 1, 0}), out = T(18, {heads, seq, seq});
+    for (uintptr_t id = 11; id <= 18; ++id) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    const float h = 0.5f;
+    f.recordFill(&h, DataType::kFloat32, View(half));
+    f.recordTri(OpType::Tril, View(sc), View(t1), 0);
+    f.record(OpType::Mul, View(t1), View(halfB), View(t2));
+    f.record(OpType::Add, View(t2), View(mskB), View(t3));
+    f.recordRowReduce(OpType::MaxTo, View(t3), View(mx), lowest, seq);
+    f.record(OpType::Sub, View(t3), View(mxB), View(out));
+    for (uintptr_t id : {12, 13, 14, 15, 17}) f.releaseBuffer(reinterpret_cast<void*>(id * 0x10000));
     f.flush();
-    CHECK(cap2.fused.size() + cap2.singles.size() >= 2);
+    CHECK(cap2.fused.size() == 1 && cap2.singles.empty());
+    if (cap2.fused.size() == 1) {
+        const auto& k = cap2.fused[0];
+        CHECK(k.rowLength == seq && k.ops.size() == 5 && k.ops[0].type == OpType::Tril && k.inputBuffers.size() == 2 && k.outputBuffers.size() == 1);
+        CHECK(k.opParams.size() == 3 && k.opParams[0] == seq && k.opParams[1] == seq);
+        CHECK(rowOperandPeriod(k.inputBuffers[1], heads * seq, seq) == seq || rowOperandPeriod(k.inputBuffers[0], heads * seq, seq) == seq);
+        CHECK(compilesRow(k));
+        std::vector<uint64_t> args;
+        const void* in[2] = {nullptr, nullptr}; void* o1[1] = {nullptr};
+        gen::packRowArgsInto(args, k, in, o1);
+        CHECK(args.size() == 2 + 1 + k.scalarData.size() / 4 + 2 + 3 + 2);             // in, out, the immediates, two periods, the triangle, rows, length
+    }
+    // a triangle of matrices whose rows are not the program's rows stays a kernel of its own
+    Capture cap3;
+    FuseEngine g(config(), cap3.callbacks());
+    auto wide = T(21, {4, 8, 128}), wtri = T(22, {4, 8, 128}), wm = T(23, {4 * 8 * 2, 1}), wflat = T(22, {4 * 8 * 2, 64});
+    for (uintptr_t id : {21, 22, 23}) g.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    g.recordTri(OpType::Triu, View(wide), View(wtri), 0);
+    g.recordRowReduce(OpType::MaxTo, View(wflat), View(wm), lowest, 64);                 // rows of 64 over matrices of 128 columns
+    g.flush();
+    CHECK(cap3.fused.size() + cap3.singles.size() == 2);
 }
 
 static void testEqualKernelsLeaveSideBySide()
 {
-    // head after head, three kernels each: b = tril(a)^2, y = b - max(b) row by row (a triangle cannot be part of a row
-    // program), c = triu(y)^2.  The planner closes a kernel when the next one reads its result, so its list goes
-    // A0 B0 A1 B1 ... and the C's last; with groupEqualKernels the A's leave side by side, then the B's, then the C's,
-    // and a kernel that depends on another never overtakes it, also through a buffer written twice.
-    auto run = [&](bool group, std::vector<FusedSubgraphDescriptor>* fused, std::vector<OpRecord>* singles) {
+    // head after head: b = a * t (t a transposed view: no operand of a row program, so the product is a kernel of its
+    // own), then y = b - max(b) row by row, then c = -y * t.  The planner closes a kernel when the next one reads its
+    // result, so in its list the products alternate with the row programs; with groupEqualKernels the four products
+    // leave side by side, and a kernel that depends on another never overtakes it, also through a buffer written twice.
+    struct Step { std::vector<const void*> reads, writes; };
+    auto run = [&](bool group) {
         Capture cap;
         FuseConfig c = config();
         c.groupEqualKernels = group;
@@ -1064,55 +1096,75 @@ static void testEqualKernelsLeaveSideBySide()
         auto P = [](uintptr_t id) { return reinterpret_cast<void*>(id * 0x10000); };
         for (uintptr_t k = 0; k < 4; ++k) {
             const uintptr_t id = 10 * (k + 1);
-            auto a = T(id + 1, {8, 256}), t = T(id + 2, {8, 256}), b = T(id + 3, {8, 256}), m = T(id + 4, {8, 1}), y = T(id + 5, {8, 256});
+            auto a = T(id + 1, {8, 256}), b = T(id + 3, {8, 256}), m = T(id + 4, {8, 1}), y = T(id + 5, {8, 256});
             auto u = T(id + 6, {8, 256}), c2 = T(id + 7, {8, 256});
+            auto t = T(id + 2, {8, 256}, DataType::kFloat32, {1, 8});
             auto mB = T(id + 4, {8, 256}, DataType::kFloat32, {1, 0});
             for (uintptr_t j = 1; j <= 7; ++j) e.retainBuffer(P(id + j));
-            e.recordTri(OpType::Tril, View(a), View(t), 0);
-            e.record(OpType::Mul, View(t), View(t), View(b));
-            e.releaseBuffer(P(id + 2));
+            e.record(OpType::Mul, View(a), View(t), View(b));
             e.recordRowReduce(OpType::MaxTo, View(b), View(m), lowest, 256);
             e.record(OpType::Sub, View(b), View(mB), View(y));
             e.releaseBuffer(P(id + 4));
-            e.recordTri(OpType::Triu, View(y), View(u), 0);
-            e.record(OpType::Mul, View(u), View(u), View(c2));
+            e.record(OpType::Negate, View(y), View(u));
+            e.record(OpType::Mul, View(u), View(t), View(c2));
             e.releaseBuffer(P(id + 6));
         }
-        // one buffer written by two kernels in turn: z = exp(a_0) (alive) is read by a row program, then z = sqrt(a_1)
-        auto a0 = T(11, {8, 256}), a1 = T(21, {8, 256}), z = T(90, {8, 256}), mz = T(91, {8, 1});
-        for (uintptr_t id : {90, 91}) e.retainBuffer(P(id));
-        e.recordTri(OpType::Tril, View(a0), View(z), 3);
+        // one buffer written by two kernels in turn: z = p * q is read by a row reduction, then z = r * s
+        auto p0 = T(81, {8, 256}), r0 = T(83, {8, 256}), z = T(90, {8, 256}), mz = T(91, {8, 1});
+        auto q0 = T(82, {8, 256}, DataType::kFloat32, {1, 8}), s0 = T(84, {8, 256}, DataType::kFloat32, {1, 8});
+        for (uintptr_t id : {81, 82, 83, 84, 90, 91}) e.retainBuffer(P(id));
+        e.record(OpType::Mul, View(p0), View(q0), View(z));
         e.recordRowReduce(OpType::MaxTo, View(z), View(mz), lowest, 256);
-        e.recordTri(OpType::Tril, View(a1), View(z), 4);
+        e.record(OpType::Mul, View(r0), View(s0), View(z));
         e.flush();
-        *fused = cap.fused; *singles = cap.singles;
         if (std::getenv("AIX_TEST_VERBOSE")) for (auto& o : cap.order) std::printf("  %s %s\n", group ? "grouped" : "plain  ", o.c_str());
-    };
-    std::vector<FusedSubgraphDescriptor> fa, fb;
-    std::vector<OpRecord> sa, sb;
-    run(false, &fa, &sa);
-    run(true, &fb, &sb);
-    CHECK(fa.size() == 12 && fb.size() == 12 && sa.size() == 3 && sb.size() == 3);
-    if (fa.size() != 12 || fb.size() != 12 || sb.size() != 3) return;
-    auto kindOf = [](const FusedSubgraphDescriptor& d) { return d.ops[0].type == OpType::Tril ? 'A' : d.ops[0].type == OpType::Triu ? 'C' : 'B'; };
-    std::string plain, grouped;
-    for (const auto& d : fa) plain += kindOf(d);
-    for (const auto& d : fb) grouped += kindOf(d);
-    CHECK(plain == "ABABABABCCCC");
-    CHECK(grouped == "AAAABBBBCCCC");
-    // each head's three kernels in order (B reads A's output, C reads B's)
-    for (uintptr_t k = 0; k < 4; ++k) {
-        const void* b = reinterpret_cast<const void*>((10 * (k + 1) + 3) * 0x10000);
-        const void* y = reinterpret_cast<const void*>((10 * (k + 1) + 5) * 0x10000);
-        size_t ia = SIZE_MAX, ib = SIZE_MAX, ic = SIZE_MAX;
-        for (size_t j = 0; j < fb.size(); ++j) {
-            for (const auto& o : fb[j].outputBuffers) { if (o.data == b) ia = j; if (o.data == y) ib = j; }
-            for (const auto& in : fb[j].inputBuffers) if (in.data == y && kindOf(fb[j]) == 'C') ic = j;
+        // what left, in the order it left: reads and writes of every kernel and single operator
+        std::vector<Step> steps;
+        size_t single = 0;
+        for (const auto& o : cap.order) {
+            Step st;
+            if (o[0] == 'F') {
+                const auto& d = cap.fused[std::stoul(o.substr(1))];
+                for (const auto& in : d.inputBuffers) st.reads.push_back(in.data);
+                for (const auto& out : d.outputBuffers) st.writes.push_back(out.data);
+            } else {
+                const auto& op = cap.singles[single++];
+                st.reads.push_back(op.input0.data);
+                if (op.hasInput1) st.reads.push_back(op.input1.data);
+                st.writes.push_back(op.output.data);
+            }
+            steps.push_back(st);
         }
-        CHECK(ia < ib && ib < ic && ic != SIZE_MAX);
+        return steps;
+    };
+    const auto plain = run(false), grouped = run(true);
+    CHECK(plain.size() == grouped.size() && plain.size() >= 11);
+    auto buf = [](uintptr_t id) { return reinterpret_cast<const void*>(id * 0x10000); };
+    auto has = [](const std::vector<const void*>& v, const void* p) { return std::find(v.begin(), v.end(), p) != v.end(); };
+    auto writer = [&](const std::vector<Step>& s, const void* p, size_t nth) { for (size_t k = 0; k < s.size(); ++k) if (has(s[k].writes, p) && nth-- == 0) return k; return (size_t)SIZE_MAX; };
+    auto reader = [&](const std::vector<Step>& s, const void* p) { for (size_t k = 0; k < s.size(); ++k) if (has(s[k].reads, p)) return k; return (size_t)SIZE_MAX; };
+    // the same work either way: every buffer is written equally often
+    for (uintptr_t id : {13, 15, 17, 23, 25, 27, 33, 35, 37, 43, 45, 47, 90, 91}) {
+        size_t n1 = 0, n2 = 0;
+        for (const auto& st : plain) n1 += has(st.writes, buf(id));
+        for (const auto& st : grouped) n2 += has(st.writes, buf(id));
+        CHECK(n1 == n2 && n1 >= 1);
     }
-    // the two writers of z and the reader between them (single operators) keep their order
-    CHECK(sb[0].type == OpType::Tril && sb[0].triDiagonal == 3 && sb[1].type == OpType::MaxTo && sb[2].type == OpType::Tril && sb[2].triDiagonal == 4);
+    // plain: something between the products of two heads; grouped: the four products are consecutive
+    CHECK(writer(plain, buf(23), 0) > writer(plain, buf(13), 0) + 1);
+    size_t first = SIZE_MAX, last = 0;
+    for (uintptr_t k = 1; k <= 4; ++k) { const size_t w = writer(grouped, buf(10 * k + 3), 0); first = std::min(first, w); last = std::max(last, w); }
+    CHECK(first != SIZE_MAX && last - first == 3);
+    // in both orders: a product before the kernel that reads it, y before its reader, the two writers of z around its reader
+    for (const auto* s : {&plain, &grouped}) {
+        for (uintptr_t k = 1; k <= 4; ++k) {
+            CHECK(writer(*s, buf(10 * k + 3), 0) < reader(*s, buf(10 * k + 3)));
+            CHECK(writer(*s, buf(10 * k + 7), 0) != SIZE_MAX);
+        }
+        const size_t w1 = writer(*s, buf(90), 0), rd = reader(*s, buf(90)), w2 = writer(*s, buf(90), 1);
+        CHECK(w1 < rd && rd < w2 && w2 != SIZE_MAX);
+        CHECK(has((*s)[w1].reads, buf(81)) && has((*s)[w2].reads, buf(83)));
+    }
 }
 
 int main(int argc, char** argv)

@@ -414,3 +414,68 @@ def test_random_programs_with_row_reductions(dev, dtype):
             T.assert_same_bits(g1, want, "fused vs oracle " + what)
             T.assert_same_bits(g2, want, "unfused vs oracle " + what)
     set_fusion(dev, True)
+
+
+# ---- triangles and blocks of rows inside a row program -------------------------------------------------------------
+def _tri(f, name, x, shape, diagonal):
+    r = f.result(shape)
+    assert getattr(CPU, name)(C.byref(x["host"].desc()), C.byref(r["host"].desc()), diagonal) == 0
+    f.dev.dev.call(name, H.ref(x["desc"]), H.ref(r["desc"]), diagonal)
+    return r
+
+
+def _block(f, node, shape, block_dims):
+    """A dense block (the last `block_dims` dims of `shape`) under leading dims of stride 0: the [seq, seq] mask of
+    attention under [batch, heads, seq, seq] scores."""
+    strides = [0] * (len(shape) - block_dims) + O.row_major(shape[-block_dims:])
+    view = T.HostTensor(node["host"].storage, f.dtype, shape, strides)
+    return {"host": view, "ptr": node["ptr"], "desc": H.kdesc(view, node["ptr"])}
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.F16], ids=lambda d: NAMES[d])
+def test_attention_scores_to_probabilities_is_one_kernel(dev, dtype):
+    """softmax(tril(s) * scale + mask) over [batch, heads, seq, seq] scores with a [seq, seq] additive mask
+    (frontend/transformer.hpp; aixNeuralNetwork.hpp:188-192 for the softmax): the triangle's rows are the rows the
+    program works on and the mask is a block of rows that every seq rows see again, so the eight operators are ONE
+    kernel.  Fused = stand-alone kernels bit for bit; both against the oracle's operator chain and float64."""
+    for k, (shape, diagonal) in enumerate([([2, 3, 64, 64], 0), ([1, 2, 128, 128], 0), ([3, 32, 256], -1), ([2, 40, 96], 2)]):
+        seq = shape[-1]
+
+        def build(f, x, rng, shape=shape, diagonal=diagonal, seq=seq):
+            mask_host = T.contiguous_tensor(rng, dtype, shape[-2:], lo=-1.0, hi=0.0)
+            upper = np.triu(np.ones(shape[-2:], bool), 1 + diagonal).reshape(-1)
+            mask_host.storage[upper] = O.to_storage(np.full(int(upper.sum()), -30000.0), dtype)
+            mask = f.leaf(mask_host)
+            t = _tri(f, "tril", x, shape, diagonal)
+            scaled = f.binary(O.MUL, t, f.over_all(f.scalar(0.125), shape), shape)
+            return softmax(f, f.binary(O.ADD, scaled, _block(f, mask, shape, 2), shape), shape)
+
+        def exact(x, m, diagonal=diagonal, shape=shape):
+            keep = np.tril(np.ones(shape[-2:]), diagonal)
+            return np_softmax(x * keep * 0.125 + m.reshape(shape[-2:]))
+
+        got = run_both(dev, dtype, shape, build, 900 + k, expect_fused_ops=8, exact=exact)
+        rows = O.to_float64(got, dtype).reshape(-1, seq).sum(axis=1)
+        assert np.all(np.abs(rows - 1.0) <= (4e-2 if dtype in (O.F16, O.BF16) else 1e-5)), shape
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32], ids=lambda d: NAMES[d])
+def test_triangle_after_a_row_sum_stays_in_the_kernel(dev, dtype):
+    """The gradient side: y = triu / tril of (x - rowsum(x) * x) * scale -- a per-row value, two products and a triangle
+    in one row program, for matrices stacked under leading dims."""
+    for k, (shape, name, diagonal) in enumerate([([4, 64, 64], "tril", 0), ([2, 2, 32, 128], "triu", 1), ([96, 512], "tril", -3)]):
+        def build(f, x, rng, shape=shape, name=name, diagonal=diagonal, k=k):
+            # the factor: a fill of this window (an immediate of the kernel) or a scalar tensor that lies in memory (the
+            # scale of attention, made in the forward pass, when the backward pass uses it): one element seen from
+            # everywhere.  (Uploaded first: an upload flushes the window.)
+            stored = f.leaf(T.HostTensor(O.to_storage(np.array([0.5]), dtype), dtype, [])) if k == 1 else None
+            s = f.row_sum(x, shape)
+            d = f.binary(O.SUB, x, f.binary(O.MUL, x, f.over_rows(s, shape), shape), shape)
+            half = stored if stored is not None else f.scalar(0.5)
+            return _tri(f, name, f.binary(O.MUL, d, f.over_all(half, shape), shape), shape, diagonal)
+
+        def exact(x, *more, shape=shape, name=name, diagonal=diagonal):
+            keep = (np.tril if name == "tril" else np.triu)(np.ones(shape[-2:]), diagonal)
+            return (x - x * x.sum(axis=-1, keepdims=True)) * 0.5 * keep
+
+        run_both(dev, dtype, shape, build, 950 + k, expect_fused_ops=5, lo=-0.5, hi=0.5, exact=exact, tol16=4e-2)
