@@ -805,7 +805,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     bool noAlias = true;                                     // in-place updates: an output that is also an input
     for (const auto& ob : d.outputBuffers) for (const auto& ib : d.inputBuffers) if (ob.data == ib.data) noAlias = false;
     size_t storedBytes = 0;                                  // large results leave through non-temporal stores
-    for (const auto& ob : d.outputBuffers) storedBytes += n * dataTypeSize(ob.dtype);
+    for (const auto& ob : d.outputBuffers) if (ob.size > 1 || n == 1) storedBytes += n * dataTypeSize(ob.dtype);      // (a sum over everything stores next to nothing)
     const bool streamOut = storedBytes >= ex.streamStoreMinBytes;
     gen::signatureInto(ex.key, d, shape, bmask, noAlias, streamOut);
     aixk_module* mod = nullptr;
@@ -819,7 +819,6 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         ++ex.misses;
     }
 
-    gen::packArgsInto(ex.args, d, shape, inPtr, outPtr, n, shape == gen::Shape::Flat ? nullptr : &space, chunks);
     uint64_t items, perBlock, cap;
     if (shape == gen::Shape::Flat) { items = n / VEC + 1; perBlock = gen::kBlock; cap = 1u << 22; }
     else if (shape == gen::Shape::Rows) { items = n / VEC; perBlock = gen::kBlock; cap = (uint64_t)m_cus * 64; }
@@ -827,13 +826,37 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     uint64_t grid = (items + perBlock - 1) / perBlock;
     grid = std::max<uint64_t>(1, std::min(grid, cap));
 
+    // Sums over everything (FuseEngine::recordWholeSum): the kernel leaves one partial sum per workgroup in scratch
+    // memory -- its "output" pointer -- and aixk_sum_partials lands their sum in the destination afterwards.
+    struct Whole { size_t output; void* scratch; uint64_t init; };
+    Whole wholes[8];
+    size_t nWholes = 0;
+    for (const auto& op : d.ops) {
+        if (!op.whole || op.outputIndex == SIZE_MAX) continue;
+        if (nWholes == 8) throw std::logic_error("DeviceHIP: more sums over everything in one kernel than the planner allows");
+        const size_t wide = d.dtype == DataType::kFloat64 ? 8 : 4;
+        void* scratch = allocateBlock(grid * wide, false);
+        m_limbo.emplace_back(scratch, bucketBytes(grid * wide));     // recycled once the work enqueued below has passed
+        m_limboBytes += bucketBytes(grid * wide);
+        uint64_t init = 0;
+        std::memcpy(&init, d.scalarData.data() + op.scalarIndex1 * esz, esz);
+        wholes[nWholes++] = Whole{op.outputIndex, scratch, init};
+        outPtr[op.outputIndex] = scratch;
+    }
+    gen::packArgsInto(ex.args, d, shape, inPtr, outPtr, n, shape == gen::Shape::Flat ? nullptr : &space, chunks);
+
     AIXHIP_TRACE("%s  %llu elements, %zu in %zu out", gen::entryName(d, shape).c_str(), (unsigned long long)n, NI, NO);
-    if (ex.batchFlatKernels) {
+    if (ex.batchFlatKernels && nWholes == 0) {
         joinBatch(d, mod, gen::entryName(d, shape), grid, [&] { return gen::source(d, shape, bmask, noAlias, streamOut, true); });
         return;
     }
     issueFlatBatch();
     check(aixk_rtc_launch(m_ctx, mod, (uint32_t)grid, gen::kBlock, ex.args.data(), ex.args.size() * sizeof(uint64_t)));
+    for (size_t k = 0; k < nWholes; ++k) {
+        aixhip_tensor dst;
+        toPod(d.outputBuffers[wholes[k].output], &dst);
+        check(aixk_sum_partials(m_ctx, wholes[k].scratch, grid, &dst, wholes[k].init));
+    }
 }
 
 // The kernel whose signature is in Extras::key and whose argument block is in Extras::args joins the kernels waiting to
@@ -1182,6 +1205,18 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
     if (folded && recordRowReduction(OpType::ReduceTo, src, dst, init)) return;
+    // The sum of ALL elements of a tensor that a recorded operator is about to produce -- the gradient of a scalar
+    // constant is the sum of a product formed for nothing else (aixCore.hpp:2384-2438, 2030-2036) -- is recorded too: the
+    // planner lets it join the kernel that holds the product in registers, which then adds it up instead of storing it.
+    if (folded && dst.size == 1 && src.size > 1 && src.isContiguous && m_extras->fuseRowReductions && m_engine->config().elementwiseFusion &&
+        (src.dtype == DataType::kFloat32 || src.dtype == DataType::kFloat16 || src.dtype == DataType::kBFloat16 || src.dtype == DataType::kFloat64) &&
+        src.shape.size() <= AIXK_MAX_RANK && dst.shape.size() <= AIXK_MAX_RANK && findBlock(src.data) && findBlock(dst.data) && m_engine->pendingWrites(src.data)) {
+        View in(src), out(dst);
+        if (in.dense) {
+            m_engine->recordWholeSum(in, out, &init);
+            return;
+        }
+    }
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
     check(folded ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &ps, &pd, init) : aixk_reduce_to(m_ctx, AIXK_SUM, &ps, &pd));

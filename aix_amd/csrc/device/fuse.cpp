@@ -368,6 +368,7 @@ public:
             if (op.type == OpType::Fill || op.type == OpType::FillMin) placeFill(i);
             else if (isElementwiseOp(op.type) && m_cfg.elementwiseFusion) placeOp(i);
             else if (isRowReduce(op.type) && op.rowLength && m_cfg.elementwiseFusion && m_cfg.supportsStridedFusion) placeReduce(i);
+            else if (op.whole && m_cfg.elementwiseFusion) placeWhole(i);
             else placeSingle(i);
         }
         for (size_t g = 0; g < m_groupCount; ++g) closeGroup(g);
@@ -441,6 +442,7 @@ public:
                 else if (operand.kind == Operand::kScalar) *sc[k] = scalarIndex(operand.index);
             }
             o.perRow = m_perRow[w] != 0;
+            o.whole = op.whole;
             if (isRowReduce(op.type)) {
                 // the value the destination was initialised with (already in the group's element type) as an immediate
                 o.scalarIndex1 = d.scalarData.size() / esz;
@@ -703,6 +705,45 @@ private:
         g.ops.push_back(i);
         m_groupOf[i] = target;
         m_perRow[i] = 1;
+    }
+
+    // ---- the sum of everything ------------------------------------------------------------------
+    // Joins the plain kernel that holds its operand in registers (every element once, whatever the launch shape), else
+    // it is a single operator.  Nothing in the kernel can use its result, and no row program takes it (its one-element
+    // destination is no row operand), so the kernel goes on growing around it.
+    void placeWhole(size_t i)
+    {
+        const auto& op = at(i);
+        const View& in = op.input0;
+        for (;;) {
+            size_t target = SIZE_MAX, def = SIZE_MAX;
+            bool closedSomething = false;
+            if (findFill(in.data)) { placeSingle(i); return; }
+            for (size_t g = 0; g < m_groupCount; ++g) {
+                if (!m_groups[g].open) continue;
+                const size_t d = findDef(m_groups[g], in.data);
+                if (d == SIZE_MAX) continue;
+                const Group& grp = m_groups[g];
+                size_t wholes = 0;
+                for (size_t w : grp.ops) wholes += at(w).whole;
+                const bool usable = target == SIZE_MAX && !grp.rowLen && !m_perRow[d] && !at(d).whole && at(d).type != OpType::Cast && sameElements(defView(d), in) &&
+                                    grp.dtype == in.dtype && grp.count == in.size && wholes < 8 &&
+                                    grp.loads.size() + grp.defs.size() + 2 <= m_cfg.maxBufferSlots;
+                if (usable) { target = g; def = d; }
+                else { closeGroup(g); closedSomething = true; }
+            }
+            if (closedSomething) continue;
+            if (target == SIZE_MAX) { placeSingle(i); return; }
+            if (closeGroupsTouching(op.output.data, SIZE_MAX, nullptr)) continue;      // (may have closed the target: look again)
+            if (findFill(op.output.data)) eraseFill(op.output.data);                   // the sum defines its destination
+            Group& g = m_groups[target];
+            m_operands[i][0] = Operand{Operand::kValue, def};
+            g.defs.push_back(i);
+            g.ops.push_back(i);
+            g.hasScalar = true;                                                        // (the destination's initial value)
+            m_groupOf[i] = target;
+            return;
+        }
     }
 
     // Can the group work on rows of `length` elements?  It does already, or everything it loads and stores fits rows.
@@ -1035,6 +1076,18 @@ void FuseEngine::recordRowReduce(OpType type, const View& input, const View& out
     wake(input.data); wake(output.data);
     OpRecord& r = append(type);
     r.input0 = input; r.output = output; r.rowLength = rowLength;
+    r.scalarDType = output.dtype;
+    std::memcpy(r.scalarData.data(), init, aix::Device::dataTypeSize(output.dtype));
+    maybeFlush();
+}
+
+void FuseEngine::recordWholeSum(const View& input, const View& output, const void* init)
+{
+    if (output.size != 1 || input.dtype != output.dtype || !input.dense)
+        throw std::invalid_argument("recordWholeSum: the sum of a dense operand into one element of its type");
+    wake(input.data); wake(output.data);
+    OpRecord& r = append(OpType::ReduceTo);
+    r.input0 = input; r.output = output; r.rowLength = 0; r.whole = true;
     r.scalarDType = output.dtype;
     std::memcpy(r.scalarData.data(), init, aix::Device::dataTypeSize(output.dtype));
     maybeFlush();

@@ -104,6 +104,8 @@ struct OpRecord {
     // ReduceTo / MaxTo recorded as a row reduction: elements per row of input0 (its last dimension); scalarData then holds
     // the value the destination was initialised with, in the destination's element type (the folded fill)
     size_t rowLength{0};
+    // ReduceTo recorded as the sum of ALL elements of input0 into a one-element output (rowLength 0); scalarData as above
+    bool whole{false};
     // Fill / FillMin: the fill has waited outside the window and was brought back because somebody names its buffer: it
     // runs with the window it is in now
     bool hasWaited{false};
@@ -132,6 +134,8 @@ struct FusedSubgraphDescriptor {
         size_t scalarIndex1 = SIZE_MAX;
         size_t paramIndex   = SIZE_MAX;    // Tril / Triu: its (rows, cols, diagonal) triple in opParams
         bool   perRow       = false;       // row programs: the operator yields one value per row (a reduction, or arithmetic on such values)
+        bool   whole        = false;       // ReduceTo: the sum of the operand over ALL elements of the kernel (plus the immediate scalarIndex1) into
+                                           // the one-element output; the kernel hands over one partial sum per workgroup, its caller adds them up
     };
     std::vector<Op> ops;
     std::vector<uint64_t> opParams;        // run-time integers of index-dependent operators, three per Tril / Triu
@@ -215,6 +219,11 @@ public:
     // ReduceTo / MaxTo over the last dimension (`rowLength` elements, dense) of `input` into the dense `output`, whose
     // pending initialisation the caller has taken out of the window: `init` is that value in output's element type.
     void recordRowReduce(OpType type, const View& input, const View& output, const void* init, size_t rowLength);
+    // The sum of all elements of the dense `input` into the one-element `output`, whose pending initialisation the caller
+    // has taken out of the window (`init`, in output's element type).  It joins the kernel that holds its operand in
+    // registers -- the product that is only formed to be summed is then never stored -- and is replayed as a plain
+    // reduction when there is no such kernel.
+    void recordWholeSum(const View& input, const View& output, const void* init);
     // Plans and emits the window.  A fill (fill / fillMin of a whole dense buffer that allocate() handed out) that no
     // other operator of the window touches, and that nobody outside is about to read, is not emitted unless `final`:
     // it waits, outside the window, until an operator naming its buffer is recorded (it then rejoins the window ahead

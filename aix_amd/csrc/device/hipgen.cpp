@@ -107,7 +107,7 @@ void emitBody(std::ostringstream& o, const FusedSubgraphDescriptor& d)
     else o << "__device__ __forceinline__ void aix_body(const T* x, const T* s, T* out)\n{\n";
     for (size_t k = 0; k < d.ops.size(); ++k) {
         const auto& op = d.ops[k];
-        if (op.type == OpType::Cast) o << "    const T v" << k << " = " << operandText(d, op.inputIndex0, op.scalarIndex0) << ";\n";
+        if (op.type == OpType::Cast || op.whole) o << "    const T v" << k << " = " << operandText(d, op.inputIndex0, op.scalarIndex0) << ";\n";   // (a sum of everything: the loops add this value up)
         else if (isTri(op.type))
             o << "    const T v" << k << " = tri_keeps(tpos[" << op.paramIndex << "], e, tp[" << 3 * op.paramIndex << "], tp[" << 3 * op.paramIndex + 1 << "], (i64)tp["
               << 3 * op.paramIndex + 2 << "], " << (op.type == OpType::Triu ? 1 : 0) << ") ? " << operandText(d, op.inputIndex0, op.scalarIndex0) << " : zero<T>();\n";
@@ -162,7 +162,7 @@ void signatureInto(std::string& s, const FusedSubgraphDescriptor& d, Shape shape
     for (size_t k = 0; k < d.outputBuffers.size(); ++k)
         if (d.outputBuffers[k].dtype != d.dtype) { s += "|y"; appendNumber(s, k); s += ':'; s += shortType(d.outputBuffers[k].dtype); }
     for (const auto& op : d.ops) {
-        s += '|'; s += fuse::opName(op.type); s += '(';
+        s += '|'; s += fuse::opName(op.type); if (op.whole) s += '!'; s += '(';
         appendOperand(s, d, op.inputIndex0, op.scalarIndex0);
         if (isBinary(op.type)) { s += ','; appendOperand(s, d, op.inputIndex1, op.scalarIndex1); }
         s += ')';
@@ -196,6 +196,20 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     for (size_t k = 0; k < NI; ++k) o << "typedef " << typeName(d.inputBuffers[k].dtype) << " I" << k << ";\n";
     for (size_t k = 0; k < NO; ++k) o << "typedef " << typeName(d.outputBuffers[k].dtype) << " O" << k << ";\n";
     o << "\n";
+    // outputs that are sums over everything: the loops add their value up per lane instead of storing it, the workgroup's
+    // total goes to slot BID of the buffer the output pointer names (partial sums in the wide type, one per workgroup)
+    std::vector<char> whole(NO, 0);
+    bool anyWhole = false;
+    for (const auto& op : d.ops) if (op.whole && op.outputIndex != SIZE_MAX) { whole[op.outputIndex] = 1; anyWhole = true; }
+    if (anyWhole) o << "typedef traits<T>::W W;\n";
+    auto wholeInit = [&](std::ostringstream& os) { for (size_t k = 0; k < NO; ++k) if (whole[k]) os << "    W acc" << k << " = (W)0;\n"; };
+    auto wholeAdd = [&](std::ostringstream& os, const char* indent) { for (size_t k = 0; k < NO; ++k) if (whole[k]) os << indent << "acc" << k << " += up(y[" << k << "]);\n"; };
+    auto wholeLand = [&](std::ostringstream& os) {
+        if (!anyWhole) return;
+        os << "    __shared__ W red[4];\n";
+        for (size_t k = 0; k < NO; ++k)
+            if (whole[k]) os << "    { const W t = row_sum<256>(acc" << k << ", red); if (threadIdx.x == 0) global_ptr<W>((u64)a.out[" << k << "])[BID] = t; }\n";
+    };
     auto in_same = [&](size_t k) { return d.inputBuffers[k].dtype == d.dtype; };
     auto out_same = [&](size_t k) { return d.outputBuffers[k].dtype == d.dtype; };
     auto to_t = [&](size_t k, const std::string& e) { return in_same(k) ? e : "convert<I" + std::to_string(k) + ", T>(" + e + ")"; };
@@ -236,6 +250,7 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
             else o << "    const vec<I" << k << ", VEC>*" << rs << " p" << k << " = (const vec<I" << k << ", VEC>*)in" << k << ";\n";
         }
         for (size_t k = 0; k < NO; ++k) o << "    vec<O" << k << ", VEC>*" << rs << " q" << k << " = (vec<O" << k << ", VEC>*)out" << k << ";\n";
+        wholeInit(o);
         o << "    const u64 nvec = a.n / VEC;\n"
           << "    for (u64 v = (u64)BID * " << kBlock << " + threadIdx.x; v < nvec; v += (u64)GDIM * " << kBlock << ") {\n";
         for (size_t k = 0; k < NI; ++k) if (!bc(k)) o << "        const vec<I" << k << ", VEC> r" << k << " = p" << k << "[v];\n";
@@ -248,9 +263,10 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         }
         if (NI == 0) o << "            x[0] = zero<T>();\n";
         o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
-        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+        for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+        wholeAdd(o, "            ");
         o << "        }\n";
-        for (size_t k = 0; k < NO; ++k) o << "        store_sel<AIX_NT>(q" << k << " + v, w" << k << ");\n";
+        for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "        store_sel<AIX_NT>(q" << k << " + v, w" << k << ");\n";
         o << "    }\n"
           << "    const u64 done = nvec * VEC;\n"
           << "    if (BID == 0 && done + threadIdx.x < a.n) {\n        const u64 i = done + threadIdx.x;\n        T x[" << AI << "], y[" << NO << "];\n";
@@ -261,12 +277,16 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         }
         if (NI == 0) o << "        x[0] = zero<T>();\n";
         o << "        aix_body(x, s, y" << (NT ? ", 0, tpos, a.tp" : "") << ");\n";
-        for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
-        o << "    }\n}\n";
+        for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+        wholeAdd(o, "        ");
+        o << "    }\n";
+        wholeLand(o);
+        o << "}\n";
         return o.str();
     }
 
     if (shape == Shape::Rows) {
+        wholeInit(o);
         o << "    const int inner = (int)a.rank - 1;\n"
           << "    const u64 total = a.n / VEC;\n"
           << "    for (u64 c = (u64)BID * " << kBlock << " + threadIdx.x; c < total; c += (u64)GDIM * " << kBlock << ") {\n"
@@ -287,14 +307,18 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
         for (size_t k = 0; k < NI; ++k) o << "            x[" << k << "] = " << to_t(k, "r" + std::to_string(k) + ".v[e]") << ";\n";
         if (NI == 0) o << "            x[0] = zero<T>();\n";
         o << "            aix_body(x, s, y" << (NT ? ", e, tpos, a.tp" : "") << ");\n";
-        for (size_t k = 0; k < NO; ++k) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+        for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "            w" << k << ".v[e] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+        wholeAdd(o, "            ");
         o << "        }\n";
-        for (size_t k = 0; k < NO; ++k) o << "        store_sel<AIX_NT>((vec<O" << k << ", VEC>*)(out" << k << " + c * VEC), w" << k << ");\n";
-        o << "    }\n}\n";
+        for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "        store_sel<AIX_NT>((vec<O" << k << ", VEC>*)(out" << k << " + c * VEC), w" << k << ");\n";
+        o << "    }\n";
+        wholeLand(o);
+        o << "}\n";
         return o.str();
     }
 
     // gather
+    wholeInit(o);
     o << "    for (u64 i = (u64)BID * " << kBlock << " + threadIdx.x; i < a.n; i += (u64)GDIM * " << kBlock << ") {\n"
       << "        u64 rest = i;\n        u64 p[" << AI << "];\n";
     if (NT) { o << "        TriPos tpos[" << NT << "];\n"; for (size_t j = 0; j < NT; ++j) o << "        tpos[" << j << "] = tri_origin(i, a.tp[" << 3 * j << "], a.tp[" << 3 * j + 1 << "]);\n"; }
@@ -305,8 +329,11 @@ std::string source(const FusedSubgraphDescriptor& d, Shape shape, uint32_t broad
     for (size_t k = 0; k < NI; ++k) o << "        x[" << k << "] = " << to_t(k, "in" + std::to_string(k) + "[p[" + std::to_string(k) + "]]") << ";\n";
     if (NI == 0) o << "        x[0] = zero<T>();\n";
     o << "        aix_body(x, s, y" << (NT ? ", 0, tpos, a.tp" : "") << ");\n";
-    for (size_t k = 0; k < NO; ++k) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
-    o << "    }\n}\n";
+    for (size_t k = 0; k < NO; ++k) if (!whole[k]) o << "        out" << k << "[i] = " << from_t(k, "y[" + std::to_string(k) + "]") << ";\n";
+    wholeAdd(o, "        ");
+    o << "    }\n";
+    wholeLand(o);
+    o << "}\n";
     return o.str();
 }
 

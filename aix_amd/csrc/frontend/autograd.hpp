@@ -187,8 +187,8 @@ public:
     }
 
     // Single-pass differentiation: nodes are visited youngest first -- the reverse of the order the program created
-    // them in, which is a reverse topological order (with the nodes that feed only leaves, and the leaves, moved to the
-    // end) -- and each one is differentiated ONCE with the sum of the seeds that reached it.  A program written stage by stage (all heads' score products, then all their softmaxes, ...) is
+    // them in, which is a reverse topological order -- and each one is differentiated ONCE with the sum of the seeds
+    // that reached it.  A program written stage by stage (all heads' score products, then all their softmaxes, ...) is
     // differentiated stage by stage too, so a device that batches runs of equal calls finds the same runs in the
     // backward pass.  The reference has no such mode (its recursion revisits a node once per path, which is
     // exponential in the number of residual branches of a transformer); the backward formulas are the same ones,
@@ -201,18 +201,11 @@ public:
         for (size_t k = 0; k < order.size(); ++k)     // everything the result depends on
             for (const auto& in : order[k]->inputs)
                 if (seen.insert(in.get()).second) order.push_back(in.get());
-        // Last of all the leaves (nothing depends on them), and before them the nodes that feed leaves only -- the
-        // broadcast of a scalar constant or of a parameter, whose backward is a reduction to the leaf's shape that
-        // nothing inside the pass waits for.  Issued where creation order puts them, between the elementwise operators
-        // of one backward formula (GeLU's has four such constants), these reductions cut the formula into several kernels.
-        auto tier = [](const Node* n) {
-            if (n->inputs.empty()) return 2;
-            for (const auto& in : n->inputs) if (!in->inputs.empty()) return 0;
-            return 1;
-        };
-        std::sort(order.begin(), order.end(), [&](const Node* a, const Node* b) {
-            const int ta = tier(a), tb = tier(b);
-            return ta != tb ? ta < tb : a->serial > b->serial;
+        // (the leaves last of all: nothing waits for them, and a scalar constant's "grad += seed", issued where the constant
+        // was created -- in the middle of a formula -- would make the kernel that forms the seed stop there)
+        std::sort(order.begin(), order.end(), [](const Node* a, const Node* b) {
+            const bool la = a->inputs.empty(), lb = b->inputs.empty();
+            return la != lb ? lb : a->serial > b->serial;
         });
         Node::accumulating() = true;
         try {

@@ -19,6 +19,8 @@
 
 #include "common.hpp"
 
+#include <type_traits>
+
 #include <algorithm>
 
 using namespace aixd;
@@ -251,6 +253,31 @@ __global__ __launch_bounds__(kBlock) void reduce_all_finish_k(const T* __restric
     }
     a = block_reduce<Op>(a, smem);
     if (threadIdx.x == 0) land(Op{}, fin, dst, 0, a, src[locate<1, IDX>(sp, 0, (IDX)0)], 0);
+}
+
+// The partial sums a generated kernel left behind (one per workgroup, in the wide type of T), folded in index order and
+// landed as reduceTo lands a sum: the value the destination was initialised with, widened, plus the sum, rounded once.
+template <class T>
+__global__ __launch_bounds__(kBlock) void sum_partials_k(const typename traits<T>::W* __restrict__ partials, unsigned count, T* dst, u64 init_bits)
+{
+    typedef SumOp<T> Op;
+    typedef typename Op::Acc Acc;
+    __shared__ Acc smem[kWaves];
+    Acc a = Op::init();
+    constexpr unsigned U = 8;
+    for (unsigned i0 = threadIdx.x; i0 < count; i0 += kBlock * U) {
+        Acc r[U];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < count) r[k] = partials[i0 + k * kBlock];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < count) a = Op::combine(a, r[k]);
+    }
+    a = block_reduce<Op>(a, smem);
+    if (threadIdx.x == 0) {
+        T init;
+        __builtin_memcpy(&init, &init_bits, sizeof(T));
+        *dst = down<T>(up(init) + a);
+    }
 }
 
 // ---- per-slot plans ------------------------------------------------------------------------------
@@ -1116,6 +1143,23 @@ int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, ui
         typedef decltype(tag) T;
         hipLaunchKernelGGL((argmax_onehot_inner_many_k<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const OnehotItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
         AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+int32_t aixk_sum_partials(aixk_ctx* ctx, const void* partials, uint64_t count, const aixhip_tensor* dst, uint64_t init_bits)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(valid_tensor(dst) && dst->data && dst->size == 1, "sum of partials: the result is one element");
+    AIXK_REQUIRE(partials && count > 0 && count < (1ull << 31), "sum of partials: no partials, or too many");
+    AIXK_REQUIRE(dst->dtype == AIXK_F64 || dst->dtype == AIXK_F32 || dst->dtype == AIXK_F16 || dst->dtype == AIXK_BF16, "sum of partials: floating-point results only");
+    return by_dtype(dst->dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        if constexpr (std::is_same<T, double>::value || std::is_same<T, float>::value || std::is_same<T, f16>::value || std::is_same<T, bf16>::value) {
+            hipLaunchKernelGGL((sum_partials_k<T>), dim3(1), dim3(kBlock), 0, ctx->stream, (const typename traits<T>::W*)partials, (unsigned)count,
+                               (T*)dst->data + dst->offset, (u64)init_bits);
+            AIXK_HIP(hipGetLastError());
+        }
         return (int)AIXK_OK;
     });
 }

@@ -77,6 +77,7 @@ _SIGNATURES = {
     "aixk_reduce_all_noalloc": [_P, C.c_int, _T, _T],
     "aixk_reduce_to": [_P, C.c_int, _T, _T],
     "aixk_reduce_to_init": [_P, C.c_int, _T, _T, C.c_uint64],
+    "aixk_sum_partials": [_P, _P, C.c_uint64, _T, C.c_uint64],
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_argmax_onehot_many": [_P, _P, C.c_uint32],
     "aixk_matmul": [_P, _T, _T, _T],

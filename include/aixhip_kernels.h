@@ -159,6 +159,12 @@ int32_t aixk_reduce_to(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const 
  * what fill(0) / fillMin() followed by reduceTo / maxTo computes (aixCore.hpp:632-639, 873-891)
  * without the separate fill pass over dst. */
 int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t init_bits);
+/* The second half of a sum over all elements that a generated kernel began (a product that is only formed to be
+ * summed -- the gradient of a scalar constant, aixCore.hpp:2384-2438 -- is summed where it is formed): `partials` holds
+ * `count` partial sums in device memory, float for f32 / f16 / bf16 results and double for f64; the one-element dst
+ * receives round(init + their sum), init being the value the destination was filled with (its bits in the low bytes of
+ * init_bits), as aixk_reduce_to_init lands a sum.  No counterpart in the reference's interface. */
+int32_t aixk_sum_partials(aixk_ctx* ctx, const void* partials, uint64_t count, const aixhip_tensor* dst, uint64_t init_bits);
 /* Device::argmaxTo / argmaxIndicesTo (aixDeviceCPU.cpp:275-298, 320-360). onehot=1 scatters ones
  * into the pre-zeroed int32 dst of src's shape; onehot=2 also zeroes dst first (the fill(0) the
  * caller issues before argmaxIndicesTo, aixCore.hpp:927-941, folded in: over a handful of rows the

@@ -1079,6 +1079,53 @@ static void testRowProgramTakesInAPlainKernel()
     CHECK(cap3.fused.size() + cap3.singles.size() == 2);
 }
 
+static void testSumOfEverythingJoinsItsProducer()
+{
+    // the gradient of a scalar constant: p = g * x is formed only to be summed; the kernel goes on around the sum
+    // (q = p + x here) and never stores p.  All three launch shapes compile; with no producer in the window the sum is a
+    // single operator; a row program does not take it.
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    auto g = T(1, {64, 96}), x = T(2, {64, 96}), p = T(3, {64, 96}), s = T(4, {}), q = T(5, {64, 96}), s2 = T(6, {});
+    for (uintptr_t id = 1; id <= 6; ++id) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    const float zero = 0.0f, seven = 7.0f;
+    e.record(OpType::Mul, View(g), View(x), View(p));
+    e.recordWholeSum(View(p), View(s), &zero);
+    e.record(OpType::Add, View(p), View(x), View(q));
+    e.recordWholeSum(View(q), View(s2), &seven);
+    e.releaseBuffer(reinterpret_cast<void*>(uintptr_t(3) * 0x10000));
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() == 1) {
+        const auto& d = cap.fused[0];
+        CHECK(d.ops.size() == 4 && d.inputBuffers.size() == 2 && d.outputBuffers.size() == 3);        // s, q, s2: p stays in registers
+        CHECK(d.ops[1].type == OpType::ReduceTo && d.ops[1].whole && d.ops[1].outputIndex != SIZE_MAX && d.ops[1].scalarIndex1 != SIZE_MAX);
+        CHECK(d.ops[3].whole && d.outputBuffers[d.ops[3].outputIndex].data == s2.data);
+        CHECK(d.rowLength == 0);
+        CHECK(compiles(d, gen::Shape::Flat) && compiles(d, gen::Shape::Rows) && compiles(d, gen::Shape::Gather));
+        const std::string src = gen::source(d, gen::Shape::Flat, 0, true);
+        CHECK(src.find("acc" + std::to_string(d.ops[1].outputIndex) + " += up(") != std::string::npos && src.find("row_sum<256>") != std::string::npos);
+        CHECK(gen::signature(d, gen::Shape::Flat, 0, true).find("ReduceTo!(") != std::string::npos);
+    }
+    // nothing in the window produces the operand: a single operator, as before
+    Capture alone;
+    FuseEngine f(config(), alone.callbacks());
+    for (uintptr_t id : {1, 4}) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    f.recordWholeSum(View(g), View(s), &zero);
+    f.flush();
+    CHECK(alone.fused.empty() && alone.singles.size() == 1 && alone.singles[0].type == OpType::ReduceTo && alone.singles[0].whole);
+    // a row program keeps its rows: the sum of everything closes it and runs as a single operator
+    Capture rows;
+    FuseEngine h(config(), rows.callbacks());
+    for (uintptr_t id = 1; id <= 30; ++id) h.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    recordSoftmax(h, DataType::kFloat32, 16, 256, 20);
+    auto y = T(26, {16, 256}), sy = T(27, {});
+    h.recordWholeSum(View(y), View(sy), &zero);
+    h.flush();
+    CHECK(rows.fused.size() == 1 && rows.singles.size() == 1 && rows.fused[0].rowLength == 256);
+    for (const auto& op : rows.fused[0].ops) CHECK(!op.whole);
+}
+
 static void testEqualKernelsLeaveSideBySide()
 {
     // head after head: b = a * t (t a transposed view: no operand of a row program, so the product is a kernel of its
@@ -1199,6 +1246,7 @@ int main(int argc, char** argv)
     testIdleFillsWaitForTheirFirstUser();
     testLoneCastsAsKernelsAndTheManyBlocksForm();
     testRowProgramTakesInAPlainKernel();
+    testSumOfEverythingJoinsItsProducer();
     testEqualKernelsLeaveSideBySide();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;

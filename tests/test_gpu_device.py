@@ -636,6 +636,65 @@ def test_fill_is_folded_into_argmax_indices_to(dev):
     dev.release()
 
 
+def test_sum_of_everything_joins_the_kernel_that_forms_it(dev):
+    """The gradient of a scalar constant (aixCore.hpp:2384-2438, 2030-2036): p = g * x, then fill(0) + reduceTo of p down to
+    one element, while the expression goes on (q = p + x, whose own sum starts from 7).  One generated kernel that adds
+    p and q up where they are formed, plus aixk_sum_partials per sum; p is never stored once its buffer is gone.
+    f32 / f64: 1e-5 / 1e-12 of the sum of |terms| against a float64 sum of the oracle's elementwise results; bf16 / f16
+    (summed in f32 here, in the 16-bit type on the CPU): 2e-2 of it.  Sizes from a ragged handful to 3 million, a strided
+    operand (the rows shape) and a higher-rank transposed one (the gather shape)."""
+    set_diag(dev)
+    rng = np.random.default_rng(45000)
+    zero, seven = np.zeros(1, np.float32), np.full(1, 7.0, np.float32)
+    cases = [(O.F32, [257], None), (O.F32, [1024, 3000], None), (O.BF16, [512, 768], None), (O.F16, [33, 1000], None), (O.F64, [100, 1001], None),
+             (O.F32, [64, 96], "rows"), (O.BF16, [6, 40, 24], "gather")]
+    for dtype, shape, kind in cases:
+        rec = Recorder(dev, dtype, shape)
+        g = rec.leaf(T.contiguous_tensor(rng, dtype, shape, lo=-1, hi=1))
+        if kind == "rows":
+            xh = T.view_tensor(rng, dtype, shape, "sliced", lo=-1, hi=1)
+        elif kind == "gather":
+            xh = T.view_tensor(rng, dtype, shape, "transposed", lo=-1, hi=1)
+        else:
+            xh = T.contiguous_tensor(rng, dtype, shape, lo=-1, hi=1)
+        x = rec.leaf(xh)
+        sums = []
+        for _ in range(2):
+            host = T.empty(dtype, [])
+            sums.append({"host": host, "ptr": dev.raw(host.storage.nbytes)})
+        dev.dev.synchronize()
+        p = rec.binary(O.MUL, g, x)
+        d0 = H.kdesc(sums[0]["host"], sums[0]["ptr"])
+        dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(d0))
+        dev.dev.call("reduce_to", H.ref(p["desc"]), H.ref(d0))
+        q = rec.binary(O.ADD, p, x)
+        d1 = H.kdesc(sums[1]["host"], sums[1]["ptr"])
+        dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(d1))
+        dev.dev.call("reduce_to", H.ref(q["desc"]), H.ref(d1))
+        pv, qv = O.to_float64(p["host"].storage, dtype), O.to_float64(q["host"].storage, dtype)
+        rec.free_temps(keep=(q,))
+        got_q = dev.fetch(q["ptr"], q["host"].storage)
+        diag = dev.dev.diagnostics()
+        assert diag.fusible_subgraphs == 1 and diag.fused_ops == 4 and diag.fallback_ops == 0, (NAMES[dtype], shape, kind, diag.subgraph_summary, diag.fallback_summary)
+        T.assert_same_bits(got_q, q["host"].storage, f"q = g * x + x beside its sums, {NAMES[dtype]} {shape} {kind}")
+        tol = {O.F64: 1e-12, O.F32: 1e-5}.get(dtype, 2e-2)
+        for node, exact, scale in ((sums[0], pv.sum(), np.abs(pv).sum()), (sums[1], 7.0 + qv.sum(), 7.0 + np.abs(qv).sum())):
+            got = float(O.to_float64(dev.fetch(node["ptr"], node["host"].storage), dtype)[0])
+            assert abs(got - exact) <= tol * scale, (NAMES[dtype], shape, kind, got, exact)
+        dev.release()
+    # a sum whose operand no recorded operator produces runs as before, and so does one taken with fusion switched off
+    x = T.contiguous_tensor(rng, O.F32, [1000], lo=-1, hi=1)
+    _, dx = dev.put(x)
+    host = T.empty(O.F32, [])
+    ps = dev.raw(4)
+    ds = H.kdesc(host, ps)
+    dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(ds))
+    dev.dev.call("reduce_to", H.ref(dx), H.ref(ds))
+    got = float(dev.fetch(ps, host.storage)[0])
+    assert abs(got - (7.0 + x.storage.astype(np.float64).sum())) <= 1e-5 * (7.0 + np.abs(x.storage).sum())
+    dev.release()
+
+
 def test_runs_of_argmax_indices_to_leave_as_one_launch(dev):
     """The masks of max()'s backward pass, head after head (aixCore.hpp:2170-2175): calls whose zero fill was folded in
     wait and leave in one launch; a recorded operator that reads a mask, a source that a recorded operator produces, and
