@@ -668,7 +668,7 @@ private:
                 const size_t def = findDef(m_groups[g], in.data);
                 if (def == SIZE_MAX) continue;
                 const Group& grp = m_groups[g];
-                const bool usable = target == SIZE_MAX && !m_perRow[def] && at(def).type != OpType::Cast && sameElements(defView(def), in) &&
+                const bool usable = target == SIZE_MAX && !m_perRow[def] && sameElements(defView(def), in) &&     // (a cast at a kernel's load included: the group has the cast's result type)
                                     grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L);
                 if (usable) { resolved = Operand{Operand::kValue, def}; target = g; }
                 else { closeGroup(g); closedSomething = true; }
@@ -726,7 +726,7 @@ private:
                 const Group& grp = m_groups[g];
                 size_t wholes = 0;
                 for (size_t w : grp.ops) wholes += at(w).whole;
-                const bool usable = target == SIZE_MAX && !grp.rowLen && !m_perRow[d] && !at(d).whole && at(d).type != OpType::Cast && sameElements(defView(d), in) &&
+                const bool usable = target == SIZE_MAX && !grp.rowLen && !m_perRow[d] && !at(d).whole && sameElements(defView(d), in) &&
                                     grp.dtype == in.dtype && grp.count == in.size && wholes < 8 &&
                                     grp.loads.size() + grp.defs.size() + 2 <= m_cfg.maxBufferSlots;
                 if (usable) { target = g; def = d; }
