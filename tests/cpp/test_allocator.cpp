@@ -233,9 +233,17 @@ static void planner_traffic(unsigned seed, int rounds)
         if (what < 25) {                                               // elementwise, full op full
             void* y = full[rng() % full.size()];
             dev.add(tensor(x, {rows, len}), tensor(y, {rows, len}), tensor(fresh_full(), {rows, len}));
-        } else if (what < 35) {                                        // full op (one value per row)
+        } else if (what < 33) {                                        // full op (one value per row)
             void* c = cols[rng() % cols.size()];
             dev.sub(tensor(x, {rows, len}), tensor(c, {rows, len}, DataType::kFloat32, {1, 0}), tensor(fresh_full(), {rows, len}));
+        } else if (what < 38) {                                        // a product that is only formed to be summed, and a triangle of a sum
+            void* prod = dev.allocate(n * 4);
+            dev.mul(tensor(x, {rows, len}), tensor(full[0], {rows, len}), tensor(prod, {rows, len}));
+            void* s = fresh_col();
+            dev.fill(&zero, DataType::kFloat32, tensor(s, {}));
+            dev.reduceTo(tensor(prod, {rows, len}), tensor(s, {}));
+            if (what & 1) dev.tril(tensor(prod, {rows, len}), tensor(fresh_full(), {rows, len}), 0);
+            dev.deallocate(prod);
         } else if (what < 45) {                                        // row maximum / row sum with the fill in front
             void* c = fresh_col();
             if (what & 1) { dev.fillMin(tensor(c, {rows, 1})); dev.maxTo(tensor(x, {rows, len}), tensor(c, {rows, 1})); }
