@@ -451,6 +451,7 @@ void DeviceHIP::flushWindow(bool final)
     issuePending();                                     // pending products were called before anything now in the window was recorded
     try { m_engine->flush(final); }
     catch (...) { m_extras->batch.clear(); m_extras->smallFills.clear(); throw; }
+    issuePending();                                         // (one-hot operators replayed on their own wait for each other: emitSingle)
     releaseLimbo();
 }
 
@@ -652,6 +653,21 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 {
     const bool smallFill = (op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels;
     if (!smallFill || m_extras->batch.count()) issueFlatBatch();            // (a fill joins the fills before it)
+    if (op.type == OpType::ArgmaxIndicesTo) {
+        // a recorded one-hot that found no company: the stand-alone operator with the zero fill folded in; several in a
+        // row wait for each other and leave in one launch (see argmaxIndicesTo())
+        auto& ex = *m_extras;
+        AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
+        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.batchFlatKernels || !ex.apartFromWaiting(op.input0.data, nullptr, op.output.data)) issuePending();
+        aixk_argmax_item item{};
+        toPod(op.input0, &item.src); toPod(op.output, &item.dst);
+        item.dim = op.input0.rank - 1;
+        ex.onehots.push_back(item);
+        ex.noteWaiting(op.input0.data, nullptr, op.output.data);
+        markTouched(op.input0.data); markTouched(op.output.data);
+        if (!ex.batchFlatKernels) issuePending();
+        return;
+    }
     issuePending();
     AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
     if ((op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels) {
@@ -1258,6 +1274,20 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
     uint64_t init = 0;
     const bool folded = takeInit(src, dst, &init);
     auto& ex = *m_extras;
+    // Rows that a row program takes (as recordRowReduction has them): recorded, so that the multiplication with the mask
+    // that always follows (max()'s backward) finds the ones and zeros in registers
+    if (folded && init == 0 && ex.fuseRowReductions && m_engine->config().elementwiseFusion && m_engine->config().supportsStridedFusion &&
+        (src.dtype == DataType::kFloat32 || src.dtype == DataType::kFloat16 || src.dtype == DataType::kBFloat16) && src.size && dst.size == src.size &&
+        findBlock(src.data) && findBlock(dst.data) && src.data != dst.data && src.isContiguous && dst.isContiguous && dst.offset == 0 && src.shape == dst.shape &&
+        !src.shape.empty() && dim + 1 == src.shape.size() && src.shape.size() <= AIXK_MAX_RANK) {
+        const size_t L = src.shape.back(), vec = 16 / dataTypeSize(src.dtype);
+        if (L >= 32 && L % vec == 0 && src.offset % vec == 0 && L / vec <= 8 * (L >= 2048 ? 256u : 64u) && L < (size_t(1) << 31)) {
+            View in(src), out(dst);
+            out.makeDense();
+            m_engine->recordRowOnehot(in, out, L);
+            return;
+        }
+    }
     if (folded && init == 0 && ex.batchFlatKernels && src.size && src.size < (size_t(1) << 31) && dst.size == src.size && findBlock(src.data) && findBlock(dst.data) &&
         src.data != dst.data && src.isContiguous && dst.isContiguous && dst.offset == 0 && src.shape == dst.shape && !src.shape.empty() &&
         dim + 1 == src.shape.size() && src.shape.size() <= AIXK_MAX_RANK) {

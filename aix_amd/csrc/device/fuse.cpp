@@ -369,6 +369,7 @@ public:
             else if (isElementwiseOp(op.type) && m_cfg.elementwiseFusion) placeOp(i);
             else if (isRowReduce(op.type) && op.rowLength && m_cfg.elementwiseFusion && m_cfg.supportsStridedFusion) placeReduce(i);
             else if (op.whole && m_cfg.elementwiseFusion) placeWhole(i);
+            else if (op.type == OpType::ArgmaxIndicesTo && op.rowLength && m_cfg.elementwiseFusion && m_cfg.supportsStridedFusion) placeOnehot(i);
             else placeSingle(i);
         }
         for (size_t g = 0; g < m_groupCount; ++g) closeGroup(g);
@@ -571,7 +572,12 @@ private:
                     if (!m_groups[g].open) continue;
                     const size_t def = findDef(m_groups[g], in[k]->data);
                     if (def == SIZE_MAX) continue;
-                    const bool usable = valueUsable(m_groups[g], def, *in[k], op) && compatible(m_groups[g], op, in[k]->dtype);
+                    // (the ones and zeros of a row program's one-hot operator are values of the program's type: only a cast to
+                    // that type may take them, and takes them as they are)
+                    const bool usable = at(def).type == OpType::ArgmaxIndicesTo
+                                            ? isCast && op.output.dtype == m_groups[g].dtype && op.output.size == m_groups[g].count && sameElements(defView(def), *in[k]) &&
+                                                  rowOperandKind(op.output, m_groups[g].rows(), m_groups[g].rowLen) == RowOperand::Dense
+                                            : valueUsable(m_groups[g], def, *in[k], op) && compatible(m_groups[g], op, in[k]->dtype);
                     if (usable && (target == SIZE_MAX || target == g)) {
                         resolved[k] = Operand{Operand::kValue, def};
                         target = g;
@@ -705,6 +711,64 @@ private:
         g.ops.push_back(i);
         m_groupOf[i] = target;
         m_perRow[i] = 1;
+    }
+
+    // ---- the place of every row's first maximum, as ones and zeros ------------------------------------
+    // Joins the row program that holds its operand in registers or loads it, else starts one.
+    void placeOnehot(size_t i)
+    {
+        const auto& op = at(i);
+        const View& in = op.input0;
+        const size_t L = op.rowLength;
+        size_t target = SIZE_MAX;
+        Operand resolved{};
+        for (;;) {
+            bool closedSomething = false;
+            target = SIZE_MAX;
+            resolved = Operand{};
+            if (findFill(in.data)) materialise(in.data);
+            resolved.kind = Operand::kMemory;
+            for (size_t g = 0; g < m_groupCount; ++g) {
+                if (!m_groups[g].open) continue;
+                const size_t def = findDef(m_groups[g], in.data);
+                if (def == SIZE_MAX) continue;
+                const Group& grp = m_groups[g];
+                const bool usable = target == SIZE_MAX && !m_perRow[def] && !at(def).whole && at(def).type != OpType::ArgmaxIndicesTo && sameElements(defView(def), in) &&
+                                    grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L);
+                if (usable) { resolved = Operand{Operand::kValue, def}; target = g; }
+                else { closeGroup(g); closedSomething = true; }
+            }
+            if (closedSomething) continue;
+            if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
+                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
+                    const Group& grp = m_groups[g];
+                    if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
+                }
+            }
+            if (closeGroupsTouching(op.output.data, target, &op.output)) continue;
+            if (target != SIZE_MAX) {
+                const Group& grp = m_groups[target];
+                size_t slots = grp.loads.size() + grp.defs.size() + 1;
+                if (resolved.kind == Operand::kMemory && !loads(grp, in)) ++slots;
+                if (slots > m_cfg.maxBufferSlots) { closeGroup(target); continue; }
+            }
+            break;
+        }
+        if (findFill(op.output.data)) eraseFill(op.output.data);     // every element of the destination is defined
+        if (target == SIZE_MAX) {
+            target = newGroup();
+            Group& fresh = m_groups[target];
+            fresh.dtype = in.dtype;
+            fresh.count = in.size;
+            fresh.shape = &op.input0;
+        }
+        Group& g = m_groups[target];
+        g.rowLen = L;
+        m_operands[i][0] = resolved;
+        if (resolved.kind == Operand::kMemory && !loads(g, in)) g.loads.push_back(ViewRef{(uint32_t)i, 0});
+        g.defs.push_back(i);
+        g.ops.push_back(i);
+        m_groupOf[i] = target;
     }
 
     // ---- the sum of everything ------------------------------------------------------------------
@@ -1078,6 +1142,16 @@ void FuseEngine::recordRowReduce(OpType type, const View& input, const View& out
     r.input0 = input; r.output = output; r.rowLength = rowLength;
     r.scalarDType = output.dtype;
     std::memcpy(r.scalarData.data(), init, aix::Device::dataTypeSize(output.dtype));
+    maybeFlush();
+}
+
+void FuseEngine::recordRowOnehot(const View& input, const View& output, size_t rowLength)
+{
+    if (rowLength == 0 || input.size % rowLength != 0 || output.size != input.size || output.dtype != DataType::kInt32 || !input.dense || !output.dense)
+        throw std::invalid_argument("recordRowOnehot: rows of a dense operand into a dense int32 result of its shape");
+    wake(input.data); wake(output.data);
+    OpRecord& r = append(OpType::ArgmaxIndicesTo);
+    r.input0 = input; r.output = output; r.rowLength = rowLength;
     maybeFlush();
 }
 

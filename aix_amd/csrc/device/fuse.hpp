@@ -224,6 +224,11 @@ public:
     // registers -- the product that is only formed to be summed is then never stored -- and is replayed as a plain
     // reduction when there is no such kernel.
     void recordWholeSum(const View& input, const View& output, const void* init);
+    // argmaxIndicesTo along the last, dense dimension (`rowLength` elements) of `input` into the dense int32 `output` of
+    // the same shape, whose zero fill the caller has taken out of the window: 1 at the first maximum of every row, 0
+    // elsewhere.  Inside a row program the ones and zeros are values of the program's type that a cast to that type
+    // takes as they are (max()'s backward multiplies the seed with them: the int32 tensor need never exist).
+    void recordRowOnehot(const View& input, const View& output, size_t rowLength);
     // Plans and emits the window.  A fill (fill / fillMin of a whole dense buffer that allocate() handed out) that no
     // other operator of the window touches, and that nobody outside is about to read, is not emitted unless `final`:
     // it waits, outside the window, until an operator naming its buffer is recorded (it then rejoins the window ahead

@@ -430,6 +430,9 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
         o << "extern \"C\" __global__ __launch_bounds__(" << kBlock << ") void " << rowEntryName(d, g) << "(Args a)\n{\n"
           << "    const u32 BID = blockIdx.x, GDIM = gridDim.x;\n";
     }
+    bool anyOnehot = false;
+    for (const auto& op : d.ops) if (op.type == OpType::ArgmaxIndicesTo) anyOnehot = true;
+    if (anyOnehot) o << "    __shared__ u32 redi[8];\n    (void)redi;\n";
     o << "    __shared__ W red[4];\n    (void)red;\n"
       << "    T s[" << AS << "];\n";
     for (size_t k = 0; k < NS; ++k) o << "    s[" << k << "] = __builtin_bit_cast(T, (word_t)a.sc[" << k << "]);\n";
@@ -509,6 +512,28 @@ std::string rowSource(const FusedSubgraphDescriptor& d, const RowGeometry& g, bo
             }
             o << ";\n";
             if (op.outputIndex != SIZE_MAX) o << "        if (lane == 0) out" << op.outputIndex << "[row] = " << from_t(op.outputIndex, "p" + std::to_string(k)) << ";\n";
+            continue;
+        }
+        if (op.type == OpType::ArgmaxIndicesTo) {
+            // 1 at the row's first maximum, 0 elsewhere (values of T; a store converts them).  Every lane scans its own
+            // elements by growing column, so a strict '>' keeps the first of equal values; NaNs are no candidates, but a
+            // NaN in column 0 wins outright (it stands in as +infinity at the smallest column), as the stand-alone operator has it.
+            const std::string x = fullOperand(op.inputIndex0, op.scalarIndex0);
+            o << "        T v" << k << "[NV][VEC];\n        {\n            W bv = lowestW; u32 bi = 0xffffffffu; bool ok = false;\n"
+              << "#pragma unroll\n            for (int j = 0; j < NV; ++j) {\n                if (lane + (u64)j * G < nvec) {\n#pragma unroll\n                    for (int e = 0; e < VEC; ++e) {\n"
+              << "                        W w = up(" << x << ");\n                        const u32 c = (u32)((lane + (u64)j * G) * VEC + e);\n"
+              << "                        if (c == 0 && w != w) w = (W)__builtin_huge_val();\n"
+              << "                        if (w == w && (!ok || w > bv)) { bv = w; bi = c; ok = true; }\n"
+              << "                    }\n                }\n            }\n"
+              << "            const u32 win = row_first_max<G>(bv, bi, ok, red, " << "redi);\n"
+              << "            const T one = down<T>((W)1);\n"
+              << "#pragma unroll\n            for (int j = 0; j < NV; ++j) {\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) v" << k << "[j][e] = (u32)((lane + (u64)j * G) * VEC + e) == win ? one : zero<T>();\n            }\n        }\n";
+            if (op.outputIndex != SIZE_MAX) {
+                const size_t qo = op.outputIndex;
+                o << "#pragma unroll\n        for (int j = 0; j < NV; ++j) {\n            const u64 v = lane + (u64)j * G;\n            if (v < nvec) {\n"
+                  << "                vec<O" << qo << ", VEC> w;\n#pragma unroll\n                for (int e = 0; e < VEC; ++e) w.v[e] = " << from_t(qo, "v" + std::to_string(k) + "[j][e]") << ";\n"
+                  << "                store_sel<AIX_NT>((vec<O" << qo << ", VEC>*)(out" << qo << " + row * a.len) + v, w);\n            }\n        }\n";
+            }
             continue;
         }
         if (isTri(op.type)) {

@@ -324,6 +324,35 @@ template <int LANES, class W> __device__ __forceinline__ W row_sum(W v, W* red)
         return ((red[0] + red[1]) + red[2]) + red[3];
     }
 }
+// The place of a row's first maximum (argmaxIndicesTo along the row): every lane brings the best of its own elements --
+// the largest value that is no NaN and the smallest column holding it -- and all lanes get the winner back.  A greater
+// value wins, between equal values the smaller column; a lane without a candidate loses to one with.
+template <int LANES, class W> __device__ __forceinline__ u32 row_first_max(W v, u32 at, bool valid, W* red, u32* redi)
+{
+    u32 ok = valid ? 1u : 0u;
+#pragma unroll
+    for (int d = 32; d > 0; d >>= 1) {
+        const W ov = __shfl_down(v, d, 64);
+        const u32 oat = __shfl_down(at, d, 64), ook = __shfl_down(ok, d, 64);
+        const bool take = (ok && ook) ? (ov > v || (ov == v && oat < at)) : (ook != 0 && ok == 0);
+        if (take) { v = ov; at = oat; ok = ook; }
+    }
+    if constexpr (LANES == 64) return __shfl(at, 0, 64);
+    else {
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) { red[threadIdx.x >> 6] = v; redi[threadIdx.x >> 6] = at; redi[4 + (threadIdx.x >> 6)] = ok; }
+        __syncthreads();
+        v = red[0]; at = redi[0]; ok = redi[4];
+#pragma unroll
+        for (int w = 1; w < 4; ++w) {
+            const W ov = red[w];
+            const u32 oat = redi[w], ook = redi[4 + w];
+            const bool take = (ok && ook) ? (ov > v || (ov == v && oat < at)) : (ook != 0 && ok == 0);
+            if (take) { v = ov; at = oat; ok = ook; }
+        }
+        return at;
+    }
+}
 template <int LANES, class W> __device__ __forceinline__ W row_max(W v, W* red)
 {
 #pragma unroll

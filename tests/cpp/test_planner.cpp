@@ -1126,6 +1126,65 @@ static void testSumOfEverythingJoinsItsProducer()
     for (const auto& op : rows.fused[0].ops) CHECK(!op.whole);
 }
 
+static void testOnehotOfRowMaximaLivesInARowProgram()
+{
+    // max()'s backward inside a softmax gradient: mask = one-hot of the row maxima of x (int32), c = cast(mask) to the
+    // seed's type, y = c * m with m a per-row value of the same program.  One row program; the int32 mask is dead after
+    // the window and never stored.  Alone in its window the one-hot is a single operator; alive, it is stored as int32.
+    Capture cap;
+    FuseEngine e(config(), cap.callbacks());
+    const size_t rows = 16, L = 512;
+    auto g = T(1, {rows, L}, DataType::kBFloat16), m = T(2, {rows, 1}, DataType::kBFloat16), x = T(3, {rows, L}, DataType::kBFloat16);
+    auto mask = T(4, {rows, L}, DataType::kInt32), c = T(5, {rows, L}, DataType::kBFloat16), y = T(6, {rows, L}, DataType::kBFloat16);
+    auto mB = T(2, {rows, L}, DataType::kBFloat16, {1, 0});
+    for (uintptr_t id = 1; id <= 6; ++id) e.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    uint8_t zero[8] = {};
+    e.recordRowReduce(OpType::ReduceTo, View(g), View(m), zero, L);
+    e.recordRowOnehot(View(x), View(mask), L);
+    e.record(OpType::Cast, View(mask), View(c));
+    e.record(OpType::Mul, View(c), View(mB), View(y));
+    for (uintptr_t id : {4, 5}) e.releaseBuffer(reinterpret_cast<void*>(id * 0x10000));
+    e.flush();
+    CHECK(cap.fused.size() == 1 && cap.singles.empty());
+    if (cap.fused.size() == 1) {
+        const auto& d = cap.fused[0];
+        CHECK(d.rowLength == L && d.ops.size() == 4 && d.inputBuffers.size() == 2 && d.outputBuffers.size() == 2);      // g, x -> m, y
+        CHECK(d.ops[1].type == OpType::ArgmaxIndicesTo && d.ops[1].outputIndex == SIZE_MAX && d.ops[2].type == OpType::Cast && d.ops[2].inputIndex0 == 2 + 1);
+        for (const auto& out : d.outputBuffers) CHECK(out.dtype == DataType::kBFloat16);
+        CHECK(compilesRow(d));
+    }
+    // the mask alive after the window: stored by the program, converted to int32
+    Capture kept;
+    FuseEngine f(config(), kept.callbacks());
+    for (uintptr_t id = 1; id <= 6; ++id) f.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    f.recordRowOnehot(View(x), View(mask), L);
+    f.record(OpType::Cast, View(mask), View(c));
+    f.record(OpType::Mul, View(c), View(g), View(y));
+    f.flush();
+    CHECK(kept.fused.size() == 1);
+    if (kept.fused.size() == 1) {
+        bool storesMask = false;
+        for (const auto& out : kept.fused[0].outputBuffers) if (out.data == mask.data && out.dtype == DataType::kInt32) storesMask = true;
+        CHECK(storesMask && kept.fused[0].rowLength == L);
+        CHECK(compilesRow(kept.fused[0]));
+    }
+    // alone: the plain operator; read by anything but a cast to the program's type: from memory
+    Capture alone;
+    FuseEngine h(config(), alone.callbacks());
+    for (uintptr_t id = 1; id <= 8; ++id) h.retainBuffer(reinterpret_cast<void*>(id * 0x10000));
+    h.recordRowOnehot(View(x), View(mask), L);
+    h.flush();
+    CHECK(alone.fused.empty() && alone.singles.size() == 1 && alone.singles[0].type == OpType::ArgmaxIndicesTo);
+    auto asF32 = T(7, {rows, L}, DataType::kFloat32);
+    h.recordRowOnehot(View(x), View(mask), L);
+    h.record(OpType::Cast, View(mask), View(asF32));            // to f32, not the program's bf16
+    h.flush();
+    CHECK(alone.singles.size() >= 2);
+    bool maskWritten = false;
+    for (const auto& s1 : alone.singles) if (s1.type == OpType::ArgmaxIndicesTo) maskWritten = true;
+    CHECK(maskWritten);
+}
+
 static void testEqualKernelsLeaveSideBySide()
 {
     // head after head: b = a * t (t a transposed view: no operand of a row program, so the product is a kernel of its
@@ -1247,6 +1306,7 @@ int main(int argc, char** argv)
     testLoneCastsAsKernelsAndTheManyBlocksForm();
     testRowProgramTakesInAPlainKernel();
     testSumOfEverythingJoinsItsProducer();
+    testOnehotOfRowMaximaLivesInARowProgram();
     testEqualKernelsLeaveSideBySide();
     std::printf(g_failed ? "%d checks FAILED\n" : "all planner checks passed\n", g_failed);
     return g_failed ? 1 : 0;

@@ -479,3 +479,48 @@ def test_triangle_after_a_row_sum_stays_in_the_kernel(dev, dtype):
             return (x - x * x.sum(axis=-1, keepdims=True)) * 0.5 * keep
 
         run_both(dev, dtype, shape, build, 950 + k, expect_fused_ops=5, lo=-0.5, hi=0.5, exact=exact, tol16=4e-2)
+
+
+# ---- the place of every row's first maximum inside a row program ----------------------------------------------------
+def _onehot_of_row_maxima(f, x, shape):
+    """fill(0) + argmaxIndicesTo along the last dim (aixCore.hpp:927-941), then the cast to the working type that
+    `seed * mask` makes (aixCore.hpp:2170-2175, 1616-1630)."""
+    mask_host = T.empty(O.I32, shape)
+    zero = np.zeros(1, np.float32)
+    assert CPU.fill(zero.ctypes.data, O.F32, C.byref(mask_host.desc())) == 0
+    assert CPU.argmax_indices_to(C.byref(x["host"].desc()), C.byref(mask_host.desc()), len(shape) - 1) == 0
+    pm = f.dev.raw(mask_host.storage.nbytes)
+    dm = H.kdesc(mask_host, pm)
+    f.temps.append({"host": mask_host, "ptr": pm, "desc": dm})
+    f.dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(dm))
+    f.dev.dev.call("argmax_indices_to", H.ref(x["desc"]), H.ref(dm), len(shape) - 1)
+    r = f.result(shape)
+    assert CPU.copy(mask_host.storage.ctypes.data, O.I32, r["host"].storage.ctypes.data, f.dtype, mask_host.size) == 0
+    f.dev.dev.call("copy", pm, O.I32, r["ptr"], f.dtype, mask_host.size)
+    return r
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.F16], ids=lambda d: NAMES[d])
+def test_onehot_of_row_maxima_stays_in_the_kernel(dev, dtype):
+    """max()'s backward as the softmax gradient has it: y = x * rowsum(x) + cast(onehot(x)) * rowsum(x) -- the row sum, the
+    one-hot of every row's first maximum, its conversion and two products in ONE row program; the int32 mask is gone
+    before the read and is never written.  Ties (values on a coarse grid), a row of NaNs, a NaN in column 0 and NaNs
+    elsewhere: as the stand-alone operator has them, bit for bit."""
+    for k, shape in enumerate([[64, 128], [3, 5, 512], [9, 1000], [4, 2048], [1, 64]]):
+        def poke(host, shape=shape):
+            vals = O.to_float64(host.storage, dtype).reshape(-1, shape[-1])
+            vals = np.round(vals * 2) / 2                                  # many equal maxima: the first one wins
+            if vals.shape[0] >= 4:
+                vals[1, :] = np.nan                                        # nothing to compare: the leading NaN wins
+                vals[2, 0] = np.nan                                        # a leading NaN wins over everything
+                vals[3, 5] = np.nan                                        # a NaN elsewhere is no candidate
+            host.storage[:] = O.to_storage(vals.reshape(-1), dtype)
+
+        def build(f, x, rng, shape=shape):
+            s = f.row_sum(x, shape)
+            a = f.binary(O.MUL, x, f.over_rows(s, shape), shape)
+            m = _onehot_of_row_maxima(f, x, shape)
+            return f.binary(O.ADD, a, f.binary(O.MUL, m, f.over_rows(s, shape), shape), shape)
+
+        got = run_both(dev, dtype, shape, build, 980 + k, expect_fused_ops=6, lo=-2.0, hi=2.0, poke=poke)
+        assert got.size == O.numel(shape)
