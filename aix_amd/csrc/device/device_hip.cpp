@@ -227,8 +227,22 @@ bool DeviceHIP::BlockTable::erase(void* base, size_t* bytes)
     const uintptr_t key = (uintptr_t)base;
     const size_t mask = m_slots.size() - 1;
     for (size_t i = slotOf(key);; i = (i + 1) & mask) {
-        if (m_slots[i].key == key) { *bytes = m_slots[i].block.bytes; m_slots[i].key = 1; --m_count; return true; }
         if (m_slots[i].key == 0) return false;
+        if (m_slots[i].key != key) continue;
+        *bytes = m_slots[i].block.bytes;
+        // no gravestone: the entries behind it in the probe sequence move up (linear probing allows that), so chains stay
+        // as short as the table's load makes them however many blocks come and go
+        size_t hole = i;
+        for (size_t j = (i + 1) & mask; m_slots[j].key != 0; j = (j + 1) & mask) {
+            const size_t home = slotOf(m_slots[j].key);
+            // j's entry may move to the hole if its home is not strictly inside (hole, j] (cyclically)
+            const bool between = hole <= j ? (home > hole && home <= j) : (home > hole || home <= j);
+            if (!between) { m_slots[hole] = m_slots[j]; hole = j; }
+        }
+        m_slots[hole] = Slot{};
+        --m_count;
+        --m_used;
+        return true;
     }
 }
 

@@ -49,6 +49,7 @@ struct Node {
     int handles{0};                                 // Tensor objects that name this node
     int readers{0};                                 // backward formulas (its own, its consumers') that read `value`
     uint64_t serial{nextSerial()};                  // creation order: a node is always younger than its inputs
+    uint64_t visited{0};                            // the last single-pass traversal that reached this node
 
     Node(Value v, bool req) : value(std::move(v)), requireGrad(req) {}
 
@@ -196,21 +197,23 @@ public:
     void backwardOnce() const
     {
         if (value().size() != 1) throw std::invalid_argument("backward() requires a one-element tensor");
-        std::vector<Node*> order{m_node.get()};
-        std::unordered_set<Node*> seen{m_node.get()};
-        for (size_t k = 0; k < order.size(); ++k)     // everything the result depends on
-            for (const auto& in : order[k]->inputs)
-                if (seen.insert(in.get()).second) order.push_back(in.get());
-        // (the leaves last of all: nothing waits for them, and a scalar constant's "grad += seed", issued where the constant
-        // was created -- in the middle of a formula -- would make the kernel that forms the seed stop there)
-        std::sort(order.begin(), order.end(), [](const Node* a, const Node* b) {
-            const bool la = a->inputs.empty(), lb = b->inputs.empty();
-            return la != lb ? lb : a->serial > b->serial;
-        });
+        // everything the result depends on, marked with this pass's number as it is found
+        static thread_local uint64_t pass = 0;
+        ++pass;
+        std::vector<std::pair<uint64_t, Node*>> order{{0, m_node.get()}};
+        m_node->visited = pass;
+        for (size_t k = 0; k < order.size(); ++k)
+            for (const auto& in : order[k].second->inputs)
+                if (in->visited != pass) { in->visited = pass; order.push_back({0, in.get()}); }
+        // youngest first; the leaves last of all: nothing waits for them, and a scalar constant's "grad += seed", issued
+        // where the constant was created -- in the middle of a formula -- would make the kernel that forms the seed stop there
+        for (auto& entry : order) entry.first = (entry.second->inputs.empty() ? 0 : uint64_t(1) << 63) | entry.second->serial;
+        std::sort(order.begin(), order.end(), [](const auto& a, const auto& b) { return a.first > b.first; });
         Node::accumulating() = true;
         try {
             m_node->pending = Value::full(device(), dtype(), shape(), 1.0f);
-            for (Node* n : order) {
+            for (const auto& entry : order) {
+                Node* n = entry.second;
                 if (!n->pending.defined() && n->windows.empty()) continue;
                 const Value seed = n->takeSeed();
                 if (n->retainGrad) n->grad() += seed;
