@@ -359,6 +359,8 @@ public:
         m_perRow.assign(ops.size(), 0);
         m_groupOf.assign(ops.size(), SIZE_MAX);
         m_groupCount = 0;
+        m_open.clear();
+        m_openCount = 0;
         m_emits.clear();
         m_fills.clear();
         m_fillsAbsorbed = 0;
@@ -487,6 +489,14 @@ private:
     {
         if (m_groupCount == m_groups.size()) m_groups.emplace_back();
         m_groups[m_groupCount].reset();
+        // the open groups in the order they were made; closed ones are weeded out now and then (never inside a loop over them)
+        if (m_open.size() > 2 * m_openCount + 8) {
+            size_t kept = 0;
+            for (size_t g : m_open) if (m_groups[g].open) m_open[kept++] = g;
+            m_open.resize(kept);
+        }
+        m_open.push_back(m_groupCount);
+        ++m_openCount;
         return m_groupCount++;
     }
 
@@ -568,7 +578,8 @@ private:
                     materialise(in[k]->data);
                 }
                 resolved[k].kind = Operand::kMemory;
-                for (size_t g = 0; g < m_groupCount; ++g) {
+                for (size_t gi = 0; gi < m_open.size(); ++gi) {
+                    const size_t g = m_open[gi];
                     if (!m_groups[g].open) continue;
                     const size_t def = findDef(m_groups[g], in[k]->data);
                     if (def == SIZE_MAX) continue;
@@ -596,7 +607,8 @@ private:
 
             // no producer inside the window: share loads with an open group of the same shape
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
+                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_open[gi];
                     if (!m_groups[g].open || !compatible(m_groups[g], op, op.output.dtype)) continue;
                     for (int k = 0; k < 2; ++k)
                         if (resolved[k].kind == Operand::kMemory && loads(m_groups[g], *in[k])) target = g;
@@ -669,7 +681,8 @@ private:
             resolved = Operand{};
             if (findFill(in.data)) materialise(in.data);
             resolved.kind = Operand::kMemory;
-            for (size_t g = 0; g < m_groupCount; ++g) {
+            for (size_t gi = 0; gi < m_open.size(); ++gi) {
+                const size_t g = m_open[gi];
                 if (!m_groups[g].open) continue;
                 const size_t def = findDef(m_groups[g], in.data);
                 if (def == SIZE_MAX) continue;
@@ -681,7 +694,8 @@ private:
             }
             if (closedSomething) continue;
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
+                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_open[gi];
                     const Group& grp = m_groups[g];
                     if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
                 }
@@ -728,7 +742,8 @@ private:
             resolved = Operand{};
             if (findFill(in.data)) materialise(in.data);
             resolved.kind = Operand::kMemory;
-            for (size_t g = 0; g < m_groupCount; ++g) {
+            for (size_t gi = 0; gi < m_open.size(); ++gi) {
+                const size_t g = m_open[gi];
                 if (!m_groups[g].open) continue;
                 const size_t def = findDef(m_groups[g], in.data);
                 if (def == SIZE_MAX) continue;
@@ -740,7 +755,8 @@ private:
             }
             if (closedSomething) continue;
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t g = 0; g < m_groupCount && target == SIZE_MAX; ++g) {
+                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_open[gi];
                     const Group& grp = m_groups[g];
                     if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
                 }
@@ -783,7 +799,8 @@ private:
             size_t target = SIZE_MAX, def = SIZE_MAX;
             bool closedSomething = false;
             if (findFill(in.data)) { placeSingle(i); return; }
-            for (size_t g = 0; g < m_groupCount; ++g) {
+            for (size_t gi = 0; gi < m_open.size(); ++gi) {
+                const size_t g = m_open[gi];
                 if (!m_groups[g].open) continue;
                 const size_t d = findDef(m_groups[g], in.data);
                 if (d == SIZE_MAX) continue;
@@ -934,6 +951,7 @@ private:
         for (size_t w : b.ops) m_groupOf[w] = into;
         b.ops.clear(); b.defs.clear(); b.loads.clear();
         b.open = false;                                     // absorbed: never emitted on its own
+        --m_openCount;
         b.absorbed = true;
     }
 
@@ -955,7 +973,8 @@ private:
     {
         bool closed = false;
         if (!buffer) return false;
-        for (size_t g = 0; g < m_groupCount; ++g) {
+        for (size_t gi = 0; gi < m_open.size(); ++gi) {
+            const size_t g = m_open[gi];
             Group& grp = m_groups[g];
             if (!grp.open) continue;
             bool touches = false, conflicting = false;
@@ -977,14 +996,15 @@ private:
 
     void closeWriters(const void* buffer)
     {
-        for (size_t g = 0; g < m_groupCount; ++g)
-            if (m_groups[g].open && findDef(m_groups[g], buffer) != SIZE_MAX) closeGroup(g);
+        for (size_t gi = 0; gi < m_open.size(); ++gi)
+            if (m_groups[m_open[gi]].open && findDef(m_groups[m_open[gi]], buffer) != SIZE_MAX) closeGroup(m_open[gi]);
     }
 
     void closeGroup(size_t g)
     {
         if (!m_groups[g].open) return;
         m_groups[g].open = false;
+        --m_openCount;
         m_emits.push_back({true, g});
     }
 
@@ -1023,6 +1043,8 @@ private:
     std::vector<uint8_t> m_perRow;           // the operator yields one value per row of its (row program) group
     std::vector<Group> m_groups;             // [0, m_groupCount) belong to the current window
     size_t m_groupCount{0};
+    std::vector<size_t> m_open;              // indices of the open groups, ascending (with some closed ones not yet weeded out)
+    size_t m_openCount{0};
     std::vector<Emit> m_emits;
     std::vector<PendingFill> m_fills;
     std::vector<uint8_t> m_store;
