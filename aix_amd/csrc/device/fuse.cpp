@@ -361,6 +361,8 @@ public:
         m_groupCount = 0;
         m_open.clear();
         m_openCount = 0;
+        m_touchIndex.clear();
+        m_touchUsed = 0;
         m_emits.clear();
         m_fills.clear();
         m_fillsAbsorbed = 0;
@@ -485,6 +487,52 @@ private:
             if (m_fills[k].buffer == buffer) { m_fills[k] = m_fills.back(); m_fills.pop_back(); return; }
     }
 
+    // ---- which open groups touch a buffer --------------------------------------------------------------
+    // Every question an operator asks of the open groups starts from one of its buffers (who defines it, who loads it,
+    // who has to close before it is overwritten), so the groups are kept per buffer: a window with hundreds of open
+    // kernels -- the same short formula applied to tensor after tensor -- costs an operator no more than a small one.
+    std::vector<uint32_t>& touchList(const void* buffer)
+    {
+        auto it = m_touchIndex.find(buffer);
+        if (it != m_touchIndex.end()) return m_touchLists[it->second];
+        if (m_touchUsed == m_touchLists.size()) m_touchLists.emplace_back();
+        m_touchLists[m_touchUsed].clear();
+        m_touchIndex.emplace(buffer, (uint32_t)m_touchUsed);
+        return m_touchLists[m_touchUsed++];
+    }
+    void addTouch(size_t g, const void* buffer)
+    {
+        if (!buffer) return;
+        auto& list = touchList(buffer);
+        for (uint32_t known : list) if (known == g) return;
+        list.insert(std::upper_bound(list.begin(), list.end(), (uint32_t)g), (uint32_t)g);     // ascending, as the groups were made
+    }
+    void dropTouches(size_t g)
+    {
+        auto drop = [&](const void* buffer) {
+            auto it = m_touchIndex.find(buffer);
+            if (it == m_touchIndex.end()) return;
+            auto& list = m_touchLists[it->second];
+            for (size_t k = 0; k < list.size(); ++k) if (list[k] == g) { list.erase(list.begin() + (long)k); break; }
+        };
+        for (const ViewRef& r : m_groups[g].loads) drop(view(r).data);
+        for (size_t def : m_groups[g].defs) drop(defView(def).data);
+    }
+    // The open groups that touch `buffer` (and `other`, if given), ascending, copied into `out` so that the caller may
+    // close and merge groups while it walks them.
+    void touching(const void* buffer, const void* other, std::vector<uint32_t>& out)
+    {
+        out.clear();
+        for (const void* p : {buffer, other}) {
+            if (!p) continue;
+            auto it = m_touchIndex.find(p);
+            if (it == m_touchIndex.end()) continue;
+            const auto& list = m_touchLists[it->second];
+            if (out.empty()) out.assign(list.begin(), list.end());
+            else { for (uint32_t g : list) if (std::find(out.begin(), out.end(), g) == out.end()) out.push_back(g); std::sort(out.begin(), out.end()); }
+        }
+    }
+
     size_t newGroup()
     {
         if (m_groupCount == m_groups.size()) m_groups.emplace_back();
@@ -578,8 +626,9 @@ private:
                     materialise(in[k]->data);
                 }
                 resolved[k].kind = Operand::kMemory;
-                for (size_t gi = 0; gi < m_open.size(); ++gi) {
-                    const size_t g = m_open[gi];
+                touching(in[k]->data, nullptr, m_candA);
+                for (size_t gi = 0; gi < m_candA.size(); ++gi) {
+                    const size_t g = m_candA[gi];
                     if (!m_groups[g].open) continue;
                     const size_t def = findDef(m_groups[g], in[k]->data);
                     if (def == SIZE_MAX) continue;
@@ -607,8 +656,9 @@ private:
 
             // no producer inside the window: share loads with an open group of the same shape
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
-                    const size_t g = m_open[gi];
+                touching(resolved[0].kind == Operand::kMemory && in[0] ? in[0]->data : nullptr, resolved[1].kind == Operand::kMemory && in[1] ? in[1]->data : nullptr, m_candA);
+                for (size_t gi = 0; gi < m_candA.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_candA[gi];
                     if (!m_groups[g].open || !compatible(m_groups[g], op, op.output.dtype)) continue;
                     for (int k = 0; k < 2; ++k)
                         if (resolved[k].kind == Operand::kMemory && loads(m_groups[g], *in[k])) target = g;
@@ -648,6 +698,7 @@ private:
             m_operands[i][k] = resolved[k];
             if (resolved[k].kind == Operand::kMemory) {
                 if (!loads(g, *in[k])) g.loads.push_back(ViewRef{(uint32_t)i, (uint32_t)k});
+                addTouch(target, in[k]->data);
                 if (!isDense(*in[k])) g.dense = false;
             } else if (resolved[k].kind == Operand::kScalar) {
                 g.hasScalar = true;
@@ -657,6 +708,7 @@ private:
         bool redefined = false;
         for (auto& def : g.defs) if (sameView(defView(def), op.output)) { def = i; redefined = true; }
         if (!redefined) g.defs.push_back(i);
+        addTouch(target, op.output.data);
         g.ops.push_back(i);
         m_groupOf[i] = target;
         if (op.type == OpType::Tril || op.type == OpType::Triu) g.hasTri = true;
@@ -681,8 +733,9 @@ private:
             resolved = Operand{};
             if (findFill(in.data)) materialise(in.data);
             resolved.kind = Operand::kMemory;
-            for (size_t gi = 0; gi < m_open.size(); ++gi) {
-                const size_t g = m_open[gi];
+            touching(in.data, nullptr, m_candA);
+            for (size_t gi = 0; gi < m_candA.size(); ++gi) {
+                const size_t g = m_candA[gi];
                 if (!m_groups[g].open) continue;
                 const size_t def = findDef(m_groups[g], in.data);
                 if (def == SIZE_MAX) continue;
@@ -694,8 +747,9 @@ private:
             }
             if (closedSomething) continue;
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
-                    const size_t g = m_open[gi];
+                touching(in.data, nullptr, m_candA);
+                for (size_t gi = 0; gi < m_candA.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_candA[gi];
                     const Group& grp = m_groups[g];
                     if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
                 }
@@ -721,7 +775,9 @@ private:
         g.rowLen = L;
         m_operands[i][0] = resolved;
         if (resolved.kind == Operand::kMemory && !loads(g, in)) g.loads.push_back(ViewRef{(uint32_t)i, 0});
+        if (resolved.kind == Operand::kMemory) addTouch(target, in.data);
         g.defs.push_back(i);
+        addTouch(target, op.output.data);
         g.ops.push_back(i);
         m_groupOf[i] = target;
         m_perRow[i] = 1;
@@ -742,8 +798,9 @@ private:
             resolved = Operand{};
             if (findFill(in.data)) materialise(in.data);
             resolved.kind = Operand::kMemory;
-            for (size_t gi = 0; gi < m_open.size(); ++gi) {
-                const size_t g = m_open[gi];
+            touching(in.data, nullptr, m_candA);
+            for (size_t gi = 0; gi < m_candA.size(); ++gi) {
+                const size_t g = m_candA[gi];
                 if (!m_groups[g].open) continue;
                 const size_t def = findDef(m_groups[g], in.data);
                 if (def == SIZE_MAX) continue;
@@ -755,8 +812,9 @@ private:
             }
             if (closedSomething) continue;
             if (target == SIZE_MAX && m_cfg.multiOutputKernels) {
-                for (size_t gi = 0; gi < m_open.size() && target == SIZE_MAX; ++gi) {
-                    const size_t g = m_open[gi];
+                touching(in.data, nullptr, m_candA);
+                for (size_t gi = 0; gi < m_candA.size() && target == SIZE_MAX; ++gi) {
+                    const size_t g = m_candA[gi];
                     const Group& grp = m_groups[g];
                     if (grp.open && grp.dtype == in.dtype && grp.count == in.size && rowsFit(grp, L) && loads(grp, in)) target = g;
                 }
@@ -782,7 +840,9 @@ private:
         g.rowLen = L;
         m_operands[i][0] = resolved;
         if (resolved.kind == Operand::kMemory && !loads(g, in)) g.loads.push_back(ViewRef{(uint32_t)i, 0});
+        if (resolved.kind == Operand::kMemory) addTouch(target, in.data);
         g.defs.push_back(i);
+        addTouch(target, op.output.data);
         g.ops.push_back(i);
         m_groupOf[i] = target;
     }
@@ -799,8 +859,9 @@ private:
             size_t target = SIZE_MAX, def = SIZE_MAX;
             bool closedSomething = false;
             if (findFill(in.data)) { placeSingle(i); return; }
-            for (size_t gi = 0; gi < m_open.size(); ++gi) {
-                const size_t g = m_open[gi];
+            touching(in.data, nullptr, m_candA);
+            for (size_t gi = 0; gi < m_candA.size(); ++gi) {
+                const size_t g = m_candA[gi];
                 if (!m_groups[g].open) continue;
                 const size_t d = findDef(m_groups[g], in.data);
                 if (d == SIZE_MAX) continue;
@@ -820,6 +881,7 @@ private:
             Group& g = m_groups[target];
             m_operands[i][0] = Operand{Operand::kValue, def};
             g.defs.push_back(i);
+            addTouch(target, op.output.data);
             g.ops.push_back(i);
             g.hasScalar = true;                                                        // (the destination's initial value)
             m_groupOf[i] = target;
@@ -941,8 +1003,9 @@ private:
         m_merged.resize(a.ops.size() + b.ops.size());
         std::merge(a.ops.begin(), a.ops.end(), b.ops.begin(), b.ops.end(), m_merged.begin());     // program order
         a.ops.assign(m_merged.begin(), m_merged.end());
-        for (size_t def : b.defs) a.defs.push_back(def);
-        for (const ViewRef& r : b.loads) if (!loads(a, view(r))) a.loads.push_back(r);
+        dropTouches(from);
+        for (size_t def : b.defs) { a.defs.push_back(def); addTouch(into, defView(def).data); }
+        for (const ViewRef& r : b.loads) { if (!loads(a, view(r))) a.loads.push_back(r); addTouch(into, view(r).data); }
         if (!a.shape->sameShape(*b.shape) && !b.dense) a.shape = b.shape;        // a is all dense then: it adopts the shape b's strided views need
         a.dense = a.dense && b.dense;
         a.hasScalar = a.hasScalar || b.hasScalar;
@@ -973,8 +1036,9 @@ private:
     {
         bool closed = false;
         if (!buffer) return false;
-        for (size_t gi = 0; gi < m_open.size(); ++gi) {
-            const size_t g = m_open[gi];
+        touching(buffer, nullptr, m_candB);
+        for (size_t gi = 0; gi < m_candB.size(); ++gi) {
+            const size_t g = m_candB[gi];
             Group& grp = m_groups[g];
             if (!grp.open) continue;
             bool touches = false, conflicting = false;
@@ -996,8 +1060,9 @@ private:
 
     void closeWriters(const void* buffer)
     {
-        for (size_t gi = 0; gi < m_open.size(); ++gi)
-            if (m_groups[m_open[gi]].open && findDef(m_groups[m_open[gi]], buffer) != SIZE_MAX) closeGroup(m_open[gi]);
+        touching(buffer, nullptr, m_candB);
+        for (size_t gi = 0; gi < m_candB.size(); ++gi)
+            if (m_groups[m_candB[gi]].open && findDef(m_groups[m_candB[gi]], buffer) != SIZE_MAX) closeGroup(m_candB[gi]);
     }
 
     void closeGroup(size_t g)
@@ -1005,6 +1070,7 @@ private:
         if (!m_groups[g].open) return;
         m_groups[g].open = false;
         --m_openCount;
+        dropTouches(g);
         m_emits.push_back({true, g});
     }
 
@@ -1018,20 +1084,21 @@ private:
         for (size_t g = 0; g < m_groupCount; ++g)
             for (size_t def : m_groups[g].defs)
                 if (m_live.count(defView(def).data)) m_store[def] = 1;
+        m_lastWriter.clear();                                   // buffer -> the latest operator so far that writes it
         for (size_t j = 0; j < n; ++j) {
             const View* in[2] = {&at(j).input0, &at(j).input1};
             for (int k = 0; k < 2; ++k) {
                 if (m_operands[j][k].kind != Operand::kMemory || !in[k]->data) continue;
-                for (size_t w = j; w-- > 0;) {
-                    if (at(w).output.data != in[k]->data) continue;
-                    if (m_groupOf[w] != SIZE_MAX) {
-                        // the value that must be in memory is the group's last definition of that view
-                        for (size_t def : m_groups[m_groupOf[w]].defs)
-                            if (sameView(defView(def), at(w).output)) m_store[def] = 1;
-                    }
-                    break;
+                const auto it = m_lastWriter.find(in[k]->data);
+                if (it == m_lastWriter.end()) continue;
+                const size_t w = it->second;
+                if (m_groupOf[w] != SIZE_MAX) {
+                    // the value that must be in memory is the group's last definition of that view
+                    for (size_t def : m_groups[m_groupOf[w]].defs)
+                        if (sameView(defView(def), at(w).output)) m_store[def] = 1;
                 }
             }
+            if (at(j).output.data) m_lastWriter[at(j).output.data] = j;
         }
     }
 
@@ -1045,6 +1112,11 @@ private:
     size_t m_groupCount{0};
     std::vector<size_t> m_open;              // indices of the open groups, ascending (with some closed ones not yet weeded out)
     size_t m_openCount{0};
+    std::unordered_map<const void*, uint32_t> m_touchIndex;      // buffer -> its list in m_touchLists
+    std::vector<std::vector<uint32_t>> m_touchLists;             // (kept from window to window: [0, m_touchUsed) are in use)
+    size_t m_touchUsed{0};
+    std::vector<uint32_t> m_candA, m_candB;                      // working copies for the loops over touching groups
+    std::unordered_map<const void*, size_t> m_lastWriter;        // decideStores()
     std::vector<Emit> m_emits;
     std::vector<PendingFill> m_fills;
     std::vector<uint8_t> m_store;
@@ -1223,6 +1295,8 @@ void FuseEngine::flush(bool final)
 
     m_window.clear();
     m_window.swap(m_pending);                // operators recorded by callbacks belong to the next window
+    m_pendingUse.clear();
+    m_counted = 0;
     if (!final && m_config.deferIdleFills && m_config.elementwiseFusion && m_config.absorbFills) setAsideIdleFills();
     const std::vector<OpRecord>& window = m_window;
     // buffers about to be read outside the planner count as alive for this window
@@ -1324,27 +1398,45 @@ bool FuseEngine::takeTrailingFill(const View& output, OpRecord* fill)
             op.output.offset != output.offset || op.output.size != output.size || !output.dense || !op.output.dense)
             return false;
         *fill = op;
+        if (k < m_counted) {                                    // (a fill: it only writes)
+            auto it = m_pendingUse.find(op.output.data);
+            if (it != m_pendingUse.end() && it->second.first) --it->second.first;
+            --m_counted;
+        }
         m_pending.erase(m_pending.begin() + (long)k);
         return true;
     }
     return false;
 }
 
+// How often the recorded operators write / read each buffer, brought up to date when somebody asks (operators are
+// appended far more often than anybody asks).
+void FuseEngine::countPending()
+{
+    for (; m_counted < m_pending.size(); ++m_counted) {
+        const OpRecord& op = m_pending[m_counted];
+        if (op.output.data) ++m_pendingUse[op.output.data].first;
+        if (op.input0.data) ++m_pendingUse[op.input0.data].second;
+        if (op.hasInput1 && op.input1.data) ++m_pendingUse[op.input1.data].second;
+    }
+}
+
 bool FuseEngine::pendingWrites(const void* buffer)
 {
     if (!buffer) return false;
     wake(buffer);
-    for (const OpRecord& op : m_pending) if (op.output.data == buffer) return true;
-    return false;
+    countPending();
+    const auto it = m_pendingUse.find(buffer);
+    return it != m_pendingUse.end() && it->second.first != 0;
 }
 
 bool FuseEngine::pendingTouches(const void* buffer)
 {
     if (!buffer) return false;
     wake(buffer);
-    for (const OpRecord& op : m_pending)
-        if (op.output.data == buffer || op.input0.data == buffer || (op.hasInput1 && op.input1.data == buffer)) return true;
-    return false;
+    countPending();
+    const auto it = m_pendingUse.find(buffer);
+    return it != m_pendingUse.end() && (it->second.first != 0 || it->second.second != 0);
 }
 
 void FuseEngine::recordExternalRead(const void* buffer)

@@ -264,6 +264,10 @@ private:
     OpRecord& append(OpType type);
     std::vector<OpRecord> m_pending;       // capacity is kept from window to window
     std::vector<OpRecord> m_window;
+    // pendingWrites() / pendingTouches(): per buffer, how many of m_pending[0, m_counted) write / read it
+    std::unordered_map<const void*, std::pair<uint32_t, uint32_t>> m_pendingUse;
+    size_t m_counted{0};
+    void countPending();
     PointerSet m_live;
     std::vector<const void*> m_externalReads;
     std::vector<OpRecord> m_waiting;       // fills set aside by flush(false), oldest first
