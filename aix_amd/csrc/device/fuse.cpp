@@ -359,8 +359,6 @@ public:
         m_perRow.assign(ops.size(), 0);
         m_groupOf.assign(ops.size(), SIZE_MAX);
         m_groupCount = 0;
-        m_open.clear();
-        m_openCount = 0;
         m_touchIndex.clear();
         m_touchUsed = 0;
         m_emits.clear();
@@ -537,14 +535,6 @@ private:
     {
         if (m_groupCount == m_groups.size()) m_groups.emplace_back();
         m_groups[m_groupCount].reset();
-        // the open groups in the order they were made; closed ones are weeded out now and then (never inside a loop over them)
-        if (m_open.size() > 2 * m_openCount + 8) {
-            size_t kept = 0;
-            for (size_t g : m_open) if (m_groups[g].open) m_open[kept++] = g;
-            m_open.resize(kept);
-        }
-        m_open.push_back(m_groupCount);
-        ++m_openCount;
         return m_groupCount++;
     }
 
@@ -1014,7 +1004,6 @@ private:
         for (size_t w : b.ops) m_groupOf[w] = into;
         b.ops.clear(); b.defs.clear(); b.loads.clear();
         b.open = false;                                     // absorbed: never emitted on its own
-        --m_openCount;
         b.absorbed = true;
     }
 
@@ -1069,7 +1058,6 @@ private:
     {
         if (!m_groups[g].open) return;
         m_groups[g].open = false;
-        --m_openCount;
         dropTouches(g);
         m_emits.push_back({true, g});
     }
@@ -1110,8 +1098,6 @@ private:
     std::vector<uint8_t> m_perRow;           // the operator yields one value per row of its (row program) group
     std::vector<Group> m_groups;             // [0, m_groupCount) belong to the current window
     size_t m_groupCount{0};
-    std::vector<size_t> m_open;              // indices of the open groups, ascending (with some closed ones not yet weeded out)
-    size_t m_openCount{0};
     std::unordered_map<const void*, uint32_t> m_touchIndex;      // buffer -> its list in m_touchLists
     std::vector<std::vector<uint32_t>> m_touchLists;             // (kept from window to window: [0, m_touchUsed) are in use)
     size_t m_touchUsed{0};
