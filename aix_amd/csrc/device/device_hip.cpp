@@ -122,7 +122,7 @@ struct DeviceHIP::Extras {
     bool fuseRowReductions = [] { const char* e = std::getenv("AIXHIP_FUSE_ROW_REDUCTIONS"); return !(e && e[0] == '0'); }();
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
     struct Group { std::vector<aixhip_tensor> a, b, out; };
-    std::array<Group, 4> groups;
+    std::array<Group, 8> groups;
     // sliceSet and argmaxIndicesTo calls waiting to leave as one launch each (see DeviceHIP::sliceSet, argmaxIndicesTo)
     std::vector<aixk_slice_item> slices;
     std::vector<aixk_argmax_item> onehots;
@@ -139,6 +139,10 @@ struct DeviceHIP::Extras {
         if ((r0 && waitWrites.contains(r0)) || (r1 && waitWrites.contains(r1))) return false;
         return !waitWrites.contains(w) && !waitReads.contains(w);
     }
+    // p is an operand or the result of a call that waits
+    bool waitingUses(const void* p) const { return p && waitReads.size() + waitWrites.size() && (waitWrites.contains(p) || waitReads.contains(p)); }
+    // p is the result of a call that waits
+    bool waitingWrites(const void* p) const { return p && waitWrites.size() && waitWrites.contains(p); }
     void noteWaiting(const void* r0, const void* r1, const void* w)
     {
         if (r0) waitReads.insert(r0);
@@ -393,7 +397,7 @@ void DeviceHIP::deallocate(void* memory)
     m_limbo.emplace_back(memory, bytes);
     m_limboBytes += bytes;
     m_liveBytes -= bytes;
-    if (m_limboBytes > (size_t(8) << 30)) flushWindow(false);   // recorded work pins too much freed memory
+    if (m_limboBytes > (size_t(8) << 30)) { issuePending(); flushWindow(false); }   // recorded and waiting work pins too much freed memory
 }
 
 void DeviceHIP::markTouched(const void* p)
@@ -417,11 +421,14 @@ void DeviceHIP::releaseLimbo()
 {
     if (m_limbo.empty()) return;
     auto& ex = *m_extras;
-    size_t kept = 0;
+    size_t kept = 0, held = 0;
     for (size_t k = 0; k < m_limbo.size(); ++k) {
         const auto entry = m_limbo[k];
         const Block* b = m_blocks.find(entry.first);        // staging blocks are not in the table: always used
-        if (b && !b->touched) {
+        if (ex.waitingUses(entry.first)) {                  // a call that has not been enqueued yet uses it: it stays
+            m_limbo[kept++] = entry;
+            ++held;
+        } else if (b && !b->touched) {
             size_t bytes = 0;
             m_blocks.erase(entry.first, &bytes);
             m_pool[entry.second].push_back(entry.first);
@@ -437,17 +444,26 @@ void DeviceHIP::releaseLimbo()
     const size_t enough = std::max<size_t>({size_t(32) << 20, m_totalBytes >> 10, (m_liveBytes + m_pooledBytes) / 8});
     if (++ex.flushesSinceEvent < 16 && m_limboBytes < enough) return;
     ex.flushesSinceEvent = 0;
-    for (const auto& entry : m_limbo) { size_t bytes = 0; m_blocks.erase(entry.first, &bytes); }
+    std::vector<std::pair<void*, size_t>> stay, leave;
+    if (held) {
+        for (const auto& entry : m_limbo) (ex.waitingUses(entry.first) ? stay : leave).push_back(entry);
+        if (leave.empty()) return;
+    } else {
+        leave.swap(m_limbo);
+    }
+    size_t stayBytes = 0;
+    for (const auto& entry : stay) stayBytes += entry.second;
+    for (const auto& entry : leave) { size_t bytes = 0; m_blocks.erase(entry.first, &bytes); }
     Cooling c{};
     if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
-        c.blocks.swap(m_limbo);
+        c.blocks.swap(leave);
         ex.cooling.push_back(std::move(c));
     } else {
         aixk_sync(m_ctx);
-        for (auto& b : m_limbo) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
-        m_limbo.clear();
+        for (auto& b : leave) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
     }
-    m_limboBytes = 0;
+    m_limbo.swap(stay);
+    m_limboBytes = stayBytes;
 }
 
 void DeviceHIP::emptyCache()
@@ -462,26 +478,39 @@ void DeviceHIP::flush() { flushWindow(true); }
 // final: nothing recorded stays behind.  Otherwise fills that nothing recorded so far uses may wait (FuseEngine::flush).
 void DeviceHIP::flushWindow(bool final)
 {
-    issuePending();                                     // pending products were called before anything now in the window was recorded
+    // Calls that wait (small products, sliceSet, one-hot masks) stay waiting across a flush: they depend on nothing
+    // recorded (their callers saw to that), and a kernel that leaves now and uses what they write, or writes what they
+    // use, sends them off first (emitFused, emitSingle).
+    if (final) issuePending();
     try { m_engine->flush(final); }
     catch (...) { m_extras->batch.clear(); m_extras->smallFills.clear(); throw; }
-    issuePending();                                         // (one-hot operators replayed on their own wait for each other: emitSingle)
+    if (final) issuePending();                              // (one-hot operators replayed on their own wait as well: emitSingle)
     releaseLimbo();
 }
 
 void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
 {
     AIXHIP_TRACE("-- operator outside the planner (%zu recorded)", m_engine->pendingOps());
+    const void* bases[3] = {nullptr, nullptr, nullptr};
+    size_t i = 0;
     for (const void* p : {a, b, c}) {
+        const size_t at = i++;
         if (!p) continue;
         m_engine->recordExternalRead(p);
         const void* base = m_blocks.baseOf(p);              // an operand may point into the middle of a block
-        if (base && base != p) m_engine->recordExternalRead(base);
+        if (base && base != p) { m_engine->recordExternalRead(base); bases[at] = base; }
     }
     markTouched(a);                                         // the caller is about to enqueue work on them
     markTouched(b);
     markTouched(c);
+    // calls that wait and have nothing to do with these operands go on waiting
+    auto& ex = *m_extras;
+    auto meets = [&] {
+        return ex.waitingUses(a) || ex.waitingUses(b) || ex.waitingUses(c) || ex.waitingUses(bases[0]) || ex.waitingUses(bases[1]) || ex.waitingUses(bases[2]);
+    };
+    if (meets()) issuePending();
     flushWindow(false);
+    if (meets()) issuePending();                            // (a one-hot replayed on its own has just begun to wait)
 }
 
 // The planner orders recorded operators by the addresses of their buffers.  An operand that points into the middle of
@@ -682,7 +711,10 @@ void DeviceHIP::emitSingle(const OpRecord& op)
         if (!ex.batchFlatKernels) issuePending();
         return;
     }
-    issuePending();
+    {
+        const auto& ex = *m_extras;                         // what waits and is used here, or uses the result's buffer, goes first
+        if (ex.waitingUses(op.output.data) || ex.waitingWrites(op.input0.data) || (op.hasInput1 && ex.waitingWrites(op.input1.data))) issuePending();
+    }
     AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
     if ((op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels) {
         // small fills that follow one another leave together (issueFlatBatch sends them off ahead of whatever comes next)
@@ -731,7 +763,16 @@ void DeviceHIP::emitSingle(const OpRecord& op)
 
 void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 {
-    issuePending();
+    {
+        // calls that wait stay waiting unless this kernel reads what they write or writes what they use
+        const auto& ex = *m_extras;
+        bool meets = false;
+        if (ex.waitReads.size() + ex.waitWrites.size()) {
+            for (const auto& v : d.inputBuffers) meets = meets || ex.waitingWrites(v.data);
+            for (const auto& v : d.outputBuffers) meets = meets || ex.waitingUses(v.data);
+        }
+        if (meets) issuePending();
+    }
     constexpr size_t kMaxOperands = 64;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
     const size_t esz = dataTypeSize(d.dtype);

@@ -296,6 +296,38 @@ static void planner_traffic(unsigned seed, int rounds)
     CHECK(dev.allocatedBytes() == 0);
 }
 
+// A small 16-bit product is not enqueued when it is called: it waits for others of its shape.  Flushes that have nothing
+// to do with it leave it waiting, and a block it uses stays out of the pool until the product has been enqueued and the
+// GPU has passed it, however long ago the caller freed the block.
+static void test_blocks_of_calls_that_wait_are_not_handed_out()
+{
+    DeviceHIP dev;
+    aixk_ctx* ctx = dev.kernelContext();
+    auto half = [](void* p) { DeviceTensorParams t = matrix(p, 64, 64); t.dtype = DataType::kBFloat16; return t; };
+    void* a = dev.allocate(8192); void* b = dev.allocate(8192); void* r = dev.allocate(8192);
+    void* x = dev.allocate(64); void* y = dev.allocate(64); void* z = dev.allocate(64);
+    const uint64_t before = stub_launches(ctx);
+    dev.matmul(half(a), half(b), half(r));
+    CHECK(stub_launches(ctx) == before);                // waits
+    dev.deallocate(a);                                  // the caller is done with an operand
+    std::set<void*> fresh;
+    for (int i = 0; i < 40; ++i) {                      // other work comes and goes; its flushes record events
+        touch(dev, x, y, z);
+        void* p = dev.allocate(8192);
+        CHECK(p != a && p != b && p != r);
+        fresh.insert(p);
+    }
+    CHECK(stub_launches(ctx) == before + 40);           // the product is still waiting
+    touch(dev, r, y, z);                                // its result is read: now it goes, ahead of the reader
+    CHECK(stub_launches(ctx) == before + 42);
+    dev.synchronize();
+    CHECK(dev.cachedBytes() == 8192);                   // and only now is the operand's block back in the pool
+    void* again = dev.allocate(8192);
+    CHECK(again == a);
+    for (void* p : fresh) dev.deallocate(p);
+    for (void* p : {again, b, r, x, y, z}) dev.deallocate(p);
+}
+
 static void test_destruction_returns_everything()
 {
     const long long before = stub_held_everywhere();
@@ -320,6 +352,7 @@ int main(int argc, char** argv)
     test_untouched_temporaries_recycle_at_the_flush();
     test_used_blocks_wait_for_the_gpu();
     test_out_of_memory_retry();
+    test_blocks_of_calls_that_wait_are_not_handed_out();
     test_destruction_returns_everything();
     for (unsigned seed = 1; seed <= 4; ++seed) stress(seed, 20000);
     for (unsigned seed = 21; seed <= 24; ++seed) planner_traffic(seed, 3000);
