@@ -1088,7 +1088,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
     if (sixteen && a.shape.size() == 2 && b.shape.size() == 2 && result.shape.size() == 2 && a.dtype == result.dtype && b.dtype == result.dtype &&
         a.size && b.size && findBlock(a.data) && findBlock(b.data)) {
         const size_t M = a.shape[0], K = a.shape[1], N = b.shape[1];
-        const bool small = K % 8 == 0 && M * N >= 64 * 64 && ((M + 63) / 64) * ((N + 63) / 64) < (size_t)m_cus * 2;
+        const bool small = K % 8 == 0 && M * N >= 64 * 64 && ((M + 63) / 64) * ((N + 63) / 64) < (size_t)m_cus * 3;
         if (small && b.shape[0] == K && result.shape[0] == M && result.shape[1] == N) {
             // recorded operators that produce an operand, or that still use the result's buffer, go first (and so does
             // every pending product); any other recorded operator may as well run after the product

@@ -1328,7 +1328,7 @@ int matmul_mfma_grouped(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tens
     const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
     if (out->dtype != AIXK_BF16 && out->dtype != AIXK_F16) return -1;
     if (count < 2 || count > 65535 || K % 8 != 0 || M * N < 64 * 64) return -1;
-    if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 2) return -1;       // each product fills the chip by itself
+    if (((M + 63) / 64) * ((N + 63) / 64) >= (uint64_t)ctx->cus * 3) return -1;       // each product fills the chip by itself
     for (uint32_t i = 0; i < count; ++i) {
         if (a[i].dtype != out->dtype || b[i].dtype != out->dtype || out[i].dtype != out->dtype) return -1;
         if (a[i].shape[0] != M || a[i].shape[1] != K || b[i].shape[0] != K || b[i].shape[1] != N) return -1;
