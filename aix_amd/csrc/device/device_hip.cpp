@@ -126,13 +126,15 @@ struct DeviceHIP::Extras {
     // sliceSet and argmaxIndicesTo calls waiting to leave as one launch each (see DeviceHIP::sliceSet, argmaxIndicesTo)
     std::vector<aixk_slice_item> slices;
     std::vector<aixk_argmax_item> onehots;
+    // reduceTo calls that sum a matrix down its columns (see DeviceHIP::reduceTo): f32, f16 and bf16 wait apart
+    std::array<std::vector<aixk_colsum_item>, 3> colsums;
     // what the waiting calls of all three kinds read and write (block starts), so that a new call knows in one lookup
     // whether it may wait beside them; per destination of waiting sliceSet calls, how it was described and the windows
     // written so far
     aixhip::fuse::PointerSet waitReads, waitWrites;
     struct SliceWindows { aixhip_tensor dst; uint64_t dim; std::vector<std::pair<uint64_t, uint64_t>> ranges; };
     std::unordered_map<const void*, SliceWindows> sliceDsts;
-    bool anyPending() const { if (!slices.empty() || !onehots.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
+    bool anyPending() const { if (!slices.empty() || !onehots.empty()) return true; for (const auto& c : colsums) if (!c.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
     // a call that reads r0, r1 and writes w neither uses what waits nor is used by it
     bool apartFromWaiting(const void* r0, const void* r1, const void* w) const
     {
@@ -503,10 +505,16 @@ void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
     markTouched(a);                                         // the caller is about to enqueue work on them
     markTouched(b);
     markTouched(c);
-    // calls that wait and have nothing to do with these operands go on waiting
+    // calls that wait and have nothing to do with these operands go on waiting: the last operand named is the one the
+    // caller writes (or the only one, which it may write), the others are read
     auto& ex = *m_extras;
+    const int last = c ? 2 : b ? 1 : 0;
+    const void* named[3] = {a, b, c};
     auto meets = [&] {
-        return ex.waitingUses(a) || ex.waitingUses(b) || ex.waitingUses(c) || ex.waitingUses(bases[0]) || ex.waitingUses(bases[1]) || ex.waitingUses(bases[2]);
+        for (int k = 0; k < 3; ++k) {
+            if (k == last ? ex.waitingUses(named[k]) || ex.waitingUses(bases[k]) : ex.waitingWrites(named[k]) || ex.waitingWrites(bases[k])) return true;
+        }
+        return false;
     };
     if (meets()) issuePending();
     flushWindow(false);
@@ -1137,6 +1145,13 @@ void DeviceHIP::issuePending()
 {
     auto& ex = *m_extras;
     int status = AIXK_OK;
+    if (ex.anyPending()) {
+        size_t products = 0, sums = 0;
+        for (const auto& g : ex.groups) products += g.out.size();
+        for (const auto& c : ex.colsums) sums += c.size();
+        AIXHIP_TRACE("-- what waited leaves: %zu sliceSet, %zu argmaxIndicesTo, %zu reduceTo, %zu matmul", ex.slices.size(), ex.onehots.size(), sums, products);
+        (void)products; (void)sums;
+    }
     if (!ex.slices.empty()) {
         status = ex.slices.size() == 1 ? aixk_slice_set(m_ctx, &ex.slices[0].src, &ex.slices[0].dst, ex.slices[0].dim, ex.slices[0].start, ex.slices[0].end, ex.slices[0].step)
                                        : aixk_slice_set_many(m_ctx, ex.slices.data(), (uint32_t)ex.slices.size());
@@ -1149,6 +1164,14 @@ void DeviceHIP::issuePending()
                                             : aixk_argmax_onehot_many(m_ctx, ex.onehots.data(), (uint32_t)ex.onehots.size());
         if (ex.onehots.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.onehots.size(); }
         ex.onehots.clear();
+    }
+    for (auto& sums : ex.colsums) {
+        if (sums.empty()) continue;
+        if (status == AIXK_OK)
+            status = sums.size() == 1 ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &sums[0].src, &sums[0].dst, sums[0].init_bits)
+                                      : aixk_sum_columns_many(m_ctx, sums.data(), (uint32_t)sums.size());
+        if (sums.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += sums.size(); }
+        sums.clear();
     }
     ex.waitReads.clear(); ex.waitWrites.clear(); ex.sliceDsts.clear();
     for (auto& g : ex.groups) {
@@ -1287,6 +1310,29 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
             m_engine->recordWholeSum(in, out, &init);
             return;
         }
+    }
+    // A dense matrix summed down its columns -- the gradient of a bias or of a LayerNorm parameter, summed to the
+    // parameter's shape (aixCore.hpp:2228-2233) and read only when the backward pass reaches the parameter: like small
+    // matmul calls it waits, and all that have gathered by then leave in one pair of launches (see matmul(), sliceSet()).
+    auto& ex = *m_extras;
+    const int slot = src.dtype == DataType::kFloat32 ? 0 : src.dtype == DataType::kFloat16 ? 1 : src.dtype == DataType::kBFloat16 ? 2 : -1;
+    if (folded && slot >= 0 && ex.batchFlatKernels && src.isContiguous && dst.isContiguous && src.shape.size() >= 2 && src.shape.size() <= AIXK_MAX_RANK &&
+        !dst.shape.empty() && dst.shape.size() <= AIXK_MAX_RANK && dst.size == src.shape.back() && dst.shape.back() == dst.size && dst.size % 4 == 0 &&
+        src.size >= 2 * dst.size && src.offset % 4 == 0 && findBlock(src.data) && findBlock(dst.data) && src.data != dst.data) {
+        if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {          // recorded producers and users go first
+            m_engine->recordExternalRead(src.data);
+            flushWindow(false);
+        }
+        auto& sums = ex.colsums[slot];
+        if (sums.size() >= AIXK_COLSUM_ITEMS_MAX || !ex.apartFromWaiting(src.data, nullptr, dst.data)) issuePending();
+        AIXHIP_TRACE("   (waits: %zu columns)", dst.size);
+        aixk_colsum_item item{};
+        toPod(src, &item.src, "reduceTo"); toPod(dst, &item.dst, "reduceTo");
+        item.init_bits = init;
+        sums.push_back(item);
+        ex.noteWaiting(src.data, nullptr, dst.data);
+        markTouched(src.data); markTouched(dst.data);
+        return;
     }
     flushFor(src.data, dst.data);
     aixhip_tensor ps, pd; stagedPod(src, &ps, "reduceTo"); toPod(dst, &pd, "reduceTo");
@@ -1471,7 +1517,7 @@ void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorPar
 {
     AIXHIP_TRACE("indexSelect");
     requireDevice(dst, "indexSelect");
-    flushFor(src.data, dst.data, indices.data);
+    flushFor(src.data, indices.data, dst.data);
     aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexSelect"); toPod(dst, &pd, "indexSelect"); stagedPod(indices, &pi, "indexSelect");
     check(aixk_index_select(m_ctx, &ps, &pd, &pi, dim));
 }
@@ -1480,7 +1526,7 @@ void DeviceHIP::indexAdd(const DeviceTensorParams& src, const DeviceTensorParams
 {
     AIXHIP_TRACE("indexAdd");
     requireDevice(dst, "indexAdd");
-    flushFor(src.data, dst.data, indices.data);
+    flushFor(src.data, indices.data, dst.data);
     aixhip_tensor ps, pd, pi; stagedPod(src, &ps, "indexAdd"); toPod(dst, &pd, "indexAdd"); stagedPod(indices, &pi, "indexAdd");
     check(aixk_index_add(m_ctx, &ps, &pd, &pi, dim));
 }

@@ -570,6 +570,92 @@ __global__ __launch_bounds__(kBlock) void argmax_onehot_inner_many_k(const Oneho
     }
 }
 
+// Column sums of several dense matrices in one launch (the gradients of biases and of LayerNorm's parameters: one
+// reduceTo each, asked for throughout a backward pass and read only at its end).  Item k is rows x cols elements with
+// `pitch` elements between rows; dst[c] = init + the sum down column c.  Stage one: a workgroup takes 256 columns (a
+// lane owns 4 neighbours, the four waves take interleaved rows) of one chunk of an item's rows and leaves its sums, in
+// the accumulator's type, in `partials`; stage two adds up the chunks of a column, adds the initial value, rounds once.
+struct ColsumItem {
+    u64 src, dst, rows, cols, pitch, init;
+    u64 partials;                       // index of the item's first partial sum
+    u32 first_wg, tiles, chunks, rows_per_chunk, first_col, pad;
+};
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void sum_columns_many_k(const ColsumItem* __restrict__ items, u32 count, typename SumOp<T>::Acc* partials)
+{
+    typedef SumOp<T> Op;
+    typedef typename Op::Acc Acc;
+    typedef vec<T, 4> V;
+    __shared__ Acc sm[kWaves][kWave * 4];
+    u32 lo = 0, hi = count;
+    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (items[mid].first_wg <= blockIdx.x) lo = mid; else hi = mid; }
+    const ColsumItem it = items[lo];
+    const u32 local = blockIdx.x - it.first_wg, tile = local % it.tiles, chunk = local / it.tiles;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const u64 c0 = ((u64)tile * kWave + lane) * 4;
+    const u64 r_begin = (u64)chunk * it.rows_per_chunk;
+    const u64 r_end = r_begin + it.rows_per_chunk < it.rows ? r_begin + it.rows_per_chunk : it.rows;
+    Acc acc[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc[e] = Op::init();
+    if (c0 < it.cols) {                                     // cols is a multiple of 4: a lane's columns are all there or none
+        const T* col = global_ptr<const T>(it.src) + c0;
+        constexpr int U = 4;
+        for (u64 r0 = r_begin + wave; r0 < r_end; r0 += (u64)kWaves * U) {
+            V x[U];
+#pragma unroll
+            for (int k = 0; k < U; ++k) { const u64 r = r0 + (u64)k * kWaves; if (r < r_end) x[k] = *(const V*)(col + r * it.pitch); }
+#pragma unroll
+            for (int k = 0; k < U; ++k) {
+                const u64 r = r0 + (u64)k * kWaves;
+                if (r < r_end) {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) Op::step(acc[e], x[k].v[e], r, false);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) sm[wave][lane * 4 + e] = acc[e];
+    __syncthreads();
+    if (wave == 0 && c0 < it.cols) {
+        Acc* out = partials + it.partials + (u64)chunk * it.cols + c0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            Acc a = sm[0][lane * 4 + e];
+#pragma unroll
+            for (int w = 1; w < kWaves; ++w) a = Op::combine(a, sm[w][lane * 4 + e]);
+            out[e] = a;
+        }
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void sum_columns_finish_many_k(const ColsumItem* __restrict__ items, u32 count, const typename SumOp<T>::Acc* __restrict__ partials,
+                                                                    u32 columns)
+{
+    typedef SumOp<T> Op;
+    typedef typename Op::Acc Acc;
+    const u32 g = blockIdx.x * kBlock + threadIdx.x;
+    if (g >= columns) return;
+    u32 lo = 0, hi = count;
+    while (hi - lo > 1) { const u32 mid = (lo + hi) / 2; if (items[mid].first_col <= g) lo = mid; else hi = mid; }
+    const ColsumItem it = items[lo];
+    const u64 c = g - it.first_col;
+    const Acc* col = partials + it.partials + c;
+    Acc a = Op::init();
+    u32 k = 0;
+    for (; k + 4 <= it.chunks; k += 4) {                    // four loads in flight
+        const Acc x0 = col[(u64)k * it.cols], x1 = col[(u64)(k + 1) * it.cols], x2 = col[(u64)(k + 2) * it.cols], x3 = col[(u64)(k + 3) * it.cols];
+        a = Op::combine(Op::combine(Op::combine(Op::combine(a, x0), x1), x2), x3);
+    }
+    for (; k < it.chunks; ++k) a = Op::combine(a, col[(u64)k * it.cols]);
+    T init;
+    __builtin_memcpy(&init, &it.init, sizeof(T));
+    global_ptr<T>(it.dst)[c] = down<T>((Acc)up(init) + a);
+}
+
 // argmax down the columns of wide rows with the rows split into chunks: the record a lane keeps per column is the
 // pair (value, row) and the scan is a bare `x > best` -- three instructions per element against the seven of
 // ArgOp::step -- and the partial records are 8 bytes instead of 12 (16 for 8-byte elements).  A strict `>` from minus
@@ -1143,6 +1229,85 @@ int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, ui
         typedef decltype(tag) T;
         hipLaunchKernelGGL((argmax_onehot_inner_many_k<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const OnehotItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
         AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    });
+}
+
+int32_t aixk_sum_columns_many(aixk_ctx* ctx, const aixk_colsum_item* items, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    if (count == 0) return AIXK_OK;
+    AIXK_REQUIRE(items, "column sums of several items: no items");
+    // one pair of launches if every item is a dense matrix of one floating-point type summed down its columns into a
+    // dense vector, else item by item
+    const int dtype = items[0].src.dtype;
+    bool together = count >= 2 && count <= AIXK_COLSUM_ITEMS_MAX && (dtype == AIXK_F32 || dtype == AIXK_F16 || dtype == AIXK_BF16);
+    const size_t esz = aixk_dtype_size(dtype);
+    uint64_t tiles_all = 0, columns = 0;
+    for (uint32_t k = 0; k < count && together; ++k) {
+        const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
+        together = valid_tensor(src) && valid_tensor(dst) && src->dtype == dtype && dst->dtype == dtype && src->rank >= 2 && dst->rank >= 1 && src->size > 0 &&
+                   src->size == numel(src) && dst->size == numel(dst) && src->data && dst->data;
+        if (!together) break;
+        const uint64_t C = src->shape[src->rank - 1], R = src->size / C;
+        uint64_t dense[AIXK_MAX_RANK];
+        row_major_strides(src->rank, src->shape, dense);
+        for (int d = 0; d < src->rank; ++d) if (src->shape[d] != 1 && src->strides[d] != dense[d]) together = false;
+        together = together && dst->size == C && dst->shape[dst->rank - 1] == C && (C == 1 || dst->strides[dst->rank - 1] == 1) && R >= 2 && C % 4 == 0 &&
+                   R < (1ull << 31) && C < (1ull << 31) && ((uintptr_t)((const char*)src->data + src->offset * esz) % (4 * esz)) == 0;
+        tiles_all += (C + 255) / 256;
+        columns += C;
+    }
+    together = together && columns < (1ull << 31);
+    const uint64_t acc_bytes = dtype == AIXK_F32 ? sizeof(SumOp<float>::Acc) : sizeof(SumOp<bf16>::Acc);
+    std::vector<ColsumItem> plan;
+    u32 grid = 0;
+    if (together) {
+        // rows in chunks of at least 64 so that the launch has about 8 workgroups per compute unit
+        const uint64_t want = (uint64_t)ctx->cus * 8;
+        const uint64_t split = std::max<uint64_t>(1, (want + tiles_all - 1) / tiles_all);
+        plan.resize(count);
+        uint64_t partials = 0, col = 0;
+        for (uint32_t k = 0; k < count; ++k) {
+            const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
+            const uint64_t C = src->shape[src->rank - 1], R = src->size / C;
+            uint64_t chunks = std::min<uint64_t>({split, (R + 63) / 64, (uint64_t)64});
+            uint64_t rpc = ((R + chunks - 1) / chunks + 15) & ~(uint64_t)15;
+            chunks = (R + rpc - 1) / rpc;
+            ColsumItem& it = plan[k];
+            it.src = (u64)(uintptr_t)((const char*)src->data + src->offset * esz);
+            it.dst = (u64)(uintptr_t)((char*)dst->data + dst->offset * esz);
+            it.rows = R; it.cols = C; it.pitch = C; it.init = items[k].init_bits;
+            it.partials = partials;
+            it.first_wg = grid; it.tiles = (u32)((C + 255) / 256); it.chunks = (u32)chunks; it.rows_per_chunk = (u32)rpc; it.first_col = (u32)col; it.pad = 0;
+            partials += chunks * C;
+            col += C;
+            const uint64_t wgs = (uint64_t)it.tiles * chunks;
+            if ((uint64_t)grid + wgs >= (1ull << 31)) { together = false; break; }
+            grid += (u32)wgs;
+        }
+        together = together && partials * acc_bytes <= ctx->scratch_bytes;
+    }
+    if (!together) {
+        for (uint32_t k = 0; k < count; ++k) AIXK_TRY(aixk_reduce_to_init(ctx, AIXK_SUM, &items[k].src, &items[k].dst, items[k].init_bits));
+        return AIXK_OK;
+    }
+    const size_t table_bytes = (size_t)count * sizeof(ColsumItem);
+    char* host = nullptr;
+    const char* dev = nullptr;
+    AIXK_TRY(table_slot(ctx, table_bytes, (void**)&host, (const void**)&dev));
+    std::memcpy(host, plan.data(), table_bytes);
+    AIXK_TRY(table_upload(ctx, host, dev, table_bytes));
+    return by_dtype(dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        if constexpr (std::is_same<T, float>::value || std::is_same<T, f16>::value || std::is_same<T, bf16>::value) {
+            typedef typename SumOp<T>::Acc Acc;
+            hipLaunchKernelGGL((sum_columns_many_k<T>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const ColsumItem*)dev, (u32)count, (Acc*)ctx->scratch);
+            AIXK_HIP(hipGetLastError());
+            hipLaunchKernelGGL((sum_columns_finish_many_k<T>), dim3((unsigned)((columns + kBlock - 1) / kBlock)), dim3(kBlock), 0, ctx->stream, (const ColsumItem*)dev,
+                               (u32)count, (const Acc*)ctx->scratch, (u32)columns);
+            AIXK_HIP(hipGetLastError());
+        }
         return (int)AIXK_OK;
     });
 }

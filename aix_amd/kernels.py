@@ -34,6 +34,11 @@ class ArgmaxItem(C.Structure):
     _fields_ = [("src", Tensor), ("dst", Tensor), ("dim", C.c_uint64)]
 
 
+class ColsumItem(C.Structure):
+    """aixk_colsum_item"""
+    _fields_ = [("src", Tensor), ("dst", Tensor), ("init_bits", C.c_uint64)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("large_bar", C.c_int32), ("wavefront", C.c_int32),
@@ -80,6 +85,7 @@ _SIGNATURES = {
     "aixk_sum_partials": [_P, _P, C.c_uint64, _T, C.c_uint64],
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_argmax_onehot_many": [_P, _P, C.c_uint32],
+    "aixk_sum_columns_many": [_P, _P, C.c_uint32],
     "aixk_matmul": [_P, _T, _T, _T],
     "aixk_matmul_batched": [_P, _T, _T, _T],
     "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],

@@ -180,6 +180,19 @@ int32_t aixk_argmax_to(aixk_ctx* ctx, int onehot, const aixhip_tensor* src, cons
 typedef struct aixk_argmax_item { aixhip_tensor src, dst; uint64_t dim; } aixk_argmax_item;
 int32_t aixk_argmax_onehot_many(aixk_ctx* ctx, const aixk_argmax_item* items, uint32_t count);
 
+/* `count` reduceTo calls that sum a dense matrix down its columns, each with the fill of its destination folded in
+ * (item k is aixk_reduce_to_init(ctx, AIXK_SUM, src, dst, init_bits) of its fields): the gradients of biases and of
+ * LayerNorm's parameters, which a backward pass asks for layer after layer (aixCore.hpp:2228-2233 sums a gradient to
+ * its parameter's shape) and reads only when it reaches the parameters.  Two launches for all items when every item is a
+ * dense f32, f16 or bf16 tensor of at least two rows whose last dim (a multiple of 4 elements) is the destination,
+ * there are at most AIXK_COLSUM_ITEMS_MAX items and the partial sums fit the context's scratch memory; otherwise item by
+ * item in order.  Sums are accumulated as aixk_reduce_to accumulates them and rounded once.  The caller guarantees
+ * that no item reads what another one writes.  No counterpart in the reference's interface (one Device::reduceTo call
+ * per tensor there). */
+#define AIXK_COLSUM_ITEMS_MAX 1024
+typedef struct aixk_colsum_item { aixhip_tensor src, dst; uint64_t init_bits; } aixk_colsum_item;
+int32_t aixk_sum_columns_many(aixk_ctx* ctx, const aixk_colsum_item* items, uint32_t count);
+
 /* ---- matmul (aixDevice.hpp:63; aixDeviceCPU.cpp:362-389) ---------------- */
 /* out[m,n] = a[m,k] . b[k,n]; a, b arbitrary 2-D views; f32/f16/bf16 run on MFMA with f32
  * accumulation, other types on a generic tiled kernel with an accumulator of the element type

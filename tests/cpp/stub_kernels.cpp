@@ -89,6 +89,7 @@ STUB_OP(aixk_reduce_to, int, const aixhip_tensor*, const aixhip_tensor*)
 STUB_OP(aixk_reduce_to_init, int, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
 STUB_OP(aixk_argmax_to, int, const aixhip_tensor*, const aixhip_tensor*, uint64_t)
 STUB_OP(aixk_argmax_onehot_many, const aixk_argmax_item*, uint32_t)
+STUB_OP(aixk_sum_columns_many, const aixk_colsum_item*, uint32_t)
 STUB_OP(aixk_sum_partials, const void*, uint64_t, const aixhip_tensor*, uint64_t)
 int32_t aixk_matmul(aixk_ctx* c, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
 {

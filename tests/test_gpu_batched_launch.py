@@ -1,7 +1,8 @@
 """The kernel-layer entry points that carry several pieces of work in one launch, through the C ABI: aixk_fill_many
 (small fills, each item a pattern already in its destination's element type), aixk_rtc_launch_many (several argument
 blocks of one runtime-compiled kernel, each with its share of the grid), aixk_slice_set_many (several sliceSet calls) and
-aixk_argmax_onehot_many (several argmaxIndicesTo calls with their zero fill).
+aixk_argmax_onehot_many (several argmaxIndicesTo calls with their zero fill) and aixk_sum_columns_many (several reduceTo
+calls down the columns of a matrix, with the fill of their destination).
 Results against numpy (fills and an exact elementwise body) and the CPU oracle's sliceSet, sizes down to one element and
 ragged tails, and the argument checks they promise."""
 import ctypes as C
@@ -247,5 +248,57 @@ def test_argmax_onehot_many_is_fill_and_argmax_indices_item_by_item(gpu, dtype):
     wrong = K.Tensor.from_buffer_copy(bad_dst)
     wrong.dtype = O.F32
     assert lib.aixk_argmax_onehot_many(h, _argmax_items([together[1][0], (bad_src, wrong, 1)]), 2) == 1      # result must be int32
+    gpu.ctx.sync()
+    gpu.release()
+
+
+def _colsum_items(entries):
+    arr = (K.ColsumItem * len(entries))()
+    for k, (src, dst, bits) in enumerate(entries):
+        arr[k].src, arr[k].dst, arr[k].init_bits = src, dst, bits
+    return arr
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.F16], ids=["bf16", "f32", "f16"])
+def test_sum_columns_many_is_fill_and_reduce_to_item_by_item(gpu, dtype):
+    """Dense matrices summed down their columns leave in two launches for all of them; a set with an item of another kind
+    (a strided source, a column count that is no multiple of 4, a row sum) runs item by item.  Either way every destination
+    equals fill(init) + the oracle's reduceTo: against the sums in wide arithmetic, 1e-5 of the sum of the terms'
+    magnitudes plus one rounding in the result's type (2^-10 for f16, 2^-8 for bf16), as for aixk_reduce_to."""
+    rng = np.random.default_rng(56000 + dtype)
+    tol, final = {O.F32: (1e-5, 0.0), O.F16: (1e-5, 2.0 ** -10), O.BF16: (1e-5, 2.0 ** -8)}[dtype]
+
+    def case(shape, dshape, init_value, kind="contig"):
+        src = T.view_tensor(rng, dtype, shape, kind, lo=-2, hi=2)
+        bits_arr = O.to_storage(np.array([init_value]), dtype)
+        bits = int.from_bytes(bits_arr.tobytes()[:O.ITEMSIZE[dtype]], "little")
+        n = max(1, int(np.prod(dshape)))
+        filled = T.HostTensor(np.resize(bits_arr.view(O.NP_STORAGE[dtype]), n).copy(), dtype, dshape)
+        exact = filled.values().reshape(-1).copy()
+        scale = np.abs(exact)
+        assert CPU.reduce_to_wide(C.byref(src.desc()), C.byref(filled.desc()), exact.ctypes.data, scale.ctypes.data) == 0
+        _, dsrc = gpu.put(src)
+        garbage = T.HostTensor(np.resize(O.to_storage(np.array([777.0]), dtype), n).copy(), dtype, dshape)      # never read
+        pd, dd = gpu.put(garbage)
+        return (dsrc, dd, bits), (pd, garbage, exact, scale, f"{shape}->{dshape} init {init_value} {kind}")
+
+    def check(cases, how):
+        for _, (pd, like, exact, scale, what) in cases:
+            got = O.to_float64(gpu.fetch(pd, like.storage), dtype)
+            G.assert_close_to_wide(got, exact, scale + (final / tol) * np.abs(exact) + 1e-30, tol, f"column sums of several items, {how}: {what}")
+
+    together = [case([8192, 768], [768], 0.0), case([2, 4], [1, 4], 3.0), case([700, 260], [260], -1.5), case([3, 50, 1024], [1024], 0.0),
+                case([16, 31, 8], [1, 1, 8], 0.25), case([4099, 12], [12], 0.0)]
+    G.run_gpu(gpu, "aixk_sum_columns_many", _colsum_items([c[0] for c in together]), len(together))
+    check(together, "together")
+    mixed = [case([64, 512], [512], 0.0), case([40, 64], [40, 1], 1.0), case([48, 8], [8], 0.0, "transposed"), case([50, 30], [30], 2.0), case([1, 16], [16], 0.0)]
+    G.run_gpu(gpu, "aixk_sum_columns_many", _colsum_items([c[0] for c in mixed]), len(mixed))
+    check(mixed, "item by item")
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    assert lib.aixk_sum_columns_many(h, None, 0) == 0
+    bad_src, bad_dst, _ = together[0][0]
+    wrong = K.Tensor.from_buffer_copy(bad_dst)
+    wrong.dtype = O.I32
+    assert lib.aixk_sum_columns_many(h, _colsum_items([together[1][0], (bad_src, wrong, 0)]), 2) == 1      # element types must agree
     gpu.ctx.sync()
     gpu.release()

@@ -905,3 +905,67 @@ def test_runs_of_equal_flat_kernels_leave_as_one_launch(dev):
         assert CPU.copy(s.storage.ctypes.data, O.F32, want.ctypes.data, O.BF16, s.size) == 0
         T.assert_same_bits(g, want, f"f32 -> bf16 over {s.size} elements, batched")
     dev.release()
+
+
+def test_runs_of_column_sums_leave_as_one_launch(dev):
+    """The gradients of biases, layer after layer (aixCore.hpp:2228-2233 sums a gradient to its parameter's shape): reduceTo
+    calls down the columns of a dense matrix whose destination's fill was folded in wait and leave together; a source that
+    a recorded operator produces, a recorded operator that reads a sum while it waits, a freed source and a second sum
+    into the same destination keep their meaning.  Against the oracle's sums in wide arithmetic: 1e-5 of the sum of the
+    terms' magnitudes plus one bf16 rounding (2^-8)."""
+    set_diag(dev)
+    rng = np.random.default_rng(45000)
+    dtype = O.BF16
+    shape, dshape = [512, 128], [128]
+    zero = np.zeros(1, np.float32)
+
+    def close(got_storage, exact, scale, what):
+        got = O.to_float64(got_storage, dtype).reshape(-1)
+        bound = 1e-5 * np.asarray(scale) + 2.0 ** -8 * np.abs(exact) + 1e-30
+        bad = np.flatnonzero(~(np.abs(got - exact) <= bound))
+        assert bad.size == 0, f"{what}: {bad.size} of {got.size} beyond the bound; first at {bad[0]}: got {got[bad[0]]!r} exact {exact[bad[0]]!r}"
+
+    def colsum_of(src_host, src_desc):
+        filled = T.empty(dtype, dshape)
+        assert CPU.fill(zero.ctypes.data, O.F32, C.byref(filled.desc())) == 0
+        exact = filled.values().reshape(-1).copy()
+        scale = np.abs(exact)
+        assert CPU.reduce_to_wide(C.byref(src_host.desc()), C.byref(filled.desc()), exact.ctypes.data, scale.ctypes.data) == 0
+        assert CPU.reduce_to(C.byref(src_host.desc()), C.byref(filled.desc())) == 0
+        ps = dev.raw(filled.storage.nbytes)
+        dd = H.kdesc(filled, ps)
+        dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(dd))
+        dev.dev.call("reduce_to", H.ref(src_desc), H.ref(dd))
+        return {"host": filled, "ptr": ps, "desc": dd, "exact": exact, "scale": scale}
+
+    srcs = [T.contiguous_tensor(rng, dtype, shape, lo=-1, hi=1) for _ in range(6)]
+    ups = [dev.put(x) for x in srcs]
+    dev.dev.synchronize()
+    before = dev.dev.batched_launch_stats()
+    sums = [colsum_of(x, d) for x, (_, d) in zip(srcs, ups)]
+    dev.free(ups[5][0])                                              # its owner is done with a source while the sum still waits
+    spare = [dev.raw(srcs[5].storage.nbytes) for _ in range(3)]      # must not be handed the freed block
+    assert all(p != ups[5][0] for p in spare)
+    got = [dev.fetch(s["ptr"], s["host"].storage) for s in sums]
+    after = dev.dev.batched_launch_stats()
+    assert after[0] - before[0] == 1 and after[1] - before[1] == len(srcs), (before, after)
+    for g, s in zip(got, sums):
+        close(g, s["exact"], s["scale"], "six column sums in one pair of launches")
+    # a source that is a recorded sum; a recorded addition that reads two sums while they wait
+    rec = Recorder(dev, dtype, shape)
+    x, y = rec.leaf(srcs[0]), rec.leaf(srcs[1])
+    total = rec.binary(O.ADD, x, y)
+    a = colsum_of(total["host"], total["desc"])
+    b = colsum_of(x["host"], x["desc"])
+    small = Recorder(dev, dtype, dshape)
+    both = small.binary(O.ADD, a, b)
+    # oracle-side values of a and b are the oracle's own sums; allow both sums' bounds plus the addition's rounding
+    exact = a["exact"] + b["exact"]
+    close(dev.fetch(both["ptr"], both["host"].storage), exact, a["scale"] + b["scale"] + (2.0 ** -8 / 1e-5) * (np.abs(a["exact"]) + np.abs(b["exact"])), "sum of two waiting column sums")
+    close(dev.fetch(a["ptr"], a["host"].storage), a["exact"], a["scale"], "column sums of a recorded sum")
+    # a second sum into a destination that a waiting sum writes: the first goes out first
+    dev.dev.call("fill", zero.ctypes.data, O.F32, H.ref(b["desc"]))
+    dev.dev.call("reduce_to", H.ref(y["desc"]), H.ref(b["desc"]))
+    c = colsum_of(y["host"], y["desc"])
+    close(dev.fetch(b["ptr"], b["host"].storage), c["exact"], c["scale"], "a destination summed into twice")
+    dev.release()
