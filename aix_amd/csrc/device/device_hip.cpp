@@ -490,26 +490,30 @@ void DeviceHIP::flushWindow(bool final)
     releaseLimbo();
 }
 
-void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
+void DeviceHIP::flushFor(const void* a, const void* b, const void* c) { flushForOperands(a, b, c, false); }
+
+// An operator is about to be enqueued at once on these operands -- the last one named is the one it writes (or the only
+// one, which it may write), the others are read.  Recorded operators go first only if one of them writes what it reads
+// or uses what it writes (`always`: whatever they touch), and so do the calls that wait; all others may as well run after
+// it, which keeps the window -- and the kernels fused from it -- whole.
+void DeviceHIP::flushForOperands(const void* a, const void* b, const void* c, bool always)
 {
     AIXHIP_TRACE("-- operator outside the planner (%zu recorded)", m_engine->pendingOps());
+    const void* named[3] = {a, b, c};
     const void* bases[3] = {nullptr, nullptr, nullptr};
-    size_t i = 0;
-    for (const void* p : {a, b, c}) {
-        const size_t at = i++;
+    const int last = c ? 2 : b ? 1 : 0;
+    bool dependent = always;
+    for (int k = 0; k < 3; ++k) {
+        const void* p = named[k];
         if (!p) continue;
-        m_engine->recordExternalRead(p);
         const void* base = m_blocks.baseOf(p);              // an operand may point into the middle of a block
-        if (base && base != p) { m_engine->recordExternalRead(base); bases[at] = base; }
+        if (base && base != p) { bases[k] = base; dependent = true; }
+        if (!dependent) dependent = k == last ? m_engine->pendingTouches(p) : m_engine->pendingWrites(p);
     }
     markTouched(a);                                         // the caller is about to enqueue work on them
     markTouched(b);
     markTouched(c);
-    // calls that wait and have nothing to do with these operands go on waiting: the last operand named is the one the
-    // caller writes (or the only one, which it may write), the others are read
     auto& ex = *m_extras;
-    const int last = c ? 2 : b ? 1 : 0;
-    const void* named[3] = {a, b, c};
     auto meets = [&] {
         for (int k = 0; k < 3; ++k) {
             if (k == last ? ex.waitingUses(named[k]) || ex.waitingUses(bases[k]) : ex.waitingWrites(named[k]) || ex.waitingWrites(bases[k])) return true;
@@ -517,6 +521,11 @@ void DeviceHIP::flushFor(const void* a, const void* b, const void* c)
         return false;
     };
     if (meets()) issuePending();
+    if (!dependent) return;
+    for (int k = 0; k < 3; ++k) {
+        if (named[k]) m_engine->recordExternalRead(named[k]);
+        if (bases[k]) m_engine->recordExternalRead(bases[k]);
+    }
     flushWindow(false);
     if (meets()) issuePending();                            // (a one-hot replayed on its own has just begun to wait)
 }
@@ -528,7 +537,7 @@ bool DeviceHIP::fenceInterior(const void* a, const void* b, const void* c)
 {
     bool any = false;
     for (const void* p : {a, b, c}) if (p && !m_blocks.find(p) && m_blocks.baseOf(p)) any = true;
-    if (any) flushFor(a, b, c);
+    if (any) flushForOperands(a, b, c, true);
     return any;
 }
 
@@ -639,7 +648,7 @@ void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const Device
     }
     const bool fenced = fenceInterior(va.data, vb.data, out.data);
     m_engine->record(t, va, vb, out);
-    if (fenced) flushFor(out.data);                         // (names the result: somebody may read it through the block's start)
+    if (fenced) flushForOperands(out.data, nullptr, nullptr, true);                         // (names the result: somebody may read it through the block's start)
 }
 
 void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op)
@@ -663,7 +672,7 @@ void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceT
     }
     const bool fenced = fenceInterior(va.data, out.data);
     m_engine->record(t, va, out);
-    if (fenced) flushFor(out.data);
+    if (fenced) flushForOperands(out.data, nullptr, nullptr, true);
 }
 
 void DeviceHIP::add(const DeviceTensorParams& a1, const DeviceTensorParams& a2, const DeviceTensorParams& result) { recordBinary(OpType::Add, a1, a2, result, "add"); }
@@ -686,7 +695,7 @@ void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTenso
     out.makeDense();
     const bool fenced = fenceInterior(out.data);
     m_engine->recordFill(scalar, scalarDType, out);
-    if (fenced) flushFor(out.data);
+    if (fenced) flushForOperands(out.data, nullptr, nullptr, true);
 }
 
 void DeviceHIP::fillMin(const DeviceTensorParams& result)
@@ -696,7 +705,7 @@ void DeviceHIP::fillMin(const DeviceTensorParams& result)
     out.makeDense();
     const bool fenced = fenceInterior(out.data);
     m_engine->recordFillMin(out);
-    if (fenced) flushFor(out.data);
+    if (fenced) flushForOperands(out.data, nullptr, nullptr, true);
 }
 
 // ---- planner callbacks -------------------------------------------------------------------------

@@ -159,6 +159,7 @@ private:
     bool recordTri(aixhip::fuse::OpType t, const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal);
     bool takeInit(const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t* bits);
     void flushFor(const void* a = nullptr, const void* b = nullptr, const void* c = nullptr);
+    void flushForOperands(const void* a, const void* b, const void* c, bool always);
     void flushWindow(bool final);
     bool fenceInterior(const void* a, const void* b = nullptr, const void* c = nullptr);   // true: flush again once the operator is recorded
     void emitFused(const aixhip::fuse::FusedSubgraphDescriptor& d);

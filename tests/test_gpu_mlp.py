@@ -85,8 +85,11 @@ def test_full_size_mlp_against_the_committed_cpu_trace(dev):
     updates have the size of the learning rate whatever the gradient's size (m / sqrt(v) = +-1 after one step), so a
     gradient entry near zero whose sign differs by rounding moves its weight by twice the learning rate: with 6 million
     weights the loss of the next steps differs at the 1e-5 level (observed 1.0e-5 at step 2), not at that of the
-    arithmetic.  Whole trace: the envelope the fixture itself measures -- 20 x the deviation of the CPU's own run with
-    1 % of W2 moved by one unit in the last place (never more than 0.1)."""
+    arithmetic.  Whole trace, step by step: three times the largest deviation that the CPU's own run with 1 % of W2 moved
+    by one unit in the last place has shown up to two steps later (at least 1e-4).  That run leaves the fixture the way the
+    GPU's does -- 1e-4 by step 11, 1e-3 by step 16, 0.108 at the bump of the loss around step 65 -- so the bound is tight
+    where the arithmetic shows (observed: at most 0.7 of it, at step 7) and follows the CPU's own sensitivity where the
+    trajectory, not the arithmetic, decides (the order in which a column sum adds its rows moves step 65 from 0.086 to 0.123)."""
     import json
     import os
     from aix_amd import drivers as GD
@@ -97,16 +100,19 @@ def test_full_size_mlp_against_the_committed_cpu_trace(dev):
     want = np.frombuffer(bytes.fromhex("".join(fixture["losses_hex"])), dtype=np.float32).astype(np.float64)
     assert np.array_equal(want, np.array(fixture["losses"]))
     other = np.array(fixture["losses_one_ulp_perturbed"])
-    spread = float((np.abs(other - want) / np.abs(want)).max())
-    tol = min(0.1, max(1e-3, 20 * spread))
+    own = np.abs(other - want) / np.abs(want)
+    spread = float(own.max())
+    so_far = np.maximum.accumulate(own)
+    tol = np.maximum(1e-4, 3 * so_far[np.minimum(np.arange(own.size) + 2, own.size - 1)])
     data = OD.mlp_data(batch, n_in, hidden, n_out)
     got, secs = GD.mlp(dev, batch, n_in, hidden, n_out, fixture["steps"], fixture["lr"], data)
     rel = np.abs(got.astype(np.float64) - want) / np.abs(want)
     print(f"full-size MLP x100: loss {want[0]:.6f} -> {want[-1]:.6f} (cpu fixture), {got[-1]:.6f} (gpu); max rel dev {rel.max():.3e} at step "
-          f"{int(rel.argmax())}; first 5 steps {rel[:5].max():.3e}; CPU's own one-ulp spread {spread:.3e} -> tolerance {tol:.3e}; "
+          f"{int(rel.argmax())}; first 5 steps {rel[:5].max():.3e}; CPU's own one-ulp spread {spread:.3e}; largest share of the step's bound {(rel / tol).max():.2f} at step {int((rel / tol).argmax())}; "
           f"gpu {np.median(secs[1:]) * 1e3:.2f} ms/step against {fixture['cpu_seconds_per_step']:.1f} s/step on {fixture['threads']} CPU threads")
     print("relative deviation per step:", " ".join(f"{v:.1e}" for v in rel))
     assert np.all(np.isfinite(got)) and got[-1] < got[0]
     assert rel[0] <= 1e-5, "first forward pass"
     assert rel[:5].max() <= 1e-4, "first 5 steps"
-    assert rel.max() <= tol
+    assert np.all(rel <= tol), f"steps beyond their bound: {np.flatnonzero(rel > tol).tolist()}"
+    assert rel.max() <= 3 * spread
