@@ -978,3 +978,37 @@ def test_runs_of_column_sums_leave_as_one_launch(dev):
     c = colsum_of(y["host"], y["desc"])
     close(dev.fetch(b["ptr"], b["host"].storage), c["exact"], c["scale"], "a destination summed into twice")
     dev.release()
+
+
+def test_operators_at_once_leave_an_unrelated_window_alone(dev):
+    """An operator that is enqueued at once (a transpose, a large matmul) goes ahead of the recorded operators when none of
+    them writes what it reads or uses what it writes: the window stays whole and what it holds fuses across the call.  One
+    that reads a recorded result flushes first.  Results against the oracle, bit for bit (add, multiply, transpose)."""
+    set_diag(dev)
+    rng = np.random.default_rng(46000)
+    shape = [96, 40]
+    rec = Recorder(dev, O.F32, shape)
+    x, y = rec.leaf(T.contiguous_tensor(rng, O.F32, shape)), rec.leaf(T.contiguous_tensor(rng, O.F32, shape))
+    other = T.contiguous_tensor(rng, O.F32, shape)
+    _, dother = dev.put(other)
+    dev.dev.synchronize()
+
+    def transposed(src_host, src_desc):
+        want = T.empty(O.F32, shape[::-1])
+        assert CPU.transpose(C.byref(src_host.desc()), C.byref(want.desc()), 0, 1) == 0
+        pt = dev.raw(want.storage.nbytes)
+        dev.dev.call("transpose", H.ref(src_desc), H.ref(H.kdesc(want, pt)), 0, 1)
+        return pt, want
+
+    total = rec.binary(O.ADD, x, y)
+    pt, want_t = transposed(other, dother)                                   # nothing recorded touches its operands
+    prod = rec.binary(O.MUL, total, x)
+    got = dev.fetch(prod["ptr"], prod["host"].storage)
+    diag = dev.dev.diagnostics()
+    assert diag.ops_recorded == 2 and diag.fusible_subgraphs == 1 and diag.fallback_ops == 0, diag.subgraph_summary
+    T.assert_same_bits(got, prod["host"].storage, "(x + y) * x around an unrelated transpose")
+    T.assert_same_bits(dev.fetch(pt, want_t.storage), want_t.storage, "the transpose")
+    again = rec.binary(O.ADD, prod, y)
+    pt2, want_t2 = transposed(again["host"], again["desc"])                  # reads a recorded result: the window goes first
+    T.assert_same_bits(dev.fetch(pt2, want_t2.storage), want_t2.storage, "transpose of a recorded sum")
+    dev.release()
