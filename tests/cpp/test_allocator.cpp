@@ -258,8 +258,17 @@ static void planner_traffic(unsigned seed, int rounds)
             for (int k = 0; k < 4; ++k) dev.unary(tensor(full[rng() % full.size()], {n}), tensor(fresh_full(), {n}));
         } else if (what < 76) {                                        // an operand inside a block
             dev.unary(tensor((char*)x + 64 * 4, {len}), tensor(fresh_full(), {len}));
-        } else if (what < 79) {                                        // an operator that runs at once
+        } else if (what < 78) {                                        // an operator that runs at once
             dev.transpose(tensor(x, {rows, len}), tensor(fresh_full(), {len, rows}), 0, 1);
+        } else if (what < 79) {                                        // column sums that wait; one source dies while its sum still waits
+            void* t = dev.allocate(n * 4);
+            dev.unary(tensor(x, {rows, len}), tensor(t, {rows, len}));
+            for (void* src : {t, x}) {
+                void* c = fresh_full();                                // (the sum is the block's first row)
+                dev.fill(&zero, DataType::kFloat32, tensor(c, {len}));
+                dev.reduceTo(tensor(src, {rows, len}), tensor(c, {len}));
+            }
+            dev.deallocate(t);
         } else if (what < 82) {                                        // a cat: row blocks of a fresh tensor, the sources may die at once
             void* whole = fresh_full();
             for (size_t k = 0; k < 4; ++k) {
