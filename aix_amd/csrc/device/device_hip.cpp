@@ -480,7 +480,7 @@ void DeviceHIP::flush() { flushWindow(true); }
 // final: nothing recorded stays behind.  Otherwise fills that nothing recorded so far uses may wait (FuseEngine::flush).
 void DeviceHIP::flushWindow(bool final)
 {
-    // Calls that wait (small products, sliceSet, one-hot masks) stay waiting across a flush: they depend on nothing
+    // Calls that wait (small products, sliceSet, one-hot masks, column sums) stay waiting across a flush: they depend on nothing
     // recorded (their callers saw to that), and a kernel that leaves now and uses what they write, or writes what they
     // use, sends them off first (emitFused, emitSingle).
     if (final) issuePending();
