@@ -128,13 +128,15 @@ struct DeviceHIP::Extras {
     std::vector<aixk_argmax_item> onehots;
     // reduceTo calls that sum a matrix down its columns (see DeviceHIP::reduceTo): f32, f16 and bf16 wait apart
     std::array<std::vector<aixk_colsum_item>, 3> colsums;
+    // second halves of sums over everything (see DeviceHIP::emitFused): one element type at a time
+    std::vector<aixk_partials_item> partialSums;
     // what the waiting calls of all three kinds read and write (block starts), so that a new call knows in one lookup
     // whether it may wait beside them; per destination of waiting sliceSet calls, how it was described and the windows
     // written so far
     aixhip::fuse::PointerSet waitReads, waitWrites;
     struct SliceWindows { aixhip_tensor dst; uint64_t dim; std::vector<std::pair<uint64_t, uint64_t>> ranges; };
     std::unordered_map<const void*, SliceWindows> sliceDsts;
-    bool anyPending() const { if (!slices.empty() || !onehots.empty()) return true; for (const auto& c : colsums) if (!c.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
+    bool anyPending() const { if (!slices.empty() || !onehots.empty() || !partialSums.empty()) return true; for (const auto& c : colsums) if (!c.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
     // a call that reads r0, r1 and writes w neither uses what waits nor is used by it
     bool apartFromWaiting(const void* r0, const void* r1, const void* w) const
     {
@@ -943,7 +945,15 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
     for (size_t k = 0; k < nWholes; ++k) {
         aixhip_tensor dst;
         toPod(d.outputBuffers[wholes[k].output], &dst);
-        check(aixk_sum_partials(m_ctx, wholes[k].scratch, grid, &dst, wholes[k].init));
+        if (!ex.batchFlatKernels) { check(aixk_sum_partials(m_ctx, wholes[k].scratch, grid, &dst, wholes[k].init)); continue; }
+        // the second half waits like a small product: the scalar gradients of a backward pass are read when it reaches
+        // its leaves, and leave together then (the partial sums' block stays in limbo until they have: releaseLimbo)
+        if (ex.partialSums.size() >= AIXK_PARTIALS_ITEMS_MAX || (!ex.partialSums.empty() && ex.partialSums[0].dst.dtype != dst.dtype) ||
+            !ex.apartFromWaiting(wholes[k].scratch, nullptr, dst.data))
+            issuePending();
+        ex.partialSums.push_back(aixk_partials_item{wholes[k].scratch, grid, dst, wholes[k].init});
+        ex.noteWaiting(wholes[k].scratch, nullptr, dst.data);
+        markTouched(dst.data);
     }
 }
 
@@ -1158,7 +1168,8 @@ void DeviceHIP::issuePending()
         size_t products = 0, sums = 0;
         for (const auto& g : ex.groups) products += g.out.size();
         for (const auto& c : ex.colsums) sums += c.size();
-        AIXHIP_TRACE("-- what waited leaves: %zu sliceSet, %zu argmaxIndicesTo, %zu reduceTo, %zu matmul", ex.slices.size(), ex.onehots.size(), sums, products);
+        AIXHIP_TRACE("-- what waited leaves: %zu sliceSet, %zu argmaxIndicesTo, %zu reduceTo, %zu sums of partials, %zu matmul", ex.slices.size(), ex.onehots.size(), sums,
+                     ex.partialSums.size(), products);
         (void)products; (void)sums;
     }
     if (!ex.slices.empty()) {
@@ -1173,6 +1184,14 @@ void DeviceHIP::issuePending()
                                             : aixk_argmax_onehot_many(m_ctx, ex.onehots.data(), (uint32_t)ex.onehots.size());
         if (ex.onehots.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.onehots.size(); }
         ex.onehots.clear();
+    }
+    if (!ex.partialSums.empty()) {
+        auto& sums = ex.partialSums;
+        if (status == AIXK_OK)
+            status = sums.size() == 1 ? aixk_sum_partials(m_ctx, sums[0].partials, sums[0].count, &sums[0].dst, sums[0].init_bits)
+                                      : aixk_sum_partials_many(m_ctx, sums.data(), (uint32_t)sums.size());
+        if (sums.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += sums.size(); }
+        sums.clear();
     }
     for (auto& sums : ex.colsums) {
         if (sums.empty()) continue;

@@ -280,6 +280,35 @@ __global__ __launch_bounds__(kBlock) void sum_partials_k(const typename traits<T
     }
 }
 
+// The same for several sums in one launch (the scalar gradients of a backward pass, which wait for each other): workgroup
+// k lands item k.
+struct PartialsItem { u64 partials, dst, init; u32 count, pad; };
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void sum_partials_many_k(const PartialsItem* __restrict__ items)
+{
+    typedef SumOp<T> Op;
+    typedef typename Op::Acc Acc;
+    __shared__ Acc smem[kWaves];
+    const PartialsItem it = items[blockIdx.x];
+    const Acc* partials = global_ptr<const Acc>(it.partials);
+    Acc a = Op::init();
+    constexpr unsigned U = 8;
+    for (unsigned i0 = threadIdx.x; i0 < it.count; i0 += kBlock * U) {
+        Acc r[U];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < it.count) r[k] = partials[i0 + k * kBlock];
+#pragma unroll
+        for (unsigned k = 0; k < U; ++k) if (i0 + k * kBlock < it.count) a = Op::combine(a, r[k]);
+    }
+    a = block_reduce<Op>(a, smem);
+    if (threadIdx.x == 0) {
+        T init;
+        __builtin_memcpy(&init, &it.init, sizeof(T));
+        *global_ptr<T>(it.dst) = down<T>(up(init) + a);
+    }
+}
+
 // ---- per-slot plans ------------------------------------------------------------------------------
 // Kept dims address the destination slot, reduced dims are folded away.  All extents/strides are
 // those of the jointly collapsed (src strides, dst weights) space; `flat` strides are the
@@ -1323,6 +1352,42 @@ int32_t aixk_sum_partials(aixk_ctx* ctx, const void* partials, uint64_t count, c
         if constexpr (std::is_same<T, double>::value || std::is_same<T, float>::value || std::is_same<T, f16>::value || std::is_same<T, bf16>::value) {
             hipLaunchKernelGGL((sum_partials_k<T>), dim3(1), dim3(kBlock), 0, ctx->stream, (const typename traits<T>::W*)partials, (unsigned)count,
                                (T*)dst->data + dst->offset, (u64)init_bits);
+            AIXK_HIP(hipGetLastError());
+        }
+        return (int)AIXK_OK;
+    });
+}
+
+int32_t aixk_sum_partials_many(aixk_ctx* ctx, const aixk_partials_item* items, uint32_t count)
+{
+    AIXK_TRY(set_device(ctx));
+    if (count == 0) return AIXK_OK;
+    AIXK_REQUIRE(items, "sums of partials: no items");
+    const int dtype = items[0].dst.dtype;
+    bool together = count >= 2 && count <= AIXK_PARTIALS_ITEMS_MAX && (dtype == AIXK_F64 || dtype == AIXK_F32 || dtype == AIXK_F16 || dtype == AIXK_BF16);
+    for (uint32_t k = 0; k < count && together; ++k)
+        together = valid_tensor(&items[k].dst) && items[k].dst.data && items[k].dst.size == 1 && items[k].dst.dtype == dtype && items[k].partials &&
+                   items[k].count > 0 && items[k].count < (1ull << 31);
+    if (!together) {
+        for (uint32_t k = 0; k < count; ++k) AIXK_TRY(aixk_sum_partials(ctx, items[k].partials, items[k].count, &items[k].dst, items[k].init_bits));
+        return AIXK_OK;
+    }
+    const size_t table_bytes = (size_t)count * sizeof(PartialsItem), esz = aixk_dtype_size(dtype);
+    PartialsItem* host = nullptr;
+    const PartialsItem* dev = nullptr;
+    AIXK_TRY(table_slot(ctx, table_bytes, (void**)&host, (const void**)&dev));
+    for (uint32_t k = 0; k < count; ++k) {
+        host[k].partials = (u64)(uintptr_t)items[k].partials;
+        host[k].dst = (u64)(uintptr_t)((char*)items[k].dst.data + items[k].dst.offset * esz);
+        host[k].init = items[k].init_bits;
+        host[k].count = (u32)items[k].count;
+        host[k].pad = 0;
+    }
+    AIXK_TRY(table_upload(ctx, host, dev, table_bytes));
+    return by_dtype(dtype, [&](auto tag) {
+        typedef decltype(tag) T;
+        if constexpr (std::is_same<T, double>::value || std::is_same<T, float>::value || std::is_same<T, f16>::value || std::is_same<T, bf16>::value) {
+            hipLaunchKernelGGL((sum_partials_many_k<T>), dim3(count), dim3(kBlock), 0, ctx->stream, dev);
             AIXK_HIP(hipGetLastError());
         }
         return (int)AIXK_OK;

@@ -39,6 +39,11 @@ class ColsumItem(C.Structure):
     _fields_ = [("src", Tensor), ("dst", Tensor), ("init_bits", C.c_uint64)]
 
 
+class PartialsItem(C.Structure):
+    """aixk_partials_item"""
+    _fields_ = [("partials", C.c_void_p), ("count", C.c_uint64), ("dst", Tensor), ("init_bits", C.c_uint64)]
+
+
 class DeviceInfo(C.Structure):
     _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
                 ("clock_khz", C.c_int32), ("large_bar", C.c_int32), ("wavefront", C.c_int32),
@@ -83,6 +88,7 @@ _SIGNATURES = {
     "aixk_reduce_to": [_P, C.c_int, _T, _T],
     "aixk_reduce_to_init": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_sum_partials": [_P, _P, C.c_uint64, _T, C.c_uint64],
+    "aixk_sum_partials_many": [_P, _P, C.c_uint32],
     "aixk_argmax_to": [_P, C.c_int, _T, _T, C.c_uint64],
     "aixk_argmax_onehot_many": [_P, _P, C.c_uint32],
     "aixk_sum_columns_many": [_P, _P, C.c_uint32],

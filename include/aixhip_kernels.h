@@ -165,6 +165,13 @@ int32_t aixk_reduce_to_init(aixk_ctx* ctx, int kind, const aixhip_tensor* src, c
  * receives round(init + their sum), init being the value the destination was filled with (its bits in the low bytes of
  * init_bits), as aixk_reduce_to_init lands a sum.  No counterpart in the reference's interface. */
 int32_t aixk_sum_partials(aixk_ctx* ctx, const void* partials, uint64_t count, const aixhip_tensor* dst, uint64_t init_bits);
+/* `count` calls of aixk_sum_partials in one launch (item k is aixk_sum_partials(ctx, partials, count, dst, init_bits) of its
+ * fields) when all destinations have one floating-point element type and there are at most AIXK_PARTIALS_ITEMS_MAX items,
+ * otherwise item by item in order.  The caller guarantees that no item reads what another one writes.  No counterpart in
+ * the reference's interface. */
+#define AIXK_PARTIALS_ITEMS_MAX 1024
+typedef struct aixk_partials_item { const void* partials; uint64_t count; aixhip_tensor dst; uint64_t init_bits; } aixk_partials_item;
+int32_t aixk_sum_partials_many(aixk_ctx* ctx, const aixk_partials_item* items, uint32_t count);
 /* Device::argmaxTo / argmaxIndicesTo (aixDeviceCPU.cpp:275-298, 320-360). onehot=1 scatters ones
  * into the pre-zeroed int32 dst of src's shape; onehot=2 also zeroes dst first (the fill(0) the
  * caller issues before argmaxIndicesTo, aixCore.hpp:927-941, folded in: over a handful of rows the

@@ -91,6 +91,7 @@ STUB_OP(aixk_argmax_to, int, const aixhip_tensor*, const aixhip_tensor*, uint64_
 STUB_OP(aixk_argmax_onehot_many, const aixk_argmax_item*, uint32_t)
 STUB_OP(aixk_sum_columns_many, const aixk_colsum_item*, uint32_t)
 STUB_OP(aixk_sum_partials, const void*, uint64_t, const aixhip_tensor*, uint64_t)
+STUB_OP(aixk_sum_partials_many, const aixk_partials_item*, uint32_t)
 int32_t aixk_matmul(aixk_ctx* c, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
 {
     if (g_fail_matmuls > 0) { --g_fail_matmuls; std::snprintf(g_error, sizeof(g_error), "stub: matmul workspace"); return AIXK_ENOMEM; }

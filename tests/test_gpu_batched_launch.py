@@ -2,7 +2,8 @@
 (small fills, each item a pattern already in its destination's element type), aixk_rtc_launch_many (several argument
 blocks of one runtime-compiled kernel, each with its share of the grid), aixk_slice_set_many (several sliceSet calls) and
 aixk_argmax_onehot_many (several argmaxIndicesTo calls with their zero fill) and aixk_sum_columns_many (several reduceTo
-calls down the columns of a matrix, with the fill of their destination).
+calls down the columns of a matrix, with the fill of their destination) and aixk_sum_partials_many (the second halves of
+several sums over everything).
 Results against numpy (fills and an exact elementwise body) and the CPU oracle's sliceSet, sizes down to one element and
 ragged tails, and the argument checks they promise."""
 import ctypes as C
@@ -300,5 +301,54 @@ def test_sum_columns_many_is_fill_and_reduce_to_item_by_item(gpu, dtype):
     wrong = K.Tensor.from_buffer_copy(bad_dst)
     wrong.dtype = O.I32
     assert lib.aixk_sum_columns_many(h, _colsum_items([together[1][0], (bad_src, wrong, 0)]), 2) == 1      # element types must agree
+    gpu.ctx.sync()
+    gpu.release()
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F32, O.F16, O.F64], ids=["bf16", "f32", "f16", "f64"])
+def test_sum_partials_many_lands_every_sum(gpu, dtype):
+    """Item k is aixk_sum_partials of its fields: dst = init + the sum of `count` partial sums (f32; f64 for f64), rounded
+    once.  One launch for destinations of one element type, item by item for a mixed set.  Against numpy's float64 sum:
+    1e-5 of the sum of magnitudes (1e-12 for f64) plus one rounding of the result."""
+    rng = np.random.default_rng(57000 + dtype)
+    bounds = {O.F64: (1e-12, 0.0), O.F32: (1e-5, 0.0), O.F16: (1e-5, 2.0 ** -10), O.BF16: (1e-5, 2.0 ** -8)}
+
+    def case(count, init_value, dt=dtype):
+        parts = rng.uniform(-1, 1, count).astype(np.float64 if dt == O.F64 else np.float32)
+        pp = gpu.raw(parts.nbytes)
+        gpu.ctx.upload(pp, parts)
+        init_arr = O.to_storage(np.array([init_value]), dt)
+        bits = int.from_bytes(init_arr.tobytes()[:O.ITEMSIZE[dt]], "little")
+        garbage = T.HostTensor(O.to_storage(np.array([777.0]), dt).copy(), dt, [])
+        pd, dd = gpu.put(garbage)
+        init_exact = float(O.to_float64(init_arr, dt)[0])
+        exact = init_exact + float(np.sum(parts.astype(np.float64)))
+        scale = abs(init_exact) + float(np.sum(np.abs(parts.astype(np.float64))))
+        return (pp, count, dd, bits), (pd, garbage, dt, exact, scale, f"{count} partials, init {init_value}")
+
+    def items_of(cases):
+        arr = (K.PartialsItem * len(cases))()
+        for k, ((pp, count, dd, bits), _) in enumerate(cases):
+            arr[k].partials, arr[k].count, arr[k].dst, arr[k].init_bits = pp, count, dd, bits
+        return arr
+
+    def check(cases, how):
+        for _, (pd, like, dt, exact, scale, what) in cases:
+            got = float(O.to_float64(gpu.fetch(pd, like.storage), dt)[0])
+            t, f = bounds[dt]
+            assert abs(got - exact) <= t * scale + f * abs(exact) + 1e-30, f"sums of partials, {how}: {what}: got {got!r}, exact {exact!r}"
+
+    together = [case(1, 0.0), case(7, 3.0), case(256, -1.5), case(2049, 0.0), case(100000, 0.25)]
+    G.run_gpu(gpu, "aixk_sum_partials_many", items_of(together), len(together))
+    check(together, "one launch")
+    if dtype != O.F64:
+        mixed = [case(300, 1.0), case(5, 0.0, O.F32 if dtype != O.F32 else O.BF16), case(4097, 2.0)]
+        G.run_gpu(gpu, "aixk_sum_partials_many", items_of(mixed), len(mixed))
+        check(mixed, "item by item")
+    lib, h = gpu.ctx.lib, gpu.ctx.handle
+    assert lib.aixk_sum_partials_many(h, None, 0) == 0
+    bad = items_of(together[:2])
+    bad[1].count = 0
+    assert lib.aixk_sum_partials_many(h, bad, 2) == 1                    # an item without partials is refused (by the single call)
     gpu.ctx.sync()
     gpu.release()
