@@ -1122,6 +1122,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             if (m_engine->pendingWrites(a.data) || m_engine->pendingWrites(b.data) || m_engine->pendingTouches(result.data)) {
                 m_engine->recordExternalRead(a.data);
                 m_engine->recordExternalRead(b.data);
+                m_engine->recordExternalRead(result.data);      // a fill of the result that nobody has read yet must not be set aside and land behind the product
                 flushWindow(false);
             }
             aixhip_tensor pa, pb, pr; toPod(a, &pa, "matmul"); toPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
@@ -1349,6 +1350,7 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
         src.size >= 2 * dst.size && src.offset % 4 == 0 && findBlock(src.data) && findBlock(dst.data) && src.data != dst.data) {
         if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {          // recorded producers and users go first
             m_engine->recordExternalRead(src.data);
+            m_engine->recordExternalRead(dst.data);             // (a fill of the destination still recorded goes first, it does not wait)
             flushWindow(false);
         }
         auto& sums = ex.colsums[slot];
@@ -1422,6 +1424,7 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
         dim + 1 == src.shape.size() && src.shape.size() <= AIXK_MAX_RANK) {
         if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {          // recorded producers and users go first
             m_engine->recordExternalRead(src.data);
+            m_engine->recordExternalRead(dst.data);             // (a fill of the destination still recorded goes first, it does not wait)
             flushWindow(false);
         }
         if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.apartFromWaiting(src.data, nullptr, dst.data)) issuePending();
@@ -1472,6 +1475,7 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
         if (window == src.size && whole == src.size && start + (count - 1) * step < dst.shape[dim]) {
             if (m_engine->pendingWrites(src.data) || m_engine->pendingTouches(dst.data)) {      // recorded producers and users go first
                 m_engine->recordExternalRead(src.data);
+                m_engine->recordExternalRead(dst.data);         // (a fill of the destination that could not be folded in goes first, it does not wait)
                 flushWindow(false);
             }
             bool independent = ex.slices.size() < AIXK_SLICE_ITEMS_MAX &&

@@ -62,6 +62,7 @@ struct aixk_ctx {
     // so the word never has to be cleared.
     unsigned int* counter{nullptr};
     unsigned int gemm_seq{0};
+    int gemm_last_route{0};            // what the last aixk_matmul took: 1 the split-plane f32 route (gemm_x3_k), 0 anything else
     // matmul: K-contiguous copies of operands whose layout the kernels cannot consume in place
     // (0: A, 1: B) and the f32 partial results of K splits (2); grown on demand, ordered on `stream`
     // like everything else

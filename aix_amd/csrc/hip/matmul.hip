@@ -109,6 +109,7 @@ extern "C" int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixh
     if (M == 0 || N == 0) return AIXK_OK;
     if (K == 0) return aixk_zero(ctx, out->data, M * N * aixk_dtype_size(out->dtype));
     AIXK_REQUIRE(out->data != nullptr, "matmul: null result");
+    ctx->gemm_last_route = 0;
 
     if (out->dtype == AIXK_F32 || out->dtype == AIXK_F16 || out->dtype == AIXK_BF16) {
         const int rc = matmul_mfma(ctx, a, b, out);
@@ -124,6 +125,18 @@ extern "C" int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixh
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     });
+}
+
+extern "C" int32_t aixk_matmul_route(aixk_ctx* ctx, int32_t* route, int32_t* redone)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(route && redone, "matmul route: null result");
+    AIXK_HIP(hipStreamSynchronize(ctx->stream));
+    unsigned int flag = 0;
+    AIXK_HIP(hipMemcpy(&flag, ctx->counter, sizeof(flag), hipMemcpyDeviceToHost));
+    *route = ctx->gemm_last_route;
+    *redone = ctx->gemm_last_route == 1 && flag == ctx->gemm_seq;
+    return AIXK_OK;
 }
 
 // out[..., m, n] = a[..., m, k] . b[..., k, n]: one product per index of the leading dims, which a, b and out share

@@ -758,11 +758,27 @@ __global__ __launch_bounds__(256) void splitk_finish_k(const float* __restrict__
 // number into a flag word, and the f32 MFMA kernel that is always launched right behind -- its workgroups return at
 // once unless the flag carries this number -- redoes the whole product with IEEE arithmetic (which also covers sums
 // that overflow on their own: the redo returns the same infinities).
+//
+// The planes also have f32's exponent range only down to where their last bits fall off the bf16 grid: the three planes
+// of x carry its 24 significand bits as multiples of 2^(e - 23), and bf16 ends at 2^-133 (its subnormals, which the
+// matrix unit takes as they are, like f32 subnormals in its products and accumulators), so an operand below 2^-110 is
+// no longer the sum of its planes (2^-116: 1e-5 off, f32 subnormals: all three planes zero).  Every lane therefore
+// follows the smallest nonzero magnitude among the values it splits, and one at or below 2^-100 raises the same flag:
+// the product is redone in IEEE f32 arithmetic, which has no such limit (aixDeviceCPU.cpp:362-389).
+constexpr u32 kX3Smallest = (127u - 100u) << 24;         // (bits << 1) - 1 of 2^-100, exclusive bound
+
 template <bool AT, bool BT> struct TileX3 {
     static constexpr int BM = 128, BN = 128, BK = 32, PA = BM + 32, PB = BN + 32;
     static constexpr int SA = AT ? BK * PA : BM * BK, SB = BT ? BK * PB : BN * BK;       // bf16 elements per plane
     static constexpr size_t kLds = (size_t)3 * (SA + SB) * 2;
 };
+
+__device__ __forceinline__ u32 min3u(u32 a, u32 b, u32 c)
+{
+    u32 r;
+    asm("v_min3_u32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 
 __device__ __forceinline__ u32 cvt_pk_bf16(float lo, float hi)
 {
@@ -771,10 +787,13 @@ __device__ __forceinline__ u32 cvt_pk_bf16(float lo, float hi)
     return r;
 }
 
-// four f32 -> three word pairs of four bf16 (element e in bits 16 (e & 1) of word e / 2)
-__device__ __forceinline__ void split3(const u32x4 x, u32x2& h, u32x2& m, u32x2& l)
+// four f32 -> three word pairs of four bf16 (element e in bits 16 (e & 1) of word e / 2).
+// `least` follows the smallest nonzero magnitude seen: (bits << 1) - 1 drops the sign and sends zeros to the top.
+__device__ __forceinline__ void split3(const u32x4 x, u32x2& h, u32x2& m, u32x2& l, u32& least)
 {
     const u32 xs[4] = {x.x, x.y, x.z, x.w};
+    least = min3u(least, (xs[0] << 1) - 1u, (xs[1] << 1) - 1u);
+    least = min3u(least, (xs[2] << 1) - 1u, (xs[3] << 1) - 1u);
     float r[4];
     u32 hb[4];
 #pragma unroll
@@ -816,6 +835,9 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
+    // smallest nonzero operand magnitude this lane has split (see split3); six vector instructions per four values, 3 % of
+    // the kernel's time at 4096^3 (watching in the first workgroup of every row and column of tiles only gained nothing)
+    u32 least = 0xFFFFFFFFu;
     u32x4 ra[CA], rb[CB];
     auto load_global = [&](u64 k0) {
 #pragma unroll
@@ -837,7 +859,7 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
             const int c = tid + 256 * i;
             const int at = AT ? (c / (BM / 4)) * PA + (c % (BM / 4)) * 4 : kplace(c);
             u32x2 h, m, l;
-            split3(ra[i], h, m, l);
+            split3(ra[i], h, m, l, least);
             *(u32x2*)(As + at) = h; *(u32x2*)(As + SA + at) = m; *(u32x2*)(As + 2 * SA + at) = l;
         }
 #pragma unroll
@@ -845,7 +867,7 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
             const int c = tid + 256 * i;
             const int at = BT ? (c / (BN / 4)) * PB + (c % (BN / 4)) * 4 : kplace(c);
             u32x2 h, m, l;
-            split3(rb[i], h, m, l);
+            split3(rb[i], h, m, l, least);
             *(u32x2*)(Bs + at) = h; *(u32x2*)(Bs + SB + at) = m; *(u32x2*)(Bs + 2 * SB + at) = l;
         }
     };
@@ -905,7 +927,7 @@ __global__ __launch_bounds__(256) void gemm_x3_k(GemmArgs g, SplitArgs sk, u32* 
                 probe = __builtin_fmaf(acc[i][j][v], 0.0f, probe);
             }
         }
-    if (probe != probe) *flag = seq;
+    if (probe != probe || least < kX3Smallest) *flag = seq;
 }
 
 __global__ __launch_bounds__(256) void splitk_finish_f32_k(const float* __restrict__ partial, float* __restrict__ out, u64 total, u32 splits)
@@ -1480,7 +1502,8 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
                                    (const float*)sk.partial, (float*)out->data, (u64)total, sk.splits);
                 AIXK_HIP(hipGetLastError());
             }
-            only_if = (const u32*)ctx->counter;                            // an infinity or a NaN among the operands: redo with IEEE arithmetic
+            only_if = (const u32*)ctx->counter;                            // operands the planes cannot carry: redo with IEEE arithmetic
+            ctx->gemm_last_route = 1;
         }
         auto launch = [&](auto kernel, uint64_t tile, size_t lds) {
             const u32 n = grid_of(g, tile, tile);

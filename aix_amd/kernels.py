@@ -93,6 +93,7 @@ _SIGNATURES = {
     "aixk_argmax_onehot_many": [_P, _P, C.c_uint32],
     "aixk_sum_columns_many": [_P, _P, C.c_uint32],
     "aixk_matmul": [_P, _T, _T, _T],
+    "aixk_matmul_route": [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32)],
     "aixk_matmul_batched": [_P, _T, _T, _T],
     "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],
     "aixk_rtc_get": [_P, C.c_char_p, C.c_char_p, C.c_char_p, C.POINTER(_P), C.POINTER(C.c_int32)],

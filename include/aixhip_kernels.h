@@ -205,6 +205,11 @@ int32_t aixk_sum_columns_many(aixk_ctx* ctx, const aixk_colsum_item* items, uint
  * accumulation, other types on a generic tiled kernel with an accumulator of the element type
  * (f64 and integers). */
 int32_t aixk_matmul(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out);
+/* Diagnostic (no counterpart in the reference): how the last aixk_matmul on this context was computed.  Waits for the
+ * stream.  *route = 1: an f32 product on the bf16 matrix pipe with every operand split into three bf16 planes, 0:
+ * anything else.  *redone = 1: that product met an operand the planes cannot carry (an infinity, a NaN, a nonzero
+ * magnitude at or below 2^-100) or an accumulator that overflowed, and was computed again in IEEE f32 arithmetic. */
+int32_t aixk_matmul_route(aixk_ctx* ctx, int32_t* route, int32_t* redone);
 /* An extension of the above: the reference multiplies 2-D operands only (aixCore.hpp:943-976), so an
  * AIX program issues attention as one matmul per (sequence, head) on sliced views.  Here a, b and out
  * may carry the same leading dims in front of the matrix dims: out[..., m, n] = a[..., m, k] . b[..., k, n],

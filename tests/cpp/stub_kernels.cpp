@@ -10,14 +10,18 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <deque>
 #include <string>
 
-struct aixk_ctx { size_t budget{SIZE_MAX}, held{0}; int event_delay{0}; uint64_t launches{0}, allocs{0}, frees{0}, syncs{0}, hits{0}, misses{0}; };
-struct aixk_module { int dummy; };
+struct aixk_module { std::string entry; };
+struct aixk_ctx {
+    size_t budget{SIZE_MAX}, held{0}; int event_delay{0}; uint64_t launches{0}, allocs{0}, frees{0}, syncs{0}, hits{0}, misses{0};
+    std::string log;                                       // what was launched, in order: "name;name;..." (generated kernels by their entry)
+    std::deque<aixk_module> modules;
+};
 struct aixk_event { int countdown{0}; bool recorded{false}; };
 
 static thread_local char g_error[256] = "";
-static aixk_module g_module;
 static std::atomic<long long> g_held_everywhere{0};        // bytes handed out and not yet returned, over all contexts
 static std::atomic<int> g_fail_matmuls{0};                 // the next n matmul calls report AIXK_ENOMEM
 
@@ -33,6 +37,8 @@ uint64_t stub_frees(aixk_ctx* c) { return c->frees; }
 uint64_t stub_syncs(aixk_ctx* c) { return c->syncs; }
 long long stub_held_everywhere(void) { return g_held_everywhere.load(); }
 void stub_fail_next_matmuls(int n) { g_fail_matmuls = n; }
+const char* stub_log(aixk_ctx* c) { return c->log.c_str(); }
+void stub_log_clear(aixk_ctx* c) { c->log.clear(); }
 
 const char* aixk_last_error(void) { return g_error; }
 size_t aixk_dtype_size(int dtype) { static const size_t sz[9] = {8, 4, 2, 2, 8, 4, 2, 1, 1}; return dtype >= 0 && dtype < 9 ? sz[dtype] : 0; }
@@ -69,7 +75,7 @@ int32_t aixk_copy_dev(aixk_ctx* c, void* d, const void* s, size_t n) { ++c->laun
 int32_t aixk_zero(aixk_ctx* c, void* d, size_t n) { ++c->launches; std::memset(d, 0, n); return AIXK_OK; }
 int32_t aixk_sync(aixk_ctx* c) { ++c->syncs; return AIXK_OK; }
 
-#define STUB_OP(name, ...) int32_t name(aixk_ctx* c, __VA_ARGS__) { ++c->launches; return AIXK_OK; }
+#define STUB_OP(name, ...) int32_t name(aixk_ctx* c, __VA_ARGS__) { ++c->launches; c->log += #name ";"; return AIXK_OK; }
 STUB_OP(aixk_binary, int, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
 STUB_OP(aixk_unary, int, const aixhip_tensor*, const aixhip_tensor*)
 STUB_OP(aixk_fill, const void*, int, const aixhip_tensor*)
@@ -95,7 +101,7 @@ STUB_OP(aixk_sum_partials_many, const aixk_partials_item*, uint32_t)
 int32_t aixk_matmul(aixk_ctx* c, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
 {
     if (g_fail_matmuls > 0) { --g_fail_matmuls; std::snprintf(g_error, sizeof(g_error), "stub: matmul workspace"); return AIXK_ENOMEM; }
-    ++c->launches;
+    ++c->launches; c->log += "aixk_matmul;";
     return AIXK_OK;
 }
 STUB_OP(aixk_matmul_batched, const aixhip_tensor*, const aixhip_tensor*, const aixhip_tensor*)
@@ -105,16 +111,17 @@ int32_t aixk_matmul_grouped(aixk_ctx* c, const aixhip_tensor* a, const aixhip_te
     return AIXK_OK;
 }
 
-int32_t aixk_rtc_get(aixk_ctx* c, const char*, const char*, const char*, aixk_module** out, int32_t* was_cached)
+int32_t aixk_rtc_get(aixk_ctx* c, const char*, const char*, const char* entry, aixk_module** out, int32_t* was_cached)
 {
     ++c->misses;
-    *out = &g_module;
+    c->modules.push_back(aixk_module{entry ? entry : ""});
+    *out = &c->modules.back();
     if (was_cached) *was_cached = 0;
     return AIXK_OK;
 }
-STUB_OP(aixk_rtc_launch, aixk_module*, uint32_t, uint32_t, const void*, size_t)
+int32_t aixk_rtc_launch(aixk_ctx* c, aixk_module* m, uint32_t, uint32_t, const void*, size_t) { ++c->launches; c->log += m->entry + ";"; return AIXK_OK; }
 STUB_OP(aixk_fill_many, const aixk_fill_item*, uint32_t)
-STUB_OP(aixk_rtc_launch_many, aixk_module*, uint32_t, const void*, size_t, size_t, uint32_t)
+int32_t aixk_rtc_launch_many(aixk_ctx* c, aixk_module* m, uint32_t, const void*, size_t, size_t, uint32_t) { ++c->launches; c->log += m->entry + "*;"; return AIXK_OK; }
 const char* aixk_rtc_prelude(void) { return ""; }
 int32_t aixk_rtc_stats(aixk_ctx* c, uint64_t* hits, uint64_t* misses) { *hits = c->hits; *misses = c->misses; return AIXK_OK; }
 

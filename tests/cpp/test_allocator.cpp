@@ -12,6 +12,7 @@
 #include <random>
 #include <set>
 #include <stdexcept>
+#include <string>
 #include <thread>
 #include <vector>
 
@@ -25,6 +26,8 @@ uint64_t stub_frees(aixk_ctx*);
 uint64_t stub_syncs(aixk_ctx*);
 long long stub_held_everywhere(void);
 void stub_fail_next_matmuls(int);
+const char* stub_log(aixk_ctx*);
+void stub_log_clear(aixk_ctx*);
 }
 
 using aix::DataType;
@@ -337,6 +340,53 @@ static void test_blocks_of_calls_that_wait_are_not_handed_out()
     for (void* p : {again, b, r, x, y, z}) dev.deallocate(p);
 }
 
+// A fill that nothing has read yet is normally set aside at a flush and waits for its first user.  A call that waits
+// (a small product, a sliceSet) and is about to overwrite the fill's buffer is such a user: the fill leaves before the call,
+// never behind it -- behind it, it would wipe the call's result, and a recorded reader would take the fill's constant.
+static void test_fills_do_not_land_behind_calls_that_wait()
+{
+    auto half = [](void* p, size_t rows = 64) { DeviceTensorParams t = matrix(p, rows, 64); t.dtype = DataType::kBFloat16; return t; };
+    auto at = [](const std::string& log, const char* what, size_t from = 0) { return log.find(what, from); };
+    const float zero = 0.0f;
+    {   // fill(r); matmul(a, b, r); exp(r) -> o
+        DeviceHIP dev;
+        aixk_ctx* ctx = dev.kernelContext();
+        void* a = dev.allocate(8192); void* b = dev.allocate(8192); void* r = dev.allocate(8192); void* o = dev.allocate(8192);
+        stub_log_clear(ctx);
+        dev.fill(&zero, DataType::kFloat32, half(r));
+        dev.matmul(half(a), half(b), half(r));
+        dev.exp(half(r), half(o));
+        dev.synchronize();
+        const std::string log = stub_log(ctx);
+        const size_t product = at(log, "aixk_matmul"), reader = std::min(at(log, "Exp"), at(log, "aixk_unary"));
+        const size_t fill = std::min(at(log, "aixk_fill"), at(log, "Fill"));
+        CHECK(product != std::string::npos && reader != std::string::npos);
+        CHECK(fill == std::string::npos || fill < product);                  // (a fill that is dropped as dead would do as well)
+        CHECK(product < reader);
+        CHECK(at(log, "aixk_fill", product) == std::string::npos && at(log, "Fill", product) == std::string::npos);
+        if (g_failed) std::printf("launch order: %s\n", log.c_str());
+        for (void* p : {a, b, r, o}) dev.deallocate(p);
+    }
+    {   // a fill through another view of the destination cannot be folded into sliceSet: it goes first all the same
+        DeviceHIP dev;
+        aixk_ctx* ctx = dev.kernelContext();
+        void* s = dev.allocate(2048); void* r = dev.allocate(8192); void* o = dev.allocate(8192);
+        stub_log_clear(ctx);
+        dev.fill(&zero, DataType::kFloat32, half(r, 32));
+        dev.sliceSet(half(s, 16), half(r), 0, 0, 16, 1);
+        dev.exp(half(r), half(o));
+        dev.synchronize();
+        const std::string log = stub_log(ctx);
+        const size_t window = at(log, "aixk_slice_set"), reader = std::min(at(log, "Exp"), at(log, "aixk_unary"));
+        const size_t fill = std::min(at(log, "aixk_fill"), at(log, "Fill"));
+        CHECK(window != std::string::npos && reader != std::string::npos && fill != std::string::npos);
+        CHECK(fill < window && window < reader);
+        CHECK(at(log, "aixk_fill", window) == std::string::npos && at(log, "Fill", window) == std::string::npos);
+        if (g_failed) std::printf("launch order: %s\n", log.c_str());
+        for (void* p : {s, r, o}) dev.deallocate(p);
+    }
+}
+
 static void test_destruction_returns_everything()
 {
     const long long before = stub_held_everywhere();
@@ -362,6 +412,7 @@ int main(int argc, char** argv)
     test_used_blocks_wait_for_the_gpu();
     test_out_of_memory_retry();
     test_blocks_of_calls_that_wait_are_not_handed_out();
+    test_fills_do_not_land_behind_calls_that_wait();
     test_destruction_returns_everything();
     for (unsigned seed = 1; seed <= 4; ++seed) stress(seed, 20000);
     for (unsigned seed = 21; seed <= 24; ++seed) planner_traffic(seed, 3000);

@@ -1012,3 +1012,44 @@ def test_operators_at_once_leave_an_unrelated_window_alone(dev):
     pt2, want_t2 = transposed(again["host"], again["desc"])                  # reads a recorded result: the window goes first
     T.assert_same_bits(dev.fetch(pt2, want_t2.storage), want_t2.storage, "transpose of a recorded sum")
     dev.release()
+
+
+def test_a_fill_of_the_destination_never_lands_behind_a_call_that_waits(dev):
+    """fill(r); matmul(a, b, r); exp(r): the small 16-bit product waits for company, and the recorded fill of its result
+    must leave before it, not be set aside as idle and wipe the product later (the reader would then take the fill's
+    constant).  The same with a fill through another view of a sliceSet's destination, which cannot be folded into the
+    copy.  Both bit for bit against the oracle's operator sequence (the device interface may be driven directly like this,
+    as Targets/AIXTests/DeviceTests.cpp does)."""
+    rng = np.random.default_rng(47000)
+    seven = np.full(1, 7.0, np.float32)
+    for dtype in (O.BF16, O.F16):
+        a, b = T.contiguous_tensor(rng, dtype, [64, 64]), T.contiguous_tensor(rng, dtype, [64, 64])
+        r, o = T.empty(dtype, [64, 64]), T.empty(dtype, [64, 64])
+        (_, da), (_, db) = dev.put(a), dev.put(b)
+        pr, po = dev.raw(r.storage.nbytes), dev.raw(o.storage.nbytes)
+        dr, do = H.kdesc(r, pr), H.kdesc(o, po)
+        dev.dev.synchronize()
+        dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(dr))
+        dev.dev.call("matmul", H.ref(da), H.ref(db), H.ref(dr))
+        dev.dev.call("exp", H.ref(dr), H.ref(do))
+        got_r, got_o = dev.fetch(pr, r.storage), dev.fetch(po, o.storage)
+        # the product itself is held to the 16-bit bar against exact accumulation; exp is then applied to the device's own product
+        exact, scale = np.zeros(64 * 64), np.zeros(64 * 64)
+        assert CPU.matmul_wide(C.byref(a.desc()), C.byref(b.desc()), exact.ctypes.data, scale.ctypes.data, 8) == 0
+        err = np.abs(O.to_float64(got_r, dtype).ravel() - exact)
+        assert (err <= 2e-2 * scale + 1e-30).all(), f"fill + matmul, {NAMES[dtype]}: {err.max()}"
+        r.storage[...] = got_r
+        assert CPU.unary(O.EXP, C.byref(r.desc()), C.byref(o.desc())) == 0
+        bad = T.ulp_distance(got_o, o.storage, dtype)
+        assert bad <= 1, f"exp of the product, {NAMES[dtype]}: {bad} ulp"
+    for dtype in (O.F32, O.BF16):
+        part, whole = T.contiguous_tensor(rng, dtype, [16, 64]), T.contiguous_tensor(rng, dtype, [64, 64])
+        upper = T.HostTensor(whole.storage, dtype, [32, 64], [64, 1])
+        (_, dp), (pw, dw) = dev.put(part), dev.put(whole)
+        dev.dev.synchronize()
+        dev.dev.call("fill", seven.ctypes.data, O.F32, H.ref(H.kdesc(upper, pw)))
+        dev.dev.call("slice_set", H.ref(dp), H.ref(dw), 0, 8, 24, 1)
+        assert CPU.fill(seven.ctypes.data, O.F32, C.byref(upper.desc())) == 0
+        assert CPU.slice_set(C.byref(part.desc()), C.byref(whole.desc()), 0, 8, 24, 1, 1) == 0
+        T.assert_same_bits(dev.fetch(pw, whole.storage), whole.storage, f"fill through another view + sliceSet, {NAMES[dtype]}")
+    dev.release()

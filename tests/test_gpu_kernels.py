@@ -710,11 +710,76 @@ def test_matmul_small_tiles(gpu, dtype):
         gpu.release()
 
 
+def _route(gpu):
+    """(took the split-plane f32 route, was redone in IEEE arithmetic) for the last aixk_matmul."""
+    route, redone = C.c_int32(-1), C.c_int32(-1)
+    G.run_gpu(gpu, "aixk_matmul_route", C.byref(route), C.byref(redone))
+    return route.value, redone.value
+
+
+def test_matmul_f32_large_tiles_small_magnitudes(gpu):
+    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes.  The planes carry
+    f32's 24 bits only down to 2^-110 (bf16's grid ends at 2^-133), so operands below that -- here in matrices WITHOUT
+    any infinity or NaN, which would send the product to the IEEE kernel for their own reasons -- must be noticed and the
+    product redone in IEEE f32 arithmetic, as the CPU device computes it (aixDeviceCPU.cpp:362-389: plain f32, no range
+    limits).  Small values the planes do carry, and products and sums that land in f32's subnormals, stay on the split-plane
+    kernel (the matrix unit keeps subnormals).  Bar: 1e-5 of the sum of |a||b| against exactly accumulated products
+    (cpuref_matmul_wide), plus K quanta of 2^-149 where results are subnormal (each f32 product rounds by up to half a
+    quantum there on the CPU too)."""
+    rng = np.random.default_rng(25600)
+    m, k, n = 4096, 256, 2048                                   # 512 tiles of 128 x 128: the split-plane route
+    U = rng.uniform(-1, 1, (m, k)).astype(np.float32)
+    P = rng.uniform(0.1, 1.0, (k, n)).astype(np.float32)
+    V = (rng.uniform(0.25, 1.0, (m, k)) * rng.choice([-1.0, 1.0], (m, k))).astype(np.float32)     # magnitudes within two binades
+    one_tiny_row = (U / np.sqrt(k)).astype(np.float32)
+    one_tiny_row[2000, :] = (U[2000] * np.float32(1e-37)).astype(np.float32)
+    one_tiny_entry = (U / np.sqrt(k)).astype(np.float32)
+    one_tiny_entry[123, 45] = np.float32(3e-39)
+    with np.errstate(under="ignore"):
+        cases = [                                               # (name, A, B, redone in IEEE arithmetic?)
+            ("ordinary", (U / np.sqrt(k)).astype(np.float32), P, 0),
+            ("A at 1e-20 (planes exact)", (V * np.float32(1e-20)).astype(np.float32), P, 0),
+            ("A at 1e-29 (planes exact)", (V * np.float32(1e-29)).astype(np.float32), P, 0),
+            ("A at 1e-33", (U * np.float32(1e-33)).astype(np.float32), P, 1),
+            ("A at 1e-36", (U * np.float32(1e-36)).astype(np.float32), P, 1),
+            ("A at 3e-38", (U * np.float32(3e-38)).astype(np.float32), P, 1),
+            ("A at 1e-41 (subnormal)", (U * np.float32(1e-41)).astype(np.float32), P, 1),
+            ("one row at 1e-37 in an ordinary A", one_tiny_row, P, 1),
+            ("one subnormal entry in an ordinary A", one_tiny_entry, P, 1),
+            ("A at 1e-36 times B at 1e30", (U * np.float32(1e-36)).astype(np.float32), (P * np.float32(1e30)).astype(np.float32), 1),
+            ("ordinary A times B at 1e-36", (U / np.sqrt(k)).astype(np.float32), (P * np.float32(1e-36)).astype(np.float32), 1),
+            ("subnormal products: A at 1e-20, B at 1e-22", (V * np.float32(1e-20)).astype(np.float32), (P * np.float32(1e-22)).astype(np.float32), 0),
+            ("products below the subnormals: A at 1e-25, B at 1e-25", (V * np.float32(1e-25)).astype(np.float32), (P * np.float32(1e-25)).astype(np.float32), 0),
+        ]
+    floor = k * 2.0 ** -149
+    for name, A, B, want_redone in cases:
+        for layout in ("NN", "TN"):
+            if layout == "TN" and name.startswith(("A at 1e-2", "A at 3e", "products below")):
+                continue                                        # (one layout is enough for the variations of one scale)
+            a = T.HostTensor(A if layout == "NN" else np.ascontiguousarray(A.T), O.F32, [m, k], None if layout == "NN" else [1, m])
+            b = T.HostTensor(B, O.F32, [k, n])
+            _, da = gpu.put(a)
+            _, db = gpu.put(b)
+            po, do = gpu.put(T.empty(O.F32, [m, n]))
+            G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+            route, redone = _route(gpu)
+            got = gpu.fetch(po, np.zeros(m * n, np.float32))
+            gpu.release()
+            assert (route, redone) == (1, want_redone), (name, layout, route, redone)
+            exact, scale = np.zeros(m * n), np.zeros(m * n)
+            okc(CPU.matmul_wide(C.byref(a.desc()), C.byref(b.desc()), exact.ctypes.data, scale.ctypes.data, 8))
+            err = np.abs(got.astype(np.float64) - exact)
+            bad = np.flatnonzero(~(err <= 1e-5 * scale + floor))
+            assert bad.size == 0, (name, layout, bad.size, int(bad[0]), float(got[bad[0]]), float(exact[bad[0]]), float(scale[bad[0]]))
+            if not want_redone and scale.min() > 2.0 ** -100:    # far inside the bar in practice: three planes carry all 24 bits
+                assert np.all(err <= 4e-7 * scale), (name, layout, float((err / scale).max()))
+
+
 def test_matmul_f32_large_tiles_special_values(gpu):
     """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes in registers.
     Rows with an infinity, a NaN, both infinities, or a value next to FLT_MAX must come out as IEEE arithmetic has
     them (inf, NaN, NaN, finite); their neighbours in the same 16-byte chunk and everything else stay within the
-    f32 matmul bar; subnormal inputs count as what they are."""
+    f32 matmul bar.  (Non-finite operands send the whole product to the IEEE kernel; small magnitudes are the test above.)"""
     rng = np.random.default_rng(25500)
     m, k, n = 4096, 256, 2048
     A = (rng.uniform(-1, 1, (m, k)) / np.sqrt(k)).astype(np.float32)
@@ -725,7 +790,6 @@ def test_matmul_f32_large_tiles_special_values(gpu):
     A[300, 3], A[300, 77] = np.inf, -np.inf
     A[1000, :] = 0.0
     A[1000, 17] = np.float32(3.3e38)                  # times at most 1: finite in f32, would be inf if rounded up to bf16 first
-    A[2000, :] = np.float32(1e-41)                    # subnormal inputs
     for layout in ("NN", "TN"):
         a = T.HostTensor(A if layout == "NN" else np.ascontiguousarray(A.T), O.F32, [m, k], None if layout == "NN" else [1, m])
         b = T.HostTensor(B, O.F32, [k, n])
@@ -733,6 +797,7 @@ def test_matmul_f32_large_tiles_special_values(gpu):
         _, db = gpu.put(b)
         po, do = gpu.put(T.empty(O.F32, [m, n]))
         G.run_gpu(gpu, "aixk_matmul", G.ref(da), G.ref(db), G.ref(do))
+        assert _route(gpu) == (1, 1), layout
         got = gpu.fetch(po, np.zeros(m * n, np.float32)).reshape(m, n)
         assert np.all(got[7] == np.inf), layout
         assert np.all(np.isnan(got[130])) and np.all(np.isnan(got[300])), layout
