@@ -2,8 +2,9 @@
 //
 // Kernels (A is [M,K], B is [K,N]; "K-contiguous" = unit stride along K, "T form" = unit stride along M / N):
 //
-//   16-bit, whole tiles   gemm_nt16_direct_k: 256x256x64 workgroup tile, LDS filled by LDS-direct
-//                         global loads, swizzled layout, explicit software pipeline; both operand forms;
+//   16-bit, whole tiles   gemm_nt16_direct_k: 256x256x64 workgroup tile, eight waves (two per SIMD) on
+//                         v_mfma_f32_16x16x32, LDS filled by LDS-direct global loads, swizzled layout,
+//                         explicit software pipeline; both operand forms;
 //   16-bit, mid-size      gemm_tile16_k: 128x128 / 128x64 / 64x64 tiles, register staging, both operand
 //                         forms, stacks of matrices (blockIdx.y) and K splits over workgroups (blockIdx.z);
 //   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
@@ -11,7 +12,7 @@
 //   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
 //   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 or 64x64 tile x BK=32, both operand forms.
 //
-// All use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
+// All but the first use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
 // resident in the 512-entry unified register file.  Every lane feeds the 16-bit MFMA with 8 consecutive K
 // values of one row; because A and B use the same lane->K assignment, the dot products are independent of
 // how the instruction numbers K internally.
@@ -29,6 +30,7 @@
 #include <cstdlib>
 #include <algorithm>
 #include <type_traits>
+#include <utility>
 
 using namespace aixd;
 using namespace aixk;
@@ -81,12 +83,16 @@ template <class T> struct Mma16;
 template <> struct Mma16<bf16> {
     static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c)
     { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0); }
+    static __device__ __forceinline__ f32x4 run16(u32x4 a, u32x4 b, f32x4 c)
+    { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0); }
     static __device__ __forceinline__ bf16 out(float v) { return bf16_down(v); }
     static __device__ __forceinline__ u32 pack(float lo, float hi) { return (u32)out(lo).bits | ((u32)out(hi).bits << 16); }
 };
 template <> struct Mma16<f16> {
     static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c)
     { return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0); }
+    static __device__ __forceinline__ f32x4 run16(u32x4 a, u32x4 b, f32x4 c)
+    { return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0); }
     static __device__ __forceinline__ f16 out(float v) { return (f16)v; }
     static __device__ __forceinline__ u32 pack(float lo, float hi)
     { return (u32)__builtin_bit_cast(u16, (f16)lo) | ((u32)__builtin_bit_cast(u16, (f16)hi) << 16); }
@@ -194,16 +200,28 @@ __global__ __launch_bounds__(256) void gemm_nt16_k(GemmArgs g)
 // registers, whole 128-byte rows per 8 lanes so every L2 request is a full line).  One load
 // instruction deposits 1 KB contiguously (lane L at byte 16 L), so padding is impossible; instead
 // the 16-byte k-chunk q of row r is kept in slot q ^ f(r), f(r) = ((r >> 1) & 7) ^ ((r & 1) << 2),
-// which makes the ds_read_b128 fragment reads (32 consecutive rows, one slot) conflict-free for
+// which makes the ds_read_b128 fragment reads (16 consecutive rows, four slots) conflict-free for
 // both 8-lane/32-bank and 16-lane/64-bank service; the producing lane applies the same
 // permutation to the global address it fetches.
 //
-// A K-step is four phases of 16 MFMAs (one 16-wide K slice each) on double-buffered fragments: the
-// LDS reads of the next slice and the loads of the tile after next are spread between the MFMAs in
-// fenced sub-blocks of 4 (the scheduler otherwise serialises "read, wait, 4 MFMAs").  The step's
-// single barrier sits before the last phase, whose MFMAs cover the first fragment reads from the
-// other stage.  The compiler does not track LDS-direct loads against LDS reads, so the waits
-// before each barrier are explicit (s_waitcnt vmcnt), and the barrier is the bare instruction.
+// EIGHT waves, two per SIMD, in a 2 x 4 arrangement: a wave owns 128 x 64 of the tile as 8 x 4
+// tiles of 16 x 16 and multiplies with v_mfma_f32_16x16x32.  Both choices are about power, which is
+// what bounds this kernel on real operands (a loop of nothing but MFMAs on U(-1,1)/64 values runs
+// at 1.81 GHz and 0.68 of the nominal peak with v_mfma_f32_32x32x16, at 2.08 GHz and 0.81 with
+// v_mfma_f32_16x16x32, which moves half the accumulator bits per flop; on all-zero operands both
+// reach 0.91-0.92 at 2.4 GHz): the 16 x 16 x 32 instruction needs two waves per SIMD to be issued
+// back to back, and with two waves the older one takes the matrix pipe whenever it can, the younger
+// one whenever the older waits -- no issue slot is lost to LDS or load latency.  The price is 1.5 x
+// the LDS fragment traffic of four waves with 128 x 128 each.
+//
+// A K-step is two slices of 32: phase A multiplies slice 0 while slice 1 is read into the other
+// fragment set, the step's single barrier, phase B multiplies slice 1 while slice 0 of the other
+// stage is read and ALL eight loads of the tile after next are issued (a whole K-step ahead of the
+// wait that needs them: spread over both phases they left 10 us on the table at 4096^3).  Reads and
+// loads sit between the MFMAs in fenced sub-blocks of eight.  The compiler does not track LDS-direct
+// loads against LDS reads, so the waits before the barrier are explicit (s_waitcnt vmcnt) and the
+// barrier is the bare instruction.  Results leave through LDS as non-temporal 16-byte stores (the
+// product is not read again by this kernel, and at its end every L2 would have to write it back).
 #define AIX_SB() __builtin_amdgcn_sched_barrier(0)
 #define AIX_WAIT(VM, LGKM) __builtin_amdgcn_s_waitcnt(((VM) & 15) | (((VM) >> 4) << 14) | 0x70 | ((LGKM) << 8))
 #define AIX_LDS(p) ((__attribute__((address_space(3))) void*)(p))
@@ -216,9 +234,11 @@ __global__ __launch_bounds__(256) void gemm_nt16_k(GemmArgs g)
 // ds_read_b64_tr_b16: in every group of 16 lanes, lane j points at 4 consecutive elements
 // ("row" j) and lane i receives element i & 3 of rows (i >> 2) + 4 e, e = 0..3.  With lane j
 // pointing at X[k + (j >> 2)][n + 4 (j & 3) ..], lane i receives X[k .. k + 3][n + i]: four k of
-// its own column; two such reads make a fragment.  The four k-rows of a group are 512 bytes
-// apart (same banks), so the 16-byte chunk c of k-row k is kept in slot c ^ 4 (k & 3): the 64 bytes
-// that two neighbouring groups read from each of their four k-rows then fall into disjoint banks.
+// its own column; two such reads make a fragment; the wave's four groups of 16 lanes read the same
+// 16 columns at k, k + 8, k + 16, k + 24.  The four k-rows of a group are 512 bytes apart (same
+// banks), and so are the rows of the next group, so the 16-byte chunk c of k-row k is kept in slot
+// c ^ 4 (k & 3) ^ 2 ((k >> 3) & 1): the 32 bytes that a group reads from each of its four k-rows,
+// and those of the neighbouring group, fall into disjoint banks.
 //
 // The read is issued through inline assembly: given the builtin, the compiler orders it behind every
 // LDS-direct load in flight (s_waitcnt vmcnt(0) before each read), which serialises the pipeline.
@@ -234,25 +254,31 @@ __device__ __forceinline__ u32x4 tr_fragment(const unsigned char* lds_addr)
     return u32x4{lo.x, lo.y, hi.x, hi.y};
 }
 
+template <int N> struct Const { static constexpr int v = N; };
+
 template <class T, bool AT, bool BT>
-__global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
+__global__ __launch_bounds__(512) void gemm_nt16_direct_k(GemmArgs g)
 {
-    constexpr int BM = 256, BK = 64, TI = 4, TJ = 4, STAGE = 2 * 256 * BK * 2;     // 65536 bytes: A rows then B rows
+    constexpr int BM = 256, BK = 64, STAGE = 2 * 256 * BK * 2;      // 65536 bytes: A rows then B rows
+    constexpr int WGN = 4, TI = 8, TJ = 4, WCOLS = TJ * 16;          // 2 x 4 waves of 128 x 64
+    constexpr int LPW = 8, LH = 4;                                   // loads per wave and tile: 4 chunks of A, 4 of B
+    constexpr int NF = TI + TJ, FPB = NF / 4;                        // fragments per slice, per sub-block
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     u32 tm, tn;
     tile_of(g, tm, tn);
     const u64 m0 = (u64)tm * 256, n0 = (u64)tn * 256;
     const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), wm = wave >> 1, wn = wave & 1;
-    // producer, K-contiguous operand: wave w fills rows 64 w .. 64 w + 63, 8 chunks of 8 rows (128 B) each
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), wm = wave / WGN, wn = wave % WGN;
+    // producer, K-contiguous operand: wave w fills rows 32 w .. 32 w + 31, 4 chunks of 8 rows (128 B each)
     const int lr = lane >> 3;
     const int fe = (lr >> 1) ^ ((lr & 1) << 2);              // f(row) in even chunks; odd chunks: fe ^ 4
     const int q0 = (lane & 7) ^ fe, q1 = q0 ^ 4;
-    // producer, T-form operand: wave w fills k-rows 16 w .. 16 w + 15, 8 chunks of 2 k-rows (512 B) each;
-    // lane = (k-row lane >> 5, slot lane & 31) fetches chunk slot ^ 4 (k & 3), k & 3 = 2 (chunk & 1) + (lane >> 5)
-    const int tk = lane >> 5, ts0 = (lane & 31) ^ (4 * tk), ts1 = ts0 ^ 8;
-    const char* A = AT ? (const char*)g.a + m0 * 2 + (u64)(wave * 16) * g.lda * 2 : (const char*)g.a + (m0 + wave * 64) * g.lda * 2;
-    const char* B = BT ? (const char*)g.b + n0 * 2 + (u64)(wave * 16) * g.ldb * 2 : (const char*)g.b + (n0 + wave * 64) * g.ldb * 2;
+    // producer, T-form operand: wave w fills k-rows 8 w .. 8 w + 7, 4 chunks of 2 k-rows (512 B each); lane = (k-row
+    // lane >> 5, slot lane & 31) fetches chunk slot ^ 4 (k & 3) ^ 2 ((k >> 3) & 1), k & 3 = 2 (chunk & 1) + (lane >> 5),
+    // (k >> 3) & 1 = w & 1
+    const int tk = lane >> 5, ts0 = (lane & 31) ^ (4 * tk) ^ (2 * (wave & 1)), ts1 = ts0 ^ 8;
+    const char* A = AT ? (const char*)g.a + m0 * 2 + (u64)(wave * 8) * g.lda * 2 : (const char*)g.a + (m0 + wave * 32) * g.lda * 2;
+    const char* B = BT ? (const char*)g.b + n0 * 2 + (u64)(wave * 8) * g.ldb * 2 : (const char*)g.b + (n0 + wave * 32) * g.ldb * 2;
     const u32 oa0 = AT ? (u32)((tk * g.lda + ts0 * 8) * 2) : (u32)((lr * g.lda + q0 * 8) * 2);
     const u32 oa1 = AT ? (u32)((tk * g.lda + ts1 * 8) * 2) : (u32)((lr * g.lda + q1 * 8) * 2);
     const u32 ob0 = BT ? (u32)((tk * g.ldb + ts0 * 8) * 2) : (u32)((lr * g.ldb + q0 * 8) * 2);
@@ -260,97 +286,106 @@ __global__ __launch_bounds__(256) void gemm_nt16_direct_k(GemmArgs g)
     const u64 ca = (AT ? 4 : 16) * g.lda, cb = (BT ? 4 : 16) * g.ldb;      // bytes between chunks
     const u64 sa = AT ? (u64)BK * g.lda * 2 : (u64)BK * 2, sb = BT ? (u64)BK * g.ldb * 2 : (u64)BK * 2;   // bytes between K-steps
     const int steps = (int)(g.K / BK);
-    // consumer, K-contiguous operand: lane reads row (lane & 31) of a 32-row block, k-chunk 2 kk + (lane >> 5)
-    const int r15 = lane & 15;
-    const int slot0 = (lane >> 5) ^ (((r15 >> 1) & 7) ^ ((r15 & 1) << 2));
-    // consumer, T-form operand: lane j of a 16-lane group points at k-row (8 (lane >> 5) + (j >> 2)) [+ 16 kk, + 4],
-    // columns 16 ((lane >> 4) & 1) + 4 (j & 3) .. + 3 of the 32-column block; the block index enters by XOR (bits 6-7)
-    const int tq = r15 >> 2, tn4 = 4 * (r15 & 3), tc = (16 * ((lane >> 4) & 1) + tn4) >> 3;
-    const int tlane = (8 * (lane >> 5) + tq) * 512 + (tn4 & 4) * 2;
-    const int fra = AT ? tlane + (((16 * wm + tc) ^ (4 * tq)) * 16) : (wm * 128 + (lane & 31)) * 128 + slot0 * 16;
-    const int frb = BM * 128 + (BT ? tlane + (((16 * wn + tc) ^ (4 * tq)) * 16) : (wn * 128 + (lane & 31)) * 128 + slot0 * 16);
+    // consumer, K-contiguous operand: lane reads row (lane & 15) of a 16-row block, k-chunk 4 s + (lane >> 4) of slice s
+    const int r15 = lane & 15, grp = lane >> 4;
+    const int slot0 = grp ^ (((r15 >> 1) & 7) ^ ((r15 & 1) << 2));
+    // consumer, T-form operand: lane j of a 16-lane group points at k-row 32 s + 8 grp + (j >> 2) [+ 4], columns
+    // 4 (j & 3) .. + 3 of the 16-column block; the block index enters by XOR (bits 5 and up of the byte address)
+    const int tq = r15 >> 2;
+    const int tlane = (8 * grp + tq) * 512 + 8 * (r15 & 1);
+    const int tsw = (4 * tq) ^ (2 * (grp & 1));
+    const int fra = AT ? tlane + (((16 * wm + ((r15 & 3) >> 1)) ^ tsw) * 16) : (wm * 128 + r15) * 128 + slot0 * 16;
+    const int frb = BM * 128 + (BT ? tlane + (((8 * wn + ((r15 & 3) >> 1)) ^ tsw) * 16) : (wn * WCOLS + r15) * 128 + slot0 * 16);
 
-    f32x16 acc[TI][TJ];
+    f32x4 acc[TI][TJ];
 #pragma unroll
     for (int i = 0; i < TI; ++i)
 #pragma unroll
-        for (int j = 0; j < TJ; ++j)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+        for (int j = 0; j < TJ; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     u32x4 fa[2][TI], fb[2][TJ];
 
-    // load n of a tile (0..15): n < 8 is chunk n of A, otherwise chunk n - 8 of B
-#define AIX_LD(N, KI, BO) { if ((N) < 8) __builtin_amdgcn_global_load_lds(AIX_GLB(A + ((N) * ca + (KI) * sa) + (((N) & 1) ? oa1 : oa0)), AIX_LDS(smem + (BO) + (wave * 8 + (N)) * 1024), 16, 0, 0); \
-    else __builtin_amdgcn_global_load_lds(AIX_GLB(B + (((N) - 8) * cb + (KI) * sb) + (((N) & 1) ? ob1 : ob0)), AIX_LDS(smem + (BO) + BM * 128 + (wave * 8 + (N) - 8) * 1024), 16, 0, 0); }
-#define AIX_RDA(F, BO, KK, I) { if constexpr (AT) fa[F][I] = tr_fragment(smem + (BO) + (fra ^ ((I) * 64)) + (KK) * 8192); \
-    else fa[F][I] = *(const u32x4*)(smem + (BO) + (fra ^ ((KK) * 32)) + (I) * 4096); }
-#define AIX_RDB(F, BO, KK, J) { if constexpr (BT) fb[F][J] = tr_fragment(smem + (BO) + (frb ^ ((J) * 64)) + (KK) * 8192); \
-    else fb[F][J] = *(const u32x4*)(smem + (BO) + (frb ^ ((KK) * 32)) + (J) * 4096); }
-#define AIX_ROW(F, I) { _Pragma("unroll") for (int j = 0; j < TJ; ++j) acc[I][j] = Mma16<T>::run(fa[F][I], fb[F][j], acc[I][j]); }
-    // MFMAs on fragment set FC while set FN is read from stage RBO, slice KK; loads L0.. of K-tile KO go to stage LBO
-#define AIX_PHASE(FC, FN, RBO, KK, KO, LBO, L0, L1, L2, L3, L4, L5) \
-    if constexpr (AT || BT) { AIX_SB(); __builtin_amdgcn_s_waitcnt(0xC07F); AIX_SB(); }     /* lgkmcnt(0): fragment set FC has arrived */ \
-    AIX_RDA(FN, RBO, KK, 0) AIX_RDA(FN, RBO, KK, 1) if (L0 >= 0) AIX_LD(L0, KO, LBO) if (L4 >= 0) AIX_LD(L4, KO, LBO) AIX_ROW(FC, 0) AIX_SB(); \
-    AIX_RDA(FN, RBO, KK, 2) AIX_RDA(FN, RBO, KK, 3) if (L1 >= 0) AIX_LD(L1, KO, LBO) if (L5 >= 0) AIX_LD(L5, KO, LBO) AIX_ROW(FC, 1) AIX_SB(); \
-    AIX_RDB(FN, RBO, KK, 0) AIX_RDB(FN, RBO, KK, 1) if (L2 >= 0) AIX_LD(L2, KO, LBO) AIX_ROW(FC, 2) AIX_SB(); \
-    AIX_RDB(FN, RBO, KK, 2) AIX_RDB(FN, RBO, KK, 3) if (L3 >= 0) AIX_LD(L3, KO, LBO) AIX_ROW(FC, 3) AIX_SB();
+    // load n of a tile (0..7): n < 4 is this wave's chunk n of A, otherwise chunk n - 4 of B
+    auto load = [&](auto n_, u64 ki, int bo) {
+        constexpr int n = decltype(n_)::v;
+        if constexpr (n < LH)
+            __builtin_amdgcn_global_load_lds(AIX_GLB(A + (n * ca + ki * sa) + ((n & 1) ? oa1 : oa0)), AIX_LDS(smem + bo + (wave * LH + n) * 1024), 16, 0, 0);
+        else
+            __builtin_amdgcn_global_load_lds(AIX_GLB(B + ((n - LH) * cb + ki * sb) + ((n & 1) ? ob1 : ob0)), AIX_LDS(smem + bo + BM * 128 + (wave * LH + n - LH) * 1024), 16, 0, 0);
+    };
+    // fragment f of slice s: f < 8 is A's 16-row block f, otherwise B's block f - 8
+    auto read = [&](int set, int bo, int s, int f) {
+        if (f < TI) {
+            if constexpr (AT) fa[set][f] = tr_fragment(smem + bo + (fra ^ (f * 32)) + s * 16384);
+            else fa[set][f] = *(const u32x4*)(smem + bo + (fra ^ (s * 64)) + f * 2048);
+        } else {
+            if constexpr (BT) fb[set][f - TI] = tr_fragment(smem + bo + (frb ^ ((f - TI) * 32)) + s * 16384);
+            else fb[set][f - TI] = *(const u32x4*)(smem + bo + (frb ^ (s * 64)) + (f - TI) * 2048);
+        }
+    };
+    // MFMAs on fragment set FC while set FN is read from stage rbo, slice S; with LOADS, the tile `ko` goes to stage lbo
+    auto phase = [&](auto FC_, auto FN_, int rbo, auto S_, auto LOADS_, u64 ko, int lbo) {
+        constexpr int FC = decltype(FC_)::v, FN = decltype(FN_)::v, S = decltype(S_)::v, LOADS = decltype(LOADS_)::v;
+        if constexpr (AT || BT) { AIX_SB(); __builtin_amdgcn_s_waitcnt(0xC07F); AIX_SB(); }     // lgkmcnt(0): fragment set FC has arrived
+        [&]<int... b>(std::integer_sequence<int, b...>) {
+            ([&] {
+#pragma unroll
+                for (int f = b * FPB; f < (b + 1) * FPB; ++f) read(FN, rbo, S, f);
+                if constexpr (LOADS) { load(Const<b>{}, ko, lbo); load(Const<b + 4>{}, ko, lbo); }
+#pragma unroll
+                for (int i = 2 * b; i < 2 * b + 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < TJ; ++j) acc[i][j] = Mma16<T>::run16(fa[FC][i], fb[FC][j], acc[i][j]);
+                AIX_SB();
+            }(), ...);
+        }(std::make_integer_sequence<int, 4>{});
+    };
 
     // Tiles past the end re-read the last tile into a stage nobody consumes any more.
     {
         const u64 k1 = 1 < steps ? 1 : 0;
-#pragma unroll
-        for (int n = 0; n < 16; ++n) AIX_LD(n, (u64)0, 0)
-#pragma unroll
-        for (int n = 0; n < 6; ++n) AIX_LD(n, k1, STAGE)
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, (u64)0, 0), ...); }(std::make_integer_sequence<int, LPW>{});
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, k1, STAGE), ...); }(std::make_integer_sequence<int, LPW>{});
     }
     AIX_SB();
-    AIX_WAIT(6, 15);                                          // tile 0 has landed (6 younger loads may be in flight)
+    AIX_WAIT(LPW, 15);                                        // tile 0 has landed (the 8 loads of tile 1 may be in flight)
     __builtin_amdgcn_s_barrier();
     AIX_SB();
-    AIX_RDA(0, 0, 0, 0) AIX_RDA(0, 0, 0, 1) AIX_RDA(0, 0, 0, 2) AIX_RDA(0, 0, 0, 3)
-    AIX_RDB(0, 0, 0, 0) AIX_RDB(0, 0, 0, 1) AIX_RDB(0, 0, 0, 2) AIX_RDB(0, 0, 0, 3)
+#pragma unroll
+    for (int f = 0; f < NF; ++f) read(0, 0, 0, f);
     for (int kt = 0; kt < steps; ++kt) {
         const int bo = (kt & 1) * STAGE, nbo = bo ^ STAGE;
-        const u64 k1 = (u64)(kt + 1 < steps ? kt + 1 : steps - 1), k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1);
-        AIX_PHASE(0, 1, bo, 1, k1, nbo, 6, 7, 8, 9, 10, -1)
-        AIX_PHASE(1, 0, bo, 2, k1, nbo, 11, 12, 13, 14, 15, -1)
-        AIX_PHASE(0, 1, bo, 3, k1, nbo, -1, -1, -1, -1, -1, -1)
+        const u64 k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1);
+        phase(Const<0>{}, Const<1>{}, bo, Const<1>{}, Const<0>{}, k2, nbo);
         AIX_WAIT(0, 0);                                       // tile kt+1 complete in the other stage; own reads of this stage done
         __builtin_amdgcn_s_barrier();
         AIX_SB();
-        AIX_PHASE(1, 0, nbo, 0, k2, bo, 0, 1, 2, 3, 4, 5)
+        phase(Const<1>{}, Const<0>{}, nbo, Const<0>{}, Const<1>{}, k2, bo);
     }
-#undef AIX_PHASE
-#undef AIX_ROW
-#undef AIX_RDB
-#undef AIX_RDA
-#undef AIX_LD
     AIX_WAIT(0, 0);                                           // stray loads have landed before LDS is reused
     __builtin_amdgcn_s_barrier();
     AIX_SB();
 
-    // Epilogue through LDS, each wave on its own 20 KB: a 32-row slab of the wave's 128 x 128 block
-    // is laid out row-major (pitch 132 floats), read back as runs of 8 columns, rounded and stored
-    // with 16-byte writes (256 contiguous bytes per row).
-    constexpr int PITCH = 132;
-    float* slab = (float*)smem + wave * (32 * PITCH + 1024);
+    // Epilogue through LDS, each wave on its own 4.5 KB: a 16-row slab of the wave's 128 x 64 block is laid out
+    // row-major (pitch 68 floats), read back as runs of 8 columns, rounded and stored with 16-byte writes (128
+    // contiguous bytes per row).  Accumulator element v of lane l: row 4 (l / 16) + v, column l % 16 of its 16 x 16 tile.
+    constexpr int PITCH = WCOLS + 4;
+    float* slab = (float*)smem + wave * (16 * PITCH + 64);
     u16* C = (u16*)g.c;
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
 #pragma unroll
         for (int j = 0; j < TJ; ++j)
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
-                slab[((v >> 2) * 8 + (lane >> 5) * 4 + (v & 3)) * PITCH + j * 32 + (lane & 31)] = acc[i][j][v];
+            for (int v = 0; v < 4; ++v) slab[(4 * grp + v) * PITCH + j * 16 + r15] = acc[i][j][v];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const int grp = lane + 64 * t, row = grp >> 4, cg = grp & 15;
+        for (int t = 0; t < 2; ++t) {
+            const int run = lane + 64 * t, row = run >> 3, cg = run & 7;
             const f32x4 lo = *(const f32x4*)(slab + row * PITCH + cg * 8);
             const f32x4 hi = *(const f32x4*)(slab + row * PITCH + cg * 8 + 4);
             u32x4 o;
             o.x = Mma16<T>::pack(lo.x, lo.y); o.y = Mma16<T>::pack(lo.z, lo.w);
             o.z = Mma16<T>::pack(hi.x, hi.y); o.w = Mma16<T>::pack(hi.z, hi.w);
-            *(u32x4*)(C + (m0 + wm * 128 + i * 32 + row) * g.N + n0 + wn * 128 + cg * 8) = o;
+            __builtin_nontemporal_store(o, (u32x4*)(C + (m0 + wm * 128 + i * 16 + row) * g.N + n0 + wn * WCOLS + cg * 8));
         }
     }
 }
@@ -1402,7 +1437,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
             const bool at = !a_k, bt = !b_k;
             auto launch = [&](auto kernel) {
                 AIXK_TRY(set_lds(kernel, lds));
-                hipLaunchKernelGGL(kernel, dim3(n), dim3(256), lds, ctx->stream, g);
+                hipLaunchKernelGGL(kernel, dim3(n), dim3(512), lds, ctx->stream, g);
                 AIXK_HIP(hipGetLastError());
                 return (int)AIXK_OK;
             };
