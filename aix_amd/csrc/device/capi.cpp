@@ -195,6 +195,7 @@ int32_t aixhip_last_flush_diagnostics(aixhip_device* dev, aixhip_flush_diagnosti
     });
 }
 
+int32_t aixhip_set_cache_limit(aixhip_device* dev, uint64_t bytes) { return guarded([&] { D(dev).setCacheLimit((size_t)bytes); }); }
 int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint64_t* kernels)
 {
     return guarded([&] {

@@ -11,6 +11,7 @@
 #include <cstdio>
 #include <cstring>
 #include <cstdlib>
+#include <dlfcn.h>
 #include <deque>
 #include <iostream>
 #include <limits>
@@ -91,6 +92,38 @@ int unaryCode(OpType t)
 // AIXHIP_TRACE=1: one line on stderr per kernel or operator the device enqueues (what ran, in which order, how large).
 static const bool kTrace = [] { const char* e = std::getenv("AIXHIP_TRACE"); return e && e[0] == '1'; }();
 #define AIXHIP_TRACE(...) do { if (kTrace) { std::fprintf(stderr, "[aixhip] " __VA_ARGS__); std::fputc('\n', stderr); } } while (0)
+
+// AIXHIP_ROCTX=1: a roctx range around every Device call, every flush of the planner's window and every send-off of the
+// calls that wait, named after the operator, so that a profiler's marker trace (rocprofv3 --marker-trace) cuts a step by
+// operator.  The marker library is looked up at run time and only then; without the variable a Marker is one branch.
+namespace {
+struct Roctx {
+    int (*push)(const char*){nullptr};
+    int (*pop)(){nullptr};
+    Roctx()
+    {
+        const char* e = std::getenv("AIXHIP_ROCTX");
+        if (!e || e[0] != '1') return;
+        for (const char* name : {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4", "libroctx64.so"}) {
+            if (void* lib = dlopen(name, RTLD_NOW | RTLD_GLOBAL)) {
+                push = reinterpret_cast<int (*)(const char*)>(dlsym(lib, "roctxRangePushA"));
+                pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+                if (push && pop) return;
+                push = nullptr; pop = nullptr;
+            }
+        }
+        std::fprintf(stderr, "[aixhip] AIXHIP_ROCTX=1 but no roctx library could be loaded: no markers\n");
+    }
+};
+const Roctx& roctx() { static const Roctx r; return r; }
+struct Marker {
+    explicit Marker(const char* name) : on(roctx().push != nullptr) { if (on) roctx().push(name); }
+    ~Marker() { if (on) roctx().pop(); }
+    Marker(const Marker&) = delete;
+    Marker& operator=(const Marker&) = delete;
+    bool on;
+};
+} // namespace
 
 struct DeviceHIP::Extras {
     std::deque<Cooling> cooling;
@@ -262,6 +295,8 @@ DeviceHIP::DeviceHIP(size_t deviceIndex)
     aixk_device_info info{};
     if (aixk_info(m_ctx, &info) == AIXK_OK && info.compute_units > 0) m_cus = info.compute_units;
     m_totalBytes = info.total_mem;
+    m_cacheLimit = (size_t)((double)info.total_mem * 0.7);
+    if (const char* env = std::getenv("AIXHIP_CACHE_LIMIT_BYTES")) m_cacheLimit = (size_t)std::strtoull(env, nullptr, 10);
     if (aixk_info(m_ctx, &info) == AIXK_OK && !info.large_bar)
         std::cerr << "DeviceHIP: device memory is not host-addressable on this system; tensors must be moved with "
                      "copy()/copyToHost() and never dereferenced on the host." << std::endl;
@@ -472,6 +507,7 @@ void DeviceHIP::releaseLimbo()
 
 void DeviceHIP::emptyCache()
 {
+    const Marker marker_("emptyCache");
     for (auto& kv : m_pool) for (void* p : kv.second) aixk_free(m_ctx, p, 0);
     m_pool.clear();
     m_pooledBytes = 0;
@@ -482,6 +518,7 @@ void DeviceHIP::flush() { flushWindow(true); }
 // final: nothing recorded stays behind.  Otherwise fills that nothing recorded so far uses may wait (FuseEngine::flush).
 void DeviceHIP::flushWindow(bool final)
 {
+    const Marker marker_("flush");
     // Calls that wait (small products, sliceSet, one-hot masks, column sums) stay waiting across a flush: they depend on nothing
     // recorded (their callers saw to that), and a kernel that leaves now and uses what they write, or writes what they
     // use, sends them off first (emitFused, emitSingle).
@@ -545,6 +582,7 @@ bool DeviceHIP::fenceInterior(const void* a, const void* b, const void* c)
 
 void DeviceHIP::synchronize()
 {
+    const Marker marker_("synchronize");
     flush();
     check(aixk_sync(m_ctx));
     auto& ex = *m_extras;
@@ -558,16 +596,39 @@ void DeviceHIP::synchronize()
     m_limbo.clear();
     m_limboBytes = 0;
     ex.flushesSinceEvent = 0;
+    trimPool();
+}
+
+// Idle blocks beyond the cache limit go back to the driver (aixDeviceMetal.cpp:1369-1373, aixDeviceMetalCache.hpp:97-124:
+// the least recently used first).  Called with the GPU idle.  Every bucket is a stack whose top is handed out first, so
+// its bottom is its coldest block; buckets are taken in the order of the bytes they hold, the fullest first.
+void DeviceHIP::trimPool()
+{
+    while (m_pooledBytes > m_cacheLimit) {
+        std::vector<void*>* fullest = nullptr;
+        size_t bucket = 0, most = 0;
+        for (auto& kv : m_pool)
+            if (kv.first * kv.second.size() > most) { most = kv.first * kv.second.size(); fullest = &kv.second; bucket = kv.first; }
+        if (!fullest) break;
+        // enough of its cold end to get under the limit, or all of it
+        const size_t over = m_pooledBytes - m_cacheLimit;
+        const size_t count = std::min(fullest->size(), (over + bucket - 1) / bucket);
+        for (size_t k = 0; k < count; ++k) aixk_free(m_ctx, (*fullest)[k], 0);
+        fullest->erase(fullest->begin(), fullest->begin() + (std::ptrdiff_t)count);
+        m_pooledBytes -= count * bucket;
+    }
 }
 
 void DeviceHIP::copyToHost(void* dstHost, const void* srcDevice, size_t bytes)
 {
+    const Marker marker_("copyToHost");
     flushFor(srcDevice);
     check(aixk_copy_out(m_ctx, dstHost, srcDevice, bytes));
 }
 
 void DeviceHIP::copyFromHost(void* dstDevice, const void* srcHost, size_t bytes)
 {
+    const Marker marker_("copyFromHost");
     if (!findBlock(dstDevice)) throw std::invalid_argument("DeviceHIP::copyFromHost() result must have GPU memory.");
     flushFor(dstDevice);
     check(aixk_copy_in(m_ctx, dstDevice, srcHost, bytes));
@@ -630,6 +691,7 @@ void DeviceHIP::stagedPod(const DeviceTensorParams& p, aixhip_tensor* out, const
 // ---- recorded (fusable) operators --------------------------------------------------------------
 void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& r, const char* op)
 {
+    const Marker marker_(op);
     requireDevice(r, op);
     if (a.dtype != r.dtype || b.dtype != r.dtype)
         throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operands must have the result's data type.");
@@ -655,6 +717,7 @@ void DeviceHIP::recordBinary(OpType t, const DeviceTensorParams& a, const Device
 
 void DeviceHIP::recordUnary(OpType t, const DeviceTensorParams& a, const DeviceTensorParams& r, const char* op)
 {
+    const Marker marker_(op);
     requireDevice(r, op);
     if (a.dtype != r.dtype)
         throw std::invalid_argument(std::string("DeviceHIP::") + op + "() operand must have the result's data type.");
@@ -692,6 +755,7 @@ void DeviceHIP::exp(const DeviceTensorParams& a, const DeviceTensorParams& resul
 
 void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTensorParams& result)
 {
+    const Marker marker_("fill");
     requireDevice(result, "fill");
     View out(result);
     out.makeDense();
@@ -702,6 +766,7 @@ void DeviceHIP::fill(const void* scalar, DataType scalarDType, const DeviceTenso
 
 void DeviceHIP::fillMin(const DeviceTensorParams& result)
 {
+    const Marker marker_("fillMin");
     requireDevice(result, "fillMin");
     View out(result);
     out.makeDense();
@@ -1065,6 +1130,7 @@ void DeviceHIP::emitRowProgram(const FusedSubgraphDescriptor& d)
 // ---- operators that run at once ------------------------------------------------------------------
 void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    const Marker marker_("sum");
     AIXHIP_TRACE("sum");
     requireDevice(result, "sum");
     flushFor(a.data, result.data);
@@ -1074,6 +1140,7 @@ void DeviceHIP::sum(const DeviceTensorParams& a, const DeviceTensorParams& resul
 
 void DeviceHIP::max(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    const Marker marker_("max");
     AIXHIP_TRACE("max");
     requireDevice(result, "max");
     flushFor(a.data, result.data);
@@ -1083,6 +1150,7 @@ void DeviceHIP::max(const DeviceTensorParams& a, const DeviceTensorParams& resul
 
 void DeviceHIP::argmax(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    const Marker marker_("argmax");
     if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmax supports only int32 data type for its result.");
     requireDevice(result, "argmax");
     flushFor(a.data, result.data);
@@ -1092,6 +1160,7 @@ void DeviceHIP::argmax(const DeviceTensorParams& a, const DeviceTensorParams& re
 
 void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorParams& result)
 {
+    const Marker marker_("argmaxIndices");
     if (result.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndices supports only int32 data type for its result.");
     requireDevice(result, "argmaxIndices");
     flushFor(a.data, result.data);
@@ -1108,6 +1177,7 @@ void DeviceHIP::argmaxIndices(const DeviceTensorParams& a, const DeviceTensorPar
 // reference batches its dispatches for the same reason (aixDeviceMetal.cpp:1344-1389).
 void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b, const DeviceTensorParams& result)
 {
+    const Marker marker_("matmul");
     requireDevice(result, "matmul");
     AIXHIP_TRACE("matmul rank %zu, %zu x %zu elements", a.shape.size(), a.size, b.size);
     auto& ex = *m_extras;
@@ -1163,6 +1233,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
 
 void DeviceHIP::issuePending()
 {
+    const Marker marker_("calls that waited leave");
     auto& ex = *m_extras;
     int status = AIXK_OK;
     if (ex.anyPending()) {
@@ -1215,6 +1286,7 @@ void DeviceHIP::issuePending()
 
 void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)
 {
+    const Marker marker_("transpose");
     AIXHIP_TRACE("transpose");
     requireDevice(result, "transpose");
     flushFor(a.data, result.data);
@@ -1224,6 +1296,7 @@ void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams&
 
 void DeviceHIP::copy(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size)
 {
+    const Marker marker_("copy");
     if (size == 0) return;
     if (!findBlock(dst)) throw std::invalid_argument("DeviceHIP::copy() result must have GPU memory.");        // aixDeviceMetal.cpp:714-715
     // Both ends whole device blocks: the conversion is recorded and fuses into the kernel that produces its
@@ -1251,12 +1324,14 @@ void DeviceHIP::copy(const void* src, DataType srcDType, void* dst, DataType dst
 
 void DeviceHIP::copyImmediate(const void* src, DataType srcDType, void* dst, DataType dstDType, size_t size)
 {
+    const Marker marker_("copyImmediate");
     copy(src, srcDType, dst, dstDType, size);
     synchronize();
 }
 
 void DeviceHIP::contiguous(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    const Marker marker_("contiguous");
     AIXHIP_TRACE("contiguous");
     requireDevice(dst, "contiguous");
     flushFor(src.data, dst.data);
@@ -1322,6 +1397,7 @@ bool DeviceHIP::recordRowReduction(OpType type, const DeviceTensorParams& src, c
 
 void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    const Marker marker_("reduceTo");
     AIXHIP_TRACE("reduceTo");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::reduceTo() requires matching source and destination data types.");
     requireDevice(dst, "reduceTo");
@@ -1371,6 +1447,7 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
 
 void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst)
 {
+    const Marker marker_("maxTo");
     AIXHIP_TRACE("maxTo");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::maxTo() requires matching source and destination data types.");
     requireDevice(dst, "maxTo");
@@ -1384,6 +1461,7 @@ void DeviceHIP::maxTo(const DeviceTensorParams& src, const DeviceTensorParams& d
 
 void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
 {
+    const Marker marker_("argmaxTo");
     AIXHIP_TRACE("argmaxTo");
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxTo");
@@ -1397,6 +1475,7 @@ void DeviceHIP::argmaxTo(const DeviceTensorParams& src, const DeviceTensorParams
 // launch (see matmul(), sliceSet()).
 void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim)
 {
+    const Marker marker_("argmaxIndicesTo");
     AIXHIP_TRACE("argmaxIndicesTo");
     if (dst.dtype != DataType::kInt32) throw std::invalid_argument("DeviceHIP::argmaxIndicesTo supports only int32 data type for its result.");
     requireDevice(dst, "argmaxIndicesTo");
@@ -1454,6 +1533,7 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
 // overlap; otherwise what waits is issued first.
 void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams& dst, size_t dim, size_t start, size_t end, size_t step)
 {
+    const Marker marker_("sliceSet");
     AIXHIP_TRACE("sliceSet");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::sliceSet() requires matching source and destination data types.");
     requireDevice(dst, "sliceSet");
@@ -1511,6 +1591,7 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
 
 void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
 {
+    const Marker marker_("tril");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::tril() requires matching source and destination data types.");   // aixDeviceMetal.cpp:1160-1161
     requireDevice(dst, "tril");
     if (recordTri(OpType::Tril, src, dst, diagonal)) return;
@@ -1521,6 +1602,7 @@ void DeviceHIP::tril(const DeviceTensorParams& src, const DeviceTensorParams& ds
 
 void DeviceHIP::triu(const DeviceTensorParams& src, const DeviceTensorParams& dst, ssize_t diagonal)
 {
+    const Marker marker_("triu");
     if (src.dtype != dst.dtype) throw std::invalid_argument("DeviceHIP::triu() requires matching source and destination data types.");
     requireDevice(dst, "triu");
     if (recordTri(OpType::Triu, src, dst, diagonal)) return;
@@ -1547,6 +1629,7 @@ bool DeviceHIP::recordTri(OpType type, const DeviceTensorParams& src, const Devi
 
 void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
 {
+    const Marker marker_("indexSelect");
     AIXHIP_TRACE("indexSelect");
     requireDevice(dst, "indexSelect");
     flushFor(src.data, indices.data, dst.data);
@@ -1556,6 +1639,7 @@ void DeviceHIP::indexSelect(const DeviceTensorParams& src, const DeviceTensorPar
 
 void DeviceHIP::indexAdd(const DeviceTensorParams& src, const DeviceTensorParams& dst, const DeviceTensorParams& indices, size_t dim)
 {
+    const Marker marker_("indexAdd");
     AIXHIP_TRACE("indexAdd");
     requireDevice(dst, "indexAdd");
     flushFor(src.data, indices.data, dst.data);

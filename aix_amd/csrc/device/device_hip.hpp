@@ -108,6 +108,10 @@ public:
     void flush();                                                            // plan + enqueue, no wait
     aixk_ctx* kernelContext() const { return m_ctx; }
     size_t cachedBytes() const { return m_pooledBytes; }
+    // The pool of idle blocks is cut back to this many bytes at every synchronize() (aixDeviceMetal.cpp:1369-1373 trims
+    // its buffer cache to the working-set limit at every commit).  Default: 0.7 of the card's memory, as there (:33).
+    void setCacheLimit(size_t bytes) { m_cacheLimit = bytes; }
+    size_t cacheLimit() const { return m_cacheLimit; }
     size_t allocatedBytes() const { return m_liveBytes; }
 
 private:
@@ -176,7 +180,8 @@ private:
     BlockTable m_blocks;
     std::unordered_map<size_t, std::vector<void*>> m_pool;     // free blocks by bucket size
     std::vector<std::pair<void*, size_t>> m_limbo;             // freed, but recorded work may still use them
-    size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0}, m_totalBytes{0};
+    size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0}, m_totalBytes{0}, m_cacheLimit{~size_t(0)};
+    void trimPool();
     int m_cus{256};
 };
 

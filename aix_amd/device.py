@@ -58,6 +58,7 @@ _SIGNATURES = {
     "aixhip_last_flush_diagnostics": [_P, C.POINTER(FlushDiagnostics)],
     "aixhip_fuse_kernel_cache_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "aixhip_batched_launch_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "aixhip_set_cache_limit": [_P, C.c_uint64],
     "aixhip_memory_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
 }
 _OTHER = {

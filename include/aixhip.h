@@ -143,6 +143,10 @@ int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint
 /* The kernel-layer context of this device (stream, events) for timing with aixk_event_*. */
 aixk_ctx* aixhip_kernel_context(aixhip_device* dev);
 int32_t aixhip_memory_stats(aixhip_device* dev, uint64_t* live_bytes, uint64_t* cached_bytes);
+/* The pool of idle blocks is cut back to `bytes` at every synchronize (the reference's GPU device trims its buffer cache
+ * to its working-set limit at every commit, aixDeviceMetal.cpp:33, 1369-1373).  Default 0.7 of the card's memory;
+ * environment override AIXHIP_CACHE_LIMIT_BYTES. */
+int32_t aixhip_set_cache_limit(aixhip_device* dev, uint64_t bytes);
 
 #ifdef __cplusplus
 }

@@ -387,6 +387,42 @@ static void test_fills_do_not_land_behind_calls_that_wait()
     }
 }
 
+// The pool of idle blocks is cut back to the cache limit at every synchronize(): the fullest bucket first, its coldest
+// blocks first (aixDeviceMetal.cpp:1369-1373, aixDeviceMetalCache.hpp:97-124).  Live blocks and blocks the GPU may still
+// use are never given back.
+static void test_the_pool_is_trimmed_to_the_cache_limit()
+{
+    DeviceHIP dev;
+    aixk_ctx* ctx = dev.kernelContext();
+    CHECK(dev.cacheLimit() == (size_t)((double)(1ull << 30) * 0.7));      // the stub's card has 1 GiB
+    std::vector<void*> big, small;
+    for (int i = 0; i < 8; ++i) big.push_back(dev.allocate(1 << 20));
+    for (int i = 0; i < 4; ++i) small.push_back(dev.allocate(4096));
+    void* live = dev.allocate(1 << 20);
+    touch(dev, big[0], big[1], live);                   // some of them have been used by the GPU
+    for (void* p : big) dev.deallocate(p);
+    for (void* p : small) dev.deallocate(p);
+    dev.synchronize();
+    CHECK(dev.cachedBytes() == 8 * (size_t(1) << 20) + 4 * 4096);         // under the default limit: all of it is kept
+    const uint64_t frees = stub_frees(ctx);
+    dev.setCacheLimit(3 * (size_t(1) << 20));
+    dev.synchronize();
+    CHECK(dev.cachedBytes() <= 3 * (size_t(1) << 20));
+    CHECK(dev.cachedBytes() == 2 * (size_t(1) << 20) + 4 * 4096);         // six of the fullest bucket went, the small ones stay
+    CHECK(stub_frees(ctx) == frees + 6);
+    CHECK(dev.allocatedBytes() == (size_t(1) << 20) && dev.isDeviceMemory(live));
+    // the two that stayed are the ones that came back to the pool last (the two the GPU had used: they waited for it, the
+    // others were idle at the flush): the top of the stack.  They are handed out again, nothing new is asked for.
+    const uint64_t allocs = stub_allocs(ctx);
+    void* a = dev.allocate(1 << 20); void* b = dev.allocate(1 << 20);
+    CHECK(stub_allocs(ctx) == allocs);
+    CHECK((a == big[1] && b == big[0]) || (a == big[0] && b == big[1]));
+    dev.setCacheLimit(0);                               // nothing idle is kept
+    dev.deallocate(a); dev.deallocate(b); dev.deallocate(live);
+    dev.synchronize();
+    CHECK(dev.cachedBytes() == 0 && dev.allocatedBytes() == 0 && stub_held(ctx) == 0);
+}
+
 static void test_destruction_returns_everything()
 {
     const long long before = stub_held_everywhere();
@@ -413,6 +449,7 @@ int main(int argc, char** argv)
     test_out_of_memory_retry();
     test_blocks_of_calls_that_wait_are_not_handed_out();
     test_fills_do_not_land_behind_calls_that_wait();
+    test_the_pool_is_trimmed_to_the_cache_limit();
     test_destruction_returns_everything();
     for (unsigned seed = 1; seed <= 4; ++seed) stress(seed, 20000);
     for (unsigned seed = 21; seed <= 24; ++seed) planner_traffic(seed, 3000);
