@@ -381,6 +381,28 @@ def main():
         extras.append({"workload": "configs[2] matmul bf16 4096^3 NN, ALL-ZERO operands (diagnostic of the power limit, not a result)",
                        "ms_per_step": round(r.wall_s * 1e3 / 100, 5), "value": round(flops * 100 / r.wall_s / 1e12, 2), "unit": "TFLOP/s",
                        "roofline": roofline("mfma", flops / (r.gpu_ms / 100 * 1e-3) / 1e12, MFMA_PEAK_TFLOPS["bf16"], "TFLOP/s")})
+        # the matrix pipe alone on this box, in this run: a loop of nothing but MFMAs on register operands of the same values
+        # (no LDS, no loads), one workgroup per compute unit, 4096^3 worth of flops per launch -- what a GEMM could reach
+        # here if its memory traffic were free
+        from aix_amd import kernels as K
+        kctx = K.Context(0)
+        vals = np.random.default_rng(3).uniform(-1, 1, 4096).astype(np.float32) / np.sqrt(4096)
+        pipe = {}
+        for label, shape_, dt_code, ops in (("bf16_16x16x32_two_waves_per_simd", 1, K.BF16, round_to_bf16_bits(vals)),
+                                            ("bf16_32x32x16_one_wave_per_simd", 0, K.BF16, round_to_bf16_bits(vals)),
+                                            ("f16_16x16x32_two_waves_per_simd", 1, K.F16, vals.astype(np.float16).view(np.uint16)),
+                                            ("bf16_16x16x32_all_zero_operands", 1, K.BF16, np.zeros(1, np.uint16))):
+            tf, ghz = C.c_float(), C.c_float()
+            ops = np.ascontiguousarray(ops)
+            kctx.call("aixk_mfma_only_rate", shape_, dt_code, ops.ctypes.data, ops.size, 2.0 * 4096 ** 3 / 1e9, C.byref(tf), C.byref(ghz))
+            pipe[label] = {"TFLOPs": round(tf.value, 1), "frac_of_nominal_peak": round(tf.value / MFMA_PEAK_TFLOPS["bf16"], 4), "shader_clock_GHz": round(ghz.value, 2)}
+        kctx.close()
+        extras.append({"workload": "the matrix pipe alone: loops of independent MFMAs on register operands (U(-1,1)/64 values unless said otherwise), no memory "
+                                   "traffic, one workgroup per compute unit, 137 GFLOP per launch (diagnostic: the ceiling a 16-bit GEMM on these operand "
+                                   "values meets on this power-limited part)", "mfma_only": pipe})
+        targets["mfma_only_bf16_frac"] = pipe["bf16_16x16x32_two_waves_per_simd"]["frac_of_nominal_peak"]
+        if "bf16_4096_nt_frac" in targets:
+            targets["bf16_4096_nt_frac_of_mfma_only"] = round(targets["bf16_4096_nt_frac"] / targets["mfma_only_bf16_frac"], 4)
         host.clear()
     if not args.no_extras and "c3" in chosen:
         # configs[3]: MLP training step (autograd + Adam); the CPU device runs the first steps of the same program

@@ -247,6 +247,17 @@ int32_t aixk_rtc_launch_many(aixk_ctx* ctx, aixk_module* mod, uint32_t block_x, 
 const char* aixk_rtc_prelude(void);
 int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);
 
+/* ---- the matrix pipe alone (no counterpart in the reference; a measurement aid) ---------------------------------- */
+/* A loop of independent 16-bit MFMAs on register operands, no LDS and no memory traffic, one workgroup per compute unit:
+ * the rate the part sustains when it only multiplies -- on a power-limited part a function of the operand values, of the
+ * instruction and of the waves per SIMD -- against which a GEMM's fraction of the nominal peak is read.  shape 0: four
+ * waves, 4 x 4 tiles of v_mfma_f32_32x32x16 each; shape 1: eight waves, 8 x 4 tiles of v_mfma_f32_16x16x32 each (the
+ * register layout of the 256 x 256 GEMM kernel).  dtype AIXK_BF16 or AIXK_F16; `operands`: `count` 16-bit patterns used
+ * round-robin as operand values; about `gflop_per_launch` GFLOP per launch, 200 untimed and 280 timed launches on the
+ * context's stream.  *tflops: the median rate; *ghz: the shader clock held during the loop. */
+int32_t aixk_mfma_only_rate(aixk_ctx* ctx, int32_t shape, int32_t dtype, const uint16_t* operands, uint32_t count, double gflop_per_launch,
+                            float* tflops, float* ghz);
+
 /* ---- timing on the context's stream ------------------------------------- */
 int32_t aixk_event_create(aixk_ctx* ctx, aixk_event** out);
 int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev);
