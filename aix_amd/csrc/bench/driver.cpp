@@ -187,6 +187,20 @@ int aixbench_mlp(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hi
     });
 }
 
+// The same with the L2 norms of the six parameters' gradients (w1, b1, w2, b2, w3, b3) of the first `norm_steps` steps in
+// grad_norms[norm_steps * 6].
+int aixbench_mlp_norms(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
+                       const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds,
+                       float* grad_norms, int norm_steps)
+{
+    return guarded([&] {
+        DeviceHIP* dev = aix::hip::fromHandle(handle);
+        const aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr, single_pass};
+        const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
+        aixfe::runMlp(dev, cfg, host, losses, step_seconds, grad_norms, norm_steps);
+    });
+}
+
 // Config 4: decoder-only transformer forward + backward (frontend/transformer.hpp); params in the order of
 // aixfe::transformerParamShapes; losses[steps], grad_norms[steps * param_count], step_seconds[steps] (may be NULL).
 // stacked_attention = 0: one 2-D matmul per (sequence, head), the reference's interface as it is; 1: matmul on stacks.
@@ -198,6 +212,30 @@ int aixbench_transformer(aixhip_device* handle, uint64_t layers, uint64_t d_mode
         DeviceHIP* dev = aix::hip::fromHandle(handle);
         const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps, stacked_attention};
         aixfe::runTransformer(dev, cfg, tokens, params, losses, grad_norms, step_seconds);
+    });
+}
+
+// The same with step `capture_at` captured into a HIP graph (DeviceHIP::beginCapture / endCapture) and that step and every
+// later one enqueued by DeviceHIP::replay: no front-end, no planner, one launch call per step.  The steps before it run
+// as usual (they compile the kernels and grow the workspaces the captured step needs).  *graph_nodes (may be NULL): the
+// number of nodes of the graph.
+int aixbench_transformer_captured(aixhip_device* handle, uint64_t layers, uint64_t d_model, uint64_t heads, uint64_t seq, uint64_t batch,
+                                  uint64_t vocab, int steps, int stacked_attention, int capture_at, const int32_t* tokens, const float* const* params,
+                                  float* losses, float* grad_norms, double* step_seconds, uint64_t* graph_nodes)
+{
+    return guarded([&] {
+        DeviceHIP* dev = aix::hip::fromHandle(handle);
+        aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps, stacked_attention};
+        cfg.captureAt = capture_at;
+        DeviceHIP::StepGraph* graph = nullptr;
+        aixfe::StepCapture capture;
+        capture.begin = [&] { dev->beginCapture(); };
+        capture.end = [&] { graph = dev->endCapture(); };
+        capture.replay = [&] { dev->replay(graph); };
+        try { aixfe::runTransformer(dev, cfg, tokens, params, losses, grad_norms, step_seconds, &capture); }
+        catch (...) { if (graph) dev->destroyGraph(graph); throw; }
+        if (graph_nodes) *graph_nodes = graph ? dev->graphNodes(graph) : 0;
+        if (graph) dev->destroyGraph(graph);
     });
 }
 

@@ -195,6 +195,16 @@ int32_t aixhip_last_flush_diagnostics(aixhip_device* dev, aixhip_flush_diagnosti
     });
 }
 
+int32_t aixhip_capture_begin(aixhip_device* dev) { return guarded([&] { D(dev).beginCapture(); }); }
+int32_t aixhip_capture_end(aixhip_device* dev, aixhip_graph** out)
+{
+    return guarded([&] {
+        if (!out) throw std::invalid_argument("aixhip_capture_end: null out pointer");
+        *out = reinterpret_cast<aixhip_graph*>(D(dev).endCapture());
+    });
+}
+int32_t aixhip_graph_replay(aixhip_device* dev, aixhip_graph* graph) { return guarded([&] { D(dev).replay(reinterpret_cast<DeviceHIP::StepGraph*>(graph)); }); }
+int32_t aixhip_graph_destroy(aixhip_device* dev, aixhip_graph* graph) { return guarded([&] { D(dev).destroyGraph(reinterpret_cast<DeviceHIP::StepGraph*>(graph)); }); }
 int32_t aixhip_set_cache_limit(aixhip_device* dev, uint64_t bytes) { return guarded([&] { D(dev).setCacheLimit((size_t)bytes); }); }
 int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint64_t* kernels)
 {

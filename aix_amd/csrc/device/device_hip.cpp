@@ -16,6 +16,7 @@
 #include <iostream>
 #include <limits>
 #include <stdexcept>
+#include <unordered_set>
 
 namespace aix {
 
@@ -126,6 +127,7 @@ struct Marker {
 } // namespace
 
 struct DeviceHIP::Extras {
+    std::unordered_set<const void*> graphBlocks;               // bases of the blocks that captured work uses
     std::deque<Cooling> cooling;
     unsigned flushesSinceEvent{0};
     std::unordered_map<std::string, aixk_module*> kernels;     // signature -> compiled kernel
@@ -316,11 +318,13 @@ DeviceHIP::~DeviceHIP()
         if (m_ctx && m_extras && m_extras->anyPending()) issuePending();           // matmul calls still waiting for company
         if (m_engine) m_engine.reset();
         if (m_ctx) {
+            if (m_capturing) { m_capturing = false; aixk_capture_abort(m_ctx); }
             aixk_sync(m_ctx);
             auto& ex = *m_extras;
             for (auto& c : ex.cooling) { aixk_event_destroy(m_ctx, c.event); for (auto& b : c.blocks) aixk_free(m_ctx, b.first, 0); }
             for (auto& b : m_limbo) aixk_free(m_ctx, b.first, 0);
             for (auto& kv : m_pool) for (void* p : kv.second) aixk_free(m_ctx, p, 0);
+            for (auto& b : m_graphReserve) aixk_free(m_ctx, b.first, 0);
             m_blocks.forEach([this](void* base, const Block& b) { if (!b.freed) aixk_free(m_ctx, base, 0); });
             aixk_destroy(m_ctx);
         }
@@ -395,7 +399,7 @@ void* DeviceHIP::allocateBlock(size_t bytes, bool track)
     while (!ex.cooling.empty()) {
         int32_t done = 0;
         if (aixk_event_query(m_ctx, ex.cooling.front().event, &done) != AIXK_OK || !done) break;
-        for (auto& b : ex.cooling.front().blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        for (auto& b : ex.cooling.front().blocks) pool(b.first, b.second);
         aixk_event_destroy(m_ctx, ex.cooling.front().event);
         ex.cooling.pop_front();
     }
@@ -444,7 +448,12 @@ void DeviceHIP::markTouched(const void* p)
     if (!p || m_blocks.empty()) return;
     Block* b = m_blocks.find(p);
     if (!b) b = m_blocks.findContaining(p);
-    if (b) b->touched = true;
+    if (!b) return;
+    b->touched = true;
+    if (m_capturing && !b->inGraph) {                       // captured work uses the block: it belongs to the graph (see pool())
+        b->inGraph = true;
+        m_extras->graphBlocks.insert(m_blocks.find(p) ? p : m_blocks.baseOf(p));
+    }
 }
 
 // Called once the recorded work that might touch freed blocks has been enqueued.
@@ -470,8 +479,7 @@ void DeviceHIP::releaseLimbo()
         } else if (b && !b->touched) {
             size_t bytes = 0;
             m_blocks.erase(entry.first, &bytes);
-            m_pool[entry.second].push_back(entry.first);
-            m_pooledBytes += entry.second;
+            pool(entry.first, entry.second);
             m_limboBytes -= entry.second;
         } else {
             m_limbo[kept++] = entry;
@@ -481,7 +489,7 @@ void DeviceHIP::releaseLimbo()
     if (m_limbo.empty()) return;
 
     const size_t enough = std::max<size_t>({size_t(32) << 20, m_totalBytes >> 10, (m_liveBytes + m_pooledBytes) / 8});
-    if (++ex.flushesSinceEvent < 16 && m_limboBytes < enough) return;
+    if (!m_capturing && ++ex.flushesSinceEvent < 16 && m_limboBytes < enough) return;      // (inside a capture no event is needed: see below)
     ex.flushesSinceEvent = 0;
     std::vector<std::pair<void*, size_t>> stay, leave;
     if (held) {
@@ -494,12 +502,16 @@ void DeviceHIP::releaseLimbo()
     for (const auto& entry : stay) stayBytes += entry.second;
     for (const auto& entry : leave) { size_t bytes = 0; m_blocks.erase(entry.first, &bytes); }
     Cooling c{};
-    if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
+    if (m_capturing) {
+        // nothing runs while the stream records, and what is recorded runs in stream order: a freed block may be used
+        // again by work captured later (the host does not write into blocks while it captures)
+        for (auto& b : leave) pool(b.first, b.second);
+    } else if (aixk_event_create(m_ctx, &c.event) == AIXK_OK && aixk_event_record(m_ctx, c.event) == AIXK_OK) {
         c.blocks.swap(leave);
         ex.cooling.push_back(std::move(c));
     } else {
         aixk_sync(m_ctx);
-        for (auto& b : leave) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        for (auto& b : leave) pool(b.first, b.second);
     }
     m_limbo.swap(stay);
     m_limboBytes = stayBytes;
@@ -583,20 +595,93 @@ bool DeviceHIP::fenceInterior(const void* a, const void* b, const void* c)
 void DeviceHIP::synchronize()
 {
     const Marker marker_("synchronize");
+    if (m_capturing) throw std::runtime_error("DeviceHIP::synchronize: nothing runs while a capture is open (endCapture() first)");
     flush();
     check(aixk_sync(m_ctx));
     auto& ex = *m_extras;
     for (auto& c : ex.cooling) {
-        for (auto& b : c.blocks) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        for (auto& b : c.blocks) pool(b.first, b.second);
         aixk_event_destroy(m_ctx, c.event);
     }
     ex.cooling.clear();
     // everything recorded has been enqueued and has finished: blocks freed since the last event are idle too
-    for (auto& b : m_limbo) { size_t bytes = 0; m_blocks.erase(b.first, &bytes); m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+    for (auto& b : m_limbo) { size_t bytes = 0; m_blocks.erase(b.first, &bytes); pool(b.first, b.second); }
     m_limbo.clear();
     m_limboBytes = 0;
     ex.flushesSinceEvent = 0;
     trimPool();
+}
+
+// An idle block goes back to its bucket -- unless a graph's kernels use it: then only work captured into a graph may
+// have it again (inside a capture, where everything is ordered on the stream), and once the capture is closed it is kept
+// aside for as long as a graph lives.
+void DeviceHIP::pool(void* p, size_t bytes)
+{
+    if (!m_capturing && m_graphs && m_extras->graphBlocks.count(p)) { m_graphReserve.emplace_back(p, bytes); return; }
+    m_pool[bytes].push_back(p);
+    m_pooledBytes += bytes;
+}
+
+void DeviceHIP::beginCapture()
+{
+    if (m_capturing) throw std::runtime_error("DeviceHIP::beginCapture: a capture is already open");
+    synchronize();                                          // everything pending runs, every freed block is idle and pooled
+    check(aixk_capture_begin(m_ctx));
+    m_capturing = true;
+}
+
+DeviceHIP::StepGraph* DeviceHIP::endCapture()
+{
+    if (!m_capturing) throw std::runtime_error("DeviceHIP::endCapture: no capture is open");
+    aixk_graph* g = nullptr;
+    try {
+        flushWindow(true);                                  // what is still recorded or waiting belongs to the graph
+        releaseLimbo();
+    } catch (...) { m_capturing = false; aixk_capture_abort(m_ctx); throw; }
+    m_capturing = false;
+    check(aixk_capture_end(m_ctx, &g));
+    ++m_graphs;
+    // blocks the captured work uses and that are idle now: aside (they were free to go round inside the capture)
+    auto& used = m_extras->graphBlocks;
+    for (auto& kv : m_pool) {
+        auto& stack = kv.second;
+        size_t kept = 0;
+        for (size_t k = 0; k < stack.size(); ++k) {
+            if (used.count(stack[k])) { m_graphReserve.emplace_back(stack[k], kv.first); m_pooledBytes -= kv.first; }
+            else stack[kept++] = stack[k];
+        }
+        stack.resize(kept);
+    }
+    // (blocks still in limbo are set aside when their turn to be pooled comes: pool())
+    return reinterpret_cast<StepGraph*>(g);
+}
+
+void DeviceHIP::replay(StepGraph* graph)
+{
+    if (m_capturing) throw std::runtime_error("DeviceHIP::replay: a capture is open");
+    if (!graph) throw std::invalid_argument("DeviceHIP::replay: null graph");
+    flushWindow(true);                                      // pending work first: the graph's kernels may read its results
+    check(aixk_graph_launch(m_ctx, reinterpret_cast<aixk_graph*>(graph)));
+}
+
+size_t DeviceHIP::graphNodes(const StepGraph* graph) const
+{
+    uint64_t n = 0;
+    if (graph) aixk_graph_nodes(reinterpret_cast<aixk_graph*>(const_cast<StepGraph*>(graph)), &n);
+    return (size_t)n;
+}
+
+void DeviceHIP::destroyGraph(StepGraph* graph)
+{
+    if (!graph) return;
+    aixk_graph_destroy(m_ctx, reinterpret_cast<aixk_graph*>(graph));      // waits for the stream
+    if (m_graphs && --m_graphs == 0) {
+        // no graph is left that could write into them: the blocks set aside are ordinary idle blocks again
+        for (auto& b : m_graphReserve) { m_pool[b.second].push_back(b.first); m_pooledBytes += b.second; }
+        m_graphReserve.clear();
+        m_extras->graphBlocks.clear();
+        m_blocks.forEach([](void*, Block& b) { b.inGraph = false; });
+    }
 }
 
 // Idle blocks beyond the cache limit go back to the driver (aixDeviceMetal.cpp:1369-1373, aixDeviceMetalCache.hpp:97-124:

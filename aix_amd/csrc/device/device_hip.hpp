@@ -108,6 +108,24 @@ public:
     void flush();                                                            // plan + enqueue, no wait
     aixk_ctx* kernelContext() const { return m_ctx; }
     size_t cachedBytes() const { return m_pooledBytes; }
+    // A stretch of the device's work as a HIP graph: a step whose operator stream, addresses and immediates repeat (a
+    // forward + backward pass, an update in place) is issued once between beginCapture() and endCapture() -- recorded,
+    // not run -- and then enqueued again and again by replay() with one call, without the front-end, the planner or a
+    // launch per kernel.  The reference's GPU device amortises dispatch by batching into command buffers
+    // (aixDeviceMetal.cpp:1344-1389); this goes one step further and has no counterpart there.
+    // Inside a capture: no synchronize(), no host transfer (copyToHost / copyFromHost / host operands), nothing that has
+    // to compile or grow a workspace for the first time (run the step once uncaptured before) -- std::runtime_error.
+    // Every block the captured work touches belongs to the graph from then on: freed, it is kept aside (never handed out
+    // again) until the last graph is destroyed, so a replay cannot write into somebody else's tensor; tensors that are
+    // still alive (parameters, gradients, the loss) are simply used in place by every replay.
+    struct StepGraph;
+    void beginCapture();                  // flushes and waits first
+    StepGraph* endCapture();              // flushes what was recorded into the graph; nothing of it has run yet
+    void replay(StepGraph* graph);        // enqueues the captured work (after whatever is pending)
+    size_t graphNodes(const StepGraph* graph) const;
+    void destroyGraph(StepGraph* graph);
+    bool capturing() const { return m_capturing; }
+
     // The pool of idle blocks is cut back to this many bytes at every synchronize() (aixDeviceMetal.cpp:1369-1373 trims
     // its buffer cache to the working-set limit at every commit).  Default: 0.7 of the card's memory, as there (:33).
     void setCacheLimit(size_t bytes) { m_cacheLimit = bytes; }
@@ -119,6 +137,7 @@ private:
         size_t bytes;
         bool touched{false};     // enqueued GPU work has referenced the block since it was allocated
         bool freed{false};       // deallocate() has been called; the block waits in m_limbo
+        bool inGraph{false};     // captured work uses the block: once freed it is kept aside, not pooled
     };
     struct Extras;
 
@@ -182,6 +201,10 @@ private:
     std::vector<std::pair<void*, size_t>> m_limbo;             // freed, but recorded work may still use them
     size_t m_liveBytes{0}, m_pooledBytes{0}, m_limboBytes{0}, m_totalBytes{0}, m_cacheLimit{~size_t(0)};
     void trimPool();
+    void pool(void* p, size_t bytes);     // an idle block goes back to its bucket, or aside if a graph uses it
+    bool m_capturing{false};
+    size_t m_graphs{0};
+    std::vector<std::pair<void*, size_t>> m_graphReserve;      // idle blocks that captured work uses: not handed out while a graph lives
     int m_cus{256};
 };
 

@@ -8,6 +8,7 @@
 #include "nn.hpp"
 
 #include <chrono>
+#include <cmath>
 
 namespace aixfe {
 
@@ -26,8 +27,11 @@ struct MlpHost {              // host arrays, f32, row-major
 };
 
 // Runs cfg.steps steps; losses[s] = loss of step s read after the step's synchronize();
-// step_seconds[s] (may be null) = wall time of step s, synchronize to synchronize.
-inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* losses, double* step_seconds)
+// step_seconds[s] (may be null) = wall time of step s, synchronize to synchronize; grad_norms (may be null) =
+// the L2 norms of the gradients of w1, b1, w2, b2, w3, b3 in the first grad_norm_steps steps, six per step, taken
+// between backward and the optimizer's update (outside the step's time).
+inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* losses, double* step_seconds, float* grad_norms = nullptr,
+                   int grad_norm_steps = 0)
 {
     const Tensor x = Tensor::fromHost(dev, DataType::kFloat32, Shape{cfg.batch, cfg.in}, h.x);
     const Tensor y = Tensor::fromHost(dev, DataType::kFloat32, Shape{cfg.batch, cfg.out}, h.y);
@@ -42,9 +46,16 @@ inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* l
         const Tensor logits = l3.forward(relu(l2.forward(relu(l1.forward(x)))));
         const Tensor loss = crossEntropy(softmax(logits, 1, true), y);
         if (cfg.singlePass) loss.backwardOnce(); else loss.backward();
+        double aside = 0;
+        if (grad_norms && s < grad_norm_steps) {
+            const auto n0 = std::chrono::steady_clock::now();
+            const Tensor* params[6] = {&l1.w, &l1.b, &l2.w, &l2.b, &l3.w, &l3.b};
+            for (int p = 0; p < 6; ++p) grad_norms[s * 6 + p] = params[p]->grad().l2Norm();
+            aside = std::chrono::duration<double>(std::chrono::steady_clock::now() - n0).count();
+        }
         opt.step();
         losses[s] = loss.value().item();          // synchronizes
-        if (step_seconds) step_seconds[s] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+        if (step_seconds) step_seconds[s] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() - aside;
     }
 }
 

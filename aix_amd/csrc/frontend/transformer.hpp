@@ -19,6 +19,7 @@
 // scores of all sequences and heads are one [batch, heads, seq, seq] tensor, and mask, softmax and
 // the product with v are one operator each over it.  The arithmetic per element is the same.
 #pragma once
+#include <functional>
 
 #include "nn.hpp"
 
@@ -31,6 +32,14 @@ struct TransformerConfig {
     uint64_t layers, dModel, heads, seq, batch, vocab;
     int32_t steps;
     int32_t stackedAttention{0};
+    int32_t captureAt{-1};        // >= 0 (and a StepCapture given): that step is captured, it and every later one is a replay
+};
+
+// How a device captures a step and enqueues it again (a HIP graph on the GPU backend); none on a device without it.
+// The step here repeats exactly -- same operators on the same tensors, gradients zeroed and accumulated in place, no
+// host-side scalar that changes -- so a replay computes what issuing it again would.
+struct StepCapture {
+    std::function<void()> begin, end, replay;
 };
 
 // Parameter order (all f32, row-major):
@@ -68,7 +77,7 @@ inline Tensor gelu(const Tensor& x)
 // losses[s], gradNorms[s * P + p] (L2 norm of parameter p's gradient after step s), step_seconds[s] (may be null).
 // tokens: int32 [batch * seq]; params: host arrays in the order above.
 inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_t* tokens, const float* const* params,
-                           float* losses, float* gradNorms, double* step_seconds)
+                           float* losses, float* gradNorms, double* step_seconds, const StepCapture* capture = nullptr)
 {
     const DataType F32 = DataType::kFloat32, BF16 = DataType::kBFloat16, I32 = DataType::kInt32;
     const uint64_t T = c.batch * c.seq, d = c.dModel, dh = d / c.heads;
@@ -93,8 +102,9 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
     const float scale = 1.0f / std::sqrt((float)dh);
     dev->synchronize();
 
-    for (int step = 0; step < c.steps; ++step) {
-        const auto t0 = std::chrono::steady_clock::now();
+    Tensor loss;                                                 // of the last step issued (a replay writes the captured step's)
+    auto issueStep = [&] {
+        loss = Tensor();                                         // the previous step's graph of nodes goes first
         for (auto& p : P) p.zeroGrad();
         std::vector<Tensor> W;                                   // bf16 working copies
         for (auto& p : P) W.push_back(p.to(BF16));
@@ -140,13 +150,18 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
         }
         const Tensor xf = layerNorm(x, P[at], P[at + 1]);
         const Tensor logits = matmul(xf, W[at + 2]).to(F32);
-        const Tensor loss = crossEntropy(softmax(logits, 1, true), target);
+        loss = crossEntropy(softmax(logits, 1, true), target);
         loss.backwardOnce();
+    };
+    for (int step = 0; step < c.steps; ++step) {
+        const auto t0 = std::chrono::steady_clock::now();
+        const bool captured = capture && c.captureAt >= 0 && step >= c.captureAt;
+        if (captured && step == c.captureAt) { capture->begin(); issueStep(); capture->end(); }
+        if (captured) capture->replay(); else issueStep();
         losses[step] = loss.value().item();                      // synchronizes: forward and backward have run
         if (step_seconds) step_seconds[step] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         for (size_t i = 0; i < P.size(); ++i) {
-            const Value g = P[i].grad();
-            gradNorms[(size_t)step * P.size() + i] = std::sqrt((g * g).sum().item());
+            gradNorms[(size_t)step * P.size() + i] = P[i].grad().l2Norm();
         }
     }
 }

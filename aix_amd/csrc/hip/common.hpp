@@ -12,6 +12,8 @@
 #include <mutex>
 #include <string>
 #include <unordered_map>
+#include <utility>
+#include <vector>
 
 #include "../../../include/aixhip_kernels.h"
 #include "aix_device.h"
@@ -75,12 +77,23 @@ struct aixk_ctx {
     size_t table_bytes{0}, table_used{0};
     hipEvent_t table_lap[2]{nullptr, nullptr};
     int table_half{0};
+    // a step being captured into a graph (aixk_capture_begin): its tables live in memory the graph owns, written once
+    struct aixk_graph* capturing{nullptr};
+    hipStream_t side{nullptr};         // for copies that must happen now while `stream` is capturing
     // runtime-compiled kernels by signature
     std::unordered_map<std::string, aixk_module*> rtc;
     uint64_t rtc_hits{0}, rtc_misses{0};
 };
 
 struct aixk_module { aixk::RtcModule m; };
+// A captured stretch of the stream.  `tables`: device memory holding the argument tables of its many-blocks launches
+// (written when they were captured; the launches read them at every replay), with the pinned memory they were staged in.
+struct aixk_graph {
+    hipGraph_t graph{nullptr};
+    hipGraphExec_t exec{nullptr};
+    std::vector<std::pair<void*, void*>> tables;          // (device, pinned host)
+    uint64_t nodes{0};
+};
 struct aixk_event { hipEvent_t ev{nullptr}; };
 
 namespace aixk {

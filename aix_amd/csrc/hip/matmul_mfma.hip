@@ -1117,6 +1117,7 @@ __global__ __launch_bounds__(256) void gemm_nt32_k(GemmArgs g, SplitArgs sk, con
 int workspace(aixk_ctx* ctx, int which, size_t bytes, void** out)
 {
     if (ctx->gemm_ws_bytes[which] < bytes) {
+        if (ctx->capturing) return fail(AIXK_EINVAL, "matmul workspace would have to grow inside a capture: run the same step once before capturing it");
         if (ctx->gemm_ws[which]) {
             AIXK_HIP(hipStreamSynchronize(ctx->stream));
             AIXK_HIP(hipFree(ctx->gemm_ws[which]));

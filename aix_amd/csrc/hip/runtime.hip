@@ -47,6 +47,16 @@ namespace aixk {
 int table_slot(aixk_ctx* ctx, size_t bytes, void** host, const void** dev)
 {
     bytes = (bytes + 255) & ~(size_t)255;
+    if (ctx->capturing) {
+        // the launch that reads this table will run again at every replay: the table gets memory of its own for as long
+        // as the graph lives (the ring's slots are written over a few hundred launches later)
+        void *d = nullptr, *h = nullptr;
+        AIXK_HIP(hipMalloc(&d, bytes));
+        if (hipHostMalloc(&h, bytes, hipHostMallocDefault) != hipSuccess) { (void)hipFree(d); return fail(AIXK_ENOMEM, "no pinned memory for a captured table of %zu bytes", bytes); }
+        ctx->capturing->tables.emplace_back(d, h);
+        *host = h; *dev = d;
+        return AIXK_OK;
+    }
     if (!ctx->table_host) {
         ctx->table_bytes = 1u << 20;
         AIXK_HIP(hipHostMalloc((void**)&ctx->table_host, ctx->table_bytes, hipHostMallocDefault));
@@ -73,6 +83,13 @@ int table_slot(aixk_ctx* ctx, size_t bytes, void** host, const void** dev)
 
 int table_upload(aixk_ctx* ctx, const void* host, const void* dev, size_t bytes)
 {
+    if (ctx->capturing) {
+        // written now, on a stream of its own (the main stream only records), and complete before this call returns: the
+        // captured launch finds it in place at every replay and no copy node enters the graph
+        AIXK_HIP(hipMemcpyAsync(const_cast<void*>(dev), host, bytes, hipMemcpyHostToDevice, ctx->side));
+        AIXK_HIP(hipStreamSynchronize(ctx->side));
+        return AIXK_OK;
+    }
     AIXK_HIP(hipMemcpyAsync(const_cast<void*>(dev), host, bytes, hipMemcpyHostToDevice, ctx->stream));
     return AIXK_OK;
 }
@@ -146,6 +163,8 @@ int32_t aixk_destroy(aixk_ctx* ctx)
     (void)hipFree(ctx->scratch);
     (void)hipFree(ctx->counter);
     for (void* ws : ctx->gemm_ws) if (ws) (void)hipFree(ws);
+    if (ctx->capturing) (void)aixk_capture_abort(ctx);
+    if (ctx->side) (void)hipStreamDestroy(ctx->side);
     (void)hipStreamDestroy(ctx->stream);
     delete ctx;
     return AIXK_OK;
@@ -210,6 +229,7 @@ int32_t aixk_copy_in(aixk_ctx* ctx, void* dst_dev, const void* src_host, size_t 
     AIXK_TRY(set_device(ctx));
     if (bytes == 0) return AIXK_OK;
     AIXK_REQUIRE(dst_dev && src_host, "copy_in: null pointer");
+    AIXK_REQUIRE(!ctx->capturing, "copy_in: no transfers from host memory inside a capture");
     // pageable source: the runtime stages it before returning, so the caller may reuse it
     AIXK_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, ctx->stream));
     AIXK_HIP(hipStreamSynchronize(ctx->stream));
@@ -221,6 +241,7 @@ int32_t aixk_copy_out(aixk_ctx* ctx, void* dst_host, const void* src_dev, size_t
     AIXK_TRY(set_device(ctx));
     if (bytes == 0) return AIXK_OK;
     AIXK_REQUIRE(dst_host && src_dev, "copy_out: null pointer");
+    AIXK_REQUIRE(!ctx->capturing, "copy_out: no transfers to host memory inside a capture");
     AIXK_HIP(hipMemcpyAsync(dst_host, src_dev, bytes, hipMemcpyDeviceToHost, ctx->stream));
     AIXK_HIP(hipStreamSynchronize(ctx->stream));
     return AIXK_OK;
@@ -258,6 +279,7 @@ int32_t aixk_zero(aixk_ctx* ctx, void* dst_dev, size_t bytes)
 int32_t aixk_sync(aixk_ctx* ctx)
 {
     AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(!ctx->capturing, "sync: nothing runs while the stream is being captured");
     AIXK_HIP(hipStreamSynchronize(ctx->stream));
     return AIXK_OK;
 }
@@ -353,6 +375,78 @@ int32_t aixk_rtc_launch(aixk_ctx* ctx, aixk_module* mod, uint32_t grid_x, uint32
     return AIXK_OK;
 }
 
+// ---- a stretch of the stream as a graph ----------------------------------------------------------------------------
+int32_t aixk_capture_begin(aixk_ctx* ctx)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(!ctx->capturing, "capture_begin: a capture is already open on this context");
+    if (!ctx->side) AIXK_HIP(hipStreamCreateWithFlags(&ctx->side, hipStreamNonBlocking));
+    AIXK_HIP(hipStreamSynchronize(ctx->stream));
+    // relaxed: the thread may go on calling hipMalloc and copying on other streams while this one records
+    AIXK_HIP(hipStreamBeginCapture(ctx->stream, hipStreamCaptureModeRelaxed));
+    ctx->capturing = new aixk_graph();
+    return AIXK_OK;
+}
+
+int32_t aixk_capture_end(aixk_ctx* ctx, aixk_graph** out)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(ctx->capturing && out, "capture_end: no capture is open on this context");
+    aixk_graph* g = ctx->capturing;
+    ctx->capturing = nullptr;
+    hipError_t e = hipStreamEndCapture(ctx->stream, &g->graph);
+    if (e == hipSuccess && !g->graph) e = hipErrorInvalidValue;
+    if (e == hipSuccess) e = hipGraphInstantiate(&g->exec, g->graph, nullptr, nullptr, 0);
+    size_t nodes = 0;
+    if (e == hipSuccess) e = hipGraphGetNodes(g->graph, nullptr, &nodes);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        aixk_graph_destroy(ctx, g);
+        return fail(AIXK_EHIP, "capture_end: %s", hipGetErrorString(e));
+    }
+    g->nodes = nodes;
+    *out = g;
+    return AIXK_OK;
+}
+
+int32_t aixk_capture_abort(aixk_ctx* ctx)
+{
+    if (!ctx || !ctx->capturing) return AIXK_OK;
+    (void)hipSetDevice(ctx->device);
+    aixk_graph* g = ctx->capturing;
+    ctx->capturing = nullptr;
+    (void)hipStreamEndCapture(ctx->stream, &g->graph);
+    (void)hipGetLastError();
+    return aixk_graph_destroy(ctx, g);
+}
+
+int32_t aixk_graph_launch(aixk_ctx* ctx, aixk_graph* g)
+{
+    AIXK_TRY(set_device(ctx));
+    AIXK_REQUIRE(g && g->exec, "graph_launch: null graph");
+    AIXK_REQUIRE(!ctx->capturing, "graph_launch: a capture is open on this context");
+    AIXK_HIP(hipGraphLaunch(g->exec, ctx->stream));
+    return AIXK_OK;
+}
+
+int32_t aixk_graph_nodes(aixk_graph* g, uint64_t* nodes)
+{
+    AIXK_REQUIRE(g && nodes, "graph_nodes: null argument");
+    *nodes = g->nodes;
+    return AIXK_OK;
+}
+
+int32_t aixk_graph_destroy(aixk_ctx* ctx, aixk_graph* g)
+{
+    if (!g) return AIXK_OK;
+    if (ctx) { (void)hipSetDevice(ctx->device); (void)hipStreamSynchronize(ctx->stream); }     // a replay may still be running
+    if (g->exec) (void)hipGraphExecDestroy(g->exec);
+    if (g->graph) (void)hipGraphDestroy(g->graph);
+    for (auto& t : g->tables) { (void)hipFree(t.first); (void)hipHostFree(t.second); }
+    delete g;
+    return AIXK_OK;
+}
+
 int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses)
 {
     AIXK_REQUIRE(ctx != nullptr, "null context");
@@ -377,6 +471,7 @@ int32_t aixk_event_record(aixk_ctx* ctx, aixk_event* ev)
 {
     AIXK_TRY(set_device(ctx));
     AIXK_REQUIRE(ev != nullptr, "event_record: null event");
+    AIXK_REQUIRE(!ctx->capturing, "event_record: no events inside a capture");
     AIXK_HIP(hipEventRecord(ev->ev, ctx->stream));
     return AIXK_OK;
 }

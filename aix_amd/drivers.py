@@ -53,18 +53,44 @@ def _pointer_array(arrays):
     return arr
 
 
-def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data, single_pass=False):
+def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data, single_pass=False, norm_steps=0):
     """Train the MLP (n_in -> hidden -> hidden -> n_out, ReLU, softmax + cross-entropy, Adam) for
     `steps` steps on `dev` from host arrays data = (x, onehot, [w1, w2, w3], [b1, b2, b3]).
     single_pass=True differentiates once per node instead of once per path (the reference's way).
-    Returns (loss per step, seconds per step)."""
+    Returns (loss per step, seconds per step); with norm_steps > 0 also the L2 norms of the gradients of
+    w1, b1, w2, b2, w3, b3 in the first norm_steps steps, [norm_steps, 6]."""
     x, y, w, b = data
     losses = np.zeros(steps, dtype=np.float32)
     secs = np.zeros(steps, dtype=np.float64)
     pw, pb = _pointer_array(w), _pointer_array(b)
+    if norm_steps:
+        lib = load()
+        lib.aixbench_mlp_norms.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int, _PF, _PF, _PPF, _PPF,
+                                           _PF, C.POINTER(C.c_double), _PF, C.c_int]
+        norms = np.zeros((norm_steps, 6), dtype=np.float32)
+        run("aixbench_mlp_norms", dev.handle, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+            pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), norms.ctypes.data_as(_PF), norm_steps)
+        return losses, secs, norms
     run("aixbench_mlp", dev.handle, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
         pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
     return losses, secs
+
+
+def transformer_captured(dev, cfg, steps, data, capture_at, stacked=False):
+    """transformer() with step `capture_at` captured into a HIP graph and that step and all later ones enqueued as replays
+    of it (one launch call per step, no front-end).  Returns (losses, gradient norms, seconds per step, graph nodes)."""
+    tokens, params = data
+    lib = load()
+    lib.aixbench_transformer_captured.argtypes = [C.c_void_p] + [C.c_uint64] * 6 + [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF,
+                                                                               C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
+    losses = np.zeros(steps, np.float32)
+    norms = np.zeros((steps, len(params)), np.float32)
+    secs = np.zeros(steps, np.float64)
+    nodes = C.c_uint64(0)
+    pp = _pointer_array(params)
+    run("aixbench_transformer_captured", dev.handle, *cfg, steps, int(stacked), capture_at, tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp,
+        losses.ctypes.data_as(_PF), norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), C.byref(nodes))
+    return losses, norms, secs, int(nodes.value)
 
 
 def transformer(dev, cfg, steps, data, stacked=False):

@@ -94,6 +94,12 @@ _SIGNATURES = {
     "aixk_sum_columns_many": [_P, _P, C.c_uint32],
     "aixk_matmul": [_P, _T, _T, _T],
     "aixk_matmul_route": [_P, C.POINTER(C.c_int32), C.POINTER(C.c_int32)],
+    "aixk_capture_begin": [_P],
+    "aixk_capture_end": [_P, C.POINTER(_P)],
+    "aixk_capture_abort": [_P],
+    "aixk_graph_launch": [_P, _P],
+    "aixk_graph_nodes": [_P, C.POINTER(C.c_uint64)],
+    "aixk_graph_destroy": [_P, _P],
     "aixk_mfma_only_rate": [_P, C.c_int32, C.c_int32, _P, C.c_uint32, C.c_double, C.POINTER(C.c_float), C.POINTER(C.c_float)],
     "aixk_matmul_batched": [_P, _T, _T, _T],
     "aixk_matmul_grouped": [_P, _T, _T, _T, C.c_uint32],

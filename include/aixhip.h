@@ -142,6 +142,18 @@ int32_t aixhip_fuse_kernel_cache_stats(aixhip_device* dev, uint64_t* hits, uint6
 int32_t aixhip_batched_launch_stats(aixhip_device* dev, uint64_t* launches, uint64_t* kernels);
 /* The kernel-layer context of this device (stream, events) for timing with aixk_event_*. */
 aixk_ctx* aixhip_kernel_context(aixhip_device* dev);
+/* A stretch of the device's work as a HIP graph (no counterpart in the reference, whose GPU device amortises dispatch by
+ * batching into command buffers, aixDeviceMetal.cpp:1344-1389): what is issued between capture_begin and capture_end is
+ * recorded, not run, and aixhip_graph_replay enqueues all of it again -- the same kernels on the same addresses with the
+ * same immediates -- with one call, for steps that repeat exactly (a forward + backward pass, updates in place).  Inside
+ * a capture: no synchronize, no transfer to or from host memory, nothing compiled or grown for the first time (run the
+ * step once before capturing it): status 2.  Blocks that captured work uses stay with the graph: freed, they are not
+ * handed out again until the last graph is destroyed; live tensors are used in place by every replay. */
+typedef struct aixhip_graph aixhip_graph;
+int32_t aixhip_capture_begin(aixhip_device* dev);
+int32_t aixhip_capture_end(aixhip_device* dev, aixhip_graph** out);
+int32_t aixhip_graph_replay(aixhip_device* dev, aixhip_graph* graph);
+int32_t aixhip_graph_destroy(aixhip_device* dev, aixhip_graph* graph);
 int32_t aixhip_memory_stats(aixhip_device* dev, uint64_t* live_bytes, uint64_t* cached_bytes);
 /* The pool of idle blocks is cut back to `bytes` at every synchronize (the reference's GPU device trims its buffer cache
  * to its working-set limit at every commit, aixDeviceMetal.cpp:33, 1369-1373).  Default 0.7 of the card's memory;

@@ -247,6 +247,22 @@ int32_t aixk_rtc_launch_many(aixk_ctx* ctx, aixk_module* mod, uint32_t block_x, 
 const char* aixk_rtc_prelude(void);
 int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);
 
+/* ---- a stretch of the stream as a HIP graph (no counterpart in the reference, whose GPU device amortises dispatch by
+ * batching into command buffers, aixDeviceMetal.cpp:1344-1389) ------------------------------------------------------ */
+/* Between aixk_capture_begin and aixk_capture_end nothing that is enqueued on the context runs: it is recorded, and
+ * aixk_graph_launch enqueues all of it again with one call, on the same addresses with the same arguments.  Inside a
+ * capture: no aixk_sync, no event, no transfer to or from host memory (status AIXK_EHIP from the driver); kernels must
+ * have been compiled and workspaces grown by an earlier, uncaptured run of the same work.  The argument tables of
+ * launches that carry several calls are written when they are captured and kept with the graph; no memset and no copy
+ * node enters a graph through this library except device-to-device copies the caller asks for. */
+typedef struct aixk_graph aixk_graph;
+int32_t aixk_capture_begin(aixk_ctx* ctx);                       /* waits for the stream first */
+int32_t aixk_capture_end(aixk_ctx* ctx, aixk_graph** out);
+int32_t aixk_capture_abort(aixk_ctx* ctx);                       /* drops an open capture; harmless without one */
+int32_t aixk_graph_launch(aixk_ctx* ctx, aixk_graph* graph);
+int32_t aixk_graph_nodes(aixk_graph* graph, uint64_t* nodes);
+int32_t aixk_graph_destroy(aixk_ctx* ctx, aixk_graph* graph);    /* waits for the stream first */
+
 /* ---- the matrix pipe alone (no counterpart in the reference; a measurement aid) ---------------------------------- */
 /* A loop of independent 16-bit MFMAs on register operands, no LDS and no memory traffic, one workgroup per compute unit:
  * the rate the part sustains when it only multiplies -- on a power-limited part a function of the operand values, of the

@@ -823,6 +823,45 @@ int cpuref_matmul_wide(const cpuref_tensor* a, const cpuref_tensor* b, double* o
     });
 }
 
+// cpuref_matmul / cpuref_matmul_stack with the products of every result element added exactly (cpuref_matmul_wide) and
+// rounded ONCE to the element type: what a device that accumulates 16-bit products in a wide type computes, as opposed to
+// the reference's running sum in the element type (aixDeviceCPU.cpp:362-389).  Rank 2 or stacks of matrices.
+int cpuref_matmul_stack_wide(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads)
+{
+    if (a->rank < 2 || a->rank != b->rank || a->rank != out->rank || a->dtype != b->dtype || a->dtype != out->dtype) return CPUREF_EINVAL;
+    const int nb = a->rank - 2;
+    uint64_t count = 1;
+    for (int d = 0; d < nb; ++d) {
+        if (a->shape[d] != b->shape[d] || a->shape[d] != out->shape[d]) return CPUREF_EINVAL;
+        count *= a->shape[d];
+    }
+    auto matrix = [nb](const cpuref_tensor* t) {
+        cpuref_tensor m = *t;
+        m.rank = 2;
+        m.shape[0] = t->shape[nb]; m.shape[1] = t->shape[nb + 1];
+        m.strides[0] = t->strides[nb]; m.strides[1] = t->strides[nb + 1];
+        m.size = m.shape[0] * m.shape[1];
+        return m;
+    };
+    cpuref_tensor a2 = matrix(a), b2 = matrix(b);
+    if (a2.shape[1] != b2.shape[0]) return CPUREF_EINVAL;
+    const uint64_t mn = a2.shape[0] * b2.shape[1], per = mn * cpuref_dtype_size(out->dtype);
+    std::vector<double> exact(mn);
+    for (uint64_t i = 0; i < count; ++i) {
+        uint64_t rest = i, oa = a->offset, ob = b->offset;
+        for (int d = nb - 1; d >= 0; --d) {
+            const uint64_t c = rest % a->shape[d];
+            rest /= a->shape[d];
+            oa += c * a->strides[d]; ob += c * b->strides[d];
+        }
+        a2.offset = oa; b2.offset = ob;
+        int rc = cpuref_matmul_wide(&a2, &b2, exact.data(), nullptr, threads);
+        if (rc == CPUREF_OK) rc = cpuref_copy(exact.data(), CPUREF_F64, (char*)out->data + i * per, out->dtype, mn);     // results are written densely
+        if (rc != CPUREF_OK) return rc;
+    }
+    return CPUREF_OK;
+}
+
 uint64_t cpuref_ulp_hist_f32(const float* x, const float* y, uint64_t n, uint64_t* hist, int nbins)
 {
     auto ordered = [](float f) -> int64_t {       // monotone map float -> integer line

@@ -100,6 +100,12 @@ int cpuref_matmul_rows(const cpuref_tensor* a, const cpuref_tensor* b, const cpu
  * dense from out->data.  Pinned by that function and, for the indexing of the stack, by integer
  * stacks against numpy.matmul (tests/test_oracle_golden.py). */
 int cpuref_matmul_stack(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads);
+/* Not in the reference either: the same products (rank 2 or stacks) with every result element added exactly
+ * (cpuref_matmul_wide) and rounded ONCE to the element type by cpuref_copy's conversion -- what a device that keeps
+ * 16-bit products in a wide accumulator computes, where the reference keeps the running sum in the element type
+ * (aixDeviceCPU.cpp:362-389).  Pinned through the two functions it is composed of and, for the composition, against
+ * float64 numpy products rounded once (tests/test_oracle_wide.py). */
+int cpuref_matmul_stack_wide(const cpuref_tensor* a, const cpuref_tensor* b, const cpuref_tensor* out, int threads);
 
 /* ---- helpers for tests --------------------------------------------------- */
 /* Distance in units in the last place between two f32 arrays: returns the maximum,

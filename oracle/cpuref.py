@@ -137,6 +137,7 @@ _CPUREF_ONLY = {
     "matmul_wide": [_T, _T, C.c_void_p, C.c_void_p, C.c_int],
     "matmul_rows": [_T, _T, _T, C.c_int],
     "matmul_stack": [_T, _T, _T, C.c_int],
+    "matmul_stack_wide": [_T, _T, _T, C.c_int],
 }
 _REF_ONLY = {
     "slice_set": [_T, _T, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64],

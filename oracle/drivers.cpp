@@ -37,12 +37,27 @@ int oracle_mlp(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
 }
 
-// Same contract as aixbench_transformer.
+// Same contract as aixbench_mlp_norms.
+int oracle_mlp_norms(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
+                     const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds,
+                     float* grad_norms, int norm_steps)
+{
+    try {
+        oracle::OracleDevice dev(threads);
+        const aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr, single_pass};
+        const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
+        aixfe::runMlp(&dev, cfg, host, losses, step_seconds, grad_norms, norm_steps);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
+
+// Same contract as aixbench_transformer.  threads < 0: -threads threads and the oracle device's wide16 mode (matmul,
+// reduceTo and sum of 16-bit tensors add exactly and round once; see oracle_device.hpp).
 int oracle_transformer(int threads, uint64_t layers, uint64_t d_model, uint64_t heads, uint64_t seq, uint64_t batch, uint64_t vocab,
                        int steps, int stacked_attention, const int32_t* tokens, const float* const* params, float* losses, float* grad_norms, double* step_seconds)
 {
     try {
-        oracle::OracleDevice dev(threads);
+        oracle::OracleDevice dev(threads < 0 ? -threads : threads, threads < 0);
         const aixfe::TransformerConfig cfg{layers, d_model, heads, seq, batch, vocab, steps, stacked_attention};
         aixfe::runTransformer(&dev, cfg, tokens, params, losses, grad_norms, step_seconds);
         return 0;

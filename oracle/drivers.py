@@ -41,6 +41,8 @@ def oracle_lib():
         _oracle = C.CDLL(path)
         _oracle.oracle_mlp.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int,
                                        _PF, _PF, _PPF, _PPF, _PF, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
+        _oracle.oracle_mlp_norms.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int,
+                                             _PF, _PF, _PPF, _PPF, _PF, C.POINTER(C.c_double), _PF, C.c_int]
         _oracle.oracle_drivers_last_error.restype = C.c_char_p
     return _oracle
 
@@ -59,13 +61,22 @@ def ref_lib():
     return _ref
 
 
-def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pass=False):
-    """Losses per step, seconds per step and (operator calls, matmul calls) of the oracle run."""
+def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pass=False, norm_steps=0):
+    """Losses per step, seconds per step and (operator calls, matmul calls) of the oracle run; with norm_steps > 0
+    instead of the counts the L2 norms of the gradients of w1, b1, w2, b2, w3, b3 in the first norm_steps steps."""
     x, y, w, b = data
     losses = np.zeros(steps, dtype=np.float32)
     secs = np.zeros(steps, dtype=np.float64)
     counts = (C.c_uint64 * 2)()
     pw, pb = pointer_array(w), pointer_array(b)
+    if norm_steps:
+        norms = np.zeros((norm_steps, 6), dtype=np.float32)
+        rc = oracle_lib().oracle_mlp_norms(threads, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF),
+                                           y.ctypes.data_as(_PF), pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)),
+                                           norms.ctypes.data_as(_PF), norm_steps)
+        if rc != 0:
+            raise RuntimeError(oracle_lib().oracle_drivers_last_error().decode())
+        return losses, secs, norms
     rc = oracle_lib().oracle_mlp(threads, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
                                  pw, pb, losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), counts)
     if rc != 0:
@@ -196,8 +207,10 @@ def ref_hip_xor_save_load(hidden1, hidden2, epochs, lr, path):
 
 
 # ---- transformer (configs[4]) ------------------------------------------------------------------------
-def oracle_transformer(cfg, steps, data, threads=1, stacked=False):
-    """cfg = (layers, d, heads, seq, batch, vocab).  Returns (losses, grad norms [steps, P], seconds)."""
+def oracle_transformer(cfg, steps, data, threads=1, stacked=False, wide16=False):
+    """cfg = (layers, d, heads, seq, batch, vocab).  Returns (losses, grad norms [steps, P], seconds).
+    wide16: matmul, reduceTo and sum of 16-bit tensors add their terms exactly and round once (the literal CPU device
+    rounds the running sum to the element type after every addition); everything else as the CPU device has it."""
     tokens, params = data
     lib = oracle_lib()
     lib.oracle_transformer.argtypes = [C.c_int] + [C.c_uint64] * 6 + [C.c_int, C.c_int, C.POINTER(C.c_int32), _PPF, _PF, _PF, C.POINTER(C.c_double)]
@@ -205,7 +218,7 @@ def oracle_transformer(cfg, steps, data, threads=1, stacked=False):
     norms = np.zeros((steps, len(params)), np.float32)
     secs = np.zeros(steps, np.float64)
     pp = pointer_array(params)
-    rc = lib.oracle_transformer(threads, *cfg, steps, int(stacked), tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
+    rc = lib.oracle_transformer(-threads if wide16 else threads, *cfg, steps, int(stacked), tokens.ctypes.data_as(C.POINTER(C.c_int32)), pp, losses.ctypes.data_as(_PF),
                                 norms.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
     if rc != 0:
         raise RuntimeError(lib.oracle_drivers_last_error().decode())

@@ -123,6 +123,23 @@ int32_t aixk_rtc_launch(aixk_ctx* c, aixk_module* m, uint32_t, uint32_t, const v
 STUB_OP(aixk_fill_many, const aixk_fill_item*, uint32_t)
 int32_t aixk_rtc_launch_many(aixk_ctx* c, aixk_module* m, uint32_t, const void*, size_t, size_t, uint32_t) { ++c->launches; c->log += m->entry + "*;"; return AIXK_OK; }
 const char* aixk_rtc_prelude(void) { return ""; }
+// captures: the stub "graph" is the stretch of the launch log recorded between begin and end; a launch appends it again
+struct aixk_graph { std::string log; uint64_t nodes{0}; };
+static thread_local size_t g_capture_from = 0;
+static thread_local uint64_t g_capture_launches = 0;
+static thread_local bool g_capturing = false;
+int32_t aixk_capture_begin(aixk_ctx* c) { if (g_capturing) return AIXK_EINVAL; g_capturing = true; g_capture_from = c->log.size(); g_capture_launches = c->launches; return AIXK_OK; }
+int32_t aixk_capture_end(aixk_ctx* c, aixk_graph** out)
+{
+    if (!g_capturing) return AIXK_EINVAL;
+    g_capturing = false;
+    *out = new aixk_graph{c->log.substr(g_capture_from), c->launches - g_capture_launches};
+    return AIXK_OK;
+}
+int32_t aixk_capture_abort(aixk_ctx*) { g_capturing = false; return AIXK_OK; }
+int32_t aixk_graph_launch(aixk_ctx* c, aixk_graph* g) { c->launches += g->nodes; c->log += g->log; return AIXK_OK; }
+int32_t aixk_graph_nodes(aixk_graph* g, uint64_t* n) { *n = g->nodes; return AIXK_OK; }
+int32_t aixk_graph_destroy(aixk_ctx*, aixk_graph* g) { delete g; return AIXK_OK; }
 int32_t aixk_rtc_stats(aixk_ctx* c, uint64_t* hits, uint64_t* misses) { *hits = c->hits; *misses = c->misses; return AIXK_OK; }
 
 int32_t aixk_event_create(aixk_ctx*, aixk_event** out) { *out = new aixk_event(); return AIXK_OK; }

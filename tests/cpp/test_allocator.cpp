@@ -423,6 +423,63 @@ static void test_the_pool_is_trimmed_to_the_cache_limit()
     CHECK(dev.cachedBytes() == 0 && dev.allocatedBytes() == 0 && stub_held(ctx) == 0);
 }
 
+// A captured step: blocks that the captured work uses may go round inside the capture (everything there is ordered on the
+// stream), but once the capture is closed they are never handed out again while a graph lives -- a replay writes into
+// them -- and come back to the pool when the last graph is destroyed.  Nothing runs inside a capture, so synchronize()
+// refuses; a replay enqueues the captured launches again, in their order.
+static void test_blocks_of_a_captured_step_stay_with_the_graph()
+{
+    DeviceHIP dev;
+    aixk_ctx* ctx = dev.kernelContext();
+    void* a = dev.allocate(64); void* b = dev.allocate(64); void* out = dev.allocate(64);
+    touch(dev, a, b, out);
+    dev.synchronize();
+    stub_log_clear(ctx);
+    dev.beginCapture();
+    CHECK(dev.capturing());
+    CHECK(throws<std::runtime_error>([&] { dev.synchronize(); }));
+    void* t1 = dev.allocate(5000);
+    touch(dev, a, b, t1);                               // captured work writes t1
+    dev.deallocate(t1);
+    dev.flush();
+    void* t2 = dev.allocate(5000);                      // inside the capture the freed block comes round again
+    CHECK(t2 == t1);
+    touch(dev, t2, b, out);
+    dev.deallocate(t2);
+    void* idle = dev.allocate(7000);                    // never used by captured work: an ordinary block
+    dev.deallocate(idle);
+    DeviceHIP::StepGraph* graph = dev.endCapture();
+    CHECK(!dev.capturing() && graph != nullptr && dev.graphNodes(graph) == 2);
+    const std::string captured = stub_log(ctx);
+    const uint64_t allocs = stub_allocs(ctx);
+    void* other = dev.allocate(5000);                   // the graph's temporary is not handed out: a fresh block
+    CHECK(other != t1 && stub_allocs(ctx) == allocs + 1);
+    void* again = dev.allocate(7000);                   // the untouched one is
+    CHECK(again == idle && stub_allocs(ctx) == allocs + 1);
+    stub_log_clear(ctx);
+    dev.replay(graph);
+    dev.replay(graph);
+    CHECK(std::string(stub_log(ctx)) == captured + captured);
+    dev.synchronize();
+    // a live block that captured work uses, freed while the graph lives: set aside as well
+    dev.deallocate(out);
+    dev.synchronize();
+    void* fresh = dev.allocate(64);
+    CHECK(fresh != out);
+    dev.deallocate(other); dev.deallocate(again); dev.deallocate(fresh);
+    dev.destroyGraph(graph);
+    dev.synchronize();
+    void* back = dev.allocate(5000);                    // with the last graph gone its blocks are ordinary idle blocks again
+    CHECK(back == t1 || back == other);
+    std::set<void*> small;
+    for (int i = 0; i < 4; ++i) small.insert(dev.allocate(64));
+    CHECK(small.count(out) == 1);
+    for (void* p : small) dev.deallocate(p);
+    for (void* p : {a, b, back}) dev.deallocate(p);
+    dev.synchronize();
+    CHECK(dev.allocatedBytes() == 0);
+}
+
 static void test_destruction_returns_everything()
 {
     const long long before = stub_held_everywhere();
@@ -450,6 +507,7 @@ int main(int argc, char** argv)
     test_blocks_of_calls_that_wait_are_not_handed_out();
     test_fills_do_not_land_behind_calls_that_wait();
     test_the_pool_is_trimmed_to_the_cache_limit();
+    test_blocks_of_a_captured_step_stay_with_the_graph();
     test_destruction_returns_everything();
     for (unsigned seed = 1; seed <= 4; ++seed) stress(seed, 20000);
     for (unsigned seed = 21; seed <= 24; ++seed) planner_traffic(seed, 3000);

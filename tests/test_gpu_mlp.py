@@ -117,3 +117,35 @@ def test_full_size_mlp_against_the_committed_cpu_trace(dev):
     assert rel[0] <= 1e-5, "first forward pass"
     assert rel[:5].max() <= 1e-4, "first 5 steps"
     assert np.all(rel <= tol), f"steps beyond their bound: {np.flatnonzero(rel > tol).tolist()}"
+
+
+def test_full_size_mlp_early_steps_gradients_and_losses(dev):
+    """Where the arithmetic, not the trajectory, decides: the L2 norms of the six parameters' gradients in steps 0-4 of the
+    full-size configuration and the losses of steps 0-10, against the CPU oracle device's figures committed in
+    tests/golden/mlp_c3_early.json (tests/golden/make_mlp_c3_early.py; its losses equal the 100-step trace bit for bit).
+    Gradient norms of steps 0 and 1: 1e-4 relative (observed 1.4e-5 and 2.4e-5: the composed ReLU's mask flips where a
+    hidden value is within rounding of zero).  From step 2 on the trajectory shows: Adam's first updates move every weight
+    by the learning rate whatever its gradient's size, so gradient entries whose sign differs by rounding put the two
+    runs 2 lr apart in those weights, and the gradients -- far more than the loss, which stays within 1e-4 -- feel it:
+    observed 4.5e-4, 5.8e-4, 2.4e-3 at steps 2, 3, 4, held to 2e-3, 2e-3, 1e-2.  Losses: steps 0-4 1e-4, steps 5-10 1e-3
+    (observed 7e-5; the CPU's own run with 1 % of one weight matrix moved by one unit in the last place is 1e-4 away by
+    step 11)."""
+    import json
+    import os
+    from aix_amd import drivers as GD
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "mlp_c3_early.json")) as f:
+        fixture = json.load(f)
+    batch, n_in, hidden, n_out = fixture["shape"]
+    steps, want_n = fixture["steps"], np.array(fixture["grad_norms"])
+    want_l = np.frombuffer(bytes.fromhex("".join(fixture["losses_hex"])), dtype=np.float32).astype(np.float64)
+    assert fixture["losses_equal_mlp_c3_trace"] and steps == 11 and want_n.shape == (5, 6)
+    data = OD.mlp_data(batch, n_in, hidden, n_out)
+    got_l, _, got_n = GD.mlp(dev, batch, n_in, hidden, n_out, steps, fixture["lr"], data, norm_steps=want_n.shape[0])
+    rel_n = np.abs(got_n.astype(np.float64) - want_n) / want_n
+    rel_l = np.abs(got_l.astype(np.float64) - want_l) / np.abs(want_l)
+    print("gradient norms, relative deviation per step (w1 b1 w2 b2 w3 b3):")
+    for s in range(rel_n.shape[0]):
+        print(f"   step {s}: " + " ".join(f"{v:.1e}" for v in rel_n[s]))
+    print("losses, relative deviation per step:", " ".join(f"{v:.1e}" for v in rel_l))
+    assert np.all(rel_n.max(axis=1) <= np.array([1e-4, 1e-4, 2e-3, 2e-3, 1e-2])), rel_n.max(axis=1)
+    assert rel_l[:5].max() <= 1e-4 and rel_l[5:].max() <= 1e-3

@@ -150,6 +150,34 @@ def test_matmul_wide_against_float64_numpy_on_views(dtype):
     assert np.array_equal(got.reshape(2, 4), np.arange(6.).reshape(2, 3) @ np.arange(12.).reshape(4, 3).T)
 
 
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16, O.F32], ids=lambda d: O.DTYPE_NAMES[d])
+def test_matmul_stack_wide_is_the_exact_product_rounded_once(dtype):
+    """cpuref_matmul_stack_wide = float64 numpy products of the logical contents, rounded once to the element type, for
+    2-D operands and for stacks whose leading dims are permuted or broadcast views (results dense); a case where the
+    reference's running sum in the element type visibly differs (256 terms of 1/256 + 1: bf16 stalls at 1 after the first
+    addition, the exact sum is 2) pins that the sum is NOT kept in the element type."""
+    rng = np.random.default_rng(640 + dtype)
+    for lead in ([], [3], [2, 3]):
+        for kind_a, kind_b in (("contig", "contig"), ("transposed", "contig"), ("sliced", "transposed"), ("contig", "broadcast")):
+            m, k, n = (int(rng.integers(1, 12)) for _ in range(3))
+            a = T.view_tensor(rng, dtype, lead + [m, k], kind_a)
+            b = T.view_tensor(rng, dtype, lead + [k, n], kind_b)
+            out = T.empty(dtype, lead + [m, n])
+            assert CPU.matmul_stack_wide(C.byref(a.desc()), C.byref(b.desc()), C.byref(out.desc()), 2) == 0
+            want = O.to_storage(np.matmul(a.values(), b.values()).reshape(-1), dtype)
+            # (float64 numpy adds in another order than the oracle: the two exact sums may round to neighbouring values at a tie)
+            assert T.ulp_distance(out.storage, want, dtype) <= 1, (lead, kind_a, kind_b)
+    if dtype != O.F32:
+        a = T.HostTensor(O.to_storage(np.array([1.0] + [1.0 / 256] * 256), dtype), dtype, [1, 257])
+        b = T.HostTensor(O.to_storage(np.ones(257), dtype), dtype, [257, 1])
+        wide, literal = T.empty(dtype, [1, 1]), T.empty(dtype, [1, 1])
+        assert CPU.matmul_stack_wide(C.byref(a.desc()), C.byref(b.desc()), C.byref(wide.desc()), 1) == 0
+        assert CPU.matmul(C.byref(a.desc()), C.byref(b.desc()), C.byref(literal.desc())) == 0
+        assert O.to_float64(wide.storage, dtype)[0] == 2.0
+        if dtype == O.BF16:
+            assert O.to_float64(literal.storage, dtype)[0] == 1.0          # the CPU device's own sum never leaves 1
+
+
 def f32_from_bits(*bits):
     return np.array(bits, dtype=np.uint32).view(np.float32)
 
