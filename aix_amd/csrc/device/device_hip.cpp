@@ -1075,6 +1075,7 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         if (!op.whole || op.outputIndex == SIZE_MAX) continue;
         if (nWholes == 8) throw std::logic_error("DeviceHIP: more sums over everything in one kernel than the planner allows");
         const size_t wide = d.dtype == DataType::kFloat64 ? 8 : 4;
+        issueFlatBatch();                                        // (an allocation that runs out of memory waits for the GPU and drops the pool: nothing enqueued may lag behind)
         void* scratch = allocateBlock(grid * wide, false);
         m_limbo.emplace_back(scratch, bucketBytes(grid * wide));     // recycled once the work enqueued below has passed
         m_limboBytes += bucketBytes(grid * wide);
@@ -1320,7 +1321,6 @@ void DeviceHIP::issuePending()
 {
     const Marker marker_("calls that waited leave");
     auto& ex = *m_extras;
-    int status = AIXK_OK;
     if (ex.anyPending()) {
         size_t products = 0, sums = 0;
         for (const auto& g : ex.groups) products += g.out.size();
@@ -1329,32 +1329,40 @@ void DeviceHIP::issuePending()
                      ex.partialSums.size(), products);
         (void)products; (void)sums;
     }
+    // A list that fails does not take the others with it: every call here was accepted earlier and returned normally, so
+    // all of them are sent off, and the first failure is reported afterwards (from whichever operator, flush or
+    // synchronize caused the send-off: errors of calls that wait are reported late).
+    int first = AIXK_OK;
+    std::string firstError;
+    size_t dropped = 0;
+    auto sent = [&](int status, size_t calls) {
+        if (status == AIXK_OK) return;
+        dropped += calls;
+        if (first == AIXK_OK) { first = status; firstError = aixk_last_error(); }
+    };
     if (!ex.slices.empty()) {
-        status = ex.slices.size() == 1 ? aixk_slice_set(m_ctx, &ex.slices[0].src, &ex.slices[0].dst, ex.slices[0].dim, ex.slices[0].start, ex.slices[0].end, ex.slices[0].step)
-                                       : aixk_slice_set_many(m_ctx, ex.slices.data(), (uint32_t)ex.slices.size());
+        sent(ex.slices.size() == 1 ? aixk_slice_set(m_ctx, &ex.slices[0].src, &ex.slices[0].dst, ex.slices[0].dim, ex.slices[0].start, ex.slices[0].end, ex.slices[0].step)
+                                   : aixk_slice_set_many(m_ctx, ex.slices.data(), (uint32_t)ex.slices.size()), ex.slices.size());
         if (ex.slices.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.slices.size(); }
         ex.slices.clear();
     }
     if (!ex.onehots.empty()) {
-        if (status == AIXK_OK)
-            status = ex.onehots.size() == 1 ? aixk_argmax_to(m_ctx, 2, &ex.onehots[0].src, &ex.onehots[0].dst, ex.onehots[0].dim)
-                                            : aixk_argmax_onehot_many(m_ctx, ex.onehots.data(), (uint32_t)ex.onehots.size());
+        sent(ex.onehots.size() == 1 ? aixk_argmax_to(m_ctx, 2, &ex.onehots[0].src, &ex.onehots[0].dst, ex.onehots[0].dim)
+                                    : aixk_argmax_onehot_many(m_ctx, ex.onehots.data(), (uint32_t)ex.onehots.size()), ex.onehots.size());
         if (ex.onehots.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += ex.onehots.size(); }
         ex.onehots.clear();
     }
     if (!ex.partialSums.empty()) {
         auto& sums = ex.partialSums;
-        if (status == AIXK_OK)
-            status = sums.size() == 1 ? aixk_sum_partials(m_ctx, sums[0].partials, sums[0].count, &sums[0].dst, sums[0].init_bits)
-                                      : aixk_sum_partials_many(m_ctx, sums.data(), (uint32_t)sums.size());
+        sent(sums.size() == 1 ? aixk_sum_partials(m_ctx, sums[0].partials, sums[0].count, &sums[0].dst, sums[0].init_bits)
+                              : aixk_sum_partials_many(m_ctx, sums.data(), (uint32_t)sums.size()), sums.size());
         if (sums.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += sums.size(); }
         sums.clear();
     }
     for (auto& sums : ex.colsums) {
         if (sums.empty()) continue;
-        if (status == AIXK_OK)
-            status = sums.size() == 1 ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &sums[0].src, &sums[0].dst, sums[0].init_bits)
-                                      : aixk_sum_columns_many(m_ctx, sums.data(), (uint32_t)sums.size());
+        sent(sums.size() == 1 ? aixk_reduce_to_init(m_ctx, AIXK_SUM, &sums[0].src, &sums[0].dst, sums[0].init_bits)
+                              : aixk_sum_columns_many(m_ctx, sums.data(), (uint32_t)sums.size()), sums.size());
         if (sums.size() > 1) { ++ex.batchedLaunches; ex.batchedKernels += sums.size(); }
         sums.clear();
     }
@@ -1362,11 +1370,14 @@ void DeviceHIP::issuePending()
     for (auto& g : ex.groups) {
         if (g.out.empty()) continue;
         const uint32_t count = (uint32_t)g.out.size();
-        if (status == AIXK_OK)
-            status = count == 1 ? aixk_matmul(m_ctx, &g.a[0], &g.b[0], &g.out[0]) : aixk_matmul_grouped(m_ctx, g.a.data(), g.b.data(), g.out.data(), count);
+        sent(count == 1 ? aixk_matmul(m_ctx, &g.a[0], &g.b[0], &g.out[0]) : aixk_matmul_grouped(m_ctx, g.a.data(), g.b.data(), g.out.data(), count), count);
         g.a.clear(); g.b.clear(); g.out.clear();
     }
-    check(status);
+    if (first == AIXK_OK) return;
+    const std::string msg = "DeviceHIP: " + firstError + " (reported when the calls that waited were sent off: " + std::to_string(dropped) +
+                            " call(s) accepted earlier did not run, their destinations keep what they held)";
+    if (first == AIXK_EINVAL) throw std::invalid_argument(msg);
+    throw std::runtime_error(msg);
 }
 
 void DeviceHIP::transpose(const DeviceTensorParams& a, const DeviceTensorParams& result, size_t dim0, size_t dim1)

@@ -1068,10 +1068,11 @@ int run_all(aixk_ctx* ctx, const aixhip_tensor* a, typename Op::Out* dst, const 
     const bool flat = (sp.rank == 0 || (sp.rank == 1 && sp.stride[0][0] == 1)) && aligned16(ps + sp.offset[0]);
     const bool small = n < (1ull << 31) && view_extent(a) < (1ull << 31);
     constexpr int VEC = vec16<T>::n;
-    unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 16, ctx->scratch_bytes / sizeof(Acc));
+    // with the fixed scratch the grid is cut to what it holds (4096 partial results of 16 bytes: every dtype on parts of up to
+    // 256 compute units runs the grid of the allocating entry point and lands the same bits; beyond that the partial
+    // sums of float types are grouped differently)
+    unsigned max_blocks = (unsigned)std::min<uint64_t>((uint64_t)ctx->cus * 16, (fixed ? kStaticScratchBytes : ctx->scratch_bytes) / sizeof(Acc));
     const unsigned grid = flat ? grid_for(n / VEC + 1, kBlock * 4, max_blocks) : grid_for(n, kBlock * 4, max_blocks);
-    if (fixed && (size_t)grid * sizeof(Acc) > kStaticScratchBytes)
-        return fail(AIXK_EINVAL, "reduce (no-allocation entry point): %u partial results of %zu bytes exceed the %zu-byte static scratch", grid, sizeof(Acc), kStaticScratchBytes);
     Acc* partials = (Acc*)(fixed ? fixed : ctx->scratch);
     if (flat) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, true>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);
     else if (small) hipLaunchKernelGGL((reduce_all_k<Op, T, u32, false>), dim3(grid), dim3(kBlock), 0, ctx->stream, ps, dst, sp, (u64)n, partials, fin);

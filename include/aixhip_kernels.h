@@ -145,11 +145,13 @@ enum aixk_reduce_kind { AIXK_SUM = 0, AIXK_MAX = 1, AIXK_ARGMAX = 2, AIXK_ARGMAX
  * (aixDeviceCPU.cpp:140-152, 244-318).  ARGMAX kinds need an int32 result. */
 int32_t aixk_reduce_all(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out);
 /* No counterpart in the reference: aixk_reduce_all for callers that cannot allocate (code under HIP graph
- * capture, tight serving loops, harnesses that forbid hipMalloc).  Same arguments, same results bit for bit; the
- * partial results of the workgroups go to a 64 KiB static device array instead of the context's pooled scratch,
- * and no hipMalloc / hipFree / allocating library call is made.  Limits: at most 2^31 elements per call, and the
- * launch's partials must fit the array (4096 workgroups x 16 bytes: always on a 256-CU part); beyond either the
- * call returns AIXK_EINVAL.  All calls on one GPU share the array: calls that overlap on one GPU race. */
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  Same arguments; the partial results of the
+ * workgroups go to a 64 KiB static device array instead of the context's pooled scratch, and no hipMalloc / hipFree /
+ * allocating library call is made.  The launch is cut to the workgroups whose partials fit the array (4096 of 16
+ * bytes): on parts of up to 256 compute units that is the launch of aixk_reduce_all and the results are the same bit
+ * for bit; on larger parts 16-byte accumulators (f64 / i64 sums, argmax of 8-byte types) run on fewer workgroups, with
+ * the same result for everything but float sums, whose partial sums are grouped differently.  Limit: at most 2^31
+ * elements per call (AIXK_EINVAL beyond).  All calls on one GPU share the array: calls that overlap on one GPU race. */
 int32_t aixk_reduce_all_noalloc(aixk_ctx* ctx, int kind, const aixhip_tensor* a, const aixhip_tensor* out);
 /* dst (op)= reduction of src over the dims dst lacks: Device::reduceTo / maxTo
  * (aixDeviceCPU.cpp:440-466).  Accumulates INTO dst (caller pre-initialises). kind = SUM|MAX. */
