@@ -630,6 +630,50 @@ def test_argmax_to_family(gpu, dtype):
     gpu.release()
 
 
+@pytest.mark.parametrize("dtype", [O.F32, O.F16, O.BF16], ids=ids)
+def test_argmax_down_wide_columns_split_into_row_chunks(gpu, dtype):
+    """argmax along dim 0 of wide rows whose rows are split into chunks over workgroups, float types: the (value, row)
+    records of a column's chunks are folded by a second stage.  What the fold must get right: the first of equal values
+    across chunks, +0 and -0 as equals, columns of nothing but NaNs and minus infinities (row 0), a leading NaN (row 0),
+    a NaN elsewhere (never wins), a value found in the last chunk only, a kept leading dim, the one-hot form -- and calls
+    in a row on different data (the records live in scratch memory that the next call reuses)."""
+    rng = np.random.default_rng(20500 + dtype)
+    ninf, nan = -np.inf, np.nan
+    for shape, dim in (([1100, 3072], 0), ([3, 700, 2048], 1), ([2000, 2048], 0), ([640, 4096], 0)):
+        R, Cw = shape[dim], shape[-1]
+        for rep in range(2):
+            vals = np.round(rng.uniform(-1, 1, size=shape) * 2) / 2            # five levels: ties everywhere
+            v2 = vals.reshape(-1, R, Cw)
+            v2[:, :, 0] = nan                                                  # nothing but NaNs
+            v2[:, :, 1] = ninf                                                 # nothing but minus infinities
+            v2[:, :, 2] = ninf; v2[:, 0, 2] = nan                              # a leading NaN above minus infinities
+            v2[:, :, 3] = 0.25; v2[:, 0, 3] = nan                              # a leading NaN wins
+            v2[:, :, 4] = 0.25; v2[:, R // 2, 4] = nan                         # a NaN elsewhere never wins: row 0
+            v2[:, :, 5] = -1.0; v2[:, R - 1, 5] = -0.0; v2[:, R - 3, 5] = 0.0  # +0 before -0: the first of the two
+            v2[:, :, 6] = -1.0; v2[:, R - 3, 6] = -0.0; v2[:, R - 1, 6] = 0.0  # -0 before +0: the first of the two
+            v2[:, :, 7] = ninf; v2[:, R - 1, 7] = -60000.0                    # found in the last chunk only
+            v2[:, :, 8] = 0.5                                                  # all equal: row 0
+            v2[:, :, 9] = ninf; v2[:, 5, 9] = np.inf; v2[:, 900 % R, 9] = np.inf
+            src = T.HostTensor(O.to_storage(vals.reshape(-1), dtype), dtype, shape)
+            _, ds = gpu.put(src)
+            keep = [1 if d == dim else e for d, e in enumerate(shape)]
+            want = T.empty(O.I32, keep, fill=-7)
+            okc(CPU.argmax_to(C.byref(src.desc()), C.byref(want.desc()), dim))
+            po, do = gpu.put(T.empty(O.I32, keep, fill=-7))
+            G.run_gpu(gpu, "aixk_argmax_to", 0, G.ref(ds), G.ref(do), dim)
+            got = gpu.fetch(po, want.storage)
+            T.assert_same_bits(got, want.storage, f"argmaxTo {NAMES[dtype]} {shape} dim={dim} call {rep}")
+            lead = got.reshape(-1, Cw)[:, :10]
+            assert (lead[:, [0, 1, 2, 3, 4, 8]] == 0).all() and (lead[:, 5] == R - 3).all() and (lead[:, 6] == R - 3).all() and (lead[:, 7] == R - 1).all()
+            assert (lead[:, 9] == min(5, 900 % R)).all()
+            want = T.empty(O.I32, shape)
+            okc(CPU.argmax_indices_to(C.byref(src.desc()), C.byref(want.desc()), dim))
+            po, do = gpu.put(T.empty(O.I32, shape))
+            G.run_gpu(gpu, "aixk_argmax_to", 1, G.ref(ds), G.ref(do), dim)
+            T.assert_same_bits(gpu.fetch(po, want.storage), want.storage, f"argmaxIndicesTo {NAMES[dtype]} {shape} dim={dim} call {rep}")
+            gpu.release()
+
+
 # ---- matmul ---------------------------------------------------------------------------------------
 MM_SIZES = [(1, 1, 1), (2, 3, 4), (1, 64, 1), (1, 257, 33), (33, 1, 17), (64, 64, 64), (65, 63, 67), (128, 256, 64),
             (257, 129, 513), (100, 300, 50), (512, 512, 512), (31, 1024, 9)]   # incl. DeviceTests.cpp:2806-2875 style edges
