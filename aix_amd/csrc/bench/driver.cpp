@@ -201,6 +201,31 @@ int aixbench_mlp_norms(aixhip_device* handle, uint64_t batch, uint64_t in, uint6
     });
 }
 
+// The whole training step -- zeroGrad, forward, loss, backward, Adam's update -- with Adam in its in-place form
+// (frontend/nn.hpp) and, with capture_at >= 0, step `capture_at` captured into a HIP graph and that step and every later one
+// enqueued by DeviceHIP::replay; capture_at < 0: every step issued eagerly (the run a captured one is compared with).
+int aixbench_mlp_captured(aixhip_device* handle, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
+                          int capture_at, const float* x, const float* y, const float* const* w, const float* const* b, float* losses,
+                          double* step_seconds, uint64_t* graph_nodes)
+{
+    return guarded([&] {
+        DeviceHIP* dev = aix::hip::fromHandle(handle);
+        aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr, single_pass};
+        cfg.adamInPlace = 1;
+        cfg.captureAt = capture_at;
+        const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
+        DeviceHIP::StepGraph* graph = nullptr;
+        aixfe::StepCapture capture;
+        capture.begin = [&] { dev->beginCapture(); };
+        capture.end = [&] { graph = dev->endCapture(); };
+        capture.replay = [&] { dev->replay(graph); };
+        try { aixfe::runMlp(dev, cfg, host, losses, step_seconds, nullptr, 0, capture_at >= 0 ? &capture : nullptr); }
+        catch (...) { if (graph) dev->destroyGraph(graph); throw; }
+        if (graph_nodes) *graph_nodes = graph ? dev->graphNodes(graph) : 0;
+        if (graph) dev->destroyGraph(graph);
+    });
+}
+
 // Config 4: decoder-only transformer forward + backward (frontend/transformer.hpp); params in the order of
 // aixfe::transformerParamShapes; losses[steps], grad_norms[steps * param_count], step_seconds[steps] (may be NULL).
 // stacked_attention = 0: one 2-D matmul per (sequence, head), the reference's interface as it is; 1: matmul on stacks.

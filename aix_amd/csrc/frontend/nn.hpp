@@ -8,6 +8,8 @@
 // max over a leading axis of the pair {x, 0}.
 #pragma once
 
+#include <functional>
+
 #include "autograd.hpp"
 
 #include <cmath>
@@ -59,14 +61,30 @@ private:
 
 // aixOptimizer.hpp:93-159.  All arithmetic is on values (no autograd); `value op scalar` is the
 // value-level form (full-shape fill + binary operator).
+// How a device captures a step and enqueues it again (a HIP graph on the GPU backend); none on a device without it.
+struct StepCapture {
+    std::function<void()> begin, end, replay;
+};
+
+// Adam (aixOptimizer.hpp:112-140).  Two forms of the same update:
+//  * as the reference writes it: m and v are new tensors every step and the bias corrections 1 - beta^t are scalars the
+//    host computes, so every step issues different constants;
+//  * inPlace: m and v are updated where they lie and beta^t lives in device memory (a rank-0 tensor multiplied by beta
+//    every step), so a step is the same device calls on the same addresses every time -- what a captured step needs
+//    (StepCapture).  The arithmetic per element is the same; beta^t is a running f32 product instead of a rounded
+//    double power, which moves the corrections by an ulp or two.
 class Adam {
 public:
-    Adam(std::vector<Tensor> params, float lr = 0.001f, float beta1 = 0.9f, float beta2 = 0.999f, float eps = 1e-8f)
-        : m_params(std::move(params)), m_lr(lr), m_beta1(beta1), m_beta2(beta2), m_eps(eps)
+    Adam(std::vector<Tensor> params, float lr = 0.001f, float beta1 = 0.9f, float beta2 = 0.999f, float eps = 1e-8f, bool inPlace = false)
+        : m_params(std::move(params)), m_lr(lr), m_beta1(beta1), m_beta2(beta2), m_eps(eps), m_inPlace(inPlace)
     {
         for (auto& p : m_params) {
             m_m.push_back(Value::full(p.device(), DataType::kFloat32, p.shape(), 0.0f));
             m_v.push_back(Value::full(p.device(), DataType::kFloat32, p.shape(), 0.0f));
+        }
+        if (m_inPlace && !m_params.empty()) {
+            m_b1t = Value::full(m_params[0].device(), DataType::kFloat32, Shape{}, 1.0f);
+            m_b2t = Value::full(m_params[0].device(), DataType::kFloat32, Shape{}, 1.0f);
         }
     }
 
@@ -75,6 +93,7 @@ public:
     void step()
     {
         ++m_t;
+        if (m_inPlace) return stepInPlace();
         for (size_t i = 0; i < m_params.size(); ++i) {
             Tensor& p = m_params[i];
             if (!p.isRequireGrad()) continue;
@@ -88,10 +107,32 @@ public:
     }
 
 private:
+    void stepInPlace()
+    {
+        if (m_params.empty()) return;
+        Device* dev = m_params[0].device();
+        m_b1t *= Value::full(dev, DataType::kFloat32, Shape{}, m_beta1);
+        m_b2t *= Value::full(dev, DataType::kFloat32, Shape{}, m_beta2);
+        const Value c1 = 1.0f - m_b1t, c2 = 1.0f - m_b2t;                       // rank-0, read by every parameter's update
+        for (size_t i = 0; i < m_params.size(); ++i) {
+            Tensor& p = m_params[i];
+            if (!p.isRequireGrad()) continue;
+            const Value g = p.grad().to(DataType::kFloat32);
+            m_m[i] *= Value::full(dev, DataType::kFloat32, p.shape(), m_beta1);
+            m_m[i] += g.withScalar(&Device::mul, float(1.0 - m_beta1), true);
+            m_v[i] *= Value::full(dev, DataType::kFloat32, p.shape(), m_beta2);
+            m_v[i] += g.withScalar(&Device::mul, float(1.0 - m_beta2), true) * g;
+            const Value mHat = m_m[i] / c1, vHat = m_v[i] / c2;
+            p.value() -= (mHat.withScalar(&Device::mul, m_lr, true) / vHat.sqrt().withScalar(&Device::add, m_eps)).to(p.dtype());
+        }
+    }
+
     std::vector<Tensor> m_params;
     float m_lr, m_beta1, m_beta2, m_eps;
+    bool m_inPlace;
     size_t m_t{0};
     std::vector<Value> m_m, m_v;
+    Value m_b1t, m_b2t;
 };
 
 } // namespace aixfe

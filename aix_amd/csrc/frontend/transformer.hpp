@@ -35,12 +35,6 @@ struct TransformerConfig {
     int32_t captureAt{-1};        // >= 0 (and a StepCapture given): that step is captured, it and every later one is a replay
 };
 
-// How a device captures a step and enqueues it again (a HIP graph on the GPU backend); none on a device without it.
-// The step here repeats exactly -- same operators on the same tensors, gradients zeroed and accumulated in place, no
-// host-side scalar that changes -- so a replay computes what issuing it again would.
-struct StepCapture {
-    std::function<void()> begin, end, replay;
-};
 
 // Parameter order (all f32, row-major):
 //   wte [vocab, d], wpe [seq, d],

@@ -83,6 +83,9 @@ struct aixk_ctx {
     // runtime-compiled kernels by signature
     std::unordered_map<std::string, aixk_module*> rtc;
     uint64_t rtc_hits{0}, rtc_misses{0};
+    // code objects of generated kernels kept on disk (AIXHIP_KERNEL_CACHE_DIR, read when the context is created; empty: off)
+    std::string rtc_disk_dir;
+    uint64_t rtc_disk_hits{0}, rtc_disk_stores{0};
 };
 
 struct aixk_module { aixk::RtcModule m; };

@@ -2,7 +2,12 @@
 
 #include "common.hpp"
 
+#include <cstdio>
 #include <cstdlib>
+#include <cstring>
+#include <string>
+#include <sys/stat.h>
+#include <unistd.h>
 
 #include <hip/hiprtc.h>
 
@@ -128,6 +133,12 @@ int32_t aixk_create(int device_index, aixk_ctx** out)
         AIXK_HIP(hipGetDeviceProperties(&ctx->prop, device_index));
         ctx->cus = ctx->prop.multiProcessorCount > 0 ? ctx->prop.multiProcessorCount : 256;
         AIXK_HIP(hipStreamCreateWithFlags(&ctx->stream, hipStreamNonBlocking));
+        if (const char* dir = std::getenv("AIXHIP_KERNEL_CACHE_DIR"); dir && *dir) {
+            ctx->rtc_disk_dir = dir;
+            while (ctx->rtc_disk_dir.size() > 1 && ctx->rtc_disk_dir.back() == '/') ctx->rtc_disk_dir.pop_back();
+            for (size_t at = 1; at <= ctx->rtc_disk_dir.size(); ++at)          // mkdir -p; an unusable directory only costs the cache
+                if (at == ctx->rtc_disk_dir.size() || ctx->rtc_disk_dir[at] == '/') (void)mkdir(ctx->rtc_disk_dir.substr(0, at).c_str(), 0777);
+        }
         ctx->scratch_bytes = 64u << 20;
         AIXK_HIP(hipMalloc(&ctx->scratch, ctx->scratch_bytes));
         AIXK_HIP(hipMalloc((void**)&ctx->counter, 256));
@@ -287,6 +298,75 @@ int32_t aixk_sync(aixk_ctx* ctx)
 // ---- hipRTC -----------------------------------------------------------------------------------
 const char* aixk_rtc_prelude(void) { return kPrelude; }
 
+// Code objects on disk.  A generated kernel takes 30-150 ms to compile and a model's first step compiles dozens of them;
+// with AIXHIP_KERNEL_CACHE_DIR set, each code object is also written to <dir>/<128-bit name>.aixk and a later process
+// loads it instead of compiling.  The name is a hash of everything the code depends on: the device header, the source,
+// the target, the compiler's options and the compiler's version.  A file is header + size + hash of the payload + payload,
+// written under a temporary name and renamed, so a reader never sees half a file and a damaged one is ignored (the kernel
+// is compiled and the file replaced).
+namespace {
+
+uint64_t fnv1a(const void* data, size_t n, uint64_t h)
+{
+    const unsigned char* p = (const unsigned char*)data;
+    for (size_t i = 0; i < n; ++i) { h ^= p[i]; h *= 0x100000001b3ull; }
+    return h;
+}
+
+const char kDiskMagic[8] = {'A', 'I', 'X', 'K', 'C', 'O', '0', '1'};
+
+std::string disk_name(const aixk_ctx* ctx, const char* source, const char* arch, const char* const* opts, int nopts)
+{
+    int major = 0, minor = 0;
+    (void)hiprtcVersion(&major, &minor);
+    uint64_t h[2] = {0xcbf29ce484222325ull, 0x84222325cbf29ce4ull};
+    for (uint64_t& x : h) {
+        x = fnv1a(kPrelude, std::strlen(kPrelude), x);
+        x = fnv1a(source, std::strlen(source) + 1, x);
+        x = fnv1a(arch, std::strlen(arch) + 1, x);
+        for (int i = 0; i < nopts; ++i) x = fnv1a(opts[i], std::strlen(opts[i]) + 1, x);
+        x = fnv1a(&major, sizeof major, x);
+        x = fnv1a(&minor, sizeof minor, x);
+        x = fnv1a(&x, sizeof x, x);                      // the two lanes start apart and stay apart
+    }
+    char name[40];
+    std::snprintf(name, sizeof name, "%016llx%016llx.aixk", (unsigned long long)h[0], (unsigned long long)h[1]);
+    return ctx->rtc_disk_dir + "/" + name;
+}
+
+bool disk_load(const std::string& path, std::vector<char>& code)
+{
+    std::FILE* f = std::fopen(path.c_str(), "rb");
+    if (!f) return false;
+    char magic[8];
+    uint64_t size = 0, hash = 0;
+    bool ok = std::fread(magic, 1, 8, f) == 8 && std::memcmp(magic, kDiskMagic, 8) == 0 && std::fread(&size, 8, 1, f) == 1 &&
+              std::fread(&hash, 8, 1, f) == 1 && size > 0 && size < (1ull << 30);
+    if (ok) {
+        code.resize(size);
+        ok = std::fread(code.data(), 1, size, f) == size && std::fgetc(f) == EOF && fnv1a(code.data(), size, 0xcbf29ce484222325ull) == hash;
+    }
+    std::fclose(f);
+    if (!ok) code.clear();
+    return ok;
+}
+
+bool disk_store(const std::string& path, const std::vector<char>& code)
+{
+    const std::string tmp = path + ".tmp." + std::to_string((long)getpid());
+    std::FILE* f = std::fopen(tmp.c_str(), "wb");
+    if (!f) return false;
+    const uint64_t size = code.size(), hash = fnv1a(code.data(), code.size(), 0xcbf29ce484222325ull);
+    bool ok = std::fwrite(kDiskMagic, 1, 8, f) == 8 && std::fwrite(&size, 8, 1, f) == 1 && std::fwrite(&hash, 8, 1, f) == 1 &&
+              std::fwrite(code.data(), 1, code.size(), f) == code.size();
+    ok = (std::fclose(f) == 0) && ok;
+    if (ok) ok = std::rename(tmp.c_str(), path.c_str()) == 0;
+    if (!ok) (void)std::remove(tmp.c_str());
+    return ok;
+}
+
+} // namespace
+
 int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const char* entry, aixk_module** out, int32_t* was_cached)
 {
     AIXK_TRY(set_device(ctx));
@@ -301,18 +381,40 @@ int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const c
     ++ctx->rtc_misses;
     if (was_cached) *was_cached = 0;
 
-    hiprtcProgram prog;
-    const char* header_names[] = {"aix_device.h"};
-    const char* header_texts[] = {kPrelude};
-    hiprtcResult r = hiprtcCreateProgram(&prog, source, "aix_fused.hip", 1, header_texts, header_names);
-    if (r != HIPRTC_SUCCESS) return fail(AIXK_EHIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
     std::string arch = std::string("--offload-arch=") + (ctx->prop.gcnArchName[0] ? ctx->prop.gcnArchName : "gfx950");
     // IEEE arithmetic: no contraction (a*b+c stays two roundings), no fast-math, correctly rounded
     // division and square root, no packed-f32 instruction selection.
     const char* opts[] = {arch.c_str(), "-O3", "-std=c++17", "-ffp-contract=off", "-fno-fast-math",
                           "-fhip-fp32-correctly-rounded-divide-sqrt",
                           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
-    r = hiprtcCompileProgram(prog, (int)(sizeof(opts) / sizeof(opts[0])), opts);
+    const int nopts = (int)(sizeof(opts) / sizeof(opts[0]));
+
+    // a code object an earlier process left on disk
+    const std::string disk_path = ctx->rtc_disk_dir.empty() ? std::string() : disk_name(ctx, source, arch.c_str(), opts, nopts);
+    if (!disk_path.empty()) {
+        std::vector<char> kept;
+        if (disk_load(disk_path, kept)) {
+            aixk_module* mod = new aixk_module();
+            hipError_t e = hipModuleLoadData(&mod->m.module, kept.data());
+            if (e == hipSuccess) e = hipModuleGetFunction(&mod->m.fn, mod->m.module, entry);
+            if (e == hipSuccess) {
+                ++ctx->rtc_disk_hits;
+                ctx->rtc.emplace(key, mod);
+                *out = mod;
+                return AIXK_OK;
+            }
+            if (mod->m.module) (void)hipModuleUnload(mod->m.module);     // not loadable here: compile, and replace the file
+            delete mod;
+            (void)hipGetLastError();
+        }
+    }
+
+    hiprtcProgram prog;
+    const char* header_names[] = {"aix_device.h"};
+    const char* header_texts[] = {kPrelude};
+    hiprtcResult r = hiprtcCreateProgram(&prog, source, "aix_fused.hip", 1, header_texts, header_names);
+    if (r != HIPRTC_SUCCESS) return fail(AIXK_EHIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+    r = hiprtcCompileProgram(prog, nopts, opts);
     if (r != HIPRTC_SUCCESS) {
         size_t n = 0;
         hiprtcGetProgramLogSize(prog, &n);
@@ -337,6 +439,15 @@ int32_t aixk_rtc_get(aixk_ctx* ctx, const char* key, const char* source, const c
     }
     ctx->rtc.emplace(key, mod);
     *out = mod;
+    if (!disk_path.empty() && disk_store(disk_path, code)) ++ctx->rtc_disk_stores;     // a cache that cannot be written is no error
+    return AIXK_OK;
+}
+
+int32_t aixk_rtc_disk_stats(aixk_ctx* ctx, uint64_t* loaded, uint64_t* stored)
+{
+    AIXK_REQUIRE(ctx != nullptr, "rtc_disk_stats: null context");
+    if (loaded) *loaded = ctx->rtc_disk_hits;
+    if (stored) *stored = ctx->rtc_disk_stores;
     return AIXK_OK;
 }
 

@@ -76,6 +76,23 @@ def mlp(dev, batch, n_in, hidden, n_out, steps, lr, data, single_pass=False, nor
     return losses, secs
 
 
+def mlp_captured(dev, batch, n_in, hidden, n_out, steps, lr, data, capture_at, single_pass=False):
+    """mlp() with Adam in its in-place form (state updated where it lies, beta^t kept in device memory) and, with
+    capture_at >= 0, step `capture_at` -- zeroGrad, forward, loss, backward and the update -- captured into a HIP graph and
+    that step and every later one enqueued as a replay of it; capture_at < 0 issues every step eagerly.
+    Returns (loss per step, seconds per step, graph nodes)."""
+    x, y, w, b = data
+    lib = load()
+    lib.aixbench_mlp_captured.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int, C.c_int, _PF, _PF,
+                                          _PPF, _PPF, _PF, C.POINTER(C.c_double), C.POINTER(C.c_uint64)]
+    losses = np.zeros(steps, dtype=np.float32)
+    secs = np.zeros(steps, dtype=np.float64)
+    nodes = C.c_uint64(0)
+    run("aixbench_mlp_captured", dev.handle, batch, n_in, hidden, n_out, steps, lr, int(single_pass), capture_at, x.ctypes.data_as(_PF),
+        y.ctypes.data_as(_PF), _pointer_array(w), _pointer_array(b), losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)), C.byref(nodes))
+    return losses, secs, int(nodes.value)
+
+
 def transformer_captured(dev, cfg, steps, data, capture_at, stacked=False):
     """transformer() with step `capture_at` captured into a HIP graph and that step and all later ones enqueued as replays
     of it (one launch call per step, no front-end).  Returns (losses, gradient norms, seconds per step, graph nodes)."""

@@ -107,6 +107,7 @@ _SIGNATURES = {
     "aixk_rtc_launch": [_P, _P, C.c_uint32, C.c_uint32, _P, C.c_size_t],
     "aixk_rtc_launch_many": [_P, _P, C.c_uint32, _P, C.c_size_t, C.c_size_t, C.c_uint32],
     "aixk_rtc_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
+    "aixk_rtc_disk_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],
     "aixk_event_create": [_P, C.POINTER(_P)],
     "aixk_event_record": [_P, _P],
     "aixk_event_query": [_P, _P, C.POINTER(C.c_int32)],

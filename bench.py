@@ -441,8 +441,21 @@ def main():
         mlp["roofline"]["note"] = ("issued work: the reference's backward recursion differentiates once per path, so the five backward products run "
                                    f"4 times ({flops_step / 1e9:.0f} GFLOP per step, what AIX issues on any device); one traversal would need "
                                    f"{useful / 1e9:.0f} GFLOP (useful_TFLOPs). The products run on the split-plane bf16 route, hence its peak.")
+        # the whole training step captured into a HIP graph once and replayed (Adam in its in-place form: state updated where it
+        # lies, beta^t in device memory), against the same program issued eagerly
+        cap_steps, cap_at = 40, 5
+        eager_l, eager_s, _ = GD.mlp_captured(dev, *shape, cap_steps, 1e-3, data, -1)
+        cap_l, cap_s, nodes = GD.mlp_captured(dev, *shape, cap_steps, 1e-3, data, cap_at)
+        replayed = float(np.median(cap_s[cap_at + 2:]))
+        mlp["captured_step_replayed"] = {"ms_per_step": round(replayed * 1e3, 4), "value": round(1.0 / replayed, 2), "unit": "steps/s", "graph_nodes": nodes,
+                                         "eager_ms_per_step": round(float(np.median(eager_s[cap_at + 2:])) * 1e3, 4),
+                                         "equals_the_eager_steps_bit_for_bit": bool(np.array_equal(eager_l, cap_l)),
+                                         "note": "zeroGrad, forward, loss, backward and Adam's update of step 5 captured (an extension: aixhip_capture_begin / "
+                                                 "_end), steps 5-39 are aixhip_graph_replay calls; all 40 losses compared with 40 eager steps"}
         extras.append(mlp)
         targets["c3_steps_per_s"] = mlp["value"]
+        targets["c3_replayed_steps_per_s"] = mlp["captured_step_replayed"]["value"]
+        targets["c3_replayed_equals_eager"] = mlp["captured_step_replayed"]["equals_the_eager_steps_bit_for_bit"]
         targets["c3_loss_ok"] = mlp["parity"]["ok"] if "parity" in mlp else None
         targets["c3_loss_max_rel_dev_first_steps"] = mlp["parity"]["max_rel_dev"] if "parity" in mlp else None
     if not args.no_extras and chosen & {"c4", "c4loop", "c4stack"}:

@@ -248,6 +248,13 @@ int32_t aixk_rtc_launch_many(aixk_ctx* ctx, aixk_module* mod, uint32_t block_x, 
 /* The device-side header every generated kernel is compiled against (types, conversions, math). */
 const char* aixk_rtc_prelude(void);
 int32_t aixk_rtc_stats(aixk_ctx* ctx, uint64_t* hits, uint64_t* misses);
+/* No counterpart in the reference (its kernel cache lives in memory and every process compiles its generated kernels
+ * anew, aixDeviceMetalKernelGen.cpp:716-768): with AIXHIP_KERNEL_CACHE_DIR set when the context is created, the
+ * code object of every kernel aixk_rtc_get compiles is also kept in that directory, named by a hash of the device header,
+ * the source, the target, the compiler's options and version, and a later context (or process) loads it instead of
+ * compiling.  A missing, damaged or unloadable file means a compilation, never an error.  loaded / stored: how many code
+ * objects this context took from / wrote to the directory. */
+int32_t aixk_rtc_disk_stats(aixk_ctx* ctx, uint64_t* loaded, uint64_t* stored);
 
 /* ---- a stretch of the stream as a HIP graph (no counterpart in the reference, whose GPU device amortises dispatch by
  * batching into command buffers, aixDeviceMetal.cpp:1344-1389) ------------------------------------------------------ */

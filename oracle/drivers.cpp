@@ -37,6 +37,21 @@ int oracle_mlp(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64
     } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
 }
 
+// The same training loop with Adam in its in-place form (frontend/nn.hpp: state updated where it lies, beta^t in device
+// memory), every step issued: what aixbench_mlp_captured's eager and replayed steps are compared with.
+int oracle_mlp_in_place(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
+                        const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds)
+{
+    try {
+        oracle::OracleDevice dev(threads);
+        aixfe::MlpConfig cfg{batch, in, hidden, out, steps, lr, single_pass};
+        cfg.adamInPlace = 1;
+        const aixfe::MlpHost host{x, y, {w[0], w[1], w[2]}, {b[0], b[1], b[2]}};
+        aixfe::runMlp(&dev, cfg, host, losses, step_seconds);
+        return 0;
+    } catch (const std::exception& e) { std::snprintf(g_err, sizeof(g_err), "%s", e.what()); return 1; }
+}
+
 // Same contract as aixbench_mlp_norms.
 int oracle_mlp_norms(int threads, uint64_t batch, uint64_t in, uint64_t hidden, uint64_t out, int steps, float lr, int single_pass,
                      const float* x, const float* y, const float* const* w, const float* const* b, float* losses, double* step_seconds,

@@ -84,6 +84,22 @@ def oracle_mlp(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pa
     return losses, secs, (int(counts[0]), int(counts[1]))
 
 
+def oracle_mlp_in_place(batch, n_in, hidden, n_out, steps, lr, data, threads=1, single_pass=False):
+    """oracle_mlp with Adam in its in-place form (state updated where it lies, beta^t kept in device memory): losses per
+    step and seconds per step."""
+    x, y, w, b = data
+    losses = np.zeros(steps, dtype=np.float32)
+    secs = np.zeros(steps, dtype=np.float64)
+    lib = oracle_lib()
+    lib.oracle_mlp_in_place.argtypes = [C.c_int, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, C.c_float, C.c_int, _PF, _PF,
+                                        C.POINTER(_PF), C.POINTER(_PF), _PF, C.POINTER(C.c_double)]
+    rc = lib.oracle_mlp_in_place(threads, batch, n_in, hidden, n_out, steps, lr, int(single_pass), x.ctypes.data_as(_PF), y.ctypes.data_as(_PF),
+                                 pointer_array(w), pointer_array(b), losses.ctypes.data_as(_PF), secs.ctypes.data_as(C.POINTER(C.c_double)))
+    if rc != 0:
+        raise RuntimeError(lib.oracle_drivers_last_error().decode())
+    return losses, secs
+
+
 def oracle_slice_gradients(which, rows, cols, x, w):
     """(gradient by the reference's recursion, gradient by the single-pass traversal) of slicing program `which`."""
     out = np.zeros((2, rows, cols), dtype=np.float32)

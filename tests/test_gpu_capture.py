@@ -94,3 +94,27 @@ def test_captured_updates_in_place_advance_step_by_step(dev):
     dev.dev.call("graph_destroy", extra)
     dev.dev.call("graph_destroy", graph)
     dev.release()
+
+
+@pytest.mark.parametrize("cfg,single_pass", [((256, 64, 128, 10), False), ((512, 96, 256, 10), True), ((4096, 784, 2048, 10), False)], ids=str)
+def test_replays_of_a_captured_training_step_equal_the_eager_steps(dev, cfg, single_pass):
+    """A whole training step of the MLP -- zeroGrad, forward, softmax + cross-entropy, backward, Adam's update -- with
+    Adam in its in-place form (its state updated where it lies, beta^t in device memory, so nothing the host computes
+    changes from step to step): steps 0-2 eager, step 3 captured, steps 3-7 replays.  The losses must equal, bit for bit,
+    those of eight eager steps of the same program, i.e. every replay advanced parameters, Adam's moments and beta^t
+    exactly as issuing the step would; and they follow the CPU device running the same program.  The last case is the
+    benchmark's full-size network (the three-plane f32 GEMM route, K splits, the workspace the eager steps grew)."""
+    from aix_amd import drivers as GD
+    steps, at = 8, 3
+    data = OD.mlp_data(*cfg)
+    eager, _, none = GD.mlp_captured(dev.dev, *cfg, steps, 1e-3, data, -1, single_pass=single_pass)
+    got, secs, nodes = GD.mlp_captured(dev.dev, *cfg, steps, 1e-3, data, at, single_pass=single_pass)
+    print(f"mlp {cfg}: {nodes} graph nodes; eager step {np.median(secs[1:at]) * 1e3:.2f} ms, replayed step {np.median(secs[at + 1:]) * 1e3:.2f} ms; losses {got}")
+    assert none == 0 and nodes > 10
+    assert np.all(np.isfinite(got)) and got[-1] < got[0]
+    assert np.array_equal(got, eager), (got, eager)
+    if cfg[0] * cfg[2] <= 1 << 17:                               # the CPU device finishes these in a second
+        want, _ = OD.oracle_mlp_in_place(*cfg, steps, 1e-3, data, threads=8, single_pass=single_pass)
+        rel = np.abs(got.astype(np.float64) - want) / np.abs(want)
+        print("   against the CPU device, relative:", " ".join(f"{v:.1e}" for v in rel))
+        assert rel[0] <= 1e-5 and rel.max() <= 1e-4

@@ -6,6 +6,7 @@ synchronize() -- and check results, fusion diagnostics, error behaviour and memo
 Patterns follow Targets/AIXTests/DeviceTests.cpp (queue tests :3074-3552, fusion tests :1774-1910).
 """
 import ctypes as C
+import os
 
 import numpy as np
 import pytest
@@ -1053,3 +1054,59 @@ def test_a_fill_of_the_destination_never_lands_behind_a_call_that_waits(dev):
         assert CPU.slice_set(C.byref(part.desc()), C.byref(whole.desc()), 0, 8, 24, 1, 1) == 0
         T.assert_same_bits(dev.fetch(pw, whole.storage), whole.storage, f"fill through another view + sliceSet, {NAMES[dtype]}")
     dev.release()
+
+
+def test_generated_kernels_are_kept_on_disk_between_contexts(tmp_path):
+    """With AIXHIP_KERNEL_CACHE_DIR set when a device is created, the code object of every kernel it compiles is kept in that
+    directory and a later device (a later process) loads it instead of compiling: the second device compiles nothing,
+    stores nothing and computes the same bits.  Damaged files -- cut short, a flipped byte, an empty file -- are ignored:
+    the third device compiles again, replaces them and computes the same bits."""
+    where = tmp_path / "kept" / "kernels"
+    rng = np.random.default_rng(34000)
+    shape = [96, 130]
+    host = T.contiguous_tensor(rng, O.F32, shape)
+    klib = K.load()
+
+    def one_device():
+        d = H.Dev()
+        try:
+            rec = Recorder(d, O.F32, shape)
+            a = rec.leaf(host)
+            y = rec.binary(O.ADD, rec.unary(O.COS, rec.binary(O.MUL, rec.scalar(0.5), a)), rec.scalar(0.25))
+            z = rec.unary(O.EXP, rec.binary(O.SUB, y, a))                       # a second kernel after a flush
+            rec.free_temps(keep=(y, z))
+            got = (d.fetch(y["ptr"], y["host"].storage).copy(), d.fetch(z["ptr"], z["host"].storage).copy())
+            assert T.ulp_distance(got[0], y["host"].storage, O.F32) <= 2
+            loaded, stored = C.c_uint64(), C.c_uint64()
+            assert klib.aixk_rtc_disk_stats(d.dev.kernel_context(), C.byref(loaded), C.byref(stored)) == 0
+            return got, loaded.value, stored.value
+        finally:
+            d.close()
+
+    os.environ["AIXHIP_KERNEL_CACHE_DIR"] = str(where) + "//"
+    try:
+        first, loaded, stored = one_device()
+        files = sorted(where.glob("*.aixk"))
+        assert loaded == 0 and stored >= 1 and len(files) == stored, (loaded, stored, files)
+        assert not list(where.glob("*.tmp.*"))
+        second, loaded, stored2 = one_device()
+        assert loaded == stored and stored2 == 0, (loaded, stored, stored2)
+        for x, y in zip(first, second):
+            T.assert_same_bits(x, y, "a kernel loaded from disk")
+        for k, f in enumerate(files):
+            blob = f.read_bytes()
+            if k % 3 == 0:
+                f.write_bytes(blob[:len(blob) // 2])
+            elif k % 3 == 1:
+                f.write_bytes(blob[:100] + bytes([blob[100] ^ 0x40]) + blob[101:])
+            else:
+                f.write_bytes(b"")
+        third, loaded, stored3 = one_device()
+        assert loaded == 0 and stored3 == stored, (loaded, stored3)
+        for x, y in zip(first, third):
+            T.assert_same_bits(x, y, "a kernel compiled again over a damaged file")
+        assert all(f.stat().st_size > 1000 for f in files)
+    finally:
+        del os.environ["AIXHIP_KERNEL_CACHE_DIR"]
+    _, loaded, stored = one_device()
+    assert loaded == 0 and stored == 0, "no directory named: nothing is read or written"
