@@ -389,6 +389,219 @@ __global__ __launch_bounds__(512) void gemm_nt16_direct_k(GemmArgs g)
         }
     }
 }
+
+// The same scheme for results that 256 x 256 tiles cannot spread over the chip: BM x BN tiles with BM = 128 and BN = 128,
+// 192 or 256 (the widths of a d = 768 model are multiples of 192, not of 256), still eight waves in a 2 x 4 arrangement,
+// a wave on 64 x BN / 4 as 4 x (BN / 64) tiles of 16 x 16, K-steps of 64 through two LDS stages filled by LDS-direct
+// loads, both operand forms consumed where they lie.  What changes with the tile:
+//  * a wave issues BM / 64 loads of A and BN / 64 of B per tile; with an odd count the parity of a load's 8-row block,
+//    which picks one of the two producer swizzles, follows the wave's number (the two offsets are swapped once);
+//  * a T-form stage keeps k-rows of 2 BM (2 BN) bytes, so a load covers 1024 / pitch k-rows and every load has its own
+//    lane -> (k-row, chunk) map (kept in a register per load); rows of 256 and 512 bytes fall on the same banks and
+//    use the slot c ^ 4 (k & 3) ^ 2 ((k >> 3) & 1) of the 256 x 256 kernel; rows of 384 bytes alternate between two
+//    halves of the banks by themselves and use c ^ 4 ((k >> 1) & 1) ^ 2 ((k >> 3) & 1), which also stays inside the
+//    row's 8-chunk groups (24 chunks do not hold a 16-chunk group);
+//  * the T-form fragment addresses are kept per 16-column block (the block's chunk enters before the swizzle, and with
+//    BN / 4 = 48 columns per wave it cannot be folded in by XOR).
+template <int P> __device__ __forceinline__ int tform_swizzle(int k_low3, int k_bit3)
+{
+    if constexpr (P == 384) return (4 * ((k_low3 >> 1) & 1)) ^ (2 * k_bit3);
+    else return (4 * (k_low3 & 3)) ^ (2 * k_bit3);
+}
+
+template <int OFF> __device__ __forceinline__ u32x4 tr_fragment_at(const unsigned char* lds_addr)
+{
+    const u32 addr = (u32)(size_t)(__attribute__((address_space(3))) const unsigned char*)lds_addr;
+    u32x2 lo, hi;
+    asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "i"(OFF));       // k + 4
+    return u32x4{lo.x, lo.y, hi.x, hi.y};
+}
+
+template <class T, bool AT, bool BT, int BM, int BN>
+__global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
+{
+    static_assert(BM == 128 && (BN == 128 || BN == 192 || BN == 256), "tiles this kernel is written for");
+    constexpr int BK = 64, ASZ = BM * 128, BSZ = BN * 128, STAGE = ASZ + BSZ;
+    constexpr int WGN = 4, TI = BM / 32, TJ = BN / 64, WROWS = TI * 16, WCOLS = TJ * 16;
+    constexpr int LHA = BM / 64, LHB = BN / 64, LPW = LHA + LHB;     // loads per wave and tile
+    constexpr int NF = TI + TJ, NB = 4;                              // fragments per slice; sub-blocks per phase
+    constexpr int PA = 2 * BM, PB = 2 * BN;                          // bytes per k-row of a T-form stage
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    u32 tm, tn;
+    tile_of(g, tm, tn);
+    const u64 m0 = (u64)tm * BM, n0 = (u64)tn * BN;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), wm = wave / WGN, wn = wave % WGN;
+    // blockIdx.y numbers the matrices of a stack, or the separate products of a group (addresses from a table)
+    u64 base_a = (u64)(size_t)g.a, base_b = (u64)(size_t)g.b, base_c = (u64)(size_t)g.c;
+    if (bt.table) {
+        const u64* entry = bt.table + 3 * (u64)blockIdx.y;
+        base_a = entry[0]; base_b = entry[1]; base_c = entry[2];
+    } else if (bt.rank) {
+        u32 rest = blockIdx.y;
+        for (int d = (int)bt.rank - 1; d >= 0; --d) {
+            const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
+            base_a += (u64)c * bt.sa[d] * 2; base_b += (u64)c * bt.sb[d] * 2;
+            rest = q;
+        }
+        base_c += (u64)blockIdx.y * bt.sc * 2;
+    }
+    const char* ga = global_ptr<const char>(base_a);
+    const char* gb = global_ptr<const char>(base_b);
+
+    // producer.  K-contiguous: load n of a wave fills the 8-row block wave * LH + n (128 bytes per row, 8 lanes per row);
+    // T form: the wave fills k-rows 8 wave .. 8 wave + 7, load n the bytes 1024 n .. 1024 n + 1023 of them.
+    const int lr = lane >> 3;
+    const int fe = (lr >> 1) ^ ((lr & 1) << 2);
+    u32 oa[AT ? LHA : 2], ob[BT ? LHB : 2];
+    const char* A;
+    const char* B;
+    if constexpr (AT) {
+        A = ga + m0 * 2 + (u64)(wave * 8) * g.lda * 2;
+#pragma unroll
+        for (int n = 0; n < LHA; ++n) {
+            const int pos = n * 1024 + lane * 16, kq = pos / PA, slot = (pos % PA) / 16;
+            oa[n] = (u32)((kq * g.lda + (u64)((slot ^ tform_swizzle<PA>(kq, wave & 1)) * 8)) * 2);
+        }
+    } else {
+        A = ga + (m0 + (u64)wave * LHA * 8) * g.lda * 2;
+        const int par = (LHA & 1) ? (wave & 1) : 0;                  // parity of the wave's first block
+        oa[0] = (u32)((lr * g.lda + (u64)(((lane & 7) ^ fe ^ (4 * par)) * 8)) * 2);
+        oa[1] = (u32)((lr * g.lda + (u64)(((lane & 7) ^ fe ^ (4 * par) ^ 4) * 8)) * 2);
+    }
+    if constexpr (BT) {
+        B = gb + n0 * 2 + (u64)(wave * 8) * g.ldb * 2;
+#pragma unroll
+        for (int n = 0; n < LHB; ++n) {
+            const int pos = n * 1024 + lane * 16, kq = pos / PB, slot = (pos % PB) / 16;
+            ob[n] = (u32)((kq * g.ldb + (u64)((slot ^ tform_swizzle<PB>(kq, wave & 1)) * 8)) * 2);
+        }
+    } else {
+        B = gb + (n0 + (u64)wave * LHB * 8) * g.ldb * 2;
+        const int par = (LHB & 1) ? (wave & 1) : 0;
+        ob[0] = (u32)((lr * g.ldb + (u64)(((lane & 7) ^ fe ^ (4 * par)) * 8)) * 2);
+        ob[1] = (u32)((lr * g.ldb + (u64)(((lane & 7) ^ fe ^ (4 * par) ^ 4) * 8)) * 2);
+    }
+    const u64 ca = 16 * g.lda, cb = 16 * g.ldb;                                          // bytes between 8-row blocks (K-contiguous)
+    const u64 sa = AT ? (u64)BK * g.lda * 2 : (u64)BK * 2, sb = BT ? (u64)BK * g.ldb * 2 : (u64)BK * 2;   // bytes between K-steps
+    const int steps = (int)(g.K / BK);
+
+    // consumer.  K-contiguous: lane reads row (lane & 15) of a 16-row block, k-chunk 4 s + (lane >> 4) of slice s.
+    // T form: lane j of a 16-lane group points at k-row 32 s + 8 grp + (j >> 2) [+ 4], columns 4 (j & 3) .. + 3 of the block.
+    const int r15 = lane & 15, grp = lane >> 4, tq = r15 >> 2;
+    const int slot0 = grp ^ (((r15 >> 1) & 7) ^ ((r15 & 1) << 2));
+    int fra[AT ? TI : 1], frb[BT ? TJ : 1];
+    if constexpr (AT) {
+#pragma unroll
+        for (int f = 0; f < TI; ++f)
+            fra[f] = (8 * grp + tq) * PA + 8 * (r15 & 1) + (((wm * (WROWS / 8) + 2 * f + ((r15 & 3) >> 1)) ^ tform_swizzle<PA>(tq, grp & 1)) * 16);
+    } else fra[0] = (wm * WROWS + r15) * 128 + slot0 * 16;
+    if constexpr (BT) {
+#pragma unroll
+        for (int f = 0; f < TJ; ++f)
+            frb[f] = ASZ + (8 * grp + tq) * PB + 8 * (r15 & 1) + (((wn * (WCOLS / 8) + 2 * f + ((r15 & 3) >> 1)) ^ tform_swizzle<PB>(tq, grp & 1)) * 16);
+    } else frb[0] = ASZ + (wn * WCOLS + r15) * 128 + slot0 * 16;
+
+    f32x4 acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; ++i)
+#pragma unroll
+        for (int j = 0; j < TJ; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    u32x4 fa[2][TI], fb[2][TJ];
+
+    auto load = [&](auto n_, u64 ki, int bo) {
+        constexpr int n = decltype(n_)::v;
+        if constexpr (n < LHA) {
+            const char* src = AT ? A + ki * sa + oa[AT ? n : 0] : A + (n * ca + ki * sa) + oa[n & 1];
+            __builtin_amdgcn_global_load_lds(AIX_GLB(src), AIX_LDS(smem + bo + (wave * LHA + n) * 1024), 16, 0, 0);
+        } else {
+            constexpr int m = n - LHA;
+            const char* src = BT ? B + ki * sb + ob[BT ? m : 0] : B + (m * cb + ki * sb) + ob[m & 1];
+            __builtin_amdgcn_global_load_lds(AIX_GLB(src), AIX_LDS(smem + bo + ASZ + (wave * LHB + m) * 1024), 16, 0, 0);
+        }
+    };
+    auto read = [&](int set, int bo, int s, auto f_) {
+        constexpr int f = decltype(f_)::v;
+        if constexpr (f < TI) {
+            if constexpr (AT) fa[set][f] = tr_fragment_at<4 * PA>(smem + bo + fra[AT ? f : 0] + s * 32 * PA);
+            else fa[set][f] = *(const u32x4*)(smem + bo + (fra[0] ^ (s * 64)) + f * 2048);
+        } else {
+            constexpr int e = f - TI;
+            if constexpr (BT) fb[set][e] = tr_fragment_at<4 * PB>(smem + bo + frb[BT ? e : 0] + s * 32 * PB);
+            else fb[set][e] = *(const u32x4*)(smem + bo + (frb[0] ^ (s * 64)) + e * 2048);
+        }
+    };
+    // MFMAs on fragment set FC while set FN is read from stage rbo, slice S; with LOADS, tile `ko` goes to stage lbo
+    auto phase = [&](auto FC_, auto FN_, int rbo, auto S_, auto LOADS_, u64 ko, int lbo) {
+        constexpr int FC = decltype(FC_)::v, FN = decltype(FN_)::v, S = decltype(S_)::v, LOADS = decltype(LOADS_)::v;
+        if constexpr (AT || BT) { AIX_SB(); __builtin_amdgcn_s_waitcnt(0xC07F); AIX_SB(); }     // lgkmcnt(0): fragment set FC has arrived
+        auto block = [&]<int b>(Const<b>) {
+            [&]<int... f>(std::integer_sequence<int, f...>) {
+                (read(FN, rbo, S, Const<b * NF / NB + f>{}), ...);
+            }(std::make_integer_sequence<int, (b + 1) * NF / NB - b * NF / NB>{});
+            if constexpr (LOADS) {
+                [&]<int... n>(std::integer_sequence<int, n...>) {
+                    (load(Const<b * LPW / NB + n>{}, ko, lbo), ...);
+                }(std::make_integer_sequence<int, (b + 1) * LPW / NB - b * LPW / NB>{});
+            }
+#pragma unroll
+            for (int i = b * TI / NB; i < (b + 1) * TI / NB; ++i)
+#pragma unroll
+                for (int j = 0; j < TJ; ++j) acc[i][j] = Mma16<T>::run16(fa[FC][i], fb[FC][j], acc[i][j]);
+            AIX_SB();
+        };
+        block(Const<0>{}); block(Const<1>{}); block(Const<2>{}); block(Const<3>{});
+    };
+
+    {
+        const u64 k1 = 1 < steps ? 1 : 0;
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, (u64)0, 0), ...); }(std::make_integer_sequence<int, LPW>{});
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, k1, STAGE), ...); }(std::make_integer_sequence<int, LPW>{});
+    }
+    AIX_SB();
+    AIX_WAIT(LPW, 15);                                        // tile 0 has landed (the loads of tile 1 may be in flight)
+    __builtin_amdgcn_s_barrier();
+    AIX_SB();
+    [&]<int... f>(std::integer_sequence<int, f...>) { (read(0, 0, 0, Const<f>{}), ...); }(std::make_integer_sequence<int, NF>{});
+    for (int kt = 0; kt < steps; ++kt) {
+        const int bo = (kt & 1) * STAGE, nbo = bo ^ STAGE;
+        const u64 k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1);
+        phase(Const<0>{}, Const<1>{}, bo, Const<1>{}, Const<0>{}, k2, nbo);
+        AIX_WAIT(0, 0);                                       // tile kt+1 complete in the other stage; own reads of this stage done
+        __builtin_amdgcn_s_barrier();
+        AIX_SB();
+        phase(Const<1>{}, Const<0>{}, nbo, Const<0>{}, Const<1>{}, k2, bo);
+    }
+    AIX_WAIT(0, 0);                                           // stray loads have landed before LDS is reused
+    __builtin_amdgcn_s_barrier();
+    AIX_SB();
+
+    // Epilogue through LDS, each wave on its own slab: 16 rows of the wave's 64 x WCOLS block row-major (pitch WCOLS + 4
+    // floats), read back as runs of 8 columns, rounded and stored with 16-byte non-temporal writes.
+    constexpr int PITCH = WCOLS + 4, RUNS = 16 * (WCOLS / 8);
+    float* slab = (float*)smem + wave * (16 * PITCH + 64);
+    u16* C = global_ptr<u16>(base_c);
+#pragma unroll
+    for (int i = 0; i < TI; ++i) {
+#pragma unroll
+        for (int j = 0; j < TJ; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) slab[(4 * grp + v) * PITCH + j * 16 + r15] = acc[i][j][v];
+#pragma unroll
+        for (int t = 0; t < (RUNS + 63) / 64; ++t) {
+            const int run = lane + 64 * t, row = run / (WCOLS / 8), cg = run % (WCOLS / 8);
+            if (RUNS % 64 == 0 || run < RUNS) {
+                const f32x4 lo = *(const f32x4*)(slab + row * PITCH + cg * 8);
+                const f32x4 hi = *(const f32x4*)(slab + row * PITCH + cg * 8 + 4);
+                u32x4 o;
+                o.x = Mma16<T>::pack(lo.x, lo.y); o.y = Mma16<T>::pack(lo.z, lo.w);
+                o.z = Mma16<T>::pack(hi.x, hi.y); o.w = Mma16<T>::pack(hi.z, hi.w);
+                __builtin_nontemporal_store(o, (u32x4*)(C + (m0 + wm * WROWS + i * 16 + row) * g.N + n0 + wn * WCOLS + cg * 8));
+            }
+        }
+    }
+}
 #undef AIX_GLB
 #undef AIX_LDS
 #undef AIX_WAIT
@@ -1283,6 +1496,78 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
     return AIXK_OK;
 }
 
+// 16-bit products of whole 128 x {128, 192, 256} x 64 tiles, at least half a tile per compute unit: the LDS-direct kernel
+// on its smaller tiles (gemm_direct16_k).  `batch` / `table` as for launch_small16 (a stack of matrices, or a group of
+// separate products).  limit > 0: only if the estimated cost stays below it (the caller has another kernel to offer).
+// -1: not for this product.
+int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch, const u64* table, double limit)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    constexpr size_t esz = 2;
+    if (!(M % 128 == 0 && N % 64 == 0 && K % 64 == 0)) return -1;
+    const char* qa = (const char*)a->data + a->offset * esz;
+    const char* qb = (const char*)b->data + b->offset * esz;
+    const bool a_k = a->strides[1] == 1, a_m = a->strides[0] == 1;
+    const bool b_k = b->strides[0] == 1, b_n = b->strides[1] == 1;
+    const uint64_t la = a_k ? a->strides[0] : a->strides[1], lb = b_k ? b->strides[1] : b->strides[0];
+    BatchArgs bt{};
+    uint64_t count = 1;
+    if (batch) {
+        if (batch->rank > 3) return -1;
+        bt.rank = (u32)batch->rank;
+        for (int d = 0; d < batch->rank; ++d) {
+            if (batch->shape[d] >= (1ull << 31) || batch->stride[0][d] % 8 != 0 || batch->stride[1][d] % 8 != 0) return -1;
+            bt.ext[d] = (u32)batch->shape[d]; bt.sa[d] = batch->stride[0][d]; bt.sb[d] = batch->stride[1][d];
+            count *= batch->shape[d];
+        }
+        if (count > 65535) return -1;
+        bt.sc = M * N;
+        bt.table = table;
+    }
+    // rounds of workgroups x tile area, a smaller tile's flop 1.35 times as dear as one of the 256 x 256 kernel (more
+    // fragment traffic per flop; measured: 4096^3 111 us on 256 x 256 tiles, 137 on 128 x 256); the larger tile on a tie
+    uint64_t bn = 0;
+    double least = 0;
+    for (uint64_t cand : {256, 192, 128}) {
+        if (N % cand != 0) continue;
+        const uint64_t tiles = (M / 128) * (N / cand) * count;
+        const double cost = 1.35 * (double)(((tiles + (uint64_t)ctx->cus - 1) / (uint64_t)ctx->cus) * cand * 128);
+        if (bn == 0 || cost < least) { bn = cand; least = cost; }
+    }
+    if (bn == 0 || (limit > 0 && least >= limit)) return -1;
+    const uint64_t tiles = (M / 128) * (N / bn);
+    if (tiles * count * 2 < (uint64_t)ctx->cus || tiles >= (1ull << 31)) return -1;
+    if (!((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && la < (1ull << 27) && lb < (1ull << 27) && aligned16(qa) && aligned16(qb))) return -1;
+    GemmArgs g{};
+    g.a = qa; g.b = qb; g.c = out->data;
+    g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+    g.tiles_m = (u32)(M / 128); g.tiles_n = (u32)(N / bn);
+    const u32 n = g.tiles_m * g.tiles_n;
+    g.swizzle = n % 8u == 0 ? 1u : 0u;
+    const size_t lds = 2 * (128 + bn) * 128;
+    const bool at = !a_k, tb = !b_k;
+    auto launch = [&](auto kernel) {
+        AIXK_TRY(set_lds(kernel, lds));
+        hipLaunchKernelGGL(kernel, dim3(n, (unsigned)count), dim3(512), lds, ctx->stream, g, bt);
+        AIXK_HIP(hipGetLastError());
+        return (int)AIXK_OK;
+    };
+    auto by_form = [&](auto dtype_tag, auto bn_tag) {
+        typedef decltype(dtype_tag) T;
+        constexpr int BN = decltype(bn_tag)::value;
+        if (!at && !tb) return launch(gemm_direct16_k<T, false, false, 128, BN>);
+        if (!at && tb) return launch(gemm_direct16_k<T, false, true, 128, BN>);
+        if (at && !tb) return launch(gemm_direct16_k<T, true, false, 128, BN>);
+        return launch(gemm_direct16_k<T, true, true, 128, BN>);
+    };
+    auto by_tile = [&](auto dtype_tag) {
+        if (bn == 256) return by_form(dtype_tag, std::integral_constant<int, 256>{});
+        if (bn == 192) return by_form(dtype_tag, std::integral_constant<int, 192>{});
+        return by_form(dtype_tag, std::integral_constant<int, 128>{});
+    };
+    return out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
+}
+
 // Which kernel multiplies 16-bit operands whose layouts are consumed in place (everything the LDS-direct kernel does
 // not take).  Measured on the shapes of a d = 768 transformer step at 8192 tokens, in microseconds, old route -> new:
 // [8192,768]x[768,768] 28 -> 23, [8192,3072]^T-free x [3072,768] 76 -> 67, weight gradients [768,8192]x[8192,768]
@@ -1304,6 +1589,10 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         // a group of separate products (table): no K splits -- their partial planes assume one dense stack of results
         if (M <= 64) return launch_tile16(ctx, a, b, out, batch, 0, table ? 1 : splits_for(t64 * count, (K + 63) / 64 * 2, 4), table);
         if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, table ? 1 : splits_for(t12864 * count, (K + 31) / 32, 2), table);
+        if (K >= 512) {                                    // whole tiles and enough K steps to pay for its prologue: the LDS-direct kernel
+            const int rc = launch_direct16(ctx, a, b, out, batch, table, 0);
+            if (rc != -1) return rc;
+        }
         return launch_tile16(ctx, a, b, out, batch, 2, table ? 1 : splits_for(t128 * count, (K + 31) / 32, 2), table);
     }
     // Tiles and K splits by a two-term cost in units of one K step (32 deep) of a lone 128 x 128 workgroup: the steps of the
@@ -1422,6 +1711,11 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
     // (K-contiguous, or "T" form with unit stride along M / N), no gathers.
     if (esz == 2 && M % 256 == 0 && N % 256 == 0 && K % 64 == 0 && (M / 256) * (N / 256) >= (uint64_t)ctx->cus / 2 &&
         (M / 256) * (N / 256) < (1ull << 31)) {
+        // unless smaller tiles fill the chip's rounds so much better that they win all the same ([8192, 768] x [768, 2304]:
+        // 288 tiles are a full round and an eighth of one, 44.7 us; 768 tiles of 128 x 192 are three full rounds, 36-39 us)
+        const uint64_t t256 = (M / 256) * (N / 256);
+        const int rc = launch_direct16(ctx, a, b, out, nullptr, nullptr, (double)(((t256 + (uint64_t)ctx->cus - 1) / (uint64_t)ctx->cus) * 65536));
+        if (rc != -1) return rc;
         const char* qa = (const char*)a->data + a->offset * esz;
         const char* qb = (const char*)b->data + b->offset * esz;
         const bool a_k = a->strides[1] == 1, a_m = a->strides[0] == 1;
@@ -1454,6 +1748,8 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
             return launch(gemm_nt16_direct_k<f16, true, true>);
         }
     }
+
+    if (esz == 2) { const int rc = launch_direct16(ctx, a, b, out, nullptr, nullptr, 0); if (rc != -1) return rc; }
 
     // 16-bit, operands consumed where they lie (K-contiguous or T form): tiles and K splits by shape
     if (esz == 2) {

@@ -65,7 +65,9 @@ def array_of(descs):
 
 @pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=lambda d: NAMES[d])
 @pytest.mark.parametrize("case", [(64, 64, 64, "N", "N", 5), (512, 64, 512, "N", "T", 7), (512, 512, 64, "N", "N", 3), (512, 512, 64, "T", "N", 4),
-                                  (128, 256, 192, "S", "S", 6), (512, 512, 512, "N", "N", 9), (96, 40, 72, "N", "N", 3)], ids=str)
+                                  (128, 256, 192, "S", "S", 6), (512, 512, 512, "N", "N", 9), (96, 40, 72, "N", "N", 3),
+                                  # whole 128 x {128, 192} tiles and K >= 512: the LDS-direct kernel's smaller tiles, addresses from the table
+                                  (768, 1024, 768, "T", "N", 6), (384, 512, 640, "N", "T", 10), (256, 576, 512, "S", "N", 16)], ids=str)
 def test_grouped_launch_matches_single_launches(gpu, dtype, case):
     m, k, n, la, lb, count = case
     rng = np.random.default_rng(9100 + m + k + n + dtype)

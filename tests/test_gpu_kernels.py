@@ -739,6 +739,34 @@ def test_matmul_mfma_tiles(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16], ids=ids)
+def test_matmul_mid_tiles(gpu, dtype):
+    """16-bit products of whole 128 x {128, 192, 256} x 64 tiles, at least half a tile per compute unit: the LDS-direct
+    kernel on its smaller tiles.  The widths pick the tile (960 = 5 x 192 and no multiple of 128; 640 = 5 x 128 and no
+    multiple of 192 or 256; 2048 under 31 tile rows: 248 tiles of 128 x 256 fill the chip in one round, 496 of 128 x 128
+    would take two), every operand layout is consumed where it lies, with 1, 2, 3 and 5 K steps, sliced operands (row
+    pitch above the extent), and the shapes of a d = 768 transformer's projections."""
+    rng = np.random.default_rng(23700 + dtype)
+    layouts = [("contig", "contig"), ("contig", "transposed"), ("transposed", "contig"), ("transposed", "transposed")]
+    cases = []
+    for n in (960, 640):
+        for k, (ka, kb) in zip((64, 128, 192, 320), layouts):
+            cases.append(((4096, k, n), ka, kb))
+        for k, (ka, kb) in zip((320, 64, 128, 192), layouts):
+            cases.append(((4096, k, n), ka, kb))
+    for k, (ka, kb) in zip((128, 192, 64, 320), layouts):
+        cases.append(((3968, k, 2048), ka, kb))
+    cases += [((4096, 128, 960), "sliced", "sliced"), ((4096, 192, 640), "sliced", "transposed"),
+              ((8192, 768, 768), "contig", "contig"), ((8192, 768, 768), "contig", "transposed"), ((8192, 768, 768), "transposed", "contig"),
+              ((8192, 3072, 768), "contig", "contig"), ((8192, 768, 2304), "contig", "transposed")]
+    for (m, k, n), ka, kb in cases:
+        scale = 1.0 / np.sqrt(k)
+        a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
+        b = T.view_tensor(rng, dtype, [k, n], kb, lo=-1, hi=1)
+        check_matmul(gpu, a, b, f"mid-tile matmul {NAMES[dtype]} {m}x{k}x{n} {ka}/{kb}")
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16], ids=ids)
 def test_matmul_small_tiles(gpu, dtype):
     """16-bit outputs too small for 64 x 64 tiles to fill the chip (attention heads and the like): the
     32 x 32-tile kernel that splits K over its four waves, every operand layout consumed in place --
@@ -962,7 +990,8 @@ def check_matmul_stack(gpu, a, b, what, against_each=True):
             single = gpu.fetch(p1, mine)
             if dtype in (O.F16, O.BF16):
                 final = 2.0 ** -10 if dtype == O.F16 else 2.0 ** -8
-                G.assert_close_to_wide(O.to_float64(mine, dtype), O.to_float64(single, dtype), 1e-5 * scale + final * np.abs(exact) + 1e-30, 1.0,
+                # two roundings of two f32 sums that differ in the order of their terms: each within half an ulp of its own sum
+                G.assert_close_to_wide(O.to_float64(mine, dtype), O.to_float64(single, dtype), 2e-5 * scale + 2 * final * np.abs(exact) + 1e-30, 1.0,
                                        f"{what} matrix {index} against the 2-D entry point")
             else:
                 T.assert_same_bits(mine, single, f"{what} matrix {index} against the 2-D entry point")
@@ -997,6 +1026,16 @@ def test_matmul_stacks(gpu, dtype):
     wide = T.HostTensor(draw(5 * 72 * 104, -0.2, 0.2), dtype, [3, 72, 88], [72 * 104, 104, 1], offset=72 * 104 + 8)
     other = T.HostTensor(draw(4 * 88 * 80, -1, 1), dtype, [3, 88, 80], None, offset=88 * 80)
     check_matmul_stack(gpu, wide, other, f"sliced stack {NAMES[dtype]}")
+    # whole 128 x {128, 192} tiles, eight K steps and half a tile per compute unit over the stack: the LDS-direct kernel's
+    # smaller tiles with blockIdx.y numbering the matrices -- plain, with permuted leading dims, a transposed first operand
+    if dtype in (O.F16, O.BF16):
+        big_a = T.HostTensor(draw(2 * 4 * 512 * 512, -0.05, 0.05), dtype, [2, 4, 512, 512], [512 * 512, 2 * 512 * 512, 512, 1])
+        big_b = T.HostTensor(draw(2 * 4 * 512 * 768, -1, 1), dtype, [2, 4, 512, 768])
+        check_matmul_stack(gpu, big_a, big_b, f"stack of whole 128 x 192 tiles {NAMES[dtype]}")
+        big_at = T.HostTensor(big_a.storage, dtype, [8, 512, 512], [512 * 512, 1, 512])
+        big_c = T.HostTensor(draw(8 * 512 * 640, -1, 1), dtype, [8, 512, 640])
+        check_matmul_stack(gpu, big_at, big_c, f"stack of whole 128 x 128 tiles, transposed first operand {NAMES[dtype]}")
+        gpu.release()
     # matrices too small or too odd for the matrix-core route
     check_matmul_stack(gpu, T.HostTensor(draw(7 * 5 * 3, -1, 1), dtype, [7, 5, 3]), T.HostTensor(draw(7 * 3 * 4, -1, 1), dtype, [7, 3, 4]),
                        f"tiny stack {NAMES[dtype]}")
