@@ -5,6 +5,8 @@
 //   16-bit, whole tiles   gemm_nt16_direct_k: 256x256x64 workgroup tile, eight waves (two per SIMD) on
 //                         v_mfma_f32_16x16x32, LDS filled by LDS-direct global loads, swizzled layout,
 //                         explicit software pipeline; both operand forms;
+//   16-bit, whole tiles   gemm_direct16_k: the same scheme on 128 x {128, 192, 256} x 64 tiles for results that 256 x 256
+//                         tiles cannot spread over the chip; stacks and groups of products by blockIdx.y;
 //   16-bit, mid-size      gemm_tile16_k: 128x128 / 128x64 / 64x64 tiles, register staging, both operand
 //                         forms, stacks of matrices (blockIdx.y) and K splits over workgroups (blockIdx.z);
 //   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
@@ -12,7 +14,7 @@
 //   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
 //   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 or 64x64 tile x BK=32, both operand forms.
 //
-// All but the first use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
+// All but the first two use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
 // resident in the 512-entry unified register file.  Every lane feeds the 16-bit MFMA with 8 consecutive K
 // values of one row; because A and B use the same lane->K assignment, the dot products are independent of
 // how the instruction numbers K internally.
