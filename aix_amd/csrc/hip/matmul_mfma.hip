@@ -12,6 +12,8 @@
 //   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
 //   16-bit, odd layouts   gemm_nt16_k: K-contiguous operands only, bounds-checked (others are gathered first);
 //   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
+//   f32, very large       split_planes_k + gemm_direct16_k<PLANES>: the planes written to memory once, six plane pairs
+//                         multiplied by the LDS-direct 16-bit kernel;
 //   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 or 64x64 tile x BK=32, both operand forms.
 //
 // All but the first two use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
@@ -420,10 +422,17 @@ template <int OFF> __device__ __forceinline__ u32x4 tr_fragment_at(const unsigne
     return u32x4{lo.x, lo.y, hi.x, hi.y};
 }
 
-template <class T, bool AT, bool BT, int BM, int BN>
-__global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
+// PLANES: an f32 product on the bf16 pipe from operands that split_planes_k has laid out as three bf16 planes each (hi, mid,
+// lo: K-contiguous, plane after plane): the K loop runs over the six plane pairs that carry the product to f32 accuracy,
+// smallest terms first -- (lo, hi), (hi, lo), (mid, mid), (mid, hi), (hi, mid), (hi, hi) -- and the accumulators leave as
+// f32; a lane whose accumulators hold an infinity or a NaN stores the launch's number into the flag word, as gemm_x3_k does.
+struct PlanesArgs { u64 plane_a, plane_b; u32* flag; u32 seq; };      // bytes from one plane to the next
+
+template <class T, bool AT, bool BT, int BM, int BN, bool PLANES = false>
+__global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt, PlanesArgs pl)
 {
-    static_assert(BM == 128 && (BN == 128 || BN == 192 || BN == 256), "tiles this kernel is written for");
+    static_assert((BM == 128 && (BN == 128 || BN == 192 || BN == 256)) || (BM == 256 && BN == 256 && PLANES), "tiles this kernel is written for");
+    static_assert(!PLANES || (!AT && !BT), "planes are laid out K-contiguous");
     constexpr int BK = 64, ASZ = BM * 128, BSZ = BN * 128, STAGE = ASZ + BSZ;
     constexpr int WGN = 4, TI = BM / 32, TJ = BN / 64, WROWS = TI * 16, WCOLS = TJ * 16;
     constexpr int LHA = BM / 64, LHB = BN / 64, LPW = LHA + LHB;     // loads per wave and tile
@@ -487,7 +496,16 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
     }
     const u64 ca = 16 * g.lda, cb = 16 * g.ldb;                                          // bytes between 8-row blocks (K-contiguous)
     const u64 sa = AT ? (u64)BK * g.lda * 2 : (u64)BK * 2, sb = BT ? (u64)BK * g.ldb * 2 : (u64)BK * 2;   // bytes between K-steps
-    const int steps = (int)(g.K / BK);
+    const int per_pair = (int)(g.K / BK), steps = PLANES ? 6 * per_pair : per_pair;
+    // where K-step `ki` starts, in bytes from the operands' bases (PLANES: pair ki / per_pair, step ki % per_pair of it)
+    auto step_a = [&](int ki) -> u64 {
+        if constexpr (PLANES) { const int pr = ki / per_pair; return (u64)((0x052u >> (2 * pr)) & 3u) * pl.plane_a + (u64)(ki - pr * per_pair) * sa; }
+        else return (u64)ki * sa;
+    };
+    auto step_b = [&](int ki) -> u64 {
+        if constexpr (PLANES) { const int pr = ki / per_pair; return (u64)((0x118u >> (2 * pr)) & 3u) * pl.plane_b + (u64)(ki - pr * per_pair) * sb; }
+        else return (u64)ki * sb;
+    };
 
     // consumer.  K-contiguous: lane reads row (lane & 15) of a 16-row block, k-chunk 4 s + (lane >> 4) of slice s.
     // T form: lane j of a 16-lane group points at k-row 32 s + 8 grp + (j >> 2) [+ 4], columns 4 (j & 3) .. + 3 of the block.
@@ -512,14 +530,15 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
         for (int j = 0; j < TJ; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     u32x4 fa[2][TI], fb[2][TJ];
 
-    auto load = [&](auto n_, u64 ki, int bo) {
+    // load n of the tile that starts ka / kb bytes into the operands
+    auto load = [&](auto n_, u64 ka, u64 kb, int bo) {
         constexpr int n = decltype(n_)::v;
         if constexpr (n < LHA) {
-            const char* src = AT ? A + ki * sa + oa[AT ? n : 0] : A + (n * ca + ki * sa) + oa[n & 1];
+            const char* src = AT ? A + ka + oa[AT ? n : 0] : A + (n * ca + ka) + oa[n & 1];
             __builtin_amdgcn_global_load_lds(AIX_GLB(src), AIX_LDS(smem + bo + (wave * LHA + n) * 1024), 16, 0, 0);
         } else {
             constexpr int m = n - LHA;
-            const char* src = BT ? B + ki * sb + ob[BT ? m : 0] : B + (m * cb + ki * sb) + ob[m & 1];
+            const char* src = BT ? B + kb + ob[BT ? m : 0] : B + (m * cb + kb) + ob[m & 1];
             __builtin_amdgcn_global_load_lds(AIX_GLB(src), AIX_LDS(smem + bo + ASZ + (wave * LHB + m) * 1024), 16, 0, 0);
         }
     };
@@ -535,7 +554,7 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
         }
     };
     // MFMAs on fragment set FC while set FN is read from stage rbo, slice S; with LOADS, tile `ko` goes to stage lbo
-    auto phase = [&](auto FC_, auto FN_, int rbo, auto S_, auto LOADS_, u64 ko, int lbo) {
+    auto phase = [&](auto FC_, auto FN_, int rbo, auto S_, auto LOADS_, u64 ka, u64 kb, int lbo) {
         constexpr int FC = decltype(FC_)::v, FN = decltype(FN_)::v, S = decltype(S_)::v, LOADS = decltype(LOADS_)::v;
         if constexpr (AT || BT) { AIX_SB(); __builtin_amdgcn_s_waitcnt(0xC07F); AIX_SB(); }     // lgkmcnt(0): fragment set FC has arrived
         auto block = [&]<int b>(Const<b>) {
@@ -544,7 +563,7 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
             }(std::make_integer_sequence<int, (b + 1) * NF / NB - b * NF / NB>{});
             if constexpr (LOADS) {
                 [&]<int... n>(std::integer_sequence<int, n...>) {
-                    (load(Const<b * LPW / NB + n>{}, ko, lbo), ...);
+                    (load(Const<b * LPW / NB + n>{}, ka, kb, lbo), ...);
                 }(std::make_integer_sequence<int, (b + 1) * LPW / NB - b * LPW / NB>{});
             }
 #pragma unroll
@@ -557,9 +576,10 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
     };
 
     {
-        const u64 k1 = 1 < steps ? 1 : 0;
-        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, (u64)0, 0), ...); }(std::make_integer_sequence<int, LPW>{});
-        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, k1, STAGE), ...); }(std::make_integer_sequence<int, LPW>{});
+        const int k1 = 1 < steps ? 1 : 0;
+        const u64 a0 = step_a(0), b0 = step_b(0), a1 = step_a(k1), b1 = step_b(k1);
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, a0, b0, 0), ...); }(std::make_integer_sequence<int, LPW>{});
+        [&]<int... n>(std::integer_sequence<int, n...>) { (load(Const<n>{}, a1, b1, STAGE), ...); }(std::make_integer_sequence<int, LPW>{});
     }
     AIX_SB();
     AIX_WAIT(LPW, 15);                                        // tile 0 has landed (the loads of tile 1 may be in flight)
@@ -568,12 +588,13 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
     [&]<int... f>(std::integer_sequence<int, f...>) { (read(0, 0, 0, Const<f>{}), ...); }(std::make_integer_sequence<int, NF>{});
     for (int kt = 0; kt < steps; ++kt) {
         const int bo = (kt & 1) * STAGE, nbo = bo ^ STAGE;
-        const u64 k2 = (u64)(kt + 2 < steps ? kt + 2 : steps - 1);
-        phase(Const<0>{}, Const<1>{}, bo, Const<1>{}, Const<0>{}, k2, nbo);
+        const int k2 = kt + 2 < steps ? kt + 2 : steps - 1;
+        const u64 a2 = step_a(k2), b2 = step_b(k2);
+        phase(Const<0>{}, Const<1>{}, bo, Const<1>{}, Const<0>{}, a2, b2, nbo);
         AIX_WAIT(0, 0);                                       // tile kt+1 complete in the other stage; own reads of this stage done
         __builtin_amdgcn_s_barrier();
         AIX_SB();
-        phase(Const<1>{}, Const<0>{}, nbo, Const<0>{}, Const<1>{}, k2, bo);
+        phase(Const<1>{}, Const<0>{}, nbo, Const<0>{}, Const<1>{}, a2, b2, bo);
     }
     AIX_WAIT(0, 0);                                           // stray loads have landed before LDS is reused
     __builtin_amdgcn_s_barrier();
@@ -583,6 +604,26 @@ __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt)
     // floats), read back as runs of 8 columns, rounded and stored with 16-byte non-temporal writes.
     constexpr int PITCH = WCOLS + 4, RUNS = 16 * (WCOLS / 8);
     float* slab = (float*)smem + wave * (16 * PITCH + 64);
+    if constexpr (PLANES) {
+        float probe = 0.0f;                                   // x * 0 is a NaN for an infinity or a NaN, else a zero
+        float* Cf = global_ptr<float>(base_c);
+#pragma unroll
+        for (int i = 0; i < TI; ++i) {
+#pragma unroll
+            for (int j = 0; j < TJ; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) { slab[(4 * grp + v) * PITCH + j * 16 + r15] = acc[i][j][v]; probe += acc[i][j][v] * 0.0f; }
+#pragma unroll
+            for (int t = 0; t < (2 * RUNS + 63) / 64; ++t) {                  // runs of 4 columns: 16 bytes of f32
+                const int run = lane + 64 * t, row = run / (WCOLS / 4), cg = run % (WCOLS / 4);
+                if ((2 * RUNS) % 64 == 0 || run < 2 * RUNS)
+                    __builtin_nontemporal_store(*(const f32x4*)(slab + row * PITCH + cg * 4),
+                                                (f32x4*)(Cf + (m0 + wm * WROWS + i * 16 + row) * g.N + n0 + wn * WCOLS + cg * 4));
+            }
+        }
+        if (probe != probe) *pl.flag = pl.seq;
+        return;
+    }
     u16* C = global_ptr<u16>(base_c);
 #pragma unroll
     for (int i = 0; i < TI; ++i) {
@@ -1053,6 +1094,65 @@ __device__ __forceinline__ void split3(const u32x4 x, u32x2& h, u32x2& m, u32x2&
     const float s0 = r[0] - __builtin_bit_cast(float, m.x << 16), s1 = r[1] - __builtin_bit_cast(float, m.x & 0xFFFF0000u);
     const float s2 = r[2] - __builtin_bit_cast(float, m.y << 16), s3 = r[3] - __builtin_bit_cast(float, m.y & 0xFFFF0000u);
     l.x = cvt_pk_bf16(s0, s1); l.y = cvt_pk_bf16(s2, s3);
+}
+
+// The three planes of a whole operand in memory, for products large enough that gemm_direct16_k<..., PLANES> (256 x 256
+// tiles, eight waves, LDS-direct loads) beats splitting in registers tile by tile: planes[p][r][k], p = hi, mid, lo, r < R,
+// k < Kp with zeros from K on, always K-contiguous whatever the source's form (TR: src[k * ld + r], a T-form operand, is
+// transposed through LDS on the way).  The operands that the planes cannot carry -- infinities, NaNs, magnitudes below
+// 2^-100 -- are noticed here: the launch's number goes into the flag word and the IEEE kernel that stands by redoes the product.
+__device__ __forceinline__ void split3_watch(const u32x4 x, u32x2& h, u32x2& m, u32x2& l, u32& least, u32& most)
+{
+    split3(x, h, m, l, least);
+    most = max(max(most, x.x & 0x7FFFFFFFu), max(x.y & 0x7FFFFFFFu, max(x.z & 0x7FFFFFFFu, x.w & 0x7FFFFFFFu)));
+}
+
+template <bool TR>
+__global__ __launch_bounds__(256) void split_planes_k(const float* __restrict__ src, u16* __restrict__ planes, u64 R, u64 K, u64 Kp, u64 ld, u32* flag, u32 seq)
+{
+    const int tid = threadIdx.x;
+    const u64 plane = R * Kp;
+    u32 least = ~0u, most = 0u;
+    if constexpr (!TR) {
+        // 32 rows x 64 k per workgroup; a lane splits 8 consecutive k of one row
+        const u64 r = (u64)blockIdx.y * 32 + tid / 8, k = (u64)blockIdx.x * 64 + (tid % 8) * 8;
+        u32x4 x0 = u32x4{0, 0, 0, 0}, x1 = u32x4{0, 0, 0, 0};
+        if (k < K) x0 = *(const u32x4*)(src + r * ld + k);
+        if (k + 4 < K) x1 = *(const u32x4*)(src + r * ld + k + 4);
+        u32x2 h0, m0, l0, h1, m1, l1;
+        split3_watch(x0, h0, m0, l0, least, most);
+        split3_watch(x1, h1, m1, l1, least, most);
+        u16* out = planes + r * Kp + k;
+        *(u32x4*)out = u32x4{h0.x, h0.y, h1.x, h1.y};
+        *(u32x4*)(out + plane) = u32x4{m0.x, m0.y, m1.x, m1.y};
+        *(u32x4*)(out + 2 * plane) = u32x4{l0.x, l0.y, l1.x, l1.y};
+    } else {
+        // 64 k x 64 r per workgroup: 16-byte loads along r, the planes transposed in LDS (pitch 72), 16-byte stores along k
+        __shared__ u16 tile[3][64][72];
+        const u64 k0 = (u64)blockIdx.x * 64, r0 = (u64)blockIdx.y * 64;
+        const int rc = tid % 16, kr = tid / 16;
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int kk = pass * 16 + kr;
+            u32x4 x = u32x4{0, 0, 0, 0};
+            if (k0 + kk < K) x = *(const u32x4*)(src + (k0 + kk) * ld + r0 + rc * 4);
+            u32x2 h, m, l;
+            split3_watch(x, h, m, l, least, most);
+            const u32 hv[4] = {h.x & 0xFFFFu, h.x >> 16, h.y & 0xFFFFu, h.y >> 16}, mv[4] = {m.x & 0xFFFFu, m.x >> 16, m.y & 0xFFFFu, m.y >> 16},
+                      lv[4] = {l.x & 0xFFFFu, l.x >> 16, l.y & 0xFFFFu, l.y >> 16};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { tile[0][rc * 4 + e][kk] = (u16)hv[e]; tile[1][rc * 4 + e][kk] = (u16)mv[e]; tile[2][rc * 4 + e][kk] = (u16)lv[e]; }
+        }
+        __syncthreads();
+        const int row = tid / 4, kc = (tid % 4) * 16;
+#pragma unroll
+        for (int p = 0; p < 3; ++p) {
+            u16* out = planes + (u64)p * plane + (r0 + row) * Kp + k0 + kc;
+            *(u32x4*)out = *(const u32x4*)&tile[p][row][kc];
+            *(u32x4*)(out + 8) = *(const u32x4*)&tile[p][row][kc + 8];
+        }
+    }
+    if (least < kX3Smallest || most >= 0x7F800000u) *flag = seq;
 }
 
 template <bool AT, bool BT>
@@ -1550,7 +1650,7 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
     const bool at = !a_k, tb = !b_k;
     auto launch = [&](auto kernel) {
         AIXK_TRY(set_lds(kernel, lds));
-        hipLaunchKernelGGL(kernel, dim3(n, (unsigned)count), dim3(512), lds, ctx->stream, g, bt);
+        hipLaunchKernelGGL(kernel, dim3(n, (unsigned)count), dim3(512), lds, ctx->stream, g, bt, PlanesArgs{});
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     };
@@ -1777,9 +1877,10 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         const bool a_k = a->strides[1] == 1 || K == 1, a_m = a->strides[0] == 1 && M % 4 == 0;
         const bool b_k = b->strides[0] == 1 || K == 1, b_n = b->strides[1] == 1 && N % 4 == 0;
         uint64_t lda = a_k ? a->strides[0] : a->strides[1], ldb = b_k ? b->strides[1] : b->strides[0];
-        bool at = !a_k && a_m, bt = !b_k && b_n;
+        bool at = !a_k && a_m, bt = !b_k && b_n, gathered = false;
         if (!(a_k || a_m) || lda % 4 != 0 || !aligned16(pa)) {
             void* ws;
+            gathered = true;
             AIXK_TRY(workspace(ctx, 0, M * K * esz, &ws));
             AIXK_TRY(gather_dense(ctx, a, ws, M * K));
             pa = (const char*)ws; lda = K; at = false;
@@ -1789,6 +1890,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
             bt_view.shape[0] = N; bt_view.shape[1] = K;
             bt_view.strides[0] = b->strides[1]; bt_view.strides[1] = b->strides[0];
             void* ws;
+            gathered = true;
             AIXK_TRY(workspace(ctx, 1, N * K * esz, &ws));
             AIXK_TRY(gather_dense(ctx, &bt_view, ws, N * K));
             pb = (const char*)ws; ldb = K; bt = false;
@@ -1796,16 +1898,49 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         GemmArgs g{};
         g.a = pa; g.b = pb; g.c = out->data;
         g.M = M; g.N = N; g.K = K; g.lda = lda; g.ldb = ldb;
+        const uint64_t t128 = ((M + 127) / 128) * ((N + 127) / 128), fill = 2 * (uint64_t)ctx->cus, steps = (K + 31) / 32;
+        const u32* only_if = nullptr;          // set: the launches below stand by behind a split-plane kernel
+        u32 seq = 0;
+        // whole 256 x 256 tiles, at least one per compute unit: the planes of both operands are written to memory once
+        // (split_planes_k) and multiplied by the LDS-direct 16-bit kernel, six plane pairs deep (4096^3: 0.73 -> 0.64 ms)
+        if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= (uint64_t)ctx->cus && (M / 256) * (N / 256) < (1ull << 31) && K >= 256 &&
+            !gathered && lda < (1ull << 27) && ldb < (1ull << 27)) {
+            const uint64_t Kp = (K + 63) / 64 * 64;
+            void *wa, *wb;
+            AIXK_TRY(workspace(ctx, 0, 3 * M * Kp * 2, &wa));
+            AIXK_TRY(workspace(ctx, 1, 3 * N * Kp * 2, &wb));
+            if (++ctx->gemm_seq == 0) ++ctx->gemm_seq;
+            seq = ctx->gemm_seq;
+            auto split = [&](const char* src, bool transposed, uint64_t rows, uint64_t ld, void* planes) {
+                if (transposed) hipLaunchKernelGGL(split_planes_k<true>, dim3((unsigned)(Kp / 64), (unsigned)(rows / 64)), dim3(256), 0, ctx->stream,
+                                                   (const float*)src, (u16*)planes, (u64)rows, (u64)K, (u64)Kp, (u64)ld, (u32*)ctx->counter, seq);
+                else hipLaunchKernelGGL(split_planes_k<false>, dim3((unsigned)(Kp / 64), (unsigned)(rows / 32)), dim3(256), 0, ctx->stream,
+                                        (const float*)src, (u16*)planes, (u64)rows, (u64)K, (u64)Kp, (u64)ld, (u32*)ctx->counter, seq);
+            };
+            split(pa, at, M, lda, wa);
+            split(pb, bt, N, ldb, wb);
+            AIXK_HIP(hipGetLastError());
+            GemmArgs gp{};
+            gp.a = wa; gp.b = wb; gp.c = out->data;
+            gp.M = M; gp.N = N; gp.K = Kp; gp.lda = Kp; gp.ldb = Kp;
+            gp.tiles_m = (u32)(M / 256); gp.tiles_n = (u32)(N / 256);
+            const u32 n = gp.tiles_m * gp.tiles_n;
+            gp.swizzle = n % 8u == 0 ? 1u : 0u;
+            constexpr size_t lds = 2 * 65536;
+            auto kernel = gemm_direct16_k<bf16, false, false, 256, 256, true>;
+            AIXK_TRY(set_lds(kernel, lds));
+            hipLaunchKernelGGL(kernel, dim3(n), dim3(512), lds, ctx->stream, gp, BatchArgs{}, PlanesArgs{M * Kp * 2, N * Kp * 2, (u32*)ctx->counter, seq});
+            AIXK_HIP(hipGetLastError());
+            only_if = (const u32*)ctx->counter;
+            ctx->gemm_last_route = 1;
+        }
         // enough 128 x 128 tiles: on the bf16 pipe, each operand as three bf16 planes (gemm_x3_k); with few tiles and a
         // long K, K is split over workgroups
-        const uint64_t t128 = ((M + 127) / 128) * ((N + 127) / 128), fill = 2 * (uint64_t)ctx->cus, steps = (K + 31) / 32;
         // two workgroups per compute unit hide each other's split-and-stage phases: with fewer tiles than that, K is split
         // over workgroups if it is long enough, else the f32 MFMA kernels below take the product
         uint64_t splits = 1;
         if (t128 < fill && K >= 2048) splits = std::min<uint64_t>({steps / 16, (fill + t128 - 1) / t128, (uint64_t)64});
-        const u32* only_if = nullptr;          // set: the launches below stand by behind gemm_x3_k
-        u32 seq = 0;
-        if (t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 4) {
+        if (!only_if && t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 4) {
             const u32 n = grid_of(g, 128, 128);
             SplitArgs sk{};
             sk.per_split = (u32)((steps + splits - 1) / splits);

@@ -789,8 +789,11 @@ def _route(gpu):
     return route.value, redone.value
 
 
-def test_matmul_f32_large_tiles_small_magnitudes(gpu):
-    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes.  The planes carry
+@pytest.mark.parametrize("mkn", [(4096, 256, 2048), (4096, 264, 4096)], ids=["planes_in_registers", "planes_in_memory"])
+def test_matmul_f32_large_tiles_small_magnitudes(gpu, mkn):
+    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes -- tile by tile in
+    registers (gemm_x3_k), or, from one whole 256 x 256 tile per compute unit on, once into memory (split_planes_k, here
+    with a K that is padded to the next multiple of 64) for the LDS-direct 16-bit kernel to multiply six plane pairs deep.  The planes carry
     f32's 24 bits only down to 2^-110 (bf16's grid ends at 2^-133), so operands below that -- here in matrices WITHOUT
     any infinity or NaN, which would send the product to the IEEE kernel for their own reasons -- must be noticed and the
     product redone in IEEE f32 arithmetic, as the CPU device computes it (aixDeviceCPU.cpp:362-389: plain f32, no range
@@ -799,7 +802,8 @@ def test_matmul_f32_large_tiles_small_magnitudes(gpu):
     (cpuref_matmul_wide), plus K quanta of 2^-149 where results are subnormal (each f32 product rounds by up to half a
     quantum there on the CPU too)."""
     rng = np.random.default_rng(25600)
-    m, k, n = 4096, 256, 2048                                   # 512 tiles of 128 x 128: the split-plane route
+    m, k, n = mkn                                               # 512 tiles of 128 x 128 / 256 tiles of 256 x 256: the split-plane routes
+    in_memory = n == 4096
     U = rng.uniform(-1, 1, (m, k)).astype(np.float32)
     P = rng.uniform(0.1, 1.0, (k, n)).astype(np.float32)
     V = (rng.uniform(0.25, 1.0, (m, k)) * rng.choice([-1.0, 1.0], (m, k))).astype(np.float32)     # magnitudes within two binades
@@ -825,11 +829,15 @@ def test_matmul_f32_large_tiles_small_magnitudes(gpu):
         ]
     floor = k * 2.0 ** -149
     for name, A, B, want_redone in cases:
-        for layout in ("NN", "TN"):
+        if in_memory and name.startswith(("A at 1e-20", "A at 1e-33", "A at 3e", "A at 1e-41", "A at 1e-36 times", "products below")):
+            continue                                            # (the scales are the first shape's business; here: who notices, in every layout)
+        for layout in ("NN", "TN", "NT", "TT"):
             if layout == "TN" and name.startswith(("A at 1e-2", "A at 3e", "products below")):
                 continue                                        # (one layout is enough for the variations of one scale)
-            a = T.HostTensor(A if layout == "NN" else np.ascontiguousarray(A.T), O.F32, [m, k], None if layout == "NN" else [1, m])
-            b = T.HostTensor(B, O.F32, [k, n])
+            if layout in ("NT", "TT") and not (in_memory and name in ("ordinary", "one subnormal entry in an ordinary A", "ordinary A times B at 1e-36")):
+                continue                                        # (a transposed B matters to the pass that writes the planes to memory)
+            a = T.HostTensor(A if layout[0] == "N" else np.ascontiguousarray(A.T), O.F32, [m, k], None if layout[0] == "N" else [1, m])
+            b = T.HostTensor(B if layout[1] == "N" else np.ascontiguousarray(B.T), O.F32, [k, n], None if layout[1] == "N" else [1, k])
             _, da = gpu.put(a)
             _, db = gpu.put(b)
             po, do = gpu.put(T.empty(O.F32, [m, n]))
@@ -847,13 +855,15 @@ def test_matmul_f32_large_tiles_small_magnitudes(gpu):
                 assert np.all(err <= 4e-7 * scale), (name, layout, float((err / scale).max()))
 
 
-def test_matmul_f32_large_tiles_special_values(gpu):
-    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes in registers.
+@pytest.mark.parametrize("mkn", [(4096, 256, 2048), (4096, 264, 4096)], ids=["planes_in_registers", "planes_in_memory"])
+def test_matmul_f32_large_tiles_special_values(gpu, mkn):
+    """Large f32 products run on the bf16 matrix pipe with every operand split into three bf16 planes (in registers tile by
+    tile, or once into memory: the two shapes).
     Rows with an infinity, a NaN, both infinities, or a value next to FLT_MAX must come out as IEEE arithmetic has
     them (inf, NaN, NaN, finite); their neighbours in the same 16-byte chunk and everything else stay within the
     f32 matmul bar.  (Non-finite operands send the whole product to the IEEE kernel; small magnitudes are the test above.)"""
     rng = np.random.default_rng(25500)
-    m, k, n = 4096, 256, 2048
+    m, k, n = mkn
     A = (rng.uniform(-1, 1, (m, k)) / np.sqrt(k)).astype(np.float32)
     B = rng.uniform(0.1, 1.0, (k, n)).astype(np.float32)
     A[7, 5] = np.inf
