@@ -1907,11 +1907,12 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         // whole 256 x 256 tiles, at least one per compute unit: the planes of both operands are written to memory once
         // (split_planes_k) and multiplied by the LDS-direct 16-bit kernel, six plane pairs deep (4096^3: 0.73 -> 0.64 ms)
         if (M % 256 == 0 && N % 256 == 0 && (M / 256) * (N / 256) >= (uint64_t)ctx->cus && (M / 256) * (N / 256) < (1ull << 31) && K >= 256 &&
-            !gathered && lda < (1ull << 27) && ldb < (1ull << 27)) {
+            !gathered && lda < (1ull << 27) && ldb < (1ull << 27) && M / 32 <= 65535 && N / 32 <= 65535) {
             const uint64_t Kp = (K + 63) / 64 * 64;
-            void *wa, *wb;
-            AIXK_TRY(workspace(ctx, 0, 3 * M * Kp * 2, &wa));
-            AIXK_TRY(workspace(ctx, 1, 3 * N * Kp * 2, &wb));
+            void *wa = nullptr, *wb = nullptr;
+            // (no room for the planes -- six bytes per operand element -- is no error: gemm_x3_k below needs none)
+            if (workspace(ctx, 0, 3 * M * Kp * 2, &wa) != AIXK_OK || workspace(ctx, 1, 3 * N * Kp * 2, &wb) != AIXK_OK) wa = nullptr;
+            if (wa) {
             if (++ctx->gemm_seq == 0) ++ctx->gemm_seq;
             seq = ctx->gemm_seq;
             auto split = [&](const char* src, bool transposed, uint64_t rows, uint64_t ld, void* planes) {
@@ -1936,6 +1937,7 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
             AIXK_HIP(hipGetLastError());
             only_if = (const u32*)ctx->counter;
             ctx->gemm_last_route = 1;
+            }
         }
         // enough 128 x 128 tiles: on the bf16 pipe, each operand as three bf16 planes (gemm_x3_k); with few tiles and a
         // long K, K is split over workgroups
