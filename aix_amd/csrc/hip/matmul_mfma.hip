@@ -1127,7 +1127,9 @@ __global__ __launch_bounds__(256) void split_planes_k(const float* __restrict__ 
         *(u32x4*)(out + plane) = u32x4{m0.x, m0.y, m1.x, m1.y};
         *(u32x4*)(out + 2 * plane) = u32x4{l0.x, l0.y, l1.x, l1.y};
     } else {
-        // 64 k x 64 r per workgroup: 16-byte loads along r, the planes transposed in LDS (pitch 72), 16-byte stores along k
+        // 64 k x 64 r per workgroup: 16-byte loads along r, the planes transposed in LDS, 16-byte stores along k.  A lane writes
+        // one k of four neighbouring rows and its 15 neighbours write the same k of the next rows, 576 bytes apart (four
+        // banks in turn): the 16-byte chunk of k is therefore kept at chunk ^ (row / 4 & 7) of its row
         __shared__ u16 tile[3][64][72];
         const u64 k0 = (u64)blockIdx.x * 64, r0 = (u64)blockIdx.y * 64;
         const int rc = tid % 16, kr = tid / 16;
@@ -1141,15 +1143,19 @@ __global__ __launch_bounds__(256) void split_planes_k(const float* __restrict__ 
             const u32 hv[4] = {h.x & 0xFFFFu, h.x >> 16, h.y & 0xFFFFu, h.y >> 16}, mv[4] = {m.x & 0xFFFFu, m.x >> 16, m.y & 0xFFFFu, m.y >> 16},
                       lv[4] = {l.x & 0xFFFFu, l.x >> 16, l.y & 0xFFFFu, l.y >> 16};
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { tile[0][rc * 4 + e][kk] = (u16)hv[e]; tile[1][rc * 4 + e][kk] = (u16)mv[e]; tile[2][rc * 4 + e][kk] = (u16)lv[e]; }
+            for (int e = 0; e < 4; ++e) {
+                const int at = (((kk >> 3) ^ (rc & 7)) << 3) | (kk & 7);
+                tile[0][rc * 4 + e][at] = (u16)hv[e]; tile[1][rc * 4 + e][at] = (u16)mv[e]; tile[2][rc * 4 + e][at] = (u16)lv[e];
+            }
         }
         __syncthreads();
         const int row = tid / 4, kc = (tid % 4) * 16;
 #pragma unroll
         for (int p = 0; p < 3; ++p) {
             u16* out = planes + (u64)p * plane + (r0 + row) * Kp + k0 + kc;
-            *(u32x4*)out = *(const u32x4*)&tile[p][row][kc];
-            *(u32x4*)(out + 8) = *(const u32x4*)&tile[p][row][kc + 8];
+            const int sw = (row >> 2) & 7;
+            *(u32x4*)out = *(const u32x4*)&tile[p][row][((kc >> 3) ^ sw) << 3];
+            *(u32x4*)(out + 8) = *(const u32x4*)&tile[p][row][(((kc >> 3) + 1) ^ sw) << 3];
         }
     }
     if (least < kX3Smallest || most >= 0x7F800000u) *flag = seq;
