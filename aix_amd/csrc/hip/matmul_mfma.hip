@@ -1645,9 +1645,10 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
     if (bn == 0 || (limit > 0 && least >= limit)) return -1;
     const uint64_t tiles = (M / 128) * (N / bn);
     if (tiles * count * 2 < (uint64_t)ctx->cus || tiles >= (1ull << 31)) return -1;
-    // a long K under less than a round of tiles: the kernels that split K over workgroups fill the chip better
-    // ([1024, 4096] x [4096, 2048]: 128 tiles, 41 us here against 37 with K split)
-    if (!batch && K >= 4096 && tiles < (uint64_t)ctx->cus) return -1;
+    // a long K under less than three quarters of a round of tiles: the kernels that split K over workgroups fill the chip
+    // better ([1024, 4096] x [4096, 2048]: 128 tiles, 41 us here against 37 with K split; [768, 8192]^T x [8192, 8192]: 192
+    // tiles, 131 us here against 146)
+    if (!batch && K >= 4096 && tiles * 4 < (uint64_t)ctx->cus * 3) return -1;
     if (!((a_k || a_m) && (b_k || b_n) && la % 8 == 0 && lb % 8 == 0 && la < (1ull << 27) && lb < (1ull << 27) && aligned16(qa) && aligned16(qb))) return -1;
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
