@@ -22,7 +22,7 @@ struct MlpConfig {
     int32_t captureAt{-1};    // >= 0 (with adamInPlace and a StepCapture): that step is captured, it and every later one is a replay
 };
 
-inline bool dev_is_capturing(const StepCapture* capture, const MlpConfig& cfg, int s) { return capture && cfg.captureAt >= 0 && s >= cfg.captureAt; }
+inline bool stepIsCaptured(const StepCapture* capture, const MlpConfig& cfg, int s) { return capture && cfg.captureAt >= 0 && s >= cfg.captureAt; }
 
 struct MlpHost {              // host arrays, f32, row-major
     const float* x;           // [batch, in]
@@ -57,7 +57,7 @@ inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* l
         const Tensor logits = l3.forward(relu(l2.forward(relu(l1.forward(x)))));
         loss = crossEntropy(softmax(logits, 1, true), y);
         if (cfg.singlePass) loss.backwardOnce(); else loss.backward();
-        if (grad_norms && s < grad_norm_steps && !dev_is_capturing(capture, cfg, s)) {
+        if (grad_norms && s < grad_norm_steps && !stepIsCaptured(capture, cfg, s)) {
             const auto n0 = std::chrono::steady_clock::now();
             const Tensor* params[6] = {&l1.w, &l1.b, &l2.w, &l2.b, &l3.w, &l3.b};
             for (int p = 0; p < 6; ++p) grad_norms[s * 6 + p] = params[p]->grad().l2Norm();

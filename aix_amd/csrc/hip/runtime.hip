@@ -2,6 +2,7 @@
 
 #include "common.hpp"
 
+#include <atomic>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -353,7 +354,8 @@ bool disk_load(const std::string& path, std::vector<char>& code)
 
 bool disk_store(const std::string& path, const std::vector<char>& code)
 {
-    const std::string tmp = path + ".tmp." + std::to_string((long)getpid());
+    static std::atomic<unsigned> serial{0};                  // two contexts of one process may store the same kernel at once
+    const std::string tmp = path + ".tmp." + std::to_string((long)getpid()) + "." + std::to_string(serial.fetch_add(1));
     std::FILE* f = std::fopen(tmp.c_str(), "wb");
     if (!f) return false;
     const uint64_t size = code.size(), hash = fnv1a(code.data(), code.size(), 0xcbf29ce484222325ull);
