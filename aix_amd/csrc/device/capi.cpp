@@ -203,6 +203,7 @@ int32_t aixhip_capture_end(aixhip_device* dev, aixhip_graph** out)
         *out = reinterpret_cast<aixhip_graph*>(D(dev).endCapture());
     });
 }
+int32_t aixhip_capture_abort(aixhip_device* dev) { return guarded([&] { D(dev).abortCapture(); }); }
 int32_t aixhip_graph_replay(aixhip_device* dev, aixhip_graph* graph) { return guarded([&] { D(dev).replay(reinterpret_cast<DeviceHIP::StepGraph*>(graph)); }); }
 int32_t aixhip_graph_destroy(aixhip_device* dev, aixhip_graph* graph) { return guarded([&] { D(dev).destroyGraph(reinterpret_cast<DeviceHIP::StepGraph*>(graph)); }); }
 int32_t aixhip_set_cache_limit(aixhip_device* dev, uint64_t bytes) { return guarded([&] { D(dev).setCacheLimit((size_t)bytes); }); }

@@ -656,6 +656,16 @@ DeviceHIP::StepGraph* DeviceHIP::endCapture()
     return reinterpret_cast<StepGraph*>(g);
 }
 
+// An open capture given up: what is still recorded or waits is flushed into the graph like at endCapture() -- nothing runs --
+// and the graph is thrown away.  The results of the abandoned stretch are undefined.
+void DeviceHIP::abortCapture()
+{
+    if (!m_capturing) return;
+    StepGraph* g = nullptr;
+    try { g = endCapture(); } catch (...) { g = nullptr; }   // (a failing flush has ended the capture itself)
+    if (g) destroyGraph(g);
+}
+
 void DeviceHIP::replay(StepGraph* graph)
 {
     if (m_capturing) throw std::runtime_error("DeviceHIP::replay: a capture is open");

@@ -121,6 +121,7 @@ public:
     struct StepGraph;
     void beginCapture();                  // flushes and waits first
     StepGraph* endCapture();              // flushes what was recorded into the graph; nothing of it has run yet
+    void abortCapture();                  // gives an open capture up (after an error inside it, say): nothing of it runs, the device is usable again
     void replay(StepGraph* graph);        // enqueues the captured work (after whatever is pending)
     size_t graphNodes(const StepGraph* graph) const;
     void destroyGraph(StepGraph* graph);

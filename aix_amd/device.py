@@ -61,6 +61,7 @@ _SIGNATURES = {
     "aixhip_set_cache_limit": [_P, C.c_uint64],
     "aixhip_capture_begin": [_P],
     "aixhip_capture_end": [_P, C.POINTER(_P)],
+    "aixhip_capture_abort": [_P],
     "aixhip_graph_replay": [_P, _P],
     "aixhip_graph_destroy": [_P, _P],
     "aixhip_memory_stats": [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)],

@@ -152,6 +152,9 @@ aixk_ctx* aixhip_kernel_context(aixhip_device* dev);
 typedef struct aixhip_graph aixhip_graph;
 int32_t aixhip_capture_begin(aixhip_device* dev);
 int32_t aixhip_capture_end(aixhip_device* dev, aixhip_graph** out);
+/* Gives an open capture up -- after an error inside it, say: nothing of it runs, its results are undefined, the device is
+ * usable again.  Without an open capture: nothing. */
+int32_t aixhip_capture_abort(aixhip_device* dev);
 int32_t aixhip_graph_replay(aixhip_device* dev, aixhip_graph* graph);
 int32_t aixhip_graph_destroy(aixhip_device* dev, aixhip_graph* graph);
 int32_t aixhip_memory_stats(aixhip_device* dev, uint64_t* live_bytes, uint64_t* cached_bytes);

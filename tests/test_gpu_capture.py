@@ -92,6 +92,18 @@ def test_captured_updates_in_place_advance_step_by_step(dev):
     extra = C.c_void_p()
     dev.dev.call("capture_end", C.byref(extra))
     dev.dev.call("graph_destroy", extra)
+    # a capture given up: nothing of it runs, the device goes on as before, another capture can be opened
+    before = dev.fetch(px, x.storage).copy()
+    dev.dev.call("capture_begin")
+    issue()
+    assert dev.dev.status("capture_begin") == 2                 # one open capture per device
+    dev.dev.call("capture_abort")
+    dev.dev.call("capture_abort")                               # (without an open capture: nothing)
+    T.assert_same_bits(dev.fetch(px, x.storage), before, "an abandoned capture has run nothing")
+    dev.dev.call("graph_replay", graph)
+    step_on_oracle()
+    T.assert_same_bits(dev.fetch(px, x.storage), x.storage, "a replay after an abandoned capture")
+    assert dev.dev.status("graph_replay", None) == 1            # a null graph is an invalid argument
     dev.dev.call("graph_destroy", graph)
     dev.release()
 
