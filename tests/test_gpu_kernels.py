@@ -767,6 +767,28 @@ def test_matmul_mid_tiles(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", [O.F16, O.BF16], ids=ids)
+def test_matmul_random_whole_tile_shapes(gpu, dtype):
+    """Random 16-bit products whose extents are multiples of the tile sizes (M of 128, N of 64, K of 64) in random operand
+    layouts: whichever kernel and tile the cost model picks -- 256 x 256, 128 x {128, 192, 256}, the register-staged
+    tiles below half a tile per compute unit, K splits under a long K -- the result must stay within the 16-bit matmul
+    bar of the exactly accumulated product.  Tile counts that are and are not multiples of 8 (the XCD-aware numbering is
+    a bijection only for the former), odd numbers of tile rows, one to twelve K steps."""
+    rng = np.random.default_rng(23900 + dtype)
+    for trial in range(14):
+        m = 128 * int(rng.integers(1, 41))
+        n = 64 * int(rng.integers(1, 41))
+        k = 64 * int(rng.integers(1, 13)) if trial % 5 else 64 * int(rng.integers(64, 80))
+        if trial == 0:
+            m, n, k = 128 * 37, 192 * 7, 64 * 3                 # 259 tiles of 128 x 192: plain numbering, a ragged last group of tile rows
+        ka, kb = (str(rng.choice(["contig", "transposed"])) for _ in range(2))
+        scale = 1.0 / np.sqrt(k)
+        a = T.view_tensor(rng, dtype, [m, k], ka, lo=-scale, hi=scale)
+        b = T.view_tensor(rng, dtype, [k, n], kb, lo=-1, hi=1)
+        check_matmul(gpu, a, b, f"random whole-tile matmul {NAMES[dtype]} {m}x{k}x{n} {ka}/{kb}")
+        gpu.release()
+
+
+@pytest.mark.parametrize("dtype", [O.F16, O.BF16], ids=ids)
 def test_matmul_small_tiles(gpu, dtype):
     """16-bit outputs too small for 64 x 64 tiles to fill the chip (attention heads and the like): the
     32 x 32-tile kernel that splits K over its four waves, every operand layout consumed in place --
