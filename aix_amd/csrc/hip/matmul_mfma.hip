@@ -431,7 +431,7 @@ struct PlanesArgs { u64 plane_a, plane_b; u32* flag; u32 seq; };      // bytes f
 template <class T, bool AT, bool BT, int BM, int BN, bool PLANES = false>
 __global__ __launch_bounds__(512) void gemm_direct16_k(GemmArgs g, BatchArgs bt, PlanesArgs pl)
 {
-    static_assert((BM == 128 && (BN == 128 || BN == 192 || BN == 256)) || (BM == 256 && BN == 256 && PLANES), "tiles this kernel is written for");
+    static_assert((BM == 128 && (BN == 128 || BN == 192 || BN == 256)) || (BM == 256 && BN == 256), "tiles this kernel is written for");
     static_assert(!PLANES || (!AT && !BT), "planes are laid out K-contiguous");
     constexpr int BK = 64, ASZ = BM * 128, BSZ = BN * 128, STAGE = ASZ + BSZ;
     constexpr int WGN = 4, TI = BM / 32, TJ = BN / 64, WROWS = TI * 16, WCOLS = TJ * 16;
@@ -1634,7 +1634,7 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
     }
     // rounds of workgroups x tile area, a smaller tile's flop 1.35 times as dear as one of the 256 x 256 kernel (more
     // fragment traffic per flop; measured: 4096^3 111 us on 256 x 256 tiles, 137 on 128 x 256); the larger tile on a tie
-    uint64_t bn = 0;
+    uint64_t bn = 0, bm = 128;
     double least = 0;
     for (uint64_t cand : {256, 192, 128}) {
         if (N % cand != 0) continue;
@@ -1642,8 +1642,16 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
         const double cost = 1.35 * (double)(((tiles + (uint64_t)ctx->cus - 1) / (uint64_t)ctx->cus) * cand * 128);
         if (bn == 0 || cost < least) { bn = cand; least = cost; }
     }
+    // stacks and groups also have the 256 x 256 tile of this kernel (a single product of whole 256 x 256 tiles has
+    // gemm_nt16_direct_k): 24 weight gradients [768, 8192]^T x [8192, 768] are 216 such tiles, one round of the chip, where
+    // 432 tiles of 128 x 256 are 1.7
+    if (batch && M % 256 == 0 && N % 256 == 0) {
+        const uint64_t tiles = (M / 256) * (N / 256) * count;
+        const double cost = (double)(((tiles + (uint64_t)ctx->cus - 1) / (uint64_t)ctx->cus) * 65536);
+        if (bn == 0 || cost < least) { bn = 256; bm = 256; least = cost; }
+    }
     if (bn == 0 || (limit > 0 && least >= limit)) return -1;
-    const uint64_t tiles = (M / 128) * (N / bn);
+    const uint64_t tiles = (M / bm) * (N / bn);
     if (tiles * count * 2 < (uint64_t)ctx->cus || tiles >= (1ull << 31)) return -1;
     // a long K under less than three quarters of a round of tiles: the kernels that split K over workgroups fill the chip
     // better ([1024, 4096] x [4096, 2048]: 128 tiles, 41 us here against 37 with K split; [768, 8192]^T x [8192, 8192]: 192
@@ -1653,10 +1661,10 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
     GemmArgs g{};
     g.a = qa; g.b = qb; g.c = out->data;
     g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
-    g.tiles_m = (u32)(M / 128); g.tiles_n = (u32)(N / bn);
+    g.tiles_m = (u32)(M / bm); g.tiles_n = (u32)(N / bn);
     const u32 n = g.tiles_m * g.tiles_n;
     g.swizzle = n % 8u == 0 ? 1u : 0u;
-    const size_t lds = 2 * (128 + bn) * 128;
+    const size_t lds = 2 * (bm + bn) * 128;
     const bool at = !a_k, tb = !b_k;
     auto launch = [&](auto kernel) {
         AIXK_TRY(set_lds(kernel, lds));
@@ -1664,18 +1672,20 @@ int launch_direct16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* 
         AIXK_HIP(hipGetLastError());
         return (int)AIXK_OK;
     };
-    auto by_form = [&](auto dtype_tag, auto bn_tag) {
+    auto by_form = [&](auto dtype_tag, auto bn_tag, auto bm_tag) {
         typedef decltype(dtype_tag) T;
-        constexpr int BN = decltype(bn_tag)::value;
-        if (!at && !tb) return launch(gemm_direct16_k<T, false, false, 128, BN>);
-        if (!at && tb) return launch(gemm_direct16_k<T, false, true, 128, BN>);
-        if (at && !tb) return launch(gemm_direct16_k<T, true, false, 128, BN>);
-        return launch(gemm_direct16_k<T, true, true, 128, BN>);
+        constexpr int BN = decltype(bn_tag)::value, BM = decltype(bm_tag)::value;
+        if (!at && !tb) return launch(gemm_direct16_k<T, false, false, BM, BN>);
+        if (!at && tb) return launch(gemm_direct16_k<T, false, true, BM, BN>);
+        if (at && !tb) return launch(gemm_direct16_k<T, true, false, BM, BN>);
+        return launch(gemm_direct16_k<T, true, true, BM, BN>);
     };
     auto by_tile = [&](auto dtype_tag) {
-        if (bn == 256) return by_form(dtype_tag, std::integral_constant<int, 256>{});
-        if (bn == 192) return by_form(dtype_tag, std::integral_constant<int, 192>{});
-        return by_form(dtype_tag, std::integral_constant<int, 128>{});
+        constexpr std::integral_constant<int, 128> rows128{};
+        if (bm == 256) return by_form(dtype_tag, std::integral_constant<int, 256>{}, std::integral_constant<int, 256>{});
+        if (bn == 256) return by_form(dtype_tag, std::integral_constant<int, 256>{}, rows128);
+        if (bn == 192) return by_form(dtype_tag, std::integral_constant<int, 192>{}, rows128);
+        return by_form(dtype_tag, std::integral_constant<int, 128>{}, rows128);
     };
     return out->dtype == AIXK_BF16 ? by_tile(bf16{}) : by_tile(f16{});
 }
