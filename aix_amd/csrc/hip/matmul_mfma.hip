@@ -1961,7 +1961,12 @@ int matmul_mfma(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, c
         // two workgroups per compute unit hide each other's split-and-stage phases: with fewer tiles than that, K is split
         // over workgroups if it is long enough, else the f32 MFMA kernels below take the product
         uint64_t splits = 1;
-        if (t128 < fill && K >= 2048) splits = std::min<uint64_t>({steps / 16, (fill + t128 - 1) / t128, (uint64_t)64});
+        // (as many splits as still fit one round of two workgroups per compute unit: [784, 4096]^T x [4096, 2048], 112 tiles,
+        // takes 107 us with 4 splits and 131 with 5, whose 560 workgroups spill into a second round)
+        if (t128 < fill && K >= 2048) {
+            const uint64_t whole = fill / t128, over = (fill + t128 - 1) / t128;
+            splits = std::max<uint64_t>(1, std::min<uint64_t>({steps / 16, t128 * whole >= fill - fill / 8 ? whole : over, (uint64_t)64}));
+        }
         if (!only_if && t128 * splits >= fill - fill / 8 && t128 >= (uint64_t)ctx->cus / 4) {
             const u32 n = grid_of(g, 128, 128);
             SplitArgs sk{};
