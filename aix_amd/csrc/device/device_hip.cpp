@@ -156,8 +156,11 @@ struct DeviceHIP::Extras {
     // row reductions are recorded and fused with the operators around them (AIXHIP_FUSE_ROW_REDUCTIONS=0 switches it off)
     bool fuseRowReductions = [] { const char* e = std::getenv("AIXHIP_FUSE_ROW_REDUCTIONS"); return !(e && e[0] == '0'); }();
     // matmul calls waiting to be issued together (see DeviceHIP::matmul): per group descriptors in three parallel arrays
-    struct Group { std::vector<aixhip_tensor> a, b, out; };
+    // and what the group reads and writes (block starts); `leaves` marks the groups that the call being looked at must
+    // come after (see meetsRead / meetsWrite)
+    struct Group { std::vector<aixhip_tensor> a, b, out; aixhip::fuse::PointerSet reads, writes; bool leaves{false}; };
     std::array<Group, 8> groups;
+    size_t grouped{0};                  // products waiting in all groups
     // sliceSet and argmaxIndicesTo calls waiting to leave as one launch each (see DeviceHIP::sliceSet, argmaxIndicesTo)
     std::vector<aixk_slice_item> slices;
     std::vector<aixk_argmax_item> onehots;
@@ -165,23 +168,49 @@ struct DeviceHIP::Extras {
     std::array<std::vector<aixk_colsum_item>, 3> colsums;
     // second halves of sums over everything (see DeviceHIP::emitFused): one element type at a time
     std::vector<aixk_partials_item> partialSums;
-    // what the waiting calls of all three kinds read and write (block starts), so that a new call knows in one lookup
+    // what the waiting calls other than products read and write (block starts), so that a new call knows in one lookup
     // whether it may wait beside them; per destination of waiting sliceSet calls, how it was described and the windows
     // written so far
     aixhip::fuse::PointerSet waitReads, waitWrites;
     struct SliceWindows { aixhip_tensor dst; uint64_t dim; std::vector<std::pair<uint64_t, uint64_t>> ranges; };
     std::unordered_map<const void*, SliceWindows> sliceDsts;
-    bool anyPending() const { if (!slices.empty() || !onehots.empty() || !partialSums.empty()) return true; for (const auto& c : colsums) if (!c.empty()) return true; for (const auto& g : groups) if (!g.out.empty()) return true; return false; }
-    // a call that reads r0, r1 and writes w neither uses what waits nor is used by it
-    bool apartFromWaiting(const void* r0, const void* r1, const void* w) const
+    bool anyPending() const { if (grouped || !slices.empty() || !onehots.empty() || !partialSums.empty()) return true; for (const auto& c : colsums) if (!c.empty()) return true; return false; }
+    bool anyUses() const { return grouped + waitReads.size() + waitWrites.size() != 0; }
+    // A call is about to read p / to write p: does it have to come after something that waits?  The groups of products it
+    // has to come after are marked, and only they leave with the other kinds of waiting calls (issuePending(true)): a
+    // weight gradient of a backward pass goes on waiting for the other layers' while the small products of attention
+    // come and go.  Whoever gets `true` sends the waiting calls off, so that no mark outlives the question.
+    bool meetsRead(const void* p)
     {
-        if ((r0 && waitWrites.contains(r0)) || (r1 && waitWrites.contains(r1))) return false;
-        return !waitWrites.contains(w) && !waitReads.contains(w);
+        if (!p) return false;
+        bool hit = waitWrites.size() && waitWrites.contains(p);
+        if (grouped) for (auto& g : groups) if (!g.out.empty() && g.writes.contains(p)) hit = g.leaves = true;
+        return hit;
+    }
+    bool meetsWrite(const void* p)
+    {
+        if (!p) return false;
+        bool hit = (waitWrites.size() && waitWrites.contains(p)) || (waitReads.size() && waitReads.contains(p));
+        if (grouped) for (auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) hit = g.leaves = true;
+        return hit;
+    }
+    // a call that reads r0, r1 and writes w neither uses what waits nor is used by it (every operand is looked at: all
+    // groups in its way are marked)
+    bool apartFromWaiting(const void* r0, const void* r1, const void* w)
+    {
+        bool hit = meetsRead(r0);
+        hit = meetsRead(r1) || hit;
+        hit = meetsWrite(w) || hit;
+        return !hit;
     }
     // p is an operand or the result of a call that waits
-    bool waitingUses(const void* p) const { return p && waitReads.size() + waitWrites.size() && (waitWrites.contains(p) || waitReads.contains(p)); }
-    // p is the result of a call that waits
-    bool waitingWrites(const void* p) const { return p && waitWrites.size() && waitWrites.contains(p); }
+    bool waitingUses(const void* p) const
+    {
+        if (!p || !anyUses()) return false;
+        if (waitWrites.contains(p) || waitReads.contains(p)) return true;
+        if (grouped) for (const auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) return true;
+        return false;
+    }
     void noteWaiting(const void* r0, const void* r1, const void* w)
     {
         if (r0) waitReads.insert(r0);
@@ -565,20 +594,23 @@ void DeviceHIP::flushForOperands(const void* a, const void* b, const void* c, bo
     markTouched(b);
     markTouched(c);
     auto& ex = *m_extras;
-    auto meets = [&] {
+    auto meets = [&] {                                      // (every operand is asked about: all the groups in the way are marked)
+        bool any = false;
+        if (!ex.anyUses()) return any;
         for (int k = 0; k < 3; ++k) {
-            if (k == last ? ex.waitingUses(named[k]) || ex.waitingUses(bases[k]) : ex.waitingWrites(named[k]) || ex.waitingWrites(bases[k])) return true;
+            if (k == last) { any = ex.meetsWrite(named[k]) || any; any = ex.meetsWrite(bases[k]) || any; }
+            else           { any = ex.meetsRead(named[k]) || any;  any = ex.meetsRead(bases[k]) || any; }
         }
-        return false;
+        return any;
     };
-    if (meets()) issuePending();
+    if (meets()) issuePending(true);
     if (!dependent) return;
     for (int k = 0; k < 3; ++k) {
         if (named[k]) m_engine->recordExternalRead(named[k]);
         if (bases[k]) m_engine->recordExternalRead(bases[k]);
     }
     flushWindow(false);
-    if (meets()) issuePending();                            // (a one-hot replayed on its own has just begun to wait)
+    if (meets()) issuePending(true);                        // (a one-hot replayed on its own has just begun to wait)
 }
 
 // The planner orders recorded operators by the addresses of their buffers.  An operand that points into the middle of
@@ -880,7 +912,8 @@ void DeviceHIP::emitSingle(const OpRecord& op)
         // row wait for each other and leave in one launch (see argmaxIndicesTo())
         auto& ex = *m_extras;
         AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
-        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.batchFlatKernels || !ex.apartFromWaiting(op.input0.data, nullptr, op.output.data)) issuePending();
+        const bool apart = ex.apartFromWaiting(op.input0.data, nullptr, op.output.data);
+        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.batchFlatKernels || !apart) issuePending(true);
         aixk_argmax_item item{};
         toPod(op.input0, &item.src); toPod(op.output, &item.dst);
         item.dim = op.input0.rank - 1;
@@ -891,8 +924,8 @@ void DeviceHIP::emitSingle(const OpRecord& op)
         return;
     }
     {
-        const auto& ex = *m_extras;                         // what waits and is used here, or uses the result's buffer, goes first
-        if (ex.waitingUses(op.output.data) || ex.waitingWrites(op.input0.data) || (op.hasInput1 && ex.waitingWrites(op.input1.data))) issuePending();
+        auto& ex = *m_extras;                               // what waits and is used here, or uses the result's buffer, goes first
+        if (ex.anyUses() && !ex.apartFromWaiting(op.input0.data, op.hasInput1 ? op.input1.data : nullptr, op.output.data)) issuePending(true);
     }
     AIXHIP_TRACE("single %s  %zu elements", aixhip::fuse::opName(op.type), op.output.size);
     if ((op.type == OpType::Fill || op.type == OpType::FillMin) && op.output.dense && op.output.size <= 65536 && m_extras->batchFlatKernels) {
@@ -944,13 +977,13 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
 {
     {
         // calls that wait stay waiting unless this kernel reads what they write or writes what they use
-        const auto& ex = *m_extras;
+        auto& ex = *m_extras;
         bool meets = false;
-        if (ex.waitReads.size() + ex.waitWrites.size()) {
-            for (const auto& v : d.inputBuffers) meets = meets || ex.waitingWrites(v.data);
-            for (const auto& v : d.outputBuffers) meets = meets || ex.waitingUses(v.data);
+        if (ex.anyUses()) {
+            for (const auto& v : d.inputBuffers) meets = ex.meetsRead(v.data) || meets;
+            for (const auto& v : d.outputBuffers) meets = ex.meetsWrite(v.data) || meets;
         }
-        if (meets) issuePending();
+        if (meets) issuePending(true);
     }
     constexpr size_t kMaxOperands = 64;
     const size_t NI = d.inputBuffers.size(), NO = d.outputBuffers.size();
@@ -1109,9 +1142,9 @@ void DeviceHIP::emitFused(const FusedSubgraphDescriptor& d)
         if (!ex.batchFlatKernels) { check(aixk_sum_partials(m_ctx, wholes[k].scratch, grid, &dst, wholes[k].init)); continue; }
         // the second half waits like a small product: the scalar gradients of a backward pass are read when it reaches
         // its leaves, and leave together then (the partial sums' block stays in limbo until they have: releaseLimbo)
-        if (ex.partialSums.size() >= AIXK_PARTIALS_ITEMS_MAX || (!ex.partialSums.empty() && ex.partialSums[0].dst.dtype != dst.dtype) ||
-            !ex.apartFromWaiting(wholes[k].scratch, nullptr, dst.data))
-            issuePending();
+        const bool apart = ex.apartFromWaiting(wholes[k].scratch, nullptr, dst.data);
+        if (ex.partialSums.size() >= AIXK_PARTIALS_ITEMS_MAX || (!ex.partialSums.empty() && ex.partialSums[0].dst.dtype != dst.dtype) || !apart)
+            issuePending(true);
         ex.partialSums.push_back(aixk_partials_item{wholes[k].scratch, grid, dst, wholes[k].init});
         ex.noteWaiting(wholes[k].scratch, nullptr, dst.data);
         markTouched(dst.data);
@@ -1294,7 +1327,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             aixhip_tensor pa, pb, pr; toPod(a, &pa, "matmul"); toPod(b, &pb, "matmul"); toPod(result, &pr, "matmul");
             // it may read no waiting result and overwrite nothing that waits: all waiting calls are then independent of
             // each other, whatever group they wait in, and the groups may be issued in any order
-            if (!ex.apartFromWaiting(pa.data, pb.data, pr.data)) issuePending();
+            if (!ex.apartFromWaiting(pa.data, pb.data, pr.data)) issuePending(true);
             // the group of its shape and operand layout (forward and backward products of attention alternate between
             // two or three of them), or the emptiest slot
             Extras::Group* into = nullptr;
@@ -1306,7 +1339,8 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             }
             if (!into) { issuePending(); into = &ex.groups[0]; }
             into->a.push_back(pa); into->b.push_back(pb); into->out.push_back(pr);
-            ex.noteWaiting(pa.data, pb.data, pr.data);
+            into->reads.insert(pa.data); into->reads.insert(pb.data); into->writes.insert(pr.data);
+            ++ex.grouped;
             markTouched(a.data); markTouched(b.data); markTouched(result.data);
             return;
         }
@@ -1327,13 +1361,15 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
     check(status);
 }
 
-void DeviceHIP::issuePending()
+// With `marked`, only those groups of products leave that the caller has just found in its way (Extras::meetsRead,
+// meetsWrite); every waiting call is independent of every other, so the rest may go on waiting.
+void DeviceHIP::issuePending(bool marked)
 {
     const Marker marker_("calls that waited leave");
     auto& ex = *m_extras;
     if (ex.anyPending()) {
         size_t products = 0, sums = 0;
-        for (const auto& g : ex.groups) products += g.out.size();
+        for (const auto& g : ex.groups) if (!marked || g.leaves) products += g.out.size();
         for (const auto& c : ex.colsums) sums += c.size();
         AIXHIP_TRACE("-- what waited leaves: %zu sliceSet, %zu argmaxIndicesTo, %zu reduceTo, %zu sums of partials, %zu matmul", ex.slices.size(), ex.onehots.size(), sums,
                      ex.partialSums.size(), products);
@@ -1378,10 +1414,13 @@ void DeviceHIP::issuePending()
     }
     ex.waitReads.clear(); ex.waitWrites.clear(); ex.sliceDsts.clear();
     for (auto& g : ex.groups) {
-        if (g.out.empty()) continue;
+        const bool leaves = !marked || g.leaves;
+        g.leaves = false;
+        if (g.out.empty() || !leaves) continue;
         const uint32_t count = (uint32_t)g.out.size();
         sent(count == 1 ? aixk_matmul(m_ctx, &g.a[0], &g.b[0], &g.out[0]) : aixk_matmul_grouped(m_ctx, g.a.data(), g.b.data(), g.out.data(), count), count);
-        g.a.clear(); g.b.clear(); g.out.clear();
+        g.a.clear(); g.b.clear(); g.out.clear(); g.reads.clear(); g.writes.clear();
+        ex.grouped -= count;
     }
     if (first == AIXK_OK) return;
     const std::string msg = "DeviceHIP: " + firstError + " (reported when the calls that waited were sent off: " + std::to_string(dropped) +
@@ -1536,7 +1575,8 @@ void DeviceHIP::reduceTo(const DeviceTensorParams& src, const DeviceTensorParams
             flushWindow(false);
         }
         auto& sums = ex.colsums[slot];
-        if (sums.size() >= AIXK_COLSUM_ITEMS_MAX || !ex.apartFromWaiting(src.data, nullptr, dst.data)) issuePending();
+        const bool apart = ex.apartFromWaiting(src.data, nullptr, dst.data);
+        if (sums.size() >= AIXK_COLSUM_ITEMS_MAX || !apart) issuePending(true);
         AIXHIP_TRACE("   (waits: %zu columns)", dst.size);
         aixk_colsum_item item{};
         toPod(src, &item.src, "reduceTo"); toPod(dst, &item.dst, "reduceTo");
@@ -1612,7 +1652,8 @@ void DeviceHIP::argmaxIndicesTo(const DeviceTensorParams& src, const DeviceTenso
             m_engine->recordExternalRead(dst.data);             // (a fill of the destination still recorded goes first, it does not wait)
             flushWindow(false);
         }
-        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !ex.apartFromWaiting(src.data, nullptr, dst.data)) issuePending();
+        const bool apart = ex.apartFromWaiting(src.data, nullptr, dst.data);
+        if (ex.onehots.size() >= AIXK_ARGMAX_ITEMS_MAX || !apart) issuePending(true);
         aixk_argmax_item item{};
         toPod(src, &item.src, "argmaxIndicesTo"); toPod(dst, &item.dst, "argmaxIndicesTo");
         item.dim = dim;
@@ -1666,8 +1707,19 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
             }
             bool independent = ex.slices.size() < AIXK_SLICE_ITEMS_MAX &&
                                (ex.slices.empty() || dataTypeSize(static_cast<DataType>(ex.slices[0].src.dtype)) == dataTypeSize(src.dtype));
+            // (products that wait: the copy comes after those that write its source or use its destination)
+            bool apartFromProducts = true;
+            if (ex.grouped) {
+                for (auto& g : ex.groups) {
+                    if (g.out.empty() || !(g.writes.contains(src.data) || g.writes.contains(dst.data) || g.reads.contains(dst.data))) continue;
+                    g.leaves = true;
+                    apartFromProducts = false;
+                }
+            }
             auto windows = ex.sliceDsts.find(dst.data);
-            if (independent && windows != ex.sliceDsts.end()) {
+            if (!apartFromProducts) {
+                independent = false;
+            } else if (independent && windows != ex.sliceDsts.end()) {
                 // another window of a destination that waits: apart if nothing that waits reads the destination, it is
                 // described the same way, and the ranges do not meet
                 const auto& w = windows->second;
@@ -1678,7 +1730,7 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
             } else if (independent) {
                 independent = ex.apartFromWaiting(src.data, nullptr, dst.data);
             }
-            if (!independent) issuePending();
+            if (!independent) issuePending(true);
             if (step == 1) {
                 auto& w = ex.sliceDsts[dst.data];
                 if (w.ranges.empty()) { w.dst = item.dst; w.dim = dim; }

@@ -192,7 +192,7 @@ private:
     void issueFlatBatch();
     bool recordRowReduction(aixhip::fuse::OpType type, const DeviceTensorParams& src, const DeviceTensorParams& dst, uint64_t init);
     void joinBatch(const aixhip::fuse::FusedSubgraphDescriptor& d, aixk_module* mod, const std::string& entry, uint64_t grid, const std::function<std::string()>& manySource);
-    void issuePending();                                     // the waiting matmul and sliceSet calls, one launch per run (see matmul(), sliceSet())
+    void issuePending(bool marked = false);                                   // the waiting matmul and sliceSet calls, one launch per run (see matmul(), sliceSet())
 
     aixk_ctx* m_ctx{nullptr};
     std::unique_ptr<aixhip::fuse::FuseEngine> m_engine;

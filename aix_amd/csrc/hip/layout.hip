@@ -8,7 +8,9 @@
 
 #include "common.hpp"
 
+#include <algorithm>
 #include <utility>
+#include <vector>
 
 using namespace aixd;
 using namespace aixk;
@@ -30,6 +32,47 @@ template <class F> int by_size(int dtype, F&& f)
         case 8: return f(u64{});
         default: return fail(AIXK_EINVAL, "unknown element type %d", dtype);
     }
+}
+
+struct alignas(16) u128 { u64 lo, hi; };
+template <class F> int by_bytes(size_t bytes, F&& f)
+{
+    switch (bytes) {
+        case 1: return f(u8{});
+        case 2: return f(u16{});
+        case 4: return f(u32{});
+        case 8: return f(u64{});
+        case 16: return f(u128{});
+        default: return fail(AIXK_EINVAL, "no word of %zu bytes", bytes);
+    }
+}
+
+// A strided copy moves words, not values, so both views may be read as arrays of wider words where their innermost runs
+// allow it: `f` elements at a time if in both views the last dim is dense and a multiple of f long, every other stride and
+// the offset are multiples of f and the storage is aligned to f elements -- flat logical indices then pair up f at a time
+// in both views.  (A head's [512, 64] slab of 2-byte elements inside a [8192, 768] activation: 16-byte words, an eighth of
+// the index arithmetic and of the memory instructions.)
+inline size_t widest_factor(const aixhip_tensor* t, size_t esz)
+{
+    if (t->rank == 0 || t->strides[t->rank - 1] != 1) return 1;
+    size_t f = 16 / esz;
+    const int last = t->rank - 1;
+    auto fits = [&](size_t k) {
+        if (t->shape[last] % k != 0 || t->offset % k != 0 || ((uintptr_t)t->data) % (k * esz) != 0) return false;
+        for (int d = 0; d < last; ++d) if (t->strides[d] % k != 0) return false;
+        return true;
+    };
+    while (f > 1 && !fits(f)) f /= 2;
+    return f;
+}
+inline void widen(aixhip_tensor* t, size_t f)
+{
+    if (f <= 1) return;
+    const int last = t->rank - 1;
+    t->shape[last] /= f;
+    for (int d = 0; d < last; ++d) t->strides[d] /= f;
+    t->offset /= f;
+    t->size /= f;
 }
 
 // Position of flat logical index i inside one collapsed view.
@@ -431,13 +474,19 @@ int gather_into(aixk_ctx* ctx, const aixhip_tensor* src, void* dst, uint64_t n)
     });
 }
 
-int copy_views(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_tensor* dst, uint64_t n)
+int copy_views(aixk_ctx* ctx, const aixhip_tensor* src_in, const aixhip_tensor* dst_in, uint64_t n)
 {
     if (n == 0) return AIXK_OK;
+    const size_t esz = aixk_dtype_size(src_in->dtype);
+    aixhip_tensor wide_src = *src_in, wide_dst = *dst_in;
+    const size_t f = n == numel(src_in) && n == numel(dst_in) ? std::min(widest_factor(src_in, esz), widest_factor(dst_in, esz)) : 1;
+    widen(&wide_src, f); widen(&wide_dst, f);
+    n /= f;
+    const aixhip_tensor *src = &wide_src, *dst = &wide_dst;
     Space<1> ssp, dsp;
     if (!collapse1(src, &ssp) || !collapse1(dst, &dsp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
     const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(dst) < (1ull << 31);
-    return by_size(src->dtype, [&](auto tag) {
+    return by_bytes(esz * f, [&](auto tag) {
         typedef decltype(tag) W;
         const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
         if (small) hipLaunchKernelGGL((copy_views_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const W*)src->data, (W*)dst->data, ssp, dsp, (u64)n);
@@ -516,6 +565,9 @@ int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_
     u32* starts = (u32*)(host + table_bytes);
     bool small = true;
     u32 grid = 0;
+    // the windows of the destinations, and the widest word every item can be copied in
+    std::vector<aixhip_tensor> windows(count);
+    size_t f = 16 / esz;
     for (uint32_t k = 0; k < count; ++k) {
         const aixhip_tensor *src = &items[k].src, *dst = &items[k].dst;
         const uint64_t dim = items[k].dim, start = items[k].start, end = items[k].end, step = items[k].step;
@@ -523,15 +575,25 @@ int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_
         AIXK_REQUIRE(src->dtype == dst->dtype, "sliceSet: element types differ");
         AIXK_REQUIRE(aixk_dtype_size(src->dtype) == esz, "sliceSet of several items: element sizes differ");
         AIXK_REQUIRE((int)dim < dst->rank && step > 0 && end >= start, "sliceSet: bad slice");
-        aixhip_tensor window = *dst;
+        aixhip_tensor& window = windows[k];
+        window = *dst;
         window.shape[dim] = (end - start + step - 1) / step;
         window.offset = dst->offset + start * dst->strides[dim];
         window.strides[dim] = dst->strides[dim] * step;
         const uint64_t n = src->size;
         AIXK_REQUIRE(n > 0 && n == numel(&window) && n == numel(src), "sliceSet: source size does not match the slice");
         AIXK_REQUIRE(start + (window.shape[dim] - 1) * step < dst->shape[dim], "sliceSet: slice exceeds the destination");
+        window.size = n;
+        f = std::min({f, widest_factor(src, esz), widest_factor(&window, esz)});
+    }
+    for (uint32_t k = 0; k < count; ++k) {
+        aixhip_tensor wide_src = items[k].src;
+        aixhip_tensor& window = windows[k];
+        widen(&wide_src, f); widen(&window, f);
+        const aixhip_tensor* src = &wide_src;
+        const uint64_t n = src->size;
         CopyItem& it = table[k];
-        it.src = (u64)(uintptr_t)src->data; it.dst = (u64)(uintptr_t)dst->data; it.n = n; it.pad = 0;
+        it.src = (u64)(uintptr_t)src->data; it.dst = (u64)(uintptr_t)window.data; it.n = n; it.pad = 0;
         if (!collapse1(src, &it.ssp) || !collapse1(&window, &it.dsp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
         small = small && n < (1ull << 31) && view_extent(src) < (1ull << 31) && view_extent(&window) < (1ull << 31);
         starts[k] = grid;
@@ -541,7 +603,7 @@ int32_t aixk_slice_set_many(aixk_ctx* ctx, const aixk_slice_item* items, uint32_
     }
     starts[count] = grid;
     AIXK_TRY(table_upload(ctx, host, dev, all_bytes));
-    return by_size(items[0].src.dtype, [&](auto tag) {
+    return by_bytes(esz * f, [&](auto tag) {
         typedef decltype(tag) W;
         if (small) hipLaunchKernelGGL((copy_views_many_k<W, u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const CopyItem*)dev, (const u32*)(dev + table_bytes), (u32)count);
         else hipLaunchKernelGGL((copy_views_many_k<W, u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const CopyItem*)dev, (const u32*)(dev + table_bytes), (u32)count);

@@ -340,6 +340,67 @@ static void test_blocks_of_calls_that_wait_are_not_handed_out()
     for (void* p : {again, b, r, x, y, z}) dev.deallocate(p);
 }
 
+// Groups of waiting products leave one by one: a reader of one group's result sends that group off and leaves the
+// others waiting (the weight gradients of a backward pass go on collecting while the small products of attention come
+// and go); a writer of an operand sends off the groups that read it; flush(true) sends off what is left.
+static void test_groups_of_products_leave_apart()
+{
+    DeviceHIP dev;
+    aixk_ctx* ctx = dev.kernelContext();
+    auto half = [](void* p, size_t rows, size_t cols) { DeviceTensorParams t = matrix(p, rows, cols); t.dtype = DataType::kBFloat16; return t; };
+    std::vector<void*> all;
+    auto block = [&](size_t bytes) { void* p = dev.allocate(bytes); all.push_back(p); return p; };
+    void* x = block(64); void* y = block(64);
+    // three "weight gradients" [128,64] x [64,128] and, in between, "attention" products [64,64] x [64,64] whose results
+    // are read at once
+    void* wa[3]; void* wb[3]; void* wr[3];
+    uint64_t expected = stub_launches(ctx);
+    for (int i = 0; i < 3; ++i) {
+        wa[i] = block(128 * 64 * 2); wb[i] = block(64 * 128 * 2); wr[i] = block(128 * 128 * 2);
+        dev.matmul(half(wa[i], 128, 64), half(wb[i], 64, 128), half(wr[i], 128, 128));
+        CHECK(stub_launches(ctx) == expected);                      // waits
+        void* a = block(8192); void* b = block(8192); void* r = block(8192); void* o = block(8192);
+        dev.matmul(half(a, 64, 64), half(b, 64, 64), half(r, 64, 64));
+        CHECK(stub_launches(ctx) == expected);                      // waits in a group of its own
+        dev.transpose(half(r, 64, 64), half(o, 64, 64), 0, 1);      // its result is read: that group leaves, the other stays
+        expected += 2;
+        CHECK(stub_launches(ctx) == expected);
+        dev.transpose(half(wa[i], 128, 64), half(o, 64, 128), 0, 1);    // reading what a waiting product reads disturbs nothing
+        expected += 1;
+        CHECK(stub_launches(ctx) == expected);
+    }
+    stub_log_clear(ctx);
+    dev.transpose(half(x, 4, 4), half(wb[1], 4, 4), 0, 1);          // an operand of a waiting product is overwritten: the three go first
+    expected += 4;
+    CHECK(stub_launches(ctx) == expected);
+    const std::string log = stub_log(ctx);
+    CHECK(log == "aixk_matmul;aixk_matmul;aixk_matmul;aixk_transpose;");
+    // two groups wait; the reader of one result leaves the other group waiting, flush(true) sends it off
+    void* a = block(8192); void* b = block(8192); void* r = block(8192);
+    dev.matmul(half(wa[0], 128, 64), half(wb[0], 64, 128), half(wr[0], 128, 128));
+    dev.matmul(half(a, 64, 64), half(b, 64, 64), half(r, 64, 64));
+    CHECK(stub_launches(ctx) == expected);
+    dev.transpose(half(wr[0], 128, 128), half(wr[2], 128, 128), 0, 1);
+    expected += 2;
+    CHECK(stub_launches(ctx) == expected);
+    dev.flush();
+    expected += 1;
+    CHECK(stub_launches(ctx) == expected);
+    // a product that reads a waiting result sends only that result's group off and then waits itself
+    dev.matmul(half(wa[0], 128, 64), half(wb[0], 64, 128), half(wr[0], 128, 128));
+    dev.matmul(half(a, 64, 64), half(b, 64, 64), half(r, 64, 64));
+    dev.matmul(half(r, 64, 64), half(b, 64, 64), half(a, 64, 64));
+    expected += 1;
+    CHECK(stub_launches(ctx) == expected);
+    dev.synchronize();
+    expected += 2;
+    CHECK(stub_launches(ctx) == expected);
+    (void)y;
+    for (void* p : all) dev.deallocate(p);
+    dev.synchronize();
+    CHECK(dev.allocatedBytes() == 0);
+}
+
 // A fill that nothing has read yet is normally set aside at a flush and waits for its first user.  A call that waits
 // (a small product, a sliceSet) and is about to overwrite the fill's buffer is such a user: the fill leaves before the call,
 // never behind it -- behind it, it would wipe the call's result, and a recorded reader would take the fill's constant.
@@ -505,6 +566,7 @@ int main(int argc, char** argv)
     test_used_blocks_wait_for_the_gpu();
     test_out_of_memory_retry();
     test_blocks_of_calls_that_wait_are_not_handed_out();
+    test_groups_of_products_leave_apart();
     test_fills_do_not_land_behind_calls_that_wait();
     test_the_pool_is_trimmed_to_the_cache_limit();
     test_blocks_of_a_captured_step_stay_with_the_graph();
