@@ -180,18 +180,26 @@ struct DeviceHIP::Extras {
     // has to come after are marked, and only they leave with the other kinds of waiting calls (issuePending(true)): a
     // weight gradient of a backward pass goes on waiting for the other layers' while the small products of attention
     // come and go.  Whoever gets `true` sends the waiting calls off, so that no mark outlives the question.
+    const BlockTable* blocks{nullptr};
+    // a waiting product may use p: its block counts them (a pointer the table does not know is looked for in every group)
+    bool productsMayUse(const void* p) const
+    {
+        if (!grouped) return false;
+        const Block* b = blocks->find(p);
+        return !b || b->waiters;
+    }
     bool meetsRead(const void* p)
     {
         if (!p) return false;
         bool hit = waitWrites.size() && waitWrites.contains(p);
-        if (grouped) for (auto& g : groups) if (!g.out.empty() && g.writes.contains(p)) hit = g.leaves = true;
+        if (productsMayUse(p)) for (auto& g : groups) if (!g.out.empty() && g.writes.contains(p)) hit = g.leaves = true;
         return hit;
     }
     bool meetsWrite(const void* p)
     {
         if (!p) return false;
         bool hit = (waitWrites.size() && waitWrites.contains(p)) || (waitReads.size() && waitReads.contains(p));
-        if (grouped) for (auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) hit = g.leaves = true;
+        if (productsMayUse(p)) for (auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) hit = g.leaves = true;
         return hit;
     }
     // a call that reads r0, r1 and writes w neither uses what waits nor is used by it (every operand is looked at: all
@@ -207,8 +215,8 @@ struct DeviceHIP::Extras {
     bool waitingUses(const void* p) const
     {
         if (!p || !anyUses()) return false;
-        if (waitWrites.contains(p) || waitReads.contains(p)) return true;
-        if (grouped) for (const auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) return true;
+        if ((waitWrites.size() && waitWrites.contains(p)) || (waitReads.size() && waitReads.contains(p))) return true;
+        if (productsMayUse(p)) for (const auto& g : groups) if (!g.out.empty() && (g.writes.contains(p) || g.reads.contains(p))) return true;
         return false;
     }
     void noteWaiting(const void* r0, const void* r1, const void* w)
@@ -336,6 +344,7 @@ DeviceHIP::DeviceHIP(size_t deviceIndex)
     if (const char* e = std::getenv("AIXHIP_MAX_BUFFER_SLOTS"); e && *e) cfg.maxBufferSlots = std::max<size_t>(4, std::min<size_t>(60, std::strtoull(e, nullptr, 10)));
     cfg.supportsStridedFusion = true;
     m_extras = std::make_unique<Extras>();
+    m_extras->blocks = &m_blocks;
     setFuseConfig(cfg);
 }
 
@@ -1340,6 +1349,7 @@ void DeviceHIP::matmul(const DeviceTensorParams& a, const DeviceTensorParams& b,
             if (!into) { issuePending(); into = &ex.groups[0]; }
             into->a.push_back(pa); into->b.push_back(pb); into->out.push_back(pr);
             into->reads.insert(pa.data); into->reads.insert(pb.data); into->writes.insert(pr.data);
+            for (const void* p : {(const void*)pa.data, (const void*)pb.data, (const void*)pr.data}) if (Block* blk = m_blocks.find(p)) ++blk->waiters;
             ++ex.grouped;
             markTouched(a.data); markTouched(b.data); markTouched(result.data);
             return;
@@ -1419,6 +1429,8 @@ void DeviceHIP::issuePending(bool marked)
         if (g.out.empty() || !leaves) continue;
         const uint32_t count = (uint32_t)g.out.size();
         sent(count == 1 ? aixk_matmul(m_ctx, &g.a[0], &g.b[0], &g.out[0]) : aixk_matmul_grouped(m_ctx, g.a.data(), g.b.data(), g.out.data(), count), count);
+        for (uint32_t i = 0; i < count; ++i)
+            for (const void* p : {(const void*)g.a[i].data, (const void*)g.b[i].data, (const void*)g.out[i].data}) if (Block* blk = m_blocks.find(p)) --blk->waiters;
         g.a.clear(); g.b.clear(); g.out.clear(); g.reads.clear(); g.writes.clear();
         ex.grouped -= count;
     }
@@ -1709,7 +1721,7 @@ void DeviceHIP::sliceSet(const DeviceTensorParams& src, const DeviceTensorParams
                                (ex.slices.empty() || dataTypeSize(static_cast<DataType>(ex.slices[0].src.dtype)) == dataTypeSize(src.dtype));
             // (products that wait: the copy comes after those that write its source or use its destination)
             bool apartFromProducts = true;
-            if (ex.grouped) {
+            if (ex.productsMayUse(src.data) || ex.productsMayUse(dst.data)) {
                 for (auto& g : ex.groups) {
                     if (g.out.empty() || !(g.writes.contains(src.data) || g.writes.contains(dst.data) || g.reads.contains(dst.data))) continue;
                     g.leaves = true;

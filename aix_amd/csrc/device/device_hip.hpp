@@ -139,6 +139,7 @@ private:
         bool touched{false};     // enqueued GPU work has referenced the block since it was allocated
         bool freed{false};       // deallocate() has been called; the block waits in m_limbo
         bool inGraph{false};     // captured work uses the block: once freed it is kept aside, not pooled
+        uint32_t waiters{0};     // operands and results of waiting products in the block (one lookup tells most callers "none")
     };
     struct Extras;
 
