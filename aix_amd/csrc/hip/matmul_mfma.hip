@@ -10,13 +10,16 @@
 //   16-bit, mid-size      gemm_tile16_k: 128x128 / 128x64 / 64x64 tiles, register staging, both operand
 //                         forms, stacks of matrices (blockIdx.y) and K splits over workgroups (blockIdx.z);
 //   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
+//   16-bit, K = 64        gemm_k64_nt_k: stacks of products with one K step (attention's scores), fragments loaded from
+//                         global memory by the waves themselves, no LDS;
 //   16-bit, odd layouts   gemm_nt16_k: K-contiguous operands only, bounds-checked (others are gathered first);
 //   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
 //   f32, very large       split_planes_k + gemm_direct16_k<PLANES>: the planes written to memory once, six plane pairs
 //                         multiplied by the LDS-direct 16-bit kernel;
 //   f32                   gemm_nt32_k: v_mfma_f32_32x32x2f32, 128x128 or 64x64 tile x BK=32, both operand forms.
 //
-// All but the first two use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split) with the accumulators
+// All but the first two use 4 waves in a 2x2 arrangement (gemm_small16_k: one 32x32 tile, K split; gemm_k64_nt_k: four
+// independent waves) with the accumulators
 // resident in the 512-entry unified register file.  Every lane feeds the 16-bit MFMA with 8 consecutive K
 // values of one row; because A and B use the same lane->K assignment, the dot products are independent of
 // how the instruction numbers K internally.
@@ -420,6 +423,84 @@ template <int OFF> __device__ __forceinline__ u32x4 tr_fragment_at(const unsigne
     asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
     asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "i"(OFF));       // k + 4
     return u32x4{lo.x, lo.y, hi.x, hi.y};
+}
+
+// K = 64 with both operands K-contiguous (A [M, 64], B given as [N, 64]: the scores q . k^T of attention and the
+// gradient dO . v^T, on stacks of a few hundred matrices).  Such a product moves a byte of result per 64 flop: it is a
+// stream of stores, and what a tile pipeline adds -- stages in LDS, barriers, a slab for the result -- only keeps its
+// loads and stores from overlapping.  Here a wave is on its own: its lanes load the MFMA fragments straight from global
+// memory (16 bytes per lane and fragment), 64 rows of A once and then STEPS blocks of 64 rows of B one after the other,
+// the next block's loads in flight while this one is multiplied and stored.  The operands are swapped in the MFMA, so
+// that the four accumulators of a lane are four neighbouring columns of one row, and the B rows of two neighbouring
+// column tiles are dealt out so that a lane's columns of both are eight in a row: 16-byte stores, no LDS, no barrier.
+// The four waves of a workgroup cover 128 rows x 128 STEPS columns; their shared fragments meet in the L1.
+template <class T, int STEPS>
+__global__ __launch_bounds__(256) void gemm_k64_nt_k(GemmArgs g, BatchArgs bt, u32 spread)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // workgroups go round the eight XCDs in the order of their numbers: with `spread` all tiles of a matrix are numbered
+    // onto one XCD, so that its operands cross the fabric once and meet in one L2
+    const u32 per = g.tiles_m * g.tiles_n;
+    u32 matrix = blockIdx.x / per, tile = blockIdx.x - matrix * per;
+    if (spread) {
+        const u32 xcd = blockIdx.x & 7u, idx = blockIdx.x >> 3;
+        matrix = (idx / per) * 8u + xcd;
+        tile = idx % per;
+    }
+    const u32 tn = tile % g.tiles_n, tm = tile / g.tiles_n;
+    const u16* A = (const u16*)g.a;
+    const u16* B = (const u16*)g.b;
+    u16* C = (u16*)g.c;
+    if (bt.table) {
+        const u64* entry = bt.table + 3 * (u64)matrix;
+        A = global_ptr<const u16>(entry[0]); B = global_ptr<const u16>(entry[1]); C = global_ptr<u16>(entry[2]);
+    } else if (bt.rank) {
+        u32 rest = matrix;
+        for (int d = (int)bt.rank - 1; d >= 0; --d) {
+            const u32 q = rest / bt.ext[d], c = rest - q * bt.ext[d];
+            A += (u64)c * bt.sa[d]; B += (u64)c * bt.sb[d];
+            rest = q;
+        }
+        C += (u64)matrix * bt.sc;
+    }
+    const u64 m0 = (u64)tm * 128 + (u64)(wave >> 1) * 64;
+    const u64 n0 = (u64)tn * (128 * STEPS) + (u64)(wave & 1) * (64 * STEPS);
+    const int r = lane & 15, kq = lane >> 4;
+    // operand row r of the even tile of a pair is B row 8 (r / 4) + r % 4 of the pair's 32, of the odd tile that row + 4
+    const int rb = 8 * (r >> 2) + (r & 3);
+    u32x4 fa[4][2], fb[2][4][2];
+    auto load_b = [&](int step, u32x4 (&f)[4][2]) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) f[j][s] = *(const u32x4*)(B + (n0 + 64 * step + 32 * (j >> 1) + 4 * (j & 1) + rb) * g.ldb + 32 * s + 8 * kq);
+    };
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int s = 0; s < 2; ++s) fa[i][s] = *(const u32x4*)(A + (m0 + 16 * i + r) * g.lda + 32 * s + 8 * kq);
+    load_b(0, fb[0]);
+#pragma unroll
+    for (int step = 0; step < STEPS; ++step) {
+        if (step + 1 < STEPS) load_b(step + 1, fb[(step + 1) & 1]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            f32x4 acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                acc[j] = Mma16<T>::run16(fb[step & 1][j][0], fa[i][0], acc[j]);
+                acc[j] = Mma16<T>::run16(fb[step & 1][j][1], fa[i][1], acc[j]);
+            }
+            // lane (kq, r): row m0 + 16 i + r, columns n0 + 64 step + 32 p + 8 kq ... + 7 of pair p
+            u16* row = C + (m0 + 16 * i + r) * g.N + n0 + 64 * step + 8 * kq;
+#pragma unroll
+            for (int pair = 0; pair < 2; ++pair) {
+                const f32x4 lo = acc[2 * pair], hi = acc[2 * pair + 1];
+                *(u32x4*)(row + 32 * pair) = u32x4{Mma16<T>::pack(lo.x, lo.y), Mma16<T>::pack(lo.z, lo.w), Mma16<T>::pack(hi.x, hi.y), Mma16<T>::pack(hi.z, hi.w)};
+            }
+        }
+    }
 }
 
 // PLANES: an f32 product on the bf16 pipe from operands that split_planes_k has laid out as three bf16 planes each (hi, mid,
@@ -1604,6 +1685,55 @@ int launch_tile16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b,
     return AIXK_OK;
 }
 
+// Stacks and groups of K = 64 products with K-contiguous operands and whole 128 x 128 tiles (gemm_k64_nt_k).  -1: not
+// for this product.
+int launch_k64(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const aixhip_tensor* out, const Space<3>* batch, const u64* table)
+{
+    const uint64_t M = a->shape[0], K = a->shape[1], N = b->shape[1];
+    constexpr size_t esz = 2;
+    if (!(K == 64 && M % 128 == 0 && N % 128 == 0 && a->strides[1] == 1 && b->strides[0] == 1)) return -1;
+    const char* qa = (const char*)a->data + a->offset * esz;
+    const char* qb = (const char*)b->data + b->offset * esz;
+    const uint64_t la = a->strides[0], lb = b->strides[1];
+    if (!(la % 8 == 0 && lb % 8 == 0 && aligned16(qa) && aligned16(qb) && aligned16(out->data))) return -1;
+    BatchArgs bt{};
+    uint64_t count = 1;
+    if (batch) {
+        if (batch->rank > 3) return -1;
+        bt.rank = (u32)batch->rank;
+        for (int d = 0; d < batch->rank; ++d) {
+            if (batch->shape[d] >= (1ull << 31) || batch->stride[0][d] % 8 != 0 || batch->stride[1][d] % 8 != 0) return -1;
+            bt.ext[d] = (u32)batch->shape[d]; bt.sa[d] = batch->stride[0][d]; bt.sb[d] = batch->stride[1][d];
+            count *= batch->shape[d];
+        }
+        if (count > 65535) return -1;
+        bt.sc = M * N;
+        bt.table = table;
+    }
+    // a wave sweeps STEPS blocks of 64 columns: as many as still leave three workgroups per compute unit
+    int steps = 1;
+    for (int cand : {2, 4, 8})
+        if ((N / 128) % cand == 0 && (M / 128) * (N / 128 / cand) * count >= 3 * (uint64_t)ctx->cus) steps = cand;
+    const uint64_t tiles = (M / 128) * (N / 128 / steps);
+    if (tiles * count >= (1ull << 31) || (M / 128) * (N / 128) * count < 2 * (uint64_t)ctx->cus) return -1;
+    GemmArgs g{};
+    g.a = qa; g.b = qb; g.c = out->data;
+    g.M = M; g.N = N; g.K = K; g.lda = la; g.ldb = lb;
+    g.tiles_m = (u32)(M / 128); g.tiles_n = (u32)(N / 128 / steps);
+    const u32 spread = count % 8 == 0 ? 1u : 0u;
+    auto launch = [&](auto kernel) { hipLaunchKernelGGL(kernel, dim3((unsigned)(tiles * count)), dim3(256), 0, ctx->stream, g, bt, spread); };
+    auto by_steps = [&](auto tag) {
+        typedef decltype(tag) T;
+        if (steps == 8) launch(gemm_k64_nt_k<T, 8>);
+        else if (steps == 4) launch(gemm_k64_nt_k<T, 4>);
+        else if (steps == 2) launch(gemm_k64_nt_k<T, 2>);
+        else launch(gemm_k64_nt_k<T, 1>);
+    };
+    if (out->dtype == AIXK_BF16) by_steps(bf16{}); else by_steps(f16{});
+    AIXK_HIP(hipGetLastError());
+    return AIXK_OK;
+}
+
 // 16-bit products of whole 128 x {128, 192, 256} x 64 tiles, at least half a tile per compute unit: the LDS-direct kernel
 // on its smaller tiles (gemm_direct16_k).  `batch` / `table` as for launch_small16 (a stack of matrices, or a group of
 // separate products).  limit > 0: only if the estimated cost stays below it (the caller has another kernel to offer).
@@ -1711,6 +1841,10 @@ int route16(aixk_ctx* ctx, const aixhip_tensor* a, const aixhip_tensor* b, const
         // a group of separate products (table): no K splits -- their partial planes assume one dense stack of results
         if (M <= 64) return launch_tile16(ctx, a, b, out, batch, 0, table ? 1 : splits_for(t64 * count, (K + 63) / 64 * 2, 4), table);
         if (N <= 64) return launch_tile16(ctx, a, b, out, batch, 1, table ? 1 : splits_for(t12864 * count, (K + 31) / 32, 2), table);
+        if (K == 64) {                                     // one K step: a stream of stores (gemm_k64_nt_k)
+            const int rc = launch_k64(ctx, a, b, out, batch, table);
+            if (rc != -1) return rc;
+        }
         if (K >= 512) {                                    // whole tiles and enough K steps to pay for its prologue: the LDS-direct kernel
             const int rc = launch_direct16(ctx, a, b, out, batch, table, 0);
             if (rc != -1) return rc;

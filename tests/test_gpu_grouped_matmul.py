@@ -68,6 +68,8 @@ def array_of(descs):
                                   (128, 256, 192, "S", "S", 6), (512, 512, 512, "N", "N", 9), (96, 40, 72, "N", "N", 3),
                                   # whole 128 x {128, 192} tiles and K >= 512: the LDS-direct kernel's smaller tiles, addresses from the table
                                   (768, 1024, 768, "T", "N", 6), (384, 512, 640, "N", "T", 10), (256, 576, 512, "S", "N", 16),
+                                  # K = 64, both operands K-contiguous, two 128 x 128 tiles per compute unit: the kernel without LDS reads the table
+                                  (512, 64, 512, "N", "T", 32), (256, 64, 384, "S", "T", 86),
                                   # 216 whole 256 x 256 tiles over the group: one round of the chip on that kernel's largest tile, in every layout
                                   (768, 576, 768, "T", "N", 24), (768, 512, 768, "N", "T", 24), (768, 512, 768, "T", "T", 24), (768, 512, 768, "N", "N", 24)], ids=str)
 def test_grouped_launch_matches_single_launches(gpu, dtype, case):

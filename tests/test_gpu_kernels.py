@@ -1068,9 +1068,42 @@ def test_matmul_stacks(gpu, dtype):
         big_c = T.HostTensor(draw(8 * 512 * 640, -1, 1), dtype, [8, 512, 640])
         check_matmul_stack(gpu, big_at, big_c, f"stack of whole 128 x 128 tiles, transposed first operand {NAMES[dtype]}")
         gpu.release()
+        # K = 64 with both operands K-contiguous and two whole 128 x 128 tiles per compute unit over the stack: the kernel
+        # without LDS (attention's scores at their real shape: heads as a permuted view, k transposed) -- 32 matrices
+        # numbered XCD by XCD, 44 in plain order, unequal tile counts per side
+        for (b2, h2, s2, t2) in ((4, 8, 512, 512), (11, 4, 512, 512), (8, 8, 256, 640)):
+            qs = draw(b2 * s2 * h2 * 64, -0.5, 0.5)
+            ks = draw(b2 * t2 * h2 * 64, -1, 1)
+            qv = T.HostTensor(qs, dtype, [b2, h2, s2, 64], [s2 * h2 * 64, 64, h2 * 64, 1])
+            kv = T.HostTensor(ks, dtype, [b2, h2, 64, t2], [t2 * h2 * 64, 64, 1, h2 * 64])
+            check_matmul_stack(gpu, qv, kv, f"{b2 * h2} score products [{s2}, 64] x [64, {t2}] {NAMES[dtype]}")
+            gpu.release()
     # matrices too small or too odd for the matrix-core route
     check_matmul_stack(gpu, T.HostTensor(draw(7 * 5 * 3, -1, 1), dtype, [7, 5, 3]), T.HostTensor(draw(7 * 3 * 4, -1, 1), dtype, [7, 3, 4]),
                        f"tiny stack {NAMES[dtype]}")
+    gpu.release()
+
+
+@pytest.mark.parametrize("dtype", [O.BF16, O.F16], ids=ids)
+@pytest.mark.parametrize("case", [(96, 512, 512), (100, 256, 2048), (192, 512, 512), (96, 1024, 1024)], ids=str)
+def test_matmul_k64_stacks_at_every_sweep_length(gpu, dtype, case):
+    """Stacks of K = 64 products with K-contiguous operands, large enough that a wave of the kernel without LDS sweeps two,
+    four and eight blocks of 64 columns (on 256 compute units: the cases in this order 2, 4, 4, 8), the matrices numbered
+    XCD by XCD (counts that are multiples of 8) and in plain order (100).  Small integers: every sum is exact in f32, so
+    the result is the one rounding of the exact product and the check is bit equality with numpy."""
+    count, m, n = case
+    rng = np.random.default_rng(25500 + count + m + dtype)
+    av = rng.integers(-3, 4, (count, m, 64)).astype(np.float32)
+    bv = rng.integers(-3, 4, (count, n, 64)).astype(np.float32)                # stored [n, k]: the transposed second operand
+    a = T.HostTensor(O.to_storage(av.reshape(-1), dtype), dtype, [count, m, 64])
+    b = T.HostTensor(O.to_storage(bv.reshape(-1), dtype), dtype, [count, 64, n], [n * 64, 1, 64])
+    pa, da = gpu.put(a)
+    pb, db = gpu.put(b)
+    po, do = gpu.put(T.empty(dtype, [count, m, n], fill=1))
+    G.run_gpu(gpu, "aixk_matmul_batched", G.ref(da), G.ref(db), G.ref(do))
+    got = gpu.fetch(po, np.zeros(count * m * n, O.NP_STORAGE[dtype]))
+    want = np.matmul(av, bv.transpose(0, 2, 1))                                # |sums| <= 576: exact in f32, rounded once to the 16-bit type below
+    T.assert_same_bits(got, O.to_storage(want.reshape(-1).astype(np.float64), dtype), f"{count} products [{m}, 64] x [64, {n}] {NAMES[dtype]}")
     gpu.release()
 
 
