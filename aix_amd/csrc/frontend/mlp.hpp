@@ -49,10 +49,11 @@ inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* l
     const bool capturing = capture && cfg.captureAt >= 0;
     if (capturing && !cfg.adamInPlace) throw std::invalid_argument("runMlp: a captured step needs Adam's in-place form (its constants must not change from step to step)");
     dev->synchronize();
-    Tensor loss;                                                  // of the last step issued (a replay writes the captured step's)
+    Tensor loss;                                                  // the captured step's graph of nodes: its tensors are what a replay writes
+    Value lossValue;                                              // of the last step issued
     double aside = 0;
-    auto issueStep = [&](int s) {
-        loss = Tensor();                                          // the previous step's graph of nodes goes first
+    auto issueStep = [&](int s, bool keepGraph) {
+        loss = Tensor();                                          // a graph that was kept goes first
         opt.zeroGrad();
         const Tensor logits = l3.forward(relu(l2.forward(relu(l1.forward(x)))));
         loss = crossEntropy(softmax(logits, 1, true), y);
@@ -64,14 +65,16 @@ inline void runMlp(Device* dev, const MlpConfig& cfg, const MlpHost& h, float* l
             aside = std::chrono::duration<double>(std::chrono::steady_clock::now() - n0).count();
         }
         opt.step();
+        lossValue = loss.value();
+        if (!keepGraph) loss = Tensor();                          // an eager step lets go of its graph while the GPU still works through the step (see runTransformer)
     };
     for (int s = 0; s < cfg.steps; ++s) {
         const auto t0 = std::chrono::steady_clock::now();
         aside = 0;
         const bool captured = capturing && s >= cfg.captureAt;
-        if (captured && s == cfg.captureAt) { capture->begin(); issueStep(s); capture->end(); }
-        if (captured) capture->replay(); else issueStep(s);
-        losses[s] = loss.value().item();          // synchronizes
+        if (captured && s == cfg.captureAt) { capture->begin(); issueStep(s, true); capture->end(); }
+        if (captured) capture->replay(); else issueStep(s, false);
+        losses[s] = lossValue.item();             // synchronizes
         if (step_seconds) step_seconds[s] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() - aside;
     }
 }

@@ -96,9 +96,10 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
     const float scale = 1.0f / std::sqrt((float)dh);
     dev->synchronize();
 
-    Tensor loss;                                                 // of the last step issued (a replay writes the captured step's)
-    auto issueStep = [&] {
-        loss = Tensor();                                         // the previous step's graph of nodes goes first
+    Tensor loss;                                                 // the captured step's graph of nodes: its tensors are what a replay writes
+    Value lossValue;                                             // of the last step issued
+    auto issueStep = [&](bool keepGraph) {
+        loss = Tensor();                                         // a graph that was kept goes first
         for (auto& p : P) p.zeroGrad();
         std::vector<Tensor> W;                                   // bf16 working copies
         for (auto& p : P) W.push_back(p.to(BF16));
@@ -146,13 +147,19 @@ inline void runTransformer(Device* dev, const TransformerConfig& c, const int32_
         const Tensor logits = matmul(xf, W[at + 2]).to(F32);
         loss = crossEntropy(softmax(logits, 1, true), target);
         loss.backwardOnce();
+        lossValue = loss.value();
+        // An eager step lets go of its graph here, before the loss is read: the host takes the nodes and their intermediate
+        // results apart while the GPU still works through the step (the device keeps a freed block until the work enqueued
+        // on it has passed), instead of opening the next step with it while the GPU idles; and results that only the graph
+        // held and nothing recorded reads any more are never stored.
+        if (!keepGraph) loss = Tensor();
     };
     for (int step = 0; step < c.steps; ++step) {
         const auto t0 = std::chrono::steady_clock::now();
         const bool captured = capture && c.captureAt >= 0 && step >= c.captureAt;
-        if (captured && step == c.captureAt) { capture->begin(); issueStep(); capture->end(); }
-        if (captured) capture->replay(); else issueStep();
-        losses[step] = loss.value().item();                      // synchronizes: forward and backward have run
+        if (captured && step == c.captureAt) { capture->begin(); issueStep(true); capture->end(); }
+        if (captured) capture->replay(); else issueStep(false);
+        losses[step] = lossValue.item();                         // synchronizes: forward and backward have run
         if (step_seconds) step_seconds[step] = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
         for (size_t i = 0; i < P.size(); ++i) {
             gradNorms[(size_t)step * P.size() + i] = P[i].grad().l2Norm();
