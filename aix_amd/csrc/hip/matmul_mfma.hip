@@ -10,8 +10,8 @@
 //   16-bit, mid-size      gemm_tile16_k: 128x128 / 128x64 / 64x64 tiles, register staging, both operand
 //                         forms, stacks of matrices (blockIdx.y) and K splits over workgroups (blockIdx.z);
 //   16-bit, small         gemm_small16_k: 32x32 tile, K split over the workgroup's four waves;
-//   16-bit, K = 64        gemm_k64_nt_k: stacks of products with one K step (attention's scores), fragments loaded from
-//                         global memory by the waves themselves, no LDS;
+//   16-bit, K = 64        gemm_k64_nt_k: stacks of products with one K step (attention's scores): every wave on its
+//                         own, rows to fragments and accumulators to rows through a slab of its own, no barrier;
 //   16-bit, odd layouts   gemm_nt16_k: K-contiguous operands only, bounds-checked (others are gathered first);
 //   f32, large            gemm_x3_k: each operand as three bf16 planes on the bf16 matrix pipe, f32 accumulation;
 //   f32, very large       split_planes_k + gemm_direct16_k<PLANES>: the planes written to memory once, six plane pairs
@@ -427,13 +427,14 @@ template <int OFF> __device__ __forceinline__ u32x4 tr_fragment_at(const unsigne
 
 // K = 64 with both operands K-contiguous (A [M, 64], B given as [N, 64]: the scores q . k^T of attention and the
 // gradient dO . v^T, on stacks of a few hundred matrices).  Such a product moves a byte of result per 64 flop: it is a
-// stream of stores, and what a tile pipeline adds -- stages in LDS, barriers, a slab for the result -- only keeps its
-// loads and stores from overlapping.  Here a wave is on its own: its lanes load the MFMA fragments straight from global
-// memory (16 bytes per lane and fragment), 64 rows of A once and then STEPS blocks of 64 rows of B one after the other,
-// the next block's loads in flight while this one is multiplied and stored.  The operands are swapped in the MFMA, so
+// stream of stores, and what a tile pipeline adds -- stages shared by a workgroup, a barrier per K step, a prologue and
+// an epilogue that do not overlap -- only keeps its loads and stores from running side by side.  Here a wave is on its
+// own: it loads 64 rows of A once and then STEPS blocks of 64 rows of B one after the other, the next block's loads in
+// flight while this one is multiplied and stored, and never meets a barrier.  The operands are swapped in the MFMA, so
 // that the four accumulators of a lane are four neighbouring columns of one row, and the B rows of two neighbouring
-// column tiles are dealt out so that a lane's columns of both are eight in a row: 16-byte stores, no LDS, no barrier.
-// The four waves of a workgroup cover 128 rows x 128 STEPS columns; their shared fragments meet in the L1.
+// column tiles are dealt out so that a lane's columns of both are eight in a row.  Rows of 128 bytes become fragments,
+// and accumulators become rows, in a slab of LDS that belongs to the wave (see below).  The four waves of a workgroup
+// cover 128 rows x 128 STEPS columns; what they share meets in the L1.
 template <class T, int STEPS>
 __global__ __launch_bounds__(256) void gemm_k64_nt_k(GemmArgs g, BatchArgs bt, u32 spread)
 {
@@ -468,37 +469,72 @@ __global__ __launch_bounds__(256) void gemm_k64_nt_k(GemmArgs g, BatchArgs bt, u
     const int r = lane & 15, kq = lane >> 4;
     // operand row r of the even tile of a pair is B row 8 (r / 4) + r % 4 of the pair's 32, of the odd tile that row + 4
     const int rb = 8 * (r >> 2) + (r & 3);
-    u32x4 fa[4][2], fb[2][4][2];
-    auto load_b = [&](int step, u32x4 (&f)[4][2]) {
+    // The wave's own slab: 32 rows of 128 bytes at a pitch of 144 (16 rows that differ in nothing else land in 16 different
+    // banks).  Global memory is only ever touched by eight neighbouring lanes per 128-byte row -- a lane per row, which is
+    // what the fragments and the accumulators are, costs the L1 a tag lookup per lane -- and the slab turns rows into
+    // fragments and accumulators into rows.  A wave's LDS operations complete in order: no barrier anywhere.
+    __shared__ __attribute__((aligned(16))) unsigned char slabs[4][32 * 144];
+    unsigned char* slab = slabs[wave];
+    const int lr = lane >> 3, lc = lane & 7;
+    auto fetch32 = [&](const u16* base, u64 row0, u64 ld, u32x4 (&t)[4]) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int s = 0; s < 2; ++s) f[j][s] = *(const u32x4*)(B + (n0 + 64 * step + 32 * (j >> 1) + 4 * (j & 1) + rb) * g.ldb + 32 * s + 8 * kq);
+        for (int q = 0; q < 4; ++q) t[q] = *(const u32x4*)(base + (row0 + 8 * q + lr) * ld + 8 * lc);
     };
+    auto to_slab = [&](const u32x4 (&t)[4]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+        for (int q = 0; q < 4; ++q) *(u32x4*)(slab + (8 * q + lr) * 144 + 16 * lc) = t[q];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    auto fragment = [&](int row, int s) { return *(const u32x4*)(slab + row * 144 + 16 * (kq + 4 * s)); };
+    u32x4 fa[4][2], fb[4][2], ta[2][4], tb[2][2][4];
+    fetch32(A, m0, g.lda, ta[0]);
+    fetch32(A, m0 + 32, g.lda, ta[1]);
+    fetch32(B, n0, g.ldb, tb[0][0]);
+    fetch32(B, n0 + 32, g.ldb, tb[0][1]);
 #pragma unroll
-        for (int s = 0; s < 2; ++s) fa[i][s] = *(const u32x4*)(A + (m0 + 16 * i + r) * g.lda + 32 * s + 8 * kq);
-    load_b(0, fb[0]);
+    for (int h = 0; h < 2; ++h) {
+        to_slab(ta[h]);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int s = 0; s < 2; ++s) fa[2 * h + t][s] = fragment(16 * t + r, s);
+        asm volatile("" ::: "memory");
+    }
 #pragma unroll
     for (int step = 0; step < STEPS; ++step) {
-        if (step + 1 < STEPS) load_b(step + 1, fb[(step + 1) & 1]);
+        if (step + 1 < STEPS) {
+            fetch32(B, n0 + 64 * (step + 1), g.ldb, tb[(step + 1) & 1][0]);
+            fetch32(B, n0 + 64 * (step + 1) + 32, g.ldb, tb[(step + 1) & 1][1]);
+        }
+#pragma unroll
+        for (int pair = 0; pair < 2; ++pair) {
+            to_slab(tb[step & 1][pair]);
+#pragma unroll
+            for (int s = 0; s < 2; ++s) { fb[2 * pair][s] = fragment(rb, s); fb[2 * pair + 1][s] = fragment(4 + rb, s); }
+            asm volatile("" ::: "memory");
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             f32x4 acc[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 acc[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-                acc[j] = Mma16<T>::run16(fb[step & 1][j][0], fa[i][0], acc[j]);
-                acc[j] = Mma16<T>::run16(fb[step & 1][j][1], fa[i][1], acc[j]);
+                acc[j] = Mma16<T>::run16(fb[j][0], fa[i][0], acc[j]);
+                acc[j] = Mma16<T>::run16(fb[j][1], fa[i][1], acc[j]);
             }
-            // lane (kq, r): row m0 + 16 i + r, columns n0 + 64 step + 32 p + 8 kq ... + 7 of pair p
-            u16* row = C + (m0 + 16 * i + r) * g.N + n0 + 64 * step + 8 * kq;
+            // lane (kq, r) holds row r, columns 32 p + 8 kq ... + 7 of pair p
 #pragma unroll
             for (int pair = 0; pair < 2; ++pair) {
                 const f32x4 lo = acc[2 * pair], hi = acc[2 * pair + 1];
-                *(u32x4*)(row + 32 * pair) = u32x4{Mma16<T>::pack(lo.x, lo.y), Mma16<T>::pack(lo.z, lo.w), Mma16<T>::pack(hi.x, hi.y), Mma16<T>::pack(hi.z, hi.w)};
+                *(u32x4*)(slab + r * 144 + 64 * pair + 16 * kq) = u32x4{Mma16<T>::pack(lo.x, lo.y), Mma16<T>::pack(lo.z, lo.w), Mma16<T>::pack(hi.x, hi.y), Mma16<T>::pack(hi.z, hi.w)};
             }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const u32x4 v = *(const u32x4*)(slab + (lr + 8 * h) * 144 + 16 * lc);
+                *(u32x4*)(C + (m0 + 16 * i + lr + 8 * h) * g.N + n0 + 64 * step + 8 * lc) = v;
+            }
+            asm volatile("" ::: "memory");
         }
     }
 }
