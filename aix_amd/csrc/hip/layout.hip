@@ -306,6 +306,21 @@ __global__ __launch_bounds__(kBlock) void index_select_k(const W* __restrict__ s
     }
 }
 
+// Rows of a dense source whose length is a whole number of 16-byte words (an embedding table's rows): a lane moves a
+// word, not an element -- one index load and one division per 16 bytes instead of per element.
+template <class IDX>
+__global__ __launch_bounds__(kBlock) void index_select_rows_k(const u128* __restrict__ src, u128* __restrict__ dst, const i32* __restrict__ idx,
+                                                              Space<1> isp, u64 words, u64 inner, u64 ni, u64 extent)
+{
+    for (u64 i = (u64)blockIdx.x * kBlock + threadIdx.x; i < words; i += (u64)gridDim.x * kBlock) {
+        const u64 e = i % inner, k = (i / inner) % ni, o = i / (ni * inner);
+        const i32 at = idx[locate<IDX>(isp, (IDX)k)];
+        u128 v{0, 0};
+        if (at >= 0 && (u64)at < extent) v = src[(o * extent + (u64)at) * inner + e];           // (an index outside the source: a zero)
+        dst[i] = v;
+    }
+}
+
 // ---- indexAdd ----------------------------------------------------------------------------------
 // dst[slot] += src[i] with duplicates summed: atomics.  32/64-bit types use native atomics;
 // 8/16-bit types update their containing 32-bit word with a compare-and-swap loop.
@@ -697,6 +712,22 @@ int32_t aixk_index_select(aixk_ctx* ctx, const aixhip_tensor* src, const aixhip_
     Space<1> ssp, isp;
     if (!collapse1(src, &ssp) || !collapse1(indices, &isp)) return fail(AIXK_EINVAL, "view does not collapse to %d dims", kMaxDims);
     const bool small = n < (1ull << 31) && view_extent(src) < (1ull << 31) && numel(src) < (1ull << 31);
+    {
+        // a dense source, rows of whole 16-byte words: word by word
+        const size_t esz = aixk_dtype_size(src->dtype);
+        bool dense = src->rank > 0;
+        uint64_t run = 1;
+        for (int d = src->rank - 1; d >= 0 && dense; --d) { dense = src->shape[d] == 1 || src->strides[d] == run; run *= src->shape[d]; }
+        const char* base = (const char*)src->data + src->offset * esz;
+        if (dense && esz && (inner * esz) % 16 == 0 && aligned16(base) && aligned16(dst->data)) {
+            const uint64_t per = inner * esz / 16, words = n * esz / 16;
+            const unsigned grid = grid_for(words, kBlock, (unsigned)ctx->cus * 32u);
+            if (small) hipLaunchKernelGGL((index_select_rows_k<u32>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const u128*)base, (u128*)dst->data, (const i32*)indices->data, isp, (u64)words, (u64)per, (u64)ni, (u64)src->shape[dim]);
+            else hipLaunchKernelGGL((index_select_rows_k<u64>), dim3(grid), dim3(kBlock), 0, ctx->stream, (const u128*)base, (u128*)dst->data, (const i32*)indices->data, isp, (u64)words, (u64)per, (u64)ni, (u64)src->shape[dim]);
+            AIXK_HIP(hipGetLastError());
+            return (int32_t)AIXK_OK;
+        }
+    }
     return by_size(src->dtype, [&](auto tag) {
         typedef decltype(tag) W;
         const unsigned grid = grid_for(n, kBlock, (unsigned)ctx->cus * 32u);
